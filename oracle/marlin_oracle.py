@@ -1,0 +1,576 @@
+"""CPU oracle for the Marlin W4A16 path.  TEST INFRASTRUCTURE ONLY.
+
+This module restates, in plain numpy, the algorithms the reference implements
+for its Marlin-family W4A16 GEMM.  It is the checker that the HIP kernels are
+compared against.  Nothing in the shipped package imports it: only tests,
+``__graft_entry__.smoke()`` and the ``cpu_baseline`` leg of ``bench.py`` do.
+
+Every function names the reference source it follows (paths relative to the
+reference checkout).  How each function is pinned (none is "parity unpinned"):
+
+* ScalarType ids           closed-form bitfield + min/max table of
+                           tests/test_scalartype.py:10-25
+* gptq/awq/col packing     unpack(pack(x)) == x, brute force against a
+                           per-element python loop
+* Marlin weight layout     two independent derivations must agree: the
+                           reshape/permute/perm-table recipe
+                           (marlin_utils_test.py:31-121) and the per-thread
+                           index arithmetic of the CUDA repack kernels
+                           (gptq_marlin_repack.cu:129-209,
+                           awq_marlin_repack.cu:89-157); bijection on nibbles
+* scale/zp/bias permutes   closed-form index tables, permutation property,
+                           inverse round trip
+* dequantised values       exhaustive over all 16 codes x all finite fp16 /
+                           bf16 scales of a sample, against exact rational
+                           arithmetic (fractions) rounded to nearest even
+* GEMM reference           textbook: dequantise then fp32 matmul; special
+                           cases that reduce to row sums / column picks
+* moe_align_block_size     the literal example in
+                           fused_moe/moe_align_block_size.py:60-73 and set
+                           equality per expert
+                           (tests/kernels/moe/test_moe_align_block_size.py)
+* gfx950 layout            this build's own format: inverse round trip and
+                           decode-to-(K,N) equality with the Marlin decode
+"""
+
+from __future__ import annotations
+
+import numpy as np
+
+# --------------------------------------------------------------------------
+# ScalarType ids  (aphrodite/scalar_type.py:129-156, csrc/core/scalar_type.hpp:131-164)
+# --------------------------------------------------------------------------
+
+NAN_REPR_IEEE_754 = 1  # scalar_type.py:65 default, also used for integer types
+
+
+def scalar_type_id(exponent: int, mantissa: int, signed: bool, bias: int,
+                   finite_values_only: bool = False,
+                   nan_repr: int = NAN_REPR_IEEE_754) -> int:
+    """Bitfield exponent[0:8] mantissa[8:16] signed[16] bias[17:49]
+    finite_only[49] nan_repr[50:58] (scalar_type.py:137-150)."""
+    val = 0
+    off = 0
+    for member, width in ((exponent, 8), (mantissa, 8), (int(signed), 1),
+                          (bias, 32), (int(finite_values_only), 1),
+                          (nan_repr, 8)):
+        val |= (int(member) & ((1 << width) - 1)) << off
+        off += width
+    return val
+
+
+UINT4B8_ID = scalar_type_id(0, 4, False, 8)      # scalar_types.uint4b8
+UINT4_ID = scalar_type_id(0, 4, False, 0)        # scalar_types.uint4
+UINT8B128_ID = scalar_type_id(0, 8, False, 128)  # scalar_types.uint8b128 (rejected by this build)
+
+
+def scalar_type_min_max(mantissa: int, signed: bool, bias: int):
+    """Integer ScalarType.min()/max() (scalar_type.py:104-127,183-196):
+    raw range minus bias."""
+    size_bits = mantissa + int(signed)
+    raw_max = (1 << mantissa) - 1
+    raw_min = -(1 << (size_bits - 1)) if signed else 0
+    return raw_min - bias, raw_max - bias
+
+
+# --------------------------------------------------------------------------
+# Checkpoint packings  (quant_utils.py:725-834)
+# --------------------------------------------------------------------------
+
+AWQ_ORDER = np.array([0, 2, 4, 6, 1, 3, 5, 7])  # quant_utils.py:823
+
+
+def pack_rows(q: np.ndarray) -> np.ndarray:
+    """GPTQ packing along K (quant_utils.py:725-746): word[k//8][n] holds
+    q[k][n] at bits 4*(k%8)."""
+    k, n = q.shape
+    assert k % 8 == 0
+    u = q.astype(np.uint32).reshape(k // 8, 8, n)
+    out = np.zeros((k // 8, n), dtype=np.uint32)
+    for i in range(8):
+        out |= u[:, i, :] << np.uint32(4 * i)
+    return out.view(np.int32)
+
+
+def unpack_rows(packed: np.ndarray) -> np.ndarray:
+    u = packed.view(np.uint32)
+    kp, n = u.shape
+    out = np.empty((kp, 8, n), dtype=np.int32)
+    for i in range(8):
+        out[:, i, :] = (u >> np.uint32(4 * i)) & np.uint32(0xF)
+    return out.reshape(kp * 8, n)
+
+
+def pack_cols(q: np.ndarray) -> np.ndarray:
+    """Packing along N (quant_utils.py:749-772): word[k][n//8] holds q[k][n]
+    at bits 4*(n%8)."""
+    k, n = q.shape
+    assert n % 8 == 0
+    u = q.astype(np.uint32).reshape(k, n // 8, 8)
+    out = np.zeros((k, n // 8), dtype=np.uint32)
+    for i in range(8):
+        out |= u[:, :, i] << np.uint32(4 * i)
+    return out.view(np.int32)
+
+
+def unpack_cols(packed: np.ndarray) -> np.ndarray:
+    """quant_utils.py:775-803."""
+    u = packed.view(np.uint32)
+    k, npk = u.shape
+    out = np.empty((k, npk, 8), dtype=np.int32)
+    for i in range(8):
+        out[:, :, i] = (u >> np.uint32(4 * i)) & np.uint32(0xF)
+    return out.reshape(k, npk * 8)
+
+
+gptq_pack = pack_rows  # quant_utils.py:806-812
+
+
+def awq_pack(q: np.ndarray) -> np.ndarray:
+    """AWQ packing (quant_utils.py:815-834): within every 8 columns, nibble
+    position p holds column AWQ_ORDER[p]."""
+    k, n = q.shape
+    r = q.reshape(k, n // 8, 8)[:, :, AWQ_ORDER].reshape(k, n)
+    return pack_cols(r)
+
+
+def awq_unpack(packed: np.ndarray) -> np.ndarray:
+    r = unpack_cols(packed)
+    k, n = r.shape
+    out = np.empty_like(r).reshape(k, n // 8, 8)
+    out[:, :, AWQ_ORDER] = r.reshape(k, n // 8, 8)
+    return out.reshape(k, n)
+
+
+# --------------------------------------------------------------------------
+# Marlin weight layout  (marlin_utils_test.py:31-121)
+# --------------------------------------------------------------------------
+
+def marlin_weight_perm_recipe() -> np.ndarray:
+    """The 1024-entry gather table of a 16(k) x 64(n) tile for 4-bit weights
+    and 16-bit activations, built the way get_weight_perm builds it
+    (marlin_utils_test.py:89-121)."""
+    table = []
+    for lane in range(32):
+        col = lane // 4
+        one = []
+        for block in (0, 1):
+            for row in (2 * (lane % 4), 2 * (lane % 4) + 1,
+                        2 * (lane % 4 + 4), 2 * (lane % 4 + 4) + 1):
+                one.append(16 * row + col + 8 * block)
+        for j in range(4):
+            table.extend(p + 256 * j for p in one)
+    perm = np.array(table)
+    return perm.reshape(-1, 8)[:, AWQ_ORDER].ravel()
+
+
+def marlin_pack_recipe(q: np.ndarray) -> np.ndarray:
+    """(K,N) codes -> Marlin (K/16, 2N) int32 following marlin_permute_weights
+    + marlin_weights (marlin_utils_test.py:31-66)."""
+    k, n = q.shape
+    assert k % 16 == 0 and n % 64 == 0
+    perm = marlin_weight_perm_recipe()
+    t = q.reshape(k // 16, 16, n // 16, 16).transpose(0, 2, 1, 3).reshape(k // 16, n * 16)
+    t = t.reshape(-1, perm.size)[:, perm].reshape(t.shape)
+    u = t.astype(np.uint32).reshape(k // 16, n * 2, 8)
+    out = np.zeros((k // 16, n * 2), dtype=np.uint32)
+    for i in range(8):
+        out |= u[:, :, i] << np.uint32(4 * i)
+    return out.view(np.int32)
+
+
+def marlin_pack_closed_form(q: np.ndarray) -> np.ndarray:
+    """Same layout derived from the repack kernels' per-thread arithmetic
+    (gptq_marlin_repack.cu:129-209): tile (kt, nt) is 128 words at
+    (kt*n_tiles+nt)*128; word lane*4+j, lane in [0,32), j = 16-column
+    sub-tile; with c = lane//4, r0 = 2*(lane%4) the eight values
+    vals[i] (i<4: column c, i>=4: column c+8; rows r0+{0,1,8,9}) are stored
+    at nibble slots pack_idx = {0,2,4,6,1,3,5,7}."""
+    k, n = q.shape
+    assert k % 16 == 0 and n % 64 == 0
+    kt_n, nt_n = k // 16, n // 64
+    tile = q.reshape(kt_n, 16, nt_n, 4, 16).astype(np.uint32)  # [kt][r][nt][j][col]
+    out = np.zeros((kt_n, nt_n, 32, 4), dtype=np.uint32)       # [kt][nt][lane][j]
+    tc_offsets = (0, 1, 8, 9)
+    pack_idx = (0, 2, 4, 6, 1, 3, 5, 7)
+    for lane in range(32):
+        c = lane // 4
+        r0 = 2 * (lane % 4)
+        vals = []
+        for i in range(4):
+            vals.append(tile[:, r0 + tc_offsets[i], :, :, c])
+        for i in range(4):
+            vals.append(tile[:, r0 + tc_offsets[i], :, :, c + 8])
+        word = np.zeros_like(vals[0])
+        for slot in range(8):
+            word |= vals[pack_idx[slot]] << np.uint32(4 * slot)
+        out[:, :, lane, :] = word
+    return out.reshape(kt_n, nt_n * 128).view(np.int32)
+
+
+marlin_pack = marlin_pack_closed_form
+
+
+def marlin_unpack(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    """Inverse of marlin_pack: Marlin (K/16, 2N) int32 -> (K,N) codes."""
+    kt_n, nt_n = size_k // 16, size_n // 64
+    u = packed.view(np.uint32).reshape(kt_n, nt_n, 32, 4)
+    q = np.empty((kt_n, 16, nt_n, 4, 16), dtype=np.int32)
+    tc_offsets = (0, 1, 8, 9)
+    pack_idx = (0, 2, 4, 6, 1, 3, 5, 7)
+    for lane in range(32):
+        c = lane // 4
+        r0 = 2 * (lane % 4)
+        w = u[:, :, lane, :]
+        for slot in range(8):
+            i = pack_idx[slot]
+            row = r0 + tc_offsets[i % 4]
+            col = c + 8 * (i // 4)
+            q[:, row, :, :, col] = (w >> np.uint32(4 * slot)) & np.uint32(0xF)
+    return q.reshape(size_k, size_n)
+
+
+def gptq_marlin_repack(b_q_weight: np.ndarray, perm: np.ndarray | None,
+                       size_k: int, size_n: int) -> np.ndarray:
+    """gptq_marlin_repack.cu:285-362: output row k takes source row perm[k]
+    when perm is non-empty (:87-96,148-161)."""
+    q = unpack_rows(b_q_weight)
+    assert q.shape == (size_k, size_n)
+    if perm is not None and perm.size > 0:
+        q = q[perm.astype(np.int64), :]
+    return marlin_pack(q)
+
+
+def awq_marlin_repack(b_q_weight: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    """awq_marlin_repack.cu:228-290."""
+    q = awq_unpack(b_q_weight)
+    assert q.shape == (size_k, size_n)
+    return marlin_pack(q)
+
+
+# --------------------------------------------------------------------------
+# Scale / zero-point / bias layouts  (marlin_utils.py:401-505)
+# --------------------------------------------------------------------------
+
+SCALE_PERM = np.array([i + 8 * j for i in range(8) for j in range(8)])           # :406-409
+SCALE_PERM_SINGLE = np.array([2 * i + j for i in range(4)
+                              for j in (0, 1, 8, 9, 16, 17, 24, 25)])          # :410-412
+
+
+def marlin_permute_scales(s: np.ndarray, size_k: int, size_n: int, group_size: int) -> np.ndarray:
+    """marlin_utils.py:415-426 (16-bit activations)."""
+    if group_size < size_k and group_size != -1:
+        out = s.reshape(-1, 64)[:, SCALE_PERM]
+    else:
+        out = s.reshape(-1, 32)[:, SCALE_PERM_SINGLE]
+    return np.ascontiguousarray(out.reshape(-1, size_n))
+
+
+def marlin_unpermute_scales(s: np.ndarray, size_k: int, size_n: int, group_size: int) -> np.ndarray:
+    if group_size < size_k and group_size != -1:
+        out = np.empty_like(s).reshape(-1, 64)
+        out[:, SCALE_PERM] = s.reshape(-1, 64)
+    else:
+        out = np.empty_like(s).reshape(-1, 32)
+        out[:, SCALE_PERM_SINGLE] = s.reshape(-1, 32)
+    return np.ascontiguousarray(out.reshape(-1, size_n))
+
+
+def marlin_permute_bias(b: np.ndarray) -> np.ndarray:
+    """marlin_utils.py:429-433."""
+    return np.ascontiguousarray(b.reshape(-1, 32)[:, SCALE_PERM_SINGLE].reshape(b.shape))
+
+
+def marlin_unpermute_bias(b: np.ndarray) -> np.ndarray:
+    out = np.empty_like(b).reshape(-1, 32)
+    out[:, SCALE_PERM_SINGLE] = b.reshape(-1, 32)
+    return np.ascontiguousarray(out.reshape(b.shape))
+
+
+def marlin_zero_points(zp: np.ndarray, num_groups: int, size_n: int) -> np.ndarray:
+    """marlin_utils.py:456-477: (groups, N) codes -> (groups, N/8) int32."""
+    t = zp.reshape(-1, 64)[:, SCALE_PERM]
+    t = t.reshape(-1, 8)[:, AWQ_ORDER].reshape(num_groups, size_n)
+    return pack_cols(t)
+
+
+def marlin_unpack_zero_points(zp_packed: np.ndarray, num_groups: int, size_n: int) -> np.ndarray:
+    t = unpack_cols(zp_packed).reshape(-1, 8)
+    u = np.empty_like(t)
+    u[:, AWQ_ORDER] = t
+    u = u.reshape(-1, 64)
+    out = np.empty_like(u)
+    out[:, SCALE_PERM] = u
+    return out.reshape(num_groups, size_n)
+
+
+def awq_to_marlin_zero_points(q_zp_packed: np.ndarray, num_groups: int, size_n: int) -> np.ndarray:
+    """marlin_utils.py:480-505: AWQ-packed zero points -> Marlin layout."""
+    return marlin_zero_points(awq_unpack(q_zp_packed), num_groups, size_n)
+
+
+def stable_sort_g_idx(g_idx: np.ndarray):
+    """marlin_sort_g_idx (marlin_utils.py:401-403) with a stable sort, so the
+    tie order is fixed; the same perm must reach repack and GEMM."""
+    order = np.argsort(g_idx, kind="stable").astype(np.int32)
+    return g_idx[order], order
+
+
+# --------------------------------------------------------------------------
+# gfx950 streaming layout (this build's own format; no reference counterpart)
+# --------------------------------------------------------------------------
+# The (K,N) code matrix is cut into 64-column strips; a strip is a contiguous
+# run of K/32 one-KiB chunks, chunk c covering rows [32c, 32c+32).  Inside a
+# chunk, wavefront lane L (0..63) owns 16 bytes = words j=0..3.  Word j of lane
+# L holds column 64*strip + 16*j + (L % 16) and the eight rows
+# 32c + 8*(L // 16) + t, t = 0..7, with row t at nibble slot GFX950_SLOT[t], so
+# that (w >> 4*i) & 0x000f000f yields the row pair (2i, 2i+1) in the low / high
+# 16-bit halves: exactly one v_mfma_f32_16x16x32 operand register each.
+
+GFX950_SLOT = np.array([0, 4, 1, 5, 2, 6, 3, 7])  # slot of row t; inverse of AWQ_ORDER
+
+
+def gfx950_pack(q: np.ndarray) -> np.ndarray:
+    k, n = q.shape
+    assert k % 32 == 0 and n % 64 == 0
+    # [strip][chunk][kb][t][j][l]
+    t = q.astype(np.uint32).reshape(k // 32, 4, 8, n // 64, 4, 16)
+    t = t.transpose(3, 0, 1, 5, 4, 2)  # [strip][chunk][kb][l][j][t]
+    out = np.zeros(t.shape[:-1], dtype=np.uint32)
+    for row in range(8):
+        out |= t[..., row] << np.uint32(4 * GFX950_SLOT[row])
+    return out.reshape(-1).view(np.int32)
+
+
+def gfx950_unpack(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    u = packed.view(np.uint32).reshape(size_n // 64, size_k // 32, 4, 16, 4)
+    t = np.empty(u.shape + (8,), dtype=np.int32)
+    for row in range(8):
+        t[..., row] = (u >> np.uint32(4 * GFX950_SLOT[row])) & np.uint32(0xF)
+    # [strip][chunk][kb][l][j][t] -> [chunk][kb][t][strip][j][l]
+    return t.transpose(1, 2, 5, 0, 4, 3).reshape(size_k, size_n)
+
+
+def marlin_to_gfx950(marlin_packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    return gfx950_pack(marlin_unpack(marlin_packed, size_k, size_n))
+
+
+# --------------------------------------------------------------------------
+# 16-bit float helpers
+# --------------------------------------------------------------------------
+
+def f32_to_bf16_bits(x: np.ndarray) -> np.ndarray:
+    """Round-to-nearest-even fp32 -> bf16 (uint16 bit patterns)."""
+    u = np.asarray(x, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    rounded = (u + np.uint64(0x7FFF) + ((u >> np.uint64(16)) & np.uint64(1))) >> np.uint64(16)
+    out = rounded.astype(np.uint16)
+    nan = np.isnan(np.asarray(x, dtype=np.float32))
+    if np.any(nan):
+        out = np.where(nan, np.uint16(0x7FC0), out)
+    return out
+
+
+def bf16_bits_to_f32(b: np.ndarray) -> np.ndarray:
+    return (np.asarray(b, dtype=np.uint16).astype(np.uint32) << np.uint32(16)).view(np.float32)
+
+
+def round_to_dtype(x32: np.ndarray, dtype: str) -> np.ndarray:
+    """fp32 -> fp16/bf16 (RNE) -> fp32."""
+    if dtype == "fp16":
+        return np.asarray(x32, dtype=np.float32).astype(np.float16).astype(np.float32)
+    if dtype == "bf16":
+        return bf16_bits_to_f32(f32_to_bf16_bits(x32))
+    raise ValueError(dtype)
+
+
+def to_bits16(x32: np.ndarray, dtype: str) -> np.ndarray:
+    """fp32 values (already representable) -> uint16 storage bits."""
+    if dtype == "fp16":
+        return np.asarray(x32, dtype=np.float32).astype(np.float16).view(np.uint16)
+    return f32_to_bf16_bits(x32)
+
+
+def from_bits16(b: np.ndarray, dtype: str) -> np.ndarray:
+    if dtype == "fp16":
+        return np.asarray(b, dtype=np.uint16).view(np.float16).astype(np.float32)
+    return bf16_bits_to_f32(b)
+
+
+# --------------------------------------------------------------------------
+# Dequantisation  (dequant.h:107-216, marlin_template.h:107-142,1182-1299;
+#                  python twin quant_utils.py:646-648)
+# --------------------------------------------------------------------------
+
+def dequantize(q: np.ndarray, scales32: np.ndarray, group_size: int, dtype: str,
+               zeros: np.ndarray | None = None, g_idx: np.ndarray | None = None) -> np.ndarray:
+    """w[k][n] = round_to_dtype((q[k][n] - z) * s[g(k)][n]) with z = 8
+    (uint4b8) or the group's zero point (uint4); s is a value of `dtype`
+    held as fp32; one rounding, to nearest even.  (q - z) is a small integer,
+    s has at most 11 significant bits, so the fp32 product is exact and the
+    single rounding happens in round_to_dtype.  g(k) = k // group_size, or
+    g_idx[k] when given (act-order)."""
+    k, n = q.shape
+    if g_idx is not None:
+        rows = np.asarray(g_idx, dtype=np.int64)
+    elif group_size in (-1, k):
+        rows = np.zeros(k, dtype=np.int64)
+    else:
+        rows = np.arange(k) // group_size
+    s = scales32.astype(np.float32)[rows, :]
+    if zeros is None:
+        centred = q.astype(np.int32) - 8
+    else:
+        centred = q.astype(np.int32) - zeros.astype(np.int32)[rows, :]
+    return round_to_dtype(centred.astype(np.float32) * s, dtype)
+
+
+def gemm_reference(a32: np.ndarray, w32: np.ndarray, bias32: np.ndarray | None = None) -> np.ndarray:
+    """Dequantise-then-fp32-matmul reference (tests/kernels/quantization/
+    test_marlin_gemm.py:483-491 uses torch.matmul(a, w_ref))."""
+    out = a32.astype(np.float32) @ w32.astype(np.float32)
+    if bias32 is not None:
+        out = out + bias32.astype(np.float32)[None, :]
+    return out
+
+
+def gemm_tolerance_ok(out32: np.ndarray, ref32: np.ndarray):
+    """The acceptance rule of this build: max|err| <= 1e-2*max|ref| and
+    |err| <= 1e-2*max|ref| + 1e-2*|ref| elementwise.  Returns (ok, max_err,
+    max_ref)."""
+    err = np.abs(out32.astype(np.float64) - ref32.astype(np.float64))
+    max_ref = float(np.max(np.abs(ref32))) if ref32.size else 0.0
+    max_err = float(np.max(err)) if err.size else 0.0
+    ok = max_err <= 1e-2 * max_ref + 1e-30
+    ok = ok and bool(np.all(err <= 1e-2 * max_ref + 1e-2 * np.abs(ref32) + 1e-30))
+    return ok, max_err, max_ref
+
+
+# --------------------------------------------------------------------------
+# Seeded synthetic layers (shapes and distributions of the benchmark configs)
+# --------------------------------------------------------------------------
+
+def make_layer(seed: int, size_k: int, size_n: int, group_size: int, dtype: str,
+               zero_points: bool = False, act_order: bool = False):
+    """Codes uniform over 0..15, scales uniform in [1e-3, 1e-2] rounded to
+    `dtype`, optional zero points uniform 0..15, optional act-order: a random
+    row permutation mapped to groups (quant_utils.py:558-585)."""
+    rng = np.random.default_rng(seed)
+    q = rng.integers(0, 16, size=(size_k, size_n), dtype=np.int32)
+    groups = 1 if group_size in (-1, size_k) else size_k // group_size
+    s = round_to_dtype(rng.uniform(1e-3, 1e-2, size=(groups, size_n)).astype(np.float32), dtype)
+    out = {"q": q, "scales": s, "group_size": group_size, "groups": groups}
+    if zero_points:
+        out["zeros"] = rng.integers(0, 16, size=(groups, size_n), dtype=np.int32)
+    if act_order:
+        rand_perm = rng.permutation(size_k)
+        g_idx = (rand_perm // group_size).astype(np.int32)  # group of each checkpoint row
+        out["g_idx"] = g_idx
+    return out
+
+
+def make_activations(seed: int, size_m: int, size_k: int, dtype: str, std: float = 1.0) -> np.ndarray:
+    rng = np.random.default_rng(seed)
+    return round_to_dtype((rng.standard_normal((size_m, size_k)) * std).astype(np.float32), dtype)
+
+
+# --------------------------------------------------------------------------
+# MoE routing  (fused_moe/moe_align_block_size.py:11-101; golden in
+# tests/kernels/moe/test_moe_align_block_size.py:85-159)
+# --------------------------------------------------------------------------
+
+def moe_align_block_size(topk_ids: np.ndarray, block_size: int, num_experts: int):
+    numel = topk_ids.size
+    max_padded = numel + num_experts * (block_size - 1)
+    if numel < num_experts:
+        max_padded = min(numel * block_size, max_padded)
+    flat = topk_ids.reshape(-1).astype(np.int64)
+    sorted_ids = np.full(max_padded, numel, dtype=np.int32)
+    expert_ids = np.full((max_padded + block_size - 1) // block_size, -1, dtype=np.int32)
+    pos = 0
+    blk = 0
+    for e in range(num_experts):
+        toks = np.nonzero(flat == e)[0].astype(np.int32)  # ascending = stable
+        if toks.size == 0:
+            continue
+        nblk = (toks.size + block_size - 1) // block_size
+        sorted_ids[pos:pos + toks.size] = toks
+        expert_ids[blk:blk + nblk] = e
+        pos += nblk * block_size
+        blk += nblk
+    return sorted_ids, expert_ids, np.array([pos], dtype=np.int32)
+
+
+def moe_block_size_rule(m: int, topk: int, num_experts: int) -> int:
+    """fused_marlin_moe block size choice (experts/marlin_moe.py:322-329)."""
+    for bs in (8, 16, 32, 48, 64):
+        if m * topk / num_experts / bs < 0.9:
+            return bs
+    return 64
+
+
+def moe_gemm_reference(a32: np.ndarray, w32_per_expert, sorted_ids: np.ndarray,
+                       expert_ids: np.ndarray, num_post_pad: int, block_size: int,
+                       top_k: int, size_m: int, topk_weights: np.ndarray | None,
+                       dtype: str) -> np.ndarray:
+    """moe_wna16_marlin_gemm semantics (moe/marlin_moe_wna16/ops.cu:544-897,
+    marlin_template.h(moe):471-570,1883-1909): for every valid slot id of
+    block b, C[id] = A[id // top_k] @ W[expert_ids[b]], rounded to dtype, then
+    optionally multiplied by dtype(topk_weights[id]) in dtype arithmetic."""
+    n = w32_per_expert[0].shape[1]
+    out = np.zeros((size_m * top_k, n), dtype=np.float32)
+    for b in range(num_post_pad // block_size):
+        e = int(expert_ids[b])
+        if e < 0:
+            continue
+        ids = sorted_ids[b * block_size:(b + 1) * block_size]
+        ids = ids[ids < size_m * top_k]
+        if ids.size == 0:
+            continue
+        rows = a32[ids // top_k, :]
+        c = round_to_dtype(rows @ w32_per_expert[e], dtype)
+        if topk_weights is not None:
+            wts = round_to_dtype(topk_weights.reshape(-1)[ids].astype(np.float32), dtype)
+            c = round_to_dtype(c * wts[:, None], dtype)
+        out[ids, :] = c
+    return out
+
+
+# --------------------------------------------------------------------------
+# CPU baseline of the layer: int4 dequantise + torch.matmul in fp32
+# --------------------------------------------------------------------------
+
+def cpu_layer_baseline(q_packed_rows: np.ndarray, scales32: np.ndarray, a32: np.ndarray,
+                       group_size: int, threads: int, repeats: int = 5, warmup: int = 2):
+    """Times W = (unpack(q) - 8) * s (fp32) followed by torch.matmul(A, W) in
+    fp32 on `threads` host threads.  Returns (seconds_dequant_plus_matmul,
+    seconds_matmul_only, output)."""
+    import time
+
+    import torch
+
+    torch.set_num_threads(threads)
+    qp = torch.from_numpy(q_packed_rows.view(np.int32).copy())
+    s = torch.from_numpy(scales32.astype(np.float32))
+    a = torch.from_numpy(a32.astype(np.float32))
+    shifts = torch.arange(0, 32, 4, dtype=torch.int32).view(1, 8, 1)
+
+    def dequant():
+        nib = (qp.unsqueeze(1) >> shifts) & 0xF            # (K/8, 8, N)
+        w = (nib.reshape(-1, qp.shape[1]).float() - 8.0)
+        return w * s.repeat_interleave(group_size, dim=0)
+
+    w = dequant()
+    for _ in range(warmup):
+        out = a @ dequant()
+    t_full = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        out = a @ dequant()
+        t_full.append(time.perf_counter() - t0)
+    t_mm = []
+    for _ in range(repeats):
+        t0 = time.perf_counter()
+        out2 = a @ w
+        t_mm.append(time.perf_counter() - t0)
+    del out2
+    return float(np.median(t_full)), float(np.median(t_mm)), out.numpy()

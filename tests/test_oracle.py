@@ -1,0 +1,313 @@
+"""Pins the CPU oracle against closed forms, invariants and the literal
+vectors the reference's own tests and docstrings hold."""
+from fractions import Fraction
+
+import numpy as np
+import pytest
+
+from oracle import marlin_oracle as mo
+
+
+# ---------------------------------------------------------------- ScalarType
+def test_scalar_type_ids_closed_form():
+    # exponent[0:8] mantissa[8:16] signed[16] bias[17:49] finite[49] nan_repr[50:58]
+    assert mo.UINT4B8_ID == (4 << 8) | (8 << 17) | (1 << 50) == 1125899907892224
+    assert mo.UINT4_ID == (4 << 8) | (1 << 50) == 1125899906843648
+    assert mo.UINT8B128_ID == (8 << 8) | (128 << 17) | (1 << 50) == 1125899923621888
+
+
+@pytest.mark.parametrize("mant,signed,bias,lo,hi", [
+    # rows of tests/test_scalartype.py:10-25 that are integer types
+    (4, False, 0, 0, 15),      # uint4
+    (4, False, 8, -8, 7),      # uint4b8
+    (8, False, 128, -128, 127),  # uint8b128
+    (3, True, 0, -8, 7),       # int4
+    (7, True, 0, -128, 127),   # int8
+])
+def test_scalar_type_min_max(mant, signed, bias, lo, hi):
+    assert mo.scalar_type_min_max(mant, signed, bias) == (lo, hi)
+
+
+# ---------------------------------------------------------------- packings
+def _brute_pack_rows(q):
+    k, n = q.shape
+    out = [[0] * n for _ in range(k // 8)]
+    for kk in range(k):
+        for nn in range(n):
+            out[kk // 8][nn] |= int(q[kk, nn]) << (4 * (kk % 8))
+    return np.array(out, dtype=np.uint32).view(np.int32)
+
+
+def _brute_awq_pack(q):
+    k, n = q.shape
+    order = [0, 2, 4, 6, 1, 3, 5, 7]
+    out = [[0] * (n // 8) for _ in range(k)]
+    for kk in range(k):
+        for w in range(n // 8):
+            for p in range(8):
+                out[kk][w] |= int(q[kk, 8 * w + order[p]]) << (4 * p)
+    return np.array(out, dtype=np.uint32).view(np.int32)
+
+
+def test_packings_brute_force_and_inverse():
+    rng = np.random.default_rng(0)
+    q = rng.integers(0, 16, size=(32, 64), dtype=np.int32)
+    assert np.array_equal(mo.pack_rows(q), _brute_pack_rows(q))
+    assert np.array_equal(mo.awq_pack(q), _brute_awq_pack(q))
+    assert np.array_equal(mo.unpack_rows(mo.pack_rows(q)), q)
+    assert np.array_equal(mo.unpack_cols(mo.pack_cols(q)), q)
+    assert np.array_equal(mo.awq_unpack(mo.awq_pack(q)), q)
+    # top nibble set: sign bit of the int32 word must survive
+    q[:] = 15
+    assert np.array_equal(mo.unpack_rows(mo.pack_rows(q)), q)
+    assert mo.pack_rows(q).dtype == np.int32 and mo.pack_rows(q)[0, 0] == -1
+
+
+# ---------------------------------------------------------------- Marlin layout
+def test_weight_perm_is_bijection():
+    perm = mo.marlin_weight_perm_recipe()
+    assert perm.shape == (1024,)
+    assert np.array_equal(np.sort(perm), np.arange(1024))
+
+
+@pytest.mark.parametrize("k,n", [(16, 64), (32, 128), (128, 256), (1024, 448)])
+def test_marlin_layout_two_derivations_agree(k, n):
+    rng = np.random.default_rng(k * 131 + n)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    a = mo.marlin_pack_recipe(q)
+    b = mo.marlin_pack_closed_form(q)
+    assert a.shape == (k // 16, 2 * n) and a.dtype == np.int32
+    assert np.array_equal(a, b)
+    assert np.array_equal(mo.marlin_unpack(a, k, n), q)
+
+
+def test_marlin_layout_single_nibble_positions():
+    """One-hot inputs: the nibble of W[r][c] lands exactly where the closed
+    form of the layout says (word lane*4+j, lane = 4*(c%8) + (r%8)//2, slot from
+    {r%2, r//8, (c%16)//8})."""
+    k, n = 16, 64
+    for r in range(16):
+        for c in range(64):
+            q = np.zeros((k, n), dtype=np.int32)
+            q[r, c] = 0xF
+            w = mo.marlin_pack_recipe(q).view(np.uint32).ravel()
+            (idx,) = np.nonzero(w)
+            assert idx.size == 1
+            j, cc = divmod(c, 16)
+            lane = 4 * (cc % 8) + (r % 8) // 2
+            slot = (r // 8) + 2 * (cc // 8) + 4 * (r % 2)
+            assert idx[0] == lane * 4 + j
+            assert w[idx[0]] == 0xF << (4 * slot)
+
+
+def test_repack_identities():
+    rng = np.random.default_rng(5)
+    k, n = 256, 192
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    g = mo.gptq_marlin_repack(mo.gptq_pack(q), None, k, n)
+    a = mo.awq_marlin_repack(mo.awq_pack(q), k, n)
+    assert np.array_equal(g, a)
+    perm = rng.permutation(k).astype(np.int32)
+    with_perm = mo.gptq_marlin_repack(mo.gptq_pack(q), perm, k, n)
+    pre_perm = mo.gptq_marlin_repack(mo.gptq_pack(q[perm]), None, k, n)
+    assert np.array_equal(with_perm, pre_perm)
+    assert np.array_equal(mo.gptq_marlin_repack(mo.gptq_pack(q), np.empty(0, np.int32), k, n), g)
+
+
+# ---------------------------------------------------------------- scale / zp / bias
+def test_scale_perm_tables():
+    assert list(mo.SCALE_PERM[:10]) == [0, 8, 16, 24, 32, 40, 48, 56, 1, 9]
+    assert list(mo.SCALE_PERM_SINGLE[:10]) == [0, 1, 8, 9, 16, 17, 24, 25, 2, 3]
+    assert np.array_equal(np.sort(mo.SCALE_PERM), np.arange(64))
+    assert np.array_equal(np.sort(mo.SCALE_PERM_SINGLE), np.arange(32))
+
+
+def test_scale_zp_bias_round_trip():
+    rng = np.random.default_rng(7)
+    k, n, g = 512, 256, 128
+    s = rng.uniform(1e-3, 1e-2, size=(k // g, n)).astype(np.float32)
+    sp = mo.marlin_permute_scales(s, k, n, g)
+    # 8x8 transpose inside every 64 columns
+    assert sp[1, 8 * 3 + 5] == s[1, 3 + 8 * 5]
+    assert np.array_equal(mo.marlin_unpermute_scales(sp, k, n, g), s)
+    s1 = s[:1]
+    sp1 = mo.marlin_permute_scales(s1, k, n, -1)
+    assert sp1[0, 1] == s1[0, 1] and sp1[0, 2] == s1[0, 8]
+    assert np.array_equal(mo.marlin_unpermute_scales(sp1, k, n, -1), s1)
+    b = rng.standard_normal(n).astype(np.float32)
+    assert np.array_equal(mo.marlin_unpermute_bias(mo.marlin_permute_bias(b)), b)
+    zp = rng.integers(0, 16, size=(k // g, n), dtype=np.int32)
+    zpp = mo.marlin_zero_points(zp, k // g, n)
+    assert zpp.shape == (k // g, n // 8) and zpp.dtype == np.int32
+    assert np.array_equal(mo.marlin_unpack_zero_points(zpp, k // g, n), zp)
+    assert np.array_equal(mo.awq_to_marlin_zero_points(mo.awq_pack(zp), k // g, n), zpp)
+
+
+def test_zero_point_slot_closed_form():
+    """Column nl of a 64-column block sits in word nl%8 of the block at slot
+    [0,4,1,5,2,6,3,7][nl//8] (derived from scale_perm then the 8-interleave)."""
+    inv = [0, 4, 1, 5, 2, 6, 3, 7]
+    for nl in range(64):
+        zp = np.zeros((1, 64), dtype=np.int32)
+        zp[0, nl] = 0xF
+        w = mo.marlin_zero_points(zp, 1, 64).view(np.uint32).ravel()
+        (idx,) = np.nonzero(w)
+        assert idx.size == 1 and idx[0] == nl % 8
+        assert w[idx[0]] == 0xF << (4 * inv[nl // 8])
+
+
+# ---------------------------------------------------------------- gfx950 layout
+@pytest.mark.parametrize("k,n", [(32, 64), (128, 128), (4096, 256)])
+def test_gfx950_layout_round_trip(k, n):
+    rng = np.random.default_rng(k + n)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    p = mo.gfx950_pack(q)
+    assert p.size == k * n // 8
+    assert np.array_equal(mo.gfx950_unpack(p, k, n), q)
+    assert np.array_equal(mo.marlin_to_gfx950(mo.marlin_pack(q), k, n), p)
+
+
+def test_gfx950_layout_word_positions():
+    k, n = 64, 128
+    for (r, c) in [(0, 0), (1, 0), (7, 15), (8, 16), (31, 63), (32, 64), (45, 101), (63, 127)]:
+        q = np.zeros((k, n), dtype=np.int32)
+        q[r, c] = 0xF
+        w = mo.gfx950_pack(q).view(np.uint32)
+        (idx,) = np.nonzero(w)
+        assert idx.size == 1
+        strip, cl = divmod(c, 64)
+        chunk, rl = divmod(r, 32)
+        j, l = divmod(cl, 16)
+        kb, t = divmod(rl, 8)
+        lane = 16 * kb + l
+        assert idx[0] == ((strip * (k // 32) + chunk) * 64 + lane) * 4 + j
+        slot = (t // 2) + 4 * (t % 2)
+        assert w[idx[0]] == 0xF << (4 * slot)
+
+
+# ---------------------------------------------------------------- dequant
+def _rne_fraction_to(dtype, value: Fraction) -> float:
+    """Exact rational -> nearest-even representable value of dtype, by
+    searching the two neighbours around the float64 approximation."""
+    if value == 0:
+        return 0.0
+    mant_bits = 10 if dtype == "fp16" else 7
+    min_exp = -14 if dtype == "fp16" else -126
+    sign = -1 if value < 0 else 1
+    v = abs(value)
+    import math
+    e = math.floor(math.log2(float(v)))
+    while Fraction(2) ** e > v:
+        e -= 1
+    while Fraction(2) ** (e + 1) <= v:
+        e += 1
+    e = max(e, min_exp)
+    ulp = Fraction(2) ** (e - mant_bits)
+    qf = v / ulp
+    lo = qf.numerator // qf.denominator
+    rem = qf - lo
+    if rem > Fraction(1, 2) or (rem == Fraction(1, 2) and lo % 2 == 1):
+        lo += 1
+    return sign * float(lo * ulp)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_dequant_exhaustive_against_exact_rationals(dtype):
+    rng = np.random.default_rng(11)
+    raw = np.concatenate([
+        rng.uniform(1e-3, 1e-2, 64), rng.uniform(1e-6, 1.0, 32),
+        np.array([0.0, 1.0, 2.0 ** -14, 2.0 ** -20, 3.0e-5, 0.333, 100.0])])
+    s = mo.round_to_dtype(raw.astype(np.float32), dtype)
+    q = np.tile(np.arange(16, dtype=np.int32)[:, None], (1, s.size))
+    w = mo.dequantize(q, s[None, :], -1, dtype)
+    zeros = np.full((1, s.size), 3, dtype=np.int32)
+    wz = mo.dequantize(q, s[None, :], -1, dtype, zeros=zeros)
+    for j, sv in enumerate(s):
+        for code in range(16):
+            want = _rne_fraction_to(dtype, Fraction(code - 8) * Fraction(float(sv)))
+            assert w[code, j] == np.float32(want), (dtype, code, sv)
+            want = _rne_fraction_to(dtype, Fraction(code - 3) * Fraction(float(sv)))
+            assert wz[code, j] == np.float32(want)
+    assert np.all(w[8] == 0)           # code 8 is zero for uint4b8
+    assert np.all(w[:, s == 0] == 0)   # zero scale (tile padding) gives zero
+
+
+def test_bf16_rounding_ties_to_even():
+    # 1 + 2^-8 is exactly between 1.0 and 1 + 2^-7 -> even mantissa (1.0)
+    x = np.array([1.0 + 2.0 ** -8, 1.0 + 3 * 2.0 ** -8, -(1.0 + 2.0 ** -8)], dtype=np.float32)
+    assert list(mo.round_to_dtype(x, "bf16")) == [1.0, 1.0 + 2.0 ** -6, -1.0]
+    assert mo.f32_to_bf16_bits(np.array([1.0], np.float32))[0] == 0x3F80
+
+
+def test_dequant_grouping_and_act_order():
+    layer = mo.make_layer(3, 256, 64, 128, "fp16", act_order=True)
+    w = mo.dequantize(layer["q"], layer["scales"], 128, "fp16", g_idx=layer["g_idx"])
+    k = 17
+    g = layer["g_idx"][k]
+    want = mo.round_to_dtype((layer["q"][k] - 8).astype(np.float32) * layer["scales"][g], "fp16")
+    assert np.array_equal(w[k], want)
+    # sorting rows by group and using contiguous groups is the same matrix, permuted
+    gs, order = mo.stable_sort_g_idx(layer["g_idx"])
+    w_sorted = mo.dequantize(layer["q"][order], layer["scales"], 128, "fp16")
+    assert np.array_equal(w_sorted, w[order])
+    assert np.array_equal(gs, np.arange(256) // 128)
+
+
+# ---------------------------------------------------------------- GEMM reference
+def test_gemm_reference_special_cases():
+    k, n, m = 128, 64, 3
+    a = mo.make_activations(1, m, k, "fp16")
+    # all codes 9, scale 1: W == 1 -> every output column is the row sum of A
+    q = np.full((k, n), 9, dtype=np.int32)
+    w = mo.dequantize(q, np.ones((1, n), np.float32), -1, "fp16")
+    out = mo.gemm_reference(a, w)
+    assert np.allclose(out, a.sum(axis=1, keepdims=True).repeat(n, 1), rtol=1e-6, atol=1e-5)
+    # a single non-zero row of W picks one column of A
+    q = np.full((k, n), 8, dtype=np.int32)
+    q[5, :] = 10
+    w = mo.dequantize(q, np.full((1, n), 0.5, np.float32), -1, "fp16")
+    out = mo.gemm_reference(a, w)
+    assert np.allclose(out, a[:, 5:6].repeat(n, 1), rtol=1e-6)
+    ok, _, _ = mo.gemm_tolerance_ok(out, out)
+    assert ok
+    ok, _, _ = mo.gemm_tolerance_ok(out * 1.05, out)
+    assert not ok
+
+
+# ---------------------------------------------------------------- MoE routing
+def test_moe_align_docstring_example():
+    # fused_moe/moe_align_block_size.py:60-73 (expert ids 1..4 -> 5 experts, 0 unused)
+    topk_ids = np.array([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]])
+    sorted_ids, expert_ids, post = mo.moe_align_block_size(topk_ids, 4, 5)
+    assert list(sorted_ids[:16]) == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    assert list(expert_ids[:4]) == [1, 2, 3, 4]
+    assert post[0] == 16
+
+
+@pytest.mark.parametrize("m,topk,e,bs", [(1, 2, 8, 8), (16, 2, 8, 8), (133, 3, 12, 16), (64, 2, 8, 64)])
+def test_moe_align_invariants(m, topk, e, bs):
+    rng = np.random.default_rng(m)
+    topk_ids = np.stack([rng.permutation(e)[:topk] for _ in range(m)])
+    sorted_ids, expert_ids, post = mo.moe_align_block_size(topk_ids, bs, e)
+    numel = m * topk
+    assert post[0] % bs == 0
+    valid = sorted_ids[:post[0]][sorted_ids[:post[0]] < numel]
+    assert np.array_equal(np.sort(valid), np.arange(numel))
+    assert np.all(sorted_ids[post[0]:] == numel)
+    for b in range(post[0] // bs):
+        ids = sorted_ids[b * bs:(b + 1) * bs]
+        ids = ids[ids < numel]
+        assert ids.size > 0
+        assert np.all(topk_ids.reshape(-1)[ids] == expert_ids[b])
+    blocks = expert_ids[:post[0] // bs]
+    assert np.all(np.diff(blocks) >= 0)
+    expect_len = numel + e * (bs - 1)
+    if numel < e:
+        expect_len = min(numel * bs, expect_len)
+    assert sorted_ids.size == expect_len
+
+
+def test_moe_block_size_rule():
+    assert mo.moe_block_size_rule(16, 2, 8) == 8
+    assert mo.moe_block_size_rule(4096, 2, 8) == 64
+    assert mo.moe_block_size_rule(64, 2, 8) == 32  # 16/8=2, 16/16=1, 16/32=.5
