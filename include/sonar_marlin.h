@@ -1,0 +1,153 @@
+/*
+ * sonar_marlin.h - C ABI of the MI355X (gfx950) W4A16 Marlin-family GEMM library.
+ *
+ * Every entry point takes plain device pointers, sizes and a HIP stream
+ * (passed as void*; NULL = the null stream).  All work is enqueued on that
+ * stream; nothing synchronises with the host.  Return value: 0 on success, a
+ * negative SONAR_E_* code on failure; sonar_marlin_last_error() then returns a
+ * message for the calling thread.  Nothing is launched when a call fails.
+ *
+ * The entry points replace these reference interfaces (paths relative to the
+ * reference checkout):
+ *   sonar_gptq_marlin_repack  -> _C::gptq_marlin_repack
+ *        csrc/libtorch_stable/torch_bindings.cpp:107-109,
+ *        csrc/libtorch_stable/quantization/marlin/gptq_marlin_repack.cu:285-362
+ *   sonar_awq_marlin_repack   -> _C::awq_marlin_repack
+ *        csrc/libtorch_stable/torch_bindings.cpp:113-115,
+ *        csrc/libtorch_stable/quantization/marlin/awq_marlin_repack.cu:228-290
+ *   sonar_marlin_gemm         -> _C::marlin_gemm
+ *        csrc/libtorch_stable/torch_bindings.cpp:96-103,
+ *        csrc/libtorch_stable/quantization/marlin/marlin.cu:546-897
+ *   sonar_moe_wna16_marlin_gemm -> _moe_C::moe_wna16_marlin_gemm
+ *        csrc/libtorch_stable/moe/torch_bindings.cpp:76-89,
+ *        csrc/libtorch_stable/moe/marlin_moe_wna16/ops.cu:544-897
+ * sonar_marlin_to_gfx950 / sonar_gfx950_to_marlin have no reference
+ * counterpart: they convert between the Marlin tile order that the repack ops
+ * return (and every reference caller stores) and the streaming order the
+ * gfx950 kernels read.
+ */
+#ifndef SONAR_MARLIN_H_
+#define SONAR_MARLIN_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define SONAR_OK 0
+#define SONAR_E_INVALID (-1)       /* bad argument (shape, alignment, null pointer) */
+#define SONAR_E_UNSUPPORTED (-2)   /* valid for the reference op, not built here */
+#define SONAR_E_RUNTIME (-3)       /* a HIP call failed */
+
+/* activation / output / scale element types */
+#define SONAR_DTYPE_F16 0
+#define SONAR_DTYPE_BF16 1
+
+/* weight orders accepted by the GEMM entry points */
+#define SONAR_LAYOUT_GFX950 0      /* output of sonar_marlin_to_gfx950 */
+
+/* ScalarType ids that cross the op boundary as b_type_id
+ * (aphrodite/scalar_type.py:129-156, csrc/core/scalar_type.hpp:131-164) */
+#define SONAR_TYPE_UINT4B8 1125899907892224LL /* GPTQ: code - 8 */
+#define SONAR_TYPE_UINT4 1125899906843648LL   /* AWQ: code - zero point */
+
+const char* sonar_marlin_last_error(void);
+const char* sonar_marlin_version(void);
+
+/* GPTQ (K/8, N) int32, nibble k%8 of word [k/8][n] = code of W[k][n]
+ * -> Marlin (K/16, 2N) int32.  perm (int32[K], may be NULL) selects source
+ * rows: output row k is source row perm[k].  num_bits must be 4. */
+int sonar_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_t* perm,
+                             uint32_t* out, int64_t size_k, int64_t size_n,
+                             int num_bits, void* stream);
+
+/* AWQ (K, N/8) int32, nibble p of word [k][n/8] = code of column
+ * 8*(n/8) + {0,2,4,6,1,3,5,7}[p] -> Marlin (K/16, 2N) int32. */
+int sonar_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out,
+                            int64_t size_k, int64_t size_n, int num_bits,
+                            void* stream);
+
+/* Marlin (K/16, 2N) int32 <-> gfx950 streaming order, same number of words.
+ * K % 32 == 0, N % 64 == 0.  in and out must not overlap. */
+int sonar_marlin_to_gfx950(const uint32_t* marlin, uint32_t* out,
+                           int64_t size_k, int64_t size_n, void* stream);
+int sonar_gfx950_to_marlin(const uint32_t* gfx950, uint32_t* out,
+                           int64_t size_k, int64_t size_n, void* stream);
+
+/* Dequantised weight matrix W[K][N] (row-major, dtype elements) exactly as the
+ * GEMM kernels form it in registers: round_to_dtype((code - z) * s).  Uses the
+ * same device routine as the GEMM; exists so the in-kernel values can be
+ * compared bit for bit.  Arguments as for sonar_marlin_gemm. */
+int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout,
+                         const void* b_scales, const uint32_t* b_zeros,
+                         const int32_t* g_idx, void* w_out, int dtype,
+                         int64_t b_type_id, int64_t size_n, int64_t size_k,
+                         int64_t num_groups, int is_k_full, void* stream);
+
+/* Bytes of scratch sonar_marlin_gemm needs for (size_m, size_n, size_k). */
+size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k);
+
+/* C[M,N] = A[M,K] * dequant(B)[K,N] (+ bias), fp32 accumulation, result
+ * rounded to dtype.
+ *   a            dtype[M][a_row_stride], 16-byte aligned, a_row_stride % 8 == 0
+ *   c            dtype[M][N] contiguous
+ *   b_q_weight   K*N/8 words in b_layout order
+ *   b_bias       dtype[N] in marlin_permute_bias order, or NULL
+ *   b_scales     dtype[num_groups][N] in marlin_permute_scales order
+ *   b_zeros      int32[num_groups][N/8] in marlin_zero_points order, or NULL
+ *                (required iff b_type_id == SONAR_TYPE_UINT4)
+ *   g_idx, perm  int32[K] each or both NULL; with both given the call is an
+ *                act-order call: perm maps weight row k to column perm[k] of
+ *                A; g_idx[k] is the group of weight row k (used only when
+ *                is_k_full == 0)
+ *   workspace    int32[workspace_len], all zero on entry, all zero on exit;
+ *                workspace_len >= number of compute units
+ *   scratch      sonar_marlin_gemm_scratch_bytes() bytes, contents don't care
+ * use_atomic_add and use_fp32_reduce are accepted for signature parity; the
+ * reduction is always fp32 and deterministic. */
+int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
+                      const uint32_t* b_q_weight, int b_layout,
+                      const void* b_bias, const void* b_scales,
+                      const uint32_t* b_zeros, const int32_t* g_idx,
+                      const int32_t* perm, int32_t* workspace,
+                      int64_t workspace_len, void* scratch,
+                      size_t scratch_bytes, int dtype, int64_t b_type_id,
+                      int64_t size_m, int64_t size_n, int64_t size_k,
+                      int64_t num_groups, int is_k_full, int use_atomic_add,
+                      int use_fp32_reduce, void* stream);
+
+/* Grouped (mixture-of-experts) variant.  For block b <
+ * num_tokens_past_padded[0] / moe_block_size with expert e = expert_ids[b]
+ * (e < 0: skipped), each slot id = sorted_token_ids[b*moe_block_size + i] with
+ * id < size_m*top_k gives C[id,:] = A[id / top_k,:] * dequant(B[e]) (+
+ * bias[e]), rounded to dtype, then multiplied in dtype by
+ * dtype(topk_weights[id]) when mul_topk_weights != 0.
+ *   a            dtype[M][K] contiguous
+ *   c            dtype[M*top_k][N] contiguous
+ *   b_q_weight   num_experts * K*N/8 words, each expert in b_layout order
+ *   b_scales     dtype[num_experts][num_groups][N]; b_zeros / b_bias likewise
+ *   g_idx, perm  int32[num_experts][K] or NULL
+ *   sorted_token_ids int32[sorted_len], expert_ids int32[ceil(sorted_len/bs)],
+ *   num_tokens_past_padded int32[1] (read on the device), topk_weights
+ *   float[M*top_k]
+ */
+size_t sonar_moe_marlin_gemm_scratch_bytes(int64_t sorted_len, int64_t moe_block_size,
+                                           int64_t size_n, int64_t size_k);
+int sonar_moe_wna16_marlin_gemm(
+    const void* a, void* c, const uint32_t* b_q_weight, int b_layout,
+    const void* b_bias, const void* b_scales, const uint32_t* b_zeros,
+    const int32_t* g_idx, const int32_t* perm, int32_t* workspace,
+    int64_t workspace_len, void* scratch, size_t scratch_bytes,
+    const int32_t* sorted_token_ids, int64_t sorted_len,
+    const int32_t* expert_ids, const int32_t* num_tokens_past_padded,
+    const float* topk_weights, int64_t moe_block_size, int64_t top_k,
+    int mul_topk_weights, int64_t num_experts, int dtype, int64_t b_type_id,
+    int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
+    int is_k_full, int use_atomic_add, int use_fp32_reduce, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SONAR_MARLIN_H_ */

@@ -1,0 +1,83 @@
+"""Builds the HIP library (and, on request, the torch op registration layer)
+in-tree.  Run as `python -m sonar_amd.build`."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+PKG = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(PKG)
+CSRC = os.path.join(PKG, "csrc")
+LIB_DIR = os.path.join(PKG, "lib")
+LIB_PATH = os.path.join(LIB_DIR, "libsonar_marlin.so")
+OPS_PATH = os.path.join(LIB_DIR, "libsonar_marlin_torch.so")
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+
+HIP_SOURCES = ["repack.hip", "gemm_stream.hip", "gemm_moe.hip"]
+HIP_FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _run(cmd):
+    proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    out = "\n".join(l for l in proc.stdout.splitlines()
+                    if "packed-fp32-ops" not in l and "unknown target feature" not in l)
+    if proc.returncode != 0:
+        raise RuntimeError("command failed: %s\n%s" % (" ".join(cmd), out))
+    return out
+
+
+def build_hip_library(verbose: bool = False) -> str:
+    os.makedirs(LIB_DIR, exist_ok=True)
+    objs = []
+    for src in HIP_SOURCES:
+        obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
+        cmd = [HIPCC, *HIP_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+               "-c", os.path.join(CSRC, src), "-o", obj]
+        out = _run(cmd)
+        if verbose and out.strip():
+            print(out)
+        objs.append(obj)
+    _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs])
+    return LIB_PATH
+
+
+def build_torch_ops(verbose: bool = False) -> str:
+    """Compiles the C++ torch op registration layer with the host compiler and
+    links it against the HIP library."""
+    import torch
+    from torch.utils import cpp_extension
+
+    src = os.path.join(CSRC, "torch_bindings.cpp")
+    inc = []
+    for d in cpp_extension.include_paths():
+        inc += ["-isystem", d]
+    torch_lib = os.path.join(os.path.dirname(torch.__file__), "lib")
+    abi = int(torch._C._GLIBCXX_USE_CXX11_ABI)
+    cmd = ["g++", "-O2", "-std=c++17", "-fPIC", "-shared", "-D_GLIBCXX_USE_CXX11_ABI=%d" % abi,
+           "-D__HIP_PLATFORM_AMD__=1", "-DUSE_ROCM=1",
+           "-I", os.path.join(ROOT, "include"), "-isystem", "/opt/rocm/include", *inc, src,
+           "-o", OPS_PATH, "-L", torch_lib, "-L", LIB_DIR,
+           "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib,
+           "-lsonar_marlin", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip"]
+    out = _run(cmd)
+    if verbose and out.strip():
+        print(out)
+    return OPS_PATH
+
+
+def build_all(verbose: bool = False):
+    paths = [build_hip_library(verbose)]
+    if os.path.exists(os.path.join(CSRC, "torch_bindings.cpp")):
+        paths.append(build_torch_ops(verbose))
+    return paths
+
+
+if __name__ == "__main__":
+    for p in build_all(verbose=True):
+        print("built", p)
+    sys.exit(0)

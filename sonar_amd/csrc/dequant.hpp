@@ -1,0 +1,161 @@
+// In-register dequantisation of one gfx950 weight word (eight 4-bit codes of
+// one column, rows t = 0..7 at nibble slots t/2 + 4*(t%2)) into the eight
+// 16-bit values of one v_mfma_f32_16x16x32 operand, plus the per-column
+// constants it needs.  The result is round_to_dtype((code - z) * s) with a
+// single round-to-nearest-even, the value the reference forms with
+// dequant<...> followed by scale()/sub_zp()
+// (csrc/libtorch_stable/quantization/marlin/dequant.h:107-216,
+// marlin_template.h:107-142,1182-1299).
+#pragma once
+
+#include "common.hpp"
+
+namespace sonar {
+
+// Where column `nl` (0..63) of a 64-column block sits after
+// marlin_permute_scales (aphrodite/.../utils/marlin_utils.py:406-426).
+// grouped: 8x8 transpose of the block; single: scale_perm_single inside each
+// 32 columns.
+__device__ __forceinline__ int scale_slot(int nl, bool grouped) {
+  if (grouped) return 8 * (nl & 7) + (nl >> 3);
+  const int n32 = nl & 31;
+  return (nl & 32) + 8 * ((n32 & 7) >> 1) + 2 * (n32 >> 3) + (n32 & 1);
+}
+
+// Zero point of column `nl` of a 64-column block from the eight words that
+// marlin_zero_points (marlin_utils.py:456-477) makes of the block: word nl%8,
+// nibble slot {0,4,1,5,2,6,3,7}[nl/8] = (nl/8)/2 + 4*((nl/8)%2).
+__device__ __forceinline__ int zero_point_word(int nl) { return nl & 7; }
+__device__ __forceinline__ int zero_point_shift(int nl) {
+  const int t = nl >> 3;
+  return 4 * ((t >> 1) + 4 * (t & 1));
+}
+
+template <typename T>
+struct Dq;
+
+// ---------------------------------------------------------------- fp16
+// (q & 0x000f000f) | 0x64006400 is the half2 (1024 + v_lo, 1024 + v_hi);
+// with mask 0x00f000f0 it is 1024 + 16 v.  Subtracting 1024 + z, or
+// fma(x, 1/16, -(64 + z)), gives v - z exactly; one packed multiply by the
+// scale then rounds once.
+template <>
+struct Dq<_Float16> {
+  typedef half8_t vec8;
+  struct Col {
+    half2_t s;    // (s, s)
+    half2_t c0;   // 1024 + z
+    half2_t c1;   // -(64 + z)
+  };
+  static __device__ __forceinline__ Col make_col(uint16_t scale_bits, int z) {
+    Col c;
+    const _Float16 s = __builtin_bit_cast(_Float16, scale_bits);
+    c.s = half2_t{s, s};
+    const _Float16 a = (_Float16)(float)(1024 + z);
+    const _Float16 b = (_Float16)(float)(-(64 + z));
+    c.c0 = half2_t{a, a};
+    c.c1 = half2_t{b, b};
+    return c;
+  }
+  static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c) {
+    const half2_t r16 = half2_t{(_Float16)0.0625f, (_Float16)0.0625f};
+    const uint32_t lo0 = (q & 0x000f000fu) | 0x64006400u;
+    const uint32_t hi0 = (q & 0x00f000f0u) | 0x64006400u;
+    q >>= 8;
+    const uint32_t lo1 = (q & 0x000f000fu) | 0x64006400u;
+    const uint32_t hi1 = (q & 0x00f000f0u) | 0x64006400u;
+    const half2_t d0 = __builtin_bit_cast(half2_t, lo0) - c.c0;
+    const half2_t d1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, hi0), r16, c.c1);
+    const half2_t d2 = __builtin_bit_cast(half2_t, lo1) - c.c0;
+    const half2_t d3 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, hi1), r16, c.c1);
+    const half2_t w0 = d0 * c.s, w1 = d1 * c.s, w2 = d2 * c.s, w3 = d3 * c.s;
+    return vec8{w0.x, w0.y, w1.x, w1.y, w2.x, w2.y, w3.x, w3.y};
+  }
+  static __device__ __forceinline__ floatx4_t mfma(vec8 w, vec8 a, floatx4_t acc) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(w, a, acc, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    return __builtin_bit_cast(uint16_t, (_Float16)f);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t b) {
+    return (float)__builtin_bit_cast(_Float16, b);
+  }
+};
+
+// ---------------------------------------------------------------- bf16
+// gfx950 has no packed bf16 arithmetic.  The same fp16 magic numbers are used
+// and each half is widened inside a mixed-precision fma: with S = float(s),
+// fma(1024 + v, S, -(1024 + z) S) and fma(1024 + 16 v, S/16, -(64 + z) S) are
+// exact in fp32 (at most 19 significant bits per term, result (v - z) S has at
+// most 12), so the only rounding is the fp32 -> bf16 conversion
+// (v_cvt_pk_bf16_f32, round to nearest even).
+template <>
+struct Dq<__bf16> {
+  typedef bf16x8_t vec8;
+  struct Col {
+    float s, s16, c0, c1;
+  };
+  static __device__ __forceinline__ Col make_col(uint16_t scale_bits, int z) {
+    Col c;
+    c.s = __builtin_bit_cast(float, (uint32_t)scale_bits << 16);
+    c.s16 = c.s * 0.0625f;
+    c.c0 = -(float)(1024 + z) * c.s;
+    c.c1 = -(float)(64 + z) * c.s;
+    return c;
+  }
+  static __device__ __forceinline__ bf16x2_t pair(uint32_t bits, float mul, float add) {
+    const half2_t h = __builtin_bit_cast(half2_t, bits);
+    const floatx2_t f = floatx2_t{__builtin_fmaf((float)h.x, mul, add),
+                                  __builtin_fmaf((float)h.y, mul, add)};
+    return __builtin_convertvector(f, bf16x2_t);
+  }
+  static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c) {
+    const uint32_t lo0 = (q & 0x000f000fu) | 0x64006400u;
+    const uint32_t hi0 = (q & 0x00f000f0u) | 0x64006400u;
+    q >>= 8;
+    const uint32_t lo1 = (q & 0x000f000fu) | 0x64006400u;
+    const uint32_t hi1 = (q & 0x00f000f0u) | 0x64006400u;
+    const bf16x2_t w0 = pair(lo0, c.s, c.c0);
+    const bf16x2_t w1 = pair(hi0, c.s16, c.c1);
+    const bf16x2_t w2 = pair(lo1, c.s, c.c0);
+    const bf16x2_t w3 = pair(hi1, c.s16, c.c1);
+    return vec8{w0.x, w0.y, w1.x, w1.y, w2.x, w2.y, w3.x, w3.y};
+  }
+  static __device__ __forceinline__ floatx4_t mfma(vec8 w, vec8 a, floatx4_t acc) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, a, acc, 0, 0, 0);
+  }
+  static __device__ __forceinline__ uint16_t from_float(float f) {
+    return __builtin_bit_cast(uint16_t, (__bf16)f);
+  }
+  static __device__ __forceinline__ float to_float(uint16_t b) {
+    return __builtin_bit_cast(float, (uint32_t)b << 16);
+  }
+};
+
+// How the scale row of a weight row is found.
+struct GroupMap {
+  int group_size;        // rows per group; >= 32 and a multiple of 32 when rows_by_g_idx == 0
+  int num_groups;
+  int rows_by_g_idx;     // 1: row k uses scale row g_idx[k] (act-order, partial K)
+  bool grouped_perm() const { return num_groups > 1; }
+};
+
+// Per-lane constants of the four columns (j = 0..3) a lane dequantises, for
+// the group `g` of strip `strip`.
+template <typename T, bool HAS_ZP>
+__device__ __forceinline__ void load_cols(typename Dq<T>::Col (&cols)[4], const uint16_t* scales,
+                                          const uint32_t* zeros, int size_n, int strip, int g,
+                                          int col16, bool grouped) {
+  const uint16_t* srow = scales + (long)g * size_n + strip * kStripN;
+  uint32_t zword = 0;
+  if (HAS_ZP) zword = zeros[(long)g * (size_n / 8) + strip * 8 + zero_point_word(col16)];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int nl = 16 * j + col16;
+    int z = 8;
+    if (HAS_ZP) z = (int)((zword >> zero_point_shift(nl)) & 0xFu);
+    cols[j] = Dq<T>::make_col(srow[scale_slot(nl, grouped)], z);
+  }
+}
+
+}  // namespace sonar

@@ -1,0 +1,223 @@
+// Weight re-ordering kernels: checkpoint packings -> Marlin tile order, and
+// Marlin tile order <-> the gfx950 streaming order.  Pure integer work; each
+// thread assembles one 32-bit output word from eight source nibbles, so the
+// stores of a wavefront are one contiguous 256-byte run.
+#include "common.hpp"
+
+namespace sonar {
+
+thread_local char g_last_error[512] = "";
+char* last_error_buffer() { return g_last_error; }
+
+namespace {
+
+// Position of a weight inside a Marlin tile (16-bit activations, 4-bit
+// weights).  Word w = lane*4 + j of the tile; lane = 4*c + h, c = column % 8
+// inside the 16-column sub-tile j, h = (row % 8) / 2.  Nibble slot s of the
+// word holds row 2h + (s >> 2) + 8*(s & 1), column c + 8*((s >> 1) & 1).
+__device__ __forceinline__ void marlin_word_sources(int word, int slot, int& row, int& col) {
+  const int lane = word >> 2;
+  const int j = word & 3;
+  const int c = lane >> 2;
+  const int h = lane & 3;
+  row = 2 * h + (slot >> 2) + 8 * (slot & 1);
+  col = 16 * j + c + 8 * ((slot >> 1) & 1);
+}
+
+template <bool HAS_PERM>
+__global__ __launch_bounds__(256) void gptq_to_marlin_kernel(
+    const uint32_t* __restrict__ in, const int32_t* __restrict__ perm,
+    uint32_t* __restrict__ out, int size_k, int size_n, long total_words) {
+  const int n_tiles = size_n / kMarlinTileN;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_words;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long tile = idx / kMarlinTileWords;
+    const int word = (int)(idx % kMarlinTileWords);
+    const int kt = (int)(tile / n_tiles);
+    const int nt = (int)(tile % n_tiles);
+    uint32_t packed = 0;
+#pragma unroll
+    for (int slot = 0; slot < 8; ++slot) {
+      int row, col;
+      marlin_word_sources(word, slot, row, col);
+      int k = kt * kMarlinTileK + row;
+      if (HAS_PERM) k = perm[k];
+      const int n = nt * kMarlinTileN + col;
+      const uint32_t src = in[(long)(k >> 3) * size_n + n];
+      packed |= ((src >> (4 * (k & 7))) & 0xFu) << (4 * slot);
+    }
+    out[idx] = packed;
+  }
+}
+
+__global__ __launch_bounds__(256) void awq_to_marlin_kernel(
+    const uint32_t* __restrict__ in, uint32_t* __restrict__ out, int size_k,
+    int size_n, long total_words) {
+  const int n_tiles = size_n / kMarlinTileN;
+  const int in_stride = size_n / 8;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_words;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long tile = idx / kMarlinTileWords;
+    const int word = (int)(idx % kMarlinTileWords);
+    const int kt = (int)(tile / n_tiles);
+    const int nt = (int)(tile % n_tiles);
+    uint32_t packed = 0;
+#pragma unroll
+    for (int slot = 0; slot < 8; ++slot) {
+      int row, col;
+      marlin_word_sources(word, slot, row, col);
+      const int k = kt * kMarlinTileK + row;
+      const int n = nt * kMarlinTileN + col;
+      // column n % 8 = 2*(p % 4) + p / 4 sits at nibble p = (n%8)/2 + 4*(n%2)
+      const int p = ((n & 7) >> 1) + 4 * (n & 1);
+      const uint32_t src = in[(long)k * in_stride + (n >> 3)];
+      packed |= ((src >> (4 * p)) & 0xFu) << (4 * slot);
+    }
+    out[idx] = packed;
+  }
+}
+
+// One thread per gfx950 word.  Word j of lane L of chunk c of strip s holds
+// column 64s + 16j + L%16, rows 32c + 8*(L/16) + t (t = 0..7) with row t at
+// nibble slot t/2 + 4*(t%2).  Those eight rows live in Marlin k-tile
+// 2c + (L/32) at tile rows 8*((L/16)%2) + t, i.e. in the four Marlin words
+// lane_m*4 + j with lane_m = 4*(col%8) + t/2.
+__global__ __launch_bounds__(256) void marlin_to_gfx950_kernel(
+    const uint32_t* __restrict__ in, uint32_t* __restrict__ out, int size_k,
+    int size_n, long total_words) {
+  const int n_tiles = size_n / kMarlinTileN;
+  const int chunks = size_k / kChunkK;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_words;
+       idx += (long)gridDim.x * blockDim.x) {
+    const int j = (int)(idx & 3);
+    const int lane = (int)((idx >> 2) & 63);
+    const long chunk_id = idx >> 8;
+    const int c = (int)(chunk_id % chunks);
+    const int s = (int)(chunk_id / chunks);
+    const int col16 = lane & 15;
+    const int kb = lane >> 4;
+    const int kt = 2 * c + (kb >> 1);
+    const int hb = kb & 1;  // upper half of the 16-row tile?
+    const uint32_t* tile = in + ((long)kt * n_tiles + s) * kMarlinTileWords;
+    // Marlin slot of (tile row 8*hb + t, column col16): hb + 2*(col16/8) + 4*(t%2)
+    const int slot_even = hb + 2 * (col16 >> 3);
+    uint32_t packed = 0;
+#pragma unroll
+    for (int h = 0; h < 4; ++h) {
+      const uint32_t w = tile[(4 * (col16 & 7) + h) * 4 + j];
+      const uint32_t even = (w >> (4 * slot_even)) & 0xFu;        // row t = 2h
+      const uint32_t odd = (w >> (4 * (slot_even + 4))) & 0xFu;   // row t = 2h+1
+      packed |= (even << (4 * h)) | (odd << (4 * (h + 4)));
+    }
+    out[idx] = packed;
+  }
+}
+
+// Inverse of the above: one thread per Marlin word.
+__global__ __launch_bounds__(256) void gfx950_to_marlin_kernel(
+    const uint32_t* __restrict__ in, uint32_t* __restrict__ out, int size_k,
+    int size_n, long total_words) {
+  const int n_tiles = size_n / kMarlinTileN;
+  const int chunks = size_k / kChunkK;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_words;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long tile = idx / kMarlinTileWords;
+    const int word = (int)(idx % kMarlinTileWords);
+    const int kt = (int)(tile / n_tiles);
+    const int nt = (int)(tile % n_tiles);
+    uint32_t packed = 0;
+#pragma unroll
+    for (int slot = 0; slot < 8; ++slot) {
+      int row, col;
+      marlin_word_sources(word, slot, row, col);
+      const int k = kt * kMarlinTileK + row;
+      const int c = k / kChunkK;
+      const int kb = (k % kChunkK) >> 3;
+      const int t = k & 7;
+      const int lane = 16 * kb + (col & 15);
+      const int j = col >> 4;
+      const uint32_t src = in[(((long)nt * chunks + c) * 64 + lane) * 4 + j];
+      const int src_slot = (t >> 1) + 4 * (t & 1);
+      packed |= ((src >> (4 * src_slot)) & 0xFu) << (4 * slot);
+    }
+    out[idx] = packed;
+  }
+}
+
+int grid_for(long total_words) {
+  long blocks = (total_words + 255) / 256;
+  if (blocks > 256L * 32) blocks = 256L * 32;
+  if (blocks < 1) blocks = 1;
+  return (int)blocks;
+}
+
+int check_repack_shape(int64_t size_k, int64_t size_n, int num_bits) {
+  if (num_bits == 8)
+    return fail(SONAR_E_UNSUPPORTED, "num_bits = 8 (uint8b128) is not built; only 4-bit weights are");
+  SONAR_REQUIRE(num_bits == 4, "num_bits must be 4 or 8. Got = %d", num_bits);
+  SONAR_REQUIRE(size_k > 0 && size_n > 0, "size_k = %ld and size_n = %ld must be positive",
+                (long)size_k, (long)size_n);
+  SONAR_REQUIRE(size_k % kMarlinTileK == 0, "size_k = %ld is not divisible by tile_k_size = %d",
+                (long)size_k, kMarlinTileK);
+  SONAR_REQUIRE(size_n % kMarlinTileN == 0, "size_n = %ld is not divisible by tile_n_size = %d",
+                (long)size_n, kMarlinTileN);
+  SONAR_REQUIRE(size_k * size_n / 8 < (1LL << 40), "weight too large");
+  SONAR_REQUIRE(size_k < (1LL << 30) && size_n < (1LL << 30), "size_k / size_n too large");
+  return SONAR_OK;
+}
+
+}  // namespace
+}  // namespace sonar
+
+using namespace sonar;
+
+extern "C" const char* sonar_marlin_last_error(void) { return last_error_buffer(); }
+extern "C" const char* sonar_marlin_version(void) { return "sonar-marlin-gfx950 0.1"; }
+
+extern "C" int sonar_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_t* perm,
+                                        uint32_t* out, int64_t size_k, int64_t size_n,
+                                        int num_bits, void* stream) {
+  if (int rc = check_repack_shape(size_k, size_n, num_bits)) return rc;
+  SONAR_REQUIRE(b_q_weight && out, "b_q_weight and out must not be NULL");
+  const long total = size_k * size_n / 8;
+  hipStream_t st = (hipStream_t)stream;
+  if (perm)
+    gptq_to_marlin_kernel<true><<<grid_for(total), 256, 0, st>>>(b_q_weight, perm, out, (int)size_k,
+                                                                (int)size_n, total);
+  else
+    gptq_to_marlin_kernel<false><<<grid_for(total), 256, 0, st>>>(b_q_weight, nullptr, out,
+                                                                 (int)size_k, (int)size_n, total);
+  return launch_status("gptq_to_marlin_kernel");
+}
+
+extern "C" int sonar_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out, int64_t size_k,
+                                       int64_t size_n, int num_bits, void* stream) {
+  if (int rc = check_repack_shape(size_k, size_n, num_bits)) return rc;
+  SONAR_REQUIRE(b_q_weight && out, "b_q_weight and out must not be NULL");
+  const long total = size_k * size_n / 8;
+  awq_to_marlin_kernel<<<grid_for(total), 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k,
+                                                                        (int)size_n, total);
+  return launch_status("awq_to_marlin_kernel");
+}
+
+extern "C" int sonar_marlin_to_gfx950(const uint32_t* marlin, uint32_t* out, int64_t size_k,
+                                      int64_t size_n, void* stream) {
+  if (int rc = check_repack_shape(size_k, size_n, 4)) return rc;
+  SONAR_REQUIRE(size_k % kChunkK == 0, "size_k = %ld is not divisible by %d", (long)size_k, kChunkK);
+  SONAR_REQUIRE(marlin && out && marlin != out, "marlin and out must be distinct non-NULL buffers");
+  const long total = size_k * size_n / 8;
+  marlin_to_gfx950_kernel<<<grid_for(total), 256, 0, (hipStream_t)stream>>>(marlin, out, (int)size_k,
+                                                                           (int)size_n, total);
+  return launch_status("marlin_to_gfx950_kernel");
+}
+
+extern "C" int sonar_gfx950_to_marlin(const uint32_t* gfx950, uint32_t* out, int64_t size_k,
+                                      int64_t size_n, void* stream) {
+  if (int rc = check_repack_shape(size_k, size_n, 4)) return rc;
+  SONAR_REQUIRE(size_k % kChunkK == 0, "size_k = %ld is not divisible by %d", (long)size_k, kChunkK);
+  SONAR_REQUIRE(gfx950 && out && gfx950 != out, "gfx950 and out must be distinct non-NULL buffers");
+  const long total = size_k * size_n / 8;
+  gfx950_to_marlin_kernel<<<grid_for(total), 256, 0, (hipStream_t)stream>>>(gfx950, out, (int)size_k,
+                                                                           (int)size_n, total);
+  return launch_status("gfx950_to_marlin_kernel");
+}

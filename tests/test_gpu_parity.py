@@ -1,0 +1,176 @@
+"""GPU parity: HIP kernels, called through the C ABI, against the CPU oracle.
+Integer results are compared bit for bit; GEMM outputs with the tolerance
+max|err| <= 1e-2*max|ref| and |err| <= 1e-2*max|ref| + 1e-2*|ref|."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import marlin_oracle as mo
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def gu():
+    from tests import gpu_util
+    return gpu_util
+
+
+# reference repack tests use K = 128*{8,5,11}, N = {64,256}*{4,7,13}
+REPACK_SHAPES = [(128 * 8, 64 * 4), (128 * 5, 64 * 7), (128 * 11, 256 * 13), (128, 64), (4096, 4096)]
+
+
+@pytest.mark.parametrize("k,n", REPACK_SHAPES)
+@pytest.mark.parametrize("act_order", [False, True])
+def test_gptq_marlin_repack_bit_exact(gu, k, n, act_order):
+    rng = np.random.default_rng(k + n)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    perm = rng.permutation(k).astype(np.int32) if act_order else None
+    out = gu.gptq_repack(gu.dev_i32(mo.gptq_pack(q)), gu.dev_i32(perm) if act_order else None, k, n)
+    want = mo.gptq_marlin_repack(mo.gptq_pack(q), perm, k, n)
+    assert out.shape == (k // 16, 2 * n)
+    assert np.array_equal(out.cpu().numpy(), want)
+
+
+@pytest.mark.parametrize("k,n", REPACK_SHAPES)
+def test_awq_marlin_repack_bit_exact(gu, k, n):
+    rng = np.random.default_rng(k * 3 + n)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    out = gu.awq_repack(gu.dev_i32(mo.awq_pack(q)), k, n)
+    assert np.array_equal(out.cpu().numpy(), mo.awq_marlin_repack(mo.awq_pack(q), k, n))
+
+
+@pytest.mark.parametrize("k,n", [(32, 64), (640, 448), (4096, 11008), (14336, 4096)])
+def test_gfx950_retile_bit_exact_and_round_trip(gu, k, n):
+    rng = np.random.default_rng(k + 7 * n)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    marlin = gu.dev_i32(mo.marlin_pack(q))
+    native = gu.to_gfx950(marlin, k, n)
+    assert np.array_equal(native.cpu().numpy(), mo.gfx950_pack(q))
+    back = gu.from_gfx950(native, k, n)
+    assert torch.equal(back.view(-1), marlin.view(-1))
+
+
+DEQUANT_CASES = [
+    # k, n, group, zero_points
+    (256, 128, 128, False), (256, 128, 64, False), (256, 128, 32, True), (512, 192, -1, False),
+    (512, 192, -1, True), (4096, 4096, 128, False), (4096, 11008, 128, True),
+]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("k,n,g,zp", DEQUANT_CASES)
+def test_in_kernel_dequant_bit_exact(gu, dtype, k, n, g, zp):
+    layer = gu.DeviceLayer(11, k, n, g, dtype, zero_points=zp)
+    w = layer.dequant()
+    got = w.view(torch.int16).cpu().numpy().view(np.uint16)
+    want = mo.to_bits16(layer.w_ref, dtype)
+    # +0 and -0 are both "zero times scale"; compare as values where the oracle has a zero
+    same = (got == want) | ((layer.w_ref == 0) & ((got & 0x7FFF) == 0))
+    assert bool(same.all()), f"{(~same).sum()} of {same.size} dequantised values differ"
+
+
+def test_dequant_extreme_scales_bit_exact(gu):
+    """Scales far outside the usual range (tiny, large, zero) still give
+    round((v - z) * s) exactly."""
+    k, n = 128, 64
+    for dtype in ("fp16", "bf16"):
+        layer = gu.DeviceLayer(5, k, n, 32, dtype, zero_points=True)
+        rng = np.random.default_rng(1)
+        s = np.concatenate([rng.uniform(1e-6, 1e-4, 64), rng.uniform(0.5, 100.0, 64),
+                            np.zeros(16), rng.uniform(1e-3, 1e-2, 112)]).astype(np.float32)
+        s = mo.round_to_dtype(s.reshape(4, 64), dtype)
+        layer.scales = gu.dev_bits16(mo.marlin_permute_scales(s, k, n, 32), dtype)
+        want = mo.dequantize(layer.layer["q"], s, 32, dtype, zeros=layer.layer["zeros"])
+        got = gu.host_f32(layer.dequant())
+        assert np.array_equal(got, want)
+
+
+GEMM_CASES = [
+    # m, k, n, group, zp, act_order, bias
+    (1, 128, 64, 128, False, False, False),
+    (16, 4096, 4096, 128, False, False, False),      # benchmark config 1
+    (1, 256, 128, 32, False, False, False),
+    (26, 1024, 256, 64, False, False, True),
+    (7, 640, 448, -1, False, False, False),
+    (33, 512, 192, 128, True, False, False),
+    (64, 2048, 1024, 128, True, False, True),
+    (1, 4096, 11008, 128, False, True, False),       # act-order, benchmark config 4
+    (1, 4096, 11008, 128, True, False, False),       # AWQ, benchmark config 4
+    (48, 1024, 512, 32, False, True, False),
+    (65, 512, 256, 128, False, False, False),
+    (257, 1280, 320, 128, False, False, True),
+    (8, 96, 64, 32, False, False, False),            # K % 64 != 0
+    (3, 14336, 4096, 128, False, False, False),
+    (5, 4096, 28672, 128, False, False, False),
+    (2, 4096, 6144, 128, False, False, False),
+]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("m,k,n,g,zp,act,bias", GEMM_CASES)
+def test_marlin_gemm_within_tolerance(gu, dtype, m, k, n, g, zp, act, bias):
+    layer = gu.DeviceLayer(21 + m, k, n, g, dtype, zero_points=zp, act_order=act, bias=bias)
+    a32 = mo.make_activations(m * 7 + 1, m, k, dtype)
+    a = gu.dev_bits16(a32, dtype)
+    c = layer.gemm(a, m)
+    torch.cuda.synchronize()
+    ref = mo.gemm_reference(a32, layer.w_ref, layer.bias32)
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), ref)
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+    assert int(layer.workspace.abs().sum().item()) == 0, "workspace must return to zero"
+    # a second call on the same workspace gives the same bits (fixed reduction order)
+    c2 = layer.gemm(a, m)
+    assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
+
+
+def test_gemm_row_strided_activations(gu):
+    m, k, n = 9, 512, 256
+    layer = gu.DeviceLayer(3, k, n, 128, "fp16")
+    big32 = mo.make_activations(5, m, k + 64, "fp16")
+    big = gu.dev_bits16(big32, "fp16")
+    a = big[:, 32:32 + k]   # row stride k + 64, 64-byte offset
+    c = layer.gemm(a, m)
+    ref = mo.gemm_reference(big32[:, 32:32 + k], layer.w_ref)
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), ref)
+    assert ok, (max_err, max_ref)
+
+
+def test_gemm_special_cases_reduce_to_row_sums(gu):
+    """All codes 9, scale 1: W == 1, so C[m][n] is the row sum of A; and M = 0
+    leaves the output untouched."""
+    m, k, n = 4, 256, 128
+    layer = gu.DeviceLayer(1, k, n, 128, "fp16")
+    q = np.full((k, n), 9, dtype=np.int32)
+    layer.native = gu.to_gfx950(gu.gptq_repack(gu.dev_i32(mo.gptq_pack(q)), None, k, n), k, n)
+    layer.scales = gu.dev_bits16(np.ones((2, n), np.float32), "fp16")
+    a32 = mo.make_activations(2, m, k, "fp16")
+    c = gu.host_f32(layer.gemm(gu.dev_bits16(a32, "fp16"), m))
+    want = a32.sum(axis=1, keepdims=True).repeat(n, 1)
+    assert np.allclose(c, want, rtol=2e-3, atol=2e-2)
+    empty = layer.gemm(torch.empty((0, k), dtype=torch.float16, device=gu.DEV), 0)
+    assert empty.shape == (0, n)
+
+
+def test_error_paths(gu):
+    from sonar_amd import _lib
+    lib = _lib.load()
+    t = torch.zeros(1024, dtype=torch.int32, device=gu.DEV)
+    with pytest.raises(_lib.SonarMarlinError, match="size_k"):
+        _lib.check(lib.sonar_gptq_marlin_repack(gu.ptr(t), None, gu.ptr(t), 24, 64, 4, gu.stream()))
+    with pytest.raises(_lib.SonarMarlinError, match="size_n"):
+        _lib.check(lib.sonar_awq_marlin_repack(gu.ptr(t), gu.ptr(t), 32, 96, 4, gu.stream()))
+    with pytest.raises(NotImplementedError):
+        _lib.check(lib.sonar_gptq_marlin_repack(gu.ptr(t), None, gu.ptr(t), 32, 64, 8, gu.stream()))
+    layer = gu.DeviceLayer(1, 128, 64, 128, "fp16")
+    a = torch.zeros((1, 128), dtype=torch.float16, device=gu.DEV)
+    layer.b_type = 1125899923621888  # uint8b128
+    with pytest.raises(NotImplementedError):
+        layer.gemm(a, 1)
+    layer.b_type = _lib.TYPE_UINT4  # uint4 needs zero points
+    with pytest.raises(_lib.SonarMarlinError, match="has_zp"):
+        layer.gemm(a, 1)
+    layer.b_type = _lib.TYPE_UINT4B8
+    layer.workspace = torch.zeros(4, dtype=torch.int32, device=gu.DEV)
+    with pytest.raises(_lib.SonarMarlinError, match="workspace"):
+        layer.gemm(a, 1)
