@@ -1,0 +1,227 @@
+#!/usr/bin/env python3
+"""Benchmark of the W4A16 Marlin-family GEMM on one MI355X.
+
+A step is one pass over the four W4A16 projection GEMMs of a Llama-3-8B decoder
+layer (qkv 4096x6144, o 4096x4096, gate_up 4096x28672, down 14336x4096;
+int4 weights, group size 128) at M = 16 bf16 activation rows, through the same
+torch ops the reference's callers use.  Weights of `--copies` distinct layers
+(more bytes than the 256 MB last-level cache) are visited round-robin so every
+step streams its weights from HBM.  The K timed steps are recorded in one HIP
+graph and replayed once between two events on the launching stream.
+
+Prints one JSON line; `--sweep` adds the M sweep of the decode and prefill
+shapes under "sweep".
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
+MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
+GROUP = 128
+LAYER_SHAPES = [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
+
+
+def algorithmic_bytes(m: int, k: int, n: int, zeros: bool = False, act_order: bool = False) -> int:
+    b = k * n // 2 + (k // GROUP) * n * 2 + m * k * 2 + m * n * 2
+    if zeros:
+        b += (k // GROUP) * n // 2
+    if act_order:
+        b += 8 * k
+    return b
+
+
+class Layer:
+    """One quantised projection with random codes and scales, already on the
+    device in the layouts the ops take."""
+
+    def __init__(self, torch, k, n, dtype, gen):
+        from sonar_amd import marlin_utils
+        self.k, self.n = k, n
+        dev = "cuda:0"
+        self.qweight = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, 2 * n), dtype=torch.int32,
+                                     device=dev, generator=gen)
+        self.scales = (torch.rand((k // GROUP, n), device=dev, generator=gen) * 9e-3 + 1e-3).to(dtype)
+        self.empty = torch.empty(0, dtype=torch.int32, device=dev)
+        self.workspace = marlin_utils.marlin_make_workspace_new(torch.device(dev))
+
+    def run(self, ops, a, wtype):
+        return ops.marlin_gemm(a, None, self.qweight, None, self.scales, None, None, self.empty,
+                               self.empty, self.empty, self.workspace, wtype, a.shape[0], self.n, self.k,
+                               True, False, True, False)
+
+
+def time_graph(torch, fn, reps):
+    """Records `reps` calls of fn() in a HIP graph, replays it once untimed and
+    once between two events; returns seconds per call."""
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        fn()
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(reps):
+                fn(i)
+        graph.replay()
+        stream.synchronize()
+        t0 = torch.cuda.Event(enable_timing=True)
+        t1 = torch.cuda.Event(enable_timing=True)
+        t0.record(stream)
+        graph.replay()
+        t1.record(stream)
+        stream.synchronize()
+    return t0.elapsed_time(t1) * 1e-3 / reps
+
+
+def cpu_baseline(threads: int):
+    """The layer's CPU path (int4 dequantise + fp32 torch.matmul) from the
+    oracle, on the o_proj shape at M = 16."""
+    import numpy as np
+
+    from oracle import marlin_oracle as mo
+    k, n, m = 4096, 4096, 16
+    layer = mo.make_layer(0, k, n, GROUP, "fp16")
+    a = mo.make_activations(1, m, k, "fp16")
+    t_full, t_mm, _ = mo.cpu_layer_baseline(mo.gptq_pack(layer["q"]), layer["scales"], a, GROUP, threads,
+                                            repeats=5, warmup=2)
+    nbytes = algorithmic_bytes(m, k, n)
+    return {"value": round(nbytes / t_full / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+            "sample": "o_proj 4096x4096, M=16, fp16: dequantise+matmul fp32, median of 5 "
+                      f"({t_full * 1e3:.1f} ms; matmul alone {t_mm * 1e3:.1f} ms)",
+            "gflops": round(2 * m * n * k / t_full / 1e9, 2)}
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--m", type=int, default=16)
+    ap.add_argument("--copies", type=int, default=6)
+    ap.add_argument("--sweep", action="store_true")
+    ap.add_argument("--no-cpu", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs on one GPU only (the GEMM is rank-local; no multi-GPU path "
+              "exists); run with --gpus 1", file=sys.stderr)
+        return 2
+
+    import torch
+    if not torch.cuda.is_available():
+        print("bench.py: needs a GPU", file=sys.stderr)
+        return 2
+    from sonar_amd import ops
+    from sonar_amd.scalar_type import scalar_types
+    torch.cuda.set_device(0)
+    gen = torch.Generator(device="cuda:0")
+    gen.manual_seed(1234)
+    dtype = torch.bfloat16
+    wtype = scalar_types.uint4b8
+    m = args.m
+
+    copies = [[Layer(torch, k, n, dtype, gen) for (_, k, n) in LAYER_SHAPES] for _ in range(args.copies)]
+    acts = {k: torch.randn((m, k), device="cuda:0", generator=gen).to(dtype) for k in (4096, 14336)}
+
+    def step(i=0):
+        for layer in copies[i % args.copies]:
+            layer.run(ops, acts[layer.k], wtype)
+
+    # warm-up (also converts every weight to the streaming order, once)
+    for i in range(max(args.warmup, args.copies)):
+        step(i)
+    torch.cuda.synchronize()
+
+    # eager timing: K steps launched one by one
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    eager_s = (time.perf_counter() - t0) / args.steps
+
+    # timed region: exactly K steps in one graph, events on the launching stream
+    torch.cuda.synchronize()
+    step_s = time_graph(torch, step, args.steps)
+
+    step_bytes = sum(algorithmic_bytes(m, k, n) for (_, k, n) in LAYER_SHAPES)
+    step_flops = sum(2 * m * k * n for (_, k, n) in LAYER_SHAPES)
+    launches = len(LAYER_SHAPES)
+    gbps = step_bytes / step_s / 1e9
+
+    per_gemm = []
+    for idx, (name, k, n) in enumerate(LAYER_SHAPES):
+        def one(i=0, idx=idx, k=k):
+            copies[i % args.copies][idx].run(ops, acts[k], wtype)
+        s = time_graph(torch, one, max(24, args.copies * 4))
+        nb = algorithmic_bytes(m, k, n)
+        per_gemm.append({"gemm": name, "k": k, "n": n, "m": m, "us": round(s * 1e6, 2),
+                         "GBps": round(nb / s / 1e9, 1), "frac_hbm": round(nb / s / 1e9 / HBM_PEAK_GBPS, 4)})
+
+    out = {
+        "metric": "W4A16 GEMM TFLOP/s + HBM GB/s (% roofline), Llama-3-8B shapes, M=1..8192",
+        "value": round(gbps, 1),
+        "unit": "GB/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(step_s * 1e3, 5),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": f"llama3-8b decoder layer W4A16 GEMMs (qkv+o+gate_up+down), M={m}, "
+                               f"bf16 activations, uint4b8 weights, group_size 128, {args.copies} "
+                               "weight copies round-robin, K steps in one HIP graph",
+                   "global_batch": m},
+        "tflops": round(step_flops / step_s / 1e12, 2),
+        "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
+                     "kernel": "marlin_stream_kernel<bf16, MB=%d>" % ((m + 15) // 16),
+                     "bytes_per_launch": step_bytes // launches,
+                     "us_per_launch": round(step_s / launches * 1e6, 3)},
+        "eager_ms_per_step": round(eager_s * 1e3, 5),
+        "per_gemm": per_gemm,
+    }
+
+    if args.sweep:
+        sweep = []
+        for (regime, ms, dt) in (("decode", (1, 2, 4, 8, 16, 32, 64), torch.bfloat16),
+                                 ("prefill", (256, 1024, 4096, 8192), torch.float16)):
+            layers = copies if dt == dtype else [[Layer(torch, k, n, dt, gen) for (_, k, n) in LAYER_SHAPES]
+                                                 for _ in range(2)]
+            for mm in ms:
+                for idx, (name, k, n) in enumerate(LAYER_SHAPES):
+                    a = torch.randn((mm, k), device="cuda:0", generator=gen).to(dt)
+                    if regime == "prefill":
+                        a = a * 0.5
+
+                    def one(i=0, idx=idx, a=a, layers=layers):
+                        layers[i % len(layers)][idx].run(ops, a, wtype)
+                    reps = 24 if regime == "decode" else 4
+                    s = time_graph(torch, one, reps)
+                    nb = algorithmic_bytes(mm, k, n)
+                    fl = 2 * mm * k * n
+                    sweep.append({"regime": regime, "gemm": name, "m": mm, "k": k, "n": n,
+                                  "us": round(s * 1e6, 2), "GBps": round(nb / s / 1e9, 1),
+                                  "TFLOPs": round(fl / s / 1e12, 2),
+                                  "frac_hbm": round(nb / s / 1e9 / HBM_PEAK_GBPS, 4),
+                                  "frac_mfma": round(fl / s / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+                    print("sweep", json.dumps(sweep[-1]), file=sys.stderr, flush=True)
+        out["sweep"] = sweep
+
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline(min(os.cpu_count() or 1, 16))
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -31,6 +31,21 @@ __device__ __forceinline__ int zero_point_shift(int nl) {
   return 4 * ((t >> 1) + 4 * (t & 1));
 }
 
+// (q & mask) | 0x64006400 in one VALU instruction.  The encoding admits one
+// scalar operand, so the constant that is OR-ed in is kept in a vector
+// register by the caller (`magic`); left to itself the compiler splits the
+// expression into an AND and an OR with literals.
+__device__ __forceinline__ uint32_t magic_register() {
+  uint32_t m = 0x64006400u;
+  asm("" : "+v"(m));
+  return m;
+}
+__device__ __forceinline__ uint32_t and_or(uint32_t q, uint32_t mask, uint32_t magic) {
+  uint32_t r;
+  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(q), "s"(mask), "v"(magic));
+  return r;
+}
+
 template <typename T>
 struct Dq;
 
@@ -57,13 +72,13 @@ struct Dq<_Float16> {
     c.c1 = half2_t{b, b};
     return c;
   }
-  static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c) {
+  static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c, uint32_t magic) {
     const half2_t r16 = half2_t{(_Float16)0.0625f, (_Float16)0.0625f};
-    const uint32_t lo0 = (q & 0x000f000fu) | 0x64006400u;
-    const uint32_t hi0 = (q & 0x00f000f0u) | 0x64006400u;
+    const uint32_t lo0 = and_or(q, 0x000f000fu, magic);
+    const uint32_t hi0 = and_or(q, 0x00f000f0u, magic);
     q >>= 8;
-    const uint32_t lo1 = (q & 0x000f000fu) | 0x64006400u;
-    const uint32_t hi1 = (q & 0x00f000f0u) | 0x64006400u;
+    const uint32_t lo1 = and_or(q, 0x000f000fu, magic);
+    const uint32_t hi1 = and_or(q, 0x00f000f0u, magic);
     const half2_t d0 = __builtin_bit_cast(half2_t, lo0) - c.c0;
     const half2_t d1 = __builtin_elementwise_fma(__builtin_bit_cast(half2_t, hi0), r16, c.c1);
     const half2_t d2 = __builtin_bit_cast(half2_t, lo1) - c.c0;
@@ -109,12 +124,12 @@ struct Dq<__bf16> {
                                   __builtin_fmaf((float)h.y, mul, add)};
     return __builtin_convertvector(f, bf16x2_t);
   }
-  static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c) {
-    const uint32_t lo0 = (q & 0x000f000fu) | 0x64006400u;
-    const uint32_t hi0 = (q & 0x00f000f0u) | 0x64006400u;
+  static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c, uint32_t magic) {
+    const uint32_t lo0 = and_or(q, 0x000f000fu, magic);
+    const uint32_t hi0 = and_or(q, 0x00f000f0u, magic);
     q >>= 8;
-    const uint32_t lo1 = (q & 0x000f000fu) | 0x64006400u;
-    const uint32_t hi1 = (q & 0x00f000f0u) | 0x64006400u;
+    const uint32_t lo1 = and_or(q, 0x000f000fu, magic);
+    const uint32_t hi1 = and_or(q, 0x00f000f0u, magic);
     const bf16x2_t w0 = pair(lo0, c.s, c.c0);
     const bf16x2_t w1 = pair(hi0, c.s16, c.c1);
     const bf16x2_t w2 = pair(lo1, c.s, c.c0);
@@ -130,14 +145,6 @@ struct Dq<__bf16> {
   static __device__ __forceinline__ float to_float(uint16_t b) {
     return __builtin_bit_cast(float, (uint32_t)b << 16);
   }
-};
-
-// How the scale row of a weight row is found.
-struct GroupMap {
-  int group_size;        // rows per group; >= 32 and a multiple of 32 when rows_by_g_idx == 0
-  int num_groups;
-  int rows_by_g_idx;     // 1: row k uses scale row g_idx[k] (act-order, partial K)
-  bool grouped_perm() const { return num_groups > 1; }
 };
 
 // Per-lane constants of the four columns (j = 0..3) a lane dequantises, for

@@ -1,28 +1,28 @@
-// Streaming W4A16 GEMM for up to 64 activation rows per launch.
+// Streaming W4A16 GEMM for up to 64 activation rows per launch (the
+// bandwidth-bound regime).
 //
 // Work decomposition.  The packed weights are a list of strips (64 output
 // columns each), every strip a contiguous run of K/32 one-KiB chunks.  The list
 // of all (strip, unit) pairs - a unit is `unit_chunks` consecutive chunks - is
 // cut into equal contiguous ranges, one per workgroup, so every compute unit
-// streams the same number of bytes whatever the shape.  A workgroup walks its
-// range strip by strip.  Inside a strip segment its eight wavefronts take
-// units round-robin, so the workgroup reads memory front to back; each
-// wavefront keeps MB x 4 accumulator tiles (16 rows x 16 columns each) and
-// feeds v_mfma_f32_16x16x32 with the weights as the row operand and the
-// activations as the column operand.  The eight partial tiles are summed
-// through LDS.  A segment that covers the whole K of its strip is written
-// straight to C.  Otherwise the partial tile goes to scratch memory and a
-// counter in `workspace` (indexed by the first workgroup that touches the
-// strip) is incremented; the workgroup that brings it to the number of
-// contributors adds the partials in a fixed order, writes C and puts the
-// counter back to zero.  The result does not depend on arrival order.
+// streams the same number of bytes whatever the shape.  The units of a range
+// are dealt round-robin to the workgroup's wavefronts; each wavefront keeps
+// MB x 4 accumulator tiles (16 rows x 16 columns) and feeds
+// v_mfma_f32_16x16x32 with the dequantised weights as the row operand and the
+// activations as the column operand.  At the end of every strip segment the
+// wavefronts' tiles are summed through LDS.  A segment that covers the whole K
+// of its strip is rounded and written to C.  A partial segment is written as
+// an fp32 tile to scratch memory; a second, tiny kernel adds the (two to five)
+// partial tiles of each split strip in a fixed order and writes C.  Nothing
+// spins, nothing is atomic, and the result does not depend on timing.
+#include <cstdlib>
+
 #include "dequant.hpp"
 
 namespace sonar {
 namespace {
 
 constexpr int kWaves = 8;
-constexpr int kThreads = kWaves * 64;
 constexpr int kSlotFloat4 = 4 * 4 * 64;  // largest partial tile: 4 row blocks x 4 column blocks x 64 lanes
 
 struct StreamParams {
@@ -33,40 +33,42 @@ struct StreamParams {
   const uint16_t* bias;
   const uint16_t* scales;
   const uint32_t* zeros;
-  const int32_t* g_idx;
   const int32_t* perm;
-  int32_t* workspace;
   float4* scratch;
   int size_m, size_n, size_k;
   int num_groups, group_size;
   int chunks_per_strip;
   int unit_chunks;
   int units_per_strip;
+  int parts;  // number of workgroups of the streaming kernel
   long total_units;
 };
 
-__device__ __forceinline__ long range_begin(long i, long total, long parts) { return i * total / parts; }
+__host__ __device__ __forceinline__ long range_begin(long i, long total, long parts) { return i * total / parts; }
 // Largest i with range_begin(i) <= x, given parts <= total.
-__device__ __forceinline__ int range_owner(long x, long total, long parts) {
+__host__ __device__ __forceinline__ int range_owner(long x, long total, long parts) {
   return (int)(((x + 1) * parts - 1) / total);
+}
+// Scratch slot of workgroup `w` for a strip whose first contributor is `first`.
+__device__ __forceinline__ float4* partial_slot(const StreamParams& p, int w, int first) {
+  return p.scratch + (long)(w == first ? p.parts + w : w) * kSlotFloat4;
 }
 
 template <typename T, bool HAS_PERM>
 __device__ __forceinline__ typename Dq<T>::vec8 load_a(const StreamParams& p, int row, int k0) {
   typedef typename Dq<T>::vec8 vec8;
-  uint4 v = make_uint4(0, 0, 0, 0);
-  if (row < p.size_m) {
-    const uint16_t* arow = p.a + (long)row * p.lda;
-    if (!HAS_PERM) {
-      v = *reinterpret_cast<const uint4*>(arow + k0);
-    } else {
-      const int4 p0 = *reinterpret_cast<const int4*>(p.perm + k0);
-      const int4 p1 = *reinterpret_cast<const int4*>(p.perm + k0 + 4);
-      v.x = (uint32_t)arow[p0.x] | ((uint32_t)arow[p0.y] << 16);
-      v.y = (uint32_t)arow[p0.z] | ((uint32_t)arow[p0.w] << 16);
-      v.z = (uint32_t)arow[p1.x] | ((uint32_t)arow[p1.y] << 16);
-      v.w = (uint32_t)arow[p1.z] | ((uint32_t)arow[p1.w] << 16);
-    }
+  // rows past M are clamped: their products are computed and never stored
+  const uint16_t* arow = p.a + (long)(row < p.size_m ? row : p.size_m - 1) * p.lda;
+  uint4 v;
+  if (!HAS_PERM) {
+    v = *reinterpret_cast<const uint4*>(arow + k0);
+  } else {
+    const int4 p0 = *reinterpret_cast<const int4*>(p.perm + k0);
+    const int4 p1 = *reinterpret_cast<const int4*>(p.perm + k0 + 4);
+    v.x = (uint32_t)arow[p0.x] | ((uint32_t)arow[p0.y] << 16);
+    v.y = (uint32_t)arow[p0.z] | ((uint32_t)arow[p0.w] << 16);
+    v.z = (uint32_t)arow[p1.x] | ((uint32_t)arow[p1.y] << 16);
+    v.w = (uint32_t)arow[p1.z] | ((uint32_t)arow[p1.w] << 16);
   }
   return __builtin_bit_cast(vec8, v);
 }
@@ -100,29 +102,158 @@ __device__ __forceinline__ void write_tiles(const StreamParams& p, int strip, in
   }
 }
 
+// Sums the wavefronts' tiles into wavefront 0 through four LDS tile slots: a
+// group of up to four wavefronts writes, the group `dist` below it adds.
+template <int MB>
+__device__ __forceinline__ void reduce_round(floatx4_t (&acc)[MB][4], float4 (*red)[MB * 4][64], int wave,
+                                             int lane, int writer_lo, int count, int dist) {
+  if (wave >= writer_lo && wave < writer_lo + count) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const floatx4_t v = acc[mb][j];
+        red[wave - writer_lo][mb * 4 + j][lane] = make_float4(v.x, v.y, v.z, v.w);
+      }
+  }
+  __syncthreads();
+  if (wave >= writer_lo - dist && wave < writer_lo - dist + count) {
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float4 v = red[wave - (writer_lo - dist)][mb * 4 + j][lane];
+        acc[mb][j] += floatx4_t{v.x, v.y, v.z, v.w};
+      }
+  }
+  __syncthreads();
+}
+
+template <int MB, int WAVES>
+__device__ __forceinline__ void reduce_waves(floatx4_t (&acc)[MB][4], float4 (*red)[MB * 4][64], int wave,
+                                             int lane) {
+  static_assert(WAVES == 8 || WAVES == 16, "8 or 16 wavefronts");
+  if (WAVES == 16) {
+    reduce_round<MB>(acc, red, wave, lane, 12, 4, 8);  // 12..15 -> 4..7
+    reduce_round<MB>(acc, red, wave, lane, 8, 4, 8);   // 8..11 -> 0..3
+  }
+  reduce_round<MB>(acc, red, wave, lane, 4, 4, 4);     // 4..7 -> 0..3
+  reduce_round<MB>(acc, red, wave, lane, 2, 2, 2);     // 2..3 -> 0..1
+  reduce_round<MB>(acc, red, wave, lane, 1, 1, 1);     // 1 -> 0
+}
+
+// Wavefront 0: a finished segment goes to C when it is the whole strip, else
+// to this workgroup's scratch slot.
+template <typename T, int MB>
+__device__ __forceinline__ void finish_segment(const StreamParams& p, int strip, long seg_begin, long seg_end,
+                                               int lane, const floatx4_t (&acc)[MB][4]) {
+  const long strip_first = (long)strip * p.units_per_strip;
+  const long strip_end = strip_first + p.units_per_strip;
+  if (seg_begin == strip_first && seg_end == strip_end) {
+    write_tiles<T, MB>(p, strip, lane, acc);
+    return;
+  }
+  const int first = range_owner(strip_first, p.total_units, p.parts);
+  float4* slot = partial_slot(p, blockIdx.x, first);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const floatx4_t v = acc[mb][j];
+      slot[(mb * 4 + j) * 64 + lane] = make_float4(v.x, v.y, v.z, v.w);
+    }
+}
+
+// The same for one 16-column block (j) of a 16-row tile, held by one wavefront.
+template <typename T>
+__device__ __forceinline__ void finish_block(const StreamParams& p, int strip, long seg_begin, long seg_end,
+                                             int lane, int j, floatx4_t v) {
+  const long strip_first = (long)strip * p.units_per_strip;
+  const long strip_end = strip_first + p.units_per_strip;
+  if (seg_begin == strip_first && seg_end == strip_end) {
+    const int m = lane & 15;
+    const int nl = 16 * j + 4 * (lane >> 4);
+    if (m < p.size_m) {
+      float b[4] = {0.f, 0.f, 0.f, 0.f};
+      if (p.bias) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+          b[r] = Dq<T>::to_float(p.bias[strip * kStripN + scale_slot(nl + r, false)]);
+      }
+      uint2 o;
+      o.x = (uint32_t)Dq<T>::from_float(v.x + b[0]) | ((uint32_t)Dq<T>::from_float(v.y + b[1]) << 16);
+      o.y = (uint32_t)Dq<T>::from_float(v.z + b[2]) | ((uint32_t)Dq<T>::from_float(v.w + b[3]) << 16);
+      *reinterpret_cast<uint2*>(p.c + (long)m * p.size_n + strip * kStripN + nl) = o;
+    }
+    return;
+  }
+  const int first = range_owner(strip_first, p.total_units, p.parts);
+  partial_slot(p, blockIdx.x, first)[j * 64 + lane] = make_float4(v.x, v.y, v.z, v.w);
+}
+
+// ---------------------------------------------------------------------------
+// General kernel: any M <= 64, any K % 32 == 0, any group size that is a
+// multiple of 32, optional act-order gather of A.  Operands are fetched into
+// registers one unit ahead.
+template <typename T, int MB>
+struct UnitBuf {
+  uint4 q[4];
+  typename Dq<T>::vec8 a[4][MB];
+  uint32_t sbits[4];
+  uint32_t zword;
+  int group;
+};
+
 template <typename T, int MB, bool HAS_ZP, bool HAS_PERM>
-__global__ __launch_bounds__(kThreads) void marlin_stream_kernel(const StreamParams p) {
+__device__ __forceinline__ void load_unit(UnitBuf<T, MB>& b, const StreamParams& p, long u, int lane,
+                                          bool grouped) {
+  const int col16 = lane & 15, kb = lane >> 4;
+  const int strip = (int)(u / p.units_per_strip);
+  const int unit = (int)(u - (long)strip * p.units_per_strip);
+  const int chunk0 = unit * p.unit_chunks;
+  const uint4* bsrc = p.b + ((long)strip * p.chunks_per_strip + chunk0) * 64 + lane;
+#pragma unroll
+  for (int cc = 0; cc < 4; ++cc)
+    if (cc < p.unit_chunks) b.q[cc] = bsrc[cc * 64];
+#pragma unroll
+  for (int cc = 0; cc < 4; ++cc)
+    if (cc < p.unit_chunks) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        b.a[cc][mb] = load_a<T, HAS_PERM>(p, 16 * mb + col16, (chunk0 + cc) * kChunkK + 8 * kb);
+    }
+  const int g = grouped ? (chunk0 * kChunkK) / p.group_size : 0;
+  b.group = g;
+  const uint16_t* srow = p.scales + (long)g * p.size_n + strip * kStripN;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) b.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
+  if (HAS_ZP) b.zword = p.zeros[(long)g * (p.size_n / 8) + strip * 8 + zero_point_word(col16)];
+}
+
+template <typename T, int MB, bool HAS_ZP, bool HAS_PERM>
+__global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const StreamParams p) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq<T>::Col Col;
-  __shared__ float4 red[kWaves / 2][MB * 4][64];
+  __shared__ float4 red[4][MB * 4][64];
 
   const int lane = threadIdx.x & 63;
-  const int wave = threadIdx.x >> 6;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col16 = lane & 15;
-  const int kb = lane >> 4;
-  const long parts = gridDim.x;
-  const long u_begin = range_begin(blockIdx.x, p.total_units, parts);
-  const long u_end = range_begin(blockIdx.x + 1, p.total_units, parts);
+  const long u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
+  const long u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
   const bool grouped = p.num_groups > 1;
+  const uint32_t magic = magic_register();
 
-  long u = u_begin;
-  while (u < u_end) {
-    const int strip = (int)(u / p.units_per_strip);
-    const int unit_a = (int)(u - (long)strip * p.units_per_strip);
-    const long strip_end = (long)(strip + 1) * p.units_per_strip;
+  UnitBuf<T, MB> cur, nxt;
+  long mine = u_begin + wave;
+  if (mine < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM>(cur, p, mine, lane, grouped);
+
+  long seg_begin = u_begin;
+  while (seg_begin < u_end) {
+    const int strip = (int)(seg_begin / p.units_per_strip);
+    const long strip_first = (long)strip * p.units_per_strip;
+    const long strip_end = strip_first + p.units_per_strip;
     const long seg_end = u_end < strip_end ? u_end : strip_end;
-    const int unit_b = unit_a + (int)(seg_end - u);
-    u = seg_end;
 
     floatx4_t acc[MB][4];
 #pragma unroll
@@ -130,115 +261,324 @@ __global__ __launch_bounds__(kThreads) void marlin_stream_kernel(const StreamPar
 #pragma unroll
       for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-    Col cols[4];
-    int cur_group = -1;
-    const uint4* bstrip = p.b + (long)strip * p.chunks_per_strip * 64 + lane;
-
-    for (int unit = unit_a + wave; unit < unit_b; unit += kWaves) {
-      const int chunk0 = unit * p.unit_chunks;
-      uint4 q[4];
-      vec8 av[4][MB];
+    while (mine < seg_end) {
+      const long next = mine + kWaves;
+      if (next < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM>(nxt, p, next, lane, grouped);
+      Col cols[4];
 #pragma unroll
-      for (int cc = 0; cc < 4; ++cc) {
-        if (cc < p.unit_chunks) {
-          q[cc] = bstrip[(long)(chunk0 + cc) * 64];
-#pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
-            av[cc][mb] = load_a<T, HAS_PERM>(p, 16 * mb + col16, (chunk0 + cc) * kChunkK + 8 * kb);
-        }
+      for (int j = 0; j < 4; ++j) {
+        int z = 8;
+        if (HAS_ZP) z = (int)((cur.zword >> zero_point_shift(16 * j + col16)) & 0xFu);
+        cols[j] = Dq<T>::make_col((uint16_t)cur.sbits[j], z);
       }
+      int cur_group = cur.group;
+      const int chunk0 = (int)(mine - strip_first) * p.unit_chunks;
 #pragma unroll
       for (int cc = 0; cc < 4; ++cc) {
         if (cc < p.unit_chunks) {
           const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
-          if (g != cur_group) {
+          if (g != cur_group) {  // groups smaller than a unit
             cur_group = g;
             load_cols<T, HAS_ZP>(cols, p.scales, p.zeros, p.size_n, strip, g, col16, grouped);
           }
-          const uint32_t words[4] = {q[cc].x, q[cc].y, q[cc].z, q[cc].w};
+          const uint32_t words[4] = {cur.q[cc].x, cur.q[cc].y, cur.q[cc].z, cur.q[cc].w};
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const vec8 w = Dq<T>::word(words[j], cols[j]);
+            const vec8 w = Dq<T>::word(words[j], cols[j], magic);
 #pragma unroll
-            for (int mb = 0; mb < MB; ++mb) acc[mb][j] = Dq<T>::mfma(w, av[cc][mb], acc[mb][j]);
+            for (int mb = 0; mb < MB; ++mb) acc[mb][j] = Dq<T>::mfma(w, cur.a[cc][mb], acc[mb][j]);
           }
         }
       }
+      cur = nxt;
+      mine = next;
     }
 
-    // Sum the eight wavefronts' tiles: the upper half of the active set
-    // writes, the lower half adds, three times.
+    reduce_waves<MB, kWaves>(acc, red, wave, lane);
+    if (wave == 0) finish_segment<T, MB>(p, strip, seg_begin, seg_end, lane, acc);
+    seg_begin = seg_end;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Fast kernel for M <= 16, K % 128 == 0, groups of 128 * 2^s rows (or one
+// group), no act-order.  Everything a wavefront consumes arrives in its own
+// region of LDS through asynchronous global->LDS copies, so bytes in flight tie
+// up no vector registers and no register is ever read while a load into it is
+// pending: two slots for the packed weights plus scale / zero-point row of one
+// 128-row unit each (filled two units ahead, HBM latency), one slot for the
+// activation slice of a unit (filled one unit ahead, L2 latency).  The copies of
+// a wavefront complete in issue order, so "the oldest unit has landed" is one
+// counter wait.  The LDS reads that follow, and the LDS traffic of the
+// cross-wavefront reduction, are issued from asm blocks: the compiler cannot
+// tell which LDS bytes an asynchronous copy writes, so before any LDS access
+// it can see it would wait for every outstanding copy, which would drain the
+// prefetch on every unit.
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(1))) const void glb_void_t;
+
+constexpr int kFastWaves = 8;
+constexpr int kSlotS = 4096;       // inside a weight slot, after 4 chunks x 1 KiB: 64 scales, 8 zero-point words
+constexpr int kSlotBytes = 4096 + 256;
+constexpr int kWaveA = 2 * kSlotBytes;            // the activation slot follows the two weight slots
+constexpr int kWaveLds = 2 * kSlotBytes + 4096;   // LDS bytes per wavefront
+constexpr int kWeightCopies = 5;   // asynchronous copies per unit: 4 weight chunks + 1 scale row
+constexpr int kFastLds = kFastWaves * kWaveLds + kFastWaves * 4 * 64 * 16;
+
+struct FastLane {
+  uint32_t a_off;       // byte offset of this lane's 16 bytes inside a 32-column slice of A
+  const char* s_ptr;    // this lane's dword of the scale / zero-point row of (group 0, strip 0)
+  long s_group_stride;  // bytes between groups for s_ptr
+  int s_strip_stride;   // bytes between strips for s_ptr
+};
+
+__device__ __forceinline__ void copy_weights(const StreamParams& p, const FastLane& fl, int strip, int unit,
+                                             char* slot, int lane, int unit_group_shift) {
+  const uint4* gq = p.b + ((long)strip * p.chunks_per_strip + unit * 4) * 64 + lane;
+  lds_void_t* lq = (lds_void_t*)slot;
+  __builtin_amdgcn_global_load_lds((glb_void_t*)gq, lq, 16, 0, 0);
+  __builtin_amdgcn_global_load_lds((glb_void_t*)gq, lq, 16, 1024, 0);
+  __builtin_amdgcn_global_load_lds((glb_void_t*)gq, lq, 16, 2048, 0);
+  __builtin_amdgcn_global_load_lds((glb_void_t*)gq, lq, 16, 3072, 0);
+  const int g = unit_group_shift >= 0 ? (unit >> unit_group_shift) : 0;
+  const char* gs = fl.s_ptr + (long)g * fl.s_group_stride + (long)strip * fl.s_strip_stride;
+  __builtin_amdgcn_global_load_lds((glb_void_t*)gs, (lds_void_t*)(slot + kSlotS), 4, 0, 0);
+}
+
+__device__ __forceinline__ void copy_activations(const StreamParams& p, const FastLane& fl, int unit,
+                                                 char* slot) {
+  const char* ga = reinterpret_cast<const char*>(p.a) + (long)unit * (4 * kChunkK * 2) + fl.a_off;
+  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga), (lds_void_t*)(slot), 16, 0, 0);
+  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 64), (lds_void_t*)(slot + 1024), 16, 0, 0);
+  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 128), (lds_void_t*)(slot + 2048), 16, 0, 0);
+  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 192), (lds_void_t*)(slot + 3072), 16, 0, 0);
+}
+
+struct UnitCursor {
+  long index;
+  int strip, unit;
+  __device__ __forceinline__ void set(long u, int units_per_strip) {
+    index = u;
+    strip = (int)(u / units_per_strip);
+    unit = (int)(u - (long)strip * units_per_strip);
+  }
+  __device__ __forceinline__ void advance(int by, int units_per_strip) {
+    index += by;
+    unit += by;
+    while (unit >= units_per_strip) {
+      unit -= units_per_strip;
+      ++strip;
+    }
+  }
+};
+
+template <typename T, bool HAS_ZP>
+__global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams p,
+                                                                             const int unit_group_shift) {
+  typedef typename Dq<T>::vec8 vec8;
+  typedef typename Dq<T>::Col Col;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int col16 = lane & 15;
+  char* ring = smem + wave * kWaveLds;
+  const uint32_t ring_lds = (uint32_t)(uintptr_t)(lds_void_t*)ring;
+  const uint32_t red_lds = (uint32_t)(uintptr_t)(lds_void_t*)(smem + kFastWaves * kWaveLds);
+  const uint32_t magic = magic_register();
+
+  const long u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
+  const long u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
+  const bool grouped = p.num_groups > 1;
+
+  FastLane fl;
+  {
+    const int row = col16 < p.size_m ? col16 : p.size_m - 1;  // rows past M are never stored
+    fl.a_off = (uint32_t)((long)row * p.lda * 2 + 16 * (lane >> 4));
+    if (HAS_ZP && lane >= 32) {
+      fl.s_ptr = reinterpret_cast<const char*>(p.zeros + (lane & 7));
+      fl.s_group_stride = (long)(p.size_n / 8) * 4;
+      fl.s_strip_stride = 8 * 4;
+    } else {
+      fl.s_ptr = reinterpret_cast<const char*>(p.scales) + 4 * (lane & 31);
+      fl.s_group_stride = (long)p.size_n * 2;
+      fl.s_strip_stride = kStripN * 2;
+    }
+  }
+  // byte offsets, inside a weight slot, of this lane's four scales and its zero-point word
+  uint32_t s_off[4];
 #pragma unroll
-    for (int half = kWaves / 2; half >= 1; half >>= 1) {
-      if (wave >= half && wave < 2 * half) {
+  for (int j = 0; j < 4; ++j) s_off[j] = kSlotS + 2 * scale_slot(16 * j + col16, grouped);
+  const uint32_t z_off = kSlotS + 128 + 4 * zero_point_word(col16);
+
+  // Issue order of a wavefront's copies, x being one of its units and W the
+  // distance to its next one:  weights(x) | A(x), weights(x+W) | A(x+W),
+  // weights(x+2W) | ...  They complete in this order.  When the arithmetic of x
+  // starts, the only copies younger than A(x) are the 5 of weights(x+W), so "at
+  // most 5 outstanding" means weights(x) and A(x) have landed.
+  UnitCursor cur, fetch;
+  cur.set(u_begin + wave, p.units_per_strip);
+  fetch = cur;
+  if (fetch.index < u_end) {
+    copy_weights(p, fl, fetch.strip, fetch.unit, ring, lane, unit_group_shift);
+    copy_activations(p, fl, fetch.unit, ring + kWaveA);
+  }
+  fetch.advance(kFastWaves, p.units_per_strip);
+  if (fetch.index < u_end)
+    copy_weights(p, fl, fetch.strip, fetch.unit, ring + kSlotBytes, lane, unit_group_shift);
+  // `fetch` names the unit whose A slice is copied next; its weights are in flight
+  int c_slot = 0;
+
+  long seg_begin = u_begin;
+  floatx4_t acc[4];
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
+  for (int j = 0; j < 4; ++j) acc[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+  for (;;) {
+    const bool have = cur.index < u_end;
+    // Close every strip segment that ends before this wavefront's next unit:
+    // every wavefront parks its four tiles in LDS, wavefront j (j < 4) adds up
+    // column block j in wavefront order and finishes it.
+    while (seg_begin < u_end) {
+      const int strip = (int)(seg_begin / p.units_per_strip);
+      const long strip_end = (long)(strip + 1) * p.units_per_strip;
+      const long seg_end = u_end < strip_end ? u_end : strip_end;
+      if (have && cur.index < seg_end) break;
+      __builtin_amdgcn_s_barrier();  // the previous segment's tiles have been consumed
+      const uint32_t park = red_lds + (wave * 4 * 64 + lane) * 16;
+      // the tiles come out of the matrix cores; an asm block is opaque to the
+      // compiler's hazard padding, so give the last MFMA time to retire
+      asm volatile(
+          "s_nop 15\n\t"
+          "s_nop 15\n\t"
+          "ds_write_b128 %0, %1\n\t"
+          "ds_write_b128 %0, %2 offset:1024\n\t"
+          "ds_write_b128 %0, %3 offset:2048\n\t"
+          "ds_write_b128 %0, %4 offset:3072\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          :
+          : "v"(park), "v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[3])
+          : "memory");
 #pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const floatx4_t v = acc[mb][j];
-            red[wave - half][mb * 4 + j][lane] = make_float4(v.x, v.y, v.z, v.w);
-          }
+      for (int j = 0; j < 4; ++j) acc[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+      __builtin_amdgcn_s_barrier();
+      if (wave < 4) {
+        floatx4_t sum = floatx4_t{0.f, 0.f, 0.f, 0.f};
+        const uint32_t src = red_lds + (wave * 64 + lane) * 16;
+#pragma unroll
+        for (int w = 0; w < kFastWaves; w += 4) {
+          floatx4_t t0, t1, t2, t3;
+          asm volatile(
+              "ds_read_b128 %0, %4\n\t"
+              "ds_read_b128 %1, %4 offset:4096\n\t"
+              "ds_read_b128 %2, %4 offset:8192\n\t"
+              "ds_read_b128 %3, %4 offset:12288\n\t"
+              "s_waitcnt lgkmcnt(0)"
+              : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
+              : "v"(src + w * 4096)
+              : "memory");
+          sum += t0;
+          sum += t1;
+          sum += t2;
+          sum += t3;
+        }
+        finish_block<T>(p, strip, seg_begin, seg_end, lane, wave, sum);
       }
-      __syncthreads();
-      if (wave < half) {
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-          for (int j = 0; j < 4; ++j) {
-            const float4 v = red[wave][mb * 4 + j][lane];
-            acc[mb][j] += floatx4_t{v.x, v.y, v.z, v.w};
-          }
-      }
-      __syncthreads();
+      seg_begin = seg_end;
+    }
+    if (!have) break;
+
+    // One unit: wait for its copies, pull them into registers, start the
+    // copies of the units after it, then do the arithmetic.
+    const uint32_t slot_lds = ring_lds + c_slot * kSlotBytes;
+    u32x4_t q0, q1, q2, q3, a0, a1, a2, a3;
+    uint32_t sb0, sb1, sb2, sb3, zw;
+    const bool more = cur.index + kFastWaves < u_end;
+    if (more) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightCopies) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    asm volatile(
+        "ds_read_b128 %0, %13\n\t"
+        "ds_read_b128 %1, %13 offset:1024\n\t"
+        "ds_read_b128 %2, %13 offset:2048\n\t"
+        "ds_read_b128 %3, %13 offset:3072\n\t"
+        "ds_read_b128 %4, %14\n\t"
+        "ds_read_b128 %5, %14 offset:1024\n\t"
+        "ds_read_b128 %6, %14 offset:2048\n\t"
+        "ds_read_b128 %7, %14 offset:3072\n\t"
+        "ds_read_u16 %8, %15\n\t"
+        "ds_read_u16 %9, %16\n\t"
+        "ds_read_u16 %10, %17\n\t"
+        "ds_read_u16 %11, %18\n\t"
+        "ds_read_b32 %12, %19\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3), "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3),
+          "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
+        : "v"(slot_lds + lane * 16), "v"(ring_lds + kWaveA + lane * 16), "v"(slot_lds + s_off[0]),
+          "v"(slot_lds + s_off[1]), "v"(slot_lds + s_off[2]), "v"(slot_lds + s_off[3]),
+          "v"(slot_lds + z_off)
+        : "memory");
+    if (more) {
+      copy_activations(p, fl, fetch.unit, ring + kWaveA);
+      fetch.advance(kFastWaves, p.units_per_strip);
+      if (fetch.index < u_end)
+        copy_weights(p, fl, fetch.strip, fetch.unit, ring + c_slot * kSlotBytes, lane, unit_group_shift);
     }
 
-    if (wave != 0) continue;
-    const bool whole = unit_a == 0 && unit_b == p.units_per_strip;
-    if (whole) {
-      write_tiles<T, MB>(p, strip, lane, acc);
-      continue;
+    Col cols[4];
+    const uint32_t sbits[4] = {sb0, sb1, sb2, sb3};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int z = 8;
+      if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
+      cols[j] = Dq<T>::make_col((uint16_t)sbits[j], z);
     }
+    const u32x4_t qs[4] = {q0, q1, q2, q3};
+    const u32x4_t as[4] = {a0, a1, a2, a3};
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) {
+      const vec8 av = __builtin_bit_cast(vec8, as[cc]);
+      const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[j] = Dq<T>::mfma(Dq<T>::word(words[j], cols[j], magic), av, acc[j]);
+    }
+    cur.advance(kFastWaves, p.units_per_strip);
+    c_slot ^= 1;
+  }
+}
 
-    // Partial strip: publish, count, and let the last contributor finish.
-    const long strip_first = (long)strip * p.units_per_strip;
-    const int first = range_owner(strip_first, p.total_units, parts);
-    const int last = range_owner(strip_end - 1, p.total_units, parts);
-    const int me = blockIdx.x;
-    float4* slot = p.scratch + (long)(me == first ? parts + me : me) * kSlotFloat4;
+// ---------------------------------------------------------------------------
+// Second pass over the strips that were split between workgroups: adds the
+// partial tiles in workgroup order and writes C.  One wavefront per strip.
+template <typename T, int MB>
+__global__ __launch_bounds__(64) void marlin_fixup_kernel(const StreamParams p) {
+  const int strip = blockIdx.x;
+  const int lane = threadIdx.x;
+  const long strip_first = (long)strip * p.units_per_strip;
+  const int first = range_owner(strip_first, p.total_units, p.parts);
+  const int last = range_owner(strip_first + p.units_per_strip - 1, p.total_units, p.parts);
+  if (first == last) return;
+  floatx4_t acc[MB][4];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  for (int w = first; w <= last; ++w) {
+    const float4* src = partial_slot(p, w, first);
 #pragma unroll
     for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        const floatx4_t v = acc[mb][j];
-        slot[(mb * 4 + j) * 64 + lane] = make_float4(v.x, v.y, v.z, v.w);
+        const float4 v = src[(mb * 4 + j) * 64 + lane];
+        acc[mb][j] += floatx4_t{v.x, v.y, v.z, v.w};
       }
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");  // partial tile visible before the count
-    int arrived = 0;
-    if (lane == 0)
-      arrived = __hip_atomic_fetch_add(p.workspace + first, 1, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-    arrived = __builtin_amdgcn_readfirstlane(arrived);
-    if (arrived != last - first) continue;
-    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-#pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-    for (int w = first; w <= last; ++w) {
-      const float4* src = p.scratch + (long)(w == first ? parts + w : w) * kSlotFloat4;
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) {
-          const float4 v = src[(mb * 4 + j) * 64 + lane];
-          acc[mb][j] += floatx4_t{v.x, v.y, v.z, v.w};
-        }
-    }
-    write_tiles<T, MB>(p, strip, lane, acc);
-    if (lane == 0) __hip_atomic_store(p.workspace + first, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  write_tiles<T, MB>(p, strip, lane, acc);
 }
 
-// Writes W[K][N]: the values the GEMM kernel feeds to the matrix cores.
+// Writes W[K][N]: the values the GEMM kernels feed to the matrix cores.
 template <typename T, bool HAS_ZP>
 __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __restrict__ b,
                                                             const uint16_t* __restrict__ scales,
@@ -252,6 +592,7 @@ __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __rest
   const int kb = lane >> 4;
   const int chunks_per_strip = size_k / kChunkK;
   const bool grouped = num_groups > 1;
+  const uint32_t magic = magic_register();
   for (long ch = (long)blockIdx.x * 4 + (threadIdx.x >> 6); ch < total_chunks; ch += (long)gridDim.x * 4) {
     const int strip = (int)(ch / chunks_per_strip);
     const int chunk = (int)(ch % chunks_per_strip);
@@ -262,7 +603,7 @@ __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __rest
     const uint32_t words[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const vec8 w = Dq<T>::word(words[j], cols[j]);
+      const vec8 w = Dq<T>::word(words[j], cols[j], magic);
       const uint16_t* bits = reinterpret_cast<const uint16_t*>(&w);
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
@@ -286,21 +627,43 @@ int cu_count() {
 }
 
 template <typename T, int MB, bool HAS_ZP>
-void launch_stream(const StreamParams& p, bool has_perm, int grid, hipStream_t st) {
+void launch_stream(const StreamParams& p, bool has_perm, hipStream_t st) {
   if (has_perm)
-    marlin_stream_kernel<T, MB, HAS_ZP, true><<<grid, kThreads, 0, st>>>(p);
+    marlin_stream_kernel<T, MB, HAS_ZP, true><<<p.parts, kWaves * 64, 0, st>>>(p);
   else
-    marlin_stream_kernel<T, MB, HAS_ZP, false><<<grid, kThreads, 0, st>>>(p);
+    marlin_stream_kernel<T, MB, HAS_ZP, false><<<p.parts, kWaves * 64, 0, st>>>(p);
 }
 
 template <typename T, bool HAS_ZP>
-void launch_stream_mb(const StreamParams& p, bool has_perm, int grid, hipStream_t st) {
-  const int mb = (p.size_m + 15) / 16;
-  switch (mb) {
-    case 1: launch_stream<T, 1, HAS_ZP>(p, has_perm, grid, st); break;
-    case 2: launch_stream<T, 2, HAS_ZP>(p, has_perm, grid, st); break;
-    case 3: launch_stream<T, 3, HAS_ZP>(p, has_perm, grid, st); break;
-    default: launch_stream<T, 4, HAS_ZP>(p, has_perm, grid, st); break;
+void launch_stream_mb(const StreamParams& p, bool has_perm, hipStream_t st) {
+  switch ((p.size_m + 15) / 16) {
+    case 1: launch_stream<T, 1, HAS_ZP>(p, has_perm, st); break;
+    case 2: launch_stream<T, 2, HAS_ZP>(p, has_perm, st); break;
+    case 3: launch_stream<T, 3, HAS_ZP>(p, has_perm, st); break;
+    default: launch_stream<T, 4, HAS_ZP>(p, has_perm, st); break;
+  }
+}
+
+template <typename T, bool HAS_ZP>
+int launch_fast(const StreamParams& p, int unit_group_shift, hipStream_t st) {
+  static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_stream_fast_kernel<T, HAS_ZP>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kFastLds));
+    attr_set = true;
+  }
+  marlin_stream_fast_kernel<T, HAS_ZP><<<p.parts, kFastWaves * 64, kFastLds, st>>>(p, unit_group_shift);
+  return SONAR_OK;
+}
+
+template <typename T>
+void launch_fixup(const StreamParams& p, hipStream_t st) {
+  const int strips = p.size_n / kStripN;
+  switch ((p.size_m + 15) / 16) {
+    case 1: marlin_fixup_kernel<T, 1><<<strips, 64, 0, st>>>(p); break;
+    case 2: marlin_fixup_kernel<T, 2><<<strips, 64, 0, st>>>(p); break;
+    case 3: marlin_fixup_kernel<T, 3><<<strips, 64, 0, st>>>(p); break;
+    default: marlin_fixup_kernel<T, 4><<<strips, 64, 0, st>>>(p); break;
   }
 }
 
@@ -383,6 +746,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   SONAR_REQUIRE(((uintptr_t)c) % 8 == 0 && ((uintptr_t)b_q_weight) % 16 == 0,
                 "c must be 8-byte and b_q_weight 16-byte aligned");
   const int cus = cu_count();
+  // The workspace is not touched (no locks are taken), but a caller that sizes
+  // it wrongly for the reference would fail there, so it fails here too.
   SONAR_REQUIRE(workspace && workspace_len >= cus,
                 "workspace.numel = %ld is below min_workspace_size = %d", (long)workspace_len, cus);
   SONAR_REQUIRE(scratch && scratch_bytes >= sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k),
@@ -393,9 +758,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   p.bias = static_cast<const uint16_t*>(b_bias);
   p.scales = static_cast<const uint16_t*>(b_scales);
   p.zeros = b_zeros;
-  p.g_idx = g_idx;
   p.perm = perm;
-  p.workspace = workspace;
   p.scratch = static_cast<float4*>(scratch);
   p.size_n = (int)size_n;
   p.size_k = (int)size_k;
@@ -406,22 +769,54 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   p.unit_chunks = p.chunks_per_strip % 4 == 0 ? 4 : (p.chunks_per_strip % 2 == 0 ? 2 : 1);
   p.units_per_strip = p.chunks_per_strip / p.unit_chunks;
   p.total_units = (long)(size_n / kStripN) * p.units_per_strip;
-  int grid = cus;
-  if (p.total_units < grid) grid = (int)p.total_units;
+  p.parts = p.total_units < cus ? (int)p.total_units : cus;
   hipStream_t st = (hipStream_t)stream;
+
+  bool any_split = false;
+  for (int i = 1; i < p.parts && !any_split; ++i)
+    any_split = range_begin(i, p.total_units, p.parts) % p.units_per_strip != 0;
+
+  // groups of 128 * 2^s rows: group of a unit = unit >> s
+  int unit_group_shift = -1;
+  bool fast_groups = num_groups == 1;
+  if (num_groups > 1 && chk.group_size % 128 == 0) {
+    const int per = chk.group_size / 128;
+    if ((per & (per - 1)) == 0) {
+      fast_groups = true;
+      unit_group_shift = 0;
+      while ((1 << unit_group_shift) < per) ++unit_group_shift;
+    }
+  }
 
   for (int64_t m0 = 0; m0 < size_m; m0 += 64) {
     p.a = static_cast<const uint16_t*>(a) + m0 * a_row_stride;
     p.c = static_cast<uint16_t*>(c) + m0 * size_n;
     p.size_m = (int)(size_m - m0 < 64 ? size_m - m0 : 64);
-    if (dtype == SONAR_DTYPE_F16) {
-      if (chk.has_zp) launch_stream_mb<_Float16, true>(p, chk.has_perm, grid, st);
-      else launch_stream_mb<_Float16, false>(p, chk.has_perm, grid, st);
+    static const bool no_fast = getenv("SONAR_MARLIN_NO_FAST") != nullptr;  // debugging aid
+    const bool fast = !no_fast && p.size_m <= 16 && !chk.has_perm && p.unit_chunks == 4 && fast_groups &&
+                      (long)p.size_m * a_row_stride * 2 < (1L << 31);
+    if (fast) {
+      int rc;
+      if (dtype == SONAR_DTYPE_F16)
+        rc = chk.has_zp ? launch_fast<_Float16, true>(p, unit_group_shift, st)
+                        : launch_fast<_Float16, false>(p, unit_group_shift, st);
+      else
+        rc = chk.has_zp ? launch_fast<__bf16, true>(p, unit_group_shift, st)
+                        : launch_fast<__bf16, false>(p, unit_group_shift, st);
+      if (rc) return rc;
+    } else if (dtype == SONAR_DTYPE_F16) {
+      if (chk.has_zp) launch_stream_mb<_Float16, true>(p, chk.has_perm, st);
+      else launch_stream_mb<_Float16, false>(p, chk.has_perm, st);
     } else {
-      if (chk.has_zp) launch_stream_mb<__bf16, true>(p, chk.has_perm, grid, st);
-      else launch_stream_mb<__bf16, false>(p, chk.has_perm, grid, st);
+      if (chk.has_zp) launch_stream_mb<__bf16, true>(p, chk.has_perm, st);
+      else launch_stream_mb<__bf16, false>(p, chk.has_perm, st);
     }
     if (int rc = launch_status("marlin_stream_kernel")) return rc;
+    if (any_split) {
+      if (dtype == SONAR_DTYPE_F16) launch_fixup<_Float16>(p, st);
+      else launch_fixup<__bf16>(p, st);
+      if (int rc = launch_status("marlin_fixup_kernel")) return rc;
+    }
   }
   return SONAR_OK;
 }

@@ -1,0 +1,468 @@
+// Torch op registration layer: defines the reference's Marlin op schemas in the
+// `_C` and `_moe_C` namespaces and forwards them to the C ABI of
+// libsonar_marlin.so.  No kernels live here.
+//
+// Schemas follow csrc/libtorch_stable/torch_bindings.cpp:96-115 and
+// csrc/libtorch_stable/moe/torch_bindings.cpp:76-89 of the reference;
+// argument checks follow marlin.cu:626-882, gptq_marlin_repack.cu:289-317,
+// awq_marlin_repack.cu:231-254 and moe/marlin_moe_wna16/ops.cu:630-879.
+//
+// The repack ops return the Marlin tile order bit for bit, because that is
+// what every caller stores.  The gfx950 kernels stream a different order, so
+// the GEMM ops convert a weight tensor the first time they see it and keep the
+// converted copy, keyed by the tensor's address.  The entry also keeps a
+// reference to the source tensor, so its address cannot be handed to another
+// tensor while the entry lives, and remembers the tensor's version counter, so
+// an in-place update triggers a new conversion.
+#include <ATen/ATen.h>
+#include <ATen/hip/HIPContext.h>
+#include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
+#include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
+#include <torch/library.h>
+
+#include <mutex>
+#include <optional>
+#include <unordered_map>
+
+#include "sonar_marlin.h"
+
+namespace {
+
+using at::Tensor;
+using OptTensor = std::optional<Tensor>;
+
+void raise_if_failed(int rc) {
+  if (rc == SONAR_OK) return;
+  const char* msg = sonar_marlin_last_error();
+  if (rc == SONAR_E_UNSUPPORTED) {
+    TORCH_CHECK_NOT_IMPLEMENTED(false, msg);
+  }
+  TORCH_CHECK(false, msg);
+}
+
+void* current_stream(const Tensor& t) {
+  return (void*)c10::hip::getCurrentHIPStreamMasqueradingAsCUDA(t.get_device()).stream();
+}
+
+int dtype_code(const Tensor& a) {
+  if (a.scalar_type() == at::kHalf) return SONAR_DTYPE_F16;
+  if (a.scalar_type() == at::kBFloat16) return SONAR_DTYPE_BF16;
+  TORCH_CHECK_NOT_IMPLEMENTED(
+      false, "unsupported `a` scalar_type: only float16 / bfloat16 activations (W4A16) are built");
+  return -1;
+}
+
+// ---------------------------------------------------------------- weight cache
+struct NativeEntry {
+  Tensor source;
+  Tensor native;
+  int64_t size_k, size_n, experts;
+  uint32_t version;
+};
+
+std::mutex g_cache_mutex;
+std::unordered_map<const void*, NativeEntry> g_cache;
+
+uint32_t version_of(const Tensor& t) { return t.is_inference() ? 0u : t._version(); }
+
+// b_q_weight: (K/16, 2N) or (E, K/16, 2N) int32 in Marlin order.
+Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, int64_t experts) {
+  const void* key = b_q_weight.const_data_ptr();
+  {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    auto it = g_cache.find(key);
+    if (it != g_cache.end() && it->second.size_k == size_k && it->second.size_n == size_n &&
+        it->second.experts == experts && it->second.version == version_of(b_q_weight))
+      return it->second.native;
+  }
+  Tensor native = at::empty_like(b_q_weight);
+  const int64_t words = size_k * size_n / 8;
+  const uint32_t* src = static_cast<const uint32_t*>(b_q_weight.const_data_ptr());
+  uint32_t* dst = static_cast<uint32_t*>(native.mutable_data_ptr());
+  for (int64_t e = 0; e < experts; ++e)
+    raise_if_failed(sonar_marlin_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
+                                           current_stream(b_q_weight)));
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  g_cache[key] = NativeEntry{b_q_weight, native, size_k, size_n, experts, version_of(b_q_weight)};
+  return native;
+}
+
+int64_t marlin_weight_cache_clear() {
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  const int64_t n = (int64_t)g_cache.size();
+  g_cache.clear();
+  return n;
+}
+
+const void* opt_ptr(const OptTensor& t) {
+  return (t.has_value() && t->numel() > 0) ? t->const_data_ptr() : nullptr;
+}
+
+// ---------------------------------------------------------------- repack
+Tensor gptq_marlin_repack(const Tensor& b_q_weight, const Tensor& perm, int64_t size_k,
+                          int64_t size_n, int64_t num_bits, bool is_a_8bit) {
+  TORCH_CHECK_NOT_IMPLEMENTED(!is_a_8bit, "is_a_8bit = True (W4A8) is not built; activations are 16-bit");
+  TORCH_CHECK(num_bits == 4 || num_bits == 8, "num_bits must be 4 or 8. Got = ", num_bits);
+  const int64_t pack_factor = 32 / num_bits;
+  TORCH_CHECK(size_k % 16 == 0, "size_k = ", size_k, " is not divisible by tile_k_size = ", 16);
+  TORCH_CHECK(size_n % 64 == 0, "size_n = ", size_n, " is not divisible by tile_n_size = ", 64);
+  TORCH_CHECK(b_q_weight.dim() == 2 && b_q_weight.size(0) == size_k / pack_factor,
+              "Shape mismatch: b_q_weight.size(0) = ", b_q_weight.size(0), ", size_k = ", size_k,
+              ", pack_factor = ", pack_factor);
+  TORCH_CHECK(b_q_weight.size(1) == size_n, "b_q_weight.size(1) = ", b_q_weight.size(1),
+              " is not size_n = ", size_n);
+  TORCH_CHECK(b_q_weight.is_cuda(), "b_q_weight is not on GPU");
+  TORCH_CHECK(b_q_weight.is_contiguous(), "b_q_weight is not contiguous");
+  TORCH_CHECK(b_q_weight.scalar_type() == at::kInt, "b_q_weight type is not kInt");
+  TORCH_CHECK(perm.is_cuda(), "perm is not on GPU");
+  TORCH_CHECK(perm.is_contiguous(), "perm is not contiguous");
+  TORCH_CHECK(perm.scalar_type() == at::kInt, "perm type is not at::kInt");
+  const bool has_perm = perm.numel() > 0;
+  TORCH_CHECK(!has_perm || perm.numel() == size_k, "perm.numel() = ", perm.numel(),
+              " is not size_k = ", size_k);
+
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(b_q_weight.device());
+  Tensor out = at::empty({size_k / 16, size_n * 16 / pack_factor}, b_q_weight.options());
+  raise_if_failed(sonar_gptq_marlin_repack(
+      static_cast<const uint32_t*>(b_q_weight.const_data_ptr()),
+      has_perm ? static_cast<const int32_t*>(perm.const_data_ptr()) : nullptr,
+      static_cast<uint32_t*>(out.mutable_data_ptr()), size_k, size_n, (int)num_bits,
+      current_stream(b_q_weight)));
+  return out;
+}
+
+Tensor awq_marlin_repack(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, int64_t num_bits,
+                         bool is_a_8bit) {
+  TORCH_CHECK_NOT_IMPLEMENTED(!is_a_8bit, "is_a_8bit = True (W4A8) is not built; activations are 16-bit");
+  TORCH_CHECK(num_bits == 4 || num_bits == 8, "num_bits must be 4 or 8. Got = ", num_bits);
+  const int64_t pack_factor = 32 / num_bits;
+  TORCH_CHECK(size_k % 16 == 0, "size_k = ", size_k, " is not divisible by tile_k_size = ", 16);
+  TORCH_CHECK(size_n % 64 == 0, "size_n = ", size_n, " is not divisible by tile_n_size = ", 64);
+  TORCH_CHECK(b_q_weight.dim() == 2 && b_q_weight.size(0) == size_k,
+              "b_q_weight.size(0) = ", b_q_weight.size(0), " is not size_k = ", size_k);
+  TORCH_CHECK(b_q_weight.size(1) == size_n / pack_factor, "Shape mismatch: b_q_weight.size(1) = ",
+              b_q_weight.size(1), ", size_n = ", size_n, ", pack_factor = ", pack_factor);
+  TORCH_CHECK(b_q_weight.is_cuda(), "b_q_weight is not on GPU");
+  TORCH_CHECK(b_q_weight.is_contiguous(), "b_q_weight is not contiguous");
+  TORCH_CHECK(b_q_weight.scalar_type() == at::kInt, "b_q_weight type is not kInt");
+
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(b_q_weight.device());
+  Tensor out = at::empty({size_k / 16, size_n * 16 / pack_factor}, b_q_weight.options());
+  raise_if_failed(sonar_awq_marlin_repack(static_cast<const uint32_t*>(b_q_weight.const_data_ptr()),
+                                          static_cast<uint32_t*>(out.mutable_data_ptr()), size_k,
+                                          size_n, (int)num_bits, current_stream(b_q_weight)));
+  return out;
+}
+
+Tensor marlin_to_gfx950(const Tensor& b_q_weight, int64_t size_k, int64_t size_n) {
+  TORCH_CHECK(b_q_weight.is_cuda() && b_q_weight.is_contiguous() && b_q_weight.scalar_type() == at::kInt,
+              "b_q_weight must be a contiguous int32 GPU tensor");
+  TORCH_CHECK(b_q_weight.numel() == size_k * size_n / 8, "b_q_weight has ", b_q_weight.numel(),
+              " words, expected ", size_k * size_n / 8);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(b_q_weight.device());
+  Tensor out = at::empty_like(b_q_weight);
+  raise_if_failed(sonar_marlin_to_gfx950(static_cast<const uint32_t*>(b_q_weight.const_data_ptr()),
+                                         static_cast<uint32_t*>(out.mutable_data_ptr()), size_k, size_n,
+                                         current_stream(b_q_weight)));
+  return out;
+}
+
+// ---------------------------------------------------------------- dense GEMM
+void check_b_type(int64_t b_type_id) {
+  TORCH_CHECK_NOT_IMPLEMENTED(
+      b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4,
+      "b_type_id = ", b_type_id,
+      " is not built here: only uint4b8 (GPTQ) and uint4 (AWQ) 4-bit weights are supported");
+}
+
+Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_q_weight,
+                   const OptTensor& b_bias_or_none, const Tensor& b_scales, const OptTensor& a_scales,
+                   const OptTensor& global_scale, const OptTensor& b_zeros_or_none,
+                   const OptTensor& g_idx_or_none, const OptTensor& perm_or_none,
+                   const Tensor& workspace, int64_t b_type_id, int64_t size_m, int64_t size_n,
+                   int64_t size_k, bool is_k_full, bool use_atomic_add, bool use_fp32_reduce,
+                   bool is_zp_float) {
+  const int dtype = dtype_code(a);
+  check_b_type(b_type_id);
+  TORCH_CHECK_NOT_IMPLEMENTED(!a_scales.has_value(), "a_scales can only be used for 8bit activation.");
+  TORCH_CHECK_NOT_IMPLEMENTED(!global_scale.has_value(), "global_scale can only be used for nvfp4 format.");
+  TORCH_CHECK_NOT_IMPLEMENTED(!is_zp_float, "is_zp_float = True is not built");
+
+  TORCH_CHECK(a.dim() == 2, "a must be 2-D");
+  TORCH_CHECK(a.size(0) == size_m, "Shape mismatch: a.size(0) = ", a.size(0), ", size_m = ", size_m);
+  TORCH_CHECK(a.size(1) == size_k, "Shape mismatch: a.size(1) = ", a.size(1), ", size_k = ", size_k);
+  TORCH_CHECK(size_k % 16 == 0, "size_k = ", size_k, " is not divisible by tile_size = ", 16);
+  TORCH_CHECK(b_q_weight.dim() == 2 && size_k / 16 == b_q_weight.size(0),
+              "Shape mismatch: b_q_weight.size(0) = ", b_q_weight.size(0), ", size_k = ", size_k,
+              ", tile_size = ", 16);
+  TORCH_CHECK(b_q_weight.size(1) % 16 == 0, "b_q_weight.size(1) = ", b_q_weight.size(1),
+              " is not divisible by tile_size = ", 16);
+  const int64_t actual_size_n = b_q_weight.size(1) / 16 * 8;
+  TORCH_CHECK(size_n == actual_size_n, "size_n = ", size_n, ", actual_size_n = ", actual_size_n);
+
+  TORCH_CHECK(a.is_cuda(), "A is not on GPU");
+  TORCH_CHECK(size_m == 0 || a.stride(1) == 1, "A.stride(1) is not 1");
+  TORCH_CHECK(size_m == 0 || a.stride(0) % 8 == 0, "A.stride(0) must divisible by 8");
+  TORCH_CHECK(((uint64_t)a.const_data_ptr()) % 16 == 0, "A must aligned to 16 bytes");
+  TORCH_CHECK(b_q_weight.is_cuda(), "b_q_weight is not on GPU");
+  TORCH_CHECK(b_q_weight.is_contiguous(), "b_q_weight is not contiguous");
+  TORCH_CHECK(b_q_weight.scalar_type() == at::kInt, "b_q_weight type is not kInt");
+  TORCH_CHECK(b_scales.is_cuda(), "b_scales is not on GPU");
+  TORCH_CHECK(b_scales.is_contiguous(), "b_scales is not contiguous");
+  TORCH_CHECK(b_scales.scalar_type() == a.scalar_type(),
+              "scalar type of b_scales must be the same as a for 16 bit activation");
+
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
+  Tensor c;
+  if (c_or_none.has_value()) {
+    c = c_or_none.value();
+    TORCH_CHECK(c.is_cuda(), "c is not on GPU");
+    TORCH_CHECK(c.is_contiguous(), "c is not contiguous");
+    TORCH_CHECK(c.size(0) == size_m, "Shape mismatch: c.size(0) = ", c.size(0), ", size_m = ", size_m);
+    TORCH_CHECK(c.size(1) == size_n, "Shape mismatch: c.size(1) = ", c.size(1), ", size_n = ", size_n);
+    TORCH_CHECK(c.scalar_type() == a.scalar_type(),
+                "scalar type of a must be the same with c for 16 bit activation");
+  } else {
+    c = at::empty({size_m, size_n}, a.options());
+  }
+  if (size_m == 0) return c;
+
+  TORCH_CHECK(b_scales.dim() == 2, "b_scales rank = ", b_scales.dim(), " is not 2");
+  TORCH_CHECK(b_scales.size(1) == size_n, "b_scales dim 1 = ", b_scales.size(1), " is not size_n = ", size_n);
+  const int64_t num_groups = b_scales.size(0);
+
+  const int32_t* g_idx = nullptr;
+  const int32_t* perm = nullptr;
+  if (g_idx_or_none.has_value() && perm_or_none.has_value()) {
+    const Tensor& g = g_idx_or_none.value();
+    const Tensor& p = perm_or_none.value();
+    TORCH_CHECK(g.is_cuda(), "g_idx is not on GPU");
+    TORCH_CHECK(g.is_contiguous(), "g_idx is not contiguous");
+    TORCH_CHECK(p.is_cuda(), "perm is not on GPU");
+    TORCH_CHECK(p.is_contiguous(), "perm is not contiguous");
+    TORCH_CHECK((g.size(-1) == 0 && p.size(-1) == 0) || (g.size(-1) == size_k && p.size(-1) == size_k),
+                "Unexpected g_idx.size(-1) = ", g.size(-1), " and perm.size(-1) = ", p.size(-1),
+                ", where size_k = ", size_k);
+    if (g.size(-1) > 0) {
+      TORCH_CHECK(g.scalar_type() == at::kInt && p.scalar_type() == at::kInt, "g_idx and perm must be int32");
+      g_idx = static_cast<const int32_t*>(g.const_data_ptr());
+      perm = static_cast<const int32_t*>(p.const_data_ptr());
+    }
+  }
+
+  if (b_bias_or_none.has_value()) {
+    const Tensor& b = b_bias_or_none.value();
+    TORCH_CHECK(b.is_cuda(), "b_bias is not on GPU");
+    TORCH_CHECK(b.is_contiguous(), "b_bias is not contiguous");
+    TORCH_CHECK(b.size(0) == size_n, "b_bias.size(0) != size_n");
+    TORCH_CHECK(b.stride(0) == 1, "b_bias.stride(0) != 1");
+    TORCH_CHECK(b.scalar_type() == a.scalar_type(), "b_bias must have the dtype of a");
+  }
+
+  const bool has_zp = b_zeros_or_none.has_value() && b_zeros_or_none->size(-1) > 0;
+  if (has_zp) {
+    const Tensor& z = b_zeros_or_none.value();
+    TORCH_CHECK(z.is_cuda(), "b_zeros is not on GPU");
+    TORCH_CHECK(z.is_contiguous(), "b_zeros is not contiguous");
+    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4, "b_type must be u4 or u8 when has_zp = True. Got = uint4b8");
+    TORCH_CHECK(z.dim() == 2, "b_zeros rank = ", z.dim(), " is not 2");
+    TORCH_CHECK(z.size(0) == num_groups, "b_zeros dim 0 = ", z.size(0), " is not num_groups = ", num_groups);
+    TORCH_CHECK(z.size(1) == size_n / 8, "b_zeros dim 1 = ", z.size(1),
+                " is not size_n / pack_factor = ", size_n / 8);
+    TORCH_CHECK(z.scalar_type() == at::kInt, "b_zeros must be int32");
+  } else {
+    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8,
+                "b_type must be uint4b8, uint8b128, int4, int8, float8_e4m3fn or float4_e2m1f when "
+                "has_zp = False. Got = uint4");
+  }
+
+  TORCH_CHECK(size_n % 64 == 0, "size_n = ", size_n, ", is not divisible by min_thread_n = ", 64);
+  TORCH_CHECK(workspace.is_cuda() && workspace.scalar_type() == at::kInt && workspace.is_contiguous(),
+              "workspace must be a contiguous int32 GPU tensor");
+
+  Tensor native = native_weights(b_q_weight, size_k, size_n, 1);
+  const size_t scratch_bytes = sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k);
+  Tensor scratch = at::empty({(int64_t)scratch_bytes}, a.options().dtype(at::kByte));
+
+  raise_if_failed(sonar_marlin_gemm(
+      a.const_data_ptr(), a.stride(0), c.mutable_data_ptr(),
+      static_cast<const uint32_t*>(native.const_data_ptr()), SONAR_LAYOUT_GFX950,
+      opt_ptr(b_bias_or_none), b_scales.const_data_ptr(),
+      has_zp ? static_cast<const uint32_t*>(b_zeros_or_none->const_data_ptr()) : nullptr, g_idx, perm,
+      static_cast<int32_t*>(workspace.mutable_data_ptr()), workspace.numel(), scratch.mutable_data_ptr(),
+      scratch_bytes, dtype, b_type_id, size_m, size_n, size_k, num_groups, is_k_full ? 1 : 0,
+      use_atomic_add ? 1 : 0, use_fp32_reduce ? 1 : 0, current_stream(a)));
+  return c;
+}
+
+// ---------------------------------------------------------------- grouped GEMM
+Tensor moe_wna16_marlin_gemm(
+    Tensor& a, const OptTensor& c_or_none, Tensor& b_q_weight, const OptTensor& b_bias_or_none,
+    Tensor& b_scales, const OptTensor& a_scales, const OptTensor& global_scale,
+    const OptTensor& b_zeros_or_none, const OptTensor& g_idx_or_none, const OptTensor& perm_or_none,
+    Tensor& workspace, const Tensor& sorted_token_ids, Tensor& expert_ids,
+    Tensor& num_tokens_past_padded, Tensor& topk_weights, int64_t moe_block_size, int64_t top_k,
+    bool mul_topk_weights, int64_t b_type_id, int64_t size_m, int64_t size_n, int64_t size_k,
+    bool is_k_full, bool use_atomic_add, bool use_fp32_reduce, bool is_zp_float, int64_t thread_k,
+    int64_t thread_n, int64_t blocks_per_sm) {
+  (void)thread_k;
+  (void)thread_n;
+  (void)blocks_per_sm;
+  const int dtype = dtype_code(a);
+  check_b_type(b_type_id);
+  TORCH_CHECK_NOT_IMPLEMENTED(!a_scales.has_value(), "a_scales can only be used for 8bit activation.");
+  TORCH_CHECK_NOT_IMPLEMENTED(!global_scale.has_value(), "global_scale can only be used for nvfp4 format.");
+  TORCH_CHECK_NOT_IMPLEMENTED(!is_zp_float, "is_zp_float = True is not built");
+  TORCH_CHECK(moe_block_size == 8 || moe_block_size % 16 == 0, "unsupported moe_block_size=", moe_block_size);
+  TORCH_CHECK(moe_block_size >= 8 && moe_block_size <= 64, "unsupported moe_block_size=", moe_block_size);
+
+  TORCH_CHECK(a.dim() == 2 && a.size(0) == size_m, "Shape mismatch: a.size(0) = ", a.size(0),
+              ", size_m = ", size_m);
+  TORCH_CHECK(a.size(1) == size_k, "Shape mismatch: a.size(1) = ", a.size(1), ", size_k = ", size_k);
+  TORCH_CHECK(a.is_cuda() && a.is_contiguous(), "A is not a contiguous GPU tensor");
+  TORCH_CHECK(b_q_weight.dim() == 3, "b_q_weight must be (E, K/16, 2N)");
+  const int64_t experts = b_q_weight.size(0);
+  TORCH_CHECK(size_k % 16 == 0 && size_k / 16 == b_q_weight.size(1),
+              "Shape mismatch: b_q_weight.size(1) = ", b_q_weight.size(1), ", size_k = ", size_k,
+              ", tile_size = ", 16);
+  TORCH_CHECK(b_q_weight.size(2) % 16 == 0 && b_q_weight.size(2) / 16 * 8 == size_n,
+              "size_n = ", size_n, ", actual_size_n = ", b_q_weight.size(2) / 16 * 8);
+  TORCH_CHECK(b_q_weight.is_cuda() && b_q_weight.is_contiguous() && b_q_weight.scalar_type() == at::kInt,
+              "b_q_weight must be a contiguous int32 GPU tensor");
+  TORCH_CHECK(b_scales.is_cuda() && b_scales.is_contiguous(), "b_scales is not a contiguous GPU tensor");
+  TORCH_CHECK(b_scales.dim() == 3 && b_scales.size(0) == experts, "b_scales rank = ", b_scales.dim(), " is not 3");
+  TORCH_CHECK(b_scales.size(2) == size_n, "b_scales dim 2 = ", b_scales.size(2), " is not size_n = ", size_n);
+  TORCH_CHECK(b_scales.scalar_type() == a.scalar_type(), "b_scales must have the dtype of a");
+  const int64_t num_groups = b_scales.size(1);
+
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
+  Tensor c;
+  if (c_or_none.has_value()) {
+    c = c_or_none.value();
+    TORCH_CHECK(c.is_cuda() && c.is_contiguous(), "c is not a contiguous GPU tensor");
+    TORCH_CHECK(c.size(0) == size_m * top_k, "Shape mismatch: c.size(0) = ", c.size(0),
+                ", size_m * topk = ", size_m * top_k);
+    TORCH_CHECK(c.size(1) == size_n, "Shape mismatch: c.size(1) = ", c.size(1), ", size_n = ", size_n);
+    TORCH_CHECK(c.scalar_type() == a.scalar_type(), "c must have the dtype of a");
+  } else {
+    c = at::empty({size_m * top_k, size_n}, a.options());
+  }
+  if (size_m == 0) return c;
+
+  const int32_t* g_idx = nullptr;
+  const int32_t* perm = nullptr;
+  if (g_idx_or_none.has_value() && perm_or_none.has_value() && g_idx_or_none->size(-1) > 0) {
+    const Tensor& g = g_idx_or_none.value();
+    const Tensor& p = perm_or_none.value();
+    TORCH_CHECK(g.is_cuda() && g.is_contiguous() && p.is_cuda() && p.is_contiguous(),
+                "g_idx and perm must be contiguous GPU tensors");
+    TORCH_CHECK(g.size(-1) == size_k && p.size(-1) == size_k, "Unexpected g_idx.size(-1) = ", g.size(-1),
+                " and perm.size(-1) = ", p.size(-1), ", where size_k = ", size_k);
+    TORCH_CHECK(g.scalar_type() == at::kInt && p.scalar_type() == at::kInt, "g_idx and perm must be int32");
+    g_idx = static_cast<const int32_t*>(g.const_data_ptr());
+    perm = static_cast<const int32_t*>(p.const_data_ptr());
+  }
+  if (b_bias_or_none.has_value()) {
+    const Tensor& b = b_bias_or_none.value();
+    TORCH_CHECK(b.is_cuda() && b.is_contiguous(), "b_bias is not a contiguous GPU tensor");
+    TORCH_CHECK(b.size(-1) == size_n, "b_bias.size(-1) != size_n");
+    TORCH_CHECK(b.scalar_type() == a.scalar_type(), "b_bias must have the dtype of a");
+  }
+  const bool has_zp = b_zeros_or_none.has_value() && b_zeros_or_none->size(-1) > 0;
+  if (has_zp) {
+    const Tensor& z = b_zeros_or_none.value();
+    TORCH_CHECK(z.is_cuda() && z.is_contiguous() && z.scalar_type() == at::kInt,
+                "b_zeros must be a contiguous int32 GPU tensor");
+    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4, "b_type must be u4 or u8 when has_zp = True. Got = uint4b8");
+    TORCH_CHECK(z.dim() == 3 && z.size(1) == num_groups && z.size(2) == size_n / 8,
+                "b_zeros must be (E, num_groups, size_n / 8)");
+  } else {
+    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8, "b_type must be uint4b8 when has_zp = False. Got = uint4");
+  }
+  TORCH_CHECK(sorted_token_ids.is_cuda() && sorted_token_ids.scalar_type() == at::kInt &&
+                  sorted_token_ids.is_contiguous(), "sorted_token_ids must be a contiguous int32 GPU tensor");
+  TORCH_CHECK(expert_ids.is_cuda() && expert_ids.scalar_type() == at::kInt && expert_ids.is_contiguous(),
+              "expert_ids must be a contiguous int32 GPU tensor");
+  TORCH_CHECK(num_tokens_past_padded.is_cuda() && num_tokens_past_padded.scalar_type() == at::kInt,
+              "num_tokens_past_padded must be an int32 GPU tensor");
+  TORCH_CHECK(topk_weights.is_cuda() && topk_weights.scalar_type() == at::kFloat &&
+                  topk_weights.is_contiguous(), "topk_weights must be a contiguous float32 GPU tensor");
+  TORCH_CHECK(workspace.is_cuda() && workspace.scalar_type() == at::kInt && workspace.is_contiguous(),
+              "workspace must be a contiguous int32 GPU tensor");
+
+  Tensor native = native_weights(b_q_weight, size_k, size_n, experts);
+  const size_t scratch_bytes =
+      sonar_moe_marlin_gemm_scratch_bytes(sorted_token_ids.numel(), moe_block_size, size_n, size_k);
+  Tensor scratch = at::empty({(int64_t)(scratch_bytes > 16 ? scratch_bytes : 16)}, a.options().dtype(at::kByte));
+
+  raise_if_failed(sonar_moe_wna16_marlin_gemm(
+      a.const_data_ptr(), c.mutable_data_ptr(), static_cast<const uint32_t*>(native.const_data_ptr()),
+      SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none), b_scales.const_data_ptr(),
+      has_zp ? static_cast<const uint32_t*>(b_zeros_or_none->const_data_ptr()) : nullptr, g_idx, perm,
+      static_cast<int32_t*>(workspace.mutable_data_ptr()), workspace.numel(), scratch.mutable_data_ptr(),
+      scratch_bytes, static_cast<const int32_t*>(sorted_token_ids.const_data_ptr()),
+      sorted_token_ids.numel(), static_cast<const int32_t*>(expert_ids.const_data_ptr()),
+      static_cast<const int32_t*>(num_tokens_past_padded.const_data_ptr()),
+      static_cast<const float*>(topk_weights.const_data_ptr()), moe_block_size, top_k,
+      mul_topk_weights ? 1 : 0, experts, dtype, b_type_id, size_m, size_n, size_k, num_groups,
+      is_k_full ? 1 : 0, use_atomic_add ? 1 : 0, use_fp32_reduce ? 1 : 0, current_stream(a)));
+  return c;
+}
+
+}  // namespace
+
+TORCH_LIBRARY_FRAGMENT(_C, m) {
+  m.def(
+      "marlin_gemm(Tensor a, Tensor? c_or_none, Tensor b_q_weight, "
+      "Tensor? b_bias_or_none,Tensor b_scales, "
+      "Tensor? a_scales, Tensor? global_scale, Tensor? b_zeros_or_none, "
+      "Tensor? "
+      "g_idx_or_none, Tensor? perm_or_none, Tensor workspace, int b_type_id, "
+      "SymInt size_m, SymInt size_n, SymInt size_k, bool is_k_full, "
+      "bool use_atomic_add, bool use_fp32_reduce, bool is_zp_float) -> Tensor");
+  // older name of the same op, still used by the reference's benchmark harness
+  m.def(
+      "gptq_marlin_gemm(Tensor a, Tensor? c_or_none, Tensor b_q_weight, "
+      "Tensor? b_bias_or_none,Tensor b_scales, "
+      "Tensor? a_scales, Tensor? global_scale, Tensor? b_zeros_or_none, "
+      "Tensor? "
+      "g_idx_or_none, Tensor? perm_or_none, Tensor workspace, int b_type_id, "
+      "SymInt size_m, SymInt size_n, SymInt size_k, bool is_k_full, "
+      "bool use_atomic_add, bool use_fp32_reduce, bool is_zp_float) -> Tensor");
+  m.def(
+      "gptq_marlin_repack(Tensor b_q_weight, Tensor perm, "
+      "SymInt size_k, SymInt size_n, int num_bits, bool is_a_8bit) -> Tensor");
+  m.def(
+      "awq_marlin_repack(Tensor b_q_weight, SymInt size_k, "
+      "SymInt size_n, int num_bits, bool is_a_8bit) -> Tensor");
+  // not in the reference: Marlin order -> gfx950 streaming order, and cache control
+  m.def("marlin_to_gfx950(Tensor b_q_weight, SymInt size_k, SymInt size_n) -> Tensor");
+  m.def("marlin_weight_cache_clear() -> int", &marlin_weight_cache_clear);
+}
+
+TORCH_LIBRARY_IMPL(_C, CUDA, m) {
+  m.impl("marlin_gemm", &marlin_gemm);
+  m.impl("gptq_marlin_gemm", &marlin_gemm);
+  m.impl("gptq_marlin_repack", &gptq_marlin_repack);
+  m.impl("awq_marlin_repack", &awq_marlin_repack);
+  m.impl("marlin_to_gfx950", &marlin_to_gfx950);
+}
+
+TORCH_LIBRARY_FRAGMENT(_moe_C, m) {
+  m.def(
+      "moe_wna16_marlin_gemm(Tensor! a, Tensor? c_or_none,"
+      "Tensor! b_q_weight, Tensor? b_bias_or_none,"
+      "Tensor! b_scales, Tensor? a_scales, Tensor? global_scale, Tensor? "
+      "b_zeros_or_none,"
+      "Tensor? g_idx_or_none, Tensor? perm_or_none, Tensor! workspace,"
+      "Tensor sorted_token_ids,"
+      "Tensor! expert_ids, Tensor! num_tokens_past_padded,"
+      "Tensor! topk_weights, int moe_block_size, int top_k, "
+      "bool mul_topk_weights, int b_type_id,"
+      "int size_m, int size_n, int size_k,"
+      "bool is_full_k, bool use_atomic_add,"
+      "bool use_fp32_reduce, bool is_zp_float,"
+      "int thread_k, int thread_n, int blocks_per_sm) -> Tensor");
+}
+
+TORCH_LIBRARY_IMPL(_moe_C, CUDA, m) { m.impl("moe_wna16_marlin_gemm", &moe_wna16_marlin_gemm); }

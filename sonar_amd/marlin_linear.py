@@ -1,0 +1,122 @@
+"""Dense caller of the Marlin ops: repack at load, GEMM at apply.  Follows the
+reference's MarlinLinearKernel
+(aphrodite/model_executor/kernels/linear/mixed_precision/marlin.py:35-235) and
+its config (MPLinearKernel.py:26-90), with plain tensors in a namespace-like
+`layer` instead of the reference's parameter classes.
+
+Checkpoint layouts taken (as the reference's GPTQ path provides them,
+layers/quantization/auto_gptq.py:304-430): qweight (K/8, N) int32 packed along
+K, scales (K/G, N), qzeros (N/8-packed per group, given here already unpacked
+to (K/G, N) codes or packed (K/G, N/8) along N), g_idx (K) int32."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+from . import ops
+from .marlin_utils import (MARLIN_SUPPORTED_GROUP_SIZES, apply_gptq_marlin_linear,
+                           check_marlin_supports_shape, marlin_is_k_full, marlin_make_empty_g_idx,
+                           marlin_make_workspace_new, marlin_pad_dim, marlin_pad_qweight,
+                           marlin_pad_scales, marlin_padded_nk, marlin_permute_bias,
+                           marlin_permute_scales, marlin_sort_g_idx, marlin_zero_points,
+                           query_marlin_supported_quant_types, unpack_cols)
+from .scalar_type import ScalarType
+
+
+@dataclass
+class MPLinearLayerConfig:
+    full_weight_shape: tuple[int, int]       # (in_features, out_features)
+    partition_weight_shape: tuple[int, int]
+    weight_type: ScalarType
+    act_type: torch.dtype
+    group_size: int
+    zero_points: bool
+    has_g_idx: bool
+
+
+class MarlinLinearKernel:
+    def __init__(self, c: MPLinearLayerConfig, w_q_param_name: str = "qweight",
+                 w_s_param_name: str = "scales", w_zp_param_name: str | None = "qzeros",
+                 w_gidx_param_name: str | None = "g_idx"):
+        ok, why = self.can_implement(c)
+        if not ok:
+            raise ValueError(why)
+        self.config = c
+        self.w_q_name = w_q_param_name
+        self.w_s_name = w_s_param_name
+        self.w_zp_name = w_zp_param_name or "w_zp"
+        self.w_gidx_name = w_gidx_param_name or "g_idx"
+
+    @classmethod
+    def can_implement(cls, c: MPLinearLayerConfig) -> tuple[bool, str | None]:
+        if c.act_type not in (torch.float16, torch.bfloat16):
+            return False, f"activation type {c.act_type} not supported: fp16 / bf16 only"
+        quant_types = query_marlin_supported_quant_types(c.zero_points)
+        if c.weight_type not in quant_types:
+            return False, (f"Quant type ({c.weight_type}) not supported by  Marlin, supported types "
+                           f"are: {quant_types}")
+        if c.group_size not in MARLIN_SUPPORTED_GROUP_SIZES:
+            return False, (f"Group size ({c.group_size}) not supported by Marlin, supported group "
+                           f"sizes are: {MARLIN_SUPPORTED_GROUP_SIZES}")
+        if c.has_g_idx:
+            return check_marlin_supports_shape(c.partition_weight_shape[1], c.partition_weight_shape[0],
+                                               c.full_weight_shape[0], c.group_size)
+        if (c.group_size != -1 and c.group_size < c.full_weight_shape[0]
+                and c.partition_weight_shape[0] % c.group_size != 0):
+            return False, (f"in_features per partition {c.partition_weight_shape[0]} is not divisible "
+                           f"by group_size = {c.group_size}.")
+        return True, None
+
+    def process_weights_after_loading(self, layer) -> None:
+        c = self.config
+        device = getattr(layer, self.w_q_name).device
+        row_parallel = c.partition_weight_shape[0] != c.full_weight_shape[0]
+        self.is_k_full = marlin_is_k_full(c.has_g_idx, row_parallel)
+        size_k, size_n = c.partition_weight_shape
+        if c.has_g_idx:
+            padded_n, padded_k = size_n, size_k
+        else:
+            padded_n, padded_k = marlin_padded_nk(size_n, size_k, c.group_size)
+        self.workspace = marlin_make_workspace_new(device, existing=getattr(self, "workspace", None))
+
+        if c.has_g_idx:
+            g_idx, g_idx_sort_indices = marlin_sort_g_idx(getattr(layer, self.w_gidx_name))
+            setattr(layer, self.w_gidx_name, g_idx)
+            layer.g_idx_sort_indices = g_idx_sort_indices
+        else:
+            setattr(layer, self.w_gidx_name, marlin_make_empty_g_idx(device))
+            layer.g_idx_sort_indices = marlin_make_empty_g_idx(device)
+
+        if c.zero_points:
+            grouped_k = size_k // c.group_size if c.group_size != -1 else 1
+            padded_grouped_k = padded_k // c.group_size if c.group_size != -1 else 1
+            zp = getattr(layer, self.w_zp_name)
+            if zp.shape == (grouped_k, size_n // 8):
+                zp = unpack_cols(zp, c.weight_type.size_bits, grouped_k, size_n)
+            zp = marlin_pad_scales(zp, size_n, size_k, padded_n, padded_k, c.group_size)
+            setattr(layer, self.w_zp_name,
+                    marlin_zero_points(zp, padded_grouped_k, padded_n, c.weight_type.size_bits))
+        else:
+            setattr(layer, self.w_zp_name, marlin_make_empty_g_idx(device))
+
+        w_q = getattr(layer, self.w_q_name)
+        setattr(layer, self.w_q_name, ops.gptq_marlin_repack(
+            marlin_pad_qweight(w_q.contiguous(), size_n, size_k, padded_n, padded_k),
+            perm=layer.g_idx_sort_indices, size_k=padded_k, size_n=padded_n,
+            num_bits=c.weight_type.size_bits, is_a_8bit=False))
+        w_s = getattr(layer, self.w_s_name)
+        setattr(layer, self.w_s_name, marlin_permute_scales(
+            marlin_pad_scales(w_s.contiguous(), size_n, size_k, padded_n, padded_k, c.group_size),
+            size_k=padded_k, size_n=padded_n, group_size=c.group_size))
+        if getattr(layer, "bias", None) is not None:
+            layer.bias = marlin_permute_bias(marlin_pad_dim(layer.bias, size_n, padded_n))
+
+    def apply_weights(self, layer, x: torch.Tensor, bias: torch.Tensor | None = None) -> torch.Tensor:
+        c = self.config
+        return apply_gptq_marlin_linear(
+            input=x, weight=getattr(layer, self.w_q_name), weight_scale=getattr(layer, self.w_s_name),
+            weight_zp=getattr(layer, self.w_zp_name), g_idx=getattr(layer, self.w_gidx_name),
+            g_idx_sort_indices=layer.g_idx_sort_indices, workspace=self.workspace, wtype=c.weight_type,
+            input_size_per_partition=c.partition_weight_shape[0],
+            output_size_per_partition=c.partition_weight_shape[1], is_k_full=self.is_k_full, bias=bias)

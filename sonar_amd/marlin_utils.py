@@ -1,0 +1,250 @@
+"""Host-side tensor preparation for the Marlin ops: the counterpart of the
+reference's aphrodite/model_executor/layers/quantization/utils/marlin_utils.py
+(:30-40 constants, :206-281 padding, :362-505 workspace / scale / zero-point /
+bias layouts, :636-700 apply_gptq_marlin_linear) and of pack_cols / unpack_cols
+in quant_utils.py:749-803.  Same names, arguments and results; implemented
+with torch index ops so tensors stay on their device."""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import ops
+from .scalar_type import ScalarType, scalar_types
+
+GPTQ_MARLIN_TILE = 16
+GPTQ_MARLIN_MIN_THREAD_N = 64
+GPTQ_MARLIN_MIN_THREAD_K = 128
+GPTQ_MARLIN_MAX_PARALLEL = 16
+MARLIN_SUPPORTED_GROUP_SIZES = [-1, 32, 64, 128]
+USE_FP32_REDUCE_DEFAULT = True
+
+_INTERLEAVE_4BIT = [0, 2, 4, 6, 1, 3, 5, 7]
+
+
+def round_up(x: int, m: int) -> int:
+    return (x + m - 1) // m * m
+
+
+def query_marlin_supported_quant_types(has_zp: bool | None = None, include_fp_type: bool = True):
+    """4-bit integer types only: uint4 with zero points, uint4b8 without."""
+    if has_zp is None:
+        return [scalar_types.uint4, scalar_types.uint4b8]
+    return [scalar_types.uint4] if has_zp else [scalar_types.uint4b8]
+
+
+def check_marlin_supports_shape(output_size_per_partition: int, input_size_per_partition: int,
+                                input_size: int, group_size: int) -> tuple[bool, str | None]:
+    if output_size_per_partition % GPTQ_MARLIN_MIN_THREAD_N != 0:
+        return False, (f"Weight output_size_per_partition = {output_size_per_partition} is not "
+                       f"divisible by  min_thread_n = {GPTQ_MARLIN_MIN_THREAD_N}. ")
+    if input_size_per_partition % GPTQ_MARLIN_MIN_THREAD_K != 0:
+        return False, (f"Weight input_size_per_partition = {input_size_per_partition} is not "
+                       f"divisible by min_thread_k = {GPTQ_MARLIN_MIN_THREAD_K}. ")
+    if group_size < input_size and input_size_per_partition % group_size != 0:
+        return False, (f"Weight input_size_per_partition = {input_size_per_partition} is not "
+                       f"divisible by group_size = {group_size}.")
+    return True, None
+
+
+# ---------------------------------------------------------------- packing
+def get_pack_factor(num_bits: int) -> int:
+    assert 32 % num_bits == 0, f"Unsupported num_bits = {num_bits}"
+    return 32 // num_bits
+
+
+def pack_cols(q_w: torch.Tensor, num_bits: int, size_k: int, size_n: int) -> torch.Tensor:
+    assert q_w.shape == (size_k, size_n)
+    pack_factor = get_pack_factor(num_bits)
+    assert size_n % pack_factor == 0
+    v = q_w.to(torch.int64).reshape(size_k, size_n // pack_factor, pack_factor)
+    shifts = torch.arange(pack_factor, device=q_w.device, dtype=torch.int64) * num_bits
+    packed = (v << shifts).sum(dim=-1)
+    packed = torch.where(packed >= 2 ** 31, packed - 2 ** 32, packed)
+    return packed.to(torch.int32).contiguous()
+
+
+def unpack_cols(packed_q_w: torch.Tensor, num_bits: int, size_k: int, size_n: int) -> torch.Tensor:
+    pack_factor = get_pack_factor(num_bits)
+    assert size_n % pack_factor == 0
+    assert packed_q_w.shape == (size_k, size_n // pack_factor), (
+        f"packed_q_w.shape = {tuple(packed_q_w.shape)} size_k = {size_k}, size_n = {size_n} "
+        f"pack_Factor = {pack_factor}")
+    u = packed_q_w.to(torch.int64) & 0xFFFFFFFF
+    shifts = torch.arange(pack_factor, device=packed_q_w.device, dtype=torch.int64) * num_bits
+    vals = (u.unsqueeze(-1) >> shifts) & ((1 << num_bits) - 1)
+    return vals.reshape(size_k, size_n).to(torch.int32).contiguous()
+
+
+# ---------------------------------------------------------------- padding helpers
+def marlin_padded_nk(size_n: int, size_k: int, group_size: int = -1) -> tuple[int, int]:
+    group = group_size if group_size > 0 else 1
+    candidates = ((round_up(size_n, 64), round_up(size_k, math.lcm(128, group))),
+                  (round_up(size_n, 128), round_up(size_k, math.lcm(64, group))))
+    return min(candidates, key=lambda nk: (nk[0] * nk[1], nk[0] + nk[1]))
+
+
+def marlin_repacked_nk(qweight: torch.Tensor, num_bits: int) -> tuple[int, int]:
+    pack_factor = 32 // num_bits
+    size_k = qweight.size(0) * GPTQ_MARLIN_TILE
+    size_n = qweight.size(1) * pack_factor // GPTQ_MARLIN_TILE
+    return size_n, size_k
+
+
+def marlin_pad_qweight(qweight: torch.Tensor, size_n: int, size_k: int, padded_n: int,
+                       padded_k: int) -> torch.Tensor:
+    if (padded_n, padded_k) == (size_n, size_k):
+        return qweight
+    pack_factor = size_k // qweight.size(0)
+    return torch.nn.functional.pad(qweight, (0, padded_n - size_n, 0, (padded_k - size_k) // pack_factor))
+
+
+def marlin_pad_scales(scales: torch.Tensor, size_n: int, size_k: int, padded_n: int, padded_k: int,
+                      group_size: int) -> torch.Tensor:
+    if (padded_n, padded_k) == (size_n, size_k):
+        return scales
+    pad_rows = padded_k // group_size - scales.size(0) if group_size > 0 else 0
+    assert pad_rows >= 0
+    return torch.nn.functional.pad(scales, (0, padded_n - size_n, 0, pad_rows))
+
+
+def marlin_pad_dim(x: torch.Tensor, size: int, padded: int) -> torch.Tensor:
+    if padded == size:
+        return x
+    return torch.nn.functional.pad(x, (0, padded - size))
+
+
+def marlin_unpad_output(output: torch.Tensor, size_n: int, padded_n: int) -> torch.Tensor:
+    if padded_n == size_n:
+        return output
+    return output[..., :size_n].contiguous()
+
+
+# ---------------------------------------------------------------- workspace, g_idx
+def num_compute_units(device_index: int | None = None) -> int:
+    return torch.cuda.get_device_properties(device_index or 0).multi_processor_count
+
+
+def marlin_make_workspace_new(device: torch.device, max_blocks_per_sm: int = 1,
+                              existing: torch.Tensor | None = None) -> torch.Tensor:
+    size = num_compute_units(device.index) * max_blocks_per_sm
+    if existing is not None:
+        if existing.device != device or existing.dtype != torch.int or existing.numel() != size:
+            raise ValueError(
+                f"Existing Marlin workspace is incompatible (device={existing.device}, "
+                f"dtype={existing.dtype}, numel={existing.numel()}; expected device={device}, "
+                f"dtype={torch.int}, numel={size}).")
+        return existing.zero_()
+    return torch.zeros(size, dtype=torch.int, device=device, requires_grad=False)
+
+
+def marlin_is_k_full(act_order: bool, is_row_parallel: bool) -> bool:
+    return (not act_order) or (act_order and not is_row_parallel)
+
+
+def marlin_repeat_scales_on_all_ranks(act_order: bool, group_size: int, is_row_parallel: bool) -> bool:
+    return act_order or (group_size == -1 and is_row_parallel)
+
+
+def marlin_make_empty_g_idx(device: torch.device) -> torch.Tensor:
+    return torch.nn.Parameter(torch.empty(0, dtype=torch.int, device=device), requires_grad=False)
+
+
+def marlin_sort_g_idx(g_idx: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    g_idx_sort_indices = torch.argsort(g_idx).to(torch.int)
+    return g_idx[g_idx_sort_indices], g_idx_sort_indices
+
+
+# ---------------------------------------------------------------- scale / zp / bias layouts
+def get_scale_perms():
+    scale_perm = [i + 8 * j for i in range(8) for j in range(8)]
+    scale_perm_single = [2 * i + j for i in range(4) for j in (0, 1, 8, 9, 16, 17, 24, 25)]
+    return scale_perm, scale_perm_single
+
+
+def marlin_permute_scales(s: torch.Tensor, size_k: int, size_n: int, group_size: int,
+                          is_a_8bit: bool = False) -> torch.Tensor:
+    assert not is_a_8bit, "8-bit activations are not built"
+    scale_perm, scale_perm_single = get_scale_perms()
+    if group_size < size_k and group_size != -1:
+        s = s.reshape((-1, len(scale_perm)))[:, scale_perm]
+    else:
+        s = s.reshape((-1, len(scale_perm_single)))[:, scale_perm_single]
+    return s.reshape((-1, size_n)).contiguous()
+
+
+def marlin_permute_bias(s: torch.Tensor) -> torch.Tensor:
+    origin_shape = s.shape
+    _, scale_perm_single = get_scale_perms()
+    s = s.reshape((-1, len(scale_perm_single)))[:, scale_perm_single]
+    return s.reshape(*origin_shape).contiguous()
+
+
+def marlin_moe_permute_scales(s: torch.Tensor, size_k: int, size_n: int, group_size: int,
+                              is_a_8bit: bool = False) -> torch.Tensor:
+    output = torch.empty_like(s)
+    for e in range(s.shape[0]):
+        output[e] = marlin_permute_scales(s[e], size_k, size_n, group_size, is_a_8bit)
+    return output
+
+
+def marlin_zero_points(zp: torch.Tensor, size_k: int, size_n: int, num_bits: int,
+                       is_a_8bit: bool = False) -> torch.Tensor:
+    """`size_k` here is the number of groups (rows of zp), as in the reference."""
+    assert num_bits == 4 and not is_a_8bit
+    scale_perm, _ = get_scale_perms()
+    zp = zp.reshape((-1, len(scale_perm)))[:, scale_perm]
+    zp = zp.reshape((-1, 8))[:, _INTERLEAVE_4BIT].reshape((-1, size_n)).contiguous()
+    return pack_cols(zp, num_bits, size_k, size_n)
+
+
+def awq_to_marlin_zero_points(q_zp_packed: torch.Tensor, size_k: int, size_n: int, num_bits: int,
+                              is_a_8bit: bool = False) -> torch.Tensor:
+    assert num_bits == 4
+    q_zp = unpack_cols(q_zp_packed, num_bits, size_k, size_n)
+    undo = sorted(range(8), key=lambda i: _INTERLEAVE_4BIT[i])
+    q_zp = q_zp.reshape((-1, 8))[:, undo].reshape((-1, size_n)).contiguous()
+    return marlin_zero_points(q_zp, size_k, size_n, num_bits, is_a_8bit)
+
+
+def moe_awq_to_marlin_zero_points(q_zp_packed: torch.Tensor, size_k: int, size_n: int, num_bits: int,
+                                  is_a_8bit: bool = False) -> torch.Tensor:
+    output = torch.empty_like(q_zp_packed)
+    for e in range(q_zp_packed.shape[0]):
+        output[e] = awq_to_marlin_zero_points(q_zp_packed[e], size_k, size_n, num_bits, is_a_8bit)
+    return output
+
+
+def should_use_atomic_add_reduce(m: int, n: int, k: int, device: torch.device, dtype: torch.dtype) -> bool:
+    """The reference turns atomic-add reduction on only behind an environment
+    flag for n < 2048, k >= 2048; the gfx950 kernels always reduce in a fixed
+    order, so the answer here is always False."""
+    return False
+
+
+# ---------------------------------------------------------------- the linear call
+def apply_gptq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+                             weight_zp: torch.Tensor, g_idx: torch.Tensor,
+                             g_idx_sort_indices: torch.Tensor, workspace: torch.Tensor,
+                             wtype: ScalarType, output_size_per_partition: int,
+                             input_size_per_partition: int, is_k_full: bool,
+                             input_global_scale: torch.Tensor | None = None,
+                             bias: torch.Tensor | None = None,
+                             use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT,
+                             input_dtype: torch.dtype | None = None) -> torch.Tensor:
+    if input_dtype is not None and input_dtype.itemsize == 1:
+        raise NotImplementedError("8-bit activations (W4A8) are not built")
+    reshaped_x = input.reshape(-1, input.shape[-1])
+    out_shape = input.shape[:-1] + (output_size_per_partition,)
+    padded_n, padded_k = marlin_repacked_nk(weight, wtype.size_bits)
+    reshaped_x = marlin_pad_dim(reshaped_x, input_size_per_partition, padded_k)
+    use_atomic_add = should_use_atomic_add_reduce(reshaped_x.size(0), padded_n, padded_k, input.device,
+                                                  input.dtype)
+    output = ops.marlin_gemm(reshaped_x, None, weight, bias, weight_scale, None, None, weight_zp, g_idx,
+                             g_idx_sort_indices, workspace, wtype, size_m=reshaped_x.shape[0],
+                             size_n=padded_n, size_k=padded_k, is_k_full=is_k_full,
+                             use_atomic_add=use_atomic_add, use_fp32_reduce=use_fp32_reduce,
+                             is_zp_float=False)
+    output = marlin_unpad_output(output, output_size_per_partition, padded_n)
+    return output.reshape(out_shape)

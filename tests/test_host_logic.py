@@ -1,0 +1,173 @@
+"""CPU tests: the C ABI library loads and exports what the header declares,
+the torch ops exist with the reference's schemas, and the host-side tensor
+preparation agrees with the oracle.  No kernel is launched here."""
+import os
+import re
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import marlin_oracle as mo
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_c_abi_exports_every_declared_symbol():
+    from sonar_amd import _lib
+    header = open(os.path.join(ROOT, "include", "sonar_marlin.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(sonar_[a-z0-9_]+)\s*\(", header))
+    assert len(declared) >= 11
+    lib = _lib.load()
+    for name in declared:
+        assert hasattr(lib, name), f"{name} declared in the header but not exported"
+    assert declared == set(_lib.PROTOTYPES), "ctypes prototypes out of step with the header"
+    assert lib.sonar_marlin_version().startswith(b"sonar-marlin-gfx950")
+
+
+def test_type_id_constants_match_header_and_oracle():
+    from sonar_amd import _lib
+    from sonar_amd.scalar_type import scalar_types
+    header = open(os.path.join(ROOT, "include", "sonar_marlin.h")).read()
+    assert int(re.search(r"SONAR_TYPE_UINT4B8 (\d+)LL", header).group(1)) == mo.UINT4B8_ID
+    assert int(re.search(r"SONAR_TYPE_UINT4 (\d+)LL", header).group(1)) == mo.UINT4_ID
+    assert scalar_types.uint4b8.id == mo.UINT4B8_ID == _lib.TYPE_UINT4B8
+    assert scalar_types.uint4.id == mo.UINT4_ID == _lib.TYPE_UINT4
+    assert scalar_types.uint8b128.id == mo.UINT8B128_ID
+    # tests/test_scalartype.py:10-25 of the reference
+    for lo, hi, t in [(-8, 7, scalar_types.int4), (0, 15, scalar_types.uint4),
+                      (-8, 7, scalar_types.uint4b8), (-128, 127, scalar_types.uint8b128),
+                      (-128, 127, scalar_types.int8), (0, 255, scalar_types.uint8)]:
+        assert (t.min(), t.max()) == (lo, hi)
+
+
+def test_torch_ops_have_the_reference_schemas():
+    import sonar_amd.ops  # noqa: F401
+    s = str(torch.ops._C.marlin_gemm.default._schema)
+    assert s == ("_C::marlin_gemm(Tensor a, Tensor? c_or_none, Tensor b_q_weight, Tensor? b_bias_or_none, "
+                 "Tensor b_scales, Tensor? a_scales, Tensor? global_scale, Tensor? b_zeros_or_none, "
+                 "Tensor? g_idx_or_none, Tensor? perm_or_none, Tensor workspace, int b_type_id, "
+                 "SymInt size_m, SymInt size_n, SymInt size_k, bool is_k_full, bool use_atomic_add, "
+                 "bool use_fp32_reduce, bool is_zp_float) -> Tensor")
+    assert str(torch.ops._C.gptq_marlin_gemm.default._schema) == s.replace("marlin_gemm", "gptq_marlin_gemm")
+    assert str(torch.ops._C.gptq_marlin_repack.default._schema) == (
+        "_C::gptq_marlin_repack(Tensor b_q_weight, Tensor perm, SymInt size_k, SymInt size_n, "
+        "int num_bits, bool is_a_8bit) -> Tensor")
+    assert str(torch.ops._C.awq_marlin_repack.default._schema) == (
+        "_C::awq_marlin_repack(Tensor b_q_weight, SymInt size_k, SymInt size_n, int num_bits, "
+        "bool is_a_8bit) -> Tensor")
+    m = str(torch.ops._moe_C.moe_wna16_marlin_gemm.default._schema)
+    assert m.startswith("_moe_C::moe_wna16_marlin_gemm(Tensor($0! -> ) a, Tensor? c_or_none, Tensor($1! -> ) b_q_weight")
+    names = re.findall(r"(\w+)(?:,|\))", m)
+    assert names[:4] == ["a", "c_or_none", "b_q_weight", "b_bias_or_none"] and len(names) == 29
+    assert m.endswith("bool is_zp_float, int thread_k, int thread_n, int blocks_per_sm) -> Tensor")
+
+
+def test_fake_impls_give_reference_shapes():
+    from sonar_amd import ops
+    from sonar_amd.scalar_type import scalar_types
+    meta = dict(device="meta")
+    qw = torch.empty((4096 // 8, 11008), dtype=torch.int32, **meta)
+    out = ops.gptq_marlin_repack(qw, torch.empty(0, dtype=torch.int32, **meta), 4096, 11008, 4)
+    assert out.shape == (256, 22016) and out.dtype == torch.int32
+    aw = torch.empty((4096, 11008 // 8), dtype=torch.int32, **meta)
+    assert ops.awq_marlin_repack(aw, 4096, 11008, 4).shape == (256, 22016)
+    a = torch.empty((7, 4096), dtype=torch.bfloat16, **meta)
+    s = torch.empty((32, 11008), dtype=torch.bfloat16, **meta)
+    ws = torch.empty(256, dtype=torch.int32, **meta)
+    c = ops.marlin_gemm(a, None, out, None, s, None, None, None, None, None, ws, scalar_types.uint4b8,
+                        7, 11008, 4096)
+    assert c.shape == (7, 11008) and c.dtype == torch.bfloat16
+    w3 = torch.empty((8, 256, 57344), dtype=torch.int32, **meta)
+    s3 = torch.empty((8, 32, 28672), dtype=torch.bfloat16, **meta)
+    ids = torch.empty(88, dtype=torch.int32, **meta)
+    c = ops.moe_wna16_marlin_gemm(a, None, w3, None, s3, None, None, None, None, None, ws, ids, ids, ids,
+                                  torch.empty((7, 2), **meta), 8, 2, False, scalar_types.uint4b8, 7, 28672,
+                                  4096, True, False, True, False)
+    assert c.shape == (14, 28672)
+
+
+def test_host_layouts_match_oracle():
+    from sonar_amd import marlin_utils as mu
+    rng = np.random.default_rng(3)
+    k, n, g = 512, 256, 128
+    s = rng.standard_normal((k // g, n)).astype(np.float32)
+    for gs in (g, -1):
+        src = s if gs == g else s[:1]
+        got = mu.marlin_permute_scales(torch.from_numpy(src), k, n, gs).numpy()
+        assert np.array_equal(got, mo.marlin_permute_scales(src, k, n, gs))
+    b = rng.standard_normal(n).astype(np.float32)
+    assert np.array_equal(mu.marlin_permute_bias(torch.from_numpy(b)).numpy(), mo.marlin_permute_bias(b))
+    zp = rng.integers(0, 16, size=(k // g, n), dtype=np.int32)
+    zp[0, :8] = 15  # top nibble of a word set: sign handling
+    got = mu.marlin_zero_points(torch.from_numpy(zp), k // g, n, 4).numpy()
+    assert got.dtype == np.int32 and np.array_equal(got, mo.marlin_zero_points(zp, k // g, n))
+    packed = mu.pack_cols(torch.from_numpy(zp), 4, k // g, n)
+    assert np.array_equal(packed.numpy(), mo.pack_cols(zp))
+    assert np.array_equal(mu.unpack_cols(packed, 4, k // g, n).numpy(), zp)
+    awq = mo.awq_pack(zp)
+    got = mu.awq_to_marlin_zero_points(torch.from_numpy(awq), k // g, n, 4).numpy()
+    assert np.array_equal(got, mo.awq_to_marlin_zero_points(awq, k // g, n))
+    g_idx = torch.from_numpy(rng.permutation(k).astype(np.int32) // g)
+    sorted_g, order = mu.marlin_sort_g_idx(g_idx)
+    assert order.dtype == torch.int32 and torch.equal(sorted_g, g_idx[order.long()])
+    assert bool((sorted_g[1:] >= sorted_g[:-1]).all())
+
+
+ODD = [(1, 1), (65, 129), (200, 208), (100, 300), (4000, 11000)]
+ALIGNED = [(64, 128), (128, 64), (256, 256), (4608, 4096)]
+
+
+def _aligned(n, k):
+    return (n % 64 == 0 and k % 128 == 0) or (n % 128 == 0 and k % 64 == 0)
+
+
+@pytest.mark.parametrize("shape", ODD + ALIGNED)
+@pytest.mark.parametrize("group_size", [-1, 16, 32, 64, 128])
+def test_marlin_padded_nk(shape, group_size):
+    """Same properties the reference checks
+    (tests/kernels/quantization/test_marlin_tile_padding.py:62-100)."""
+    from sonar_amd import marlin_utils as mu
+    size_n, size_k = shape
+    pn, pk = mu.marlin_padded_nk(size_n, size_k, group_size)
+    assert pn >= size_n and pk >= size_k and _aligned(pn, pk)
+    if group_size > 0:
+        assert pk % group_size == 0
+    if _aligned(size_n, size_k) and (group_size <= 0 or size_k % group_size == 0):
+        assert (pn, pk) == (size_n, size_k)
+    if pn * pk <= 300 * 400:
+        for cn in range(size_n, pn + 1):
+            for ck in range(size_k, pk + 1):
+                if _aligned(cn, ck) and (group_size <= 0 or ck % group_size == 0):
+                    assert cn * ck >= pn * pk
+    repacked = torch.empty((pk // 16, pn * 16 // 8), device="meta")
+    assert mu.marlin_repacked_nk(repacked, 4) == (pn, pk)
+
+
+def test_pad_helpers_shapes():
+    from sonar_amd import marlin_utils as mu
+    size_n, size_k, group = 200, 208, 16
+    pn, pk = mu.marlin_padded_nk(size_n, size_k, group)
+    assert mu.marlin_pad_qweight(torch.zeros(size_k // 8, size_n, dtype=torch.int32), size_n, size_k, pn,
+                                 pk).shape == (pk // 8, pn)
+    padded = mu.marlin_pad_scales(torch.ones(size_k // group, size_n), size_n, size_k, pn, pk, group)
+    assert padded.shape == (pk // group, pn) and padded[:, size_n:].abs().sum() == 0
+    assert mu.marlin_pad_scales(torch.ones(1, size_n), size_n, size_k, pn, pk, -1).shape == (1, pn)
+
+
+def test_marlin_linear_kernel_gates():
+    from sonar_amd.marlin_linear import MarlinLinearKernel, MPLinearLayerConfig
+    from sonar_amd.scalar_type import scalar_types as st
+    ok = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4b8, torch.float16, 128, False, False)
+    assert MarlinLinearKernel.can_implement(ok) == (True, None)
+    bad_type = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint8b128, torch.float16, 128, False, False)
+    assert not MarlinLinearKernel.can_implement(bad_type)[0]
+    bad_group = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4b8, torch.float16, 100, False, False)
+    assert not MarlinLinearKernel.can_implement(bad_group)[0]
+    zp_needs_uint4 = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4b8, torch.float16, 128, True, False)
+    assert not MarlinLinearKernel.can_implement(zp_needs_uint4)[0]
+    act_order_odd = MPLinearLayerConfig((4096, 4000), (4096, 4000), st.uint4b8, torch.float16, 128, False, True)
+    assert not MarlinLinearKernel.can_implement(act_order_odd)[0]
+    straddle = MPLinearLayerConfig((4096, 4096), (1000, 4096), st.uint4b8, torch.float16, 128, False, False)
+    assert not MarlinLinearKernel.can_implement(straddle)[0]
