@@ -41,13 +41,16 @@ struct StreamParams {
   int unit_chunks;
   int units_per_strip;
   int parts;  // number of workgroups of the streaming kernel
-  long total_units;
+  int total_units;
 };
 
-__host__ __device__ __forceinline__ long range_begin(long i, long total, long parts) { return i * total / parts; }
+// Unit indices are 32-bit: the host checks total_units * parts < 2^31.
+__host__ __device__ __forceinline__ int range_begin(int i, int total, int parts) {
+  return (int)((unsigned)i * (unsigned)total / (unsigned)parts);
+}
 // Largest i with range_begin(i) <= x, given parts <= total.
-__host__ __device__ __forceinline__ int range_owner(long x, long total, long parts) {
-  return (int)(((x + 1) * parts - 1) / total);
+__host__ __device__ __forceinline__ int range_owner(int x, int total, int parts) {
+  return (int)((((unsigned)x + 1u) * (unsigned)parts - 1u) / (unsigned)total);
 }
 // Scratch slot of workgroup `w` for a strip whose first contributor is `first`.
 __device__ __forceinline__ float4* partial_slot(const StreamParams& p, int w, int first) {
@@ -145,10 +148,10 @@ __device__ __forceinline__ void reduce_waves(floatx4_t (&acc)[MB][4], float4 (*r
 // Wavefront 0: a finished segment goes to C when it is the whole strip, else
 // to this workgroup's scratch slot.
 template <typename T, int MB>
-__device__ __forceinline__ void finish_segment(const StreamParams& p, int strip, long seg_begin, long seg_end,
+__device__ __forceinline__ void finish_segment(const StreamParams& p, int strip, int seg_begin, int seg_end,
                                                int lane, const floatx4_t (&acc)[MB][4]) {
-  const long strip_first = (long)strip * p.units_per_strip;
-  const long strip_end = strip_first + p.units_per_strip;
+  const int strip_first = strip * p.units_per_strip;
+  const int strip_end = strip_first + p.units_per_strip;
   if (seg_begin == strip_first && seg_end == strip_end) {
     write_tiles<T, MB>(p, strip, lane, acc);
     return;
@@ -166,10 +169,10 @@ __device__ __forceinline__ void finish_segment(const StreamParams& p, int strip,
 
 // The same for one 16-column block (j) of a 16-row tile, held by one wavefront.
 template <typename T>
-__device__ __forceinline__ void finish_block(const StreamParams& p, int strip, long seg_begin, long seg_end,
+__device__ __forceinline__ void finish_block(const StreamParams& p, int strip, int seg_begin, int seg_end,
                                              int lane, int j, floatx4_t v) {
-  const long strip_first = (long)strip * p.units_per_strip;
-  const long strip_end = strip_first + p.units_per_strip;
+  const int strip_first = strip * p.units_per_strip;
+  const int strip_end = strip_first + p.units_per_strip;
   if (seg_begin == strip_first && seg_end == strip_end) {
     const int m = lane & 15;
     const int nl = 16 * j + 4 * (lane >> 4);
@@ -205,11 +208,11 @@ struct UnitBuf {
 };
 
 template <typename T, int MB, bool HAS_ZP, bool HAS_PERM>
-__device__ __forceinline__ void load_unit(UnitBuf<T, MB>& b, const StreamParams& p, long u, int lane,
+__device__ __forceinline__ void load_unit(UnitBuf<T, MB>& b, const StreamParams& p, int u, int lane,
                                           bool grouped) {
   const int col16 = lane & 15, kb = lane >> 4;
-  const int strip = (int)(u / p.units_per_strip);
-  const int unit = (int)(u - (long)strip * p.units_per_strip);
+  const int strip = u / p.units_per_strip;
+  const int unit = u - strip * p.units_per_strip;
   const int chunk0 = unit * p.unit_chunks;
   const uint4* bsrc = p.b + ((long)strip * p.chunks_per_strip + chunk0) * 64 + lane;
 #pragma unroll
@@ -239,21 +242,21 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col16 = lane & 15;
-  const long u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
-  const long u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
+  const int u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
+  const int u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
   const bool grouped = p.num_groups > 1;
   const uint32_t magic = magic_register();
 
   UnitBuf<T, MB> cur, nxt;
-  long mine = u_begin + wave;
+  int mine = u_begin + wave;
   if (mine < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM>(cur, p, mine, lane, grouped);
 
-  long seg_begin = u_begin;
+  int seg_begin = u_begin;
   while (seg_begin < u_end) {
-    const int strip = (int)(seg_begin / p.units_per_strip);
-    const long strip_first = (long)strip * p.units_per_strip;
-    const long strip_end = strip_first + p.units_per_strip;
-    const long seg_end = u_end < strip_end ? u_end : strip_end;
+    const int strip = seg_begin / p.units_per_strip;
+    const int strip_first = strip * p.units_per_strip;
+    const int strip_end = strip_first + p.units_per_strip;
+    const int seg_end = u_end < strip_end ? u_end : strip_end;
 
     floatx4_t acc[MB][4];
 #pragma unroll
@@ -262,7 +265,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
       for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
     while (mine < seg_end) {
-      const long next = mine + kWaves;
+      const int next = mine + kWaves;
       if (next < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM>(nxt, p, next, lane, grouped);
       Col cols[4];
 #pragma unroll
@@ -272,7 +275,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
         cols[j] = Dq<T>::make_col((uint16_t)cur.sbits[j], z);
       }
       int cur_group = cur.group;
-      const int chunk0 = (int)(mine - strip_first) * p.unit_chunks;
+      const int chunk0 = (mine - strip_first) * p.unit_chunks;
 #pragma unroll
       for (int cc = 0; cc < 4; ++cc) {
         if (cc < p.unit_chunks) {
@@ -335,7 +338,7 @@ struct FastLane {
 
 __device__ __forceinline__ void copy_weights(const StreamParams& p, const FastLane& fl, int strip, int unit,
                                              char* slot, int lane, int unit_group_shift) {
-  const uint4* gq = p.b + ((long)strip * p.chunks_per_strip + unit * 4) * 64 + lane;
+  const uint4* gq = p.b + (size_t)(unsigned)(strip * p.chunks_per_strip + unit * 4) * 64 + lane;
   lds_void_t* lq = (lds_void_t*)slot;
   __builtin_amdgcn_global_load_lds((glb_void_t*)gq, lq, 16, 0, 0);
   __builtin_amdgcn_global_load_lds((glb_void_t*)gq, lq, 16, 1024, 0);
@@ -356,12 +359,12 @@ __device__ __forceinline__ void copy_activations(const StreamParams& p, const Fa
 }
 
 struct UnitCursor {
-  long index;
+  int index;
   int strip, unit;
-  __device__ __forceinline__ void set(long u, int units_per_strip) {
+  __device__ __forceinline__ void set(int u, int units_per_strip) {
     index = u;
-    strip = (int)(u / units_per_strip);
-    unit = (int)(u - (long)strip * units_per_strip);
+    strip = u / units_per_strip;
+    unit = u - strip * units_per_strip;
   }
   __device__ __forceinline__ void advance(int by, int units_per_strip) {
     index += by;
@@ -387,8 +390,8 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   const uint32_t red_lds = (uint32_t)(uintptr_t)(lds_void_t*)(smem + kFastWaves * kWaveLds);
   const uint32_t magic = magic_register();
 
-  const long u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
-  const long u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
+  const int u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
+  const int u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
   const bool grouped = p.num_groups > 1;
 
   FastLane fl;
@@ -429,7 +432,9 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   // `fetch` names the unit whose A slice is copied next; its weights are in flight
   int c_slot = 0;
 
-  long seg_begin = u_begin;
+  // the current segment starts at seg_begin, inside strip seg_strip
+  int seg_begin = u_begin;
+  int seg_strip = u_begin / p.units_per_strip;
   floatx4_t acc[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) acc[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
@@ -440,9 +445,9 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     // every wavefront parks its four tiles in LDS, wavefront j (j < 4) adds up
     // column block j in wavefront order and finishes it.
     while (seg_begin < u_end) {
-      const int strip = (int)(seg_begin / p.units_per_strip);
-      const long strip_end = (long)(strip + 1) * p.units_per_strip;
-      const long seg_end = u_end < strip_end ? u_end : strip_end;
+      const int strip = seg_strip;
+      const int strip_end = (strip + 1) * p.units_per_strip;
+      const int seg_end = u_end < strip_end ? u_end : strip_end;
       if (have && cur.index < seg_end) break;
       __builtin_amdgcn_s_barrier();  // the previous segment's tiles have been consumed
       const uint32_t park = red_lds + (wave * 4 * 64 + lane) * 16;
@@ -485,6 +490,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
         finish_block<T>(p, strip, seg_begin, seg_end, lane, wave, sum);
       }
       seg_begin = seg_end;
+      ++seg_strip;
     }
     if (!have) break;
 
@@ -556,7 +562,7 @@ template <typename T, int MB>
 __global__ __launch_bounds__(64) void marlin_fixup_kernel(const StreamParams p) {
   const int strip = blockIdx.x;
   const int lane = threadIdx.x;
-  const long strip_first = (long)strip * p.units_per_strip;
+  const int strip_first = strip * p.units_per_strip;
   const int first = range_owner(strip_first, p.total_units, p.parts);
   const int last = range_owner(strip_first + p.units_per_strip - 1, p.total_units, p.parts);
   if (first == last) return;
@@ -768,8 +774,11 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   p.chunks_per_strip = (int)(size_k / kChunkK);
   p.unit_chunks = p.chunks_per_strip % 4 == 0 ? 4 : (p.chunks_per_strip % 2 == 0 ? 2 : 1);
   p.units_per_strip = p.chunks_per_strip / p.unit_chunks;
-  p.total_units = (long)(size_n / kStripN) * p.units_per_strip;
-  p.parts = p.total_units < cus ? (int)p.total_units : cus;
+  const int64_t total_units = (size_n / kStripN) * p.units_per_strip;
+  SONAR_REQUIRE(total_units * cus < (1LL << 31), "size_k * size_n = %ld x %ld is too large", (long)size_k,
+                (long)size_n);
+  p.total_units = (int)total_units;
+  p.parts = p.total_units < cus ? p.total_units : cus;
   hipStream_t st = (hipStream_t)stream;
 
   bool any_split = false;
