@@ -20,6 +20,12 @@
 #include "dequant.hpp"
 
 namespace sonar {
+
+// gemm_tile.hip: the MFMA-bound kernel for more than 64 rows
+int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
+              const void* scales, const uint32_t* zeros, const int32_t* perm, int dtype, int64_t size_m,
+              int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, hipStream_t st);
+
 namespace {
 
 constexpr int kWaves = 8;
@@ -796,6 +802,11 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
       while ((1 << unit_group_shift) < per) ++unit_group_shift;
     }
   }
+
+  static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
+  if (size_m > 64 && size_k % 64 == 0 && !no_tile)
+    return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
+                     size_k, num_groups, chk.group_size, st);
 
   for (int64_t m0 = 0; m0 < size_m; m0 += 64) {
     p.a = static_cast<const uint16_t*>(a) + m0 * a_row_stride;

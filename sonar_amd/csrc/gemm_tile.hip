@@ -1,0 +1,269 @@
+// Tiled W4A16 GEMM for more than 64 activation rows (the MFMA-bound regime).
+//
+// A workgroup of eight wavefronts owns a 256 (rows of A) x 256 (columns of W)
+// tile of C and walks K in steps of 64.  Per step, four wavefronts each fetch
+// one 1-KiB chunk of packed weights per 32 rows (64 columns x 32 rows, already
+// in operand order), dequantise it in registers and store the result to LDS as
+// four 16-column operand blocks; all eight wavefronts fetch the 256 x 64 slice
+// of A and store it to LDS as 16-row operand blocks.  An operand block is 64
+// lanes x 16 bytes: exactly what one v_mfma_f32_16x16x32 reads, so every LDS
+// read of the inner loop is a linear, conflict-free ds_read_b128.  LDS is
+// double-buffered; the global loads of step i+1 are issued before the matrix
+// work of step i and land in registers meanwhile.  Each wavefront computes a
+// 128 x 64 sub-tile: 8 x 4 accumulator tiles, weights as the row operand
+// (D[n][m]) so a lane ends up with four consecutive columns of one row of C.
+//
+// Workgroup ids are dealt so that the 32 workgroups resident on one XCD (ids
+// congruent mod 8) take neighbouring tiles that share weight columns, which
+// keeps the packed weights in that XCD's L2.
+#include "dequant.hpp"
+
+namespace sonar {
+namespace {
+
+constexpr int kTileM = 256;
+constexpr int kTileN = 256;
+constexpr int kTileK = 64;
+constexpr int kTileWaves = 8;
+constexpr int kBlockBytes = 1024;                          // one operand block
+constexpr int kStageA = (kTileM / 16) * (kTileK / 32) * kBlockBytes;  // 32 KiB
+constexpr int kStageB = (kTileN / 16) * (kTileK / 32) * kBlockBytes;  // 32 KiB
+constexpr int kStageBytes = kStageA + kStageB;
+constexpr int kTileLds = 2 * kStageBytes;                  // 128 KiB
+
+struct TileParams {
+  const uint16_t* a;
+  long lda;
+  uint16_t* c;
+  const uint4* b;
+  const uint16_t* bias;
+  const uint16_t* scales;
+  const uint32_t* zeros;
+  const int32_t* perm;
+  int size_m, size_n, size_k;
+  int num_groups, group_size;
+  int chunks_per_strip;
+  int tiles_m, tiles_n;
+};
+
+// 16 bytes (8 consecutive k) of row `row` of A, gathered through perm when given.
+template <bool HAS_PERM>
+__device__ __forceinline__ uint4 load_a16(const TileParams& p, int row, int k0) {
+  const uint16_t* arow = p.a + (long)(row < p.size_m ? row : p.size_m - 1) * p.lda;
+  if (!HAS_PERM) return *reinterpret_cast<const uint4*>(arow + k0);
+  const int4 p0 = *reinterpret_cast<const int4*>(p.perm + k0);
+  const int4 p1 = *reinterpret_cast<const int4*>(p.perm + k0 + 4);
+  uint4 v;
+  v.x = (uint32_t)arow[p0.x] | ((uint32_t)arow[p0.y] << 16);
+  v.y = (uint32_t)arow[p0.z] | ((uint32_t)arow[p0.w] << 16);
+  v.z = (uint32_t)arow[p1.x] | ((uint32_t)arow[p1.y] << 16);
+  v.w = (uint32_t)arow[p1.z] | ((uint32_t)arow[p1.w] << 16);
+  return v;
+}
+
+template <typename T, bool HAS_ZP, bool HAS_PERM>
+__global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const TileParams p) {
+  typedef typename Dq<T>::vec8 vec8;
+  typedef typename Dq<T>::Col Col;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col16 = lane & 15;
+  const int kb = lane >> 4;
+  const uint32_t magic = magic_register();
+  const bool grouped = p.num_groups > 1;
+
+  // XCD-aware tile order: ids congruent mod 8 run on one XCD; give each XCD a
+  // contiguous run of tiles, rows of A innermost so neighbours share weights.
+  const int total = p.tiles_m * p.tiles_n;
+  const int per_xcd = (total + 7) / 8;
+  const int id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  if (id >= total) return;
+  const int tile_n = id / p.tiles_m;
+  const int tile_m = id - tile_n * p.tiles_m;
+  const int m0 = tile_m * kTileM;
+  const int strip0 = tile_n * (kTileN / kStripN);
+  const int strips_here = min(kTileN / kStripN, p.size_n / kStripN - strip0);
+
+  // ---- what this thread fetches per K step
+  // A: the 256 x 64 slice is 32 operand blocks (16 row blocks x 2 k blocks);
+  // thread t fills lane t%64 of blocks t/64 + 8*i, i = 0..3.
+  // W: wavefronts 0..3 each own one strip of the tile and fetch its two chunks.
+  const bool loads_b = wave < strips_here;
+  const uint4* b_src = p.b + (size_t)(unsigned)((strip0 + (loads_b ? wave : 0)) * p.chunks_per_strip) * 64 + lane;
+  const uint16_t* s_src = p.scales + (strip0 + (loads_b ? wave : 0)) * kStripN;
+  const uint32_t* z_src = HAS_ZP ? p.zeros + (strip0 + (loads_b ? wave : 0)) * 8 + zero_point_word(col16) : nullptr;
+  int s_slot[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) s_slot[j] = scale_slot(16 * j + col16, grouped);
+
+  // ---- what this wavefront computes
+  const int wm = wave >> 2;   // rows 128*wm .. +128 of the tile
+  const int wn = wave & 3;    // strip wn of the tile
+  floatx4_t acc[4][8];
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < 8; ++mb) acc[nb][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+  uint4 a_reg[4];
+  uint4 b_reg[2];
+  uint32_t s_reg[2][4];
+  uint32_t z_reg[2];
+
+  auto fetch = [&](int kt) {
+    const int k0 = kt * kTileK;
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int blk = wave + 8 * i;          // 0..31: row block blk>>1, k block blk&1
+      a_reg[i] = load_a16<HAS_PERM>(p, m0 + 16 * (blk >> 1) + col16, k0 + 32 * (blk & 1) + 8 * kb);
+    }
+    if (loads_b) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        const int chunk = kt * 2 + h;
+        b_reg[h] = b_src[(size_t)chunk * 64];
+        const int g = grouped ? (chunk * kChunkK) / p.group_size : 0;
+        const uint16_t* srow = s_src + (long)g * p.size_n;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) s_reg[h][j] = srow[s_slot[j]];
+        if (HAS_ZP) z_reg[h] = z_src[(long)g * (p.size_n / 8)];
+      }
+    }
+  };
+
+  auto stash = [&](int stage) {
+    char* sa = smem + stage * kStageBytes;
+    char* sb = sa + kStageA;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      *reinterpret_cast<uint4*>(sa + (wave + 8 * i) * kBlockBytes + lane * 16) = a_reg[i];
+    if (loads_b) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        Col cols[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          int z = 8;
+          if (HAS_ZP) z = (int)((z_reg[h] >> zero_point_shift(16 * j + col16)) & 0xFu);
+          cols[j] = Dq<T>::make_col((uint16_t)s_reg[h][j], z);
+        }
+        const uint32_t words[4] = {b_reg[h].x, b_reg[h].y, b_reg[h].z, b_reg[h].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const vec8 w = Dq<T>::word(words[j], cols[j], magic);
+          // column block 4*wave + j of the tile, k block h
+          *reinterpret_cast<vec8*>(sb + ((4 * wave + j) * 2 + h) * kBlockBytes + lane * 16) = w;
+        }
+      }
+    }
+  };
+
+  const int k_tiles = p.size_k / kTileK;
+  fetch(0);
+  stash(0);
+  __syncthreads();
+
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    if (kt + 1 < k_tiles) fetch(kt + 1);
+    const char* sa = smem + (kt & 1) * kStageBytes;
+    const char* sb = sa + kStageA;
+    if (wn < strips_here) {
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        vec8 wv[4];
+#pragma unroll
+        for (int nb = 0; nb < 4; ++nb)
+          wv[nb] = *reinterpret_cast<const vec8*>(sb + ((4 * wn + nb) * 2 + h) * kBlockBytes + lane * 16);
+#pragma unroll
+        for (int mb = 0; mb < 8; ++mb) {
+          const vec8 av =
+              *reinterpret_cast<const vec8*>(sa + ((8 * wm + mb) * 2 + h) * kBlockBytes + lane * 16);
+#pragma unroll
+          for (int nb = 0; nb < 4; ++nb) acc[nb][mb] = Dq<T>::mfma(wv[nb], av, acc[nb][mb]);
+        }
+      }
+    }
+    if (kt + 1 < k_tiles) stash((kt + 1) & 1);
+    __syncthreads();
+  }
+
+  // ---- epilogue: lane holds C[m][n .. n+3] for m = row block + lane%16
+  if (wn >= strips_here) return;
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) {
+    const int n = (strip0 + wn) * kStripN + 16 * nb + 4 * kb;
+    float bias[4] = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        bias[r] = Dq<T>::to_float(p.bias[(strip0 + wn) * kStripN + scale_slot(16 * nb + 4 * kb + r, false)]);
+    }
+#pragma unroll
+    for (int mb = 0; mb < 8; ++mb) {
+      const int m = m0 + 128 * wm + 16 * mb + col16;
+      if (m < p.size_m) {
+        const floatx4_t v = acc[nb][mb];
+        uint2 o;
+        o.x = (uint32_t)Dq<T>::from_float(v.x + bias[0]) | ((uint32_t)Dq<T>::from_float(v.y + bias[1]) << 16);
+        o.y = (uint32_t)Dq<T>::from_float(v.z + bias[2]) | ((uint32_t)Dq<T>::from_float(v.w + bias[3]) << 16);
+        *reinterpret_cast<uint2*>(p.c + (long)m * p.size_n + n) = o;
+      }
+    }
+  }
+}
+
+template <typename T, bool HAS_ZP, bool HAS_PERM>
+int launch_tile(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_kernel<T, HAS_ZP, HAS_PERM>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kTileLds));
+    attr_set = true;
+  }
+  const int total = p.tiles_m * p.tiles_n;
+  const int grid = ((total + 7) / 8) * 8;
+  marlin_tile_kernel<T, HAS_ZP, HAS_PERM><<<grid, kTileWaves * 64, kTileLds, st>>>(p);
+  return SONAR_OK;
+}
+
+}  // namespace
+
+// Called by sonar_marlin_gemm for size_m > 64.  Shapes and pointers have been
+// validated by the caller; size_k % 64 == 0 is required here.
+int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
+              const void* scales, const uint32_t* zeros, const int32_t* perm, int dtype, int64_t size_m,
+              int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, hipStream_t st) {
+  TileParams p;
+  p.a = static_cast<const uint16_t*>(a);
+  p.lda = a_row_stride;
+  p.c = static_cast<uint16_t*>(c);
+  p.b = reinterpret_cast<const uint4*>(b);
+  p.bias = static_cast<const uint16_t*>(bias);
+  p.scales = static_cast<const uint16_t*>(scales);
+  p.zeros = zeros;
+  p.perm = perm;
+  p.size_m = (int)size_m;
+  p.size_n = (int)size_n;
+  p.size_k = (int)size_k;
+  p.num_groups = (int)num_groups;
+  p.group_size = group_size;
+  p.chunks_per_strip = (int)(size_k / kChunkK);
+  p.tiles_m = (int)((size_m + kTileM - 1) / kTileM);
+  p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);
+  const bool zp = zeros != nullptr, pm = perm != nullptr;
+  int rc;
+  if (dtype == SONAR_DTYPE_F16) {
+    rc = zp ? (pm ? launch_tile<_Float16, true, true>(p, st) : launch_tile<_Float16, true, false>(p, st))
+            : (pm ? launch_tile<_Float16, false, true>(p, st) : launch_tile<_Float16, false, false>(p, st));
+  } else {
+    rc = zp ? (pm ? launch_tile<__bf16, true, true>(p, st) : launch_tile<__bf16, true, false>(p, st))
+            : (pm ? launch_tile<__bf16, false, true>(p, st) : launch_tile<__bf16, false, false>(p, st));
+  }
+  if (rc) return rc;
+  return launch_status("marlin_tile_kernel");
+}
+
+}  // namespace sonar

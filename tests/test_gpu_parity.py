@@ -174,3 +174,30 @@ def test_error_paths(gu):
     layer.workspace = torch.zeros(4, dtype=torch.int32, device=gu.DEV)
     with pytest.raises(_lib.SonarMarlinError, match="workspace"):
         layer.gemm(a, 1)
+
+
+TILE_CASES = [
+    # m, k, n, group, zp, act_order, bias   (more than 64 rows: the MFMA-tiled kernel)
+    (65, 512, 256, 128, False, False, False),
+    (256, 4096, 4096, 128, False, False, False),
+    (257, 1280, 320, 128, False, False, True),
+    (300, 1024, 448, 32, True, False, False),
+    (512, 4096, 11008, 128, False, True, False),     # act-order, benchmark config 4
+    (512, 4096, 11008, 128, True, False, False),     # AWQ, benchmark config 4
+    (1000, 2048, 64, -1, False, False, True),
+    (129, 14336, 4096, 128, False, False, False),
+]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("m,k,n,g,zp,act,bias", TILE_CASES)
+def test_marlin_gemm_tiled_within_tolerance(gu, dtype, m, k, n, g, zp, act, bias):
+    layer = gu.DeviceLayer(31 + m, k, n, g, dtype, zero_points=zp, act_order=act, bias=bias)
+    a32 = mo.make_activations(m * 3 + 1, m, k, dtype, std=0.5)
+    a = gu.dev_bits16(a32, dtype)
+    c = layer.gemm(a, m)
+    ref = mo.gemm_reference(a32, layer.w_ref, layer.bias32)
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), ref)
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+    c2 = layer.gemm(a, m)
+    assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
