@@ -1,12 +1,243 @@
-// Grouped (mixture-of-experts) W4A16 GEMM entry points.
+// Grouped (mixture-of-experts) W4A16 GEMM for gfx950.
+//
+// moe_align_block_size hands the kernel blocks of `moe_block_size` slots, all
+// of one expert; slot id < M * top_k stands for row id of C and row id / top_k
+// of A (csrc/libtorch_stable/moe/marlin_moe_wna16/marlin_template.h:471-570).
+// One workgroup owns one (block, 64-column strip) pair: its eight wavefronts
+// split the strip's 128-row units of the block's expert between them, keep
+// the next unit's operands in flight in registers, sum their accumulators
+// through LDS and wavefront 0 scatters the rows to C, multiplied by the
+// routing weight when asked (marlin_template.h:1883-1909).  K is never split
+// across workgroups, so nothing is reduced through memory and results do not
+// depend on the launch: scratch and workspace are not used.
 #include "common.hpp"
+#include "dequant.hpp"
+#include "wave_reduce.hpp"
+
+namespace sonar {
+namespace {
+
+constexpr int kMoeWaves = 8;
+
+struct MoeParams {
+  const uint16_t* a;
+  uint16_t* c;
+  const uint4* b;
+  const uint16_t* bias;
+  const uint16_t* scales;
+  const uint32_t* zeros;
+  const int32_t* perm;
+  const int32_t* sorted_ids;
+  const int32_t* expert_ids;
+  const int32_t* num_post_pad;
+  const float* topk_weights;
+  int size_m, size_n, size_k;
+  int num_groups, group_size;
+  int chunks_per_strip, unit_chunks, units_per_strip;
+  int strips;
+  int block_size, top_k, num_experts, num_blocks;
+  int sorted_len;
+  int mul_topk;
+};
+
+template <typename T, bool HAS_PERM>
+__device__ __forceinline__ typename Dq<T>::vec8 moe_load_a(const uint16_t* arow, const int32_t* perm, int k0) {
+  typedef typename Dq<T>::vec8 vec8;
+  uint4 v;
+  if (!HAS_PERM) {
+    v = *reinterpret_cast<const uint4*>(arow + k0);
+  } else {
+    const int4 p0 = *reinterpret_cast<const int4*>(perm + k0);
+    const int4 p1 = *reinterpret_cast<const int4*>(perm + k0 + 4);
+    v.x = (uint32_t)arow[p0.x] | ((uint32_t)arow[p0.y] << 16);
+    v.y = (uint32_t)arow[p0.z] | ((uint32_t)arow[p0.w] << 16);
+    v.z = (uint32_t)arow[p1.x] | ((uint32_t)arow[p1.y] << 16);
+    v.w = (uint32_t)arow[p1.z] | ((uint32_t)arow[p1.w] << 16);
+  }
+  return __builtin_bit_cast(vec8, v);
+}
+
+template <typename T, int MB>
+struct MoeUnit {
+  uint4 q[4];
+  typename Dq<T>::vec8 a[4][MB];
+  uint32_t sbits[4];
+  uint32_t zword;
+  int group;
+};
+
+template <typename T, int MB, bool HAS_ZP, bool HAS_PERM>
+__global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoeParams p) {
+  typedef typename Dq<T>::vec8 vec8;
+  typedef typename Dq<T>::Col Col;
+  __shared__ float4 red[4][MB * 4][64];
+  __shared__ int slot_id[16 * MB];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int col16 = lane & 15, kb = lane >> 4;
+  const int block = blockIdx.x / p.strips;
+  const int strip = blockIdx.x - block * p.strips;
+
+  // the whole workgroup leaves together: nothing below is reached by a part of it
+  const int past = p.num_post_pad[0];
+  if (block * p.block_size >= past) return;
+  const int expert = p.expert_ids[block];
+  if (expert < 0 || expert >= p.num_experts) return;
+
+  const int rows_total = p.size_m * p.top_k;
+  if (threadIdx.x < 16 * MB) {
+    int id = -1;
+    const int at = block * p.block_size + (int)threadIdx.x;
+    if ((int)threadIdx.x < p.block_size && at < p.sorted_len) {
+      id = p.sorted_ids[at];
+      if (id < 0 || id >= rows_total) id = -1;
+    }
+    slot_id[threadIdx.x] = id;
+  }
+  __syncthreads();
+
+  const uint16_t* arow[MB];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int id = slot_id[16 * mb + col16];
+    // padding slots read row 0; their products are never stored
+    arow[mb] = p.a + (long)(id >= 0 ? id / p.top_k : 0) * p.size_k;
+  }
+  const long expert_l = expert;
+  const uint4* bsrc = p.b + (expert_l * p.strips + strip) * (long)p.chunks_per_strip * 64 + lane;
+  const uint16_t* scales = p.scales + expert_l * p.num_groups * p.size_n;
+  const uint32_t* zeros = HAS_ZP ? p.zeros + expert_l * p.num_groups * (p.size_n / 8) : nullptr;
+  const int32_t* perm = HAS_PERM ? p.perm + expert_l * p.size_k : nullptr;
+  const bool grouped = p.num_groups > 1;
+  const uint32_t magic = magic_register();
+
+  auto load_unit = [&](MoeUnit<T, MB>& u, int unit) {
+    const int chunk0 = unit * p.unit_chunks;
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc)
+      if (cc < p.unit_chunks) u.q[cc] = bsrc[(long)(chunk0 + cc) * 64];
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc)
+      if (cc < p.unit_chunks) {
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          u.a[cc][mb] = moe_load_a<T, HAS_PERM>(arow[mb], perm, (chunk0 + cc) * kChunkK + 8 * kb);
+      }
+    const int g = grouped ? (chunk0 * kChunkK) / p.group_size : 0;
+    u.group = g;
+    const uint16_t* srow = scales + (long)g * p.size_n + strip * kStripN;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) u.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
+    if (HAS_ZP) u.zword = zeros[(long)g * (p.size_n / 8) + strip * 8 + zero_point_word(col16)];
+  };
+
+  floatx4_t acc[MB][4];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+  MoeUnit<T, MB> cur, nxt;
+  int mine = wave;
+  if (mine < p.units_per_strip) load_unit(cur, mine);
+  while (mine < p.units_per_strip) {
+    const int next = mine + kMoeWaves;
+    if (next < p.units_per_strip) load_unit(nxt, next);
+    Col cols[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int z = 8;
+      if (HAS_ZP) z = (int)((cur.zword >> zero_point_shift(16 * j + col16)) & 0xFu);
+      cols[j] = Dq<T>::make_col((uint16_t)cur.sbits[j], z);
+    }
+    int cur_group = cur.group;
+    const int chunk0 = mine * p.unit_chunks;
+#pragma unroll
+    for (int cc = 0; cc < 4; ++cc) {
+      if (cc < p.unit_chunks) {
+        const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
+        if (g != cur_group) {  // groups smaller than a unit
+          cur_group = g;
+          load_cols<T, HAS_ZP>(cols, scales, zeros, p.size_n, strip, g, col16, grouped);
+        }
+        const uint32_t words[4] = {cur.q[cc].x, cur.q[cc].y, cur.q[cc].z, cur.q[cc].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const vec8 w = Dq<T>::word(words[j], cols[j], magic);
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) acc[mb][j] = Dq<T>::mfma(w, cur.a[cc][mb], acc[mb][j]);
+        }
+      }
+    }
+    cur = nxt;
+    mine = next;
+  }
+
+  reduce_waves<MB, kMoeWaves>(acc, red, wave, lane);
+  if (wave != 0) return;
+
+  const uint16_t* bias = p.bias ? p.bias + expert_l * p.size_n + strip * kStripN : nullptr;
+  const int n_in = 4 * (lane >> 4);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int id = slot_id[16 * mb + col16];
+    if (id < 0) continue;
+    float tw = 1.f;
+    // the routing weight is rounded to the activation type and the product is
+    // formed and rounded in that type (marlin_template.h:1893-1897)
+    if (p.mul_topk) tw = Dq<T>::to_float(Dq<T>::from_float(p.topk_weights[id]));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int nl = 16 * j + n_in;
+      const floatx4_t v = acc[mb][j];
+      float r[4] = {v.x, v.y, v.z, v.w};
+      uint16_t o[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        float x = r[t];
+        if (bias) x += Dq<T>::to_float(bias[scale_slot(nl + t, false)]);
+        o[t] = Dq<T>::from_float(x);
+        if (p.mul_topk) o[t] = Dq<T>::from_float(Dq<T>::to_float(o[t]) * tw);
+      }
+      uint2 packed;
+      packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+      packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+      *reinterpret_cast<uint2*>(p.c + (long)id * p.size_n + strip * kStripN + nl) = packed;
+    }
+  }
+}
+
+template <typename T, int MB, bool HAS_ZP>
+void launch_moe(const MoeParams& p, bool has_perm, int grid, hipStream_t st) {
+  if (has_perm)
+    marlin_moe_kernel<T, MB, HAS_ZP, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  else
+    marlin_moe_kernel<T, MB, HAS_ZP, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
+}
+
+template <typename T, bool HAS_ZP>
+void launch_moe_mb(const MoeParams& p, bool has_perm, int grid, hipStream_t st) {
+  switch ((p.block_size + 15) / 16) {
+    case 1: launch_moe<T, 1, HAS_ZP>(p, has_perm, grid, st); break;
+    case 2: launch_moe<T, 2, HAS_ZP>(p, has_perm, grid, st); break;
+    case 3: launch_moe<T, 3, HAS_ZP>(p, has_perm, grid, st); break;
+    default: launch_moe<T, 4, HAS_ZP>(p, has_perm, grid, st); break;
+  }
+}
+
+}  // namespace
+}  // namespace sonar
 
 using namespace sonar;
 
 extern "C" size_t sonar_moe_marlin_gemm_scratch_bytes(int64_t sorted_len, int64_t moe_block_size,
                                                       int64_t size_n, int64_t size_k) {
-  (void)sorted_len; (void)moe_block_size; (void)size_n; (void)size_k;
-  return 0;
+  (void)sorted_len;
+  (void)moe_block_size;
+  (void)size_n;
+  (void)size_k;
+  return 0;  // K is not split across workgroups: no partial sums leave the chip
 }
 
 extern "C" int sonar_moe_wna16_marlin_gemm(
@@ -18,5 +249,97 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     int64_t top_k, int mul_topk_weights, int64_t num_experts, int dtype, int64_t b_type_id,
     int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int is_k_full,
     int use_atomic_add, int use_fp32_reduce, void* stream) {
-  return fail(SONAR_E_UNSUPPORTED, "moe_wna16_marlin_gemm is not built yet");
+  (void)workspace;
+  (void)workspace_len;
+  (void)scratch;
+  (void)scratch_bytes;
+  (void)use_atomic_add;
+  (void)use_fp32_reduce;
+  SONAR_REQUIRE(b_layout == SONAR_LAYOUT_GFX950, "unknown b_layout = %d", b_layout);
+  SONAR_REQUIRE(dtype == SONAR_DTYPE_F16 || dtype == SONAR_DTYPE_BF16, "unsupported `a` scalar_type");
+  // marlin_moe_wna16/ops.cu:560-566
+  SONAR_REQUIRE(moe_block_size == 8 || (moe_block_size > 0 && moe_block_size % 16 == 0 && moe_block_size <= 64),
+                "unsupported moe_block_size=%ld", (long)moe_block_size);
+  SONAR_REQUIRE(top_k >= 1 && num_experts >= 1, "top_k = %ld and num_experts = %ld must be >= 1",
+                (long)top_k, (long)num_experts);
+  SONAR_REQUIRE(size_m >= 0 && size_m * top_k < (1LL << 30), "size_m = %ld out of range", (long)size_m);
+  SONAR_REQUIRE(size_k > 0 && size_k % kChunkK == 0 && size_k < (1LL << 30),
+                "size_k = %ld is not divisible by %d", (long)size_k, kChunkK);
+  SONAR_REQUIRE(size_n > 0 && size_n % kStripN == 0 && size_n < (1LL << 30),
+                "size_n = %ld, is not divisible by min_thread_n = %d", (long)size_n, kStripN);
+  SONAR_REQUIRE(b_scales != nullptr, "b_scales must not be NULL");
+  SONAR_REQUIRE(num_groups >= 1, "num_groups = %ld must be >= 1", (long)num_groups);
+  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4)
+    return fail(SONAR_E_UNSUPPORTED,
+                "b_type id %ld is not built here: only uint4b8 (GPTQ) and uint4 (AWQ) weights are",
+                (long)b_type_id);
+  const bool has_zp = b_zeros != nullptr;
+  if (has_zp)
+    SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4, "b_type must be u4 or u8 when has_zp = True");
+  else
+    SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4B8,
+                  "b_type must be uint4b8 when has_zp = False (uint4 needs b_zeros)");
+  SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
+  const bool has_perm = perm != nullptr;
+  if (has_perm) {
+    if (!is_k_full)
+      return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False is not built yet");
+    SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
+  }
+  int group_size = (int)size_k;
+  if (num_groups > 1) {
+    SONAR_REQUIRE(size_k % num_groups == 0, "size_k = %ld, is not divisible by num_groups = %ld",
+                  (long)size_k, (long)num_groups);
+    group_size = (int)(size_k / num_groups);
+    SONAR_REQUIRE(group_size % kChunkK == 0, "group_size = %d must be a multiple of %d", group_size,
+                  kChunkK);
+  }
+  if (size_m == 0 || sorted_len == 0) return SONAR_OK;
+  SONAR_REQUIRE(a && c && b_q_weight, "a, c and b_q_weight must not be NULL");
+  SONAR_REQUIRE(sorted_token_ids && expert_ids && num_tokens_past_padded,
+                "sorted_token_ids, expert_ids and num_tokens_past_padded must not be NULL");
+  SONAR_REQUIRE(!mul_topk_weights || topk_weights, "topk_weights must be given when mul_topk_weights is set");
+  SONAR_REQUIRE(((uintptr_t)a) % 16 == 0 && ((uintptr_t)c) % 8 == 0 && ((uintptr_t)b_q_weight) % 16 == 0,
+                "a and b_q_weight must be 16-byte and c 8-byte aligned");
+  SONAR_REQUIRE(sorted_len > 0 && sorted_len < (1LL << 30), "sorted_token_ids.numel = %ld out of range",
+                (long)sorted_len);
+
+  MoeParams p;
+  p.a = static_cast<const uint16_t*>(a);
+  p.c = static_cast<uint16_t*>(c);
+  p.b = reinterpret_cast<const uint4*>(b_q_weight);
+  p.bias = static_cast<const uint16_t*>(b_bias);
+  p.scales = static_cast<const uint16_t*>(b_scales);
+  p.zeros = b_zeros;
+  p.perm = perm;
+  p.sorted_ids = sorted_token_ids;
+  p.expert_ids = expert_ids;
+  p.num_post_pad = num_tokens_past_padded;
+  p.topk_weights = topk_weights;
+  p.size_m = (int)size_m;
+  p.size_n = (int)size_n;
+  p.size_k = (int)size_k;
+  p.num_groups = (int)num_groups;
+  p.group_size = group_size;
+  p.chunks_per_strip = (int)(size_k / kChunkK);
+  p.unit_chunks = p.chunks_per_strip % 4 == 0 ? 4 : (p.chunks_per_strip % 2 == 0 ? 2 : 1);
+  p.units_per_strip = p.chunks_per_strip / p.unit_chunks;
+  p.strips = (int)(size_n / kStripN);
+  p.block_size = (int)moe_block_size;
+  p.top_k = (int)top_k;
+  p.num_experts = (int)num_experts;
+  p.sorted_len = (int)sorted_len;
+  p.num_blocks = (int)((sorted_len + moe_block_size - 1) / moe_block_size);
+  p.mul_topk = mul_topk_weights ? 1 : 0;
+  const int64_t grid = (int64_t)p.num_blocks * p.strips;
+  SONAR_REQUIRE(grid < (1LL << 31), "too many (block, strip) pairs: %ld", (long)grid);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == SONAR_DTYPE_F16) {
+    if (has_zp) launch_moe_mb<_Float16, true>(p, has_perm, (int)grid, st);
+    else launch_moe_mb<_Float16, false>(p, has_perm, (int)grid, st);
+  } else {
+    if (has_zp) launch_moe_mb<__bf16, true>(p, has_perm, (int)grid, st);
+    else launch_moe_mb<__bf16, false>(p, has_perm, (int)grid, st);
+  }
+  return launch_status("marlin_moe_kernel");
 }

@@ -393,14 +393,16 @@ Tensor moe_wna16_marlin_gemm(
   Tensor native = native_weights(b_q_weight, size_k, size_n, experts);
   const size_t scratch_bytes =
       sonar_moe_marlin_gemm_scratch_bytes(sorted_token_ids.numel(), moe_block_size, size_n, size_k);
-  Tensor scratch = at::empty({(int64_t)(scratch_bytes > 16 ? scratch_bytes : 16)}, a.options().dtype(at::kByte));
+  Tensor scratch;
+  if (scratch_bytes > 0) scratch = at::empty({(int64_t)scratch_bytes}, a.options().dtype(at::kByte));
 
   raise_if_failed(sonar_moe_wna16_marlin_gemm(
       a.const_data_ptr(), c.mutable_data_ptr(), static_cast<const uint32_t*>(native.const_data_ptr()),
       SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none), b_scales.const_data_ptr(),
       has_zp ? static_cast<const uint32_t*>(b_zeros_or_none->const_data_ptr()) : nullptr, g_idx, perm,
-      static_cast<int32_t*>(workspace.mutable_data_ptr()), workspace.numel(), scratch.mutable_data_ptr(),
-      scratch_bytes, static_cast<const int32_t*>(sorted_token_ids.const_data_ptr()),
+      static_cast<int32_t*>(workspace.mutable_data_ptr()), workspace.numel(),
+      scratch_bytes > 0 ? scratch.mutable_data_ptr() : nullptr, scratch_bytes,
+      static_cast<const int32_t*>(sorted_token_ids.const_data_ptr()),
       sorted_token_ids.numel(), static_cast<const int32_t*>(expert_ids.const_data_ptr()),
       static_cast<const int32_t*>(num_tokens_past_padded.const_data_ptr()),
       static_cast<const float*>(topk_weights.const_data_ptr()), moe_block_size, top_k,

@@ -1,0 +1,177 @@
+"""GPU parity of the grouped (mixture-of-experts) W4A16 GEMM, through the C ABI,
+against the oracle's restatement of moe_wna16_marlin_gemm
+(csrc/libtorch_stable/moe/marlin_moe_wna16/ops.cu:544-897).  The routing
+(moe_align_block_size) is the oracle's; the cases follow
+tests/kernels/moe/test_moe.py:560-700 (experts, top-k, group sizes, act-order,
+zero points) at sizes the oracle finishes in seconds."""
+from __future__ import annotations
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import marlin_oracle as mo
+from sonar_amd import _lib
+from tests import gpu_util as gu
+
+pytestmark = pytest.mark.gpu
+
+
+class Experts:
+    def __init__(self, seed, e, k, n, group_size, dtype, zero_points=False, act_order=False, bias=False):
+        self.layers = [gu.DeviceLayer(seed + 17 * i, k, n, group_size, dtype, zero_points, act_order, bias)
+                       for i in range(e)]
+        first = self.layers[0]
+        self.e, self.k, self.n, self.dtype = e, k, n, dtype
+        self.groups, self.b_type = first.groups, first.b_type
+        cat = lambda name: (torch.stack([getattr(l, name) for l in self.layers]).contiguous()
+                            if getattr(first, name) is not None else None)
+        self.native = cat("native")
+        self.scales = cat("scales")
+        self.zeros = cat("zeros")
+        self.bias = cat("bias")
+        self.g_idx = cat("g_idx")
+        self.perm = cat("perm")
+        self.workspace = first.workspace
+
+    def reference(self, a32, sorted_ids, expert_ids, past, bs, top_k, m, weights):
+        w = [l.w_ref for l in self.layers]
+        if self.bias is None:
+            return mo.moe_gemm_reference(a32, w, sorted_ids, expert_ids, past, bs, top_k, m, weights, self.dtype)
+        # bias is added before the routing weight is applied
+        out = np.zeros((m * top_k, self.n), dtype=np.float32)
+        for b in range(past // bs):
+            ex = int(expert_ids[b])
+            if ex < 0:
+                continue
+            ids = sorted_ids[b * bs:(b + 1) * bs]
+            ids = ids[ids < m * top_k]
+            c = mo.round_to_dtype(a32[ids // top_k] @ w[ex] + self.layers[ex].bias32[None, :], self.dtype)
+            if weights is not None:
+                wt = mo.round_to_dtype(weights.reshape(-1)[ids].astype(np.float32), self.dtype)
+                c = mo.round_to_dtype(c * wt[:, None], self.dtype)
+            out[ids] = c
+        return out
+
+    def gemm(self, a, sorted_ids, expert_ids, past, weights, bs, top_k, m, mul):
+        lib = _lib.load()
+        tdt = torch.float16 if self.dtype == "fp16" else torch.bfloat16
+        c = torch.zeros((m * top_k, self.n), dtype=tdt, device=gu.DEV)
+        sid = gu.dev_i32(sorted_ids)
+        eid = gu.dev_i32(expert_ids)
+        npp = gu.dev_i32(np.array([past], dtype=np.int32))
+        tw = torch.from_numpy(weights.astype(np.float32).reshape(-1)).to(gu.DEV) if weights is not None else None
+        _lib.check(lib.sonar_moe_wna16_marlin_gemm(
+            gu.ptr(a), gu.ptr(c), gu.ptr(self.native), _lib.LAYOUT_GFX950, gu.ptr(self.bias),
+            gu.ptr(self.scales), gu.ptr(self.zeros), gu.ptr(self.g_idx), gu.ptr(self.perm),
+            gu.ptr(self.workspace), self.workspace.numel(), None, 0, gu.ptr(sid), sid.numel(),
+            gu.ptr(eid), gu.ptr(npp), gu.ptr(tw), bs, top_k, int(mul), self.e,
+            gu.dtype_code(self.dtype), self.b_type, m, self.n, self.k, self.groups, 1, 0, 1, gu.stream()))
+        torch.cuda.synchronize()
+        return c
+
+
+def route(seed, m, e, top_k):
+    rng = np.random.default_rng(seed)
+    ids = np.stack([rng.permutation(e)[:top_k] for _ in range(m)]).astype(np.int32)
+    w = rng.random((m, top_k)).astype(np.float32)
+    w /= w.sum(axis=1, keepdims=True)
+    return ids, w
+
+
+# (m, e, top_k, k, n, group, dtype, zero_points, act_order, bias, block_size or None, mul)
+MOE_CASES = [
+    (1, 8, 2, 256, 128, 128, "fp16", False, False, False, None, False),
+    (7, 8, 2, 512, 256, 128, "bf16", False, False, False, None, True),
+    (33, 4, 2, 512, 192, 64, "fp16", True, False, False, None, True),
+    (64, 8, 3, 384, 128, 32, "bf16", False, False, True, None, True),
+    (20, 4, 1, 256, 128, -1, "fp16", False, False, False, None, False),
+    (40, 6, 2, 512, 128, 128, "fp16", False, True, False, None, True),
+    (16, 8, 2, 256, 128, 128, "bf16", True, False, False, 8, False),
+    (150, 4, 2, 256, 256, 128, "fp16", False, False, False, 48, True),
+    (222, 3, 2, 288, 128, 32, "bf16", False, False, False, 64, True),
+    (5, 64, 6, 256, 128, 128, "fp16", False, False, False, 16, True),
+]
+
+
+@pytest.mark.parametrize("case", MOE_CASES, ids=lambda c: "-".join(str(x) for x in c))
+def test_moe_gemm_within_tolerance(case):
+    m, e, top_k, k, n, g, dtype, zp, act, bias, bs, mul = case
+    print("moe case", case, flush=True)
+    ex = Experts(500 + m, e, k, n, g, dtype, zp, act, bias)
+    topk_ids, topk_w = route(m, m, e, top_k)
+    if bs is None:
+        bs = mo.moe_block_size_rule(m, top_k, e)
+    sorted_ids, expert_ids, past = mo.moe_align_block_size(topk_ids, bs, e)
+    a32 = mo.make_activations(m + 3, m, k, dtype)
+    a = gu.dev_bits16(a32, dtype)
+    got = gu.host_f32(ex.gemm(a, sorted_ids, expert_ids, int(past[0]), topk_w, bs, top_k, m, mul))
+    want = ex.reference(a32, sorted_ids, expert_ids, int(past[0]), bs, top_k, m, topk_w if mul else None)
+    # every row of C is produced by exactly one slot
+    assert np.all(np.isfinite(got))
+    ok, *worst = mo.gemm_tolerance_ok(got, want)
+    assert ok, worst
+
+
+def test_moe_skips_invalid_blocks_and_rows():
+    """Blocks with expert id -1, blocks past num_tokens_past_padded and padding
+    slots leave C untouched (marlin_template.h(moe):471-570)."""
+    m, e, top_k, k, n, bs = 12, 4, 2, 256, 128, 16
+    ex = Experts(77, e, k, n, 128, "fp16")
+    topk_ids, topk_w = route(5, m, e, top_k)
+    sorted_ids, expert_ids, past = mo.moe_align_block_size(topk_ids, bs, e)
+    expert_ids = expert_ids.copy()
+    expert_ids[1] = -1
+    past_cut = int(past[0]) - bs      # the last block is declared padding
+    a32 = mo.make_activations(9, m, k, "fp16")
+    a = gu.dev_bits16(a32, "fp16")
+    got = gu.host_f32(ex.gemm(a, sorted_ids, expert_ids, past_cut, topk_w, bs, top_k, m, False))
+    want = ex.reference(a32, sorted_ids, expert_ids, past_cut, bs, top_k, m, None)
+    ok, *worst = mo.gemm_tolerance_ok(got, want)
+    assert ok, worst
+    untouched = np.ones(m * top_k, dtype=bool)
+    for b in range(past_cut // bs):
+        if expert_ids[b] >= 0:
+            ids = sorted_ids[b * bs:(b + 1) * bs]
+            untouched[ids[ids < m * top_k]] = False
+    assert untouched.any()
+    assert np.all(got[untouched] == 0.0)
+
+
+def test_moe_matches_dense_gemm_per_expert():
+    """With top_k = 1 and all tokens routed to one expert the grouped GEMM is
+    the dense GEMM of that expert, bit for bit up to the summation order: both
+    must satisfy the tolerance against the same reference and each other."""
+    m, e, k, n, bs = 16, 3, 512, 128, 16
+    ex = Experts(31, e, k, n, 128, "bf16")
+    topk_ids = np.full((m, 1), 2, dtype=np.int32)
+    sorted_ids, expert_ids, past = mo.moe_align_block_size(topk_ids, bs, e)
+    a32 = mo.make_activations(2, m, k, "bf16")
+    a = gu.dev_bits16(a32, "bf16")
+    got = gu.host_f32(ex.gemm(a, sorted_ids, expert_ids, int(past[0]), None, bs, 1, m, False))
+    dense = gu.host_f32(ex.layers[2].gemm(a, m))
+    ok, *worst = mo.gemm_tolerance_ok(got, dense)
+    assert ok, worst
+
+
+def test_moe_error_paths():
+    lib = _lib.load()
+    ex = Experts(3, 2, 256, 128, 128, "fp16")
+    a = torch.zeros((4, 256), dtype=torch.float16, device=gu.DEV)
+    c = torch.zeros((8, 128), dtype=torch.float16, device=gu.DEV)
+    sid = torch.zeros(32, dtype=torch.int32, device=gu.DEV)
+    eid = torch.zeros(2, dtype=torch.int32, device=gu.DEV)
+    npp = torch.zeros(1, dtype=torch.int32, device=gu.DEV)
+
+    def call(bs=16, b_type=_lib.TYPE_UINT4B8, k=256):
+        return lib.sonar_moe_wna16_marlin_gemm(
+            gu.ptr(a), gu.ptr(c), gu.ptr(ex.native), _lib.LAYOUT_GFX950, None, gu.ptr(ex.scales), None, None,
+            None, gu.ptr(ex.workspace), ex.workspace.numel(), None, 0, gu.ptr(sid), sid.numel(), gu.ptr(eid),
+            gu.ptr(npp), None, bs, 2, 0, 2, _lib.DTYPE_F16, b_type, 4, 128, k, 2, 1, 0, 1, gu.stream())
+
+    assert call() == _lib.OK
+    assert call(bs=24) == _lib.E_INVALID
+    assert b"moe_block_size" in lib.sonar_marlin_last_error()
+    assert call(b_type=_lib.TYPE_UINT4) == _lib.E_INVALID
+    assert call(k=250) == _lib.E_INVALID
+    torch.cuda.synchronize()
