@@ -1,0 +1,191 @@
+"""Host side of the Marlin mixture-of-experts layer: token routing into blocks
+and the two grouped W4A16 GEMMs around the gated activation.
+
+Mirrors aphrodite/model_executor/layers/fused_moe/moe_align_block_size.py:11-101
+(`moe_align_block_size`) and .../fused_moe/experts/marlin_moe.py:57-392
+(`fused_marlin_moe`) for 4-bit integer weights with fp16 / bf16 activations.
+The routing, the activation and the final sum are torch expressions that never
+read a device value on the host, so the whole layer can be recorded in a HIP
+graph; the two GEMMs are the `_moe_C::moe_wna16_marlin_gemm` op.
+"""
+from __future__ import annotations
+
+import math
+
+import torch
+
+from . import ops
+from .marlin_utils import marlin_make_workspace_new
+from .scalar_type import ScalarType, scalar_types
+
+_SUPPORTED = {t.id: t for t in (scalar_types.uint4, scalar_types.uint4b8)}
+
+
+def moe_block_size(num_tokens: int, top_k: int, num_experts: int) -> int:
+    """Smallest block size whose expected fill is below 0.9 (marlin_moe.py:322-329)."""
+    for block_size_m in (8, 16, 32, 48, 64):
+        if num_tokens * top_k / num_experts / block_size_m < 0.9:
+            break
+    return block_size_m
+
+
+def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int,
+                         expert_map: torch.Tensor | None = None, pad_sorted_ids: bool = False,
+                         ignore_invalid_experts: bool = False
+                         ) -> tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Sorts the flattened (token, k) slots by expert, pads every expert's run
+    to a multiple of `block_size` with the sentinel `topk_ids.numel()`, and
+    names the expert of each block.  Returns (sorted_token_ids int32
+    [max_num_tokens_padded], expert_ids int32 [blocks], num_tokens_post_padded
+    int32 [1]).  Slots of one expert keep ascending order.  Blocks past
+    num_tokens_post_padded carry expert id -1.
+
+    With `expert_map` (global -> local id, -1 = not on this rank): when
+    `ignore_invalid_experts` the slots of absent experts are dropped before
+    counting and expert_ids holds local ids; otherwise every expert is counted
+    and expert_ids of absent experts become -1."""
+    numel = topk_ids.numel()
+    dev = topk_ids.device
+    max_num_tokens_padded = numel + num_experts * (block_size - 1)
+    if pad_sorted_ids:
+        max_num_tokens_padded = -(-max_num_tokens_padded // block_size) * block_size
+    if numel < num_experts:
+        max_num_tokens_padded = min(numel * block_size, max_num_tokens_padded)
+    max_blocks = -(-max_num_tokens_padded // block_size)
+
+    flat = topk_ids.reshape(-1).to(torch.int64)
+    valid = (flat >= 0) & (flat < num_experts)
+    if expert_map is not None and ignore_invalid_experts:
+        valid &= expert_map.to(torch.int64)[flat.clamp(0, num_experts - 1)] >= 0
+    # invalid slots sort behind every expert and are never placed
+    key = torch.where(valid, flat, torch.full_like(flat, num_experts))
+    counts = torch.zeros(num_experts + 1, dtype=torch.int64, device=dev).scatter_add_(
+        0, key, torch.ones_like(key))[:num_experts]
+    padded = (counts + block_size - 1) // block_size * block_size
+    pad_end = torch.cumsum(padded, 0)
+    pad_begin = pad_end - padded
+    run_begin = torch.cumsum(counts, 0) - counts
+
+    order = torch.sort(key, stable=True).indices          # slot ids, expert-major, ascending inside
+    sorted_key = key[order]
+    placed = sorted_key < num_experts
+    e_of = sorted_key.clamp(max=num_experts - 1)
+    rank = torch.arange(numel, device=dev) - run_begin[e_of]
+    dest = torch.where(placed, pad_begin[e_of] + rank, torch.full_like(rank, max_num_tokens_padded))
+    sorted_ids = torch.full((max_num_tokens_padded + 1,), numel, dtype=torch.int32, device=dev)
+    sorted_ids.scatter_(0, dest, order.to(torch.int32))
+    sorted_ids = sorted_ids[:max_num_tokens_padded]
+
+    block_start = torch.arange(max_blocks, device=dev) * block_size
+    expert_of_block = torch.searchsorted(pad_end, block_start, right=True)
+    total = pad_end[-1]
+    in_range = block_start < total
+    expert_ids = torch.where(in_range, expert_of_block, torch.full_like(expert_of_block, -1))
+    if expert_map is not None:
+        mapped = expert_map.to(torch.int64)[expert_ids.clamp(0, num_experts - 1)]
+        expert_ids = torch.where(in_range, mapped, expert_ids)
+    return sorted_ids, expert_ids.to(torch.int32), total.to(torch.int32).reshape(1)
+
+
+def silu_and_mul(out: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
+    """out = silu(x[:, :d]) * x[:, d:] in the tensor's own dtype."""
+    d = x.shape[-1] // 2
+    torch.mul(torch.nn.functional.silu(x[..., :d]), x[..., d:], out=out)
+    return out
+
+
+def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, num_topk,
+                      quant_type: ScalarType, apply_router_weight_on_input, block_size_m, sorted_token_ids,
+                      expert_ids, num_tokens_post_padded, g_idx1=None, g_idx2=None, sort_indices1=None,
+                      sort_indices2=None, w1_zeros=None, w2_zeros=None, workspace=None,
+                      intermediate_cache13=None, intermediate_cache2=None, output=None, is_k_full=True):
+    """Gate/up GEMM -> silu_and_mul -> down GEMM over already routed slots
+    (marlin_moe.py:57-223).  Returns the [M * top_k, K] per-slot outputs."""
+    assert hidden_states.ndim == 2
+    M, K = hidden_states.shape
+    N = w2.shape[1] * 16                       # intermediate size: w2 is (E, N/16, 2K)
+    dev, dt = hidden_states.device, hidden_states.dtype
+    if workspace is None:
+        workspace = marlin_make_workspace_new(dev, 4)
+    if intermediate_cache13 is None:
+        intermediate_cache13 = torch.empty((M * num_topk * max(2 * N, K),), device=dev, dtype=dt)
+    if intermediate_cache2 is None:
+        intermediate_cache2 = torch.empty((M * num_topk, N), device=dev, dtype=dt)
+    cache1 = intermediate_cache13[:M * num_topk * 2 * N].view(M * num_topk, 2 * N)
+    cache3 = intermediate_cache13[:M * num_topk * K].view(M * num_topk, K)
+    cache2 = intermediate_cache2.view(-1)[:M * num_topk * N].view(M * num_topk, N)
+
+    cache1 = ops.moe_wna16_marlin_gemm(
+        hidden_states, cache1, w1, bias1, w1_scale, None, None, w1_zeros, g_idx1, sort_indices1, workspace,
+        sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, moe_block_size=block_size_m,
+        top_k=num_topk, mul_topk_weights=apply_router_weight_on_input, b_q_type=quant_type, size_m=M,
+        size_n=2 * N, size_k=K, is_k_full=is_k_full, use_atomic_add=False, use_fp32_reduce=True,
+        is_zp_float=False)
+    silu_and_mul(cache2, cache1.view(-1, 2 * N))
+    if output is None:
+        output = cache3
+    return ops.moe_wna16_marlin_gemm(
+        cache2, output, w2, bias2, w2_scale, None, None, w2_zeros, g_idx2, sort_indices2, workspace,
+        sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, moe_block_size=block_size_m,
+        top_k=1, mul_topk_weights=not apply_router_weight_on_input, b_q_type=quant_type,
+        size_m=M * num_topk, size_n=K, size_k=N, is_k_full=is_k_full, use_atomic_add=False,
+        use_fp32_reduce=True, is_zp_float=False)
+
+
+def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Tensor,
+                     bias1: torch.Tensor | None, bias2: torch.Tensor | None, w1_scale: torch.Tensor,
+                     w2_scale: torch.Tensor, topk_weights: torch.Tensor, topk_ids: torch.Tensor,
+                     quant_type_id: int, apply_router_weight_on_input: bool = False,
+                     global_num_experts: int = -1, expert_map: torch.Tensor | None = None,
+                     g_idx1: torch.Tensor | None = None, g_idx2: torch.Tensor | None = None,
+                     sort_indices1: torch.Tensor | None = None, sort_indices2: torch.Tensor | None = None,
+                     w1_zeros: torch.Tensor | None = None, w2_zeros: torch.Tensor | None = None,
+                     workspace: torch.Tensor | None = None,
+                     intermediate_cache13: torch.Tensor | None = None,
+                     intermediate_cache2: torch.Tensor | None = None, is_k_full: bool = True,
+                     output: torch.Tensor | None = None, input_dtype: torch.dtype | None = None
+                     ) -> torch.Tensor:
+    """Mixture-of-experts layer with Marlin int4 expert weights and top-k gating
+    (marlin_moe.py:226-392).  w1: (E, K/16, 2 * 2N) gate and up projections,
+    w2: (E, N/16, 2K); scales (E, groups, 2N) / (E, groups, K); topk_weights
+    fp32 [M, top_k]; topk_ids [M, top_k].  Returns [M, K]."""
+    if quant_type_id not in _SUPPORTED:
+        raise NotImplementedError(f"quant type id {quant_type_id}: only uint4 and uint4b8 expert weights "
+                                  "are built")
+    if input_dtype is not None:
+        raise NotImplementedError("8-bit activations are not built")
+    quant_type = _SUPPORTED[quant_type_id]
+    M, K = hidden_states.shape
+    E = w1.shape[0]
+    topk = topk_ids.shape[1]
+    assert w1.shape[1] * 16 == K, "Hidden size mismatch w1"
+    assert w2.shape[2] // 2 == K, "Hidden size mismatch w2"
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert w1.is_contiguous(), "Expert weights1 must be contiguous"
+    assert w2.is_contiguous(), "Expert weights2 must be contiguous"
+    assert hidden_states.dtype in (torch.float16, torch.bfloat16)
+    assert topk_weights.dtype == torch.float32
+
+    m_est = M
+    if global_num_experts == -1:
+        global_num_experts = E
+    else:
+        m_est = math.ceil(M * E / global_num_experts)   # expected tokens for the local experts
+    block_size_m = moe_block_size(m_est, topk, E)
+    sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(
+        topk_ids, block_size_m, global_num_experts, expert_map, ignore_invalid_experts=True)
+
+    moe_output = _fused_marlin_moe(
+        hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, topk, quant_type,
+        apply_router_weight_on_input, block_size_m, sorted_token_ids, expert_ids, num_tokens_post_padded,
+        g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1, sort_indices2=sort_indices2,
+        w1_zeros=w1_zeros, w2_zeros=w2_zeros, workspace=workspace,
+        intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2, output=None,
+        is_k_full=is_k_full).view(-1, topk, K)
+    if expert_map is not None:
+        # slots of experts held elsewhere were never written
+        local = expert_map.to(torch.int64)[topk_ids.to(torch.int64).clamp(0, global_num_experts - 1)] >= 0
+        moe_output = torch.where(local.unsqueeze(-1), moe_output, torch.zeros_like(moe_output))
+    if output is None:
+        output = torch.empty_like(hidden_states)
+    return torch.sum(moe_output, dim=1, out=output)

@@ -1,0 +1,83 @@
+#!/usr/bin/env python3
+"""Writes the golden fixtures of this directory from the CPU oracle.
+
+The reference's own tests hold no stored vectors for the Marlin path (they
+compare against helper code at run time), so these fixtures are this
+repository's: seeded inputs and the oracle's outputs, frozen so that a later
+change of the oracle or of a kernel shows up as a diff against committed data.
+`moe_align_example` is the one literal vector the reference gives
+(fused_moe/moe_align_block_size.py:60-73).
+
+Run from the repository root:  python tests/golden/make_fixtures.py
+"""
+from __future__ import annotations
+
+import os
+import sys
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.dirname(os.path.dirname(HERE)))
+
+from oracle import marlin_oracle as mo  # noqa: E402
+
+
+def layer_fixture(seed, k, n, g, dtype, zero_points, act_order, m):
+    layer = mo.make_layer(seed, k, n, g, dtype, zero_points, act_order)
+    q = layer["q"]
+    out = {"size_k": np.int64(k), "size_n": np.int64(n), "group_size": np.int64(g), "size_m": np.int64(m),
+           "q": q.astype(np.uint8), "gptq_packed": mo.gptq_pack(q), "awq_packed": mo.awq_pack(q),
+           "scales_bits": mo.to_bits16(layer["scales"], dtype)}
+    perm = None
+    if act_order:
+        g_sorted, perm = mo.stable_sort_g_idx(layer["g_idx"])
+        out["g_idx"] = layer["g_idx"].astype(np.int32)
+        out["g_idx_sorted"] = g_sorted.astype(np.int32)
+        out["perm"] = perm.astype(np.int32)
+    marlin = mo.gptq_marlin_repack(mo.gptq_pack(q), perm, k, n)
+    out["marlin"] = marlin
+    out["gfx950"] = mo.marlin_to_gfx950(marlin, k, n)
+    gs = g if g < k else -1
+    out["scales_marlin_bits"] = mo.to_bits16(mo.marlin_permute_scales(layer["scales"], k, n, gs), dtype)
+    if zero_points:
+        out["zeros"] = layer["zeros"].astype(np.uint8)
+        out["zeros_marlin"] = mo.marlin_zero_points(layer["zeros"], layer["groups"], n)
+    w = mo.dequantize(q, layer["scales"], g, dtype, zeros=layer.get("zeros"), g_idx=layer.get("g_idx"))
+    out["dequant_bits"] = mo.to_bits16(w, dtype)
+    a = mo.make_activations(seed + 1, m, k, dtype)
+    out["a_bits"] = mo.to_bits16(a, dtype)
+    out["c_ref"] = mo.gemm_reference(a, w)
+    return out
+
+
+def main():
+    np.savez_compressed(os.path.join(HERE, "gptq_fp16_k128_n128_g64.npz"),
+                        **layer_fixture(101, 128, 128, 64, "fp16", False, False, 5))
+    np.savez_compressed(os.path.join(HERE, "awq_bf16_k128_n64_g32.npz"),
+                        **layer_fixture(102, 128, 64, 32, "bf16", True, False, 3))
+    np.savez_compressed(os.path.join(HERE, "actorder_fp16_k256_n64_g128.npz"),
+                        **layer_fixture(103, 256, 64, 128, "fp16", False, True, 17))
+    ids = np.array([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]], dtype=np.int32)
+    s, e, p = mo.moe_align_block_size(ids, 4, 5)
+    np.savez_compressed(os.path.join(HERE, "moe_align_example.npz"), topk_ids=ids, block_size=np.int64(4),
+                        num_experts=np.int64(5), sorted_ids=s, expert_ids=e, num_post_pad=p)
+    # every 4-bit code against zero points 0..15 and a spread of scale bit patterns
+    rng = np.random.default_rng(7)
+    for dtype in ("fp16", "bf16"):
+        scales = mo.round_to_dtype(np.concatenate([rng.uniform(1e-3, 1e-2, 24), [0.0, 1.0, 6.1e-5, 3.0e-3]])
+                                   .astype(np.float32), dtype)
+        codes = np.arange(16, dtype=np.int64)
+        table = np.zeros((16, 16, scales.size), dtype=np.uint16)
+        for z in range(16):
+            table[z] = mo.to_bits16(mo.round_to_dtype(((codes - z)[:, None] * scales[None, :])
+                                                      .astype(np.float32), dtype), dtype)
+        np.savez_compressed(os.path.join(HERE, f"dequant_table_{dtype}.npz"),
+                            scales_bits=mo.to_bits16(scales, dtype), table_bits=table)
+    for f in sorted(os.listdir(HERE)):
+        if f.endswith(".npz"):
+            print(f, os.path.getsize(os.path.join(HERE, f)))
+
+
+if __name__ == "__main__":
+    main()

@@ -1,0 +1,113 @@
+"""The committed fixtures of tests/golden (written by tests/golden/make_fixtures.py
+from the oracle) against the oracle as it is now (CPU) and against the HIP
+kernels through the C ABI (GPU)."""
+from __future__ import annotations
+
+import os
+
+import numpy as np
+import pytest
+
+from oracle import marlin_oracle as mo
+
+
+def U32(x):
+    return np.ascontiguousarray(x).view(np.uint32)
+
+GOLDEN = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+LAYERS = [("gptq_fp16_k128_n128_g64.npz", "fp16"), ("awq_bf16_k128_n64_g32.npz", "bf16"),
+          ("actorder_fp16_k256_n64_g128.npz", "fp16")]
+
+
+def load(name):
+    return np.load(os.path.join(GOLDEN, name), allow_pickle=False)
+
+
+@pytest.mark.parametrize("name,dtype", LAYERS)
+def test_oracle_reproduces_layer_fixture(name, dtype):
+    f = load(name)
+    k, n, g = int(f["size_k"]), int(f["size_n"]), int(f["group_size"])
+    q = f["q"].astype(np.int64)
+    assert np.array_equal(mo.gptq_pack(q), f["gptq_packed"])
+    assert np.array_equal(mo.awq_pack(q), f["awq_packed"])
+    perm = f["perm"] if "perm" in f.files else None
+    assert np.array_equal(mo.gptq_marlin_repack(f["gptq_packed"], perm, k, n), f["marlin"])
+    if perm is None:
+        assert np.array_equal(mo.awq_marlin_repack(f["awq_packed"], k, n), f["marlin"])
+    else:
+        g_sorted, order = mo.stable_sort_g_idx(f["g_idx"])
+        assert np.array_equal(order, perm) and np.array_equal(g_sorted, f["g_idx_sorted"])
+    assert np.array_equal(mo.marlin_to_gfx950(f["marlin"], k, n), f["gfx950"])
+    scales = mo.from_bits16(f["scales_bits"], dtype)
+    gs = g if g < k else -1
+    assert np.array_equal(mo.to_bits16(mo.marlin_permute_scales(scales, k, n, gs), dtype), f["scales_marlin_bits"])
+    zeros = f["zeros"].astype(np.int64) if "zeros" in f.files else None
+    if zeros is not None:
+        assert np.array_equal(mo.marlin_zero_points(zeros, k // g, n), f["zeros_marlin"])
+    w = mo.dequantize(q, scales, g, dtype, zeros=zeros, g_idx=f["g_idx"] if perm is not None else None)
+    assert np.array_equal(mo.to_bits16(w, dtype), f["dequant_bits"])
+    a = mo.from_bits16(f["a_bits"], dtype)
+    assert np.allclose(mo.gemm_reference(a, w), f["c_ref"], rtol=1e-6, atol=1e-6)
+
+
+def test_oracle_reproduces_moe_align_and_dequant_tables():
+    f = load("moe_align_example.npz")
+    s, e, p = mo.moe_align_block_size(f["topk_ids"], int(f["block_size"]), int(f["num_experts"]))
+    assert np.array_equal(s, f["sorted_ids"]) and np.array_equal(e, f["expert_ids"]) and p[0] == f["num_post_pad"][0]
+    assert s[:16].tolist() == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    for dtype in ("fp16", "bf16"):
+        t = load(f"dequant_table_{dtype}.npz")
+        scales = mo.from_bits16(t["scales_bits"], dtype)
+        for z in range(16):
+            q = np.arange(16, dtype=np.int64)[:, None].repeat(scales.size, 1)     # [16 rows][S columns]
+            w = mo.dequantize(q, scales[None, :], 16, dtype, zeros=np.full((1, scales.size), z, dtype=np.int64))
+            assert np.array_equal(mo.to_bits16(w, dtype), t["table_bits"][z])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,dtype", LAYERS)
+def test_hip_kernels_reproduce_layer_fixture(name, dtype):
+    import torch
+
+    from sonar_amd import _lib
+    from tests import gpu_util as gu
+    f = load(name)
+    k, n, g, m = int(f["size_k"]), int(f["size_n"]), int(f["group_size"]), int(f["size_m"])
+    has_perm = "perm" in f.files
+    has_zp = "zeros" in f.files
+    perm = gu.dev_i32(f["perm"]) if has_perm else None
+    marlin = gu.gptq_repack(gu.dev_i32(f["gptq_packed"]), perm, k, n)
+    assert np.array_equal(marlin.cpu().numpy().view(np.uint32), U32(f["marlin"]))
+    if not has_perm:
+        awq = gu.awq_repack(gu.dev_i32(f["awq_packed"]), k, n)
+        assert np.array_equal(awq.cpu().numpy().view(np.uint32), U32(f["marlin"]))
+    native = gu.to_gfx950(marlin, k, n)
+    assert np.array_equal(native.cpu().numpy().view(np.uint32), U32(f["gfx950"].reshape(-1)))
+    assert np.array_equal(gu.from_gfx950(native, k, n).cpu().numpy().view(np.uint32), U32(f["marlin"]))
+
+    lib = _lib.load()
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    scales = torch.from_numpy(f["scales_marlin_bits"].view(np.int16).copy()).to(gu.DEV).view(tdt)
+    zeros = gu.dev_i32(f["zeros_marlin"]) if has_zp else None
+    b_type = _lib.TYPE_UINT4 if has_zp else _lib.TYPE_UINT4B8
+    groups = k // g
+    # in-kernel dequantised values, bit for bit.  With act-order the kernel sees
+    # the rows in sorted-group order: row i of its matrix is row perm[i] of W.
+    w = torch.empty((k, n), dtype=tdt, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_dequant(gu.ptr(native), _lib.LAYOUT_GFX950, gu.ptr(scales), gu.ptr(zeros), None,
+                                        gu.ptr(w), gu.dtype_code(dtype), b_type, n, k, groups, 1, gu.stream()))
+    want = f["dequant_bits"][f["perm"]] if has_perm else f["dequant_bits"]
+    assert np.array_equal(w.view(torch.int16).cpu().numpy().view(np.uint16), want)
+
+    a = torch.from_numpy(f["a_bits"].view(np.int16).copy()).to(gu.DEV).view(tdt)
+    c = torch.empty((m, n), dtype=tdt, device=gu.DEV)
+    ws = torch.zeros(torch.cuda.get_device_properties(0).multi_processor_count, dtype=torch.int32, device=gu.DEV)
+    nbytes = lib.sonar_marlin_gemm_scratch_bytes(m, n, k)
+    scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=gu.DEV)
+    g_idx = gu.dev_i32(f["g_idx_sorted"]) if has_perm else None
+    _lib.check(lib.sonar_marlin_gemm(gu.ptr(a), k, gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None,
+                                     gu.ptr(scales), gu.ptr(zeros), gu.ptr(g_idx), gu.ptr(perm), gu.ptr(ws),
+                                     ws.numel(), gu.ptr(scratch), scratch.numel(), gu.dtype_code(dtype), b_type,
+                                     m, n, k, groups, 1, 0, 1, gu.stream()))
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(c), f["c_ref"])
+    assert ok, worst

@@ -1,0 +1,260 @@
+"""GPU tests of the torch-op layer and the host mirror above it: the ops are
+called the way the reference's callers call them (apply_gptq_marlin_linear,
+MarlinLinearKernel, fused_marlin_moe) and compared with the oracle."""
+from __future__ import annotations
+
+import types
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import marlin_oracle as mo
+from tests import gpu_util as gu
+
+pytestmark = pytest.mark.gpu
+
+
+def U32(x):
+    return np.ascontiguousarray(x).view(np.uint32)
+
+
+def _tdt(dtype):
+    return torch.float16 if dtype == "fp16" else torch.bfloat16
+
+
+def test_repack_ops_bit_exact_and_fresh_output():
+    from sonar_amd import ops
+    k, n = 256, 192
+    layer = mo.make_layer(3, k, n, 128, "fp16", zero_points=True, act_order=True)
+    q = layer["q"]
+    g_sorted, order = mo.stable_sort_g_idx(layer["g_idx"])
+    got = ops.gptq_marlin_repack(gu.dev_i32(mo.gptq_pack(q)), gu.dev_i32(order), k, n, 4)
+    want = mo.gptq_marlin_repack(mo.gptq_pack(q), order, k, n)
+    assert got.shape == (k // 16, 2 * n) and got.dtype == torch.int32
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), U32(want))
+    empty = torch.empty(0, dtype=torch.int32, device=gu.DEV)
+    got = ops.gptq_marlin_repack(gu.dev_i32(mo.gptq_pack(q)), empty, k, n, 4)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), U32(mo.gptq_marlin_repack(mo.gptq_pack(q), None, k, n)))
+    got = ops.awq_marlin_repack(gu.dev_i32(mo.awq_pack(q)), k, n, 4)
+    assert np.array_equal(got.cpu().numpy().view(np.uint32), U32(mo.awq_marlin_repack(mo.awq_pack(q), k, n)))
+    with pytest.raises(RuntimeError):
+        ops.gptq_marlin_repack(gu.dev_i32(mo.gptq_pack(q)), empty, k, n, 8)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("m", [1, 16, 48, 300])
+def test_marlin_gemm_op_and_weight_cache(dtype, m):
+    from sonar_amd import ops
+    from sonar_amd.scalar_type import scalar_types
+    k, n = 512, 256
+    dl = gu.DeviceLayer(21, k, n, 128, dtype)
+    a32 = mo.make_activations(m, m, k, dtype)
+    a = gu.dev_bits16(a32, dtype)
+    empty = torch.empty(0, dtype=torch.int32, device=gu.DEV)
+    ops.marlin_weight_cache_clear()
+    outs = []
+    for _ in range(2):   # second call takes the cached streaming-order copy
+        outs.append(ops.marlin_gemm(a, None, dl.marlin, None, dl.scales, None, None, empty, empty, empty,
+                                    dl.workspace, scalar_types.uint4b8, m, n, k, True, False, True, False))
+    torch.cuda.synchronize()
+    assert torch.equal(outs[0], outs[1])
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(outs[0]), mo.gemm_reference(a32, dl.w_ref))
+    assert ok, worst
+    assert int(dl.workspace.abs().sum()) == 0
+    # writing into a caller's tensor returns that tensor
+    c = torch.empty((m, n), dtype=_tdt(dtype), device=gu.DEV)
+    r = ops.marlin_gemm(a, c, dl.marlin, None, dl.scales, None, None, empty, empty, empty, dl.workspace,
+                        scalar_types.uint4b8, m, n, k, True, False, True, False)
+    assert r.data_ptr() == c.data_ptr() and torch.equal(r, outs[0])
+    # the cache notices an in-place change of the weight
+    dl.marlin.copy_(gu.DeviceLayer(22, k, n, 128, dtype).marlin)
+    other = ops.marlin_gemm(a, None, dl.marlin, None, dl.scales, None, None, empty, empty, empty,
+                            dl.workspace, scalar_types.uint4b8, m, n, k, True, False, True, False)
+    assert not torch.equal(other, outs[0])
+    assert ops.marlin_weight_cache_clear() >= 1
+
+
+def test_marlin_gemm_op_rejects_like_the_reference():
+    from sonar_amd import ops
+    from sonar_amd.scalar_type import scalar_types
+    k, n, m = 256, 128, 4
+    dl = gu.DeviceLayer(5, k, n, 128, "fp16")
+    a = gu.dev_bits16(mo.make_activations(1, m, k, "fp16"), "fp16")
+    empty = torch.empty(0, dtype=torch.int32, device=gu.DEV)
+
+    def call(**kw):
+        args = dict(a=a, c=None, b=dl.marlin, s=dl.scales, z=empty, ws=dl.workspace, t=scalar_types.uint4b8,
+                    m=m, n=n, k=k)
+        args.update(kw)
+        return ops.marlin_gemm(args["a"], args["c"], args["b"], None, args["s"], None, None, args["z"], empty,
+                               empty, args["ws"], args["t"], args["m"], args["n"], args["k"], True, False, True,
+                               False)
+
+    call()
+    with pytest.raises(RuntimeError, match="size_m"):
+        call(m=m + 1)
+    with pytest.raises(RuntimeError):
+        call(t=scalar_types.uint4)            # uint4 needs zero points
+    with pytest.raises(RuntimeError):
+        call(t=scalar_types.uint8b128)        # 8-bit weights are not built
+    with pytest.raises(RuntimeError, match="workspace"):
+        call(ws=dl.workspace[:8])
+    with pytest.raises(RuntimeError):
+        call(s=dl.scales.to(torch.bfloat16))  # scales must have the activation type
+    assert call(a=a[:0], m=0).shape == (0, n)
+
+
+@pytest.mark.parametrize("cfg", [
+    # (k, n, group, dtype, zero_points, act_order, bias, batch shape)
+    (256, 128, 128, "fp16", False, False, False, (5,)),
+    (512, 192, 64, "bf16", False, False, True, (2, 3)),
+    (256, 128, -1, "fp16", False, False, False, (1,)),
+    (256, 128, 128, "bf16", True, False, False, (7,)),
+    (512, 128, 128, "fp16", False, True, True, (9,)),
+    (136, 72, 8 * 17, "fp16", False, False, False, (4,)),     # padded N and K (one group)
+], ids=str)
+def test_marlin_linear_kernel_round_trip(cfg):
+    """Checkpoint-format tensors -> process_weights_after_loading -> apply_weights
+    (kernels/linear/mixed_precision/marlin.py:88-235)."""
+    from sonar_amd.marlin_linear import MarlinLinearKernel, MPLinearLayerConfig
+    from sonar_amd.marlin_utils import pack_cols
+    from sonar_amd.scalar_type import scalar_types
+    k, n, g, dtype, zp, act, bias, batch = cfg
+    gs = k if g == -1 or g >= k else g
+    layer_np = mo.make_layer(11, k, n, gs, dtype, zero_points=zp, act_order=act)
+    w_ref = mo.dequantize(layer_np["q"], layer_np["scales"], gs, dtype, zeros=layer_np.get("zeros"),
+                          g_idx=layer_np.get("g_idx"))
+    layer = types.SimpleNamespace()
+    layer.qweight = gu.dev_i32(mo.gptq_pack(layer_np["q"]))
+    layer.scales = gu.dev_bits16(layer_np["scales"], dtype)
+    layer.bias = None
+    if zp:
+        layer.qzeros = pack_cols(torch.from_numpy(layer_np["zeros"].astype(np.int32)).to(gu.DEV), 4,
+                                 layer_np["groups"], n)
+    if act:
+        layer.g_idx = gu.dev_i32(layer_np["g_idx"])
+    bias32 = None
+    if bias:
+        bias32 = mo.round_to_dtype(np.random.default_rng(4).standard_normal(n).astype(np.float32), dtype)
+        layer.bias = gu.dev_bits16(bias32, dtype)
+    cfgobj = MPLinearLayerConfig((k, n), (k, n), scalar_types.uint4 if zp else scalar_types.uint4b8,
+                                 _tdt(dtype), g if g != 8 * 17 else -1, zp, act)
+    kern = MarlinLinearKernel(cfgobj, w_zp_param_name="qzeros" if zp else None,
+                              w_gidx_param_name="g_idx" if act else None)
+    kern.process_weights_after_loading(layer)
+    rows = int(np.prod(batch))
+    x32 = mo.make_activations(8, rows, k, dtype)
+    x = gu.dev_bits16(x32, dtype).reshape(*batch, k)
+    y = kern.apply_weights(layer, x, layer.bias)
+    assert y.shape == (*batch, n)
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y).reshape(rows, n), mo.gemm_reference(x32, w_ref, bias32))
+    assert ok, worst
+
+
+def _moe_layer(seed, e, hidden, inter, g, dtype, zp):
+    """Expert weights in the layouts fused_marlin_moe takes, plus dequantised references."""
+    from sonar_amd import marlin_utils as mu
+    from sonar_amd import ops
+    w13, w2 = [], []
+    for i in range(e):
+        w13.append(mo.make_layer(seed + i, hidden, 2 * inter, g, dtype, zero_points=zp))
+        w2.append(mo.make_layer(seed + 100 + i, inter, hidden, g, dtype, zero_points=zp))
+
+    def pack(layers, k, n):
+        q = torch.stack([gu.dev_i32(mo.gptq_pack(l["q"])) for l in layers])
+        empty = torch.empty((e, 0), dtype=torch.int32, device=gu.DEV)
+        marlin = ops.gptq_marlin_moe_repack(q, empty, k, n, 4)
+        s = torch.stack([gu.dev_bits16(l["scales"], dtype) for l in layers])
+        s = mu.marlin_moe_permute_scales(s, k, n, g)
+        z = None
+        if zp:
+            z = torch.stack([mu.marlin_zero_points(torch.from_numpy(l["zeros"].astype(np.int32)).to(gu.DEV),
+                                                   l["groups"], n, 4) for l in layers])
+        ref = [mo.dequantize(l["q"], l["scales"], g, dtype, zeros=l.get("zeros")) for l in layers]
+        return marlin, s, z, ref
+
+    return pack(w13, hidden, 2 * inter), pack(w2, inter, hidden)
+
+
+def _moe_reference(x32, ref13, ref2, topk_ids, topk_w, dtype):
+    """torch_experts restated (tests/kernels/utils.py:817-931): per routed
+    slot silu(x W_gate) * (x W_up) -> W_down, weighted sum over the slots."""
+    m, hidden = x32.shape
+    inter = ref2[0].shape[0]
+    out = np.zeros((m, hidden), dtype=np.float32)
+    for t in range(m):
+        for j in range(topk_ids.shape[1]):
+            ex = int(topk_ids[t, j])
+            h = mo.round_to_dtype(x32[t:t + 1] @ ref13[ex], dtype)
+            gate, up = h[:, :inter], h[:, inter:]
+            act = mo.round_to_dtype(mo.round_to_dtype(gate / (1.0 + np.exp(-gate)), dtype) * up, dtype)
+            y = mo.round_to_dtype(act @ ref2[ex], dtype)
+            out[t] += topk_w[t, j] * y[0]
+    return out
+
+
+@pytest.mark.parametrize("cfg", [
+    (4, 8, 2, 256, 128, 128, "bf16", False),
+    (40, 4, 2, 256, 256, 64, "fp16", False),
+    (200, 4, 2, 128, 128, 128, "bf16", True),
+    (3, 16, 4, 256, 128, 128, "fp16", False),
+], ids=str)
+def test_fused_marlin_moe_against_per_token_reference(cfg):
+    from sonar_amd.fused_moe import fused_marlin_moe
+    from sonar_amd.scalar_type import scalar_types
+    m, e, topk, hidden, inter, g, dtype, zp = cfg
+    (w1, s1, z1, ref13), (w2, s2, z2, ref2) = _moe_layer(40, e, hidden, inter, g, dtype, zp)
+    rng = np.random.default_rng(m)
+    logits = rng.standard_normal((m, e)).astype(np.float32)
+    prob = np.exp(logits - logits.max(1, keepdims=True))
+    prob /= prob.sum(1, keepdims=True)
+    topk_ids = np.argsort(-prob, axis=1, kind="stable")[:, :topk].astype(np.int32)
+    topk_w = np.take_along_axis(prob, topk_ids, axis=1).astype(np.float32)
+    x32 = mo.round_to_dtype(0.5 * mo.make_activations(m, m, hidden, dtype), dtype)
+    x = gu.dev_bits16(x32, dtype)
+    qtype = scalar_types.uint4 if zp else scalar_types.uint4b8
+    y = fused_marlin_moe(x, w1, w2, None, None, s1, s2, torch.from_numpy(topk_w).to(gu.DEV),
+                         torch.from_numpy(topk_ids).to(gu.DEV), qtype.id, w1_zeros=z1, w2_zeros=z2)
+    torch.cuda.synchronize()
+    want = _moe_reference(x32, ref13, ref2, topk_ids, topk_w, dtype)
+    got = gu.host_f32(y)
+    max_ref = np.abs(want).max()
+    # two chained GEMMs and three roundings per slot: 2x the single-GEMM bound
+    assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)
+
+
+def test_fused_marlin_moe_replays_in_a_hip_graph():
+    """The layer reads no device value on the host, so it can be recorded; every
+    replay must reproduce the eager result, also after the routing changed."""
+    from sonar_amd.fused_moe import fused_marlin_moe
+    from sonar_amd.scalar_type import scalar_types
+    m, e, topk, hidden, inter = 6, 8, 2, 256, 128
+    (w1, s1, _, _), (w2, s2, _, _) = _moe_layer(60, e, hidden, inter, 128, "bf16", False)
+    x = gu.dev_bits16(mo.make_activations(1, m, hidden, "bf16"), "bf16")
+    gen = torch.Generator(device="cpu").manual_seed(0)
+
+    def routing():
+        w = torch.softmax(torch.randn((m, e), generator=gen), dim=1)
+        tw, ti = torch.topk(w, topk, dim=1)
+        return tw.to(gu.DEV), ti.to(torch.int32).to(gu.DEV)
+
+    tw, ti = routing()
+    run = lambda: fused_marlin_moe(x, w1, w2, None, None, s1, s2, tw, ti, scalar_types.uint4b8.id)
+    eager = run().clone()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        run()
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            out = run()
+    for rep in range(3):
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), rep
+        tw2, ti2 = routing()
+        tw.copy_(tw2)
+        ti.copy_(ti2)
+        eager = run().clone()
+        torch.cuda.synchronize()

@@ -171,3 +171,51 @@ def test_marlin_linear_kernel_gates():
     assert not MarlinLinearKernel.can_implement(act_order_odd)[0]
     straddle = MPLinearLayerConfig((4096, 4096), (1000, 4096), st.uint4b8, torch.float16, 128, False, False)
     assert not MarlinLinearKernel.can_implement(straddle)[0]
+
+
+# ---------------------------------------------------------------- MoE routing (torch mirror)
+@pytest.mark.parametrize("m,topk,e,bs", [(4, 3, 5, 4), (1, 2, 8, 8), (33, 2, 8, 16), (257, 2, 4, 64),
+                                         (5, 6, 64, 16), (100, 1, 3, 48)])
+def test_torch_moe_align_block_size_matches_oracle(m, topk, e, bs):
+    import torch
+
+    from sonar_amd import fused_moe
+    rng = np.random.default_rng(m * 31 + e)
+    ids = np.stack([rng.permutation(e)[:topk] for _ in range(m)]).astype(np.int32)
+    want = mo.moe_align_block_size(ids, bs, e)
+    got = fused_moe.moe_align_block_size(torch.from_numpy(ids), bs, e)
+    past = int(want[2][0])
+    assert int(got[2][0]) == past and got[2].dtype == torch.int32
+    assert got[0].shape[0] == want[0].shape[0] and got[1].shape[0] == want[1].shape[0]
+    assert np.array_equal(got[0].numpy()[:past], want[0][:past])
+    assert np.all(got[0].numpy()[past:] == ids.size)
+    assert np.array_equal(got[1].numpy(), want[1])
+
+
+def test_torch_moe_align_docstring_example_and_expert_map():
+    import torch
+
+    from sonar_amd import fused_moe
+    ids = torch.tensor([[2, 3, 4], [1, 2, 4], [1, 3, 4], [1, 2, 3]], dtype=torch.int32)
+    s, e, p = fused_moe.moe_align_block_size(ids, 4, 5)
+    assert s[:16].tolist() == [3, 6, 9, 12, 0, 4, 10, 12, 1, 7, 11, 12, 2, 5, 8, 12]
+    assert e[:4].tolist() == [1, 2, 3, 4] and int(p) == 16
+    # experts 1 and 3 live on this rank as local experts 0 and 1
+    emap = torch.tensor([-1, 0, -1, 1, -1], dtype=torch.int32)
+    s2, e2, p2 = fused_moe.moe_align_block_size(ids, 4, 5, emap, ignore_invalid_experts=True)
+    assert int(p2) == 8 and e2[:2].tolist() == [0, 1] and s2[:8].tolist() == [3, 6, 9, 12, 1, 7, 11, 12]
+    assert (e2[2:] == -1).all() and (s2[8:] == 12).all()
+    s3, e3, p3 = fused_moe.moe_align_block_size(ids, 4, 5, emap, ignore_invalid_experts=False)
+    assert int(p3) == 16 and e3[:4].tolist() == [0, -1, 1, -1] and torch.equal(s3, s)
+
+
+def test_moe_block_size_and_silu_and_mul():
+    import torch
+
+    from sonar_amd import fused_moe
+    for m, topk, e in [(16, 2, 8), (4096, 2, 8), (1, 2, 8), (64, 6, 64), (300, 2, 8)]:
+        assert fused_moe.moe_block_size(m, topk, e) == mo.moe_block_size_rule(m, topk, e)
+    x = torch.randn(5, 8)
+    out = torch.empty(5, 4)
+    fused_moe.silu_and_mul(out, x)
+    assert torch.allclose(out, x[:, :4] / (1 + torch.exp(-x[:, :4])) * x[:, 4:], atol=1e-6)
