@@ -31,19 +31,18 @@ __device__ __forceinline__ int zero_point_shift(int nl) {
   return 4 * ((t >> 1) + 4 * (t & 1));
 }
 
-// (q & mask) | 0x64006400 in one VALU instruction.  The encoding admits one
-// scalar operand, so the constant that is OR-ed in is kept in a vector
-// register by the caller (`magic`); left to itself the compiler splits the
-// expression into an AND and an OR with literals.
-__device__ __forceinline__ uint32_t magic_register() {
-  uint32_t m = 0x64006400u;
+// (q & mask) | magic, which the compiler emits as one v_and_or_b32 when the
+// constant that is OR-ed in sits in a vector register it cannot see through
+// (`magic_register`); with a visible constant it splits the expression into
+// an AND and an OR with literals.  The expression itself must stay visible to
+// the compiler: it pads the matrix-core hazards (a VALU write to a register an
+// MFMA in flight still reads) only around instructions it generated itself.
+__device__ __forceinline__ uint32_t magic_register(uint32_t m = 0x64006400u) {
   asm("" : "+v"(m));
   return m;
 }
 __device__ __forceinline__ uint32_t and_or(uint32_t q, uint32_t mask, uint32_t magic) {
-  uint32_t r;
-  asm("v_and_or_b32 %0, %1, %2, %3" : "=v"(r) : "v"(q), "s"(mask), "v"(magic));
-  return r;
+  return (q & mask) | magic;
 }
 
 template <typename T>

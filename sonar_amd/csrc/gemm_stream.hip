@@ -343,6 +343,57 @@ struct UnitCursor {
   }
 };
 
+// bf16 only.  gfx950 has no packed bf16 arithmetic, so forming (v - z) * s per
+// weight costs a mixed-precision fma and half a conversion per element.  The
+// fast kernel instead feeds the matrix cores the exact integers 128 + v (the
+// nibble OR-ed into the mantissa of bf16 128.0) and folds offset and scale into
+// the accumulator once per 128-row unit, which lies inside one group:
+//   sum_k (v_k - z) s a_k = s * (sum_k (128 + v_k) a_k - (128 + z) * sum_k a_k),
+// the last sum coming from one more MFMA per chunk with an all-ones operand.
+// Products and sums are exact or fp32, so the result differs from the
+// dequantise-then-multiply form only by not rounding (v - z) * s to bf16 first.
+__device__ __forceinline__ bf16x8_t raw_operand_bf16(uint32_t q, uint32_t magic) {
+  const uint32_t e0 = and_or(q, 0x000f000fu, magic);
+  const uint32_t e1 = and_or(q >> 4, 0x000f000fu, magic);
+  const uint32_t e2 = and_or(q >> 8, 0x000f000fu, magic);
+  const uint32_t e3 = and_or(q >> 12, 0x000f000fu, magic);
+  return __builtin_bit_cast(bf16x8_t, u32x4_t{e0, e1, e2, e3});
+}
+
+// One unit's operands for the deferred-scale path, issued and awaited inside a
+// single asm block (a register must not be touched between the issue of the LDS
+// read that fills it and the counter wait): four weight chunks, four activation
+// slices, the lane's four zero-point words, and the 16 scales of the output
+// rows the lane holds (column 16 j + 4 (lane / 16) + r of the strip, register
+// 4 j + r).  O0..O15 are the byte offsets of those scales from `s_at`.
+#define SONAR_UNIT_READS(O0, O1, O2, O3, O4, O5, O6, O7, O8, O9, O10, O11, O12, O13, O14, O15)      \
+  asm volatile(                                                                                    \
+      "ds_read_b128 %0, %25\n\t"                                                                   \
+      "ds_read_b128 %1, %25 offset:1024\n\t"                                                       \
+      "ds_read_b128 %2, %25 offset:2048\n\t"                                                       \
+      "ds_read_b128 %3, %25 offset:3072\n\t"                                                       \
+      "ds_read_b128 %4, %26\n\t"                                                                   \
+      "ds_read_b128 %5, %26 offset:1024\n\t"                                                       \
+      "ds_read_b128 %6, %26 offset:2048\n\t"                                                       \
+      "ds_read_b128 %7, %26 offset:3072\n\t"                                                       \
+      "ds_read_b128 %8, %27\n\t"                                                                   \
+      "ds_read_u16 %9, %28 offset:" #O0 "\n\tds_read_u16 %10, %28 offset:" #O1 "\n\t"              \
+      "ds_read_u16 %11, %28 offset:" #O2 "\n\tds_read_u16 %12, %28 offset:" #O3 "\n\t"             \
+      "ds_read_u16 %13, %28 offset:" #O4 "\n\tds_read_u16 %14, %28 offset:" #O5 "\n\t"             \
+      "ds_read_u16 %15, %28 offset:" #O6 "\n\tds_read_u16 %16, %28 offset:" #O7 "\n\t"             \
+      "ds_read_u16 %17, %28 offset:" #O8 "\n\tds_read_u16 %18, %28 offset:" #O9 "\n\t"             \
+      "ds_read_u16 %19, %28 offset:" #O10 "\n\tds_read_u16 %20, %28 offset:" #O11 "\n\t"           \
+      "ds_read_u16 %21, %28 offset:" #O12 "\n\tds_read_u16 %22, %28 offset:" #O13 "\n\t"           \
+      "ds_read_u16 %23, %28 offset:" #O14 "\n\tds_read_u16 %24, %28 offset:" #O15 "\n\t"           \
+      "s_waitcnt lgkmcnt(0)"                                                                       \
+      : "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3), "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3),    \
+        "=&v"(row_z), "=&v"(row_s[0]), "=&v"(row_s[1]), "=&v"(row_s[2]), "=&v"(row_s[3]),          \
+        "=&v"(row_s[4]), "=&v"(row_s[5]), "=&v"(row_s[6]), "=&v"(row_s[7]), "=&v"(row_s[8]),       \
+        "=&v"(row_s[9]), "=&v"(row_s[10]), "=&v"(row_s[11]), "=&v"(row_s[12]), "=&v"(row_s[13]),   \
+        "=&v"(row_s[14]), "=&v"(row_s[15])                                                         \
+      : "v"(q_at), "v"(a_at), "v"(z_at), "v"(s_at)                                                 \
+      : "memory")
+
 template <typename T, bool HAS_ZP>
 __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams p,
                                                                              const int unit_group_shift) {
@@ -380,6 +431,15 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
 #pragma unroll
   for (int j = 0; j < 4; ++j) s_off[j] = kSlotS + 2 * scale_slot(16 * j + col16, grouped);
   const uint32_t z_off = kSlotS + 128 + 4 * zero_point_word(col16);
+  // deferred-scale path (bf16): where the scales / zero points of this lane's output rows sit
+  constexpr bool kDeferred = __is_same(T, __bf16);
+  const int q4 = lane >> 4;
+  const uint32_t row_s_off = kSlotS + (grouped ? 64 * (q4 & 1) + 2 * (q4 >> 1) : 32 * (q4 & 1) + 4 * (q4 >> 1));
+  const uint32_t row_z_off = kSlotS + 128 + 16 * (q4 & 1);
+  const uint32_t row_z_shift = 16 * (q4 >> 1);
+  const uint32_t magic_bf16 = magic_register(0x43004300u);
+  u32x4_t ones = u32x4_t{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  asm("" : "+v"(ones));
 
   // Issue order of a wavefront's copies, x being one of its units and W the
   // distance to its next one:  weights(x) | A(x), weights(x+W) | A(x+W),
@@ -465,34 +525,46 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     // copies of the units after it, then do the arithmetic.
     const uint32_t slot_lds = ring_lds + c_slot * kSlotBytes;
     u32x4_t q0, q1, q2, q3, a0, a1, a2, a3;
-    uint32_t sb0, sb1, sb2, sb3, zw;
+    uint32_t sb0 = 0, sb1 = 0, sb2 = 0, sb3 = 0, zw = 0;
+    uint32_t row_s[16];
+    u32x4_t row_z = u32x4_t{0u, 0u, 0u, 0u};
     const bool more = cur.index + kFastWaves < u_end;
     if (more) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightCopies) : "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    asm volatile(
-        "ds_read_b128 %0, %13\n\t"
-        "ds_read_b128 %1, %13 offset:1024\n\t"
-        "ds_read_b128 %2, %13 offset:2048\n\t"
-        "ds_read_b128 %3, %13 offset:3072\n\t"
-        "ds_read_b128 %4, %14\n\t"
-        "ds_read_b128 %5, %14 offset:1024\n\t"
-        "ds_read_b128 %6, %14 offset:2048\n\t"
-        "ds_read_b128 %7, %14 offset:3072\n\t"
-        "ds_read_u16 %8, %15\n\t"
-        "ds_read_u16 %9, %16\n\t"
-        "ds_read_u16 %10, %17\n\t"
-        "ds_read_u16 %11, %18\n\t"
-        "ds_read_b32 %12, %19\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3), "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3),
-          "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
-        : "v"(slot_lds + lane * 16), "v"(ring_lds + kWaveA + lane * 16), "v"(slot_lds + s_off[0]),
-          "v"(slot_lds + s_off[1]), "v"(slot_lds + s_off[2]), "v"(slot_lds + s_off[3]),
-          "v"(slot_lds + z_off)
-        : "memory");
+    if constexpr (kDeferred) {
+      const uint32_t q_at = slot_lds + lane * 16, a_at = ring_lds + kWaveA + lane * 16;
+      const uint32_t z_at = slot_lds + row_z_off, s_at = slot_lds + row_s_off;
+      if (grouped) {  // scale of (j, r) at byte 16 r + 4 j past s_at
+        SONAR_UNIT_READS(0, 16, 32, 48, 4, 20, 36, 52, 8, 24, 40, 56, 12, 28, 44, 60);
+      } else {        // at byte 64 (j >> 1) + 8 (j & 1) + 16 (r >> 1) + 2 (r & 1)
+        SONAR_UNIT_READS(0, 2, 16, 18, 8, 10, 24, 26, 64, 66, 80, 82, 72, 74, 88, 90);
+      }
+    } else {
+      asm volatile(
+          "ds_read_b128 %0, %13\n\t"
+          "ds_read_b128 %1, %13 offset:1024\n\t"
+          "ds_read_b128 %2, %13 offset:2048\n\t"
+          "ds_read_b128 %3, %13 offset:3072\n\t"
+          "ds_read_b128 %4, %14\n\t"
+          "ds_read_b128 %5, %14 offset:1024\n\t"
+          "ds_read_b128 %6, %14 offset:2048\n\t"
+          "ds_read_b128 %7, %14 offset:3072\n\t"
+          "ds_read_u16 %8, %15\n\t"
+          "ds_read_u16 %9, %16\n\t"
+          "ds_read_u16 %10, %17\n\t"
+          "ds_read_u16 %11, %18\n\t"
+          "ds_read_b32 %12, %19\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          : "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3), "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3),
+            "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
+          : "v"(slot_lds + lane * 16), "v"(ring_lds + kWaveA + lane * 16), "v"(slot_lds + s_off[0]),
+            "v"(slot_lds + s_off[1]), "v"(slot_lds + s_off[2]), "v"(slot_lds + s_off[3]),
+            "v"(slot_lds + z_off)
+          : "memory");
+    }
     if (more) {
       copy_activations(p, fl, fetch.unit, ring + kWaveA);
       fetch.advance(kFastWaves, p.units_per_strip);
@@ -500,22 +572,49 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
         copy_weights(p, fl, fetch.strip, fetch.unit, ring + c_slot * kSlotBytes, lane, unit_group_shift);
     }
 
-    Col cols[4];
-    const uint32_t sbits[4] = {sb0, sb1, sb2, sb3};
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int z = 8;
-      if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
-      cols[j] = Dq<T>::make_col((uint16_t)sbits[j], z);
-    }
     const u32x4_t qs[4] = {q0, q1, q2, q3};
     const u32x4_t as[4] = {a0, a1, a2, a3};
+    if constexpr (kDeferred) {
+      const floatx4_t zero4 = floatx4_t{0.f, 0.f, 0.f, 0.f};
+      floatx4_t part[4], asum;
 #pragma unroll
-    for (int cc = 0; cc < 4; ++cc) {
-      const vec8 av = __builtin_bit_cast(vec8, as[cc]);
-      const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
+      for (int cc = 0; cc < 4; ++cc) {
+        const bf16x8_t av = __builtin_bit_cast(bf16x8_t, as[cc]);
+        const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[j] = Dq<T>::mfma(Dq<T>::word(words[j], cols[j], magic), av, acc[j]);
+        for (int j = 0; j < 4; ++j)
+          part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(raw_operand_bf16(words[j], magic_bf16), av,
+                                                            cc == 0 ? zero4 : part[j], 0, 0, 0);
+        asum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ones), av,
+                                                       cc == 0 ? zero4 : asum, 0, 0, 0);
+      }
+      const uint32_t zrow[4] = {row_z.x >> row_z_shift, row_z.y >> row_z_shift, row_z.z >> row_z_shift,
+                                row_z.w >> row_z_shift};
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float sc = __builtin_bit_cast(float, row_s[4 * j + r] << 16);
+          float off = -136.f;
+          if (HAS_ZP) off = -128.f - (float)((zrow[r] >> (4 * j)) & 0xFu);
+          acc[j][r] = __builtin_fmaf(sc, __builtin_fmaf(off, asum[r], part[j][r]), acc[j][r]);
+        }
+    } else {
+      Col cols[4];
+      const uint32_t sbits[4] = {sb0, sb1, sb2, sb3};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        int z = 8;
+        if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
+        cols[j] = Dq<T>::make_col((uint16_t)sbits[j], z);
+      }
+#pragma unroll
+      for (int cc = 0; cc < 4; ++cc) {
+        const vec8 av = __builtin_bit_cast(vec8, as[cc]);
+        const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = Dq<T>::mfma(Dq<T>::word(words[j], cols[j], magic), av, acc[j]);
+      }
     }
     cur.advance(kFastWaves, p.units_per_strip);
     c_slot ^= 1;
