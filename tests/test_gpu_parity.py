@@ -104,6 +104,8 @@ GEMM_CASES = [
     (3, 14336, 4096, 128, False, False, False),
     (5, 4096, 28672, 128, False, False, False),
     (2, 4096, 6144, 128, False, False, False),
+    (2, 14336, 6144, 128, False, False, False),      # more than four activation slices per wavefront
+    (11, 4096, 512, 128, True, False, True),
 ]
 
 
