@@ -50,6 +50,10 @@ typedef __bf16 bf16x2_t __attribute__((ext_vector_type(2)));
 typedef __bf16 bf16x8_t __attribute__((ext_vector_type(8)));
 typedef float floatx2_t __attribute__((ext_vector_type(2)));
 typedef float floatx4_t __attribute__((ext_vector_type(4)));
+typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+// address spaces of the asynchronous global -> LDS copy builtin
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef __attribute__((address_space(1))) const void glb_void_t;
 
 // ---- layout constants -----------------------------------------------------
 // Marlin order: tiles of 16 (k) x 64 (n), 128 words each, stored k-tile major.

@@ -284,9 +284,6 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
 // tell which LDS bytes an asynchronous copy writes, so before any LDS access
 // it can see it would wait for every outstanding copy, which would drain the
 // prefetch on every unit.
-typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
-typedef __attribute__((address_space(3))) void lds_void_t;
-typedef __attribute__((address_space(1))) const void glb_void_t;
 
 constexpr int kFastWaves = 8;
 constexpr int kSlotS = 4096;       // inside a weight slot, after 4 chunks x 1 KiB: 64 scales, 8 zero-point words
@@ -864,7 +861,11 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   }
 
   static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
-  if (size_m > 64 && size_k % 64 == 0 && !no_tile)
+  // Up to 256 rows a problem with few 256 x 256 tiles leaves most compute units
+  // idle in the tile kernel; 64-row slabs of the streaming kernel use them all.
+  const int64_t tiles = ((size_m + 255) / 256) * ((size_n + 255) / 256);
+  const bool slabs = size_m <= 128 || (size_m <= 256 && tiles < 64);
+  if (size_m > 64 && size_k % 64 == 0 && !no_tile && !slabs)
     return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
                      size_k, num_groups, chk.group_size, st);
 

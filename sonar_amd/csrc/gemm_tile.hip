@@ -14,8 +14,9 @@
 // (D[n][m]) so a lane ends up with four consecutive columns of one row of C.
 //
 // Workgroup ids are dealt so that the 32 workgroups resident on one XCD (ids
-// congruent mod 8) take neighbouring tiles that share weight columns, which
-// keeps the packed weights in that XCD's L2.
+// congruent mod 8) take neighbouring tiles (tile_of_workgroup).
+#include <cstdlib>
+
 #include "dequant.hpp"
 
 namespace sonar {
@@ -61,6 +62,21 @@ __device__ __forceinline__ uint4 load_a16(const TileParams& p, int row, int k0) 
   return v;
 }
 
+// Workgroup id -> tile.  Workgroups whose ids are congruent mod 8 run on one
+// XCD and share its L2: each XCD takes a contiguous run of tiles, rows of A
+// innermost, so the workgroups resident on it share a few panels of W.
+// Returns false for the padding ids of the last run.
+__device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile_m, int& tile_n) {
+  const int total = p.tiles_m * p.tiles_n;
+  const int per_xcd = (total + 7) / 8;
+  const int id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
+  tile_n = id / p.tiles_m;
+  tile_m = id - tile_n * p.tiles_m;
+  return id < total;
+}
+
+inline int tile_grid(const TileParams& p) { return ((p.tiles_m * p.tiles_n + 7) / 8) * 8; }
+
 template <typename T, bool HAS_ZP, bool HAS_PERM>
 __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
@@ -75,14 +91,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const Tile
   const uint32_t magic = magic_register();
   const bool grouped = p.num_groups > 1;
 
-  // XCD-aware tile order: ids congruent mod 8 run on one XCD; give each XCD a
-  // contiguous run of tiles, rows of A innermost so neighbours share weights.
-  const int total = p.tiles_m * p.tiles_n;
-  const int per_xcd = (total + 7) / 8;
-  const int id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  if (id >= total) return;
-  const int tile_n = id / p.tiles_m;
-  const int tile_m = id - tile_n * p.tiles_m;
+  int tile_m, tile_n;
+  if (!tile_of_workgroup(p, tile_m, tile_n)) return;
   const int m0 = tile_m * kTileM;
   const int strip0 = tile_n * (kTileN / kStripN);
   const int strips_here = min(kTileN / kStripN, p.size_n / kStripN - strip0);
@@ -215,6 +225,260 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const Tile
   }
 }
 
+// ---------------------------------------------------------------------------
+// The same tile with every operand arriving through asynchronous global -> LDS
+// copies, three K steps deep, so no vector register holds bytes in flight and
+// the copies of step i+2 are issued before the matrix work of step i.
+//   * A: a ring of three 32-KiB stages shared by the workgroup; wavefront w
+//     copies both k blocks of row blocks w and w+8 of a stage.
+//   * W: the packed chunks are already in operand order, so each wavefront
+//     copies the two chunks of its own strip (and the scale / zero-point row of
+//     the step's group) into a private ring and dequantises them straight into
+//     MFMA operands; dequantised weights never pass through LDS.  The two
+//     wavefronts that share a strip each dequantise it.
+// Copies of a wavefront complete in issue order, seven per stage, so "stage i
+// has landed" is s_waitcnt vmcnt(7); one barrier per step then makes every
+// wavefront's share of A visible and frees the stage consumed in step i-1.
+// LDS is read from asm blocks only (the compiler cannot tell which LDS bytes a
+// copy writes and would otherwise wait for all copies before any LDS access).
+// Needs group_size % 64 == 0 (or one group) and no act-order.
+constexpr int kAsyncStages = 3;
+constexpr int kWaveStage = 2 * kBlockBytes + 256;   // two weight chunks + 64 scales + 8 zero-point words
+constexpr int kAsyncA = kAsyncStages * kStageA;
+constexpr int kAsyncLds = kAsyncA + kTileWaves * kAsyncStages * kWaveStage;
+constexpr int kAsyncCopies = 7;
+
+#define SONAR_TILE_A4(h_off)                                                                       \
+  asm volatile(                                                                                    \
+      "ds_read_b128 %0, %4 offset:" #h_off "\n\t"                                                  \
+      "ds_read_b128 %1, %4 offset:" #h_off "+2048\n\t"                                             \
+      "ds_read_b128 %2, %4 offset:" #h_off "+4096\n\t"                                             \
+      "ds_read_b128 %3, %4 offset:" #h_off "+6144\n\t"                                             \
+      "s_waitcnt lgkmcnt(0)"                                                                       \
+      : "=&v"(av[0]), "=&v"(av[1]), "=&v"(av[2]), "=&v"(av[3])                                     \
+      : "v"(a_at)                                                                                  \
+      : "memory")
+
+template <typename T, bool HAS_ZP>
+__global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(const TileParams p) {
+  typedef typename Dq<T>::vec8 vec8;
+  typedef typename Dq<T>::Col Col;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col16 = lane & 15;
+  const int kb = lane >> 4;
+  const uint32_t magic = magic_register();
+  const bool grouped = p.num_groups > 1;
+
+  int tile_m, tile_n;
+  if (!tile_of_workgroup(p, tile_m, tile_n)) return;
+  const int m0 = tile_m * kTileM;
+  const int strip0 = tile_n * (kTileN / kStripN);
+  const int strips_here = min(kTileN / kStripN, p.size_n / kStripN - strip0);
+  const int wm = wave >> 2;
+  const int wn = wave & 3;
+  const bool active = wn < strips_here;
+  // a wavefront past the last strip copies the last strip again and computes nothing
+  const int strip = strip0 + (active ? wn : strips_here - 1);
+
+  // ---- copy sources
+  const char* a_src[4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    // operand block of copy i: row block wave + 8 (i / 2), k block i % 2, so that the
+    // two halves of every 128-byte line of A are requested back to back by one wavefront
+    const int blk = 2 * (wave + 8 * (i >> 1)) + (i & 1);
+    int row = m0 + 16 * (blk >> 1) + col16;
+    if (row >= p.size_m) row = p.size_m - 1;  // rows past M are computed and never stored
+    a_src[i] = reinterpret_cast<const char*>(p.a) + ((long)row * p.lda + 32 * (blk & 1) + 8 * kb) * 2;
+  }
+  const uint4* b_src = p.b + (size_t)(unsigned)(strip * p.chunks_per_strip) * 64 + lane;
+  const char* s_src;
+  long s_group_stride;
+  if (HAS_ZP && lane >= 32) {
+    s_src = reinterpret_cast<const char*>(p.zeros + strip * 8 + (lane & 7));
+    s_group_stride = (long)(p.size_n / 8) * 4;
+  } else {
+    s_src = reinterpret_cast<const char*>(p.scales + strip * kStripN) + 4 * (lane & 31);
+    s_group_stride = (long)p.size_n * 2;
+  }
+  char* wring = smem + kAsyncA + wave * (kAsyncStages * kWaveStage);
+  const uint32_t a_lds = (uint32_t)(uintptr_t)(lds_void_t*)smem;
+  const uint32_t w_lds = (uint32_t)(uintptr_t)(lds_void_t*)wring;
+
+  auto issue = [&](int kt, int slot) {
+    char* sa = smem + slot * kStageA;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      __builtin_amdgcn_global_load_lds((glb_void_t*)(a_src[i] + (long)kt * (kTileK * 2)),
+                                       (lds_void_t*)(sa + (2 * (wave + 8 * (i >> 1)) + (i & 1)) * kBlockBytes), 16, 0,
+                                       0);
+    char* sw = wring + slot * kWaveStage;
+    const uint4* g = b_src + (size_t)(2 * kt) * 64;
+    __builtin_amdgcn_global_load_lds((glb_void_t*)g, (lds_void_t*)sw, 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((glb_void_t*)g, (lds_void_t*)sw, 16, 1024, 0);
+    const int grp = grouped ? (kt * kTileK) / p.group_size : 0;
+    __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)grp * s_group_stride),
+                                     (lds_void_t*)(sw + 2 * kBlockBytes), 4, 0, 0);
+  };
+
+  uint32_t s_off[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) s_off[j] = 2 * kBlockBytes + 2 * scale_slot(16 * j + col16, grouped);
+  const uint32_t z_off = 2 * kBlockBytes + 128 + 4 * zero_point_word(col16);
+
+  floatx4_t acc[4][8];
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < 8; ++mb) acc[nb][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+  const int k_tiles = p.size_k / kTileK;
+  issue(0, 0);
+  if (k_tiles > 1) issue(1, 1);
+
+  // Dequantisation runs in the shadow of the matrix work, half a step ahead:
+  // while the MFMAs of k block 0 run, k block 1 of the same step is
+  // dequantised (wv[1]); while those of k block 1 run, k block 0 of the next
+  // step (wv[0]), whose packed words sit in the wavefront's private ring and
+  // need no barrier.  qb holds the packed words of k block 1 in between.
+  vec8 wv[2][4];
+  u32x4_t qa, qb;
+  uint32_t sb0, sb1, sb2, sb3, zw;
+  Col cols[4];
+  auto make_cols = [&]() {
+    const uint32_t sbits[4] = {sb0, sb1, sb2, sb3};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int z = 8;
+      if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
+      cols[j] = Dq<T>::make_col((uint16_t)sbits[j], z);
+    }
+  };
+#define SONAR_TILE_W(w_at)                                                                         \
+  asm volatile(                                                                                    \
+      "ds_read_b128 %0, %7\n\t"                                                                    \
+      "ds_read_b128 %1, %7 offset:1024\n\t"                                                        \
+      "ds_read_u16 %2, %8\n\t"                                                                     \
+      "ds_read_u16 %3, %9\n\t"                                                                     \
+      "ds_read_u16 %4, %10\n\t"                                                                    \
+      "ds_read_u16 %5, %11\n\t"                                                                    \
+      "ds_read_b32 %6, %12\n\t"                                                                    \
+      "s_waitcnt lgkmcnt(0)"                                                                       \
+      : "=&v"(qa), "=&v"(qb), "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)            \
+      : "v"((w_at) + lane * 16), "v"((w_at) + s_off[0]), "v"((w_at) + s_off[1]),                   \
+        "v"((w_at) + s_off[2]), "v"((w_at) + s_off[3]), "v"((w_at) + z_off)                        \
+      : "memory")
+#define SONAR_TILE_MFMA16(h, mb0)                                                                  \
+  _Pragma("unroll") for (int i = 0; i < 4; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j)      \
+      acc[j][(mb0) + i] = Dq<T>::mfma(wv[h][j], __builtin_bit_cast(vec8, av[i]), acc[j][(mb0) + i])
+  if (active) {
+    if (k_tiles > 1) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    SONAR_TILE_W(w_lds);
+    make_cols();
+    wv[0][0] = Dq<T>::word(qa.x, cols[0], magic);
+    wv[0][1] = Dq<T>::word(qa.y, cols[1], magic);
+    wv[0][2] = Dq<T>::word(qa.z, cols[2], magic);
+    wv[0][3] = Dq<T>::word(qa.w, cols[3], magic);
+  }
+
+  int slot = 0;        // stage of step kt
+  int fill = 2;        // stage step kt + 2 goes to
+  for (int kt = 0; kt < k_tiles; ++kt) {
+    if (kt + 1 < k_tiles) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    }
+    __builtin_amdgcn_s_barrier();
+    if (kt + 2 < k_tiles) issue(kt + 2, fill);
+
+    if (active) {
+      const uint32_t a_at = a_lds + slot * kStageA + (8 * wm * 2) * kBlockBytes + lane * 16;
+      const int next_slot = slot == kAsyncStages - 1 ? 0 : slot + 1;
+      const bool has_next = kt + 1 < k_tiles;
+      u32x4_t av[4];
+      SONAR_TILE_A4(0);
+      wv[1][0] = Dq<T>::word(qb.x, cols[0], magic);
+      wv[1][1] = Dq<T>::word(qb.y, cols[1], magic);
+      SONAR_TILE_MFMA16(0, 0);
+      SONAR_TILE_A4(8192);
+      wv[1][2] = Dq<T>::word(qb.z, cols[2], magic);
+      wv[1][3] = Dq<T>::word(qb.w, cols[3], magic);
+      SONAR_TILE_MFMA16(0, 4);
+      if (has_next) {
+        // stage kt + 1 has landed once at most the copies of stage kt + 2 are outstanding
+        if (kt + 2 < k_tiles) {
+          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
+        } else {
+          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        }
+        SONAR_TILE_W(w_lds + next_slot * kWaveStage);
+      }
+      SONAR_TILE_A4(1024);
+      if (has_next) {
+        make_cols();
+        wv[0][0] = Dq<T>::word(qa.x, cols[0], magic);
+        wv[0][1] = Dq<T>::word(qa.y, cols[1], magic);
+      }
+      SONAR_TILE_MFMA16(1, 0);
+      SONAR_TILE_A4(9216);
+      if (has_next) {
+        wv[0][2] = Dq<T>::word(qa.z, cols[2], magic);
+        wv[0][3] = Dq<T>::word(qa.w, cols[3], magic);
+      }
+      SONAR_TILE_MFMA16(1, 4);
+    }
+    slot = slot == kAsyncStages - 1 ? 0 : slot + 1;
+    fill = fill == kAsyncStages - 1 ? 0 : fill + 1;
+  }
+#undef SONAR_TILE_MFMA16
+#undef SONAR_TILE_W
+
+  if (!active) return;
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) {
+    const int n = strip * kStripN + 16 * nb + 4 * kb;
+    float bias[4] = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        bias[r] = Dq<T>::to_float(p.bias[strip * kStripN + scale_slot(16 * nb + 4 * kb + r, false)]);
+    }
+#pragma unroll
+    for (int mb = 0; mb < 8; ++mb) {
+      const int m = m0 + 128 * wm + 16 * mb + col16;
+      if (m < p.size_m) {
+        const floatx4_t v = acc[nb][mb];
+        uint2 o;
+        o.x = (uint32_t)Dq<T>::from_float(v.x + bias[0]) | ((uint32_t)Dq<T>::from_float(v.y + bias[1]) << 16);
+        o.y = (uint32_t)Dq<T>::from_float(v.z + bias[2]) | ((uint32_t)Dq<T>::from_float(v.w + bias[3]) << 16);
+        *reinterpret_cast<uint2*>(p.c + (long)m * p.size_n + n) = o;
+      }
+    }
+  }
+}
+
+template <typename T, bool HAS_ZP>
+int launch_tile_async(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, HAS_ZP>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kAsyncLds));
+    attr_set = true;
+  }
+  const int grid = tile_grid(p);
+  marlin_tile_async_kernel<T, HAS_ZP><<<grid, kTileWaves * 64, kAsyncLds, st>>>(p);
+  return SONAR_OK;
+}
+
 template <typename T, bool HAS_ZP, bool HAS_PERM>
 int launch_tile(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
@@ -223,8 +487,7 @@ int launch_tile(const TileParams& p, hipStream_t st) {
                                   hipFuncAttributeMaxDynamicSharedMemorySize, kTileLds));
     attr_set = true;
   }
-  const int total = p.tiles_m * p.tiles_n;
-  const int grid = ((total + 7) / 8) * 8;
+  const int grid = tile_grid(p);
   marlin_tile_kernel<T, HAS_ZP, HAS_PERM><<<grid, kTileWaves * 64, kTileLds, st>>>(p);
   return SONAR_OK;
 }
@@ -255,6 +518,15 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);
   const bool zp = zeros != nullptr, pm = perm != nullptr;
   int rc;
+  static const bool no_async = getenv("SONAR_MARLIN_NO_ASYNC_TILE") != nullptr;  // debugging aid
+  if (!pm && !no_async && (num_groups == 1 || group_size % kTileK == 0)) {
+    if (dtype == SONAR_DTYPE_F16)
+      rc = zp ? launch_tile_async<_Float16, true>(p, st) : launch_tile_async<_Float16, false>(p, st);
+    else
+      rc = zp ? launch_tile_async<__bf16, true>(p, st) : launch_tile_async<__bf16, false>(p, st);
+    if (rc) return rc;
+    return launch_status("marlin_tile_async_kernel");
+  }
   if (dtype == SONAR_DTYPE_F16) {
     rc = zp ? (pm ? launch_tile<_Float16, true, true>(p, st) : launch_tile<_Float16, true, false>(p, st))
             : (pm ? launch_tile<_Float16, false, true>(p, st) : launch_tile<_Float16, false, false>(p, st));
