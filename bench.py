@@ -105,6 +105,110 @@ def cpu_baseline(threads: int):
             "gflops": round(2 * m * n * k / t_full / 1e9, 2)}
 
 
+def variants_sweep(torch, ops, gen, time_graph):
+    """K = 4096, N = 11008 at M = 1 and 512: act-order (perm gathers the columns
+    of A, weights repacked in sorted-group order) and AWQ (per-group zero points)."""
+    from sonar_amd import marlin_utils
+    from sonar_amd.scalar_type import scalar_types
+    dev = "cuda:0"
+    k, n = 4096, 11008
+    out = []
+    for name in ("act_order", "awq"):
+        layers = []
+        for _ in range(6):
+            qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, 2 * n), dtype=torch.int32, device=dev, generator=gen)
+            sc = (torch.rand((k // GROUP, n), device=dev, generator=gen) * 9e-3 + 1e-3).to(torch.float16)
+            ws = marlin_utils.marlin_make_workspace_new(torch.device(dev))
+            empty = torch.empty(0, dtype=torch.int32, device=dev)
+            if name == "act_order":
+                g_idx = (torch.arange(k, device=dev) // GROUP).to(torch.int32)
+                perm = torch.randperm(k, device=dev, generator=gen).to(torch.int32)
+                layers.append((qw, sc, empty, g_idx, perm, ws, scalar_types.uint4b8))
+            else:
+                zp = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // GROUP, n // 8), dtype=torch.int32, device=dev,
+                                   generator=gen)
+                layers.append((qw, sc, zp, empty, empty, ws, scalar_types.uint4))
+        for m in (1, 512):
+            a = torch.randn((m, k), device=dev, generator=gen).to(torch.float16)
+
+            def one(i=0, a=a, m=m):
+                qw, sc, zp, g_idx, perm, ws, wt = layers[i % len(layers)]
+                ops.marlin_gemm(a, None, qw, None, sc, None, None, zp, g_idx, perm, ws, wt, m, n, k, True,
+                                False, True, False)
+            s = time_graph(torch, one, 24 if m == 1 else 6)
+            nb = algorithmic_bytes(m, k, n, zeros=name == "awq", act_order=name == "act_order")
+            fl = 2 * m * k * n
+            out.append({"variant": name, "m": m, "k": k, "n": n, "us": round(s * 1e6, 2),
+                        "GBps": round(nb / s / 1e9, 1), "TFLOPs": round(fl / s / 1e12, 2),
+                        "frac_hbm": round(nb / s / 1e9 / HBM_PEAK_GBPS, 4),
+                        "frac_mfma": round(fl / s / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+            print("variant", json.dumps(out[-1]), file=sys.stderr, flush=True)
+    return out
+
+
+def moe_sweep(torch, gen, time_graph):
+    """Mixtral-8x7B-shaped grouped GEMMs (8 experts, hidden 4096, intermediate
+    14336, top-2, bf16) at T = 16 and 4096 tokens: gate/up GEMM, down GEMM and
+    the whole layer (routing + both GEMMs + activation + sum)."""
+    from sonar_amd import fused_moe, ops
+    from sonar_amd.scalar_type import scalar_types
+    dev = "cuda:0"
+    e, hidden, inter, topk = 8, 4096, 14336, 2
+    dt = torch.bfloat16
+    w1 = torch.randint(-2 ** 31, 2 ** 31 - 1, (e, hidden // 16, 2 * 2 * inter), dtype=torch.int32, device=dev,
+                       generator=gen)
+    w2 = torch.randint(-2 ** 31, 2 ** 31 - 1, (e, inter // 16, 2 * hidden), dtype=torch.int32, device=dev,
+                       generator=gen)
+    s1 = (torch.rand((e, hidden // GROUP, 2 * inter), device=dev, generator=gen) * 9e-3 + 1e-3).to(dt)
+    s2 = (torch.rand((e, inter // GROUP, hidden), device=dev, generator=gen) * 9e-3 + 1e-3).to(dt)
+    out = []
+    for t in (16, 4096):
+        x = torch.randn((t, hidden), device=dev, generator=gen).to(dt)
+        logits = torch.randn((t, e), device=dev, generator=gen)
+        tw, ti = torch.topk(torch.softmax(logits, dim=1), topk, dim=1)
+        ti = ti.to(torch.int32)
+        bs = fused_moe.moe_block_size(t, topk, e)
+        sorted_ids, expert_ids, past = fused_moe.moe_align_block_size(ti, bs, e)
+        ws = torch.zeros(1024, dtype=torch.int32, device=dev)
+        h1 = torch.empty((t * topk, 2 * inter), dtype=dt, device=dev)
+        h2 = torch.randn((t * topk, inter), device=dev, generator=gen).to(dt)
+        y = torch.empty((t * topk, hidden), dtype=dt, device=dev)
+        routed = int(torch.unique(ti).numel())
+
+        def gemm1(i=0):
+            ops.moe_wna16_marlin_gemm(x, h1, w1, None, s1, None, None, None, None, None, ws, sorted_ids,
+                                      expert_ids, past, tw, bs, topk, False, scalar_types.uint4b8, t, 2 * inter,
+                                      hidden, True, False, True, False)
+
+        def gemm2(i=0):
+            ops.moe_wna16_marlin_gemm(h2, y, w2, None, s2, None, None, None, None, None, ws, sorted_ids,
+                                      expert_ids, past, tw, bs, 1, True, scalar_types.uint4b8, t * topk, hidden,
+                                      inter, True, False, True, False)
+
+        def layer(i=0):
+            fused_moe.fused_marlin_moe(x, w1, w2, None, None, s1, s2, tw, ti, scalar_types.uint4b8.id)
+
+        reps = 8 if t == 16 else 2
+        for name, fn, k, n, rows in (("gate_up", gemm1, hidden, 2 * inter, t), ("down", gemm2, inter, hidden, t * topk)):
+            s = time_graph(torch, fn, reps)
+            weights = routed * (k * n // 2 + (k // GROUP) * n * 2)
+            nb = weights + rows * k * 2 + t * topk * n * 2 + sorted_ids.numel() * 4 + expert_ids.numel() * 4
+            fl = 2 * t * topk * n * k
+            out.append({"tokens": t, "gemm": name, "block_size": bs, "experts_routed": routed,
+                        "us": round(s * 1e6, 1), "GBps": round(nb / s / 1e9, 1), "TFLOPs": round(fl / s / 1e12, 2),
+                        "frac_hbm": round(nb / s / 1e9 / HBM_PEAK_GBPS, 4),
+                        "frac_mfma": round(fl / s / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+            print("moe", json.dumps(out[-1]), file=sys.stderr, flush=True)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(reps):
+            layer()
+        torch.cuda.synchronize()
+        out.append({"tokens": t, "gemm": "whole layer (eager)", "us": round((time.perf_counter() - t0) / reps * 1e6, 1)})
+        print("moe", json.dumps(out[-1]), file=sys.stderr, flush=True)
+    return out
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -236,6 +340,8 @@ def main() -> int:
                                   "frac_mfma": round(fl / s / 1e12 / MFMA_PEAK_TFLOPS, 4)})
                     print("sweep", json.dumps(sweep[-1]), file=sys.stderr, flush=True)
         out["sweep"] = sweep
+        out["variants"] = variants_sweep(torch, ops, gen, time_graph)
+        out["moe"] = moe_sweep(torch, gen, time_graph)
 
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(min(os.cpu_count() or 1, 16))

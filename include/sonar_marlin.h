@@ -104,7 +104,10 @@ size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n, int64_t s
  *                is_k_full == 0)
  *   workspace    int32[workspace_len], all zero on entry, all zero on exit;
  *                workspace_len >= number of compute units
- *   scratch      sonar_marlin_gemm_scratch_bytes() bytes, contents don't care
+ *   scratch      sonar_marlin_gemm_scratch_bytes() bytes, contents don't care;
+ *                an act-order call given size_m * size_k * 2 bytes more uses
+ *                them for a column-permuted copy of A, which is much faster
+ *                than gathering A inside the GEMM
  * use_atomic_add and use_fp32_reduce are accepted for signature parity; the
  * reduction is always fp32 and deterministic. */
 int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
@@ -146,6 +149,35 @@ int sonar_moe_wna16_marlin_gemm(
     int mul_topk_weights, int64_t num_experts, int dtype, int64_t b_type_id,
     int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
     int is_k_full, int use_atomic_add, int use_fp32_reduce, void* stream);
+
+/* The small kernels around the two grouped GEMMs of a mixture-of-experts layer.
+ * They have counterparts in every build of the reference (also on ROCm):
+ *   sonar_moe_align_block_size -> _moe_C::moe_align_block_size
+ *        csrc/libtorch_stable/moe/torch_bindings.cpp:36-41,
+ *        csrc/libtorch_stable/moe/moe_align_sum_kernels.cu:626-725
+ *   sonar_moe_sum              -> _moe_C::moe_sum (moe_align_sum_kernels.cu:759+)
+ *   sonar_silu_and_mul         -> _C::silu_and_mul
+ *        csrc/libtorch_stable/torch_bindings.cpp:640, activation_kernels.cu
+ * so the torch layer registers them under its own namespace, not under _C.
+ *
+ * sonar_moe_align_block_size: topk_ids int32[numel] (expert of every
+ * (token, k) slot).  Slots are grouped by expert, ascending slot id inside an
+ * expert, every expert's run padded to a multiple of block_size with the
+ * sentinel `numel`; expert_ids[b] is the expert of block b, -1 past the
+ * padded total, which goes to num_tokens_post_pad[0].  With expert_map
+ * (int32[num_experts], -1 = absent) slots of absent experts are dropped and
+ * experts are numbered and ordered by their mapped ids.  sorted_len must be
+ * at least numel + num_experts * (block_size - 1) (or numel * block_size when
+ * that is smaller and numel < num_experts); offsets_scratch is int32[num_experts].
+ * sonar_silu_and_mul: out[rows][d] = T(T(silu(in[r][c])) * in[r][d + c]),
+ * in is [rows][2 d].  sonar_moe_sum: out[tokens][d] = T(sum_k in[t][k][d]) in fp32. */
+int sonar_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int64_t num_experts,
+                               int64_t block_size, int32_t* sorted_token_ids, int64_t sorted_len,
+                               int32_t* expert_ids, int64_t expert_len, int32_t* num_tokens_post_pad,
+                               const int32_t* expert_map, int32_t* offsets_scratch, void* stream);
+int sonar_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int dtype, void* stream);
+int sonar_moe_sum(void* out, const void* in, int64_t tokens, int64_t topk, int64_t d, int dtype,
+                  void* stream);
 
 #ifdef __cplusplus
 }

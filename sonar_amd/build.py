@@ -14,7 +14,7 @@ LIB_PATH = os.path.join(LIB_DIR, "libsonar_marlin.so")
 OPS_PATH = os.path.join(LIB_DIR, "libsonar_marlin_torch.so")
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-HIP_SOURCES = ["repack.hip", "gemm_stream.hip", "gemm_tile.hip", "gemm_moe.hip"]
+HIP_SOURCES = ["repack.hip", "gemm_stream.hip", "gemm_tile.hip", "gemm_moe.hip", "moe_aux.hip"]
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

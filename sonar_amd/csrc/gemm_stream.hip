@@ -695,6 +695,30 @@ int cu_count() {
   return cached;
 }
 
+// A'[m][k] = A[m][perm[k]]: with act-order weights (rows in sorted-group order)
+// the GEMM on A' is a plain grouped GEMM, which every kernel here runs without
+// gathering (the reference permutes A the same way, marlin.cu:760-762).
+__global__ __launch_bounds__(256) void permute_columns_kernel(const uint16_t* __restrict__ a, long lda,
+                                                             const int32_t* __restrict__ perm,
+                                                             uint16_t* __restrict__ out, int size_m,
+                                                             int size_k) {
+  const int per_row = size_k / 8;
+  const long total = (long)size_m * per_row;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const int m = (int)(i / per_row);
+    const int k0 = (int)(i - (long)m * per_row) * 8;
+    const uint16_t* arow = a + (long)m * lda;
+    const int4 p0 = *reinterpret_cast<const int4*>(perm + k0);
+    const int4 p1 = *reinterpret_cast<const int4*>(perm + k0 + 4);
+    uint4 v;
+    v.x = (uint32_t)arow[p0.x] | ((uint32_t)arow[p0.y] << 16);
+    v.y = (uint32_t)arow[p0.z] | ((uint32_t)arow[p0.w] << 16);
+    v.z = (uint32_t)arow[p1.x] | ((uint32_t)arow[p1.y] << 16);
+    v.w = (uint32_t)arow[p1.z] | ((uint32_t)arow[p1.w] << 16);
+    *reinterpret_cast<uint4*>(out + (long)m * size_k + k0) = v;
+  }
+}
+
 template <typename T, int MB, bool HAS_ZP>
 void launch_stream(const StreamParams& p, bool has_perm, hipStream_t st) {
   if (has_perm)
@@ -822,6 +846,23 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   SONAR_REQUIRE(scratch && scratch_bytes >= sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k),
                 "scratch of %zu bytes is too small", scratch_bytes);
 
+  hipStream_t st = (hipStream_t)stream;
+  // Act-order with room in the scratch buffer for a copy of A: permute the
+  // columns of A once and run the plain grouped kernels on the copy.
+  const size_t base_scratch = sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k);
+  if (chk.has_perm && scratch_bytes >= base_scratch + (size_t)size_m * size_k * 2) {
+    uint16_t* a_tmp = reinterpret_cast<uint16_t*>(static_cast<char*>(scratch) + base_scratch);
+    const long vecs = (long)size_m * (size_k / 8);
+    const int blocks = (int)((vecs + 255) / 256 < 4096 ? (vecs + 255) / 256 : 4096);
+    permute_columns_kernel<<<blocks, 256, 0, st>>>(static_cast<const uint16_t*>(a), a_row_stride, perm, a_tmp,
+                                                   (int)size_m, (int)size_k);
+    if (int rc = launch_status("permute_columns_kernel")) return rc;
+    a = a_tmp;
+    a_row_stride = size_k;
+    perm = nullptr;
+    chk.has_perm = false;
+  }
+
   StreamParams p;
   p.b = reinterpret_cast<const uint4*>(b_q_weight);
   p.bias = static_cast<const uint16_t*>(b_bias);
@@ -842,7 +883,6 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                 (long)size_n);
   p.total_units = (int)total_units;
   p.parts = p.total_units < cus ? p.total_units : cus;
-  hipStream_t st = (hipStream_t)stream;
 
   bool any_split = false;
   for (int i = 1; i < p.parts && !any_split; ++i)

@@ -281,7 +281,8 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
               "workspace must be a contiguous int32 GPU tensor");
 
   Tensor native = native_weights(b_q_weight, size_k, size_n, 1);
-  const size_t scratch_bytes = sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k);
+  size_t scratch_bytes = sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k);
+  if (perm != nullptr) scratch_bytes += (size_t)size_m * size_k * 2;  // room for the column-permuted copy of A
   Tensor scratch = at::empty({(int64_t)scratch_bytes}, a.options().dtype(at::kByte));
 
   raise_if_failed(sonar_marlin_gemm(
@@ -411,7 +412,72 @@ Tensor moe_wna16_marlin_gemm(
   return c;
 }
 
+// ---------------------------------------------------------------- MoE helper ops
+void moe_align_block_size(const Tensor& topk_ids, int64_t num_experts, int64_t block_size,
+                          Tensor& sorted_token_ids, Tensor& experts_ids, Tensor& num_tokens_post_pad,
+                          const OptTensor& maybe_expert_map) {
+  TORCH_CHECK(topk_ids.is_cuda() && topk_ids.is_contiguous() && topk_ids.scalar_type() == at::kInt,
+              "topk_ids must be a contiguous int32 GPU tensor");
+  for (const Tensor* t : {&sorted_token_ids, &experts_ids, &num_tokens_post_pad})
+    TORCH_CHECK(t->is_cuda() && t->is_contiguous() && t->scalar_type() == at::kInt,
+                "outputs must be contiguous int32 GPU tensors");
+  const int32_t* map = nullptr;
+  if (maybe_expert_map.has_value()) {
+    const Tensor& m = maybe_expert_map.value();
+    TORCH_CHECK(m.is_cuda() && m.is_contiguous() && m.scalar_type() == at::kInt && m.numel() == num_experts,
+                "expert_map must be a contiguous int32 GPU tensor of num_experts entries");
+    map = static_cast<const int32_t*>(m.const_data_ptr());
+  }
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(topk_ids.device());
+  Tensor offsets = at::empty({num_experts}, topk_ids.options());
+  raise_if_failed(sonar_moe_align_block_size(
+      static_cast<const int32_t*>(topk_ids.const_data_ptr()), topk_ids.numel(), num_experts, block_size,
+      static_cast<int32_t*>(sorted_token_ids.mutable_data_ptr()), sorted_token_ids.numel(),
+      static_cast<int32_t*>(experts_ids.mutable_data_ptr()), experts_ids.numel(),
+      static_cast<int32_t*>(num_tokens_post_pad.mutable_data_ptr()), map,
+      static_cast<int32_t*>(offsets.mutable_data_ptr()), current_stream(topk_ids)));
+}
+
+void silu_and_mul(Tensor& result, const Tensor& input) {
+  TORCH_CHECK(input.is_cuda() && input.is_contiguous() && result.is_cuda() && result.is_contiguous(),
+              "silu_and_mul needs contiguous GPU tensors");
+  TORCH_CHECK(result.scalar_type() == input.scalar_type(), "result must have the dtype of input");
+  const int64_t d = input.size(-1) / 2;
+  TORCH_CHECK(input.size(-1) == 2 * d && result.size(-1) == d && result.numel() * 2 == input.numel(),
+              "result must be input with the last dimension halved");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+  raise_if_failed(sonar_silu_and_mul(result.mutable_data_ptr(), input.const_data_ptr(), input.numel() / (2 * d),
+                                     d, dtype_code(input), current_stream(input)));
+}
+
+void moe_sum(const Tensor& input, Tensor& output) {
+  TORCH_CHECK(input.is_cuda() && input.is_contiguous() && output.is_cuda() && output.is_contiguous(),
+              "moe_sum needs contiguous GPU tensors");
+  TORCH_CHECK(input.dim() == 3 && output.dim() == 2 && output.size(0) == input.size(0) &&
+                  output.size(1) == input.size(2), "moe_sum: input [tokens, topk, d], output [tokens, d]");
+  TORCH_CHECK(output.scalar_type() == input.scalar_type(), "output must have the dtype of input");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+  raise_if_failed(sonar_moe_sum(output.mutable_data_ptr(), input.const_data_ptr(), input.size(0), input.size(1),
+                                input.size(2), dtype_code(input), current_stream(input)));
+}
+
 }  // namespace
+
+// Ops every build of the reference already has under _C / _moe_C (they are not
+// CUDA-only there); registered under a namespace of their own so that loading
+// this library next to the reference's extension defines nothing twice.
+TORCH_LIBRARY(sonar_amd, m) {
+  m.def(
+      "moe_align_block_size(Tensor topk_ids, int num_experts, int block_size, Tensor! sorted_token_ids, "
+      "Tensor! experts_ids, Tensor! num_tokens_post_pad, Tensor? maybe_expert_map) -> ()");
+  m.def("silu_and_mul(Tensor! result, Tensor input) -> ()");
+  m.def("moe_sum(Tensor input, Tensor! output) -> ()");
+}
+TORCH_LIBRARY_IMPL(sonar_amd, CUDA, m) {
+  m.impl("moe_align_block_size", &moe_align_block_size);
+  m.impl("silu_and_mul", &silu_and_mul);
+  m.impl("moe_sum", &moe_sum);
+}
 
 TORCH_LIBRARY_FRAGMENT(_C, m) {
   m.def(

@@ -4,9 +4,11 @@ and the two grouped W4A16 GEMMs around the gated activation.
 Mirrors aphrodite/model_executor/layers/fused_moe/moe_align_block_size.py:11-101
 (`moe_align_block_size`) and .../fused_moe/experts/marlin_moe.py:57-392
 (`fused_marlin_moe`) for 4-bit integer weights with fp16 / bf16 activations.
-The routing, the activation and the final sum are torch expressions that never
-read a device value on the host, so the whole layer can be recorded in a HIP
-graph; the two GEMMs are the `_moe_C::moe_wna16_marlin_gemm` op.
+On the GPU the routing, the activation and the final sum are the HIP kernels
+behind `torch.ops.sonar_amd.{moe_align_block_size, silu_and_mul, moe_sum}`; the
+torch expressions kept here serve CPU tensors (and the tests of those kernels).
+Neither reads a device value on the host, so the whole layer can be recorded
+in a HIP graph; the two GEMMs are the `_moe_C::moe_wna16_marlin_gemm` op.
 """
 from __future__ import annotations
 
@@ -53,12 +55,38 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
         max_num_tokens_padded = min(numel * block_size, max_num_tokens_padded)
     max_blocks = -(-max_num_tokens_padded // block_size)
 
+    if topk_ids.is_cuda:
+        sorted_ids = torch.empty((max_num_tokens_padded,), dtype=torch.int32, device=dev)
+        expert_ids = torch.empty((max_blocks,), dtype=torch.int32, device=dev)
+        num_tokens_post_pad = torch.empty((1,), dtype=torch.int32, device=dev)
+        ids = topk_ids if topk_ids.dtype == torch.int32 else topk_ids.to(torch.int32)
+        emap = None
+        if expert_map is not None and ignore_invalid_experts:
+            emap = expert_map if expert_map.dtype == torch.int32 else expert_map.to(torch.int32)
+        torch.ops.sonar_amd.moe_align_block_size(ids.contiguous(), num_experts, block_size, sorted_ids,
+                                                 expert_ids, num_tokens_post_pad, emap)
+        if expert_map is not None and not ignore_invalid_experts:
+            mapped = expert_map.to(torch.int32)[expert_ids.clamp(min=0).to(torch.int64)]
+            expert_ids = torch.where(expert_ids >= 0, mapped, expert_ids)
+        return sorted_ids, expert_ids, num_tokens_post_pad
+    return _moe_align_block_size_torch(topk_ids, block_size, num_experts, expert_map, ignore_invalid_experts,
+                                       max_num_tokens_padded, max_blocks)
+
+
+def _moe_align_block_size_torch(topk_ids, block_size, num_experts, expert_map, ignore_invalid_experts,
+                                max_num_tokens_padded, max_blocks):
+    """The same routing as torch expressions (any device)."""
+    numel = topk_ids.numel()
+    dev = topk_ids.device
     flat = topk_ids.reshape(-1).to(torch.int64)
     valid = (flat >= 0) & (flat < num_experts)
+    key = flat
     if expert_map is not None and ignore_invalid_experts:
-        valid &= expert_map.to(torch.int64)[flat.clamp(0, num_experts - 1)] >= 0
+        # experts are numbered and ordered by their mapped (local) ids
+        key = expert_map.to(torch.int64)[flat.clamp(0, num_experts - 1)]
+        valid &= (key >= 0) & (key < num_experts)
     # invalid slots sort behind every expert and are never placed
-    key = torch.where(valid, flat, torch.full_like(flat, num_experts))
+    key = torch.where(valid, key, torch.full_like(flat, num_experts))
     counts = torch.zeros(num_experts + 1, dtype=torch.int64, device=dev).scatter_add_(
         0, key, torch.ones_like(key))[:num_experts]
     padded = (counts + block_size - 1) // block_size * block_size
@@ -81,7 +109,7 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     total = pad_end[-1]
     in_range = block_start < total
     expert_ids = torch.where(in_range, expert_of_block, torch.full_like(expert_of_block, -1))
-    if expert_map is not None:
+    if expert_map is not None and not ignore_invalid_experts:
         mapped = expert_map.to(torch.int64)[expert_ids.clamp(0, num_experts - 1)]
         expert_ids = torch.where(in_range, mapped, expert_ids)
     return sorted_ids, expert_ids.to(torch.int32), total.to(torch.int32).reshape(1)
@@ -90,8 +118,19 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
 def silu_and_mul(out: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     """out = silu(x[:, :d]) * x[:, d:] in the tensor's own dtype."""
     d = x.shape[-1] // 2
+    if x.is_cuda and x.is_contiguous() and out.is_contiguous() and d % 8 == 0:
+        torch.ops.sonar_amd.silu_and_mul(out, x)
+        return out
     torch.mul(torch.nn.functional.silu(x[..., :d]), x[..., d:], out=out)
     return out
+
+
+def moe_sum(moe_output: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+    """out[t] = sum over k of moe_output[t, k], accumulated in fp32."""
+    if moe_output.is_cuda and moe_output.is_contiguous() and out.is_contiguous() and out.shape[-1] % 8 == 0:
+        torch.ops.sonar_amd.moe_sum(moe_output, out)
+        return out
+    return torch.sum(moe_output, dim=1, out=out)
 
 
 def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, num_topk,
@@ -182,10 +221,10 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
         w1_zeros=w1_zeros, w2_zeros=w2_zeros, workspace=workspace,
         intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2, output=None,
         is_k_full=is_k_full).view(-1, topk, K)
+    if output is None:
+        output = torch.empty_like(hidden_states)
     if expert_map is not None:
         # slots of experts held elsewhere were never written
         local = expert_map.to(torch.int64)[topk_ids.to(torch.int64).clamp(0, global_num_experts - 1)] >= 0
         moe_output = torch.where(local.unsqueeze(-1), moe_output, torch.zeros_like(moe_output))
-    if output is None:
-        output = torch.empty_like(hidden_states)
-    return torch.sum(moe_output, dim=1, out=output)
+    return moe_sum(moe_output.contiguous(), output)

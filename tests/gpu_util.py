@@ -107,12 +107,12 @@ class DeviceLayer:
         props = torch.cuda.get_device_properties(0)
         self.workspace = torch.zeros(props.multi_processor_count, dtype=torch.int32, device=DEV)
 
-    def gemm(self, a: torch.Tensor, m: int, is_k_full: bool = True) -> torch.Tensor:
+    def gemm(self, a: torch.Tensor, m: int, is_k_full: bool = True, extra_scratch: int = 0) -> torch.Tensor:
         lib = _lib.load()
         tdt = torch.float16 if self.dtype == "fp16" else torch.bfloat16
         c = torch.empty((m, self.n), dtype=tdt, device=DEV)
         nbytes = lib.sonar_marlin_gemm_scratch_bytes(m, self.n, self.k)
-        scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=DEV)
+        scratch = torch.empty(max(nbytes, 16) + extra_scratch, dtype=torch.uint8, device=DEV)
         _lib.check(lib.sonar_marlin_gemm(
             ptr(a), a.stride(0) if m > 0 else self.k, ptr(c), ptr(self.native), _lib.LAYOUT_GFX950,
             ptr(self.bias), ptr(self.scales), ptr(self.zeros), ptr(self.g_idx), ptr(self.perm),

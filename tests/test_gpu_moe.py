@@ -175,3 +175,67 @@ def test_moe_error_paths():
     assert call(b_type=_lib.TYPE_UINT4) == _lib.E_INVALID
     assert call(k=250) == _lib.E_INVALID
     torch.cuda.synchronize()
+
+
+# ---------------------------------------------------------------- helper kernels around the GEMMs
+@pytest.mark.parametrize("m,topk,e,bs", [(4, 3, 5, 4), (1, 2, 8, 8), (33, 2, 8, 16), (257, 2, 4, 64),
+                                         (5, 6, 64, 16), (100, 1, 3, 48), (4096, 2, 8, 64), (700, 8, 256, 16)])
+def test_moe_align_kernel_matches_oracle(m, topk, e, bs):
+    lib = _lib.load()
+    rng = np.random.default_rng(m * 31 + e)
+    ids = np.stack([rng.permutation(e)[:topk] for _ in range(m)]).astype(np.int32)
+    want_sorted, want_experts, want_past = mo.moe_align_block_size(ids, bs, e)
+    d_ids = gu.dev_i32(ids.reshape(-1))
+    sorted_ids = torch.empty(want_sorted.size, dtype=torch.int32, device=gu.DEV)
+    expert_ids = torch.empty(want_experts.size, dtype=torch.int32, device=gu.DEV)
+    past = torch.empty(1, dtype=torch.int32, device=gu.DEV)
+    offsets = torch.empty(e, dtype=torch.int32, device=gu.DEV)
+    _lib.check(lib.sonar_moe_align_block_size(gu.ptr(d_ids), ids.size, e, bs, gu.ptr(sorted_ids), sorted_ids.numel(),
+                                              gu.ptr(expert_ids), expert_ids.numel(), gu.ptr(past), None,
+                                              gu.ptr(offsets), gu.stream()))
+    torch.cuda.synchronize()
+    assert int(past[0]) == int(want_past[0])
+    assert np.array_equal(sorted_ids.cpu().numpy(), want_sorted)        # bit-exact, padding included
+    assert np.array_equal(expert_ids.cpu().numpy(), want_experts)
+
+
+def test_moe_align_op_with_expert_map_matches_torch_expressions():
+    from sonar_amd import fused_moe
+    rng = np.random.default_rng(3)
+    m, topk, e, bs = 50, 2, 8, 16
+    ids = torch.from_numpy(np.stack([rng.permutation(e)[:topk] for _ in range(m)]).astype(np.int32))
+    emap = torch.tensor([-1, 2, -1, 0, 1, -1, 3, -1], dtype=torch.int32)
+    for ignore in (True, False):
+        want = fused_moe.moe_align_block_size(ids, bs, e, emap, ignore_invalid_experts=ignore)        # CPU: torch
+        got = fused_moe.moe_align_block_size(ids.to(gu.DEV), bs, e, emap.to(gu.DEV), ignore_invalid_experts=ignore)
+        torch.cuda.synchronize()
+        past = int(want[2][0])
+        assert int(got[2][0]) == past
+        assert torch.equal(got[0].cpu()[:past], want[0][:past]) and bool((got[0].cpu()[past:] == ids.numel()).all())
+        assert torch.equal(got[1].cpu(), want[1])
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_silu_and_mul_and_moe_sum_kernels(dtype):
+    lib = _lib.load()
+    rng = np.random.default_rng(11)
+    rows, d, topk = 37, 264, 3
+    x32 = mo.round_to_dtype((rng.standard_normal((rows, 2 * d)) * 3).astype(np.float32), dtype)
+    x = gu.dev_bits16(x32, dtype)
+    out = torch.empty((rows, d), dtype=x.dtype, device=gu.DEV)
+    _lib.check(lib.sonar_silu_and_mul(gu.ptr(out), gu.ptr(x), rows, d, gu.dtype_code(dtype), gu.stream()))
+    g, u = x32[:, :d].astype(np.float64), x32[:, d:]
+    silu = mo.round_to_dtype((g / (1.0 + np.exp(-g))).astype(np.float32), dtype)
+    want = mo.round_to_dtype(silu * u, dtype)
+    got = gu.host_f32(out)
+    # expf in the kernel vs exp here: allow one unit in the last place of the activation
+    ulp = 2.0 ** (-10 if dtype == "fp16" else -7)
+    assert np.all(np.abs(got - want) <= ulp * np.abs(want) * 2 + 1e-6)
+    assert np.mean(got == want) > 0.98
+
+    y32 = mo.round_to_dtype(rng.standard_normal((rows, topk, d)).astype(np.float32), dtype)
+    y = gu.dev_bits16(y32.reshape(rows * topk, d), dtype).reshape(rows, topk, d)
+    s = torch.empty((rows, d), dtype=y.dtype, device=gu.DEV)
+    _lib.check(lib.sonar_moe_sum(gu.ptr(s), gu.ptr(y), rows, topk, d, gu.dtype_code(dtype), gu.stream()))
+    want = mo.round_to_dtype(((y32[:, 0] + y32[:, 1]) + y32[:, 2]).astype(np.float32), dtype)
+    assert np.array_equal(gu.host_f32(s), want)        # fp32 sum in k order, one rounding

@@ -188,6 +188,7 @@ TILE_CASES = [
     (512, 4096, 11008, 128, True, False, False),     # AWQ, benchmark config 4
     (1000, 2048, 64, -1, False, False, True),
     (129, 14336, 4096, 128, False, False, False),
+    (600, 1024, 768, 64, True, False, True),
 ]
 
 
@@ -203,3 +204,20 @@ def test_marlin_gemm_tiled_within_tolerance(gu, dtype, m, k, n, g, zp, act, bias
     assert ok, f"max_err={max_err} max_ref={max_ref}"
     c2 = layer.gemm(a, m)
     assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("m,k,n", [(1, 4096, 11008), (16, 512, 256), (48, 1024, 512), (512, 4096, 1024)])
+def test_act_order_with_permuted_copy_of_a(gu, dtype, m, k, n):
+    """With size_m * size_k * 2 bytes more scratch an act-order call permutes A
+    once and runs the plain kernels; it must agree with the gathering path."""
+    layer = gu.DeviceLayer(77 + m, k, n, 128, dtype, act_order=True)
+    a32 = mo.make_activations(m + 5, m, k, dtype, std=0.5)
+    a = gu.dev_bits16(a32, dtype)
+    fast = layer.gemm(a, m, extra_scratch=m * k * 2)
+    ref = mo.gemm_reference(a32, layer.w_ref)
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(fast), ref)
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+    gathered = layer.gemm(a, m)
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(fast), gu.host_f32(gathered))
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
