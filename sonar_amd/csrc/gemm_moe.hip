@@ -10,11 +10,22 @@
 // routing weight when asked (marlin_template.h:1883-1909).  K is never split
 // across workgroups, so nothing is reduced through memory and results do not
 // depend on the launch: scratch and workspace are not used.
+#include <cstdlib>
+
 #include "common.hpp"
 #include "dequant.hpp"
 #include "wave_reduce.hpp"
 
 namespace sonar {
+
+// gemm_tile.hip: the MFMA-tiled grouped kernel for 64-slot blocks
+int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, const void* scales,
+                  const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
+                  const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
+                  int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
+                  int64_t num_groups, int group_size, hipStream_t st);
+size_t moe_tile_table_bytes(int64_t sorted_len, int64_t num_experts);
+
 namespace {
 
 constexpr int kMoeWaves = 8;
@@ -233,11 +244,12 @@ using namespace sonar;
 
 extern "C" size_t sonar_moe_marlin_gemm_scratch_bytes(int64_t sorted_len, int64_t moe_block_size,
                                                       int64_t size_n, int64_t size_k) {
-  (void)sorted_len;
-  (void)moe_block_size;
   (void)size_n;
   (void)size_k;
-  return 0;  // K is not split across workgroups: no partial sums leave the chip
+  // K is never split across workgroups, so no partial sums leave the chip; the
+  // tiled kernel for 64-slot blocks keeps its table of row tiles here (sized
+  // for any number of experts up to 1024)
+  return moe_block_size == 64 ? moe_tile_table_bytes(sorted_len, 1024) : 0;
 }
 
 extern "C" int sonar_moe_wna16_marlin_gemm(
@@ -251,8 +263,6 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     int use_atomic_add, int use_fp32_reduce, void* stream) {
   (void)workspace;
   (void)workspace_len;
-  (void)scratch;
-  (void)scratch_bytes;
   (void)use_atomic_add;
   (void)use_fp32_reduce;
   SONAR_REQUIRE(b_layout == SONAR_LAYOUT_GFX950, "unknown b_layout = %d", b_layout);
@@ -304,6 +314,16 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
   SONAR_REQUIRE(sorted_len > 0 && sorted_len < (1LL << 30), "sorted_token_ids.numel = %ld out of range",
                 (long)sorted_len);
 
+  hipStream_t st = (hipStream_t)stream;
+  static const bool no_tile = getenv("SONAR_MARLIN_NO_MOE_TILE") != nullptr;  // debugging aid
+  // Full blocks of 64 slots mean many rows per expert: the MFMA-tiled kernel
+  if (moe_block_size == 64 && !has_perm && !no_tile && size_k % 64 == 0 && num_experts <= 1024 &&
+      (num_groups == 1 || group_size % 64 == 0) && scratch != nullptr &&
+      scratch_bytes >= moe_tile_table_bytes(sorted_len, num_experts) && ((uintptr_t)scratch) % 4 == 0)
+    return moe_tile_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
+                         num_tokens_past_padded, topk_weights, top_k, mul_topk_weights ? 1 : 0, num_experts,
+                         static_cast<int32_t*>(scratch), dtype, size_m, size_n, size_k, num_groups, group_size, st);
+
   MoeParams p;
   p.a = static_cast<const uint16_t*>(a);
   p.c = static_cast<uint16_t*>(c);
@@ -333,7 +353,6 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
   p.mul_topk = mul_topk_weights ? 1 : 0;
   const int64_t grid = (int64_t)p.num_blocks * p.strips;
   SONAR_REQUIRE(grid < (1LL << 31), "too many (block, strip) pairs: %ld", (long)grid);
-  hipStream_t st = (hipStream_t)stream;
   if (dtype == SONAR_DTYPE_F16) {
     if (has_zp) launch_moe_mb<_Float16, true>(p, has_perm, (int)grid, st);
     else launch_moe_mb<_Float16, false>(p, has_perm, (int)grid, st);

@@ -45,6 +45,13 @@ struct TileParams {
   int num_groups, group_size;
   int chunks_per_strip;
   int tiles_m, tiles_n;
+  // grouped (mixture-of-experts) calls only
+  const int32_t* sorted_ids;   // slot -> row id of C (row id / top_k of A), >= rows_total: padding
+  const float* topk_weights;
+  const int32_t* tile_table;   // [0]: number of row tiles, then (first block, blocks, expert) per tile
+  int rows_total, top_k, mul_topk;
+  long expert_b_stride;        // uint4 units between experts in b
+  long expert_s_stride, expert_z_stride, expert_bias_stride;  // elements between experts
 };
 
 // 16 bytes (8 consecutive k) of row `row` of A, gathered through perm when given.
@@ -259,7 +266,7 @@ constexpr int kAsyncCopies = 7;
       : "v"(a_at)                                                                                  \
       : "memory")
 
-template <typename T, bool HAS_ZP>
+template <typename T, bool HAS_ZP, bool GROUPED>
 __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq<T>::Col Col;
@@ -275,6 +282,16 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 
   int tile_m, tile_n;
   if (!tile_of_workgroup(p, tile_m, tile_n)) return;
+  // Grouped calls: row tile t is up to four consecutive 64-slot blocks of one
+  // expert, listed in tile_table; rows are slots of sorted_ids.
+  int first_slot = 0, tile_rows = kTileM;
+  long expert = 0;
+  if (GROUPED) {
+    if (tile_m >= p.tile_table[0]) return;
+    first_slot = p.tile_table[1 + 3 * tile_m] * 64;
+    tile_rows = p.tile_table[2 + 3 * tile_m] * 64;
+    expert = p.tile_table[3 + 3 * tile_m];
+  }
   const int m0 = tile_m * kTileM;
   const int strip0 = tile_n * (kTileN / kStripN);
   const int strips_here = min(kTileN / kStripN, p.size_n / kStripN - strip0);
@@ -291,18 +308,25 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     // operand block of copy i: row block wave + 8 (i / 2), k block i % 2, so that the
     // two halves of every 128-byte line of A are requested back to back by one wavefront
     const int blk = 2 * (wave + 8 * (i >> 1)) + (i & 1);
-    int row = m0 + 16 * (blk >> 1) + col16;
-    if (row >= p.size_m) row = p.size_m - 1;  // rows past M are computed and never stored
+    int row;
+    if (GROUPED) {
+      const int r = 16 * (blk >> 1) + col16;
+      const int id = r < tile_rows ? p.sorted_ids[first_slot + r] : p.rows_total;
+      row = (unsigned)id < (unsigned)p.rows_total ? id / p.top_k : 0;  // padding slots read row 0, never stored
+    } else {
+      row = m0 + 16 * (blk >> 1) + col16;
+      if (row >= p.size_m) row = p.size_m - 1;  // rows past M are computed and never stored
+    }
     a_src[i] = reinterpret_cast<const char*>(p.a) + ((long)row * p.lda + 32 * (blk & 1) + 8 * kb) * 2;
   }
-  const uint4* b_src = p.b + (size_t)(unsigned)(strip * p.chunks_per_strip) * 64 + lane;
+  const uint4* b_src = p.b + expert * p.expert_b_stride + (size_t)(unsigned)(strip * p.chunks_per_strip) * 64 + lane;
   const char* s_src;
   long s_group_stride;
   if (HAS_ZP && lane >= 32) {
-    s_src = reinterpret_cast<const char*>(p.zeros + strip * 8 + (lane & 7));
+    s_src = reinterpret_cast<const char*>(p.zeros + expert * p.expert_z_stride + strip * 8 + (lane & 7));
     s_group_stride = (long)(p.size_n / 8) * 4;
   } else {
-    s_src = reinterpret_cast<const char*>(p.scales + strip * kStripN) + 4 * (lane & 31);
+    s_src = reinterpret_cast<const char*>(p.scales + expert * p.expert_s_stride + strip * kStripN) + 4 * (lane & 31);
     s_group_stride = (long)p.size_n * 2;
   }
   char* wring = smem + kAsyncA + wave * (kAsyncStages * kWaveStage);
@@ -443,39 +467,105 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 #undef SONAR_TILE_W
 
   if (!active) return;
+  // rows of C this lane writes: one per row block
+  long c_row[8];
+  float row_w[8];
+#pragma unroll
+  for (int mb = 0; mb < 8; ++mb) {
+    const int r = 128 * wm + 16 * mb + col16;
+    c_row[mb] = -1;
+    row_w[mb] = 1.f;
+    if (GROUPED) {
+      const int id = r < tile_rows ? p.sorted_ids[first_slot + r] : p.rows_total;
+      if ((unsigned)id < (unsigned)p.rows_total) {
+        c_row[mb] = id;
+        // the routing weight is rounded to the activation type and the product is
+        // formed and rounded in that type (marlin_template.h(moe):1893-1897)
+        if (p.mul_topk) row_w[mb] = Dq<T>::to_float(Dq<T>::from_float(p.topk_weights[id]));
+      }
+    } else if (m0 + r < p.size_m) {
+      c_row[mb] = m0 + r;
+    }
+  }
+  const uint16_t* bias_src = p.bias ? p.bias + expert * p.expert_bias_stride + strip * kStripN : nullptr;
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb) {
     const int n = strip * kStripN + 16 * nb + 4 * kb;
     float bias[4] = {0.f, 0.f, 0.f, 0.f};
-    if (p.bias) {
+    if (bias_src) {
 #pragma unroll
-      for (int r = 0; r < 4; ++r)
-        bias[r] = Dq<T>::to_float(p.bias[strip * kStripN + scale_slot(16 * nb + 4 * kb + r, false)]);
+      for (int r = 0; r < 4; ++r) bias[r] = Dq<T>::to_float(bias_src[scale_slot(16 * nb + 4 * kb + r, false)]);
     }
 #pragma unroll
     for (int mb = 0; mb < 8; ++mb) {
-      const int m = m0 + 128 * wm + 16 * mb + col16;
-      if (m < p.size_m) {
-        const floatx4_t v = acc[nb][mb];
-        uint2 o;
-        o.x = (uint32_t)Dq<T>::from_float(v.x + bias[0]) | ((uint32_t)Dq<T>::from_float(v.y + bias[1]) << 16);
-        o.y = (uint32_t)Dq<T>::from_float(v.z + bias[2]) | ((uint32_t)Dq<T>::from_float(v.w + bias[3]) << 16);
-        *reinterpret_cast<uint2*>(p.c + (long)m * p.size_n + n) = o;
+      if (c_row[mb] < 0) continue;
+      const floatx4_t v = acc[nb][mb];
+      uint16_t o[4] = {Dq<T>::from_float(v.x + bias[0]), Dq<T>::from_float(v.y + bias[1]),
+                       Dq<T>::from_float(v.z + bias[2]), Dq<T>::from_float(v.w + bias[3])};
+      if (GROUPED && p.mul_topk) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) o[r] = Dq<T>::from_float(Dq<T>::to_float(o[r]) * row_w[mb]);
       }
+      uint2 packed;
+      packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+      packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+      *reinterpret_cast<uint2*>(p.c + c_row[mb] * p.size_n + n) = packed;
     }
   }
+}
+
+// Builds the row-tile table of a grouped call: runs of blocks with the same
+// expert are cut into tiles of up to four blocks.  One workgroup; expert_ids
+// is staged in LDS and scanned by one thread (a few hundred entries).
+__global__ __launch_bounds__(256) void moe_tile_table_kernel(const int32_t* __restrict__ expert_ids,
+                                                            const int32_t* __restrict__ num_post_pad,
+                                                            int num_blocks_max, int block_size, int num_experts,
+                                                            int32_t* __restrict__ table, int max_tiles) {
+  extern __shared__ int32_t ids[];
+  int blocks = num_post_pad[0] / block_size;
+  if (blocks > num_blocks_max) blocks = num_blocks_max;
+  for (int b = threadIdx.x; b < blocks; b += blockDim.x) ids[b] = expert_ids[b];
+  __syncthreads();
+  if (threadIdx.x != 0) return;
+  int tiles = 0;
+  int b = 0;
+  while (b < blocks && tiles < max_tiles) {
+    const int e = ids[b];
+    int n = 1;
+    while (n < 4 && b + n < blocks && ids[b + n] == e) ++n;
+    if (e >= 0 && e < num_experts) {
+      table[1 + 3 * tiles] = b;
+      table[2 + 3 * tiles] = n;
+      table[3 + 3 * tiles] = e;
+      ++tiles;
+    }
+    b += n;
+  }
+  table[0] = tiles;
 }
 
 template <typename T, bool HAS_ZP>
 int launch_tile_async(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, HAS_ZP>,
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, HAS_ZP, false>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, kAsyncLds));
     attr_set = true;
   }
   const int grid = tile_grid(p);
-  marlin_tile_async_kernel<T, HAS_ZP><<<grid, kTileWaves * 64, kAsyncLds, st>>>(p);
+  marlin_tile_async_kernel<T, HAS_ZP, false><<<grid, kTileWaves * 64, kAsyncLds, st>>>(p);
+  return SONAR_OK;
+}
+
+template <typename T, bool HAS_ZP>
+int launch_tile_grouped(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, HAS_ZP, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kAsyncLds));
+    attr_set = true;
+  }
+  marlin_tile_async_kernel<T, HAS_ZP, true><<<tile_grid(p), kTileWaves * 64, kAsyncLds, st>>>(p);
   return SONAR_OK;
 }
 
@@ -516,6 +606,11 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   p.chunks_per_strip = (int)(size_k / kChunkK);
   p.tiles_m = (int)((size_m + kTileM - 1) / kTileM);
   p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);
+  p.sorted_ids = nullptr;
+  p.topk_weights = nullptr;
+  p.tile_table = nullptr;
+  p.rows_total = p.top_k = p.mul_topk = 0;
+  p.expert_b_stride = p.expert_s_stride = p.expert_z_stride = p.expert_bias_stride = 0;
   const bool zp = zeros != nullptr, pm = perm != nullptr;
   int rc;
   static const bool no_async = getenv("SONAR_MARLIN_NO_ASYNC_TILE") != nullptr;  // debugging aid
@@ -536,6 +631,63 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   }
   if (rc) return rc;
   return launch_status("marlin_tile_kernel");
+}
+
+// Row tiles a grouped call can have at most, and the bytes of its tile table.
+int moe_tile_max(int64_t sorted_len, int64_t num_experts) {
+  const int64_t blocks = (sorted_len + 63) / 64;
+  return (int)((blocks + 3) / 4 + num_experts);
+}
+size_t moe_tile_table_bytes(int64_t sorted_len, int64_t num_experts) {
+  return (size_t)(1 + 3 * moe_tile_max(sorted_len, num_experts)) * sizeof(int32_t);
+}
+
+// Called by sonar_moe_wna16_marlin_gemm for 64-slot blocks without act-order
+// when group_size % 64 == 0 (or one group) and size_k % 64 == 0.
+int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, const void* scales,
+                  const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
+                  const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
+                  int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
+                  int64_t num_groups, int group_size, hipStream_t st) {
+  const int max_tiles = moe_tile_max(sorted_len, num_experts);
+  const int blocks_max = (int)((sorted_len + 63) / 64);
+  moe_tile_table_kernel<<<1, 256, (size_t)blocks_max * sizeof(int32_t), st>>>(expert_ids, num_post_pad, blocks_max, 64,
+                                                                             (int)num_experts, table, max_tiles);
+  if (int rc = launch_status("moe_tile_table_kernel")) return rc;
+  TileParams p;
+  p.a = static_cast<const uint16_t*>(a);
+  p.lda = size_k;
+  p.c = static_cast<uint16_t*>(c);
+  p.b = reinterpret_cast<const uint4*>(b);
+  p.bias = static_cast<const uint16_t*>(bias);
+  p.scales = static_cast<const uint16_t*>(scales);
+  p.zeros = zeros;
+  p.perm = nullptr;
+  p.size_m = (int)size_m;
+  p.size_n = (int)size_n;
+  p.size_k = (int)size_k;
+  p.num_groups = (int)num_groups;
+  p.group_size = group_size;
+  p.chunks_per_strip = (int)(size_k / kChunkK);
+  p.tiles_m = max_tiles;
+  p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);
+  p.sorted_ids = sorted_ids;
+  p.topk_weights = topk_weights;
+  p.tile_table = table;
+  p.rows_total = (int)(size_m * top_k);
+  p.top_k = (int)top_k;
+  p.mul_topk = mul_topk;
+  p.expert_b_stride = (long)(size_k * size_n / 8 / 4);
+  p.expert_s_stride = (long)(num_groups * size_n);
+  p.expert_z_stride = (long)(num_groups * (size_n / 8));
+  p.expert_bias_stride = (long)size_n;
+  int rc;
+  if (dtype == SONAR_DTYPE_F16)
+    rc = zeros ? launch_tile_grouped<_Float16, true>(p, st) : launch_tile_grouped<_Float16, false>(p, st);
+  else
+    rc = zeros ? launch_tile_grouped<__bf16, true>(p, st) : launch_tile_grouped<__bf16, false>(p, st);
+  if (rc) return rc;
+  return launch_status("marlin_tile_async_kernel (grouped)");
 }
 
 }  // namespace sonar

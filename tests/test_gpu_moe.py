@@ -53,7 +53,7 @@ class Experts:
             out[ids] = c
         return out
 
-    def gemm(self, a, sorted_ids, expert_ids, past, weights, bs, top_k, m, mul):
+    def gemm(self, a, sorted_ids, expert_ids, past, weights, bs, top_k, m, mul, scratch=True):
         lib = _lib.load()
         tdt = torch.float16 if self.dtype == "fp16" else torch.bfloat16
         c = torch.zeros((m * top_k, self.n), dtype=tdt, device=gu.DEV)
@@ -61,10 +61,12 @@ class Experts:
         eid = gu.dev_i32(expert_ids)
         npp = gu.dev_i32(np.array([past], dtype=np.int32))
         tw = torch.from_numpy(weights.astype(np.float32).reshape(-1)).to(gu.DEV) if weights is not None else None
+        nbytes = lib.sonar_moe_marlin_gemm_scratch_bytes(sid.numel(), bs, self.n, self.k) if scratch else 0
+        scr = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=gu.DEV) if scratch else None
         _lib.check(lib.sonar_moe_wna16_marlin_gemm(
             gu.ptr(a), gu.ptr(c), gu.ptr(self.native), _lib.LAYOUT_GFX950, gu.ptr(self.bias),
             gu.ptr(self.scales), gu.ptr(self.zeros), gu.ptr(self.g_idx), gu.ptr(self.perm),
-            gu.ptr(self.workspace), self.workspace.numel(), None, 0, gu.ptr(sid), sid.numel(),
+            gu.ptr(self.workspace), self.workspace.numel(), gu.ptr(scr), nbytes, gu.ptr(sid), sid.numel(),
             gu.ptr(eid), gu.ptr(npp), gu.ptr(tw), bs, top_k, int(mul), self.e,
             gu.dtype_code(self.dtype), self.b_type, m, self.n, self.k, self.groups, 1, 0, 1, gu.stream()))
         torch.cuda.synchronize()
@@ -91,6 +93,11 @@ MOE_CASES = [
     (150, 4, 2, 256, 256, 128, "fp16", False, False, False, 48, True),
     (222, 3, 2, 288, 128, 32, "bf16", False, False, False, 64, True),
     (5, 64, 6, 256, 128, 128, "fp16", False, False, False, 16, True),
+    # 64-slot blocks with groups of at least 64 rows: the MFMA-tiled grouped kernel
+    (300, 4, 2, 512, 256, 128, "fp16", False, False, False, 64, True),
+    (513, 3, 2, 256, 320, 64, "bf16", True, False, True, 64, True),
+    (90, 8, 2, 384, 128, -1, "fp16", False, False, False, 64, False),
+    (1100, 2, 1, 128, 512, 128, "bf16", False, False, True, 64, False),
 ]
 
 
@@ -239,3 +246,23 @@ def test_silu_and_mul_and_moe_sum_kernels(dtype):
     _lib.check(lib.sonar_moe_sum(gu.ptr(s), gu.ptr(y), rows, topk, d, gu.dtype_code(dtype), gu.stream()))
     want = mo.round_to_dtype(((y32[:, 0] + y32[:, 1]) + y32[:, 2]).astype(np.float32), dtype)
     assert np.array_equal(gu.host_f32(s), want)        # fp32 sum in k order, one rounding
+
+
+def test_moe_tiled_and_streaming_kernels_agree():
+    """The same 64-slot-block call with and without the scratch the tiled kernel
+    needs for its table takes two different kernels; both meet the tolerance
+    against the reference and each other."""
+    m, e, top_k, k, n, bs = 260, 4, 2, 512, 256, 64
+    ex = Experts(91, e, k, n, 128, "bf16")
+    topk_ids, topk_w = route(7, m, e, top_k)
+    sorted_ids, expert_ids, past = mo.moe_align_block_size(topk_ids, bs, e)
+    a32 = mo.make_activations(4, m, k, "bf16")
+    a = gu.dev_bits16(a32, "bf16")
+    tiled = gu.host_f32(ex.gemm(a, sorted_ids, expert_ids, int(past[0]), topk_w, bs, top_k, m, True, scratch=True))
+    streamed = gu.host_f32(ex.gemm(a, sorted_ids, expert_ids, int(past[0]), topk_w, bs, top_k, m, True, scratch=False))
+    want = ex.reference(a32, sorted_ids, expert_ids, int(past[0]), bs, top_k, m, topk_w)
+    for got in (tiled, streamed):
+        ok, *worst = mo.gemm_tolerance_ok(got, want)
+        assert ok, worst
+    ok, *worst = mo.gemm_tolerance_ok(tiled, streamed)
+    assert ok, worst
