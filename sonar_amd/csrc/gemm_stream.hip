@@ -165,10 +165,16 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, int strip, i
 // General kernel: any M <= 64, any K % 32 == 0, any group size that is a
 // multiple of 32, optional act-order gather of A.  Operands are fetched into
 // registers one unit ahead.
+// With three or four 16-row blocks a unit buffer holds two chunks instead of
+// four (the host halves the unit), which keeps the two buffers and the
+// accumulators inside the register file.
+template <int MB>
+constexpr int unit_buffer_chunks() { return MB >= 3 ? 2 : 4; }
+
 template <typename T, int MB>
 struct UnitBuf {
-  uint4 q[4];
-  typename Dq<T>::vec8 a[4][MB];
+  uint4 q[unit_buffer_chunks<MB>()];
+  typename Dq<T>::vec8 a[unit_buffer_chunks<MB>()][MB];
   uint32_t sbits[4];
   uint32_t zword;
   int group;
@@ -183,10 +189,10 @@ __device__ __forceinline__ void load_unit(UnitBuf<T, MB>& b, const StreamParams&
   const int chunk0 = unit * p.unit_chunks;
   const uint4* bsrc = p.b + ((long)strip * p.chunks_per_strip + chunk0) * 64 + lane;
 #pragma unroll
-  for (int cc = 0; cc < 4; ++cc)
+  for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc)
     if (cc < p.unit_chunks) b.q[cc] = bsrc[cc * 64];
 #pragma unroll
-  for (int cc = 0; cc < 4; ++cc)
+  for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc)
     if (cc < p.unit_chunks) {
 #pragma unroll
       for (int mb = 0; mb < MB; ++mb)
@@ -244,7 +250,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
       int cur_group = cur.group;
       const int chunk0 = (mine - strip_first) * p.unit_chunks;
 #pragma unroll
-      for (int cc = 0; cc < 4; ++cc) {
+      for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc) {
         if (cc < p.unit_chunks) {
           const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
           if (g != cur_group) {  // groups smaller than a unit
@@ -620,31 +626,45 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
 
 // ---------------------------------------------------------------------------
 // Second pass over the strips that were split between workgroups: adds the
-// partial tiles in workgroup order and writes C.  One wavefront per strip.
+// partial tiles in workgroup order and writes C.  One wavefront per strip and
+// 16-row block.
 template <typename T, int MB>
 __global__ __launch_bounds__(64) void marlin_fixup_kernel(const StreamParams p) {
-  const int strip = blockIdx.x;
+  const int strip = blockIdx.x / MB;
+  const int mb = blockIdx.x - strip * MB;
   const int lane = threadIdx.x;
   const int strip_first = strip * p.units_per_strip;
   const int first = range_owner(strip_first, p.total_units, p.parts);
   const int last = range_owner(strip_first + p.units_per_strip - 1, p.total_units, p.parts);
   if (first == last) return;
-  floatx4_t acc[MB][4];
+  floatx4_t acc[4];
 #pragma unroll
-  for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-    for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  for (int j = 0; j < 4; ++j) acc[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
   for (int w = first; w <= last; ++w) {
     const float4* src = partial_slot(p, w, first);
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const float4 v = src[(mb * 4 + j) * 64 + lane];
-        acc[mb][j] += floatx4_t{v.x, v.y, v.z, v.w};
-      }
+    for (int j = 0; j < 4; ++j) {
+      const float4 v = src[(mb * 4 + j) * 64 + lane];
+      acc[j] += floatx4_t{v.x, v.y, v.z, v.w};
+    }
   }
-  write_tiles<T, MB>(p, strip, lane, acc);
+  const int m = 16 * mb + (lane & 15);
+  if (m >= p.size_m) return;
+  const int n_in = 4 * (lane >> 4);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int nl = 16 * j + n_in;
+    float b[4] = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) b[r] = Dq<T>::to_float(p.bias[strip * kStripN + scale_slot(nl + r, false)]);
+    }
+    const floatx4_t v = acc[j];
+    uint2 o;
+    o.x = (uint32_t)Dq<T>::from_float(v.x + b[0]) | ((uint32_t)Dq<T>::from_float(v.y + b[1]) << 16);
+    o.y = (uint32_t)Dq<T>::from_float(v.z + b[2]) | ((uint32_t)Dq<T>::from_float(v.w + b[3]) << 16);
+    *reinterpret_cast<uint2*>(p.c + (long)m * p.size_n + strip * kStripN + nl) = o;
+  }
 }
 
 // Writes W[K][N]: the values the GEMM kernels feed to the matrix cores.
@@ -754,9 +774,9 @@ void launch_fixup(const StreamParams& p, hipStream_t st) {
   const int strips = p.size_n / kStripN;
   switch ((p.size_m + 15) / 16) {
     case 1: marlin_fixup_kernel<T, 1><<<strips, 64, 0, st>>>(p); break;
-    case 2: marlin_fixup_kernel<T, 2><<<strips, 64, 0, st>>>(p); break;
-    case 3: marlin_fixup_kernel<T, 3><<<strips, 64, 0, st>>>(p); break;
-    default: marlin_fixup_kernel<T, 4><<<strips, 64, 0, st>>>(p); break;
+    case 2: marlin_fixup_kernel<T, 2><<<strips * 2, 64, 0, st>>>(p); break;
+    case 3: marlin_fixup_kernel<T, 3><<<strips * 3, 64, 0, st>>>(p); break;
+    default: marlin_fixup_kernel<T, 4><<<strips * 4, 64, 0, st>>>(p); break;
   }
 }
 
@@ -877,6 +897,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   p.group_size = chk.group_size;
   p.chunks_per_strip = (int)(size_k / kChunkK);
   p.unit_chunks = p.chunks_per_strip % 4 == 0 ? 4 : (p.chunks_per_strip % 2 == 0 ? 2 : 1);
+  // slabs of more than 32 rows work on half units (see unit_buffer_chunks)
+  if (size_m > 32 && p.unit_chunks == 4) p.unit_chunks = 2;
   p.units_per_strip = p.chunks_per_strip / p.unit_chunks;
   const int64_t total_units = (size_n / kStripN) * p.units_per_strip;
   SONAR_REQUIRE(total_units * cus < (1LL << 31), "size_k * size_n = %ld x %ld is too large", (long)size_k,
@@ -901,10 +923,10 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   }
 
   static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
-  // Up to 256 rows a problem with few 256 x 256 tiles leaves most compute units
+  // Up to 512 rows a problem with few 256 x 256 tiles leaves most compute units
   // idle in the tile kernel; 64-row slabs of the streaming kernel use them all.
   const int64_t tiles = ((size_m + 255) / 256) * ((size_n + 255) / 256);
-  const bool slabs = size_m <= 128 || (size_m <= 256 && tiles < 64);
+  const bool slabs = size_m <= 128 || (size_m <= 512 && tiles < 64);
   if (size_m > 64 && size_k % 64 == 0 && !no_tile && !slabs)
     return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
                      size_k, num_groups, chk.group_size, st);
