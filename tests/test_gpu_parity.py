@@ -189,6 +189,7 @@ TILE_CASES = [
     (1000, 2048, 64, -1, False, False, True),
     (129, 14336, 4096, 128, False, False, False),
     (600, 1024, 768, 64, True, False, True),
+    (520, 512, 192, 32, True, False, False),         # groups of 32 rows: the register-staged tile kernel
 ]
 
 

@@ -219,3 +219,36 @@ def test_moe_block_size_and_silu_and_mul():
     out = torch.empty(5, 4)
     fused_moe.silu_and_mul(out, x)
     assert torch.allclose(out, x[:, :4] / (1 + torch.exp(-x[:, :4])) * x[:, 4:], atol=1e-6)
+
+
+def test_kernels_with_hand_counted_waits_do_not_spill():
+    """The LDS-DMA kernels wait for their copies with hand-counted
+    `s_waitcnt vmcnt(N)`; a register spill adds scratch loads and stores to the
+    same counter and would silently weaken those waits."""
+    import re
+    import shutil
+    import subprocess
+    hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
+    if not os.path.exists(hipcc):
+        pytest.skip("hipcc not available")
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    watched = {"gemm_tile.hip": "marlin_tile_async_kernel", "gemm_stream.hip": "marlin_stream_fast_kernel"}
+    for src, kernel in watched.items():
+        out = subprocess.run(
+            [hipcc, "-O3", "--offload-arch=gfx950", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
+             "-packed-fp32-ops", "-I", os.path.join(root, "include"), "-I", os.path.join(root, "sonar_amd", "csrc"),
+             "-c", "--offload-device-only", "-Rpass-analysis=kernel-resource-usage",
+             os.path.join(root, "sonar_amd", "csrc", src), "-o", os.devnull],
+            capture_output=True, text=True, timeout=600)
+        assert out.returncode == 0, out.stderr[-2000:]
+        name = None
+        seen = 0
+        for line in out.stderr.splitlines():
+            m = re.search(r"Function Name: (\S+)", line)
+            if m:
+                name = m.group(1)
+            m = re.search(r"VGPRs Spill: (\d+)", line)
+            if m and name and kernel in name:
+                seen += 1
+                assert int(m.group(1)) == 0, f"{name} spills {m.group(1)} VGPRs"
+        assert seen >= 4, f"no resource report for {kernel}"
