@@ -238,22 +238,28 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const Tile
 // the copies of step i+2 are issued before the matrix work of step i.
 //   * A: a ring of three 32-KiB stages shared by the workgroup; wavefront w
 //     copies both k blocks of row blocks w and w+8 of a stage.
-//   * W: the packed chunks are already in operand order, so each wavefront
-//     copies the two chunks of its own strip (and the scale / zero-point row of
-//     the step's group) into a private ring and dequantises them straight into
-//     MFMA operands; dequantised weights never pass through LDS.  The two
-//     wavefronts that share a strip each dequantise it.
-// Copies of a wavefront complete in issue order, seven per stage, so "stage i
-// has landed" is s_waitcnt vmcnt(7); one barrier per step then makes every
-// wavefront's share of A visible and frees the stage consumed in step i-1.
+//   * W: the packed chunks are already in operand order.  The two wavefronts
+//     that share a strip split its two chunks of a step: each copies one chunk
+//     (and the scale / zero-point row of the step's group) into a private
+//     ring, dequantises it one step ahead in the shadow of its MFMAs and
+//     parks the four operand blocks in a 32-KiB exchange buffer, from which
+//     both read the step's eight blocks.  Every packed word is therefore
+//     dequantised once per workgroup (the VALU work, 13 instructions per word,
+//     is what bounds this loop once the copies are hidden).
+// Copies of a wavefront complete in issue order, six per stage, so "stage i
+// has landed" is s_waitcnt vmcnt(6); a barrier at the top of a step makes
+// every wavefront's share of A and of the dequantised weights visible and frees
+// the stage consumed in step i-1; a second one, after the last read of the
+// exchange buffer, lets the weights of step i+1 be written into it.
 // LDS is read from asm blocks only (the compiler cannot tell which LDS bytes a
 // copy writes and would otherwise wait for all copies before any LDS access).
 // Needs group_size % 64 == 0 (or one group) and no act-order.
 constexpr int kAsyncStages = 3;
-constexpr int kWaveStage = 2 * kBlockBytes + 256;   // two weight chunks + 64 scales + 8 zero-point words
+constexpr int kWaveStage = kBlockBytes + 256;       // one weight chunk + 64 scales + 8 zero-point words
 constexpr int kAsyncA = kAsyncStages * kStageA;
-constexpr int kAsyncLds = kAsyncA + kTileWaves * kAsyncStages * kWaveStage;
-constexpr int kAsyncCopies = 7;
+constexpr int kAsyncW = kTileWaves * kAsyncStages * kWaveStage;
+constexpr int kAsyncLds = kAsyncA + kAsyncW + kStageB;   // + the dequantised weights of one step
+constexpr int kAsyncCopies = 6;
 
 #define SONAR_TILE_A4(h_off)                                                                       \
   asm volatile(                                                                                    \
@@ -341,18 +347,21 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
                                        (lds_void_t*)(sa + (2 * (wave + 8 * (i >> 1)) + (i & 1)) * kBlockBytes), 16, 0,
                                        0);
     char* sw = wring + slot * kWaveStage;
-    const uint4* g = b_src + (size_t)(2 * kt) * 64;
+    const uint4* g = b_src + (size_t)(2 * kt + wm) * 64;   // this wavefront's chunk: k block wm
     __builtin_amdgcn_global_load_lds((glb_void_t*)g, (lds_void_t*)sw, 16, 0, 0);
-    __builtin_amdgcn_global_load_lds((glb_void_t*)g, (lds_void_t*)sw, 16, 1024, 0);
     const int grp = grouped ? (kt * kTileK) / p.group_size : 0;
     __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)grp * s_group_stride),
-                                     (lds_void_t*)(sw + 2 * kBlockBytes), 4, 0, 0);
+                                     (lds_void_t*)(sw + kBlockBytes), 4, 0, 0);
   };
 
   uint32_t s_off[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) s_off[j] = 2 * kBlockBytes + 2 * scale_slot(16 * j + col16, grouped);
-  const uint32_t z_off = 2 * kBlockBytes + 128 + 4 * zero_point_word(col16);
+  for (int j = 0; j < 4; ++j) s_off[j] = kBlockBytes + 2 * scale_slot(16 * j + col16, grouped);
+  const uint32_t z_off = kBlockBytes + 128 + 4 * zero_point_word(col16);
+  // exchange buffer: operand block ((strip * 2 + k block) * 4 + column block)
+  const uint32_t x_lds = a_lds + kAsyncA + kAsyncW;
+  const uint32_t x_own = x_lds + ((wn * 2 + wm) * 4) * kBlockBytes + lane * 16;
+  const uint32_t x_strip = x_lds + (wn * 2 * 4) * kBlockBytes + lane * 16;
 
   floatx4_t acc[4][8];
 #pragma unroll
@@ -364,16 +373,23 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   issue(0, 0);
   if (k_tiles > 1) issue(1, 1);
 
-  // Dequantisation runs in the shadow of the matrix work, half a step ahead:
-  // while the MFMAs of k block 0 run, k block 1 of the same step is
-  // dequantised (wv[1]); while those of k block 1 run, k block 0 of the next
-  // step (wv[0]), whose packed words sit in the wavefront's private ring and
-  // need no barrier.  qb holds the packed words of k block 1 in between.
-  vec8 wv[2][4];
-  u32x4_t qa, qb;
+  u32x4_t qraw;
   uint32_t sb0, sb1, sb2, sb3, zw;
   Col cols[4];
-  auto make_cols = [&]() {
+  // packed words, scales and zero points of this wavefront's chunk of a stage
+  auto read_own = [&](uint32_t w_at) {
+    asm volatile(
+        "ds_read_b128 %0, %6\n\t"
+        "ds_read_u16 %1, %7\n\t"
+        "ds_read_u16 %2, %8\n\t"
+        "ds_read_u16 %3, %9\n\t"
+        "ds_read_u16 %4, %10\n\t"
+        "ds_read_b32 %5, %11\n\t"
+        "s_waitcnt lgkmcnt(0)"
+        : "=&v"(qraw), "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
+        : "v"(w_at + lane * 16), "v"(w_at + s_off[0]), "v"(w_at + s_off[1]), "v"(w_at + s_off[2]),
+          "v"(w_at + s_off[3]), "v"(w_at + z_off)
+        : "memory");
     const uint32_t sbits[4] = {sb0, sb1, sb2, sb3};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -382,35 +398,48 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
       cols[j] = Dq<T>::make_col((uint16_t)sbits[j], z);
     }
   };
-#define SONAR_TILE_W(w_at)                                                                         \
-  asm volatile(                                                                                    \
-      "ds_read_b128 %0, %7\n\t"                                                                    \
-      "ds_read_b128 %1, %7 offset:1024\n\t"                                                        \
-      "ds_read_u16 %2, %8\n\t"                                                                     \
-      "ds_read_u16 %3, %9\n\t"                                                                     \
-      "ds_read_u16 %4, %10\n\t"                                                                    \
-      "ds_read_u16 %5, %11\n\t"                                                                    \
-      "ds_read_b32 %6, %12\n\t"                                                                    \
-      "s_waitcnt lgkmcnt(0)"                                                                       \
-      : "=&v"(qa), "=&v"(qb), "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)            \
-      : "v"((w_at) + lane * 16), "v"((w_at) + s_off[0]), "v"((w_at) + s_off[1]),                   \
-        "v"((w_at) + s_off[2]), "v"((w_at) + s_off[3]), "v"((w_at) + z_off)                        \
-      : "memory")
-#define SONAR_TILE_MFMA16(h, mb0)                                                                  \
+  // dequantises column blocks j0 and j0 + 1 of the chunk and parks them
+  auto park_pair = [&](uint32_t w0, uint32_t w1, const Col& c0, const Col& c1, int j0, bool last) {
+    const vec8 v0 = Dq<T>::word(w0, c0, magic);
+    const vec8 v1 = Dq<T>::word(w1, c1, magic);
+    if (j0 == 0) {
+      asm volatile("ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:1024" ::"v"(x_own), "v"(v0), "v"(v1) : "memory");
+    } else {
+      asm volatile("ds_write_b128 %0, %1 offset:2048\n\tds_write_b128 %0, %2 offset:3072" ::"v"(x_own), "v"(v0),
+                   "v"(v1)
+                   : "memory");
+    }
+    if (last) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  };
+#define SONAR_TILE_MFMA16(wv, mb0)                                                                 \
   _Pragma("unroll") for (int i = 0; i < 4; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j)      \
-      acc[j][(mb0) + i] = Dq<T>::mfma(wv[h][j], __builtin_bit_cast(vec8, av[i]), acc[j][(mb0) + i])
+      acc[j][(mb0) + i] = Dq<T>::mfma(__builtin_bit_cast(vec8, wv[j]), __builtin_bit_cast(vec8, av[i]), acc[j][(mb0) + i])
+// four weight operand blocks of k block h of this strip and four blocks of A
+#define SONAR_TILE_XA(wv, x_off, a_off)                                                            \
+  asm volatile(                                                                                    \
+      "ds_read_b128 %0, %8 offset:" #x_off "\n\t"                                                  \
+      "ds_read_b128 %1, %8 offset:" #x_off "+1024\n\t"                                             \
+      "ds_read_b128 %2, %8 offset:" #x_off "+2048\n\t"                                             \
+      "ds_read_b128 %3, %8 offset:" #x_off "+3072\n\t"                                             \
+      "ds_read_b128 %4, %9 offset:" #a_off "\n\t"                                                  \
+      "ds_read_b128 %5, %9 offset:" #a_off "+2048\n\t"                                             \
+      "ds_read_b128 %6, %9 offset:" #a_off "+4096\n\t"                                             \
+      "ds_read_b128 %7, %9 offset:" #a_off "+6144\n\t"                                             \
+      "s_waitcnt lgkmcnt(0)"                                                                       \
+      : "=&v"(wv[0]), "=&v"(wv[1]), "=&v"(wv[2]), "=&v"(wv[3]), "=&v"(av[0]), "=&v"(av[1]),        \
+        "=&v"(av[2]), "=&v"(av[3])                                                                 \
+      : "v"(x_strip), "v"(a_at)                                                                    \
+      : "memory")
+
   if (active) {
     if (k_tiles > 1) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    SONAR_TILE_W(w_lds);
-    make_cols();
-    wv[0][0] = Dq<T>::word(qa.x, cols[0], magic);
-    wv[0][1] = Dq<T>::word(qa.y, cols[1], magic);
-    wv[0][2] = Dq<T>::word(qa.z, cols[2], magic);
-    wv[0][3] = Dq<T>::word(qa.w, cols[3], magic);
+    read_own(w_lds);
+    park_pair(qraw.x, qraw.y, cols[0], cols[1], 0, false);
+    park_pair(qraw.z, qraw.w, cols[2], cols[3], 2, true);
   }
 
   int slot = 0;        // stage of step kt
@@ -424,19 +453,20 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     __builtin_amdgcn_s_barrier();
     if (kt + 2 < k_tiles) issue(kt + 2, fill);
 
+    const uint32_t a_at = a_lds + slot * kStageA + (8 * wm * 2) * kBlockBytes + lane * 16;
+    const int next_slot = slot == kAsyncStages - 1 ? 0 : slot + 1;
+    const bool has_next = kt + 1 < k_tiles;
+    u32x4_t av[4], wa[4], wb[4];
     if (active) {
-      const uint32_t a_at = a_lds + slot * kStageA + (8 * wm * 2) * kBlockBytes + lane * 16;
-      const int next_slot = slot == kAsyncStages - 1 ? 0 : slot + 1;
-      const bool has_next = kt + 1 < k_tiles;
-      u32x4_t av[4];
-      SONAR_TILE_A4(0);
-      wv[1][0] = Dq<T>::word(qb.x, cols[0], magic);
-      wv[1][1] = Dq<T>::word(qb.y, cols[1], magic);
-      SONAR_TILE_MFMA16(0, 0);
+      SONAR_TILE_XA(wa, 0, 0);
+      SONAR_TILE_MFMA16(wa, 0);
       SONAR_TILE_A4(8192);
-      wv[1][2] = Dq<T>::word(qb.z, cols[2], magic);
-      wv[1][3] = Dq<T>::word(qb.w, cols[3], magic);
-      SONAR_TILE_MFMA16(0, 4);
+      SONAR_TILE_MFMA16(wa, 4);
+      SONAR_TILE_XA(wb, 4096, 1024);
+    }
+    // every wavefront has read the weights of this step: those of the next may be parked
+    __builtin_amdgcn_s_barrier();
+    if (active) {
       if (has_next) {
         // stage kt + 1 has landed once at most the copies of stage kt + 2 are outstanding
         if (kt + 2 < k_tiles) {
@@ -444,25 +474,18 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
         } else {
           asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         }
-        SONAR_TILE_W(w_lds + next_slot * kWaveStage);
+        read_own(w_lds + next_slot * kWaveStage);
+        park_pair(qraw.x, qraw.y, cols[0], cols[1], 0, false);
       }
-      SONAR_TILE_A4(1024);
-      if (has_next) {
-        make_cols();
-        wv[0][0] = Dq<T>::word(qa.x, cols[0], magic);
-        wv[0][1] = Dq<T>::word(qa.y, cols[1], magic);
-      }
-      SONAR_TILE_MFMA16(1, 0);
+      SONAR_TILE_MFMA16(wb, 0);
       SONAR_TILE_A4(9216);
-      if (has_next) {
-        wv[0][2] = Dq<T>::word(qa.z, cols[2], magic);
-        wv[0][3] = Dq<T>::word(qa.w, cols[3], magic);
-      }
-      SONAR_TILE_MFMA16(1, 4);
+      if (has_next) park_pair(qraw.z, qraw.w, cols[2], cols[3], 2, true);
+      SONAR_TILE_MFMA16(wb, 4);
     }
     slot = slot == kAsyncStages - 1 ? 0 : slot + 1;
     fill = fill == kAsyncStages - 1 ? 0 : fill + 1;
   }
+#undef SONAR_TILE_XA
 #undef SONAR_TILE_MFMA16
 #undef SONAR_TILE_W
 
