@@ -1,0 +1,46 @@
+// Which kernel a dense call takes and how much scratch it needs: shared by the
+// dispatcher, the tile kernels and sonar_marlin_gemm_scratch_bytes.
+#pragma once
+
+#include <stdint.h>
+
+namespace sonar {
+
+struct GemmPlan {
+  bool tile;        // MFMA-tiled kernel (else the streaming kernels, in 64-row slabs)
+  int k_splits;     // workgroups per 256 x 256 tile along K (tile kernel only)
+  int k_steps_per_split;
+};
+
+inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool async_tile) {
+  GemmPlan plan = {false, 1, 0};
+  if (size_m <= 64 || size_k % 64 != 0) return plan;
+  const int64_t tiles = ((size_m + 255) / 256) * ((size_n + 255) / 256);
+  const int k_steps = (int)(size_k / 64);
+  plan.k_steps_per_split = k_steps;
+  // Few tiles leave compute units idle: split K so that about 256 workgroups
+  // run, each with at least eight K steps.  Partial tiles cost 256 KiB of
+  // fp32 traffic each way, so up to 128 rows the streaming kernels stay ahead.
+  int splits = 1;
+  if (async_tile && tiles < 256) {
+    splits = (int)(256 / tiles);
+    if (splits > k_steps / 8) splits = k_steps / 8;
+    if (splits > 16) splits = 16;
+    if (splits < 1) splits = 1;
+  }
+  if (size_m <= 128) return plan;
+  if (splits == 1 && size_m <= 512 && tiles < 64) return plan;  // slabs use every compute unit
+  plan.tile = true;
+  plan.k_splits = splits;
+  plan.k_steps_per_split = (k_steps + splits - 1) / splits;
+  plan.k_splits = (k_steps + plan.k_steps_per_split - 1) / plan.k_steps_per_split;  // no empty split
+  return plan;
+}
+
+inline size_t plan_partial_bytes(const GemmPlan& plan, int64_t size_m, int64_t size_n) {
+  if (!plan.tile || plan.k_splits <= 1) return 0;
+  const int64_t tiles = ((size_m + 255) / 256) * ((size_n + 255) / 256);
+  return (size_t)plan.k_splits * tiles * 256 * 1024;
+}
+
+}  // namespace sonar

@@ -18,6 +18,7 @@
 #include <cstdlib>
 
 #include "dequant.hpp"
+#include "gemm_plan.hpp"
 #include "wave_reduce.hpp"
 
 namespace sonar {
@@ -25,7 +26,9 @@ namespace sonar {
 // gemm_tile.hip: the MFMA-bound kernel for more than 64 rows
 int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
               const void* scales, const uint32_t* zeros, const int32_t* perm, int dtype, int64_t size_m,
-              int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, hipStream_t st);
+              int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
+              size_t partial_bytes, hipStream_t st);
+bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size);
 
 namespace {
 
@@ -831,11 +834,13 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
 
 using namespace sonar;
 
+namespace {
+size_t stream_scratch_bytes() { return (size_t)2 * cu_count() * kSlotFloat4 * sizeof(float4); }
+}  // namespace
+
 extern "C" size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k) {
-  (void)size_m;
-  (void)size_n;
-  (void)size_k;
-  return (size_t)2 * cu_count() * kSlotFloat4 * sizeof(float4);
+  // partial tiles of the streaming kernels, then those of a split-K tile launch
+  return stream_scratch_bytes() + plan_partial_bytes(plan_gemm(size_m, size_n, size_k, true), size_m, size_n);
 }
 
 extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
@@ -923,13 +928,14 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   }
 
   static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
-  // Up to 512 rows a problem with few 256 x 256 tiles leaves most compute units
-  // idle in the tile kernel; 64-row slabs of the streaming kernel use them all.
-  const int64_t tiles = ((size_m + 255) / 256) * ((size_n + 255) / 256);
-  const bool slabs = size_m <= 128 || (size_m <= 512 && tiles < 64);
-  if (size_m > 64 && size_k % 64 == 0 && !no_tile && !slabs)
+  const bool async_tile = tile_async_applies(chk.has_perm, num_groups, chk.group_size);
+  const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
+  if (plan.tile && !no_tile) {
+    const size_t used = stream_scratch_bytes();
     return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
-                     size_k, num_groups, chk.group_size, st);
+                     size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used,
+                     scratch_bytes > used ? scratch_bytes - used : 0, st);
+  }
 
   for (int64_t m0 = 0; m0 < size_m; m0 += 64) {
     p.a = static_cast<const uint16_t*>(a) + m0 * a_row_stride;

@@ -18,6 +18,7 @@
 #include <cstdlib>
 
 #include "dequant.hpp"
+#include "gemm_plan.hpp"
 
 namespace sonar {
 namespace {
@@ -45,6 +46,10 @@ struct TileParams {
   int num_groups, group_size;
   int chunks_per_strip;
   int tiles_m, tiles_n;
+  // split K: workgroup (tile, split) covers K steps [split * k_steps_per_split, ...) and, when
+  // k_splits > 1, leaves its fp32 tile in `partial` for tile_reduce_kernel
+  int k_splits, k_steps_per_split;
+  float4* partial;
   // grouped (mixture-of-experts) calls only
   const int32_t* sorted_ids;   // slot -> row id of C (row id / top_k of A), >= rows_total: padding
   const float* topk_weights;
@@ -73,16 +78,19 @@ __device__ __forceinline__ uint4 load_a16(const TileParams& p, int row, int k0) 
 // XCD and share its L2: each XCD takes a contiguous run of tiles, rows of A
 // innermost, so the workgroups resident on it share a few panels of W.
 // Returns false for the padding ids of the last run.
-__device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile_m, int& tile_n) {
-  const int total = p.tiles_m * p.tiles_n;
+__device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile_m, int& tile_n, int& split) {
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int total = tiles * p.k_splits;
   const int per_xcd = (total + 7) / 8;
   const int id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  tile_n = id / p.tiles_m;
-  tile_m = id - tile_n * p.tiles_m;
+  split = id / tiles;
+  const int tile = id - split * tiles;
+  tile_n = tile / p.tiles_m;
+  tile_m = tile - tile_n * p.tiles_m;
   return id < total;
 }
 
-inline int tile_grid(const TileParams& p) { return ((p.tiles_m * p.tiles_n + 7) / 8) * 8; }
+inline int tile_grid(const TileParams& p) { return ((p.tiles_m * p.tiles_n * p.k_splits + 7) / 8) * 8; }
 
 template <typename T, bool HAS_ZP, bool HAS_PERM>
 __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const TileParams p) {
@@ -98,8 +106,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const Tile
   const uint32_t magic = magic_register();
   const bool grouped = p.num_groups > 1;
 
-  int tile_m, tile_n;
-  if (!tile_of_workgroup(p, tile_m, tile_n)) return;
+  int tile_m, tile_n, split;
+  if (!tile_of_workgroup(p, tile_m, tile_n, split)) return;  // this kernel is launched with k_splits == 1
   const int m0 = tile_m * kTileM;
   const int strip0 = tile_n * (kTileN / kStripN);
   const int strips_here = min(kTileN / kStripN, p.size_n / kStripN - strip0);
@@ -286,8 +294,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   const uint32_t magic = magic_register();
   const bool grouped = p.num_groups > 1;
 
-  int tile_m, tile_n;
-  if (!tile_of_workgroup(p, tile_m, tile_n)) return;
+  int tile_m, tile_n, split;
+  if (!tile_of_workgroup(p, tile_m, tile_n, split)) return;
   // Grouped calls: row tile t is up to four consecutive 64-slot blocks of one
   // expert, listed in tile_table; rows are slots of sorted_ids.
   int first_slot = 0, tile_rows = kTileM;
@@ -369,9 +377,11 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 #pragma unroll
     for (int mb = 0; mb < 8; ++mb) acc[nb][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-  const int k_tiles = p.size_k / kTileK;
-  issue(0, 0);
-  if (k_tiles > 1) issue(1, 1);
+  // K steps [k_first, k_tiles) of this workgroup
+  const int k_first = split * p.k_steps_per_split;
+  const int k_tiles = min(p.size_k / kTileK, k_first + p.k_steps_per_split);
+  issue(k_first, 0);
+  if (k_first + 1 < k_tiles) issue(k_first + 1, 1);
 
   u32x4_t qraw;
   uint32_t sb0, sb1, sb2, sb3, zw;
@@ -432,7 +442,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
       : "memory")
 
   if (active) {
-    if (k_tiles > 1) {
+    if (k_first + 1 < k_tiles) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -444,7 +454,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 
   int slot = 0;        // stage of step kt
   int fill = 2;        // stage step kt + 2 goes to
-  for (int kt = 0; kt < k_tiles; ++kt) {
+  for (int kt = k_first; kt < k_tiles; ++kt) {
     if (kt + 1 < k_tiles) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
     } else {
@@ -490,6 +500,18 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 #undef SONAR_TILE_W
 
   if (!active) return;
+  if (!GROUPED && p.k_splits > 1) {
+    // partial tile of this K range: one 1-KiB block per accumulator tile
+    float4* dst = p.partial + ((size_t)(split * p.tiles_m * p.tiles_n + tile_n * p.tiles_m + tile_m) * 256 + wave * 32) * 64 + lane;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < 8; ++mb) {
+        const floatx4_t v = acc[nb][mb];
+        dst[(nb * 8 + mb) * 64] = make_float4(v.x, v.y, v.z, v.w);
+      }
+    return;
+  }
   // rows of C this lane writes: one per row block
   long c_row[8];
   float row_w[8];
@@ -535,6 +557,40 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
       *reinterpret_cast<uint2*>(p.c + c_row[mb] * p.size_n + n) = packed;
     }
   }
+}
+
+// Sums the partial tiles of a split-K launch in split order, adds the bias and
+// writes C.  One wavefront per accumulator tile (16 rows x 16 columns).
+template <typename T>
+__global__ __launch_bounds__(256) void tile_reduce_kernel(const TileParams p) {
+  const int lane = threadIdx.x & 63;
+  const int col16 = lane & 15, kb = lane >> 4;
+  const long unit = (long)blockIdx.x * 4 + (threadIdx.x >> 6);   // (tile, wavefront, accumulator tile)
+  const int tiles = p.tiles_m * p.tiles_n;
+  if (unit >= (long)tiles * 256) return;
+  const int tile = (int)(unit >> 8);
+  const int wave = (int)(unit >> 5) & 7;
+  const int nb = (int)(unit & 31) >> 3, mb = (int)unit & 7;
+  const int tile_n = tile / p.tiles_m, tile_m = tile - tile_n * p.tiles_m;
+  const int strip = tile_n * (kTileN / kStripN) + (wave & 3);
+  const int m = tile_m * kTileM + 128 * (wave >> 2) + 16 * mb + col16;
+  if (strip * kStripN >= p.size_n) return;
+  floatx4_t acc = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < p.k_splits; ++s) {
+    const float4 v = p.partial[((size_t)(s * tiles + tile) * 256 + (unit & 255)) * 64 + lane];
+    acc += floatx4_t{v.x, v.y, v.z, v.w};
+  }
+  if (m >= p.size_m) return;
+  const int nl = 16 * nb + 4 * kb;
+  float bias[4] = {0.f, 0.f, 0.f, 0.f};
+  if (p.bias) {
+#pragma unroll
+    for (int r = 0; r < 4; ++r) bias[r] = Dq<T>::to_float(p.bias[strip * kStripN + scale_slot(nl + r, false)]);
+  }
+  uint2 o;
+  o.x = (uint32_t)Dq<T>::from_float(acc.x + bias[0]) | ((uint32_t)Dq<T>::from_float(acc.y + bias[1]) << 16);
+  o.y = (uint32_t)Dq<T>::from_float(acc.z + bias[2]) | ((uint32_t)Dq<T>::from_float(acc.w + bias[3]) << 16);
+  *reinterpret_cast<uint2*>(p.c + (long)m * p.size_n + strip * kStripN + nl) = o;
 }
 
 // Builds the row-tile table of a grouped call: runs of blocks with the same
@@ -607,11 +663,17 @@ int launch_tile(const TileParams& p, hipStream_t st) {
 
 }  // namespace
 
+// The asynchronous tile kernel needs groups of at least 64 rows and no gather of A.
+bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size) {
+  return !has_perm && (num_groups == 1 || group_size % kTileK == 0);
+}
+
 // Called by sonar_marlin_gemm for size_m > 64.  Shapes and pointers have been
 // validated by the caller; size_k % 64 == 0 is required here.
 int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
               const void* scales, const uint32_t* zeros, const int32_t* perm, int dtype, int64_t size_m,
-              int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, hipStream_t st) {
+              int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
+              size_t partial_bytes, hipStream_t st) {
   TileParams p;
   p.a = static_cast<const uint16_t*>(a);
   p.lda = a_row_stride;
@@ -629,6 +691,9 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   p.chunks_per_strip = (int)(size_k / kChunkK);
   p.tiles_m = (int)((size_m + kTileM - 1) / kTileM);
   p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);
+  p.k_splits = 1;
+  p.k_steps_per_split = (int)(size_k / kTileK);
+  p.partial = nullptr;
   p.sorted_ids = nullptr;
   p.topk_weights = nullptr;
   p.tile_table = nullptr;
@@ -637,13 +702,26 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   const bool zp = zeros != nullptr, pm = perm != nullptr;
   int rc;
   static const bool no_async = getenv("SONAR_MARLIN_NO_ASYNC_TILE") != nullptr;  // debugging aid
-  if (!pm && !no_async && (num_groups == 1 || group_size % kTileK == 0)) {
+  if (tile_async_applies(pm, num_groups, group_size) && !no_async) {
+    const GemmPlan plan = plan_gemm(size_m, size_n, size_k, true);
+    if (plan.k_splits > 1 && partial != nullptr && partial_bytes >= plan_partial_bytes(plan, size_m, size_n)) {
+      p.k_splits = plan.k_splits;
+      p.k_steps_per_split = plan.k_steps_per_split;
+      p.partial = static_cast<float4*>(partial);
+    }
     if (dtype == SONAR_DTYPE_F16)
       rc = zp ? launch_tile_async<_Float16, true>(p, st) : launch_tile_async<_Float16, false>(p, st);
     else
       rc = zp ? launch_tile_async<__bf16, true>(p, st) : launch_tile_async<__bf16, false>(p, st);
     if (rc) return rc;
-    return launch_status("marlin_tile_async_kernel");
+    if (int rc2 = launch_status("marlin_tile_async_kernel")) return rc2;
+    if (p.k_splits > 1) {
+      const int blocks = p.tiles_m * p.tiles_n * 64;
+      if (dtype == SONAR_DTYPE_F16) tile_reduce_kernel<_Float16><<<blocks, 256, 0, st>>>(p);
+      else tile_reduce_kernel<__bf16><<<blocks, 256, 0, st>>>(p);
+      return launch_status("tile_reduce_kernel");
+    }
+    return SONAR_OK;
   }
   if (dtype == SONAR_DTYPE_F16) {
     rc = zp ? (pm ? launch_tile<_Float16, true, true>(p, st) : launch_tile<_Float16, true, false>(p, st))
@@ -693,6 +771,9 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.group_size = group_size;
   p.chunks_per_strip = (int)(size_k / kChunkK);
   p.tiles_m = max_tiles;
+  p.k_splits = 1;
+  p.k_steps_per_split = (int)(size_k / kTileK);
+  p.partial = nullptr;
   p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);
   p.sorted_ids = sorted_ids;
   p.topk_weights = topk_weights;
