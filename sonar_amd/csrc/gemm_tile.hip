@@ -461,7 +461,10 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     __builtin_amdgcn_s_barrier();
-    if (kt + 2 < k_tiles) issue(kt + 2, fill);
+    // The two wavefronts of a SIMD (same strip, wm = 0 and 1) issue their copies
+    // at different points of the step, so that one computes while the other is
+    // held up by the memory pipeline.
+    if (wm == 0 && kt + 2 < k_tiles) issue(kt + 2, fill);
 
     const uint32_t a_at = a_lds + slot * kStageA + (8 * wm * 2) * kBlockBytes + lane * 16;
     const int next_slot = slot == kAsyncStages - 1 ? 0 : slot + 1;
@@ -478,8 +481,9 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     __builtin_amdgcn_s_barrier();
     if (active) {
       if (has_next) {
-        // stage kt + 1 has landed once at most the copies of stage kt + 2 are outstanding
-        if (kt + 2 < k_tiles) {
+        // stage kt + 1 has landed once nothing but the copies of stage kt + 2 (issued
+        // already only by the wm = 0 wavefronts) is outstanding
+        if (wm == 0 && kt + 2 < k_tiles) {
           asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
         } else {
           asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -488,6 +492,9 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
         park_pair(qraw.x, qraw.y, cols[0], cols[1], 0, false);
       }
       SONAR_TILE_MFMA16(wb, 0);
+    }
+    if (wm == 1 && kt + 2 < k_tiles) issue(kt + 2, fill);
+    if (active) {
       SONAR_TILE_A4(9216);
       if (has_next) park_pair(qraw.z, qraw.w, cols[2], cols[3], 2, true);
       SONAR_TILE_MFMA16(wb, 4);
