@@ -423,21 +423,26 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   };
 #define SONAR_TILE_MFMA16(wv, mb0)                                                                 \
   _Pragma("unroll") for (int i = 0; i < 4; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j)      \
-      acc[j][(mb0) + i] = Dq<T>::mfma(__builtin_bit_cast(vec8, wv[j]), __builtin_bit_cast(vec8, av[i]), acc[j][(mb0) + i])
-// four weight operand blocks of k block h of this strip and four blocks of A
+      acc[j][(mb0) + i] =                                                                          \
+          Dq<T>::mfma(__builtin_bit_cast(vec8, wv[j]), __builtin_bit_cast(vec8, av[(mb0) + i]), acc[j][(mb0) + i])
+// four weight operand blocks of k block h of this strip and the eight blocks of A of that k block
 #define SONAR_TILE_XA(wv, x_off, a_off)                                                            \
   asm volatile(                                                                                    \
-      "ds_read_b128 %0, %8 offset:" #x_off "\n\t"                                                  \
-      "ds_read_b128 %1, %8 offset:" #x_off "+1024\n\t"                                             \
-      "ds_read_b128 %2, %8 offset:" #x_off "+2048\n\t"                                             \
-      "ds_read_b128 %3, %8 offset:" #x_off "+3072\n\t"                                             \
-      "ds_read_b128 %4, %9 offset:" #a_off "\n\t"                                                  \
-      "ds_read_b128 %5, %9 offset:" #a_off "+2048\n\t"                                             \
-      "ds_read_b128 %6, %9 offset:" #a_off "+4096\n\t"                                             \
-      "ds_read_b128 %7, %9 offset:" #a_off "+6144\n\t"                                             \
+      "ds_read_b128 %0, %12 offset:" #x_off "\n\t"                                                 \
+      "ds_read_b128 %1, %12 offset:" #x_off "+1024\n\t"                                            \
+      "ds_read_b128 %2, %12 offset:" #x_off "+2048\n\t"                                            \
+      "ds_read_b128 %3, %12 offset:" #x_off "+3072\n\t"                                            \
+      "ds_read_b128 %4, %13 offset:" #a_off "\n\t"                                                 \
+      "ds_read_b128 %5, %13 offset:" #a_off "+2048\n\t"                                            \
+      "ds_read_b128 %6, %13 offset:" #a_off "+4096\n\t"                                            \
+      "ds_read_b128 %7, %13 offset:" #a_off "+6144\n\t"                                            \
+      "ds_read_b128 %8, %13 offset:" #a_off "+8192\n\t"                                            \
+      "ds_read_b128 %9, %13 offset:" #a_off "+10240\n\t"                                           \
+      "ds_read_b128 %10, %13 offset:" #a_off "+12288\n\t"                                          \
+      "ds_read_b128 %11, %13 offset:" #a_off "+14336\n\t"                                          \
       "s_waitcnt lgkmcnt(0)"                                                                       \
       : "=&v"(wv[0]), "=&v"(wv[1]), "=&v"(wv[2]), "=&v"(wv[3]), "=&v"(av[0]), "=&v"(av[1]),        \
-        "=&v"(av[2]), "=&v"(av[3])                                                                 \
+        "=&v"(av[2]), "=&v"(av[3]), "=&v"(av[4]), "=&v"(av[5]), "=&v"(av[6]), "=&v"(av[7])         \
       : "v"(x_strip), "v"(a_at)                                                                    \
       : "memory")
 
@@ -469,11 +474,10 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     const uint32_t a_at = a_lds + slot * kStageA + (8 * wm * 2) * kBlockBytes + lane * 16;
     const int next_slot = slot == kAsyncStages - 1 ? 0 : slot + 1;
     const bool has_next = kt + 1 < k_tiles;
-    u32x4_t av[4], wa[4], wb[4];
+    u32x4_t av[8], wa[4], wb[4];
     if (active) {
       SONAR_TILE_XA(wa, 0, 0);
       SONAR_TILE_MFMA16(wa, 0);
-      SONAR_TILE_A4(8192);
       SONAR_TILE_MFMA16(wa, 4);
       SONAR_TILE_XA(wb, 4096, 1024);
     }
@@ -495,7 +499,6 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     }
     if (wm == 1 && kt + 2 < k_tiles) issue(kt + 2, fill);
     if (active) {
-      SONAR_TILE_A4(9216);
       if (has_next) park_pair(qraw.z, qraw.w, cols[2], cols[3], 2, true);
       SONAR_TILE_MFMA16(wb, 4);
     }
