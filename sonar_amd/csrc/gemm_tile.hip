@@ -269,17 +269,6 @@ constexpr int kAsyncW = kTileWaves * kAsyncStages * kWaveStage;
 constexpr int kAsyncLds = kAsyncA + kAsyncW + kStageB;   // + the dequantised weights of one step
 constexpr int kAsyncCopies = 6;
 
-#define SONAR_TILE_A4(h_off)                                                                       \
-  asm volatile(                                                                                    \
-      "ds_read_b128 %0, %4 offset:" #h_off "\n\t"                                                  \
-      "ds_read_b128 %1, %4 offset:" #h_off "+2048\n\t"                                             \
-      "ds_read_b128 %2, %4 offset:" #h_off "+4096\n\t"                                             \
-      "ds_read_b128 %3, %4 offset:" #h_off "+6144\n\t"                                             \
-      "s_waitcnt lgkmcnt(0)"                                                                       \
-      : "=&v"(av[0]), "=&v"(av[1]), "=&v"(av[2]), "=&v"(av[3])                                     \
-      : "v"(a_at)                                                                                  \
-      : "memory")
-
 template <typename T, bool HAS_ZP, bool GROUPED>
 __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
