@@ -266,3 +266,30 @@ def test_moe_tiled_and_streaming_kernels_agree():
         assert ok, worst
     ok, *worst = mo.gemm_tolerance_ok(tiled, streamed)
     assert ok, worst
+
+
+def test_full_size_grouped_tile_gemm_agrees_with_dense_rows():
+    """Mixtral-sized grouped GEMM at 4096 tokens (64-slot blocks, tiled kernel):
+    every routed slot must equal the dense GEMM of its token with its expert."""
+    from sonar_amd import fused_moe
+    m, e, top_k, k, n = 4096, 8, 2, 4096, 2048
+    ex = Experts(13, e, k, n, 128, "bf16")
+    gen = torch.Generator(device=gu.DEV).manual_seed(2)
+    a = (torch.randn((m, k), device=gu.DEV, generator=gen) * 0.5).to(torch.bfloat16)
+    logits = torch.randn((m, e), device=gu.DEV, generator=gen)
+    tw, ti = torch.topk(torch.softmax(logits, dim=1), top_k, dim=1)
+    ti = ti.to(torch.int32)
+    bs = fused_moe.moe_block_size(m, top_k, e)
+    assert bs == 64
+    sorted_ids, expert_ids, past = fused_moe.moe_align_block_size(ti, bs, e)
+    got = ex.gemm(a, sorted_ids.cpu().numpy(), expert_ids.cpu().numpy(), int(past[0]), tw.cpu().numpy(), bs, top_k, m,
+                  False)
+    assert bool(torch.isfinite(got.float()).all())
+    scale = float(got.float().abs().max())
+    ti_host = ti.cpu().numpy()
+    rng = np.random.default_rng(0)
+    for t in rng.integers(0, m, 6):
+        for j in range(top_k):
+            dense = ex.layers[int(ti_host[t, j])].gemm(a[t:t + 1].contiguous(), 1)
+            err = float((dense.float() - got[t * top_k + j].float()).abs().max())
+            assert err <= 1e-2 * scale, (t, j, err, scale)
