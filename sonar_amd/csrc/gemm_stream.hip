@@ -294,13 +294,15 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
 // it can see it would wait for every outstanding copy, which would drain the
 // prefetch on every unit.
 
-constexpr int kFastWaves = 8;
 constexpr int kSlotS = 4096;       // inside a weight slot, after 4 chunks x 1 KiB: 64 scales, 8 zero-point words
 constexpr int kSlotBytes = 4096 + 256;
 constexpr int kWaveA = 2 * kSlotBytes;            // the activation slot follows the two weight slots
 constexpr int kWaveLds = 2 * kSlotBytes + 4096;   // LDS bytes per wavefront
 constexpr int kWeightCopies = 5;   // asynchronous copies per unit: 4 weight chunks + 1 scale row
-constexpr int kFastLds = kFastWaves * kWaveLds + kFastWaves * 4 * 64 * 16;
+// A workgroup of the fast kernel has 8 wavefronts (one workgroup per compute
+// unit), or 4 (two per compute unit: a grid with more workgroups than compute
+// units then runs them side by side instead of one after the other).
+constexpr int fast_lds_bytes(int waves) { return waves * kWaveLds + waves * 4 * 64 * 16; }
 
 struct FastLane {
   uint32_t a_off;       // byte offset of this lane's 16 bytes inside a 32-column slice of A
@@ -400,7 +402,7 @@ __device__ __forceinline__ bf16x8_t raw_operand_bf16(uint32_t q, uint32_t magic)
       : "v"(q_at), "v"(a_at), "v"(z_at), "v"(s_at)                                                 \
       : "memory")
 
-template <typename T, bool HAS_ZP>
+template <typename T, bool HAS_ZP, int kFastWaves>
 __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams p,
                                                                              const int unit_group_shift) {
   typedef typename Dq<T>::vec8 vec8;
@@ -760,16 +762,23 @@ void launch_stream_mb(const StreamParams& p, bool has_perm, hipStream_t st) {
   }
 }
 
-template <typename T, bool HAS_ZP>
-int launch_fast(const StreamParams& p, int unit_group_shift, hipStream_t st) {
+template <typename T, bool HAS_ZP, int WAVES>
+int launch_fast_waves(const StreamParams& p, int unit_group_shift, hipStream_t st) {
   static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_stream_fast_kernel<T, HAS_ZP>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kFastLds));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_stream_fast_kernel<T, HAS_ZP, WAVES>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds_bytes(WAVES)));
     attr_set = true;
   }
-  marlin_stream_fast_kernel<T, HAS_ZP><<<p.parts, kFastWaves * 64, kFastLds, st>>>(p, unit_group_shift);
+  marlin_stream_fast_kernel<T, HAS_ZP, WAVES>
+      <<<p.parts, WAVES * 64, fast_lds_bytes(WAVES), st>>>(p, unit_group_shift);
   return SONAR_OK;
+}
+
+template <typename T, bool HAS_ZP>
+int launch_fast(const StreamParams& p, int unit_group_shift, bool half_workgroups, hipStream_t st) {
+  return half_workgroups ? launch_fast_waves<T, HAS_ZP, 4>(p, unit_group_shift, st)
+                         : launch_fast_waves<T, HAS_ZP, 8>(p, unit_group_shift, st);
 }
 
 template <typename T>
@@ -953,12 +962,15 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                       (long)p.size_m * a_row_stride * 2 < (1L << 31);
     if (fast) {
       int rc;
+      // more workgroups than compute units (one per strip): two small ones per compute unit
+      static const bool no_half = getenv("SONAR_MARLIN_NO_HALF_WG") != nullptr;  // debugging aid
+      const bool half = !no_half && p.parts > cus;
       if (dtype == SONAR_DTYPE_F16)
-        rc = chk.has_zp ? launch_fast<_Float16, true>(p, unit_group_shift, st)
-                        : launch_fast<_Float16, false>(p, unit_group_shift, st);
+        rc = chk.has_zp ? launch_fast<_Float16, true>(p, unit_group_shift, half, st)
+                        : launch_fast<_Float16, false>(p, unit_group_shift, half, st);
       else
-        rc = chk.has_zp ? launch_fast<__bf16, true>(p, unit_group_shift, st)
-                        : launch_fast<__bf16, false>(p, unit_group_shift, st);
+        rc = chk.has_zp ? launch_fast<__bf16, true>(p, unit_group_shift, half, st)
+                        : launch_fast<__bf16, false>(p, unit_group_shift, half, st);
       if (rc) return rc;
     } else if (dtype == SONAR_DTYPE_F16) {
       if (chk.has_zp) launch_stream_mb<_Float16, true>(p, chk.has_perm, st);
