@@ -244,30 +244,39 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const Tile
 // The same tile with every operand arriving through asynchronous global -> LDS
 // copies, three K steps deep, so no vector register holds bytes in flight and
 // the copies of step i+2 are issued before the matrix work of step i.
-//   * A: a ring of three 32-KiB stages shared by the workgroup; wavefront w
-//     copies both k blocks of row blocks w and w+8 of a stage.
-//   * W: the packed chunks are already in operand order.  The two wavefronts
-//     that share a strip split its two chunks of a step: each copies one chunk
-//     (and the scale / zero-point row of the step's group) into a private
-//     ring, dequantises it one step ahead in the shadow of its MFMAs and
-//     parks the four operand blocks in a 32-KiB exchange buffer, from which
-//     both read the step's eight blocks.  Every packed word is therefore
-//     dequantised once per workgroup (the VALU work, 13 instructions per word,
-//     is what bounds this loop once the copies are hidden).
-// Copies of a wavefront complete in issue order, six per stage, so "stage i
-// has landed" is s_waitcnt vmcnt(6); a barrier at the top of a step makes
-// every wavefront's share of A and of the dequantised weights visible and frees
-// the stage consumed in step i-1; a second one, after the last read of the
-// exchange buffer, lets the weights of step i+1 be written into it.
+//   * A: a ring of three 32-KiB stages shared by the workgroup, each 32
+//     regions of 8 rows x 128 bytes; wavefront w copies regions 4w..4w+3, one
+//     copy per region, eight whole 128-byte lines per copy.
+//   * W: the packed chunks are already in operand order.  Every wavefront
+//     copies the two chunks of its strip (and the scale / zero-point row of the
+//     step's group) into a private ring and dequantises them in registers.
+// The eight wavefronts form two groups (wm = 0: rows 0..127 of the tile, wm = 1:
+// rows 128..255); each SIMD holds one wavefront of either group.  A K step is
+// two half steps (k blocks 0 and 1), a half step is a "fetch" phase (LDS reads
+// of the 8 blocks of A and of one packed chunk, dequantisation: LDS and VALU
+// work) followed by a "multiply" phase (32 MFMAs).  Phases end with a
+// workgroup barrier and group 1 runs one phase behind group 0, so that on
+// every SIMD one wavefront multiplies while the other fetches: the matrix
+// cores see a steady stream although a single wavefront never overlaps its own
+// LDS waits, VALU work and MFMAs.
+// Copies of a wavefront complete in issue order, seven per stage, so "stage i
+// has landed" is s_waitcnt vmcnt(7) while the copies of stage i+1 are
+// outstanding.  With p = 4 kt + 2 b (+1 for group 1) the phase in which the
+// fetch of (step kt, k block b) runs: stage kt is read in phases 4kt..4kt+3; the
+// copies of stage kt+2 go to the slot of stage kt-1 and are issued in the two
+// fetch phases of step kt, phases 4kt..4kt+3, after the barrier that ends
+// phase 4kt-1; every wavefront waits for its copies of stage kt+1 at the end of
+// its fetch of (kt, 1), phases 4kt+2 and 4kt+3, before the barrier that starts
+// phase 4kt+4.
 // LDS is read from asm blocks only (the compiler cannot tell which LDS bytes a
 // copy writes and would otherwise wait for all copies before any LDS access).
 // Needs group_size % 64 == 0 (or one group) and no act-order.
 constexpr int kAsyncStages = 3;
-constexpr int kWaveStage = kBlockBytes + 256;       // one weight chunk + 64 scales + 8 zero-point words
+constexpr int kWaveStage = 2 * kBlockBytes + 256;   // two weight chunks + 64 scales + 8 zero-point words
 constexpr int kAsyncA = kAsyncStages * kStageA;
 constexpr int kAsyncW = kTileWaves * kAsyncStages * kWaveStage;
-constexpr int kAsyncLds = kAsyncA + kAsyncW + kStageB;   // + the dequantised weights of one step
-constexpr int kAsyncCopies = 6;
+constexpr int kAsyncLds = kAsyncA + kAsyncW;
+constexpr int kAsyncCopies = 7;
 
 template <typename T, bool HAS_ZP, bool GROUPED>
 __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(const TileParams p) {
@@ -305,22 +314,29 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   const int strip = strip0 + (active ? wn : strips_here - 1);
 
   // ---- copy sources
+  // A stage is 32 regions of 1 KiB: region 2 rb + h holds rows 8h..8h+7 of row
+  // block rb, 128 bytes (both k blocks) each.  One copy fills one region: its
+  // lanes 8r..8r+7 fetch the eight 16-byte pieces of one 128-byte line of row r,
+  // so an instruction touches 8 whole lines (16 rows x 64 bytes per instruction,
+  // the operand-block shape, moves a third of the bytes per cycle).  Piece q of
+  // row r sits at 16-byte slot q ^ r of the row, which keeps the operand reads
+  // (16 rows, one piece each) off each other's banks.  Wavefront w fills
+  // regions 4w..4w+3.
   const char* a_src[4];
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
-    // operand block of copy i: row block wave + 8 (i / 2), k block i % 2, so that the
-    // two halves of every 128-byte line of A are requested back to back by one wavefront
-    const int blk = 2 * (wave + 8 * (i >> 1)) + (i & 1);
+    const int region = 4 * wave + i;
+    const int r8 = lane >> 3;
+    const int in_tile = 16 * (region >> 1) + 8 * (region & 1) + r8;
     int row;
     if (GROUPED) {
-      const int r = 16 * (blk >> 1) + col16;
-      const int id = r < tile_rows ? p.sorted_ids[first_slot + r] : p.rows_total;
+      const int id = in_tile < tile_rows ? p.sorted_ids[first_slot + in_tile] : p.rows_total;
       row = (unsigned)id < (unsigned)p.rows_total ? id / p.top_k : 0;  // padding slots read row 0, never stored
     } else {
-      row = m0 + 16 * (blk >> 1) + col16;
+      row = m0 + in_tile;
       if (row >= p.size_m) row = p.size_m - 1;  // rows past M are computed and never stored
     }
-    a_src[i] = reinterpret_cast<const char*>(p.a) + ((long)row * p.lda + 32 * (blk & 1) + 8 * kb) * 2;
+    a_src[i] = reinterpret_cast<const char*>(p.a) + ((long)row * p.lda + 8 * ((lane & 7) ^ r8)) * 2;
   }
   const uint4* b_src = p.b + expert * p.expert_b_stride + (size_t)(unsigned)(strip * p.chunks_per_strip) * 64 + lane;
   const char* s_src;
@@ -336,29 +352,33 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   const uint32_t a_lds = (uint32_t)(uintptr_t)(lds_void_t*)smem;
   const uint32_t w_lds = (uint32_t)(uintptr_t)(lds_void_t*)wring;
 
-  auto issue = [&](int kt, int slot) {
-    char* sa = smem + slot * kStageA;
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-      __builtin_amdgcn_global_load_lds((glb_void_t*)(a_src[i] + (long)kt * (kTileK * 2)),
-                                       (lds_void_t*)(sa + (2 * (wave + 8 * (i >> 1)) + (i & 1)) * kBlockBytes), 16, 0,
-                                       0);
+  // copy `idx` (0..6) of the stage of step kt: four blocks of A, two weight chunks, one scale row
+  auto issue_one = [&](int kt, int slot, int idx) {
+    if (idx < 4) {
+      char* sa = smem + slot * kStageA;
+      __builtin_amdgcn_global_load_lds((glb_void_t*)(a_src[idx] + (long)kt * (kTileK * 2)),
+                                       (lds_void_t*)(sa + (4 * wave + idx) * kBlockBytes), 16, 0, 0);
+      return;
+    }
     char* sw = wring + slot * kWaveStage;
-    const uint4* g = b_src + (size_t)(2 * kt + wm) * 64;   // this wavefront's chunk: k block wm
-    __builtin_amdgcn_global_load_lds((glb_void_t*)g, (lds_void_t*)sw, 16, 0, 0);
+    if (idx < 6) {
+      const uint4* g = b_src + (size_t)(2 * kt + (idx - 4)) * 64;   // the two chunks of this step
+      __builtin_amdgcn_global_load_lds((glb_void_t*)g, (lds_void_t*)(sw + (idx - 4) * kBlockBytes), 16, 0, 0);
+      return;
+    }
     const int grp = grouped ? (kt * kTileK) / p.group_size : 0;
     __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)grp * s_group_stride),
-                                     (lds_void_t*)(sw + kBlockBytes), 4, 0, 0);
+                                     (lds_void_t*)(sw + 2 * kBlockBytes), 4, 0, 0);
+  };
+  auto issue = [&](int kt, int slot) {
+#pragma unroll
+    for (int idx = 0; idx < kAsyncCopies; ++idx) issue_one(kt, slot, idx);
   };
 
   uint32_t s_off[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) s_off[j] = kBlockBytes + 2 * scale_slot(16 * j + col16, grouped);
-  const uint32_t z_off = kBlockBytes + 128 + 4 * zero_point_word(col16);
-  // exchange buffer: operand block ((strip * 2 + k block) * 4 + column block)
-  const uint32_t x_lds = a_lds + kAsyncA + kAsyncW;
-  const uint32_t x_own = x_lds + ((wn * 2 + wm) * 4) * kBlockBytes + lane * 16;
-  const uint32_t x_strip = x_lds + (wn * 2 * 4) * kBlockBytes + lane * 16;
+  for (int j = 0; j < 4; ++j) s_off[j] = 2 * kBlockBytes + 2 * scale_slot(16 * j + col16, grouped);
+  const uint32_t z_off = 2 * kBlockBytes + 128 + 4 * zero_point_word(col16);
 
   floatx4_t acc[4][8];
 #pragma unroll
@@ -370,133 +390,141 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   const int k_first = split * p.k_steps_per_split;
   const int k_tiles = min(p.size_k / kTileK, k_first + p.k_steps_per_split);
   issue(k_first, 0);
-  if (k_first + 1 < k_tiles) issue(k_first + 1, 1);
+  issue(min(k_first + 1, k_tiles - 1), 1);
 
-  u32x4_t qraw;
-  uint32_t sb0, sb1, sb2, sb3, zw;
+  u32x4_t av[8], wv[4], qraw;
+  uint32_t sb0 = 0, sb1 = 0, sb2 = 0, sb3 = 0, zw = 0;
   Col cols[4];
-  // packed words, scales and zero points of this wavefront's chunk of a stage
-  auto read_own = [&](uint32_t w_at) {
-    asm volatile(
-        "ds_read_b128 %0, %6\n\t"
-        "ds_read_u16 %1, %7\n\t"
-        "ds_read_u16 %2, %8\n\t"
-        "ds_read_u16 %3, %9\n\t"
-        "ds_read_u16 %4, %10\n\t"
-        "ds_read_b32 %5, %11\n\t"
-        "s_waitcnt lgkmcnt(0)"
-        : "=&v"(qraw), "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
-        : "v"(w_at + lane * 16), "v"(w_at + s_off[0]), "v"(w_at + s_off[1]), "v"(w_at + s_off[2]),
-          "v"(w_at + s_off[3]), "v"(w_at + z_off)
-        : "memory");
-    const uint32_t sbits[4] = {sb0, sb1, sb2, sb3};
+// Starts one 16-byte LDS read into `dst`; the data is there after the next
+// s_waitcnt lgkmcnt(0) that names `dst` as an operand.  Until then nothing may
+// name `dst` (the hardware does not interlock).
+#define SONAR_TILE_READ(dst, base, off) \
+  asm volatile("ds_read_b128 %0, %1 offset:" #off : "=&v"(dst) : "v"(base) : "memory")
+// Waits for every LDS read in flight; the registers they fill are operands so
+// that no use of them can be scheduled ahead of the wait.
+#define SONAR_TILE_LANDED()                                                                        \
+  asm volatile("s_waitcnt lgkmcnt(0)"                                                              \
+               : "+v"(av[0]), "+v"(av[1]), "+v"(av[2]), "+v"(av[3]), "+v"(av[4]), "+v"(av[5]),     \
+                 "+v"(av[6]), "+v"(av[7])                                                          \
+               :                                                                                   \
+               : "memory")
+  // Starts the reads of the packed chunk of (stage in `slot`, k block b), with
+  // the scales and zero points of the step when `with_scales` (they hold for
+  // both k blocks: a step lies inside one group).  The wavefront's own copies of
+  // that stage must have landed.  The data is picked up by the next fetch().
+  auto raw_start = [&](int slot, int b, bool with_scales) {
+    const uint32_t w_at = w_lds + slot * kWaveStage;
+    const uint32_t q_at = w_at + b * kBlockBytes + lane * 16;
+    if (with_scales) {
+      asm volatile(
+          "ds_read_b128 %0, %6\n\t"
+          "ds_read_u16 %1, %7\n\t"
+          "ds_read_u16 %2, %8\n\t"
+          "ds_read_u16 %3, %9\n\t"
+          "ds_read_u16 %4, %10\n\t"
+          "ds_read_b32 %5, %11"
+          : "=&v"(qraw), "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
+          : "v"(q_at), "v"(w_at + s_off[0]), "v"(w_at + s_off[1]), "v"(w_at + s_off[2]), "v"(w_at + s_off[3]),
+            "v"(w_at + z_off)
+          : "memory");
+    } else {
+      asm volatile("ds_read_b128 %0, %1" : "=&v"(qraw) : "v"(q_at) : "memory");
+    }
+  };
+  // Fetch phase of (stage in `slot`, k block b): picks up the packed chunk
+  // started by raw_start, starts the reads of the eight blocks of A and
+  // dequantises the chunk while they are in flight.
+  auto fetch = [&](int slot, int b, bool with_scales) {
+    asm volatile("s_waitcnt lgkmcnt(0)"
+                 : "+v"(qraw), "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw)
+                 :
+                 : "memory");
+    // operand lane (kb, col16) of row block rb, k block b: piece 4 b + kb of row col16
+    const uint32_t a_at = a_lds + slot * kStageA + (8 * wm * 2 + (col16 >> 3)) * kBlockBytes + (col16 & 7) * 128 +
+                          (((4 * b + kb) ^ (col16 & 7)) * 16);
+    SONAR_TILE_READ(av[0], a_at, 0);
+    SONAR_TILE_READ(av[1], a_at, 2048);
+    SONAR_TILE_READ(av[2], a_at, 4096);
+    SONAR_TILE_READ(av[3], a_at, 6144);
+    SONAR_TILE_READ(av[4], a_at, 8192);
+    SONAR_TILE_READ(av[5], a_at, 10240);
+    SONAR_TILE_READ(av[6], a_at, 12288);
+    SONAR_TILE_READ(av[7], a_at, 14336);
+    if (with_scales) {
+      const uint32_t sbits[4] = {sb0, sb1, sb2, sb3};
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int z = 8;
-      if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
-      cols[j] = Dq<T>::make_col((uint16_t)sbits[j], z);
+      for (int j = 0; j < 4; ++j) {
+        int z = 8;
+        if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
+        cols[j] = Dq<T>::make_col((uint16_t)sbits[j], z);
+      }
     }
+    wv[0] = __builtin_bit_cast(u32x4_t, Dq<T>::word(qraw.x, cols[0], magic));
+    wv[1] = __builtin_bit_cast(u32x4_t, Dq<T>::word(qraw.y, cols[1], magic));
+    wv[2] = __builtin_bit_cast(u32x4_t, Dq<T>::word(qraw.z, cols[2], magic));
+    wv[3] = __builtin_bit_cast(u32x4_t, Dq<T>::word(qraw.w, cols[3], magic));
+    SONAR_TILE_LANDED();
   };
-  // dequantises column blocks j0 and j0 + 1 of the chunk and parks them
-  auto park_pair = [&](uint32_t w0, uint32_t w1, const Col& c0, const Col& c1, int j0, bool last) {
-    const vec8 v0 = Dq<T>::word(w0, c0, magic);
-    const vec8 v1 = Dq<T>::word(w1, c1, magic);
-    if (j0 == 0) {
-      asm volatile("ds_write_b128 %0, %1\n\tds_write_b128 %0, %2 offset:1024" ::"v"(x_own), "v"(v0), "v"(v1) : "memory");
-    } else {
-      asm volatile("ds_write_b128 %0, %1 offset:2048\n\tds_write_b128 %0, %2 offset:3072" ::"v"(x_own), "v"(v0),
-                   "v"(v1)
-                   : "memory");
-    }
-    if (last) asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+  // Multiply phase: 32 MFMAs, ahead of the other wavefront's VALU work in the issue order.
+  auto multiply = [&]() {
+    __builtin_amdgcn_s_setprio(2);
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        acc[j][i] = Dq<T>::mfma(__builtin_bit_cast(vec8, wv[j]), __builtin_bit_cast(vec8, av[i]), acc[j][i]);
+    __builtin_amdgcn_s_setprio(0);
   };
-#define SONAR_TILE_MFMA16(wv, mb0)                                                                 \
-  _Pragma("unroll") for (int i = 0; i < 4; ++i) _Pragma("unroll") for (int j = 0; j < 4; ++j)      \
-      acc[j][(mb0) + i] =                                                                          \
-          Dq<T>::mfma(__builtin_bit_cast(vec8, wv[j]), __builtin_bit_cast(vec8, av[(mb0) + i]), acc[j][(mb0) + i])
-// four weight operand blocks of k block h of this strip and the eight blocks of A of that k block
-#define SONAR_TILE_XA(wv, x_off, a_off)                                                            \
-  asm volatile(                                                                                    \
-      "ds_read_b128 %0, %12 offset:" #x_off "\n\t"                                                 \
-      "ds_read_b128 %1, %12 offset:" #x_off "+1024\n\t"                                            \
-      "ds_read_b128 %2, %12 offset:" #x_off "+2048\n\t"                                            \
-      "ds_read_b128 %3, %12 offset:" #x_off "+3072\n\t"                                            \
-      "ds_read_b128 %4, %13 offset:" #a_off "\n\t"                                                 \
-      "ds_read_b128 %5, %13 offset:" #a_off "+2048\n\t"                                            \
-      "ds_read_b128 %6, %13 offset:" #a_off "+4096\n\t"                                            \
-      "ds_read_b128 %7, %13 offset:" #a_off "+6144\n\t"                                            \
-      "ds_read_b128 %8, %13 offset:" #a_off "+8192\n\t"                                            \
-      "ds_read_b128 %9, %13 offset:" #a_off "+10240\n\t"                                           \
-      "ds_read_b128 %10, %13 offset:" #a_off "+12288\n\t"                                          \
-      "ds_read_b128 %11, %13 offset:" #a_off "+14336\n\t"                                          \
-      "s_waitcnt lgkmcnt(0)"                                                                       \
-      : "=&v"(wv[0]), "=&v"(wv[1]), "=&v"(wv[2]), "=&v"(wv[3]), "=&v"(av[0]), "=&v"(av[1]),        \
-        "=&v"(av[2]), "=&v"(av[3]), "=&v"(av[4]), "=&v"(av[5]), "=&v"(av[6]), "=&v"(av[7])         \
-      : "v"(x_strip), "v"(a_at)                                                                    \
-      : "memory")
+  // end of a phase; nothing may be scheduled across it
+  auto phase_end = [&]() {
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+  };
 
-  if (active) {
-    if (k_first + 1 < k_tiles) {
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    read_own(w_lds);
-    park_pair(qraw.x, qraw.y, cols[0], cols[1], 0, false);
-    park_pair(qraw.z, qraw.w, cols[2], cols[3], 2, true);
-  }
+  // The loop body has no branches: a wavefront past the last strip of the
+  // matrix works on a second copy of the last strip (its results are dropped),
+  // and the copies for steps past the end fetch the last step again, into a
+  // slot nobody reads any more.  So seven copies are outstanding at every wait.
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");  // stage k_first has landed
+  raw_start(0, 0, true);
+  phase_end();
+  if (wm == 1) phase_end();  // group 1 runs one phase behind
 
   int slot = 0;        // stage of step kt
   int fill = 2;        // stage step kt + 2 goes to
   for (int kt = k_first; kt < k_tiles; ++kt) {
-    if (kt + 1 < k_tiles) {
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    }
-    __builtin_amdgcn_s_barrier();
-    // The two wavefronts of a SIMD (same strip, wm = 0 and 1) issue their copies
-    // at different points of the step, so that one computes while the other is
-    // held up by the memory pipeline.
-    if (wm == 0 && kt + 2 < k_tiles) issue(kt + 2, fill);
-
-    const uint32_t a_at = a_lds + slot * kStageA + (8 * wm * 2) * kBlockBytes + lane * 16;
     const int next_slot = slot == kAsyncStages - 1 ? 0 : slot + 1;
-    const bool has_next = kt + 1 < k_tiles;
-    u32x4_t av[8], wa[4], wb[4];
-    if (active) {
-      SONAR_TILE_XA(wa, 0, 0);
-      SONAR_TILE_MFMA16(wa, 0);
-      SONAR_TILE_MFMA16(wa, 4);
-      SONAR_TILE_XA(wb, 4096, 1024);
-    }
-    // every wavefront has read the weights of this step: those of the next may be parked
-    __builtin_amdgcn_s_barrier();
-    if (active) {
-      if (has_next) {
-        // stage kt + 1 has landed once nothing but the copies of stage kt + 2 (issued
-        // already only by the wm = 0 wavefronts) is outstanding
-        if (wm == 0 && kt + 2 < k_tiles) {
-          asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
-        } else {
-          asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        }
-        read_own(w_lds + next_slot * kWaveStage);
-        park_pair(qraw.x, qraw.y, cols[0], cols[1], 0, false);
-      }
-      SONAR_TILE_MFMA16(wb, 0);
-    }
-    if (wm == 1 && kt + 2 < k_tiles) issue(kt + 2, fill);
-    if (active) {
-      if (has_next) park_pair(qraw.z, qraw.w, cols[2], cols[3], 2, true);
-      SONAR_TILE_MFMA16(wb, 4);
-    }
-    slot = slot == kAsyncStages - 1 ? 0 : slot + 1;
+    // ---- half step (kt, 0)
+    // the copies of stage kt + 2 go out in the fetch phases, four and three: a
+    // wavefront waits at a copy while the memory pipeline is busy, which would
+    // starve the matrix cores if it happened between MFMAs
+    const int copy_kt = min(kt + 2, k_tiles - 1);
+#pragma unroll
+    for (int idx = 0; idx < 4; ++idx) issue_one(copy_kt, fill, idx);
+    fetch(slot, 0, true);
+    raw_start(slot, 1, false);
+    phase_end();
+    multiply();
+    phase_end();
+    // ---- half step (kt, 1)
+#pragma unroll
+    for (int idx = 4; idx < kAsyncCopies; ++idx) issue_one(copy_kt, fill, idx);
+    fetch(slot, 1, false);
+    // stage kt + 1 has landed once nothing but the copies of stage kt + 2 is outstanding
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
+    raw_start(next_slot, 0, true);
+    phase_end();
+    multiply();
+    phase_end();
+    slot = next_slot;
     fill = fill == kAsyncStages - 1 ? 0 : fill + 1;
   }
-#undef SONAR_TILE_XA
-#undef SONAR_TILE_MFMA16
-#undef SONAR_TILE_W
+  if (wm == 0) phase_end();  // the barrier that ends group 1's last phase
+  // the last copies and the last read started by raw_start must not outlive the wavefront
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(qraw), "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw)::"memory");
+#undef SONAR_TILE_LANDED
+#undef SONAR_TILE_READ
 
   if (!active) return;
   if (!GROUPED && p.k_splits > 1) {
