@@ -305,7 +305,7 @@ constexpr int kWeightCopies = 5;   // asynchronous copies per unit: 4 weight chu
 constexpr int fast_lds_bytes(int waves) { return waves * kWaveLds + waves * 4 * 64 * 16; }
 
 struct FastLane {
-  uint32_t a_off;       // byte offset of this lane's 16 bytes inside a 32-column slice of A
+  uint32_t a_off[2];    // byte offset of the 16 bytes this lane copies from rows 0..7 / 8..15 of a 64-column slice of A
   const char* s_ptr;    // this lane's dword of the scale / zero-point row of (group 0, strip 0)
   long s_group_stride;  // bytes between groups for s_ptr
   int s_strip_stride;   // bytes between strips for s_ptr
@@ -324,13 +324,20 @@ __device__ __forceinline__ void copy_weights(const StreamParams& p, const FastLa
   __builtin_amdgcn_global_load_lds((glb_void_t*)gs, (lds_void_t*)(slot + kSlotS), 4, 0, 0);
 }
 
+// The 16 x 128 slice of A of one unit, as four regions of 1 KiB: region
+// 2 * half + h holds rows 8h..8h+7, 128 bytes (64 columns) each.  One copy fills
+// one region; its lanes 8r..8r+7 fetch the eight 16-byte pieces of one
+// 128-byte line of row r, so a copy touches 8 whole lines (16 rows x 64 bytes per
+// copy, the operand shape, moves a third of the bytes per cycle).  Piece q of
+// row r sits at 16-byte slot q ^ (r % 8) of the row, which keeps the operand
+// reads (16 rows, one piece each) off each other's banks.
 __device__ __forceinline__ void copy_activations(const StreamParams& p, const FastLane& fl, int unit,
                                                  char* slot) {
-  const char* ga = reinterpret_cast<const char*>(p.a) + (long)unit * (4 * kChunkK * 2) + fl.a_off;
-  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga), (lds_void_t*)(slot), 16, 0, 0);
-  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 64), (lds_void_t*)(slot + 1024), 16, 0, 0);
-  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 128), (lds_void_t*)(slot + 2048), 16, 0, 0);
-  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 192), (lds_void_t*)(slot + 3072), 16, 0, 0);
+  const char* ga = reinterpret_cast<const char*>(p.a) + (long)unit * (4 * kChunkK * 2);
+  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + fl.a_off[0]), (lds_void_t*)(slot), 16, 0, 0);
+  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + fl.a_off[1]), (lds_void_t*)(slot + 1024), 16, 0, 0);
+  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 128 + fl.a_off[0]), (lds_void_t*)(slot + 2048), 16, 0, 0);
+  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 128 + fl.a_off[1]), (lds_void_t*)(slot + 3072), 16, 0, 0);
 }
 
 struct UnitCursor {
@@ -381,9 +388,9 @@ __device__ __forceinline__ bf16x8_t raw_operand_bf16(uint32_t q, uint32_t magic)
       "ds_read_b128 %2, %25 offset:2048\n\t"                                                       \
       "ds_read_b128 %3, %25 offset:3072\n\t"                                                       \
       "ds_read_b128 %4, %26\n\t"                                                                   \
-      "ds_read_b128 %5, %26 offset:1024\n\t"                                                       \
+      "ds_read_b128 %5, %29\n\t"                                                                   \
       "ds_read_b128 %6, %26 offset:2048\n\t"                                                       \
-      "ds_read_b128 %7, %26 offset:3072\n\t"                                                       \
+      "ds_read_b128 %7, %29 offset:2048\n\t"                                                       \
       "ds_read_b128 %8, %27\n\t"                                                                   \
       "ds_read_u16 %9, %28 offset:" #O0 "\n\tds_read_u16 %10, %28 offset:" #O1 "\n\t"              \
       "ds_read_u16 %11, %28 offset:" #O2 "\n\tds_read_u16 %12, %28 offset:" #O3 "\n\t"             \
@@ -399,7 +406,7 @@ __device__ __forceinline__ bf16x8_t raw_operand_bf16(uint32_t q, uint32_t magic)
         "=&v"(row_s[4]), "=&v"(row_s[5]), "=&v"(row_s[6]), "=&v"(row_s[7]), "=&v"(row_s[8]),       \
         "=&v"(row_s[9]), "=&v"(row_s[10]), "=&v"(row_s[11]), "=&v"(row_s[12]), "=&v"(row_s[13]),   \
         "=&v"(row_s[14]), "=&v"(row_s[15])                                                         \
-      : "v"(q_at), "v"(a_at), "v"(z_at), "v"(s_at)                                                 \
+      : "v"(q_at), "v"(a_at), "v"(z_at), "v"(s_at), "v"(a_at ^ 64u)                                \
       : "memory")
 
 template <typename T, bool HAS_ZP, int kFastWaves>
@@ -422,8 +429,12 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
 
   FastLane fl;
   {
-    const int row = col16 < p.size_m ? col16 : p.size_m - 1;  // rows past M are never stored
-    fl.a_off = (uint32_t)((long)row * p.lda * 2 + 16 * (lane >> 4));
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      const int r = 8 * h + (lane >> 3);
+      const int row = r < p.size_m ? r : p.size_m - 1;  // rows past M are never stored
+      fl.a_off[h] = (uint32_t)((long)row * p.lda * 2 + 16 * ((lane & 7) ^ (lane >> 3)));
+    }
     if (HAS_ZP && lane >= 32) {
       fl.s_ptr = reinterpret_cast<const char*>(p.zeros + (lane & 7));
       fl.s_group_stride = (long)(p.size_n / 8) * 4;
@@ -439,6 +450,12 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
 #pragma unroll
   for (int j = 0; j < 4; ++j) s_off[j] = kSlotS + 2 * scale_slot(16 * j + col16, grouped);
   const uint32_t z_off = kSlotS + 128 + 4 * zero_point_word(col16);
+  // Operand lane (k group q4 = lane / 16, row col16) of chunk cc of a unit reads
+  // piece 4 (cc % 2) + q4 of row col16 in region 2 (cc / 2) + col16 / 8 of the
+  // activation slot: a_at for chunk 0, a_at ^ 64 for chunk 1, both + 2048 for
+  // chunks 2 and 3.
+  const uint32_t a_at = ring_lds + kWaveA + (col16 >> 3) * 1024 + (col16 & 7) * 128 +
+                        ((uint32_t)((lane >> 4) ^ (col16 & 7)) * 16);
   // deferred-scale path (bf16): where the scales / zero points of this lane's output rows sit
   constexpr bool kDeferred = __is_same(T, __bf16);
   const int q4 = lane >> 4;
@@ -543,7 +560,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     if constexpr (kDeferred) {
-      const uint32_t q_at = slot_lds + lane * 16, a_at = ring_lds + kWaveA + lane * 16;
+      const uint32_t q_at = slot_lds + lane * 16;
       const uint32_t z_at = slot_lds + row_z_off, s_at = slot_lds + row_s_off;
       if (grouped) {  // scale of (j, r) at byte 16 r + 4 j past s_at
         SONAR_UNIT_READS(0, 16, 32, 48, 4, 20, 36, 52, 8, 24, 40, 56, 12, 28, 44, 60);
@@ -557,9 +574,9 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
           "ds_read_b128 %2, %13 offset:2048\n\t"
           "ds_read_b128 %3, %13 offset:3072\n\t"
           "ds_read_b128 %4, %14\n\t"
-          "ds_read_b128 %5, %14 offset:1024\n\t"
+          "ds_read_b128 %5, %20\n\t"
           "ds_read_b128 %6, %14 offset:2048\n\t"
-          "ds_read_b128 %7, %14 offset:3072\n\t"
+          "ds_read_b128 %7, %20 offset:2048\n\t"
           "ds_read_u16 %8, %15\n\t"
           "ds_read_u16 %9, %16\n\t"
           "ds_read_u16 %10, %17\n\t"
@@ -568,9 +585,8 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
           "s_waitcnt lgkmcnt(0)"
           : "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3), "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3),
             "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
-          : "v"(slot_lds + lane * 16), "v"(ring_lds + kWaveA + lane * 16), "v"(slot_lds + s_off[0]),
-            "v"(slot_lds + s_off[1]), "v"(slot_lds + s_off[2]), "v"(slot_lds + s_off[3]),
-            "v"(slot_lds + z_off)
+          : "v"(slot_lds + lane * 16), "v"(a_at), "v"(slot_lds + s_off[0]), "v"(slot_lds + s_off[1]),
+            "v"(slot_lds + s_off[2]), "v"(slot_lds + s_off[3]), "v"(slot_lds + z_off), "v"(a_at ^ 64u)
           : "memory");
     }
     if (more) {
