@@ -358,21 +358,37 @@ struct UnitCursor {
   }
 };
 
-// bf16 only.  gfx950 has no packed bf16 arithmetic, so forming (v - z) * s per
-// weight costs a mixed-precision fma and half a conversion per element.  The
-// fast kernel instead feeds the matrix cores the exact integers 128 + v (the
-// nibble OR-ed into the mantissa of bf16 128.0) and folds offset and scale into
-// the accumulator once per 128-row unit, which lies inside one group:
-//   sum_k (v_k - z) s a_k = s * (sum_k (128 + v_k) a_k - (128 + z) * sum_k a_k),
+// Forming (v - z) * s per weight costs 13 VALU instructions per packed word in
+// fp16 and 17 in bf16 (gfx950 has no packed bf16 arithmetic), more than the
+// matrix work of a 16-row tile is worth.  The fast kernel instead feeds the
+// matrix cores the exact integers B + v (the nibble OR-ed into the mantissa of
+// B = 1024.0 in fp16, 128.0 in bf16: 7 instructions per word) and folds offset
+// and scale into the accumulator once per 128-row unit, which lies inside one
+// group:
+//   sum_k (v_k - z) s a_k = s * (sum_k (B + v_k) a_k - (B + z) * sum_k a_k),
 // the last sum coming from one more MFMA per chunk with an all-ones operand.
 // Products and sums are exact or fp32, so the result differs from the
-// dequantise-then-multiply form only by not rounding (v - z) * s to bf16 first.
-__device__ __forceinline__ bf16x8_t raw_operand_bf16(uint32_t q, uint32_t magic) {
+// dequantise-then-multiply form only by not rounding (v - z) * s to 16 bits first.
+template <typename T>
+struct RawOperand;
+template <>
+struct RawOperand<_Float16> {
+  static constexpr uint32_t kMagic = 0x64006400u;  // 1024.0 twice
+  static constexpr uint32_t kOnes = 0x3c003c00u;
+  static constexpr float kBase = 1024.f;
+};
+template <>
+struct RawOperand<__bf16> {
+  static constexpr uint32_t kMagic = 0x43004300u;  // 128.0 twice
+  static constexpr uint32_t kOnes = 0x3f803f80u;
+  static constexpr float kBase = 128.f;
+};
+__device__ __forceinline__ u32x4_t raw_operand(uint32_t q, uint32_t magic) {
   const uint32_t e0 = and_or(q, 0x000f000fu, magic);
   const uint32_t e1 = and_or(q >> 4, 0x000f000fu, magic);
   const uint32_t e2 = and_or(q >> 8, 0x000f000fu, magic);
   const uint32_t e3 = and_or(q >> 12, 0x000f000fu, magic);
-  return __builtin_bit_cast(bf16x8_t, u32x4_t{e0, e1, e2, e3});
+  return u32x4_t{e0, e1, e2, e3};
 }
 
 // One unit's operands for the deferred-scale path, issued and awaited inside a
@@ -413,7 +429,6 @@ template <typename T, bool HAS_ZP, int kFastWaves>
 __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams p,
                                                                              const int unit_group_shift) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq<T>::Col Col;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
@@ -421,7 +436,6 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   char* ring = smem + wave * kWaveLds;
   const uint32_t ring_lds = (uint32_t)(uintptr_t)(lds_void_t*)ring;
   const uint32_t red_lds = (uint32_t)(uintptr_t)(lds_void_t*)(smem + kFastWaves * kWaveLds);
-  const uint32_t magic = magic_register();
 
   const int u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
   const int u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
@@ -445,25 +459,19 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
       fl.s_strip_stride = kStripN * 2;
     }
   }
-  // byte offsets, inside a weight slot, of this lane's four scales and its zero-point word
-  uint32_t s_off[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) s_off[j] = kSlotS + 2 * scale_slot(16 * j + col16, grouped);
-  const uint32_t z_off = kSlotS + 128 + 4 * zero_point_word(col16);
   // Operand lane (k group q4 = lane / 16, row col16) of chunk cc of a unit reads
   // piece 4 (cc % 2) + q4 of row col16 in region 2 (cc / 2) + col16 / 8 of the
   // activation slot: a_at for chunk 0, a_at ^ 64 for chunk 1, both + 2048 for
   // chunks 2 and 3.
   const uint32_t a_at = ring_lds + kWaveA + (col16 >> 3) * 1024 + (col16 & 7) * 128 +
                         ((uint32_t)((lane >> 4) ^ (col16 & 7)) * 16);
-  // deferred-scale path (bf16): where the scales / zero points of this lane's output rows sit
-  constexpr bool kDeferred = __is_same(T, __bf16);
+  // where the scales / zero points of this lane's output rows sit inside a weight slot
   const int q4 = lane >> 4;
   const uint32_t row_s_off = kSlotS + (grouped ? 64 * (q4 & 1) + 2 * (q4 >> 1) : 32 * (q4 & 1) + 4 * (q4 >> 1));
   const uint32_t row_z_off = kSlotS + 128 + 16 * (q4 & 1);
   const uint32_t row_z_shift = 16 * (q4 >> 1);
-  const uint32_t magic_bf16 = magic_register(0x43004300u);
-  u32x4_t ones = u32x4_t{0x3f803f80u, 0x3f803f80u, 0x3f803f80u, 0x3f803f80u};
+  const uint32_t magic = magic_register(RawOperand<T>::kMagic);
+  u32x4_t ones = u32x4_t{RawOperand<T>::kOnes, RawOperand<T>::kOnes, RawOperand<T>::kOnes, RawOperand<T>::kOnes};
   asm("" : "+v"(ones));
 
   // Issue order of a wavefront's copies, x being one of its units and W the
@@ -550,7 +558,6 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     // copies of the units after it, then do the arithmetic.
     const uint32_t slot_lds = ring_lds + c_slot * kSlotBytes;
     u32x4_t q0, q1, q2, q3, a0, a1, a2, a3;
-    uint32_t sb0 = 0, sb1 = 0, sb2 = 0, sb3 = 0, zw = 0;
     uint32_t row_s[16];
     u32x4_t row_z = u32x4_t{0u, 0u, 0u, 0u};
     const bool more = cur.index + kFastWaves < u_end;
@@ -559,7 +566,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     } else {
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
-    if constexpr (kDeferred) {
+    {
       const uint32_t q_at = slot_lds + lane * 16;
       const uint32_t z_at = slot_lds + row_z_off, s_at = slot_lds + row_s_off;
       if (grouped) {  // scale of (j, r) at byte 16 r + 4 j past s_at
@@ -567,27 +574,6 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
       } else {        // at byte 64 (j >> 1) + 8 (j & 1) + 16 (r >> 1) + 2 (r & 1)
         SONAR_UNIT_READS(0, 2, 16, 18, 8, 10, 24, 26, 64, 66, 80, 82, 72, 74, 88, 90);
       }
-    } else {
-      asm volatile(
-          "ds_read_b128 %0, %13\n\t"
-          "ds_read_b128 %1, %13 offset:1024\n\t"
-          "ds_read_b128 %2, %13 offset:2048\n\t"
-          "ds_read_b128 %3, %13 offset:3072\n\t"
-          "ds_read_b128 %4, %14\n\t"
-          "ds_read_b128 %5, %20\n\t"
-          "ds_read_b128 %6, %14 offset:2048\n\t"
-          "ds_read_b128 %7, %20 offset:2048\n\t"
-          "ds_read_u16 %8, %15\n\t"
-          "ds_read_u16 %9, %16\n\t"
-          "ds_read_u16 %10, %17\n\t"
-          "ds_read_u16 %11, %18\n\t"
-          "ds_read_b32 %12, %19\n\t"
-          "s_waitcnt lgkmcnt(0)"
-          : "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3), "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3),
-            "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
-          : "v"(slot_lds + lane * 16), "v"(a_at), "v"(slot_lds + s_off[0]), "v"(slot_lds + s_off[1]),
-            "v"(slot_lds + s_off[2]), "v"(slot_lds + s_off[3]), "v"(slot_lds + z_off), "v"(a_at ^ 64u)
-          : "memory");
     }
     if (more) {
       copy_activations(p, fl, fetch.unit, ring + kWaveA);
@@ -598,48 +584,28 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
 
     const u32x4_t qs[4] = {q0, q1, q2, q3};
     const u32x4_t as[4] = {a0, a1, a2, a3};
-    if constexpr (kDeferred) {
-      const floatx4_t zero4 = floatx4_t{0.f, 0.f, 0.f, 0.f};
-      floatx4_t part[4], asum;
+    const floatx4_t zero4 = floatx4_t{0.f, 0.f, 0.f, 0.f};
+    floatx4_t part[4], asum;
 #pragma unroll
-      for (int cc = 0; cc < 4; ++cc) {
-        const bf16x8_t av = __builtin_bit_cast(bf16x8_t, as[cc]);
-        const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-          part[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(raw_operand_bf16(words[j], magic_bf16), av,
-                                                            cc == 0 ? zero4 : part[j], 0, 0, 0);
-        asum = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(bf16x8_t, ones), av,
-                                                       cc == 0 ? zero4 : asum, 0, 0, 0);
-      }
-      const uint32_t zrow[4] = {row_z.x >> row_z_shift, row_z.y >> row_z_shift, row_z.z >> row_z_shift,
-                                row_z.w >> row_z_shift};
+    for (int cc = 0; cc < 4; ++cc) {
+      const vec8 av = __builtin_bit_cast(vec8, as[cc]);
+      const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
 #pragma unroll
       for (int j = 0; j < 4; ++j)
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float sc = __builtin_bit_cast(float, row_s[4 * j + r] << 16);
-          float off = -136.f;
-          if (HAS_ZP) off = -128.f - (float)((zrow[r] >> (4 * j)) & 0xFu);
-          acc[j][r] = __builtin_fmaf(sc, __builtin_fmaf(off, asum[r], part[j][r]), acc[j][r]);
-        }
-    } else {
-      Col cols[4];
-      const uint32_t sbits[4] = {sb0, sb1, sb2, sb3};
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int z = 8;
-        if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
-        cols[j] = Dq<T>::make_col((uint16_t)sbits[j], z);
-      }
-#pragma unroll
-      for (int cc = 0; cc < 4; ++cc) {
-        const vec8 av = __builtin_bit_cast(vec8, as[cc]);
-        const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = Dq<T>::mfma(Dq<T>::word(words[j], cols[j], magic), av, acc[j]);
-      }
+        part[j] = Dq<T>::mfma(__builtin_bit_cast(vec8, raw_operand(words[j], magic)), av, cc == 0 ? zero4 : part[j]);
+      asum = Dq<T>::mfma(__builtin_bit_cast(vec8, ones), av, cc == 0 ? zero4 : asum);
     }
+    const uint32_t zrow[4] = {row_z.x >> row_z_shift, row_z.y >> row_z_shift, row_z.z >> row_z_shift,
+                              row_z.w >> row_z_shift};
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) {
+        const float sc = Dq<T>::to_float((uint16_t)row_s[4 * j + r]);
+        float off = -(RawOperand<T>::kBase + 8.f);
+        if (HAS_ZP) off = -RawOperand<T>::kBase - (float)((zrow[r] >> (4 * j)) & 0xFu);
+        acc[j][r] = __builtin_fmaf(sc, __builtin_fmaf(off, asum[r], part[j][r]), acc[j][r]);
+      }
     cur.advance(kFastWaves, p.units_per_strip);
     c_slot ^= 1;
   }
