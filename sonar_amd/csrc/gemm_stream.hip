@@ -52,6 +52,10 @@ struct StreamParams {
   int units_per_strip;
   int parts;  // number of workgroups of the streaming kernel
   int total_units;
+  // fast kernel only: the launch covers `slabs` blocks of 16 rows, workgroup
+  // slab * grid_parts + part works on rows 16 slab.. of part `part` (ids past
+  // `parts` inside a slab are padding)
+  int slabs, grid_parts;
 };
 
 // Unit indices are 32-bit: the host checks total_units * parts < 2^31.
@@ -426,10 +430,20 @@ __device__ __forceinline__ u32x4_t raw_operand(uint32_t q, uint32_t magic) {
       : "memory")
 
 template <typename T, bool HAS_ZP, int kFastWaves>
-__global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams p,
+__global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams params,
                                                                              const int unit_group_shift) {
   typedef typename Dq<T>::vec8 vec8;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
+  // The slabs of one part have ids congruent mod 8 (grid_parts is a multiple of
+  // 8 when there are several), so they run on one XCD and the second to ask
+  // for a weight chunk finds it in that XCD's L2.
+  StreamParams p = params;
+  const int part = blockIdx.x % p.grid_parts;
+  const int slab = blockIdx.x / p.grid_parts;
+  if (part >= p.parts) return;
+  p.a += (long)slab * 16 * p.lda;
+  p.c += (long)slab * 16 * p.size_n;
+  p.size_m = min(16, p.size_m - 16 * slab);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col16 = lane & 15;
@@ -437,8 +451,8 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   const uint32_t ring_lds = (uint32_t)(uintptr_t)(lds_void_t*)ring;
   const uint32_t red_lds = (uint32_t)(uintptr_t)(lds_void_t*)(smem + kFastWaves * kWaveLds);
 
-  const int u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
-  const int u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
+  const int u_begin = range_begin(part, p.total_units, p.parts);
+  const int u_end = range_begin(part + 1, p.total_units, p.parts);
   const bool grouped = p.num_groups > 1;
 
   FastLane fl;
@@ -753,7 +767,7 @@ int launch_fast_waves(const StreamParams& p, int unit_group_shift, hipStream_t s
     attr_set = true;
   }
   marlin_stream_fast_kernel<T, HAS_ZP, WAVES>
-      <<<p.parts, WAVES * 64, fast_lds_bytes(WAVES), st>>>(p, unit_group_shift);
+      <<<p.grid_parts * p.slabs, WAVES * 64, fast_lds_bytes(WAVES), st>>>(p, unit_group_shift);
   return SONAR_OK;
 }
 
@@ -892,26 +906,6 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   p.num_groups = (int)num_groups;
   p.group_size = chk.group_size;
   p.chunks_per_strip = (int)(size_k / kChunkK);
-  p.unit_chunks = p.chunks_per_strip % 4 == 0 ? 4 : (p.chunks_per_strip % 2 == 0 ? 2 : 1);
-  // slabs of more than 32 rows work on half units (see unit_buffer_chunks)
-  if (size_m > 32 && p.unit_chunks == 4) p.unit_chunks = 2;
-  p.units_per_strip = p.chunks_per_strip / p.unit_chunks;
-  const int64_t total_units = (size_n / kStripN) * p.units_per_strip;
-  SONAR_REQUIRE(total_units * cus < (1LL << 31), "size_k * size_n = %ld x %ld is too large", (long)size_k,
-                (long)size_n);
-  p.total_units = (int)total_units;
-  p.parts = p.total_units < cus ? p.total_units : cus;
-  // Short strips (K <= 4096) on a matrix with at least 64 of them: one workgroup
-  // per strip.  No strip is shared, so no partial tile goes through memory and
-  // the fix-up launch is skipped; measured equal or faster than the even split
-  // (qkv 8.7 vs 10.4 us) although fewer compute units stream at a time.  No
-  // scratch slot is touched in this mode (slots are sized for `cus` workgroups).
-  const int64_t n_strips = size_n / kStripN;
-  if (p.units_per_strip <= 32 && n_strips >= 64 && total_units * n_strips < (1LL << 31)) p.parts = (int)n_strips;
-
-  bool any_split = false;
-  for (int i = 1; i < p.parts && !any_split; ++i)
-    any_split = range_begin(i, p.total_units, p.parts) % p.units_per_strip != 0;
 
   // groups of 128 * 2^s rows: group of a unit = unit >> s
   int unit_group_shift = -1;
@@ -924,6 +918,40 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
       while ((1 << unit_group_shift) < per) ++unit_group_shift;
     }
   }
+  static const bool no_fast = getenv("SONAR_MARLIN_NO_FAST") != nullptr;  // debugging aid
+  const bool fast_shape = !no_fast && !chk.has_perm && p.chunks_per_strip % 4 == 0 && fast_groups &&
+                          size_m * a_row_stride * 2 < (1LL << 31);
+  // Short strips (K <= 4096) on a matrix with at least 64 of them: one workgroup
+  // per strip.  No strip is shared, so no partial tile goes through memory and
+  // the fix-up launch is skipped; measured equal or faster than the even split
+  // (qkv 8.7 vs 10.4 us) although fewer compute units stream at a time.  No
+  // scratch slot is touched in this mode (slots are sized for `cus` workgroups).
+  const int64_t n_strips = size_n / kStripN;
+  const bool strip_per_workgroup = p.chunks_per_strip % 4 == 0 && p.chunks_per_strip / 4 <= 32 && n_strips >= 64 &&
+                                   (n_strips * (p.chunks_per_strip / 4)) * n_strips < (1LL << 31);
+  // 17 to 128 rows on such a matrix: the fast kernel once, with one workgroup
+  // per strip and block of 16 rows.  The blocks of a strip stream the same
+  // weights at the same time on compute units of one XCD, which would
+  // otherwise idle (a Llama-3-8B attention projection has 64 to 96 strips).
+  static const bool no_slabs = getenv("SONAR_MARLIN_NO_SLABS") != nullptr;  // debugging aid
+  const bool slab_fast = !no_slabs && fast_shape && strip_per_workgroup && size_m > 16 && size_m <= 128;
+
+  p.unit_chunks = p.chunks_per_strip % 4 == 0 ? 4 : (p.chunks_per_strip % 2 == 0 ? 2 : 1);
+  // the general kernel works on half units when it holds more than 32 rows (see unit_buffer_chunks)
+  if (size_m > 32 && p.unit_chunks == 4 && !slab_fast) p.unit_chunks = 2;
+  p.units_per_strip = p.chunks_per_strip / p.unit_chunks;
+  const int64_t total_units = n_strips * p.units_per_strip;
+  SONAR_REQUIRE(total_units * cus < (1LL << 31), "size_k * size_n = %ld x %ld is too large", (long)size_k,
+                (long)size_n);
+  p.total_units = (int)total_units;
+  p.parts = p.total_units < cus ? p.total_units : cus;
+  if (strip_per_workgroup && p.unit_chunks == 4) p.parts = (int)n_strips;
+  p.slabs = 1;
+  p.grid_parts = p.parts;
+
+  bool any_split = false;
+  for (int i = 1; i < p.parts && !any_split; ++i)
+    any_split = range_begin(i, p.total_units, p.parts) % p.units_per_strip != 0;
 
   static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
   const bool async_tile = tile_async_applies(chk.has_perm, num_groups, chk.group_size);
@@ -939,14 +967,18 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
     p.a = static_cast<const uint16_t*>(a) + m0 * a_row_stride;
     p.c = static_cast<uint16_t*>(c) + m0 * size_n;
     p.size_m = (int)(size_m - m0 < 64 ? size_m - m0 : 64);
-    static const bool no_fast = getenv("SONAR_MARLIN_NO_FAST") != nullptr;  // debugging aid
-    const bool fast = !no_fast && p.size_m <= 16 && !chk.has_perm && p.unit_chunks == 4 && fast_groups &&
-                      (long)p.size_m * a_row_stride * 2 < (1L << 31);
+    const bool fast = fast_shape && p.unit_chunks == 4 && (p.size_m <= 16 || slab_fast);
     if (fast) {
+      if (slab_fast) {  // every row in this one launch
+        p.size_m = (int)size_m;
+        p.slabs = (int)((size_m + 15) / 16);
+        p.grid_parts = (p.parts + 7) / 8 * 8;
+        m0 = size_m;
+      }
       int rc;
-      // more workgroups than compute units (one per strip): two small ones per compute unit
+      // more workgroups than compute units: two small ones per compute unit
       static const bool no_half = getenv("SONAR_MARLIN_NO_HALF_WG") != nullptr;  // debugging aid
-      const bool half = !no_half && p.parts > cus;
+      const bool half = !no_half && p.parts * p.slabs > cus;
       if (dtype == SONAR_DTYPE_F16)
         rc = chk.has_zp ? launch_fast<_Float16, true>(p, unit_group_shift, half, st)
                         : launch_fast<_Float16, false>(p, unit_group_shift, half, st);

@@ -106,6 +106,13 @@ GEMM_CASES = [
     (2, 4096, 6144, 128, False, False, False),
     (2, 14336, 6144, 128, False, False, False),      # more than four activation slices per wavefront
     (11, 4096, 512, 128, True, False, True),
+    # 17..128 rows on a matrix with at least 64 short strips: one launch of the
+    # 16-row kernel with a block of rows per workgroup
+    (33, 512, 4096, 128, False, False, True),
+    (100, 1024, 4224, 128, True, False, False),
+    (128, 256, 4096, -1, False, False, False),
+    (64, 4096, 6144, 128, False, False, False),
+    (17, 384, 8192, 128, True, False, True),
 ]
 
 
