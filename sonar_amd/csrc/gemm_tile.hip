@@ -27,6 +27,7 @@ constexpr int kTileM = 256;
 constexpr int kTileN = 256;
 constexpr int kTileK = 64;
 constexpr int kTileWaves = 8;
+constexpr int kTileBand = 4;                               // see tile_of_workgroup
 constexpr int kBlockBytes = 1024;                          // one operand block
 constexpr int kStageA = (kTileM / 16) * (kTileK / 32) * kBlockBytes;  // 32 KiB
 constexpr int kStageB = (kTileN / 16) * (kTileK / 32) * kBlockBytes;  // 32 KiB
@@ -85,8 +86,13 @@ __device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile
   const int id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   split = id / tiles;
   const int tile = id - split * tiles;
-  tile_n = tile / p.tiles_m;
-  tile_m = tile - tile_n * p.tiles_m;
+  // tiles are numbered band by band (kTileBand rows of tiles), inside a band
+  // column by column: 32 consecutive tiles are 4 panels of A x 8 panels of W
+  const int band = tile / (kTileBand * p.tiles_n);
+  const int rem = tile - band * kTileBand * p.tiles_n;
+  const int rows = min(kTileBand, p.tiles_m - band * kTileBand);
+  tile_n = rem / rows;
+  tile_m = band * kTileBand + rem - tile_n * rows;
   return id < total;
 }
 
