@@ -30,7 +30,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 # `bench.py --eager --calibrate`: FETCH_SIZE scaled by 2.000 and WRITE_SIZE by
 # 1.000, the factors that make the `--calibrate` pass (256 MiB read, 256 MiB
 # written) come out right.  Average over the four GEMMs of the layer at M = 16.
-MEASURED_TRAFFIC_M16 = 30_090_000
+MEASURED_TRAFFIC_M16 = 30_100_000
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 GROUP = 128
 LAYER_SHAPES = [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
@@ -339,6 +339,17 @@ def main() -> int:
                                   "TFLOPs": round(fl / s / 1e12, 2),
                                   "frac_hbm": round(nb / s / 1e9 / HBM_PEAK_GBPS, 4),
                                   "frac_mfma": round(fl / s / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+                    if regime == "prefill" and mm >= 4096:
+                        # yardstick: the vendor library's dense 16-bit GEMM on the same activations
+                        # and a dense matrix of the same shape (what the box sustains on this much
+                        # matrix work with real data; not part of the product path)
+                        w_dense = torch.randn((k, n), device="cuda:0", generator=gen).to(dt) * 0.05
+
+                        def dense(i=0, a=a, w_dense=w_dense):
+                            torch.matmul(a, w_dense)
+                        sd = time_graph(torch, dense, reps)
+                        sweep[-1]["dense_matmul_TFLOPs"] = round(fl / sd / 1e12, 2)
+                        del w_dense
                     print("sweep", json.dumps(sweep[-1]), file=sys.stderr, flush=True)
         out["sweep"] = sweep
         out["variants"] = variants_sweep(torch, ops, gen, time_graph)

@@ -27,7 +27,6 @@ constexpr int kTileM = 256;
 constexpr int kTileN = 256;
 constexpr int kTileK = 64;
 constexpr int kTileWaves = 8;
-constexpr int kTileBand = 4;                               // see tile_of_workgroup
 constexpr int kBlockBytes = 1024;                          // one operand block
 constexpr int kStageA = (kTileM / 16) * (kTileK / 32) * kBlockBytes;  // 32 KiB
 constexpr int kStageB = (kTileN / 16) * (kTileK / 32) * kBlockBytes;  // 32 KiB
@@ -47,6 +46,7 @@ struct TileParams {
   int num_groups, group_size;
   int chunks_per_strip;
   int tiles_m, tiles_n;
+  int tile_band;               // rows of tiles per band of the tile numbering (tile_of_workgroup)
   // split K: workgroup (tile, split) covers K steps [split * k_steps_per_split, ...) and, when
   // k_splits > 1, leaves its fp32 tile in `partial` for tile_reduce_kernel
   int k_splits, k_steps_per_split;
@@ -86,13 +86,14 @@ __device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile
   const int id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
   split = id / tiles;
   const int tile = id - split * tiles;
-  // tiles are numbered band by band (kTileBand rows of tiles), inside a band
-  // column by column: 32 consecutive tiles are 4 panels of A x 8 panels of W
-  const int band = tile / (kTileBand * p.tiles_n);
-  const int rem = tile - band * kTileBand * p.tiles_n;
-  const int rows = min(kTileBand, p.tiles_m - band * kTileBand);
+  // tiles are numbered band by band (tile_band rows of tiles), inside a band
+  // column by column: with bands of 4 rows, 32 consecutive tiles are 4 panels
+  // of A x 8 panels of W
+  const int band = tile / (p.tile_band * p.tiles_n);
+  const int rem = tile - band * p.tile_band * p.tiles_n;
+  const int rows = min(p.tile_band, p.tiles_m - band * p.tile_band);
   tile_n = rem / rows;
-  tile_m = band * kTileBand + rem - tile_n * rows;
+  tile_m = band * p.tile_band + rem - tile_n * rows;
   return id < total;
 }
 
@@ -723,6 +724,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   p.group_size = group_size;
   p.chunks_per_strip = (int)(size_k / kChunkK);
   p.tiles_m = (int)((size_m + kTileM - 1) / kTileM);
+  p.tile_band = 4;
   p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);
   p.k_splits = 1;
   p.k_steps_per_split = (int)(size_k / kTileK);
@@ -804,6 +806,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.group_size = group_size;
   p.chunks_per_strip = (int)(size_k / kChunkK);
   p.tiles_m = max_tiles;
+  p.tile_band = max_tiles > 0 ? max_tiles : 1;  // row tiles of different experts share no panel of W: whole columns
   p.k_splits = 1;
   p.k_steps_per_split = (int)(size_k / kTileK);
   p.partial = nullptr;
