@@ -142,9 +142,12 @@ __device__ __forceinline__ void finish_segment(const StreamParams& p, int strip,
 }
 
 // The same for one 16-column block (j) of a 16-row tile, held by one wavefront.
+// `part` is the workgroup's index in the partition and `slab` its block of 16
+// rows (fast kernel: several blocks of rows share one launch; the scratch slot
+// of a part holds one partial tile per block of rows).
 template <typename T>
-__device__ __forceinline__ void finish_block(const StreamParams& p, int strip, int seg_begin, int seg_end,
-                                             int lane, int j, floatx4_t v) {
+__device__ __forceinline__ void finish_block(const StreamParams& p, int part, int slab, int strip, int seg_begin,
+                                             int seg_end, int lane, int j, floatx4_t v) {
   const int strip_first = strip * p.units_per_strip;
   const int strip_end = strip_first + p.units_per_strip;
   if (seg_begin == strip_first && seg_end == strip_end) {
@@ -165,7 +168,7 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, int strip, i
     return;
   }
   const int first = range_owner(strip_first, p.total_units, p.parts);
-  partial_slot(p, blockIdx.x, first)[j * 64 + lane] = make_float4(v.x, v.y, v.z, v.w);
+  partial_slot(p, part, first)[(slab * 4 + j) * 64 + lane] = make_float4(v.x, v.y, v.z, v.w);
 }
 
 // ---------------------------------------------------------------------------
@@ -561,7 +564,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
           sum += t2;
           sum += t3;
         }
-        finish_block<T>(p, strip, seg_begin, seg_end, lane, wave, sum);
+        finish_block<T>(p, part, slab, strip, seg_begin, seg_end, lane, wave, sum);
       }
       seg_begin = seg_end;
       ++seg_strip;
@@ -934,7 +937,10 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   // weights at the same time on compute units of one XCD, which would
   // otherwise idle (a Llama-3-8B attention projection has 64 to 96 strips).
   static const bool no_slabs = getenv("SONAR_MARLIN_NO_SLABS") != nullptr;  // debugging aid
-  const bool slab_fast = !no_slabs && fast_shape && strip_per_workgroup && size_m > 16 && size_m <= 128;
+  // Up to 64 rows this also pays on matrices whose strips are shared between
+  // workgroups (a scratch slot has room for four blocks of rows).
+  const bool slab_fast = !no_slabs && fast_shape && size_m > 16 &&
+                         (size_m <= 64 || (strip_per_workgroup && size_m <= 128));
 
   p.unit_chunks = p.chunks_per_strip % 4 == 0 ? 4 : (p.chunks_per_strip % 2 == 0 ? 2 : 1);
   // the general kernel works on half units when it holds more than 32 rows (see unit_buffer_chunks)

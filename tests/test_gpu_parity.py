@@ -113,6 +113,10 @@ GEMM_CASES = [
     (128, 256, 4096, -1, False, False, False),
     (64, 4096, 6144, 128, False, False, False),
     (17, 384, 8192, 128, True, False, True),
+    # the same with strips shared between workgroups (partial tiles per block of rows)
+    (33, 14336, 1024, 128, False, False, True),
+    (64, 2048, 512, 128, True, False, False),
+    (40, 4096, 640, -1, False, False, False),
 ]
 
 
