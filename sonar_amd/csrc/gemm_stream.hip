@@ -56,6 +56,10 @@ struct StreamParams {
   // slab * grid_parts + part works on rows 16 slab.. of part `part` (ids past
   // `parts` inside a slab are padding)
   int slabs, grid_parts;
+  // fast kernel only: the tiles of the cross-wavefront sum are parked on top of
+  // the copy rings instead of behind them.  Allowed when every workgroup owns
+  // whole strips: it then sums once, after its last copy has been consumed.
+  int sum_over_rings;
 };
 
 // Unit indices are 32-bit: the host checks total_units * parts < 2^31.
@@ -452,7 +456,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   const int col16 = lane & 15;
   char* ring = smem + wave * kWaveLds;
   const uint32_t ring_lds = (uint32_t)(uintptr_t)(lds_void_t*)ring;
-  const uint32_t red_lds = (uint32_t)(uintptr_t)(lds_void_t*)(smem + kFastWaves * kWaveLds);
+  const uint32_t red_lds = (uint32_t)(uintptr_t)(lds_void_t*)(smem + (p.sum_over_rings ? 0 : kFastWaves * kWaveLds));
 
   const int u_begin = range_begin(part, p.total_units, p.parts);
   const int u_end = range_begin(part + 1, p.total_units, p.parts);
@@ -769,8 +773,8 @@ int launch_fast_waves(const StreamParams& p, int unit_group_shift, hipStream_t s
                                   hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds_bytes(WAVES)));
     attr_set = true;
   }
-  marlin_stream_fast_kernel<T, HAS_ZP, WAVES>
-      <<<p.grid_parts * p.slabs, WAVES * 64, fast_lds_bytes(WAVES), st>>>(p, unit_group_shift);
+  const int lds = p.sum_over_rings ? WAVES * kWaveLds : fast_lds_bytes(WAVES);
+  marlin_stream_fast_kernel<T, HAS_ZP, WAVES><<<p.grid_parts * p.slabs, WAVES * 64, lds, st>>>(p, unit_group_shift);
   return SONAR_OK;
 }
 
@@ -954,6 +958,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   if (strip_per_workgroup && p.unit_chunks == 4) p.parts = (int)n_strips;
   p.slabs = 1;
   p.grid_parts = p.parts;
+  p.sum_over_rings = 0;
 
   bool any_split = false;
   for (int i = 1; i < p.parts && !any_split; ++i)
@@ -982,9 +987,11 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
         m0 = size_m;
       }
       int rc;
-      // more workgroups than compute units: two small ones per compute unit
+      // more workgroups than compute units: small ones, two per compute unit, or three
+      // when they need no LDS of their own for the sum
       static const bool no_half = getenv("SONAR_MARLIN_NO_HALF_WG") != nullptr;  // debugging aid
       const bool half = !no_half && p.parts * p.slabs > cus;
+      p.sum_over_rings = half && (int64_t)p.parts == n_strips && p.parts * p.slabs > 2 * cus;
       if (dtype == SONAR_DTYPE_F16)
         rc = chk.has_zp ? launch_fast<_Float16, true>(p, unit_group_shift, half, st)
                         : launch_fast<_Float16, false>(p, unit_group_shift, half, st);
