@@ -137,8 +137,8 @@ def test_marlin_gemm_within_tolerance(gu, dtype, m, k, n, g, zp, act, bias):
     assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
 
 
-def test_gemm_row_strided_activations(gu):
-    m, k, n = 9, 512, 256
+@pytest.mark.parametrize("m,k,n", [(9, 512, 256), (37, 512, 4096), (50, 1024, 256), (300, 512, 512)])
+def test_gemm_row_strided_activations(gu, m, k, n):
     layer = gu.DeviceLayer(3, k, n, 128, "fp16")
     big32 = mo.make_activations(5, m, k + 64, "fp16")
     big = gu.dev_bits16(big32, "fp16")
