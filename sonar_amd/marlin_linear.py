@@ -7,7 +7,8 @@ its config (MPLinearKernel.py:26-90), with plain tensors in a namespace-like
 Checkpoint layouts taken (as the reference's GPTQ path provides them,
 layers/quantization/auto_gptq.py:304-430): qweight (K/8, N) int32 packed along
 K, scales (K/G, N), qzeros (N/8-packed per group, given here already unpacked
-to (K/G, N) codes or packed (K/G, N/8) along N), g_idx (K) int32."""
+to (K/G, N) codes, packed (K/G, N/8) along N, or that transposed), g_idx (K)
+int32.  AutoAWQ checkpoints go through convert_awq_to_standard_format first."""
 from __future__ import annotations
 
 from dataclasses import dataclass
@@ -22,6 +23,34 @@ from .marlin_utils import (MARLIN_SUPPORTED_GROUP_SIZES, apply_gptq_marlin_linea
                            marlin_permute_scales, marlin_sort_g_idx, marlin_zero_points,
                            query_marlin_supported_quant_types, unpack_cols)
 from .scalar_type import ScalarType
+
+
+_AWQ_SLOT_OF_COLUMN = (0, 4, 1, 5, 2, 6, 3, 7)   # nibble slot of column j of an AWQ-packed int32
+
+
+def convert_awq_to_standard_format(layer, w_q_name: str = "qweight", w_zp_name: str = "qzeros",
+                                   size_bits: int = 4) -> None:
+    """AutoAWQ checkpoint tensors -> the GPTQ-like ones MarlinLinearKernel takes
+    (the reference's `_convert_awq_to_standard_format`,
+    layers/quantization/auto_awq.py:93-153): qweight (K, N/8), packed along N
+    with AWQ's interleaved nibble order, becomes (K/8, N) packed along K in
+    plain order; qzeros (G, N/8) in the same AWQ packing becomes (N/8, G),
+    packed along N in plain order and transposed."""
+    if size_bits != 4:
+        raise NotImplementedError("AWQ conversion: 4-bit only")
+    qw = getattr(layer, w_q_name)
+    shifts = 4 * torch.tensor(_AWQ_SLOT_OF_COLUMN, dtype=torch.int32, device=qw.device)
+    plain = 4 * torch.arange(8, dtype=torch.int32, device=qw.device)
+
+    def codes(packed: torch.Tensor) -> torch.Tensor:       # (R, N/8) -> (R, N), column order restored
+        return ((packed.unsqueeze(-1) >> shifts) & 0xF).reshape(packed.shape[0], -1)
+
+    def pack_dim0(q: torch.Tensor) -> torch.Tensor:        # (8 R, C) -> (R, C): row 8 r + t in nibble t
+        q = q.reshape(q.shape[0] // 8, 8, q.shape[1]).to(torch.int32)
+        return (q << plain[None, :, None]).sum(dim=1, dtype=torch.int32).contiguous()
+
+    setattr(layer, w_q_name, pack_dim0(codes(qw)))
+    setattr(layer, w_zp_name, pack_dim0(codes(getattr(layer, w_zp_name)).t().contiguous()))
 
 
 @dataclass
@@ -92,6 +121,8 @@ class MarlinLinearKernel:
             grouped_k = size_k // c.group_size if c.group_size != -1 else 1
             padded_grouped_k = padded_k // c.group_size if c.group_size != -1 else 1
             zp = getattr(layer, self.w_zp_name)
+            if zp.shape == (size_n // 8, grouped_k) and grouped_k != size_n // 8:
+                zp = zp.t().contiguous()      # packed along N and transposed (the converted AWQ form)
             if zp.shape == (grouped_k, size_n // 8):
                 zp = unpack_cols(zp, c.weight_type.size_bits, grouped_k, size_n)
             zp = marlin_pad_scales(zp, size_n, size_k, padded_n, padded_k, c.group_size)

@@ -152,6 +152,29 @@ def test_marlin_linear_kernel_round_trip(cfg):
     assert ok, worst
 
 
+@pytest.mark.parametrize("k,n,g,dtype,rows", [(512, 256, 128, "fp16", 5), (1024, 4096, 128, "bf16", 40)])
+def test_awq_checkpoint_through_the_linear_kernel(k, n, g, dtype, rows):
+    """AutoAWQ tensors -> convert_awq_to_standard_format -> MarlinLinearKernel
+    (auto_awq.py:93-153 feeding kernels/linear/mixed_precision/marlin.py)."""
+    from sonar_amd.marlin_linear import (MarlinLinearKernel, MPLinearLayerConfig,
+                                         convert_awq_to_standard_format)
+    from sonar_amd.scalar_type import scalar_types
+    layer_np = mo.make_layer(19, k, n, g, dtype, zero_points=True)
+    w_ref = mo.dequantize(layer_np["q"], layer_np["scales"], g, dtype, zeros=layer_np["zeros"])
+    layer = types.SimpleNamespace(bias=None)
+    layer.qweight = gu.dev_i32(mo.awq_pack(layer_np["q"]))
+    layer.qzeros = gu.dev_i32(mo.awq_pack(layer_np["zeros"].astype(np.int32)))
+    layer.scales = gu.dev_bits16(layer_np["scales"], dtype)
+    convert_awq_to_standard_format(layer)
+    kern = MarlinLinearKernel(MPLinearLayerConfig((k, n), (k, n), scalar_types.uint4, _tdt(dtype), g, True, False),
+                              w_gidx_param_name=None)
+    kern.process_weights_after_loading(layer)
+    x32 = mo.make_activations(3, rows, k, dtype)
+    y = kern.apply_weights(layer, gu.dev_bits16(x32, dtype), None)
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y), mo.gemm_reference(x32, w_ref))
+    assert ok, worst
+
+
 def _moe_layer(seed, e, hidden, inter, g, dtype, zp):
     """Expert weights in the layouts fused_marlin_moe takes, plus dequantised references."""
     from sonar_amd import marlin_utils as mu

@@ -252,3 +252,24 @@ def test_kernels_with_hand_counted_waits_do_not_spill():
                 seen += 1
                 assert int(m.group(1)) == 0, f"{name} spills {m.group(1)} VGPRs"
         assert seen >= 4, f"no resource report for {kernel}"
+
+
+def test_awq_checkpoint_conversion_matches_gptq_packing():
+    """AutoAWQ tensors through convert_awq_to_standard_format give what packing the
+    same codes the GPTQ way gives (layers/quantization/auto_awq.py:93-153)."""
+    import types
+    from sonar_amd.marlin_linear import convert_awq_to_standard_format
+    rng = np.random.default_rng(12)
+    k, n, g = 256, 192, 64
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    zp = rng.integers(0, 16, size=(k // g, n), dtype=np.int32)
+    q[:, :8] = 15       # top nibble of a word set: sign handling
+    zp[:, -8:] = 15
+    layer = types.SimpleNamespace(qweight=torch.from_numpy(mo.awq_pack(q)), qzeros=torch.from_numpy(mo.awq_pack(zp)))
+    convert_awq_to_standard_format(layer)
+    assert layer.qweight.dtype == torch.int32 and layer.qweight.shape == (k // 8, n)
+    assert np.array_equal(layer.qweight.numpy(), mo.pack_rows(q))
+    assert layer.qzeros.shape == (n // 8, k // g)
+    assert np.array_equal(layer.qzeros.numpy(), mo.pack_rows(np.ascontiguousarray(zp.T)))
+    # and the converted zero points unpack to the codes again (pack_cols form, transposed)
+    assert np.array_equal(mo.unpack_cols(np.ascontiguousarray(layer.qzeros.numpy().T)), zp)
