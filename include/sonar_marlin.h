@@ -100,8 +100,11 @@ size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n, int64_t s
  *                (required iff b_type_id == SONAR_TYPE_UINT4)
  *   g_idx, perm  int32[K] each or both NULL; with both given the call is an
  *                act-order call: perm maps weight row k to column perm[k] of
- *                A; g_idx[k] is the group of weight row k (used only when
- *                is_k_full == 0)
+ *                A; g_idx[k] is the group of weight row k, read only when
+ *                is_k_full == 0 (a shard that does not hold whole groups:
+ *                b_scales then has every group of the unsharded matrix,
+ *                num_groups need not divide K, b_zeros must be NULL, and the
+ *                size_m * size_k * 2 extra scratch bytes below are required)
  *   workspace    int32[workspace_len], all zero on entry, all zero on exit;
  *                workspace_len >= number of compute units
  *   scratch      sonar_marlin_gemm_scratch_bytes() bytes, contents don't care;

@@ -164,4 +164,32 @@ __device__ __forceinline__ void load_cols(typename Dq<T>::Col (&cols)[4], const 
   }
 }
 
+// One packed word whose eight rows (8 consecutive k) may lie in different groups:
+// a shard of an act-order matrix that does not hold whole groups.  `groups`
+// holds the group of each row, `scale_col` points at this column's scale of
+// group 0, `group_stride` is the distance between groups in elements.  The
+// exact integers v - 8 times the scale of the row's group, rounded once, as
+// the reference's dequantise-then-scale (products of two 16-bit floats are
+// exact in fp32, so rounding the fp32 product is the 16-bit multiply).
+template <typename T>
+__device__ __forceinline__ typename Dq<T>::vec8 word_by_row_groups(uint32_t q, const int (&groups)[8],
+                                                                  const uint16_t* scale_col, long group_stride,
+                                                                  uint32_t magic) {
+  typedef typename Dq<T>::vec8 vec8;
+  const typename Dq<T>::Col unit = Dq<T>::make_col(Dq<T>::from_float(1.0f), 8);
+  const vec8 w0 = Dq<T>::word(q, unit, magic);
+  const u32x4_t in = __builtin_bit_cast(u32x4_t, w0);
+  const uint32_t regs[4] = {in.x, in.y, in.z, in.w};
+  uint32_t out[4];
+#pragma unroll
+  for (int r = 0; r < 4; ++r) {
+    const float lo = Dq<T>::to_float((uint16_t)(regs[r] & 0xffffu)) *
+                     Dq<T>::to_float(scale_col[(long)groups[2 * r] * group_stride]);
+    const float hi = Dq<T>::to_float((uint16_t)(regs[r] >> 16)) *
+                     Dq<T>::to_float(scale_col[(long)groups[2 * r + 1] * group_stride]);
+    out[r] = (uint32_t)Dq<T>::from_float(lo) | ((uint32_t)Dq<T>::from_float(hi) << 16);
+  }
+  return __builtin_bit_cast(vec8, u32x4_t{out[0], out[1], out[2], out[3]});
+}
+
 }  // namespace sonar

@@ -44,6 +44,7 @@ struct StreamParams {
   const uint16_t* scales;
   const uint32_t* zeros;
   const int32_t* perm;
+  const int32_t* g_idx;  // group of every row of W; null when groups are runs of group_size rows
   float4* scratch;
   int size_m, size_n, size_k;
   int num_groups, group_size;
@@ -220,7 +221,7 @@ __device__ __forceinline__ void load_unit(UnitBuf<T, MB>& b, const StreamParams&
   if (HAS_ZP) b.zword = p.zeros[(long)g * (p.size_n / 8) + strip * 8 + zero_point_word(col16)];
 }
 
-template <typename T, int MB, bool HAS_ZP, bool HAS_PERM>
+template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX>
 __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const StreamParams p) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq<T>::Col Col;
@@ -272,9 +273,22 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
             load_cols<T, HAS_ZP>(cols, p.scales, p.zeros, p.size_n, strip, g, col16, grouped);
           }
           const uint32_t words[4] = {cur.q[cc].x, cur.q[cc].y, cur.q[cc].z, cur.q[cc].w};
+          int row_groups[8];
+          if (HAS_GIDX) {  // the lane's eight rows of this chunk: k = 32 chunk + 8 (lane / 16) + t
+            const int4* gsrc = reinterpret_cast<const int4*>(p.g_idx + (chunk0 + cc) * kChunkK + 8 * (lane >> 4));
+            const int4 g0 = gsrc[0], g1 = gsrc[1];
+            row_groups[0] = g0.x, row_groups[1] = g0.y, row_groups[2] = g0.z, row_groups[3] = g0.w;
+            row_groups[4] = g1.x, row_groups[5] = g1.y, row_groups[6] = g1.z, row_groups[7] = g1.w;
+          }
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const vec8 w = Dq<T>::word(words[j], cols[j], magic);
+            vec8 w;
+            if (HAS_GIDX)
+              w = word_by_row_groups<T>(words[j], row_groups,
+                                        p.scales + strip * kStripN + scale_slot(16 * j + col16, true), p.size_n,
+                                        magic);
+            else
+              w = Dq<T>::word(words[j], cols[j], magic);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) acc[mb][j] = Dq<T>::mfma(w, cur.a[cc][mb], acc[mb][j]);
           }
@@ -676,10 +690,12 @@ __global__ __launch_bounds__(64) void marlin_fixup_kernel(const StreamParams p) 
 }
 
 // Writes W[K][N]: the values the GEMM kernels feed to the matrix cores.
+// With g_idx (symmetric weights only) the group of every row is looked up there.
 template <typename T, bool HAS_ZP>
 __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __restrict__ b,
                                                             const uint16_t* __restrict__ scales,
                                                             const uint32_t* __restrict__ zeros,
+                                                            const int32_t* __restrict__ g_idx,
                                                             uint16_t* __restrict__ w_out, int size_n,
                                                             int size_k, int num_groups, int group_size,
                                                             long total_chunks) {
@@ -693,14 +709,24 @@ __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __rest
   for (long ch = (long)blockIdx.x * 4 + (threadIdx.x >> 6); ch < total_chunks; ch += (long)gridDim.x * 4) {
     const int strip = (int)(ch / chunks_per_strip);
     const int chunk = (int)(ch % chunks_per_strip);
-    const int g = grouped ? (chunk * kChunkK) / group_size : 0;
+    const int g = grouped && !g_idx ? (chunk * kChunkK) / group_size : 0;
     typename Dq<T>::Col cols[4];
     load_cols<T, HAS_ZP>(cols, scales, zeros, size_n, strip, g, col16, grouped);
+    int row_groups[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+    if (g_idx) {
+#pragma unroll
+      for (int t = 0; t < 8; ++t) row_groups[t] = g_idx[chunk * kChunkK + 8 * kb + t];
+    }
     const uint4 q = b[ch * 64 + lane];
     const uint32_t words[4] = {q.x, q.y, q.z, q.w};
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const vec8 w = Dq<T>::word(words[j], cols[j], magic);
+      vec8 w;
+      if (!HAS_ZP && g_idx)
+        w = word_by_row_groups<T>(words[j], row_groups, scales + strip * kStripN + scale_slot(16 * j + col16, true),
+                                  size_n, magic);
+      else
+        w = Dq<T>::word(words[j], cols[j], magic);
       const uint16_t* bits = reinterpret_cast<const uint16_t*>(&w);
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
@@ -749,10 +775,13 @@ __global__ __launch_bounds__(256) void permute_columns_kernel(const uint16_t* __
 
 template <typename T, int MB, bool HAS_ZP>
 void launch_stream(const StreamParams& p, bool has_perm, hipStream_t st) {
-  if (has_perm)
-    marlin_stream_kernel<T, MB, HAS_ZP, true><<<p.parts, kWaves * 64, 0, st>>>(p);
-  else
-    marlin_stream_kernel<T, MB, HAS_ZP, false><<<p.parts, kWaves * 64, 0, st>>>(p);
+  if (p.g_idx) {  // row -> group lookup: symmetric weights, activations already permuted
+    if constexpr (!HAS_ZP) marlin_stream_kernel<T, MB, false, false, true><<<p.parts, kWaves * 64, 0, st>>>(p);
+  } else if (has_perm) {
+    marlin_stream_kernel<T, MB, HAS_ZP, true, false><<<p.parts, kWaves * 64, 0, st>>>(p);
+  } else {
+    marlin_stream_kernel<T, MB, HAS_ZP, false, false><<<p.parts, kWaves * 64, 0, st>>>(p);
+  }
 }
 
 template <typename T, bool HAS_ZP>
@@ -798,6 +827,7 @@ void launch_fixup(const StreamParams& p, hipStream_t st) {
 struct Checked {
   bool has_zp;
   bool has_perm;
+  bool row_groups;  // act-order shard without whole groups: the group of a row comes from g_idx
   int group_size;
 };
 
@@ -824,12 +854,14 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
                   "b_type must be uint4b8 when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   out.has_perm = perm != nullptr;
-  if (out.has_perm) {
-    if (!is_k_full)
-      return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False is not built yet");
-    SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
-  }
-  if (num_groups > 1) {
+  out.row_groups = out.has_perm && !is_k_full;
+  if (out.has_perm) SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
+  if (out.row_groups) {
+    // marlin.cu:343-351,763-769: group_size = 0, every row looks its group up
+    if (out.has_zp)
+      return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False and zero points is not built");
+    out.group_size = 0;
+  } else if (num_groups > 1) {
     SONAR_REQUIRE(size_k % num_groups == 0, "size_k = %ld, is not divisible by num_groups = %ld",
                   (long)size_k, (long)num_groups);
     out.group_size = (int)(size_k / num_groups);
@@ -899,6 +931,10 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
     perm = nullptr;
     chk.has_perm = false;
   }
+  if (chk.row_groups && chk.has_perm)
+    return fail(SONAR_E_INVALID,
+                "act-order with is_k_full = False needs size_m * size_k * 2 more scratch bytes "
+                "(the column-permuted copy of A)");
 
   StreamParams p;
   p.b = reinterpret_cast<const uint4*>(b_q_weight);
@@ -906,18 +942,19 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   p.scales = static_cast<const uint16_t*>(b_scales);
   p.zeros = b_zeros;
   p.perm = perm;
+  p.g_idx = chk.row_groups ? g_idx : nullptr;
   p.scratch = static_cast<float4*>(scratch);
   p.size_n = (int)size_n;
   p.size_k = (int)size_k;
   p.lda = a_row_stride;
   p.num_groups = (int)num_groups;
-  p.group_size = chk.group_size;
+  p.group_size = chk.row_groups ? (int)size_k : chk.group_size;  // the kernels' own group arithmetic is unused then
   p.chunks_per_strip = (int)(size_k / kChunkK);
 
   // groups of 128 * 2^s rows: group of a unit = unit >> s
   int unit_group_shift = -1;
   bool fast_groups = num_groups == 1;
-  if (num_groups > 1 && chk.group_size % 128 == 0) {
+  if (num_groups > 1 && chk.group_size > 0 && chk.group_size % 128 == 0) {
     const int per = chk.group_size / 128;
     if ((per & (per - 1)) == 0) {
       fast_groups = true;
@@ -926,7 +963,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
     }
   }
   static const bool no_fast = getenv("SONAR_MARLIN_NO_FAST") != nullptr;  // debugging aid
-  const bool fast_shape = !no_fast && !chk.has_perm && p.chunks_per_strip % 4 == 0 && fast_groups &&
+  const bool fast_shape = !no_fast && !chk.has_perm && !chk.row_groups && p.chunks_per_strip % 4 == 0 && fast_groups &&
                           size_m * a_row_stride * 2 < (1LL << 31);
   // Short strips (K <= 4096) on a matrix with at least 64 of them: one workgroup
   // per strip.  No strip is shared, so no partial tile goes through memory and
@@ -967,7 +1004,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
   const bool async_tile = tile_async_applies(chk.has_perm, num_groups, chk.group_size);
   const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
-  if (plan.tile && !no_tile) {
+  if (plan.tile && !no_tile && !chk.row_groups) {  // the row -> group lookup exists in the streaming kernel only
     const size_t used = stream_scratch_bytes();
     return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
                      size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used,
@@ -1033,12 +1070,13 @@ extern "C" int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout, co
   const uint16_t* s = static_cast<const uint16_t*>(b_scales);
   uint16_t* w = static_cast<uint16_t*>(w_out);
   const int ng = (int)num_groups, gs = chk.group_size, n = (int)size_n, k = (int)size_k;
+  const int32_t* gi = chk.row_groups ? g_idx : nullptr;
   if (dtype == SONAR_DTYPE_F16) {
-    if (chk.has_zp) marlin_dequant_kernel<_Float16, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, w, n, k, ng, gs, total_chunks);
-    else marlin_dequant_kernel<_Float16, false><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, w, n, k, ng, gs, total_chunks);
+    if (chk.has_zp) marlin_dequant_kernel<_Float16, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);
+    else marlin_dequant_kernel<_Float16, false><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);
   } else {
-    if (chk.has_zp) marlin_dequant_kernel<__bf16, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, w, n, k, ng, gs, total_chunks);
-    else marlin_dequant_kernel<__bf16, false><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, w, n, k, ng, gs, total_chunks);
+    if (chk.has_zp) marlin_dequant_kernel<__bf16, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);
+    else marlin_dequant_kernel<__bf16, false><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);
   }
   return launch_status("marlin_dequant_kernel");
 }

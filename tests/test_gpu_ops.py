@@ -175,6 +175,32 @@ def test_awq_checkpoint_through_the_linear_kernel(k, n, g, dtype, rows):
     assert ok, worst
 
 
+@pytest.mark.parametrize("dtype,rows", [("fp16", 3), ("bf16", 70)])
+def test_linear_kernel_row_parallel_act_order_shard(dtype, rows):
+    """A row-parallel rank's slice of an act-order layer: is_k_full = False, the
+    scales of every group on every rank (marlin_utils.py: marlin_is_k_full,
+    marlin_repeat_scales_on_all_ranks; marlin.py:88-235)."""
+    from sonar_amd.marlin_linear import MarlinLinearKernel, MPLinearLayerConfig
+    from sonar_amd.scalar_type import scalar_types
+    k_full, n, g = 1024, 256, 128
+    full = mo.make_layer(23, k_full, n, g, dtype, act_order=True)
+    lo, hi = 512, 1024                       # rank 1 of 2
+    k = hi - lo
+    w_ref = mo.dequantize(full["q"][lo:hi], full["scales"], g, dtype, g_idx=full["g_idx"][lo:hi])
+    layer = types.SimpleNamespace(bias=None)
+    layer.qweight = gu.dev_i32(mo.gptq_pack(full["q"][lo:hi]))
+    layer.scales = gu.dev_bits16(full["scales"], dtype)
+    layer.g_idx = gu.dev_i32(full["g_idx"][lo:hi])
+    kern = MarlinLinearKernel(MPLinearLayerConfig((k_full, n), (k, n), scalar_types.uint4b8, _tdt(dtype), g, False,
+                                                  True), w_zp_param_name=None)
+    kern.process_weights_after_loading(layer)
+    assert kern.is_k_full is False
+    x32 = mo.make_activations(6, rows, k, dtype)
+    y = kern.apply_weights(layer, gu.dev_bits16(x32, dtype), None)
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y), mo.gemm_reference(x32, w_ref))
+    assert ok, worst
+
+
 def _moe_layer(seed, e, hidden, inter, g, dtype, zp):
     """Expert weights in the layouts fused_marlin_moe takes, plus dequantised references."""
     from sonar_amd import marlin_utils as mu

@@ -235,6 +235,57 @@ def test_act_order_with_permuted_copy_of_a(gu, dtype, m, k, n):
     assert ok, f"max_err={max_err} max_ref={max_ref}"
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("m", [1, 16, 40, 100, 300])
+def test_act_order_shard_without_whole_groups(gu, dtype, m):
+    """A row-parallel shard of an act-order matrix (is_k_full = False,
+    marlin.cu:343-351,763-769): the shard's rows lie in all groups, no group is
+    whole, every row finds its scale through g_idx.  Dequantised values bit
+    for bit, GEMM within the tolerance."""
+    from sonar_amd import _lib
+    k_full, n, g = 1024, 320, 128
+    full = mo.make_layer(91, k_full, n, g, dtype, act_order=True)
+    lo, hi = 256, 768
+    k = hi - lo
+    q, g_idx, scales = full["q"][lo:hi], full["g_idx"][lo:hi], full["scales"]
+    assert len(np.unique(g_idx)) == k_full // g and np.bincount(g_idx).max() < g
+    w_ref = mo.dequantize(q, scales, g, dtype, g_idx=g_idx)
+    g_sorted, order = mo.stable_sort_g_idx(g_idx)
+    perm, g_dev = gu.dev_i32(order), gu.dev_i32(g_sorted)
+    native = gu.to_gfx950(gu.gptq_repack(gu.dev_i32(mo.gptq_pack(q)), perm, k, n), k, n)
+    s_dev = gu.dev_bits16(mo.marlin_permute_scales(scales, k_full, n, g), dtype)
+    lib = _lib.load()
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+
+    w = torch.empty((k, n), dtype=tdt, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_dequant(gu.ptr(native), _lib.LAYOUT_GFX950, gu.ptr(s_dev), None, gu.ptr(g_dev),
+                                        gu.ptr(w), gu.dtype_code(dtype), _lib.TYPE_UINT4B8, n, k, k_full // g, 0,
+                                        gu.stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(gu.host_f32(w), w_ref[order])      # weight rows are in sorted-group order
+
+    a32 = mo.make_activations(m, m, k, dtype, std=0.5)
+    a = gu.dev_bits16(a32, dtype)
+    c = torch.empty((m, n), dtype=tdt, device=gu.DEV)
+    workspace = torch.zeros(torch.cuda.get_device_properties(0).multi_processor_count, dtype=torch.int32,
+                            device=gu.DEV)
+    base = lib.sonar_marlin_gemm_scratch_bytes(m, n, k)
+
+    def call(scratch_bytes):
+        scratch = torch.empty(scratch_bytes, dtype=torch.uint8, device=gu.DEV)
+        return lib.sonar_marlin_gemm(
+            gu.ptr(a), k, gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None, gu.ptr(s_dev), None, gu.ptr(g_dev),
+            gu.ptr(perm), gu.ptr(workspace), workspace.numel(), gu.ptr(scratch), scratch.numel(),
+            gu.dtype_code(dtype), _lib.TYPE_UINT4B8, m, n, k, k_full // g, 0, 0, 1, gu.stream())
+
+    _lib.check(call(base + m * k * 2))
+    torch.cuda.synchronize()
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), mo.gemm_reference(a32, w_ref))
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+    # without room for the permuted copy of A the call is refused, not mis-computed
+    assert call(base) != 0 and b"more scratch" in lib.sonar_marlin_last_error()
+
+
 @pytest.mark.parametrize("dtype,m,k,n", [("fp16", 4096, 4096, 4096), ("bf16", 8192, 4096, 6144),
                                           ("fp16", 1024, 14336, 4096), ("fp16", 256, 4096, 28672)])
 def test_full_size_tile_gemm_agrees_with_streamed_rows(gu, dtype, m, k, n):
