@@ -31,6 +31,12 @@ reference checkout).  How each function is pinned (none is "parity unpinned"):
                            (tests/kernels/moe/test_moe_align_block_size.py)
 * gfx950 layout            this build's own format: inverse round trip and
                            decode-to-(K,N) equality with the Marlin decode
+* 8-bit weights (W8A16)    the same pinning as the 4-bit functions: recipe
+                           (get_weight_perm(8), interleave [0,2,1,3]) against
+                           the repack kernel's arithmetic
+                           (gptq_marlin_repack.cu:129-236), bijection on
+                           bytes, round trips, exhaustive dequantisation over
+                           256 codes
 """
 
 from __future__ import annotations
@@ -249,6 +255,150 @@ def awq_marlin_repack(b_q_weight: np.ndarray, size_k: int, size_n: int) -> np.nd
 
 
 # --------------------------------------------------------------------------
+# 8-bit weights (uint8b128, W8A16): same tile shape, four codes per word
+# --------------------------------------------------------------------------
+
+def pack_rows8(q: np.ndarray) -> np.ndarray:
+    """GPTQ packing along K with 8-bit codes (quant_utils.py:725-746 with
+    num_bits = 8): word[k//4][n] holds q[k][n] at bits 8*(k%4)."""
+    k, n = q.shape
+    assert k % 4 == 0
+    u = q.astype(np.uint32).reshape(k // 4, 4, n)
+    out = np.zeros((k // 4, n), dtype=np.uint32)
+    for i in range(4):
+        out |= u[:, i, :] << np.uint32(8 * i)
+    return out.view(np.int32)
+
+
+def unpack_rows8(packed: np.ndarray) -> np.ndarray:
+    u = packed.view(np.uint32)
+    kp, n = u.shape
+    out = np.empty((kp, 4, n), dtype=np.int32)
+    for i in range(4):
+        out[:, i, :] = (u >> np.uint32(8 * i)) & np.uint32(0xFF)
+    return out.reshape(kp * 4, n)
+
+
+def marlin_weight_perm_recipe8() -> np.ndarray:
+    """get_weight_perm(num_bits=8) (marlin_utils_test.py:69-121): the same
+    1024-entry table as for 4 bits, interleaved in fours by [0, 2, 1, 3]."""
+    table = []
+    for lane in range(32):
+        col = lane // 4
+        one = []
+        for block in (0, 1):
+            for row in (2 * (lane % 4), 2 * (lane % 4) + 1,
+                        2 * (lane % 4 + 4), 2 * (lane % 4 + 4) + 1):
+                one.append(16 * row + col + 8 * block)
+        for j in range(4):
+            table.extend(p + 256 * j for p in one)
+    return np.array(table).reshape(-1, 4)[:, [0, 2, 1, 3]].ravel()
+
+
+def marlin_pack8_recipe(q: np.ndarray) -> np.ndarray:
+    """(K,N) 8-bit codes -> Marlin (K/16, 4N) int32 following
+    marlin_permute_weights + marlin_weights (marlin_utils_test.py:31-66)."""
+    k, n = q.shape
+    assert k % 16 == 0 and n % 64 == 0
+    perm = marlin_weight_perm_recipe8()
+    t = q.reshape(k // 16, 16, n // 16, 16).transpose(0, 2, 1, 3).reshape(k // 16, n * 16)
+    t = t.reshape(-1, perm.size)[:, perm].reshape(t.shape)
+    u = t.astype(np.uint32).reshape(k // 16, n * 4, 4)
+    out = np.zeros((k // 16, n * 4), dtype=np.uint32)
+    for i in range(4):
+        out |= u[:, :, i] << np.uint32(8 * i)
+    return out.view(np.int32)
+
+
+def marlin_pack8_closed_form(q: np.ndarray) -> np.ndarray:
+    """The repack kernel's arithmetic for num_bits = 8
+    (gptq_marlin_repack.cu:129-236): tile (kt, nt) is 256 words; thread
+    `lane` of warp j (16-column sub-tile) writes words lane*8 + 2j (column
+    c = lane//4) and lane*8 + 2j + 1 (column c + 8); byte i of a word holds
+    row 2*(lane%4) + {0, 1, 8, 9}[pack_idx[i]], pack_idx = {0, 2, 1, 3}."""
+    k, n = q.shape
+    assert k % 16 == 0 and n % 64 == 0
+    kt_n, nt_n = k // 16, n // 64
+    tile = q.reshape(kt_n, 16, nt_n, 4, 16).astype(np.uint32)  # [kt][r][nt][j][col]
+    out = np.zeros((kt_n, nt_n, 32, 4, 2), dtype=np.uint32)    # [kt][nt][lane][j][half]
+    tc_offsets = (0, 1, 8, 9)
+    pack_idx = (0, 2, 1, 3)
+    for lane in range(32):
+        c = lane // 4
+        r0 = 2 * (lane % 4)
+        for half in (0, 1):
+            word = np.zeros((kt_n, nt_n, 4), dtype=np.uint32)
+            for i in range(4):
+                word |= tile[:, r0 + tc_offsets[pack_idx[i]], :, :, c + 8 * half] << np.uint32(8 * i)
+            out[:, :, lane, :, half] = word
+    return out.reshape(kt_n, nt_n * 256).view(np.int32)
+
+
+marlin_pack8 = marlin_pack8_closed_form
+
+
+def marlin_unpack8(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    kt_n, nt_n = size_k // 16, size_n // 64
+    u = packed.view(np.uint32).reshape(kt_n, nt_n, 32, 4, 2)
+    q = np.empty((kt_n, 16, nt_n, 4, 16), dtype=np.int32)
+    tc_offsets = (0, 1, 8, 9)
+    pack_idx = (0, 2, 1, 3)
+    for lane in range(32):
+        c = lane // 4
+        r0 = 2 * (lane % 4)
+        for half in (0, 1):
+            w = u[:, :, lane, :, half]
+            for i in range(4):
+                q[:, r0 + tc_offsets[pack_idx[i]], :, :, c + 8 * half] = (w >> np.uint32(8 * i)) & np.uint32(0xFF)
+    return q.reshape(size_k, size_n)
+
+
+def gptq_marlin_repack8(b_q_weight: np.ndarray, perm: np.ndarray | None,
+                        size_k: int, size_n: int) -> np.ndarray:
+    """gptq_marlin_repack.cu:285-362 with num_bits = 8."""
+    q = unpack_rows8(b_q_weight)
+    assert q.shape == (size_k, size_n)
+    if perm is not None and perm.size > 0:
+        q = q[perm.astype(np.int64), :]
+    return marlin_pack8(q)
+
+
+# The gfx950 order for 8-bit codes: per strip a stream of 1-KiB blocks of 16
+# rows each; block b = 2c + h belongs to 32-row chunk c.  Word j of lane L holds
+# column 64*strip + 16*j + L%16 and rows 32c + 8*(L//16) + 4h + t, t = 0..3, row
+# t at byte GFX950_BYTE[t], so that w & 0x00ff00ff is the row pair (0, 1) and
+# (w >> 8) & 0x00ff00ff the pair (2, 3); blocks 2c and 2c+1 together give a
+# lane the eight consecutive rows of one MFMA operand.
+
+GFX950_BYTE = np.array([0, 2, 1, 3])
+
+
+def gfx950_pack8(q: np.ndarray) -> np.ndarray:
+    k, n = q.shape
+    assert k % 32 == 0 and n % 64 == 0
+    # [chunk][kb][h][t][strip][j][l]
+    t = q.astype(np.uint32).reshape(k // 32, 4, 2, 4, n // 64, 4, 16)
+    t = t.transpose(4, 0, 2, 1, 6, 5, 3)  # [strip][chunk][h][kb][l][j][t]
+    out = np.zeros(t.shape[:-1], dtype=np.uint32)
+    for row in range(4):
+        out |= t[..., row] << np.uint32(8 * GFX950_BYTE[row])
+    return out.reshape(-1).view(np.int32)
+
+
+def gfx950_unpack8(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    u = packed.view(np.uint32).reshape(size_n // 64, size_k // 32, 2, 4, 16, 4)
+    t = np.empty(u.shape + (4,), dtype=np.int32)
+    for row in range(4):
+        t[..., row] = (u >> np.uint32(8 * GFX950_BYTE[row])) & np.uint32(0xFF)
+    # [strip][chunk][h][kb][l][j][t] -> [chunk][kb][h][t][strip][j][l]
+    return t.transpose(1, 3, 2, 6, 0, 5, 4).reshape(size_k, size_n)
+
+
+def marlin8_to_gfx950(marlin_packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    return gfx950_pack8(marlin_unpack8(marlin_packed, size_k, size_n))
+
+
+# --------------------------------------------------------------------------
 # Scale / zero-point / bias layouts  (marlin_utils.py:401-505)
 # --------------------------------------------------------------------------
 
@@ -402,7 +552,8 @@ def from_bits16(b: np.ndarray, dtype: str) -> np.ndarray:
 # --------------------------------------------------------------------------
 
 def dequantize(q: np.ndarray, scales32: np.ndarray, group_size: int, dtype: str,
-               zeros: np.ndarray | None = None, g_idx: np.ndarray | None = None) -> np.ndarray:
+               zeros: np.ndarray | None = None, g_idx: np.ndarray | None = None,
+               num_bits: int = 4) -> np.ndarray:
     """w[k][n] = round_to_dtype((q[k][n] - z) * s[g(k)][n]) with z = 8
     (uint4b8) or the group's zero point (uint4); s is a value of `dtype`
     held as fp32; one rounding, to nearest even.  (q - z) is a small integer,
@@ -418,7 +569,7 @@ def dequantize(q: np.ndarray, scales32: np.ndarray, group_size: int, dtype: str,
         rows = np.arange(k) // group_size
     s = scales32.astype(np.float32)[rows, :]
     if zeros is None:
-        centred = q.astype(np.int32) - 8
+        centred = q.astype(np.int32) - (8 if num_bits == 4 else 128)   # uint4b8 / uint8b128
     else:
         centred = q.astype(np.int32) - zeros.astype(np.int32)[rows, :]
     return round_to_dtype(centred.astype(np.float32) * s, dtype)

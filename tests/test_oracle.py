@@ -311,3 +311,85 @@ def test_moe_block_size_rule():
     assert mo.moe_block_size_rule(16, 2, 8) == 8
     assert mo.moe_block_size_rule(4096, 2, 8) == 64
     assert mo.moe_block_size_rule(64, 2, 8) == 32  # 16/8=2, 16/16=1, 16/32=.5
+
+
+# ---------------------------------------------------------------- 8-bit weights (W8A16)
+def test_packings8_brute_force_and_inverse():
+    rng = np.random.default_rng(8)
+    q = rng.integers(0, 256, size=(16, 5), dtype=np.int32)
+    q[3, 2] = 255        # top byte of a word set: sign handling
+    p = mo.pack_rows8(q)
+    assert p.dtype == np.int32 and p.shape == (4, 5)
+    for k in range(16):
+        for n in range(5):
+            assert ((int(p.view(np.uint32)[k // 4, n]) >> (8 * (k % 4))) & 0xFF) == q[k, n]
+    assert np.array_equal(mo.unpack_rows8(p), q)
+
+
+@pytest.mark.parametrize("k,n", [(16, 64), (64, 128), (128, 320)])
+def test_marlin8_layout_two_derivations_agree(k, n):
+    rng = np.random.default_rng(k + n)
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    a, b = mo.marlin_pack8_recipe(q), mo.marlin_pack8_closed_form(q)
+    assert a.shape == (k // 16, 4 * n) and np.array_equal(a, b)
+    assert np.array_equal(mo.marlin_unpack8(a, k, n), q)
+    perm = mo.marlin_weight_perm_recipe8()
+    assert sorted(perm.tolist()) == list(range(1024))
+
+
+def test_marlin8_layout_single_byte_positions():
+    """One code set at a time: word lane*8 + 2j + half of its tile, byte i with
+    row 2*(lane%4) + {0,8,1,9}[i] (gptq_marlin_repack.cu:216-236)."""
+    for (row, col) in [(0, 0), (1, 0), (8, 0), (9, 0), (5, 8), (15, 63), (6, 37)]:
+        q = np.zeros((16, 64), dtype=np.int32)
+        q[row, col] = 0xAB
+        u = mo.marlin_pack8(q).view(np.uint32).ravel()
+        (word,) = np.nonzero(u)[0]
+        j, c16 = col // 16, col % 16
+        lane = 4 * (c16 % 8) + (row % 8) // 2
+        assert word == lane * 8 + 2 * j + c16 // 8
+        byte = [b for b in range(4) if (int(u[word]) >> (8 * b)) & 0xFF][0]
+        assert row == 2 * (lane % 4) + (0, 8, 1, 9)[byte]
+
+
+def test_repack8_identities():
+    rng = np.random.default_rng(5)
+    k, n = 64, 128
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    packed = mo.pack_rows8(q)
+    assert np.array_equal(mo.gptq_marlin_repack8(packed, None, k, n), mo.marlin_pack8(q))
+    perm = rng.permutation(k).astype(np.int32)
+    assert np.array_equal(mo.gptq_marlin_repack8(packed, perm, k, n), mo.marlin_pack8(q[perm]))
+
+
+@pytest.mark.parametrize("k,n", [(32, 64), (96, 192)])
+def test_gfx950_layout8_round_trip_and_positions(k, n):
+    rng = np.random.default_rng(k)
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    g = mo.gfx950_pack8(q)
+    assert g.size == k * n // 4
+    assert np.array_equal(mo.gfx950_unpack8(g, k, n), q)
+    assert np.array_equal(mo.marlin8_to_gfx950(mo.marlin_pack8(q), k, n), g)
+    # word ((strip*chunks + c)*2 + h)*256 + lane*4 + j, byte GFX950_BYTE[t]
+    u = g.view(np.uint32)
+    chunks = k // 32
+    for (kk, nn) in [(0, 0), (5, 17), (31, 63), (k - 1, n - 1), (13, 40)]:
+        strip, j, l16 = nn // 64, (nn % 64) // 16, nn % 16
+        c, r = kk // 32, kk % 32
+        kb, h, t = r // 8, (r % 8) // 4, r % 4
+        word = ((strip * chunks + c) * 2 + h) * 256 + (16 * kb + l16) * 4 + j
+        assert (int(u[word]) >> (8 * int(mo.GFX950_BYTE[t]))) & 0xFF == q[kk, nn]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_dequant8_exhaustive_against_exact_rationals(dtype):
+    rng = np.random.default_rng(12)
+    raw = np.concatenate([rng.uniform(1e-4, 1e-2, 24), np.array([0.0, 1.0, 2.0 ** -14, 3.0e-5, 0.333])])
+    s = mo.round_to_dtype(raw.astype(np.float32), dtype)
+    q = np.tile(np.arange(256, dtype=np.int32)[:, None], (1, s.size))
+    w = mo.dequantize(q, s[None, :], -1, dtype, num_bits=8)
+    for j, sv in enumerate(s):
+        for code in range(256):
+            want = _rne_fraction_to(dtype, Fraction(code - 128) * Fraction(float(sv)))
+            assert w[code, j] == np.float32(want), (dtype, code, sv)
+    assert np.all(w[128] == 0)
