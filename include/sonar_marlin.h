@@ -52,13 +52,16 @@ extern "C" {
  * (aphrodite/scalar_type.py:129-156, csrc/core/scalar_type.hpp:131-164) */
 #define SONAR_TYPE_UINT4B8 1125899907892224LL /* GPTQ: code - 8 */
 #define SONAR_TYPE_UINT4 1125899906843648LL   /* AWQ: code - zero point */
+#define SONAR_TYPE_UINT8B128 1125899923621888LL /* GPTQ 8-bit: code - 128 */
 
 const char* sonar_marlin_last_error(void);
 const char* sonar_marlin_version(void);
 
 /* GPTQ (K/8, N) int32, nibble k%8 of word [k/8][n] = code of W[k][n]
- * -> Marlin (K/16, 2N) int32.  perm (int32[K], may be NULL) selects source
- * rows: output row k is source row perm[k].  num_bits must be 4. */
+ * -> Marlin (K/16, 2N) int32; with num_bits == 8: (K/4, N) int32, byte k%4
+ * -> Marlin (K/16, 4N) int32.  perm (int32[K], may be NULL) selects source
+ * rows: output row k is source row perm[k].
+ * (gptq_marlin_repack, csrc/libtorch_stable/quantization/marlin/gptq_marlin_repack.cu:285-362) */
 int sonar_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_t* perm,
                              uint32_t* out, int64_t size_k, int64_t size_n,
                              int num_bits, void* stream);
@@ -75,6 +78,14 @@ int sonar_marlin_to_gfx950(const uint32_t* marlin, uint32_t* out,
                            int64_t size_k, int64_t size_n, void* stream);
 int sonar_gfx950_to_marlin(const uint32_t* gfx950, uint32_t* out,
                            int64_t size_k, int64_t size_n, void* stream);
+
+/* The same for 8-bit codes (uint8b128): Marlin (K/16, 4N) int32 <-> the
+ * streaming order of 1-KiB blocks of 16 rows x 64 columns.  No counterpart in
+ * the reference (its kernels read the Marlin order directly). */
+int sonar_marlin8_to_gfx950(const uint32_t* marlin, uint32_t* out,
+                            int64_t size_k, int64_t size_n, void* stream);
+int sonar_gfx950_to_marlin8(const uint32_t* gfx950, uint32_t* out,
+                            int64_t size_k, int64_t size_n, void* stream);
 
 /* Dequantised weight matrix W[K][N] (row-major, dtype elements) exactly as the
  * GEMM kernels form it in registers: round_to_dtype((code - z) * s).  Uses the

@@ -15,6 +15,7 @@ DTYPE_BF16 = 1
 LAYOUT_GFX950 = 0
 TYPE_UINT4B8 = 1125899907892224
 TYPE_UINT4 = 1125899906843648
+TYPE_UINT8B128 = 1125899923621888
 
 OK = 0
 E_INVALID = -1
@@ -29,6 +30,8 @@ PROTOTYPES = {
     "sonar_awq_marlin_repack": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "sonar_marlin_to_gfx950": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "sonar_gfx950_to_marlin": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "sonar_marlin8_to_gfx950": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "sonar_gfx950_to_marlin8": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "sonar_marlin_dequant": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                      c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "sonar_marlin_gemm_scratch_bytes": (c_size_t, [c_int64, c_int64, c_int64]),

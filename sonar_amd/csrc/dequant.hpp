@@ -164,6 +164,54 @@ __device__ __forceinline__ void load_cols(typename Dq<T>::Col (&cols)[4], const 
   }
 }
 
+// 8-bit codes (uint8b128, symmetric): (v - 128) * s with one rounding.  A
+// packed word holds four rows of one column; word4 returns them as two
+// registers (rows 0,1 and rows 2,3).  The code is OR-ed into the mantissa of
+// fp16 1024.0 for both activation types (bf16 has too few mantissa bits for
+// 128 + v); 1024 + 128 = 1152 comes off exactly, in fp16 or in fp32.
+template <typename T>
+struct Dq8;
+
+template <>
+struct Dq8<_Float16> {
+  struct Col {
+    half2_t s;
+  };
+  static __device__ __forceinline__ Col make_col(uint16_t scale_bits) {
+    const _Float16 s = __builtin_bit_cast(_Float16, scale_bits);
+    return Col{half2_t{s, s}};
+  }
+  static __device__ __forceinline__ uint2 word4(uint32_t q, const Col& c, uint32_t magic) {
+    const half2_t off = half2_t{(_Float16)1152.f, (_Float16)1152.f};
+    const uint32_t lo = and_or(q, 0x00ff00ffu, magic);
+    const uint32_t hi = and_or(q >> 8, 0x00ff00ffu, magic);
+    const half2_t w0 = (__builtin_bit_cast(half2_t, lo) - off) * c.s;
+    const half2_t w1 = (__builtin_bit_cast(half2_t, hi) - off) * c.s;
+    return make_uint2(__builtin_bit_cast(uint32_t, w0), __builtin_bit_cast(uint32_t, w1));
+  }
+};
+
+template <>
+struct Dq8<__bf16> {
+  struct Col {
+    float s, c0;
+  };
+  static __device__ __forceinline__ Col make_col(uint16_t scale_bits) {
+    Col c;
+    c.s = __builtin_bit_cast(float, (uint32_t)scale_bits << 16);
+    c.c0 = -1152.f * c.s;  // 9 * 2^7 times an 8-bit mantissa: exact
+    return c;
+  }
+  static __device__ __forceinline__ uint2 word4(uint32_t q, const Col& c, uint32_t magic) {
+    const uint32_t lo = and_or(q, 0x00ff00ffu, magic);
+    const uint32_t hi = and_or(q >> 8, 0x00ff00ffu, magic);
+    // (1024 + v) * s - 1152 s: both products and their sum are exact in fp32
+    const bf16x2_t w0 = Dq<__bf16>::pair(lo, c.s, c.c0);
+    const bf16x2_t w1 = Dq<__bf16>::pair(hi, c.s, c.c0);
+    return make_uint2(__builtin_bit_cast(uint32_t, w0), __builtin_bit_cast(uint32_t, w1));
+  }
+};
+
 // One packed word whose eight rows (8 consecutive k) may lie in different groups:
 // a shard of an act-order matrix that does not hold whole groups.  `groups`
 // holds the group of each row, `scale_col` points at this column's scale of

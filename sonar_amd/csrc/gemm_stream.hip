@@ -305,6 +305,118 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
 }
 
 // ---------------------------------------------------------------------------
+// The general kernel for 8-bit codes (uint8b128, symmetric, no act-order
+// gather): the same partition, reduction and fix-up; a 32-row chunk of a strip
+// is two 1-KiB blocks of 16 rows, whose words give a lane the low and the high
+// four of the eight consecutive rows of an MFMA operand.
+template <typename T, int MB>
+struct UnitBuf8 {
+  uint4 q[unit_buffer_chunks<MB>()][2];
+  typename Dq<T>::vec8 a[unit_buffer_chunks<MB>()][MB];
+  uint32_t sbits[4];
+  int group;
+};
+
+template <typename T, int MB>
+__device__ __forceinline__ void load_unit8(UnitBuf8<T, MB>& b, const StreamParams& p, int u, int lane,
+                                           bool grouped) {
+  const int col16 = lane & 15, kb = lane >> 4;
+  const int strip = u / p.units_per_strip;
+  const int unit = u - strip * p.units_per_strip;
+  const int chunk0 = unit * p.unit_chunks;
+  const uint4* bsrc = p.b + ((long)strip * p.chunks_per_strip + chunk0) * 128 + lane;
+#pragma unroll
+  for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc)
+    if (cc < p.unit_chunks) {
+      b.q[cc][0] = bsrc[(2 * cc) * 64];
+      b.q[cc][1] = bsrc[(2 * cc + 1) * 64];
+    }
+#pragma unroll
+  for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc)
+    if (cc < p.unit_chunks) {
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        b.a[cc][mb] = load_a<T, false>(p, 16 * mb + col16, (chunk0 + cc) * kChunkK + 8 * kb);
+    }
+  const int g = grouped ? (chunk0 * kChunkK) / p.group_size : 0;
+  b.group = g;
+  const uint16_t* srow = p.scales + (long)g * p.size_n + strip * kStripN;
+#pragma unroll
+  for (int j = 0; j < 4; ++j) b.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
+}
+
+template <typename T, int MB>
+__global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const StreamParams p) {
+  typedef typename Dq<T>::vec8 vec8;
+  typedef typename Dq8<T>::Col Col;
+  __shared__ float4 red[4][MB * 4][64];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int col16 = lane & 15;
+  const int u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
+  const int u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
+  const bool grouped = p.num_groups > 1;
+  const uint32_t magic = magic_register();
+
+  UnitBuf8<T, MB> cur, nxt;
+  int mine = u_begin + wave;
+  if (mine < u_end) load_unit8<T, MB>(cur, p, mine, lane, grouped);
+
+  int seg_begin = u_begin;
+  while (seg_begin < u_end) {
+    const int strip = seg_begin / p.units_per_strip;
+    const int strip_first = strip * p.units_per_strip;
+    const int strip_end = strip_first + p.units_per_strip;
+    const int seg_end = u_end < strip_end ? u_end : strip_end;
+
+    floatx4_t acc[MB][4];
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+    while (mine < seg_end) {
+      const int next = mine + kWaves;
+      if (next < u_end) load_unit8<T, MB>(nxt, p, next, lane, grouped);
+      Col cols[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) cols[j] = Dq8<T>::make_col((uint16_t)cur.sbits[j]);
+      int cur_group = cur.group;
+      const int chunk0 = (mine - strip_first) * p.unit_chunks;
+#pragma unroll
+      for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc) {
+        if (cc < p.unit_chunks) {
+          const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
+          if (g != cur_group) {  // groups smaller than a unit
+            cur_group = g;
+            const uint16_t* srow = p.scales + (long)g * p.size_n + strip * kStripN;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) cols[j] = Dq8<T>::make_col(srow[scale_slot(16 * j + col16, grouped)]);
+          }
+          const uint32_t lo[4] = {cur.q[cc][0].x, cur.q[cc][0].y, cur.q[cc][0].z, cur.q[cc][0].w};
+          const uint32_t hi[4] = {cur.q[cc][1].x, cur.q[cc][1].y, cur.q[cc][1].z, cur.q[cc][1].w};
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const uint2 w_lo = Dq8<T>::word4(lo[j], cols[j], magic);
+            const uint2 w_hi = Dq8<T>::word4(hi[j], cols[j], magic);
+            const vec8 w = __builtin_bit_cast(vec8, u32x4_t{w_lo.x, w_lo.y, w_hi.x, w_hi.y});
+#pragma unroll
+            for (int mb = 0; mb < MB; ++mb) acc[mb][j] = Dq<T>::mfma(w, cur.a[cc][mb], acc[mb][j]);
+          }
+        }
+      }
+      cur = nxt;
+      mine = next;
+    }
+
+    reduce_waves<MB, kWaves>(acc, red, wave, lane);
+    if (wave == 0) finish_segment<T, MB>(p, strip, seg_begin, seg_end, lane, acc);
+    seg_begin = seg_end;
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Fast kernel for M <= 16, K % 128 == 0, groups of 128 * 2^s rows (or one
 // group), no act-order.  Everything a wavefront consumes arrives in its own
 // region of LDS through asynchronous global->LDS copies, so bytes in flight tie
@@ -737,6 +849,40 @@ __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __rest
   }
 }
 
+// The same for 8-bit codes: one wavefront per 1-KiB block of 16 rows.
+template <typename T>
+__global__ __launch_bounds__(256) void marlin_dequant8_kernel(const uint4* __restrict__ b,
+                                                             const uint16_t* __restrict__ scales,
+                                                             uint16_t* __restrict__ w_out, int size_n, int size_k,
+                                                             int num_groups, int group_size, long total_blocks) {
+  const int lane = threadIdx.x & 63;
+  const int col16 = lane & 15;
+  const int kb = lane >> 4;
+  const int blocks_per_strip = size_k / 16;
+  const bool grouped = num_groups > 1;
+  const uint32_t magic = magic_register();
+  for (long blk = (long)blockIdx.x * 4 + (threadIdx.x >> 6); blk < total_blocks; blk += (long)gridDim.x * 4) {
+    const int strip = (int)(blk / blocks_per_strip);
+    const int in_strip = (int)(blk % blocks_per_strip);
+    const int chunk = in_strip >> 1, h = in_strip & 1;
+    const int g = grouped ? (chunk * kChunkK) / group_size : 0;
+    const uint16_t* srow = scales + (long)g * size_n + strip * kStripN;
+    const uint4 q = b[blk * 64 + lane];
+    const uint32_t words[4] = {q.x, q.y, q.z, q.w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint2 w = Dq8<T>::word4(words[j], Dq8<T>::make_col(srow[scale_slot(16 * j + col16, grouped)]), magic);
+      const uint16_t bits[4] = {(uint16_t)(w.x & 0xffffu), (uint16_t)(w.x >> 16), (uint16_t)(w.y & 0xffffu),
+                                (uint16_t)(w.y >> 16)};
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        const long k = (long)chunk * kChunkK + 8 * kb + 4 * h + t;
+        w_out[k * size_n + strip * kStripN + 16 * j + col16] = bits[t];
+      }
+    }
+  }
+}
+
 int cu_count() {
   static int cached = 0;
   if (cached == 0) {
@@ -794,6 +940,16 @@ void launch_stream_mb(const StreamParams& p, bool has_perm, hipStream_t st) {
   }
 }
 
+template <typename T>
+void launch_stream8_mb(const StreamParams& p, hipStream_t st) {
+  switch ((p.size_m + 15) / 16) {
+    case 1: marlin_stream8_kernel<T, 1><<<p.parts, kWaves * 64, 0, st>>>(p); break;
+    case 2: marlin_stream8_kernel<T, 2><<<p.parts, kWaves * 64, 0, st>>>(p); break;
+    case 3: marlin_stream8_kernel<T, 3><<<p.parts, kWaves * 64, 0, st>>>(p); break;
+    default: marlin_stream8_kernel<T, 4><<<p.parts, kWaves * 64, 0, st>>>(p); break;
+  }
+}
+
 template <typename T, bool HAS_ZP, int WAVES>
 int launch_fast_waves(const StreamParams& p, int unit_group_shift, hipStream_t st) {
   static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
@@ -829,6 +985,7 @@ struct Checked {
   bool has_perm;
   bool row_groups;  // act-order shard without whole groups: the group of a row comes from g_idx
   int group_size;
+  int bits;         // 4 or 8
 };
 
 int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_t* b_zeros,
@@ -842,22 +999,25 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
                 "size_n = %ld, is not divisible by min_thread_n = %d", (long)size_n, kStripN);
   SONAR_REQUIRE(b_scales != nullptr, "b_scales must not be NULL");
   SONAR_REQUIRE(num_groups >= 1, "num_groups = %ld must be >= 1", (long)num_groups);
-  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4)
+  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4 && b_type_id != SONAR_TYPE_UINT8B128)
     return fail(SONAR_E_UNSUPPORTED,
-                "b_type id %ld is not built here: only uint4b8 (GPTQ) and uint4 (AWQ) weights are",
+                "b_type id %ld is not built here: only uint4b8, uint8b128 (GPTQ) and uint4 (AWQ) weights are",
                 (long)b_type_id);
+  out.bits = b_type_id == SONAR_TYPE_UINT8B128 ? 8 : 4;
   out.has_zp = b_zeros != nullptr;
   if (out.has_zp)
     SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4, "b_type must be u4 or u8 when has_zp = True");
   else
-    SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4B8,
-                  "b_type must be uint4b8 when has_zp = False (uint4 needs b_zeros)");
+    SONAR_REQUIRE(b_type_id != SONAR_TYPE_UINT4,
+                  "b_type must be uint4b8 or uint8b128 when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   out.has_perm = perm != nullptr;
   out.row_groups = out.has_perm && !is_k_full;
   if (out.has_perm) SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
   if (out.row_groups) {
     // marlin.cu:343-351,763-769: group_size = 0, every row looks its group up
+    if (out.bits == 8)
+      return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False and 8-bit weights is not built");
     if (out.has_zp)
       return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False and zero points is not built");
     out.group_size = 0;
@@ -931,6 +1091,10 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
     perm = nullptr;
     chk.has_perm = false;
   }
+  if (chk.bits == 8 && chk.has_perm)
+    return fail(SONAR_E_INVALID,
+                "act-order with 8-bit weights needs size_m * size_k * 2 more scratch bytes "
+                "(the column-permuted copy of A)");
   if (chk.row_groups && chk.has_perm)
     return fail(SONAR_E_INVALID,
                 "act-order with is_k_full = False needs size_m * size_k * 2 more scratch bytes "
@@ -963,7 +1127,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
     }
   }
   static const bool no_fast = getenv("SONAR_MARLIN_NO_FAST") != nullptr;  // debugging aid
-  const bool fast_shape = !no_fast && !chk.has_perm && !chk.row_groups && p.chunks_per_strip % 4 == 0 && fast_groups &&
+  const bool fast_shape = !no_fast && chk.bits == 4 && !chk.has_perm && !chk.row_groups &&
+                          p.chunks_per_strip % 4 == 0 && fast_groups &&
                           size_m * a_row_stride * 2 < (1LL << 31);
   // Short strips (K <= 4096) on a matrix with at least 64 of them: one workgroup
   // per strip.  No strip is shared, so no partial tile goes through memory and
@@ -1004,7 +1169,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
   const bool async_tile = tile_async_applies(chk.has_perm, num_groups, chk.group_size);
   const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
-  if (plan.tile && !no_tile && !chk.row_groups) {  // the row -> group lookup exists in the streaming kernel only
+  // the row -> group lookup and 8-bit codes exist in the streaming kernels only
+  if (plan.tile && !no_tile && !chk.row_groups && chk.bits == 4) {
     const size_t used = stream_scratch_bytes();
     return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
                      size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used,
@@ -1036,6 +1202,9 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
         rc = chk.has_zp ? launch_fast<__bf16, true>(p, unit_group_shift, half, st)
                         : launch_fast<__bf16, false>(p, unit_group_shift, half, st);
       if (rc) return rc;
+    } else if (chk.bits == 8) {
+      if (dtype == SONAR_DTYPE_F16) launch_stream8_mb<_Float16>(p, st);
+      else launch_stream8_mb<__bf16>(p, st);
     } else if (dtype == SONAR_DTYPE_F16) {
       if (chk.has_zp) launch_stream_mb<_Float16, true>(p, chk.has_perm, st);
       else launch_stream_mb<_Float16, false>(p, chk.has_perm, st);
@@ -1070,6 +1239,14 @@ extern "C" int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout, co
   const uint16_t* s = static_cast<const uint16_t*>(b_scales);
   uint16_t* w = static_cast<uint16_t*>(w_out);
   const int ng = (int)num_groups, gs = chk.group_size, n = (int)size_n, k = (int)size_k;
+  if (chk.bits == 8) {
+    const long total_blocks = (size_n / kStripN) * (size_k / 16);
+    long grid = (total_blocks + 3) / 4;
+    if (grid > 8192) grid = 8192;
+    if (dtype == SONAR_DTYPE_F16) marlin_dequant8_kernel<_Float16><<<(int)grid, 256, 0, st>>>(b, s, w, n, k, ng, gs, total_blocks);
+    else marlin_dequant8_kernel<__bf16><<<(int)grid, 256, 0, st>>>(b, s, w, n, k, ng, gs, total_blocks);
+    return launch_status("marlin_dequant8_kernel");
+  }
   const int32_t* gi = chk.row_groups ? g_idx : nullptr;
   if (dtype == SONAR_DTYPE_F16) {
     if (chk.has_zp) marlin_dequant_kernel<_Float16, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);

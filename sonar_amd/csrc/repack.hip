@@ -144,6 +144,107 @@ __global__ __launch_bounds__(256) void gfx950_to_marlin_kernel(
   }
 }
 
+// ---- 8-bit codes (uint8b128): the same 16 x 64 tile in 256 words.  Word
+// lane*8 + 2j + half of the tile; lane = 4*c + h as above; byte s of the word
+// holds row 2h + (s >> 1) + 8*(s & 1), column 16j + c + 8*half
+// (gptq_marlin_repack.cu:216-236).
+constexpr int kMarlinTileWords8 = 256;
+
+__device__ __forceinline__ void marlin8_word_sources(int word, int byte, int& row, int& col) {
+  const int lane = word >> 3;
+  const int j = (word >> 1) & 3;
+  const int half = word & 1;
+  row = 2 * (lane & 3) + (byte >> 1) + 8 * (byte & 1);
+  col = 16 * j + (lane >> 2) + 8 * half;
+}
+
+// GPTQ (K/4, N) int32, byte k % 4 of word [k / 4][n] -> Marlin 8-bit order.
+template <bool HAS_PERM>
+__global__ __launch_bounds__(256) void gptq8_to_marlin_kernel(
+    const uint32_t* __restrict__ in, const int32_t* __restrict__ perm,
+    uint32_t* __restrict__ out, int size_k, int size_n, long total_words) {
+  const int n_tiles = size_n / kMarlinTileN;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_words;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long tile = idx / kMarlinTileWords8;
+    const int word = (int)(idx % kMarlinTileWords8);
+    const int kt = (int)(tile / n_tiles);
+    const int nt = (int)(tile % n_tiles);
+    uint32_t packed = 0;
+#pragma unroll
+    for (int byte = 0; byte < 4; ++byte) {
+      int row, col;
+      marlin8_word_sources(word, byte, row, col);
+      int k = kt * kMarlinTileK + row;
+      if (HAS_PERM) k = perm[k];
+      const int n = nt * kMarlinTileN + col;
+      const uint32_t src = in[(long)(k >> 2) * size_n + n];
+      packed |= ((src >> (8 * (k & 3))) & 0xFFu) << (8 * byte);
+    }
+    out[idx] = packed;
+  }
+}
+
+// Position of W[k][n] in the Marlin 8-bit order: word index and byte.
+__device__ __forceinline__ long marlin8_position(int k, int n, int n_tiles, int& byte) {
+  const int kt = k / kMarlinTileK, row = k % kMarlinTileK;
+  const int nt = n / kMarlinTileN, col = n % kMarlinTileN;
+  const int c16 = col & 15;
+  const int lane = 4 * (c16 & 7) + ((row & 7) >> 1);
+  byte = ((row & 1) << 1) | (row >> 3);
+  return ((long)kt * n_tiles + nt) * kMarlinTileWords8 + lane * 8 + 2 * (col >> 4) + (c16 >> 3);
+}
+
+// The gfx950 order for 8-bit codes: per strip a stream of 1-KiB blocks of 16
+// rows, block 2c + h in chunk c; word j of lane L: column 64s + 16j + L%16,
+// rows 32c + 8*(L/16) + 4h + t, row t at byte {0, 2, 1, 3}[t].
+__device__ __forceinline__ long gfx950_8_position(int k, int n, int chunks, int& byte) {
+  const int s = n / kStripN, j = (n % kStripN) >> 4, l16 = n & 15;
+  const int c = k / kChunkK, r = k % kChunkK;
+  const int kb = r >> 3, h = (r >> 2) & 1, t = r & 3;
+  byte = ((t & 1) << 1) | (t >> 1);
+  return ((((long)s * chunks + c) * 2 + h) * 64 + 16 * kb + l16) * 4 + j;
+}
+
+// One thread per output word; TO_GFX950 selects the direction.
+template <bool TO_GFX950>
+__global__ __launch_bounds__(256) void marlin8_gfx950_kernel(const uint32_t* __restrict__ in,
+                                                            uint32_t* __restrict__ out, int size_k, int size_n,
+                                                            long total_words) {
+  const int n_tiles = size_n / kMarlinTileN;
+  const int chunks = size_k / kChunkK;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_words;
+       idx += (long)gridDim.x * blockDim.x) {
+    uint32_t packed = 0;
+#pragma unroll
+    for (int byte = 0; byte < 4; ++byte) {
+      int k, n;
+      if (TO_GFX950) {  // which (k, n) does byte `byte` of gfx950 word idx hold?
+        const int j = (int)(idx & 3);
+        const int lane = (int)((idx >> 2) & 63);
+        const long block = idx >> 8;
+        const int h = (int)(block & 1);
+        const int c = (int)((block >> 1) % chunks);
+        const int s = (int)((block >> 1) / chunks);
+        const int t = ((byte & 1) << 1) | (byte >> 1);
+        k = c * kChunkK + 8 * (lane >> 4) + 4 * h + t;
+        n = s * kStripN + 16 * j + (lane & 15);
+      } else {
+        const long tile = idx / kMarlinTileWords8;
+        int row, col;
+        marlin8_word_sources((int)(idx % kMarlinTileWords8), byte, row, col);
+        k = (int)(tile / n_tiles) * kMarlinTileK + row;
+        n = (int)(tile % n_tiles) * kMarlinTileN + col;
+      }
+      int src_byte;
+      const long src = TO_GFX950 ? marlin8_position(k, n, n_tiles, src_byte)
+                                 : gfx950_8_position(k, n, chunks, src_byte);
+      packed |= ((in[src] >> (8 * src_byte)) & 0xFFu) << (8 * byte);
+    }
+    out[idx] = packed;
+  }
+}
+
 int grid_for(long total_words) {
   long blocks = (total_words + 255) / 256;
   if (blocks > 256L * 32) blocks = 256L * 32;
@@ -152,9 +253,7 @@ int grid_for(long total_words) {
 }
 
 int check_repack_shape(int64_t size_k, int64_t size_n, int num_bits) {
-  if (num_bits == 8)
-    return fail(SONAR_E_UNSUPPORTED, "num_bits = 8 (uint8b128) is not built; only 4-bit weights are");
-  SONAR_REQUIRE(num_bits == 4, "num_bits must be 4 or 8. Got = %d", num_bits);
+  SONAR_REQUIRE(num_bits == 4 || num_bits == 8, "num_bits must be 4 or 8. Got = %d", num_bits);
   SONAR_REQUIRE(size_k > 0 && size_n > 0, "size_k = %ld and size_n = %ld must be positive",
                 (long)size_k, (long)size_n);
   SONAR_REQUIRE(size_k % kMarlinTileK == 0, "size_k = %ld is not divisible by tile_k_size = %d",
@@ -179,8 +278,18 @@ extern "C" int sonar_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_
                                         int num_bits, void* stream) {
   if (int rc = check_repack_shape(size_k, size_n, num_bits)) return rc;
   SONAR_REQUIRE(b_q_weight && out, "b_q_weight and out must not be NULL");
-  const long total = size_k * size_n / 8;
   hipStream_t st = (hipStream_t)stream;
+  if (num_bits == 8) {
+    const long words = size_k * size_n / 4;
+    if (perm)
+      gptq8_to_marlin_kernel<true><<<grid_for(words), 256, 0, st>>>(b_q_weight, perm, out, (int)size_k,
+                                                                   (int)size_n, words);
+    else
+      gptq8_to_marlin_kernel<false><<<grid_for(words), 256, 0, st>>>(b_q_weight, nullptr, out, (int)size_k,
+                                                                    (int)size_n, words);
+    return launch_status("gptq8_to_marlin_kernel");
+  }
+  const long total = size_k * size_n / 8;
   if (perm)
     gptq_to_marlin_kernel<true><<<grid_for(total), 256, 0, st>>>(b_q_weight, perm, out, (int)size_k,
                                                                 (int)size_n, total);
@@ -193,6 +302,7 @@ extern "C" int sonar_gptq_marlin_repack(const uint32_t* b_q_weight, const int32_
 extern "C" int sonar_awq_marlin_repack(const uint32_t* b_q_weight, uint32_t* out, int64_t size_k,
                                        int64_t size_n, int num_bits, void* stream) {
   if (int rc = check_repack_shape(size_k, size_n, num_bits)) return rc;
+  if (num_bits != 4) return fail(SONAR_E_UNSUPPORTED, "awq_marlin_repack: 8-bit AWQ weights are not built");
   SONAR_REQUIRE(b_q_weight && out, "b_q_weight and out must not be NULL");
   const long total = size_k * size_n / 8;
   awq_to_marlin_kernel<<<grid_for(total), 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k,
@@ -220,4 +330,26 @@ extern "C" int sonar_gfx950_to_marlin(const uint32_t* gfx950, uint32_t* out, int
   gfx950_to_marlin_kernel<<<grid_for(total), 256, 0, (hipStream_t)stream>>>(gfx950, out, (int)size_k,
                                                                            (int)size_n, total);
   return launch_status("gfx950_to_marlin_kernel");
+}
+
+extern "C" int sonar_marlin8_to_gfx950(const uint32_t* marlin, uint32_t* out, int64_t size_k,
+                                       int64_t size_n, void* stream) {
+  if (int rc = check_repack_shape(size_k, size_n, 8)) return rc;
+  SONAR_REQUIRE(size_k % kChunkK == 0, "size_k = %ld is not divisible by %d", (long)size_k, kChunkK);
+  SONAR_REQUIRE(marlin && out && marlin != out, "marlin and out must be distinct non-NULL buffers");
+  const long total = size_k * size_n / 4;
+  marlin8_gfx950_kernel<true><<<grid_for(total), 256, 0, (hipStream_t)stream>>>(marlin, out, (int)size_k,
+                                                                               (int)size_n, total);
+  return launch_status("marlin8_gfx950_kernel");
+}
+
+extern "C" int sonar_gfx950_to_marlin8(const uint32_t* gfx950, uint32_t* out, int64_t size_k,
+                                       int64_t size_n, void* stream) {
+  if (int rc = check_repack_shape(size_k, size_n, 8)) return rc;
+  SONAR_REQUIRE(size_k % kChunkK == 0, "size_k = %ld is not divisible by %d", (long)size_k, kChunkK);
+  SONAR_REQUIRE(gfx950 && out && gfx950 != out, "gfx950 and out must be distinct non-NULL buffers");
+  const long total = size_k * size_n / 4;
+  marlin8_gfx950_kernel<false><<<grid_for(total), 256, 0, (hipStream_t)stream>>>(gfx950, out, (int)size_k,
+                                                                                (int)size_n, total);
+  return launch_status("marlin8_gfx950_kernel");
 }

@@ -65,8 +65,8 @@ std::unordered_map<const void*, NativeEntry> g_cache;
 
 uint32_t version_of(const Tensor& t) { return t.is_inference() ? 0u : t._version(); }
 
-// b_q_weight: (K/16, 2N) or (E, K/16, 2N) int32 in Marlin order.
-Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, int64_t experts) {
+// b_q_weight: (K/16, 2N) or (E, K/16, 2N) int32 in Marlin order; (K/16, 4N) for 8-bit codes.
+Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, int64_t experts, int bits = 4) {
   const void* key = b_q_weight.const_data_ptr();
   {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
@@ -76,12 +76,14 @@ Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, 
       return it->second.native;
   }
   Tensor native = at::empty_like(b_q_weight);
-  const int64_t words = size_k * size_n / 8;
+  const int64_t words = size_k * size_n / (32 / bits);
   const uint32_t* src = static_cast<const uint32_t*>(b_q_weight.const_data_ptr());
   uint32_t* dst = static_cast<uint32_t*>(native.mutable_data_ptr());
   for (int64_t e = 0; e < experts; ++e)
-    raise_if_failed(sonar_marlin_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
-                                           current_stream(b_q_weight)));
+    raise_if_failed(bits == 8 ? sonar_marlin8_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
+                                                        current_stream(b_q_weight))
+                              : sonar_marlin_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
+                                                       current_stream(b_q_weight)));
   std::lock_guard<std::mutex> lock(g_cache_mutex);
   g_cache[key] = NativeEntry{b_q_weight, native, size_k, size_n, experts, version_of(b_q_weight)};
   return native;
@@ -170,9 +172,9 @@ Tensor marlin_to_gfx950(const Tensor& b_q_weight, int64_t size_k, int64_t size_n
 // ---------------------------------------------------------------- dense GEMM
 void check_b_type(int64_t b_type_id) {
   TORCH_CHECK_NOT_IMPLEMENTED(
-      b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4,
+      b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4 || b_type_id == SONAR_TYPE_UINT8B128,
       "b_type_id = ", b_type_id,
-      " is not built here: only uint4b8 (GPTQ) and uint4 (AWQ) 4-bit weights are supported");
+      " is not built here: only uint4b8, uint8b128 (GPTQ) and uint4 (AWQ) weights are supported");
 }
 
 Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_q_weight,
@@ -197,7 +199,8 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
               ", tile_size = ", 16);
   TORCH_CHECK(b_q_weight.size(1) % 16 == 0, "b_q_weight.size(1) = ", b_q_weight.size(1),
               " is not divisible by tile_size = ", 16);
-  const int64_t actual_size_n = b_q_weight.size(1) / 16 * 8;
+  const int bits = b_type_id == SONAR_TYPE_UINT8B128 ? 8 : 4;
+  const int64_t actual_size_n = b_q_weight.size(1) / 16 * (32 / bits);
   TORCH_CHECK(size_n == actual_size_n, "size_n = ", size_n, ", actual_size_n = ", actual_size_n);
 
   TORCH_CHECK(a.is_cuda(), "A is not on GPU");
@@ -271,7 +274,7 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
                 " is not size_n / pack_factor = ", size_n / 8);
     TORCH_CHECK(z.scalar_type() == at::kInt, "b_zeros must be int32");
   } else {
-    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8,
+    TORCH_CHECK(b_type_id != SONAR_TYPE_UINT4,
                 "b_type must be uint4b8, uint8b128, int4, int8, float8_e4m3fn or float4_e2m1f when "
                 "has_zp = False. Got = uint4");
   }
@@ -280,7 +283,7 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
   TORCH_CHECK(workspace.is_cuda() && workspace.scalar_type() == at::kInt && workspace.is_contiguous(),
               "workspace must be a contiguous int32 GPU tensor");
 
-  Tensor native = native_weights(b_q_weight, size_k, size_n, 1);
+  Tensor native = native_weights(b_q_weight, size_k, size_n, 1, bits);
   size_t scratch_bytes = sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k);
   if (perm != nullptr) scratch_bytes += (size_t)size_m * size_k * 2;  // room for the column-permuted copy of A
   Tensor scratch = at::empty({(int64_t)scratch_bytes}, a.options().dtype(at::kByte));

@@ -97,7 +97,7 @@ def test_marlin_gemm_op_rejects_like_the_reference():
     with pytest.raises(RuntimeError):
         call(t=scalar_types.uint4)            # uint4 needs zero points
     with pytest.raises(RuntimeError):
-        call(t=scalar_types.uint8b128)        # 8-bit weights are not built
+        call(t=scalar_types.uint8b128)        # 4-bit packing under the 8-bit type: wrong size_n
     with pytest.raises(RuntimeError, match="workspace"):
         call(ws=dl.workspace[:8])
     with pytest.raises(RuntimeError):
@@ -197,6 +197,32 @@ def test_linear_kernel_row_parallel_act_order_shard(dtype, rows):
     assert kern.is_k_full is False
     x32 = mo.make_activations(6, rows, k, dtype)
     y = kern.apply_weights(layer, gu.dev_bits16(x32, dtype), None)
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y), mo.gemm_reference(x32, w_ref))
+    assert ok, worst
+
+
+@pytest.mark.parametrize("k,n,g,dtype,rows", [(512, 256, 128, "fp16", 3), (1024, 4096, 128, "bf16", 70),
+                                              (4000, 192, -1, "fp16", 9)])
+def test_w8a16_through_the_ops_and_the_linear_kernel(k, n, g, dtype, rows):
+    """uint8b128 checkpoint tensors (qweight (K/4, N), scales) -> gptq_marlin_repack
+    with num_bits = 8 -> marlin_gemm, through MarlinLinearKernel (with tile
+    padding of K for the third case)."""
+    from sonar_amd.marlin_linear import MarlinLinearKernel, MPLinearLayerConfig
+    from sonar_amd.scalar_type import scalar_types
+    rng = np.random.default_rng(k + n)
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    groups = 1 if g == -1 else k // g
+    scales = mo.round_to_dtype(rng.uniform(1e-4, 1e-3, size=(groups, n)).astype(np.float32), dtype)
+    w_ref = mo.dequantize(q, scales, g, dtype, num_bits=8)
+    layer = types.SimpleNamespace(bias=None)
+    layer.qweight = gu.dev_i32(mo.pack_rows8(q))
+    layer.scales = gu.dev_bits16(scales, dtype)
+    kern = MarlinLinearKernel(MPLinearLayerConfig((k, n), (k, n), scalar_types.uint8b128, _tdt(dtype), g, False,
+                                                  False), w_zp_param_name=None, w_gidx_param_name=None)
+    kern.process_weights_after_loading(layer)
+    x32 = mo.make_activations(2, rows, k, dtype, std=0.5)
+    y = kern.apply_weights(layer, gu.dev_bits16(x32, dtype), None)
+    assert y.shape == (rows, n)
     ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y), mo.gemm_reference(x32, w_ref))
     assert ok, worst
 

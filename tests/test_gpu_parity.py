@@ -173,11 +173,11 @@ def test_error_paths(gu):
         _lib.check(lib.sonar_gptq_marlin_repack(gu.ptr(t), None, gu.ptr(t), 24, 64, 4, gu.stream()))
     with pytest.raises(_lib.SonarMarlinError, match="size_n"):
         _lib.check(lib.sonar_awq_marlin_repack(gu.ptr(t), gu.ptr(t), 32, 96, 4, gu.stream()))
-    with pytest.raises(NotImplementedError):
-        _lib.check(lib.sonar_gptq_marlin_repack(gu.ptr(t), None, gu.ptr(t), 32, 64, 8, gu.stream()))
+    with pytest.raises(NotImplementedError):   # 8-bit AWQ weights
+        _lib.check(lib.sonar_awq_marlin_repack(gu.ptr(t), gu.ptr(t), 32, 64, 8, gu.stream()))
     layer = gu.DeviceLayer(1, 128, 64, 128, "fp16")
     a = torch.zeros((1, 128), dtype=torch.float16, device=gu.DEV)
-    layer.b_type = 1125899923621888  # uint8b128
+    layer.b_type = 1125899906844672  # uint8: 8-bit codes with zero points
     with pytest.raises(NotImplementedError):
         layer.gemm(a, 1)
     layer.b_type = _lib.TYPE_UINT4  # uint4 needs zero points
@@ -232,6 +232,98 @@ def test_act_order_with_permuted_copy_of_a(gu, dtype, m, k, n):
     assert ok, f"max_err={max_err} max_ref={max_ref}"
     gathered = layer.gemm(a, m)
     ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(fast), gu.host_f32(gathered))
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+
+
+def _layer8(gu, seed, k, n, g, dtype, act_order=False):
+    """An 8-bit (uint8b128) layer on the device: GPTQ packing -> repack op ->
+    streaming order, plus the oracle's dequantised matrix."""
+    from sonar_amd import _lib
+    rng = np.random.default_rng(seed)
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    groups = 1 if g in (-1, k) else k // g
+    scales = mo.round_to_dtype(rng.uniform(1e-4, 1e-3, size=(groups, n)).astype(np.float32), dtype)
+    g_idx = perm = None
+    order = None
+    if act_order:
+        g_idx_np = (rng.permutation(k) // g).astype(np.int32)
+        g_sorted, order = mo.stable_sort_g_idx(g_idx_np)
+        g_idx, perm = gu.dev_i32(g_sorted), gu.dev_i32(order)
+        w_ref = mo.dequantize(q, scales, g, dtype, g_idx=g_idx_np, num_bits=8)
+    else:
+        w_ref = mo.dequantize(q, scales, g, dtype, num_bits=8)
+    lib = _lib.load()
+    marlin = torch.empty((k // 16, 4 * n), dtype=torch.int32, device=gu.DEV)
+    _lib.check(lib.sonar_gptq_marlin_repack(gu.ptr(gu.dev_i32(mo.pack_rows8(q))), gu.ptr(perm), gu.ptr(marlin),
+                                            k, n, 8, gu.stream()))
+    native = torch.empty_like(marlin)
+    _lib.check(lib.sonar_marlin8_to_gfx950(gu.ptr(marlin), gu.ptr(native), k, n, gu.stream()))
+    s_dev = gu.dev_bits16(mo.marlin_permute_scales(scales, k, n, -1 if groups == 1 else g), dtype)
+    return dict(q=q, order=order, marlin=marlin, native=native, scales=s_dev, groups=groups, w_ref=w_ref,
+                g_idx=g_idx, perm=perm)
+
+
+@pytest.mark.parametrize("k,n", [(128, 64), (640, 448), (4096, 1024)])
+@pytest.mark.parametrize("act_order", [False, True])
+def test_repack8_and_layout_bit_exact(gu, k, n, act_order):
+    from sonar_amd import _lib
+    L = _layer8(gu, k + n, k, n, 128, "fp16", act_order)
+    torch.cuda.synchronize()
+    q_rows = L["q"] if L["order"] is None else L["q"][L["order"]]
+    assert np.array_equal(L["marlin"].cpu().numpy(), mo.marlin_pack8(q_rows).reshape(k // 16, 4 * n))
+    assert np.array_equal(L["native"].cpu().numpy().ravel(), mo.gfx950_pack8(q_rows))
+    back = torch.empty_like(L["marlin"])
+    _lib.check(_lib.load().sonar_gfx950_to_marlin8(gu.ptr(L["native"]), gu.ptr(back), k, n, gu.stream()))
+    assert torch.equal(back, L["marlin"])
+
+
+W8_CASES = [
+    # m, k, n, g, act_order, bias
+    (1, 128, 64, 128, False, False),
+    (7, 512, 256, 128, False, True),
+    (16, 4096, 1024, 128, False, False),
+    (33, 1024, 320, 64, False, False),
+    (64, 256, 4096, -1, False, True),
+    (100, 1024, 512, 128, False, False),
+    (13, 1024, 256, 128, True, False),
+    (300, 512, 192, 32, False, False),
+]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("m,k,n,g,act,bias", W8_CASES)
+def test_w8a16_dequant_bit_exact_and_gemm_within_tolerance(gu, dtype, m, k, n, g, act, bias):
+    """uint8b128 weights through the same entry points (generate_kernels.py:80-86,
+    dequant.h: code - 128, then the scale)."""
+    from sonar_amd import _lib
+    lib = _lib.load()
+    L = _layer8(gu, 3 * m + k, k, n, g, dtype, act)
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    w = torch.empty((k, n), dtype=tdt, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_dequant(gu.ptr(L["native"]), _lib.LAYOUT_GFX950, gu.ptr(L["scales"]), None,
+                                        gu.ptr(L["g_idx"]), gu.ptr(w), gu.dtype_code(dtype), _lib.TYPE_UINT8B128,
+                                        n, k, L["groups"], 1, gu.stream()))
+    torch.cuda.synchronize()
+    want = L["w_ref"] if L["order"] is None else L["w_ref"][L["order"]]
+    assert np.array_equal(gu.host_f32(w), want)
+
+    bias32 = bias_dev = None
+    if bias:
+        bias32 = mo.round_to_dtype(np.random.default_rng(m).standard_normal(n).astype(np.float32), dtype)
+        bias_dev = gu.dev_bits16(mo.marlin_permute_bias(bias32), dtype)
+    a32 = mo.make_activations(m + 1, m, k, dtype, std=0.5)
+    a = gu.dev_bits16(a32, dtype)
+    c = torch.empty((m, n), dtype=tdt, device=gu.DEV)
+    workspace = torch.zeros(torch.cuda.get_device_properties(0).multi_processor_count, dtype=torch.int32,
+                            device=gu.DEV)
+    nbytes = lib.sonar_marlin_gemm_scratch_bytes(m, n, k) + (m * k * 2 if act else 0)
+    scratch = torch.empty(nbytes, dtype=torch.uint8, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_gemm(
+        gu.ptr(a), k, gu.ptr(c), gu.ptr(L["native"]), _lib.LAYOUT_GFX950, gu.ptr(bias_dev), gu.ptr(L["scales"]), None,
+        gu.ptr(L["g_idx"]), gu.ptr(L["perm"]), gu.ptr(workspace), workspace.numel(), gu.ptr(scratch), scratch.numel(),
+        gu.dtype_code(dtype), _lib.TYPE_UINT8B128, m, n, k, L["groups"], 1, 0, 1, gu.stream()))
+    torch.cuda.synchronize()
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), mo.gemm_reference(a32, L["w_ref"], bias32))
     assert ok, f"max_err={max_err} max_ref={max_ref}"
 
 

@@ -161,7 +161,9 @@ def test_marlin_linear_kernel_gates():
     from sonar_amd.scalar_type import scalar_types as st
     ok = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4b8, torch.float16, 128, False, False)
     assert MarlinLinearKernel.can_implement(ok) == (True, None)
-    bad_type = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint8b128, torch.float16, 128, False, False)
+    eight_bit = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint8b128, torch.float16, 128, False, False)
+    assert MarlinLinearKernel.can_implement(eight_bit) == (True, None)
+    bad_type = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint8, torch.float16, 128, True, False)
     assert not MarlinLinearKernel.can_implement(bad_type)[0]
     bad_group = MPLinearLayerConfig((4096, 4096), (4096, 4096), st.uint4b8, torch.float16, 100, False, False)
     assert not MarlinLinearKernel.can_implement(bad_group)[0]
