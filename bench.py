@@ -107,16 +107,18 @@ def cpu_baseline(threads: int):
 
 def variants_sweep(torch, ops, gen, time_graph):
     """K = 4096, N = 11008 at M = 1 and 512: act-order (perm gathers the columns
-    of A, weights repacked in sorted-group order) and AWQ (per-group zero points)."""
+    of A, weights repacked in sorted-group order), AWQ (per-group zero points)
+    and 8-bit weights (uint8b128)."""
     from sonar_amd import marlin_utils
     from sonar_amd.scalar_type import scalar_types
     dev = "cuda:0"
     k, n = 4096, 11008
     out = []
-    for name in ("act_order", "awq"):
+    for name in ("act_order", "awq", "w8a16"):
         layers = []
+        words = 4 * n if name == "w8a16" else 2 * n     # 8-bit codes: four per word
         for _ in range(6):
-            qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, 2 * n), dtype=torch.int32, device=dev, generator=gen)
+            qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, words), dtype=torch.int32, device=dev, generator=gen)
             sc = (torch.rand((k // GROUP, n), device=dev, generator=gen) * 9e-3 + 1e-3).to(torch.float16)
             ws = marlin_utils.marlin_make_workspace_new(torch.device(dev))
             empty = torch.empty(0, dtype=torch.int32, device=dev)
@@ -124,6 +126,8 @@ def variants_sweep(torch, ops, gen, time_graph):
                 g_idx = (torch.arange(k, device=dev) // GROUP).to(torch.int32)
                 perm = torch.randperm(k, device=dev, generator=gen).to(torch.int32)
                 layers.append((qw, sc, empty, g_idx, perm, ws, scalar_types.uint4b8))
+            elif name == "w8a16":
+                layers.append((qw, sc * 0.0625, empty, empty, empty, ws, scalar_types.uint8b128))
             else:
                 zp = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // GROUP, n // 8), dtype=torch.int32, device=dev,
                                    generator=gen)
@@ -137,6 +141,8 @@ def variants_sweep(torch, ops, gen, time_graph):
                                 False, True, False)
             s = time_graph(torch, one, 24 if m == 1 else 6)
             nb = algorithmic_bytes(m, k, n, zeros=name == "awq", act_order=name == "act_order")
+            if name == "w8a16":
+                nb += k * n // 2                        # a byte per weight instead of half
             fl = 2 * m * k * n
             out.append({"variant": name, "m": m, "k": k, "n": n, "us": round(s * 1e6, 2),
                         "GBps": round(nb / s / 1e9, 1), "TFLOPs": round(fl / s / 1e12, 2),
