@@ -51,7 +51,25 @@ def layer_fixture(seed, k, n, g, dtype, zero_points, act_order, m):
     return out
 
 
+def layer8_fixture(seed, k, n, g, dtype, m):
+    """8-bit (uint8b128) weights: codes, the three packings, dequantised bits, GEMM."""
+    rng = np.random.default_rng(seed)
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    scales = mo.round_to_dtype(rng.uniform(1e-4, 1e-3, size=(k // g, n)).astype(np.float32), dtype)
+    marlin = mo.gptq_marlin_repack8(mo.pack_rows8(q), None, k, n)
+    w = mo.dequantize(q, scales, g, dtype, num_bits=8)
+    a = mo.make_activations(seed + 1, m, k, dtype)
+    return {"size_k": np.int64(k), "size_n": np.int64(n), "group_size": np.int64(g), "size_m": np.int64(m),
+            "q": q.astype(np.uint8), "gptq_packed": mo.pack_rows8(q), "marlin": marlin,
+            "gfx950": mo.marlin8_to_gfx950(marlin, k, n), "scales_bits": mo.to_bits16(scales, dtype),
+            "scales_marlin_bits": mo.to_bits16(mo.marlin_permute_scales(scales, k, n, g), dtype),
+            "dequant_bits": mo.to_bits16(w, dtype), "a_bits": mo.to_bits16(a, dtype),
+            "c_ref": mo.gemm_reference(a, w)}
+
+
 def main():
+    np.savez_compressed(os.path.join(HERE, "gptq8_bf16_k128_n64_g64.npz"),
+                        **layer8_fixture(104, 128, 64, 64, "bf16", 6))
     np.savez_compressed(os.path.join(HERE, "gptq_fp16_k128_n128_g64.npz"),
                         **layer_fixture(101, 128, 128, 64, "fp16", False, False, 5))
     np.savez_compressed(os.path.join(HERE, "awq_bf16_k128_n64_g32.npz"),

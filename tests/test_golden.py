@@ -111,3 +111,51 @@ def test_hip_kernels_reproduce_layer_fixture(name, dtype):
                                      m, n, k, groups, 1, 0, 1, gu.stream()))
     ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(c), f["c_ref"])
     assert ok, worst
+
+
+def test_oracle_reproduces_8bit_fixture():
+    f = load("gptq8_bf16_k128_n64_g64.npz")
+    k, n, g = int(f["size_k"]), int(f["size_n"]), int(f["group_size"])
+    q = f["q"].astype(np.int64)
+    assert np.array_equal(mo.pack_rows8(q), f["gptq_packed"])
+    assert np.array_equal(mo.gptq_marlin_repack8(f["gptq_packed"], None, k, n), f["marlin"])
+    assert np.array_equal(mo.marlin_pack8_recipe(q), f["marlin"])
+    assert np.array_equal(mo.marlin8_to_gfx950(f["marlin"], k, n), f["gfx950"])
+    scales = mo.from_bits16(f["scales_bits"], "bf16")
+    assert np.array_equal(mo.to_bits16(mo.marlin_permute_scales(scales, k, n, g), "bf16"), f["scales_marlin_bits"])
+    w = mo.dequantize(q, scales, g, "bf16", num_bits=8)
+    assert np.array_equal(mo.to_bits16(w, "bf16"), f["dequant_bits"])
+    assert np.allclose(mo.gemm_reference(mo.from_bits16(f["a_bits"], "bf16"), w), f["c_ref"], rtol=1e-6, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_hip_kernels_reproduce_8bit_fixture():
+    import torch
+
+    from sonar_amd import _lib
+    from tests import gpu_util as gu
+    f = load("gptq8_bf16_k128_n64_g64.npz")
+    k, n, g, m = int(f["size_k"]), int(f["size_n"]), int(f["group_size"]), int(f["size_m"])
+    lib = _lib.load()
+    marlin = torch.empty((k // 16, 4 * n), dtype=torch.int32, device=gu.DEV)
+    _lib.check(lib.sonar_gptq_marlin_repack(gu.ptr(gu.dev_i32(f["gptq_packed"])), None, gu.ptr(marlin), k, n, 8,
+                                            gu.stream()))
+    assert np.array_equal(marlin.cpu().numpy().view(np.uint32), U32(f["marlin"]))
+    native = torch.empty_like(marlin)
+    _lib.check(lib.sonar_marlin8_to_gfx950(gu.ptr(marlin), gu.ptr(native), k, n, gu.stream()))
+    assert np.array_equal(native.cpu().numpy().view(np.uint32).ravel(), U32(f["gfx950"].reshape(-1)))
+    scales = torch.from_numpy(f["scales_marlin_bits"].view(np.int16).copy()).to(gu.DEV).view(torch.bfloat16)
+    w = torch.empty((k, n), dtype=torch.bfloat16, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_dequant(gu.ptr(native), _lib.LAYOUT_GFX950, gu.ptr(scales), None, None, gu.ptr(w),
+                                        gu.dtype_code("bf16"), _lib.TYPE_UINT8B128, n, k, k // g, 1, gu.stream()))
+    assert np.array_equal(w.view(torch.int16).cpu().numpy().view(np.uint16), f["dequant_bits"])
+    a = torch.from_numpy(f["a_bits"].view(np.int16).copy()).to(gu.DEV).view(torch.bfloat16)
+    c = torch.empty((m, n), dtype=torch.bfloat16, device=gu.DEV)
+    ws = torch.zeros(torch.cuda.get_device_properties(0).multi_processor_count, dtype=torch.int32, device=gu.DEV)
+    scratch = torch.empty(lib.sonar_marlin_gemm_scratch_bytes(m, n, k), dtype=torch.uint8, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_gemm(gu.ptr(a), k, gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None,
+                                     gu.ptr(scales), None, None, None, gu.ptr(ws), ws.numel(), gu.ptr(scratch),
+                                     scratch.numel(), gu.dtype_code("bf16"), _lib.TYPE_UINT8B128, m, n, k, k // g,
+                                     1, 0, 1, gu.stream()))
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(c), f["c_ref"])
+    assert ok, worst
