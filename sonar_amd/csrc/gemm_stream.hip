@@ -1,5 +1,5 @@
-// Streaming W4A16 GEMM for up to 64 activation rows per launch (the
-// bandwidth-bound regime).
+// Streaming W4A16 / W8A16 GEMM for the bandwidth-bound regime: up to 64
+// activation rows per workgroup (up to 128 rows per launch of the fast kernel).
 //
 // Work decomposition.  The packed weights are a list of strips (64 output
 // columns each), every strip a contiguous run of K/32 one-KiB chunks.  The list
@@ -14,7 +14,9 @@
 // of its strip is rounded and written to C.  A partial segment is written as
 // an fp32 tile to scratch memory; a second, tiny kernel adds the (two to five)
 // partial tiles of each split strip in a fixed order and writes C.  Nothing
-// spins, nothing is atomic, and the result does not depend on timing.
+// spins, nothing is atomic, and the result does not depend on timing.  Short
+// strips (K <= 4096) on a wide matrix get one workgroup each instead, which
+// shares nothing and needs no second kernel.
 #include <cstdlib>
 
 #include "dequant.hpp"
@@ -417,8 +419,9 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
 }
 
 // ---------------------------------------------------------------------------
-// Fast kernel for M <= 16, K % 128 == 0, groups of 128 * 2^s rows (or one
-// group), no act-order.  Everything a wavefront consumes arrives in its own
+// Fast kernel for 16 rows per workgroup (several blocks of 16 rows per launch),
+// K % 128 == 0, groups of 128 * 2^s rows (or one group), 4-bit codes, no
+// act-order.  Everything a wavefront consumes arrives in its own
 // region of LDS through asynchronous global->LDS copies, so bytes in flight tie
 // up no vector registers and no register is ever read while a load into it is
 // pending: two slots for the packed weights plus scale / zero-point row of one
