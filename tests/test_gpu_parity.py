@@ -1,6 +1,8 @@
 """GPU parity: HIP kernels, called through the C ABI, against the CPU oracle.
 Integer results are compared bit for bit; GEMM outputs with the tolerance
 max|err| <= 1e-2*max|ref| and |err| <= 1e-2*max|ref| + 1e-2*|ref|."""
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -233,6 +235,40 @@ def test_act_order_with_permuted_copy_of_a(gu, dtype, m, k, n):
     gathered = layer.gemm(a, m)
     ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(fast), gu.host_f32(gathered))
     assert ok, f"max_err={max_err} max_ref={max_ref}"
+
+
+def _random_cases(count=int(os.environ.get("SONAR_RANDOM_CASES", "56"))):
+    """Seeded draws over the dispatcher's decision variables: rows around the
+    kernel boundaries, short and long strips, narrow and wide matrices, every
+    group size, zero points, act-order, bias."""
+    rng = np.random.default_rng(2024)
+    ms = [1, 2, 15, 16, 17, 31, 32, 33, 48, 64, 65, 100, 128, 129, 200, 256, 300, 520]
+    ks = [32, 64, 96, 128, 256, 384, 512, 1024, 2048, 4096]
+    ns = [64, 128, 192, 320, 1024, 4096, 4160, 8192]
+    cases = []
+    while len(cases) < count:
+        m, k, n = int(rng.choice(ms)), int(rng.choice(ks)), int(rng.choice(ns))
+        g = int(rng.choice([32, 64, 128, -1]))
+        if g != -1 and (k % g != 0 or g > k):
+            continue
+        if m * k * n > 3e9:
+            continue
+        zp = bool(rng.integers(0, 2))
+        act = (not zp) and g != -1 and k // g > 1 and bool(rng.integers(0, 3) == 0)
+        cases.append((m, k, n, g, zp, act, bool(rng.integers(0, 2)), "fp16" if rng.integers(0, 2) else "bf16"))
+    return cases
+
+
+@pytest.mark.parametrize("m,k,n,g,zp,act,bias,dtype", _random_cases())
+def test_random_shapes_against_oracle(gu, m, k, n, g, zp, act, bias, dtype):
+    layer = gu.DeviceLayer(m + k + n, k, n, g, dtype, zero_points=zp, act_order=act, bias=bias)
+    a32 = mo.make_activations(m, m, k, dtype, std=0.5)
+    a = gu.dev_bits16(a32, dtype)
+    c = layer.gemm(a, m, extra_scratch=m * k * 2 if act and m % 2 else 0)   # with and without the permuted copy
+    torch.cuda.synchronize()
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), mo.gemm_reference(a32, layer.w_ref, layer.bias32))
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+    assert int(layer.workspace.abs().sum().item()) == 0
 
 
 def _layer8(gu, seed, k, n, g, dtype, act_order=False):
