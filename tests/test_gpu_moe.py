@@ -6,6 +6,8 @@ tests/kernels/moe/test_moe.py:560-700 (experts, top-k, group sizes, act-order,
 zero points) at sizes the oracle finishes in seconds."""
 from __future__ import annotations
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -118,6 +120,35 @@ def test_moe_gemm_within_tolerance(case):
     assert np.all(np.isfinite(got))
     ok, *worst = mo.gemm_tolerance_ok(got, want)
     assert ok, worst
+
+
+def _random_moe_cases(count=int(os.environ.get("SONAR_RANDOM_CASES", "32"))):
+    """Seeded draws over tokens, experts, top_k, shapes, group sizes, block sizes
+    (8, 16, 32, 48, 64 or the reference's rule), zero points, act-order, bias."""
+    rng = np.random.default_rng(77)
+    cases = []
+    while len(cases) < count:
+        m = int(rng.choice([1, 3, 16, 17, 40, 64, 130, 300, 700]))
+        e = int(rng.choice([2, 4, 8, 16]))
+        top_k = int(rng.choice([1, 2, 4]))
+        if top_k > e:
+            continue
+        k = int(rng.choice([128, 256, 384, 512]))
+        n = int(rng.choice([64, 128, 256, 320]))
+        g = int(rng.choice([32, 64, 128, -1]))
+        if g != -1 and k % g != 0:
+            continue
+        zp = bool(rng.integers(0, 2))
+        act = (not zp) and g != -1 and k // g > 1 and bool(rng.integers(0, 4) == 0)
+        bs = rng.choice([None, 8, 16, 32, 48, 64])
+        cases.append((m, e, top_k, k, n, g, "fp16" if rng.integers(0, 2) else "bf16", zp, act,
+                      bool(rng.integers(0, 2)), None if bs is None else int(bs), bool(rng.integers(0, 2))))
+    return cases
+
+
+@pytest.mark.parametrize("case", _random_moe_cases(), ids=lambda c: "-".join(str(x) for x in c))
+def test_random_moe_cases_against_oracle(case):
+    test_moe_gemm_within_tolerance(case)
 
 
 def test_moe_skips_invalid_blocks_and_rows():
