@@ -8,12 +8,15 @@ namespace sonar {
 
 struct GemmPlan {
   bool tile;        // MFMA-tiled kernel (else the streaming kernels, in 64-row slabs)
-  int k_splits;     // workgroups per 256 x 256 tile along K (tile kernel only)
+  int k_splits;     // workgroups per split 256 x 256 tile along K (tile kernel only)
   int k_steps_per_split;
+  // With k_splits > 1: the first `whole_tiles` tiles of the tile numbering are
+  // each computed by one workgroup over the whole of K, the rest are split.
+  int64_t whole_tiles;
 };
 
 inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool async_tile) {
-  GemmPlan plan = {false, 1, 0};
+  GemmPlan plan = {false, 1, 0, 0};
   if (size_m <= 64 || size_k % 64 != 0) return plan;
   const int64_t tiles = ((size_m + 255) / 256) * ((size_n + 255) / 256);
   const int k_steps = (int)(size_k / 64);
@@ -28,19 +31,35 @@ inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool a
     if (splits > 16) splits = 16;
     if (splits < 1) splits = 1;
   }
+  // More tiles than compute units, the last round of workgroups a half or less
+  // of the chip: split the tiles of that round so that it is as wide as the
+  // others and 1 / splits as long.  Worth the partial-tile traffic (at most
+  // 64 MiB each way, about 30 us) once a tile takes about 80 us (48 K steps).
+  int64_t whole_tiles = 0;
+  if (async_tile && tiles > 256 && k_steps >= 48) {
+    const int64_t last_round = tiles % 256;
+    if (last_round != 0 && last_round <= 128) {
+      splits = (int)(256 / last_round);
+      if (splits > k_steps / 8) splits = k_steps / 8;
+      if (splits > 16) splits = 16;
+      if (splits < 2) splits = 1;
+      else whole_tiles = tiles - last_round;
+    }
+  }
   if (size_m <= 128) return plan;
   if (splits == 1 && size_m <= 512 && tiles < 64) return plan;  // slabs use every compute unit
   plan.tile = true;
   plan.k_splits = splits;
   plan.k_steps_per_split = (k_steps + splits - 1) / splits;
   plan.k_splits = (k_steps + plan.k_steps_per_split - 1) / plan.k_steps_per_split;  // no empty split
+  plan.whole_tiles = plan.k_splits > 1 ? whole_tiles : tiles;
   return plan;
 }
 
 inline size_t plan_partial_bytes(const GemmPlan& plan, int64_t size_m, int64_t size_n) {
   if (!plan.tile || plan.k_splits <= 1) return 0;
   const int64_t tiles = ((size_m + 255) / 256) * ((size_n + 255) / 256);
-  return (size_t)plan.k_splits * tiles * 256 * 1024;
+  return (size_t)plan.k_splits * (size_t)(tiles - plan.whole_tiles) * 256 * 1024;
 }
 
 }  // namespace sonar

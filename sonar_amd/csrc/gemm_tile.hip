@@ -47,9 +47,10 @@ struct TileParams {
   int chunks_per_strip;
   int tiles_m, tiles_n;
   int tile_band;               // rows of tiles per band of the tile numbering (tile_of_workgroup)
-  // split K: workgroup (tile, split) covers K steps [split * k_steps_per_split, ...) and, when
-  // k_splits > 1, leaves its fp32 tile in `partial` for tile_reduce_kernel
+  // split K (k_splits > 1): workgroup (tile, split) of a split tile covers K steps
+  // [split * k_steps_per_split, ...) and leaves its fp32 tile in `partial` for tile_reduce_kernel
   int k_splits, k_steps_per_split;
+  int whole_tiles;             // with k_splits > 1: tiles 0..whole_tiles-1 of the numbering are not split
   float4* partial;
   // grouped (mixture-of-experts) calls only
   const int32_t* sorted_ids;   // slot -> row id of C (row id / top_k of A), >= rows_total: padding
@@ -75,29 +76,52 @@ __device__ __forceinline__ uint4 load_a16(const TileParams& p, int row, int k0) 
   return v;
 }
 
-// Workgroup id -> tile.  Workgroups whose ids are congruent mod 8 run on one
-// XCD and share its L2: each XCD takes a contiguous run of tiles, rows of A
-// innermost, so the workgroups resident on it share a few panels of W.
-// Returns false for the padding ids of the last run.
-__device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile_m, int& tile_n, int& split) {
-  const int tiles = p.tiles_m * p.tiles_n;
-  const int total = tiles * p.k_splits;
-  const int per_xcd = (total + 7) / 8;
-  const int id = (blockIdx.x & 7) * per_xcd + (blockIdx.x >> 3);
-  split = id / tiles;
-  const int tile = id - split * tiles;
-  // tiles are numbered band by band (tile_band rows of tiles), inside a band
-  // column by column: with bands of 4 rows, 32 consecutive tiles are 4 panels
-  // of A x 8 panels of W
+// Tiles are numbered band by band (tile_band rows of tiles), inside a band
+// column by column: with bands of 4 rows, 32 consecutive tiles are 4 panels
+// of A x 8 panels of W.
+__device__ __forceinline__ void tile_coords(const TileParams& p, int tile, int& tile_m, int& tile_n) {
   const int band = tile / (p.tile_band * p.tiles_n);
   const int rem = tile - band * p.tile_band * p.tiles_n;
   const int rows = min(p.tile_band, p.tiles_m - band * p.tile_band);
   tile_n = rem / rows;
   tile_m = band * p.tile_band + rem - tile_n * rows;
-  return id < total;
+}
+// Tiles computed by one workgroup over the whole of K (the first ones of the numbering).
+__host__ __device__ __forceinline__ int whole_tiles(const TileParams& p) {
+  return p.k_splits > 1 ? p.whole_tiles : p.tiles_m * p.tiles_n;
 }
 
-inline int tile_grid(const TileParams& p) { return ((p.tiles_m * p.tiles_n * p.k_splits + 7) / 8) * 8; }
+// Workgroup id -> (tile, K range).  Workgroups whose ids are congruent mod 8
+// run on one XCD and share its L2: each XCD takes a contiguous run of the
+// whole tiles, rows of A innermost, so the workgroups resident on it share a
+// few panels of W, and after those a contiguous run of the (tile, split) pairs
+// of the split tiles, so that the short workgroups start last on every XCD.
+// Returns false for the padding ids of a run.
+__device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile, int& split, bool& whole_k) {
+  const int tiles = p.tiles_m * p.tiles_n;
+  const int whole = whole_tiles(p);
+  const int split_tiles = tiles - whole;
+  const int whole_per_xcd = (whole + 7) / 8;
+  const int split_per_xcd = (split_tiles * p.k_splits + 7) / 8;
+  const int xcd = blockIdx.x & 7, i = blockIdx.x >> 3;
+  whole_k = i < whole_per_xcd;
+  if (whole_k) {
+    tile = xcd * whole_per_xcd + i;
+    split = 0;
+    return tile < whole;
+  }
+  const int t = xcd * split_per_xcd + (i - whole_per_xcd);
+  if (t >= split_tiles * p.k_splits) return false;
+  split = t / split_tiles;
+  tile = whole + t - split * split_tiles;
+  return true;
+}
+
+inline int tile_grid(const TileParams& p) {
+  const int whole = whole_tiles(p);
+  const int split_work = (p.tiles_m * p.tiles_n - whole) * p.k_splits;
+  return 8 * ((whole + 7) / 8 + (split_work + 7) / 8);
+}
 
 template <typename T, bool HAS_ZP, bool HAS_PERM>
 __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const TileParams p) {
@@ -113,8 +137,10 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const Tile
   const uint32_t magic = magic_register();
   const bool grouped = p.num_groups > 1;
 
-  int tile_m, tile_n, split;
-  if (!tile_of_workgroup(p, tile_m, tile_n, split)) return;  // this kernel is launched with k_splits == 1
+  int tile, tile_m, tile_n, split;
+  bool whole_k;
+  if (!tile_of_workgroup(p, tile, split, whole_k)) return;  // this kernel is launched with k_splits == 1
+  tile_coords(p, tile, tile_m, tile_n);
   const int m0 = tile_m * kTileM;
   const int strip0 = tile_n * (kTileN / kStripN);
   const int strips_here = min(kTileN / kStripN, p.size_n / kStripN - strip0);
@@ -299,8 +325,10 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   const uint32_t magic = magic_register();
   const bool grouped = p.num_groups > 1;
 
-  int tile_m, tile_n, split;
-  if (!tile_of_workgroup(p, tile_m, tile_n, split)) return;
+  int tile, tile_m, tile_n, split;
+  bool whole_k;
+  if (!tile_of_workgroup(p, tile, split, whole_k)) return;
+  tile_coords(p, tile, tile_m, tile_n);
   // Grouped calls: row tile t is up to four consecutive 64-slot blocks of one
   // expert, listed in tile_table; rows are slots of sorted_ids.
   int first_slot = 0, tile_rows = kTileM;
@@ -394,8 +422,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     for (int mb = 0; mb < 8; ++mb) acc[nb][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
   // K steps [k_first, k_tiles) of this workgroup
-  const int k_first = split * p.k_steps_per_split;
-  const int k_tiles = min(p.size_k / kTileK, k_first + p.k_steps_per_split);
+  const int k_first = whole_k ? 0 : split * p.k_steps_per_split;
+  const int k_tiles = whole_k ? p.size_k / kTileK : min(p.size_k / kTileK, k_first + p.k_steps_per_split);
   issue(k_first, 0);
   issue(min(k_first + 1, k_tiles - 1), 1);
 
@@ -534,9 +562,11 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 #undef SONAR_TILE_READ
 
   if (!active) return;
-  if (!GROUPED && p.k_splits > 1) {
+  if (!GROUPED && !whole_k) {
     // partial tile of this K range: one 1-KiB block per accumulator tile
-    float4* dst = p.partial + ((size_t)(split * p.tiles_m * p.tiles_n + tile_n * p.tiles_m + tile_m) * 256 + wave * 32) * 64 + lane;
+    const int first_split = whole_tiles(p);
+    const int split_tiles = p.tiles_m * p.tiles_n - first_split;
+    float4* dst = p.partial + ((size_t)(split * split_tiles + tile - first_split) * 256 + wave * 32) * 64 + lane;
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
@@ -593,19 +623,21 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   }
 }
 
-// Sums the partial tiles of a split-K launch in split order, adds the bias and
-// writes C.  One wavefront per accumulator tile (16 rows x 16 columns).
+// Sums the partial tiles of the split tiles of a launch in split order, adds the
+// bias and writes C.  One wavefront per accumulator tile (16 rows x 16 columns).
 template <typename T>
 __global__ __launch_bounds__(256) void tile_reduce_kernel(const TileParams p) {
   const int lane = threadIdx.x & 63;
   const int col16 = lane & 15, kb = lane >> 4;
   const long unit = (long)blockIdx.x * 4 + (threadIdx.x >> 6);   // (tile, wavefront, accumulator tile)
-  const int tiles = p.tiles_m * p.tiles_n;
+  const int first_split = whole_tiles(p);
+  const int tiles = p.tiles_m * p.tiles_n - first_split;  // split tiles
   if (unit >= (long)tiles * 256) return;
   const int tile = (int)(unit >> 8);
   const int wave = (int)(unit >> 5) & 7;
   const int nb = (int)(unit & 31) >> 3, mb = (int)unit & 7;
-  const int tile_n = tile / p.tiles_m, tile_m = tile - tile_n * p.tiles_m;
+  int tile_m, tile_n;
+  tile_coords(p, first_split + tile, tile_m, tile_n);
   const int strip = tile_n * (kTileN / kStripN) + (wave & 3);
   const int m = tile_m * kTileM + 128 * (wave >> 2) + 16 * mb + col16;
   if (strip * kStripN >= p.size_n) return;
@@ -727,6 +759,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   p.tile_band = 4;
   p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);
   p.k_splits = 1;
+  p.whole_tiles = 0;  // read only with k_splits > 1
   p.k_steps_per_split = (int)(size_k / kTileK);
   p.partial = nullptr;
   p.sorted_ids = nullptr;
@@ -742,6 +775,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     if (plan.k_splits > 1 && partial != nullptr && partial_bytes >= plan_partial_bytes(plan, size_m, size_n)) {
       p.k_splits = plan.k_splits;
       p.k_steps_per_split = plan.k_steps_per_split;
+      p.whole_tiles = (int)plan.whole_tiles;
       p.partial = static_cast<float4*>(partial);
     }
     if (dtype == SONAR_DTYPE_F16)
@@ -751,7 +785,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     if (rc) return rc;
     if (int rc2 = launch_status("marlin_tile_async_kernel")) return rc2;
     if (p.k_splits > 1) {
-      const int blocks = p.tiles_m * p.tiles_n * 64;
+      const int blocks = (p.tiles_m * p.tiles_n - p.whole_tiles) * 64;
       if (dtype == SONAR_DTYPE_F16) tile_reduce_kernel<_Float16><<<blocks, 256, 0, st>>>(p);
       else tile_reduce_kernel<__bf16><<<blocks, 256, 0, st>>>(p);
       return launch_status("tile_reduce_kernel");
@@ -808,6 +842,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.tiles_m = max_tiles;
   p.tile_band = max_tiles > 0 ? max_tiles : 1;  // row tiles of different experts share no panel of W: whole columns
   p.k_splits = 1;
+  p.whole_tiles = 0;  // read only with k_splits > 1
   p.k_steps_per_split = (int)(size_k / kTileK);
   p.partial = nullptr;
   p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);

@@ -203,6 +203,8 @@ TILE_CASES = [
     (129, 14336, 4096, 128, False, False, False),
     (600, 1024, 768, 64, True, False, True),
     (520, 512, 192, 32, True, False, False),         # groups of 32 rows: the register-staged tile kernel
+    # 9 x 29 = 261 tiles: 256 whole ones, then the last 5 split six ways along K
+    (2200, 3072, 7360, 128, True, False, True),
 ]
 
 
@@ -415,10 +417,12 @@ def test_act_order_shard_without_whole_groups(gu, dtype, m):
 
 
 @pytest.mark.parametrize("dtype,m,k,n", [("fp16", 4096, 4096, 4096), ("bf16", 8192, 4096, 6144),
-                                          ("fp16", 1024, 14336, 4096), ("fp16", 256, 4096, 28672)])
+                                          ("fp16", 1024, 14336, 4096), ("fp16", 256, 4096, 28672),
+                                          ("fp16", 4096, 4096, 6144)])   # 384 tiles: the last 128 split in two
 def test_full_size_tile_gemm_agrees_with_streamed_rows(gu, dtype, m, k, n):
     """At the benchmark's prefill sizes the CPU oracle is too slow, so the tile
-    kernels (with and without split K) are checked through a size-independent
+    kernels (without split K, with every tile split, with the last round of
+    tiles split) are checked through a size-independent
     property: any subset of rows of A gives the same rows of C, and 16 rows go
     through the decode kernel, which is checked against the oracle elsewhere."""
     layer = gu.DeviceLayer(5, k, n, 128, dtype)
