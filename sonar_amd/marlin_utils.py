@@ -1,7 +1,8 @@
 """Host-side tensor preparation for the Marlin ops: the counterpart of the
 reference's aphrodite/model_executor/layers/quantization/utils/marlin_utils.py
-(:30-40 constants, :206-281 padding, :362-505 workspace / scale / zero-point /
-bias layouts, :636-700 apply_gptq_marlin_linear) and of pack_cols / unpack_cols
+(:30-40 constants, :111-203 and :284-359 support checks, :206-281 padding,
+:362-559 workspace / scale / zero-point / bias layouts, :636-700
+apply_gptq_marlin_linear) and of pack_cols / unpack_cols
 in quant_utils.py:749-803.  Same names, arguments and results; implemented
 with torch index ops so tensors stay on their device."""
 from __future__ import annotations
@@ -48,6 +49,78 @@ def check_marlin_supports_shape(output_size_per_partition: int, input_size_per_p
         return False, (f"Weight input_size_per_partition = {input_size_per_partition} is not "
                        f"divisible by group_size = {group_size}.")
     return True, None
+
+
+def _check_marlin_supported(quant_type: ScalarType, group_size: int | None, has_zp: bool):
+    supported = query_marlin_supported_quant_types(has_zp, True)
+    if quant_type not in supported:
+        return False, (f"Marlin does not support weight_bits = {quant_type}. Only types = {supported} "
+                       f"are supported (for group_size = {group_size}, zp = {has_zp}).")
+    if group_size is None or group_size not in MARLIN_SUPPORTED_GROUP_SIZES:
+        return False, (f"Marlin does not support group_size = {group_size}. "
+                       f"Only group_sizes = {MARLIN_SUPPORTED_GROUP_SIZES} are supported.")
+    return True, None
+
+
+def check_marlin_supported(quant_type: ScalarType, group_size: int, has_zp: bool = False,
+                           device_capability: int | None = None) -> bool:
+    """marlin_utils.py:142-149.  `device_capability` is accepted for the
+    reference's callers and ignored: there is one target, gfx950."""
+    return _check_marlin_supported(quant_type, group_size, has_zp)[0]
+
+
+def verify_marlin_supported(quant_type: ScalarType, group_size: int, has_zp: bool = False) -> None:
+    ok, why = _check_marlin_supported(quant_type, group_size, has_zp)
+    if not ok:
+        raise ValueError(why)
+
+
+def verify_marlin_supports_shape(output_size_per_partition: int, input_size_per_partition: int,
+                                 input_size: int, group_size: int) -> None:
+    """Raises ValueError where check_marlin_supports_shape returns False
+    (marlin_utils.py:159-190)."""
+    ok, why = check_marlin_supports_shape(output_size_per_partition, input_size_per_partition,
+                                          input_size, group_size)
+    if not ok:
+        raise ValueError(why)
+
+
+def check_marlin_supports_layer(layer, group_size: int, allow_tile_padding: bool = False) -> bool:
+    """marlin_utils.py:284-300: `layer` has output_size / input_size and, when
+    sharded, the *_per_partition sizes.  With tile padding only a group that
+    straddles the shard boundary stays unsupported."""
+    out_part = getattr(layer, "output_size_per_partition", None) or layer.output_size
+    in_part = getattr(layer, "input_size_per_partition", None) or layer.input_size
+    if allow_tile_padding:
+        return group_size == -1 or group_size >= layer.input_size or in_part % group_size == 0
+    return check_marlin_supports_shape(out_part, in_part, layer.input_size, group_size)[0]
+
+
+def marlin_moe_padded_intermediate(intermediate_size: int, group_size: int = -1) -> int:
+    """Smallest intermediate size >= the given one that the grouped op takes
+    (a multiple of 64 and of the group size; marlin_utils.py:303-321).  The
+    padding is zero scales, so padded channels contribute nothing."""
+    return round_up(intermediate_size, math.lcm(64, group_size if group_size > 0 else 1))
+
+
+def check_moe_marlin_supports_layer(layer, group_size: int, allow_tile_padding: bool = False) -> bool:
+    """Shape rule of marlin_utils.py:324-350 (hidden % 128, intermediate a
+    multiple of max(64, group), no router weight on the input).  The reference
+    answers False on ROCm before looking at the shape; with this library loaded
+    that early return is the line a maintainer removes."""
+    hidden = layer.hidden_size
+    inter = layer.moe_config.intermediate_size_per_partition_unpadded
+    if allow_tile_padding:
+        shape_ok = hidden % 128 == 0 and (group_size <= 0 or inter % group_size == 0)
+    else:
+        shape_ok = hidden % 128 == 0 and inter % max(64, group_size) == 0
+    return shape_ok and group_size in (-1, 32, 64, 128) and not layer.apply_router_weight_on_input
+
+
+def marlin_moe_intermediate_size(w1_packed: torch.Tensor, w2_packed: torch.Tensor) -> int:
+    """Intermediate size from the packed down-projection [E, K / 16, ...]
+    (marlin_utils.py:353-359)."""
+    return w2_packed.size(1) * GPTQ_MARLIN_TILE
 
 
 # ---------------------------------------------------------------- packing
@@ -216,6 +289,18 @@ def moe_awq_to_marlin_zero_points(q_zp_packed: torch.Tensor, size_k: int, size_n
     for e in range(q_zp_packed.shape[0]):
         output[e] = awq_to_marlin_zero_points(q_zp_packed[e], size_k, size_n, num_bits, is_a_8bit)
     return output
+
+
+def moe_packed_to_marlin_zero_points(q_zp_packed: torch.Tensor, size_k: int, size_n: int, num_bits: int,
+                                     is_a_8bit: bool = False) -> torch.Tensor:
+    """Per-expert zero points packed along columns in plain order (the
+    compressed-tensors format, no AWQ interleave) to the op's layout
+    (marlin_utils.py:538-559)."""
+    out = torch.empty_like(q_zp_packed)
+    for e in range(q_zp_packed.shape[0]):
+        out[e] = marlin_zero_points(unpack_cols(q_zp_packed[e], num_bits, size_k, size_n), size_k, size_n,
+                                    num_bits, is_a_8bit)
+    return out
 
 
 def should_use_atomic_add_reduce(m: int, n: int, k: int, device: torch.device, dtype: torch.dtype) -> bool:

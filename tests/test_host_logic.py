@@ -275,3 +275,66 @@ def test_awq_checkpoint_conversion_matches_gptq_packing():
     assert np.array_equal(layer.qzeros.numpy(), mo.pack_rows(np.ascontiguousarray(zp.T)))
     # and the converted zero points unpack to the codes again (pack_cols form, transposed)
     assert np.array_equal(mo.unpack_cols(np.ascontiguousarray(layer.qzeros.numpy().T)), zp)
+
+
+def test_support_checks_follow_the_reference_rules():
+    """marlin_utils.py:111-203, 284-359 of the reference: type / group-size
+    gate, shape gate (N % 64, K % 128, groups dividing the shard), layer gates
+    and the MoE intermediate-size helpers, on values worked out by hand."""
+    from types import SimpleNamespace as NS
+    from sonar_amd import marlin_utils as mu
+    from sonar_amd.scalar_type import scalar_types as st
+    assert mu.check_marlin_supported(st.uint4b8, 128)
+    assert mu.check_marlin_supported(st.uint8b128, -1)
+    assert mu.check_marlin_supported(st.uint4, 64, has_zp=True)
+    assert not mu.check_marlin_supported(st.uint4, 64, has_zp=False)
+    assert not mu.check_marlin_supported(st.uint4b8, 100)
+    assert not mu.check_marlin_supported(st.uint8, 128, has_zp=True)   # 8-bit codes with zero points: not built
+    mu.verify_marlin_supported(st.uint4b8, 32)
+    with pytest.raises(ValueError, match="group_size = 256"):
+        mu.verify_marlin_supported(st.uint4b8, 256)
+    with pytest.raises(ValueError, match="weight_bits"):
+        mu.verify_marlin_supported(st.uint8, 128, has_zp=True)
+    mu.verify_marlin_supports_shape(4096, 4096, 4096, 128)
+    with pytest.raises(ValueError, match="min_thread_n"):
+        mu.verify_marlin_supports_shape(4000, 4096, 4096, 128)
+    with pytest.raises(ValueError, match="min_thread_k"):
+        mu.verify_marlin_supports_shape(4096, 4160, 8320, 128)
+    # a row-parallel shard of 1408 rows (11 groups of 128) passes, one of 1344 rows does not
+    layer = NS(output_size=4096, input_size=5632, output_size_per_partition=4096, input_size_per_partition=1408)
+    assert mu.check_marlin_supports_layer(layer, 128)
+    layer.input_size_per_partition = 1344
+    assert not mu.check_marlin_supports_layer(layer, 128)
+    assert not mu.check_marlin_supports_layer(layer, 128, allow_tile_padding=True)   # a group straddles the shard
+    assert mu.check_marlin_supports_layer(layer, 64, allow_tile_padding=True)
+    assert mu.check_marlin_supports_layer(layer, -1, allow_tile_padding=True)
+    # MoE: lcm(64, group) granularity
+    assert mu.marlin_moe_padded_intermediate(1408, 128) == 1408
+    assert mu.marlin_moe_padded_intermediate(1000, 128) == 1024
+    assert mu.marlin_moe_padded_intermediate(1000, -1) == 1024
+    assert mu.marlin_moe_padded_intermediate(100, 32) == 128
+    moe = NS(hidden_size=2048, apply_router_weight_on_input=False,
+             moe_config=NS(intermediate_size_per_partition_unpadded=1408))
+    assert mu.check_moe_marlin_supports_layer(moe, 128)
+    assert mu.check_moe_marlin_supports_layer(moe, 64)
+    assert not mu.check_moe_marlin_supports_layer(moe, 256)
+    moe.moe_config.intermediate_size_per_partition_unpadded = 1376      # 43 * 32
+    assert not mu.check_moe_marlin_supports_layer(moe, 32)
+    assert mu.check_moe_marlin_supports_layer(moe, 32, allow_tile_padding=True)
+    moe.apply_router_weight_on_input = True
+    assert not mu.check_moe_marlin_supports_layer(moe, 32, allow_tile_padding=True)
+    w2 = torch.zeros((4, 1408 // 16, 2048 * 2), dtype=torch.int32)
+    assert mu.marlin_moe_intermediate_size(None, w2) == 1408
+
+
+def test_moe_packed_zero_points_match_oracle():
+    """Zero points packed eight to a word along the columns, in plain order,
+    per expert: unpack, then the op's layout (marlin_utils.py:538-559)."""
+    from sonar_amd import marlin_utils as mu
+    rng = np.random.default_rng(12)
+    experts, groups, n = 3, 4, 128
+    zp = rng.integers(0, 16, size=(experts, groups, n)).astype(np.int32)
+    packed = np.stack([mo.pack_cols(zp[e]) for e in range(experts)])
+    got = mu.moe_packed_to_marlin_zero_points(torch.from_numpy(packed.view(np.int32)), groups, n, 4)
+    want = np.stack([mo.marlin_zero_points(zp[e], groups, n) for e in range(experts)])
+    assert np.array_equal(got.numpy().view(np.uint32), want.view(np.uint32))
