@@ -252,7 +252,7 @@ def _moe_layer(seed, e, hidden, inter, g, dtype, zp):
     return pack(w13, hidden, 2 * inter), pack(w2, inter, hidden)
 
 
-def _moe_reference(x32, ref13, ref2, topk_ids, topk_w, dtype):
+def _moe_reference(x32, ref13, ref2, topk_ids, topk_w, dtype, bias13=None, bias2=None):
     """torch_experts restated (tests/kernels/utils.py:817-931): per routed
     slot silu(x W_gate) * (x W_up) -> W_down, weighted sum over the slots."""
     m, hidden = x32.shape
@@ -261,10 +261,12 @@ def _moe_reference(x32, ref13, ref2, topk_ids, topk_w, dtype):
     for t in range(m):
         for j in range(topk_ids.shape[1]):
             ex = int(topk_ids[t, j])
-            h = mo.round_to_dtype(x32[t:t + 1] @ ref13[ex], dtype)
+            h = x32[t:t + 1] @ ref13[ex]
+            h = mo.round_to_dtype(h if bias13 is None else h + bias13[ex][None, :], dtype)
             gate, up = h[:, :inter], h[:, inter:]
             act = mo.round_to_dtype(mo.round_to_dtype(gate / (1.0 + np.exp(-gate)), dtype) * up, dtype)
-            y = mo.round_to_dtype(act @ ref2[ex], dtype)
+            y = act @ ref2[ex]
+            y = mo.round_to_dtype(y if bias2 is None else y + bias2[ex][None, :], dtype)
             out[t] += topk_w[t, j] * y[0]
     return out
 
@@ -296,6 +298,73 @@ def test_fused_marlin_moe_against_per_token_reference(cfg):
     got = gu.host_f32(y)
     max_ref = np.abs(want).max()
     # two chained GEMMs and three roundings per slot: 2x the single-GEMM bound
+    assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)
+
+
+def _route(m, e, topk, seed):
+    rng = np.random.default_rng(seed)
+    logits = rng.standard_normal((m, e)).astype(np.float32)
+    prob = np.exp(logits - logits.max(1, keepdims=True))
+    prob /= prob.sum(1, keepdims=True)
+    ids = np.argsort(-prob, axis=1, kind="stable")[:, :topk].astype(np.int32)
+    return ids, np.take_along_axis(prob, ids, axis=1).astype(np.float32)
+
+
+@pytest.mark.parametrize("cfg", [
+    # m, experts, topk, hidden, intermediate, group, dtype, format, act_order, bias
+    (5, 4, 2, 256, 128, 128, "fp16", "gptq", False, False),
+    (70, 4, 2, 256, 256, 64, "bf16", "gptq", True, True),
+    (33, 8, 2, 128, 128, 128, "bf16", "gptq_zp", False, False),
+    (40, 4, 2, 256, 128, 128, "fp16", "awq", False, True),
+    (9, 4, 2, 256, 96, 32, "fp16", "gptq", False, True),      # intermediate size padded 96 -> 128
+    (9, 4, 2, 128, 160, 32, "bf16", "awq", False, False),     # 160 -> 192
+], ids=str)
+def test_moe_checkpoint_tensors_through_weight_processing(cfg):
+    """Stacked expert tensors as a GPTQ / AWQ checkpoint holds them ->
+    process_*_moe_weights -> fused_marlin_moe, against the per-token reference
+    on the weights dequantised from the same checkpoint tensors."""
+    from sonar_amd import moe_weights as mw
+    from sonar_amd.fused_moe import fused_marlin_moe
+    from sonar_amd.scalar_type import scalar_types
+    m, e, topk, hidden, inter, g, dtype, fmt, act, bias = cfg
+    zp = fmt != "gptq"
+    rng = np.random.default_rng(hidden + inter)
+
+    def expert_set(seed, k, n):
+        layers = [mo.make_layer(seed + i, k, n, g, dtype, zero_points=zp, act_order=act) for i in range(e)]
+        ref = [mo.dequantize(l["q"], l["scales"], g, dtype, zeros=l.get("zeros"), g_idx=l.get("g_idx"))
+               for l in layers]
+        if fmt == "awq":
+            qw = torch.stack([gu.dev_i32(mo.awq_pack(l["q"])) for l in layers])
+            qz = torch.stack([gu.dev_i32(mo.awq_pack(l["zeros"])) for l in layers])
+        else:
+            qw = torch.stack([gu.dev_i32(mo.gptq_pack(l["q"])) for l in layers])
+            qz = torch.stack([gu.dev_i32(mo.pack_cols(l["zeros"])) for l in layers]) if zp else None
+        sc = torch.stack([gu.dev_bits16(l["scales"], dtype) for l in layers])
+        gi = torch.stack([gu.dev_i32(l["g_idx"]) for l in layers]) if act else None
+        b32 = mo.round_to_dtype(rng.standard_normal((e, n)).astype(np.float32), dtype) if bias else None
+        return qw, qz, sc, gi, ref, b32
+
+    qw13, qz13, s13, gi13, ref13, b13 = expert_set(300, hidden, 2 * inter)
+    qw2, qz2, s2, gi2, ref2, b2 = expert_set(400, inter, hidden)
+    dev_bias = lambda b: None if b is None else gu.dev_bits16(b, dtype)
+    if fmt == "awq":
+        w = mw.process_awq_moe_weights(inter, 4, g, qw13, qw2, s13, s2, qz13, qz2, dev_bias(b13), dev_bias(b2))
+    else:
+        w = mw.process_gptq_moe_weights(inter, 4, g, act, qw13, qw2, s13, s2, gi13, gi2, qz13, qz2,
+                                        dev_bias(b13), dev_bias(b2))
+    assert w.intermediate_size == mw.marlin_moe_padded_intermediate(inter, g)
+    topk_ids, topk_w = _route(m, e, topk, m)
+    x32 = mo.round_to_dtype(0.5 * mo.make_activations(m, m, hidden, dtype), dtype)
+    qtype = scalar_types.uint4 if zp else scalar_types.uint4b8
+    y = fused_marlin_moe(gu.dev_bits16(x32, dtype), w.w1, w.w2, w.bias1, w.bias2, w.w1_scale, w.w2_scale,
+                         torch.from_numpy(topk_w).to(gu.DEV), torch.from_numpy(topk_ids).to(gu.DEV), qtype.id,
+                         g_idx1=w.g_idx1, g_idx2=w.g_idx2, sort_indices1=w.sort_indices1,
+                         sort_indices2=w.sort_indices2, w1_zeros=w.w1_zeros, w2_zeros=w.w2_zeros)
+    torch.cuda.synchronize()
+    want = _moe_reference(x32, ref13, ref2, topk_ids, topk_w, dtype, b13, b2)
+    got = gu.host_f32(y)
+    max_ref = np.abs(want).max()
     assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)
 
 
