@@ -64,6 +64,23 @@ class MPLinearLayerConfig:
     has_g_idx: bool
 
 
+def _input_major(x: torch.Tensor, rows: int, cols: int) -> torch.Tensor:
+    """A weight or scale tensor with the input (K) dimension first.  The
+    reference's parameters carry `input_dim` / `output_dim` and are permuted by
+    `permute_param_layout_` (marlin.py:120-135): compressed-tensors checkpoints
+    hold `weight_packed` as (N, K / pack) and `weight_scale` as (N, groups).
+    Here the attributes are honoured when present, else the layout is read off
+    the shape, (rows, cols) winning when both fit."""
+    input_dim = getattr(x, "input_dim", None)
+    output_dim = getattr(x, "output_dim", None)
+    if input_dim == 1 or (input_dim is None and output_dim == 0 and x.shape != (rows, cols)):
+        x = x.t()
+    elif input_dim is None and output_dim is None and x.shape != (rows, cols) and x.shape == (cols, rows):
+        x = x.t()
+    assert x.shape == (rows, cols), f"expected {(rows, cols)} or its transpose, got {tuple(x.shape)}"
+    return x
+
+
 class MarlinLinearKernel:
     def __init__(self, c: MPLinearLayerConfig, w_q_param_name: str = "qweight",
                  w_s_param_name: str = "scales", w_zp_param_name: str | None = "qzeros",
@@ -131,12 +148,14 @@ class MarlinLinearKernel:
         else:
             setattr(layer, self.w_zp_name, marlin_make_empty_g_idx(device))
 
-        w_q = getattr(layer, self.w_q_name)
+        pack = 32 // c.weight_type.size_bits
+        w_q = _input_major(getattr(layer, self.w_q_name), size_k // pack, size_n)
         setattr(layer, self.w_q_name, ops.gptq_marlin_repack(
             marlin_pad_qweight(w_q.contiguous(), size_n, size_k, padded_n, padded_k),
             perm=layer.g_idx_sort_indices, size_k=padded_k, size_n=padded_n,
             num_bits=c.weight_type.size_bits, is_a_8bit=False))
         w_s = getattr(layer, self.w_s_name)
+        w_s = _input_major(w_s, w_s.numel() // size_n, size_n)
         setattr(layer, self.w_s_name, marlin_permute_scales(
             marlin_pad_scales(w_s.contiguous(), size_n, size_k, padded_n, padded_k, c.group_size),
             size_k=padded_k, size_n=padded_n, group_size=c.group_size))

@@ -113,6 +113,10 @@ def test_marlin_gemm_op_rejects_like_the_reference():
     (256, 128, 128, "bf16", True, False, False, (7,)),
     (512, 128, 128, "fp16", False, True, True, (9,)),
     (136, 72, 8 * 17, "fp16", False, False, False, (4,)),     # padded N and K (one group)
+    # compressed-tensors layout: weight_packed (N, K/8), weight_scale (N, groups), zero points (N/8, groups)
+    (512, 192, 128, "bf16", False, False, False, (6,), "ct"),
+    (256, 128, 64, "fp16", True, False, True, (3,), "ct"),
+    (512, 128, 128, "fp16", False, True, False, (20,), "ct"),
 ], ids=str)
 def test_marlin_linear_kernel_round_trip(cfg):
     """Checkpoint-format tensors -> process_weights_after_loading -> apply_weights
@@ -120,7 +124,8 @@ def test_marlin_linear_kernel_round_trip(cfg):
     from sonar_amd.marlin_linear import MarlinLinearKernel, MPLinearLayerConfig
     from sonar_amd.marlin_utils import pack_cols
     from sonar_amd.scalar_type import scalar_types
-    k, n, g, dtype, zp, act, bias, batch = cfg
+    k, n, g, dtype, zp, act, bias, batch = cfg[:8]
+    ct = len(cfg) > 8
     gs = k if g == -1 or g >= k else g
     layer_np = mo.make_layer(11, k, n, gs, dtype, zero_points=zp, act_order=act)
     w_ref = mo.dequantize(layer_np["q"], layer_np["scales"], gs, dtype, zeros=layer_np.get("zeros"),
@@ -134,6 +139,11 @@ def test_marlin_linear_kernel_round_trip(cfg):
                                  layer_np["groups"], n)
     if act:
         layer.g_idx = gu.dev_i32(layer_np["g_idx"])
+    if ct:
+        layer.qweight = layer.qweight.t().contiguous()
+        layer.scales = layer.scales.t().contiguous()
+        if zp:
+            layer.qzeros = layer.qzeros.t().contiguous()
     bias32 = None
     if bias:
         bias32 = mo.round_to_dtype(np.random.default_rng(4).standard_normal(n).astype(np.float32), dtype)
