@@ -149,18 +149,19 @@ __device__ __forceinline__ void finish_segment(const StreamParams& p, int strip,
 }
 
 // The same for one 16-column block (j) of a 16-row tile, held by one wavefront.
-// `part` is the workgroup's index in the partition and `slab` its block of 16
-// rows (fast kernel: several blocks of rows share one launch; the scratch slot
-// of a part holds one partial tile per block of rows).
+// `c_block` is row 0 of the tile in C and `rows` the rows of it that exist;
+// `part` is the workgroup's index in the partition and `slab` the tile's block
+// of 16 rows (fast kernel: several blocks of rows share one launch; the scratch
+// slot of a part holds one partial tile per block of rows).
 template <typename T>
-__device__ __forceinline__ void finish_block(const StreamParams& p, int part, int slab, int strip, int seg_begin,
-                                             int seg_end, int lane, int j, floatx4_t v) {
+__device__ __forceinline__ void finish_block(const StreamParams& p, uint16_t* c_block, int rows, int part, int slab,
+                                             int strip, int seg_begin, int seg_end, int lane, int j, floatx4_t v) {
   const int strip_first = strip * p.units_per_strip;
   const int strip_end = strip_first + p.units_per_strip;
   if (seg_begin == strip_first && seg_end == strip_end) {
     const int m = lane & 15;
     const int nl = 16 * j + 4 * (lane >> 4);
-    if (m < p.size_m) {
+    if (m < rows) {
       float b[4] = {0.f, 0.f, 0.f, 0.f};
       if (p.bias) {
 #pragma unroll
@@ -170,7 +171,7 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, int part, in
       uint2 o;
       o.x = (uint32_t)Dq<T>::from_float(v.x + b[0]) | ((uint32_t)Dq<T>::from_float(v.y + b[1]) << 16);
       o.y = (uint32_t)Dq<T>::from_float(v.z + b[2]) | ((uint32_t)Dq<T>::from_float(v.w + b[3]) << 16);
-      *reinterpret_cast<uint2*>(p.c + (long)m * p.size_n + strip * kStripN + nl) = o;
+      *reinterpret_cast<uint2*>(c_block + (long)m * p.size_n + strip * kStripN + nl) = o;
     }
     return;
   }
@@ -437,21 +438,28 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
 constexpr int kSlotS = 4096;       // inside a weight slot, after 4 chunks x 1 KiB: 64 scales, 8 zero-point words
 constexpr int kSlotBytes = 4096 + 256;
 constexpr int kWaveA = 2 * kSlotBytes;            // the activation slot follows the two weight slots
-constexpr int kWaveLds = 2 * kSlotBytes + 4096;   // LDS bytes per wavefront
+// LDS bytes per wavefront: the activation slot holds 4 KiB per block of 16 rows
+constexpr int wave_lds(int mb) { return 2 * kSlotBytes + 4096 * mb; }
+// Tiles (16 x 16 fp32, 1 KiB) a wavefront parks per pass of the cross-wavefront
+// sum: all four of its one block of rows, or two of the eight of two blocks
+// (four passes), which keeps 8 wavefronts with two blocks inside 160 KiB.
+constexpr int park_tiles(int mb) { return mb == 1 ? 4 : 2; }
 constexpr int kWeightCopies = 5;   // asynchronous copies per unit: 4 weight chunks + 1 scale row
 // A workgroup of the fast kernel has 8 wavefronts (one workgroup per compute
 // unit), or 4 (two per compute unit: a grid with more workgroups than compute
 // units then runs them side by side instead of one after the other).
-constexpr int fast_lds_bytes(int waves) { return waves * kWaveLds + waves * 4 * 64 * 16; }
+constexpr int fast_lds_bytes(int waves, int mb) { return waves * (wave_lds(mb) + park_tiles(mb) * 1024); }
 
+template <int MB>
 struct FastLane {
-  uint32_t a_off[2];    // byte offset of the 16 bytes this lane copies from rows 0..7 / 8..15 of a 64-column slice of A
+  uint32_t a_off[2 * MB];  // byte offset of the 16 bytes this lane copies from rows 8h..8h+7 of a 64-column slice of A
   const char* s_ptr;    // this lane's dword of the scale / zero-point row of (group 0, strip 0)
   long s_group_stride;  // bytes between groups for s_ptr
   int s_strip_stride;   // bytes between strips for s_ptr
 };
 
-__device__ __forceinline__ void copy_weights(const StreamParams& p, const FastLane& fl, int strip, int unit,
+template <int MB>
+__device__ __forceinline__ void copy_weights(const StreamParams& p, const FastLane<MB>& fl, int strip, int unit,
                                              char* slot, int lane, int unit_group_shift) {
   const uint4* gq = p.b + (size_t)(unsigned)(strip * p.chunks_per_strip + unit * 4) * 64 + lane;
   lds_void_t* lq = (lds_void_t*)slot;
@@ -464,20 +472,26 @@ __device__ __forceinline__ void copy_weights(const StreamParams& p, const FastLa
   __builtin_amdgcn_global_load_lds((glb_void_t*)gs, (lds_void_t*)(slot + kSlotS), 4, 0, 0);
 }
 
-// The 16 x 128 slice of A of one unit, as four regions of 1 KiB: region
+// The 16 x 128 slice of A of one unit and block of 16 rows, as four regions of
+// 1 KiB (a second block of rows follows 4 KiB later): region
 // 2 * half + h holds rows 8h..8h+7, 128 bytes (64 columns) each.  One copy fills
 // one region; its lanes 8r..8r+7 fetch the eight 16-byte pieces of one
 // 128-byte line of row r, so a copy touches 8 whole lines (16 rows x 64 bytes per
 // copy, the operand shape, moves a third of the bytes per cycle).  Piece q of
 // row r sits at 16-byte slot q ^ (r % 8) of the row, which keeps the operand
 // reads (16 rows, one piece each) off each other's banks.
-__device__ __forceinline__ void copy_activations(const StreamParams& p, const FastLane& fl, int unit,
+template <int MB>
+__device__ __forceinline__ void copy_activations(const StreamParams& p, const FastLane<MB>& fl, int unit,
                                                  char* slot) {
   const char* ga = reinterpret_cast<const char*>(p.a) + (long)unit * (4 * kChunkK * 2);
-  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + fl.a_off[0]), (lds_void_t*)(slot), 16, 0, 0);
-  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + fl.a_off[1]), (lds_void_t*)(slot + 1024), 16, 0, 0);
-  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 128 + fl.a_off[0]), (lds_void_t*)(slot + 2048), 16, 0, 0);
-  __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 128 + fl.a_off[1]), (lds_void_t*)(slot + 3072), 16, 0, 0);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    char* s = slot + 4096 * mb;
+    __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + fl.a_off[2 * mb]), (lds_void_t*)(s), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + fl.a_off[2 * mb + 1]), (lds_void_t*)(s + 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 128 + fl.a_off[2 * mb]), (lds_void_t*)(s + 2048), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 128 + fl.a_off[2 * mb + 1]), (lds_void_t*)(s + 3072), 16, 0, 0);
+  }
 }
 
 struct UnitCursor {
@@ -565,10 +579,27 @@ __device__ __forceinline__ u32x4_t raw_operand(uint32_t q, uint32_t magic) {
       : "v"(q_at), "v"(a_at), "v"(z_at), "v"(s_at), "v"(a_at ^ 64u)                                \
       : "memory")
 
-template <typename T, bool HAS_ZP, int kFastWaves>
+// The activation operands of a second block of 16 rows (4 KiB after the first).
+#define SONAR_UNIT_READS_ROWS2(B0, B1, B2, B3)                                                      \
+  asm volatile(                                                                                    \
+      "ds_read_b128 %0, %4 offset:4096\n\t"                                                        \
+      "ds_read_b128 %1, %5 offset:4096\n\t"                                                        \
+      "ds_read_b128 %2, %4 offset:6144\n\t"                                                        \
+      "ds_read_b128 %3, %5 offset:6144\n\t"                                                        \
+      "s_waitcnt lgkmcnt(0)"                                                                       \
+      : "=&v"(B0), "=&v"(B1), "=&v"(B2), "=&v"(B3)                                                 \
+      : "v"(a_at), "v"(a_at ^ 64u)                                                                 \
+      : "memory")
+
+// MB blocks of 16 rows per workgroup (1 or 2): the weights of a unit are pulled
+// out of LDS and turned into operands once and multiplied with every block.
+template <typename T, bool HAS_ZP, int kFastWaves, int MB>
 __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams params,
                                                                              const int unit_group_shift) {
   typedef typename Dq<T>::vec8 vec8;
+  constexpr int kWaveLds = wave_lds(MB);
+  constexpr int kPark = park_tiles(MB);       // tiles per wavefront and pass of the cross-wavefront sum
+  constexpr int kPasses = 4 * MB / kPark;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
   // The slabs of one part have ids congruent mod 8 (grid_parts is a multiple of
   // 8 when there are several), so they run on one XCD and the second to ask
@@ -577,9 +608,9 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   const int part = blockIdx.x % p.grid_parts;
   const int slab = blockIdx.x / p.grid_parts;
   if (part >= p.parts) return;
-  p.a += (long)slab * 16 * p.lda;
-  p.c += (long)slab * 16 * p.size_n;
-  p.size_m = min(16, p.size_m - 16 * slab);
+  p.a += (long)slab * (16 * MB) * p.lda;
+  p.c += (long)slab * (16 * MB) * p.size_n;
+  p.size_m = min(16 * MB, p.size_m - 16 * MB * slab);
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col16 = lane & 15;
@@ -591,10 +622,10 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   const int u_end = range_begin(part + 1, p.total_units, p.parts);
   const bool grouped = p.num_groups > 1;
 
-  FastLane fl;
+  FastLane<MB> fl;
   {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
+    for (int h = 0; h < 2 * MB; ++h) {
       const int r = 8 * h + (lane >> 3);
       const int row = r < p.size_m ? r : p.size_m - 1;  // rows past M are never stored
       fl.a_off[h] = (uint32_t)((long)row * p.lda * 2 + 16 * ((lane & 7) ^ (lane >> 3)));
@@ -612,7 +643,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   // Operand lane (k group q4 = lane / 16, row col16) of chunk cc of a unit reads
   // piece 4 (cc % 2) + q4 of row col16 in region 2 (cc / 2) + col16 / 8 of the
   // activation slot: a_at for chunk 0, a_at ^ 64 for chunk 1, both + 2048 for
-  // chunks 2 and 3.
+  // chunks 2 and 3 (+ 4096 for the second block of rows).
   const uint32_t a_at = ring_lds + kWaveA + (col16 >> 3) * 1024 + (col16 & 7) * 128 +
                         ((uint32_t)((lane >> 4) ^ (col16 & 7)) * 16);
   // where the scales / zero points of this lane's output rows sit inside a weight slot
@@ -633,72 +664,94 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   cur.set(u_begin + wave, p.units_per_strip);
   fetch = cur;
   if (fetch.index < u_end) {
-    copy_weights(p, fl, fetch.strip, fetch.unit, ring, lane, unit_group_shift);
-    copy_activations(p, fl, fetch.unit, ring + kWaveA);
+    copy_weights<MB>(p, fl, fetch.strip, fetch.unit, ring, lane, unit_group_shift);
+    copy_activations<MB>(p, fl, fetch.unit, ring + kWaveA);
   }
   fetch.advance(kFastWaves, p.units_per_strip);
   if (fetch.index < u_end)
-    copy_weights(p, fl, fetch.strip, fetch.unit, ring + kSlotBytes, lane, unit_group_shift);
+    copy_weights<MB>(p, fl, fetch.strip, fetch.unit, ring + kSlotBytes, lane, unit_group_shift);
   // `fetch` names the unit whose A slice is copied next; its weights are in flight
   int c_slot = 0;
 
   // the current segment starts at seg_begin, inside strip seg_strip
   int seg_begin = u_begin;
   int seg_strip = u_begin / p.units_per_strip;
-  floatx4_t acc[4];
+  floatx4_t acc[MB][4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) acc[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
   for (;;) {
     const bool have = cur.index < u_end;
     // Close every strip segment that ends before this wavefront's next unit:
-    // every wavefront parks its four tiles in LDS, wavefront j (j < 4) adds up
-    // column block j in wavefront order and finishes it.
+    // in each pass every wavefront parks kPark of its tiles in LDS and
+    // wavefront w (w < kPark) adds up one column block of one block of rows in
+    // wavefront order and finishes it.
     while (seg_begin < u_end) {
       const int strip = seg_strip;
       const int strip_end = (strip + 1) * p.units_per_strip;
       const int seg_end = u_end < strip_end ? u_end : strip_end;
       if (have && cur.index < seg_end) break;
-      __builtin_amdgcn_s_barrier();  // the previous segment's tiles have been consumed
-      const uint32_t park = red_lds + (wave * 4 * 64 + lane) * 16;
-      // the tiles come out of the matrix cores; an asm block is opaque to the
-      // compiler's hazard padding, so give the last MFMA time to retire
-      asm volatile(
-          "s_nop 15\n\t"
-          "s_nop 15\n\t"
-          "ds_write_b128 %0, %1\n\t"
-          "ds_write_b128 %0, %2 offset:1024\n\t"
-          "ds_write_b128 %0, %3 offset:2048\n\t"
-          "ds_write_b128 %0, %4 offset:3072\n\t"
-          "s_waitcnt lgkmcnt(0)"
-          :
-          : "v"(park), "v"(acc[0]), "v"(acc[1]), "v"(acc[2]), "v"(acc[3])
-          : "memory");
 #pragma unroll
-      for (int j = 0; j < 4; ++j) acc[j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-      __builtin_amdgcn_s_barrier();
-      if (wave < 4) {
-        floatx4_t sum = floatx4_t{0.f, 0.f, 0.f, 0.f};
-        const uint32_t src = red_lds + (wave * 64 + lane) * 16;
-#pragma unroll
-        for (int w = 0; w < kFastWaves; w += 4) {
-          floatx4_t t0, t1, t2, t3;
+      for (int ps = 0; ps < kPasses; ++ps) {
+        const int mb = ps * kPark / 4, jb = ps * kPark % 4;
+        __builtin_amdgcn_s_barrier();  // the previous pass's tiles have been consumed
+        const uint32_t park = red_lds + (wave * kPark * 64 + lane) * 16;
+        // the tiles come out of the matrix cores; an asm block is opaque to the
+        // compiler's hazard padding, so give the last MFMA time to retire
+        if constexpr (kPark == 4) {
           asm volatile(
-              "ds_read_b128 %0, %4\n\t"
-              "ds_read_b128 %1, %4 offset:4096\n\t"
-              "ds_read_b128 %2, %4 offset:8192\n\t"
-              "ds_read_b128 %3, %4 offset:12288\n\t"
+              "s_nop 15\n\t"
+              "s_nop 15\n\t"
+              "ds_write_b128 %0, %1\n\t"
+              "ds_write_b128 %0, %2 offset:1024\n\t"
+              "ds_write_b128 %0, %3 offset:2048\n\t"
+              "ds_write_b128 %0, %4 offset:3072\n\t"
               "s_waitcnt lgkmcnt(0)"
-              : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
-              : "v"(src + w * 4096)
+              :
+              : "v"(park), "v"(acc[mb][0]), "v"(acc[mb][1]), "v"(acc[mb][2]), "v"(acc[mb][3])
               : "memory");
-          sum += t0;
-          sum += t1;
-          sum += t2;
-          sum += t3;
+        } else {
+          asm volatile(
+              "s_nop 15\n\t"
+              "s_nop 15\n\t"
+              "ds_write_b128 %0, %1\n\t"
+              "ds_write_b128 %0, %2 offset:1024\n\t"
+              "s_waitcnt lgkmcnt(0)"
+              :
+              : "v"(park), "v"(acc[mb][jb]), "v"(acc[mb][jb + 1])
+              : "memory");
         }
-        finish_block<T>(p, part, slab, strip, seg_begin, seg_end, lane, wave, sum);
+        __builtin_amdgcn_s_barrier();
+        if (wave < kPark) {
+          floatx4_t sum = floatx4_t{0.f, 0.f, 0.f, 0.f};
+          const uint32_t src = red_lds + (wave * 64 + lane) * 16;
+#pragma unroll
+          for (int w = 0; w < kFastWaves; w += 4) {
+            floatx4_t t0, t1, t2, t3;
+            asm volatile(
+                "ds_read_b128 %0, %4\n\t"
+                "ds_read_b128 %1, %4 offset:%5\n\t"
+                "ds_read_b128 %2, %4 offset:%6\n\t"
+                "ds_read_b128 %3, %4 offset:%7\n\t"
+                "s_waitcnt lgkmcnt(0)"
+                : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
+                : "v"(src + w * kPark * 1024), "n"(kPark * 1024), "n"(2 * kPark * 1024), "n"(3 * kPark * 1024)
+                : "memory");
+            sum += t0;
+            sum += t1;
+            sum += t2;
+            sum += t3;
+          }
+          finish_block<T>(p, p.c + (long)(16 * mb) * p.size_n, p.size_m - 16 * mb, part, slab * MB + mb, strip,
+                          seg_begin, seg_end, lane, jb + wave, sum);
+        }
       }
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
       seg_begin = seg_end;
       ++seg_strip;
     }
@@ -708,6 +761,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     // copies of the units after it, then do the arithmetic.
     const uint32_t slot_lds = ring_lds + c_slot * kSlotBytes;
     u32x4_t q0, q1, q2, q3, a0, a1, a2, a3;
+    u32x4_t b0 = u32x4_t{0u, 0u, 0u, 0u}, b1 = b0, b2 = b0, b3 = b0;  // second block of rows
     uint32_t row_s[16];
     u32x4_t row_z = u32x4_t{0u, 0u, 0u, 0u};
     const bool more = cur.index + kFastWaves < u_end;
@@ -724,26 +778,33 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
       } else {        // at byte 64 (j >> 1) + 8 (j & 1) + 16 (r >> 1) + 2 (r & 1)
         SONAR_UNIT_READS(0, 2, 16, 18, 8, 10, 24, 26, 64, 66, 80, 82, 72, 74, 88, 90);
       }
+      if constexpr (MB == 2) SONAR_UNIT_READS_ROWS2(b0, b1, b2, b3);
     }
     if (more) {
-      copy_activations(p, fl, fetch.unit, ring + kWaveA);
+      copy_activations<MB>(p, fl, fetch.unit, ring + kWaveA);
       fetch.advance(kFastWaves, p.units_per_strip);
       if (fetch.index < u_end)
-        copy_weights(p, fl, fetch.strip, fetch.unit, ring + c_slot * kSlotBytes, lane, unit_group_shift);
+        copy_weights<MB>(p, fl, fetch.strip, fetch.unit, ring + c_slot * kSlotBytes, lane, unit_group_shift);
     }
 
     const u32x4_t qs[4] = {q0, q1, q2, q3};
-    const u32x4_t as[4] = {a0, a1, a2, a3};
+    const u32x4_t as[2][4] = {{a0, a1, a2, a3}, {b0, b1, b2, b3}};
     const floatx4_t zero4 = floatx4_t{0.f, 0.f, 0.f, 0.f};
-    floatx4_t part[4], asum;
+    floatx4_t part_sum[MB][4], asum[MB];
 #pragma unroll
     for (int cc = 0; cc < 4; ++cc) {
-      const vec8 av = __builtin_bit_cast(vec8, as[cc]);
       const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
 #pragma unroll
-      for (int j = 0; j < 4; ++j)
-        part[j] = Dq<T>::mfma(__builtin_bit_cast(vec8, raw_operand(words[j], magic)), av, cc == 0 ? zero4 : part[j]);
-      asum = Dq<T>::mfma(__builtin_bit_cast(vec8, ones), av, cc == 0 ? zero4 : asum);
+      for (int j = 0; j < 4; ++j) {
+        const vec8 wv = __builtin_bit_cast(vec8, raw_operand(words[j], magic));
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          part_sum[mb][j] = Dq<T>::mfma(wv, __builtin_bit_cast(vec8, as[mb][cc]), cc == 0 ? zero4 : part_sum[mb][j]);
+      }
+#pragma unroll
+      for (int mb = 0; mb < MB; ++mb)
+        asum[mb] = Dq<T>::mfma(__builtin_bit_cast(vec8, ones), __builtin_bit_cast(vec8, as[mb][cc]),
+                               cc == 0 ? zero4 : asum[mb]);
     }
     const uint32_t zrow[4] = {row_z.x >> row_z_shift, row_z.y >> row_z_shift, row_z.z >> row_z_shift,
                               row_z.w >> row_z_shift};
@@ -754,12 +815,15 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
         const float sc = Dq<T>::to_float((uint16_t)row_s[4 * j + r]);
         float off = -(RawOperand<T>::kBase + 8.f);
         if (HAS_ZP) off = -RawOperand<T>::kBase - (float)((zrow[r] >> (4 * j)) & 0xFu);
-        acc[j][r] = __builtin_fmaf(sc, __builtin_fmaf(off, asum[r], part[j][r]), acc[j][r]);
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          acc[mb][j][r] = __builtin_fmaf(sc, __builtin_fmaf(off, asum[mb][r], part_sum[mb][j][r]), acc[mb][j][r]);
       }
     cur.advance(kFastWaves, p.units_per_strip);
     c_slot ^= 1;
   }
 }
+#undef SONAR_UNIT_READS_ROWS2
 
 // ---------------------------------------------------------------------------
 // Second pass over the strips that were split between workgroups: adds the
@@ -953,23 +1017,27 @@ void launch_stream8_mb(const StreamParams& p, hipStream_t st) {
   }
 }
 
-template <typename T, bool HAS_ZP, int WAVES>
+template <typename T, bool HAS_ZP, int WAVES, int MB>
 int launch_fast_waves(const StreamParams& p, int unit_group_shift, hipStream_t st) {
   static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_stream_fast_kernel<T, HAS_ZP, WAVES>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds_bytes(WAVES)));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds_bytes(WAVES, MB)));
     attr_set = true;
   }
-  const int lds = p.sum_over_rings ? WAVES * kWaveLds : fast_lds_bytes(WAVES);
-  marlin_stream_fast_kernel<T, HAS_ZP, WAVES><<<p.grid_parts * p.slabs, WAVES * 64, lds, st>>>(p, unit_group_shift);
+  const int lds = p.sum_over_rings ? WAVES * wave_lds(MB) : fast_lds_bytes(WAVES, MB);
+  marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB><<<p.grid_parts * p.slabs, WAVES * 64, lds, st>>>(p, unit_group_shift);
   return SONAR_OK;
 }
 
+// `row_blocks`: blocks of 16 rows per workgroup (1 or 2).
 template <typename T, bool HAS_ZP>
-int launch_fast(const StreamParams& p, int unit_group_shift, bool half_workgroups, hipStream_t st) {
-  return half_workgroups ? launch_fast_waves<T, HAS_ZP, 4>(p, unit_group_shift, st)
-                         : launch_fast_waves<T, HAS_ZP, 8>(p, unit_group_shift, st);
+int launch_fast(const StreamParams& p, int unit_group_shift, bool half_workgroups, int row_blocks, hipStream_t st) {
+  if (row_blocks == 2)
+    return half_workgroups ? launch_fast_waves<T, HAS_ZP, 4, 2>(p, unit_group_shift, st)
+                           : launch_fast_waves<T, HAS_ZP, 8, 2>(p, unit_group_shift, st);
+  return half_workgroups ? launch_fast_waves<T, HAS_ZP, 4, 1>(p, unit_group_shift, st)
+                         : launch_fast_waves<T, HAS_ZP, 8, 1>(p, unit_group_shift, st);
 }
 
 template <typename T>
@@ -1186,10 +1254,16 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
     p.size_m = (int)(size_m - m0 < 64 ? size_m - m0 : 64);
     const bool fast = fast_shape && p.unit_chunks == 4 && (p.size_m <= 16 || slab_fast);
     if (fast) {
+      // Two blocks of rows per workgroup once one block each would make more
+      // workgroups than compute units: the weights are then fetched from L2 and
+      // unpacked once for 32 rows.
+      static const bool no_pairs = getenv("SONAR_MARLIN_NO_ROW_PAIRS") != nullptr;  // debugging aid
+      int row_blocks = 1;
       if (slab_fast) {  // every row in this one launch
         p.size_m = (int)size_m;
-        p.slabs = (int)((size_m + 15) / 16);
-        p.grid_parts = (p.parts + 7) / 8 * 8;
+        if (!no_pairs && p.parts * ((size_m + 15) / 16) > cus) row_blocks = 2;
+        p.slabs = (int)((size_m + 16 * row_blocks - 1) / (16 * row_blocks));
+        p.grid_parts = p.slabs > 1 ? (p.parts + 7) / 8 * 8 : p.parts;
         m0 = size_m;
       }
       int rc;
@@ -1199,11 +1273,11 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
       const bool half = !no_half && p.parts * p.slabs > cus;
       p.sum_over_rings = half && (int64_t)p.parts == n_strips && p.parts * p.slabs > 2 * cus;
       if (dtype == SONAR_DTYPE_F16)
-        rc = chk.has_zp ? launch_fast<_Float16, true>(p, unit_group_shift, half, st)
-                        : launch_fast<_Float16, false>(p, unit_group_shift, half, st);
+        rc = chk.has_zp ? launch_fast<_Float16, true>(p, unit_group_shift, half, row_blocks, st)
+                        : launch_fast<_Float16, false>(p, unit_group_shift, half, row_blocks, st);
       else
-        rc = chk.has_zp ? launch_fast<__bf16, true>(p, unit_group_shift, half, st)
-                        : launch_fast<__bf16, false>(p, unit_group_shift, half, st);
+        rc = chk.has_zp ? launch_fast<__bf16, true>(p, unit_group_shift, half, row_blocks, st)
+                        : launch_fast<__bf16, false>(p, unit_group_shift, half, row_blocks, st);
       if (rc) return rc;
     } else if (chk.bits == 8) {
       if (dtype == SONAR_DTYPE_F16) launch_stream8_mb<_Float16>(p, st);
