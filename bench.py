@@ -313,8 +313,8 @@ def main() -> int:
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_M16 if (m == 16 and args.copies == 6) else None,
-                     "kernel": ("marlin_stream_fast_kernel<bf16>" if m <= 16 else
-                                "marlin_stream_kernel<bf16, MB=%d>" % ((m + 15) // 16)) +
+                     "kernel": "marlin_stream_fast_kernel<bf16>" +
+                               ("" if m <= 16 else " (blocks of 16 or 32 rows per workgroup)") +
                                " (+ marlin_fixup_kernel for down_proj)",
                      "bytes_per_launch": step_bytes // launches,
                      "us_per_launch": round(step_s / launches * 1e6, 3)},

@@ -777,6 +777,14 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
       p.k_steps_per_split = plan.k_steps_per_split;
       p.whole_tiles = (int)plan.whole_tiles;
       p.partial = static_cast<float4*>(partial);
+      static const char* max_splits = getenv("SONAR_MARLIN_MAX_K_SPLITS");  // debugging aid
+      if (max_splits && atoi(max_splits) >= 1 && p.k_splits > atoi(max_splits)) {
+        const int k_steps = (int)(size_k / kTileK);
+        p.k_splits = atoi(max_splits);
+        p.k_steps_per_split = (k_steps + p.k_splits - 1) / p.k_splits;
+        p.k_splits = (k_steps + p.k_steps_per_split - 1) / p.k_steps_per_split;
+        if (p.k_splits == 1) p.partial = nullptr;
+      }
     }
     if (dtype == SONAR_DTYPE_F16)
       rc = zp ? launch_tile_async<_Float16, true>(p, st) : launch_tile_async<_Float16, false>(p, st);
