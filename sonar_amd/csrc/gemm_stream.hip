@@ -1216,8 +1216,14 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   static const bool no_slabs = getenv("SONAR_MARLIN_NO_SLABS") != nullptr;  // debugging aid
   // Up to 64 rows this also pays on matrices whose strips are shared between
   // workgroups (a scratch slot has room for four blocks of rows).
+  // Beyond 128 rows the tile kernel takes over, except where it would have few
+  // tiles and split K through memory while this kernel needs at most four
+  // workgroups of 32 rows per compute unit (measured at K = 4096: N = 4096,
+  // M = 256: 21 us against 37; N = 6144, M = 256: 32 against 40; N = 4096,
+  // M = 512: 37 against 44; N = 6144, M = 512: 54 against 50).
+  const bool few_row_blocks = n_strips * ((size_m + 31) / 32) <= 4 * (int64_t)cus;
   const bool slab_fast = !no_slabs && fast_shape && size_m > 16 &&
-                         (size_m <= 64 || (strip_per_workgroup && size_m <= 128));
+                         (size_m <= 64 || (strip_per_workgroup && (size_m <= 128 || few_row_blocks)));
 
   p.unit_chunks = p.chunks_per_strip % 4 == 0 ? 4 : (p.chunks_per_strip % 2 == 0 ? 2 : 1);
   // the general kernel works on half units when it holds more than 32 rows (see unit_buffer_chunks)
@@ -1241,7 +1247,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   const bool async_tile = tile_async_applies(chk.has_perm, num_groups, chk.group_size);
   const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
   // the row -> group lookup and 8-bit codes exist in the streaming kernels only
-  if (plan.tile && !no_tile && !chk.row_groups && chk.bits == 4) {
+  if (plan.tile && !no_tile && !chk.row_groups && chk.bits == 4 && !(slab_fast && p.unit_chunks == 4)) {
     const size_t used = stream_scratch_bytes();
     return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
                      size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used,

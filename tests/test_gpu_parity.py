@@ -115,6 +115,10 @@ GEMM_CASES = [
     (128, 256, 4096, -1, False, False, False),
     (64, 4096, 6144, 128, False, False, False),
     (17, 384, 8192, 128, True, False, True),
+    # more than 128 rows where that is at most four workgroups of 32 rows per compute unit
+    (200, 512, 4096, 128, False, False, True),
+    (300, 1024, 4224, 128, True, False, False),
+    (512, 256, 4096, -1, False, False, False),
     # the same with strips shared between workgroups (partial tiles per block of rows)
     (33, 14336, 1024, 128, False, False, True),
     (64, 2048, 512, 128, True, False, False),
