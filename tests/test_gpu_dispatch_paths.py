@@ -1,0 +1,38 @@
+"""Every kernel the dispatcher can fall back to, on shapes the faster kernels
+normally take: the debugging switches of the library (read once per process)
+turn the faster paths off one at a time, and the same cases must still meet
+the oracle.  One child process per switch, one after the other."""
+from __future__ import annotations
+
+import os
+import subprocess
+import sys
+
+import pytest
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+SWITCHES = [
+    None,                            # the default dispatch
+    "SONAR_MARLIN_NO_FAST",          # the register-prefetch streaming kernel for every M <= 64
+    "SONAR_MARLIN_NO_SLABS",         # no blocks of rows in the 16-row kernel
+    "SONAR_MARLIN_NO_ROW_PAIRS",     # blocks of 16 rows only
+    "SONAR_MARLIN_NO_HALF_WG",       # 8-wavefront workgroups only
+    "SONAR_MARLIN_NO_TILE",          # the streaming kernels in 64-row slabs for every M
+    "SONAR_MARLIN_NO_ASYNC_TILE",    # the register-staged tile kernel
+    "SONAR_MARLIN_MAX_K_SPLITS=1",   # no split K in the tile kernel
+    "SONAR_MARLIN_NO_MOE_TILE",      # the grouped streaming kernel for 64-slot blocks
+]
+
+
+@pytest.mark.parametrize("switch", SWITCHES, ids=lambda s: s or "default")
+def test_every_dispatch_path_meets_the_oracle(switch):
+    env = dict(os.environ)
+    if switch:
+        name, _, value = switch.partition("=")
+        env[name] = value or "1"
+    out = subprocess.run([sys.executable, "-u", "-m", "tests.dispatch_paths_child"], cwd=ROOT, env=env,
+                         capture_output=True, text=True, timeout=110)
+    assert out.returncode == 0 and "all paths ok" in out.stdout, out.stdout[-1500:] + out.stderr[-1500:]
