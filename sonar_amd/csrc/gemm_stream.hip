@@ -63,6 +63,16 @@ struct StreamParams {
   // the copy rings instead of behind them.  Allowed when every workgroup owns
   // whole strips: it then sums once, after its last copy has been consumed.
   int sum_over_rings;
+  // grouped (mixture-of-experts) calls of the fast kernel only: workgroup
+  // block * grid_parts + strip works on the slots [block * block_size, ...) of
+  // sorted_ids with the weights of expert_ids[block]
+  const int32_t* sorted_ids;   // slot -> row id of C (row id / top_k of A); outside [0, rows_total): padding
+  const int32_t* expert_ids;
+  const int32_t* num_post_pad;
+  const float* topk_weights;
+  int block_size, top_k, num_experts, rows_total, sorted_len, mul_topk;
+  long expert_b_stride;        // uint4 units between experts in b
+  long expert_s_stride, expert_z_stride, expert_bias_stride;  // elements between experts
 };
 
 // Unit indices are 32-bit: the host checks total_units * parts < 2^31.
@@ -177,6 +187,32 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, uint16_t* c_
   }
   const int first = range_owner(strip_first, p.total_units, p.parts);
   partial_slot(p, part, first)[(slab * 4 + j) * 64 + lane] = make_float4(v.x, v.y, v.z, v.w);
+}
+
+// Grouped calls: the tile's row (lane & 15) goes to row `id` of C (none when
+// id < 0), with the expert's bias and, when asked, the routing weight: the
+// weight is rounded to the activation type and the product is formed and
+// rounded in that type (marlin_moe_wna16/marlin_template.h:1883-1909).
+template <typename T>
+__device__ __forceinline__ void finish_block_grouped(const StreamParams& p, int id, int strip, int lane, int j,
+                                                     floatx4_t v) {
+  if (id < 0) return;
+  const int nl = 16 * j + 4 * (lane >> 4);
+  const float r[4] = {v.x, v.y, v.z, v.w};
+  float tw = 1.f;
+  if (p.mul_topk) tw = Dq<T>::to_float(Dq<T>::from_float(p.topk_weights[id]));
+  uint16_t o[4];
+#pragma unroll
+  for (int t = 0; t < 4; ++t) {
+    float x = r[t];
+    if (p.bias) x += Dq<T>::to_float(p.bias[strip * kStripN + scale_slot(nl + t, false)]);
+    o[t] = Dq<T>::from_float(x);
+    if (p.mul_topk) o[t] = Dq<T>::from_float(Dq<T>::to_float(o[t]) * tw);
+  }
+  uint2 packed;
+  packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+  packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+  *reinterpret_cast<uint2*>(p.c + (long)id * p.size_n + strip * kStripN + nl) = packed;
 }
 
 // ---------------------------------------------------------------------------
@@ -450,6 +486,14 @@ constexpr int kWeightCopies = 5;   // asynchronous copies per unit: 4 weight chu
 // units then runs them side by side instead of one after the other).
 constexpr int fast_lds_bytes(int waves, int mb) { return waves * (wave_lds(mb) + park_tiles(mb) * 1024); }
 
+// Row id of C of row `r` of block `block` of a grouped call, -1 for padding.
+__device__ __forceinline__ int moe_row_id(const StreamParams& p, int block, int r) {
+  const int at = block * p.block_size + r;
+  if (r >= p.block_size || at >= p.sorted_len) return -1;
+  const int id = p.sorted_ids[at];
+  return (id < 0 || id >= p.rows_total) ? -1 : id;
+}
+
 template <int MB>
 struct FastLane {
   uint32_t a_off[2 * MB];  // byte offset of the 16 bytes this lane copies from rows 8h..8h+7 of a 64-column slice of A
@@ -593,7 +637,10 @@ __device__ __forceinline__ u32x4_t raw_operand(uint32_t q, uint32_t magic) {
 
 // MB blocks of 16 rows per workgroup (1 or 2): the weights of a unit are pulled
 // out of LDS and turned into operands once and multiplied with every block.
-template <typename T, bool HAS_ZP, int kFastWaves, int MB>
+// GROUPED: one workgroup per (block of slots, strip) of a mixture-of-experts
+// call; the rows of A are gathered and the rows of C scattered through
+// sorted_ids, everything else is the dense kernel on the expert's matrices.
+template <typename T, bool HAS_ZP, int kFastWaves, int MB, bool GROUPED = false>
 __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams params,
                                                                              const int unit_group_shift) {
   typedef typename Dq<T>::vec8 vec8;
@@ -608,10 +655,25 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   const int part = blockIdx.x % p.grid_parts;
   const int slab = blockIdx.x / p.grid_parts;
   if (part >= p.parts) return;
-  p.a += (long)slab * (16 * MB) * p.lda;
-  p.c += (long)slab * (16 * MB) * p.size_n;
-  p.size_m = min(16 * MB, p.size_m - 16 * MB * slab);
   const int lane = threadIdx.x & 63;
+  int row_id[MB] = {};  // grouped calls: the row of C that row (lane & 15) of block of rows mb goes to, or -1
+  if constexpr (GROUPED) {
+    // `slab` is the block of slots here; the whole workgroup leaves together
+    if (slab * p.block_size >= p.num_post_pad[0]) return;
+    const long expert = p.expert_ids[slab];
+    if (expert < 0 || expert >= p.num_experts) return;
+    p.b += expert * p.expert_b_stride;
+    p.scales += expert * p.expert_s_stride;
+    if (HAS_ZP) p.zeros += expert * p.expert_z_stride;
+    if (p.bias) p.bias += expert * p.expert_bias_stride;
+    p.size_m = 16 * MB;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) row_id[mb] = moe_row_id(p, slab, 16 * mb + (lane & 15));
+  } else {
+    p.a += (long)slab * (16 * MB) * p.lda;
+    p.c += (long)slab * (16 * MB) * p.size_n;
+    p.size_m = min(16 * MB, p.size_m - 16 * MB * slab);
+  }
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col16 = lane & 15;
   char* ring = smem + wave * kWaveLds;
@@ -627,7 +689,11 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
 #pragma unroll
     for (int h = 0; h < 2 * MB; ++h) {
       const int r = 8 * h + (lane >> 3);
-      const int row = r < p.size_m ? r : p.size_m - 1;  // rows past M are never stored
+      int row = r < p.size_m ? r : p.size_m - 1;  // rows past M are never stored
+      if constexpr (GROUPED) {                    // padding slots read row 0 and are never stored
+        const int id = moe_row_id(p, slab, r);
+        row = id >= 0 ? id / p.top_k : 0;
+      }
       fl.a_off[h] = (uint32_t)((long)row * p.lda * 2 + 16 * ((lane & 7) ^ (lane >> 3)));
     }
     if (HAS_ZP && lane >= 32) {
@@ -744,8 +810,11 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
             sum += t2;
             sum += t3;
           }
-          finish_block<T>(p, p.c + (long)(16 * mb) * p.size_n, p.size_m - 16 * mb, part, slab * MB + mb, strip,
-                          seg_begin, seg_end, lane, jb + wave, sum);
+          if constexpr (GROUPED)
+            finish_block_grouped<T>(p, row_id[mb], strip, lane, jb + wave, sum);
+          else
+            finish_block<T>(p, p.c + (long)(16 * mb) * p.size_n, p.size_m - 16 * mb, part, slab * MB + mb, strip,
+                            seg_begin, seg_end, lane, jb + wave, sum);
         }
       }
 #pragma unroll
@@ -1017,27 +1086,28 @@ void launch_stream8_mb(const StreamParams& p, hipStream_t st) {
   }
 }
 
-template <typename T, bool HAS_ZP, int WAVES, int MB>
+template <typename T, bool HAS_ZP, int WAVES, int MB, bool GROUPED>
 int launch_fast_waves(const StreamParams& p, int unit_group_shift, hipStream_t st) {
   static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB>,
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB, GROUPED>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds_bytes(WAVES, MB)));
     attr_set = true;
   }
   const int lds = p.sum_over_rings ? WAVES * wave_lds(MB) : fast_lds_bytes(WAVES, MB);
-  marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB><<<p.grid_parts * p.slabs, WAVES * 64, lds, st>>>(p, unit_group_shift);
+  marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB, GROUPED>
+      <<<p.grid_parts * p.slabs, WAVES * 64, lds, st>>>(p, unit_group_shift);
   return SONAR_OK;
 }
 
 // `row_blocks`: blocks of 16 rows per workgroup (1 or 2).
-template <typename T, bool HAS_ZP>
+template <typename T, bool HAS_ZP, bool GROUPED = false>
 int launch_fast(const StreamParams& p, int unit_group_shift, bool half_workgroups, int row_blocks, hipStream_t st) {
   if (row_blocks == 2)
-    return half_workgroups ? launch_fast_waves<T, HAS_ZP, 4, 2>(p, unit_group_shift, st)
-                           : launch_fast_waves<T, HAS_ZP, 8, 2>(p, unit_group_shift, st);
-  return half_workgroups ? launch_fast_waves<T, HAS_ZP, 4, 1>(p, unit_group_shift, st)
-                         : launch_fast_waves<T, HAS_ZP, 8, 1>(p, unit_group_shift, st);
+    return half_workgroups ? launch_fast_waves<T, HAS_ZP, 4, 2, GROUPED>(p, unit_group_shift, st)
+                           : launch_fast_waves<T, HAS_ZP, 8, 2, GROUPED>(p, unit_group_shift, st);
+  return half_workgroups ? launch_fast_waves<T, HAS_ZP, 4, 1, GROUPED>(p, unit_group_shift, st)
+                         : launch_fast_waves<T, HAS_ZP, 8, 1, GROUPED>(p, unit_group_shift, st);
 }
 
 template <typename T>
@@ -1104,7 +1174,94 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
   return SONAR_OK;
 }
 
+// log2 of the 128-row units per group when groups are runs of 128 * 2^s rows,
+// -1 for one group; false when the fast kernel cannot index the groups.
+bool fast_group_shift(int64_t num_groups, int group_size, int& unit_group_shift) {
+  unit_group_shift = -1;
+  if (num_groups == 1) return true;
+  if (group_size <= 0 || group_size % 128 != 0) return false;
+  const int per = group_size / 128;
+  if ((per & (per - 1)) != 0) return false;
+  unit_group_shift = 0;
+  while ((1 << unit_group_shift) < per) ++unit_group_shift;
+  return true;
+}
+
 }  // namespace
+
+// The grouped (mixture-of-experts) op can use the 16-row kernel for blocks of up
+// to 32 slots when the expert matrices meet its conditions.
+bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t size_m, int64_t size_n, int64_t size_k,
+                      int64_t num_groups, int group_size) {
+  static const bool no_fast = getenv("SONAR_MARLIN_NO_MOE_FAST") != nullptr;  // debugging aid
+  int shift;
+  const int64_t n_strips = size_n / kStripN, units = size_k / (4 * kChunkK);
+  return !no_fast && !has_perm && moe_block_size <= 32 && size_k % (4 * kChunkK) == 0 &&
+         fast_group_shift(num_groups, group_size, shift) && size_m * size_k * 2 < (1LL << 31) &&
+         n_strips * units * n_strips < (1LL << 31);
+}
+
+// Called by sonar_moe_wna16_marlin_gemm when moe_fast_applies: one workgroup
+// per (block of slots, strip), nothing reduced through memory.  Arguments have
+// been validated by the caller.
+int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, const void* scales,
+                  const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
+                  const int32_t* num_post_pad, const float* topk_weights, int64_t moe_block_size, int64_t top_k,
+                  int mul_topk, int64_t num_experts, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
+                  int64_t num_groups, int group_size, hipStream_t st) {
+  StreamParams p = {};
+  p.a = static_cast<const uint16_t*>(a);
+  p.lda = size_k;
+  p.c = static_cast<uint16_t*>(c);
+  p.b = reinterpret_cast<const uint4*>(b);
+  p.bias = static_cast<const uint16_t*>(bias);
+  p.scales = static_cast<const uint16_t*>(scales);
+  p.zeros = zeros;
+  p.size_m = (int)size_m;
+  p.size_n = (int)size_n;
+  p.size_k = (int)size_k;
+  p.num_groups = (int)num_groups;
+  p.group_size = group_size;
+  p.chunks_per_strip = (int)(size_k / kChunkK);
+  p.unit_chunks = 4;
+  p.units_per_strip = p.chunks_per_strip / 4;
+  const int n_strips = (int)(size_n / kStripN);
+  p.parts = n_strips;                       // part i is strip i
+  p.total_units = n_strips * p.units_per_strip;
+  p.slabs = (int)((sorted_len + moe_block_size - 1) / moe_block_size);   // blocks of slots
+  p.grid_parts = n_strips;
+  p.sum_over_rings = 1;                     // every workgroup owns a whole strip
+  p.sorted_ids = sorted_ids;
+  p.expert_ids = expert_ids;
+  p.num_post_pad = num_post_pad;
+  p.topk_weights = topk_weights;
+  p.block_size = (int)moe_block_size;
+  p.top_k = (int)top_k;
+  p.num_experts = (int)num_experts;
+  p.rows_total = (int)(size_m * top_k);
+  p.sorted_len = (int)sorted_len;
+  p.mul_topk = mul_topk;
+  p.expert_b_stride = (long)n_strips * p.chunks_per_strip * 64;
+  p.expert_s_stride = (long)num_groups * size_n;
+  p.expert_z_stride = (long)num_groups * (size_n / 8);
+  p.expert_bias_stride = size_n;
+  SONAR_REQUIRE((int64_t)p.slabs * n_strips < (1LL << 31), "too many (block, strip) pairs: %ld",
+                (long)((int64_t)p.slabs * n_strips));
+  int unit_group_shift;
+  fast_group_shift(num_groups, group_size, unit_group_shift);
+  const bool half = (int64_t)p.slabs * n_strips > cu_count();   // small workgroups, three per compute unit
+  const int row_blocks = moe_block_size <= 16 ? 1 : 2;
+  int rc;
+  if (dtype == SONAR_DTYPE_F16)
+    rc = zeros ? launch_fast<_Float16, true, true>(p, unit_group_shift, half, row_blocks, st)
+               : launch_fast<_Float16, false, true>(p, unit_group_shift, half, row_blocks, st);
+  else
+    rc = zeros ? launch_fast<__bf16, true, true>(p, unit_group_shift, half, row_blocks, st)
+               : launch_fast<__bf16, false, true>(p, unit_group_shift, half, row_blocks, st);
+  if (rc) return rc;
+  return launch_status("marlin_stream_fast_kernel (grouped)");
+}
+
 }  // namespace sonar
 
 using namespace sonar;
@@ -1171,7 +1328,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                 "act-order with is_k_full = False needs size_m * size_k * 2 more scratch bytes "
                 "(the column-permuted copy of A)");
 
-  StreamParams p;
+  StreamParams p = {};
   p.b = reinterpret_cast<const uint4*>(b_q_weight);
   p.bias = static_cast<const uint16_t*>(b_bias);
   p.scales = static_cast<const uint16_t*>(b_scales);
@@ -1187,16 +1344,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   p.chunks_per_strip = (int)(size_k / kChunkK);
 
   // groups of 128 * 2^s rows: group of a unit = unit >> s
-  int unit_group_shift = -1;
-  bool fast_groups = num_groups == 1;
-  if (num_groups > 1 && chk.group_size > 0 && chk.group_size % 128 == 0) {
-    const int per = chk.group_size / 128;
-    if ((per & (per - 1)) == 0) {
-      fast_groups = true;
-      unit_group_shift = 0;
-      while ((1 << unit_group_shift) < per) ++unit_group_shift;
-    }
-  }
+  int unit_group_shift;
+  const bool fast_groups = fast_group_shift(num_groups, chk.group_size, unit_group_shift);
   static const bool no_fast = getenv("SONAR_MARLIN_NO_FAST") != nullptr;  // debugging aid
   const bool fast_shape = !no_fast && chk.bits == 4 && !chk.has_perm && !chk.row_groups &&
                           p.chunks_per_strip % 4 == 0 && fast_groups &&

@@ -45,7 +45,9 @@ def grouped() -> None:
     from tests import test_gpu_moe as tm
     for case in [(300, 4, 2, 256, 256, 128, "fp16", False, False, False, 64, True),
                  (700, 8, 2, 512, 128, 64, "bf16", True, False, True, 64, False),
-                 (40, 4, 2, 256, 128, 128, "fp16", False, False, False, 16, True)]:
+                 (40, 4, 2, 256, 128, 128, "fp16", False, False, False, 16, True),
+                 (3, 8, 2, 512, 256, 128, "bf16", True, False, True, 8, False),
+                 (130, 4, 2, 256, 320, -1, "fp16", False, False, True, 32, True)]:
         print("grouped", case, flush=True)
         tm.test_moe_gemm_within_tolerance(case)   # raises on a mismatch
 
