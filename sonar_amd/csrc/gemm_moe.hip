@@ -25,9 +25,9 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
                   int64_t num_groups, int group_size, hipStream_t st);
 size_t moe_tile_table_bytes(int64_t sorted_len, int64_t num_experts);
-// gemm_stream.hip: the 16-row decode kernel in grouped form, for blocks of up to 32 slots
-bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t size_m, int64_t size_n, int64_t size_k,
-                      int64_t num_groups, int group_size);
+// gemm_stream.hip: the 16-row decode kernel in grouped form, for few rows per expert
+bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t sorted_len, int64_t num_experts,
+                      int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size);
 int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, const void* scales,
                   const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t moe_block_size, int64_t top_k,
@@ -323,6 +323,12 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                 (long)sorted_len);
 
   hipStream_t st = (hipStream_t)stream;
+  // Few rows per expert: the decode kernel, one workgroup per strip and 32 slots of a block
+  if (moe_fast_applies(has_perm, moe_block_size, sorted_len, num_experts, size_m, size_n, size_k, num_groups,
+                       group_size))
+    return moe_fast_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
+                         num_tokens_past_padded, topk_weights, moe_block_size, top_k, mul_topk_weights ? 1 : 0,
+                         num_experts, dtype, size_m, size_n, size_k, num_groups, group_size, st);
   static const bool no_tile = getenv("SONAR_MARLIN_NO_MOE_TILE") != nullptr;  // debugging aid
   // Full blocks of 64 slots mean many rows per expert: the MFMA-tiled kernel
   if (moe_block_size == 64 && !has_perm && !no_tile && size_k % 64 == 0 && num_experts <= 1024 &&
@@ -331,13 +337,6 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     return moe_tile_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
                          num_tokens_past_padded, topk_weights, top_k, mul_topk_weights ? 1 : 0, num_experts,
                          static_cast<int32_t*>(scratch), dtype, size_m, size_n, size_k, num_groups, group_size, st);
-
-  // Few rows per expert (blocks of 8 to 32 slots): the decode kernel, one
-  // workgroup per block and strip
-  if (moe_fast_applies(has_perm, moe_block_size, size_m, size_n, size_k, num_groups, group_size))
-    return moe_fast_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
-                         num_tokens_past_padded, topk_weights, moe_block_size, top_k, mul_topk_weights ? 1 : 0,
-                         num_experts, dtype, size_m, size_n, size_k, num_groups, group_size, st);
 
   MoeParams p;
   p.a = static_cast<const uint16_t*>(a);

@@ -65,12 +65,14 @@ struct StreamParams {
   int sum_over_rings;
   // grouped (mixture-of-experts) calls of the fast kernel only: workgroup
   // block * grid_parts + strip works on the slots [block * block_size, ...) of
-  // sorted_ids with the weights of expert_ids[block]
+  // sorted_ids with the weights of expert_ids[block]; blocks of 48 and 64 slots
+  // are split between two workgroups (`slab` = block * sub_blocks + half)
   const int32_t* sorted_ids;   // slot -> row id of C (row id / top_k of A); outside [0, rows_total): padding
   const int32_t* expert_ids;
   const int32_t* num_post_pad;
   const float* topk_weights;
   int block_size, top_k, num_experts, rows_total, sorted_len, mul_topk;
+  int sub_blocks;              // workgroups (of up to 32 rows) per block of slots and strip
   long expert_b_stride;        // uint4 units between experts in b
   long expert_s_stride, expert_z_stride, expert_bias_stride;  // elements between experts
 };
@@ -658,9 +660,11 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   const int lane = threadIdx.x & 63;
   int row_id[MB] = {};  // grouped calls: the row of C that row (lane & 15) of block of rows mb goes to, or -1
   if constexpr (GROUPED) {
-    // `slab` is the block of slots here; the whole workgroup leaves together
-    if (slab * p.block_size >= p.num_post_pad[0]) return;
-    const long expert = p.expert_ids[slab];
+    // `slab` names the block of slots and the 32 rows of it; the whole workgroup leaves together
+    const int block = slab / p.sub_blocks;
+    const int row0 = 32 * (slab - block * p.sub_blocks);
+    if (block * p.block_size >= p.num_post_pad[0]) return;
+    const long expert = p.expert_ids[block];
     if (expert < 0 || expert >= p.num_experts) return;
     p.b += expert * p.expert_b_stride;
     p.scales += expert * p.expert_s_stride;
@@ -668,7 +672,13 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     if (p.bias) p.bias += expert * p.expert_bias_stride;
     p.size_m = 16 * MB;
 #pragma unroll
-    for (int mb = 0; mb < MB; ++mb) row_id[mb] = moe_row_id(p, slab, 16 * mb + (lane & 15));
+    for (int mb = 0; mb < MB; ++mb) row_id[mb] = moe_row_id(p, block, row0 + 16 * mb + (lane & 15));
+    // nothing but padding in these rows (the tail of an expert's last block): every
+    // wavefront sees the same ids, so the workgroup leaves as one
+    bool any_row = false;
+#pragma unroll
+    for (int mb = 0; mb < MB; ++mb) any_row |= row_id[mb] >= 0;
+    if (__builtin_amdgcn_ballot_w64(any_row) == 0) return;
   } else {
     p.a += (long)slab * (16 * MB) * p.lda;
     p.c += (long)slab * (16 * MB) * p.size_n;
@@ -691,7 +701,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
       const int r = 8 * h + (lane >> 3);
       int row = r < p.size_m ? r : p.size_m - 1;  // rows past M are never stored
       if constexpr (GROUPED) {                    // padding slots read row 0 and are never stored
-        const int id = moe_row_id(p, slab, r);
+        const int id = moe_row_id(p, slab / p.sub_blocks, 32 * (slab % p.sub_blocks) + r);
         row = id >= 0 ? id / p.top_k : 0;
       }
       fl.a_off[h] = (uint32_t)((long)row * p.lda * 2 + 16 * ((lane & 7) ^ (lane >> 3)));
@@ -1189,16 +1199,26 @@ bool fast_group_shift(int64_t num_groups, int group_size, int& unit_group_shift)
 
 }  // namespace
 
-// The grouped (mixture-of-experts) op can use the 16-row kernel for blocks of up
-// to 32 slots when the expert matrices meet its conditions.
-bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t size_m, int64_t size_n, int64_t size_k,
-                      int64_t num_groups, int group_size) {
+// The grouped (mixture-of-experts) op can use the 16-row kernel when the expert
+// matrices meet its conditions (blocks of 48 or 64 slots as two halves).
+bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t sorted_len, int64_t num_experts,
+                      int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size) {
   static const bool no_fast = getenv("SONAR_MARLIN_NO_MOE_FAST") != nullptr;  // debugging aid
   int shift;
   const int64_t n_strips = size_n / kStripN, units = size_k / (4 * kChunkK);
-  return !no_fast && !has_perm && moe_block_size <= 32 && size_k % (4 * kChunkK) == 0 &&
-         fast_group_shift(num_groups, group_size, shift) && size_m * size_k * 2 < (1LL << 31) &&
-         n_strips * units * n_strips < (1LL << 31);
+  if (no_fast || has_perm || size_k % (4 * kChunkK) != 0 || !fast_group_shift(num_groups, group_size, shift) ||
+      size_m * size_k * 2 >= (1LL << 31) || n_strips * units * n_strips >= (1LL << 31))
+    return false;
+  if (moe_block_size < 64) return true;
+  // 64-slot blocks also have the tile kernel, which wins once the experts have
+  // rows enough to fill its 256-row tiles.  Measured on Mixtral shapes (8
+  // experts, top 2): 1016 slots (256 tokens): 285 / 128 us here against 459 /
+  // 349 in the tile kernel (gate_up / down); 1528 slots: 559 / 237 against 493 /
+  // 355; 2552 slots: 977 / 406 against 753 / 369.  The tile kernel launches at
+  // least experts x N / 256 workgroups; where that is under one per compute
+  // unit (down) it stays behind for longer.
+  const int64_t tile_workgroups = num_experts * ((size_n + 255) / 256);
+  return sorted_len <= (tile_workgroups < cu_count() ? 1600 : 1100);
 }
 
 // Called by sonar_moe_wna16_marlin_gemm when moe_fast_applies: one workgroup
@@ -1228,7 +1248,8 @@ int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   const int n_strips = (int)(size_n / kStripN);
   p.parts = n_strips;                       // part i is strip i
   p.total_units = n_strips * p.units_per_strip;
-  p.slabs = (int)((sorted_len + moe_block_size - 1) / moe_block_size);   // blocks of slots
+  p.sub_blocks = moe_block_size > 32 ? 2 : 1;
+  p.slabs = (int)((sorted_len + moe_block_size - 1) / moe_block_size) * p.sub_blocks;   // blocks of slots x halves
   p.grid_parts = n_strips;
   p.sum_over_rings = 1;                     // every workgroup owns a whole strip
   p.sorted_ids = sorted_ids;
