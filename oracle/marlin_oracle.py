@@ -651,6 +651,26 @@ def moe_align_block_size(topk_ids: np.ndarray, block_size: int, num_experts: int
     return sorted_ids, expert_ids, np.array([pos], dtype=np.int32)
 
 
+def batched_moe_align_block_size(max_tokens_per_batch: int, block_size: int, expert_num_tokens):
+    """Tokens already batched by expert (csrc/libtorch_stable/moe/
+    moe_align_sum_kernels.cu:26-82): batch b owns ceil(n_b / bs) blocks laid end
+    to end; slot i of its range holds row b * max_tokens + i for i < n_b, the
+    rest B * max_tokens; blocks of no batch hold expert -1."""
+    n = [int(x) for x in expert_num_tokens]
+    batches = len(n)
+    per_batch = -(-max_tokens_per_batch // block_size) * block_size
+    sentinel = batches * max_tokens_per_batch
+    sorted_ids = np.full(batches * per_batch, sentinel, dtype=np.int32)
+    expert_ids = np.full(batches * per_batch // block_size, -1, dtype=np.int32)
+    at = 0
+    for b, count in enumerate(n):
+        padded = -(-count // block_size) * block_size
+        sorted_ids[at:at + count] = b * max_tokens_per_batch + np.arange(count)
+        expert_ids[at // block_size:(at + padded) // block_size] = b
+        at += padded
+    return sorted_ids, expert_ids, np.array([at], dtype=np.int32)
+
+
 def moe_block_size_rule(m: int, topk: int, num_experts: int) -> int:
     """fused_marlin_moe block size choice (experts/marlin_moe.py:322-329)."""
     for bs in (8, 16, 32, 48, 64):

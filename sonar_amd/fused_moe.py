@@ -115,6 +115,39 @@ def _moe_align_block_size_torch(topk_ids, block_size, num_experts, expert_map, i
     return sorted_ids, expert_ids.to(torch.int32), total.to(torch.int32).reshape(1)
 
 
+def batched_moe_align_block_size(max_tokens_per_batch: int, block_size: int,
+                                 expert_num_tokens: torch.Tensor):
+    """Routing tables for tokens that are already batched by expert: batch b holds
+    the tokens of expert b in rows b * max_tokens_per_batch .., the first
+    expert_num_tokens[b] of them valid (moe_align_block_size.py:100-186; the
+    arithmetic follows batched_moe_align_block_size_kernel,
+    csrc/libtorch_stable/moe/moe_align_sum_kernels.cu:26-82).  Every batch is
+    padded to whole blocks; padding slots hold B * max_tokens_per_batch, unused
+    blocks expert -1.  Index arithmetic only: nothing is read back to the host."""
+    B = expert_num_tokens.size(0)
+    dev = expert_num_tokens.device
+    total = B * ((max_tokens_per_batch + block_size - 1) // block_size * block_size)
+    sentinel = B * max_tokens_per_batch
+    n = expert_num_tokens.to(torch.int64)
+    padded = (n + block_size - 1) // block_size * block_size
+    ends = torch.cumsum(padded, 0)
+    starts = ends - padded
+
+    def owner(pos):                      # batch whose padded range holds slot pos, B past the last one
+        return torch.searchsorted(ends, pos, right=True)
+
+    pos = torch.arange(total, device=dev)
+    b = owner(pos)
+    bc = b.clamp(max=B - 1)
+    off = pos - starts[bc]
+    valid = (b < B) & (off < n[bc])
+    sorted_ids = torch.where(valid, bc * max_tokens_per_batch + off,
+                             torch.full_like(pos, sentinel)).to(torch.int32)
+    bb = owner(torch.arange(total // block_size, device=dev) * block_size)
+    expert_ids = torch.where(bb < B, bb, torch.full_like(bb, -1)).to(torch.int32)
+    return sorted_ids, expert_ids, ends[-1:].to(torch.int32)
+
+
 def silu_and_mul(out: torch.Tensor, x: torch.Tensor) -> torch.Tensor:
     """out = silu(x[:, :d]) * x[:, d:] in the tensor's own dtype."""
     d = x.shape[-1] // 2
@@ -228,3 +261,51 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
         local = expert_map.to(torch.int64)[topk_ids.to(torch.int64).clamp(0, global_num_experts - 1)] >= 0
         moe_output = torch.where(local.unsqueeze(-1), moe_output, torch.zeros_like(moe_output))
     return moe_sum(moe_output.contiguous(), output)
+
+
+def batched_fused_marlin_moe(hidden_states: torch.Tensor, expert_num_tokens: torch.Tensor, w1: torch.Tensor,
+                             w2: torch.Tensor, bias1: torch.Tensor | None, bias2: torch.Tensor | None,
+                             w1_scale: torch.Tensor, w2_scale: torch.Tensor, quant_type_id: int,
+                             apply_router_weight_on_input: bool = False,
+                             g_idx1: torch.Tensor | None = None, g_idx2: torch.Tensor | None = None,
+                             sort_indices1: torch.Tensor | None = None, sort_indices2: torch.Tensor | None = None,
+                             w1_zeros: torch.Tensor | None = None, w2_zeros: torch.Tensor | None = None,
+                             workspace: torch.Tensor | None = None,
+                             intermediate_cache13: torch.Tensor | None = None,
+                             intermediate_cache2: torch.Tensor | None = None, is_k_full: bool = True,
+                             output: torch.Tensor | None = None) -> torch.Tensor:
+    """The layer on tokens already batched by expert (marlin_moe.py:395-560):
+    hidden_states [E, max_tokens, K], of which the first expert_num_tokens[e] rows
+    of batch e are valid.  Every row belongs to one expert, so top_k = 1 and the
+    routing weights are ones.  Returns [E, max_tokens, K]; rows of invalid tokens
+    are not written."""
+    if quant_type_id not in _SUPPORTED:
+        raise NotImplementedError(f"quant type id {quant_type_id}: only uint4 and uint4b8 expert weights "
+                                  "are built")
+    assert hidden_states.ndim == 3, f"hidden states must be batched. e.g. [B, MAX_TOKENS, K].But got {hidden_states.size()}"
+    B, max_tokens, K = hidden_states.shape
+    E = w1.shape[0]
+    assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
+    assert hidden_states.dtype in (torch.float16, torch.bfloat16)
+    assert expert_num_tokens.size(0) == E
+    assert B == E, "Batch must be as big as number of experts as the tokens are sorted into the batch/expert they belong to"
+    assert w1.shape[1] * 16 == K, "Hidden size mismatch w1"
+    assert w2.shape[2] // 2 == K, "Hidden size mismatch w2"
+    assert w1.is_contiguous() and w2.is_contiguous(), "Expert weights must be contiguous"
+    block_size_m = 64
+    for b_m in (8, 16, 32, 48, 64):
+        if max_tokens / b_m < 0.9:
+            block_size_m = b_m
+            break
+    sorted_token_ids, expert_ids, num_tokens_post_padded = batched_moe_align_block_size(
+        max_tokens, block_size_m, expert_num_tokens)
+    M = B * max_tokens
+    topk_weights = torch.ones((M, 1), device=hidden_states.device, dtype=torch.float32)
+    out = _fused_marlin_moe(
+        hidden_states.view(-1, K), w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, 1,
+        _SUPPORTED[quant_type_id], apply_router_weight_on_input, block_size_m, sorted_token_ids, expert_ids,
+        num_tokens_post_padded, g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1,
+        sort_indices2=sort_indices2, w1_zeros=w1_zeros, w2_zeros=w2_zeros, workspace=workspace,
+        intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2,
+        output=output.view(-1, K) if output is not None else None, is_k_full=is_k_full)
+    return out.view(B, max_tokens, K)

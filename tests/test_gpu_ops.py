@@ -378,6 +378,41 @@ def test_moe_checkpoint_tensors_through_weight_processing(cfg):
     assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)
 
 
+@pytest.mark.parametrize("cfg", [
+    # experts, max tokens per expert, hidden, intermediate, group, dtype, zero points
+    (4, 5, 256, 128, 128, "fp16", False),
+    (8, 20, 256, 256, 64, "bf16", False),
+    (4, 70, 128, 128, 128, "bf16", True),
+], ids=str)
+def test_batched_fused_marlin_moe_against_per_token_reference(cfg):
+    """Tokens already batched by expert (marlin_moe.py:395-560): the valid rows of
+    batch e go through expert e; rows past expert_num_tokens[e] are left alone."""
+    from sonar_amd.fused_moe import batched_fused_marlin_moe
+    from sonar_amd.scalar_type import scalar_types
+    e, max_tokens, hidden, inter, g, dtype, zp = cfg
+    (w1, s1, z1, ref13), (w2, s2, z2, ref2) = _moe_layer(60, e, hidden, inter, g, dtype, zp)
+    rng = np.random.default_rng(max_tokens)
+    counts = rng.integers(0, max_tokens + 1, size=e).astype(np.int32)
+    counts[0] = max_tokens                  # one full batch, and
+    counts[-1] = 0                          # one empty
+    x32 = mo.round_to_dtype(0.5 * mo.make_activations(7, e * max_tokens, hidden, dtype), dtype)
+    x = gu.dev_bits16(x32, dtype).view(e, max_tokens, hidden)
+    qtype = scalar_types.uint4 if zp else scalar_types.uint4b8
+    marker = torch.full((e, max_tokens, hidden), 7.0, dtype=x.dtype, device=gu.DEV)
+    y = batched_fused_marlin_moe(x, torch.from_numpy(counts).to(gu.DEV), w1, w2, None, None, s1, s2, qtype.id,
+                                 w1_zeros=z1, w2_zeros=z2, output=marker)
+    torch.cuda.synchronize()
+    got = gu.host_f32(y)
+    for b in range(e):
+        rows = x32[b * max_tokens:b * max_tokens + counts[b]]
+        if counts[b]:
+            ids = np.full((counts[b], 1), b, dtype=np.int32)
+            want = _moe_reference(rows, ref13, ref2, ids, np.ones((counts[b], 1), np.float32), dtype)
+            max_ref = np.abs(want).max()
+            assert np.abs(got[b, :counts[b]] - want).max() <= 2e-2 * max_ref, (b, counts[b])
+        assert np.all(got[b, counts[b]:] == 7.0), "rows of invalid tokens must not be written"
+
+
 def test_fused_marlin_moe_replays_in_a_hip_graph():
     """The layer reads no device value on the host, so it can be recorded; every
     replay must reproduce the eager result, also after the routing changed."""

@@ -338,3 +338,29 @@ def test_moe_packed_zero_points_match_oracle():
     got = mu.moe_packed_to_marlin_zero_points(torch.from_numpy(packed.view(np.int32)), groups, n, 4)
     want = np.stack([mo.marlin_zero_points(zp[e], groups, n) for e in range(experts)])
     assert np.array_equal(got.numpy().view(np.uint32), want.view(np.uint32))
+
+
+def test_batched_moe_align_matches_docstring_example_and_oracle():
+    """The literal example of moe_align_block_size.py:129-162 (5 batches of 8
+    rows, blocks of 4, 2 / 3 / 0 / 6 / 8 valid rows).  Its expert_ids line lists
+    experts 5, which five batches cannot have; the kernel
+    (moe_align_sum_kernels.cu:70-81) gives a block the id of its batch, hence
+    0 1 3 3 4 4.  Then the torch version against the oracle on random counts."""
+    from sonar_amd.fused_moe import batched_moe_align_block_size
+    counts = [2, 3, 0, 6, 8]
+    want_ids = [0, 1, 40, 40, 8, 9, 10, 40, 24, 25, 26, 27, 28, 29, 40, 40, 32, 33, 34, 35, 36, 37, 38, 39] + [40] * 16
+    want_experts = [0, 1, 3, 3, 4, 4, -1, -1, -1, -1]
+    for fn in (mo.batched_moe_align_block_size,
+               lambda m, b, c: [t.numpy() for t in batched_moe_align_block_size(m, b, torch.tensor(c, dtype=torch.int32))]):
+        ids, experts, past = fn(8, 4, counts)
+        assert ids.tolist() == want_ids and experts.tolist() == want_experts and past.tolist() == [24]
+    rng = np.random.default_rng(3)
+    for _ in range(40):
+        batches = int(rng.integers(1, 12))
+        max_tokens = int(rng.integers(1, 70))
+        bs = int(rng.choice([4, 8, 16, 32, 48, 64]))
+        counts = rng.integers(0, max_tokens + 1, size=batches).astype(np.int32)
+        got = batched_moe_align_block_size(max_tokens, bs, torch.from_numpy(counts))
+        want = mo.batched_moe_align_block_size(max_tokens, bs, counts)
+        for g, w in zip(got, want):
+            assert g.dtype == torch.int32 and np.array_equal(g.numpy(), w), (batches, max_tokens, bs, counts)
