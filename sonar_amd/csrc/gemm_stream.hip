@@ -141,8 +141,8 @@ __device__ __forceinline__ void write_tiles(const StreamParams& p, int strip, in
 // Wavefront 0: a finished segment goes to C when it is the whole strip, else
 // to this workgroup's scratch slot.
 template <typename T, int MB>
-__device__ __forceinline__ void finish_segment(const StreamParams& p, int strip, int seg_begin, int seg_end,
-                                               int lane, const floatx4_t (&acc)[MB][4]) {
+__device__ __forceinline__ void finish_segment(const StreamParams& p, int part, int strip, int seg_begin,
+                                               int seg_end, int lane, const floatx4_t (&acc)[MB][4]) {
   const int strip_first = strip * p.units_per_strip;
   const int strip_end = strip_first + p.units_per_strip;
   if (seg_begin == strip_first && seg_end == strip_end) {
@@ -150,7 +150,7 @@ __device__ __forceinline__ void finish_segment(const StreamParams& p, int strip,
     return;
   }
   const int first = range_owner(strip_first, p.total_units, p.parts);
-  float4* slot = partial_slot(p, blockIdx.x, first);
+  float4* slot = partial_slot(p, part, first);
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
@@ -263,16 +263,28 @@ __device__ __forceinline__ void load_unit(UnitBuf<T, MB>& b, const StreamParams&
 }
 
 template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX>
-__global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const StreamParams p) {
+__global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const StreamParams params) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq<T>::Col Col;
   __shared__ float4 red[4][MB * 4][64];
+  // Several 64-row slabs can share a launch when no strip is shared between
+  // workgroups (nothing goes through the scratch slots): workgroup
+  // slab * grid_parts + part, ids of one part congruent mod 8 (one XCD).
+  StreamParams p = params;
+  const int part = blockIdx.x % p.grid_parts;
+  if (part >= p.parts) return;
+  {
+    const int slab = blockIdx.x / p.grid_parts;
+    p.a += (long)slab * 64 * p.lda;
+    p.c += (long)slab * 64 * p.size_n;
+    p.size_m = min(64, p.size_m - 64 * slab);
+  }
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col16 = lane & 15;
-  const int u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
-  const int u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
+  const int u_begin = range_begin(part, p.total_units, p.parts);
+  const int u_end = range_begin(part + 1, p.total_units, p.parts);
   const bool grouped = p.num_groups > 1;
   const uint32_t magic = magic_register();
 
@@ -340,7 +352,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
     }
 
     reduce_waves<MB, kWaves>(acc, red, wave, lane);
-    if (wave == 0) finish_segment<T, MB>(p, strip, seg_begin, seg_end, lane, acc);
+    if (wave == 0) finish_segment<T, MB>(p, part, strip, seg_begin, seg_end, lane, acc);
     seg_begin = seg_end;
   }
 }
@@ -387,16 +399,28 @@ __device__ __forceinline__ void load_unit8(UnitBuf8<T, MB>& b, const StreamParam
 }
 
 template <typename T, int MB>
-__global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const StreamParams p) {
+__global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const StreamParams params) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq8<T>::Col Col;
   __shared__ float4 red[4][MB * 4][64];
+  // Several 64-row slabs can share a launch when no strip is shared between
+  // workgroups (nothing goes through the scratch slots): workgroup
+  // slab * grid_parts + part, ids of one part congruent mod 8 (one XCD).
+  StreamParams p = params;
+  const int part = blockIdx.x % p.grid_parts;
+  if (part >= p.parts) return;
+  {
+    const int slab = blockIdx.x / p.grid_parts;
+    p.a += (long)slab * 64 * p.lda;
+    p.c += (long)slab * 64 * p.size_n;
+    p.size_m = min(64, p.size_m - 64 * slab);
+  }
 
   const int lane = threadIdx.x & 63;
   const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int col16 = lane & 15;
-  const int u_begin = range_begin(blockIdx.x, p.total_units, p.parts);
-  const int u_end = range_begin(blockIdx.x + 1, p.total_units, p.parts);
+  const int u_begin = range_begin(part, p.total_units, p.parts);
+  const int u_end = range_begin(part + 1, p.total_units, p.parts);
   const bool grouped = p.num_groups > 1;
   const uint32_t magic = magic_register();
 
@@ -452,7 +476,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
     }
 
     reduce_waves<MB, kWaves>(acc, red, wave, lane);
-    if (wave == 0) finish_segment<T, MB>(p, strip, seg_begin, seg_end, lane, acc);
+    if (wave == 0) finish_segment<T, MB>(p, part, strip, seg_begin, seg_end, lane, acc);
     seg_begin = seg_end;
   }
 }
@@ -1068,11 +1092,11 @@ __global__ __launch_bounds__(256) void permute_columns_kernel(const uint16_t* __
 template <typename T, int MB, bool HAS_ZP>
 void launch_stream(const StreamParams& p, bool has_perm, hipStream_t st) {
   if (p.g_idx) {  // row -> group lookup: symmetric weights, activations already permuted
-    if constexpr (!HAS_ZP) marlin_stream_kernel<T, MB, false, false, true><<<p.parts, kWaves * 64, 0, st>>>(p);
+    if constexpr (!HAS_ZP) marlin_stream_kernel<T, MB, false, false, true><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p);
   } else if (has_perm) {
-    marlin_stream_kernel<T, MB, HAS_ZP, true, false><<<p.parts, kWaves * 64, 0, st>>>(p);
+    marlin_stream_kernel<T, MB, HAS_ZP, true, false><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p);
   } else {
-    marlin_stream_kernel<T, MB, HAS_ZP, false, false><<<p.parts, kWaves * 64, 0, st>>>(p);
+    marlin_stream_kernel<T, MB, HAS_ZP, false, false><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p);
   }
 }
 
@@ -1089,10 +1113,10 @@ void launch_stream_mb(const StreamParams& p, bool has_perm, hipStream_t st) {
 template <typename T>
 void launch_stream8_mb(const StreamParams& p, hipStream_t st) {
   switch ((p.size_m + 15) / 16) {
-    case 1: marlin_stream8_kernel<T, 1><<<p.parts, kWaves * 64, 0, st>>>(p); break;
-    case 2: marlin_stream8_kernel<T, 2><<<p.parts, kWaves * 64, 0, st>>>(p); break;
-    case 3: marlin_stream8_kernel<T, 3><<<p.parts, kWaves * 64, 0, st>>>(p); break;
-    default: marlin_stream8_kernel<T, 4><<<p.parts, kWaves * 64, 0, st>>>(p); break;
+    case 1: marlin_stream8_kernel<T, 1><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 2: marlin_stream8_kernel<T, 2><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 3: marlin_stream8_kernel<T, 3><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    default: marlin_stream8_kernel<T, 4><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
   }
 }
 
@@ -1403,8 +1427,21 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   SONAR_REQUIRE(total_units * cus < (1LL << 31), "size_k * size_n = %ld x %ld is too large", (long)size_k,
                 (long)size_n);
   p.total_units = (int)total_units;
+  static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
+  const bool async_tile = tile_async_applies(chk.has_perm, num_groups, chk.group_size);
+  const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
+  // the row -> group lookup and 8-bit codes exist in the streaming kernels only
+  const bool use_tile = plan.tile && !no_tile && !chk.row_groups && chk.bits == 4 && !(slab_fast && p.unit_chunks == 4);
+  // More than 64 rows in the general kernels (8-bit codes, is_k_full = false,
+  // the tile path switched off) on a matrix of short strips: one workgroup per
+  // strip as well, so that every 64-row slab can run in the same launch and the
+  // slabs of a strip share its weights in L2, instead of one launch per slab
+  // that streams all of W again (8-bit, K = 4096, N = 11008, M = 512: 214 us as
+  // eight launches).
+  const bool row_slabs = !use_tile && !slab_fast && size_m > 64 && strip_per_workgroup &&
+                         total_units * n_strips < (1LL << 31);
   p.parts = p.total_units < cus ? p.total_units : cus;
-  if (strip_per_workgroup && p.unit_chunks == 4) p.parts = (int)n_strips;
+  if (strip_per_workgroup && (p.unit_chunks == 4 || row_slabs)) p.parts = (int)n_strips;
   p.slabs = 1;
   p.grid_parts = p.parts;
   p.sum_over_rings = 0;
@@ -1413,11 +1450,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   for (int i = 1; i < p.parts && !any_split; ++i)
     any_split = range_begin(i, p.total_units, p.parts) % p.units_per_strip != 0;
 
-  static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
-  const bool async_tile = tile_async_applies(chk.has_perm, num_groups, chk.group_size);
-  const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
-  // the row -> group lookup and 8-bit codes exist in the streaming kernels only
-  if (plan.tile && !no_tile && !chk.row_groups && chk.bits == 4 && !(slab_fast && p.unit_chunks == 4)) {
+  if (use_tile) {
     const size_t used = stream_scratch_bytes();
     return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
                      size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used,
@@ -1455,15 +1488,23 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
         rc = chk.has_zp ? launch_fast<__bf16, true>(p, unit_group_shift, half, row_blocks, st)
                         : launch_fast<__bf16, false>(p, unit_group_shift, half, row_blocks, st);
       if (rc) return rc;
-    } else if (chk.bits == 8) {
-      if (dtype == SONAR_DTYPE_F16) launch_stream8_mb<_Float16>(p, st);
-      else launch_stream8_mb<__bf16>(p, st);
-    } else if (dtype == SONAR_DTYPE_F16) {
-      if (chk.has_zp) launch_stream_mb<_Float16, true>(p, chk.has_perm, st);
-      else launch_stream_mb<_Float16, false>(p, chk.has_perm, st);
     } else {
-      if (chk.has_zp) launch_stream_mb<__bf16, true>(p, chk.has_perm, st);
-      else launch_stream_mb<__bf16, false>(p, chk.has_perm, st);
+      if (row_slabs && !any_split) {   // every 64-row slab in this one launch
+        p.size_m = (int)size_m;
+        p.slabs = (int)((size_m + 63) / 64);
+        p.grid_parts = (p.parts + 7) / 8 * 8;
+        m0 = size_m;
+      }
+      if (chk.bits == 8) {
+        if (dtype == SONAR_DTYPE_F16) launch_stream8_mb<_Float16>(p, st);
+        else launch_stream8_mb<__bf16>(p, st);
+      } else if (dtype == SONAR_DTYPE_F16) {
+        if (chk.has_zp) launch_stream_mb<_Float16, true>(p, chk.has_perm, st);
+        else launch_stream_mb<_Float16, false>(p, chk.has_perm, st);
+      } else {
+        if (chk.has_zp) launch_stream_mb<__bf16, true>(p, chk.has_perm, st);
+        else launch_stream_mb<__bf16, false>(p, chk.has_perm, st);
+      }
     }
     if (int rc = launch_status("marlin_stream_kernel")) return rc;
     if (any_split) {
