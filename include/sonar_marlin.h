@@ -145,7 +145,9 @@ int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
  *   c            dtype[M*top_k][N] contiguous
  *   b_q_weight   num_experts * K*N/8 words, each expert in b_layout order
  *   b_scales     dtype[num_experts][num_groups][N]; b_zeros / b_bias likewise
- *   g_idx, perm  int32[num_experts][K] or NULL
+ *   g_idx, perm  int32[num_experts][K] or NULL; with is_k_full == 0 (shards that
+ *                hold no whole group; uint4b8 only) g_idx is the group of
+ *                every sorted row and num_groups the groups of the whole matrix
  *   sorted_token_ids int32[sorted_len], expert_ids int32[ceil(sorted_len/bs)],
  *   num_tokens_past_padded int32[1] (read on the device), topk_weights
  *   float[M*top_k]

@@ -46,6 +46,7 @@ struct MoeParams {
   const uint16_t* scales;
   const uint32_t* zeros;
   const int32_t* perm;
+  const int32_t* g_idx;        // [experts][size_k] group of every (sorted) row; null when groups are runs of rows
   const int32_t* sorted_ids;
   const int32_t* expert_ids;
   const int32_t* num_post_pad;
@@ -85,7 +86,10 @@ struct MoeUnit {
   int group;
 };
 
-template <typename T, int MB, bool HAS_ZP, bool HAS_PERM>
+// HAS_GIDX (with HAS_PERM, symmetric weights): an act-order shard that does not
+// hold whole groups (is_k_full = false); every row finds its scale through g_idx
+// (marlin_moe_wna16/ops.cu:343-351).
+template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX>
 __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoeParams p) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq<T>::Col Col;
@@ -128,6 +132,7 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
   const uint16_t* scales = p.scales + expert_l * p.num_groups * p.size_n;
   const uint32_t* zeros = HAS_ZP ? p.zeros + expert_l * p.num_groups * (p.size_n / 8) : nullptr;
   const int32_t* perm = HAS_PERM ? p.perm + expert_l * p.size_k : nullptr;
+  const int32_t* row_group = HAS_GIDX ? p.g_idx + expert_l * p.size_k : nullptr;
   const bool grouped = p.num_groups > 1;
   const uint32_t magic = magic_register();
 
@@ -181,9 +186,21 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
           load_cols<T, HAS_ZP>(cols, scales, zeros, p.size_n, strip, g, col16, grouped);
         }
         const uint32_t words[4] = {cur.q[cc].x, cur.q[cc].y, cur.q[cc].z, cur.q[cc].w};
+        int row_groups[8];
+        if (HAS_GIDX) {  // the lane's eight rows of this chunk: k = 32 chunk + 8 (lane / 16) + t
+          const int4* gsrc = reinterpret_cast<const int4*>(row_group + (chunk0 + cc) * kChunkK + 8 * kb);
+          const int4 g0 = gsrc[0], g1 = gsrc[1];
+          row_groups[0] = g0.x, row_groups[1] = g0.y, row_groups[2] = g0.z, row_groups[3] = g0.w;
+          row_groups[4] = g1.x, row_groups[5] = g1.y, row_groups[6] = g1.z, row_groups[7] = g1.w;
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const vec8 w = Dq<T>::word(words[j], cols[j], magic);
+          vec8 w;
+          if (HAS_GIDX)
+            w = word_by_row_groups<T>(words[j], row_groups,
+                                      scales + strip * kStripN + scale_slot(16 * j + col16, true), p.size_n, magic);
+          else
+            w = Dq<T>::word(words[j], cols[j], magic);
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb) acc[mb][j] = Dq<T>::mfma(w, cur.a[cc][mb], acc[mb][j]);
         }
@@ -229,10 +246,13 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
 
 template <typename T, int MB, bool HAS_ZP>
 void launch_moe(const MoeParams& p, bool has_perm, int grid, hipStream_t st) {
-  if (has_perm)
-    marlin_moe_kernel<T, MB, HAS_ZP, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
-  else
-    marlin_moe_kernel<T, MB, HAS_ZP, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  if (has_perm && p.g_idx) {
+    if constexpr (!HAS_ZP) marlin_moe_kernel<T, MB, false, true, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  } else if (has_perm) {
+    marlin_moe_kernel<T, MB, HAS_ZP, true, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  } else {
+    marlin_moe_kernel<T, MB, HAS_ZP, false, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  }
 }
 
 template <typename T, bool HAS_ZP>
@@ -299,13 +319,17 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                   "b_type must be uint4b8 when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   const bool has_perm = perm != nullptr;
+  const bool row_groups = has_perm && !is_k_full;
   if (has_perm) {
-    if (!is_k_full)
-      return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False is not built yet");
     SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
+    if (row_groups && has_zp)
+      return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False and zero points is not built");
   }
   int group_size = (int)size_k;
-  if (num_groups > 1) {
+  if (row_groups) {
+    // the shard holds no whole groups: every row looks its group up in g_idx, and the
+    // kernels' own group arithmetic (one group of size_k rows) is unused
+  } else if (num_groups > 1) {
     SONAR_REQUIRE(size_k % num_groups == 0, "size_k = %ld, is not divisible by num_groups = %ld",
                   (long)size_k, (long)num_groups);
     group_size = (int)(size_k / num_groups);
@@ -346,6 +370,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
   p.scales = static_cast<const uint16_t*>(b_scales);
   p.zeros = b_zeros;
   p.perm = perm;
+  p.g_idx = row_groups ? g_idx : nullptr;
   p.sorted_ids = sorted_token_ids;
   p.expert_ids = expert_ids;
   p.num_post_pad = num_tokens_past_padded;

@@ -151,6 +151,54 @@ def test_random_moe_cases_against_oracle(case):
     test_moe_gemm_within_tolerance(case)
 
 
+@pytest.mark.parametrize("cfg", [(9, 4, 2, 16, "fp16", True), (70, 3, 2, 32, "bf16", False), (200, 2, 1, 64, "fp16", True)],
+                         ids=str)
+def test_moe_act_order_shard_without_whole_groups(cfg):
+    """Row-parallel shards of act-order experts (is_k_full = False; the
+    reference's scenario (133, 256, 256, 5, 2, 1, act_order, k_full = False),
+    tests/kernels/moe/test_moe.py:688-710): the shard's rows lie in all groups
+    and every row finds its scale through g_idx."""
+    m, e, top_k, bs, dtype, mul = cfg
+    k_full, n, g = 1024, 192, 128
+    lo, hi = 384, 768
+    k = hi - lo
+    native, scales, perms, g_sorted_all, w_ref = [], [], [], [], []
+    for i in range(e):
+        full = mo.make_layer(700 + i, k_full, n, g, dtype, act_order=True)
+        q, g_idx = full["q"][lo:hi], full["g_idx"][lo:hi]
+        assert np.bincount(g_idx, minlength=k_full // g).max() < g     # no whole group in the shard
+        w_ref.append(mo.dequantize(q, full["scales"], g, dtype, g_idx=g_idx))
+        g_sorted, order = mo.stable_sort_g_idx(g_idx)
+        perm = gu.dev_i32(order)
+        native.append(gu.to_gfx950(gu.gptq_repack(gu.dev_i32(mo.gptq_pack(q)), perm, k, n), k, n))
+        scales.append(gu.dev_bits16(mo.marlin_permute_scales(full["scales"], k_full, n, g), dtype))
+        perms.append(perm)
+        g_sorted_all.append(gu.dev_i32(g_sorted))
+    native, scales = torch.stack(native).contiguous(), torch.stack(scales).contiguous()
+    perm, g_dev = torch.stack(perms).contiguous(), torch.stack(g_sorted_all).contiguous()
+    topk_ids, topk_w = route(m + 1, m, e, top_k)
+    sorted_ids, expert_ids, past = mo.moe_align_block_size(topk_ids, bs, e)
+    a32 = mo.make_activations(m + 9, m, k, dtype, std=0.5)
+    a = gu.dev_bits16(a32, dtype)
+    lib = _lib.load()
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    c = torch.zeros((m * top_k, n), dtype=tdt, device=gu.DEV)
+    sid, eid = gu.dev_i32(sorted_ids), gu.dev_i32(expert_ids)
+    npp = gu.dev_i32(np.array([int(past[0])], dtype=np.int32))
+    tw = torch.from_numpy(topk_w.astype(np.float32).reshape(-1)).to(gu.DEV)
+    workspace = torch.zeros(1024, dtype=torch.int32, device=gu.DEV)
+    _lib.check(lib.sonar_moe_wna16_marlin_gemm(
+        gu.ptr(a), gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None, gu.ptr(scales), None, gu.ptr(g_dev),
+        gu.ptr(perm), gu.ptr(workspace), workspace.numel(), None, 0, gu.ptr(sid), sid.numel(), gu.ptr(eid),
+        gu.ptr(npp), gu.ptr(tw), bs, top_k, int(mul), e, gu.dtype_code(dtype), _lib.TYPE_UINT4B8, m, n, k,
+        k_full // g, 0, 0, 1, gu.stream()))
+    torch.cuda.synchronize()
+    want = mo.moe_gemm_reference(a32, w_ref, sorted_ids, expert_ids, int(past[0]), bs, top_k, m,
+                                 topk_w if mul else None, dtype)
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(c), want)
+    assert ok, worst
+
+
 def test_moe_skips_invalid_blocks_and_rows():
     """Blocks with expert id -1, blocks past num_tokens_past_padded and padding
     slots leave C untouched (marlin_template.h(moe):471-570)."""
