@@ -215,6 +215,9 @@ def moe_sweep(torch, gen, time_graph):
         torch.cuda.synchronize()
         out.append({"tokens": t, "gemm": "whole layer (eager)", "us": round((time.perf_counter() - t0) / reps * 1e6, 1)})
         print("moe", json.dumps(out[-1]), file=sys.stderr, flush=True)
+        # routing, both GEMMs, activation and sum recorded in one HIP graph
+        out.append({"tokens": t, "gemm": "whole layer (graph)", "us": round(time_graph(torch, layer, reps) * 1e6, 1)})
+        print("moe", json.dumps(out[-1]), file=sys.stderr, flush=True)
     return out
 
 
