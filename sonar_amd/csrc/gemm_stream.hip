@@ -55,9 +55,9 @@ struct StreamParams {
   int units_per_strip;
   int parts;  // number of workgroups of the streaming kernel
   int total_units;
-  // fast kernel only: the launch covers `slabs` blocks of 16 rows, workgroup
-  // slab * grid_parts + part works on rows 16 slab.. of part `part` (ids past
-  // `parts` inside a slab are padding)
+  // The launch covers `slabs` blocks of rows (16 or 32 in the fast kernel, 64 in
+  // the general kernels) times `grid_parts` >= parts workgroups per block
+  // (part_and_slab; parts past `parts` are padding)
   int slabs, grid_parts;
   // fast kernel only: the tiles of the cross-wavefront sum are parked on top of
   // the copy rings instead of behind them.  Allowed when every workgroup owns
@@ -84,6 +84,20 @@ __host__ __device__ __forceinline__ int range_begin(int i, int total, int parts)
 // Largest i with range_begin(i) <= x, given parts <= total.
 __host__ __device__ __forceinline__ int range_owner(int x, int total, int parts) {
   return (int)((((unsigned)x + 1u) * (unsigned)parts - 1u) / (unsigned)total);
+}
+// Workgroup id -> (part, slab) of a launch that covers `slabs` blocks of rows.
+// With several slabs grid_parts is a multiple of 8 and the slabs of a part get
+// consecutive ids on one XCD (ids congruent mod 8), so that they are dispatched
+// together and the second to ask for a weight chunk finds it in that XCD's L2.
+__device__ __forceinline__ void part_and_slab(const int grid_parts, const int slabs, int& part, int& slab) {
+  if (slabs == 1) {
+    part = blockIdx.x;
+    slab = 0;
+    return;
+  }
+  const int t = blockIdx.x >> 3;
+  slab = t % slabs;
+  part = (t / slabs) * 8 + (blockIdx.x & 7);
 }
 // Scratch slot of workgroup `w` for a strip whose first contributor is `first`.
 __device__ __forceinline__ float4* partial_slot(const StreamParams& p, int w, int first) {
@@ -268,13 +282,12 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
   typedef typename Dq<T>::Col Col;
   __shared__ float4 red[4][MB * 4][64];
   // Several 64-row slabs can share a launch when no strip is shared between
-  // workgroups (nothing goes through the scratch slots): workgroup
-  // slab * grid_parts + part, ids of one part congruent mod 8 (one XCD).
+  // workgroups (nothing goes through the scratch slots).
   StreamParams p = params;
-  const int part = blockIdx.x % p.grid_parts;
+  int part, slab;
+  part_and_slab(p.grid_parts, p.slabs, part, slab);
   if (part >= p.parts) return;
   {
-    const int slab = blockIdx.x / p.grid_parts;
     p.a += (long)slab * 64 * p.lda;
     p.c += (long)slab * 64 * p.size_n;
     p.size_m = min(64, p.size_m - 64 * slab);
@@ -404,13 +417,12 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
   typedef typename Dq8<T>::Col Col;
   __shared__ float4 red[4][MB * 4][64];
   // Several 64-row slabs can share a launch when no strip is shared between
-  // workgroups (nothing goes through the scratch slots): workgroup
-  // slab * grid_parts + part, ids of one part congruent mod 8 (one XCD).
+  // workgroups (nothing goes through the scratch slots).
   StreamParams p = params;
-  const int part = blockIdx.x % p.grid_parts;
+  int part, slab;
+  part_and_slab(p.grid_parts, p.slabs, part, slab);
   if (part >= p.parts) return;
   {
-    const int slab = blockIdx.x / p.grid_parts;
     p.a += (long)slab * 64 * p.lda;
     p.c += (long)slab * 64 * p.size_n;
     p.size_m = min(64, p.size_m - 64 * slab);
@@ -674,12 +686,14 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   constexpr int kPark = park_tiles(MB);       // tiles per wavefront and pass of the cross-wavefront sum
   constexpr int kPasses = 4 * MB / kPark;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  // The slabs of one part have ids congruent mod 8 (grid_parts is a multiple of
-  // 8 when there are several), so they run on one XCD and the second to ask
-  // for a weight chunk finds it in that XCD's L2.
   StreamParams p = params;
-  const int part = blockIdx.x % p.grid_parts;
-  const int slab = blockIdx.x / p.grid_parts;
+  int part, slab;
+  if constexpr (GROUPED) {   // strip-major inside a block of slots
+    part = blockIdx.x % p.grid_parts;
+    slab = blockIdx.x / p.grid_parts;
+  } else {
+    part_and_slab(p.grid_parts, p.slabs, part, slab);
+  }
   if (part >= p.parts) return;
   const int lane = threadIdx.x & 63;
   int row_id[MB] = {};  // grouped calls: the row of C that row (lane & 15) of block of rows mb goes to, or -1
