@@ -90,6 +90,31 @@ def time_graph(torch, fn, reps):
     return t0.elapsed_time(t1) * 1e-3 / reps
 
 
+def memory_yardsticks(torch):
+    """What the box sustains on plain streaming passes over 1 GiB, with the
+    framework's own kernels (not part of the product path): a reduction (reads
+    1 GiB) and a copy (reads and writes 1 GiB each).  Puts the GEMM's GB/s next
+    to a measured ceiling instead of the 8 TB/s headline alone."""
+    x = torch.empty(256 * 1024 * 1024, dtype=torch.float32, device="cuda:0").normal_()
+    y = torch.empty_like(x)
+    out = {}
+    for name, fn, nbytes in (("read_1GiB_GBps", lambda: x.sum(), x.numel() * 4),
+                             ("copy_1GiB_GBps", lambda: y.copy_(x), 2 * x.numel() * 4)):
+        for _ in range(3):
+            fn()
+        torch.cuda.synchronize()
+        t0 = torch.cuda.Event(enable_timing=True)
+        t1 = torch.cuda.Event(enable_timing=True)
+        t0.record()
+        for _ in range(10):
+            fn()
+        t1.record()
+        torch.cuda.synchronize()
+        out[name] = round(nbytes * 10 / (t0.elapsed_time(t1) * 1e-3) / 1e9, 1)
+    del x, y
+    return out
+
+
 def cpu_baseline(threads: int):
     """The layer's CPU path (int4 dequantise + fp32 torch.matmul) from the
     oracle, on the o_proj shape at M = 16."""
@@ -367,6 +392,7 @@ def main() -> int:
         out["variants"] = variants_sweep(torch, ops, gen, time_graph)
         out["moe"] = moe_sweep(torch, gen, time_graph)
 
+    out["yardsticks"] = memory_yardsticks(torch)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(min(os.cpu_count() or 1, 16))
     print(json.dumps(out))
