@@ -240,6 +240,59 @@ def test_moe_matches_dense_gemm_per_expert():
     assert ok, worst
 
 
+@pytest.mark.parametrize("tokens,k,n", [(16, 4096, 28672), (64, 14336, 4096), (256, 4096, 28672), (600, 14336, 4096)])
+def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n):
+    """Mixtral-8x7B expert shapes (8 experts, top 2, the block size of the
+    reference's rule), where the CPU oracle is too slow: every routed slot must
+    equal, within the GEMM tolerance, the dense op on the same token row and
+    the same expert's weights (the dense decode kernel is checked against the
+    oracle elsewhere).  Random device weights; the grouped call covers blocks
+    of 8, 32 and 64 slots, i.e. the grouped decode kernel with one and two
+    blocks of rows, its two-halves form and the tile kernel."""
+    e, top_k, dtype = 8, 2, torch.bfloat16
+    gen = torch.Generator(device=gu.DEV).manual_seed(tokens + n)
+    lib = _lib.load()
+    words = k * n // 8
+    native = torch.randint(-2 ** 31, 2 ** 31 - 1, (e, words), dtype=torch.int32, device=gu.DEV, generator=gen)
+    scales = (torch.rand((e, k // 128, n), device=gu.DEV, generator=gen) * 9e-3 + 1e-3).to(dtype)
+    a = torch.randn((tokens, k), device=gu.DEV, generator=gen).to(dtype)
+    topk_ids, topk_w = route(tokens, tokens, e, top_k)
+    bs = mo.moe_block_size_rule(tokens, top_k, e)
+    sorted_ids, expert_ids, past = mo.moe_align_block_size(topk_ids, bs, e)
+    sid, eid = gu.dev_i32(sorted_ids), gu.dev_i32(expert_ids)
+    npp = gu.dev_i32(np.array([int(past[0])], dtype=np.int32))
+    c = torch.zeros((tokens * top_k, n), dtype=dtype, device=gu.DEV)
+    workspace = torch.zeros(1024, dtype=torch.int32, device=gu.DEV)
+    nbytes = lib.sonar_moe_marlin_gemm_scratch_bytes(sid.numel(), bs, n, k)
+    scr = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=gu.DEV)
+    _lib.check(lib.sonar_moe_wna16_marlin_gemm(
+        gu.ptr(a), gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None, gu.ptr(scales), None, None, None,
+        gu.ptr(workspace), workspace.numel(), gu.ptr(scr), nbytes, gu.ptr(sid), sid.numel(), gu.ptr(eid),
+        gu.ptr(npp), None, bs, top_k, 0, e, _lib.DTYPE_BF16, _lib.TYPE_UINT4B8, tokens, n, k, k // 128, 1, 0, 1,
+        gu.stream()))
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(c.float()).all())
+    scale = float(c.float().abs().max())
+    checked = 0
+    for ex in range(e):
+        slots = np.nonzero(topk_ids.reshape(-1) == ex)[0][:16]      # up to 16 slots of this expert
+        if len(slots) == 0:
+            continue
+        rows = a[torch.from_numpy(slots // top_k).to(gu.DEV)].contiguous()
+        m = rows.shape[0]
+        dense = torch.empty((m, n), dtype=dtype, device=gu.DEV)
+        dscr = torch.empty(max(lib.sonar_marlin_gemm_scratch_bytes(m, n, k), 16), dtype=torch.uint8, device=gu.DEV)
+        _lib.check(lib.sonar_marlin_gemm(
+            gu.ptr(rows), k, gu.ptr(dense), gu.ptr(native[ex]), _lib.LAYOUT_GFX950, None, gu.ptr(scales[ex]), None,
+            None, None, gu.ptr(workspace), workspace.numel(), gu.ptr(dscr), dscr.numel(), _lib.DTYPE_BF16,
+            _lib.TYPE_UINT4B8, m, n, k, k // 128, 1, 0, 1, gu.stream()))
+        got = c[torch.from_numpy(slots).to(gu.DEV)].float()
+        err = float((got - dense.float()).abs().max())
+        assert err <= 1e-2 * scale, (ex, err, scale)
+        checked += m
+    assert checked >= min(16, tokens)
+
+
 def test_moe_error_paths():
     lib = _lib.load()
     ex = Experts(3, 2, 256, 128, 128, "fp16")
