@@ -23,16 +23,16 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
                   int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, hipStream_t st);
+                  int64_t num_groups, int group_size, int a_by_slot, hipStream_t st);
 size_t moe_tile_table_bytes(int64_t sorted_len, int64_t num_experts);
 // gemm_stream.hip: the 16-row decode kernel in grouped form, for few rows per expert
 bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t sorted_len, int64_t num_experts,
-                      int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size);
+                      int64_t a_rows, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size);
 int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, const void* scales,
                   const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t moe_block_size, int64_t top_k,
                   int mul_topk, int64_t num_experts, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, hipStream_t st);
+                  int64_t num_groups, int group_size, int a_by_slot, hipStream_t st);
 
 namespace {
 
@@ -58,6 +58,7 @@ struct MoeParams {
   int block_size, top_k, num_experts, num_blocks;
   int sorted_len;
   int mul_topk;
+  int a_by_slot;               // row of A = slot index (a column-permuted copy made per slot), else row id / top_k
 };
 
 template <typename T, bool HAS_PERM>
@@ -125,7 +126,8 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
   for (int mb = 0; mb < MB; ++mb) {
     const int id = slot_id[16 * mb + col16];
     // padding slots read row 0; their products are never stored
-    arow[mb] = p.a + (long)(id >= 0 ? id / p.top_k : 0) * p.size_k;
+    const int a_row = id < 0 ? 0 : (p.a_by_slot ? block * p.block_size + 16 * mb + col16 : id / p.top_k);
+    arow[mb] = p.a + (long)a_row * p.size_k;
   }
   const long expert_l = expert;
   const uint4* bsrc = p.b + (expert_l * p.strips + strip) * (long)p.chunks_per_strip * 64 + lane;
@@ -244,6 +246,39 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
   }
 }
 
+// Act-order with room in scratch: A'[slot][k] = A[row id / top_k][perm[expert][k]]
+// for every valid slot, once, so that the kernels without a gather can run on
+// A' (what the dense op does with permute_columns_kernel, here per slot because
+// every expert has its own permutation).  One thread per 8 columns.
+__global__ __launch_bounds__(256) void moe_permute_rows_kernel(const uint16_t* __restrict__ a,
+                                                              const int32_t* __restrict__ perm,
+                                                              const int32_t* __restrict__ sorted_ids,
+                                                              const int32_t* __restrict__ expert_ids,
+                                                              const int32_t* __restrict__ num_post_pad,
+                                                              uint16_t* __restrict__ out, int size_k, int top_k,
+                                                              int rows_total, int block_size, int sorted_len,
+                                                              int num_experts) {
+  const int per_row = size_k / 8;
+  const long total = (long)min(sorted_len, num_post_pad[0]) * per_row;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const int slot = (int)(i / per_row);
+    const int k0 = 8 * (int)(i - (long)slot * per_row);
+    const int expert = expert_ids[slot / block_size];
+    const int id = sorted_ids[slot];
+    if (expert < 0 || expert >= num_experts || id < 0 || id >= rows_total) continue;
+    const uint16_t* arow = a + (long)(id / top_k) * size_k;
+    const int32_t* pe = perm + (long)expert * size_k + k0;
+    const int4 p0 = *reinterpret_cast<const int4*>(pe);
+    const int4 p1 = *reinterpret_cast<const int4*>(pe + 4);
+    uint4 v;
+    v.x = (uint32_t)arow[p0.x] | ((uint32_t)arow[p0.y] << 16);
+    v.y = (uint32_t)arow[p0.z] | ((uint32_t)arow[p0.w] << 16);
+    v.z = (uint32_t)arow[p1.x] | ((uint32_t)arow[p1.y] << 16);
+    v.w = (uint32_t)arow[p1.z] | ((uint32_t)arow[p1.w] << 16);
+    *reinterpret_cast<uint4*>(out + (long)slot * size_k + k0) = v;
+  }
+}
+
 template <typename T, int MB, bool HAS_ZP>
 void launch_moe(const MoeParams& p, bool has_perm, int grid, hipStream_t st) {
   if (has_perm && p.g_idx) {
@@ -318,7 +353,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4B8,
                   "b_type must be uint4b8 when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
-  const bool has_perm = perm != nullptr;
+  bool has_perm = perm != nullptr;
   const bool row_groups = has_perm && !is_k_full;
   if (has_perm) {
     SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
@@ -347,12 +382,40 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                 (long)sorted_len);
 
   hipStream_t st = (hipStream_t)stream;
+  // Act-order with whole groups and room for a copy of A per slot behind the
+  // table of row tiles: permute the columns once and go on without a gather.
+  int a_by_slot = 0;
+  int64_t a_rows = size_m;
+  {
+    const size_t base = (sonar_moe_marlin_gemm_scratch_bytes(sorted_len, moe_block_size, size_n, size_k) + 255) & ~(size_t)255;
+    const size_t copy_bytes = (size_t)sorted_len * size_k * 2;
+    static const bool no_copy = getenv("SONAR_MARLIN_NO_MOE_PERMUTED_COPY") != nullptr;  // debugging aid
+    if (has_perm && !row_groups && !no_copy && scratch != nullptr && scratch_bytes >= base + copy_bytes &&
+        ((uintptr_t)scratch) % 16 == 0 && size_k % 8 == 0) {
+      uint16_t* a_copy = reinterpret_cast<uint16_t*>(static_cast<char*>(scratch) + base);
+      const long work = (long)sorted_len * (size_k / 8);
+      long grid = (work + 255) / 256;
+      if (grid > 16384) grid = 16384;
+      moe_permute_rows_kernel<<<(int)grid, 256, 0, st>>>(static_cast<const uint16_t*>(a), perm, sorted_token_ids,
+                                                         expert_ids, num_tokens_past_padded, a_copy, (int)size_k,
+                                                         (int)top_k, (int)(size_m * top_k), (int)moe_block_size,
+                                                         (int)sorted_len, (int)num_experts);
+      if (int rc = launch_status("moe_permute_rows_kernel")) return rc;
+      a = a_copy;
+      a_by_slot = 1;
+      a_rows = sorted_len;
+      has_perm = false;
+      perm = nullptr;
+      g_idx = nullptr;
+      scratch_bytes = base;   // what is left for the table of row tiles
+    }
+  }
   // Few rows per expert: the decode kernel, one workgroup per strip and 32 slots of a block
-  if (moe_fast_applies(has_perm, moe_block_size, sorted_len, num_experts, size_m, size_n, size_k, num_groups,
+  if (moe_fast_applies(has_perm, moe_block_size, sorted_len, num_experts, a_rows, size_n, size_k, num_groups,
                        group_size))
     return moe_fast_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
                          num_tokens_past_padded, topk_weights, moe_block_size, top_k, mul_topk_weights ? 1 : 0,
-                         num_experts, dtype, size_m, size_n, size_k, num_groups, group_size, st);
+                         num_experts, dtype, size_m, size_n, size_k, num_groups, group_size, a_by_slot, st);
   static const bool no_tile = getenv("SONAR_MARLIN_NO_MOE_TILE") != nullptr;  // debugging aid
   // Full blocks of 64 slots mean many rows per expert: the MFMA-tiled kernel
   if (moe_block_size == 64 && !has_perm && !no_tile && size_k % 64 == 0 && num_experts <= 1024 &&
@@ -360,7 +423,8 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
       scratch_bytes >= moe_tile_table_bytes(sorted_len, num_experts) && ((uintptr_t)scratch) % 4 == 0)
     return moe_tile_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
                          num_tokens_past_padded, topk_weights, top_k, mul_topk_weights ? 1 : 0, num_experts,
-                         static_cast<int32_t*>(scratch), dtype, size_m, size_n, size_k, num_groups, group_size, st);
+                         static_cast<int32_t*>(scratch), dtype, size_m, size_n, size_k, num_groups, group_size,
+                         a_by_slot, st);
 
   MoeParams p;
   p.a = static_cast<const uint16_t*>(a);
@@ -390,6 +454,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
   p.sorted_len = (int)sorted_len;
   p.num_blocks = (int)((sorted_len + moe_block_size - 1) / moe_block_size);
   p.mul_topk = mul_topk_weights ? 1 : 0;
+  p.a_by_slot = a_by_slot;
   const int64_t grid = (int64_t)p.num_blocks * p.strips;
   SONAR_REQUIRE(grid < (1LL << 31), "too many (block, strip) pairs: %ld", (long)grid);
   if (dtype == SONAR_DTYPE_F16) {

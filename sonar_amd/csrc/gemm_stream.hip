@@ -73,6 +73,7 @@ struct StreamParams {
   const float* topk_weights;
   int block_size, top_k, num_experts, rows_total, sorted_len, mul_topk;
   int sub_blocks;              // workgroups (of up to 32 rows) per block of slots and strip
+  int a_by_slot;               // row of A = slot index (a column-permuted copy made per slot), else row id / top_k
   long expert_b_stride;        // uint4 units between experts in b
   long expert_s_stride, expert_z_stride, expert_bias_stride;  // elements between experts
 };
@@ -739,8 +740,9 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
       const int r = 8 * h + (lane >> 3);
       int row = r < p.size_m ? r : p.size_m - 1;  // rows past M are never stored
       if constexpr (GROUPED) {                    // padding slots read row 0 and are never stored
-        const int id = moe_row_id(p, slab / p.sub_blocks, 32 * (slab % p.sub_blocks) + r);
-        row = id >= 0 ? id / p.top_k : 0;
+        const int in_block = 32 * (slab % p.sub_blocks) + r;
+        const int id = moe_row_id(p, slab / p.sub_blocks, in_block);
+        row = id >= 0 ? (p.a_by_slot ? (slab / p.sub_blocks) * p.block_size + in_block : id / p.top_k) : 0;
       }
       fl.a_off[h] = (uint32_t)((long)row * p.lda * 2 + 16 * ((lane & 7) ^ (lane >> 3)));
     }
@@ -1240,12 +1242,12 @@ bool fast_group_shift(int64_t num_groups, int group_size, int& unit_group_shift)
 // The grouped (mixture-of-experts) op can use the 16-row kernel when the expert
 // matrices meet its conditions (blocks of 48 or 64 slots as two halves).
 bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t sorted_len, int64_t num_experts,
-                      int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size) {
+                      int64_t a_rows, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size) {
   static const bool no_fast = getenv("SONAR_MARLIN_NO_MOE_FAST") != nullptr;  // debugging aid
   int shift;
   const int64_t n_strips = size_n / kStripN, units = size_k / (4 * kChunkK);
   if (no_fast || has_perm || size_k % (4 * kChunkK) != 0 || !fast_group_shift(num_groups, group_size, shift) ||
-      size_m * size_k * 2 >= (1LL << 31) || n_strips * units * n_strips >= (1LL << 31))
+      a_rows * size_k * 2 >= (1LL << 31) || n_strips * units * n_strips >= (1LL << 31))
     return false;
   if (moe_block_size < 64) return true;
   // 64-slot blocks also have the tile kernel, which wins once the experts have
@@ -1266,8 +1268,9 @@ int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t moe_block_size, int64_t top_k,
                   int mul_topk, int64_t num_experts, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, hipStream_t st) {
+                  int64_t num_groups, int group_size, int a_by_slot, hipStream_t st) {
   StreamParams p = {};
+  p.a_by_slot = a_by_slot;
   p.a = static_cast<const uint16_t*>(a);
   p.lda = size_k;
   p.c = static_cast<uint16_t*>(c);

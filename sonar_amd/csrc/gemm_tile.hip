@@ -57,6 +57,7 @@ struct TileParams {
   const float* topk_weights;
   const int32_t* tile_table;   // [0]: number of row tiles, then (first block, blocks, expert) per tile
   int rows_total, top_k, mul_topk;
+  int a_by_slot;               // grouped: row of A = slot index (a column-permuted copy made per slot), else row id / top_k
   long expert_b_stride;        // uint4 units between experts in b
   long expert_s_stride, expert_z_stride, expert_bias_stride;  // elements between experts
 };
@@ -366,7 +367,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     int row;
     if (GROUPED) {
       const int id = in_tile < tile_rows ? p.sorted_ids[first_slot + in_tile] : p.rows_total;
-      row = (unsigned)id < (unsigned)p.rows_total ? id / p.top_k : 0;  // padding slots read row 0, never stored
+      // padding slots read row 0, never stored
+      row = (unsigned)id < (unsigned)p.rows_total ? (p.a_by_slot ? first_slot + in_tile : id / p.top_k) : 0;
     } else {
       row = m0 + in_tile;
       if (row >= p.size_m) row = p.size_m - 1;  // rows past M are computed and never stored
@@ -765,7 +767,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   p.sorted_ids = nullptr;
   p.topk_weights = nullptr;
   p.tile_table = nullptr;
-  p.rows_total = p.top_k = p.mul_topk = 0;
+  p.rows_total = p.top_k = p.mul_topk = p.a_by_slot = 0;
   p.expert_b_stride = p.expert_s_stride = p.expert_z_stride = p.expert_bias_stride = 0;
   const bool zp = zeros != nullptr, pm = perm != nullptr;
   int rc;
@@ -826,7 +828,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
                   int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, hipStream_t st) {
+                  int64_t num_groups, int group_size, int a_by_slot, hipStream_t st) {
   const int max_tiles = moe_tile_max(sorted_len, num_experts);
   const int blocks_max = (int)((sorted_len + 63) / 64);
   moe_tile_table_kernel<<<1, 256, (size_t)blocks_max * sizeof(int32_t), st>>>(expert_ids, num_post_pad, blocks_max, 64,
@@ -860,6 +862,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.rows_total = (int)(size_m * top_k);
   p.top_k = (int)top_k;
   p.mul_topk = mul_topk;
+  p.a_by_slot = a_by_slot;
   p.expert_b_stride = (long)(size_k * size_n / 8 / 4);
   p.expert_s_stride = (long)(num_groups * size_n);
   p.expert_z_stride = (long)(num_groups * (size_n / 8));

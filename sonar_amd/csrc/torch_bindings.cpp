@@ -395,8 +395,11 @@ Tensor moe_wna16_marlin_gemm(
               "workspace must be a contiguous int32 GPU tensor");
 
   Tensor native = native_weights(b_q_weight, size_k, size_n, experts);
-  const size_t scratch_bytes =
+  size_t scratch_bytes =
       sonar_moe_marlin_gemm_scratch_bytes(sorted_token_ids.numel(), moe_block_size, size_n, size_k);
+  // act-order: room for the column-permuted copy of A, one row per slot, behind the table of row tiles
+  if (perm != nullptr && is_k_full)
+    scratch_bytes = ((scratch_bytes + 255) & ~(size_t)255) + (size_t)sorted_token_ids.numel() * size_k * 2;
   Tensor scratch;
   if (scratch_bytes > 0) scratch = at::empty({(int64_t)scratch_bytes}, a.options().dtype(at::kByte));
 

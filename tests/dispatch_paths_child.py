@@ -47,7 +47,8 @@ def grouped() -> None:
                  (700, 8, 2, 512, 128, 64, "bf16", True, False, True, 64, False),
                  (40, 4, 2, 256, 128, 128, "fp16", False, False, False, 16, True),
                  (3, 8, 2, 512, 256, 128, "bf16", True, False, True, 8, False),
-                 (130, 4, 2, 256, 320, -1, "fp16", False, False, True, 32, True)]:
+                 (130, 4, 2, 256, 320, -1, "fp16", False, False, True, 32, True),
+                 (50, 4, 2, 512, 128, 128, "bf16", False, True, False, 16, True)]:     # act-order
         print("grouped", case, flush=True)
         tm.test_moe_gemm_within_tolerance(case)   # raises on a mismatch
 

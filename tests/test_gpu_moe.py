@@ -55,7 +55,7 @@ class Experts:
             out[ids] = c
         return out
 
-    def gemm(self, a, sorted_ids, expert_ids, past, weights, bs, top_k, m, mul, scratch=True):
+    def gemm(self, a, sorted_ids, expert_ids, past, weights, bs, top_k, m, mul, scratch=True, permuted_copy=False):
         lib = _lib.load()
         tdt = torch.float16 if self.dtype == "fp16" else torch.bfloat16
         c = torch.zeros((m * top_k, self.n), dtype=tdt, device=gu.DEV)
@@ -64,6 +64,8 @@ class Experts:
         npp = gu.dev_i32(np.array([past], dtype=np.int32))
         tw = torch.from_numpy(weights.astype(np.float32).reshape(-1)).to(gu.DEV) if weights is not None else None
         nbytes = lib.sonar_moe_marlin_gemm_scratch_bytes(sid.numel(), bs, self.n, self.k) if scratch else 0
+        if permuted_copy:   # act-order: room for a column-permuted copy of A per slot
+            nbytes = (nbytes + 255) // 256 * 256 + sid.numel() * self.k * 2
         scr = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=gu.DEV) if scratch else None
         _lib.check(lib.sonar_moe_wna16_marlin_gemm(
             gu.ptr(a), gu.ptr(c), gu.ptr(self.native), _lib.LAYOUT_GFX950, gu.ptr(self.bias),
@@ -120,6 +122,11 @@ def test_moe_gemm_within_tolerance(case):
     assert np.all(np.isfinite(got))
     ok, *worst = mo.gemm_tolerance_ok(got, want)
     assert ok, worst
+    if act:   # with room for the permuted copy of A the kernels without a gather run
+        got = gu.host_f32(ex.gemm(a, sorted_ids, expert_ids, int(past[0]), topk_w, bs, top_k, m, mul,
+                                  permuted_copy=True))
+        ok, *worst = mo.gemm_tolerance_ok(got, want)
+        assert ok, worst
 
 
 def _random_moe_cases(count=int(os.environ.get("SONAR_RANDOM_CASES", "32"))):
