@@ -155,6 +155,20 @@ def test_gemm_row_strided_activations(gu, m, k, n):
     assert ok, (max_err, max_ref)
 
 
+@pytest.mark.parametrize("m", [32, 300])
+def test_gemm_subset_input_like_the_reference(gu, m):
+    """tests/kernels/quantization/test_marlin_gemm.py:494-537: A is the window
+    [8:m+8, 8:k+8] of a matrix twice as large (row stride 2k, 16-byte offset)."""
+    k, n = 1024, 2048
+    layer = gu.DeviceLayer(8, k, n, 128, "fp16")
+    big32 = mo.make_activations(6, 2 * m, 2 * k, "fp16")
+    a = gu.dev_bits16(big32, "fp16")[8:m + 8, 8:k + 8]
+    assert not a.is_contiguous() and a.data_ptr() % 16 == 0
+    c = layer.gemm(a, m)
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), mo.gemm_reference(big32[8:m + 8, 8:k + 8], layer.w_ref))
+    assert ok, (max_err, max_ref)
+
+
 def test_gemm_special_cases_reduce_to_row_sums(gu):
     """All codes 9, scale 1: W == 1, so C[m][n] is the row sum of A; and M = 0
     leaves the output untouched."""
