@@ -240,4 +240,23 @@ __device__ __forceinline__ typename Dq<T>::vec8 word_by_row_groups(uint32_t q, c
   return __builtin_bit_cast(vec8, u32x4_t{out[0], out[1], out[2], out[3]});
 }
 
+// The same for one packed word of 8-bit codes (four rows of one column, uint8b128):
+// the exact integers v - 128 times the scale of each row's group, rounded once.
+template <typename T>
+__device__ __forceinline__ uint2 word4_by_row_groups8(uint32_t q, const int* groups4, const uint16_t* scale_col,
+                                                      long group_stride, uint32_t magic) {
+  const uint2 w0 = Dq8<T>::word4(q, Dq8<T>::make_col(Dq<T>::from_float(1.0f)), magic);
+  const uint32_t regs[2] = {w0.x, w0.y};
+  uint32_t out[2];
+#pragma unroll
+  for (int r = 0; r < 2; ++r) {
+    const float lo = Dq<T>::to_float((uint16_t)(regs[r] & 0xffffu)) *
+                     Dq<T>::to_float(scale_col[(long)groups4[2 * r] * group_stride]);
+    const float hi = Dq<T>::to_float((uint16_t)(regs[r] >> 16)) *
+                     Dq<T>::to_float(scale_col[(long)groups4[2 * r + 1] * group_stride]);
+    out[r] = (uint32_t)Dq<T>::from_float(lo) | ((uint32_t)Dq<T>::from_float(hi) << 16);
+  }
+  return make_uint2(out[0], out[1]);
+}
+
 }  // namespace sonar

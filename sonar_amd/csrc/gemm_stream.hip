@@ -412,7 +412,7 @@ __device__ __forceinline__ void load_unit8(UnitBuf8<T, MB>& b, const StreamParam
   for (int j = 0; j < 4; ++j) b.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
 }
 
-template <typename T, int MB>
+template <typename T, int MB, bool HAS_GIDX>
 __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const StreamParams params) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq8<T>::Col Col;
@@ -474,10 +474,24 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
           }
           const uint32_t lo[4] = {cur.q[cc][0].x, cur.q[cc][0].y, cur.q[cc][0].z, cur.q[cc][0].w};
           const uint32_t hi[4] = {cur.q[cc][1].x, cur.q[cc][1].y, cur.q[cc][1].z, cur.q[cc][1].w};
+          int row_groups[8];
+          if (HAS_GIDX) {  // the lane's eight rows of this chunk: k = 32 chunk + 8 (lane / 16) + t
+            const int4* gsrc = reinterpret_cast<const int4*>(p.g_idx + (chunk0 + cc) * kChunkK + 8 * (lane >> 4));
+            const int4 g0 = gsrc[0], g1 = gsrc[1];
+            row_groups[0] = g0.x, row_groups[1] = g0.y, row_groups[2] = g0.z, row_groups[3] = g0.w;
+            row_groups[4] = g1.x, row_groups[5] = g1.y, row_groups[6] = g1.z, row_groups[7] = g1.w;
+          }
 #pragma unroll
           for (int j = 0; j < 4; ++j) {
-            const uint2 w_lo = Dq8<T>::word4(lo[j], cols[j], magic);
-            const uint2 w_hi = Dq8<T>::word4(hi[j], cols[j], magic);
+            uint2 w_lo, w_hi;
+            if (HAS_GIDX) {
+              const uint16_t* scale_col = p.scales + strip * kStripN + scale_slot(16 * j + col16, true);
+              w_lo = word4_by_row_groups8<T>(lo[j], row_groups, scale_col, p.size_n, magic);
+              w_hi = word4_by_row_groups8<T>(hi[j], row_groups + 4, scale_col, p.size_n, magic);
+            } else {
+              w_lo = Dq8<T>::word4(lo[j], cols[j], magic);
+              w_hi = Dq8<T>::word4(hi[j], cols[j], magic);
+            }
             const vec8 w = __builtin_bit_cast(vec8, u32x4_t{w_lo.x, w_lo.y, w_hi.x, w_hi.y});
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) acc[mb][j] = Dq<T>::mfma(w, cur.a[cc][mb], acc[mb][j]);
@@ -1039,6 +1053,7 @@ __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __rest
 template <typename T>
 __global__ __launch_bounds__(256) void marlin_dequant8_kernel(const uint4* __restrict__ b,
                                                              const uint16_t* __restrict__ scales,
+                                                             const int32_t* __restrict__ g_idx,
                                                              uint16_t* __restrict__ w_out, int size_n, int size_k,
                                                              int num_groups, int group_size, long total_blocks) {
   const int lane = threadIdx.x & 63;
@@ -1051,13 +1066,23 @@ __global__ __launch_bounds__(256) void marlin_dequant8_kernel(const uint4* __res
     const int strip = (int)(blk / blocks_per_strip);
     const int in_strip = (int)(blk % blocks_per_strip);
     const int chunk = in_strip >> 1, h = in_strip & 1;
-    const int g = grouped ? (chunk * kChunkK) / group_size : 0;
+    const int g = (grouped && !g_idx) ? (chunk * kChunkK) / group_size : 0;
     const uint16_t* srow = scales + (long)g * size_n + strip * kStripN;
     const uint4 q = b[blk * 64 + lane];
     const uint32_t words[4] = {q.x, q.y, q.z, q.w};
+    int row_groups[4] = {0, 0, 0, 0};
+    if (g_idx) {
+#pragma unroll
+      for (int t = 0; t < 4; ++t) row_groups[t] = g_idx[chunk * kChunkK + 8 * kb + 4 * h + t];
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint2 w = Dq8<T>::word4(words[j], Dq8<T>::make_col(srow[scale_slot(16 * j + col16, grouped)]), magic);
+      uint2 w;
+      if (g_idx)
+        w = word4_by_row_groups8<T>(words[j], row_groups, scales + strip * kStripN + scale_slot(16 * j + col16, true),
+                                    size_n, magic);
+      else
+        w = Dq8<T>::word4(words[j], Dq8<T>::make_col(srow[scale_slot(16 * j + col16, grouped)]), magic);
       const uint16_t bits[4] = {(uint16_t)(w.x & 0xffffu), (uint16_t)(w.x >> 16), (uint16_t)(w.y & 0xffffu),
                                 (uint16_t)(w.y >> 16)};
 #pragma unroll
@@ -1126,14 +1151,20 @@ void launch_stream_mb(const StreamParams& p, bool has_perm, hipStream_t st) {
   }
 }
 
+template <typename T, bool HAS_GIDX>
+void launch_stream8_gidx(const StreamParams& p, hipStream_t st) {
+  switch ((p.size_m + 15) / 16) {
+    case 1: marlin_stream8_kernel<T, 1, HAS_GIDX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 2: marlin_stream8_kernel<T, 2, HAS_GIDX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 3: marlin_stream8_kernel<T, 3, HAS_GIDX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    default: marlin_stream8_kernel<T, 4, HAS_GIDX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+  }
+}
+
 template <typename T>
 void launch_stream8_mb(const StreamParams& p, hipStream_t st) {
-  switch ((p.size_m + 15) / 16) {
-    case 1: marlin_stream8_kernel<T, 1><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    case 2: marlin_stream8_kernel<T, 2><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    case 3: marlin_stream8_kernel<T, 3><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    default: marlin_stream8_kernel<T, 4><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-  }
+  if (p.g_idx) launch_stream8_gidx<T, true>(p, st);
+  else launch_stream8_gidx<T, false>(p, st);
 }
 
 template <typename T, bool HAS_ZP, int WAVES, int MB, bool GROUPED>
@@ -1207,8 +1238,6 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
   if (out.has_perm) SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
   if (out.row_groups) {
     // marlin.cu:343-351,763-769: group_size = 0, every row looks its group up
-    if (out.bits == 8)
-      return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False and 8-bit weights is not built");
     if (out.has_zp)
       return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False and zero points is not built");
     out.group_size = 0;
@@ -1554,8 +1583,9 @@ extern "C" int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout, co
     const long total_blocks = (size_n / kStripN) * (size_k / 16);
     long grid = (total_blocks + 3) / 4;
     if (grid > 8192) grid = 8192;
-    if (dtype == SONAR_DTYPE_F16) marlin_dequant8_kernel<_Float16><<<(int)grid, 256, 0, st>>>(b, s, w, n, k, ng, gs, total_blocks);
-    else marlin_dequant8_kernel<__bf16><<<(int)grid, 256, 0, st>>>(b, s, w, n, k, ng, gs, total_blocks);
+    const int32_t* gi8 = chk.row_groups ? g_idx : nullptr;
+    if (dtype == SONAR_DTYPE_F16) marlin_dequant8_kernel<_Float16><<<(int)grid, 256, 0, st>>>(b, s, gi8, w, n, k, ng, gs, total_blocks);
+    else marlin_dequant8_kernel<__bf16><<<(int)grid, 256, 0, st>>>(b, s, gi8, w, n, k, ng, gs, total_blocks);
     return launch_status("marlin_dequant8_kernel");
   }
   const int32_t* gi = chk.row_groups ? g_idx : nullptr;

@@ -434,6 +434,52 @@ def test_act_order_shard_without_whole_groups(gu, dtype, m):
     assert call(base) != 0 and b"more scratch" in lib.sonar_marlin_last_error()
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("m", [1, 40, 200])
+def test_act_order_shard_without_whole_groups_8bit(gu, dtype, m):
+    """The same for uint8b128 codes (the reference's test grid runs GPTQ-INT8
+    with act-order and is_k_full = False, test_marlin_gemm.py:86-91,304-333)."""
+    from sonar_amd import _lib
+    k_full, n, g = 1024, 192, 128
+    lo, hi = 128, 640
+    k = hi - lo
+    rng = np.random.default_rng(5 + m)
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    scales = mo.round_to_dtype(rng.uniform(1e-4, 1e-3, size=(k_full // g, n)).astype(np.float32), dtype)
+    g_idx = (rng.permutation(k_full) // g).astype(np.int32)[lo:hi]
+    assert np.bincount(g_idx, minlength=k_full // g).max() < g
+    w_ref = mo.dequantize(q, scales, g, dtype, g_idx=g_idx, num_bits=8)
+    g_sorted, order = mo.stable_sort_g_idx(g_idx)
+    perm, g_dev = gu.dev_i32(order), gu.dev_i32(g_sorted)
+    lib = _lib.load()
+    marlin = torch.empty((k // 16, 4 * n), dtype=torch.int32, device=gu.DEV)
+    _lib.check(lib.sonar_gptq_marlin_repack(gu.ptr(gu.dev_i32(mo.pack_rows8(q))), gu.ptr(perm), gu.ptr(marlin), k, n, 8,
+                                            gu.stream()))
+    native = torch.empty_like(marlin)
+    _lib.check(lib.sonar_marlin8_to_gfx950(gu.ptr(marlin), gu.ptr(native), k, n, gu.stream()))
+    s_dev = gu.dev_bits16(mo.marlin_permute_scales(scales, k_full, n, g), dtype)
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    w = torch.empty((k, n), dtype=tdt, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_dequant(gu.ptr(native), _lib.LAYOUT_GFX950, gu.ptr(s_dev), None, gu.ptr(g_dev),
+                                        gu.ptr(w), gu.dtype_code(dtype), _lib.TYPE_UINT8B128, n, k, k_full // g, 0,
+                                        gu.stream()))
+    torch.cuda.synchronize()
+    assert np.array_equal(gu.host_f32(w), w_ref[order])
+    a32 = mo.make_activations(m, m, k, dtype, std=0.5)
+    a = gu.dev_bits16(a32, dtype)
+    c = torch.empty((m, n), dtype=tdt, device=gu.DEV)
+    workspace = torch.zeros(torch.cuda.get_device_properties(0).multi_processor_count, dtype=torch.int32,
+                            device=gu.DEV)
+    scratch = torch.empty(lib.sonar_marlin_gemm_scratch_bytes(m, n, k) + m * k * 2, dtype=torch.uint8, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_gemm(
+        gu.ptr(a), k, gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None, gu.ptr(s_dev), None, gu.ptr(g_dev),
+        gu.ptr(perm), gu.ptr(workspace), workspace.numel(), gu.ptr(scratch), scratch.numel(),
+        gu.dtype_code(dtype), _lib.TYPE_UINT8B128, m, n, k, k_full // g, 0, 0, 1, gu.stream()))
+    torch.cuda.synchronize()
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), mo.gemm_reference(a32, w_ref))
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+
+
 @pytest.mark.parametrize("dtype,m,k,n", [("fp16", 4096, 4096, 4096), ("bf16", 8192, 4096, 6144),
                                           ("fp16", 1024, 14336, 4096), ("fp16", 256, 4096, 28672),
                                           ("fp16", 4096, 4096, 6144)])   # 384 tiles: the last 128 split in two

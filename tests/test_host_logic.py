@@ -364,3 +364,57 @@ def test_batched_moe_align_matches_docstring_example_and_oracle():
         want = mo.batched_moe_align_block_size(max_tokens, bs, counts)
         for g, w in zip(got, want):
             assert g.dtype == torch.int32 and np.array_equal(g.numpy(), w), (batches, max_tokens, bs, counts)
+
+
+def test_marlin_test_utils_match_the_oracle_layout():
+    """get_weight_perm / marlin_weights (marlin_utils_test.py:31-121) against the
+    oracle's restatement of the same recipe and its closed form, 4 and 8 bits;
+    gptq_pack / awq_pack against the oracle's packings."""
+    from sonar_amd import marlin_utils_test as mt
+    from sonar_amd import quant_utils as qu
+    assert np.array_equal(mt.get_weight_perm(4).numpy(), mo.marlin_weight_perm_recipe())
+    assert np.array_equal(mt.get_weight_perm(8).numpy(), mo.marlin_weight_perm_recipe8())
+    rng = np.random.default_rng(0)
+    q = rng.integers(0, 16, size=(128, 192)).astype(np.int32)
+    got = mt.marlin_weights(torch.from_numpy(q), 128, 192, 4, mt.get_weight_perm(4)).numpy()
+    assert np.array_equal(got.view(np.uint32).ravel(), mo.marlin_pack_closed_form(q).view(np.uint32).ravel())
+    q8 = rng.integers(0, 256, size=(64, 128)).astype(np.int32)
+    got = mt.marlin_weights(torch.from_numpy(q8), 64, 128, 8, mt.get_weight_perm(8)).numpy()
+    assert np.array_equal(got.view(np.uint32).ravel(), mo.marlin_pack8_closed_form(q8).view(np.uint32).ravel())
+    assert np.array_equal(qu.gptq_pack(torch.from_numpy(q), 4, 128, 192).numpy(), mo.gptq_pack(q))
+    assert np.array_equal(qu.awq_pack(torch.from_numpy(q), 4, 128, 192).numpy(), mo.awq_pack(q))
+    assert np.array_equal(qu.gptq_pack(torch.from_numpy(q8), 8, 64, 128).numpy(), mo.pack_rows8(q8))
+
+
+def test_quantize_weights_on_hand_worked_groups():
+    """quant_utils.py:588-679 on columns whose answer is known: a symmetric
+    group spanning [-8, 7] has scale 1 and codes value + 8; an asymmetric group
+    spanning [-3, 12] has scale 1 and zero point 3; and in general the codes
+    are in range, w_ref = (code - zero) * scale and |w - w_ref| <= scale / 2."""
+    from sonar_amd import quant_utils as qu
+    from sonar_amd.scalar_type import scalar_types as st
+    col = torch.tensor([-8.0, 7.0, 0.0, 3.0, -1.0, 2.0, -5.0, 6.0]).repeat(4)      # one group of 32 rows
+    w = torch.stack([col, 0.5 * col], dim=1)
+    w_ref, q, s, zp = qu.quantize_weights(w, st.uint4b8, 32)
+    assert zp is None and s.tolist() == [[1.0, 0.5]]
+    assert torch.equal(q[:, 0], (col + 8).int()) and torch.equal(q[:, 1], (col + 8).int())
+    assert torch.equal(w_ref, w)
+    col = torch.tensor([-3.0, 12.0, 0.0, 5.0]).repeat(8)
+    w_ref, q, s, zp = qu.quantize_weights(col.view(-1, 1), st.uint4, 32, zero_points=True)
+    assert s.item() == 1.0 and zp.item() == 3 and torch.equal(q[:, 0], (col + 3).int())
+    assert torch.equal(w_ref[:, 0], col)
+    gen = torch.Generator().manual_seed(1)
+    w = torch.randn((256, 64), generator=gen)
+    for qt, zero in ((st.uint4b8, False), (st.uint8b128, False), (st.uint4, True)):
+        w_ref, q, s, zp = qu.quantize_weights(w, qt, 64, zero_points=zero)
+        top = 2 ** qt.size_bits - 1
+        assert q.min() >= 0 and q.max() <= top and s.shape == (4, 64)
+        z = zp.repeat_interleave(64, 0) if zero else (top + 1) // 2
+        assert torch.allclose(w_ref, (q - z).float() * s.repeat_interleave(64, 0))
+        inside = (q > 0) & (q < top)        # not clamped
+        assert ((w - w_ref).abs()[inside] <= 0.5 * s.repeat_interleave(64, 0)[inside] + 1e-6).all()
+    # act-order: rows permuted, g_idx names the group each row came from; sorting restores runs of groups
+    w_ref, q, s, g_idx, rand_perm = qu.gptq_quantize_weights(w, st.uint4b8, 64, True)
+    assert torch.equal(g_idx, (rand_perm // 64).int())
+    q_sorted, g_sorted, sort_indices = qu.sort_weights(q, g_idx)
+    assert torch.equal(g_sorted, torch.arange(256).int() // 64) and torch.equal(q_sorted, q[sort_indices.long()])
