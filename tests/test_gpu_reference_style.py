@@ -150,3 +150,144 @@ def test_marlin_gemm_with_bias(size_m):
     output_ref = torch.matmul(a_input, w_ref) + b_bias.view(1, -1)
     torch.cuda.synchronize()
     assert compute_max_diff(output, output_ref) < 0.04
+
+
+# ---------------------------------------------------------------------------
+# tests/kernels/moe/test_moe.py:129-143, 688-1010 of the reference: the fused
+# Marlin MoE layer against a plain torch mixture of experts on the dequantised
+# weights, atol 4e-2, over the reference's scenarios for integer weights.
+MOE_CONFIGS = [
+    {"b_type": scalar_types.uint4, "group_blocks": [-1, 2, 4, 8]},
+    {"b_type": scalar_types.uint4b8, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]},
+]
+MARLIN_MOE_SCENARIOS = [
+    # (m, n, k, e, topk, ep_size, act_order, is_k_full)
+    (1, 128, 256, 5, 2, 1, False, True),
+    (1, 1024, 2048, 5, 2, 1, False, True),
+    (133, 256, 256, 5, 2, 1, False, True),
+    (133, 1024, 2048, 12, 3, 1, False, True),
+    (128, 256, 256, 5, 2, 1, False, True),
+    (128, 1024, 2048, 12, 3, 1, False, True),
+    (64, 1024, 2048, 12, 3, 4, False, True),
+    (1, 1024, 2048, 5, 2, 1, True, True),
+    (133, 256, 256, 5, 2, 1, True, False),
+]
+
+
+def _moe_cases():
+    cases = []
+    for cfg in MOE_CONFIGS:
+        for group_blocks in cfg["group_blocks"]:
+            group_size = group_blocks if group_blocks <= 0 else group_blocks * 16
+            for (m, n, k, e, topk, ep_size, act_order, is_k_full) in MARLIN_MOE_SCENARIOS:
+                if act_order and not cfg.get("support_act_order", False):
+                    continue
+                if group_size > 0 and k % group_size != 0:
+                    continue
+                if act_order and group_size in (-1, k, n):
+                    continue
+                if group_size in (k, n):
+                    continue
+                cases.append((cfg["b_type"], group_size, m, n, k, e, topk, ep_size, act_order, is_k_full))
+    return cases
+
+
+def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None):
+    """MarlinMoEWeightData.make (test_moe.py:774-892): every expert's (N, K)
+    matrix quantised and laid out on its own, then stacked."""
+    from sonar_amd.marlin_utils import marlin_permute_bias
+    from sonar_amd.marlin_utils_test import awq_marlin_quantize, marlin_quantize
+    k = w.shape[-1]
+    out = {"w_ref": [], "qweight": [], "scales": [], "zeros": [], "g_idx": [], "sort_indices": [], "bias": []}
+    for i in range(w.shape[0]):
+        if quant_type == scalar_types.uint4:
+            w_ref, qweight, scales, zeros = awq_marlin_quantize(w[i].transpose(1, 0), quant_type, group_size)
+            out["zeros"].append(zeros)
+        else:
+            w_ref, qweight, scales, g_idx, sort_indices, _ = marlin_quantize(
+                w[i].transpose(1, 0), quant_type, group_size, act_order, torch.randperm(k))
+            out["g_idx"].append(g_idx)
+            out["sort_indices"].append(sort_indices)
+        out["w_ref"].append(w_ref.T)
+        out["qweight"].append(qweight)
+        out["scales"].append(scales)
+        if bias is not None:
+            out["bias"].append(marlin_permute_bias(bias[i]))
+    return {name: (torch.stack(v).contiguous() if v else None) for name, v in out.items()}
+
+
+def _torch_experts(a, w1, w2, topk_weight, topk_ids, expert_map=None, b1=None, b2=None):
+    """Plain mixture of experts on (E, 2N, K) / (E, K, N) matrices: for every
+    token and routed expert silu(x W1_gate^T) * (x W1_up^T) through W2^T, summed
+    with the routing weights; experts mapped to -1 contribute nothing."""
+    m, k = a.shape
+    n = w2.shape[-1]
+    out = torch.zeros((m, k), dtype=torch.float32, device=a.device)
+    a32 = a.float()
+    for ex in torch.unique(topk_ids).tolist():
+        local = ex if expert_map is None else int(expert_map[ex])
+        if local < 0:
+            continue
+        rows, slot = torch.nonzero(topk_ids == ex, as_tuple=True)
+        h = a32[rows] @ w1[local].float().T
+        if b1 is not None:
+            h = h + b1[local].float()
+        h = h.to(a.dtype).float()
+        act = (torch.nn.functional.silu(h[:, :n]) * h[:, n:]).to(a.dtype).float()
+        y = act @ w2[local].float().T
+        if b2 is not None:
+            y = y + b2[local].float()
+        out.index_add_(0, rows, y.to(a.dtype).float() * topk_weight[rows, slot].float().unsqueeze(1))
+    return out.to(a.dtype)
+
+
+@pytest.mark.parametrize("b_type,group_size,m,n,k,e,topk,ep_size,act_order,is_k_full", _moe_cases(), ids=str)
+def test_fused_marlin_moe(b_type, group_size, m, n, k, e, topk, ep_size, act_order, is_k_full):
+    from sonar_amd.fused_moe import fused_marlin_moe
+    torch.manual_seed(1)
+    dtype = torch.float16
+    a = torch.randn((m, k), device="cuda", dtype=dtype) / 10
+    w1 = torch.randn((e, 2 * n, k), device="cuda", dtype=dtype) / 10
+    w2 = torch.randn((e, k, n), device="cuda", dtype=dtype) / 10
+    e_map = None
+    if ep_size > 1:
+        local_e = e // ep_size
+        e_ids = torch.randperm(e, device="cuda")[:local_e]
+        e_map = torch.full((e,), -1, device="cuda", dtype=torch.int32)
+        e_map[e_ids] = torch.arange(local_e, device="cuda", dtype=torch.int32)
+        w1, w2 = w1[e_ids], w2[e_ids]
+    d1 = _marlin_moe_weights(w1, b_type, group_size, act_order)
+    d2 = _marlin_moe_weights(w2, b_type, group_size, act_order)
+    score = torch.randn((m, e), device="cuda", dtype=dtype)
+    topk_weights, topk_ids = torch.topk(torch.softmax(score, dim=-1, dtype=torch.float32), topk)
+    want = _torch_experts(a, d1["w_ref"], d2["w_ref"], topk_weights, topk_ids, e_map)
+    got = fused_marlin_moe(a, d1["qweight"], d2["qweight"], None, None, d1["scales"], d2["scales"], topk_weights,
+                           topk_ids.to(torch.int32), global_num_experts=e, expert_map=e_map, g_idx1=d1["g_idx"],
+                           g_idx2=d2["g_idx"], sort_indices1=d1["sort_indices"], sort_indices2=d2["sort_indices"],
+                           w1_zeros=d1["zeros"], w2_zeros=d2["zeros"], quant_type_id=b_type.id, is_k_full=is_k_full)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(got, want, atol=4e-2, rtol=0)
+
+
+@pytest.mark.parametrize("m", [1, 256])
+def test_fused_marlin_moe_with_bias(m):
+    """test_moe.py:1013-1090: 32 experts, top 4, N = K = 2048, biases on both GEMMs."""
+    from sonar_amd.fused_moe import fused_marlin_moe
+    torch.manual_seed(0)
+    e, topk, n, k, group_size = 32, 4, 2048, 2048, 128
+    dtype = torch.half
+    a = torch.randn((m, k), device="cuda", dtype=dtype) / 10
+    w1 = torch.randn((e, 2 * n, k), device="cuda", dtype=dtype) / 10
+    w2 = torch.randn((e, k, n), device="cuda", dtype=dtype) / 10
+    b_bias1 = torch.randn((e, 2 * n), device="cuda", dtype=dtype) / 10
+    b_bias2 = torch.randn((e, k), device="cuda", dtype=dtype) / 10
+    d1 = _marlin_moe_weights(w1, scalar_types.uint4b8, group_size, False, b_bias1)
+    d2 = _marlin_moe_weights(w2, scalar_types.uint4b8, group_size, False, b_bias2)
+    score = torch.randn((m, e), device="cuda", dtype=dtype)
+    topk_weights, topk_ids = torch.topk(torch.softmax(score, dim=-1, dtype=torch.float32), topk)
+    want = _torch_experts(a, d1["w_ref"], d2["w_ref"], topk_weights, topk_ids, None, b_bias1, b_bias2)
+    got = fused_marlin_moe(a, d1["qweight"], d2["qweight"], d1["bias"], d2["bias"], d1["scales"], d2["scales"],
+                           topk_weights, topk_ids.to(torch.int32), global_num_experts=e, expert_map=None,
+                           quant_type_id=scalar_types.uint4b8.id, is_k_full=True)
+    torch.cuda.synchronize()
+    torch.testing.assert_close(got, want, atol=4e-2, rtol=0)
