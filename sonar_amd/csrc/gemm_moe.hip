@@ -78,6 +78,43 @@ __device__ __forceinline__ typename Dq<T>::vec8 moe_load_a(const uint16_t* arow,
   return __builtin_bit_cast(vec8, v);
 }
 
+// Wavefront 0, after the cross-wavefront sum: row `id` of C for every valid slot
+// of the block, with the expert's bias and, when asked, the routing weight.
+template <typename T, int MB>
+__device__ __forceinline__ void moe_scatter(const MoeParams& p, const floatx4_t (&acc)[MB][4], const int* slot_id,
+                                            long expert_l, int strip, int lane) {
+  const int col16 = lane & 15;
+  const uint16_t* bias = p.bias ? p.bias + expert_l * p.size_n + strip * kStripN : nullptr;
+  const int n_in = 4 * (lane >> 4);
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb) {
+    const int id = slot_id[16 * mb + col16];
+    if (id < 0) continue;
+    float tw = 1.f;
+    // the routing weight is rounded to the activation type and the product is
+    // formed and rounded in that type (marlin_template.h:1893-1897)
+    if (p.mul_topk) tw = Dq<T>::to_float(Dq<T>::from_float(p.topk_weights[id]));
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int nl = 16 * j + n_in;
+      const floatx4_t v = acc[mb][j];
+      float r[4] = {v.x, v.y, v.z, v.w};
+      uint16_t o[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) {
+        float x = r[t];
+        if (bias) x += Dq<T>::to_float(bias[scale_slot(nl + t, false)]);
+        o[t] = Dq<T>::from_float(x);
+        if (p.mul_topk) o[t] = Dq<T>::from_float(Dq<T>::to_float(o[t]) * tw);
+      }
+      uint2 packed;
+      packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+      packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+      *reinterpret_cast<uint2*>(p.c + (long)id * p.size_n + strip * kStripN + nl) = packed;
+    }
+  }
+}
+
 template <typename T, int MB>
 struct MoeUnit {
   uint4 q[4];
@@ -214,36 +251,146 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
 
   reduce_waves<MB, kMoeWaves>(acc, red, wave, lane);
   if (wave != 0) return;
+  moe_scatter<T, MB>(p, acc, slot_id, expert_l, strip, lane);
+}
 
-  const uint16_t* bias = p.bias ? p.bias + expert_l * p.size_n + strip * kStripN : nullptr;
-  const int n_in = 4 * (lane >> 4);
+// The same for 8-bit codes (uint8b128, symmetric): a 32-row chunk is two 1-KiB
+// blocks of 16 rows.  No gather of A: act-order experts come here through the
+// per-slot permuted copy (a_by_slot).  HAS_GIDX: every row finds its scale
+// through g_idx (is_k_full = false).
+template <typename T, int MB>
+struct MoeUnit8 {
+  static constexpr int kChunks = MB >= 3 ? 2 : 4;   // two units of this size and the accumulators fit the register file
+  uint4 q[kChunks][2];
+  typename Dq<T>::vec8 a[kChunks][MB];
+  uint32_t sbits[4];
+  int group;
+};
+
+template <typename T, int MB, bool HAS_GIDX>
+__global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe8_kernel(const MoeParams p) {
+  typedef typename Dq<T>::vec8 vec8;
+  typedef typename Dq8<T>::Col Col;
+  __shared__ float4 red[4][MB * 4][64];
+  __shared__ int slot_id[16 * MB];
+
+  const int lane = threadIdx.x & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
+  const int col16 = lane & 15, kb = lane >> 4;
+  const int block = blockIdx.x / p.strips;
+  const int strip = blockIdx.x - block * p.strips;
+
+  // the whole workgroup leaves together: nothing below is reached by a part of it
+  const int past = p.num_post_pad[0];
+  if (block * p.block_size >= past) return;
+  const int expert = p.expert_ids[block];
+  if (expert < 0 || expert >= p.num_experts) return;
+
+  const int rows_total = p.size_m * p.top_k;
+  if (threadIdx.x < 16 * MB) {
+    int id = -1;
+    const int at = block * p.block_size + (int)threadIdx.x;
+    if ((int)threadIdx.x < p.block_size && at < p.sorted_len) {
+      id = p.sorted_ids[at];
+      if (id < 0 || id >= rows_total) id = -1;
+    }
+    slot_id[threadIdx.x] = id;
+  }
+  __syncthreads();
+
+  const uint16_t* arow[MB];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     const int id = slot_id[16 * mb + col16];
-    if (id < 0) continue;
-    float tw = 1.f;
-    // the routing weight is rounded to the activation type and the product is
-    // formed and rounded in that type (marlin_template.h:1893-1897)
-    if (p.mul_topk) tw = Dq<T>::to_float(Dq<T>::from_float(p.topk_weights[id]));
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int nl = 16 * j + n_in;
-      const floatx4_t v = acc[mb][j];
-      float r[4] = {v.x, v.y, v.z, v.w};
-      uint16_t o[4];
-#pragma unroll
-      for (int t = 0; t < 4; ++t) {
-        float x = r[t];
-        if (bias) x += Dq<T>::to_float(bias[scale_slot(nl + t, false)]);
-        o[t] = Dq<T>::from_float(x);
-        if (p.mul_topk) o[t] = Dq<T>::from_float(Dq<T>::to_float(o[t]) * tw);
-      }
-      uint2 packed;
-      packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
-      packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
-      *reinterpret_cast<uint2*>(p.c + (long)id * p.size_n + strip * kStripN + nl) = packed;
-    }
+    // padding slots read row 0; their products are never stored
+    const int a_row = id < 0 ? 0 : (p.a_by_slot ? block * p.block_size + 16 * mb + col16 : id / p.top_k);
+    arow[mb] = p.a + (long)a_row * p.size_k;
   }
+  const long expert_l = expert;
+  const uint4* bsrc = p.b + (expert_l * p.strips + strip) * (long)p.chunks_per_strip * 128 + lane;
+  const uint16_t* scales = p.scales + expert_l * p.num_groups * p.size_n;
+  const int32_t* row_group = HAS_GIDX ? p.g_idx + expert_l * p.size_k : nullptr;
+  const bool grouped = p.num_groups > 1;
+  const uint32_t magic = magic_register();
+
+  auto load_unit = [&](MoeUnit8<T, MB>& u, int unit) {
+    const int chunk0 = unit * p.unit_chunks;
+#pragma unroll
+    for (int cc = 0; cc < MoeUnit8<T, MB>::kChunks; ++cc)
+      if (cc < p.unit_chunks) {
+        u.q[cc][0] = bsrc[(long)(chunk0 + cc) * 128];
+        u.q[cc][1] = bsrc[(long)(chunk0 + cc) * 128 + 64];
+#pragma unroll
+        for (int mb = 0; mb < MB; ++mb)
+          u.a[cc][mb] = moe_load_a<T, false>(arow[mb], nullptr, (chunk0 + cc) * kChunkK + 8 * kb);
+      }
+    const int g = grouped ? (chunk0 * kChunkK) / p.group_size : 0;
+    u.group = g;
+    const uint16_t* srow = scales + (long)g * p.size_n + strip * kStripN;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) u.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
+  };
+
+  floatx4_t acc[MB][4];
+#pragma unroll
+  for (int mb = 0; mb < MB; ++mb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+
+  MoeUnit8<T, MB> cur, nxt;
+  int mine = wave;
+  if (mine < p.units_per_strip) load_unit(cur, mine);
+  while (mine < p.units_per_strip) {
+    const int next = mine + kMoeWaves;
+    if (next < p.units_per_strip) load_unit(nxt, next);
+    Col cols[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) cols[j] = Dq8<T>::make_col((uint16_t)cur.sbits[j]);
+    int cur_group = cur.group;
+    const int chunk0 = mine * p.unit_chunks;
+#pragma unroll
+    for (int cc = 0; cc < MoeUnit8<T, MB>::kChunks; ++cc) {
+      if (cc < p.unit_chunks) {
+        const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
+        if (g != cur_group) {  // groups smaller than a unit
+          cur_group = g;
+          const uint16_t* srow = scales + (long)g * p.size_n + strip * kStripN;
+#pragma unroll
+          for (int j = 0; j < 4; ++j) cols[j] = Dq8<T>::make_col(srow[scale_slot(16 * j + col16, grouped)]);
+        }
+        const uint32_t lo[4] = {cur.q[cc][0].x, cur.q[cc][0].y, cur.q[cc][0].z, cur.q[cc][0].w};
+        const uint32_t hi[4] = {cur.q[cc][1].x, cur.q[cc][1].y, cur.q[cc][1].z, cur.q[cc][1].w};
+        int row_groups[8];
+        if (HAS_GIDX) {  // the lane's eight rows of this chunk: k = 32 chunk + 8 (lane / 16) + t
+          const int4* gsrc = reinterpret_cast<const int4*>(row_group + (chunk0 + cc) * kChunkK + 8 * kb);
+          const int4 g0 = gsrc[0], g1 = gsrc[1];
+          row_groups[0] = g0.x, row_groups[1] = g0.y, row_groups[2] = g0.z, row_groups[3] = g0.w;
+          row_groups[4] = g1.x, row_groups[5] = g1.y, row_groups[6] = g1.z, row_groups[7] = g1.w;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint2 w_lo, w_hi;
+          if (HAS_GIDX) {
+            const uint16_t* scale_col = scales + strip * kStripN + scale_slot(16 * j + col16, true);
+            w_lo = word4_by_row_groups8<T>(lo[j], row_groups, scale_col, p.size_n, magic);
+            w_hi = word4_by_row_groups8<T>(hi[j], row_groups + 4, scale_col, p.size_n, magic);
+          } else {
+            w_lo = Dq8<T>::word4(lo[j], cols[j], magic);
+            w_hi = Dq8<T>::word4(hi[j], cols[j], magic);
+          }
+          const vec8 w = __builtin_bit_cast(vec8, u32x4_t{w_lo.x, w_lo.y, w_hi.x, w_hi.y});
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb) acc[mb][j] = Dq<T>::mfma(w, cur.a[cc][mb], acc[mb][j]);
+        }
+      }
+    }
+    cur = nxt;
+    mine = next;
+  }
+
+  reduce_waves<MB, kMoeWaves>(acc, red, wave, lane);
+  if (wave != 0) return;
+  moe_scatter<T, MB>(p, acc, slot_id, expert_l, strip, lane);
 }
 
 // Act-order with room in scratch: A'[slot][k] = A[row id / top_k][perm[expert][k]]
@@ -283,10 +430,28 @@ template <typename T, int MB, bool HAS_ZP>
 void launch_moe(const MoeParams& p, bool has_perm, int grid, hipStream_t st) {
   if (has_perm && p.g_idx) {
     if constexpr (!HAS_ZP) marlin_moe_kernel<T, MB, false, true, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  } else if (p.g_idx) {   // rows already permuted into a copy of A, groups still looked up per row
+    if constexpr (!HAS_ZP) marlin_moe_kernel<T, MB, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
   } else if (has_perm) {
     marlin_moe_kernel<T, MB, HAS_ZP, true, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
   } else {
     marlin_moe_kernel<T, MB, HAS_ZP, false, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  }
+}
+
+template <typename T, int MB>
+void launch_moe8(const MoeParams& p, int grid, hipStream_t st) {
+  if (p.g_idx) marlin_moe8_kernel<T, MB, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  else marlin_moe8_kernel<T, MB, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
+}
+
+template <typename T>
+void launch_moe8_mb(const MoeParams& p, int grid, hipStream_t st) {
+  switch ((p.block_size + 15) / 16) {
+    case 1: launch_moe8<T, 1>(p, grid, st); break;
+    case 2: launch_moe8<T, 2>(p, grid, st); break;
+    case 3: launch_moe8<T, 3>(p, grid, st); break;
+    default: launch_moe8<T, 4>(p, grid, st); break;
   }
 }
 
@@ -342,16 +507,17 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                 "size_n = %ld, is not divisible by min_thread_n = %d", (long)size_n, kStripN);
   SONAR_REQUIRE(b_scales != nullptr, "b_scales must not be NULL");
   SONAR_REQUIRE(num_groups >= 1, "num_groups = %ld must be >= 1", (long)num_groups);
-  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4)
+  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4 && b_type_id != SONAR_TYPE_UINT8B128)
     return fail(SONAR_E_UNSUPPORTED,
-                "b_type id %ld is not built here: only uint4b8 (GPTQ) and uint4 (AWQ) weights are",
+                "b_type id %ld is not built here: only uint4b8, uint8b128 (GPTQ) and uint4 (AWQ) weights are",
                 (long)b_type_id);
   const bool has_zp = b_zeros != nullptr;
+  const bool bits8 = b_type_id == SONAR_TYPE_UINT8B128;
   if (has_zp)
     SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4, "b_type must be u4 or u8 when has_zp = True");
   else
-    SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4B8,
-                  "b_type must be uint4b8 when has_zp = False (uint4 needs b_zeros)");
+    SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4B8 || bits8,
+                  "b_type must be uint4b8 or uint8b128 when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   bool has_perm = perm != nullptr;
   const bool row_groups = has_perm && !is_k_full;
@@ -390,7 +556,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     const size_t base = (sonar_moe_marlin_gemm_scratch_bytes(sorted_len, moe_block_size, size_n, size_k) + 255) & ~(size_t)255;
     const size_t copy_bytes = (size_t)sorted_len * size_k * 2;
     static const bool no_copy = getenv("SONAR_MARLIN_NO_MOE_PERMUTED_COPY") != nullptr;  // debugging aid
-    if (has_perm && !row_groups && !no_copy && scratch != nullptr && scratch_bytes >= base + copy_bytes &&
+    if (has_perm && !no_copy && scratch != nullptr && scratch_bytes >= base + copy_bytes &&
         ((uintptr_t)scratch) % 16 == 0 && size_k % 8 == 0) {
       uint16_t* a_copy = reinterpret_cast<uint16_t*>(static_cast<char*>(scratch) + base);
       const long work = (long)sorted_len * (size_k / 8);
@@ -406,19 +572,25 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
       a_rows = sorted_len;
       has_perm = false;
       perm = nullptr;
-      g_idx = nullptr;
+      if (!row_groups) g_idx = nullptr;   // shards without whole groups still look every row's group up
       scratch_bytes = base;   // what is left for the table of row tiles
     }
   }
+  if (bits8 && has_perm)
+    return fail(SONAR_E_INVALID,
+                "act-order with 8-bit expert weights needs sorted_len * size_k * 2 more scratch bytes "
+                "(the column-permuted copy of A per slot)");
   // Few rows per expert: the decode kernel, one workgroup per strip and 32 slots of a block
-  if (moe_fast_applies(has_perm, moe_block_size, sorted_len, num_experts, a_rows, size_n, size_k, num_groups,
+  if (!bits8 && !row_groups &&
+      moe_fast_applies(has_perm, moe_block_size, sorted_len, num_experts, a_rows, size_n, size_k, num_groups,
                        group_size))
     return moe_fast_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
                          num_tokens_past_padded, topk_weights, moe_block_size, top_k, mul_topk_weights ? 1 : 0,
                          num_experts, dtype, size_m, size_n, size_k, num_groups, group_size, a_by_slot, st);
   static const bool no_tile = getenv("SONAR_MARLIN_NO_MOE_TILE") != nullptr;  // debugging aid
   // Full blocks of 64 slots mean many rows per expert: the MFMA-tiled kernel
-  if (moe_block_size == 64 && !has_perm && !no_tile && size_k % 64 == 0 && num_experts <= 1024 &&
+  if (moe_block_size == 64 && !has_perm && !bits8 && !row_groups && !no_tile && size_k % 64 == 0 &&
+      num_experts <= 1024 &&
       (num_groups == 1 || group_size % 64 == 0) && scratch != nullptr &&
       scratch_bytes >= moe_tile_table_bytes(sorted_len, num_experts) && ((uintptr_t)scratch) % 4 == 0)
     return moe_tile_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
@@ -457,6 +629,15 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
   p.a_by_slot = a_by_slot;
   const int64_t grid = (int64_t)p.num_blocks * p.strips;
   SONAR_REQUIRE(grid < (1LL << 31), "too many (block, strip) pairs: %ld", (long)grid);
+  if (bits8) {
+    if (p.block_size > 32 && p.unit_chunks == 4) {   // MoeUnit8 holds two chunks from three blocks of rows on
+      p.unit_chunks = 2;
+      p.units_per_strip = p.chunks_per_strip / 2;
+    }
+    if (dtype == SONAR_DTYPE_F16) launch_moe8_mb<_Float16>(p, (int)grid, st);
+    else launch_moe8_mb<__bf16>(p, (int)grid, st);
+    return launch_status("marlin_moe8_kernel");
+  }
   if (dtype == SONAR_DTYPE_F16) {
     if (has_zp) launch_moe_mb<_Float16, true>(p, has_perm, (int)grid, st);
     else launch_moe_mb<_Float16, false>(p, has_perm, (int)grid, st);

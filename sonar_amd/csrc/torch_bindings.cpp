@@ -329,8 +329,10 @@ Tensor moe_wna16_marlin_gemm(
   TORCH_CHECK(size_k % 16 == 0 && size_k / 16 == b_q_weight.size(1),
               "Shape mismatch: b_q_weight.size(1) = ", b_q_weight.size(1), ", size_k = ", size_k,
               ", tile_size = ", 16);
-  TORCH_CHECK(b_q_weight.size(2) % 16 == 0 && b_q_weight.size(2) / 16 * 8 == size_n,
-              "size_n = ", size_n, ", actual_size_n = ", b_q_weight.size(2) / 16 * 8);
+  const int bits = b_type_id == SONAR_TYPE_UINT8B128 ? 8 : 4;
+  const int64_t pack_factor = 32 / bits;
+  TORCH_CHECK(b_q_weight.size(2) % 16 == 0 && b_q_weight.size(2) / 16 * pack_factor == size_n,
+              "size_n = ", size_n, ", actual_size_n = ", b_q_weight.size(2) / 16 * pack_factor);
   TORCH_CHECK(b_q_weight.is_cuda() && b_q_weight.is_contiguous() && b_q_weight.scalar_type() == at::kInt,
               "b_q_weight must be a contiguous int32 GPU tensor");
   TORCH_CHECK(b_scales.is_cuda() && b_scales.is_contiguous(), "b_scales is not a contiguous GPU tensor");
@@ -381,7 +383,8 @@ Tensor moe_wna16_marlin_gemm(
     TORCH_CHECK(z.dim() == 3 && z.size(1) == num_groups && z.size(2) == size_n / 8,
                 "b_zeros must be (E, num_groups, size_n / 8)");
   } else {
-    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8, "b_type must be uint4b8 when has_zp = False. Got = uint4");
+    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT8B128,
+                "b_type must be uint4b8 or uint8b128 when has_zp = False. Got = uint4");
   }
   TORCH_CHECK(sorted_token_ids.is_cuda() && sorted_token_ids.scalar_type() == at::kInt &&
                   sorted_token_ids.is_contiguous(), "sorted_token_ids must be a contiguous int32 GPU tensor");
@@ -394,11 +397,11 @@ Tensor moe_wna16_marlin_gemm(
   TORCH_CHECK(workspace.is_cuda() && workspace.scalar_type() == at::kInt && workspace.is_contiguous(),
               "workspace must be a contiguous int32 GPU tensor");
 
-  Tensor native = native_weights(b_q_weight, size_k, size_n, experts);
+  Tensor native = native_weights(b_q_weight, size_k, size_n, experts, bits);
   size_t scratch_bytes =
       sonar_moe_marlin_gemm_scratch_bytes(sorted_token_ids.numel(), moe_block_size, size_n, size_k);
   // act-order: room for the column-permuted copy of A, one row per slot, behind the table of row tiles
-  if (perm != nullptr && is_k_full)
+  if (perm != nullptr)
     scratch_bytes = ((scratch_bytes + 255) & ~(size_t)255) + (size_t)sorted_token_ids.numel() * size_k * 2;
   Tensor scratch;
   if (scratch_bytes > 0) scratch = at::empty({(int64_t)scratch_bytes}, a.options().dtype(at::kByte));

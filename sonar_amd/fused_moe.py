@@ -20,7 +20,7 @@ from . import ops
 from .marlin_utils import marlin_make_workspace_new
 from .scalar_type import ScalarType, scalar_types
 
-_SUPPORTED = {t.id: t for t in (scalar_types.uint4, scalar_types.uint4b8)}
+_SUPPORTED = {t.id: t for t in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128)}
 
 
 def moe_block_size(num_tokens: int, top_k: int, num_experts: int) -> int:
@@ -222,8 +222,8 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
     w2: (E, N/16, 2K); scales (E, groups, 2N) / (E, groups, K); topk_weights
     fp32 [M, top_k]; topk_ids [M, top_k].  Returns [M, K]."""
     if quant_type_id not in _SUPPORTED:
-        raise NotImplementedError(f"quant type id {quant_type_id}: only uint4 and uint4b8 expert weights "
-                                  "are built")
+        raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8 and uint8b128 expert "
+                                  "weights are built")
     if input_dtype is not None:
         raise NotImplementedError("8-bit activations are not built")
     quant_type = _SUPPORTED[quant_type_id]
@@ -231,7 +231,7 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
     E = w1.shape[0]
     topk = topk_ids.shape[1]
     assert w1.shape[1] * 16 == K, "Hidden size mismatch w1"
-    assert w2.shape[2] // 2 == K, "Hidden size mismatch w2"
+    assert w2.shape[2] // (_SUPPORTED[quant_type_id].size_bits // 2) == K, "Hidden size mismatch w2"
     assert hidden_states.is_contiguous(), "Hidden_states must be contiguous"
     assert w1.is_contiguous(), "Expert weights1 must be contiguous"
     assert w2.is_contiguous(), "Expert weights2 must be contiguous"
@@ -280,8 +280,8 @@ def batched_fused_marlin_moe(hidden_states: torch.Tensor, expert_num_tokens: tor
     routing weights are ones.  Returns [E, max_tokens, K]; rows of invalid tokens
     are not written."""
     if quant_type_id not in _SUPPORTED:
-        raise NotImplementedError(f"quant type id {quant_type_id}: only uint4 and uint4b8 expert weights "
-                                  "are built")
+        raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8 and uint8b128 expert "
+                                  "weights are built")
     assert hidden_states.ndim == 3, f"hidden states must be batched. e.g. [B, MAX_TOKENS, K].But got {hidden_states.size()}"
     B, max_tokens, K = hidden_states.shape
     E = w1.shape[0]
@@ -290,7 +290,7 @@ def batched_fused_marlin_moe(hidden_states: torch.Tensor, expert_num_tokens: tor
     assert expert_num_tokens.size(0) == E
     assert B == E, "Batch must be as big as number of experts as the tokens are sorted into the batch/expert they belong to"
     assert w1.shape[1] * 16 == K, "Hidden size mismatch w1"
-    assert w2.shape[2] // 2 == K, "Hidden size mismatch w2"
+    assert w2.shape[2] // (_SUPPORTED[quant_type_id].size_bits // 2) == K, "Hidden size mismatch w2"
     assert w1.is_contiguous() and w2.is_contiguous(), "Expert weights must be contiguous"
     block_size_m = 64
     for b_m in (8, 16, 32, 48, 64):
