@@ -143,13 +143,15 @@ int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
  * dtype(topk_weights[id]) when mul_topk_weights != 0.
  *   a            dtype[M][K] contiguous
  *   c            dtype[M*top_k][N] contiguous
- *   b_q_weight   num_experts * K*N/8 words, each expert in b_layout order
+ *   b_q_weight   num_experts * K*N/8 words (K*N/4 for uint8b128), each expert
+ *                in b_layout order; b_type_id uint4b8, uint4 or uint8b128
  *   b_scales     dtype[num_experts][num_groups][N]; b_zeros / b_bias likewise
  *   scratch      sonar_moe_marlin_gemm_scratch_bytes(); act-order calls run 4 to
  *                20 times faster with sorted_len * K * 2 bytes more behind that
- *                size rounded up to 256 (a column-permuted copy of A per slot)
+ *                size rounded up to 256 (a column-permuted copy of A per slot;
+ *                required for act-order with uint8b128)
  *   g_idx, perm  int32[num_experts][K] or NULL; with is_k_full == 0 (shards that
- *                hold no whole group; uint4b8 only) g_idx is the group of
+ *                hold no whole group; no zero points) g_idx is the group of
  *                every sorted row and num_groups the groups of the whole matrix
  *   sorted_token_ids int32[sorted_len], expert_ids int32[ceil(sorted_len/bs)],
  *   num_tokens_past_padded int32[1] (read on the device), topk_weights
