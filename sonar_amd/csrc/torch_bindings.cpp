@@ -20,6 +20,7 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/library.h>
 
+#include <iterator>
 #include <mutex>
 #include <optional>
 #include <unordered_map>
@@ -54,7 +55,7 @@ int dtype_code(const Tensor& a) {
 
 // ---------------------------------------------------------------- weight cache
 struct NativeEntry {
-  Tensor source;
+  c10::weak_intrusive_ptr<c10::TensorImpl> source;   // the Marlin tensor, not kept alive by the cache
   Tensor native;
   int64_t size_k, size_n, experts;
   uint32_t version;
@@ -71,8 +72,10 @@ Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, 
   {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     auto it = g_cache.find(key);
-    if (it != g_cache.end() && it->second.size_k == size_k && it->second.size_n == size_n &&
-        it->second.experts == experts && it->second.version == version_of(b_q_weight))
+    if (it != g_cache.end() && !it->second.source.expired() &&
+        it->second.source._unsafe_get_target() == b_q_weight.unsafeGetTensorImpl() &&
+        it->second.size_k == size_k && it->second.size_n == size_n && it->second.experts == experts &&
+        it->second.version == version_of(b_q_weight))
       return it->second.native;
   }
   Tensor native = at::empty_like(b_q_weight);
@@ -85,7 +88,12 @@ Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, 
                               : sonar_marlin_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
                                                        current_stream(b_q_weight)));
   std::lock_guard<std::mutex> lock(g_cache_mutex);
-  g_cache[key] = NativeEntry{b_q_weight, native, size_k, size_n, experts, version_of(b_q_weight)};
+  // Weights whose Marlin tensor is gone (a layer that was reloaded or dropped)
+  // leave the cache with their streaming-order copies.
+  for (auto it = g_cache.begin(); it != g_cache.end();)
+    it = it->second.source.expired() ? g_cache.erase(it) : std::next(it);
+  g_cache.insert_or_assign(key, NativeEntry{c10::weak_intrusive_ptr<c10::TensorImpl>(b_q_weight.getIntrusivePtr()),
+                                            native, size_k, size_n, experts, version_of(b_q_weight)});
   return native;
 }
 

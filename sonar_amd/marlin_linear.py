@@ -129,7 +129,15 @@ class MarlinLinearKernel:
         if c.has_g_idx:
             g_idx, g_idx_sort_indices = marlin_sort_g_idx(getattr(layer, self.w_gidx_name))
             setattr(layer, self.w_gidx_name, g_idx)
-            layer.g_idx_sort_indices = g_idx_sort_indices
+            # A reload keeps the tensor the GEMM (and any recorded graph) reads: new
+            # values are copied into it (marlin.py:160-163, replace_parameter with
+            # prefer_copy; tests/model_executor/model_loader/test_reload.py:235-258).
+            held = getattr(layer, "g_idx_sort_indices", None)
+            if (isinstance(held, torch.Tensor) and held.shape == g_idx_sort_indices.shape
+                    and held.dtype == g_idx_sort_indices.dtype and held.device == g_idx_sort_indices.device):
+                held.data.copy_(g_idx_sort_indices)
+            else:
+                layer.g_idx_sort_indices = torch.nn.Parameter(g_idx_sort_indices, requires_grad=False)
         else:
             setattr(layer, self.w_gidx_name, marlin_make_empty_g_idx(device))
             layer.g_idx_sort_indices = marlin_make_empty_g_idx(device)

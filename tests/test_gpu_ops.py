@@ -75,6 +75,31 @@ def test_marlin_gemm_op_and_weight_cache(dtype, m):
     assert ops.marlin_weight_cache_clear() >= 1
 
 
+def test_weight_cache_lets_go_of_dropped_weights():
+    """The streaming-order copy of a weight whose Marlin tensor the caller has
+    dropped (a reloaded layer) leaves the cache at the next conversion."""
+    from sonar_amd import ops
+    from sonar_amd.scalar_type import scalar_types
+    k, n, m = 256, 128, 4
+    a = gu.dev_bits16(mo.make_activations(1, m, k, "fp16"), "fp16")
+    empty = torch.empty(0, dtype=torch.int32, device=gu.DEV)
+
+    def run(dl):
+        ops.marlin_gemm(a, None, dl.marlin, None, dl.scales, None, None, empty, empty, empty, dl.workspace,
+                        scalar_types.uint4b8, m, n, k, True, False, True, False)
+
+    ops.marlin_weight_cache_clear()
+    first, second = gu.DeviceLayer(1, k, n, 128, "fp16"), gu.DeviceLayer(2, k, n, 128, "fp16")
+    run(first)
+    run(second)
+    assert ops.marlin_weight_cache_clear() == 2
+    run(first)
+    del first                      # the only holder of its Marlin tensor
+    run(second)
+    torch.cuda.synchronize()
+    assert ops.marlin_weight_cache_clear() == 1
+
+
 def test_marlin_gemm_op_rejects_like_the_reference():
     from sonar_amd import ops
     from sonar_amd.scalar_type import scalar_types

@@ -418,3 +418,43 @@ def test_quantize_weights_on_hand_worked_groups():
     assert torch.equal(g_idx, (rand_perm // 64).int())
     q_sorted, g_sorted, sort_indices = qu.sort_weights(q, g_idx)
     assert torch.equal(g_sorted, torch.arange(256).int() // 64) and torch.equal(q_sorted, q[sort_indices.long()])
+
+
+def test_marlin_post_load_preserves_runtime_tensor_addresses(monkeypatch):
+    """tests/model_executor/model_loader/test_reload.py:158-258 of the reference:
+    loading new checkpoint tensors into a layer and running
+    process_weights_after_loading again keeps the workspace and the sort
+    indices at their addresses (zeroed / refilled in place), so a recorded
+    graph keeps reading live tensors."""
+    import types
+    from sonar_amd import marlin_linear, marlin_utils, ops
+    from sonar_amd.scalar_type import scalar_types
+    size_k, size_n, group = 128, 64, 64
+    monkeypatch.setattr(marlin_utils, "num_compute_units", lambda _=None: 4)
+    monkeypatch.setattr(ops, "gptq_marlin_repack",
+                        lambda w, perm, size_k, size_n, num_bits, is_a_8bit=False:
+                        torch.zeros(size_k // 16, size_n * 2, dtype=torch.int32))
+    cfg = marlin_linear.MPLinearLayerConfig((size_k, size_n), (size_k, size_n), scalar_types.uint4b8,
+                                            torch.float16, group, False, True)
+    kernel = marlin_linear.MarlinLinearKernel(cfg, w_zp_param_name=None, w_gidx_param_name="g_idx")
+    gen = torch.Generator().manual_seed(0)
+    layer = types.SimpleNamespace()
+
+    def load(g_idx):
+        layer.qweight = torch.zeros(size_k // 8, size_n, dtype=torch.int32)
+        layer.scales = torch.ones(size_k // group, size_n, dtype=torch.float16)
+        layer.g_idx = g_idx.clone()
+
+    first = torch.randint(0, size_k // group, (size_k,), dtype=torch.int32, generator=gen)
+    second = torch.randint(0, size_k // group, (size_k,), dtype=torch.int32, generator=gen)
+    load(first)
+    kernel.process_weights_after_loading(layer)
+    workspace_ptr = kernel.workspace.data_ptr()
+    sort_ptr = layer.g_idx_sort_indices.data_ptr()
+    kernel.workspace.fill_(3)           # a reload must hand the workspace back zeroed
+    load(second)
+    kernel.process_weights_after_loading(layer)
+    assert kernel.workspace.data_ptr() == workspace_ptr and torch.all(kernel.workspace == 0)
+    assert layer.g_idx_sort_indices.data_ptr() == sort_ptr
+    assert torch.equal(layer.g_idx_sort_indices.data, marlin_utils.marlin_sort_g_idx(second)[1])
+    assert isinstance(layer.g_idx_sort_indices, torch.nn.Parameter)
