@@ -525,19 +525,24 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
 // prefetch on every unit.
 
 constexpr int kSlotS = 4096;       // inside a weight slot, after 4 chunks x 1 KiB: 64 scales, 8 zero-point words
-constexpr int kSlotBytes = 4096 + 256;
-constexpr int kWaveA = 2 * kSlotBytes;            // the activation slot follows the two weight slots
+// GPU below is the number of groups per 128-row unit (1 for groups of 128 rows
+// or more, 2 / 4 for groups of 64 / 32 rows): one 256-byte scale / zero-point
+// row per group follows the four chunks of a weight slot.
+constexpr int slot_bytes(int gpu) { return 4096 + 256 * gpu; }
+constexpr int wave_a(int gpu) { return 2 * slot_bytes(gpu); }   // the activation slot follows the two weight slots
 // LDS bytes per wavefront: the activation slot holds 4 KiB per block of 16 rows
-constexpr int wave_lds(int mb) { return 2 * kSlotBytes + 4096 * mb; }
+constexpr int wave_lds(int mb, int gpu = 1) { return 2 * slot_bytes(gpu) + 4096 * mb; }
 // Tiles (16 x 16 fp32, 1 KiB) a wavefront parks per pass of the cross-wavefront
 // sum: all four of its one block of rows, or two of the eight of two blocks
 // (four passes), which keeps 8 wavefronts with two blocks inside 160 KiB.
 constexpr int park_tiles(int mb) { return mb == 1 ? 4 : 2; }
-constexpr int kWeightCopies = 5;   // asynchronous copies per unit: 4 weight chunks + 1 scale row
+constexpr int weight_copies(int gpu) { return 4 + gpu; }   // asynchronous copies per unit: 4 weight chunks + the scale rows
 // A workgroup of the fast kernel has 8 wavefronts (one workgroup per compute
 // unit), or 4 (two per compute unit: a grid with more workgroups than compute
 // units then runs them side by side instead of one after the other).
-constexpr int fast_lds_bytes(int waves, int mb) { return waves * (wave_lds(mb) + park_tiles(mb) * 1024); }
+constexpr int fast_lds_bytes(int waves, int mb, int gpu = 1) {
+  return waves * (wave_lds(mb, gpu) + park_tiles(mb) * 1024);
+}
 
 // Row id of C of row `r` of block `block` of a grouped call, -1 for padding.
 __device__ __forceinline__ int moe_row_id(const StreamParams& p, int block, int r) {
@@ -555,7 +560,9 @@ struct FastLane {
   int s_strip_stride;   // bytes between strips for s_ptr
 };
 
-template <int MB>
+// unit_group_shift: s >= 0 for groups of 128 * 2^s rows, -1 for one group; with
+// GPU > 1 the unit holds groups GPU * unit .. GPU * unit + GPU - 1.
+template <int MB, int GPU>
 __device__ __forceinline__ void copy_weights(const StreamParams& p, const FastLane<MB>& fl, int strip, int unit,
                                              char* slot, int lane, int unit_group_shift) {
   const uint4* gq = p.b + (size_t)(unsigned)(strip * p.chunks_per_strip + unit * 4) * 64 + lane;
@@ -564,9 +571,12 @@ __device__ __forceinline__ void copy_weights(const StreamParams& p, const FastLa
   __builtin_amdgcn_global_load_lds((glb_void_t*)gq, lq, 16, 1024, 0);
   __builtin_amdgcn_global_load_lds((glb_void_t*)gq, lq, 16, 2048, 0);
   __builtin_amdgcn_global_load_lds((glb_void_t*)gq, lq, 16, 3072, 0);
-  const int g = unit_group_shift >= 0 ? (unit >> unit_group_shift) : 0;
+  const int g = GPU > 1 ? unit * GPU : (unit_group_shift >= 0 ? (unit >> unit_group_shift) : 0);
   const char* gs = fl.s_ptr + (long)g * fl.s_group_stride + (long)strip * fl.s_strip_stride;
-  __builtin_amdgcn_global_load_lds((glb_void_t*)gs, (lds_void_t*)(slot + kSlotS), 4, 0, 0);
+#pragma unroll
+  for (int gi = 0; gi < GPU; ++gi)
+    __builtin_amdgcn_global_load_lds((glb_void_t*)(gs + gi * fl.s_group_stride),
+                                     (lds_void_t*)(slot + kSlotS + 256 * gi), 4, 0, 0);
 }
 
 // The 16 x 128 slice of A of one unit and block of 16 rows, as four regions of
@@ -688,16 +698,42 @@ __device__ __forceinline__ u32x4_t raw_operand(uint32_t q, uint32_t magic) {
       : "v"(a_at), "v"(a_at ^ 64u)                                                                 \
       : "memory")
 
+// Zero-point words and the 16 scales of one more group of the unit (GI = 1..3, 256 bytes per group).
+#define SONAR_GROUP_READS(GI)                                                                       \
+  asm volatile(                                                                                    \
+      "ds_read_b128 %0, %17\n\t"                                                                   \
+      "ds_read_u16 %1, %18\n\tds_read_u16 %2, %18 offset:16\n\t"                                  \
+      "ds_read_u16 %3, %18 offset:32\n\tds_read_u16 %4, %18 offset:48\n\t"                        \
+      "ds_read_u16 %5, %18 offset:4\n\tds_read_u16 %6, %18 offset:20\n\t"                         \
+      "ds_read_u16 %7, %18 offset:36\n\tds_read_u16 %8, %18 offset:52\n\t"                        \
+      "ds_read_u16 %9, %18 offset:8\n\tds_read_u16 %10, %18 offset:24\n\t"                        \
+      "ds_read_u16 %11, %18 offset:40\n\tds_read_u16 %12, %18 offset:56\n\t"                      \
+      "ds_read_u16 %13, %18 offset:12\n\tds_read_u16 %14, %18 offset:28\n\t"                      \
+      "ds_read_u16 %15, %18 offset:44\n\tds_read_u16 %16, %18 offset:60\n\t"                      \
+      "s_waitcnt lgkmcnt(0)"                                                                       \
+      : "=&v"(more_z[GI - 1]), "=&v"(more_s[GI - 1][0]), "=&v"(more_s[GI - 1][1]),                  \
+        "=&v"(more_s[GI - 1][2]), "=&v"(more_s[GI - 1][3]), "=&v"(more_s[GI - 1][4]),                \
+        "=&v"(more_s[GI - 1][5]), "=&v"(more_s[GI - 1][6]), "=&v"(more_s[GI - 1][7]),                \
+        "=&v"(more_s[GI - 1][8]), "=&v"(more_s[GI - 1][9]), "=&v"(more_s[GI - 1][10]),               \
+        "=&v"(more_s[GI - 1][11]), "=&v"(more_s[GI - 1][12]), "=&v"(more_s[GI - 1][13]),             \
+        "=&v"(more_s[GI - 1][14]), "=&v"(more_s[GI - 1][15])                                         \
+      : "v"(z_at + 256u * (GI)), "v"(s_at + 256u * (GI))                                           \
+      : "memory")
+
 // MB blocks of 16 rows per workgroup (1 or 2): the weights of a unit are pulled
 // out of LDS and turned into operands once and multiplied with every block.
 // GROUPED: one workgroup per (block of slots, strip) of a mixture-of-experts
 // call; the rows of A are gathered and the rows of C scattered through
 // sorted_ids, everything else is the dense kernel on the expert's matrices.
-template <typename T, bool HAS_ZP, int kFastWaves, int MB, bool GROUPED = false>
+// GPU: groups per 128-row unit (2 or 4 for groups of 64 or 32 rows, else 1).
+template <typename T, bool HAS_ZP, int kFastWaves, int MB, bool GROUPED = false, int GPU = 1>
 __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams params,
                                                                              const int unit_group_shift) {
   typedef typename Dq<T>::vec8 vec8;
-  constexpr int kWaveLds = wave_lds(MB);
+  constexpr int kWaveLds = wave_lds(MB, GPU);
+  constexpr int kSlotBytes = slot_bytes(GPU);
+  constexpr int kWaveA = wave_a(GPU);
+  constexpr int kWeightCopies = weight_copies(GPU);
   constexpr int kPark = park_tiles(MB);       // tiles per wavefront and pass of the cross-wavefront sum
   constexpr int kPasses = 4 * MB / kPark;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -794,12 +830,12 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   cur.set(u_begin + wave, p.units_per_strip);
   fetch = cur;
   if (fetch.index < u_end) {
-    copy_weights<MB>(p, fl, fetch.strip, fetch.unit, ring, lane, unit_group_shift);
+    copy_weights<MB, GPU>(p, fl, fetch.strip, fetch.unit, ring, lane, unit_group_shift);
     copy_activations<MB>(p, fl, fetch.unit, ring + kWaveA);
   }
   fetch.advance(kFastWaves, p.units_per_strip);
   if (fetch.index < u_end)
-    copy_weights<MB>(p, fl, fetch.strip, fetch.unit, ring + kSlotBytes, lane, unit_group_shift);
+    copy_weights<MB, GPU>(p, fl, fetch.strip, fetch.unit, ring + kSlotBytes, lane, unit_group_shift);
   // `fetch` names the unit whose A slice is copied next; its weights are in flight
   int c_slot = 0;
 
@@ -897,6 +933,8 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     u32x4_t b0 = u32x4_t{0u, 0u, 0u, 0u}, b1 = b0, b2 = b0, b3 = b0;  // second block of rows
     uint32_t row_s[16];
     u32x4_t row_z = u32x4_t{0u, 0u, 0u, 0u};
+    uint32_t more_s[GPU > 1 ? GPU - 1 : 1][16];   // the other groups of the unit
+    u32x4_t more_z[GPU > 1 ? GPU - 1 : 1];
     const bool more = cur.index + kFastWaves < u_end;
     if (more) {
       asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightCopies) : "memory");
@@ -912,51 +950,64 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
         SONAR_UNIT_READS(0, 2, 16, 18, 8, 10, 24, 26, 64, 66, 80, 82, 72, 74, 88, 90);
       }
       if constexpr (MB == 2) SONAR_UNIT_READS_ROWS2(b0, b1, b2, b3);
+      if constexpr (GPU >= 2) SONAR_GROUP_READS(1);
+      if constexpr (GPU == 4) {
+        SONAR_GROUP_READS(2);
+        SONAR_GROUP_READS(3);
+      }
     }
     if (more) {
       copy_activations<MB>(p, fl, fetch.unit, ring + kWaveA);
       fetch.advance(kFastWaves, p.units_per_strip);
       if (fetch.index < u_end)
-        copy_weights<MB>(p, fl, fetch.strip, fetch.unit, ring + c_slot * kSlotBytes, lane, unit_group_shift);
+        copy_weights<MB, GPU>(p, fl, fetch.strip, fetch.unit, ring + c_slot * kSlotBytes, lane, unit_group_shift);
     }
 
     const u32x4_t qs[4] = {q0, q1, q2, q3};
     const u32x4_t as[2][4] = {{a0, a1, a2, a3}, {b0, b1, b2, b3}};
     const floatx4_t zero4 = floatx4_t{0.f, 0.f, 0.f, 0.f};
     floatx4_t part_sum[MB][4], asum[MB];
+    constexpr int kChunksPerGroup = 4 / GPU;
 #pragma unroll
-    for (int cc = 0; cc < 4; ++cc) {
-      const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
+    for (int gi = 0; gi < GPU; ++gi) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const vec8 wv = __builtin_bit_cast(vec8, raw_operand(words[j], magic));
+      for (int cg = 0; cg < kChunksPerGroup; ++cg) {
+        const int cc = gi * kChunksPerGroup + cg;
+        const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const vec8 wv = __builtin_bit_cast(vec8, raw_operand(words[j], magic));
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            part_sum[mb][j] = Dq<T>::mfma(wv, __builtin_bit_cast(vec8, as[mb][cc]), cg == 0 ? zero4 : part_sum[mb][j]);
+        }
 #pragma unroll
         for (int mb = 0; mb < MB; ++mb)
-          part_sum[mb][j] = Dq<T>::mfma(wv, __builtin_bit_cast(vec8, as[mb][cc]), cc == 0 ? zero4 : part_sum[mb][j]);
+          asum[mb] = Dq<T>::mfma(__builtin_bit_cast(vec8, ones), __builtin_bit_cast(vec8, as[mb][cc]),
+                                 cg == 0 ? zero4 : asum[mb]);
       }
+      // scale and offset of this group (the whole unit when GPU == 1)
+      const u32x4_t gz = gi == 0 ? row_z : more_z[gi == 0 ? 0 : gi - 1];
+      const uint32_t zrow[4] = {gz.x >> row_z_shift, gz.y >> row_z_shift, gz.z >> row_z_shift, gz.w >> row_z_shift};
 #pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-        asum[mb] = Dq<T>::mfma(__builtin_bit_cast(vec8, ones), __builtin_bit_cast(vec8, as[mb][cc]),
-                               cc == 0 ? zero4 : asum[mb]);
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const uint32_t sbits = gi == 0 ? row_s[4 * j + r] : more_s[gi == 0 ? 0 : gi - 1][4 * j + r];
+          const float sc = Dq<T>::to_float((uint16_t)sbits);
+          float off = -(RawOperand<T>::kBase + 8.f);
+          if (HAS_ZP) off = -RawOperand<T>::kBase - (float)((zrow[r] >> (4 * j)) & 0xFu);
+#pragma unroll
+          for (int mb = 0; mb < MB; ++mb)
+            acc[mb][j][r] = __builtin_fmaf(sc, __builtin_fmaf(off, asum[mb][r], part_sum[mb][j][r]), acc[mb][j][r]);
+        }
     }
-    const uint32_t zrow[4] = {row_z.x >> row_z_shift, row_z.y >> row_z_shift, row_z.z >> row_z_shift,
-                              row_z.w >> row_z_shift};
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int r = 0; r < 4; ++r) {
-        const float sc = Dq<T>::to_float((uint16_t)row_s[4 * j + r]);
-        float off = -(RawOperand<T>::kBase + 8.f);
-        if (HAS_ZP) off = -RawOperand<T>::kBase - (float)((zrow[r] >> (4 * j)) & 0xFu);
-#pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          acc[mb][j][r] = __builtin_fmaf(sc, __builtin_fmaf(off, asum[mb][r], part_sum[mb][j][r]), acc[mb][j][r]);
-      }
     cur.advance(kFastWaves, p.units_per_strip);
     c_slot ^= 1;
   }
 }
 #undef SONAR_UNIT_READS_ROWS2
+#undef SONAR_GROUP_READS
 
 // ---------------------------------------------------------------------------
 // Second pass over the strips that were split between workgroups: adds the
@@ -1167,18 +1218,34 @@ void launch_stream8_mb(const StreamParams& p, hipStream_t st) {
   else launch_stream8_gidx<T, false>(p, st);
 }
 
-template <typename T, bool HAS_ZP, int WAVES, int MB, bool GROUPED>
-int launch_fast_waves(const StreamParams& p, int unit_group_shift, hipStream_t st) {
+template <typename T, bool HAS_ZP, int WAVES, int MB, bool GROUPED, int GPU>
+int launch_fast_groups(const StreamParams& p, int unit_group_shift, hipStream_t st) {
   static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB, GROUPED>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds_bytes(WAVES, MB)));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB, GROUPED, GPU>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds_bytes(WAVES, MB, GPU)));
     attr_set = true;
   }
-  const int lds = p.sum_over_rings ? WAVES * wave_lds(MB) : fast_lds_bytes(WAVES, MB);
-  marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB, GROUPED>
+  const int lds = p.sum_over_rings ? WAVES * wave_lds(MB, GPU) : fast_lds_bytes(WAVES, MB, GPU);
+  marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB, GROUPED, GPU>
       <<<p.grid_parts * p.slabs, WAVES * 64, lds, st>>>(p, unit_group_shift);
   return SONAR_OK;
+}
+
+// unit_group_shift -2 / -4: two / four groups per 128-row unit (groups of 64 / 32 rows)
+template <typename T, bool HAS_ZP, int WAVES, int MB, bool GROUPED>
+int launch_fast_waves(const StreamParams& p, int unit_group_shift, hipStream_t st) {
+  if (unit_group_shift <= -2) {
+    // several sets of scales per unit and two blocks of rows do not fit the register file (and were measured
+    // slower than the general kernel): callers pass one block of rows
+    if constexpr (MB == 1) {
+      return unit_group_shift == -2 ? launch_fast_groups<T, HAS_ZP, WAVES, 1, GROUPED, 2>(p, unit_group_shift, st)
+                                    : launch_fast_groups<T, HAS_ZP, WAVES, 1, GROUPED, 4>(p, unit_group_shift, st);
+    } else {
+      return fail(SONAR_E_INVALID, "internal: groups of 32 / 64 rows with two blocks of rows per workgroup");
+    }
+  }
+  return launch_fast_groups<T, HAS_ZP, WAVES, MB, GROUPED, 1>(p, unit_group_shift, st);
 }
 
 // `row_blocks`: blocks of 16 rows per workgroup (1 or 2).
@@ -1254,10 +1321,15 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
 }
 
 // log2 of the 128-row units per group when groups are runs of 128 * 2^s rows,
-// -1 for one group; false when the fast kernel cannot index the groups.
+// -1 for one group, -2 / -4 for groups of 64 / 32 rows (two / four per unit);
+// false when the fast kernel cannot index the groups.
 bool fast_group_shift(int64_t num_groups, int group_size, int& unit_group_shift) {
   unit_group_shift = -1;
   if (num_groups == 1) return true;
+  if (group_size == 64 || group_size == 32) {   // two / four groups per 128-row unit
+    unit_group_shift = group_size == 64 ? -2 : -4;
+    return true;
+  }
   if (group_size <= 0 || group_size % 128 != 0) return false;
   const int per = group_size / 128;
   if ((per & (per - 1)) != 0) return false;
@@ -1278,6 +1350,7 @@ bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t sorted_len,
   if (no_fast || has_perm || size_k % (4 * kChunkK) != 0 || !fast_group_shift(num_groups, group_size, shift) ||
       a_rows * size_k * 2 >= (1LL << 31) || n_strips * units * n_strips >= (1LL << 31))
     return false;
+  if (shift <= -2 && moe_block_size > 16) return false;   // groups of 32 / 64 rows: one block of 16 rows only
   if (moe_block_size < 64) return true;
   // 64-slot blocks also have the tile kernel, which wins once the experts have
   // rows enough to fill its 256-row tiles.  Measured on Mixtral shapes (8
@@ -1462,7 +1535,9 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   // M = 256: 21 us against 37; N = 6144, M = 256: 32 against 40; N = 4096,
   // M = 512: 37 against 44; N = 6144, M = 512: 54 against 50).
   const bool few_row_blocks = n_strips * ((size_m + 31) / 32) <= 4 * (int64_t)cus;
-  const bool slab_fast = !no_slabs && fast_shape && size_m > 16 &&
+  // (groups of 32 / 64 rows take the 16-row kernel up to 16 rows only: measured at K = 4096, N = 11008,
+  // M = 64: 43 / 30 us in blocks of rows against 30 / 27 in the general kernel)
+  const bool slab_fast = !no_slabs && fast_shape && size_m > 16 && unit_group_shift >= -1 &&
                          (size_m <= 64 || (strip_per_workgroup && (size_m <= 128 || few_row_blocks)));
 
   p.unit_chunks = p.chunks_per_strip % 4 == 0 ? 4 : (p.chunks_per_strip % 2 == 0 ? 2 : 1);
