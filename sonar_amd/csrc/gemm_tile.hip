@@ -304,18 +304,21 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const Tile
 // phase 4kt+4.
 // LDS is read from asm blocks only (the compiler cannot tell which LDS bytes a
 // copy writes and would otherwise wait for all copies before any LDS access).
-// Needs group_size % 64 == 0 (or one group) and no act-order.
+// Needs groups of 32 rows or a multiple of 64 (or one group) and no act-order.
 constexpr int kAsyncStages = 3;
-constexpr int kWaveStage = 2 * kBlockBytes + 256;   // two weight chunks + 64 scales + 8 zero-point words
+// G32: groups of 32 rows, i.e. one group per k block: a stage then carries two
+// scale / zero-point rows (256 bytes each) and takes one copy more.
+constexpr int wave_stage(bool g32) { return 2 * kBlockBytes + (g32 ? 512 : 256); }   // two weight chunks + scale rows
 constexpr int kAsyncA = kAsyncStages * kStageA;
-constexpr int kAsyncW = kTileWaves * kAsyncStages * kWaveStage;
-constexpr int kAsyncLds = kAsyncA + kAsyncW;
-constexpr int kAsyncCopies = 7;
+constexpr int async_lds(bool g32) { return kAsyncA + kTileWaves * kAsyncStages * wave_stage(g32); }
+constexpr int async_copies(bool g32) { return g32 ? 8 : 7; }
 
-template <typename T, bool HAS_ZP, bool GROUPED>
+template <typename T, bool HAS_ZP, bool GROUPED, bool G32 = false>
 __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq<T>::Col Col;
+  constexpr int kWaveStage = wave_stage(G32);
+  constexpr int kAsyncCopies = async_copies(G32);
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int tid = threadIdx.x;
@@ -403,6 +406,11 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
       __builtin_amdgcn_global_load_lds((glb_void_t*)g, (lds_void_t*)(sw + (idx - 4) * kBlockBytes), 16, 0, 0);
       return;
     }
+    if (G32) {   // idx 6 / 7: the rows of groups 2 kt and 2 kt + 1
+      __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)(2 * kt + (idx - 6)) * s_group_stride),
+                                       (lds_void_t*)(sw + 2 * kBlockBytes + 256 * (idx - 6)), 4, 0, 0);
+      return;
+    }
     const int grp = grouped ? (kt * kTileK) / p.group_size : 0;
     __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)grp * s_group_stride),
                                      (lds_void_t*)(sw + 2 * kBlockBytes), 4, 0, 0);
@@ -452,6 +460,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   auto raw_start = [&](int slot, int b, bool with_scales) {
     const uint32_t w_at = w_lds + slot * kWaveStage;
     const uint32_t q_at = w_at + b * kBlockBytes + lane * 16;
+    const uint32_t r_at = w_at + (G32 ? 256 * b : 0);   // this k block's scale row
     if (with_scales) {
       asm volatile(
           "ds_read_b128 %0, %6\n\t"
@@ -461,8 +470,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
           "ds_read_u16 %4, %10\n\t"
           "ds_read_b32 %5, %11"
           : "=&v"(qraw), "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
-          : "v"(q_at), "v"(w_at + s_off[0]), "v"(w_at + s_off[1]), "v"(w_at + s_off[2]), "v"(w_at + s_off[3]),
-            "v"(w_at + z_off)
+          : "v"(q_at), "v"(r_at + s_off[0]), "v"(r_at + s_off[1]), "v"(r_at + s_off[2]), "v"(r_at + s_off[3]),
+            "v"(r_at + z_off)
           : "memory");
     } else {
       asm volatile("ds_read_b128 %0, %1" : "=&v"(qraw) : "v"(q_at) : "memory");
@@ -540,14 +549,14 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 #pragma unroll
     for (int idx = 0; idx < 4; ++idx) issue_one(copy_kt, fill, idx);
     fetch(slot, 0, true);
-    raw_start(slot, 1, false);
+    raw_start(slot, 1, G32);
     phase_end();
     multiply();
     phase_end();
     // ---- half step (kt, 1)
 #pragma unroll
     for (int idx = 4; idx < kAsyncCopies; ++idx) issue_one(copy_kt, fill, idx);
-    fetch(slot, 1, false);
+    fetch(slot, 1, G32);
     // stage kt + 1 has landed once nothing but the copies of stage kt + 2 is outstanding
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
     raw_start(next_slot, 0, true);
@@ -691,17 +700,23 @@ __global__ __launch_bounds__(256) void moe_tile_table_kernel(const int32_t* __re
   table[0] = tiles;
 }
 
-template <typename T, bool HAS_ZP>
-int launch_tile_async(const TileParams& p, hipStream_t st) {
+template <typename T, bool HAS_ZP, bool G32>
+int launch_tile_async_groups(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;  // raising the dynamic LDS limit is needed once per kernel
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, HAS_ZP, false>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kAsyncLds));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, HAS_ZP, false, G32>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, async_lds(G32)));
     attr_set = true;
   }
   const int grid = tile_grid(p);
-  marlin_tile_async_kernel<T, HAS_ZP, false><<<grid, kTileWaves * 64, kAsyncLds, st>>>(p);
+  marlin_tile_async_kernel<T, HAS_ZP, false, G32><<<grid, kTileWaves * 64, async_lds(G32), st>>>(p);
   return SONAR_OK;
+}
+
+template <typename T, bool HAS_ZP>
+int launch_tile_async(const TileParams& p, hipStream_t st) {
+  return (p.num_groups > 1 && p.group_size == 32) ? launch_tile_async_groups<T, HAS_ZP, true>(p, st)
+                                                  : launch_tile_async_groups<T, HAS_ZP, false>(p, st);
 }
 
 template <typename T, bool HAS_ZP>
@@ -709,10 +724,10 @@ int launch_tile_grouped(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
     SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, HAS_ZP, true>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kAsyncLds));
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, async_lds(false)));
     attr_set = true;
   }
-  marlin_tile_async_kernel<T, HAS_ZP, true><<<tile_grid(p), kTileWaves * 64, kAsyncLds, st>>>(p);
+  marlin_tile_async_kernel<T, HAS_ZP, true><<<tile_grid(p), kTileWaves * 64, async_lds(false), st>>>(p);
   return SONAR_OK;
 }
 
@@ -731,9 +746,9 @@ int launch_tile(const TileParams& p, hipStream_t st) {
 
 }  // namespace
 
-// The asynchronous tile kernel needs groups of at least 64 rows and no gather of A.
+// The asynchronous tile kernel needs groups of 32 rows or a multiple of 64 and no gather of A.
 bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size) {
-  return !has_perm && (num_groups == 1 || group_size % kTileK == 0);
+  return !has_perm && (num_groups == 1 || group_size % kTileK == 0 || group_size == 32);
 }
 
 // Called by sonar_marlin_gemm for size_m > 64.  Shapes and pointers have been

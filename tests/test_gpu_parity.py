@@ -220,7 +220,8 @@ TILE_CASES = [
     (1000, 2048, 64, -1, False, False, True),
     (129, 14336, 4096, 128, False, False, False),
     (600, 1024, 768, 64, True, False, True),
-    (520, 512, 192, 32, True, False, False),         # groups of 32 rows: the register-staged tile kernel
+    (520, 512, 192, 32, True, False, False),         # groups of 32 rows: two scale rows per K step
+    (1000, 2048, 1024, 32, False, False, True),
     # 9 x 29 = 261 tiles: 256 whole ones, then the last 5 split six ways along K
     (2200, 3072, 7360, 128, True, False, True),
 ]
