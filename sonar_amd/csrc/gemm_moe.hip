@@ -591,7 +591,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
   // Full blocks of 64 slots mean many rows per expert: the MFMA-tiled kernel
   if (moe_block_size == 64 && !has_perm && !bits8 && !row_groups && !no_tile && size_k % 64 == 0 &&
       num_experts <= 1024 &&
-      (num_groups == 1 || group_size % 64 == 0) && scratch != nullptr &&
+      (num_groups == 1 || group_size % 64 == 0 || group_size == 32) && scratch != nullptr &&
       scratch_bytes >= moe_tile_table_bytes(sorted_len, num_experts) && ((uintptr_t)scratch) % 4 == 0)
     return moe_tile_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
                          num_tokens_past_padded, topk_weights, top_k, mul_topk_weights ? 1 : 0, num_experts,

@@ -719,16 +719,22 @@ int launch_tile_async(const TileParams& p, hipStream_t st) {
                                                   : launch_tile_async_groups<T, HAS_ZP, false>(p, st);
 }
 
-template <typename T, bool HAS_ZP>
-int launch_tile_grouped(const TileParams& p, hipStream_t st) {
+template <typename T, bool HAS_ZP, bool G32>
+int launch_tile_grouped_groups(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, HAS_ZP, true>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, async_lds(false)));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, HAS_ZP, true, G32>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, async_lds(G32)));
     attr_set = true;
   }
-  marlin_tile_async_kernel<T, HAS_ZP, true><<<tile_grid(p), kTileWaves * 64, async_lds(false), st>>>(p);
+  marlin_tile_async_kernel<T, HAS_ZP, true, G32><<<tile_grid(p), kTileWaves * 64, async_lds(G32), st>>>(p);
   return SONAR_OK;
+}
+
+template <typename T, bool HAS_ZP>
+int launch_tile_grouped(const TileParams& p, hipStream_t st) {
+  return (p.num_groups > 1 && p.group_size == 32) ? launch_tile_grouped_groups<T, HAS_ZP, true>(p, st)
+                                                  : launch_tile_grouped_groups<T, HAS_ZP, false>(p, st);
 }
 
 template <typename T, bool HAS_ZP, bool HAS_PERM>

@@ -102,6 +102,7 @@ MOE_CASES = [
     (513, 3, 2, 256, 320, 64, "bf16", True, False, True, 64, True),
     (90, 8, 2, 384, 128, -1, "fp16", False, False, False, 64, False),
     (1100, 2, 1, 128, 512, 128, "bf16", False, False, True, 64, False),
+    (900, 2, 2, 256, 512, 32, "fp16", True, False, True, 64, True),      # groups of 32 rows in the tile kernel
 ]
 
 
