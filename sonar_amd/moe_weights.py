@@ -4,12 +4,13 @@
 Mirrors `_process_weights_marlin` (GPTQ-style experts, packed along K) and
 `_process_awq_weights_marlin` (AWQ-style experts, packed along N with the AWQ
 nibble order) of aphrodite/model_executor/layers/fused_moe/oracle/
-int_wna16.py:464-700 and :787-940, for 4-bit weights with fp16 / bf16
-activations: pad the intermediate size to what the grouped op takes, sort the
+int_wna16.py:464-700 and :787-940, for fp16 / bf16 activations (GPTQ-style: 4-
+and 8-bit codes with a fixed offset, 4-bit codes with zero points; AWQ-style:
+4-bit): pad the intermediate size to what the grouped op takes, sort the
 act-order group indices per expert, repack every expert, permute scales, zero
 points and biases.  Stacked tensors, expert first:
 
-  GPTQ:  w13_qweight (E, K/8, 2N)   w2_qweight (E, N/8, K)   int32
+  GPTQ:  w13_qweight (E, K/8, 2N)   w2_qweight (E, N/8, K)   int32 (K/4, N/4 for 8 bits)
          w13_scales  (E, K/G, 2N)   w2_scales  (E, N/G, K)
          w13_qzeros  (E, K/G, 2N/8) w2_qzeros  (E, N/G, K/8) plain column packing
          w13_g_idx   (E, K)         w2_g_idx   (E, N)
@@ -85,8 +86,10 @@ def process_gptq_moe_weights(intermediate_size: int, num_bits: int, group_size: 
     K of their own matrix (hidden size for w13, intermediate size for w2); the
     reference passes the intermediate size for both, which selects the same
     permutation unless exactly one of the two sizes is at most group_size."""
-    if num_bits != 4:
-        raise NotImplementedError("expert weights of 4 bits only")
+    if num_bits not in (4, 8):
+        raise NotImplementedError("expert weights of 4 or 8 bits only")
+    if num_bits == 8 and (w13_qzeros is not None or w2_qzeros is not None):
+        raise NotImplementedError("8-bit expert weights with zero points")
     pack = 32 // num_bits
     n = intermediate_size
     padded_n = marlin_moe_padded_intermediate(n, group_size)

@@ -353,6 +353,9 @@ def _route(m, e, topk, seed):
     (40, 4, 2, 256, 128, 128, "fp16", "awq", False, True),
     (9, 4, 2, 256, 96, 32, "fp16", "gptq", False, True),      # intermediate size padded 96 -> 128
     (9, 4, 2, 128, 160, 32, "bf16", "awq", False, False),     # 160 -> 192
+    (21, 4, 2, 256, 128, 128, "fp16", "gptq8", False, True),  # 8-bit codes
+    (70, 4, 2, 256, 256, 64, "bf16", "gptq8", True, False),
+    (9, 4, 2, 256, 96, 32, "fp16", "gptq8", False, False),    # 8-bit codes, 96 -> 128
 ], ids=str)
 def test_moe_checkpoint_tensors_through_weight_processing(cfg):
     """Stacked expert tensors as a GPTQ / AWQ checkpoint holds them ->
@@ -362,14 +365,22 @@ def test_moe_checkpoint_tensors_through_weight_processing(cfg):
     from sonar_amd.fused_moe import fused_marlin_moe
     from sonar_amd.scalar_type import scalar_types
     m, e, topk, hidden, inter, g, dtype, fmt, act, bias = cfg
-    zp = fmt != "gptq"
+    zp = fmt in ("gptq_zp", "awq")
+    bits = 8 if fmt == "gptq8" else 4
     rng = np.random.default_rng(hidden + inter)
 
     def expert_set(seed, k, n):
         layers = [mo.make_layer(seed + i, k, n, g, dtype, zero_points=zp, act_order=act) for i in range(e)]
-        ref = [mo.dequantize(l["q"], l["scales"], g, dtype, zeros=l.get("zeros"), g_idx=l.get("g_idx"))
-               for l in layers]
-        if fmt == "awq":
+        if bits == 8:
+            for i, l in enumerate(layers):   # codes over all of 0..255, scales a sixteenth
+                l["q"] = np.random.default_rng(seed + 50 + i).integers(0, 256, size=(k, n), dtype=np.int32)
+                l["scales"] = mo.round_to_dtype(l["scales"] / 16, dtype)
+        ref = [mo.dequantize(l["q"], l["scales"], g, dtype, zeros=l.get("zeros"), g_idx=l.get("g_idx"),
+                             num_bits=bits) for l in layers]
+        if bits == 8:
+            qw = torch.stack([gu.dev_i32(mo.pack_rows8(l["q"])) for l in layers])
+            qz = None
+        elif fmt == "awq":
             qw = torch.stack([gu.dev_i32(mo.awq_pack(l["q"])) for l in layers])
             qz = torch.stack([gu.dev_i32(mo.awq_pack(l["zeros"])) for l in layers])
         else:
@@ -386,12 +397,12 @@ def test_moe_checkpoint_tensors_through_weight_processing(cfg):
     if fmt == "awq":
         w = mw.process_awq_moe_weights(inter, 4, g, qw13, qw2, s13, s2, qz13, qz2, dev_bias(b13), dev_bias(b2))
     else:
-        w = mw.process_gptq_moe_weights(inter, 4, g, act, qw13, qw2, s13, s2, gi13, gi2, qz13, qz2,
+        w = mw.process_gptq_moe_weights(inter, bits, g, act, qw13, qw2, s13, s2, gi13, gi2, qz13, qz2,
                                         dev_bias(b13), dev_bias(b2))
     assert w.intermediate_size == mw.marlin_moe_padded_intermediate(inter, g)
     topk_ids, topk_w = _route(m, e, topk, m)
     x32 = mo.round_to_dtype(0.5 * mo.make_activations(m, m, hidden, dtype), dtype)
-    qtype = scalar_types.uint4 if zp else scalar_types.uint4b8
+    qtype = scalar_types.uint8b128 if bits == 8 else scalar_types.uint4 if zp else scalar_types.uint4b8
     y = fused_marlin_moe(gu.dev_bits16(x32, dtype), w.w1, w.w2, w.bias1, w.bias2, w.w1_scale, w.w2_scale,
                          torch.from_numpy(topk_w).to(gu.DEV), torch.from_numpy(topk_ids).to(gu.DEV), qtype.id,
                          g_idx1=w.g_idx1, g_idx2=w.g_idx2, sort_indices1=w.sort_indices1,
