@@ -53,6 +53,11 @@ extern "C" {
 #define SONAR_TYPE_UINT4B8 1125899907892224LL /* GPTQ: code - 8 */
 #define SONAR_TYPE_UINT4 1125899906843648LL   /* AWQ: code - zero point */
 #define SONAR_TYPE_UINT8B128 1125899923621888LL /* GPTQ 8-bit: code - 128 */
+/* 8-bit floating-point codes (sign, 4 exponent bits, 3 mantissa bits, no infinities), in the 8-bit
+ * weight order; b_scales then hold the scales times 2^8 (fp16) or 2^120 (bf16), as
+ * fp8_fused_exponent_bias_into_scales makes them (quantization/utils/marlin_utils_fp8.py:35-46);
+ * one scale per column or per group of 128 rows, no act-order (marlin/generate_kernels.py:87-93) */
+#define SONAR_TYPE_FLOAT8_E4M3FN 2814749767172868LL
 
 const char* sonar_marlin_last_error(void);
 const char* sonar_marlin_version(void);
@@ -79,7 +84,7 @@ int sonar_marlin_to_gfx950(const uint32_t* marlin, uint32_t* out,
 int sonar_gfx950_to_marlin(const uint32_t* gfx950, uint32_t* out,
                            int64_t size_k, int64_t size_n, void* stream);
 
-/* The same for 8-bit codes (uint8b128): Marlin (K/16, 4N) int32 <-> the
+/* The same for 8-bit codes (uint8b128, float8_e4m3fn): Marlin (K/16, 4N) int32 <-> the
  * streaming order of 1-KiB blocks of 16 rows x 64 columns.  No counterpart in
  * the reference (its kernels read the Marlin order directly). */
 int sonar_marlin8_to_gfx950(const uint32_t* marlin, uint32_t* out,
@@ -88,7 +93,8 @@ int sonar_gfx950_to_marlin8(const uint32_t* gfx950, uint32_t* out,
                             int64_t size_k, int64_t size_n, void* stream);
 
 /* Dequantised weight matrix W[K][N] (row-major, dtype elements) exactly as the
- * GEMM kernels form it in registers: round_to_dtype((code - z) * s).  Uses the
+ * GEMM kernels form it in registers: round_to_dtype((code - z) * s), for
+ * float8_e4m3fn round_to_dtype(value(code) * scale).  Uses the
  * same device routine as the GEMM; exists so the in-kernel values can be
  * compared bit for bit.  Arguments as for sonar_marlin_gemm. */
 int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout,
@@ -104,7 +110,7 @@ size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n, int64_t s
  * rounded to dtype.
  *   a            dtype[M][a_row_stride], 16-byte aligned, a_row_stride % 8 == 0
  *   c            dtype[M][N] contiguous
- *   b_q_weight   K*N/8 words in b_layout order
+ *   b_q_weight   K*N/8 words (K*N/4 for the 8-bit types) in b_layout order
  *   b_bias       dtype[N] in marlin_permute_bias order, or NULL
  *   b_scales     dtype[num_groups][N] in marlin_permute_scales order
  *   b_zeros      int32[num_groups][N/8] in marlin_zero_points order, or NULL
@@ -144,7 +150,7 @@ int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
  *   a            dtype[M][K] contiguous
  *   c            dtype[M*top_k][N] contiguous
  *   b_q_weight   num_experts * K*N/8 words (K*N/4 for uint8b128), each expert
- *                in b_layout order; b_type_id uint4b8, uint4 or uint8b128
+ *                in b_layout order; b_type_id uint4b8, uint4, uint8b128 or float8_e4m3fn
  *   b_scales     dtype[num_experts][num_groups][N]; b_zeros / b_bias likewise
  *   scratch      sonar_moe_marlin_gemm_scratch_bytes(); act-order calls run 4 to
  *                20 times faster with sorted_len * K * 2 bytes more behind that

@@ -37,6 +37,14 @@ reference checkout).  How each function is pinned (none is "parity unpinned"):
                            (gptq_marlin_repack.cu:129-236), bijection on
                            bytes, round trips, exhaustive dequantisation over
                            256 codes
+* fp8 weights (W8A16-fp8)  the table of the 254 finite codes against torch's
+                           own float8_e4m3fn -> float32 conversion on the CPU
+                           and hand values (0x38 = 1, 0x7e = 448, 0x01 =
+                           2^-9); the kernel-side recipe (code read as a
+                           16-bit float, scale with the exponent bias folded
+                           in; dequant.h:320-380, marlin_utils_fp8.py:35-46)
+                           against value * scale in exact rational arithmetic
+                           rounded to nearest even, over all codes
 """
 
 from __future__ import annotations
@@ -67,7 +75,9 @@ def scalar_type_id(exponent: int, mantissa: int, signed: bool, bias: int,
 
 UINT4B8_ID = scalar_type_id(0, 4, False, 8)      # scalar_types.uint4b8
 UINT4_ID = scalar_type_id(0, 4, False, 0)        # scalar_types.uint4
-UINT8B128_ID = scalar_type_id(0, 8, False, 128)  # scalar_types.uint8b128 (rejected by this build)
+UINT8B128_ID = scalar_type_id(0, 8, False, 128)  # scalar_types.uint8b128
+NAN_REPR_EXTD_RANGE_MAX_MIN = 2                  # scalar_type.py:16
+FLOAT8_E4M3FN_ID = scalar_type_id(4, 3, True, 0, True, NAN_REPR_EXTD_RANGE_MAX_MIN)  # scalar_type.py:314
 
 
 def scalar_type_min_max(mantissa: int, signed: bool, bias: int):
@@ -396,6 +406,53 @@ def gfx950_unpack8(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
 
 def marlin8_to_gfx950(marlin_packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
     return gfx950_pack8(marlin_unpack8(marlin_packed, size_k, size_n))
+
+
+# --------------------------------------------------------------------------
+# 8-bit floating-point weights: float8_e4m3fn codes in the 8-bit packings above
+# (dequant.h:320-380; marlin_utils_fp8.py:35-46, 366-378, 591-631)
+# --------------------------------------------------------------------------
+
+def fp8_e4m3fn_values() -> np.ndarray:
+    """The value of each of the 256 codes: sign bit, 4 exponent bits with bias
+    7, 3 mantissa bits, subnormals at exponent 0, no infinities.  The codes
+    0x7f and 0xff are NaN in the format; the kernels' bit trick reads them as
+    the next step of the sequence, +-480, and so does this table."""
+    code = np.arange(256)
+    e, m = (code >> 3) & 15, code & 7
+    mag = np.where(e == 0, m / 8.0 * 2.0 ** -6, (1 + m / 8.0) * 2.0 ** (e.astype(np.float64) - 7))
+    return np.where(code & 0x80, -mag, mag).astype(np.float32)
+
+
+FP8_EXPONENT_BIAS_SHIFT = {"fp16": 8, "bf16": 120}   # 2^(e-1) - 2^3 for e = 5 / 8 exponent bits
+
+
+def fp8_fuse_exponent_bias(scales32: np.ndarray, dtype: str) -> np.ndarray:
+    """marlin_utils_fp8.py:35-46: the scales the op receives, scales * 2^8
+    (fp16) or * 2^120 (bf16), as values of `dtype` held in fp32."""
+    return round_to_dtype((scales32.astype(np.float64) * 2.0 ** FP8_EXPONENT_BIAS_SHIFT[dtype]).astype(np.float32),
+                          dtype)
+
+
+def fp8_code_as_16bit_float(codes: np.ndarray, dtype: str) -> np.ndarray:
+    """dequant.h:321-337, 357-374: the sign stays, the other seven bits move
+    right by (exponent bits of `dtype`) - 4 below it; the 16-bit pattern read
+    as `dtype` is value * 2^-8 (fp16) or value * 2^-120 (bf16).  Returned in
+    fp32 (exact; bf16 subnormals are fp32 subnormals)."""
+    c = codes.astype(np.uint32)
+    shift = 1 if dtype == "fp16" else 4
+    bits = ((c & 0x80) << 8) | (((c & 0x7F) << 8) >> shift)
+    return from_bits16(bits.astype(np.uint16), dtype)
+
+
+def dequantize_fp8(codes: np.ndarray, fused_scales32: np.ndarray, group_size: int, dtype: str) -> np.ndarray:
+    """w[k][n] = round_to_dtype(code_as_16bit_float * fused_scale[g(k)][n]): the
+    reference's one 16-bit multiply (marlin_template.h:1172-1299 with
+    dequant_skip_flop, :353-357); the fp32 product of a 4-bit and an 11-bit
+    significand is exact, so the rounding is the single one."""
+    k, n = codes.shape
+    rows = np.zeros(k, dtype=np.int64) if group_size in (-1, k) else np.arange(k) // group_size
+    return round_to_dtype(fp8_code_as_16bit_float(codes, dtype) * fused_scales32.astype(np.float32)[rows, :], dtype)
 
 
 # --------------------------------------------------------------------------

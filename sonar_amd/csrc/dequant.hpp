@@ -212,6 +212,64 @@ struct Dq8<__bf16> {
   }
 };
 
+// 8-bit floating-point codes (float8_e4m3fn: sign, 4 exponent bits with bias
+// 7, 3 mantissa bits; dequant.h:320-380 of the reference).  Moved one bit to
+// the right below the sign, a code is the fp16 number v * 2^-8 (subnormal
+// codes become fp16 subnormals, so this holds for all of them; the two NaN
+// codes read as +-480).  The scales arrive with the exponent bias already
+// folded in (marlin_utils_fp8.py:35-46): s * 2^8 for fp16, s * 2^120 for bf16.
+// fp16: one packed multiply by that scale, as the reference's.  bf16: the
+// reference reads the code as the bf16 number v * 2^-120 and multiplies by
+// s * 2^120; here the fp16 reading is widened and multiplied by
+// (s * 2^120) * 2^-112 in fp32 -- the same exact product v * s, rounded once.
+// Same interface and row order as Dq8.
+template <typename T>
+struct Dq8F;
+
+__device__ __forceinline__ uint32_t fp8_pair_as_fp16(uint32_t y) {  // codes in bits 8-15 and 24-31
+  return (y & 0x80008000u) | ((y & 0x7f007f00u) >> 1);
+}
+
+template <>
+struct Dq8F<_Float16> {
+  typedef Dq8<_Float16>::Col Col;
+  static __device__ __forceinline__ Col make_col(uint16_t scale_bits) { return Dq8<_Float16>::make_col(scale_bits); }
+  static __device__ __forceinline__ uint2 word4(uint32_t q, const Col& c, uint32_t) {
+    const half2_t w0 = __builtin_bit_cast(half2_t, fp8_pair_as_fp16(q << 8)) * c.s;
+    const half2_t w1 = __builtin_bit_cast(half2_t, fp8_pair_as_fp16(q)) * c.s;
+    return make_uint2(__builtin_bit_cast(uint32_t, w0), __builtin_bit_cast(uint32_t, w1));
+  }
+};
+
+template <>
+struct Dq8F<__bf16> {
+  struct Col {
+    float s;
+  };
+  static __device__ __forceinline__ Col make_col(uint16_t scale_bits) {
+    return Col{__builtin_bit_cast(float, (uint32_t)scale_bits << 16) * 0x1p-112f};
+  }
+  static __device__ __forceinline__ bf16x2_t scaled(uint32_t fp16_pair, float s) {
+    const half2_t h = __builtin_bit_cast(half2_t, fp16_pair);
+    return __builtin_convertvector(floatx2_t{(float)h.x * s, (float)h.y * s}, bf16x2_t);
+  }
+  static __device__ __forceinline__ uint2 word4(uint32_t q, const Col& c, uint32_t) {
+    const bf16x2_t w0 = scaled(fp8_pair_as_fp16(q << 8), c.s);
+    const bf16x2_t w1 = scaled(fp8_pair_as_fp16(q), c.s);
+    return make_uint2(__builtin_bit_cast(uint32_t, w0), __builtin_bit_cast(uint32_t, w1));
+  }
+};
+
+// The dequantiser of an 8-bit weight type.
+template <typename T, bool FP8>
+struct Dq8Of {
+  typedef Dq8<T> type;
+};
+template <typename T>
+struct Dq8Of<T, true> {
+  typedef Dq8F<T> type;
+};
+
 // One packed word whose eight rows (8 consecutive k) may lie in different groups:
 // a shard of an act-order matrix that does not hold whole groups.  `groups`
 // holds the group of each row, `scale_col` points at this column's scale of

@@ -254,7 +254,7 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
   moe_scatter<T, MB>(p, acc, slot_id, expert_l, strip, lane);
 }
 
-// The same for 8-bit codes (uint8b128, symmetric): a 32-row chunk is two 1-KiB
+// The same for 8-bit codes (uint8b128, symmetric, or float8_e4m3fn with FP8): a 32-row chunk is two 1-KiB
 // blocks of 16 rows.  No gather of A: act-order experts come here through the
 // per-slot permuted copy (a_by_slot).  HAS_GIDX: every row finds its scale
 // through g_idx (is_k_full = false).
@@ -267,10 +267,11 @@ struct MoeUnit8 {
   int group;
 };
 
-template <typename T, int MB, bool HAS_GIDX>
+template <typename T, int MB, bool HAS_GIDX, bool FP8>
 __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe8_kernel(const MoeParams p) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq8<T>::Col Col;
+  typedef typename Dq8Of<T, FP8>::type D8;
+  typedef typename D8::Col Col;
   __shared__ float4 red[4][MB * 4][64];
   __shared__ int slot_id[16 * MB];
 
@@ -345,7 +346,7 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe8_kernel(const MoePa
     if (next < p.units_per_strip) load_unit(nxt, next);
     Col cols[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) cols[j] = Dq8<T>::make_col((uint16_t)cur.sbits[j]);
+    for (int j = 0; j < 4; ++j) cols[j] = D8::make_col((uint16_t)cur.sbits[j]);
     int cur_group = cur.group;
     const int chunk0 = mine * p.unit_chunks;
 #pragma unroll
@@ -356,7 +357,7 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe8_kernel(const MoePa
           cur_group = g;
           const uint16_t* srow = scales + (long)g * p.size_n + strip * kStripN;
 #pragma unroll
-          for (int j = 0; j < 4; ++j) cols[j] = Dq8<T>::make_col(srow[scale_slot(16 * j + col16, grouped)]);
+          for (int j = 0; j < 4; ++j) cols[j] = D8::make_col(srow[scale_slot(16 * j + col16, grouped)]);
         }
         const uint32_t lo[4] = {cur.q[cc][0].x, cur.q[cc][0].y, cur.q[cc][0].z, cur.q[cc][0].w};
         const uint32_t hi[4] = {cur.q[cc][1].x, cur.q[cc][1].y, cur.q[cc][1].z, cur.q[cc][1].w};
@@ -375,8 +376,8 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe8_kernel(const MoePa
             w_lo = word4_by_row_groups8<T>(lo[j], row_groups, scale_col, p.size_n, magic);
             w_hi = word4_by_row_groups8<T>(hi[j], row_groups + 4, scale_col, p.size_n, magic);
           } else {
-            w_lo = Dq8<T>::word4(lo[j], cols[j], magic);
-            w_hi = Dq8<T>::word4(hi[j], cols[j], magic);
+            w_lo = D8::word4(lo[j], cols[j], magic);
+            w_hi = D8::word4(hi[j], cols[j], magic);
           }
           const vec8 w = __builtin_bit_cast(vec8, u32x4_t{w_lo.x, w_lo.y, w_hi.x, w_hi.y});
 #pragma unroll
@@ -440,18 +441,19 @@ void launch_moe(const MoeParams& p, bool has_perm, int grid, hipStream_t st) {
 }
 
 template <typename T, int MB>
-void launch_moe8(const MoeParams& p, int grid, hipStream_t st) {
-  if (p.g_idx) marlin_moe8_kernel<T, MB, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
-  else marlin_moe8_kernel<T, MB, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
+void launch_moe8(const MoeParams& p, bool fp8, int grid, hipStream_t st) {
+  if (fp8) marlin_moe8_kernel<T, MB, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  else if (p.g_idx) marlin_moe8_kernel<T, MB, true, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  else marlin_moe8_kernel<T, MB, false, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
 }
 
 template <typename T>
-void launch_moe8_mb(const MoeParams& p, int grid, hipStream_t st) {
+void launch_moe8_mb(const MoeParams& p, bool fp8, int grid, hipStream_t st) {
   switch ((p.block_size + 15) / 16) {
-    case 1: launch_moe8<T, 1>(p, grid, st); break;
-    case 2: launch_moe8<T, 2>(p, grid, st); break;
-    case 3: launch_moe8<T, 3>(p, grid, st); break;
-    default: launch_moe8<T, 4>(p, grid, st); break;
+    case 1: launch_moe8<T, 1>(p, fp8, grid, st); break;
+    case 2: launch_moe8<T, 2>(p, fp8, grid, st); break;
+    case 3: launch_moe8<T, 3>(p, fp8, grid, st); break;
+    default: launch_moe8<T, 4>(p, fp8, grid, st); break;
   }
 }
 
@@ -507,19 +509,29 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                 "size_n = %ld, is not divisible by min_thread_n = %d", (long)size_n, kStripN);
   SONAR_REQUIRE(b_scales != nullptr, "b_scales must not be NULL");
   SONAR_REQUIRE(num_groups >= 1, "num_groups = %ld must be >= 1", (long)num_groups);
-  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4 && b_type_id != SONAR_TYPE_UINT8B128)
+  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4 && b_type_id != SONAR_TYPE_UINT8B128 &&
+      b_type_id != SONAR_TYPE_FLOAT8_E4M3FN)
     return fail(SONAR_E_UNSUPPORTED,
-                "b_type id %ld is not built here: only uint4b8, uint8b128 (GPTQ) and uint4 (AWQ) weights are",
+                "b_type id %ld is not built here: only uint4b8, uint8b128 (GPTQ), uint4 (AWQ) and "
+                "float8_e4m3fn weights are",
                 (long)b_type_id);
   const bool has_zp = b_zeros != nullptr;
-  const bool bits8 = b_type_id == SONAR_TYPE_UINT8B128;
+  const bool fp8 = b_type_id == SONAR_TYPE_FLOAT8_E4M3FN;
+  const bool bits8 = b_type_id == SONAR_TYPE_UINT8B128 || fp8;
   if (has_zp)
     SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4, "b_type must be u4 or u8 when has_zp = True");
   else
     SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4B8 || bits8,
-                  "b_type must be uint4b8 or uint8b128 when has_zp = False (uint4 needs b_zeros)");
+                  "b_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   bool has_perm = perm != nullptr;
+  if (fp8) {
+    // moe/marlin_moe_wna16/generate_kernels.py: channelwise scales or groups of 128 rows, no act-order
+    SONAR_REQUIRE(!has_perm, "act-order is not supported with float8_e4m3fn weights");
+    SONAR_REQUIRE(num_groups == 1 || size_k == 128 * num_groups,
+                  "float8_e4m3fn weights take one scale per column or per group of 128 rows; got size_k = %ld, "
+                  "num_groups = %ld", (long)size_k, (long)num_groups);
+  }
   const bool row_groups = has_perm && !is_k_full;
   if (has_perm) {
     SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
@@ -634,8 +646,8 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
       p.unit_chunks = 2;
       p.units_per_strip = p.chunks_per_strip / 2;
     }
-    if (dtype == SONAR_DTYPE_F16) launch_moe8_mb<_Float16>(p, (int)grid, st);
-    else launch_moe8_mb<__bf16>(p, (int)grid, st);
+    if (dtype == SONAR_DTYPE_F16) launch_moe8_mb<_Float16>(p, fp8, (int)grid, st);
+    else launch_moe8_mb<__bf16>(p, fp8, (int)grid, st);
     return launch_status("marlin_moe8_kernel");
   }
   if (dtype == SONAR_DTYPE_F16) {

@@ -372,8 +372,8 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
 }
 
 // ---------------------------------------------------------------------------
-// The general kernel for 8-bit codes (uint8b128, symmetric, no act-order
-// gather): the same partition, reduction and fix-up; a 32-row chunk of a strip
+// The general kernel for 8-bit codes (uint8b128, symmetric, or float8_e4m3fn
+// with FP8; no act-order gather): the same partition, reduction and fix-up; a 32-row chunk of a strip
 // is two 1-KiB blocks of 16 rows, whose words give a lane the low and the high
 // four of the eight consecutive rows of an MFMA operand.
 template <typename T, int MB>
@@ -412,10 +412,11 @@ __device__ __forceinline__ void load_unit8(UnitBuf8<T, MB>& b, const StreamParam
   for (int j = 0; j < 4; ++j) b.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
 }
 
-template <typename T, int MB, bool HAS_GIDX>
+template <typename T, int MB, bool HAS_GIDX, bool FP8>
 __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const StreamParams params) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq8<T>::Col Col;
+  typedef typename Dq8Of<T, FP8>::type D8;
+  typedef typename D8::Col Col;
   __shared__ float4 red[4][MB * 4][64];
   // Several 64-row slabs can share a launch when no strip is shared between
   // workgroups (nothing goes through the scratch slots).
@@ -459,7 +460,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
       if (next < u_end) load_unit8<T, MB>(nxt, p, next, lane, grouped);
       Col cols[4];
 #pragma unroll
-      for (int j = 0; j < 4; ++j) cols[j] = Dq8<T>::make_col((uint16_t)cur.sbits[j]);
+      for (int j = 0; j < 4; ++j) cols[j] = D8::make_col((uint16_t)cur.sbits[j]);
       int cur_group = cur.group;
       const int chunk0 = (mine - strip_first) * p.unit_chunks;
 #pragma unroll
@@ -470,7 +471,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
             cur_group = g;
             const uint16_t* srow = p.scales + (long)g * p.size_n + strip * kStripN;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) cols[j] = Dq8<T>::make_col(srow[scale_slot(16 * j + col16, grouped)]);
+            for (int j = 0; j < 4; ++j) cols[j] = D8::make_col(srow[scale_slot(16 * j + col16, grouped)]);
           }
           const uint32_t lo[4] = {cur.q[cc][0].x, cur.q[cc][0].y, cur.q[cc][0].z, cur.q[cc][0].w};
           const uint32_t hi[4] = {cur.q[cc][1].x, cur.q[cc][1].y, cur.q[cc][1].z, cur.q[cc][1].w};
@@ -489,8 +490,8 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
               w_lo = word4_by_row_groups8<T>(lo[j], row_groups, scale_col, p.size_n, magic);
               w_hi = word4_by_row_groups8<T>(hi[j], row_groups + 4, scale_col, p.size_n, magic);
             } else {
-              w_lo = Dq8<T>::word4(lo[j], cols[j], magic);
-              w_hi = Dq8<T>::word4(hi[j], cols[j], magic);
+              w_lo = D8::word4(lo[j], cols[j], magic);
+              w_hi = D8::word4(hi[j], cols[j], magic);
             }
             const vec8 w = __builtin_bit_cast(vec8, u32x4_t{w_lo.x, w_lo.y, w_hi.x, w_hi.y});
 #pragma unroll
@@ -1101,7 +1102,7 @@ __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __rest
 }
 
 // The same for 8-bit codes: one wavefront per 1-KiB block of 16 rows.
-template <typename T>
+template <typename T, bool FP8>
 __global__ __launch_bounds__(256) void marlin_dequant8_kernel(const uint4* __restrict__ b,
                                                              const uint16_t* __restrict__ scales,
                                                              const int32_t* __restrict__ g_idx,
@@ -1133,7 +1134,8 @@ __global__ __launch_bounds__(256) void marlin_dequant8_kernel(const uint4* __res
         w = word4_by_row_groups8<T>(words[j], row_groups, scales + strip * kStripN + scale_slot(16 * j + col16, true),
                                     size_n, magic);
       else
-        w = Dq8<T>::word4(words[j], Dq8<T>::make_col(srow[scale_slot(16 * j + col16, grouped)]), magic);
+        w = Dq8Of<T, FP8>::type::word4(
+            words[j], Dq8Of<T, FP8>::type::make_col(srow[scale_slot(16 * j + col16, grouped)]), magic);
       const uint16_t bits[4] = {(uint16_t)(w.x & 0xffffu), (uint16_t)(w.x >> 16), (uint16_t)(w.y & 0xffffu),
                                 (uint16_t)(w.y >> 16)};
 #pragma unroll
@@ -1202,20 +1204,21 @@ void launch_stream_mb(const StreamParams& p, bool has_perm, hipStream_t st) {
   }
 }
 
-template <typename T, bool HAS_GIDX>
+template <typename T, bool HAS_GIDX, bool FP8>
 void launch_stream8_gidx(const StreamParams& p, hipStream_t st) {
   switch ((p.size_m + 15) / 16) {
-    case 1: marlin_stream8_kernel<T, 1, HAS_GIDX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    case 2: marlin_stream8_kernel<T, 2, HAS_GIDX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    case 3: marlin_stream8_kernel<T, 3, HAS_GIDX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    default: marlin_stream8_kernel<T, 4, HAS_GIDX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 1: marlin_stream8_kernel<T, 1, HAS_GIDX, FP8><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 2: marlin_stream8_kernel<T, 2, HAS_GIDX, FP8><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 3: marlin_stream8_kernel<T, 3, HAS_GIDX, FP8><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    default: marlin_stream8_kernel<T, 4, HAS_GIDX, FP8><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
   }
 }
 
 template <typename T>
-void launch_stream8_mb(const StreamParams& p, hipStream_t st) {
-  if (p.g_idx) launch_stream8_gidx<T, true>(p, st);
-  else launch_stream8_gidx<T, false>(p, st);
+void launch_stream8_mb(const StreamParams& p, bool fp8, hipStream_t st) {
+  if (fp8) launch_stream8_gidx<T, false, true>(p, st);   // no act-order with floating-point codes
+  else if (p.g_idx) launch_stream8_gidx<T, true, false>(p, st);
+  else launch_stream8_gidx<T, false, false>(p, st);
 }
 
 template <typename T, bool HAS_ZP, int WAVES, int MB, bool GROUPED, int GPU>
@@ -1275,6 +1278,7 @@ struct Checked {
   bool row_groups;  // act-order shard without whole groups: the group of a row comes from g_idx
   int group_size;
   int bits;         // 4 or 8
+  bool fp8;         // 8-bit floating-point codes (float8_e4m3fn)
 };
 
 int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_t* b_zeros,
@@ -1288,19 +1292,29 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
                 "size_n = %ld, is not divisible by min_thread_n = %d", (long)size_n, kStripN);
   SONAR_REQUIRE(b_scales != nullptr, "b_scales must not be NULL");
   SONAR_REQUIRE(num_groups >= 1, "num_groups = %ld must be >= 1", (long)num_groups);
-  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4 && b_type_id != SONAR_TYPE_UINT8B128)
+  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4 && b_type_id != SONAR_TYPE_UINT8B128 &&
+      b_type_id != SONAR_TYPE_FLOAT8_E4M3FN)
     return fail(SONAR_E_UNSUPPORTED,
-                "b_type id %ld is not built here: only uint4b8, uint8b128 (GPTQ) and uint4 (AWQ) weights are",
+                "b_type id %ld is not built here: only uint4b8, uint8b128 (GPTQ), uint4 (AWQ) and "
+                "float8_e4m3fn weights are",
                 (long)b_type_id);
-  out.bits = b_type_id == SONAR_TYPE_UINT8B128 ? 8 : 4;
+  out.fp8 = b_type_id == SONAR_TYPE_FLOAT8_E4M3FN;
+  out.bits = (b_type_id == SONAR_TYPE_UINT8B128 || out.fp8) ? 8 : 4;
   out.has_zp = b_zeros != nullptr;
   if (out.has_zp)
     SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4, "b_type must be u4 or u8 when has_zp = True");
   else
     SONAR_REQUIRE(b_type_id != SONAR_TYPE_UINT4,
-                  "b_type must be uint4b8 or uint8b128 when has_zp = False (uint4 needs b_zeros)");
+                  "b_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   out.has_perm = perm != nullptr;
+  if (out.fp8) {
+    // generate_kernels.py:87-93: channelwise scales or groups of 128 rows, no act-order
+    SONAR_REQUIRE(!out.has_perm, "act-order is not supported with float8_e4m3fn weights");
+    SONAR_REQUIRE(num_groups == 1 || size_k == 128 * num_groups,
+                  "float8_e4m3fn weights take one scale per column or per group of 128 rows; got size_k = %ld, "
+                  "num_groups = %ld", (long)size_k, (long)num_groups);
+  }
   out.row_groups = out.has_perm && !is_k_full;
   if (out.has_perm) SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
   if (out.row_groups) {
@@ -1617,8 +1631,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
         m0 = size_m;
       }
       if (chk.bits == 8) {
-        if (dtype == SONAR_DTYPE_F16) launch_stream8_mb<_Float16>(p, st);
-        else launch_stream8_mb<__bf16>(p, st);
+        if (dtype == SONAR_DTYPE_F16) launch_stream8_mb<_Float16>(p, chk.fp8, st);
+        else launch_stream8_mb<__bf16>(p, chk.fp8, st);
       } else if (dtype == SONAR_DTYPE_F16) {
         if (chk.has_zp) launch_stream_mb<_Float16, true>(p, chk.has_perm, st);
         else launch_stream_mb<_Float16, false>(p, chk.has_perm, st);
@@ -1659,8 +1673,14 @@ extern "C" int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout, co
     long grid = (total_blocks + 3) / 4;
     if (grid > 8192) grid = 8192;
     const int32_t* gi8 = chk.row_groups ? g_idx : nullptr;
-    if (dtype == SONAR_DTYPE_F16) marlin_dequant8_kernel<_Float16><<<(int)grid, 256, 0, st>>>(b, s, gi8, w, n, k, ng, gs, total_blocks);
-    else marlin_dequant8_kernel<__bf16><<<(int)grid, 256, 0, st>>>(b, s, gi8, w, n, k, ng, gs, total_blocks);
+    if (chk.fp8) {
+      if (dtype == SONAR_DTYPE_F16) marlin_dequant8_kernel<_Float16, true><<<(int)grid, 256, 0, st>>>(b, s, gi8, w, n, k, ng, gs, total_blocks);
+      else marlin_dequant8_kernel<__bf16, true><<<(int)grid, 256, 0, st>>>(b, s, gi8, w, n, k, ng, gs, total_blocks);
+    } else if (dtype == SONAR_DTYPE_F16) {
+      marlin_dequant8_kernel<_Float16, false><<<(int)grid, 256, 0, st>>>(b, s, gi8, w, n, k, ng, gs, total_blocks);
+    } else {
+      marlin_dequant8_kernel<__bf16, false><<<(int)grid, 256, 0, st>>>(b, s, gi8, w, n, k, ng, gs, total_blocks);
+    }
     return launch_status("marlin_dequant8_kernel");
   }
   const int32_t* gi = chk.row_groups ? g_idx : nullptr;

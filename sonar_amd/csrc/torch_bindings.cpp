@@ -180,9 +180,10 @@ Tensor marlin_to_gfx950(const Tensor& b_q_weight, int64_t size_k, int64_t size_n
 // ---------------------------------------------------------------- dense GEMM
 void check_b_type(int64_t b_type_id) {
   TORCH_CHECK_NOT_IMPLEMENTED(
-      b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4 || b_type_id == SONAR_TYPE_UINT8B128,
+      b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4 || b_type_id == SONAR_TYPE_UINT8B128 ||
+          b_type_id == SONAR_TYPE_FLOAT8_E4M3FN,
       "b_type_id = ", b_type_id,
-      " is not built here: only uint4b8, uint8b128 (GPTQ) and uint4 (AWQ) weights are supported");
+      " is not built here: only uint4b8, uint8b128 (GPTQ), uint4 (AWQ) and float8_e4m3fn weights are supported");
 }
 
 Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_q_weight,
@@ -207,7 +208,7 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
               ", tile_size = ", 16);
   TORCH_CHECK(b_q_weight.size(1) % 16 == 0, "b_q_weight.size(1) = ", b_q_weight.size(1),
               " is not divisible by tile_size = ", 16);
-  const int bits = b_type_id == SONAR_TYPE_UINT8B128 ? 8 : 4;
+  const int bits = (b_type_id == SONAR_TYPE_UINT8B128 || b_type_id == SONAR_TYPE_FLOAT8_E4M3FN) ? 8 : 4;
   const int64_t actual_size_n = b_q_weight.size(1) / 16 * (32 / bits);
   TORCH_CHECK(size_n == actual_size_n, "size_n = ", size_n, ", actual_size_n = ", actual_size_n);
 
@@ -337,7 +338,7 @@ Tensor moe_wna16_marlin_gemm(
   TORCH_CHECK(size_k % 16 == 0 && size_k / 16 == b_q_weight.size(1),
               "Shape mismatch: b_q_weight.size(1) = ", b_q_weight.size(1), ", size_k = ", size_k,
               ", tile_size = ", 16);
-  const int bits = b_type_id == SONAR_TYPE_UINT8B128 ? 8 : 4;
+  const int bits = (b_type_id == SONAR_TYPE_UINT8B128 || b_type_id == SONAR_TYPE_FLOAT8_E4M3FN) ? 8 : 4;
   const int64_t pack_factor = 32 / bits;
   TORCH_CHECK(b_q_weight.size(2) % 16 == 0 && b_q_weight.size(2) / 16 * pack_factor == size_n,
               "size_n = ", size_n, ", actual_size_n = ", b_q_weight.size(2) / 16 * pack_factor);
@@ -391,8 +392,8 @@ Tensor moe_wna16_marlin_gemm(
     TORCH_CHECK(z.dim() == 3 && z.size(1) == num_groups && z.size(2) == size_n / 8,
                 "b_zeros must be (E, num_groups, size_n / 8)");
   } else {
-    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT8B128,
-                "b_type must be uint4b8 or uint8b128 when has_zp = False. Got = uint4");
+    TORCH_CHECK(b_type_id != SONAR_TYPE_UINT4,
+                "b_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False. Got = uint4");
   }
   TORCH_CHECK(sorted_token_ids.is_cuda() && sorted_token_ids.scalar_type() == at::kInt &&
                   sorted_token_ids.is_contiguous(), "sorted_token_ids must be a contiguous int32 GPU tensor");

@@ -29,12 +29,15 @@ def round_up(x: int, m: int) -> int:
 
 
 def query_marlin_supported_quant_types(has_zp: bool | None = None, include_fp_type: bool = True):
-    """Integer types only: uint4 with zero points; uint4b8 and uint8b128 without
-    (marlin_utils.py:64-108 of the reference lists more: uint8 with zero points
-    and the fp8 / fp4 types are not built here)."""
+    """uint4 with zero points; uint4b8, uint8b128 and (with include_fp_type)
+    float8_e4m3fn without (marlin_utils.py:64-108 of the reference lists more:
+    uint8 with zero points and float4_e2m1f are not built here)."""
+    without = [scalar_types.uint4b8, scalar_types.uint8b128]
+    if include_fp_type:
+        without.append(scalar_types.float8_e4m3fn)
     if has_zp is None:
-        return [scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128]
-    return [scalar_types.uint4] if has_zp else [scalar_types.uint4b8, scalar_types.uint8b128]
+        return without + [scalar_types.uint4]
+    return [scalar_types.uint4] if has_zp else without
 
 
 def check_marlin_supports_shape(output_size_per_partition: int, input_size_per_partition: int,

@@ -1,12 +1,15 @@
 """Sub-byte scalar type descriptor whose integer id crosses the op boundary as
 `b_type_id`.  Mirrors aphrodite/scalar_type.py:22-340 of the reference (id
-bitfield :129-156) for the integer types this build handles."""
+bitfield :129-156) for the integer types this build handles and the 8-bit
+floating-point weight type float8_e4m3fn."""
 from __future__ import annotations
 
 import functools
 from dataclasses import dataclass
 
+_NAN_REPR_NONE = 0
 _NAN_REPR_IEEE_754 = 1
+_NAN_REPR_EXTD_RANGE_MAX_MIN = 2   # NaN: exponent and mantissa all ones; no infinities
 
 
 @dataclass(frozen=True)
@@ -53,7 +56,12 @@ class ScalarType:
         return val
 
     def __str__(self) -> str:
-        assert self.is_integer()
+        if self.is_floating_point():   # scalar_type.py:223-233: f = no infinities, n = non-standard NaNs
+            s = f"float{self.size_bits}_e{self.exponent}m{self.mantissa}"
+            if self.nan_repr != _NAN_REPR_IEEE_754 or self._finite_values_only:
+                s += "f" if self._finite_values_only else ""
+                s += "n" if self.nan_repr != _NAN_REPR_NONE else ""
+            return s
         s = ("int" if self.signed else "uint") + str(self.size_bits)
         return s + (f"b{self.bias}" if self.bias else "")
 
@@ -65,6 +73,12 @@ class ScalarType:
     def uint(cls, size_bits: int, bias: int | None) -> "ScalarType":
         return cls(0, size_bits, False, bias or 0)
 
+    @classmethod
+    def float_(cls, exponent: int, mantissa: int, finite_values_only: bool, nan_repr: int) -> "ScalarType":
+        """A floating-point type that does not follow IEEE 754 (scalar_type.py:276-289)."""
+        assert mantissa > 0 and exponent > 0 and nan_repr != _NAN_REPR_IEEE_754
+        return cls(exponent, mantissa, True, 0, finite_values_only, nan_repr)
+
 
 class scalar_types:
     int4 = ScalarType.int_(4, None)
@@ -73,3 +87,4 @@ class scalar_types:
     uint8 = ScalarType.uint(8, None)
     uint4b8 = ScalarType.uint(4, 8)
     uint8b128 = ScalarType.uint(8, 128)
+    float8_e4m3fn = ScalarType.float_(4, 3, True, _NAN_REPR_EXTD_RANGE_MAX_MIN)

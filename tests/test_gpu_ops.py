@@ -483,3 +483,129 @@ def test_fused_marlin_moe_replays_in_a_hip_graph():
         ti.copy_(ti2)
         eager = run().clone()
         torch.cuda.synchronize()
+
+
+# ---------------------------------------------------------------- fp8 weights (float8_e4m3fn)
+@pytest.mark.parametrize("m,k,n,g,dtype", [(1, 512, 256, -1, "fp16"), (33, 1024, 320, 128, "bf16"),
+                                           (16, 4096, 4096, 128, "fp16"), (200, 256, 512, -1, "bf16")])
+def test_fp8_quantise_helper_and_marlin_gemm(m, k, n, g, dtype):
+    """The reference's fp8 case of its Marlin GEMM test (tests/kernels/quantization/
+    test_marlin_gemm.py with marlin_quant_fp8_torch): quantise a random weight,
+    run the op, compare with the matmul on the dequantised weight."""
+    from sonar_amd import marlin_utils_fp8 as f8
+    from sonar_amd import ops
+    from sonar_amd.marlin_utils import marlin_make_workspace_new
+    from sonar_amd.scalar_type import scalar_types
+    gen = torch.Generator(device="cpu").manual_seed(m + k)
+    weight = torch.randn((n, k), generator=gen).to(_tdt(dtype)).to(gu.DEV)
+    a = (0.5 * torch.randn((m, k), generator=gen)).to(_tdt(dtype)).to(gu.DEV)
+    w_ref, qweight, scales = f8.marlin_quant_fp8_torch(weight, g)
+    assert qweight.shape == (k // 16, 4 * n) and scales.shape == (1 if g == -1 else k // g, n)
+    out = ops.marlin_gemm(a, None, qweight, None, scales, None, None, None, None, None,
+                          marlin_make_workspace_new(a.device), scalar_types.float8_e4m3fn, m, n, k)
+    torch.cuda.synchronize()
+    want = (a.float() @ w_ref.float()).cpu().numpy()
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(out), want)
+    assert ok, worst
+
+
+@pytest.mark.parametrize("mode,dtype", [("block", "bf16"), ("tensor", "fp16"), ("shards", "bf16"),
+                                        ("channel", "fp16"), ("block_padded", "fp16")])
+def test_prepare_fp8_layer_and_apply(mode, dtype):
+    """An fp8 checkpoint layer (weight (N, K) fp8, scales per tensor / per fused
+    shard / per channel / per 128 x 128 block) -> prepare_fp8_layer_for_marlin ->
+    apply_fp8_marlin_linear, against the oracle on the same bytes and scales."""
+    from sonar_amd import marlin_utils_fp8 as f8
+    k, n = (512, 384) if mode != "block_padded" else (384, 320)   # 320 columns: padded to 384 inside
+    rng = np.random.default_rng(len(mode))
+    codes = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    codes[(codes & 0x7F) == 0x7F] = 0x30
+    layer = types.SimpleNamespace(output_size_per_partition=n, input_size_per_partition=k, orig_dtype=_tdt(dtype))
+    layer.weight = torch.from_numpy(codes.T.astype(np.uint8)).contiguous().to(gu.DEV).view(torch.float8_e4m3fn)
+    g = -1
+    if mode.startswith("block"):
+        layer.weight_block_size = [128, 128]
+        g = 128
+        blocks = rng.uniform(2e-4, 2e-3, size=((n + 127) // 128, k // 128)).astype(np.float32)
+        layer.weight_scale_inv = torch.from_numpy(blocks).to(gu.DEV)
+        s_full = np.repeat(blocks.T, 128, axis=1)[:, :n]
+    elif mode == "tensor":
+        layer.weight_scale = torch.tensor(7e-4, device=gu.DEV)
+        s_full = np.full((1, n), 7e-4, dtype=np.float32)
+    elif mode == "shards":
+        layer.logical_widths = [128, 64, 192]
+        per = np.array([3e-4, 9e-4, 5e-4], dtype=np.float32)
+        layer.weight_scale = torch.from_numpy(per).to(gu.DEV)
+        s_full = np.repeat(per, layer.logical_widths)[None, :]
+    else:
+        per = rng.uniform(2e-4, 2e-3, size=n).astype(np.float32)
+        layer.weight_scale = torch.from_numpy(per).to(gu.DEV)
+        s_full = per[None, :]
+    bias32 = mo.round_to_dtype(rng.standard_normal(n).astype(np.float32), dtype)
+    layer.bias = gu.dev_bits16(bias32, dtype)
+    s_full = mo.round_to_dtype(s_full, dtype)
+    w_ref = mo.dequantize_fp8(codes, mo.fp8_fuse_exponent_bias(s_full, dtype), g, dtype)
+
+    f8.prepare_fp8_layer_for_marlin(layer, size_k_first=False)
+    scales = layer.weight_scale_inv if mode.startswith("block") else layer.weight_scale
+    x32 = mo.make_activations(3, 5, k, dtype, std=0.5)
+    y = f8.apply_fp8_marlin_linear(gu.dev_bits16(x32, dtype).view(1, 5, k), layer.weight, scales, layer.workspace,
+                                   n, k, layer.bias)
+    torch.cuda.synchronize()
+    assert y.shape == (1, 5, n)
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y.view(5, n)), mo.gemm_reference(x32, w_ref, bias32))
+    assert ok, worst
+
+
+@pytest.mark.parametrize("cfg", [
+    # m, experts, topk, hidden, intermediate, dtype, scales
+    (5, 4, 2, 256, 128, "fp16", "tensor"),
+    (70, 4, 2, 256, 256, "bf16", "block"),
+    (33, 8, 2, 128, 128, "bf16", "channel"),
+    (9, 4, 2, 256, 96, "fp16", "channel"),      # intermediate size padded 96 -> 128
+], ids=str)
+def test_prepare_fp8_moe_layer_and_fused_marlin_moe(cfg):
+    """fp8 expert weights (w13 (E, 2N, K), w2 (E, K, N)) -> prepare_fp8_moe_layer_for_marlin
+    -> fused_marlin_moe, against the per-token reference on the same bytes."""
+    from sonar_amd import marlin_utils_fp8 as f8
+    from sonar_amd.fused_moe import fused_marlin_moe
+    from sonar_amd.scalar_type import scalar_types
+    m, e, topk, hidden, inter, dtype, mode = cfg
+    rng = np.random.default_rng(hidden + inter + m)
+    layer = types.SimpleNamespace(num_experts=e, hidden_size=hidden, intermediate_size_per_partition=inter,
+                                  orig_dtype=_tdt(dtype))
+    if mode == "block":
+        layer.weight_block_size = [128, 128]
+
+    def expert_set(rows, cols):   # checkpoint shape (E, rows = N of the GEMM, cols = K of the GEMM)
+        codes = rng.integers(0, 256, size=(e, rows, cols), dtype=np.int32)
+        codes[(codes & 0x7F) == 0x7F] = 0x30
+        weight = torch.from_numpy(codes.astype(np.uint8)).to(gu.DEV).view(torch.float8_e4m3fn)
+        if mode == "tensor":
+            raw = rng.uniform(2e-4, 2e-3, size=e).astype(np.float32)
+            full = np.broadcast_to(raw[:, None, None], (e, 1, rows))
+        elif mode == "channel":
+            raw = rng.uniform(2e-4, 2e-3, size=(e, rows)).astype(np.float32)
+            full = raw[:, None, :]
+        else:
+            raw = rng.uniform(2e-4, 2e-3, size=(e, (rows + 127) // 128, cols // 128)).astype(np.float32)
+            full = np.repeat(raw.transpose(0, 2, 1), 128, axis=2)[..., :rows]
+        full = mo.round_to_dtype(np.ascontiguousarray(full), dtype)
+        g = 128 if mode == "block" else -1
+        ref = [mo.dequantize_fp8(codes[i].T, mo.fp8_fuse_exponent_bias(full[i], dtype), g, dtype) for i in range(e)]
+        return weight, torch.from_numpy(raw).to(gu.DEV), ref
+
+    w13, s13, ref13 = expert_set(2 * inter, hidden)
+    w2, s2, ref2 = expert_set(hidden, inter)
+    layer.w13_weight = w13
+    mw13, mw2, ms13, ms2 = f8.prepare_fp8_moe_layer_for_marlin(layer, w13, w2, s13, s2)
+    topk_ids, topk_w = _route(m, e, topk, m)
+    x32 = mo.round_to_dtype(0.5 * mo.make_activations(m, m, hidden, dtype), dtype)
+    y = fused_marlin_moe(gu.dev_bits16(x32, dtype), mw13, mw2, None, None, ms13, ms2,
+                         torch.from_numpy(topk_w).to(gu.DEV), torch.from_numpy(topk_ids).to(gu.DEV),
+                         scalar_types.float8_e4m3fn.id)
+    torch.cuda.synchronize()
+    want = _moe_reference(x32, ref13, ref2, topk_ids, topk_w, dtype)
+    got = gu.host_f32(y)
+    max_ref = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)

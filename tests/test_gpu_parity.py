@@ -384,6 +384,101 @@ def test_w8a16_dequant_bit_exact_and_gemm_within_tolerance(gu, dtype, m, k, n, g
     assert ok, f"max_err={max_err} max_ref={max_ref}"
 
 
+def _layer_fp8(gu, seed, k, n, g, dtype, all_codes=False):
+    """A float8_e4m3fn layer on the device: the codes packed four to a word along
+    K -> repack op (num_bits = 8) -> streaming order; scales permuted, with the
+    exponent bias folded in; plus the oracle's dequantised matrix."""
+    from sonar_amd import _lib
+    rng = np.random.default_rng(seed)
+    codes = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    if all_codes:
+        codes[:256, 0] = np.arange(256)   # every code, the two NaN codes included, in one column
+    else:
+        codes[(codes & 0x7F) == 0x7F] = 0x3C
+    groups = 1 if g in (-1, k) else k // g
+    scales = mo.round_to_dtype(rng.uniform(2e-4, 2e-3, size=(groups, n)).astype(np.float32), dtype)
+    fused = mo.fp8_fuse_exponent_bias(scales, dtype)
+    w_ref = mo.dequantize_fp8(codes, fused, g, dtype)
+    lib = _lib.load()
+    marlin = torch.empty((k // 16, 4 * n), dtype=torch.int32, device=gu.DEV)
+    _lib.check(lib.sonar_gptq_marlin_repack(gu.ptr(gu.dev_i32(mo.pack_rows8(codes))), None, gu.ptr(marlin),
+                                            k, n, 8, gu.stream()))
+    native = torch.empty_like(marlin)
+    _lib.check(lib.sonar_marlin8_to_gfx950(gu.ptr(marlin), gu.ptr(native), k, n, gu.stream()))
+    s_dev = gu.dev_bits16(mo.marlin_permute_scales(fused, k, n, -1 if groups == 1 else g), dtype)
+    return dict(codes=codes, native=native, scales=s_dev, groups=groups, w_ref=w_ref)
+
+
+FP8_CASES = [
+    # m, k, n, g, bias
+    (1, 128, 64, 128, False),
+    (7, 512, 256, -1, True),
+    (16, 4096, 1024, 128, False),
+    (33, 1024, 320, 128, True),
+    (64, 256, 4096, -1, False),
+    (100, 1024, 512, 128, False),
+    (300, 512, 192, -1, True),
+    (1, 4096, 4096, 128, False),
+]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("m,k,n,g,bias", FP8_CASES)
+def test_fp8_weights_dequant_bit_exact_and_gemm_within_tolerance(gu, dtype, m, k, n, g, bias):
+    """float8_e4m3fn weights through the same entry points (generate_kernels.py:
+    87-93; dequant.h:320-380: the code read as a 16-bit float, times the scale
+    with the exponent bias folded in)."""
+    from sonar_amd import _lib
+    lib = _lib.load()
+    L = _layer_fp8(gu, 5 * m + k, k, n, g, dtype, all_codes=k >= 256)
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    w = torch.empty((k, n), dtype=tdt, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_dequant(gu.ptr(L["native"]), _lib.LAYOUT_GFX950, gu.ptr(L["scales"]), None,
+                                        None, gu.ptr(w), gu.dtype_code(dtype), _lib.TYPE_FLOAT8_E4M3FN,
+                                        n, k, L["groups"], 1, gu.stream()))
+    torch.cuda.synchronize()
+    got = w.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, mo.to_bits16(L["w_ref"], dtype))   # bits: the code 0x80 gives -0
+
+    bias32 = bias_dev = None
+    if bias:
+        bias32 = mo.round_to_dtype(np.random.default_rng(m).standard_normal(n).astype(np.float32), dtype)
+        bias_dev = gu.dev_bits16(mo.marlin_permute_bias(bias32), dtype)
+    a32 = mo.make_activations(m + 1, m, k, dtype, std=0.5)
+    a = gu.dev_bits16(a32, dtype)
+    c = torch.empty((m, n), dtype=tdt, device=gu.DEV)
+    workspace = torch.zeros(torch.cuda.get_device_properties(0).multi_processor_count, dtype=torch.int32,
+                            device=gu.DEV)
+    scratch = torch.empty(max(lib.sonar_marlin_gemm_scratch_bytes(m, n, k), 16), dtype=torch.uint8, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_gemm(
+        gu.ptr(a), k, gu.ptr(c), gu.ptr(L["native"]), _lib.LAYOUT_GFX950, gu.ptr(bias_dev), gu.ptr(L["scales"]), None,
+        None, None, gu.ptr(workspace), workspace.numel(), gu.ptr(scratch), scratch.numel(),
+        gu.dtype_code(dtype), _lib.TYPE_FLOAT8_E4M3FN, m, n, k, L["groups"], 1, 0, 1, gu.stream()))
+    torch.cuda.synchronize()
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), mo.gemm_reference(a32, L["w_ref"], bias32))
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+
+
+def test_fp8_weights_rejected_configurations(gu):
+    """Groups other than 128 rows and act-order do not exist for fp8 weights
+    (generate_kernels.py:87-93: group_blocks -1 and 8 only)."""
+    from sonar_amd import _lib
+    lib = _lib.load()
+    k, n = 256, 64
+    L = _layer_fp8(gu, 1, k, n, 128, "fp16")
+    w = torch.empty((k, n), dtype=torch.float16, device=gu.DEV)
+    idx = torch.zeros(k, dtype=torch.int32, device=gu.DEV)
+
+    def dequant(groups, g_idx):
+        return lib.sonar_marlin_dequant(gu.ptr(L["native"]), _lib.LAYOUT_GFX950, gu.ptr(L["scales"]), None,
+                                        gu.ptr(g_idx), gu.ptr(w), 0, _lib.TYPE_FLOAT8_E4M3FN, n, k, groups, 1,
+                                        gu.stream())
+    assert dequant(2, None) == 0
+    assert dequant(4, None) != 0 and "128" in lib.sonar_marlin_last_error().decode()
+    assert dequant(2, idx) != 0 and "act-order" in lib.sonar_marlin_last_error().decode()
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("m", [1, 16, 40, 100, 300])
 def test_act_order_shard_without_whole_groups(gu, dtype, m):

@@ -34,7 +34,11 @@ def test_type_id_constants_match_header_and_oracle():
     assert int(re.search(r"SONAR_TYPE_UINT4 (\d+)LL", header).group(1)) == mo.UINT4_ID
     assert scalar_types.uint4b8.id == mo.UINT4B8_ID == _lib.TYPE_UINT4B8
     assert scalar_types.uint4.id == mo.UINT4_ID == _lib.TYPE_UINT4
-    assert scalar_types.uint8b128.id == mo.UINT8B128_ID
+    assert scalar_types.uint8b128.id == mo.UINT8B128_ID == _lib.TYPE_UINT8B128
+    assert int(re.search(r"SONAR_TYPE_FLOAT8_E4M3FN (\d+)LL", header).group(1)) == mo.FLOAT8_E4M3FN_ID
+    assert scalar_types.float8_e4m3fn.id == mo.FLOAT8_E4M3FN_ID == _lib.TYPE_FLOAT8_E4M3FN
+    assert str(scalar_types.float8_e4m3fn) == "float8_e4m3fn" and scalar_types.float8_e4m3fn.size_bits == 8
+    assert str(scalar_types.uint8b128) == "uint8b128" and str(scalar_types.int4) == "int4"
     # tests/test_scalartype.py:10-25 of the reference
     for lo, hi, t in [(-8, 7, scalar_types.int4), (0, 15, scalar_types.uint4),
                       (-8, 7, scalar_types.uint4b8), (-128, 127, scalar_types.uint8b128),
@@ -458,3 +462,31 @@ def test_marlin_post_load_preserves_runtime_tensor_addresses(monkeypatch):
     assert layer.g_idx_sort_indices.data_ptr() == sort_ptr
     assert torch.equal(layer.g_idx_sort_indices.data, marlin_utils.marlin_sort_g_idx(second)[1])
     assert isinstance(layer.g_idx_sort_indices, torch.nn.Parameter)
+
+
+def test_fp8_host_helpers():
+    """marlin_utils_fp8.py:35-46, 366-378 of the reference: the exponent-bias
+    factor (2^8 / 2^120) and the packing of four consecutive K to a word, on
+    values worked out by hand; fp8 joins the supported types without zero points."""
+    from sonar_amd import marlin_utils as mu
+    from sonar_amd import marlin_utils_fp8 as f8
+    from sonar_amd.scalar_type import scalar_types as st
+    s = torch.tensor([[0.5, 3.0]], dtype=torch.float16)
+    assert torch.equal(f8.fp8_fused_exponent_bias_into_scales(s), torch.tensor([[128.0, 768.0]], dtype=torch.float16))
+    s = torch.tensor([[2.0 ** -10]], dtype=torch.bfloat16)
+    assert f8.fp8_fused_exponent_bias_into_scales(s).float().item() == 2.0 ** 110
+    with pytest.raises(TypeError):
+        f8.fp8_fused_exponent_bias_into_scales(torch.ones(1))
+    # (K, N) = (8, 2): word [k/4][n] holds codes k%4 = 0..3 from the low byte up
+    codes = torch.arange(16, dtype=torch.uint8).view(8, 2)
+    words = f8.pack_fp8_to_int32(codes.view(torch.float8_e4m3fn), size_k_first=True)
+    assert words.shape == (2, 2) and words.dtype == torch.int32
+    assert words[0, 0].item() == 0 | (2 << 8) | (4 << 16) | (6 << 24)
+    assert words[1, 1].item() == 9 | (11 << 8) | (13 << 16) | (15 << 24)
+    by_n = f8.pack_fp8_to_int32(codes.T.contiguous().view(torch.float8_e4m3fn), size_k_first=False)
+    assert torch.equal(by_n.T, words)
+    assert np.array_equal(words.numpy().view(np.uint32), mo.pack_rows8(codes.numpy().astype(np.int32)).view(np.uint32))
+    assert mu.check_marlin_supported(st.float8_e4m3fn, 128) and mu.check_marlin_supported(st.float8_e4m3fn, -1)
+    assert not mu.check_marlin_supported(st.float8_e4m3fn, 128, has_zp=True)
+    assert st.float8_e4m3fn not in mu.query_marlin_supported_quant_types(False, include_fp_type=False)
+    assert f8.is_fp8_marlin_supported()

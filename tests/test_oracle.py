@@ -393,3 +393,52 @@ def test_dequant8_exhaustive_against_exact_rationals(dtype):
             want = _rne_fraction_to(dtype, Fraction(code - 128) * Fraction(float(sv)))
             assert w[code, j] == np.float32(want), (dtype, code, sv)
     assert np.all(w[128] == 0)
+
+
+# ---------------------------------------------------------------- fp8 weights (float8_e4m3fn)
+def test_fp8_type_id_and_value_table():
+    import torch
+    assert mo.FLOAT8_E4M3FN_ID == 4 | (3 << 8) | (1 << 16) | (1 << 49) | (2 << 50) == 2814749767172868
+    v = mo.fp8_e4m3fn_values()
+    # torch's own conversion of the 254 finite codes (the two NaN codes aside)
+    t = torch.arange(256, dtype=torch.uint8).view(torch.float8_e4m3fn).float().numpy()
+    finite = np.isfinite(t)
+    assert finite.sum() == 254 and not finite[0x7F] and not finite[0xFF]
+    assert np.array_equal(v[finite], t[finite])
+    assert np.array_equal(np.signbit(v[finite]), np.signbit(t[finite]))   # 0x80 is -0
+    # hand values: 1, the largest (1.75 * 2^8), the smallest subnormal, the smallest normal, -2
+    assert v[0x38] == 1.0 and v[0x7E] == 448.0 and v[0x01] == 2.0 ** -9 and v[0x08] == 2.0 ** -6 and v[0xC0] == -2.0
+    assert v[0x7F] == 480.0 and v[0xFF] == -480.0   # what the bit trick makes of the NaN codes
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_fp8_kernel_recipe_equals_value_times_scale(dtype):
+    """The code read as a 16-bit float is value * 2^-8 / 2^-120 for every code,
+    and the recipe (that reading times the scale with the bias folded in) is
+    round-to-nearest-even of value * scale in exact arithmetic."""
+    v = mo.fp8_e4m3fn_values()
+    shift = mo.FP8_EXPONENT_BIAS_SHIFT[dtype]
+    as16 = mo.fp8_code_as_16bit_float(np.arange(256), dtype)
+    assert all(Fraction(float(as16[c])) * Fraction(2) ** shift == Fraction(float(v[c])) for c in range(256))
+    rng = np.random.default_rng(13)
+    raw = np.concatenate([rng.uniform(1e-4, 1e-2, 24), np.array([1.0, 2.0 ** -10, 3.0e-5, 0.333, 0.0])])
+    s = mo.round_to_dtype(raw.astype(np.float32), dtype)
+    fused = mo.fp8_fuse_exponent_bias(s, dtype)
+    assert all(Fraction(float(f)) == Fraction(float(x)) * Fraction(2) ** shift for f, x in zip(fused, s))
+    codes = np.tile(np.arange(256, dtype=np.int32)[:, None], (1, s.size))
+    w = mo.dequantize_fp8(codes, fused[None, :], -1, dtype)
+    for j, sv in enumerate(s):
+        for code in range(256):
+            want = _rne_fraction_to(dtype, Fraction(float(v[code])) * Fraction(float(sv)))
+            assert w[code, j] == np.float32(want), (dtype, code, sv)
+    assert np.all(w[0] == 0) and np.all(w[0x80] == 0)
+
+
+def test_fp8_dequant_groups():
+    rng = np.random.default_rng(14)
+    codes = rng.integers(0, 256, size=(256, 8), dtype=np.int32)
+    s = mo.round_to_dtype(rng.uniform(1e-3, 1e-2, size=(2, 8)).astype(np.float32), "fp16")
+    w = mo.dequantize_fp8(codes, mo.fp8_fuse_exponent_bias(s, "fp16"), 128, "fp16")
+    v = mo.fp8_e4m3fn_values()
+    assert np.array_equal(w[:128], mo.round_to_dtype(v[codes[:128]] * s[0], "fp16"))
+    assert np.array_equal(w[128:], mo.round_to_dtype(v[codes[128:]] * s[1], "fp16"))
