@@ -8,7 +8,8 @@ laid out in Marlin order by the index recipe of `marlin_utils_test.py`
   * `marlin_gemm` must agree with `torch.matmul(a, w_ref)` under the
     reference's criterion mean|out - ref| / mean|ref| < 0.04 (test_marlin_gemm,
     test_marlin_gemm_with_bias), over the reference's grid of shapes, group
-    sizes, weight types, act-order and is_k_full for 16-bit activations.
+    sizes, weight types (integer and fp8), act-order and is_k_full for 16-bit
+    activations.
 No oracle here: the expected values come from torch on the GPU, as in the
 reference."""
 from __future__ import annotations
@@ -30,6 +31,7 @@ DENSE_CONFIGS = [
     {"b_type": scalar_types.uint4, "group_blocks": [-1, 2, 4, 8]},                                # AWQ int4
     {"b_type": scalar_types.uint4b8, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]},   # GPTQ int4
     {"b_type": scalar_types.uint8b128, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]}, # GPTQ int8
+    {"b_type": scalar_types.float8_e4m3fn, "group_blocks": [-1, 8]},                              # FP8
 ]
 
 
@@ -110,12 +112,16 @@ def _gemm_cases():
 def test_marlin_gemm(b_type, dtype, group_size, size_m, size_n, size_k, act_order, is_k_full):
     from sonar_amd import ops
     from sonar_amd.marlin_utils import marlin_make_workspace_new
+    from sonar_amd.marlin_utils_fp8 import marlin_quant_fp8_torch
     from sonar_amd.marlin_utils_test import awq_marlin_quantize, marlin_quantize
     a_input = rand_data((size_m, size_k), dtype=dtype)
     b_weight = rand_data((size_k, size_n), dtype=dtype)
     if b_type == scalar_types.uint4:
         w_ref, marlin_q_w, marlin_s, marlin_zp = awq_marlin_quantize(b_weight, b_type, group_size)
         g_idx = sort_indices = None
+    elif b_type == scalar_types.float8_e4m3fn:
+        w_ref, marlin_q_w, marlin_s = marlin_quant_fp8_torch(b_weight.T.contiguous(), group_size)
+        g_idx = sort_indices = marlin_zp = None
     else:
         w_ref, marlin_q_w, marlin_s, g_idx, sort_indices, _ = marlin_quantize(b_weight, b_type, group_size, act_order)
         marlin_zp = None
@@ -155,11 +161,12 @@ def test_marlin_gemm_with_bias(size_m):
 # ---------------------------------------------------------------------------
 # tests/kernels/moe/test_moe.py:129-143, 688-1010 of the reference: the fused
 # Marlin MoE layer against a plain torch mixture of experts on the dequantised
-# weights, atol 4e-2, over the reference's scenarios for integer weights.
+# weights, atol 4e-2, over the reference's scenarios for integer and fp8 weights.
 MOE_CONFIGS = [
     {"b_type": scalar_types.uint4, "group_blocks": [-1, 2, 4, 8]},
     {"b_type": scalar_types.uint4b8, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]},
     {"b_type": scalar_types.uint8b128, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]},
+    {"b_type": scalar_types.float8_e4m3fn, "group_blocks": [-1, 8]},
 ]
 MARLIN_MOE_SCENARIOS = [
     # (m, n, k, e, topk, ep_size, act_order, is_k_full)
@@ -197,6 +204,7 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None):
     """MarlinMoEWeightData.make (test_moe.py:774-892): every expert's (N, K)
     matrix quantised and laid out on its own, then stacked."""
     from sonar_amd.marlin_utils import marlin_permute_bias
+    from sonar_amd.marlin_utils_fp8 import marlin_quant_fp8_torch
     from sonar_amd.marlin_utils_test import awq_marlin_quantize, marlin_quantize
     k = w.shape[-1]
     out = {"w_ref": [], "qweight": [], "scales": [], "zeros": [], "g_idx": [], "sort_indices": [], "bias": []}
@@ -204,6 +212,8 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None):
         if quant_type == scalar_types.uint4:
             w_ref, qweight, scales, zeros = awq_marlin_quantize(w[i].transpose(1, 0), quant_type, group_size)
             out["zeros"].append(zeros)
+        elif quant_type == scalar_types.float8_e4m3fn:
+            w_ref, qweight, scales = marlin_quant_fp8_torch(w[i].contiguous(), group_size)
         else:
             w_ref, qweight, scales, g_idx, sort_indices, _ = marlin_quantize(
                 w[i].transpose(1, 0), quant_type, group_size, act_order, torch.randperm(k))
