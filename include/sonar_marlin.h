@@ -58,6 +58,13 @@ extern "C" {
  * fp8_fused_exponent_bias_into_scales makes them (quantization/utils/marlin_utils_fp8.py:35-46);
  * one scale per column or per group of 128 rows, no act-order (marlin/generate_kernels.py:87-93) */
 #define SONAR_TYPE_FLOAT8_E4M3FN 2814749767172868LL
+/* 4-bit floating-point codes (sign, 2 exponent bits, 1 mantissa bit) in the 4-bit weight order,
+ * with one power-of-two scale per column and group of 32 rows (MXFP4): bfloat16 activations only;
+ * b_scales hold the block scales 2^(e - 127) as bfloat16 in marlin_permute_scales order (the
+ * reference passes the exponent bytes e, reordered by mxfp4_marlin_process_scales,
+ * quantization/utils/marlin_utils_fp4.py:123-135; the torch op takes those and converts them);
+ * no zero points, no act-order (marlin/generate_kernels.py:102-110) */
+#define SONAR_TYPE_FLOAT4_E2M1F 562949953487106LL
 
 const char* sonar_marlin_last_error(void);
 const char* sonar_marlin_version(void);

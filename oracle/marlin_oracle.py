@@ -45,6 +45,14 @@ reference checkout).  How each function is pinned (none is "parity unpinned"):
                            in; dequant.h:320-380, marlin_utils_fp8.py:35-46)
                            against value * scale in exact rational arithmetic
                            rounded to nearest even, over all codes
+* MXFP4 weights            the 16 values against the list in the OCP MX
+                           format (0, 0.5, 1, 1.5, 2, 3, 4, 6 and negatives) and
+                           against the reference's own test recipe (the code
+                           moved into a float8_e4m3fn byte, converted by torch
+                           on the CPU, times 2^6; marlin_utils_fp4.py:720-727);
+                           scales 2^(e - 127) against torch's float8_e8m0fnu
+                           conversion; the (0, 2, 1, 3) reorder is its own
+                           inverse
 """
 
 from __future__ import annotations
@@ -78,6 +86,7 @@ UINT4_ID = scalar_type_id(0, 4, False, 0)        # scalar_types.uint4
 UINT8B128_ID = scalar_type_id(0, 8, False, 128)  # scalar_types.uint8b128
 NAN_REPR_EXTD_RANGE_MAX_MIN = 2                  # scalar_type.py:16
 FLOAT8_E4M3FN_ID = scalar_type_id(4, 3, True, 0, True, NAN_REPR_EXTD_RANGE_MAX_MIN)  # scalar_type.py:314
+FLOAT4_E2M1F_ID = scalar_type_id(2, 1, True, 0, True, 0)                              # scalar_type.py:327 (NanRepr.NONE)
 
 
 def scalar_type_min_max(mantissa: int, signed: bool, bias: int):
@@ -453,6 +462,40 @@ def dequantize_fp8(codes: np.ndarray, fused_scales32: np.ndarray, group_size: in
     k, n = codes.shape
     rows = np.zeros(k, dtype=np.int64) if group_size in (-1, k) else np.arange(k) // group_size
     return round_to_dtype(fp8_code_as_16bit_float(codes, dtype) * fused_scales32.astype(np.float32)[rows, :], dtype)
+
+
+# --------------------------------------------------------------------------
+# MXFP4 weights: float4_e2m1f codes in the 4-bit packings above, one
+# power-of-two scale per column and 32 rows, bf16 activations
+# (dequant.h:397-470; marlin_utils_fp4.py:123-135, 217-290, 701-753)
+# --------------------------------------------------------------------------
+
+def fp4_e2m1_values() -> np.ndarray:
+    """The value of each of the 16 codes: sign bit, 2 exponent bits with bias 1,
+    1 mantissa bit, subnormal at exponent 0; no infinities, no NaN."""
+    code = np.arange(16)
+    e, m = (code >> 1) & 3, code & 1
+    mag = np.where(e == 0, 0.5 * m, (1 + 0.5 * m) * 2.0 ** (e - 1))
+    return np.where(code & 8, -mag, mag).astype(np.float32)
+
+
+def mx_scale_values(exponent_bytes: np.ndarray) -> np.ndarray:
+    """float8_e8m0fnu: 2^(e - 127) for e = 0..254 (255 is NaN, not used here)."""
+    return np.ldexp(np.float32(1.0), exponent_bytes.astype(np.int32) - 127).astype(np.float32)
+
+
+def mxfp4_process_scales(permuted: np.ndarray) -> np.ndarray:
+    """marlin_utils_fp4.py:123-127: every four neighbours of the (already
+    permuted) scale rows in the order 0, 2, 1, 3."""
+    return permuted.reshape(-1, 4)[:, [0, 2, 1, 3]].reshape(permuted.shape)
+
+
+def dequantize_mxfp4(codes: np.ndarray, exponent_bytes: np.ndarray, dtype: str = "bf16") -> np.ndarray:
+    """w[k][n] = value(code[k][n]) * 2^(e[k // 32][n] - 127): a 2-bit significand
+    times a power of two, exact in bf16."""
+    k, n = codes.shape
+    rows = np.arange(k) // 32
+    return round_to_dtype(fp4_e2m1_values()[codes] * mx_scale_values(exponent_bytes)[rows, :], dtype)
 
 
 # --------------------------------------------------------------------------

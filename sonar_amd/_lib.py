@@ -17,6 +17,7 @@ TYPE_UINT4B8 = 1125899907892224
 TYPE_UINT4 = 1125899906843648
 TYPE_UINT8B128 = 1125899923621888
 TYPE_FLOAT8_E4M3FN = 2814749767172868
+TYPE_FLOAT4_E2M1F = 562949953487106
 
 OK = 0
 E_INVALID = -1

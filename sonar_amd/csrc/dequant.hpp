@@ -148,8 +148,8 @@ struct Dq<__bf16> {
 
 // Per-lane constants of the four columns (j = 0..3) a lane dequantises, for
 // the group `g` of strip `strip`.
-template <typename T, bool HAS_ZP>
-__device__ __forceinline__ void load_cols(typename Dq<T>::Col (&cols)[4], const uint16_t* scales,
+template <typename T, bool HAS_ZP, typename D = Dq<T>>
+__device__ __forceinline__ void load_cols(typename D::Col (&cols)[4], const uint16_t* scales,
                                           const uint32_t* zeros, int size_n, int strip, int g,
                                           int col16, bool grouped) {
   const uint16_t* srow = scales + (long)g * size_n + strip * kStripN;
@@ -160,9 +160,47 @@ __device__ __forceinline__ void load_cols(typename Dq<T>::Col (&cols)[4], const 
     const int nl = 16 * j + col16;
     int z = 8;
     if (HAS_ZP) z = (int)((zword >> zero_point_shift(nl)) & 0xFu);
-    cols[j] = Dq<T>::make_col(srow[scale_slot(nl, grouped)], z);
+    cols[j] = D::make_col(srow[scale_slot(nl, grouped)], z);
   }
 }
+
+// 4-bit floating-point codes (float4_e2m1f: sign, 2 exponent bits with bias 1,
+// 1 mantissa bit: 0, 0.5, 1, 1.5, 2, 3, 4, 6 and their negatives;
+// dequant.h:397-470 of the reference).  With its sign at bit 15 and the other
+// three bits at bits 11-9, a code is the fp16 number value * 2^-14 (the two
+// subnormal codes become fp16 subnormals).  The scales are powers of two held
+// in the activation type (the MX block scales, 2^(e - 127)); value * scale is
+// exact, so the one conversion rounds nothing.  Same interface and row order
+// as Dq: word() returns rows 0..7 of the column.
+template <typename T>
+struct DqF4 {
+  typedef typename Dq<T>::vec8 vec8;
+  struct Col {
+    float s;   // scale * 2^14
+  };
+  static __device__ __forceinline__ Col make_col(uint16_t scale_bits, int) {
+    return Col{Dq<T>::to_float(scale_bits) * 0x1p14f};
+  }
+  // codes in bits 12-15 and 28-31 of y -> two scaled values of T
+  static __device__ __forceinline__ uint32_t pair(uint32_t y, float s) {
+    const half2_t h = __builtin_bit_cast(half2_t, (y & 0x80008000u) | ((y & 0x70007000u) >> 3));
+    return (uint32_t)Dq<T>::from_float((float)h.x * s) | ((uint32_t)Dq<T>::from_float((float)h.y * s) << 16);
+  }
+  static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c, uint32_t) {
+    // rows 0,1 are nibbles 0,4; rows 2,3 nibbles 1,5; rows 4,5 nibbles 2,6; rows 6,7 nibbles 3,7
+    return __builtin_bit_cast(vec8, u32x4_t{pair(q << 12, c.s), pair(q << 8, c.s), pair(q << 4, c.s), pair(q, c.s)});
+  }
+};
+
+// The dequantiser of a 4-bit weight type.
+template <typename T, bool FP4>
+struct Dq4Of {
+  typedef Dq<T> type;
+};
+template <typename T>
+struct Dq4Of<T, true> {
+  typedef DqF4<T> type;
+};
 
 // 8-bit codes (uint8b128, symmetric): (v - 128) * s with one rounding.  A
 // packed word holds four rows of one column; word4 returns them as two

@@ -127,10 +127,11 @@ struct MoeUnit {
 // HAS_GIDX (with HAS_PERM, symmetric weights): an act-order shard that does not
 // hold whole groups (is_k_full = false); every row finds its scale through g_idx
 // (marlin_moe_wna16/ops.cu:343-351).
-template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX>
+template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX, bool FP4 = false>
 __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoeParams p) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq<T>::Col Col;
+  typedef typename Dq4Of<T, FP4>::type D4;   // integer codes, or float4_e2m1f
+  typedef typename D4::Col Col;
   __shared__ float4 red[4][MB * 4][64];
   __shared__ int slot_id[16 * MB];
 
@@ -212,7 +213,7 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
     for (int j = 0; j < 4; ++j) {
       int z = 8;
       if (HAS_ZP) z = (int)((cur.zword >> zero_point_shift(16 * j + col16)) & 0xFu);
-      cols[j] = Dq<T>::make_col((uint16_t)cur.sbits[j], z);
+      cols[j] = D4::make_col((uint16_t)cur.sbits[j], z);
     }
     int cur_group = cur.group;
     const int chunk0 = mine * p.unit_chunks;
@@ -222,7 +223,7 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
         const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
         if (g != cur_group) {  // groups smaller than a unit
           cur_group = g;
-          load_cols<T, HAS_ZP>(cols, scales, zeros, p.size_n, strip, g, col16, grouped);
+          load_cols<T, HAS_ZP, D4>(cols, scales, zeros, p.size_n, strip, g, col16, grouped);
         }
         const uint32_t words[4] = {cur.q[cc].x, cur.q[cc].y, cur.q[cc].z, cur.q[cc].w};
         int row_groups[8];
@@ -239,7 +240,7 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
             w = word_by_row_groups<T>(words[j], row_groups,
                                       scales + strip * kStripN + scale_slot(16 * j + col16, true), p.size_n, magic);
           else
-            w = Dq<T>::word(words[j], cols[j], magic);
+            w = D4::word(words[j], cols[j], magic);
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb) acc[mb][j] = Dq<T>::mfma(w, cur.a[cc][mb], acc[mb][j]);
         }
@@ -457,6 +458,17 @@ void launch_moe8_mb(const MoeParams& p, bool fp8, int grid, hipStream_t st) {
   }
 }
 
+// float4_e2m1f codes: no zero points, no act-order
+template <typename T>
+void launch_moe_fp4(const MoeParams& p, int grid, hipStream_t st) {
+  switch ((p.block_size + 15) / 16) {
+    case 1: marlin_moe_kernel<T, 1, false, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
+    case 2: marlin_moe_kernel<T, 2, false, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
+    case 3: marlin_moe_kernel<T, 3, false, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
+    default: marlin_moe_kernel<T, 4, false, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
+  }
+}
+
 template <typename T, bool HAS_ZP>
 void launch_moe_mb(const MoeParams& p, bool has_perm, int grid, hipStream_t st) {
   switch ((p.block_size + 15) / 16) {
@@ -510,21 +522,31 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
   SONAR_REQUIRE(b_scales != nullptr, "b_scales must not be NULL");
   SONAR_REQUIRE(num_groups >= 1, "num_groups = %ld must be >= 1", (long)num_groups);
   if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4 && b_type_id != SONAR_TYPE_UINT8B128 &&
-      b_type_id != SONAR_TYPE_FLOAT8_E4M3FN)
+      b_type_id != SONAR_TYPE_FLOAT8_E4M3FN && b_type_id != SONAR_TYPE_FLOAT4_E2M1F)
     return fail(SONAR_E_UNSUPPORTED,
-                "b_type id %ld is not built here: only uint4b8, uint8b128 (GPTQ), uint4 (AWQ) and "
-                "float8_e4m3fn weights are",
+                "b_type id %ld is not built here: only uint4b8, uint8b128 (GPTQ), uint4 (AWQ), "
+                "float8_e4m3fn and float4_e2m1f (MXFP4) weights are",
                 (long)b_type_id);
   const bool has_zp = b_zeros != nullptr;
   const bool fp8 = b_type_id == SONAR_TYPE_FLOAT8_E4M3FN;
+  const bool fp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F;
   const bool bits8 = b_type_id == SONAR_TYPE_UINT8B128 || fp8;
   if (has_zp)
     SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4, "b_type must be u4 or u8 when has_zp = True");
   else
-    SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4B8 || bits8,
+    SONAR_REQUIRE(b_type_id == SONAR_TYPE_UINT4B8 || bits8 || fp4,
                   "b_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   bool has_perm = perm != nullptr;
+  if (fp4) {
+    // moe/marlin_moe_wna16/generate_kernels.py:102-110: MXFP4, bfloat16 activations, a scale per 32 rows
+    SONAR_REQUIRE(!has_perm, "act-order is not supported with float4_e2m1f weights");
+    SONAR_REQUIRE(dtype == SONAR_DTYPE_BF16, "float4_e2m1f weights with power-of-two block scales (MXFP4) "
+                  "need bfloat16 activations");
+    SONAR_REQUIRE(size_k == 32 * num_groups,
+                  "float4_e2m1f weights (MXFP4) take one scale per group of 32 rows; got size_k = %ld, "
+                  "num_groups = %ld", (long)size_k, (long)num_groups);
+  }
   if (fp8) {
     // moe/marlin_moe_wna16/generate_kernels.py: channelwise scales or groups of 128 rows, no act-order
     SONAR_REQUIRE(!has_perm, "act-order is not supported with float8_e4m3fn weights");
@@ -593,7 +615,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                 "act-order with 8-bit expert weights needs sorted_len * size_k * 2 more scratch bytes "
                 "(the column-permuted copy of A per slot)");
   // Few rows per expert: the decode kernel, one workgroup per strip and 32 slots of a block
-  if (!bits8 && !row_groups &&
+  if (!bits8 && !fp4 && !row_groups &&
       moe_fast_applies(has_perm, moe_block_size, sorted_len, num_experts, a_rows, size_n, size_k, num_groups,
                        group_size))
     return moe_fast_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
@@ -601,7 +623,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                          num_experts, dtype, size_m, size_n, size_k, num_groups, group_size, a_by_slot, st);
   static const bool no_tile = getenv("SONAR_MARLIN_NO_MOE_TILE") != nullptr;  // debugging aid
   // Full blocks of 64 slots mean many rows per expert: the MFMA-tiled kernel
-  if (moe_block_size == 64 && !has_perm && !bits8 && !row_groups && !no_tile && size_k % 64 == 0 &&
+  if (moe_block_size == 64 && !has_perm && !bits8 && !fp4 && !row_groups && !no_tile && size_k % 64 == 0 &&
       num_experts <= 1024 &&
       (num_groups == 1 || group_size % 64 == 0 || group_size == 32) && scratch != nullptr &&
       scratch_bytes >= moe_tile_table_bytes(sorted_len, num_experts) && ((uintptr_t)scratch) % 4 == 0)
@@ -649,6 +671,10 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     if (dtype == SONAR_DTYPE_F16) launch_moe8_mb<_Float16>(p, fp8, (int)grid, st);
     else launch_moe8_mb<__bf16>(p, fp8, (int)grid, st);
     return launch_status("marlin_moe8_kernel");
+  }
+  if (fp4) {
+    launch_moe_fp4<__bf16>(p, (int)grid, st);
+    return launch_status("marlin_moe_kernel");
   }
   if (dtype == SONAR_DTYPE_F16) {
     if (has_zp) launch_moe_mb<_Float16, true>(p, has_perm, (int)grid, st);

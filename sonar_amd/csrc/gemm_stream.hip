@@ -277,10 +277,11 @@ __device__ __forceinline__ void load_unit(UnitBuf<T, MB>& b, const StreamParams&
   if (HAS_ZP) b.zword = p.zeros[(long)g * (p.size_n / 8) + strip * 8 + zero_point_word(col16)];
 }
 
-template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX>
+template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX, bool FP4 = false>
 __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const StreamParams params) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq<T>::Col Col;
+  typedef typename Dq4Of<T, FP4>::type D4;   // integer codes, or float4_e2m1f
+  typedef typename D4::Col Col;
   __shared__ float4 red[4][MB * 4][64];
   // Several 64-row slabs can share a launch when no strip is shared between
   // workgroups (nothing goes through the scratch slots).
@@ -327,7 +328,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
       for (int j = 0; j < 4; ++j) {
         int z = 8;
         if (HAS_ZP) z = (int)((cur.zword >> zero_point_shift(16 * j + col16)) & 0xFu);
-        cols[j] = Dq<T>::make_col((uint16_t)cur.sbits[j], z);
+        cols[j] = D4::make_col((uint16_t)cur.sbits[j], z);
       }
       int cur_group = cur.group;
       const int chunk0 = (mine - strip_first) * p.unit_chunks;
@@ -337,7 +338,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
           const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
           if (g != cur_group) {  // groups smaller than a unit
             cur_group = g;
-            load_cols<T, HAS_ZP>(cols, p.scales, p.zeros, p.size_n, strip, g, col16, grouped);
+            load_cols<T, HAS_ZP, D4>(cols, p.scales, p.zeros, p.size_n, strip, g, col16, grouped);
           }
           const uint32_t words[4] = {cur.q[cc].x, cur.q[cc].y, cur.q[cc].z, cur.q[cc].w};
           int row_groups[8];
@@ -355,7 +356,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
                                         p.scales + strip * kStripN + scale_slot(16 * j + col16, true), p.size_n,
                                         magic);
             else
-              w = Dq<T>::word(words[j], cols[j], magic);
+              w = D4::word(words[j], cols[j], magic);
 #pragma unroll
             for (int mb = 0; mb < MB; ++mb) acc[mb][j] = Dq<T>::mfma(w, cur.a[cc][mb], acc[mb][j]);
           }
@@ -1055,7 +1056,7 @@ __global__ __launch_bounds__(64) void marlin_fixup_kernel(const StreamParams p) 
 
 // Writes W[K][N]: the values the GEMM kernels feed to the matrix cores.
 // With g_idx (symmetric weights only) the group of every row is looked up there.
-template <typename T, bool HAS_ZP>
+template <typename T, bool HAS_ZP, bool FP4 = false>
 __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __restrict__ b,
                                                             const uint16_t* __restrict__ scales,
                                                             const uint32_t* __restrict__ zeros,
@@ -1074,8 +1075,9 @@ __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __rest
     const int strip = (int)(ch / chunks_per_strip);
     const int chunk = (int)(ch % chunks_per_strip);
     const int g = grouped && !g_idx ? (chunk * kChunkK) / group_size : 0;
-    typename Dq<T>::Col cols[4];
-    load_cols<T, HAS_ZP>(cols, scales, zeros, size_n, strip, g, col16, grouped);
+    typedef typename Dq4Of<T, FP4>::type D4;
+    typename D4::Col cols[4];
+    load_cols<T, HAS_ZP, D4>(cols, scales, zeros, size_n, strip, g, col16, grouped);
     int row_groups[8] = {0, 0, 0, 0, 0, 0, 0, 0};
     if (g_idx) {
 #pragma unroll
@@ -1090,7 +1092,7 @@ __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __rest
         w = word_by_row_groups<T>(words[j], row_groups, scales + strip * kStripN + scale_slot(16 * j + col16, true),
                                   size_n, magic);
       else
-        w = Dq<T>::word(words[j], cols[j], magic);
+        w = D4::word(words[j], cols[j], magic);
       const uint16_t* bits = reinterpret_cast<const uint16_t*>(&w);
 #pragma unroll
       for (int t = 0; t < 8; ++t) {
@@ -1204,6 +1206,17 @@ void launch_stream_mb(const StreamParams& p, bool has_perm, hipStream_t st) {
   }
 }
 
+// float4_e2m1f codes: no zero points, no act-order
+template <typename T>
+void launch_stream_fp4(const StreamParams& p, hipStream_t st) {
+  switch ((p.size_m + 15) / 16) {
+    case 1: marlin_stream_kernel<T, 1, false, false, false, true><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 2: marlin_stream_kernel<T, 2, false, false, false, true><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 3: marlin_stream_kernel<T, 3, false, false, false, true><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    default: marlin_stream_kernel<T, 4, false, false, false, true><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+  }
+}
+
 template <typename T, bool HAS_GIDX, bool FP8>
 void launch_stream8_gidx(const StreamParams& p, hipStream_t st) {
   switch ((p.size_m + 15) / 16) {
@@ -1279,6 +1292,7 @@ struct Checked {
   int group_size;
   int bits;         // 4 or 8
   bool fp8;         // 8-bit floating-point codes (float8_e4m3fn)
+  bool fp4;         // 4-bit floating-point codes (float4_e2m1f) with power-of-two scales per 32 rows
 };
 
 int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_t* b_zeros,
@@ -1293,12 +1307,13 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
   SONAR_REQUIRE(b_scales != nullptr, "b_scales must not be NULL");
   SONAR_REQUIRE(num_groups >= 1, "num_groups = %ld must be >= 1", (long)num_groups);
   if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4 && b_type_id != SONAR_TYPE_UINT8B128 &&
-      b_type_id != SONAR_TYPE_FLOAT8_E4M3FN)
+      b_type_id != SONAR_TYPE_FLOAT8_E4M3FN && b_type_id != SONAR_TYPE_FLOAT4_E2M1F)
     return fail(SONAR_E_UNSUPPORTED,
-                "b_type id %ld is not built here: only uint4b8, uint8b128 (GPTQ), uint4 (AWQ) and "
-                "float8_e4m3fn weights are",
+                "b_type id %ld is not built here: only uint4b8, uint8b128 (GPTQ), uint4 (AWQ), "
+                "float8_e4m3fn and float4_e2m1f (MXFP4) weights are",
                 (long)b_type_id);
   out.fp8 = b_type_id == SONAR_TYPE_FLOAT8_E4M3FN;
+  out.fp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F;
   out.bits = (b_type_id == SONAR_TYPE_UINT8B128 || out.fp8) ? 8 : 4;
   out.has_zp = b_zeros != nullptr;
   if (out.has_zp)
@@ -1308,6 +1323,15 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
                   "b_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   out.has_perm = perm != nullptr;
+  if (out.fp4) {
+    // generate_kernels.py:102-110: MXFP4, bfloat16 activations, one power-of-two scale per 32 rows
+    SONAR_REQUIRE(!out.has_perm, "act-order is not supported with float4_e2m1f weights");
+    SONAR_REQUIRE(dtype == SONAR_DTYPE_BF16, "float4_e2m1f weights with power-of-two block scales (MXFP4) "
+                  "need bfloat16 activations");
+    SONAR_REQUIRE(size_k == 32 * num_groups,
+                  "float4_e2m1f weights (MXFP4) take one scale per group of 32 rows; got size_k = %ld, "
+                  "num_groups = %ld", (long)size_k, (long)num_groups);
+  }
   if (out.fp8) {
     // generate_kernels.py:87-93: channelwise scales or groups of 128 rows, no act-order
     SONAR_REQUIRE(!out.has_perm, "act-order is not supported with float8_e4m3fn weights");
@@ -1525,7 +1549,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   int unit_group_shift;
   const bool fast_groups = fast_group_shift(num_groups, chk.group_size, unit_group_shift);
   static const bool no_fast = getenv("SONAR_MARLIN_NO_FAST") != nullptr;  // debugging aid
-  const bool fast_shape = !no_fast && chk.bits == 4 && !chk.has_perm && !chk.row_groups &&
+  const bool fast_shape = !no_fast && chk.bits == 4 && !chk.fp4 && !chk.has_perm && !chk.row_groups &&
                           p.chunks_per_strip % 4 == 0 && fast_groups &&
                           size_m * a_row_stride * 2 < (1LL << 31);
   // Short strips (K <= 4096) on a matrix with at least 64 of them: one workgroup
@@ -1566,7 +1590,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   const bool async_tile = tile_async_applies(chk.has_perm, num_groups, chk.group_size);
   const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
   // the row -> group lookup and 8-bit codes exist in the streaming kernels only
-  const bool use_tile = plan.tile && !no_tile && !chk.row_groups && chk.bits == 4 && !(slab_fast && p.unit_chunks == 4);
+  const bool use_tile = plan.tile && !no_tile && !chk.row_groups && chk.bits == 4 && !chk.fp4 &&
+                        !(slab_fast && p.unit_chunks == 4);
   // More than 64 rows in the general kernels (8-bit codes, is_k_full = false,
   // the tile path switched off) on a matrix of short strips: one workgroup per
   // strip as well, so that every 64-row slab can run in the same launch and the
@@ -1633,6 +1658,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
       if (chk.bits == 8) {
         if (dtype == SONAR_DTYPE_F16) launch_stream8_mb<_Float16>(p, chk.fp8, st);
         else launch_stream8_mb<__bf16>(p, chk.fp8, st);
+      } else if (chk.fp4) {
+        launch_stream_fp4<__bf16>(p, st);
       } else if (dtype == SONAR_DTYPE_F16) {
         if (chk.has_zp) launch_stream_mb<_Float16, true>(p, chk.has_perm, st);
         else launch_stream_mb<_Float16, false>(p, chk.has_perm, st);
@@ -1684,7 +1711,9 @@ extern "C" int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout, co
     return launch_status("marlin_dequant8_kernel");
   }
   const int32_t* gi = chk.row_groups ? g_idx : nullptr;
-  if (dtype == SONAR_DTYPE_F16) {
+  if (chk.fp4) {
+    marlin_dequant_kernel<__bf16, false, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);
+  } else if (dtype == SONAR_DTYPE_F16) {
     if (chk.has_zp) marlin_dequant_kernel<_Float16, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);
     else marlin_dequant_kernel<_Float16, false><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);
   } else {

@@ -97,6 +97,37 @@ Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, 
   return native;
 }
 
+// MXFP4 block scales as the reference's callers pass them (float8_e8m0fnu exponent
+// bytes in marlin_permute_scales order with every four neighbours in the order
+// 0, 2, 1, 3; marlin_utils_fp4.py:123-135) -> bfloat16 powers of two in plain
+// marlin_permute_scales order, which the kernels read.  Cached like the weights.
+Tensor mx_scales_as_bf16(const Tensor& b_scales) {
+  const void* key = b_scales.const_data_ptr();
+  {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    auto it = g_cache.find(key);
+    if (it != g_cache.end() && !it->second.source.expired() &&
+        it->second.source._unsafe_get_target() == b_scales.unsafeGetTensorImpl() && it->second.size_k == -1 &&
+        it->second.version == version_of(b_scales))
+      return it->second.native;
+  }
+  TORCH_CHECK(b_scales.numel() % 4 == 0, "b_scales.numel() must be a multiple of 4");
+  const Tensor bytes = b_scales.view(at::kByte);
+  const Tensor order = at::tensor({0, 2, 1, 3}, at::TensorOptions().dtype(at::kLong).device(b_scales.device()));
+  const Tensor e = bytes.reshape({-1, 4}).index_select(1, order).reshape(bytes.sizes()).to(at::kShort);
+  // bfloat16 2^(e - 127): exponent field e; e = 0 is the subnormal 2^-127
+  const Tensor bits = at::where(e == 0, at::full_like(e, 0x40), e * 128);
+  Tensor out = bits.view(at::kBFloat16);
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  g_cache.insert_or_assign(key, NativeEntry{c10::weak_intrusive_ptr<c10::TensorImpl>(b_scales.getIntrusivePtr()),
+                                            out, -1, -1, -1, version_of(b_scales)});
+  return out;
+}
+
+bool is_mx_scale_type(const Tensor& t) {
+  return t.scalar_type() == at::kFloat8_e8m0fnu || t.scalar_type() == at::kByte;
+}
+
 int64_t marlin_weight_cache_clear() {
   std::lock_guard<std::mutex> lock(g_cache_mutex);
   const int64_t n = (int64_t)g_cache.size();
@@ -181,9 +212,10 @@ Tensor marlin_to_gfx950(const Tensor& b_q_weight, int64_t size_k, int64_t size_n
 void check_b_type(int64_t b_type_id) {
   TORCH_CHECK_NOT_IMPLEMENTED(
       b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4 || b_type_id == SONAR_TYPE_UINT8B128 ||
-          b_type_id == SONAR_TYPE_FLOAT8_E4M3FN,
+          b_type_id == SONAR_TYPE_FLOAT8_E4M3FN || b_type_id == SONAR_TYPE_FLOAT4_E2M1F,
       "b_type_id = ", b_type_id,
-      " is not built here: only uint4b8, uint8b128 (GPTQ), uint4 (AWQ) and float8_e4m3fn weights are supported");
+      " is not built here: only uint4b8, uint8b128 (GPTQ), uint4 (AWQ), float8_e4m3fn and float4_e2m1f (MXFP4) "
+      "weights are supported");
 }
 
 Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_q_weight,
@@ -221,8 +253,17 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
   TORCH_CHECK(b_q_weight.scalar_type() == at::kInt, "b_q_weight type is not kInt");
   TORCH_CHECK(b_scales.is_cuda(), "b_scales is not on GPU");
   TORCH_CHECK(b_scales.is_contiguous(), "b_scales is not contiguous");
-  TORCH_CHECK(b_scales.scalar_type() == a.scalar_type(),
-              "scalar type of b_scales must be the same as a for 16 bit activation");
+  const bool fp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F;
+  if (fp4) {   // marlin.cu:600-611; the fp8 block scales of NVFP4 are not built
+    TORCH_CHECK_NOT_IMPLEMENTED(b_scales.scalar_type() != at::kFloat8_e4m3fn,
+                                "float4_e2m1f weights with float8_e4m3fn scales (NVFP4) are not built");
+    TORCH_CHECK(is_mx_scale_type(b_scales),
+                "When b_type = float4_e2m1f, b_scale scalar type must be",
+                "float8_e4m3fn (for NVFP4) or float8_e8m0fnu (for MXFP4).");
+  } else {
+    TORCH_CHECK(b_scales.scalar_type() == a.scalar_type(),
+                "scalar type of b_scales must be the same as a for 16 bit activation");
+  }
 
   c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
   Tensor c;
@@ -300,7 +341,7 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
   raise_if_failed(sonar_marlin_gemm(
       a.const_data_ptr(), a.stride(0), c.mutable_data_ptr(),
       static_cast<const uint32_t*>(native.const_data_ptr()), SONAR_LAYOUT_GFX950,
-      opt_ptr(b_bias_or_none), b_scales.const_data_ptr(),
+      opt_ptr(b_bias_or_none), (fp4 ? mx_scales_as_bf16(b_scales) : b_scales).const_data_ptr(),
       has_zp ? static_cast<const uint32_t*>(b_zeros_or_none->const_data_ptr()) : nullptr, g_idx, perm,
       static_cast<int32_t*>(workspace.mutable_data_ptr()), workspace.numel(), scratch.mutable_data_ptr(),
       scratch_bytes, dtype, b_type_id, size_m, size_n, size_k, num_groups, is_k_full ? 1 : 0,
@@ -347,7 +388,16 @@ Tensor moe_wna16_marlin_gemm(
   TORCH_CHECK(b_scales.is_cuda() && b_scales.is_contiguous(), "b_scales is not a contiguous GPU tensor");
   TORCH_CHECK(b_scales.dim() == 3 && b_scales.size(0) == experts, "b_scales rank = ", b_scales.dim(), " is not 3");
   TORCH_CHECK(b_scales.size(2) == size_n, "b_scales dim 2 = ", b_scales.size(2), " is not size_n = ", size_n);
-  TORCH_CHECK(b_scales.scalar_type() == a.scalar_type(), "b_scales must have the dtype of a");
+  const bool fp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F;
+  if (fp4) {
+    TORCH_CHECK_NOT_IMPLEMENTED(b_scales.scalar_type() != at::kFloat8_e4m3fn,
+                                "float4_e2m1f weights with float8_e4m3fn scales (NVFP4) are not built");
+    TORCH_CHECK(is_mx_scale_type(b_scales),
+                "When b_type = float4_e2m1f, b_scale scalar type must be",
+                "float8_e4m3fn (for NVFP4) or float8_e8m0fnu (for MXFP4).");
+  } else {
+    TORCH_CHECK(b_scales.scalar_type() == a.scalar_type(), "b_scales must have the dtype of a");
+  }
   const int64_t num_groups = b_scales.size(1);
 
   c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
@@ -417,7 +467,7 @@ Tensor moe_wna16_marlin_gemm(
 
   raise_if_failed(sonar_moe_wna16_marlin_gemm(
       a.const_data_ptr(), c.mutable_data_ptr(), static_cast<const uint32_t*>(native.const_data_ptr()),
-      SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none), b_scales.const_data_ptr(),
+      SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none), (fp4 ? mx_scales_as_bf16(b_scales) : b_scales).const_data_ptr(),
       has_zp ? static_cast<const uint32_t*>(b_zeros_or_none->const_data_ptr()) : nullptr, g_idx, perm,
       static_cast<int32_t*>(workspace.mutable_data_ptr()), workspace.numel(),
       scratch_bytes > 0 ? scratch.mutable_data_ptr() : nullptr, scratch_bytes,

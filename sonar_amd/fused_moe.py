@@ -21,7 +21,7 @@ from .marlin_utils import marlin_make_workspace_new
 from .scalar_type import ScalarType, scalar_types
 
 _SUPPORTED = {t.id: t for t in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128,
-                                scalar_types.float8_e4m3fn)}
+                                scalar_types.float8_e4m3fn, scalar_types.float4_e2m1f)}
 
 
 def moe_block_size(num_tokens: int, top_k: int, num_experts: int) -> int:
@@ -223,8 +223,8 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
     w2: (E, N/16, 2K); scales (E, groups, 2N) / (E, groups, K); topk_weights
     fp32 [M, top_k]; topk_ids [M, top_k].  Returns [M, K]."""
     if quant_type_id not in _SUPPORTED:
-        raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8, uint8b128 and "
-                                  "float8_e4m3fn expert weights are built")
+        raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8, uint8b128, "
+                                  "float8_e4m3fn and float4_e2m1f (MXFP4) expert weights are built")
     if input_dtype is not None:
         raise NotImplementedError("8-bit activations are not built")
     quant_type = _SUPPORTED[quant_type_id]
@@ -281,8 +281,8 @@ def batched_fused_marlin_moe(hidden_states: torch.Tensor, expert_num_tokens: tor
     routing weights are ones.  Returns [E, max_tokens, K]; rows of invalid tokens
     are not written."""
     if quant_type_id not in _SUPPORTED:
-        raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8, uint8b128 and "
-                                  "float8_e4m3fn expert weights are built")
+        raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8, uint8b128, "
+                                  "float8_e4m3fn and float4_e2m1f (MXFP4) expert weights are built")
     assert hidden_states.ndim == 3, f"hidden states must be batched. e.g. [B, MAX_TOKENS, K].But got {hidden_states.size()}"
     B, max_tokens, K = hidden_states.shape
     E = w1.shape[0]

@@ -30,11 +30,11 @@ def round_up(x: int, m: int) -> int:
 
 def query_marlin_supported_quant_types(has_zp: bool | None = None, include_fp_type: bool = True):
     """uint4 with zero points; uint4b8, uint8b128 and (with include_fp_type)
-    float8_e4m3fn without (marlin_utils.py:64-108 of the reference lists more:
-    uint8 with zero points and float4_e2m1f are not built here)."""
+    float8_e4m3fn and float4_e2m1f without (marlin_utils.py:64-82 of the
+    reference; of the float4_e2m1f formats MXFP4 is built, NVFP4 is not)."""
     without = [scalar_types.uint4b8, scalar_types.uint8b128]
     if include_fp_type:
-        without.append(scalar_types.float8_e4m3fn)
+        without += [scalar_types.float8_e4m3fn, scalar_types.float4_e2m1f]
     if has_zp is None:
         return without + [scalar_types.uint4]
     return [scalar_types.uint4] if has_zp else without

@@ -1,0 +1,145 @@
+"""MXFP4 weights (float4_e2m1f codes, one power-of-two scale per 32 rows, bf16
+activations) through the Marlin ops.  Mirrors the MXFP4 half of
+aphrodite/model_executor/layers/quantization/utils/marlin_utils_fp4.py:34-36,
+123-135, 153-290, 293-322, 556-649, 701-753 of the reference: the checkpoint
+bytes (two codes each, low nibble first along K) are GPTQ words as they stand
+and go through gptq_marlin_repack with num_bits = 4; the scales (exponent bytes
+e, value 2^(e - 127)) are permuted as for any Marlin layer, every four
+neighbours are put in the order 0, 2, 1, 3, and they travel as float8_e8m0fnu.
+NVFP4 (float8_e4m3fn scales per 16 rows and a global scale) is not built.
+"""
+from __future__ import annotations
+
+import torch
+
+from . import ops
+from .marlin_utils import (USE_FP32_REDUCE_DEFAULT, marlin_make_workspace_new, marlin_pad_dim, marlin_pad_qweight,
+                           marlin_pad_scales, marlin_padded_nk, marlin_permute_bias, marlin_permute_scales,
+                           marlin_repacked_nk, marlin_unpad_output, should_use_atomic_add_reduce)
+from .scalar_type import scalar_types
+
+MXFP4_GROUP_SIZE = 32
+
+
+def is_fp4_marlin_supported() -> bool:
+    """marlin_utils_fp4.py:34-35; one target here, which runs MXFP4."""
+    return True
+
+
+def mxfp4_marlin_process_scales(marlin_scales: torch.Tensor, input_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """marlin_utils_fp4.py:123-135 for 16-bit activations: (0, 2, 1, 3) inside
+    every four, then the exponent bytes."""
+    if input_dtype is not None and input_dtype.itemsize == 1:
+        raise NotImplementedError("8-bit activations are not built")
+    reordered = marlin_scales.view(-1, 4)[:, [0, 2, 1, 3]].view(marlin_scales.size(0), -1)
+    return reordered.to(torch.float8_e8m0fnu)
+
+
+def apply_fp4_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+                            weight_global_scale: torch.Tensor | None, workspace: torch.Tensor, size_n: int,
+                            size_k: int, bias: torch.Tensor | None = None, input_dtype: torch.dtype | None = None,
+                            use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
+    """marlin_utils_fp4.py:153-214."""
+    if weight_global_scale is not None:
+        raise NotImplementedError("NVFP4 (a global scale) is not built; MXFP4 only")
+    if input_dtype is not None and input_dtype.itemsize == 1:
+        raise NotImplementedError("8-bit activations are not built")
+    x = input.reshape(-1, input.shape[-1])
+    out_shape = input.shape[:-1] + (size_n,)
+    padded_n, padded_k = marlin_repacked_nk(weight, num_bits=4)
+    x = marlin_pad_dim(x, size_k, padded_k)
+    use_atomic_add = should_use_atomic_add_reduce(m=x.size(0), n=padded_n, k=padded_k, device=input.device,
+                                                  dtype=input.dtype)
+    out = ops.marlin_gemm(a=x, c=None, b_q_weight=weight, b_bias=bias, b_scales=weight_scale, a_scales=None,
+                          global_scale=None, b_zeros=None, g_idx=None, perm=None, workspace=workspace,
+                          b_q_type=scalar_types.float4_e2m1f, size_m=x.size(0), size_n=padded_n, size_k=padded_k,
+                          use_atomic_add=use_atomic_add, use_fp32_reduce=use_fp32_reduce)
+    return marlin_unpad_output(out, size_n, padded_n).reshape(out_shape)
+
+
+def _set(layer, name: str, value: torch.Tensor) -> None:
+    setattr(layer, name, torch.nn.Parameter(value, requires_grad=False)
+            if isinstance(layer, torch.nn.Module) else value)
+
+
+def prepare_fp4_layer_for_marlin(layer, input_dtype: torch.dtype | None = None) -> None:
+    """marlin_utils_fp4.py:217-290 for MXFP4.  The layer holds `weight` (N, K/2)
+    uint8, `weight_scale` (N, K/32) exponent bytes, `params_dtype` (bfloat16),
+    `output_size_per_partition`, `input_size_per_partition`, optionally `bias`."""
+    if hasattr(layer, "weight_global_scale"):
+        raise NotImplementedError("NVFP4 (a global scale) is not built; MXFP4 only")
+    if input_dtype is not None and input_dtype.itemsize == 1:
+        raise NotImplementedError("8-bit activations are not built")
+    part_n, part_k = layer.output_size_per_partition, layer.input_size_per_partition
+    padded_n, padded_k = marlin_padded_nk(part_n, part_k, MXFP4_GROUP_SIZE)
+    assert layer.weight.shape == (part_n, part_k // 2)
+    device = layer.weight.device
+    layer.workspace = marlin_make_workspace_new(device)
+    perm = torch.empty(0, dtype=torch.int, device=device)
+    qweight = marlin_pad_qweight(layer.weight.view(torch.int32).T.contiguous(), part_n, part_k, padded_n, padded_k)
+    _set(layer, "weight", ops.gptq_marlin_repack(qweight, perm, padded_k, padded_n, 4))
+
+    scales = layer.weight_scale.T.contiguous().view(torch.float8_e8m0fnu).to(layer.params_dtype)
+    scales = marlin_pad_scales(scales, part_n, part_k, padded_n, padded_k, MXFP4_GROUP_SIZE)
+    scales = marlin_permute_scales(scales, padded_k, padded_n, MXFP4_GROUP_SIZE)
+    _set(layer, "weight_scale", mxfp4_marlin_process_scales(scales))
+
+    if getattr(layer, "bias", None) is not None:
+        assert layer.bias.shape == (part_n,)
+        _set(layer, "bias", marlin_permute_bias(marlin_pad_dim(layer.bias, part_n, padded_n)))
+
+
+def prepare_moe_mxfp4_layer_for_marlin(layer, w13: torch.Tensor, w2: torch.Tensor, w13_scale: torch.Tensor,
+                                       w2_scale: torch.Tensor, w13_bias: torch.Tensor | None,
+                                       w2_bias: torch.Tensor | None):
+    """marlin_utils_fp4.py:556-649.  w13 (E, 2N, K/2), w2 (E, K, N/2) uint8; scales
+    (E, 2N, K/32), (E, K, N/32) exponent bytes; `layer.params_dtype` is the
+    activation type.  Returns (w13, w2, w13_scale, w2_scale, w13_bias, w2_bias)
+    for fused_marlin_moe; nothing on the layer changes."""
+    e, n, k = w13.shape[0], w13.shape[1] // 2, w13.shape[2] * 2
+    perm = torch.empty(0, dtype=torch.int, device=w13.device)
+
+    def repack(weight: torch.Tensor, size_n: int, size_k: int) -> torch.Tensor:
+        assert weight.shape == (e, size_n, size_k // 2)
+        return torch.stack([ops.gptq_marlin_repack(weight[i].view(torch.int32).T.contiguous(), perm, size_k, size_n, 4)
+                            for i in range(e)])
+
+    def permute(scales: torch.Tensor, size_n: int, size_k: int) -> torch.Tensor:
+        scales = scales.view(torch.float8_e8m0fnu).to(layer.params_dtype)
+        return torch.stack([mxfp4_marlin_process_scales(
+            marlin_permute_scales(scales[i].T, size_k, size_n, MXFP4_GROUP_SIZE)) for i in range(e)])
+
+    def permute_bias(bias: torch.Tensor | None) -> torch.Tensor | None:
+        if bias is None:
+            return None
+        bias = bias.to(layer.params_dtype)
+        return torch.stack([marlin_permute_bias(bias[i]) for i in range(e)])
+
+    return (repack(w13, 2 * n, k), repack(w2, k, n), permute(w13_scale, 2 * n, k), permute(w2_scale, k, n),
+            permute_bias(w13_bias), permute_bias(w2_bias))
+
+
+def rand_marlin_weight_mxfp4_like(weight: torch.Tensor, group_size: int, input_dtype: torch.dtype | None = None):
+    """The reference's test helper (marlin_utils_fp4.py:701-753): random codes of
+    the shape of `weight` (N, K) and random exponents 110..119; returns
+    (dequantised reference (K, N), Marlin weight, Marlin scales)."""
+    assert input_dtype is None or input_dtype.itemsize != 1, "8-bit activations are not built"
+    assert group_size > 0
+    size_n, size_k = weight.shape
+    device = weight.device
+    scales = torch.randint(110, 120, (size_n, size_k // group_size), dtype=torch.uint8, device=device)
+    scales = scales.view(torch.float8_e8m0fnu)
+    codes = torch.randint(0, 256, (size_n, size_k // 2), dtype=torch.uint8, device=device)
+
+    def values(nibble_high: torch.Tensor) -> torch.Tensor:
+        # sign and the three other bits at the top of a byte: as float8_e4m3fn that is value * 2^-6
+        as_fp8 = (nibble_high & 0b10000000) | ((nibble_high & 0b01110000) >> 2)
+        return as_fp8.view(torch.float8_e4m3fn).to(weight.dtype) * (2 ** 6)
+
+    odd, even = values(codes), values(codes << 4)   # k odd: high nibble; k even: low nibble
+    weight_ref = torch.cat([even.unsqueeze(2), odd.unsqueeze(2)], 2).view(size_n, size_k)
+    weight_ref = weight_ref * scales.repeat_interleave(group_size, 1).to(weight.dtype)
+    perm = torch.empty(0, dtype=torch.int, device=device)
+    marlin_qweight = ops.gptq_marlin_repack(codes.view(torch.int32).T.contiguous(), perm, size_k, size_n, 4)
+    marlin_scales = marlin_permute_scales(scales.T.to(weight.dtype), size_k, size_n, group_size)
+    return weight_ref.T, marlin_qweight, mxfp4_marlin_process_scales(marlin_scales)

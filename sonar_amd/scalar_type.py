@@ -1,7 +1,8 @@
 """Sub-byte scalar type descriptor whose integer id crosses the op boundary as
 `b_type_id`.  Mirrors aphrodite/scalar_type.py:22-340 of the reference (id
 bitfield :129-156) for the integer types this build handles and the 8-bit
-floating-point weight type float8_e4m3fn."""
+floating-point weight type float8_e4m3fn, the 4-bit one float4_e2m1f and the
+scale type float8_e8m0fnu."""
 from __future__ import annotations
 
 import functools
@@ -88,3 +89,5 @@ class scalar_types:
     uint4b8 = ScalarType.uint(4, 8)
     uint8b128 = ScalarType.uint(8, 128)
     float8_e4m3fn = ScalarType.float_(4, 3, True, _NAN_REPR_EXTD_RANGE_MAX_MIN)
+    float8_e8m0fnu = ScalarType(8, 0, False, 0, True, _NAN_REPR_EXTD_RANGE_MAX_MIN)
+    float4_e2m1f = ScalarType.float_(2, 1, True, _NAN_REPR_NONE)

@@ -609,3 +609,108 @@ def test_prepare_fp8_moe_layer_and_fused_marlin_moe(cfg):
     got = gu.host_f32(y)
     max_ref = np.abs(want).max()
     assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)
+
+
+# ---------------------------------------------------------------- MXFP4 weights (float4_e2m1f, e8m0 block scales)
+@pytest.mark.parametrize("m,k,n", [(1, 512, 256), (33, 1024, 320), (16, 2880, 5760), (200, 256, 512)])
+def test_mxfp4_random_weight_helper_and_marlin_gemm(m, k, n):
+    """The reference's MXFP4 case of its Marlin GEMM test (test_marlin_gemm.py with
+    rand_marlin_weight_mxfp4_like): the op takes the float8_e8m0fnu scales in the
+    reference's order; compared with the matmul on the dequantised weight."""
+    from sonar_amd import marlin_utils_fp4 as f4
+    from sonar_amd import ops
+    from sonar_amd.marlin_utils import marlin_make_workspace_new
+    from sonar_amd.scalar_type import scalar_types
+    torch.manual_seed(m + k)
+    weight = torch.empty((n, k), dtype=torch.bfloat16, device=gu.DEV)
+    a = (0.5 * torch.randn((m, k), device=gu.DEV)).to(torch.bfloat16)
+    w_ref, qweight, scales = f4.rand_marlin_weight_mxfp4_like(weight, 32)
+    assert qweight.shape == (k // 16, 2 * n) and scales.shape == (k // 32, n)
+    assert scales.dtype == torch.float8_e8m0fnu
+    workspace = marlin_make_workspace_new(a.device)
+    out = ops.marlin_gemm(a, None, qweight, None, scales, None, None, None, None, None, workspace,
+                          scalar_types.float4_e2m1f, m, n, k)
+    again = ops.marlin_gemm(a, None, qweight, None, scales, None, None, None, None, None, workspace,
+                            scalar_types.float4_e2m1f, m, n, k)     # converted scales come from the cache
+    torch.cuda.synchronize()
+    assert torch.equal(out, again)
+    want = (a.float() @ w_ref.float()).cpu().numpy()
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(out), want)
+    assert ok, worst
+    with pytest.raises(RuntimeError, match="bfloat16"):
+        ops.marlin_gemm(a.half(), None, qweight, None, scales, None, None, None, None, None, workspace,
+                        scalar_types.float4_e2m1f, m, n, k)
+    with pytest.raises(NotImplementedError, match="NVFP4"):
+        ops.marlin_gemm(a, None, qweight, None, scales.view(torch.float8_e4m3fn), None, None, None, None, None,
+                        workspace, scalar_types.float4_e2m1f, m, n, k)
+
+
+@pytest.mark.parametrize("k,n", [(512, 384), (384, 320)])   # 320 columns: padded to 384 inside
+def test_prepare_mxfp4_layer_and_apply(k, n):
+    """An MXFP4 checkpoint layer (weight (N, K/2) bytes, low nibble first; scales
+    (N, K/32) exponent bytes) -> prepare_fp4_layer_for_marlin ->
+    apply_fp4_marlin_linear, against the oracle on the same bytes."""
+    from sonar_amd import marlin_utils_fp4 as f4
+    rng = np.random.default_rng(k + n)
+    codes = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    e = rng.integers(108, 122, size=(k // 32, n)).astype(np.uint8)
+    w_ref = mo.dequantize_mxfp4(codes, e)
+    by_n = codes.T                                            # (N, K)
+    packed = np.ascontiguousarray((by_n[:, 0::2] | (by_n[:, 1::2] << 4)).astype(np.uint8))
+    layer = types.SimpleNamespace(output_size_per_partition=n, input_size_per_partition=k,
+                                  params_dtype=torch.bfloat16)
+    layer.weight = torch.from_numpy(packed).to(gu.DEV)
+    layer.weight_scale = torch.from_numpy(np.ascontiguousarray(e.T)).to(gu.DEV)
+    bias32 = mo.round_to_dtype(1e-2 * rng.standard_normal(n).astype(np.float32), "bf16")
+    layer.bias = gu.dev_bits16(bias32, "bf16")
+    f4.prepare_fp4_layer_for_marlin(layer)
+    assert layer.weight_scale.dtype == torch.float8_e8m0fnu
+    x32 = mo.make_activations(4, 6, k, "bf16", std=0.5)
+    y = f4.apply_fp4_marlin_linear(gu.dev_bits16(x32, "bf16").view(2, 3, k), layer.weight, layer.weight_scale, None,
+                                   layer.workspace, n, k, layer.bias)
+    torch.cuda.synchronize()
+    assert y.shape == (2, 3, n)
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y.view(6, n)), mo.gemm_reference(x32, w_ref, bias32))
+    assert ok, worst
+
+
+@pytest.mark.parametrize("cfg", [
+    # m, experts, topk, hidden, intermediate, bias
+    (5, 4, 2, 256, 128, False),
+    (70, 4, 2, 256, 256, True),
+    (200, 8, 2, 128, 128, False),
+], ids=str)
+def test_prepare_moe_mxfp4_layer_and_fused_marlin_moe(cfg):
+    """MXFP4 expert weights (w13 (E, 2N, K/2), w2 (E, K, N/2) bytes, exponent-byte
+    scales) -> prepare_moe_mxfp4_layer_for_marlin -> fused_marlin_moe, against the
+    per-token reference on the same bytes."""
+    from sonar_amd import marlin_utils_fp4 as f4
+    from sonar_amd.fused_moe import fused_marlin_moe
+    from sonar_amd.scalar_type import scalar_types
+    m, e, topk, hidden, inter, bias = cfg
+    rng = np.random.default_rng(hidden + inter + m)
+    layer = types.SimpleNamespace(params_dtype=torch.bfloat16)
+
+    def expert_set(rows, cols):   # checkpoint shape (E, rows = N of the GEMM, cols = K of the GEMM)
+        codes = rng.integers(0, 16, size=(e, rows, cols), dtype=np.int32)
+        ex = rng.integers(116, 124, size=(e, rows, cols // 32)).astype(np.uint8)
+        packed = np.ascontiguousarray((codes[:, :, 0::2] | (codes[:, :, 1::2] << 4)).astype(np.uint8))
+        ref = [mo.dequantize_mxfp4(codes[i].T, np.ascontiguousarray(ex[i].T)) for i in range(e)]
+        b32 = mo.round_to_dtype(0.1 * rng.standard_normal((e, rows)).astype(np.float32), "bf16") if bias else None
+        return torch.from_numpy(packed).to(gu.DEV), torch.from_numpy(ex).to(gu.DEV), ref, b32
+
+    w13, s13, ref13, b13 = expert_set(2 * inter, hidden)
+    w2, s2, ref2, b2 = expert_set(hidden, inter)
+    dev_bias = lambda b: None if b is None else gu.dev_bits16(b, "bf16")
+    mw13, mw2, ms13, ms2, mb13, mb2 = f4.prepare_moe_mxfp4_layer_for_marlin(layer, w13, w2, s13, s2, dev_bias(b13),
+                                                                            dev_bias(b2))
+    topk_ids, topk_w = _route(m, e, topk, m)
+    x32 = mo.round_to_dtype(0.5 * mo.make_activations(m, m, hidden, "bf16"), "bf16")
+    y = fused_marlin_moe(gu.dev_bits16(x32, "bf16"), mw13, mw2, mb13, mb2, ms13, ms2,
+                         torch.from_numpy(topk_w).to(gu.DEV), torch.from_numpy(topk_ids).to(gu.DEV),
+                         scalar_types.float4_e2m1f.id)
+    torch.cuda.synchronize()
+    want = _moe_reference(x32, ref13, ref2, topk_ids, topk_w, "bf16", b13, b2)
+    got = gu.host_f32(y)
+    max_ref = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)

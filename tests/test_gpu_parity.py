@@ -479,6 +479,90 @@ def test_fp8_weights_rejected_configurations(gu):
     torch.cuda.synchronize()
 
 
+def _layer_mxfp4(gu, seed, k, n):
+    """An MXFP4 layer on the device: float4_e2m1f codes in GPTQ words -> repack op
+    -> streaming order; the block scales 2^(e - 127) as bf16 in
+    marlin_permute_scales order (what the C entry points take); plus the
+    oracle's dequantised matrix."""
+    rng = np.random.default_rng(seed)
+    codes = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    codes[:16, 0] = np.arange(16)                      # every code in one column
+    e = rng.integers(108, 122, size=(k // 32, n)).astype(np.uint8)
+    w_ref = mo.dequantize_mxfp4(codes, e)
+    marlin = gu.gptq_repack(gu.dev_i32(mo.gptq_pack(codes)), None, k, n)
+    native = gu.to_gfx950(marlin, k, n)
+    s_dev = gu.dev_bits16(mo.marlin_permute_scales(mo.mx_scale_values(e), k, n, 32), "bf16")
+    return dict(codes=codes, e=e, native=native, scales=s_dev, groups=k // 32, w_ref=w_ref)
+
+
+MXFP4_CASES = [
+    # m, k, n, bias
+    (1, 128, 64, False),
+    (7, 512, 256, True),
+    (16, 4096, 1024, False),
+    (33, 1024, 320, True),
+    (64, 256, 4096, False),
+    (100, 1024, 512, False),
+    (300, 512, 192, True),
+    (1, 2880, 5760, False),     # gpt-oss expert shape: K is 90 groups of 32 rows
+]
+
+
+@pytest.mark.parametrize("m,k,n,bias", MXFP4_CASES)
+def test_mxfp4_weights_dequant_bit_exact_and_gemm_within_tolerance(gu, m, k, n, bias):
+    """float4_e2m1f weights with power-of-two scales per 32 rows, bf16 activations
+    (generate_kernels.py:102-110; dequant.h:397-470)."""
+    from sonar_amd import _lib
+    lib = _lib.load()
+    L = _layer_mxfp4(gu, 7 * m + k, k, n)
+    w = torch.empty((k, n), dtype=torch.bfloat16, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_dequant(gu.ptr(L["native"]), _lib.LAYOUT_GFX950, gu.ptr(L["scales"]), None,
+                                        None, gu.ptr(w), gu.dtype_code("bf16"), _lib.TYPE_FLOAT4_E2M1F,
+                                        n, k, L["groups"], 1, gu.stream()))
+    torch.cuda.synchronize()
+    got = w.view(torch.int16).cpu().numpy().view(np.uint16)
+    assert np.array_equal(got, mo.to_bits16(L["w_ref"], "bf16"))   # bits: the code 8 gives -0
+
+    bias32 = bias_dev = None
+    if bias:
+        bias32 = mo.round_to_dtype(1e-2 * np.random.default_rng(m).standard_normal(n).astype(np.float32), "bf16")
+        bias_dev = gu.dev_bits16(mo.marlin_permute_bias(bias32), "bf16")
+    a32 = mo.make_activations(m + 1, m, k, "bf16", std=0.5)
+    a = gu.dev_bits16(a32, "bf16")
+    c = torch.empty((m, n), dtype=torch.bfloat16, device=gu.DEV)
+    workspace = torch.zeros(torch.cuda.get_device_properties(0).multi_processor_count, dtype=torch.int32,
+                            device=gu.DEV)
+    scratch = torch.empty(max(lib.sonar_marlin_gemm_scratch_bytes(m, n, k), 16), dtype=torch.uint8, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_gemm(
+        gu.ptr(a), k, gu.ptr(c), gu.ptr(L["native"]), _lib.LAYOUT_GFX950, gu.ptr(bias_dev), gu.ptr(L["scales"]), None,
+        None, None, gu.ptr(workspace), workspace.numel(), gu.ptr(scratch), scratch.numel(),
+        gu.dtype_code("bf16"), _lib.TYPE_FLOAT4_E2M1F, m, n, k, L["groups"], 1, 0, 1, gu.stream()))
+    torch.cuda.synchronize()
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), mo.gemm_reference(a32, L["w_ref"], bias32))
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+
+
+def test_mxfp4_weights_rejected_configurations(gu):
+    """MXFP4 exists for bfloat16 activations and groups of 32 rows only
+    (generate_kernels.py:102-110), without act-order."""
+    from sonar_amd import _lib
+    lib = _lib.load()
+    k, n = 256, 64
+    L = _layer_mxfp4(gu, 1, k, n)
+    w = torch.empty((k, n), dtype=torch.bfloat16, device=gu.DEV)
+    idx = torch.zeros(k, dtype=torch.int32, device=gu.DEV)
+
+    def dequant(dtype, groups, g_idx):
+        return lib.sonar_marlin_dequant(gu.ptr(L["native"]), _lib.LAYOUT_GFX950, gu.ptr(L["scales"]), None,
+                                        gu.ptr(g_idx), gu.ptr(w), dtype, _lib.TYPE_FLOAT4_E2M1F, n, k, groups, 1,
+                                        gu.stream())
+    assert dequant(1, 8, None) == 0
+    assert dequant(0, 8, None) != 0 and "bfloat16" in lib.sonar_marlin_last_error().decode()
+    assert dequant(1, 2, None) != 0 and "32 rows" in lib.sonar_marlin_last_error().decode()
+    assert dequant(1, 8, idx) != 0 and "act-order" in lib.sonar_marlin_last_error().decode()
+    torch.cuda.synchronize()
+
+
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("m", [1, 16, 40, 100, 300])
 def test_act_order_shard_without_whole_groups(gu, dtype, m):

@@ -8,7 +8,7 @@ laid out in Marlin order by the index recipe of `marlin_utils_test.py`
   * `marlin_gemm` must agree with `torch.matmul(a, w_ref)` under the
     reference's criterion mean|out - ref| / mean|ref| < 0.04 (test_marlin_gemm,
     test_marlin_gemm_with_bias), over the reference's grid of shapes, group
-    sizes, weight types (integer and fp8), act-order and is_k_full for 16-bit
+    sizes, weight types (integer, fp8, MXFP4), act-order and is_k_full for 16-bit
     activations.
 No oracle here: the expected values come from torch on the GPU, as in the
 reference."""
@@ -32,6 +32,7 @@ DENSE_CONFIGS = [
     {"b_type": scalar_types.uint4b8, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]},   # GPTQ int4
     {"b_type": scalar_types.uint8b128, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]}, # GPTQ int8
     {"b_type": scalar_types.float8_e4m3fn, "group_blocks": [-1, 8]},                              # FP8
+    {"b_type": scalar_types.float4_e2m1f, "a_type": [torch.bfloat16], "group_blocks": [2]},       # MXFP4
 ]
 
 
@@ -93,7 +94,8 @@ def _gemm_cases():
         size_m, size_n, size_k = mf, nf * n_chunk, kf * 128
         if act_order and not cfg.get("support_act_order", False):
             continue
-        for dtype, group_blocks in itertools.product([torch.float16, torch.bfloat16], cfg["group_blocks"]):
+        for dtype, group_blocks in itertools.product(cfg.get("a_type", [torch.float16, torch.bfloat16]),
+                                                     cfg["group_blocks"]):
             group_size = group_blocks if group_blocks <= 0 else group_blocks * 16
             if group_size > 0 and size_k % group_size != 0:
                 continue
@@ -112,6 +114,7 @@ def _gemm_cases():
 def test_marlin_gemm(b_type, dtype, group_size, size_m, size_n, size_k, act_order, is_k_full):
     from sonar_amd import ops
     from sonar_amd.marlin_utils import marlin_make_workspace_new
+    from sonar_amd.marlin_utils_fp4 import rand_marlin_weight_mxfp4_like
     from sonar_amd.marlin_utils_fp8 import marlin_quant_fp8_torch
     from sonar_amd.marlin_utils_test import awq_marlin_quantize, marlin_quantize
     a_input = rand_data((size_m, size_k), dtype=dtype)
@@ -121,6 +124,9 @@ def test_marlin_gemm(b_type, dtype, group_size, size_m, size_n, size_k, act_orde
         g_idx = sort_indices = None
     elif b_type == scalar_types.float8_e4m3fn:
         w_ref, marlin_q_w, marlin_s = marlin_quant_fp8_torch(b_weight.T.contiguous(), group_size)
+        g_idx = sort_indices = marlin_zp = None
+    elif b_type == scalar_types.float4_e2m1f:
+        w_ref, marlin_q_w, marlin_s = rand_marlin_weight_mxfp4_like(b_weight.T, group_size)
         g_idx = sort_indices = marlin_zp = None
     else:
         w_ref, marlin_q_w, marlin_s, g_idx, sort_indices, _ = marlin_quantize(b_weight, b_type, group_size, act_order)
@@ -161,12 +167,13 @@ def test_marlin_gemm_with_bias(size_m):
 # ---------------------------------------------------------------------------
 # tests/kernels/moe/test_moe.py:129-143, 688-1010 of the reference: the fused
 # Marlin MoE layer against a plain torch mixture of experts on the dequantised
-# weights, atol 4e-2, over the reference's scenarios for integer and fp8 weights.
+# weights, atol 4e-2, over the reference's scenarios for integer, fp8 and MXFP4 weights.
 MOE_CONFIGS = [
     {"b_type": scalar_types.uint4, "group_blocks": [-1, 2, 4, 8]},
     {"b_type": scalar_types.uint4b8, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]},
     {"b_type": scalar_types.uint8b128, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]},
     {"b_type": scalar_types.float8_e4m3fn, "group_blocks": [-1, 8]},
+    {"b_type": scalar_types.float4_e2m1f, "a_type": torch.bfloat16, "group_blocks": [2]},
 ]
 MARLIN_MOE_SCENARIOS = [
     # (m, n, k, e, topk, ep_size, act_order, is_k_full)
@@ -196,7 +203,8 @@ def _moe_cases():
                     continue
                 if group_size in (k, n):
                     continue
-                cases.append((cfg["b_type"], group_size, m, n, k, e, topk, ep_size, act_order, is_k_full))
+                cases.append((cfg["b_type"], cfg.get("a_type", torch.float16), group_size, m, n, k, e, topk, ep_size,
+                              act_order, is_k_full))
     return cases
 
 
@@ -204,6 +212,7 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None):
     """MarlinMoEWeightData.make (test_moe.py:774-892): every expert's (N, K)
     matrix quantised and laid out on its own, then stacked."""
     from sonar_amd.marlin_utils import marlin_permute_bias
+    from sonar_amd.marlin_utils_fp4 import rand_marlin_weight_mxfp4_like
     from sonar_amd.marlin_utils_fp8 import marlin_quant_fp8_torch
     from sonar_amd.marlin_utils_test import awq_marlin_quantize, marlin_quantize
     k = w.shape[-1]
@@ -214,6 +223,8 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None):
             out["zeros"].append(zeros)
         elif quant_type == scalar_types.float8_e4m3fn:
             w_ref, qweight, scales = marlin_quant_fp8_torch(w[i].contiguous(), group_size)
+        elif quant_type == scalar_types.float4_e2m1f:
+            w_ref, qweight, scales = rand_marlin_weight_mxfp4_like(w[i], group_size)
         else:
             w_ref, qweight, scales, g_idx, sort_indices, _ = marlin_quantize(
                 w[i].transpose(1, 0), quant_type, group_size, act_order, torch.randperm(k))
@@ -252,11 +263,11 @@ def _torch_experts(a, w1, w2, topk_weight, topk_ids, expert_map=None, b1=None, b
     return out.to(a.dtype)
 
 
-@pytest.mark.parametrize("b_type,group_size,m,n,k,e,topk,ep_size,act_order,is_k_full", _moe_cases(), ids=str)
-def test_fused_marlin_moe(b_type, group_size, m, n, k, e, topk, ep_size, act_order, is_k_full):
+@pytest.mark.parametrize("b_type,dtype,group_size,m,n,k,e,topk,ep_size,act_order,is_k_full", _moe_cases(),
+                         ids=lambda v: str(v).replace("torch.", ""))
+def test_fused_marlin_moe(b_type, dtype, group_size, m, n, k, e, topk, ep_size, act_order, is_k_full):
     from sonar_amd.fused_moe import fused_marlin_moe
     torch.manual_seed(1)
-    dtype = torch.float16
     a = torch.randn((m, k), device="cuda", dtype=dtype) / 10
     w1 = torch.randn((e, 2 * n, k), device="cuda", dtype=dtype) / 10
     w2 = torch.randn((e, k, n), device="cuda", dtype=dtype) / 10

@@ -37,6 +37,9 @@ def test_type_id_constants_match_header_and_oracle():
     assert scalar_types.uint8b128.id == mo.UINT8B128_ID == _lib.TYPE_UINT8B128
     assert int(re.search(r"SONAR_TYPE_FLOAT8_E4M3FN (\d+)LL", header).group(1)) == mo.FLOAT8_E4M3FN_ID
     assert scalar_types.float8_e4m3fn.id == mo.FLOAT8_E4M3FN_ID == _lib.TYPE_FLOAT8_E4M3FN
+    assert int(re.search(r"SONAR_TYPE_FLOAT4_E2M1F (\d+)LL", header).group(1)) == mo.FLOAT4_E2M1F_ID
+    assert scalar_types.float4_e2m1f.id == mo.FLOAT4_E2M1F_ID == _lib.TYPE_FLOAT4_E2M1F
+    assert str(scalar_types.float4_e2m1f) == "float4_e2m1f" and scalar_types.float4_e2m1f.size_bits == 4
     assert str(scalar_types.float8_e4m3fn) == "float8_e4m3fn" and scalar_types.float8_e4m3fn.size_bits == 8
     assert str(scalar_types.uint8b128) == "uint8b128" and str(scalar_types.int4) == "int4"
     # tests/test_scalartype.py:10-25 of the reference
@@ -490,3 +493,24 @@ def test_fp8_host_helpers():
     assert not mu.check_marlin_supported(st.float8_e4m3fn, 128, has_zp=True)
     assert st.float8_e4m3fn not in mu.query_marlin_supported_quant_types(False, include_fp_type=False)
     assert f8.is_fp8_marlin_supported()
+
+
+def test_mxfp4_host_helpers():
+    """marlin_utils_fp4.py:123-135 of the reference: the scale rows with every
+    four neighbours in the order 0, 2, 1, 3, as exponent bytes; float4_e2m1f
+    joins the supported types without zero points."""
+    from sonar_amd import marlin_utils as mu
+    from sonar_amd import marlin_utils_fp4 as f4
+    from sonar_amd.scalar_type import scalar_types as st
+    e = torch.tensor([[120, 121, 122, 123, 124, 125, 126, 127]], dtype=torch.uint8)
+    s = e.view(torch.float8_e8m0fnu).to(torch.bfloat16)
+    assert s[0, 7].item() == 1.0 and s[0, 0].item() == 2.0 ** -7
+    out = f4.mxfp4_marlin_process_scales(s)
+    assert out.dtype == torch.float8_e8m0fnu
+    assert out.view(torch.uint8).tolist() == [[120, 122, 121, 123, 124, 126, 125, 127]]
+    assert np.array_equal(out.view(torch.uint8).numpy(), mo.mxfp4_process_scales(e.numpy()))
+    with pytest.raises(NotImplementedError):
+        f4.mxfp4_marlin_process_scales(s, input_dtype=torch.float8_e4m3fn)
+    assert mu.check_marlin_supported(st.float4_e2m1f, 32)
+    assert not mu.check_marlin_supported(st.float4_e2m1f, 32, has_zp=True)
+    assert f4.is_fp4_marlin_supported()

@@ -442,3 +442,40 @@ def test_fp8_dequant_groups():
     v = mo.fp8_e4m3fn_values()
     assert np.array_equal(w[:128], mo.round_to_dtype(v[codes[:128]] * s[0], "fp16"))
     assert np.array_equal(w[128:], mo.round_to_dtype(v[codes[128:]] * s[1], "fp16"))
+
+
+# ---------------------------------------------------------------- MXFP4 weights (float4_e2m1f, e8m0 scales)
+def test_fp4_type_id_values_and_scales():
+    import torch
+    assert mo.FLOAT4_E2M1F_ID == 2 | (1 << 8) | (1 << 16) | (1 << 49) == 562949953487106
+    v = mo.fp4_e2m1_values()
+    # the list of the OCP microscaling format, codes 0..7, and its negatives for 8..15
+    assert v[:8].tolist() == [0.0, 0.5, 1.0, 1.5, 2.0, 3.0, 4.0, 6.0]
+    assert v[8:].tolist() == [-0.0, -0.5, -1.0, -1.5, -2.0, -3.0, -4.0, -6.0] and np.signbit(v[8])
+    # the reference's test recipe (marlin_utils_fp4.py:720-727): sign and the three other bits at
+    # the top of a float8_e4m3fn byte, torch's conversion, times 2^6
+    code = torch.arange(16, dtype=torch.uint8) << 4
+    as_fp8 = ((code & 0x80) | ((code & 0x70) >> 2)).view(torch.float8_e4m3fn).float() * 64
+    assert np.array_equal(v, as_fp8.numpy())
+    # the kernel's reading: sign at bit 15, the other three bits at bits 11-9 of an fp16, times 2^14
+    c = np.arange(16, dtype=np.uint16)
+    h = (((c & 8) << 12) | ((c & 7) << 9)).astype(np.uint16).view(np.float16).astype(np.float64)
+    assert np.array_equal(h * 2.0 ** 14, v.astype(np.float64))
+    e = np.arange(255, dtype=np.uint8)
+    t = torch.from_numpy(e).view(torch.float8_e8m0fnu).float().numpy()
+    assert np.array_equal(mo.mx_scale_values(e), t)
+    assert mo.mx_scale_values(np.array([127, 120, 0]))[:2].tolist() == [1.0, 2.0 ** -7]
+
+
+def test_mxfp4_dequant_and_scale_reorder():
+    rng = np.random.default_rng(15)
+    codes = rng.integers(0, 16, size=(64, 8), dtype=np.int32)
+    e = rng.integers(100, 130, size=(2, 8)).astype(np.uint8)
+    w = mo.dequantize_mxfp4(codes, e)
+    v = mo.fp4_e2m1_values()
+    for k in (0, 31, 32, 63):
+        for n in (0, 7):
+            assert w[k, n] == v[codes[k, n]] * 2.0 ** (int(e[k // 32, n]) - 127)
+    x = np.arange(16).reshape(2, 8)
+    y = mo.mxfp4_process_scales(x)
+    assert y[0].tolist() == [0, 2, 1, 3, 4, 6, 5, 7] and np.array_equal(mo.mxfp4_process_scales(y), x)
