@@ -192,6 +192,15 @@ struct DqF4 {
   }
 };
 
+// Eight neighbours of a permuted scale row of grouped scales, slots
+// 8 (col16 % 8) .. + 7, hold the scales of columns 16 j + col16 (j = 0..3) and
+// of their partners col16 +- 8: column 16 j + col16 is slot 2 j + col16 / 8
+// (scale_slot with grouped = true).
+__device__ __forceinline__ uint16_t chunk_scale(const uint4& sv, int j, int col16) {
+  const uint32_t word = j == 0 ? sv.x : (j == 1 ? sv.y : (j == 2 ? sv.z : sv.w));
+  return (uint16_t)(word >> (16 * (col16 >> 3)));
+}
+
 // The dequantiser of a 4-bit weight type.
 template <typename T, bool FP4>
 struct Dq4Of {

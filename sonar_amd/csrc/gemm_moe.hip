@@ -115,13 +115,16 @@ __device__ __forceinline__ void moe_scatter(const MoeParams& p, const floatx4_t 
   }
 }
 
-template <typename T, int MB>
+// CHUNK_SCALES (groups of 32 rows, one per chunk: MXFP4): the scales of every
+// chunk travel with the unit (eight neighbours of the permuted scale row per lane).
+template <typename T, int MB, bool CHUNK_SCALES = false>
 struct MoeUnit {
   uint4 q[4];
   typename Dq<T>::vec8 a[4][MB];
   uint32_t sbits[4];
   uint32_t zword;
   int group;
+  uint4 sv[CHUNK_SCALES ? 4 : 1];
 };
 
 // HAS_GIDX (with HAS_PERM, symmetric weights): an act-order shard that does not
@@ -176,7 +179,8 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
   const bool grouped = p.num_groups > 1;
   const uint32_t magic = magic_register();
 
-  auto load_unit = [&](MoeUnit<T, MB>& u, int unit) {
+  const bool chunk_scales = FP4 && grouped;
+  auto load_unit = [&](MoeUnit<T, MB, FP4>& u, int unit) {
     const int chunk0 = unit * p.unit_chunks;
 #pragma unroll
     for (int cc = 0; cc < 4; ++cc)
@@ -191,6 +195,13 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
     const int g = grouped ? (chunk0 * kChunkK) / p.group_size : 0;
     u.group = g;
     const uint16_t* srow = scales + (long)g * p.size_n + strip * kStripN;
+    if (chunk_scales) {   // group = chunk
+#pragma unroll
+      for (int cc = 0; cc < 4; ++cc)
+        if (cc < p.unit_chunks)
+          u.sv[FP4 ? cc : 0] = *reinterpret_cast<const uint4*>(srow + (long)cc * p.size_n + 8 * (col16 & 7));
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) u.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
     if (HAS_ZP) u.zword = zeros[(long)g * (p.size_n / 8) + strip * 8 + zero_point_word(col16)];
@@ -202,18 +213,20 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-  MoeUnit<T, MB> cur, nxt;
+  MoeUnit<T, MB, FP4> cur, nxt;
   int mine = wave;
   if (mine < p.units_per_strip) load_unit(cur, mine);
   while (mine < p.units_per_strip) {
     const int next = mine + kMoeWaves;
     if (next < p.units_per_strip) load_unit(nxt, next);
     Col cols[4];
+    if (!chunk_scales) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      int z = 8;
-      if (HAS_ZP) z = (int)((cur.zword >> zero_point_shift(16 * j + col16)) & 0xFu);
-      cols[j] = D4::make_col((uint16_t)cur.sbits[j], z);
+      for (int j = 0; j < 4; ++j) {
+        int z = 8;
+        if (HAS_ZP) z = (int)((cur.zword >> zero_point_shift(16 * j + col16)) & 0xFu);
+        cols[j] = D4::make_col((uint16_t)cur.sbits[j], z);
+      }
     }
     int cur_group = cur.group;
     const int chunk0 = mine * p.unit_chunks;
@@ -221,7 +234,10 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
     for (int cc = 0; cc < 4; ++cc) {
       if (cc < p.unit_chunks) {
         const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
-        if (g != cur_group) {  // groups smaller than a unit
+        if (chunk_scales) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) cols[j] = D4::make_col(chunk_scale(cur.sv[FP4 ? cc : 0], j, col16), 0);
+        } else if (g != cur_group) {  // groups smaller than a unit
           cur_group = g;
           load_cols<T, HAS_ZP, D4>(cols, scales, zeros, p.size_n, strip, g, col16, grouped);
         }
@@ -546,6 +562,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     SONAR_REQUIRE(size_k == 32 * num_groups,
                   "float4_e2m1f weights (MXFP4) take one scale per group of 32 rows; got size_k = %ld, "
                   "num_groups = %ld", (long)size_k, (long)num_groups);
+    SONAR_REQUIRE(((uintptr_t)b_scales) % 16 == 0, "b_scales must be 16-byte aligned");
   }
   if (fp8) {
     // moe/marlin_moe_wna16/generate_kernels.py: channelwise scales or groups of 128 rows, no act-order

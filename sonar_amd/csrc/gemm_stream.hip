@@ -242,17 +242,22 @@ __device__ __forceinline__ void finish_block_grouped(const StreamParams& p, int 
 template <int MB>
 constexpr int unit_buffer_chunks() { return MB >= 3 ? 2 : 4; }
 
-template <typename T, int MB>
+// CHUNK_SCALES (groups of 32 rows, one per chunk: MXFP4): the scales of every
+// chunk travel with the unit, eight neighbours of the permuted scale row per
+// lane (16 bytes) of which it uses four, instead of being fetched when the
+// chunk is reached.
+template <typename T, int MB, bool CHUNK_SCALES = false>
 struct UnitBuf {
   uint4 q[unit_buffer_chunks<MB>()];
   typename Dq<T>::vec8 a[unit_buffer_chunks<MB>()][MB];
   uint32_t sbits[4];
   uint32_t zword;
   int group;
+  uint4 sv[CHUNK_SCALES ? unit_buffer_chunks<MB>() : 1];
 };
 
-template <typename T, int MB, bool HAS_ZP, bool HAS_PERM>
-__device__ __forceinline__ void load_unit(UnitBuf<T, MB>& b, const StreamParams& p, int u, int lane,
+template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool CHUNK_SCALES = false>
+__device__ __forceinline__ void load_unit(UnitBuf<T, MB, CHUNK_SCALES>& b, const StreamParams& p, int u, int lane,
                                           bool grouped) {
   const int col16 = lane & 15, kb = lane >> 4;
   const int strip = u / p.units_per_strip;
@@ -272,6 +277,13 @@ __device__ __forceinline__ void load_unit(UnitBuf<T, MB>& b, const StreamParams&
   const int g = grouped ? (chunk0 * kChunkK) / p.group_size : 0;
   b.group = g;
   const uint16_t* srow = p.scales + (long)g * p.size_n + strip * kStripN;
+  if (CHUNK_SCALES && grouped) {   // group = chunk
+#pragma unroll
+    for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc)
+      if (cc < p.unit_chunks)
+        b.sv[cc] = *reinterpret_cast<const uint4*>(srow + (long)cc * p.size_n + 8 * (col16 & 7));
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) b.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
   if (HAS_ZP) b.zword = p.zeros[(long)g * (p.size_n / 8) + strip * 8 + zero_point_word(col16)];
@@ -303,9 +315,9 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
   const bool grouped = p.num_groups > 1;
   const uint32_t magic = magic_register();
 
-  UnitBuf<T, MB> cur, nxt;
+  UnitBuf<T, MB, FP4> cur, nxt;
   int mine = u_begin + wave;
-  if (mine < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM>(cur, p, mine, lane, grouped);
+  if (mine < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM, FP4>(cur, p, mine, lane, grouped);
 
   int seg_begin = u_begin;
   while (seg_begin < u_end) {
@@ -322,13 +334,16 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
 
     while (mine < seg_end) {
       const int next = mine + kWaves;
-      if (next < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM>(nxt, p, next, lane, grouped);
+      if (next < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM, FP4>(nxt, p, next, lane, grouped);
       Col cols[4];
+      const bool chunk_scales = FP4 && grouped;   // the scales of every chunk came with the unit
+      if (!chunk_scales) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        int z = 8;
-        if (HAS_ZP) z = (int)((cur.zword >> zero_point_shift(16 * j + col16)) & 0xFu);
-        cols[j] = D4::make_col((uint16_t)cur.sbits[j], z);
+        for (int j = 0; j < 4; ++j) {
+          int z = 8;
+          if (HAS_ZP) z = (int)((cur.zword >> zero_point_shift(16 * j + col16)) & 0xFu);
+          cols[j] = D4::make_col((uint16_t)cur.sbits[j], z);
+        }
       }
       int cur_group = cur.group;
       const int chunk0 = (mine - strip_first) * p.unit_chunks;
@@ -336,7 +351,10 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
       for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc) {
         if (cc < p.unit_chunks) {
           const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
-          if (g != cur_group) {  // groups smaller than a unit
+          if (chunk_scales) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) cols[j] = D4::make_col(chunk_scale(cur.sv[FP4 ? cc : 0], j, col16), 0);
+          } else if (g != cur_group) {  // groups smaller than a unit
             cur_group = g;
             load_cols<T, HAS_ZP, D4>(cols, p.scales, p.zeros, p.size_n, strip, g, col16, grouped);
           }
@@ -1331,6 +1349,7 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
     SONAR_REQUIRE(size_k == 32 * num_groups,
                   "float4_e2m1f weights (MXFP4) take one scale per group of 32 rows; got size_k = %ld, "
                   "num_groups = %ld", (long)size_k, (long)num_groups);
+    SONAR_REQUIRE(((uintptr_t)b_scales) % 16 == 0, "b_scales must be 16-byte aligned");
   }
   if (out.fp8) {
     // generate_kernels.py:87-93: channelwise scales or groups of 128 rows, no act-order
