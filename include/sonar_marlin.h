@@ -56,7 +56,9 @@ extern "C" {
 /* 8-bit floating-point codes (sign, 4 exponent bits, 3 mantissa bits, no infinities), in the 8-bit
  * weight order; b_scales then hold the scales times 2^8 (fp16) or 2^120 (bf16), as
  * fp8_fused_exponent_bias_into_scales makes them (quantization/utils/marlin_utils_fp8.py:35-46);
- * one scale per column or per group of 128 rows, no act-order (marlin/generate_kernels.py:87-93) */
+ * one scale per column, per group of 128 rows (marlin/generate_kernels.py:87-93) or, for MXFP8, per
+ * group of 32 rows (:111-119; the torch op takes the exponent bytes of the reference's callers and
+ * makes such scales of them); no act-order */
 #define SONAR_TYPE_FLOAT8_E4M3FN 2814749767172868LL
 /* 4-bit floating-point codes (sign, 2 exponent bits, 1 mantissa bit) in the 4-bit weight order,
  * with one power-of-two scale per column and group of 32 rows (MXFP4): bfloat16 activations only;

@@ -565,11 +565,11 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     SONAR_REQUIRE(((uintptr_t)b_scales) % 16 == 0, "b_scales must be 16-byte aligned");
   }
   if (fp8) {
-    // moe/marlin_moe_wna16/generate_kernels.py: channelwise scales or groups of 128 rows, no act-order
+    // moe/marlin_moe_wna16/generate_kernels.py: channelwise scales or groups of 128 rows (:111-119: MXFP8, groups of 32), no act-order
     SONAR_REQUIRE(!has_perm, "act-order is not supported with float8_e4m3fn weights");
-    SONAR_REQUIRE(num_groups == 1 || size_k == 128 * num_groups,
-                  "float8_e4m3fn weights take one scale per column or per group of 128 rows; got size_k = %ld, "
-                  "num_groups = %ld", (long)size_k, (long)num_groups);
+    SONAR_REQUIRE(num_groups == 1 || size_k == 128 * num_groups || size_k == 32 * num_groups,
+                  "float8_e4m3fn weights take one scale per column, per group of 128 rows or (MXFP8) per group "
+                  "of 32 rows; got size_k = %ld, num_groups = %ld", (long)size_k, (long)num_groups);
   }
   const bool row_groups = has_perm && !is_k_full;
   if (has_perm) {

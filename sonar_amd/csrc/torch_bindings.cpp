@@ -101,26 +101,30 @@ Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, 
 // bytes in marlin_permute_scales order with every four neighbours in the order
 // 0, 2, 1, 3; marlin_utils_fp4.py:123-135) -> bfloat16 powers of two in plain
 // marlin_permute_scales order, which the kernels read.  Cached like the weights.
-Tensor mx_scales_as_bf16(const Tensor& b_scales) {
+// `exponent_offset` is added to every exponent: 0 for MXFP4, 120 for MXFP8, whose
+// kernels expect the scales times 2^120 (the fp8 codes are read as bf16 numbers
+// with the same exponent field); exponents past the bf16 range become infinity.
+Tensor mx_scales_as_bf16(const Tensor& b_scales, int64_t exponent_offset) {
   const void* key = b_scales.const_data_ptr();
   {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     auto it = g_cache.find(key);
     if (it != g_cache.end() && !it->second.source.expired() &&
         it->second.source._unsafe_get_target() == b_scales.unsafeGetTensorImpl() && it->second.size_k == -1 &&
-        it->second.version == version_of(b_scales))
+        it->second.size_n == exponent_offset && it->second.version == version_of(b_scales))
       return it->second.native;
   }
   TORCH_CHECK(b_scales.numel() % 4 == 0, "b_scales.numel() must be a multiple of 4");
   const Tensor bytes = b_scales.view(at::kByte);
   const Tensor order = at::tensor({0, 2, 1, 3}, at::TensorOptions().dtype(at::kLong).device(b_scales.device()));
-  const Tensor e = bytes.reshape({-1, 4}).index_select(1, order).reshape(bytes.sizes()).to(at::kShort);
+  const Tensor e = bytes.reshape({-1, 4}).index_select(1, order).reshape(bytes.sizes()).to(at::kShort) +
+                   exponent_offset;
   // bfloat16 2^(e - 127): exponent field e; e = 0 is the subnormal 2^-127
-  const Tensor bits = at::where(e == 0, at::full_like(e, 0x40), e * 128);
+  const Tensor bits = at::where(e == 0, at::full_like(e, 0x40), at::clamp_max(e, 255) * 128);
   Tensor out = bits.view(at::kBFloat16);
   std::lock_guard<std::mutex> lock(g_cache_mutex);
   g_cache.insert_or_assign(key, NativeEntry{c10::weak_intrusive_ptr<c10::TensorImpl>(b_scales.getIntrusivePtr()),
-                                            out, -1, -1, -1, version_of(b_scales)});
+                                            out, -1, exponent_offset, -1, version_of(b_scales)});
   return out;
 }
 
@@ -254,7 +258,12 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
   TORCH_CHECK(b_scales.is_cuda(), "b_scales is not on GPU");
   TORCH_CHECK(b_scales.is_contiguous(), "b_scales is not contiguous");
   const bool fp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F;
-  if (fp4) {   // marlin.cu:600-611; the fp8 block scales of NVFP4 are not built
+  // marlin.cu:612-617: fp8 weights with exponent-byte scales per 32 rows (MXFP8, bfloat16 activations)
+  const bool mxfp8 = b_type_id == SONAR_TYPE_FLOAT8_E4M3FN && b_scales.scalar_type() == at::kFloat8_e8m0fnu;
+  if (mxfp8) {
+    TORCH_CHECK(a.scalar_type() == at::kBFloat16, "float8_e4m3fn weights with float8_e8m0fnu scales (MXFP8) "
+                "need bfloat16 activations");
+  } else if (fp4) {   // marlin.cu:600-611; the fp8 block scales of NVFP4 are not built
     TORCH_CHECK_NOT_IMPLEMENTED(b_scales.scalar_type() != at::kFloat8_e4m3fn,
                                 "float4_e2m1f weights with float8_e4m3fn scales (NVFP4) are not built");
     TORCH_CHECK(is_mx_scale_type(b_scales),
@@ -341,7 +350,8 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
   raise_if_failed(sonar_marlin_gemm(
       a.const_data_ptr(), a.stride(0), c.mutable_data_ptr(),
       static_cast<const uint32_t*>(native.const_data_ptr()), SONAR_LAYOUT_GFX950,
-      opt_ptr(b_bias_or_none), (fp4 ? mx_scales_as_bf16(b_scales) : b_scales).const_data_ptr(),
+      opt_ptr(b_bias_or_none),
+      (fp4 || mxfp8 ? mx_scales_as_bf16(b_scales, mxfp8 ? 120 : 0) : b_scales).const_data_ptr(),
       has_zp ? static_cast<const uint32_t*>(b_zeros_or_none->const_data_ptr()) : nullptr, g_idx, perm,
       static_cast<int32_t*>(workspace.mutable_data_ptr()), workspace.numel(), scratch.mutable_data_ptr(),
       scratch_bytes, dtype, b_type_id, size_m, size_n, size_k, num_groups, is_k_full ? 1 : 0,
@@ -389,7 +399,11 @@ Tensor moe_wna16_marlin_gemm(
   TORCH_CHECK(b_scales.dim() == 3 && b_scales.size(0) == experts, "b_scales rank = ", b_scales.dim(), " is not 3");
   TORCH_CHECK(b_scales.size(2) == size_n, "b_scales dim 2 = ", b_scales.size(2), " is not size_n = ", size_n);
   const bool fp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F;
-  if (fp4) {
+  const bool mxfp8 = b_type_id == SONAR_TYPE_FLOAT8_E4M3FN && b_scales.scalar_type() == at::kFloat8_e8m0fnu;
+  if (mxfp8) {
+    TORCH_CHECK(a.scalar_type() == at::kBFloat16, "float8_e4m3fn weights with float8_e8m0fnu scales (MXFP8) "
+                "need bfloat16 activations");
+  } else if (fp4) {
     TORCH_CHECK_NOT_IMPLEMENTED(b_scales.scalar_type() != at::kFloat8_e4m3fn,
                                 "float4_e2m1f weights with float8_e4m3fn scales (NVFP4) are not built");
     TORCH_CHECK(is_mx_scale_type(b_scales),
@@ -467,7 +481,8 @@ Tensor moe_wna16_marlin_gemm(
 
   raise_if_failed(sonar_moe_wna16_marlin_gemm(
       a.const_data_ptr(), c.mutable_data_ptr(), static_cast<const uint32_t*>(native.const_data_ptr()),
-      SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none), (fp4 ? mx_scales_as_bf16(b_scales) : b_scales).const_data_ptr(),
+      SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none),
+      (fp4 || mxfp8 ? mx_scales_as_bf16(b_scales, mxfp8 ? 120 : 0) : b_scales).const_data_ptr(),
       has_zp ? static_cast<const uint32_t*>(b_zeros_or_none->const_data_ptr()) : nullptr, g_idx, perm,
       static_cast<int32_t*>(workspace.mutable_data_ptr()), workspace.numel(),
       scratch_bytes > 0 ? scratch.mutable_data_ptr() : nullptr, scratch_bytes,

@@ -1,11 +1,11 @@
 """Weight-only FP8 (float8_e4m3fn weights, fp16 / bf16 activations) through the
 Marlin ops.  Mirrors aphrodite/model_executor/layers/quantization/utils/
-marlin_utils_fp8.py:31-365, 591-631 of the reference: the bytes of the fp8
+marlin_utils_fp8.py:31-631 of the reference: the bytes of the fp8
 weights travel as 8-bit codes (packed four to an int32 along K, then
 gptq_marlin_repack with num_bits = 8); the scales are permuted as for any Marlin
 layer and multiplied by 2^8 (fp16) or 2^120 (bf16), the difference between the
 exponent biases, because the kernels read a code as the 16-bit number with the
-same exponent field.
+same exponent field.  MXFP8 (exponent-byte scales per 32 rows) is at the end.
 """
 from __future__ import annotations
 
@@ -201,3 +201,85 @@ def marlin_quant_fp8_torch(weight: torch.Tensor, group_size: int, input_dtype: t
     marlin_qweight = ops.gptq_marlin_repack(packed, perm, size_k, size_n, 8)
     marlin_scales = marlin_permute_scales(scales.T, size_k, size_n, group_size)
     return weight_ref.T, marlin_qweight, fp8_fused_exponent_bias_into_scales(marlin_scales)
+
+
+# ---------------------------------------------------------------- MXFP8
+# float8_e4m3fn weights with one power-of-two scale (an exponent byte) per 32
+# rows, bfloat16 activations (marlin_utils_fp8.py:381-588 of the reference).
+MXFP8_GROUP_SIZE = 32
+
+
+def mxfp8_marlin_process_scales(marlin_scales: torch.Tensor) -> torch.Tensor:
+    """marlin_utils_fp8.py:381-386: every four neighbours of the permuted scale
+    rows in the order 0, 2, 1, 3, then the exponent bytes."""
+    reordered = marlin_scales.view(-1, 4)[:, [0, 2, 1, 3]].view(marlin_scales.size(0), -1)
+    return reordered.to(torch.float8_e8m0fnu)
+
+
+def apply_mxfp8_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
+                              workspace: torch.Tensor, size_n: int, size_k: int, bias: torch.Tensor | None = None,
+                              use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
+    """marlin_utils_fp8.py:389-434: the fp8 call with float8_e8m0fnu scales."""
+    return apply_fp8_marlin_linear(input, weight, weight_scale, workspace, size_n, size_k, bias,
+                                   use_fp32_reduce=use_fp32_reduce)
+
+
+def _mx_scales_for_marlin(exponent_bytes: torch.Tensor, size_n: int, size_k: int, padded_n: int, padded_k: int,
+                          dtype: torch.dtype) -> torch.Tensor:
+    """(N, K/32) exponent bytes -> permuted, reordered float8_e8m0fnu (K/32, N)."""
+    scales = exponent_bytes[:size_n, :size_k // MXFP8_GROUP_SIZE].contiguous()
+    scales = scales.view(torch.float8_e8m0fnu).to(dtype).T.contiguous()
+    scales = marlin_pad_scales(scales, size_n, size_k, padded_n, padded_k, MXFP8_GROUP_SIZE)
+    return mxfp8_marlin_process_scales(marlin_permute_scales(scales, padded_k, padded_n, MXFP8_GROUP_SIZE))
+
+
+def prepare_mxfp8_layer_for_marlin(layer) -> None:
+    """marlin_utils_fp8.py:437-496.  The layer holds `weight` (N, K) fp8,
+    `weight_scale` (N, K/32) exponent bytes, `output_size_per_partition`,
+    `input_size_per_partition`, optionally `bias`."""
+    part_n, part_k = layer.output_size_per_partition, layer.input_size_per_partition
+    padded_n, padded_k = marlin_padded_nk(part_n, part_k, MXFP8_GROUP_SIZE)
+    device = layer.weight.device
+    layer.workspace = marlin_make_workspace_new(device)
+    perm = torch.empty(0, dtype=torch.int, device=device)
+    qweight = pack_fp8_to_int32(layer.weight, size_k_first=False).T.contiguous()
+    qweight = marlin_pad_qweight(qweight, part_n, part_k, padded_n, padded_k)
+    _set(layer, "weight", ops.gptq_marlin_repack(qweight, perm, padded_k, padded_n, 8))
+    _set(layer, "weight_scale", _mx_scales_for_marlin(layer.weight_scale.data, part_n, part_k, padded_n, padded_k,
+                                                      torch.bfloat16))
+    if getattr(layer, "bias", None) is not None:
+        assert layer.bias.shape == (part_n,)
+        _set(layer, "bias", marlin_permute_bias(marlin_pad_dim(layer.bias, part_n, padded_n)))
+
+
+def prepare_mxfp8_moe_layer_for_marlin(layer, w13: torch.Tensor, w2: torch.Tensor, w13_scale: torch.Tensor,
+                                       w2_scale: torch.Tensor):
+    """marlin_utils_fp8.py:499-588.  w13 (E, 2N, K), w2 (E, K, N) fp8; scales
+    (E, 2N, K/32), (E, K, N/32) exponent bytes.  Returns the Marlin weights and
+    scales of fused_marlin_moe; adds `workspace` to the layer."""
+    g = MXFP8_GROUP_SIZE
+    e, k, n = w13.shape[0], w13.shape[2], w2.shape[2]
+    padded_n = marlin_moe_padded_intermediate(n, g)
+    if padded_n != n:   # the code 0 is 0.0: padded weights add nothing, whatever their scales
+        pad = padded_n - n
+        w13 = F.pad(w13.view(torch.uint8).view(e, 2, n, k), (0, 0, 0, pad)).reshape(e, 2 * padded_n, k) \
+            .view(torch.float8_e4m3fn)
+        w13_scale = F.pad(w13_scale.view(e, 2, n, -1), (0, 0, 0, pad)).reshape(e, 2 * padded_n, -1)
+        w2 = F.pad(w2.view(torch.uint8), (0, pad)).view(torch.float8_e4m3fn)
+        w2_scale = F.pad(w2_scale, (0, pad // g))
+        n = padded_n
+    w13_n = w13.shape[1]
+    device = w13.device
+    layer.workspace = marlin_make_workspace_new(device, 4)
+    perm = torch.empty(0, dtype=torch.int, device=device)
+
+    def repack(weight: torch.Tensor, size_n: int, size_k: int) -> torch.Tensor:
+        assert weight.shape == (e, size_n, size_k)
+        return torch.stack([ops.gptq_marlin_repack(pack_fp8_to_int32(weight[i], size_k_first=False).T.contiguous(),
+                                                   perm, size_k, size_n, 8) for i in range(e)])
+
+    def permute(scales: torch.Tensor, size_n: int, size_k: int) -> torch.Tensor:
+        return torch.stack([_mx_scales_for_marlin(scales[i], size_n, size_k, size_n, size_k, torch.bfloat16)
+                            for i in range(e)])
+
+    return repack(w13, w13_n, k), repack(w2, k, n), permute(w13_scale, w13_n, k), permute(w2_scale, k, n)

@@ -714,3 +714,74 @@ def test_prepare_moe_mxfp4_layer_and_fused_marlin_moe(cfg):
     got = gu.host_f32(y)
     max_ref = np.abs(want).max()
     assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)
+
+
+# ---------------------------------------------------------------- MXFP8 weights (float8_e4m3fn, e8m0 block scales)
+def _mxfp8_reference(codes_kn, exps_gn):
+    """Oracle matrix for fp8 codes (K, N) and exponent bytes (K/32, N), bf16."""
+    fused = mo.fp8_fuse_exponent_bias(mo.mx_scale_values(exps_gn), "bf16")
+    return mo.dequantize_fp8(codes_kn, fused, 32, "bf16")
+
+
+@pytest.mark.parametrize("m,k,n", [(3, 512, 384), (40, 384, 320), (16, 4096, 1024)])   # 320 columns: padded inside
+def test_prepare_mxfp8_layer_and_apply(m, k, n):
+    """An MXFP8 checkpoint layer (weight (N, K) fp8, scales (N, K/32) exponent
+    bytes) -> prepare_mxfp8_layer_for_marlin -> apply_mxfp8_marlin_linear (the op
+    takes the float8_e8m0fnu scales), against the oracle on the same bytes."""
+    from sonar_amd import marlin_utils_fp8 as f8
+    rng = np.random.default_rng(k + n + m)
+    codes = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    codes[(codes & 0x7F) == 0x7F] = 0x30
+    e = rng.integers(112, 122, size=(k // 32, n)).astype(np.uint8)
+    w_ref = _mxfp8_reference(codes, e)
+    layer = types.SimpleNamespace(output_size_per_partition=n, input_size_per_partition=k)
+    layer.weight = torch.from_numpy(np.ascontiguousarray(codes.T.astype(np.uint8))).to(gu.DEV).view(torch.float8_e4m3fn)
+    layer.weight_scale = torch.from_numpy(np.ascontiguousarray(e.T)).to(gu.DEV)
+    bias32 = mo.round_to_dtype(rng.standard_normal(n).astype(np.float32), "bf16")
+    layer.bias = gu.dev_bits16(bias32, "bf16")
+    f8.prepare_mxfp8_layer_for_marlin(layer)
+    assert layer.weight_scale.dtype == torch.float8_e8m0fnu
+    x32 = mo.make_activations(4, m, k, "bf16", std=0.5)
+    y = f8.apply_mxfp8_marlin_linear(gu.dev_bits16(x32, "bf16"), layer.weight, layer.weight_scale, layer.workspace,
+                                     n, k, layer.bias)
+    torch.cuda.synchronize()
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y), mo.gemm_reference(x32, w_ref, bias32))
+    assert ok, worst
+    with pytest.raises(RuntimeError, match="bfloat16"):
+        f8.apply_mxfp8_marlin_linear(gu.dev_bits16(x32, "bf16").half(), layer.weight, layer.weight_scale,
+                                     layer.workspace, n, k, None)
+
+
+@pytest.mark.parametrize("cfg", [(5, 4, 2, 256, 128), (70, 4, 2, 256, 256), (9, 4, 2, 256, 96)], ids=str)
+def test_prepare_mxfp8_moe_layer_and_fused_marlin_moe(cfg):
+    """MXFP8 expert weights -> prepare_mxfp8_moe_layer_for_marlin -> fused_marlin_moe,
+    against the per-token reference on the same bytes (the third case pads the
+    intermediate size 96 -> 128)."""
+    from sonar_amd import marlin_utils_fp8 as f8
+    from sonar_amd.fused_moe import fused_marlin_moe
+    from sonar_amd.scalar_type import scalar_types
+    m, e, topk, hidden, inter = cfg
+    rng = np.random.default_rng(hidden + inter + m)
+    layer = types.SimpleNamespace()
+
+    def expert_set(rows, cols):   # checkpoint shape (E, rows = N of the GEMM, cols = K of the GEMM)
+        codes = rng.integers(0, 256, size=(e, rows, cols), dtype=np.int32)
+        codes[(codes & 0x7F) == 0x7F] = 0x30
+        ex = rng.integers(114, 120, size=(e, rows, cols // 32)).astype(np.uint8)
+        ref = [_mxfp8_reference(codes[i].T, np.ascontiguousarray(ex[i].T)) for i in range(e)]
+        weight = torch.from_numpy(codes.astype(np.uint8)).to(gu.DEV).view(torch.float8_e4m3fn)
+        return weight, torch.from_numpy(ex).to(gu.DEV), ref
+
+    w13, s13, ref13 = expert_set(2 * inter, hidden)
+    w2, s2, ref2 = expert_set(hidden, inter)
+    mw13, mw2, ms13, ms2 = f8.prepare_mxfp8_moe_layer_for_marlin(layer, w13, w2, s13, s2)
+    topk_ids, topk_w = _route(m, e, topk, m)
+    x32 = mo.round_to_dtype(0.5 * mo.make_activations(m, m, hidden, "bf16"), "bf16")
+    y = fused_marlin_moe(gu.dev_bits16(x32, "bf16"), mw13, mw2, None, None, ms13, ms2,
+                         torch.from_numpy(topk_w).to(gu.DEV), torch.from_numpy(topk_ids).to(gu.DEV),
+                         scalar_types.float8_e4m3fn.id)
+    torch.cuda.synchronize()
+    want = _moe_reference(x32, ref13, ref2, topk_ids, topk_w, "bf16")
+    got = gu.host_f32(y)
+    max_ref = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)

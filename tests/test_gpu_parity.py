@@ -419,6 +419,8 @@ FP8_CASES = [
     (100, 1024, 512, 128, False),
     (300, 512, 192, -1, True),
     (1, 4096, 4096, 128, False),
+    (16, 1024, 256, 32, False),       # groups of 32 rows: MXFP8
+    (100, 512, 192, 32, True),
 ]
 
 

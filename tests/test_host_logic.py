@@ -511,6 +511,8 @@ def test_mxfp4_host_helpers():
     assert np.array_equal(out.view(torch.uint8).numpy(), mo.mxfp4_process_scales(e.numpy()))
     with pytest.raises(NotImplementedError):
         f4.mxfp4_marlin_process_scales(s, input_dtype=torch.float8_e4m3fn)
+    from sonar_amd import marlin_utils_fp8 as f8   # MXFP8: the same reorder (marlin_utils_fp8.py:381-386)
+    assert torch.equal(f8.mxfp8_marlin_process_scales(s).view(torch.uint8), out.view(torch.uint8))
     assert mu.check_marlin_supported(st.float4_e2m1f, 32)
     assert not mu.check_marlin_supported(st.float4_e2m1f, 32, has_zp=True)
     assert f4.is_fp4_marlin_supported()
