@@ -171,7 +171,8 @@ __device__ __forceinline__ void load_cols(typename D::Col (&cols)[4], const uint
 // subnormal codes become fp16 subnormals).  The scales are powers of two held
 // in the activation type (the MX block scales, 2^(e - 127)); value * scale is
 // exact, so the one conversion rounds nothing.  Same interface and row order
-// as Dq: word() returns rows 0..7 of the column.
+// as Dq: word() returns rows 0..7 of the column.  (This generic form is the
+// arithmetic the bf16 specialisation below must reproduce; only bf16 is launched.)
 template <typename T>
 struct DqF4 {
   typedef typename Dq<T>::vec8 vec8;
@@ -189,6 +190,34 @@ struct DqF4 {
   static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c, uint32_t) {
     // rows 0,1 are nibbles 0,4; rows 2,3 nibbles 1,5; rows 4,5 nibbles 2,6; rows 6,7 nibbles 3,7
     return __builtin_bit_cast(vec8, u32x4_t{pair(q << 12, c.s), pair(q << 8, c.s), pair(q << 4, c.s), pair(q, c.s)});
+  }
+};
+
+// bf16: the matrix-core generation this is written for converts two 4-bit
+// floats of a byte to bf16 and applies a power-of-two scale in one instruction
+// (v_cvt_scalef32_pk_bf16_fp4: low nibble to the low half; only the exponent of
+// the scale operand counts, and the MX block scales are powers of two).  Byte b
+// of a word holds nibble slots 2b, 2b + 1, i.e. rows (0,2), (4,6), (1,3), (5,7);
+// four byte permutes put the rows in order.
+template <>
+struct DqF4<__bf16> {
+  typedef Dq<__bf16>::vec8 vec8;
+  struct Col {
+    float s;   // the block scale, a power of two
+  };
+  static __device__ __forceinline__ Col make_col(uint16_t scale_bits, int) {
+    return Col{Dq<__bf16>::to_float(scale_bits)};
+  }
+  static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c, uint32_t) {
+    const uint32_t r02 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, c.s, 0));
+    const uint32_t r46 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, c.s, 1));
+    const uint32_t r13 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, c.s, 2));
+    const uint32_t r57 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, c.s, 3));
+    // __builtin_amdgcn_perm(a, b, sel): bytes 0-3 of the selector space are b, 4-7 are a
+    return __builtin_bit_cast(vec8, u32x4_t{__builtin_amdgcn_perm(r13, r02, 0x05040100u),
+                                            __builtin_amdgcn_perm(r13, r02, 0x07060302u),
+                                            __builtin_amdgcn_perm(r57, r46, 0x05040100u),
+                                            __builtin_amdgcn_perm(r57, r46, 0x07060302u)});
   }
 };
 
