@@ -232,10 +232,28 @@ def moe_sweep(torch, gen, time_graph):
         def layer(i=0):
             fused_moe.fused_marlin_moe(x, w1, w2, None, None, s1, s2, tw, ti, scalar_types.uint4b8.id)
 
+        # the same codes read as MXFP4 (float4_e2m1f, an exponent byte per 32 rows)
+        e1 = torch.randint(110, 120, (e, hidden // 32, 2 * inter), dtype=torch.uint8, device=dev, generator=gen)
+        e2 = torch.randint(110, 120, (e, inter // 32, hidden), dtype=torch.uint8, device=dev, generator=gen)
+        e1, e2 = e1.view(torch.float8_e8m0fnu), e2.view(torch.float8_e8m0fnu)
+
+        def gemm1_mx(i=0):
+            ops.moe_wna16_marlin_gemm(x, h1, w1, None, e1, None, None, None, None, None, ws, sorted_ids,
+                                      expert_ids, past, tw, bs, topk, False, scalar_types.float4_e2m1f, t, 2 * inter,
+                                      hidden, True, False, True, False)
+
+        def gemm2_mx(i=0):
+            ops.moe_wna16_marlin_gemm(h2, y, w2, None, e2, None, None, None, None, None, ws, sorted_ids,
+                                      expert_ids, past, tw, bs, 1, True, scalar_types.float4_e2m1f, t * topk, hidden,
+                                      inter, True, False, True, False)
+
         reps = 8 if t == 16 else 2
-        for name, fn, k, n, rows in (("gate_up", gemm1, hidden, 2 * inter, t), ("down", gemm2, inter, hidden, t * topk)):
+        cases = [("gate_up", gemm1, hidden, 2 * inter, t, GROUP, 2), ("down", gemm2, inter, hidden, t * topk, GROUP, 2),
+                 ("gate_up (mxfp4)", gemm1_mx, hidden, 2 * inter, t, 32, 1),
+                 ("down (mxfp4)", gemm2_mx, inter, hidden, t * topk, 32, 1)]
+        for name, fn, k, n, rows, group, scale_bytes in cases:
             s = time_graph(torch, fn, reps)
-            weights = routed * (k * n // 2 + (k // GROUP) * n * 2)
+            weights = routed * (k * n // 2 + (k // group) * n * scale_bytes)
             nb = weights + rows * k * 2 + t * topk * n * 2 + sorted_ids.numel() * 4 + expert_ids.numel() * 4
             fl = 2 * t * topk * n * k
             out.append({"tokens": t, "gemm": name, "block_size": bs, "experts_routed": routed,

@@ -29,7 +29,7 @@ namespace sonar {
 int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
               const void* scales, const uint32_t* zeros, const int32_t* perm, int dtype, int64_t size_m,
               int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
-              size_t partial_bytes, hipStream_t st);
+              size_t partial_bytes, bool fp4, hipStream_t st);
 bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size);
 
 namespace {
@@ -1609,7 +1609,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   const bool async_tile = tile_async_applies(chk.has_perm, num_groups, chk.group_size);
   const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
   // the row -> group lookup and 8-bit codes exist in the streaming kernels only
-  const bool use_tile = plan.tile && !no_tile && !chk.row_groups && chk.bits == 4 && !chk.fp4 &&
+  // (MXFP4 only through the asynchronous tile kernel: the older one has no float4 dequantiser)
+  const bool use_tile = plan.tile && !no_tile && !chk.row_groups && chk.bits == 4 && (!chk.fp4 || async_tile) &&
                         !(slab_fast && p.unit_chunks == 4);
   // More than 64 rows in the general kernels (8-bit codes, is_k_full = false,
   // the tile path switched off) on a matrix of short strips: one workgroup per
@@ -1633,7 +1634,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
     const size_t used = stream_scratch_bytes();
     return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
                      size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used,
-                     scratch_bytes > used ? scratch_bytes - used : 0, st);
+                     scratch_bytes > used ? scratch_bytes - used : 0, chk.fp4, st);
   }
 
   for (int64_t m0 = 0; m0 < size_m; m0 += 64) {

@@ -313,10 +313,11 @@ constexpr int kAsyncA = kAsyncStages * kStageA;
 constexpr int async_lds(bool g32) { return kAsyncA + kTileWaves * kAsyncStages * wave_stage(g32); }
 constexpr int async_copies(bool g32) { return g32 ? 8 : 7; }
 
-template <typename T, bool HAS_ZP, bool GROUPED, bool G32 = false>
+template <typename T, bool HAS_ZP, bool GROUPED, bool G32 = false, bool FP4 = false>
 __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq<T>::Col Col;
+  typedef typename Dq4Of<T, FP4>::type D4;   // integer codes, or float4_e2m1f (MXFP4: with G32)
+  typedef typename D4::Col Col;
   constexpr int kWaveStage = wave_stage(G32);
   constexpr int kAsyncCopies = async_copies(G32);
   extern __shared__ __attribute__((aligned(1024))) char smem[];
@@ -502,13 +503,13 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
       for (int j = 0; j < 4; ++j) {
         int z = 8;
         if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
-        cols[j] = Dq<T>::make_col((uint16_t)sbits[j], z);
+        cols[j] = D4::make_col((uint16_t)sbits[j], z);
       }
     }
-    wv[0] = __builtin_bit_cast(u32x4_t, Dq<T>::word(qraw.x, cols[0], magic));
-    wv[1] = __builtin_bit_cast(u32x4_t, Dq<T>::word(qraw.y, cols[1], magic));
-    wv[2] = __builtin_bit_cast(u32x4_t, Dq<T>::word(qraw.z, cols[2], magic));
-    wv[3] = __builtin_bit_cast(u32x4_t, Dq<T>::word(qraw.w, cols[3], magic));
+    wv[0] = __builtin_bit_cast(u32x4_t, D4::word(qraw.x, cols[0], magic));
+    wv[1] = __builtin_bit_cast(u32x4_t, D4::word(qraw.y, cols[1], magic));
+    wv[2] = __builtin_bit_cast(u32x4_t, D4::word(qraw.z, cols[2], magic));
+    wv[3] = __builtin_bit_cast(u32x4_t, D4::word(qraw.w, cols[3], magic));
     SONAR_TILE_LANDED();
   };
   // Multiply phase: 32 MFMAs, ahead of the other wavefront's VALU work in the issue order.
@@ -713,6 +714,29 @@ int launch_tile_async_groups(const TileParams& p, hipStream_t st) {
   return SONAR_OK;
 }
 
+// MXFP4: bf16, groups of 32 rows, float4_e2m1f codes
+int launch_tile_async_fp4(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<__bf16, false, false, true, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, async_lds(true)));
+    attr_set = true;
+  }
+  marlin_tile_async_kernel<__bf16, false, false, true, true><<<tile_grid(p), kTileWaves * 64, async_lds(true), st>>>(p);
+  return SONAR_OK;
+}
+
+int launch_tile_grouped_fp4(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<__bf16, false, true, true, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, async_lds(true)));
+    attr_set = true;
+  }
+  marlin_tile_async_kernel<__bf16, false, true, true, true><<<tile_grid(p), kTileWaves * 64, async_lds(true), st>>>(p);
+  return SONAR_OK;
+}
+
 template <typename T, bool HAS_ZP>
 int launch_tile_async(const TileParams& p, hipStream_t st) {
   return (p.num_groups > 1 && p.group_size == 32) ? launch_tile_async_groups<T, HAS_ZP, true>(p, st)
@@ -762,7 +786,7 @@ bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size) {
 int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
               const void* scales, const uint32_t* zeros, const int32_t* perm, int dtype, int64_t size_m,
               int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
-              size_t partial_bytes, hipStream_t st) {
+              size_t partial_bytes, bool fp4, hipStream_t st) {
   TileParams p;
   p.a = static_cast<const uint16_t*>(a);
   p.lda = a_row_stride;
@@ -793,7 +817,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   const bool zp = zeros != nullptr, pm = perm != nullptr;
   int rc;
   static const bool no_async = getenv("SONAR_MARLIN_NO_ASYNC_TILE") != nullptr;  // debugging aid
-  if (tile_async_applies(pm, num_groups, group_size) && !no_async) {
+  if (tile_async_applies(pm, num_groups, group_size) && (!no_async || fp4)) {   // float4 codes exist here only
     const GemmPlan plan = plan_gemm(size_m, size_n, size_k, true);
     if (plan.k_splits > 1 && partial != nullptr && partial_bytes >= plan_partial_bytes(plan, size_m, size_n)) {
       p.k_splits = plan.k_splits;
@@ -809,7 +833,9 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
         if (p.k_splits == 1) p.partial = nullptr;
       }
     }
-    if (dtype == SONAR_DTYPE_F16)
+    if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
+      rc = launch_tile_async_fp4(p, st);
+    else if (dtype == SONAR_DTYPE_F16)
       rc = zp ? launch_tile_async<_Float16, true>(p, st) : launch_tile_async<_Float16, false>(p, st);
     else
       rc = zp ? launch_tile_async<__bf16, true>(p, st) : launch_tile_async<__bf16, false>(p, st);
@@ -849,7 +875,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
                   int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, int a_by_slot, hipStream_t st) {
+                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, hipStream_t st) {
   const int max_tiles = moe_tile_max(sorted_len, num_experts);
   const int blocks_max = (int)((sorted_len + 63) / 64);
   moe_tile_table_kernel<<<1, 256, (size_t)blocks_max * sizeof(int32_t), st>>>(expert_ids, num_post_pad, blocks_max, 64,
@@ -889,7 +915,9 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.expert_z_stride = (long)(num_groups * (size_n / 8));
   p.expert_bias_stride = (long)size_n;
   int rc;
-  if (dtype == SONAR_DTYPE_F16)
+  if (fp4)
+    rc = launch_tile_grouped_fp4(p, st);
+  else if (dtype == SONAR_DTYPE_F16)
     rc = zeros ? launch_tile_grouped<_Float16, true>(p, st) : launch_tile_grouped<_Float16, false>(p, st);
   else
     rc = zeros ? launch_tile_grouped<__bf16, true>(p, st) : launch_tile_grouped<__bf16, false>(p, st);

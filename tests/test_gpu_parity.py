@@ -507,6 +507,8 @@ MXFP4_CASES = [
     (100, 1024, 512, False),
     (300, 512, 192, True),
     (1, 2880, 5760, False),     # gpt-oss expert shape: K is 90 groups of 32 rows
+    (1024, 2880, 5760, True),   # the same through the tile kernel (K = 45 steps of 64 rows)
+    (4096, 4096, 1024, False),  # tile kernel, several rounds of tiles
 ]
 
 
