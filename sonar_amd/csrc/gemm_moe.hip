@@ -32,7 +32,7 @@ int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t moe_block_size, int64_t top_k,
                   int mul_topk, int64_t num_experts, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, int a_by_slot, hipStream_t st);
+                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, hipStream_t st);
 
 namespace {
 
@@ -632,12 +632,12 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                 "act-order with 8-bit expert weights needs sorted_len * size_k * 2 more scratch bytes "
                 "(the column-permuted copy of A per slot)");
   // Few rows per expert: the decode kernel, one workgroup per strip and 32 slots of a block
-  if (!bits8 && !fp4 && !row_groups &&
+  if (!bits8 && !row_groups &&
       moe_fast_applies(has_perm, moe_block_size, sorted_len, num_experts, a_rows, size_n, size_k, num_groups,
                        group_size))
     return moe_fast_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
                          num_tokens_past_padded, topk_weights, moe_block_size, top_k, mul_topk_weights ? 1 : 0,
-                         num_experts, dtype, size_m, size_n, size_k, num_groups, group_size, a_by_slot, st);
+                         num_experts, dtype, size_m, size_n, size_k, num_groups, group_size, a_by_slot, fp4, st);
   static const bool no_tile = getenv("SONAR_MARLIN_NO_MOE_TILE") != nullptr;  // debugging aid
   // Full blocks of 64 slots mean many rows per expert: the MFMA-tiled kernel
   if (moe_block_size == 64 && !has_perm && !bits8 && !row_groups && !no_tile && size_k % 64 == 0 &&

@@ -746,7 +746,9 @@ __device__ __forceinline__ u32x4_t raw_operand(uint32_t q, uint32_t magic) {
 // call; the rows of A are gathered and the rows of C scattered through
 // sorted_ids, everything else is the dense kernel on the expert's matrices.
 // GPU: groups per 128-row unit (2 or 4 for groups of 64 or 32 rows, else 1).
-template <typename T, bool HAS_ZP, int kFastWaves, int MB, bool GROUPED = false, int GPU = 1>
+// FP4 (with GPU = 4, no zero points): float4_e2m1f codes; the operands are the
+// converted values themselves, so only the scale is left for after the unit.
+template <typename T, bool HAS_ZP, int kFastWaves, int MB, bool GROUPED = false, int GPU = 1, bool FP4 = false>
 __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams params,
                                                                              const int unit_group_shift) {
   typedef typename Dq<T>::vec8 vec8;
@@ -996,15 +998,19 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
         const uint32_t words[4] = {qs[cc].x, qs[cc].y, qs[cc].z, qs[cc].w};
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-          const vec8 wv = __builtin_bit_cast(vec8, raw_operand(words[j], magic));
+          vec8 wv;
+          if constexpr (FP4) wv = DqF4<T>::word(words[j], typename DqF4<T>::Col{1.0f}, magic);
+          else wv = __builtin_bit_cast(vec8, raw_operand(words[j], magic));
 #pragma unroll
           for (int mb = 0; mb < MB; ++mb)
             part_sum[mb][j] = Dq<T>::mfma(wv, __builtin_bit_cast(vec8, as[mb][cc]), cg == 0 ? zero4 : part_sum[mb][j]);
         }
+        if constexpr (!FP4) {
 #pragma unroll
-        for (int mb = 0; mb < MB; ++mb)
-          asum[mb] = Dq<T>::mfma(__builtin_bit_cast(vec8, ones), __builtin_bit_cast(vec8, as[mb][cc]),
-                                 cg == 0 ? zero4 : asum[mb]);
+          for (int mb = 0; mb < MB; ++mb)
+            asum[mb] = Dq<T>::mfma(__builtin_bit_cast(vec8, ones), __builtin_bit_cast(vec8, as[mb][cc]),
+                                   cg == 0 ? zero4 : asum[mb]);
+        }
       }
       // scale and offset of this group (the whole unit when GPU == 1)
       const u32x4_t gz = gi == 0 ? row_z : more_z[gi == 0 ? 0 : gi - 1];
@@ -1018,8 +1024,10 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
           float off = -(RawOperand<T>::kBase + 8.f);
           if (HAS_ZP) off = -RawOperand<T>::kBase - (float)((zrow[r] >> (4 * j)) & 0xFu);
 #pragma unroll
-          for (int mb = 0; mb < MB; ++mb)
-            acc[mb][j][r] = __builtin_fmaf(sc, __builtin_fmaf(off, asum[mb][r], part_sum[mb][j][r]), acc[mb][j][r]);
+          for (int mb = 0; mb < MB; ++mb) {
+            if constexpr (FP4) acc[mb][j][r] = __builtin_fmaf(sc, part_sum[mb][j][r], acc[mb][j][r]);
+            else acc[mb][j][r] = __builtin_fmaf(sc, __builtin_fmaf(off, asum[mb][r], part_sum[mb][j][r]), acc[mb][j][r]);
+          }
         }
     }
     cur.advance(kFastWaves, p.units_per_strip);
@@ -1282,6 +1290,26 @@ int launch_fast_waves(const StreamParams& p, int unit_group_shift, hipStream_t s
   return launch_fast_groups<T, HAS_ZP, WAVES, MB, GROUPED, 1>(p, unit_group_shift, st);
 }
 
+// MXFP4: bf16, four groups of 32 rows per unit, one block of 16 rows per workgroup
+template <int WAVES, bool GROUPED>
+int launch_fast_fp4_waves(const StreamParams& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_stream_fast_kernel<__bf16, false, WAVES, 1, GROUPED, 4, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds_bytes(WAVES, 1, 4)));
+    attr_set = true;
+  }
+  const int lds = p.sum_over_rings ? WAVES * wave_lds(1, 4) : fast_lds_bytes(WAVES, 1, 4);
+  marlin_stream_fast_kernel<__bf16, false, WAVES, 1, GROUPED, 4, true>
+      <<<p.grid_parts * p.slabs, WAVES * 64, lds, st>>>(p, -4);
+  return SONAR_OK;
+}
+
+template <bool GROUPED>
+int launch_fast_fp4(const StreamParams& p, bool half_workgroups, hipStream_t st) {
+  return half_workgroups ? launch_fast_fp4_waves<4, GROUPED>(p, st) : launch_fast_fp4_waves<8, GROUPED>(p, st);
+}
+
 // `row_blocks`: blocks of 16 rows per workgroup (1 or 2).
 template <typename T, bool HAS_ZP, bool GROUPED = false>
 int launch_fast(const StreamParams& p, int unit_group_shift, bool half_workgroups, int row_blocks, hipStream_t st) {
@@ -1427,7 +1455,7 @@ int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t moe_block_size, int64_t top_k,
                   int mul_topk, int64_t num_experts, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, int a_by_slot, hipStream_t st) {
+                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, hipStream_t st) {
   StreamParams p = {};
   p.a_by_slot = a_by_slot;
   p.a = static_cast<const uint16_t*>(a);
@@ -1473,7 +1501,9 @@ int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   const bool half = (int64_t)p.slabs * n_strips > cu_count();   // small workgroups, three per compute unit
   const int row_blocks = moe_block_size <= 16 ? 1 : 2;
   int rc;
-  if (dtype == SONAR_DTYPE_F16)
+  if (fp4)   // bf16, groups of 32 rows, blocks of at most 16 slots: moe_fast_applies has seen to it
+    rc = launch_fast_fp4<true>(p, half, st);
+  else if (dtype == SONAR_DTYPE_F16)
     rc = zeros ? launch_fast<_Float16, true, true>(p, unit_group_shift, half, row_blocks, st)
                : launch_fast<_Float16, false, true>(p, unit_group_shift, half, row_blocks, st);
   else
@@ -1568,7 +1598,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   int unit_group_shift;
   const bool fast_groups = fast_group_shift(num_groups, chk.group_size, unit_group_shift);
   static const bool no_fast = getenv("SONAR_MARLIN_NO_FAST") != nullptr;  // debugging aid
-  const bool fast_shape = !no_fast && chk.bits == 4 && !chk.fp4 && !chk.has_perm && !chk.row_groups &&
+  const bool fast_shape = !no_fast && chk.bits == 4 && !chk.has_perm && !chk.row_groups &&
                           p.chunks_per_strip % 4 == 0 && fast_groups &&
                           size_m * a_row_stride * 2 < (1LL << 31);
   // Short strips (K <= 4096) on a matrix with at least 64 of them: one workgroup
@@ -1661,7 +1691,9 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
       static const bool no_half = getenv("SONAR_MARLIN_NO_HALF_WG") != nullptr;  // debugging aid
       const bool half = !no_half && p.parts * p.slabs > cus;
       p.sum_over_rings = half && (int64_t)p.parts == n_strips && p.parts * p.slabs > 2 * cus;
-      if (dtype == SONAR_DTYPE_F16)
+      if (chk.fp4)   // groups of 32 rows: never in blocks of rows (slab_fast is off), so one block of 16 rows
+        rc = launch_fast_fp4<false>(p, half, st);
+      else if (dtype == SONAR_DTYPE_F16)
         rc = chk.has_zp ? launch_fast<_Float16, true>(p, unit_group_shift, half, row_blocks, st)
                         : launch_fast<_Float16, false>(p, unit_group_shift, half, row_blocks, st);
       else
