@@ -158,8 +158,9 @@ int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
  * dtype(topk_weights[id]) when mul_topk_weights != 0.
  *   a            dtype[M][K] contiguous
  *   c            dtype[M*top_k][N] contiguous
- *   b_q_weight   num_experts * K*N/8 words (K*N/4 for uint8b128), each expert
- *                in b_layout order; b_type_id uint4b8, uint4, uint8b128 or float8_e4m3fn
+ *   b_q_weight   num_experts * K*N/8 words (K*N/4 for the 8-bit types), each expert
+ *                in b_layout order; b_type_id uint4b8, uint4, uint8b128, float8_e4m3fn
+ *                or float4_e2m1f (scales as described at the type ids)
  *   b_scales     dtype[num_experts][num_groups][N]; b_zeros / b_bias likewise
  *   scratch      sonar_moe_marlin_gemm_scratch_bytes(); act-order calls run 4 to
  *                20 times faster with sorted_len * K * 2 bytes more behind that
