@@ -92,6 +92,23 @@ def main():
                                                       .astype(np.float32), dtype), dtype)
         np.savez_compressed(os.path.join(HERE, f"dequant_table_{dtype}.npz"),
                             scales_bits=mo.to_bits16(scales, dtype), table_bits=table)
+    # floating-point weight types: every fp8 code (rows) under 64 channel scales with the exponent bias
+    # folded in, and every fp4 code under power-of-two block scales (MXFP4, one exponent byte per 32 rows)
+    for dtype in ("fp16", "bf16"):
+        scales = mo.round_to_dtype(np.concatenate([rng.uniform(1e-4, 1e-2, 60), [1.0, 0.333, 6.1e-5, 2.0 ** -9]])
+                                   .astype(np.float32), dtype)
+        fused = mo.fp8_fuse_exponent_bias(scales[None, :], dtype)
+        codes = np.arange(256, dtype=np.int32)[:, None].repeat(64, 1)
+        np.savez_compressed(os.path.join(HERE, f"fp8_dequant_table_{dtype}.npz"), codes=codes.astype(np.uint8),
+                            fused_scales_bits=mo.to_bits16(fused, dtype),
+                            dequant_bits=mo.to_bits16(mo.dequantize_fp8(codes, fused, -1, dtype), dtype))
+    codes4 = rng.integers(0, 16, size=(128, 64), dtype=np.int32)
+    codes4[:16, :] = np.arange(16)[:, None]
+    exps = rng.integers(90, 140, size=(4, 64)).astype(np.uint8)
+    exps[0, :4] = [0, 1, 127, 250]
+    np.savez_compressed(os.path.join(HERE, "mxfp4_dequant_k128_n64.npz"), codes=codes4.astype(np.uint8),
+                        exponent_bytes=exps, gptq_packed=mo.gptq_pack(codes4),
+                        dequant_bits=mo.to_bits16(mo.dequantize_mxfp4(codes4, exps), "bf16"))
     for f in sorted(os.listdir(HERE)):
         if f.endswith(".npz"):
             print(f, os.path.getsize(os.path.join(HERE, f)))

@@ -159,3 +159,53 @@ def test_hip_kernels_reproduce_8bit_fixture():
                                      1, 0, 1, gu.stream()))
     ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(c), f["c_ref"])
     assert ok, worst
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_oracle_reproduces_fp8_and_mxfp4_tables(dtype):
+    t = load(f"fp8_dequant_table_{dtype}.npz")
+    fused = mo.from_bits16(t["fused_scales_bits"], dtype)
+    w = mo.dequantize_fp8(t["codes"].astype(np.int32), fused, -1, dtype)
+    assert np.array_equal(mo.to_bits16(w, dtype), t["dequant_bits"])
+    if dtype == "bf16":
+        f = load("mxfp4_dequant_k128_n64.npz")
+        codes = f["codes"].astype(np.int32)
+        assert np.array_equal(mo.gptq_pack(codes), f["gptq_packed"])
+        assert np.array_equal(mo.to_bits16(mo.dequantize_mxfp4(codes, f["exponent_bytes"]), "bf16"), f["dequant_bits"])
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_hip_kernels_reproduce_fp8_and_mxfp4_tables(dtype):
+    """In-kernel dequantised values of the floating-point weight types, bit for
+    bit: all 256 fp8 codes under 64 channel scales; MXFP4 codes under block
+    scales that include the exponent bytes 0, 1 and 250."""
+    import torch
+
+    from sonar_amd import _lib
+    from tests import gpu_util as gu
+    lib = _lib.load()
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    t = load(f"fp8_dequant_table_{dtype}.npz")
+    k, n = t["codes"].shape
+    marlin = torch.empty((k // 16, 4 * n), dtype=torch.int32, device=gu.DEV)
+    _lib.check(lib.sonar_gptq_marlin_repack(gu.ptr(gu.dev_i32(mo.pack_rows8(t["codes"].astype(np.int32)))), None,
+                                            gu.ptr(marlin), k, n, 8, gu.stream()))
+    native = torch.empty_like(marlin)
+    _lib.check(lib.sonar_marlin8_to_gfx950(gu.ptr(marlin), gu.ptr(native), k, n, gu.stream()))
+    fused = mo.from_bits16(t["fused_scales_bits"], dtype)
+    scales = gu.dev_bits16(mo.marlin_permute_scales(fused, k, n, -1), dtype)
+    w = torch.empty((k, n), dtype=tdt, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_dequant(gu.ptr(native), _lib.LAYOUT_GFX950, gu.ptr(scales), None, None, gu.ptr(w),
+                                        gu.dtype_code(dtype), _lib.TYPE_FLOAT8_E4M3FN, n, k, 1, 1, gu.stream()))
+    assert np.array_equal(w.view(torch.int16).cpu().numpy().view(np.uint16), t["dequant_bits"])
+    if dtype != "bf16":
+        return
+    f = load("mxfp4_dequant_k128_n64.npz")
+    k, n = f["codes"].shape
+    native = gu.to_gfx950(gu.gptq_repack(gu.dev_i32(f["gptq_packed"]), None, k, n), k, n)
+    scales = gu.dev_bits16(mo.marlin_permute_scales(mo.mx_scale_values(f["exponent_bytes"]), k, n, 32), "bf16")
+    w = torch.empty((k, n), dtype=torch.bfloat16, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_dequant(gu.ptr(native), _lib.LAYOUT_GFX950, gu.ptr(scales), None, None, gu.ptr(w),
+                                        gu.dtype_code("bf16"), _lib.TYPE_FLOAT4_E2M1F, n, k, k // 32, 1, gu.stream()))
+    assert np.array_equal(w.view(torch.int16).cpu().numpy().view(np.uint16), f["dequant_bits"])
