@@ -41,6 +41,30 @@ def dense() -> None:
             sys.exit(1)
 
 
+def dense_mxfp4() -> None:
+    """float4_e2m1f weights take the decode, the general and the tile kernel; every
+    switch must leave them on a kernel that has the float4 dequantiser."""
+    from sonar_amd import _lib
+    from tests import test_gpu_parity as tp
+    lib = _lib.load()
+    for (m, k, n) in [(16, 1024, 4096), (48, 1024, 512), (300, 1024, 768)]:
+        L = tp._layer_mxfp4(gu, 9 + m, k, n)
+        a32 = mo.make_activations(m + 1, m, k, "bf16", std=0.5)
+        a = gu.dev_bits16(a32, "bf16")
+        c = torch.empty((m, n), dtype=torch.bfloat16, device=gu.DEV)
+        ws = torch.zeros(torch.cuda.get_device_properties(0).multi_processor_count, dtype=torch.int32, device=gu.DEV)
+        scratch = torch.empty(max(lib.sonar_marlin_gemm_scratch_bytes(m, n, k), 16), dtype=torch.uint8, device=gu.DEV)
+        _lib.check(lib.sonar_marlin_gemm(
+            gu.ptr(a), k, gu.ptr(c), gu.ptr(L["native"]), _lib.LAYOUT_GFX950, None, gu.ptr(L["scales"]), None, None,
+            None, gu.ptr(ws), ws.numel(), gu.ptr(scratch), scratch.numel(), gu.dtype_code("bf16"),
+            _lib.TYPE_FLOAT4_E2M1F, m, n, k, L["groups"], 1, 0, 1, gu.stream()))
+        torch.cuda.synchronize()
+        ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), mo.gemm_reference(a32, L["w_ref"]))
+        print("mxfp4", m, k, n, "ok" if ok else f"FAILED max_err={max_err} max_ref={max_ref}", flush=True)
+        if not ok:
+            sys.exit(1)
+
+
 def grouped() -> None:
     from tests import test_gpu_moe as tm
     for case in [(300, 4, 2, 256, 256, 128, "fp16", False, False, False, 64, True),
@@ -55,5 +79,6 @@ def grouped() -> None:
 
 if __name__ == "__main__":
     dense()
+    dense_mxfp4()
     grouped()
     print("all paths ok", flush=True)
