@@ -3,7 +3,8 @@ and the two grouped W4A16 GEMMs around the gated activation.
 
 Mirrors aphrodite/model_executor/layers/fused_moe/moe_align_block_size.py:11-101
 (`moe_align_block_size`) and .../fused_moe/experts/marlin_moe.py:57-392
-(`fused_marlin_moe`) for 4-bit integer weights with fp16 / bf16 activations.
+(`fused_marlin_moe`) for 4- and 8-bit integer, fp8 and MXFP4 weights with fp16 / bf16
+activations.
 On the GPU the routing, the activation and the final sum are the HIP kernels
 behind `torch.ops.sonar_amd.{moe_align_block_size, silu_and_mul, moe_sum}`; the
 torch expressions kept here serve CPU tensors (and the tests of those kernels).
