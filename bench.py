@@ -137,17 +137,17 @@ def variants_sweep(torch, ops, gen, time_graph):
     """K = 4096, N = 11008 at M = 1 and 512: act-order (perm gathers the columns
     of A, weights repacked in sorted-group order), AWQ (per-group zero points),
     8-bit weights (uint8b128), fp8 weights (float8_e4m3fn, scales with the
-    exponent bias folded in) and MXFP4 weights (float4_e2m1f, exponent-byte
-    scales per 32 rows, bf16 activations)."""
+    exponent bias folded in), MXFP8 and MXFP4 weights (float8_e4m3fn /
+    float4_e2m1f, exponent-byte scales per 32 rows, bf16 activations)."""
     from sonar_amd import marlin_utils
     from sonar_amd.scalar_type import scalar_types
     dev = "cuda:0"
     k, n = 4096, 11008
     out = []
-    for name in ("act_order", "awq", "w8a16", "fp8", "mxfp4"):
+    for name in ("act_order", "awq", "w8a16", "fp8", "mxfp8", "mxfp4"):
         layers = []
-        words = 4 * n if name in ("w8a16", "fp8") else 2 * n     # 8-bit codes: four per word
-        act_dtype = torch.bfloat16 if name == "mxfp4" else torch.float16
+        words = 4 * n if name in ("w8a16", "fp8", "mxfp8") else 2 * n     # 8-bit codes: four per word
+        act_dtype = torch.bfloat16 if name in ("mxfp4", "mxfp8") else torch.float16
         for _ in range(6):
             qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, words), dtype=torch.int32, device=dev, generator=gen)
             sc = (torch.rand((k // GROUP, n), device=dev, generator=gen) * 9e-3 + 1e-3).to(torch.float16)
@@ -161,9 +161,10 @@ def variants_sweep(torch, ops, gen, time_graph):
                 layers.append((qw, sc * 0.0625, empty, empty, empty, ws, scalar_types.uint8b128))
             elif name == "fp8":
                 layers.append((qw, sc * 0.0625 * 256, empty, empty, empty, ws, scalar_types.float8_e4m3fn))
-            elif name == "mxfp4":
+            elif name in ("mxfp4", "mxfp8"):
                 e8 = torch.randint(110, 120, (k // 32, n), dtype=torch.uint8, device=dev, generator=gen)
-                layers.append((qw, e8.view(torch.float8_e8m0fnu), empty, empty, empty, ws, scalar_types.float4_e2m1f))
+                wt = scalar_types.float4_e2m1f if name == "mxfp4" else scalar_types.float8_e4m3fn
+                layers.append((qw, e8.view(torch.float8_e8m0fnu), empty, empty, empty, ws, wt))
             else:
                 zp = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // GROUP, n // 8), dtype=torch.int32, device=dev,
                                    generator=gen)
@@ -177,9 +178,9 @@ def variants_sweep(torch, ops, gen, time_graph):
                                 False, True, False)
             s = time_graph(torch, one, 24 if m == 1 else 6)
             nb = algorithmic_bytes(m, k, n, zeros=name == "awq", act_order=name == "act_order")
-            if name in ("w8a16", "fp8"):
+            if name in ("w8a16", "fp8", "mxfp8"):
                 nb += k * n // 2                        # a byte per weight instead of half
-            if name == "mxfp4":
+            if name in ("mxfp4", "mxfp8"):
                 nb += (k // 32 - 2 * (k // GROUP)) * n  # a byte per 32 rows instead of two per 128
             fl = 2 * m * k * n
             out.append({"variant": name, "m": m, "k": k, "n": n, "us": round(s * 1e6, 2),

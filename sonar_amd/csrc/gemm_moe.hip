@@ -275,16 +275,18 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
 // blocks of 16 rows.  No gather of A: act-order experts come here through the
 // per-slot permuted copy (a_by_slot).  HAS_GIDX: every row finds its scale
 // through g_idx (is_k_full = false).
-template <typename T, int MB>
+template <typename T, int MB, bool CHUNK_SCALES = false>
 struct MoeUnit8 {
   static constexpr int kChunks = MB >= 3 ? 2 : 4;   // two units of this size and the accumulators fit the register file
   uint4 q[kChunks][2];
   typename Dq<T>::vec8 a[kChunks][MB];
   uint32_t sbits[4];
   int group;
+  uint4 sv[CHUNK_SCALES ? kChunks : 1];   // groups of 32 rows: the scales of every chunk
 };
 
-template <typename T, int MB, bool HAS_GIDX, bool FP8>
+// MX: float8 codes with groups of 32 rows (the host launches it for nothing else).
+template <typename T, int MB, bool HAS_GIDX, bool FP8, bool MX = false>
 __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe8_kernel(const MoeParams p) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq8Of<T, FP8>::type D8;
@@ -331,10 +333,10 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe8_kernel(const MoePa
   const bool grouped = p.num_groups > 1;
   const uint32_t magic = magic_register();
 
-  auto load_unit = [&](MoeUnit8<T, MB>& u, int unit) {
+  auto load_unit = [&](MoeUnit8<T, MB, MX>& u, int unit) {
     const int chunk0 = unit * p.unit_chunks;
 #pragma unroll
-    for (int cc = 0; cc < MoeUnit8<T, MB>::kChunks; ++cc)
+    for (int cc = 0; cc < MoeUnit8<T, MB, MX>::kChunks; ++cc)
       if (cc < p.unit_chunks) {
         u.q[cc][0] = bsrc[(long)(chunk0 + cc) * 128];
         u.q[cc][1] = bsrc[(long)(chunk0 + cc) * 128 + 64];
@@ -345,6 +347,13 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe8_kernel(const MoePa
     const int g = grouped ? (chunk0 * kChunkK) / p.group_size : 0;
     u.group = g;
     const uint16_t* srow = scales + (long)g * p.size_n + strip * kStripN;
+    if (MX) {   // group = chunk
+#pragma unroll
+      for (int cc = 0; cc < MoeUnit8<T, MB, MX>::kChunks; ++cc)
+        if (cc < p.unit_chunks)
+          u.sv[MX ? cc : 0] = *reinterpret_cast<const uint4*>(srow + (long)cc * p.size_n + 8 * (col16 & 7));
+      return;
+    }
 #pragma unroll
     for (int j = 0; j < 4; ++j) u.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
   };
@@ -355,22 +364,27 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe8_kernel(const MoePa
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-  MoeUnit8<T, MB> cur, nxt;
+  MoeUnit8<T, MB, MX> cur, nxt;
   int mine = wave;
   if (mine < p.units_per_strip) load_unit(cur, mine);
   while (mine < p.units_per_strip) {
     const int next = mine + kMoeWaves;
     if (next < p.units_per_strip) load_unit(nxt, next);
     Col cols[4];
+    if (!MX) {
 #pragma unroll
-    for (int j = 0; j < 4; ++j) cols[j] = D8::make_col((uint16_t)cur.sbits[j]);
+      for (int j = 0; j < 4; ++j) cols[j] = D8::make_col((uint16_t)cur.sbits[j]);
+    }
     int cur_group = cur.group;
     const int chunk0 = mine * p.unit_chunks;
 #pragma unroll
-    for (int cc = 0; cc < MoeUnit8<T, MB>::kChunks; ++cc) {
+    for (int cc = 0; cc < MoeUnit8<T, MB, MX>::kChunks; ++cc) {
       if (cc < p.unit_chunks) {
         const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
-        if (g != cur_group) {  // groups smaller than a unit
+        if (MX) {
+#pragma unroll
+          for (int j = 0; j < 4; ++j) cols[j] = D8::make_col(chunk_scale(cur.sv[MX ? cc : 0], j, col16));
+        } else if (g != cur_group) {  // groups smaller than a unit
           cur_group = g;
           const uint16_t* srow = scales + (long)g * p.size_n + strip * kStripN;
 #pragma unroll
@@ -459,7 +473,10 @@ void launch_moe(const MoeParams& p, bool has_perm, int grid, hipStream_t st) {
 
 template <typename T, int MB>
 void launch_moe8(const MoeParams& p, bool fp8, int grid, hipStream_t st) {
-  if (fp8) marlin_moe8_kernel<T, MB, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  // groups of 32 rows (MXFP8): the scales of every chunk are fetched with the unit
+  if (fp8 && p.num_groups > 1 && p.group_size == 32 && ((uintptr_t)p.scales) % 16 == 0)
+    marlin_moe8_kernel<T, MB, false, true, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  else if (fp8) marlin_moe8_kernel<T, MB, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
   else if (p.g_idx) marlin_moe8_kernel<T, MB, true, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
   else marlin_moe8_kernel<T, MB, false, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
 }

@@ -395,16 +395,19 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
 // with FP8; no act-order gather): the same partition, reduction and fix-up; a 32-row chunk of a strip
 // is two 1-KiB blocks of 16 rows, whose words give a lane the low and the high
 // four of the eight consecutive rows of an MFMA operand.
-template <typename T, int MB>
+// CHUNK_SCALES (groups of 32 rows, one per chunk: MXFP8): the scales of every
+// chunk travel with the unit, as in UnitBuf.
+template <typename T, int MB, bool CHUNK_SCALES = false>
 struct UnitBuf8 {
   uint4 q[unit_buffer_chunks<MB>()][2];
   typename Dq<T>::vec8 a[unit_buffer_chunks<MB>()][MB];
   uint32_t sbits[4];
   int group;
+  uint4 sv[CHUNK_SCALES ? unit_buffer_chunks<MB>() : 1];
 };
 
-template <typename T, int MB>
-__device__ __forceinline__ void load_unit8(UnitBuf8<T, MB>& b, const StreamParams& p, int u, int lane,
+template <typename T, int MB, bool CHUNK_SCALES = false>
+__device__ __forceinline__ void load_unit8(UnitBuf8<T, MB, CHUNK_SCALES>& b, const StreamParams& p, int u, int lane,
                                            bool grouped) {
   const int col16 = lane & 15, kb = lane >> 4;
   const int strip = u / p.units_per_strip;
@@ -427,11 +430,19 @@ __device__ __forceinline__ void load_unit8(UnitBuf8<T, MB>& b, const StreamParam
   const int g = grouped ? (chunk0 * kChunkK) / p.group_size : 0;
   b.group = g;
   const uint16_t* srow = p.scales + (long)g * p.size_n + strip * kStripN;
+  if (CHUNK_SCALES) {   // group = chunk
+#pragma unroll
+    for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc)
+      if (cc < p.unit_chunks)
+        b.sv[CHUNK_SCALES ? cc : 0] = *reinterpret_cast<const uint4*>(srow + (long)cc * p.size_n + 8 * (col16 & 7));
+    return;
+  }
 #pragma unroll
   for (int j = 0; j < 4; ++j) b.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
 }
 
-template <typename T, int MB, bool HAS_GIDX, bool FP8>
+// MX: float8 codes with groups of 32 rows (the host launches it for nothing else).
+template <typename T, int MB, bool HAS_GIDX, bool FP8, bool MX = false>
 __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const StreamParams params) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq8Of<T, FP8>::type D8;
@@ -457,9 +468,9 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
   const bool grouped = p.num_groups > 1;
   const uint32_t magic = magic_register();
 
-  UnitBuf8<T, MB> cur, nxt;
+  UnitBuf8<T, MB, MX> cur, nxt;
   int mine = u_begin + wave;
-  if (mine < u_end) load_unit8<T, MB>(cur, p, mine, lane, grouped);
+  if (mine < u_end) load_unit8<T, MB, MX>(cur, p, mine, lane, grouped);
 
   int seg_begin = u_begin;
   while (seg_begin < u_end) {
@@ -476,17 +487,22 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const Strea
 
     while (mine < seg_end) {
       const int next = mine + kWaves;
-      if (next < u_end) load_unit8<T, MB>(nxt, p, next, lane, grouped);
+      if (next < u_end) load_unit8<T, MB, MX>(nxt, p, next, lane, grouped);
       Col cols[4];
+      if (!MX) {
 #pragma unroll
-      for (int j = 0; j < 4; ++j) cols[j] = D8::make_col((uint16_t)cur.sbits[j]);
+        for (int j = 0; j < 4; ++j) cols[j] = D8::make_col((uint16_t)cur.sbits[j]);
+      }
       int cur_group = cur.group;
       const int chunk0 = (mine - strip_first) * p.unit_chunks;
 #pragma unroll
       for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc) {
         if (cc < p.unit_chunks) {
           const int g = grouped ? ((chunk0 + cc) * kChunkK) / p.group_size : 0;
-          if (g != cur_group) {  // groups smaller than a unit
+          if (MX) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) cols[j] = D8::make_col(chunk_scale(cur.sv[MX ? cc : 0], j, col16));
+          } else if (g != cur_group) {  // groups smaller than a unit
             cur_group = g;
             const uint16_t* srow = p.scales + (long)g * p.size_n + strip * kStripN;
 #pragma unroll
@@ -1243,19 +1259,22 @@ void launch_stream_fp4(const StreamParams& p, hipStream_t st) {
   }
 }
 
-template <typename T, bool HAS_GIDX, bool FP8>
+template <typename T, bool HAS_GIDX, bool FP8, bool MX = false>
 void launch_stream8_gidx(const StreamParams& p, hipStream_t st) {
   switch ((p.size_m + 15) / 16) {
-    case 1: marlin_stream8_kernel<T, 1, HAS_GIDX, FP8><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    case 2: marlin_stream8_kernel<T, 2, HAS_GIDX, FP8><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    case 3: marlin_stream8_kernel<T, 3, HAS_GIDX, FP8><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    default: marlin_stream8_kernel<T, 4, HAS_GIDX, FP8><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 1: marlin_stream8_kernel<T, 1, HAS_GIDX, FP8, MX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 2: marlin_stream8_kernel<T, 2, HAS_GIDX, FP8, MX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 3: marlin_stream8_kernel<T, 3, HAS_GIDX, FP8, MX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    default: marlin_stream8_kernel<T, 4, HAS_GIDX, FP8, MX><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
   }
 }
 
 template <typename T>
 void launch_stream8_mb(const StreamParams& p, bool fp8, hipStream_t st) {
-  if (fp8) launch_stream8_gidx<T, false, true>(p, st);   // no act-order with floating-point codes
+  // groups of 32 rows (MXFP8): the scales of every chunk are fetched with the unit
+  if (fp8 && p.num_groups > 1 && p.group_size == 32 && ((uintptr_t)p.scales) % 16 == 0)
+    launch_stream8_gidx<T, false, true, true>(p, st);
+  else if (fp8) launch_stream8_gidx<T, false, true>(p, st);   // no act-order with floating-point codes
   else if (p.g_idx) launch_stream8_gidx<T, true, false>(p, st);
   else launch_stream8_gidx<T, false, false>(p, st);
 }
