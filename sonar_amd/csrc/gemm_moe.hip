@@ -285,7 +285,7 @@ struct MoeUnit8 {
   uint4 sv[CHUNK_SCALES ? kChunks : 1];   // groups of 32 rows: the scales of every chunk
 };
 
-// MX: float8 codes with groups of 32 rows (the host launches it for nothing else).
+// MX: groups of 32 rows, one per chunk (MXFP8; integer codes with such groups too).
 template <typename T, int MB, bool HAS_GIDX, bool FP8, bool MX = false>
 __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe8_kernel(const MoeParams p) {
   typedef typename Dq<T>::vec8 vec8;
@@ -473,9 +473,10 @@ void launch_moe(const MoeParams& p, bool has_perm, int grid, hipStream_t st) {
 
 template <typename T, int MB>
 void launch_moe8(const MoeParams& p, bool fp8, int grid, hipStream_t st) {
-  // groups of 32 rows (MXFP8): the scales of every chunk are fetched with the unit
-  if (fp8 && p.num_groups > 1 && p.group_size == 32 && ((uintptr_t)p.scales) % 16 == 0)
-    marlin_moe8_kernel<T, MB, false, true, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  // groups of 32 rows (MXFP8, or integer codes): the scales of every chunk are fetched with the unit
+  const bool chunk_groups = !p.g_idx && p.num_groups > 1 && p.group_size == 32 && ((uintptr_t)p.scales) % 16 == 0;
+  if (fp8 && chunk_groups) marlin_moe8_kernel<T, MB, false, true, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  else if (chunk_groups) marlin_moe8_kernel<T, MB, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
   else if (fp8) marlin_moe8_kernel<T, MB, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
   else if (p.g_idx) marlin_moe8_kernel<T, MB, true, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
   else marlin_moe8_kernel<T, MB, false, false><<<grid, kMoeWaves * 64, 0, st>>>(p);

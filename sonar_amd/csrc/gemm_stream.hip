@@ -441,7 +441,7 @@ __device__ __forceinline__ void load_unit8(UnitBuf8<T, MB, CHUNK_SCALES>& b, con
   for (int j = 0; j < 4; ++j) b.sbits[j] = srow[scale_slot(16 * j + col16, grouped)];
 }
 
-// MX: float8 codes with groups of 32 rows (the host launches it for nothing else).
+// MX: groups of 32 rows, one per chunk (MXFP8; integer codes with such groups too).
 template <typename T, int MB, bool HAS_GIDX, bool FP8, bool MX = false>
 __global__ __launch_bounds__(kWaves * 64) void marlin_stream8_kernel(const StreamParams params) {
   typedef typename Dq<T>::vec8 vec8;
@@ -1271,9 +1271,10 @@ void launch_stream8_gidx(const StreamParams& p, hipStream_t st) {
 
 template <typename T>
 void launch_stream8_mb(const StreamParams& p, bool fp8, hipStream_t st) {
-  // groups of 32 rows (MXFP8): the scales of every chunk are fetched with the unit
-  if (fp8 && p.num_groups > 1 && p.group_size == 32 && ((uintptr_t)p.scales) % 16 == 0)
-    launch_stream8_gidx<T, false, true, true>(p, st);
+  // groups of 32 rows (MXFP8, or integer codes): the scales of every chunk are fetched with the unit
+  const bool chunk_groups = !p.g_idx && p.num_groups > 1 && p.group_size == 32 && ((uintptr_t)p.scales) % 16 == 0;
+  if (fp8 && chunk_groups) launch_stream8_gidx<T, false, true, true>(p, st);
+  else if (chunk_groups) launch_stream8_gidx<T, false, false, true>(p, st);
   else if (fp8) launch_stream8_gidx<T, false, true>(p, st);   // no act-order with floating-point codes
   else if (p.g_idx) launch_stream8_gidx<T, true, false>(p, st);
   else launch_stream8_gidx<T, false, false>(p, st);
