@@ -5,6 +5,7 @@ from __future__ import annotations
 import os
 import subprocess
 import sys
+from concurrent.futures import ThreadPoolExecutor
 
 PKG = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(PKG)
@@ -31,17 +32,25 @@ def _run(cmd):
     return out
 
 
-def build_hip_library(verbose: bool = False) -> str:
+def build_hip_library(verbose: bool = False, only=None) -> str:
+    """Compiles every HIP source (or, with `only`, those sources; the other objects are
+    reused when they exist) and links the shared library."""
     os.makedirs(LIB_DIR, exist_ok=True)
-    objs = []
-    for src in HIP_SOURCES:
+    only = set(only or HIP_SOURCES)
+
+    def compile_one(src):
         obj = os.path.join(LIB_DIR, src.replace(".hip", ".o"))
-        cmd = [HIPCC, *HIP_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
-               "-c", os.path.join(CSRC, src), "-o", obj]
-        out = _run(cmd)
-        if verbose and out.strip():
-            print(out)
-        objs.append(obj)
+        if src in only or not os.path.exists(obj):
+            cmd = [HIPCC, *HIP_FLAGS, "-I", os.path.join(ROOT, "include"), "-I", CSRC,
+                   "-c", os.path.join(CSRC, src), "-o", obj]
+            out = _run(cmd)
+            if verbose and out.strip():
+                print(out)
+        return obj
+
+    # one hipcc per source file, side by side
+    with ThreadPoolExecutor(max_workers=min(len(HIP_SOURCES), os.cpu_count() or 1)) as pool:
+        objs = list(pool.map(compile_one, HIP_SOURCES))
     _run([HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH, *objs])
     return LIB_PATH
 
@@ -78,6 +87,9 @@ def build_all(verbose: bool = False):
 
 
 if __name__ == "__main__":
-    for p in build_all(verbose=True):
-        print("built", p)
+    if len(sys.argv) > 1:   # python -m sonar_amd.build gemm_stream.hip ...: recompile these, relink
+        print("built", build_hip_library(verbose=True, only=sys.argv[1:]))
+    else:
+        for p in build_all(verbose=True):
+            print("built", p)
     sys.exit(0)

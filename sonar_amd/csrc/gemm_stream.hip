@@ -32,6 +32,17 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
               size_t partial_bytes, bool fp4, hipStream_t st);
 bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size);
 
+#ifdef SONAR_TRACE
+__device__ unsigned long long* g_trace;
+#define TRACE(i)                                                                   \
+  do {                                                                             \
+    if (g_trace && (threadIdx.x & 63) == 0)                                        \
+      g_trace[((long)blockIdx.x * 8 + (threadIdx.x >> 6)) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+  } while (0)
+#else
+#define TRACE(i)
+#endif
+
 namespace {
 
 constexpr int kWaves = 8;
@@ -59,6 +70,21 @@ struct StreamParams {
   // the general kernels) times `grid_parts` >= parts workgroups per block
   // (part_and_slab; parts past `parts` are padding)
   int slabs, grid_parts;
+  // fast kernel only: with `tickets` the strips shared between workgroups are
+  // summed inside the kernel.  Every contributor stores its fp32 partial tiles
+  // with agent-scope (write-through) stores, waits for them, and draws a ticket
+  // of the strip with one relaxed atomic add; the workgroup that draws the last
+  // ticket reads all the partial tiles back with agent-scope loads, adds them in
+  // workgroup order (the same bits whoever comes last), writes C and puts the
+  // ticket back to zero.  Nobody waits for anybody, so nothing can hang.  Ticket
+  // of the strip whose first contributor is `first`, for block of rows `slab`:
+  // tickets[(first * slabs + slab) * ticket_stride].  Without `tickets` the
+  // fix-up kernel adds the partial tiles.
+  unsigned int* tickets;
+  int ticket_stride;
+  // workgroup ids are dealt to the parts so that consecutive parts (which share
+  // strips and rows of A) have ids congruent mod 8, i.e. sit on one XCD
+  int xcd_ranges;
   // fast kernel only: the tiles of the cross-wavefront sum are parked on top of
   // the copy rings instead of behind them.  Allowed when every workgroup owns
   // whole strips: it then sums once, after its last copy has been consumed.
@@ -90,9 +116,11 @@ __host__ __device__ __forceinline__ int range_owner(int x, int total, int parts)
 // With several slabs grid_parts is a multiple of 8 and the slabs of a part get
 // consecutive ids on one XCD (ids congruent mod 8), so that they are dispatched
 // together and the second to ask for a weight chunk finds it in that XCD's L2.
-__device__ __forceinline__ void part_and_slab(const int grid_parts, const int slabs, int& part, int& slab) {
+__device__ __forceinline__ void part_and_slab(const int grid_parts, const int slabs, int& part, int& slab,
+                                              const int xcd_ranges = 0) {
   if (slabs == 1) {
-    part = blockIdx.x;
+    // xcd_ranges (grid_parts % 8 == 0): ids congruent mod 8 get a contiguous run of parts
+    part = xcd_ranges ? (int)(blockIdx.x & 7) * (grid_parts >> 3) + (int)(blockIdx.x >> 3) : (int)blockIdx.x;
     slab = 0;
     return;
   }
@@ -180,30 +208,58 @@ __device__ __forceinline__ void finish_segment(const StreamParams& p, int part, 
 // `part` is the workgroup's index in the partition and `slab` the tile's block
 // of 16 rows (fast kernel: several blocks of rows share one launch; the scratch
 // slot of a part holds one partial tile per block of rows).
+// Adds bias, rounds and stores one 16 x 16 block (column block j of a strip) held by one wavefront.
+template <typename T>
+__device__ __forceinline__ void store_c_block(const StreamParams& p, uint16_t* c_block, int rows, int strip, int lane,
+                                              int j, floatx4_t v) {
+  const int m = lane & 15;
+  const int nl = 16 * j + 4 * (lane >> 4);
+  if (m < rows) {
+    float b[4] = {0.f, 0.f, 0.f, 0.f};
+    if (p.bias) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+        b[r] = Dq<T>::to_float(p.bias[strip * kStripN + scale_slot(nl + r, false)]);
+    }
+    uint2 o;
+    o.x = (uint32_t)Dq<T>::from_float(v.x + b[0]) | ((uint32_t)Dq<T>::from_float(v.y + b[1]) << 16);
+    o.y = (uint32_t)Dq<T>::from_float(v.z + b[2]) | ((uint32_t)Dq<T>::from_float(v.w + b[3]) << 16);
+    *reinterpret_cast<uint2*>(c_block + (long)m * p.size_n + strip * kStripN + nl) = o;
+  }
+}
+
 template <typename T>
 __device__ __forceinline__ void finish_block(const StreamParams& p, uint16_t* c_block, int rows, int part, int slab,
                                              int strip, int seg_begin, int seg_end, int lane, int j, floatx4_t v) {
   const int strip_first = strip * p.units_per_strip;
   const int strip_end = strip_first + p.units_per_strip;
   if (seg_begin == strip_first && seg_end == strip_end) {
-    const int m = lane & 15;
-    const int nl = 16 * j + 4 * (lane >> 4);
-    if (m < rows) {
-      float b[4] = {0.f, 0.f, 0.f, 0.f};
-      if (p.bias) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-          b[r] = Dq<T>::to_float(p.bias[strip * kStripN + scale_slot(nl + r, false)]);
-      }
-      uint2 o;
-      o.x = (uint32_t)Dq<T>::from_float(v.x + b[0]) | ((uint32_t)Dq<T>::from_float(v.y + b[1]) << 16);
-      o.y = (uint32_t)Dq<T>::from_float(v.z + b[2]) | ((uint32_t)Dq<T>::from_float(v.w + b[3]) << 16);
-      *reinterpret_cast<uint2*>(c_block + (long)m * p.size_n + strip * kStripN + nl) = o;
-    }
+    store_c_block<T>(p, c_block, rows, strip, lane, j, v);
     return;
   }
   const int first = range_owner(strip_first, p.total_units, p.parts);
-  partial_slot(p, part, first)[(slab * 4 + j) * 64 + lane] = make_float4(v.x, v.y, v.z, v.w);
+  float4* dst = partial_slot(p, part, first) + (slab * 4 + j) * 64 + lane;
+  if (p.tickets) {  // read back by another workgroup of this launch: write through to memory
+    unsigned long long* d = reinterpret_cast<unsigned long long*>(dst);
+    const unsigned long long lo = ((unsigned long long)__float_as_uint(v.y) << 32) | __float_as_uint(v.x);
+    const unsigned long long hi = ((unsigned long long)__float_as_uint(v.w) << 32) | __float_as_uint(v.z);
+    __hip_atomic_store(d, lo, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_store(d + 1, hi, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+    *dst = make_float4(v.x, v.y, v.z, v.w);
+  }
+}
+
+// The partial tile (block of rows `slab`, column block j) that workgroup w left for a
+// strip whose first contributor is `first`, read with agent-scope loads.
+__device__ __forceinline__ floatx4_t load_partial_tile(const StreamParams& p, int w, int first, int slab, int j,
+                                                       int lane) {
+  const unsigned long long* src =
+      reinterpret_cast<const unsigned long long*>(partial_slot(p, w, first) + (slab * 4 + j) * 64 + lane);
+  const unsigned long long lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  const unsigned long long hi = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return floatx4_t{__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)),
+                   __uint_as_float((unsigned)hi), __uint_as_float((unsigned)(hi >> 32))};
 }
 
 // Grouped calls: the tile's row (lane & 15) goes to row `id` of C (none when
@@ -565,9 +621,9 @@ constexpr int kSlotS = 4096;       // inside a weight slot, after 4 chunks x 1 K
 // or more, 2 / 4 for groups of 64 / 32 rows): one 256-byte scale / zero-point
 // row per group follows the four chunks of a weight slot.
 constexpr int slot_bytes(int gpu) { return 4096 + 256 * gpu; }
-constexpr int wave_a(int gpu) { return 2 * slot_bytes(gpu); }   // the activation slot follows the two weight slots
+constexpr int wave_a(int gpu, int slots = 2) { return slots * slot_bytes(gpu); }   // the activation slot follows the weight slots
 // LDS bytes per wavefront: the activation slot holds 4 KiB per block of 16 rows
-constexpr int wave_lds(int mb, int gpu = 1) { return 2 * slot_bytes(gpu) + 4096 * mb; }
+constexpr int wave_lds(int mb, int gpu = 1, int slots = 2) { return slots * slot_bytes(gpu) + 4096 * mb; }
 // Tiles (16 x 16 fp32, 1 KiB) a wavefront parks per pass of the cross-wavefront
 // sum: all four of its one block of rows, or two of the eight of two blocks
 // (four passes), which keeps 8 wavefronts with two blocks inside 160 KiB.
@@ -576,8 +632,8 @@ constexpr int weight_copies(int gpu) { return 4 + gpu; }   // asynchronous copie
 // A workgroup of the fast kernel has 8 wavefronts (one workgroup per compute
 // unit), or 4 (two per compute unit: a grid with more workgroups than compute
 // units then runs them side by side instead of one after the other).
-constexpr int fast_lds_bytes(int waves, int mb, int gpu = 1) {
-  return waves * (wave_lds(mb, gpu) + park_tiles(mb) * 1024);
+constexpr int fast_lds_bytes(int waves, int mb, int gpu = 1, int slots = 2) {
+  return waves * (wave_lds(mb, gpu, slots) + park_tiles(mb) * 1024);
 }
 
 // Row id of C of row `r` of block `block` of a grouped call, -1 for padding.
@@ -627,6 +683,9 @@ template <int MB>
 __device__ __forceinline__ void copy_activations(const StreamParams& p, const FastLane<MB>& fl, int unit,
                                                  char* slot) {
   const char* ga = reinterpret_cast<const char*>(p.a) + (long)unit * (4 * kChunkK * 2);
+#ifdef SONAR_EXP_NO_A
+  return;
+#endif
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     char* s = slot + 4096 * mb;
@@ -764,24 +823,38 @@ __device__ __forceinline__ u32x4_t raw_operand(uint32_t q, uint32_t magic) {
 // GPU: groups per 128-row unit (2 or 4 for groups of 64 or 32 rows, else 1).
 // FP4 (with GPU = 4, no zero points): float4_e2m1f codes; the operands are the
 // converted values themselves, so only the scale is left for after the unit.
-template <typename T, bool HAS_ZP, int kFastWaves, int MB, bool GROUPED = false, int GPU = 1, bool FP4 = false>
+// SLOTS: weight slots per wavefront, i.e. units of weights in flight.  Three were measured
+// slower than two on every Llama-3-8B shape (M = 16: down 12.2 against 11.4 us, gate_up
+// 19.1 against 17.4), so only two are instantiated.
+template <typename T, bool HAS_ZP, int kFastWaves, int MB, bool GROUPED = false, int GPU = 1, bool FP4 = false,
+          int SLOTS = 2>
 __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams params,
                                                                              const int unit_group_shift) {
   typedef typename Dq<T>::vec8 vec8;
-  constexpr int kWaveLds = wave_lds(MB, GPU);
+  constexpr int kWaveLds = wave_lds(MB, GPU, SLOTS);
   constexpr int kSlotBytes = slot_bytes(GPU);
-  constexpr int kWaveA = wave_a(GPU);
+  constexpr int kWaveA = wave_a(GPU, SLOTS);
   constexpr int kWeightCopies = weight_copies(GPU);
   constexpr int kPark = park_tiles(MB);       // tiles per wavefront and pass of the cross-wavefront sum
   constexpr int kPasses = 4 * MB / kPark;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
+  TRACE(0);
   StreamParams p = params;
+  // Every argument the dense path reads, fetched now in one batch of scalar loads: left to
+  // itself the compiler fetches them where they are first used, four round trips to a cold
+  // argument buffer one after the other (about 2 us of a kernel that takes 6).
+  if constexpr (!GROUPED)
+    asm volatile("" ::"s"(p.a), "s"(p.lda), "s"(p.c), "s"(p.b), "s"(p.bias), "s"(p.scales), "s"(p.zeros),
+                 "s"(p.scratch), "s"(p.size_m), "s"(p.size_n), "s"(p.num_groups), "s"(p.chunks_per_strip),
+                 "s"(p.units_per_strip), "s"(p.parts), "s"(p.total_units), "s"(p.slabs), "s"(p.grid_parts),
+                 "s"(p.tickets), "s"(p.ticket_stride), "s"(p.xcd_ranges), "s"(p.sum_over_rings),
+                 "s"(unit_group_shift));
   int part, slab;
   if constexpr (GROUPED) {   // strip-major inside a block of slots
     part = blockIdx.x % p.grid_parts;
     slab = blockIdx.x / p.grid_parts;
   } else {
-    part_and_slab(p.grid_parts, p.slabs, part, slab);
+    part_and_slab(p.grid_parts, p.slabs, part, slab, p.xcd_ranges);
   }
   if (part >= p.parts) return;
   const int lane = threadIdx.x & 63;
@@ -860,26 +933,38 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   asm("" : "+v"(ones));
 
   // Issue order of a wavefront's copies, x being one of its units and W the
-  // distance to its next one:  weights(x) | A(x), weights(x+W) | A(x+W),
-  // weights(x+2W) | ...  They complete in this order.  When the arithmetic of x
-  // starts, the only copies younger than A(x) are the 5 of weights(x+W), so "at
-  // most 5 outstanding" means weights(x) and A(x) have landed.
-  UnitCursor cur, fetch;
+  // distance to its next one (two slots):  weights(x) | A(x), weights(x+W) | A(x+W),
+  // weights(x+2W) | ...; with three slots weights(x+2W) follows weights(x+W) at the
+  // start and every later A(y) is followed by weights(y+2W).  They complete in this
+  // order.  When the arithmetic of x starts, the copies younger than A(x) are those of
+  // one unit of weights (of SLOTS - 1 units before the first unit), so "at most that
+  // many outstanding" means weights(x) and A(x) have landed.
+  UnitCursor cur, fetch, fetch_w;
   cur.set(u_begin + wave, p.units_per_strip);
-  fetch = cur;
-  if (fetch.index < u_end) {
-    copy_weights<MB, GPU>(p, fl, fetch.strip, fetch.unit, ring, lane, unit_group_shift);
-    copy_activations<MB>(p, fl, fetch.unit, ring + kWaveA);
+  fetch_w = cur;
+#pragma unroll
+  for (int sl = 0; sl < SLOTS; ++sl) {
+    if (fetch_w.index < u_end) {
+      copy_weights<MB, GPU>(p, fl, fetch_w.strip, fetch_w.unit, ring + sl * kSlotBytes, lane, unit_group_shift);
+      if (sl == 0) copy_activations<MB>(p, fl, fetch_w.unit, ring + kWaveA);
+    }
+    fetch_w.advance(kFastWaves, p.units_per_strip);
   }
+  // `fetch` names the unit whose A slice is copied next, `fetch_w` the one whose weights are
+  fetch = cur;
   fetch.advance(kFastWaves, p.units_per_strip);
-  if (fetch.index < u_end)
-    copy_weights<MB, GPU>(p, fl, fetch.strip, fetch.unit, ring + kSlotBytes, lane, unit_group_shift);
-  // `fetch` names the unit whose A slice is copied next; its weights are in flight
   int c_slot = 0;
+  bool first_unit = true;
+  TRACE(1);
 
   // the current segment starts at seg_begin, inside strip seg_strip
   int seg_begin = u_begin;
   int seg_strip = u_begin / p.units_per_strip;
+  // strips of which this workgroup has left partial tiles in memory (at most two: the
+  // one its range starts inside and the one it ends inside); their tickets are drawn
+  // when all its units are done, so that the streaming is not held up in between
+  int pending_strip[2] = {0, 0};
+  int pending = 0;
   floatx4_t acc[MB][4];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
@@ -959,6 +1044,13 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
       for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
         for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+      if constexpr (!GROUPED) {
+        if (seg_begin != strip * p.units_per_strip || seg_end != strip_end) {
+          if (pending == 0) pending_strip[0] = strip;
+          else pending_strip[1] = strip;
+          ++pending;
+        }
+      }
       seg_begin = seg_end;
       ++seg_strip;
     }
@@ -973,11 +1065,20 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     u32x4_t row_z = u32x4_t{0u, 0u, 0u, 0u};
     uint32_t more_s[GPU > 1 ? GPU - 1 : 1][16];   // the other groups of the unit
     u32x4_t more_z[GPU > 1 ? GPU - 1 : 1];
-    const bool more = cur.index + kFastWaves < u_end;
-    if (more) {
-      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightCopies) : "memory");
-    } else {
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // this wavefront's units after the current one
+    const int after = (u_end - 1 - cur.index) / kFastWaves;
+    const bool more = after >= 1;
+    {
+      // units of weights whose copies were issued after those of A(x)
+      const int younger = first_unit ? (after < SLOTS - 1 ? after : SLOTS - 1) : (after >= SLOTS - 1 ? 1 : 0);
+      if (younger == 0) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      } else if (SLOTS == 2 || younger == 1) {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightCopies) : "memory");
+      } else {
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kWeightCopies) : "memory");
+      }
+      first_unit = false;
     }
     {
       const uint32_t q_at = slot_lds + lane * 16;
@@ -994,13 +1095,26 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
         SONAR_GROUP_READS(3);
       }
     }
+    TRACE(2);
     if (more) {
       copy_activations<MB>(p, fl, fetch.unit, ring + kWaveA);
       fetch.advance(kFastWaves, p.units_per_strip);
-      if (fetch.index < u_end)
-        copy_weights<MB, GPU>(p, fl, fetch.strip, fetch.unit, ring + c_slot * kSlotBytes, lane, unit_group_shift);
+      if (fetch_w.index < u_end) {
+        copy_weights<MB, GPU>(p, fl, fetch_w.strip, fetch_w.unit, ring + c_slot * kSlotBytes, lane,
+                              unit_group_shift);
+        fetch_w.advance(kFastWaves, p.units_per_strip);
+      }
     }
 
+#ifdef SONAR_EXP_NO_COMPUTE
+    {
+      const u32x4_t x = q0 ^ q1 ^ q2 ^ q3 ^ a0 ^ a1 ^ a2 ^ a3 ^ row_z;
+      acc[0][0][0] += __uint_as_float((x.x ^ x.y ^ x.z ^ x.w ^ row_s[0] ^ row_s[15]) & 0x3fffffu);
+      cur.advance(kFastWaves, p.units_per_strip);
+      c_slot = c_slot + 1 == SLOTS ? 0 : c_slot + 1;
+      continue;
+    }
+#endif
     const u32x4_t qs[4] = {q0, q1, q2, q3};
     const u32x4_t as[2][4] = {{a0, a1, a2, a3}, {b0, b1, b2, b3}};
     const floatx4_t zero4 = floatx4_t{0.f, 0.f, 0.f, 0.f};
@@ -1047,7 +1161,61 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
         }
     }
     cur.advance(kFastWaves, p.units_per_strip);
-    c_slot ^= 1;
+    c_slot = c_slot + 1 == SLOTS ? 0 : c_slot + 1;
+    TRACE(3);
+  }
+  TRACE(4);
+
+  // Strips shared with other workgroups: draw their tickets; whoever holds the last
+  // ticket of a strip adds its partial tiles up.
+  if constexpr (!GROUPED) {
+    if (p.tickets != nullptr && pending > 0) {
+      const uint32_t flag_lds = (uint32_t)(uintptr_t)(lds_void_t*)smem;
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's partial tiles are in memory
+      TRACE(5);
+      __builtin_amdgcn_s_barrier();                      // ... and every wavefront's; all LDS traffic is over
+      if (wave == 0 && lane < pending) {
+        const int strip = lane == 0 ? pending_strip[0] : pending_strip[1];
+        const int first = range_owner(strip * p.units_per_strip, p.total_units, p.parts);
+        unsigned int* ticket = p.tickets + ((long)first * p.slabs + slab) * p.ticket_stride;
+        const unsigned int drawn = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(flag_lds + 4u * lane), "v"(drawn) : "memory");
+      }
+      __builtin_amdgcn_s_barrier();
+      TRACE(6);
+      for (int k = 0; k < pending; ++k) {
+        uint32_t drawn;
+        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(drawn) : "v"(flag_lds + 4u * k) : "memory");
+        drawn = __builtin_amdgcn_readfirstlane(drawn);
+        const int strip = k == 0 ? pending_strip[0] : pending_strip[1];
+        const int strip_first = strip * p.units_per_strip;
+        const int first = range_owner(strip_first, p.total_units, p.parts);
+        const int last = range_owner(strip_first + p.units_per_strip - 1, p.total_units, p.parts);
+        if ((int)drawn != last - first) continue;   // somebody is still at work on this strip
+        for (int t = wave; t < 4 * MB; t += kFastWaves) {
+          const int mb = t >> 2, j = t & 3;
+          // four loads in flight at a time, added in workgroup order
+          floatx4_t sum = floatx4_t{0.f, 0.f, 0.f, 0.f};
+          for (int w0 = first; w0 <= last; w0 += 4) {
+            floatx4_t part4[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              part4[i] = load_partial_tile(p, w0 + i <= last ? w0 + i : last, first, slab * MB + mb, j, lane);
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+              if (w0 + i <= last) sum += part4[i];
+          }
+          store_c_block<T>(p, p.c + (long)(16 * mb) * p.size_n, p.size_m - 16 * mb, strip, lane, j, sum);
+        }
+        if (threadIdx.x == 0)
+          __hip_atomic_store(p.tickets + ((long)first * p.slabs + slab) * p.ticket_stride, 0u, __ATOMIC_RELAXED,
+                             __HIP_MEMORY_SCOPE_AGENT);
+      }
+#ifdef SONAR_TRACE
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+#endif
+      TRACE(7);
+    }
   }
 }
 #undef SONAR_UNIT_READS_ROWS2
@@ -1541,6 +1709,12 @@ namespace {
 size_t stream_scratch_bytes() { return (size_t)2 * cu_count() * kSlotFloat4 * sizeof(float4); }
 }  // namespace
 
+#ifdef SONAR_TRACE
+extern "C" void sonar_debug_set_trace(void* ptr) {
+  (void)hipMemcpyToSymbol(HIP_SYMBOL(sonar::g_trace), &ptr, sizeof(ptr));
+}
+#endif
+
 extern "C" size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k) {
   // partial tiles of the streaming kernels, then those of a split-K tile launch
   return stream_scratch_bytes() + plan_partial_bytes(plan_gemm(size_m, size_n, size_k, true), size_m, size_n);
@@ -1567,8 +1741,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   SONAR_REQUIRE(((uintptr_t)c) % 8 == 0 && ((uintptr_t)b_q_weight) % 16 == 0,
                 "c must be 8-byte and b_q_weight 16-byte aligned");
   const int cus = cu_count();
-  // The workspace is not touched (no locks are taken), but a caller that sizes
-  // it wrongly for the reference would fail there, so it fails here too.
+  // The workspace holds the tickets of the strips that workgroups of the decode kernel share
+  // (all zero again when the kernel ends; nobody ever waits on one).
   SONAR_REQUIRE(workspace && workspace_len >= cus,
                 "workspace.numel = %ld is below min_workspace_size = %d", (long)workspace_len, cus);
   SONAR_REQUIRE(scratch && scratch_bytes >= sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k),
@@ -1671,10 +1845,35 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   const bool row_slabs = !use_tile && !slab_fast && size_m > 64 && strip_per_workgroup &&
                          total_units * n_strips < (1LL << 31);
   p.parts = p.total_units < cus ? p.total_units : cus;
-  if (strip_per_workgroup && (p.unit_chunks == 4 || row_slabs)) p.parts = (int)n_strips;
+  // Up to 16 rows in the fast kernel: every strip is cut into the same number of pieces, as
+  // many as make at most one workgroup per compute unit (a Llama-3-8B attention output
+  // projection: 64 strips x 4), and the pieces of a strip are summed inside the kernel
+  // (tickets in the workspace).  With more strips than compute units every strip is one
+  // workgroup.  Either way a workgroup works on one strip only, sums its wavefronts once,
+  // at the end, and can park the tiles of that sum on top of its copy rings, which leaves
+  // LDS for a third weight slot per wavefront.
+  static const bool no_inline_sum = getenv("SONAR_MARLIN_NO_INLINE_SUM") != nullptr;   // debugging aids
+  static const char* split_env = getenv("SONAR_MARLIN_SPLIT");
+  const bool piece_split = fast_shape && p.unit_chunks == 4 && size_m <= 16 && !no_inline_sum &&
+                           n_strips * n_strips * p.units_per_strip < (1LL << 31);
+  int pieces = 1;
+  if (piece_split) {
+    pieces = (int)(cus / n_strips);
+    if (split_env) pieces = atoi(split_env);
+    if (pieces > p.units_per_strip) pieces = p.units_per_strip;
+    if (pieces > 16) pieces = 16;
+    if (pieces < 1) pieces = 1;
+    if (n_strips * pieces > workspace_len) pieces = 1;
+    p.parts = (int)n_strips * pieces;   // range_begin(strip * pieces + i) = strip * units_per_strip + i * units_per_strip / pieces
+  } else if (strip_per_workgroup && (p.unit_chunks == 4 || row_slabs)) {
+    p.parts = (int)n_strips;
+  }
   p.slabs = 1;
   p.grid_parts = p.parts;
   p.sum_over_rings = 0;
+  p.tickets = nullptr;
+  p.ticket_stride = 1;
+  p.xcd_ranges = 0;
 
   bool any_split = false;
   for (int i = 1; i < p.parts && !any_split; ++i)
@@ -1692,6 +1891,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
     p.c = static_cast<uint16_t*>(c) + m0 * size_n;
     p.size_m = (int)(size_m - m0 < 64 ? size_m - m0 : 64);
     const bool fast = fast_shape && p.unit_chunks == 4 && (p.size_m <= 16 || slab_fast);
+    bool inline_sum = false;
     if (fast) {
       // Two blocks of rows per workgroup once one block each would make more
       // workgroups than compute units: the weights are then fetched from L2 and
@@ -1711,6 +1911,18 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
       static const bool no_half = getenv("SONAR_MARLIN_NO_HALF_WG") != nullptr;  // debugging aid
       const bool half = !no_half && p.parts * p.slabs > cus;
       p.sum_over_rings = half && (int64_t)p.parts == n_strips && p.parts * p.slabs > 2 * cus;
+      if (piece_split) {
+        p.sum_over_rings = 1;
+      }
+      // Shared strips are summed inside the kernel when the workspace has a ticket for every
+      // part and block of rows; tickets four words apart do not hold each other up.
+      inline_sum = any_split && !no_inline_sum && (int64_t)p.parts * p.slabs <= workspace_len;
+      if (inline_sum) {
+        p.tickets = reinterpret_cast<unsigned int*>(workspace);
+        const int64_t room = workspace_len / ((int64_t)p.parts * p.slabs);
+        p.ticket_stride = room >= 4 ? 4 : (int)room;
+        p.xcd_ranges = p.slabs == 1 && p.parts % 8 == 0;
+      }
       if (chk.fp4)   // groups of 32 rows: never in blocks of rows (slab_fast is off), so one block of 16 rows
         rc = launch_fast_fp4<false>(p, half, st);
       else if (dtype == SONAR_DTYPE_F16)
@@ -1741,7 +1953,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
       }
     }
     if (int rc = launch_status("marlin_stream_kernel")) return rc;
-    if (any_split) {
+    if (any_split && !inline_sum) {
       if (dtype == SONAR_DTYPE_F16) launch_fixup<_Float16>(p, st);
       else launch_fixup<__bf16>(p, st);
       if (int rc = launch_status("marlin_fixup_kernel")) return rc;
