@@ -150,6 +150,29 @@ int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                       int64_t num_groups, int is_k_full, int use_atomic_add,
                       int use_fp32_reduce, void* stream);
 
+/* sonar_marlin_gemm for callers that cannot allocate device memory (code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the
+ * reference.  Same arguments without `scratch` / `scratch_bytes`: the scratch memory (fp32
+ * partial tiles of strips or tiles whose K range is shared between workgroups; with act-order the
+ * column-permuted copy of A when it fits) is a static array in device memory of 24 MiB, one
+ * per GPU, held until the process ends.  The call allocates and frees nothing.  A call whose
+ * sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k) exceeds 24 MiB fails with
+ * SONAR_E_INVALID and launches nothing (every size_m <= 128 fits for any matrix; beyond that
+ * only calls whose K range is split over many workgroups can exceed it).  All calls on one
+ * GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two
+ * threads) race and give wrong results; calls on one stream, or ordered by events, do not.
+ * Nothing in the array has to be zero between calls.  The first call on a device looks the
+ * array's address up (hipGetSymbolAddress); make it outside graph capture. */
+int sonar_marlin_gemm_noalloc(const void* a, int64_t a_row_stride, void* c,
+                              const uint32_t* b_q_weight, int b_layout,
+                              const void* b_bias, const void* b_scales,
+                              const uint32_t* b_zeros, const int32_t* g_idx,
+                              const int32_t* perm, int32_t* workspace,
+                              int64_t workspace_len, int dtype, int64_t b_type_id,
+                              int64_t size_m, int64_t size_n, int64_t size_k,
+                              int64_t num_groups, int is_k_full, int use_atomic_add,
+                              int use_fp32_reduce, void* stream);
+
 /* Grouped (mixture-of-experts) variant.  For block b <
  * num_tokens_past_padded[0] / moe_block_size with expert e = expert_ids[b]
  * (e < 0: skipped), each slot id = sorted_token_ids[b*moe_block_size + i] with

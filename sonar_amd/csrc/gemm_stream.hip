@@ -1962,6 +1962,50 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   return SONAR_OK;
 }
 
+// ---------------------------------------------------------------------------
+// The GEMM for callers that cannot allocate: the scratch memory is this array,
+// one copy per GPU that the library runs on, held until the process ends.
+namespace {
+constexpr size_t kStaticScratchBytes = (size_t)24 << 20;
+static __device__ __align__(256) unsigned char scratch[kStaticScratchBytes];
+constexpr int kMaxDevices = 64;
+void* g_static_scratch[kMaxDevices];   // device address of `scratch` on every device, once asked for
+}  // namespace
+
+extern "C" int sonar_marlin_gemm_noalloc(const void* a, int64_t a_row_stride, void* c, const uint32_t* b_q_weight,
+                                         int b_layout, const void* b_bias, const void* b_scales,
+                                         const uint32_t* b_zeros, const int32_t* g_idx, const int32_t* perm,
+                                         int32_t* workspace, int64_t workspace_len, int dtype, int64_t b_type_id,
+                                         int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
+                                         int is_k_full, int use_atomic_add, int use_fp32_reduce, void* stream) {
+  SONAR_REQUIRE(size_m >= 0 && size_m < (1LL << 30) && size_n > 0 && size_n < (1LL << 30) && size_k > 0 &&
+                    size_k < (1LL << 30),
+                "size_m, size_n, size_k = %ld, %ld, %ld out of range", (long)size_m, (long)size_n, (long)size_k);
+  int dev = 0;
+  SONAR_HIP(hipGetDevice(&dev));
+  SONAR_REQUIRE(dev >= 0 && dev < kMaxDevices, "device index %d is beyond the %d this entry point keeps", dev,
+                kMaxDevices);
+  void* base = __atomic_load_n(&g_static_scratch[dev], __ATOMIC_ACQUIRE);
+  if (base == nullptr) {   // first call on this device: the array's address there
+    SONAR_HIP(hipGetSymbolAddress(&base, HIP_SYMBOL(scratch)));
+    SONAR_REQUIRE(base != nullptr, "hipGetSymbolAddress returned no address for the static scratch array");
+    __atomic_store_n(&g_static_scratch[dev], base, __ATOMIC_RELEASE);
+  }
+  const size_t need = sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k);
+  if (need > kStaticScratchBytes)
+    return fail(SONAR_E_INVALID,
+                "sonar_marlin_gemm_noalloc: size_m, size_n, size_k = %ld, %ld, %ld need %zu bytes of scratch, "
+                "the static array holds %zu; call sonar_marlin_gemm with a buffer of the caller's",
+                (long)size_m, (long)size_n, (long)size_k, need, kStaticScratchBytes);
+  // an act-order call also gets room for the column-permuted copy of A when that fits
+  size_t give = need;
+  if (perm != nullptr && need + (size_t)size_m * (size_t)size_k * 2 <= kStaticScratchBytes)
+    give = need + (size_t)size_m * (size_t)size_k * 2;
+  return sonar_marlin_gemm(a, a_row_stride, c, b_q_weight, b_layout, b_bias, b_scales, b_zeros, g_idx, perm,
+                           workspace, workspace_len, base, give, dtype, b_type_id, size_m, size_n, size_k,
+                           num_groups, is_k_full, use_atomic_add, use_fp32_reduce, stream);
+}
+
 extern "C" int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout, const void* b_scales,
                                     const uint32_t* b_zeros, const int32_t* g_idx, void* w_out,
                                     int dtype, int64_t b_type_id, int64_t size_n, int64_t size_k,
