@@ -33,11 +33,11 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
 bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size);
 
 #ifdef SONAR_TRACE
-__device__ unsigned long long* g_trace;
+unsigned long long* g_trace_host;
 #define TRACE(i)                                                                   \
   do {                                                                             \
-    if (g_trace && (threadIdx.x & 63) == 0)                                        \
-      g_trace[((long)blockIdx.x * 8 + (threadIdx.x >> 6)) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+    if (params.trace && (threadIdx.x & 63) == 0)                                   \
+      params.trace[((long)blockIdx.x * 8 + (threadIdx.x >> 6)) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
   } while (0)
 #else
 #define TRACE(i)
@@ -49,6 +49,9 @@ constexpr int kWaves = 8;
 constexpr int kSlotFloat4 = 4 * 4 * 64;  // largest partial tile: 4 row blocks x 4 column blocks x 64 lanes
 
 struct StreamParams {
+#ifdef SONAR_TRACE
+  unsigned long long* trace;
+#endif
   const uint16_t* a;
   long lda;
   uint16_t* c;
@@ -85,6 +88,12 @@ struct StreamParams {
   // workgroup ids are dealt to the parts so that consecutive parts (which share
   // strips and rows of A) have ids congruent mod 8, i.e. sit on one XCD
   int xcd_ranges;
+  // fast kernel only: piece_units > 0 says that every strip is cut into 2^piece_shift
+  // pieces of piece_units units, part (strip << piece_shift) + i being piece i: the
+  // kernel then finds its range with shifts instead of the divisions of the general
+  // split (a wavefront's scalar unit is shared with seven others: the index arithmetic
+  // of the general split alone took about 0.4 us before the first copy was issued)
+  int piece_shift, piece_units;
   // fast kernel only: the tiles of the cross-wavefront sum are parked on top of
   // the copy rings instead of behind them.  Allowed when every workgroup owns
   // whole strips: it then sums once, after its last copy has been consumed.
@@ -127,6 +136,17 @@ __device__ __forceinline__ void part_and_slab(const int grid_parts, const int sl
   const int t = blockIdx.x >> 3;
   slab = t % slabs;
   part = (t / slabs) * 8 + (blockIdx.x & 7);
+}
+// First and last workgroup that work on `strip`.
+__device__ __forceinline__ void strip_contributors(const StreamParams& p, int strip, int& first, int& last) {
+  if (p.piece_units > 0) {
+    first = strip << p.piece_shift;
+    last = first + (1 << p.piece_shift) - 1;
+  } else {
+    const int strip_first = strip * p.units_per_strip;
+    first = range_owner(strip_first, p.total_units, p.parts);
+    last = range_owner(strip_first + p.units_per_strip - 1, p.total_units, p.parts);
+  }
 }
 // Scratch slot of workgroup `w` for a strip whose first contributor is `first`.
 __device__ __forceinline__ float4* partial_slot(const StreamParams& p, int w, int first) {
@@ -237,7 +257,8 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, uint16_t* c_
     store_c_block<T>(p, c_block, rows, strip, lane, j, v);
     return;
   }
-  const int first = range_owner(strip_first, p.total_units, p.parts);
+  int first, last;
+  strip_contributors(p, strip, first, last);
   float4* dst = partial_slot(p, part, first) + (slab * 4 + j) * 64 + lane;
   if (p.tickets) {  // read back by another workgroup of this launch: write through to memory
     unsigned long long* d = reinterpret_cast<unsigned long long*>(dst);
@@ -251,15 +272,44 @@ __device__ __forceinline__ void finish_block(const StreamParams& p, uint16_t* c_
 }
 
 // The partial tile (block of rows `slab`, column block j) that workgroup w left for a
-// strip whose first contributor is `first`, read with agent-scope loads.
+// strip whose first contributor is `first`.  NEAR: the writer ran on this workgroup's
+// XCD, whose L2 is the point of coherence for its compute units, so the load only has
+// to pass the compute unit's own cache (which cannot hold the line: this workgroup has
+// not read it since the cache was invalidated at kernel start); otherwise an
+// agent-scope load, which is answered from beyond the L2.
+template <bool NEAR>
 __device__ __forceinline__ floatx4_t load_partial_tile(const StreamParams& p, int w, int first, int slab, int j,
                                                        int lane) {
   const unsigned long long* src =
       reinterpret_cast<const unsigned long long*>(partial_slot(p, w, first) + (slab * 4 + j) * 64 + lane);
-  const unsigned long long lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-  const unsigned long long hi = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  unsigned long long lo, hi;
+  if constexpr (NEAR) {
+    lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    hi = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  } else {
+    lo = __hip_atomic_load(src, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    hi = __hip_atomic_load(src + 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
   return floatx4_t{__uint_as_float((unsigned)lo), __uint_as_float((unsigned)(lo >> 32)),
                    __uint_as_float((unsigned)hi), __uint_as_float((unsigned)(hi >> 32))};
+}
+
+// Sum of the partial tiles of workgroups first..last, four loads in flight at a time, added
+// in workgroup order.
+template <bool NEAR>
+__device__ __forceinline__ floatx4_t sum_partial_tiles(const StreamParams& p, int first, int last, int slab, int j,
+                                                       int lane) {
+  floatx4_t sum = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  for (int w0 = first; w0 <= last; w0 += 4) {
+    floatx4_t part4[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      part4[i] = load_partial_tile<NEAR>(p, w0 + i <= last ? w0 + i : last, first, slab, j, lane);
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      if (w0 + i <= last) sum += part4[i];
+  }
+  return sum;
 }
 
 // Grouped calls: the tile's row (lane & 15) goes to row `id` of C (none when
@@ -848,7 +898,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
                  "s"(p.scratch), "s"(p.size_m), "s"(p.size_n), "s"(p.num_groups), "s"(p.chunks_per_strip),
                  "s"(p.units_per_strip), "s"(p.parts), "s"(p.total_units), "s"(p.slabs), "s"(p.grid_parts),
                  "s"(p.tickets), "s"(p.ticket_stride), "s"(p.xcd_ranges), "s"(p.sum_over_rings),
-                 "s"(unit_group_shift));
+                 "s"(p.piece_shift), "s"(p.piece_units), "s"(unit_group_shift));
   int part, slab;
   if constexpr (GROUPED) {   // strip-major inside a block of slots
     part = blockIdx.x % p.grid_parts;
@@ -890,8 +940,16 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   const uint32_t ring_lds = (uint32_t)(uintptr_t)(lds_void_t*)ring;
   const uint32_t red_lds = (uint32_t)(uintptr_t)(lds_void_t*)(smem + (p.sum_over_rings ? 0 : kFastWaves * kWaveLds));
 
-  const int u_begin = range_begin(part, p.total_units, p.parts);
-  const int u_end = range_begin(part + 1, p.total_units, p.parts);
+  int u_begin, u_end, first_strip;
+  if (p.piece_units > 0) {
+    first_strip = part >> p.piece_shift;
+    u_begin = first_strip * p.units_per_strip + (part & ((1 << p.piece_shift) - 1)) * p.piece_units;
+    u_end = u_begin + p.piece_units;
+  } else {
+    u_begin = range_begin(part, p.total_units, p.parts);
+    u_end = range_begin(part + 1, p.total_units, p.parts);
+    first_strip = u_begin / p.units_per_strip;
+  }
   const bool grouped = p.num_groups > 1;
 
   FastLane<MB> fl;
@@ -940,7 +998,10 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   // one unit of weights (of SLOTS - 1 units before the first unit), so "at most that
   // many outstanding" means weights(x) and A(x) have landed.
   UnitCursor cur, fetch, fetch_w;
-  cur.set(u_begin + wave, p.units_per_strip);
+  cur.index = u_begin;
+  cur.strip = first_strip;
+  cur.unit = u_begin - first_strip * p.units_per_strip;
+  cur.advance(wave, p.units_per_strip);
   fetch_w = cur;
 #pragma unroll
   for (int sl = 0; sl < SLOTS; ++sl) {
@@ -959,7 +1020,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
 
   // the current segment starts at seg_begin, inside strip seg_strip
   int seg_begin = u_begin;
-  int seg_strip = u_begin / p.units_per_strip;
+  int seg_strip = first_strip;
   // strips of which this workgroup has left partial tiles in memory (at most two: the
   // one its range starts inside and the one it ends inside); their tickets are drawn
   // when all its units are done, so that the streaming is not held up in between
@@ -1174,37 +1235,36 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's partial tiles are in memory
       TRACE(5);
       __builtin_amdgcn_s_barrier();                      // ... and every wavefront's; all LDS traffic is over
+      // A ticket counts arrivals per XCD, four bits each (the host keeps a strip to at most
+      // 15 contributors): their sum says who is last, and a single non-zero field that every
+      // contributor ran on one XCD.
+      const unsigned int xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7u;   // XCC_ID: the XCD this workgroup runs on
       if (wave == 0 && lane < pending) {
         const int strip = lane == 0 ? pending_strip[0] : pending_strip[1];
-        const int first = range_owner(strip * p.units_per_strip, p.total_units, p.parts);
+        int first, last;
+        strip_contributors(p, strip, first, last);
         unsigned int* ticket = p.tickets + ((long)first * p.slabs + slab) * p.ticket_stride;
-        const unsigned int drawn = __hip_atomic_fetch_add(ticket, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(flag_lds + 4u * lane), "v"(drawn) : "memory");
+        const unsigned int mine = 1u << (4u * xcc);
+        const unsigned int now = mine + __hip_atomic_fetch_add(ticket, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(flag_lds + 4u * lane), "v"(now) : "memory");
       }
       __builtin_amdgcn_s_barrier();
       TRACE(6);
       for (int k = 0; k < pending; ++k) {
-        uint32_t drawn;
-        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(drawn) : "v"(flag_lds + 4u * k) : "memory");
-        drawn = __builtin_amdgcn_readfirstlane(drawn);
+        uint32_t now;
+        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(now) : "v"(flag_lds + 4u * k) : "memory");
+        now = __builtin_amdgcn_readfirstlane(now);
         const int strip = k == 0 ? pending_strip[0] : pending_strip[1];
-        const int strip_first = strip * p.units_per_strip;
-        const int first = range_owner(strip_first, p.total_units, p.parts);
-        const int last = range_owner(strip_first + p.units_per_strip - 1, p.total_units, p.parts);
-        if ((int)drawn != last - first) continue;   // somebody is still at work on this strip
+        int first, last;
+        strip_contributors(p, strip, first, last);
+        const unsigned int pairs = (now & 0x0f0f0f0fu) + ((now >> 4) & 0x0f0f0f0fu);
+        const int arrived = (int)((pairs * 0x01010101u) >> 24);
+        if (arrived != last - first + 1) continue;   // somebody is still at work on this strip
+        const bool near = now == ((unsigned int)(last - first + 1) << (4u * xcc));
         for (int t = wave; t < 4 * MB; t += kFastWaves) {
           const int mb = t >> 2, j = t & 3;
-          // four loads in flight at a time, added in workgroup order
-          floatx4_t sum = floatx4_t{0.f, 0.f, 0.f, 0.f};
-          for (int w0 = first; w0 <= last; w0 += 4) {
-            floatx4_t part4[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              part4[i] = load_partial_tile(p, w0 + i <= last ? w0 + i : last, first, slab * MB + mb, j, lane);
-#pragma unroll
-            for (int i = 0; i < 4; ++i)
-              if (w0 + i <= last) sum += part4[i];
-          }
+          const floatx4_t sum = near ? sum_partial_tiles<true>(p, first, last, slab * MB + mb, j, lane)
+                                     : sum_partial_tiles<false>(p, first, last, slab * MB + mb, j, lane);
           store_c_block<T>(p, p.c + (long)(16 * mb) * p.size_n, p.size_m - 16 * mb, strip, lane, j, sum);
         }
         if (threadIdx.x == 0)
@@ -1668,6 +1728,8 @@ int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.slabs = (int)((sorted_len + moe_block_size - 1) / moe_block_size) * p.sub_blocks;   // blocks of slots x halves
   p.grid_parts = n_strips;
   p.sum_over_rings = 1;                     // every workgroup owns a whole strip
+  p.piece_shift = 0;
+  p.piece_units = p.units_per_strip;
   p.sorted_ids = sorted_ids;
   p.expert_ids = expert_ids;
   p.num_post_pad = num_post_pad;
@@ -1710,9 +1772,7 @@ size_t stream_scratch_bytes() { return (size_t)2 * cu_count() * kSlotFloat4 * si
 }  // namespace
 
 #ifdef SONAR_TRACE
-extern "C" void sonar_debug_set_trace(void* ptr) {
-  (void)hipMemcpyToSymbol(HIP_SYMBOL(sonar::g_trace), &ptr, sizeof(ptr));
-}
+extern "C" void sonar_debug_set_trace(void* ptr) { sonar::g_trace_host = (unsigned long long*)ptr; }
 #endif
 
 extern "C" size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k) {
@@ -1774,6 +1834,9 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                 "(the column-permuted copy of A)");
 
   StreamParams p = {};
+#ifdef SONAR_TRACE
+  p.trace = g_trace_host;
+#endif
   p.b = reinterpret_cast<const uint4*>(b_q_weight);
   p.bias = static_cast<const uint16_t*>(b_bias);
   p.scales = static_cast<const uint16_t*>(b_scales);
@@ -1856,14 +1919,21 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   static const char* split_env = getenv("SONAR_MARLIN_SPLIT");
   const bool piece_split = fast_shape && p.unit_chunks == 4 && size_m <= 16 && !no_inline_sum &&
                            n_strips * n_strips * p.units_per_strip < (1LL << 31);
-  int pieces = 1;
+  int pieces = 1, piece_shift = 0, piece_units = 0;
   if (piece_split) {
     pieces = (int)(cus / n_strips);
-    if (split_env) pieces = atoi(split_env);
+    if (split_env && atoi(split_env) < pieces) pieces = atoi(split_env);   // never more parts than scratch slots
     if (pieces > p.units_per_strip) pieces = p.units_per_strip;
-    if (pieces > 16) pieces = 16;
+    if (pieces > 15) pieces = 15;   // a ticket field counts up to 15 contributors
     if (pieces < 1) pieces = 1;
     if (n_strips * pieces > workspace_len) pieces = 1;
+    // equal pieces, a power of two of them, when the strip can be cut that way
+    int shift = 0;
+    while ((2 << shift) <= pieces && p.units_per_strip % (2 << shift) == 0) ++shift;
+    if ((1 << shift) == pieces) {
+      piece_shift = shift;
+      piece_units = p.units_per_strip >> shift;
+    }
     p.parts = (int)n_strips * pieces;   // range_begin(strip * pieces + i) = strip * units_per_strip + i * units_per_strip / pieces
   } else if (strip_per_workgroup && (p.unit_chunks == 4 || row_slabs)) {
     p.parts = (int)n_strips;
@@ -1874,10 +1944,17 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   p.tickets = nullptr;
   p.ticket_stride = 1;
   p.xcd_ranges = 0;
+  p.piece_shift = piece_shift;
+  p.piece_units = piece_units;
 
   bool any_split = false;
   for (int i = 1; i < p.parts && !any_split; ++i)
     any_split = range_begin(i, p.total_units, p.parts) % p.units_per_strip != 0;
+
+  // a split strip leaves one partial tile set per contributor in scratch slot `part` or `parts + part`
+  if (any_split && !use_tile)
+    SONAR_REQUIRE((size_t)2 * p.parts * kSlotFloat4 * sizeof(float4) <= stream_scratch_bytes(),
+                  "internal: %d parts share strips but the scratch has slots for %d", p.parts, cus);
 
   if (use_tile) {
     const size_t used = stream_scratch_bytes();
@@ -1916,7 +1993,9 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
       }
       // Shared strips are summed inside the kernel when the workspace has a ticket for every
       // part and block of rows; tickets four words apart do not hold each other up.
-      inline_sum = any_split && !no_inline_sum && (int64_t)p.parts * p.slabs <= workspace_len;
+      const int smallest_part = p.total_units / p.parts;   // parts <= total_units
+      const int contributors = (p.units_per_strip + smallest_part - 1) / smallest_part + 1;   // upper bound
+      inline_sum = any_split && !no_inline_sum && (int64_t)p.parts * p.slabs <= workspace_len && contributors <= 15;
       if (inline_sum) {
         p.tickets = reinterpret_cast<unsigned int*>(workspace);
         const int64_t room = workspace_len / ((int64_t)p.parts * p.slabs);
