@@ -94,10 +94,6 @@ struct StreamParams {
   // split (a wavefront's scalar unit is shared with seven others: the index arithmetic
   // of the general split alone took about 0.4 us before the first copy was issued)
   int piece_shift, piece_units;
-  // fast kernel only: the tiles of the cross-wavefront sum are parked on top of
-  // the copy rings instead of behind them.  Allowed when every workgroup owns
-  // whole strips: it then sums once, after its last copy has been consumed.
-  int sum_over_rings;
   // grouped (mixture-of-experts) calls of the fast kernel only: workgroup
   // block * grid_parts + strip works on the slots [block * block_size, ...) of
   // sorted_ids with the weights of expert_ids[block]; blocks of 48 and 64 slots
@@ -136,17 +132,6 @@ __device__ __forceinline__ void part_and_slab(const int grid_parts, const int sl
   const int t = blockIdx.x >> 3;
   slab = t % slabs;
   part = (t / slabs) * 8 + (blockIdx.x & 7);
-}
-// First and last workgroup that work on `strip`.
-__device__ __forceinline__ void strip_contributors(const StreamParams& p, int strip, int& first, int& last) {
-  if (p.piece_units > 0) {
-    first = strip << p.piece_shift;
-    last = first + (1 << p.piece_shift) - 1;
-  } else {
-    const int strip_first = strip * p.units_per_strip;
-    first = range_owner(strip_first, p.total_units, p.parts);
-    last = range_owner(strip_first + p.units_per_strip - 1, p.total_units, p.parts);
-  }
 }
 // Scratch slot of workgroup `w` for a strip whose first contributor is `first`.
 __device__ __forceinline__ float4* partial_slot(const StreamParams& p, int w, int first) {
@@ -248,18 +233,11 @@ __device__ __forceinline__ void store_c_block(const StreamParams& p, uint16_t* c
   }
 }
 
-template <typename T>
-__device__ __forceinline__ void finish_block(const StreamParams& p, uint16_t* c_block, int rows, int part, int slab,
-                                             int strip, int seg_begin, int seg_end, int lane, int j, floatx4_t v) {
-  const int strip_first = strip * p.units_per_strip;
-  const int strip_end = strip_first + p.units_per_strip;
-  if (seg_begin == strip_first && seg_end == strip_end) {
-    store_c_block<T>(p, c_block, rows, strip, lane, j, v);
-    return;
-  }
-  int first, last;
-  strip_contributors(p, strip, first, last);
-  float4* dst = partial_slot(p, part, first) + (slab * 4 + j) * 64 + lane;
+// One 16 x 16 fp32 block of a strip that several workgroups share goes to this
+// workgroup's scratch slot (`tile` = 4 x block of rows + column block).
+__device__ __forceinline__ void store_partial_block(const StreamParams& p, int part, int first, int tile, int lane,
+                                                    floatx4_t v) {
+  float4* dst = partial_slot(p, part, first) + tile * 64 + lane;
   if (p.tickets) {  // read back by another workgroup of this launch: write through to memory
     unsigned long long* d = reinterpret_cast<unsigned long long*>(dst);
     const unsigned long long lo = ((unsigned long long)__float_as_uint(v.y) << 32) | __float_as_uint(v.x);
@@ -671,20 +649,21 @@ constexpr int kSlotS = 4096;       // inside a weight slot, after 4 chunks x 1 K
 // or more, 2 / 4 for groups of 64 / 32 rows): one 256-byte scale / zero-point
 // row per group follows the four chunks of a weight slot.
 constexpr int slot_bytes(int gpu) { return 4096 + 256 * gpu; }
-constexpr int wave_a(int gpu, int slots = 2) { return slots * slot_bytes(gpu); }   // the activation slot follows the weight slots
+constexpr int wave_a(int gpu) { return 2 * slot_bytes(gpu); }   // the activation slot follows the two weight slots
 // LDS bytes per wavefront: the activation slot holds 4 KiB per block of 16 rows
-constexpr int wave_lds(int mb, int gpu = 1, int slots = 2) { return slots * slot_bytes(gpu) + 4096 * mb; }
+constexpr int wave_lds(int mb, int gpu = 1) { return 2 * slot_bytes(gpu) + 4096 * mb; }
 // Tiles (16 x 16 fp32, 1 KiB) a wavefront parks per pass of the cross-wavefront
 // sum: all four of its one block of rows, or two of the eight of two blocks
 // (four passes), which keeps 8 wavefronts with two blocks inside 160 KiB.
 constexpr int park_tiles(int mb) { return mb == 1 ? 4 : 2; }
 constexpr int weight_copies(int gpu) { return 4 + gpu; }   // asynchronous copies per unit: 4 weight chunks + the scale rows
 // A workgroup of the fast kernel has 8 wavefronts (one workgroup per compute
-// unit), or 4 (two per compute unit: a grid with more workgroups than compute
-// units then runs them side by side instead of one after the other).
-constexpr int fast_lds_bytes(int waves, int mb, int gpu = 1, int slots = 2) {
-  return waves * (wave_lds(mb, gpu, slots) + park_tiles(mb) * 1024);
-}
+// unit), or 4 (three per compute unit: a grid with more workgroups than compute
+// units then runs them side by side instead of one after the other).  The tiles of
+// the cross-wavefront sum are parked on top of the copy rings.
+constexpr int fast_lds_bytes(int waves, int mb, int gpu = 1) { return waves * wave_lds(mb, gpu); }
+static_assert(fast_lds_bytes(4, 1) >= 4 * park_tiles(1) * 1024 && fast_lds_bytes(4, 2) >= 4 * park_tiles(2) * 1024,
+              "the parked tiles must fit the rings");
 
 // Row id of C of row `r` of block `block` of a grouped call, -1 for padding.
 __device__ __forceinline__ int moe_row_id(const StreamParams& p, int block, int r) {
@@ -745,24 +724,6 @@ __device__ __forceinline__ void copy_activations(const StreamParams& p, const Fa
     __builtin_amdgcn_global_load_lds((glb_void_t*)(ga + 128 + fl.a_off[2 * mb + 1]), (lds_void_t*)(s + 3072), 16, 0, 0);
   }
 }
-
-struct UnitCursor {
-  int index;
-  int strip, unit;
-  __device__ __forceinline__ void set(int u, int units_per_strip) {
-    index = u;
-    strip = u / units_per_strip;
-    unit = u - strip * units_per_strip;
-  }
-  __device__ __forceinline__ void advance(int by, int units_per_strip) {
-    index += by;
-    unit += by;
-    while (unit >= units_per_strip) {
-      unit -= units_per_strip;
-      ++strip;
-    }
-  }
-};
 
 // Forming (v - z) * s per weight costs 13 VALU instructions per packed word in
 // fp16 and 17 in bf16 (gfx950 has no packed bf16 arithmetic), more than the
@@ -831,6 +792,31 @@ __device__ __forceinline__ u32x4_t raw_operand(uint32_t q, uint32_t magic) {
       : "v"(q_at), "v"(a_at), "v"(z_at), "v"(s_at), "v"(a_at ^ 64u)                                \
       : "memory")
 
+// The same with the 16 scales fetched as four 16-byte vectors (grouped scales, whose
+// permuted row holds the scales of columns 16 j + 4 (lane / 16) + r, j = 0..3, as the
+// low (lane / 32 == 0) or high 16 bits of the four words at byte 64 ((lane / 16) & 1) + 16 r):
+// 4 LDS instructions instead of 16.
+#define SONAR_UNIT_READS_VEC()                                                                     \
+  asm volatile(                                                                                    \
+      "ds_read_b128 %0, %13\n\t"                                                                   \
+      "ds_read_b128 %1, %13 offset:1024\n\t"                                                       \
+      "ds_read_b128 %2, %13 offset:2048\n\t"                                                       \
+      "ds_read_b128 %3, %13 offset:3072\n\t"                                                       \
+      "ds_read_b128 %4, %14\n\t"                                                                   \
+      "ds_read_b128 %5, %17\n\t"                                                                   \
+      "ds_read_b128 %6, %14 offset:2048\n\t"                                                       \
+      "ds_read_b128 %7, %17 offset:2048\n\t"                                                       \
+      "ds_read_b128 %8, %15\n\t"                                                                   \
+      "ds_read_b128 %9, %16\n\t"                                                                   \
+      "ds_read_b128 %10, %16 offset:16\n\t"                                                        \
+      "ds_read_b128 %11, %16 offset:32\n\t"                                                        \
+      "ds_read_b128 %12, %16 offset:48\n\t"                                                        \
+      "s_waitcnt lgkmcnt(0)"                                                                       \
+      : "=&v"(q0), "=&v"(q1), "=&v"(q2), "=&v"(q3), "=&v"(a0), "=&v"(a1), "=&v"(a2), "=&v"(a3),    \
+        "=&v"(row_z), "=&v"(sv0), "=&v"(sv1), "=&v"(sv2), "=&v"(sv3)                               \
+      : "v"(q_at), "v"(a_at), "v"(z_at), "v"(sv_at), "v"(a_at ^ 64u)                               \
+      : "memory")
+
 // The activation operands of a second block of 16 rows (4 KiB after the first).
 #define SONAR_UNIT_READS_ROWS2(B0, B1, B2, B3)                                                      \
   asm volatile(                                                                                    \
@@ -873,17 +859,20 @@ __device__ __forceinline__ u32x4_t raw_operand(uint32_t q, uint32_t magic) {
 // GPU: groups per 128-row unit (2 or 4 for groups of 64 or 32 rows, else 1).
 // FP4 (with GPU = 4, no zero points): float4_e2m1f codes; the operands are the
 // converted values themselves, so only the scale is left for after the unit.
-// SLOTS: weight slots per wavefront, i.e. units of weights in flight.  Three were measured
-// slower than two on every Llama-3-8B shape (M = 16: down 12.2 against 11.4 us, gate_up
-// 19.1 against 17.4), so only two are instantiated.
-template <typename T, bool HAS_ZP, int kFastWaves, int MB, bool GROUPED = false, int GPU = 1, bool FP4 = false,
-          int SLOTS = 2>
+// A workgroup works on one piece of one strip (StreamParams::piece_shift / piece_units):
+// units unit0 .. unit0 + piece_units - 1 of strip `part >> piece_shift`, dealt round-robin
+// to its wavefronts.  It sums its wavefronts once, at the end (the tiles of that sum are
+// parked on top of the copy rings, every copy having been consumed by then), and either
+// writes C (the piece is the whole strip) or leaves fp32 partial tiles and draws the
+// strip's ticket.  (A third weight slot per wavefront was measured slower than two on every
+// Llama-3-8B shape: M = 16, down 12.2 against 11.4 us, gate_up 19.1 against 17.4.)
+template <typename T, bool HAS_ZP, int kFastWaves, int MB, bool GROUPED = false, int GPU = 1, bool FP4 = false>
 __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(const StreamParams params,
                                                                              const int unit_group_shift) {
   typedef typename Dq<T>::vec8 vec8;
-  constexpr int kWaveLds = wave_lds(MB, GPU, SLOTS);
+  constexpr int kWaveLds = wave_lds(MB, GPU);
   constexpr int kSlotBytes = slot_bytes(GPU);
-  constexpr int kWaveA = wave_a(GPU, SLOTS);
+  constexpr int kWaveA = wave_a(GPU);
   constexpr int kWeightCopies = weight_copies(GPU);
   constexpr int kPark = park_tiles(MB);       // tiles per wavefront and pass of the cross-wavefront sum
   constexpr int kPasses = 4 * MB / kPark;
@@ -892,13 +881,13 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   StreamParams p = params;
   // Every argument the dense path reads, fetched now in one batch of scalar loads: left to
   // itself the compiler fetches them where they are first used, four round trips to a cold
-  // argument buffer one after the other (about 2 us of a kernel that takes 6).
+  // argument buffer one after the other.
   if constexpr (!GROUPED)
     asm volatile("" ::"s"(p.a), "s"(p.lda), "s"(p.c), "s"(p.b), "s"(p.bias), "s"(p.scales), "s"(p.zeros),
                  "s"(p.scratch), "s"(p.size_m), "s"(p.size_n), "s"(p.num_groups), "s"(p.chunks_per_strip),
-                 "s"(p.units_per_strip), "s"(p.parts), "s"(p.total_units), "s"(p.slabs), "s"(p.grid_parts),
-                 "s"(p.tickets), "s"(p.ticket_stride), "s"(p.xcd_ranges), "s"(p.sum_over_rings),
-                 "s"(p.piece_shift), "s"(p.piece_units), "s"(unit_group_shift));
+                 "s"(p.units_per_strip), "s"(p.parts), "s"(p.slabs), "s"(p.grid_parts), "s"(p.tickets),
+                 "s"(p.ticket_stride), "s"(p.xcd_ranges), "s"(p.piece_shift), "s"(p.piece_units),
+                 "s"(unit_group_shift));
   int part, slab;
   if constexpr (GROUPED) {   // strip-major inside a block of slots
     part = blockIdx.x % p.grid_parts;
@@ -938,18 +927,13 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   const int col16 = lane & 15;
   char* ring = smem + wave * kWaveLds;
   const uint32_t ring_lds = (uint32_t)(uintptr_t)(lds_void_t*)ring;
-  const uint32_t red_lds = (uint32_t)(uintptr_t)(lds_void_t*)(smem + (p.sum_over_rings ? 0 : kFastWaves * kWaveLds));
+  const uint32_t red_lds = (uint32_t)(uintptr_t)(lds_void_t*)smem;
 
-  int u_begin, u_end, first_strip;
-  if (p.piece_units > 0) {
-    first_strip = part >> p.piece_shift;
-    u_begin = first_strip * p.units_per_strip + (part & ((1 << p.piece_shift) - 1)) * p.piece_units;
-    u_end = u_begin + p.piece_units;
-  } else {
-    u_begin = range_begin(part, p.total_units, p.parts);
-    u_end = range_begin(part + 1, p.total_units, p.parts);
-    first_strip = u_begin / p.units_per_strip;
-  }
+  // this workgroup's piece and this wavefront's share of it: units unit, unit + kFastWaves, ...
+  const int strip = part >> p.piece_shift;
+  const int pieces = 1 << p.piece_shift;
+  int unit = (part & (pieces - 1)) * p.piece_units + wave;
+  const int mine = wave < p.piece_units ? (p.piece_units - wave + kFastWaves - 1) / kFastWaves : 0;
   const bool grouped = p.num_groups > 1;
 
   FastLane<MB> fl;
@@ -986,137 +970,33 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   const uint32_t row_s_off = kSlotS + (grouped ? 64 * (q4 & 1) + 2 * (q4 >> 1) : 32 * (q4 & 1) + 4 * (q4 >> 1));
   const uint32_t row_z_off = kSlotS + 128 + 16 * (q4 & 1);
   const uint32_t row_z_shift = 16 * (q4 >> 1);
+  // bfloat16 scales of one group per unit: row_s holds float bits
+  constexpr bool kVecScales = sizeof(typename Dq<T>::vec8) == 16 && __is_same(T, __bf16) && GPU == 1;
+  const uint32_t scale_half = (q4 >> 1) ? 0x07060c0cu : 0x05040c0cu;   // byte selector: high or low 16 bits, shifted up
   const uint32_t magic = magic_register(RawOperand<T>::kMagic);
   u32x4_t ones = u32x4_t{RawOperand<T>::kOnes, RawOperand<T>::kOnes, RawOperand<T>::kOnes, RawOperand<T>::kOnes};
   asm("" : "+v"(ones));
 
-  // Issue order of a wavefront's copies, x being one of its units and W the
-  // distance to its next one (two slots):  weights(x) | A(x), weights(x+W) | A(x+W),
-  // weights(x+2W) | ...; with three slots weights(x+2W) follows weights(x+W) at the
-  // start and every later A(y) is followed by weights(y+2W).  They complete in this
-  // order.  When the arithmetic of x starts, the copies younger than A(x) are those of
-  // one unit of weights (of SLOTS - 1 units before the first unit), so "at most that
-  // many outstanding" means weights(x) and A(x) have landed.
-  UnitCursor cur, fetch, fetch_w;
-  cur.index = u_begin;
-  cur.strip = first_strip;
-  cur.unit = u_begin - first_strip * p.units_per_strip;
-  cur.advance(wave, p.units_per_strip);
-  fetch_w = cur;
-#pragma unroll
-  for (int sl = 0; sl < SLOTS; ++sl) {
-    if (fetch_w.index < u_end) {
-      copy_weights<MB, GPU>(p, fl, fetch_w.strip, fetch_w.unit, ring + sl * kSlotBytes, lane, unit_group_shift);
-      if (sl == 0) copy_activations<MB>(p, fl, fetch_w.unit, ring + kWaveA);
-    }
-    fetch_w.advance(kFastWaves, p.units_per_strip);
+  // Issue order of a wavefront's copies, x being one of its units and W the distance
+  // to its next one:  weights(x) | A(x), weights(x+W) | A(x+W), weights(x+2W) | ...
+  // They complete in this order.  When the arithmetic of x starts, the only copies
+  // younger than A(x) are those of weights(x+W), so "at most that many outstanding"
+  // means weights(x) and A(x) have landed.
+  if (mine > 0) {
+    copy_weights<MB, GPU>(p, fl, strip, unit, ring, lane, unit_group_shift);
+    copy_activations<MB>(p, fl, unit, ring + kWaveA);
   }
-  // `fetch` names the unit whose A slice is copied next, `fetch_w` the one whose weights are
-  fetch = cur;
-  fetch.advance(kFastWaves, p.units_per_strip);
+  if (mine > 1) copy_weights<MB, GPU>(p, fl, strip, unit + kFastWaves, ring + kSlotBytes, lane, unit_group_shift);
   int c_slot = 0;
-  bool first_unit = true;
   TRACE(1);
 
-  // the current segment starts at seg_begin, inside strip seg_strip
-  int seg_begin = u_begin;
-  int seg_strip = first_strip;
-  // strips of which this workgroup has left partial tiles in memory (at most two: the
-  // one its range starts inside and the one it ends inside); their tickets are drawn
-  // when all its units are done, so that the streaming is not held up in between
-  int pending_strip[2] = {0, 0};
-  int pending = 0;
   floatx4_t acc[MB][4];
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb)
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
 
-  for (;;) {
-    const bool have = cur.index < u_end;
-    // Close every strip segment that ends before this wavefront's next unit:
-    // in each pass every wavefront parks kPark of its tiles in LDS and
-    // wavefront w (w < kPark) adds up one column block of one block of rows in
-    // wavefront order and finishes it.
-    while (seg_begin < u_end) {
-      const int strip = seg_strip;
-      const int strip_end = (strip + 1) * p.units_per_strip;
-      const int seg_end = u_end < strip_end ? u_end : strip_end;
-      if (have && cur.index < seg_end) break;
-#pragma unroll
-      for (int ps = 0; ps < kPasses; ++ps) {
-        const int mb = ps * kPark / 4, jb = ps * kPark % 4;
-        __builtin_amdgcn_s_barrier();  // the previous pass's tiles have been consumed
-        const uint32_t park = red_lds + (wave * kPark * 64 + lane) * 16;
-        // the tiles come out of the matrix cores; an asm block is opaque to the
-        // compiler's hazard padding, so give the last MFMA time to retire
-        if constexpr (kPark == 4) {
-          asm volatile(
-              "s_nop 15\n\t"
-              "s_nop 15\n\t"
-              "ds_write_b128 %0, %1\n\t"
-              "ds_write_b128 %0, %2 offset:1024\n\t"
-              "ds_write_b128 %0, %3 offset:2048\n\t"
-              "ds_write_b128 %0, %4 offset:3072\n\t"
-              "s_waitcnt lgkmcnt(0)"
-              :
-              : "v"(park), "v"(acc[mb][0]), "v"(acc[mb][1]), "v"(acc[mb][2]), "v"(acc[mb][3])
-              : "memory");
-        } else {
-          asm volatile(
-              "s_nop 15\n\t"
-              "s_nop 15\n\t"
-              "ds_write_b128 %0, %1\n\t"
-              "ds_write_b128 %0, %2 offset:1024\n\t"
-              "s_waitcnt lgkmcnt(0)"
-              :
-              : "v"(park), "v"(acc[mb][jb]), "v"(acc[mb][jb + 1])
-              : "memory");
-        }
-        __builtin_amdgcn_s_barrier();
-        if (wave < kPark) {
-          floatx4_t sum = floatx4_t{0.f, 0.f, 0.f, 0.f};
-          const uint32_t src = red_lds + (wave * 64 + lane) * 16;
-#pragma unroll
-          for (int w = 0; w < kFastWaves; w += 4) {
-            floatx4_t t0, t1, t2, t3;
-            asm volatile(
-                "ds_read_b128 %0, %4\n\t"
-                "ds_read_b128 %1, %4 offset:%5\n\t"
-                "ds_read_b128 %2, %4 offset:%6\n\t"
-                "ds_read_b128 %3, %4 offset:%7\n\t"
-                "s_waitcnt lgkmcnt(0)"
-                : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
-                : "v"(src + w * kPark * 1024), "n"(kPark * 1024), "n"(2 * kPark * 1024), "n"(3 * kPark * 1024)
-                : "memory");
-            sum += t0;
-            sum += t1;
-            sum += t2;
-            sum += t3;
-          }
-          if constexpr (GROUPED)
-            finish_block_grouped<T>(p, row_id[mb], strip, lane, jb + wave, sum);
-          else
-            finish_block<T>(p, p.c + (long)(16 * mb) * p.size_n, p.size_m - 16 * mb, part, slab * MB + mb, strip,
-                            seg_begin, seg_end, lane, jb + wave, sum);
-        }
-      }
-#pragma unroll
-      for (int mb = 0; mb < MB; ++mb)
-#pragma unroll
-        for (int j = 0; j < 4; ++j) acc[mb][j] = floatx4_t{0.f, 0.f, 0.f, 0.f};
-      if constexpr (!GROUPED) {
-        if (seg_begin != strip * p.units_per_strip || seg_end != strip_end) {
-          if (pending == 0) pending_strip[0] = strip;
-          else pending_strip[1] = strip;
-          ++pending;
-        }
-      }
-      seg_begin = seg_end;
-      ++seg_strip;
-    }
-    if (!have) break;
-
+  for (int left = mine; left > 0; --left) {
     // One unit: wait for its copies, pull them into registers, start the
     // copies of the units after it, then do the arithmetic.
     const uint32_t slot_lds = ring_lds + c_slot * kSlotBytes;
@@ -1126,28 +1006,31 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     u32x4_t row_z = u32x4_t{0u, 0u, 0u, 0u};
     uint32_t more_s[GPU > 1 ? GPU - 1 : 1][16];   // the other groups of the unit
     u32x4_t more_z[GPU > 1 ? GPU - 1 : 1];
-    // this wavefront's units after the current one
-    const int after = (u_end - 1 - cur.index) / kFastWaves;
-    const bool more = after >= 1;
-    {
-      // units of weights whose copies were issued after those of A(x)
-      const int younger = first_unit ? (after < SLOTS - 1 ? after : SLOTS - 1) : (after >= SLOTS - 1 ? 1 : 0);
-      if (younger == 0) {
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-      } else if (SLOTS == 2 || younger == 1) {
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightCopies) : "memory");
-      } else {
-        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * kWeightCopies) : "memory");
-      }
-      first_unit = false;
+    if (left > 1) {
+      asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kWeightCopies) : "memory");
+    } else {
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     }
     {
       const uint32_t q_at = slot_lds + lane * 16;
       const uint32_t z_at = slot_lds + row_z_off, s_at = slot_lds + row_s_off;
-      if (grouped) {  // scale of (j, r) at byte 16 r + 4 j past s_at
+      if (kVecScales && grouped) {   // bfloat16: the float bits of a scale are a byte permute of its word
+        const uint32_t sv_at = slot_lds + kSlotS + 64 * (q4 & 1);
+        u32x4_t sv0, sv1, sv2, sv3;
+        SONAR_UNIT_READS_VEC();
+        const u32x4_t sv[4] = {sv0, sv1, sv2, sv3};
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int r = 0; r < 4; ++r) row_s[4 * j + r] = __builtin_amdgcn_perm(sv[r][j], 0u, scale_half);
+      } else if (grouped) {  // scale of (j, r) at byte 16 r + 4 j past s_at
         SONAR_UNIT_READS(0, 16, 32, 48, 4, 20, 36, 52, 8, 24, 40, 56, 12, 28, 44, 60);
       } else {        // at byte 64 (j >> 1) + 8 (j & 1) + 16 (r >> 1) + 2 (r & 1)
         SONAR_UNIT_READS(0, 2, 16, 18, 8, 10, 24, 26, 64, 66, 80, 82, 72, 74, 88, 90);
+      }
+      if (kVecScales && !grouped) {
+#pragma unroll
+        for (int i = 0; i < 16; ++i) row_s[i] <<= 16;
       }
       if constexpr (MB == 2) SONAR_UNIT_READS_ROWS2(b0, b1, b2, b3);
       if constexpr (GPU >= 2) SONAR_GROUP_READS(1);
@@ -1157,22 +1040,19 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
       }
     }
     TRACE(2);
-    if (more) {
-      copy_activations<MB>(p, fl, fetch.unit, ring + kWaveA);
-      fetch.advance(kFastWaves, p.units_per_strip);
-      if (fetch_w.index < u_end) {
-        copy_weights<MB, GPU>(p, fl, fetch_w.strip, fetch_w.unit, ring + c_slot * kSlotBytes, lane,
+    if (left > 1) {
+      copy_activations<MB>(p, fl, unit + kFastWaves, ring + kWaveA);
+      if (left > 2)
+        copy_weights<MB, GPU>(p, fl, strip, unit + 2 * kFastWaves, ring + c_slot * kSlotBytes, lane,
                               unit_group_shift);
-        fetch_w.advance(kFastWaves, p.units_per_strip);
-      }
     }
+    unit += kFastWaves;
+    c_slot ^= 1;
 
 #ifdef SONAR_EXP_NO_COMPUTE
     {
       const u32x4_t x = q0 ^ q1 ^ q2 ^ q3 ^ a0 ^ a1 ^ a2 ^ a3 ^ row_z;
       acc[0][0][0] += __uint_as_float((x.x ^ x.y ^ x.z ^ x.w ^ row_s[0] ^ row_s[15]) & 0x3fffffu);
-      cur.advance(kFastWaves, p.units_per_strip);
-      c_slot = c_slot + 1 == SLOTS ? 0 : c_slot + 1;
       continue;
     }
 #endif
@@ -1211,7 +1091,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
           const uint32_t sbits = gi == 0 ? row_s[4 * j + r] : more_s[gi == 0 ? 0 : gi - 1][4 * j + r];
-          const float sc = Dq<T>::to_float((uint16_t)sbits);
+          const float sc = (kVecScales && gi == 0) ? __uint_as_float(sbits) : Dq<T>::to_float((uint16_t)sbits);
           float off = -(RawOperand<T>::kBase + 8.f);
           if (HAS_ZP) off = -RawOperand<T>::kBase - (float)((zrow[r] >> (4 * j)) & 0xFu);
 #pragma unroll
@@ -1221,16 +1101,84 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
           }
         }
     }
-    cur.advance(kFastWaves, p.units_per_strip);
-    c_slot = c_slot + 1 == SLOTS ? 0 : c_slot + 1;
     TRACE(3);
   }
   TRACE(4);
 
-  // Strips shared with other workgroups: draw their tickets; whoever holds the last
-  // ticket of a strip adds its partial tiles up.
+  // The cross-wavefront sum: in each pass every wavefront parks kPark of its tiles in
+  // LDS and wavefront w (w < kPark) adds up one column block of one block of rows in
+  // wavefront order and finishes it.
+  int first = 0, last = 0;   // the workgroups that share this strip
   if constexpr (!GROUPED) {
-    if (p.tickets != nullptr && pending > 0) {
+    first = strip << p.piece_shift;
+    last = first + pieces - 1;
+  }
+#pragma unroll
+  for (int ps = 0; ps < kPasses; ++ps) {
+    const int mb = ps * kPark / 4, jb = ps * kPark % 4;
+    __builtin_amdgcn_s_barrier();  // every copy has been consumed; the previous pass's tiles too
+    const uint32_t park = red_lds + (wave * kPark * 64 + lane) * 16;
+    // the tiles come out of the matrix cores; an asm block is opaque to the
+    // compiler's hazard padding, so give the last MFMA time to retire
+    if constexpr (kPark == 4) {
+      asm volatile(
+          "s_nop 15\n\t"
+          "s_nop 15\n\t"
+          "ds_write_b128 %0, %1\n\t"
+          "ds_write_b128 %0, %2 offset:1024\n\t"
+          "ds_write_b128 %0, %3 offset:2048\n\t"
+          "ds_write_b128 %0, %4 offset:3072\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          :
+          : "v"(park), "v"(acc[mb][0]), "v"(acc[mb][1]), "v"(acc[mb][2]), "v"(acc[mb][3])
+          : "memory");
+    } else {
+      asm volatile(
+          "s_nop 15\n\t"
+          "s_nop 15\n\t"
+          "ds_write_b128 %0, %1\n\t"
+          "ds_write_b128 %0, %2 offset:1024\n\t"
+          "s_waitcnt lgkmcnt(0)"
+          :
+          : "v"(park), "v"(acc[mb][jb]), "v"(acc[mb][jb + 1])
+          : "memory");
+    }
+    __builtin_amdgcn_s_barrier();
+    if (wave < kPark) {
+      floatx4_t sum = floatx4_t{0.f, 0.f, 0.f, 0.f};
+      const uint32_t src = red_lds + (wave * 64 + lane) * 16;
+#pragma unroll
+      for (int w = 0; w < kFastWaves; w += 4) {
+        floatx4_t t0, t1, t2, t3;
+        asm volatile(
+            "ds_read_b128 %0, %4\n\t"
+            "ds_read_b128 %1, %4 offset:%5\n\t"
+            "ds_read_b128 %2, %4 offset:%6\n\t"
+            "ds_read_b128 %3, %4 offset:%7\n\t"
+            "s_waitcnt lgkmcnt(0)"
+            : "=&v"(t0), "=&v"(t1), "=&v"(t2), "=&v"(t3)
+            : "v"(src + w * kPark * 1024), "n"(kPark * 1024), "n"(2 * kPark * 1024), "n"(3 * kPark * 1024)
+            : "memory");
+        sum += t0;
+        sum += t1;
+        sum += t2;
+        sum += t3;
+      }
+      const int j = jb + wave;
+      if constexpr (GROUPED) {
+        finish_block_grouped<T>(p, row_id[mb], strip, lane, j, sum);
+      } else if (pieces == 1) {
+        store_c_block<T>(p, p.c + (long)(16 * mb) * p.size_n, p.size_m - 16 * mb, strip, lane, j, sum);
+      } else {
+        store_partial_block(p, part, first, (slab * MB + mb) * 4 + j, lane, sum);
+      }
+    }
+  }
+
+  // A strip shared with other workgroups: draw its ticket; whoever holds the last ticket
+  // adds its partial tiles up.
+  if constexpr (!GROUPED) {
+    if (p.tickets != nullptr && pieces > 1) {
       const uint32_t flag_lds = (uint32_t)(uintptr_t)(lds_void_t*)smem;
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's partial tiles are in memory
       TRACE(5);
@@ -1239,37 +1187,29 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
       // 15 contributors): their sum says who is last, and a single non-zero field that every
       // contributor ran on one XCD.
       const unsigned int xcc = __builtin_amdgcn_s_getreg((3 << 11) | 20) & 7u;   // XCC_ID: the XCD this workgroup runs on
-      if (wave == 0 && lane < pending) {
-        const int strip = lane == 0 ? pending_strip[0] : pending_strip[1];
-        int first, last;
-        strip_contributors(p, strip, first, last);
-        unsigned int* ticket = p.tickets + ((long)first * p.slabs + slab) * p.ticket_stride;
-        const unsigned int mine = 1u << (4u * xcc);
-        const unsigned int now = mine + __hip_atomic_fetch_add(ticket, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(flag_lds + 4u * lane), "v"(now) : "memory");
+      unsigned int* ticket = p.tickets + ((long)first * p.slabs + slab) * p.ticket_stride;
+      if (threadIdx.x == 0) {
+        const unsigned int mine_field = 1u << (4u * xcc);
+        const unsigned int now =
+            mine_field + __hip_atomic_fetch_add(ticket, mine_field, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(flag_lds), "v"(now) : "memory");
       }
       __builtin_amdgcn_s_barrier();
       TRACE(6);
-      for (int k = 0; k < pending; ++k) {
-        uint32_t now;
-        asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(now) : "v"(flag_lds + 4u * k) : "memory");
-        now = __builtin_amdgcn_readfirstlane(now);
-        const int strip = k == 0 ? pending_strip[0] : pending_strip[1];
-        int first, last;
-        strip_contributors(p, strip, first, last);
-        const unsigned int pairs = (now & 0x0f0f0f0fu) + ((now >> 4) & 0x0f0f0f0fu);
-        const int arrived = (int)((pairs * 0x01010101u) >> 24);
-        if (arrived != last - first + 1) continue;   // somebody is still at work on this strip
-        const bool near = now == ((unsigned int)(last - first + 1) << (4u * xcc));
+      uint32_t now;
+      asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(now) : "v"(flag_lds) : "memory");
+      now = __builtin_amdgcn_readfirstlane(now);
+      const unsigned int pairs = (now & 0x0f0f0f0fu) + ((now >> 4) & 0x0f0f0f0fu);
+      const int arrived = (int)((pairs * 0x01010101u) >> 24);
+      if (arrived == pieces) {   // nobody is still at work on this strip
+        const bool near = now == ((unsigned int)pieces << (4u * xcc));
         for (int t = wave; t < 4 * MB; t += kFastWaves) {
           const int mb = t >> 2, j = t & 3;
           const floatx4_t sum = near ? sum_partial_tiles<true>(p, first, last, slab * MB + mb, j, lane)
                                      : sum_partial_tiles<false>(p, first, last, slab * MB + mb, j, lane);
           store_c_block<T>(p, p.c + (long)(16 * mb) * p.size_n, p.size_m - 16 * mb, strip, lane, j, sum);
         }
-        if (threadIdx.x == 0)
-          __hip_atomic_store(p.tickets + ((long)first * p.slabs + slab) * p.ticket_stride, 0u, __ATOMIC_RELAXED,
-                             __HIP_MEMORY_SCOPE_AGENT);
+        if (threadIdx.x == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
 #ifdef SONAR_TRACE
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
@@ -1278,6 +1218,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     }
   }
 }
+#undef SONAR_UNIT_READS_VEC
 #undef SONAR_UNIT_READS_ROWS2
 #undef SONAR_GROUP_READS
 
@@ -1516,7 +1457,7 @@ int launch_fast_groups(const StreamParams& p, int unit_group_shift, hipStream_t 
                                   hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds_bytes(WAVES, MB, GPU)));
     attr_set = true;
   }
-  const int lds = p.sum_over_rings ? WAVES * wave_lds(MB, GPU) : fast_lds_bytes(WAVES, MB, GPU);
+  const int lds = fast_lds_bytes(WAVES, MB, GPU);
   marlin_stream_fast_kernel<T, HAS_ZP, WAVES, MB, GROUPED, GPU>
       <<<p.grid_parts * p.slabs, WAVES * 64, lds, st>>>(p, unit_group_shift);
   return SONAR_OK;
@@ -1547,7 +1488,7 @@ int launch_fast_fp4_waves(const StreamParams& p, hipStream_t st) {
                                   hipFuncAttributeMaxDynamicSharedMemorySize, fast_lds_bytes(WAVES, 1, 4)));
     attr_set = true;
   }
-  const int lds = p.sum_over_rings ? WAVES * wave_lds(1, 4) : fast_lds_bytes(WAVES, 1, 4);
+  const int lds = fast_lds_bytes(WAVES, 1, 4);
   marlin_stream_fast_kernel<__bf16, false, WAVES, 1, GROUPED, 4, true>
       <<<p.grid_parts * p.slabs, WAVES * 64, lds, st>>>(p, -4);
   return SONAR_OK;
@@ -1727,7 +1668,6 @@ int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.sub_blocks = moe_block_size > 32 ? 2 : 1;
   p.slabs = (int)((sorted_len + moe_block_size - 1) / moe_block_size) * p.sub_blocks;   // blocks of slots x halves
   p.grid_parts = n_strips;
-  p.sum_over_rings = 1;                     // every workgroup owns a whole strip
   p.piece_shift = 0;
   p.piece_units = p.units_per_strip;
   p.sorted_ids = sorted_ids;
@@ -1908,53 +1848,14 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   const bool row_slabs = !use_tile && !slab_fast && size_m > 64 && strip_per_workgroup &&
                          total_units * n_strips < (1LL << 31);
   p.parts = p.total_units < cus ? p.total_units : cus;
-  // Up to 16 rows in the fast kernel: every strip is cut into the same number of pieces, as
-  // many as make at most one workgroup per compute unit (a Llama-3-8B attention output
-  // projection: 64 strips x 4), and the pieces of a strip are summed inside the kernel
-  // (tickets in the workspace).  With more strips than compute units every strip is one
-  // workgroup.  Either way a workgroup works on one strip only, sums its wavefronts once,
-  // at the end, and can park the tiles of that sum on top of its copy rings, which leaves
-  // LDS for a third weight slot per wavefront.
-  static const bool no_inline_sum = getenv("SONAR_MARLIN_NO_INLINE_SUM") != nullptr;   // debugging aids
-  static const char* split_env = getenv("SONAR_MARLIN_SPLIT");
-  const bool piece_split = fast_shape && p.unit_chunks == 4 && size_m <= 16 && !no_inline_sum &&
-                           n_strips * n_strips * p.units_per_strip < (1LL << 31);
-  int pieces = 1, piece_shift = 0, piece_units = 0;
-  if (piece_split) {
-    pieces = (int)(cus / n_strips);
-    if (split_env && atoi(split_env) < pieces) pieces = atoi(split_env);   // never more parts than scratch slots
-    if (pieces > p.units_per_strip) pieces = p.units_per_strip;
-    if (pieces > 15) pieces = 15;   // a ticket field counts up to 15 contributors
-    if (pieces < 1) pieces = 1;
-    if (n_strips * pieces > workspace_len) pieces = 1;
-    // equal pieces, a power of two of them, when the strip can be cut that way
-    int shift = 0;
-    while ((2 << shift) <= pieces && p.units_per_strip % (2 << shift) == 0) ++shift;
-    if ((1 << shift) == pieces) {
-      piece_shift = shift;
-      piece_units = p.units_per_strip >> shift;
-    }
-    p.parts = (int)n_strips * pieces;   // range_begin(strip * pieces + i) = strip * units_per_strip + i * units_per_strip / pieces
-  } else if (strip_per_workgroup && (p.unit_chunks == 4 || row_slabs)) {
-    p.parts = (int)n_strips;
-  }
+  if (strip_per_workgroup && row_slabs) p.parts = (int)n_strips;
   p.slabs = 1;
   p.grid_parts = p.parts;
-  p.sum_over_rings = 0;
   p.tickets = nullptr;
   p.ticket_stride = 1;
   p.xcd_ranges = 0;
-  p.piece_shift = piece_shift;
-  p.piece_units = piece_units;
-
-  bool any_split = false;
-  for (int i = 1; i < p.parts && !any_split; ++i)
-    any_split = range_begin(i, p.total_units, p.parts) % p.units_per_strip != 0;
-
-  // a split strip leaves one partial tile set per contributor in scratch slot `part` or `parts + part`
-  if (any_split && !use_tile)
-    SONAR_REQUIRE((size_t)2 * p.parts * kSlotFloat4 * sizeof(float4) <= stream_scratch_bytes(),
-                  "internal: %d parts share strips but the scratch has slots for %d", p.parts, cus);
+  p.piece_shift = 0;
+  p.piece_units = 0;
 
   if (use_tile) {
     const size_t used = stream_scratch_bytes();
@@ -1963,55 +1864,87 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                      scratch_bytes > used ? scratch_bytes - used : 0, chk.fp4, st);
   }
 
+  // The fast kernel: up to 16 rows, or more rows in blocks of 16 or 32 (slab_fast), all in
+  // one launch.  Every strip is cut into the same number of pieces, a power of two, as many
+  // as keep the launch at one workgroup per compute unit (a Llama-3-8B attention output
+  // projection at M <= 16: 64 strips x 4 pieces), and the pieces of a strip are summed inside
+  // the kernel (tickets in the workspace; the fix-up launch when the workspace is too small
+  // for them).  With more strips than compute units every strip is one workgroup of four
+  // wavefronts, three of which fit a compute unit.
+  if (fast_shape && p.unit_chunks == 4 && (size_m <= 16 || slab_fast)) {
+    static const bool no_inline_sum = getenv("SONAR_MARLIN_NO_INLINE_SUM") != nullptr;   // debugging aids
+    static const char* split_env = getenv("SONAR_MARLIN_SPLIT");
+    static const bool no_pairs = getenv("SONAR_MARLIN_NO_ROW_PAIRS") != nullptr;
+    static const bool no_half = getenv("SONAR_MARLIN_NO_HALF_WG") != nullptr;
+    p.a = static_cast<const uint16_t*>(a);
+    p.c = static_cast<uint16_t*>(c);
+    p.size_m = (int)size_m;
+    const int blocks16 = (int)((size_m + 15) / 16);
+    int shift = 0;
+    // a scratch slot holds the partial tiles of four blocks of 16 rows, a ticket field counts to 15
+    if (size_m <= 64) {
+      while (shift < 3 && n_strips * (2 << shift) * blocks16 <= cus && p.units_per_strip % (2 << shift) == 0 &&
+             n_strips * (2 << shift) * blocks16 <= workspace_len)
+        ++shift;
+      if (split_env)
+        while (shift > 0 && (1 << shift) > atoi(split_env)) --shift;
+    }
+    p.piece_shift = shift;
+    p.piece_units = p.units_per_strip >> shift;
+    p.parts = (int)(n_strips << shift);
+    SONAR_REQUIRE(n_strips << shift < (1LL << 30), "size_n = %ld is too large", (long)size_n);
+    // Two blocks of rows per workgroup once one block each would make more
+    // workgroups than compute units: the weights are then fetched from L2 and
+    // unpacked once for 32 rows.
+    int row_blocks = 1;
+    if (size_m > 16 && !no_pairs && (int64_t)p.parts * blocks16 > cus) row_blocks = 2;
+    p.slabs = (int)((size_m + 16 * row_blocks - 1) / (16 * row_blocks));
+    p.grid_parts = p.slabs > 1 ? (p.parts + 7) / 8 * 8 : p.parts;
+    // more workgroups than compute units: small ones, three per compute unit
+    const bool half = !no_half && (int64_t)p.parts * p.slabs > cus;
+    const bool split = shift > 0;
+    // a split strip leaves one set of partial tiles per contributor in scratch slot `part` or `parts + part`
+    if (split)
+      SONAR_REQUIRE((size_t)2 * p.parts * kSlotFloat4 * sizeof(float4) <= stream_scratch_bytes() &&
+                        p.slabs * row_blocks <= 4,
+                    "internal: %d parts x %d blocks of rows share strips but the scratch has slots for %d x 4",
+                    p.parts, p.slabs * row_blocks, cus);
+    const bool inline_sum = split && !no_inline_sum && (int64_t)p.parts * p.slabs <= workspace_len;
+    if (inline_sum) {
+      p.tickets = reinterpret_cast<unsigned int*>(workspace);
+      const int64_t room = workspace_len / ((int64_t)p.parts * p.slabs);
+      p.ticket_stride = room >= 4 ? 4 : (int)room;
+      p.xcd_ranges = p.slabs == 1 && p.parts % 8 == 0;
+    }
+    int rc;
+    if (chk.fp4)   // groups of 32 rows: never in blocks of rows (slab_fast is off), so one block of 16 rows
+      rc = launch_fast_fp4<false>(p, half, st);
+    else if (dtype == SONAR_DTYPE_F16)
+      rc = chk.has_zp ? launch_fast<_Float16, true>(p, unit_group_shift, half, row_blocks, st)
+                      : launch_fast<_Float16, false>(p, unit_group_shift, half, row_blocks, st);
+    else
+      rc = chk.has_zp ? launch_fast<__bf16, true>(p, unit_group_shift, half, row_blocks, st)
+                      : launch_fast<__bf16, false>(p, unit_group_shift, half, row_blocks, st);
+    if (rc) return rc;
+    if (int rc2 = launch_status("marlin_stream_fast_kernel")) return rc2;
+    if (split && !inline_sum) {   // the fix-up kernel reads the split as ranges of units: part i = units [i, i + 1) * piece_units
+      p.total_units = (int)total_units;
+      if (dtype == SONAR_DTYPE_F16) launch_fixup<_Float16>(p, st);
+      else launch_fixup<__bf16>(p, st);
+      if (int rc2 = launch_status("marlin_fixup_kernel")) return rc2;
+    }
+    return SONAR_OK;
+  }
+
+  bool any_split = false;
+  for (int i = 1; i < p.parts && !any_split; ++i)
+    any_split = range_begin(i, p.total_units, p.parts) % p.units_per_strip != 0;
+
   for (int64_t m0 = 0; m0 < size_m; m0 += 64) {
     p.a = static_cast<const uint16_t*>(a) + m0 * a_row_stride;
     p.c = static_cast<uint16_t*>(c) + m0 * size_n;
     p.size_m = (int)(size_m - m0 < 64 ? size_m - m0 : 64);
-    const bool fast = fast_shape && p.unit_chunks == 4 && (p.size_m <= 16 || slab_fast);
-    bool inline_sum = false;
-    if (fast) {
-      // Two blocks of rows per workgroup once one block each would make more
-      // workgroups than compute units: the weights are then fetched from L2 and
-      // unpacked once for 32 rows.
-      static const bool no_pairs = getenv("SONAR_MARLIN_NO_ROW_PAIRS") != nullptr;  // debugging aid
-      int row_blocks = 1;
-      if (slab_fast) {  // every row in this one launch
-        p.size_m = (int)size_m;
-        if (!no_pairs && p.parts * ((size_m + 15) / 16) > cus) row_blocks = 2;
-        p.slabs = (int)((size_m + 16 * row_blocks - 1) / (16 * row_blocks));
-        p.grid_parts = p.slabs > 1 ? (p.parts + 7) / 8 * 8 : p.parts;
-        m0 = size_m;
-      }
-      int rc;
-      // more workgroups than compute units: small ones, two per compute unit, or three
-      // when they need no LDS of their own for the sum
-      static const bool no_half = getenv("SONAR_MARLIN_NO_HALF_WG") != nullptr;  // debugging aid
-      const bool half = !no_half && p.parts * p.slabs > cus;
-      p.sum_over_rings = half && (int64_t)p.parts == n_strips && p.parts * p.slabs > 2 * cus;
-      if (piece_split) {
-        p.sum_over_rings = 1;
-      }
-      // Shared strips are summed inside the kernel when the workspace has a ticket for every
-      // part and block of rows; tickets four words apart do not hold each other up.
-      const int smallest_part = p.total_units / p.parts;   // parts <= total_units
-      const int contributors = (p.units_per_strip + smallest_part - 1) / smallest_part + 1;   // upper bound
-      inline_sum = any_split && !no_inline_sum && (int64_t)p.parts * p.slabs <= workspace_len && contributors <= 15;
-      if (inline_sum) {
-        p.tickets = reinterpret_cast<unsigned int*>(workspace);
-        const int64_t room = workspace_len / ((int64_t)p.parts * p.slabs);
-        p.ticket_stride = room >= 4 ? 4 : (int)room;
-        p.xcd_ranges = p.slabs == 1 && p.parts % 8 == 0;
-      }
-      if (chk.fp4)   // groups of 32 rows: never in blocks of rows (slab_fast is off), so one block of 16 rows
-        rc = launch_fast_fp4<false>(p, half, st);
-      else if (dtype == SONAR_DTYPE_F16)
-        rc = chk.has_zp ? launch_fast<_Float16, true>(p, unit_group_shift, half, row_blocks, st)
-                        : launch_fast<_Float16, false>(p, unit_group_shift, half, row_blocks, st);
-      else
-        rc = chk.has_zp ? launch_fast<__bf16, true>(p, unit_group_shift, half, row_blocks, st)
-                        : launch_fast<__bf16, false>(p, unit_group_shift, half, row_blocks, st);
-      if (rc) return rc;
-    } else {
+    {
       if (row_slabs && !any_split) {   // every 64-row slab in this one launch
         p.size_m = (int)size_m;
         p.slabs = (int)((size_m + 63) / 64);
@@ -2032,7 +1965,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
       }
     }
     if (int rc = launch_status("marlin_stream_kernel")) return rc;
-    if (any_split && !inline_sum) {
+    if (any_split) {
       if (dtype == SONAR_DTYPE_F16) launch_fixup<_Float16>(p, st);
       else launch_fixup<__bf16>(p, st);
       if (int rc = launch_status("marlin_fixup_kernel")) return rc;
