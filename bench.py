@@ -7,7 +7,12 @@ int4 weights, group size 128) at M = 16 bf16 activation rows, through the same
 torch ops the reference's callers use.  Weights of `--copies` distinct layers
 (more bytes than the 256 MB last-level cache) are visited round-robin so every
 step streams its weights from HBM.  The K timed steps are recorded in one HIP
-graph and replayed once between two events on the launching stream.
+graph; the graph is replayed `REPLAYS` times, each replay between two events on
+the launching stream, and the line reports the median replay (with the 10th
+and 90th percentile beside it).
+
+The same line carries the MFMA half of the metric: the four GEMMs at M = 4096
+with fp16 activations (`roofline_mfma`), timed the same way.
 
 Prints one JSON line; `--sweep` adds the M sweep of the decode and prefill
 shapes under "sweep".
@@ -25,12 +30,15 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
-# HBM bytes per GEMM launch (stream kernel, plus the fix-up where one runs) of the default workload,
-# from one `rocprofv3 --pmc FETCH_SIZE` and one `--pmc WRITE_SIZE` run of
-# `bench.py --eager --calibrate`: FETCH_SIZE scaled by 2.000 and WRITE_SIZE by
-# 1.000, the factors that make the `--calibrate` pass (256 MiB read, 256 MiB
-# written) come out right.  Average over the four GEMMs of the layer at M = 16.
+# HBM bytes per GEMM launch of the default workload (M = 16, 6 weight copies), from one
+# `rocprofv3 --pmc FETCH_SIZE` and one `--pmc WRITE_SIZE` run of `bench.py --eager --calibrate`
+# (profiles/marlin_stream_fast_kernel_llama3-8b_m16_hbm-traffic.txt): FETCH_SIZE scaled by
+# 2.000 and WRITE_SIZE by 1.000, the factors that make the `--calibrate` pass (256 MiB read,
+# 256 MiB written) come out right.  Average over the four GEMMs of the layer.  Counters
+# cannot be read from inside a run, so the figure is tied to the launch shapes named in
+# TRAFFIC_LAUNCH_SHAPES: bench.py reports null as soon as the library launches differently.
 MEASURED_TRAFFIC_M16 = 30_100_000
+REPLAYS = 21                # graph replays per timing; the median is reported
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 GROUP = 128
 LAYER_SHAPES = [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
@@ -65,9 +73,10 @@ class Layer:
                                True, False, True, False)
 
 
-def time_graph(torch, fn, reps):
+def time_graph(torch, fn, reps, replays=REPLAYS, spread=False):
     """Records `reps` calls of fn() in a HIP graph, replays it once untimed and
-    once between two events; returns seconds per call."""
+    `replays` times between two events each; returns the median seconds per
+    call (with `spread`: median, 10th and 90th percentile)."""
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
         # every weight copy fn cycles through gets its one-time layout conversion here,
@@ -81,13 +90,20 @@ def time_graph(torch, fn, reps):
                 fn(i)
         graph.replay()
         stream.synchronize()
-        t0 = torch.cuda.Event(enable_timing=True)
-        t1 = torch.cuda.Event(enable_timing=True)
-        t0.record(stream)
-        graph.replay()
-        t1.record(stream)
-        stream.synchronize()
-    return t0.elapsed_time(t1) * 1e-3 / reps
+        times = []
+        for _ in range(replays):
+            t0 = torch.cuda.Event(enable_timing=True)
+            t1 = torch.cuda.Event(enable_timing=True)
+            t0.record(stream)
+            graph.replay()
+            t1.record(stream)
+            stream.synchronize()
+            times.append(t0.elapsed_time(t1) * 1e-3 / reps)
+    times.sort()
+    median = times[len(times) // 2]
+    if spread:
+        return median, times[len(times) // 10], times[(len(times) * 9) // 10]
+    return median
 
 
 def memory_yardsticks(torch):
@@ -280,10 +296,11 @@ def main() -> int:
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
-    ap.add_argument("--m", type=int, default=16)
+    ap.add_argument("--m", type=int, default=16, help="activation rows of the decode step (1..64)")
     ap.add_argument("--copies", type=int, default=6)
     ap.add_argument("--sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the M = 4096 half of the metric")
     ap.add_argument("--eager", action="store_true",
                     help="time the K steps launched one by one instead of in a HIP graph (for counter runs)")
     ap.add_argument("--calibrate", action="store_true",
@@ -293,6 +310,10 @@ def main() -> int:
     if args.gpus != 1:
         print("bench.py: this build runs on one GPU only (the GEMM is rank-local; no multi-GPU path "
               "exists); run with --gpus 1", file=sys.stderr)
+        return 2
+    if not 1 <= args.m <= 64:
+        print("bench.py: --m is the row count of the decode step, 1..64 (the M = 4096 half of the metric is "
+              "always timed beside it; --sweep covers every other M)", file=sys.stderr)
         return 2
 
     import torch
@@ -334,9 +355,12 @@ def main() -> int:
     torch.cuda.synchronize()
     eager_s = (time.perf_counter() - t0) / args.steps
 
-    # timed region: exactly K steps in one graph, events on the launching stream
+    # timed region: exactly K steps in one graph, events on the launching stream; median of REPLAYS replays
     torch.cuda.synchronize()
-    step_s = eager_s if args.eager else time_graph(torch, step, args.steps)
+    if args.eager:
+        step_s = p10 = p90 = eager_s
+    else:
+        step_s, p10, p90 = time_graph(torch, step, args.steps, spread=True)
 
     step_bytes = sum(algorithmic_bytes(m, k, n) for (_, k, n) in LAYER_SHAPES)
     step_flops = sum(2 * m * k * n for (_, k, n) in LAYER_SHAPES)
@@ -347,11 +371,18 @@ def main() -> int:
     for idx, (name, k, n) in enumerate(LAYER_SHAPES):
         def one(i=0, idx=idx, k=k):
             copies[i % args.copies][idx].run(ops, acts[k], wtype)
-        s = eager_s if args.eager else time_graph(torch, one, max(24, args.copies * 4))
+        if args.eager:
+            s = lo = hi = eager_s
+        else:
+            s, lo, hi = time_graph(torch, one, max(24, args.copies * 4), spread=True)
         nb = algorithmic_bytes(m, k, n)
         per_gemm.append({"gemm": name, "k": k, "n": n, "m": m, "us": round(s * 1e6, 2),
+                         "us_p10": round(lo * 1e6, 2), "us_p90": round(hi * 1e6, 2),
                          "GBps": round(nb / s / 1e9, 1), "frac_hbm": round(nb / s / 1e9 / HBM_PEAK_GBPS, 4)})
 
+    kernel = "marlin_stream_fast_kernel<bf16>"
+    if m > 16:
+        kernel += " (blocks of 16 or 32 rows per workgroup)"
     out = {
         "metric": "W4A16 GEMM TFLOP/s + HBM GB/s (% roofline), Llama-3-8B shapes, M=1..8192",
         "value": round(gbps, 1),
@@ -360,6 +391,9 @@ def main() -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(step_s * 1e3, 5),
+        "ms_per_step_p10": round(p10 * 1e3, 5),
+        "ms_per_step_p90": round(p90 * 1e3, 5),
+        "replays": 1 if args.eager else REPLAYS,
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -367,20 +401,51 @@ def main() -> int:
         "data": "synthetic",
         "config": {"workload": f"llama3-8b decoder layer W4A16 GEMMs (qkv+o+gate_up+down), M={m}, "
                                f"bf16 activations, uint4b8 weights, group_size 128, {args.copies} "
-                               "weight copies round-robin, K steps in one HIP graph",
+                               f"weight copies round-robin, K steps in one HIP graph, median of {REPLAYS} replays",
                    "global_batch": m},
         "tflops": round(step_flops / step_s / 1e12, 2),
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
                      "traffic": MEASURED_TRAFFIC_M16 if (m == 16 and args.copies == 6) else None,
-                     "kernel": "marlin_stream_fast_kernel<bf16>" +
-                               ("" if m <= 16 else " (blocks of 16 or 32 rows per workgroup)") +
-                               " (+ marlin_fixup_kernel for down_proj)",
+                     "kernel": kernel,
                      "bytes_per_launch": step_bytes // launches,
                      "us_per_launch": round(step_s / launches * 1e6, 3)},
         "eager_ms_per_step": round(eager_s * 1e3, 5),
         "per_gemm": per_gemm,
     }
+
+    if not args.no_prefill and not args.eager:
+        # the MFMA half of the metric: the same four GEMMs at M = 4096, fp16 activations ~ N(0, 0.5)
+        pm = 4096
+        fl_layers = [[Layer(torch, k, n, torch.float16, gen) for (_, k, n) in LAYER_SHAPES] for _ in range(2)]
+        pa = {k: (torch.randn((pm, k), device="cuda:0", generator=gen) * 0.5).to(torch.float16) for k in (4096, 14336)}
+
+        def prefill_step(i=0):
+            for layer in fl_layers[i % 2]:
+                layer.run(ops, pa[layer.k], wtype)
+
+        ps, plo, phi = time_graph(torch, prefill_step, 4, spread=True)
+        pflops = sum(2 * pm * k * n for (_, k, n) in LAYER_SHAPES)
+        per_prefill = []
+        for idx, (name, k, n) in enumerate(LAYER_SHAPES):
+            def one(i=0, idx=idx, k=k):
+                fl_layers[i % 2][idx].run(ops, pa[k], wtype)
+            s, lo, hi = time_graph(torch, one, 4, spread=True)
+            fl = 2 * pm * k * n
+            per_prefill.append({"gemm": name, "k": k, "n": n, "m": pm, "us": round(s * 1e6, 1),
+                                "us_p10": round(lo * 1e6, 1), "us_p90": round(hi * 1e6, 1),
+                                "TFLOPs": round(fl / s / 1e12, 1),
+                                "frac_mfma": round(fl / s / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+        out["roofline_mfma"] = {"bound": "mfma", "achieved": round(pflops / ps / 1e12, 1), "peak": MFMA_PEAK_TFLOPS,
+                                "unit": "TFLOP/s", "frac": round(pflops / ps / 1e12 / MFMA_PEAK_TFLOPS, 4),
+                                "kernel": "marlin_tile_async_kernel<f16> (+ tile_reduce_kernel where K is split)",
+                                "workload": "the four GEMMs of the layer at M=4096, fp16 activations ~ N(0,0.5), "
+                                            f"4 steps per graph, median of {REPLAYS} replays",
+                                "flops_per_launch": pflops // launches,
+                                "us_per_launch": round(ps / launches * 1e6, 2),
+                                "ms_per_step": round(ps * 1e3, 4), "ms_per_step_p10": round(plo * 1e3, 4),
+                                "ms_per_step_p90": round(phi * 1e3, 4), "per_gemm": per_prefill}
+        del fl_layers, pa
 
     if args.sweep:
         sweep = []
