@@ -9,9 +9,9 @@ from __future__ import annotations
 
 import torch
 
-from .marlin_utils import (GPTQ_MARLIN_TILE, get_pack_factor, marlin_permute_scales, marlin_zero_points)
-from .quant_utils import gptq_quantize_weights, quantize_weights, sort_weights
-from .scalar_type import ScalarType
+from sonar_amd.marlin_utils import (GPTQ_MARLIN_TILE, get_pack_factor, marlin_permute_scales, marlin_zero_points)
+from tests.quant_utils import gptq_quantize_weights, quantize_weights, sort_weights
+from sonar_amd.scalar_type import ScalarType
 
 
 class MarlinWorkspace:

@@ -8,8 +8,8 @@ from __future__ import annotations
 
 import torch
 
-from .marlin_utils import get_pack_factor, pack_cols
-from .scalar_type import ScalarType, scalar_types
+from sonar_amd.marlin_utils import get_pack_factor, pack_cols
+from sonar_amd.scalar_type import ScalarType, scalar_types
 
 SUPPORTED_GPTQ_QUANT_TYPES = [scalar_types.uint4b8, scalar_types.uint8b128]
 SUPPORTED_GROUP_SIZES = [-1, 32, 64, 128]

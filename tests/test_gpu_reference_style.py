@@ -50,8 +50,8 @@ def rand_data(shape, dtype=torch.float16):
 @pytest.mark.parametrize("nk_factors", MARLIN_REPACK_NK_FACTORS)
 def test_gptq_marlin_repack(n_chunk, quant_type, act_order, nk_factors):
     from sonar_amd import ops
-    from sonar_amd.marlin_utils_test import get_weight_perm, marlin_weights
-    from sonar_amd.quant_utils import gptq_pack, gptq_quantize_weights, sort_weights
+    from tests.marlin_utils_for_tests import get_weight_perm, marlin_weights
+    from tests.quant_utils import gptq_pack, gptq_quantize_weights, sort_weights
     n_factor, k_factor = nk_factors
     size_k, size_n, group_size = 128 * k_factor, n_chunk * n_factor, 128
     b_weight = rand_data((size_k, size_n))
@@ -70,8 +70,8 @@ def test_gptq_marlin_repack(n_chunk, quant_type, act_order, nk_factors):
 @pytest.mark.parametrize("nk_factors", MARLIN_REPACK_NK_FACTORS)
 def test_awq_marlin_repack(n_chunk, nk_factors):
     from sonar_amd import ops
-    from sonar_amd.marlin_utils_test import get_weight_perm, marlin_weights
-    from sonar_amd.quant_utils import awq_pack, quantize_weights
+    from tests.marlin_utils_for_tests import get_weight_perm, marlin_weights
+    from tests.quant_utils import awq_pack, quantize_weights
     quant_type = scalar_types.uint4
     n_factor, k_factor = nk_factors
     size_k, size_n = 128 * k_factor, n_chunk * n_factor
@@ -116,7 +116,7 @@ def test_marlin_gemm(b_type, dtype, group_size, size_m, size_n, size_k, act_orde
     from sonar_amd.marlin_utils import marlin_make_workspace_new
     from sonar_amd.marlin_utils_fp4 import rand_marlin_weight_mxfp4_like
     from sonar_amd.marlin_utils_fp8 import marlin_quant_fp8_torch
-    from sonar_amd.marlin_utils_test import awq_marlin_quantize, marlin_quantize
+    from tests.marlin_utils_for_tests import awq_marlin_quantize, marlin_quantize
     a_input = rand_data((size_m, size_k), dtype=dtype)
     b_weight = rand_data((size_k, size_n), dtype=dtype)
     if b_type == scalar_types.uint4:
@@ -145,7 +145,7 @@ def test_marlin_gemm(b_type, dtype, group_size, size_m, size_n, size_k, act_orde
 def test_marlin_gemm_with_bias(size_m):
     from sonar_amd import ops
     from sonar_amd.marlin_utils import marlin_make_empty_g_idx, marlin_make_workspace_new, marlin_permute_bias
-    from sonar_amd.marlin_utils_test import marlin_quantize
+    from tests.marlin_utils_for_tests import marlin_quantize
     quant_type, group_size = scalar_types.uint4b8, 128
     size_k, size_n = 1024, 2048
     a_input = rand_data((size_m, size_k))
@@ -214,7 +214,7 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None):
     from sonar_amd.marlin_utils import marlin_permute_bias
     from sonar_amd.marlin_utils_fp4 import rand_marlin_weight_mxfp4_like
     from sonar_amd.marlin_utils_fp8 import marlin_quant_fp8_torch
-    from sonar_amd.marlin_utils_test import awq_marlin_quantize, marlin_quantize
+    from tests.marlin_utils_for_tests import awq_marlin_quantize, marlin_quantize
     k = w.shape[-1]
     out = {"w_ref": [], "qweight": [], "scales": [], "zeros": [], "g_idx": [], "sort_indices": [], "bias": []}
     for i in range(w.shape[0]):

@@ -377,8 +377,8 @@ def test_marlin_test_utils_match_the_oracle_layout():
     """get_weight_perm / marlin_weights (marlin_utils_test.py:31-121) against the
     oracle's restatement of the same recipe and its closed form, 4 and 8 bits;
     gptq_pack / awq_pack against the oracle's packings."""
-    from sonar_amd import marlin_utils_test as mt
-    from sonar_amd import quant_utils as qu
+    from tests import marlin_utils_for_tests as mt
+    from tests import quant_utils as qu
     assert np.array_equal(mt.get_weight_perm(4).numpy(), mo.marlin_weight_perm_recipe())
     assert np.array_equal(mt.get_weight_perm(8).numpy(), mo.marlin_weight_perm_recipe8())
     rng = np.random.default_rng(0)
@@ -398,7 +398,7 @@ def test_quantize_weights_on_hand_worked_groups():
     group spanning [-8, 7] has scale 1 and codes value + 8; an asymmetric group
     spanning [-3, 12] has scale 1 and zero point 3; and in general the codes
     are in range, w_ref = (code - zero) * scale and |w - w_ref| <= scale / 2."""
-    from sonar_amd import quant_utils as qu
+    from tests import quant_utils as qu
     from sonar_amd.scalar_type import scalar_types as st
     col = torch.tensor([-8.0, 7.0, 0.0, 3.0, -1.0, 2.0, -5.0, 6.0]).repeat(4)      # one group of 32 rows
     w = torch.stack([col, 0.5 * col], dim=1)

@@ -479,3 +479,48 @@ def test_mxfp4_dequant_and_scale_reorder():
     x = np.arange(16).reshape(2, 8)
     y = mo.mxfp4_process_scales(x)
     assert y[0].tolist() == [0, 2, 1, 3, 4, 6, 5, 7] and np.array_equal(mo.mxfp4_process_scales(y), x)
+
+
+def test_moe_gemm_reference_against_per_slot_brute_force():
+    """moe_gemm_reference (the oracle of the grouped GEMM) follows sorted_ids / expert_ids
+    block by block.  Brute force from the routing itself, slot by slot, without any of
+    that bookkeeping: C[t * top_k + j] = A[t] @ W[topk_ids[t][j]], rounded, times the
+    rounded routing weight, rounded.  Integer-valued matrices keep every product and sum
+    exact in fp32, so the two must agree exactly; a wrong row index (id % top_k for
+    id // top_k), a wrong expert, a dropped rounding of the weight or a block that is
+    skipped or written twice all show."""
+    rng = np.random.default_rng(11)
+    m, e, top_k, k, n, bs = 13, 5, 3, 16, 8, 4
+    a = rng.integers(-4, 5, size=(m, k)).astype(np.float32)
+    w = [rng.integers(-3, 4, size=(k, n)).astype(np.float32) for _ in range(e)]
+    topk_ids = np.stack([rng.permutation(e)[:top_k] for _ in range(m)]).astype(np.int32)
+    weights = rng.random((m, top_k)).astype(np.float32)
+    sorted_ids, expert_ids, past = mo.moe_align_block_size(topk_ids, bs, e)
+    for dtype in ("fp16", "bf16"):
+        for tw in (None, weights):
+            got = mo.moe_gemm_reference(a, w, sorted_ids, expert_ids, int(past[0]), bs, top_k, m, tw, dtype)
+            want = np.zeros((m * top_k, n), dtype=np.float32)
+            for t in range(m):
+                for j in range(top_k):
+                    row = np.zeros(n, dtype=np.float32)
+                    for col in range(n):
+                        acc = 0.0
+                        for kk in range(k):
+                            acc += float(a[t, kk]) * float(w[topk_ids[t, j]][kk, col])
+                        row[col] = acc
+                    row = mo.round_to_dtype(row, dtype)
+                    if tw is not None:
+                        wt = mo.round_to_dtype(np.array([tw[t, j]], dtype=np.float32), dtype)[0]
+                        row = mo.round_to_dtype(row * wt, dtype)
+                    want[t * top_k + j] = row
+            assert np.array_equal(got, want), (dtype, tw is None)
+    # a block whose expert is not on this rank (-1) and slots past the padded total write nothing
+    expert_ids2 = expert_ids.copy()
+    expert_ids2[0] = -1
+    got = mo.moe_gemm_reference(a, w, sorted_ids, expert_ids2, int(past[0]), bs, top_k, m, None, "fp16")
+    dropped = sorted_ids[:bs]
+    dropped = dropped[dropped < m * top_k]
+    assert np.all(got[dropped] == 0) and dropped.size > 0
+    kept = np.setdiff1d(np.arange(m * top_k), dropped)
+    full = mo.moe_gemm_reference(a, w, sorted_ids, expert_ids, int(past[0]), bs, top_k, m, None, "fp16")
+    assert np.array_equal(got[kept], full[kept])
