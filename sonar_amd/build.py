@@ -72,7 +72,8 @@ def build_torch_ops(verbose: bool = False) -> str:
            "-I", os.path.join(ROOT, "include"), "-isystem", "/opt/rocm/include", *inc, src,
            "-o", OPS_PATH, "-L", torch_lib, "-L", LIB_DIR,
            "-Wl,-rpath,$ORIGIN", "-Wl,-rpath," + torch_lib,
-           "-lsonar_marlin", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip"]
+           "-L", "/opt/rocm/lib", "-lsonar_marlin", "-ltorch", "-ltorch_cpu", "-lc10", "-lc10_hip", "-ltorch_hip",
+           "-lamdhip64"]
     out = _run(cmd)
     if verbose and out.strip():
         print(out)

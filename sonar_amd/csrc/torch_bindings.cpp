@@ -10,11 +10,24 @@
 // The repack ops return the Marlin tile order bit for bit, because that is
 // what every caller stores.  The gfx950 kernels stream a different order, so
 // the GEMM ops convert a weight tensor the first time they see it and keep the
-// converted copy, keyed by the tensor's address.  The entry also keeps a
-// reference to the source tensor, so its address cannot be handed to another
-// tensor while the entry lives, and remembers the tensor's version counter, so
-// an in-place update triggers a new conversion.
+// converted copy, keyed by the tensor's address.  An entry is valid for one
+// (address, tensor object, shape, version counter).  What invalidates it:
+//   * the repack ops drop every entry whose source memory overlaps the tensor
+//     they have just written (a reload through `x.data = ops.gptq_marlin_repack(...)`
+//     is safe even when the allocator hands the old address back);
+//   * a miss drops every entry of the same tensor object at another address
+//     (`x.data = ...` keeps the object) and every entry whose tensor is gone;
+//   * an in-place op on the tensor itself bumps its version counter;
+//   * marlin_weight_cache_invalidate(tensor) / marlin_weight_cache_clear().
+// What nothing here can see: bytes rewritten in place through another view
+// (`x.data.copy_(...)`, any write to an inference-mode tensor).  After such a
+// write the caller must call marlin_weight_cache_invalidate on the tensor.
+// A miss while the stream is being captured into a graph is an error (the
+// conversion would be recorded instead of run): warm every weight up before
+// capture.  The conversion runs on the calling stream; a hit from another
+// stream waits for it through an event.
 #include <ATen/ATen.h>
+#include <hip/hip_runtime_api.h>
 #include <ATen/hip/HIPContext.h>
 #include <ATen/hip/impl/HIPGuardImplMasqueradingAsCUDA.h>
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
@@ -59,6 +72,9 @@ struct NativeEntry {
   Tensor native;
   int64_t size_k, size_n, experts;
   uint32_t version;
+  size_t source_bytes;
+  hipStream_t stream;    // the stream the conversion ran on
+  hipEvent_t ready;      // recorded behind the conversion; null once it is known to have finished
 };
 
 std::mutex g_cache_mutex;
@@ -66,18 +82,91 @@ std::unordered_map<const void*, NativeEntry> g_cache;
 
 uint32_t version_of(const Tensor& t) { return t.is_inference() ? 0u : t._version(); }
 
+void drop_event(NativeEntry& e) {
+  if (e.ready != nullptr) (void)hipEventDestroy(e.ready);
+  e.ready = nullptr;
+}
+
+// Refuses a conversion while `stream` is being captured: the conversion kernels would be
+// recorded into the graph instead of run, and the cached copy would be read before it exists.
+void refuse_during_capture(hipStream_t stream, const char* what) {
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) {
+    (void)hipGetLastError();
+    return;
+  }
+  TORCH_CHECK(status == hipStreamCaptureStatusNone, what,
+              " has not been used before and the stream is being captured into a graph: its one-time "
+              "conversion to the gfx950 streaming order cannot run inside a capture.  Call the op once on "
+              "every weight (a warm-up step) before capturing.");
+}
+
+// A hit from another stream than the one that converted must not overtake the conversion.
+void wait_for_conversion(NativeEntry& e, hipStream_t stream) {
+  if (e.ready == nullptr) return;
+  if (hipEventQuery(e.ready) == hipSuccess) {
+    drop_event(e);
+    return;
+  }
+  (void)hipGetLastError();   // hipErrorNotReady
+  if (stream != e.stream) (void)hipStreamWaitEvent(stream, e.ready, 0);
+}
+
+// Drops every entry whose source bytes overlap [begin, begin + bytes).
+void invalidate_range_locked(const void* begin, size_t bytes) {
+  const char* lo = static_cast<const char*>(begin);
+  const char* hi = lo + bytes;
+  for (auto it = g_cache.begin(); it != g_cache.end();) {
+    const char* s = static_cast<const char*>(it->first);
+    if (s < hi && lo < s + it->second.source_bytes) {
+      drop_event(it->second);
+      it = g_cache.erase(it);
+    } else {
+      ++it;
+    }
+  }
+}
+
+void record_conversion(NativeEntry& e, hipStream_t stream) {
+  e.stream = stream;
+  e.ready = nullptr;
+  if (hipEventCreateWithFlags(&e.ready, hipEventDisableTiming) != hipSuccess || hipEventRecord(e.ready, stream) != hipSuccess) {
+    (void)hipGetLastError();
+    drop_event(e);
+  }
+}
+
+// Before a new entry for `t` goes in: entries of tensors that are gone, and entries of this
+// tensor object at another address (`x.data = ...` keeps the object alive), leave.
+void evict_stale_locked(const Tensor& t, const void* key) {
+  for (auto it = g_cache.begin(); it != g_cache.end();) {
+    const bool gone = it->second.source.expired();
+    const bool moved = !gone && it->first != key && it->second.source._unsafe_get_target() == t.unsafeGetTensorImpl();
+    if (gone || moved) {
+      drop_event(it->second);
+      it = g_cache.erase(it);
+    } else {
+      ++it;
+    }
+  }
+}
+
 // b_q_weight: (K/16, 2N) or (E, K/16, 2N) int32 in Marlin order; (K/16, 4N) for 8-bit codes.
 Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, int64_t experts, int bits = 4) {
   const void* key = b_q_weight.const_data_ptr();
+  hipStream_t stream = (hipStream_t)current_stream(b_q_weight);
   {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     auto it = g_cache.find(key);
     if (it != g_cache.end() && !it->second.source.expired() &&
         it->second.source._unsafe_get_target() == b_q_weight.unsafeGetTensorImpl() &&
         it->second.size_k == size_k && it->second.size_n == size_n && it->second.experts == experts &&
-        it->second.version == version_of(b_q_weight))
+        it->second.version == version_of(b_q_weight)) {
+      wait_for_conversion(it->second, stream);
       return it->second.native;
+    }
   }
+  refuse_during_capture(stream, "This weight tensor");
   Tensor native = at::empty_like(b_q_weight);
   const int64_t words = size_k * size_n / (32 / bits);
   const uint32_t* src = static_cast<const uint32_t*>(b_q_weight.const_data_ptr());
@@ -88,12 +177,12 @@ Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, 
                               : sonar_marlin_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
                                                        current_stream(b_q_weight)));
   std::lock_guard<std::mutex> lock(g_cache_mutex);
-  // Weights whose Marlin tensor is gone (a layer that was reloaded or dropped)
-  // leave the cache with their streaming-order copies.
-  for (auto it = g_cache.begin(); it != g_cache.end();)
-    it = it->second.source.expired() ? g_cache.erase(it) : std::next(it);
-  g_cache.insert_or_assign(key, NativeEntry{c10::weak_intrusive_ptr<c10::TensorImpl>(b_q_weight.getIntrusivePtr()),
-                                            native, size_k, size_n, experts, version_of(b_q_weight)});
+  evict_stale_locked(b_q_weight, key);
+  invalidate_range_locked(key, b_q_weight.nbytes());
+  NativeEntry entry{c10::weak_intrusive_ptr<c10::TensorImpl>(b_q_weight.getIntrusivePtr()), native, size_k, size_n,
+                    experts, version_of(b_q_weight), b_q_weight.nbytes(), stream, nullptr};
+  record_conversion(entry, stream);
+  g_cache.insert_or_assign(key, entry);
   return native;
 }
 
@@ -106,14 +195,18 @@ Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, 
 // with the same exponent field); exponents past the bf16 range become infinity.
 Tensor mx_scales_as_bf16(const Tensor& b_scales, int64_t exponent_offset) {
   const void* key = b_scales.const_data_ptr();
+  hipStream_t stream = (hipStream_t)current_stream(b_scales);
   {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     auto it = g_cache.find(key);
     if (it != g_cache.end() && !it->second.source.expired() &&
         it->second.source._unsafe_get_target() == b_scales.unsafeGetTensorImpl() && it->second.size_k == -1 &&
-        it->second.size_n == exponent_offset && it->second.version == version_of(b_scales))
+        it->second.size_n == exponent_offset && it->second.version == version_of(b_scales)) {
+      wait_for_conversion(it->second, stream);
       return it->second.native;
+    }
   }
+  refuse_during_capture(stream, "This tensor of float8_e8m0fnu block scales");
   TORCH_CHECK(b_scales.numel() % 4 == 0, "b_scales.numel() must be a multiple of 4");
   const Tensor bytes = b_scales.view(at::kByte);
   const Tensor order = at::tensor({0, 2, 1, 3}, at::TensorOptions().dtype(at::kLong).device(b_scales.device()));
@@ -123,8 +216,12 @@ Tensor mx_scales_as_bf16(const Tensor& b_scales, int64_t exponent_offset) {
   const Tensor bits = at::where(e == 0, at::full_like(e, 0x40), at::clamp_max(e, 255) * 128);
   Tensor out = bits.view(at::kBFloat16);
   std::lock_guard<std::mutex> lock(g_cache_mutex);
-  g_cache.insert_or_assign(key, NativeEntry{c10::weak_intrusive_ptr<c10::TensorImpl>(b_scales.getIntrusivePtr()),
-                                            out, -1, exponent_offset, -1, version_of(b_scales)});
+  evict_stale_locked(b_scales, key);
+  invalidate_range_locked(key, b_scales.nbytes());
+  NativeEntry entry{c10::weak_intrusive_ptr<c10::TensorImpl>(b_scales.getIntrusivePtr()), out, -1, exponent_offset,
+                    -1, version_of(b_scales), b_scales.nbytes(), stream, nullptr};
+  record_conversion(entry, stream);
+  g_cache.insert_or_assign(key, entry);
   return out;
 }
 
@@ -135,8 +232,24 @@ bool is_mx_scale_type(const Tensor& t) {
 int64_t marlin_weight_cache_clear() {
   std::lock_guard<std::mutex> lock(g_cache_mutex);
   const int64_t n = (int64_t)g_cache.size();
+  for (auto& kv : g_cache) drop_event(kv.second);
   g_cache.clear();
   return n;
+}
+
+// Drops the converted copies made from the memory of `t` (weights or block scales): to be called
+// after the bytes of `t` were rewritten in place in a way that leaves its version counter alone.
+int64_t marlin_weight_cache_invalidate(const Tensor& t) {
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  const size_t before = g_cache.size();
+  if (t.defined() && t.numel() > 0) invalidate_range_locked(t.const_data_ptr(), t.nbytes());
+  return (int64_t)(before - g_cache.size());
+}
+
+// The repack ops have just written `out`: whatever was converted from that memory before is stale.
+void forget_memory_of(const Tensor& out) {
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  if (out.numel() > 0) invalidate_range_locked(out.const_data_ptr(), out.nbytes());
 }
 
 const void* opt_ptr(const OptTensor& t) {
@@ -173,6 +286,7 @@ Tensor gptq_marlin_repack(const Tensor& b_q_weight, const Tensor& perm, int64_t 
       has_perm ? static_cast<const int32_t*>(perm.const_data_ptr()) : nullptr,
       static_cast<uint32_t*>(out.mutable_data_ptr()), size_k, size_n, (int)num_bits,
       current_stream(b_q_weight)));
+  forget_memory_of(out);
   return out;
 }
 
@@ -196,6 +310,7 @@ Tensor awq_marlin_repack(const Tensor& b_q_weight, int64_t size_k, int64_t size_
   raise_if_failed(sonar_awq_marlin_repack(static_cast<const uint32_t*>(b_q_weight.const_data_ptr()),
                                           static_cast<uint32_t*>(out.mutable_data_ptr()), size_k,
                                           size_n, (int)num_bits, current_stream(b_q_weight)));
+  forget_memory_of(out);
   return out;
 }
 
@@ -589,6 +704,7 @@ TORCH_LIBRARY_FRAGMENT(_C, m) {
   // not in the reference: Marlin order -> gfx950 streaming order, and cache control
   m.def("marlin_to_gfx950(Tensor b_q_weight, SymInt size_k, SymInt size_n) -> Tensor");
   m.def("marlin_weight_cache_clear() -> int", &marlin_weight_cache_clear);
+  m.def("marlin_weight_cache_invalidate(Tensor t) -> int", &marlin_weight_cache_invalidate);
 }
 
 TORCH_LIBRARY_IMPL(_C, CUDA, m) {

@@ -144,3 +144,12 @@ def marlin_to_gfx950(b_q_weight: torch.Tensor, size_k: int, size_n: int) -> torc
 def marlin_weight_cache_clear() -> int:
     """Drops the converted weight copies the GEMM ops keep; returns how many there were."""
     return torch.ops._C.marlin_weight_cache_clear()
+
+
+def marlin_weight_cache_invalidate(t: torch.Tensor) -> int:
+    """Drops the converted copies made from the memory of `t` (a Marlin weight tensor or a
+    tensor of float8_e8m0fnu block scales); returns how many.  Needed after the bytes of `t`
+    were rewritten in place in a way its version counter does not show (`t.data.copy_(...)`,
+    any write to an inference-mode tensor).  Weights that come out of the repack ops, and
+    in-place ops on `t` itself, need no call."""
+    return torch.ops._C.marlin_weight_cache_invalidate(t)

@@ -100,6 +100,117 @@ def test_weight_cache_lets_go_of_dropped_weights():
     assert ops.marlin_weight_cache_clear() == 1
 
 
+def _gemm_through_op(a, marlin, scales, ws, m, n, k):
+    from sonar_amd import ops
+    from sonar_amd.scalar_type import scalar_types
+    empty = torch.empty(0, dtype=torch.int32, device=gu.DEV)
+    return ops.marlin_gemm(a, None, marlin, None, scales, None, None, empty, empty, empty, ws,
+                           scalar_types.uint4b8, m, n, k, True, False, True, False)
+
+
+def test_weight_cache_follows_the_reference_reload_idioms():
+    """The ways a caller replaces a weight after its first GEMM: `x.data = repack(...)`
+    (the reference's own idiom, marlin.py transform_w_q), also when the allocator
+    hands the old address back; `x.data.copy_(...)` followed by
+    marlin_weight_cache_invalidate; an inference-mode tensor refilled in place."""
+    from sonar_amd import ops
+    k, n, m = 512, 256, 8
+    a32 = mo.make_activations(3, m, k, "fp16")
+    a = gu.dev_bits16(a32, "fp16")
+    first, second = gu.DeviceLayer(31, k, n, 128, "fp16"), gu.DeviceLayer(32, k, n, 128, "fp16")
+
+    def check(out, layer):
+        ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(out), mo.gemm_reference(a32, layer.w_ref))
+        assert ok, worst
+
+    ops.marlin_weight_cache_clear()
+    # 1. x.data = new tensor from the repack op
+    param = torch.nn.Parameter(first.marlin.clone(), requires_grad=False)
+    check(_gemm_through_op(a, param, first.scales, first.workspace, m, n, k), first)
+    param.data = gu.gptq_repack(gu.dev_i32(mo.gptq_pack(second.layer["q"])), None, k, n)
+    check(_gemm_through_op(a, param, second.scales, first.workspace, m, n, k), second)
+    assert ops.marlin_weight_cache_clear() == 1      # the entry of the old address is gone
+
+    # 2. the same when the new weight lands on the old address: the repack op itself forgets that memory
+    qw_first, qw_second = gu.dev_i32(mo.gptq_pack(first.layer["q"])), gu.dev_i32(mo.gptq_pack(second.layer["q"]))
+    empty = torch.empty(0, dtype=torch.int32, device=gu.DEV)
+    holder = ops.gptq_marlin_repack(qw_first, empty, k, n, 4)
+    param = torch.nn.Parameter(holder, requires_grad=False)
+    check(_gemm_through_op(a, param, first.scales, first.workspace, m, n, k), first)
+    address = param.data_ptr()
+    del holder
+    param.data = torch.empty(0, dtype=torch.int32, device=gu.DEV)     # frees the block; the allocator reuses it
+    param.data = ops.gptq_marlin_repack(qw_second, empty, k, n, 4)
+    if param.data_ptr() != address:
+        pytest.skip("the allocator did not hand the old block back")
+    check(_gemm_through_op(a, param, second.scales, first.workspace, m, n, k), second)
+
+    # 3. bytes rewritten through .data (no version bump): the caller invalidates
+    param = torch.nn.Parameter(first.marlin.clone(), requires_grad=False)
+    check(_gemm_through_op(a, param, first.scales, first.workspace, m, n, k), first)
+    version = param._version
+    param.data.copy_(second.marlin)
+    assert param._version == version
+    assert ops.marlin_weight_cache_invalidate(param) == 1
+    check(_gemm_through_op(a, param, second.scales, first.workspace, m, n, k), second)
+
+    # 4. an inference-mode tensor refilled in place
+    with torch.inference_mode():
+        w = first.marlin.clone()
+        check(_gemm_through_op(a, w, first.scales, first.workspace, m, n, k), first)
+        w.copy_(second.marlin)
+        assert ops.marlin_weight_cache_invalidate(w) == 1
+        check(_gemm_through_op(a, w, second.scales, first.workspace, m, n, k), second)
+    ops.marlin_weight_cache_clear()
+
+
+def test_first_use_of_a_weight_inside_graph_capture_is_refused():
+    from sonar_amd import ops
+    k, n, m = 256, 128, 4
+    dl = gu.DeviceLayer(41, k, n, 128, "fp16")
+    a = gu.dev_bits16(mo.make_activations(1, m, k, "fp16"), "fp16")
+    ops.marlin_weight_cache_clear()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with pytest.raises(RuntimeError, match="warm-up"):
+            with torch.cuda.graph(graph, stream=stream):
+                _gemm_through_op(a, dl.marlin, dl.scales, dl.workspace, m, n, k)
+    torch.cuda.synchronize()
+    # after a warm-up call the capture goes through and replays give the eager result
+    want = _gemm_through_op(a, dl.marlin, dl.scales, dl.workspace, m, n, k)
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            got = _gemm_through_op(a, dl.marlin, dl.scales, dl.workspace, m, n, k)
+        for _ in range(3):
+            got.zero_()
+            graph.replay()
+            stream.synchronize()
+            assert torch.equal(got, want)
+
+
+def test_weight_converted_on_one_stream_is_safe_on_another():
+    from sonar_amd import ops
+    k, n, m = 4096, 4096, 4
+    dl = gu.DeviceLayer(43, 512, 256, 128, "fp16")          # oracle-sized reference
+    big = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, 2 * n), dtype=torch.int32, device=gu.DEV)
+    scales = torch.full((k // 128, n), 0.01, dtype=torch.float16, device=gu.DEV)
+    a = torch.randn((m, k), device=gu.DEV, dtype=torch.float16)
+    ws = dl.workspace
+    ops.marlin_weight_cache_clear()
+    s1, s2 = torch.cuda.Stream(), torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(s1):
+        first = _gemm_through_op(a, big, scales, ws, m, n, k)      # converts on s1
+    with torch.cuda.stream(s2):
+        second = _gemm_through_op(a, big, scales, torch.zeros_like(ws), m, n, k)   # hits the cache from s2
+    torch.cuda.synchronize()
+    assert torch.equal(first, second)
+    ops.marlin_weight_cache_clear()
+
+
 def test_marlin_gemm_op_rejects_like_the_reference():
     from sonar_amd import ops
     from sonar_amd.scalar_type import scalar_types
