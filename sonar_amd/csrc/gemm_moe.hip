@@ -523,9 +523,8 @@ extern "C" size_t sonar_moe_marlin_gemm_scratch_bytes(int64_t sorted_len, int64_
   (void)size_n;
   (void)size_k;
   // K is never split across workgroups, so no partial sums leave the chip; the
-  // tiled kernel for 64-slot blocks keeps its table of row tiles here (sized
-  // for any number of experts up to 1024)
-  return moe_block_size == 64 ? moe_tile_table_bytes(sorted_len, 1024) : 0;
+  // tiled kernel for 64-slot blocks keeps its table of row tiles here (one entry per block)
+  return moe_block_size == 64 ? moe_tile_table_bytes(sorted_len, 0) : 0;
 }
 
 extern "C" int sonar_moe_wna16_marlin_gemm(
@@ -659,7 +658,6 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
   static const bool no_tile = getenv("SONAR_MARLIN_NO_MOE_TILE") != nullptr;  // debugging aid
   // Full blocks of 64 slots mean many rows per expert: the MFMA-tiled kernel
   if (moe_block_size == 64 && !has_perm && !bits8 && !row_groups && !no_tile && size_k % 64 == 0 &&
-      num_experts <= 1024 &&
       (num_groups == 1 || group_size % 64 == 0 || group_size == 32) && scratch != nullptr &&
       scratch_bytes >= moe_tile_table_bytes(sorted_len, num_experts) && ((uintptr_t)scratch) % 4 == 0)
     return moe_tile_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,

@@ -860,10 +860,13 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   return launch_status("marlin_tile_kernel");
 }
 
-// Row tiles a grouped call can have at most, and the bytes of its tile table.
+// Row tiles a grouped call can have at most, and the bytes of its tile table.  A tile is a
+// run of up to four blocks of one expert; expert_ids need not be grouped by expert (blocks of
+// absent experts, -1, may sit between runs), so the bound is one tile per block: the table
+// can never be short of an entry, whatever the routing.
 int moe_tile_max(int64_t sorted_len, int64_t num_experts) {
-  const int64_t blocks = (sorted_len + 63) / 64;
-  return (int)((blocks + 3) / 4 + num_experts);
+  (void)num_experts;
+  return (int)((sorted_len + 63) / 64);
 }
 size_t moe_tile_table_bytes(int64_t sorted_len, int64_t num_experts) {
   return (size_t)(1 + 3 * moe_tile_max(sorted_len, num_experts)) * sizeof(int32_t);

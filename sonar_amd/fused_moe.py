@@ -168,13 +168,45 @@ def moe_sum(moe_output: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
     return torch.sum(moe_output, dim=1, out=out)
 
 
+def _activation_name(activation) -> str:
+    """`activation` as the reference passes it (a MoEActivation enum member, whose value is
+    the name) or as a plain string."""
+    return str(getattr(activation, "value", activation)).lower()
+
+
+def _check_unbuilt(activation, clamp_limit, gemm1_alpha, gemm1_beta, input_dtype, global_scales,
+                   activation_situ_beta=None, activation_situ_linear_beta=None) -> None:
+    if _activation_name(activation) != "silu":
+        raise NotImplementedError(f"activation {activation!r}: only SILU (silu(gate) * up) is built; the "
+                                  "reference's GELU, RELU2, SWIGLUOAI, SITU and no-mul variants are not")
+    if clamp_limit is not None or gemm1_alpha != 1.0 or gemm1_beta != 0.0:
+        raise NotImplementedError("clamp_limit / gemm1_alpha / gemm1_beta (SWIGLUOAI parameters) are not built")
+    if activation_situ_beta is not None or activation_situ_linear_beta is not None:
+        raise NotImplementedError("activation_situ_beta / activation_situ_linear_beta are not built")
+    if input_dtype is not None:
+        raise NotImplementedError("8-bit activations (input_dtype) are not built")
+    if any(g is not None for g in global_scales):
+        raise NotImplementedError("global scales (NVFP4 / 8-bit activations) are not built")
+
+
 def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, num_topk,
-                      quant_type: ScalarType, apply_router_weight_on_input, block_size_m, sorted_token_ids,
-                      expert_ids, num_tokens_post_padded, g_idx1=None, g_idx2=None, sort_indices1=None,
+                      quant_type: ScalarType, apply_router_weight_on_input, expert_map, block_size_m,
+                      sorted_token_ids, expert_ids, num_tokens_post_padded, activation="silu",
+                      activation_func=None, topk_ids=None, input_global_scale1=None, input_global_scale2=None,
+                      global_scale1=None, global_scale2=None, g_idx1=None, g_idx2=None, sort_indices1=None,
                       sort_indices2=None, w1_zeros=None, w2_zeros=None, workspace=None,
-                      intermediate_cache13=None, intermediate_cache2=None, output=None, is_k_full=True):
-    """Gate/up GEMM -> silu_and_mul -> down GEMM over already routed slots
-    (marlin_moe.py:57-223).  Returns the [M * top_k, K] per-slot outputs."""
+                      intermediate_cache13=None, intermediate_cache2=None, output=None, input_dtype=None,
+                      is_k_full=True, clamp_limit=None, gemm1_alpha=1.0, gemm1_beta=0.0,
+                      activation_situ_beta=None, activation_situ_linear_beta=None):
+    """Gate/up GEMM -> activation -> down GEMM over already routed slots
+    (marlin_moe.py:57-223; same parameters in the same order).  `activation_func`, when
+    given, is called as activation_func(activation, out [M * top_k, N], in [M * top_k, 2N])
+    like the reference's apply_moe_activation; the default is the HIP silu_and_mul.
+    `expert_map` and `topk_ids` are accepted for signature parity (the routing passed in
+    already reflects them).  Returns the [M * top_k, K] per-slot outputs."""
+    _check_unbuilt(activation, clamp_limit, gemm1_alpha, gemm1_beta, input_dtype,
+                   (input_global_scale1, input_global_scale2, global_scale1, global_scale2),
+                   activation_situ_beta, activation_situ_linear_beta)
     assert hidden_states.ndim == 2
     M, K = hidden_states.shape
     N = w2.shape[1] * 16                       # intermediate size: w2 is (E, N/16, 2K)
@@ -195,7 +227,10 @@ def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, t
         top_k=num_topk, mul_topk_weights=apply_router_weight_on_input, b_q_type=quant_type, size_m=M,
         size_n=2 * N, size_k=K, is_k_full=is_k_full, use_atomic_add=False, use_fp32_reduce=True,
         is_zp_float=False)
-    silu_and_mul(cache2, cache1.view(-1, 2 * N))
+    if activation_func is not None:
+        activation_func(activation, cache2, cache1.view(-1, 2 * N))
+    else:
+        silu_and_mul(cache2, cache1.view(-1, 2 * N))
     if output is None:
         output = cache3
     return ops.moe_wna16_marlin_gemm(
@@ -210,24 +245,35 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
                      bias1: torch.Tensor | None, bias2: torch.Tensor | None, w1_scale: torch.Tensor,
                      w2_scale: torch.Tensor, topk_weights: torch.Tensor, topk_ids: torch.Tensor,
                      quant_type_id: int, apply_router_weight_on_input: bool = False,
-                     global_num_experts: int = -1, expert_map: torch.Tensor | None = None,
+                     global_num_experts: int = -1, activation="silu", activation_func=None,
+                     moe_sum=None, expert_map: torch.Tensor | None = None,
+                     input_global_scale1: torch.Tensor | None = None,
+                     input_global_scale2: torch.Tensor | None = None,
+                     global_scale1: torch.Tensor | None = None, global_scale2: torch.Tensor | None = None,
                      g_idx1: torch.Tensor | None = None, g_idx2: torch.Tensor | None = None,
                      sort_indices1: torch.Tensor | None = None, sort_indices2: torch.Tensor | None = None,
                      w1_zeros: torch.Tensor | None = None, w2_zeros: torch.Tensor | None = None,
                      workspace: torch.Tensor | None = None,
                      intermediate_cache13: torch.Tensor | None = None,
                      intermediate_cache2: torch.Tensor | None = None, is_k_full: bool = True,
-                     output: torch.Tensor | None = None, input_dtype: torch.dtype | None = None
-                     ) -> torch.Tensor:
+                     output: torch.Tensor | None = None, input_dtype: torch.dtype | None = None,
+                     clamp_limit: float | None = None, gemm1_alpha: float = 1.0, gemm1_beta: float = 0.0,
+                     activation_situ_beta: float | None = None,
+                     activation_situ_linear_beta: float | None = None) -> torch.Tensor:
     """Mixture-of-experts layer with Marlin int4 expert weights and top-k gating
     (marlin_moe.py:226-392).  w1: (E, K/16, 2 * 2N) gate and up projections,
     w2: (E, N/16, 2K); scales (E, groups, 2N) / (E, groups, K); topk_weights
-    fp32 [M, top_k]; topk_ids [M, top_k].  Returns [M, K]."""
+    fp32 [M, top_k]; topk_ids [M, top_k].  Returns [M, K].  Parameters and their order are
+    the reference's; of its activations only SILU is built (anything else, and clamp_limit /
+    gemm1_alpha / gemm1_beta / global scales / input_dtype, raise NotImplementedError).
+    `activation_func(activation, out, in)` and `moe_sum(moe_output [M, top_k, K], output)`
+    replace the built-in HIP kernels when given, as in the reference."""
+    _check_unbuilt(activation, clamp_limit, gemm1_alpha, gemm1_beta, input_dtype,
+                   (input_global_scale1, input_global_scale2, global_scale1, global_scale2),
+                   activation_situ_beta, activation_situ_linear_beta)
     if quant_type_id not in _SUPPORTED:
         raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8, uint8b128, "
                                   "float8_e4m3fn and float4_e2m1f (MXFP4) expert weights are built")
-    if input_dtype is not None:
-        raise NotImplementedError("8-bit activations are not built")
     quant_type = _SUPPORTED[quant_type_id]
     M, K = hidden_states.shape
     E = w1.shape[0]
@@ -249,9 +295,11 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
     sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(
         topk_ids, block_size_m, global_num_experts, expert_map, ignore_invalid_experts=True)
 
+    sum_rows = moe_sum
     moe_output = _fused_marlin_moe(
         hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, topk, quant_type,
-        apply_router_weight_on_input, block_size_m, sorted_token_ids, expert_ids, num_tokens_post_padded,
+        apply_router_weight_on_input, expert_map, block_size_m, sorted_token_ids, expert_ids,
+        num_tokens_post_padded, activation=activation, activation_func=activation_func, topk_ids=topk_ids,
         g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1, sort_indices2=sort_indices2,
         w1_zeros=w1_zeros, w2_zeros=w2_zeros, workspace=workspace,
         intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2, output=None,
@@ -259,10 +307,15 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
     if output is None:
         output = torch.empty_like(hidden_states)
     if expert_map is not None:
-        # slots of experts held elsewhere were never written
-        local = expert_map.to(torch.int64)[topk_ids.to(torch.int64).clamp(0, global_num_experts - 1)] >= 0
+        # slots of experts held elsewhere (or with an id outside the table) were never written
+        ids = topk_ids.to(torch.int64)
+        inside = (ids >= 0) & (ids < global_num_experts)
+        local = inside & (expert_map.to(torch.int64)[ids.clamp(0, global_num_experts - 1)] >= 0)
         moe_output = torch.where(local.unsqueeze(-1), moe_output, torch.zeros_like(moe_output))
-    return moe_sum(moe_output.contiguous(), output)
+    if sum_rows is not None:
+        sum_rows(moe_output.contiguous(), output)
+        return output
+    return globals()["moe_sum"](moe_output.contiguous(), output)
 
 
 def batched_fused_marlin_moe(hidden_states: torch.Tensor, expert_num_tokens: torch.Tensor, w1: torch.Tensor,
@@ -305,8 +358,8 @@ def batched_fused_marlin_moe(hidden_states: torch.Tensor, expert_num_tokens: tor
     topk_weights = torch.ones((M, 1), device=hidden_states.device, dtype=torch.float32)
     out = _fused_marlin_moe(
         hidden_states.view(-1, K), w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, 1,
-        _SUPPORTED[quant_type_id], apply_router_weight_on_input, block_size_m, sorted_token_ids, expert_ids,
-        num_tokens_post_padded, g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1,
+        _SUPPORTED[quant_type_id], apply_router_weight_on_input, None, block_size_m, sorted_token_ids,
+        expert_ids, num_tokens_post_padded, g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1,
         sort_indices2=sort_indices2, w1_zeros=w1_zeros, w2_zeros=w2_zeros, workspace=workspace,
         intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2,
         output=output.view(-1, K) if output is not None else None, is_k_full=is_k_full)

@@ -433,3 +433,27 @@ def test_full_size_grouped_tile_gemm_agrees_with_dense_rows():
             dense = ex.layers[int(ti_host[t, j])].gemm(a[t:t + 1].contiguous(), 1)
             err = float((dense.float() - got[t * top_k + j].float()).abs().max())
             assert err <= 1e-2 * scale, (t, j, err, scale)
+
+
+def test_tile_kernel_with_expert_ids_that_are_not_grouped_by_expert():
+    """64-slot blocks whose experts alternate, with blocks of absent experts (-1) in
+    between: every block is a run of its own, more runs than experts.  The table of
+    row tiles has an entry per block, so no block may be dropped."""
+    m, e, top_k, k, n, bs = 64 * 14, 3, 1, 256, 256, 64
+    ex = Experts(301, e, k, n, 128, "bf16")
+    blocks = m // bs
+    pattern = [0, 1, -1, 2, 0, -1, 1, 2, 0, 1, 2, -1, 0, 2]
+    assert len(pattern) == blocks
+    expert_ids = np.array(pattern, dtype=np.int32)
+    rng = np.random.default_rng(5)
+    sorted_ids = rng.permutation(m).astype(np.int32)          # every block full, ids in any order
+    weights = rng.random((m, top_k)).astype(np.float32)
+    a32 = mo.make_activations(9, m, k, "bf16")
+    a = gu.dev_bits16(a32, "bf16")
+    got = gu.host_f32(ex.gemm(a, sorted_ids, expert_ids, m, weights, bs, top_k, m, True))
+    want = ex.reference(a32, sorted_ids, expert_ids, m, bs, top_k, m, weights)
+    written = np.concatenate([sorted_ids[b * bs:(b + 1) * bs] for b in range(blocks) if pattern[b] >= 0])
+    ok, *worst = mo.gemm_tolerance_ok(got[written], want[written])
+    assert ok, worst
+    skipped = np.concatenate([sorted_ids[b * bs:(b + 1) * bs] for b in range(blocks) if pattern[b] < 0])
+    assert np.all(got[skipped] == 0)          # Experts.gemm hands the op a zeroed output
