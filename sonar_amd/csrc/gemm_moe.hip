@@ -23,7 +23,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
                   int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, hipStream_t st);
+                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, int bits, bool fp8, hipStream_t st);
 size_t moe_tile_table_bytes(int64_t sorted_len, int64_t num_experts);
 // gemm_stream.hip: the 16-row decode kernel in grouped form, for few rows per expert
 bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t sorted_len, int64_t num_experts,
@@ -657,13 +657,13 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                          num_experts, dtype, size_m, size_n, size_k, num_groups, group_size, a_by_slot, fp4, st);
   static const bool no_tile = getenv("SONAR_MARLIN_NO_MOE_TILE") != nullptr;  // debugging aid
   // Full blocks of 64 slots mean many rows per expert: the MFMA-tiled kernel
-  if (moe_block_size == 64 && !has_perm && !bits8 && !row_groups && !no_tile && size_k % 64 == 0 &&
+  if (moe_block_size == 64 && !has_perm && !row_groups && !no_tile && size_k % 64 == 0 &&
       (num_groups == 1 || group_size % 64 == 0 || group_size == 32) && scratch != nullptr &&
       scratch_bytes >= moe_tile_table_bytes(sorted_len, num_experts) && ((uintptr_t)scratch) % 4 == 0)
     return moe_tile_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
                          num_tokens_past_padded, topk_weights, top_k, mul_topk_weights ? 1 : 0, num_experts,
                          static_cast<int32_t*>(scratch), dtype, size_m, size_n, size_k, num_groups, group_size,
-                         a_by_slot, fp4, st);
+                         a_by_slot, fp4, bits8 ? 8 : 4, fp8, st);
 
   MoeParams p;
   p.a = static_cast<const uint16_t*>(a);

@@ -29,7 +29,7 @@ namespace sonar {
 int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
               const void* scales, const uint32_t* zeros, const int32_t* perm, int dtype, int64_t size_m,
               int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
-              size_t partial_bytes, bool fp4, hipStream_t st);
+              size_t partial_bytes, bool fp4, int bits, bool fp8, hipStream_t st);
 bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size);
 
 #ifdef SONAR_TRACE
@@ -1837,7 +1837,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
   // the row -> group lookup and 8-bit codes exist in the streaming kernels only
   // (MXFP4 only through the asynchronous tile kernel: the older one has no float4 dequantiser)
-  const bool use_tile = plan.tile && !no_tile && !chk.row_groups && chk.bits == 4 && (!chk.fp4 || async_tile) &&
+  // (8-bit codes and MXFP4 only through the asynchronous tile kernel: the older one has neither dequantiser)
+  const bool use_tile = plan.tile && !no_tile && !chk.row_groups && ((chk.bits == 4 && !chk.fp4) || async_tile) &&
                         !(slab_fast && p.unit_chunks == 4);
   // More than 64 rows in the general kernels (8-bit codes, is_k_full = false,
   // the tile path switched off) on a matrix of short strips: one workgroup per
@@ -1861,7 +1862,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
     const size_t used = stream_scratch_bytes();
     return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
                      size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used,
-                     scratch_bytes > used ? scratch_bytes - used : 0, chk.fp4, st);
+                     scratch_bytes > used ? scratch_bytes - used : 0, chk.fp4, chk.bits, chk.fp8, st);
   }
 
   // The fast kernel: up to 16 rows, or more rows in blocks of 16 or 32 (slab_fast), all in

@@ -16,6 +16,7 @@
 // Workgroup ids are dealt so that the 32 workgroups resident on one XCD (ids
 // congruent mod 8) take neighbouring tiles (tile_of_workgroup).
 #include <cstdlib>
+#include <type_traits>
 
 #include "dequant.hpp"
 #include "gemm_plan.hpp"
@@ -312,13 +313,26 @@ constexpr int wave_stage(bool g32) { return 2 * kBlockBytes + (g32 ? 512 : 256);
 constexpr int kAsyncA = kAsyncStages * kStageA;
 constexpr int async_lds(bool g32) { return kAsyncA + kTileWaves * kAsyncStages * wave_stage(g32); }
 constexpr int async_copies(bool g32) { return g32 ? 8 : 7; }
+// 8-bit codes (W8 = 1: uint8b128, 2: float8_e4m3fn): a K step of a strip is four 1-KiB blocks
+// of 16 rows (block 2 b holds the low four, block 2 b + 1 the high four of the eight
+// consecutive rows of a lane's operand of k block b).  Private rings of that size would not
+// fit, so the two wavefronts of a strip (one per group of rows) share one ring: the
+// wavefront of group 0 copies the two blocks of k block 0, that of group 1 those of k block
+// 1, the same number of copies per stage as with 4-bit codes.  The barriers that order the
+// shared stages of A order these too: group 1 reads k block 0 one phase after group 0 has
+// waited for its copies, group 0 reads k block 1 two barriers after group 1 has.
+constexpr int strip_stage8(bool g32) { return 4 * kBlockBytes + (g32 ? 512 : 256); }
+constexpr int async_lds8(bool g32) { return kAsyncA + (kTileN / kStripN) * kAsyncStages * strip_stage8(g32); }
 
-template <typename T, bool HAS_ZP, bool GROUPED, bool G32 = false, bool FP4 = false>
+template <typename T, bool HAS_ZP, bool GROUPED, bool G32 = false, bool FP4 = false, int W8 = 0>
 __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq4Of<T, FP4>::type D4;   // integer codes, or float4_e2m1f (MXFP4: with G32)
-  typedef typename D4::Col Col;
-  constexpr int kWaveStage = wave_stage(G32);
+  typedef typename Dq8Of<T, W8 == 2>::type D8;   // 8-bit integer or floating-point codes (W8 != 0)
+  typedef typename std::conditional<W8 != 0, typename D8::Col, typename D4::Col>::type Col;
+  static_assert(W8 == 0 || (!HAS_ZP && !FP4), "8-bit codes are symmetric");
+  constexpr int kWaveStage = W8 ? strip_stage8(G32) : wave_stage(G32);
+  constexpr int kWeightBytes = (W8 ? 4 : 2) * kBlockBytes;   // packed weights of a stage, scale rows behind them
   constexpr int kAsyncCopies = async_copies(G32);
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -379,7 +393,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     }
     a_src[i] = reinterpret_cast<const char*>(p.a) + ((long)row * p.lda + 8 * ((lane & 7) ^ r8)) * 2;
   }
-  const uint4* b_src = p.b + expert * p.expert_b_stride + (size_t)(unsigned)(strip * p.chunks_per_strip) * 64 + lane;
+  const uint4* b_src = p.b + expert * p.expert_b_stride +
+                       (size_t)(unsigned)(strip * p.chunks_per_strip) * (W8 ? 128 : 64) + lane;
   const char* s_src;
   long s_group_stride;
   if (HAS_ZP && lane >= 32) {
@@ -389,7 +404,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     s_src = reinterpret_cast<const char*>(p.scales + expert * p.expert_s_stride + strip * kStripN) + 4 * (lane & 31);
     s_group_stride = (long)p.size_n * 2;
   }
-  char* wring = smem + kAsyncA + wave * (kAsyncStages * kWaveStage);
+  // the weight ring: private to the wavefront, or shared by the two wavefronts of a strip (8-bit codes)
+  char* wring = smem + kAsyncA + (W8 ? wn : wave) * (kAsyncStages * kWaveStage);
   const uint32_t a_lds = (uint32_t)(uintptr_t)(lds_void_t*)smem;
   const uint32_t w_lds = (uint32_t)(uintptr_t)(lds_void_t*)wring;
 
@@ -403,18 +419,25 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     }
     char* sw = wring + slot * kWaveStage;
     if (idx < 6) {
+      if (W8) {   // blocks 2 wm, 2 wm + 1 of the four of this step: the two of k block wm
+        const int blk = 2 * wm + (idx - 4);
+        const uint4* g = b_src + (size_t)(4 * kt + blk) * 64;
+        __builtin_amdgcn_global_load_lds((glb_void_t*)g, (lds_void_t*)(sw + blk * kBlockBytes), 16, 0, 0);
+        return;
+      }
       const uint4* g = b_src + (size_t)(2 * kt + (idx - 4)) * 64;   // the two chunks of this step
       __builtin_amdgcn_global_load_lds((glb_void_t*)g, (lds_void_t*)(sw + (idx - 4) * kBlockBytes), 16, 0, 0);
       return;
     }
+    // the scale rows (with a shared ring both wavefronts of the strip copy them: the same bytes twice)
     if (G32) {   // idx 6 / 7: the rows of groups 2 kt and 2 kt + 1
       __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)(2 * kt + (idx - 6)) * s_group_stride),
-                                       (lds_void_t*)(sw + 2 * kBlockBytes + 256 * (idx - 6)), 4, 0, 0);
+                                       (lds_void_t*)(sw + kWeightBytes + 256 * (idx - 6)), 4, 0, 0);
       return;
     }
     const int grp = grouped ? (kt * kTileK) / p.group_size : 0;
     __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)grp * s_group_stride),
-                                     (lds_void_t*)(sw + 2 * kBlockBytes), 4, 0, 0);
+                                     (lds_void_t*)(sw + kWeightBytes), 4, 0, 0);
   };
   auto issue = [&](int kt, int slot) {
 #pragma unroll
@@ -423,8 +446,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 
   uint32_t s_off[4];
 #pragma unroll
-  for (int j = 0; j < 4; ++j) s_off[j] = 2 * kBlockBytes + 2 * scale_slot(16 * j + col16, grouped);
-  const uint32_t z_off = 2 * kBlockBytes + 128 + 4 * zero_point_word(col16);
+  for (int j = 0; j < 4; ++j) s_off[j] = kWeightBytes + 2 * scale_slot(16 * j + col16, grouped);
+  const uint32_t z_off = kWeightBytes + 128 + 4 * zero_point_word(col16);
 
   floatx4_t acc[4][8];
 #pragma unroll
@@ -439,6 +462,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   issue(min(k_first + 1, k_tiles - 1), 1);
 
   u32x4_t av[8], wv[4], qraw;
+  u32x4_t qhigh = u32x4_t{0u, 0u, 0u, 0u};   // 8-bit codes: the block with the high four rows
   uint32_t sb0 = 0, sb1 = 0, sb2 = 0, sb3 = 0, zw = 0;
   Col cols[4];
 // Starts one 16-byte LDS read into `dst`; the data is there after the next
@@ -460,8 +484,9 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   // that stage must have landed.  The data is picked up by the next fetch().
   auto raw_start = [&](int slot, int b, bool with_scales) {
     const uint32_t w_at = w_lds + slot * kWaveStage;
-    const uint32_t q_at = w_at + b * kBlockBytes + lane * 16;
+    const uint32_t q_at = w_at + (W8 ? 2 * b : b) * kBlockBytes + lane * 16;
     const uint32_t r_at = w_at + (G32 ? 256 * b : 0);   // this k block's scale row
+    if constexpr (W8 != 0) asm volatile("ds_read_b128 %0, %1 offset:1024" : "=&v"(qhigh) : "v"(q_at) : "memory");
     if (with_scales) {
       asm volatile(
           "ds_read_b128 %0, %6\n\t"
@@ -482,10 +507,17 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   // started by raw_start, starts the reads of the eight blocks of A and
   // dequantises the chunk while they are in flight.
   auto fetch = [&](int slot, int b, bool with_scales) {
-    asm volatile("s_waitcnt lgkmcnt(0)"
-                 : "+v"(qraw), "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw)
-                 :
-                 : "memory");
+    if constexpr (W8 != 0) {
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(qraw), "+v"(qhigh), "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw)
+                   :
+                   : "memory");
+    } else {
+      asm volatile("s_waitcnt lgkmcnt(0)"
+                   : "+v"(qraw), "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw)
+                   :
+                   : "memory");
+    }
     // operand lane (kb, col16) of row block rb, k block b: piece 4 b + kb of row col16
     const uint32_t a_at = a_lds + slot * kStageA + (8 * wm * 2 + (col16 >> 3)) * kBlockBytes + (col16 & 7) * 128 +
                           (((4 * b + kb) ^ (col16 & 7)) * 16);
@@ -501,15 +533,28 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
       const uint32_t sbits[4] = {sb0, sb1, sb2, sb3};
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
-        int z = 8;
-        if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
-        cols[j] = D4::make_col((uint16_t)sbits[j], z);
+        if constexpr (W8 != 0) {
+          cols[j] = D8::make_col((uint16_t)sbits[j]);
+        } else {
+          int z = 8;
+          if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
+          cols[j] = D4::make_col((uint16_t)sbits[j], z);
+        }
       }
     }
-    wv[0] = __builtin_bit_cast(u32x4_t, D4::word(qraw.x, cols[0], magic));
-    wv[1] = __builtin_bit_cast(u32x4_t, D4::word(qraw.y, cols[1], magic));
-    wv[2] = __builtin_bit_cast(u32x4_t, D4::word(qraw.z, cols[2], magic));
-    wv[3] = __builtin_bit_cast(u32x4_t, D4::word(qraw.w, cols[3], magic));
+    if constexpr (W8 != 0) {
+      const uint32_t lo[4] = {qraw.x, qraw.y, qraw.z, qraw.w}, hi[4] = {qhigh.x, qhigh.y, qhigh.z, qhigh.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const uint2 w_lo = D8::word4(lo[j], cols[j], magic), w_hi = D8::word4(hi[j], cols[j], magic);
+        wv[j] = u32x4_t{w_lo.x, w_lo.y, w_hi.x, w_hi.y};
+      }
+    } else {
+      wv[0] = __builtin_bit_cast(u32x4_t, D4::word(qraw.x, cols[0], magic));
+      wv[1] = __builtin_bit_cast(u32x4_t, D4::word(qraw.y, cols[1], magic));
+      wv[2] = __builtin_bit_cast(u32x4_t, D4::word(qraw.z, cols[2], magic));
+      wv[3] = __builtin_bit_cast(u32x4_t, D4::word(qraw.w, cols[3], magic));
+    }
     SONAR_TILE_LANDED();
   };
   // Multiply phase: 32 MFMAs, ahead of the other wavefront's VALU work in the issue order.
@@ -569,7 +614,12 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   }
   if (wm == 0) phase_end();  // the barrier that ends group 1's last phase
   // the last copies and the last read started by raw_start must not outlive the wavefront
-  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(qraw), "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw)::"memory");
+  if constexpr (W8 != 0) {
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)"
+                 : "+v"(qraw), "+v"(qhigh), "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw)::"memory");
+  } else {
+    asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(qraw), "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw)::"memory");
+  }
 #undef SONAR_TILE_LANDED
 #undef SONAR_TILE_READ
 
@@ -737,6 +787,28 @@ int launch_tile_grouped_fp4(const TileParams& p, hipStream_t st) {
   return SONAR_OK;
 }
 
+// 8-bit codes (W8 = 1: uint8b128, 2: float8_e4m3fn), dense or grouped
+template <typename T, bool GROUPED, bool G32, int W8>
+int launch_tile_async8_groups(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, false, GROUPED, G32, false, W8>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, async_lds8(G32)));
+    attr_set = true;
+  }
+  marlin_tile_async_kernel<T, false, GROUPED, G32, false, W8>
+      <<<tile_grid(p), kTileWaves * 64, async_lds8(G32), st>>>(p);
+  return SONAR_OK;
+}
+template <typename T, bool GROUPED>
+int launch_tile_async8(const TileParams& p, bool fp8, hipStream_t st) {
+  const bool g32 = p.num_groups > 1 && p.group_size == 32;
+  if (fp8) return g32 ? launch_tile_async8_groups<T, GROUPED, true, 2>(p, st)
+                      : launch_tile_async8_groups<T, GROUPED, false, 2>(p, st);
+  return g32 ? launch_tile_async8_groups<T, GROUPED, true, 1>(p, st)
+             : launch_tile_async8_groups<T, GROUPED, false, 1>(p, st);
+}
+
 template <typename T, bool HAS_ZP>
 int launch_tile_async(const TileParams& p, hipStream_t st) {
   return (p.num_groups > 1 && p.group_size == 32) ? launch_tile_async_groups<T, HAS_ZP, true>(p, st)
@@ -786,7 +858,7 @@ bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size) {
 int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
               const void* scales, const uint32_t* zeros, const int32_t* perm, int dtype, int64_t size_m,
               int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
-              size_t partial_bytes, bool fp4, hipStream_t st) {
+              size_t partial_bytes, bool fp4, int bits, bool fp8, hipStream_t st) {
   TileParams p;
   p.a = static_cast<const uint16_t*>(a);
   p.lda = a_row_stride;
@@ -835,6 +907,9 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     }
     if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
       rc = launch_tile_async_fp4(p, st);
+    else if (bits == 8)   // symmetric 8-bit codes: the caller has checked
+      rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, false>(p, fp8, st)
+                                    : launch_tile_async8<__bf16, false>(p, fp8, st);
     else if (dtype == SONAR_DTYPE_F16)
       rc = zp ? launch_tile_async<_Float16, true>(p, st) : launch_tile_async<_Float16, false>(p, st);
     else
@@ -849,6 +924,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     }
     return SONAR_OK;
   }
+  if (bits == 8) return fail(SONAR_E_INVALID, "internal: 8-bit codes exist in the asynchronous tile kernel only");
   if (dtype == SONAR_DTYPE_F16) {
     rc = zp ? (pm ? launch_tile<_Float16, true, true>(p, st) : launch_tile<_Float16, true, false>(p, st))
             : (pm ? launch_tile<_Float16, false, true>(p, st) : launch_tile<_Float16, false, false>(p, st));
@@ -878,7 +954,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
                   int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, hipStream_t st) {
+                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, int bits, bool fp8, hipStream_t st) {
   const int max_tiles = moe_tile_max(sorted_len, num_experts);
   const int blocks_max = (int)((sorted_len + 63) / 64);
   moe_tile_table_kernel<<<1, 256, (size_t)blocks_max * sizeof(int32_t), st>>>(expert_ids, num_post_pad, blocks_max, 64,
@@ -913,13 +989,16 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.top_k = (int)top_k;
   p.mul_topk = mul_topk;
   p.a_by_slot = a_by_slot;
-  p.expert_b_stride = (long)(size_k * size_n / 8 / 4);
+  p.expert_b_stride = (long)(size_k * size_n / (32 / bits) / 4);
   p.expert_s_stride = (long)(num_groups * size_n);
   p.expert_z_stride = (long)(num_groups * (size_n / 8));
   p.expert_bias_stride = (long)size_n;
   int rc;
   if (fp4)
     rc = launch_tile_grouped_fp4(p, st);
+  else if (bits == 8)
+    rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, true>(p, fp8, st)
+                                  : launch_tile_async8<__bf16, true>(p, fp8, st);
   else if (dtype == SONAR_DTYPE_F16)
     rc = zeros ? launch_tile_grouped<_Float16, true>(p, st) : launch_tile_grouped<_Float16, false>(p, st);
   else

@@ -248,8 +248,12 @@ def test_moe_matches_dense_gemm_per_expert():
     assert ok, worst
 
 
-@pytest.mark.parametrize("tokens,k,n", [(16, 4096, 28672), (64, 14336, 4096), (256, 4096, 28672), (600, 14336, 4096)])
-def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n):
+@pytest.mark.parametrize("tokens,k,n,wtype", [
+    (16, 4096, 28672, "uint4b8"), (64, 14336, 4096, "uint4b8"), (256, 4096, 28672, "uint4b8"),
+    (600, 14336, 4096, "uint4b8"),
+    # 8-bit codes: blocks of 64 slots run the tile kernel's 8-bit form, smaller ones the general grouped kernel
+    (700, 4096, 2048, "uint8b128"), (2048, 2048, 1024, "fp8"), (64, 2048, 1024, "uint8b128")])
+def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     """Mixtral-8x7B expert shapes (8 experts, top 2, the block size of the
     reference's rule), where the CPU oracle is too slow: every routed slot must
     equal, within the GEMM tolerance, the dense op on the same token row and
@@ -260,9 +264,15 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n):
     e, top_k, dtype = 8, 2, torch.bfloat16
     gen = torch.Generator(device=gu.DEV).manual_seed(tokens + n)
     lib = _lib.load()
-    words = k * n // 8
+    b_type = {"uint4b8": _lib.TYPE_UINT4B8, "uint8b128": _lib.TYPE_UINT8B128, "fp8": _lib.TYPE_FLOAT8_E4M3FN}[wtype]
+    words = k * n // (8 if wtype == "uint4b8" else 4)
     native = torch.randint(-2 ** 31, 2 ** 31 - 1, (e, words), dtype=torch.int32, device=gu.DEV, generator=gen)
-    scales = (torch.rand((e, k // 128, n), device=gu.DEV, generator=gen) * 9e-3 + 1e-3).to(dtype)
+    scales = torch.rand((e, k // 128, n), device=gu.DEV, generator=gen) * 9e-3 + 1e-3
+    if wtype == "uint8b128":
+        scales = scales / 16
+    if wtype == "fp8":   # the exponent bias of the codes is folded into the scales: 2^120 for bf16
+        scales = scales * 2.0 ** 120
+    scales = scales.to(dtype)
     a = torch.randn((tokens, k), device=gu.DEV, generator=gen).to(dtype)
     topk_ids, topk_w = route(tokens, tokens, e, top_k)
     bs = mo.moe_block_size_rule(tokens, top_k, e)
@@ -276,7 +286,7 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n):
     _lib.check(lib.sonar_moe_wna16_marlin_gemm(
         gu.ptr(a), gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None, gu.ptr(scales), None, None, None,
         gu.ptr(workspace), workspace.numel(), gu.ptr(scr), nbytes, gu.ptr(sid), sid.numel(), gu.ptr(eid),
-        gu.ptr(npp), None, bs, top_k, 0, e, _lib.DTYPE_BF16, _lib.TYPE_UINT4B8, tokens, n, k, k // 128, 1, 0, 1,
+        gu.ptr(npp), None, bs, top_k, 0, e, _lib.DTYPE_BF16, b_type, tokens, n, k, k // 128, 1, 0, 1,
         gu.stream()))
     torch.cuda.synchronize()
     assert bool(torch.isfinite(c.float()).all())
@@ -293,7 +303,7 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n):
         _lib.check(lib.sonar_marlin_gemm(
             gu.ptr(rows), k, gu.ptr(dense), gu.ptr(native[ex]), _lib.LAYOUT_GFX950, None, gu.ptr(scales[ex]), None,
             None, None, gu.ptr(workspace), workspace.numel(), gu.ptr(dscr), dscr.numel(), _lib.DTYPE_BF16,
-            _lib.TYPE_UINT4B8, m, n, k, k // 128, 1, 0, 1, gu.stream()))
+            b_type, m, n, k, k // 128, 1, 0, 1, gu.stream()))
         got = c[torch.from_numpy(slots).to(gu.DEV)].float()
         err = float((got - dense.float()).abs().max())
         assert err <= 1e-2 * scale, (ex, err, scale)

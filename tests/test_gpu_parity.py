@@ -344,6 +344,12 @@ W8_CASES = [
     (100, 1024, 512, 128, False, False),
     (13, 1024, 256, 128, True, False),
     (300, 512, 192, 32, False, False),
+    # more than 128 rows on enough K steps or tiles: the MFMA tile kernel's 8-bit form
+    (300, 2048, 512, 128, False, True),      # K split over workgroups
+    (1024, 1024, 832, 128, False, False),    # a last column of tiles that is not full
+    (260, 1024, 4160, -1, False, False),     # one group
+    (512, 2048, 320, 32, False, True),       # groups of 32 rows
+    (300, 2048, 512, 128, True, False),      # act-order through the permuted copy of A
 ]
 
 
@@ -421,6 +427,10 @@ FP8_CASES = [
     (1, 4096, 4096, 128, False),
     (16, 1024, 256, 32, False),       # groups of 32 rows: MXFP8
     (100, 512, 192, 32, True),
+    # the MFMA tile kernel's form for 8-bit floating-point codes
+    (300, 2048, 512, 128, True),
+    (1024, 1024, 832, -1, False),
+    (512, 2048, 320, 32, True),
 ]
 
 
