@@ -32,26 +32,12 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
               size_t partial_bytes, bool fp4, int bits, bool fp8, hipStream_t st);
 bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size);
 
-#ifdef SONAR_TRACE
-unsigned long long* g_trace_host;
-#define TRACE(i)                                                                   \
-  do {                                                                             \
-    if (params.trace && (threadIdx.x & 63) == 0)                                   \
-      params.trace[((long)blockIdx.x * 8 + (threadIdx.x >> 6)) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
-  } while (0)
-#else
-#define TRACE(i)
-#endif
-
 namespace {
 
 constexpr int kWaves = 8;
 constexpr int kSlotFloat4 = 4 * 4 * 64;  // largest partial tile: 4 row blocks x 4 column blocks x 64 lanes
 
 struct StreamParams {
-#ifdef SONAR_TRACE
-  unsigned long long* trace;
-#endif
   const uint16_t* a;
   long lda;
   uint16_t* c;
@@ -712,9 +698,6 @@ template <int MB>
 __device__ __forceinline__ void copy_activations(const StreamParams& p, const FastLane<MB>& fl, int unit,
                                                  char* slot) {
   const char* ga = reinterpret_cast<const char*>(p.a) + (long)unit * (4 * kChunkK * 2);
-#ifdef SONAR_EXP_NO_A
-  return;
-#endif
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
     char* s = slot + 4096 * mb;
@@ -877,7 +860,6 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   constexpr int kPark = park_tiles(MB);       // tiles per wavefront and pass of the cross-wavefront sum
   constexpr int kPasses = 4 * MB / kPark;
   extern __shared__ __attribute__((aligned(1024))) char smem[];
-  TRACE(0);
   StreamParams p = params;
   // Every argument the dense path reads, fetched now in one batch of scalar loads: left to
   // itself the compiler fetches them where they are first used, four round trips to a cold
@@ -988,7 +970,6 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
   }
   if (mine > 1) copy_weights<MB, GPU>(p, fl, strip, unit + kFastWaves, ring + kSlotBytes, lane, unit_group_shift);
   int c_slot = 0;
-  TRACE(1);
 
   floatx4_t acc[MB][4];
 #pragma unroll
@@ -1039,7 +1020,6 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
         SONAR_GROUP_READS(3);
       }
     }
-    TRACE(2);
     if (left > 1) {
       copy_activations<MB>(p, fl, unit + kFastWaves, ring + kWaveA);
       if (left > 2)
@@ -1049,13 +1029,6 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     unit += kFastWaves;
     c_slot ^= 1;
 
-#ifdef SONAR_EXP_NO_COMPUTE
-    {
-      const u32x4_t x = q0 ^ q1 ^ q2 ^ q3 ^ a0 ^ a1 ^ a2 ^ a3 ^ row_z;
-      acc[0][0][0] += __uint_as_float((x.x ^ x.y ^ x.z ^ x.w ^ row_s[0] ^ row_s[15]) & 0x3fffffu);
-      continue;
-    }
-#endif
     const u32x4_t qs[4] = {q0, q1, q2, q3};
     const u32x4_t as[2][4] = {{a0, a1, a2, a3}, {b0, b1, b2, b3}};
     const floatx4_t zero4 = floatx4_t{0.f, 0.f, 0.f, 0.f};
@@ -1101,9 +1074,7 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
           }
         }
     }
-    TRACE(3);
   }
-  TRACE(4);
 
   // The cross-wavefront sum: in each pass every wavefront parks kPark of its tiles in
   // LDS and wavefront w (w < kPark) adds up one column block of one block of rows in
@@ -1181,7 +1152,6 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
     if (p.tickets != nullptr && pieces > 1) {
       const uint32_t flag_lds = (uint32_t)(uintptr_t)(lds_void_t*)smem;
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");   // this wavefront's partial tiles are in memory
-      TRACE(5);
       __builtin_amdgcn_s_barrier();                      // ... and every wavefront's; all LDS traffic is over
       // A ticket counts arrivals per XCD, four bits each (the host keeps a strip to at most
       // 15 contributors): their sum says who is last, and a single non-zero field that every
@@ -1195,7 +1165,6 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
         asm volatile("ds_write_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" ::"v"(flag_lds), "v"(now) : "memory");
       }
       __builtin_amdgcn_s_barrier();
-      TRACE(6);
       uint32_t now;
       asm volatile("ds_read_b32 %0, %1\n\ts_waitcnt lgkmcnt(0)" : "=&v"(now) : "v"(flag_lds) : "memory");
       now = __builtin_amdgcn_readfirstlane(now);
@@ -1211,10 +1180,6 @@ __global__ __launch_bounds__(kFastWaves * 64) void marlin_stream_fast_kernel(con
         }
         if (threadIdx.x == 0) __hip_atomic_store(ticket, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       }
-#ifdef SONAR_TRACE
-      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
-      TRACE(7);
     }
   }
 }
@@ -1711,9 +1676,6 @@ namespace {
 size_t stream_scratch_bytes() { return (size_t)2 * cu_count() * kSlotFloat4 * sizeof(float4); }
 }  // namespace
 
-#ifdef SONAR_TRACE
-extern "C" void sonar_debug_set_trace(void* ptr) { sonar::g_trace_host = (unsigned long long*)ptr; }
-#endif
 
 extern "C" size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k) {
   // partial tiles of the streaming kernels, then those of a split-K tile launch
@@ -1774,9 +1736,6 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                 "(the column-permuted copy of A)");
 
   StreamParams p = {};
-#ifdef SONAR_TRACE
-  p.trace = g_trace_host;
-#endif
   p.b = reinterpret_cast<const uint4*>(b_q_weight);
   p.bias = static_cast<const uint16_t*>(b_bias);
   p.scales = static_cast<const uint16_t*>(b_scales);

@@ -102,8 +102,14 @@ void refuse_during_capture(hipStream_t stream, const char* what) {
 }
 
 // A hit from another stream than the one that converted must not overtake the conversion.
+// While `stream` is being captured nothing is asked of the event (event queries and waits on
+// events from outside the capture invalidate it): a capture starts behind a device-wide
+// synchronisation, so the conversion has finished.
 void wait_for_conversion(NativeEntry& e, hipStream_t stream) {
   if (e.ready == nullptr) return;
+  hipStreamCaptureStatus status = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(stream, &status) != hipSuccess) (void)hipGetLastError();
+  if (status != hipStreamCaptureStatusNone) return;
   if (hipEventQuery(e.ready) == hipSuccess) {
     drop_event(e);
     return;

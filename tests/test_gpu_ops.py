@@ -191,6 +191,34 @@ def test_first_use_of_a_weight_inside_graph_capture_is_refused():
             assert torch.equal(got, want)
 
 
+def test_capture_on_the_stream_that_converted_the_weight():
+    """One warm-up call on a side stream, then a capture on that same stream: the hit
+    inside the capture must not touch the conversion's event (an event query there
+    invalidates the capture)."""
+    from sonar_amd import ops
+    k, n, m = 256, 128, 4
+    dl = gu.DeviceLayer(42, k, n, 128, "fp16")
+    a = gu.dev_bits16(mo.make_activations(2, m, k, "fp16"), "fp16")
+    ops.marlin_weight_cache_clear()
+    stream = torch.cuda.Stream()
+    torch.cuda.synchronize()
+    with torch.cuda.stream(stream):
+        want = _gemm_through_op(a, dl.marlin, dl.scales, dl.workspace, m, n, k)
+        stream.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            got = _gemm_through_op(a, dl.marlin, dl.scales, dl.workspace, m, n, k)
+        for _ in range(3):
+            got.zero_()
+            graph.replay()
+            stream.synchronize()
+            assert torch.equal(got, want)
+        again = _gemm_through_op(a, dl.marlin, dl.scales, dl.workspace, m, n, k)   # eager hit drops the event
+        stream.synchronize()
+        assert torch.equal(again, want)
+    ops.marlin_weight_cache_clear()
+
+
 def test_weight_converted_on_one_stream_is_safe_on_another():
     from sonar_amd import ops
     k, n, m = 4096, 4096, 4
