@@ -287,13 +287,16 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_kernel(const Tile
 //     step's group) into a private ring and dequantises them in registers.
 // The eight wavefronts form two groups (wm = 0: rows 0..127 of the tile, wm = 1:
 // rows 128..255); each SIMD holds one wavefront of either group.  A K step is
-// two half steps (k blocks 0 and 1), a half step is a "fetch" phase (LDS reads
-// of the 8 blocks of A and of one packed chunk, dequantisation: LDS and VALU
-// work) followed by a "multiply" phase (32 MFMAs).  Phases end with a
-// workgroup barrier and group 1 runs one phase behind group 0, so that on
-// every SIMD one wavefront multiplies while the other fetches: the matrix
-// cores see a steady stream although a single wavefront never overlaps its own
-// LDS waits, VALU work and MFMAs.
+// two half steps (k blocks 0 and 1), a half step is a "fetch" phase (the copies
+// of a later stage, the LDS read of one packed chunk, dequantisation: VALU
+// work) followed by a "multiply" phase (32 MFMAs and, behind the four of a row
+// block, the LDS read of that row block's operand of the next half step; a
+// group reads only rows of A that its own wavefronts copied).  Phases end with
+// a workgroup barrier and group 1 runs one phase behind group 0, so that on
+// every SIMD one wavefront multiplies while the other fetches.  The fetch phase
+// is the longer one: while its sibling issues MFMAs a wavefront gets a VALU
+// instruction through every eight cycles or so, and its copies and LDS
+// instructions take their issue time on top of that.
 // Copies of a wavefront complete in issue order, seven per stage, so "stage i
 // has landed" is s_waitcnt vmcnt(7) while the copies of stage i+1 are
 // outstanding.  With p = 4 kt + 2 b (+1 for group 1) the phase in which the
@@ -503,9 +506,9 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
       asm volatile("ds_read_b128 %0, %1" : "=&v"(qraw) : "v"(q_at) : "memory");
     }
   };
-  // Fetch phase of (stage in `slot`, k block b): picks up the packed chunk
-  // started by raw_start, starts the reads of the eight blocks of A and
-  // dequantises the chunk while they are in flight.
+  // Fetch phase of a half step: picks up the packed chunk started by raw_start
+  // and dequantises it, then waits for the operands of A the last multiply
+  // phase started to read.
   auto fetch = [&](int slot, int b, bool with_scales) {
     if constexpr (W8 != 0) {
       asm volatile("s_waitcnt lgkmcnt(0)"
@@ -518,17 +521,6 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
                    :
                    : "memory");
     }
-    // operand lane (kb, col16) of row block rb, k block b: piece 4 b + kb of row col16
-    const uint32_t a_at = a_lds + slot * kStageA + (8 * wm * 2 + (col16 >> 3)) * kBlockBytes + (col16 & 7) * 128 +
-                          (((4 * b + kb) ^ (col16 & 7)) * 16);
-    SONAR_TILE_READ(av[0], a_at, 0);
-    SONAR_TILE_READ(av[1], a_at, 2048);
-    SONAR_TILE_READ(av[2], a_at, 4096);
-    SONAR_TILE_READ(av[3], a_at, 6144);
-    SONAR_TILE_READ(av[4], a_at, 8192);
-    SONAR_TILE_READ(av[5], a_at, 10240);
-    SONAR_TILE_READ(av[6], a_at, 12288);
-    SONAR_TILE_READ(av[7], a_at, 14336);
     if (with_scales) {
       const uint32_t sbits[4] = {sb0, sb1, sb2, sb3};
 #pragma unroll
@@ -557,14 +549,31 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     }
     SONAR_TILE_LANDED();
   };
-  // Multiply phase: 32 MFMAs, ahead of the other wavefront's VALU work in the issue order.
-  auto multiply = [&]() {
+  // operand lane (kb, col16) of row block rb, k block b: piece 4 b + kb of row col16
+  auto a_address = [&](int slot, int b) {
+    return a_lds + slot * kStageA + (8 * wm * 2 + (col16 >> 3)) * kBlockBytes + (col16 & 7) * 128 +
+           (((4 * b + kb) ^ (col16 & 7)) * 16);
+  };
+  // Multiply phase: 32 MFMAs, ahead of the other wavefront's VALU work in the
+  // issue order; behind the four of a row block, the read of that row block's
+  // operand of half step (slot, b), which the next multiply phase uses: the
+  // reads of A cost the fetch phases nothing.
+  auto multiply_and_read = [&](int slot, int b) {
+    const uint32_t a_at = a_address(slot, b);
     __builtin_amdgcn_s_setprio(2);
-#pragma unroll
-    for (int i = 0; i < 8; ++i)
-#pragma unroll
-      for (int j = 0; j < 4; ++j)
-        acc[j][i] = Dq<T>::mfma(__builtin_bit_cast(vec8, wv[j]), __builtin_bit_cast(vec8, av[i]), acc[j][i]);
+#define SONAR_TILE_ROW(i, off)                                                                          \
+  _Pragma("unroll") for (int j = 0; j < 4; ++j) acc[j][i] =                                             \
+      Dq<T>::mfma(__builtin_bit_cast(vec8, wv[j]), __builtin_bit_cast(vec8, av[i]), acc[j][i]);         \
+  SONAR_TILE_READ(av[i], a_at, off)
+    SONAR_TILE_ROW(0, 0);
+    SONAR_TILE_ROW(1, 2048);
+    SONAR_TILE_ROW(2, 4096);
+    SONAR_TILE_ROW(3, 6144);
+    SONAR_TILE_ROW(4, 8192);
+    SONAR_TILE_ROW(5, 10240);
+    SONAR_TILE_ROW(6, 12288);
+    SONAR_TILE_ROW(7, 14336);
+#undef SONAR_TILE_ROW
     __builtin_amdgcn_s_setprio(0);
   };
   // end of a phase; nothing may be scheduled across it
@@ -581,6 +590,17 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");  // stage k_first has landed
   raw_start(0, 0, true);
   phase_end();
+  {
+    const uint32_t a_at = a_address(0, 0);
+    SONAR_TILE_READ(av[0], a_at, 0);
+    SONAR_TILE_READ(av[1], a_at, 2048);
+    SONAR_TILE_READ(av[2], a_at, 4096);
+    SONAR_TILE_READ(av[3], a_at, 6144);
+    SONAR_TILE_READ(av[4], a_at, 8192);
+    SONAR_TILE_READ(av[5], a_at, 10240);
+    SONAR_TILE_READ(av[6], a_at, 12288);
+    SONAR_TILE_READ(av[7], a_at, 14336);
+  }
   if (wm == 1) phase_end();  // group 1 runs one phase behind
 
   int slot = 0;        // stage of step kt
@@ -597,7 +617,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     fetch(slot, 0, true);
     raw_start(slot, 1, G32);
     phase_end();
-    multiply();
+    multiply_and_read(slot, 1);
     phase_end();
     // ---- half step (kt, 1)
 #pragma unroll
@@ -607,7 +627,9 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");
     raw_start(next_slot, 0, true);
     phase_end();
-    multiply();
+    // the rows of stage kt + 1 this group reads are the ones it copied, and its four
+    // wavefronts have waited for their copies before the barrier above
+    multiply_and_read(next_slot, 0);
     phase_end();
     slot = next_slot;
     fill = fill == kAsyncStages - 1 ? 0 : fill + 1;
@@ -620,6 +642,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   } else {
     asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)" : "+v"(qraw), "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw)::"memory");
   }
+  SONAR_TILE_LANDED();   // the operand reads started by the last multiply phase
 #undef SONAR_TILE_LANDED
 #undef SONAR_TILE_READ
 
