@@ -31,13 +31,14 @@ if ROOT not in sys.path:
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 # HBM bytes per GEMM launch of the default workload (M = 16, 6 weight copies), from one
-# `rocprofv3 --pmc FETCH_SIZE` and one `--pmc WRITE_SIZE` run of `bench.py --eager --calibrate`
-# (profiles/marlin_stream_fast_kernel_llama3-8b_m16_hbm-traffic.txt): FETCH_SIZE scaled by
-# 2.000 and WRITE_SIZE by 1.000, the factors that make the `--calibrate` pass (256 MiB read,
-# 256 MiB written) come out right.  Average over the four GEMMs of the layer.  Counters
-# cannot be read from inside a run, so the figure is tied to the launch shapes named in
-# TRAFFIC_LAUNCH_SHAPES: bench.py reports null as soon as the library launches differently.
-MEASURED_TRAFFIC_M16 = 30_100_000
+# `rocprofv3 --pmc FETCH_SIZE` and one `--pmc WRITE_SIZE` run of
+# `bench.py --no-prefill --eager --calibrate`
+# (profiles/marlin_stream_fast_kernel_llama3-8b-layer_m16_hbm-traffic.txt): FETCH_SIZE scaled
+# by 2.000 and WRITE_SIZE by 1.000, the factors that make the `--calibrate` pass (256 MiB
+# read, 256 MiB written) come out right.  Average over the four GEMMs of the layer.  Counters
+# cannot be read from inside a run: the figure belongs to the launch shapes of that profile
+# (192 / 256 / 448 / 256 workgroups) and is reported for M = 16 with six weight copies only.
+MEASURED_TRAFFIC_M16 = 32_400_000
 REPLAYS = 21                # graph replays per timing; the median is reported
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 GROUP = 128
@@ -414,7 +415,7 @@ def main() -> int:
         "per_gemm": per_gemm,
     }
 
-    if not args.no_prefill and not args.eager:
+    if not args.no_prefill:
         # the MFMA half of the metric: the same four GEMMs at M = 4096, fp16 activations ~ N(0, 0.5)
         pm = 4096
         fl_layers = [[Layer(torch, k, n, torch.float16, gen) for (_, k, n) in LAYER_SHAPES] for _ in range(2)]
@@ -424,13 +425,27 @@ def main() -> int:
             for layer in fl_layers[i % 2]:
                 layer.run(ops, pa[layer.k], wtype)
 
-        ps, plo, phi = time_graph(torch, prefill_step, 4, spread=True)
+        def timed(fn, reps):
+            """(median, p10, p90) seconds per call of fn: graph replays, or with --eager `reps` plain launches."""
+            if not args.eager:
+                return time_graph(torch, fn, reps, spread=True)
+            for i in range(2):
+                fn(i)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            for i in range(reps):
+                fn(i)
+            torch.cuda.synchronize()
+            dt = (time.perf_counter() - t0) / reps
+            return dt, dt, dt
+
+        ps, plo, phi = timed(prefill_step, 4)
         pflops = sum(2 * pm * k * n for (_, k, n) in LAYER_SHAPES)
         per_prefill = []
         for idx, (name, k, n) in enumerate(LAYER_SHAPES):
             def one(i=0, idx=idx, k=k):
                 fl_layers[i % 2][idx].run(ops, pa[k], wtype)
-            s, lo, hi = time_graph(torch, one, 4, spread=True)
+            s, lo, hi = timed(one, 4)
             fl = 2 * pm * k * n
             per_prefill.append({"gemm": name, "k": k, "n": n, "m": pm, "us": round(s * 1e6, 1),
                                 "us_p10": round(lo * 1e6, 1), "us_p90": round(hi * 1e6, 1),
@@ -440,7 +455,8 @@ def main() -> int:
                                 "unit": "TFLOP/s", "frac": round(pflops / ps / 1e12 / MFMA_PEAK_TFLOPS, 4),
                                 "kernel": "marlin_tile_async_kernel<f16> (+ tile_reduce_kernel where K is split)",
                                 "workload": "the four GEMMs of the layer at M=4096, fp16 activations ~ N(0,0.5), "
-                                            f"4 steps per graph, median of {REPLAYS} replays",
+                                            + ("4 plain launches of the step" if args.eager else
+                                               f"4 steps per graph, median of {REPLAYS} replays"),
                                 "flops_per_launch": pflops // launches,
                                 "us_per_launch": round(ps / launches * 1e6, 2),
                                 "ms_per_step": round(ps * 1e3, 4), "ms_per_step_p10": round(plo * 1e3, 4),
