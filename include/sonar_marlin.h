@@ -18,6 +18,8 @@
  *   sonar_marlin_gemm         -> _C::marlin_gemm
  *        csrc/libtorch_stable/torch_bindings.cpp:96-103,
  *        csrc/libtorch_stable/quantization/marlin/marlin.cu:546-897
+ *   sonar_marlin_gemm_nvfp4   -> the same op called with b_q_type = float4_e2m1f, float8_e4m3fn
+ *        block scales and a global_scale (marlin.cu:600-611,784-796)
  *   sonar_moe_wna16_marlin_gemm -> _moe_C::moe_wna16_marlin_gemm
  *        csrc/libtorch_stable/moe/torch_bindings.cpp:76-89,
  *        csrc/libtorch_stable/moe/marlin_moe_wna16/ops.cu:544-897
@@ -149,6 +151,31 @@ int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                       int64_t size_m, int64_t size_n, int64_t size_k,
                       int64_t num_groups, int is_k_full, int use_atomic_add,
                       int use_fp32_reduce, void* stream);
+
+/* NVFP4 (marlin.cu:600-611,784-796 of the reference; marlin_template.h:1661-1665;
+ * marlin_utils_fp4.py:59-151): float4_e2m1f codes (b_q_weight as for the other 4-bit types),
+ * one block scale per 16 rows and column, and one global scale.
+ *   C = round_to_dtype((A * W) * *global_scale (+ bias)),  W[k][n] = value(code) * b_scales[k / 16][n]
+ *   b_scales      dtype[size_k / 16][N] in marlin_permute_scales order: the block scales as
+ *                 numbers of the activation type.  value * scale must be exact in that type
+ *                 (it is for the reference's fp8 block scales: 1 + 3 mantissa bits).  The
+ *                 reference's callers hold the scales as bytes of a special 8-bit format
+ *                 (nvfp4_marlin_process_scales); a byte b stands for the half-precision
+ *                 number with the bits b << 7 times 2^-14 (half) or 2^-126 (bfloat16), which
+ *                 is what this argument takes; the torch op converts.
+ *   global_scale  one float in device memory (what nvfp4_marlin_process_global_scale
+ *                 returns, divided by the scale factor of the block scales)
+ * dtype is SONAR_DTYPE_F16 or SONAR_DTYPE_BF16; num_groups == size_k / 16; no zero points,
+ * no act-order.  The other arguments as for sonar_marlin_gemm.  sonar_marlin_dequant takes
+ * the same b_scales with num_groups == size_k / 16 and returns value(code) * scale. */
+int sonar_marlin_gemm_nvfp4(const void* a, int64_t a_row_stride, void* c,
+                            const uint32_t* b_q_weight, int b_layout,
+                            const void* b_bias, const void* b_scales,
+                            const float* global_scale, int32_t* workspace,
+                            int64_t workspace_len, void* scratch,
+                            size_t scratch_bytes, int dtype, int64_t size_m,
+                            int64_t size_n, int64_t size_k, int64_t num_groups,
+                            void* stream);
 
 /* sonar_marlin_gemm for callers that cannot allocate device memory (code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc).  No counterpart in the

@@ -53,6 +53,16 @@ reference checkout).  How each function is pinned (none is "parity unpinned"):
                            scales 2^(e - 127) against torch's float8_e8m0fnu
                            conversion; the (0, 2, 1, 3) reorder is its own
                            inverse
+* NVFP4 weights            the scale bytes (nvfp4_process_scales) decoded by both
+                           of the kernel's readings (dequant.h:520-549: b << 7
+                           as fp16, and sign / exponent / mantissa moved into a
+                           bf16) against scale * 2^7 for every non-negative
+                           float8_e4m3fn scale (torch's own conversion on the
+                           CPU), the >= 2 cut, the scale factor against its
+                           definition; global-scale processing against
+                           2^(bias - 7); the dequantised weight times the
+                           processed global scale against value * scale *
+                           global scale in exact arithmetic
 """
 
 from __future__ import annotations
@@ -496,6 +506,83 @@ def dequantize_mxfp4(codes: np.ndarray, exponent_bytes: np.ndarray, dtype: str =
     k, n = codes.shape
     rows = np.arange(k) // 32
     return round_to_dtype(fp4_e2m1_values()[codes] * mx_scale_values(exponent_bytes)[rows, :], dtype)
+
+
+# --------------------------------------------------------------------------
+# NVFP4 weights: float4_e2m1f codes, one float8_e4m3fn scale per column and 16
+# rows, one fp32 global scale, fp16 or bf16 activations
+# (marlin_utils_fp4.py:37-151, 640-697; dequant.h:397-470, 518-549;
+#  marlin_template.h:360-364, 1661-1665)
+# --------------------------------------------------------------------------
+
+NVFP4_EXPONENT_BIAS = {"fp16": 14, "bf16": 126}   # 2^(e-1) - 2^1 for e = 5 / 8 exponent bits (:143-149)
+
+
+def nvfp4_scale_factor(scales32: np.ndarray, dtype: str) -> float:
+    """marlin_utils_fp4.py:37-58: the power of two (>= 1) that lifts the largest
+    scale times 2^7 towards 448 * 2^7; 1 for fp16 activations."""
+    if dtype == "fp16":
+        return 1.0
+    ws = scales32.astype(np.float64) * 2.0 ** 7
+    pos = ws[ws > 0]
+    if pos.size and pos.max() < 448 * 2.0 ** 7:
+        return float(2.0 ** np.floor(np.log2(448 * 2.0 ** 7 / pos.max())))
+    return 1.0
+
+
+def nvfp4_process_scales(permuted32: np.ndarray, dtype: str, scale_factor: float | None = None):
+    """marlin_utils_fp4.py:61-120: (bytes, scale_factor).  The scales (values of
+    float8_e4m3fn, >= 0, already in marlin_permute_scales order) go to fp16, every
+    four neighbours into the order 0, 2, 1, 3, times the scale factor, times
+    2^7; what is below 2 becomes 0; the byte is bits 14..7 of the fp16 number."""
+    s = round_to_dtype(permuted32.astype(np.float32), "fp16")
+    s = s.reshape(-1, 4)[:, [0, 2, 1, 3]].reshape(s.shape)
+    if scale_factor is None:
+        scale_factor = nvfp4_scale_factor(s, dtype)
+    if scale_factor > 1.0:
+        s = round_to_dtype((s.astype(np.float32) * np.float32(scale_factor)), "fp16")
+    s = round_to_dtype(s * np.float32(2.0 ** 7), "fp16")
+    s = np.where(s < 2, np.float32(0), s)
+    bits = to_bits16(s, "fp16").astype(np.uint32)
+    return ((bits << 1) >> 8 & 0xFF).astype(np.uint8), scale_factor
+
+
+def nvfp4_scale_bytes_as_16bit_float(b: np.ndarray, dtype: str) -> np.ndarray:
+    """dequant.h:520-549: what the kernel reads a scale byte as.  fp16: the bits
+    b << 7.  bf16: bit 7 to bit 14, the other seven bits to bits 10..4.  Both are
+    the fp16 reading's value when bit 7 is set (or the byte is 0)."""
+    b = b.astype(np.uint32)
+    if dtype == "fp16":
+        return from_bits16((b << 7).astype(np.uint16), "fp16")
+    return from_bits16((((b & 0x80) << 7) | ((b & 0x7F) << 4)).astype(np.uint16), "bf16")
+
+
+def nvfp4_process_global_scale(global_scale: float, dtype: str, scale_factor: float = 1.0) -> np.float32:
+    """marlin_utils_fp4.py:138-151 and :289-291: times 2^(exponent bias - 7), over
+    the scale factor of the block scales; fp32."""
+    return np.float32(np.float32(global_scale) * np.float32(2.0 ** (NVFP4_EXPONENT_BIAS[dtype] - 7))
+                      / np.float32(scale_factor))
+
+
+def nvfp4_kernel_scales(scale_bytes: np.ndarray, dtype: str) -> np.ndarray:
+    """The block scales as this build's kernels take them: the kernel-side reading
+    of a byte times 2^-(exponent bias), the factor the reference's dequantised
+    code carries (dequant.h:397-470: a code read as fp16 / bf16 is value *
+    2^-bias).  Plain marlin_permute_scales order (the 0, 2, 1, 3 reorder undone).
+    Exact in `dtype` (held in fp32)."""
+    v = nvfp4_scale_bytes_as_16bit_float(scale_bytes, dtype).astype(np.float64)
+    v = v.reshape(-1, 4)[:, [0, 2, 1, 3]].reshape(v.shape)
+    return (v * 2.0 ** -NVFP4_EXPONENT_BIAS[dtype]).astype(np.float32)
+
+
+def dequantize_nvfp4(codes: np.ndarray, kernel_scales32: np.ndarray, dtype: str) -> np.ndarray:
+    """w[k][n] = value(code[k][n]) * scale[k // 16][n] with the scales of
+    nvfp4_kernel_scales in plain (K / 16, N) order: at most five significant
+    bits, exact in fp16 and bf16 (the reference's one 16-bit multiply,
+    marlin_template.h:1172-1299)."""
+    k, n = codes.shape
+    rows = np.arange(k) // 16
+    return round_to_dtype(fp4_e2m1_values()[codes] * kernel_scales32.astype(np.float32)[rows, :], dtype)
 
 
 # --------------------------------------------------------------------------

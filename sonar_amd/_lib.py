@@ -41,6 +41,9 @@ PROTOTYPES = {
                                   c_void_p, c_void_p, c_void_p, c_void_p, c_int64, c_void_p, c_size_t,
                                   c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int,
                                   c_int, c_void_p]),
+    "sonar_marlin_gemm_nvfp4": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                        c_void_p, c_void_p, c_int64, c_void_p, c_size_t,
+                                        c_int, c_int64, c_int64, c_int64, c_int64, c_void_p]),
     "sonar_marlin_gemm_noalloc": (c_int, [c_void_p, c_int64, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                           c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
                                           c_int, c_int64, c_int64, c_int64, c_int64, c_int64, c_int, c_int,

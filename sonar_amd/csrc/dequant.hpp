@@ -174,7 +174,7 @@ __device__ __forceinline__ void load_cols(typename D::Col (&cols)[4], const uint
 // as Dq: word() returns rows 0..7 of the column.  (This generic form is the
 // arithmetic the bf16 specialisation below must reproduce; only bf16 is launched.)
 template <typename T>
-struct DqF4 {
+struct DqF4Generic {
   typedef typename Dq<T>::vec8 vec8;
   struct Col {
     float s;   // scale * 2^14
@@ -192,6 +192,14 @@ struct DqF4 {
     return __builtin_bit_cast(vec8, u32x4_t{pair(q << 12, c.s), pair(q << 8, c.s), pair(q << 4, c.s), pair(q, c.s)});
   }
 };
+template <typename T>
+struct DqF4 : DqF4Generic<T> {};
+// NVFP4 (dequant.h:397-470,518-549 of the reference): the same codes with one scale per column
+// and 16 rows that is any number of the activation type with few significant bits (the
+// reference's fp8 block scales, decoded by the caller): value * scale has at most five, so the
+// generic form, which multiplies in fp32 and converts once, rounds nothing either.
+template <typename T>
+struct DqNvF4 : DqF4Generic<T> {};
 
 // bf16: the matrix-core generation this is written for converts two 4-bit
 // floats of a byte to bf16 and applies a power-of-two scale in one instruction
@@ -230,14 +238,18 @@ __device__ __forceinline__ uint16_t chunk_scale(const uint4& sv, int j, int col1
   return (uint16_t)(word >> (16 * (col16 >> 3)));
 }
 
-// The dequantiser of a 4-bit weight type.
-template <typename T, bool FP4>
+// The dequantiser of a 4-bit weight type (NV: float4 codes with arbitrary scales per 16 rows).
+template <typename T, bool FP4, bool NV = false>
 struct Dq4Of {
   typedef Dq<T> type;
 };
 template <typename T>
-struct Dq4Of<T, true> {
+struct Dq4Of<T, true, false> {
   typedef DqF4<T> type;
+};
+template <typename T>
+struct Dq4Of<T, true, true> {
+  typedef DqNvF4<T> type;
 };
 
 // 8-bit codes (uint8b128, symmetric): (v - 128) * s with one rounding.  A

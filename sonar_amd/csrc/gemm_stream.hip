@@ -27,7 +27,8 @@ namespace sonar {
 
 // gemm_tile.hip: the MFMA-bound kernel for more than 64 rows
 int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
-              const void* scales, const uint32_t* zeros, const int32_t* perm, int dtype, int64_t size_m,
+              const void* scales, const float* global_scale, const uint32_t* zeros, const int32_t* perm, int dtype,
+              int64_t size_m,
               int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
               size_t partial_bytes, bool fp4, int bits, bool fp8, hipStream_t st);
 bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size);
@@ -43,6 +44,7 @@ struct StreamParams {
   uint16_t* c;
   const uint4* b;
   const uint16_t* bias;
+  const float* global_scale;   // NVFP4: one number the output is multiplied by; else nullptr
   const uint16_t* scales;
   const uint32_t* zeros;
   const int32_t* perm;
@@ -149,6 +151,7 @@ __device__ __forceinline__ void write_tiles(const StreamParams& p, int strip, in
                                             const floatx4_t (&acc)[MB][4]) {
   const int m_in = lane & 15;
   const int n_in = 4 * (lane >> 4);
+  const float gs = p.global_scale ? *p.global_scale : 1.f;   // marlin_template.h:1661-1665
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int nl = 16 * j + n_in;
@@ -162,7 +165,7 @@ __device__ __forceinline__ void write_tiles(const StreamParams& p, int strip, in
     for (int mb = 0; mb < MB; ++mb) {
       const int m = 16 * mb + m_in;
       if (m < p.size_m) {
-        const floatx4_t v = acc[mb][j];
+        const floatx4_t v = acc[mb][j] * gs;
         uint2 o;
         o.x = (uint32_t)Dq<T>::from_float(v.x + b[0]) | ((uint32_t)Dq<T>::from_float(v.y + b[1]) << 16);
         o.y = (uint32_t)Dq<T>::from_float(v.z + b[2]) | ((uint32_t)Dq<T>::from_float(v.w + b[3]) << 16);
@@ -326,7 +329,9 @@ struct UnitBuf {
   uint4 sv[CHUNK_SCALES ? unit_buffer_chunks<MB>() : 1];
 };
 
-template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool CHUNK_SCALES = false>
+// NV (with CHUNK_SCALES): groups of 16 rows, two per chunk; a lane's eight rows, 8 kb .. 8 kb + 7,
+// lie in group kb / 2 of the chunk, and that is the row of scales it fetches.
+template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool CHUNK_SCALES = false, bool NV = false>
 __device__ __forceinline__ void load_unit(UnitBuf<T, MB, CHUNK_SCALES>& b, const StreamParams& p, int u, int lane,
                                           bool grouped) {
   const int col16 = lane & 15, kb = lane >> 4;
@@ -351,7 +356,8 @@ __device__ __forceinline__ void load_unit(UnitBuf<T, MB, CHUNK_SCALES>& b, const
 #pragma unroll
     for (int cc = 0; cc < unit_buffer_chunks<MB>(); ++cc)
       if (cc < p.unit_chunks)
-        b.sv[cc] = *reinterpret_cast<const uint4*>(srow + (long)cc * p.size_n + 8 * (col16 & 7));
+        b.sv[cc] = *reinterpret_cast<const uint4*>(srow + (long)(NV ? 2 * cc + (kb >> 1) : cc) * p.size_n +
+                                                   8 * (col16 & 7));
     return;
   }
 #pragma unroll
@@ -359,10 +365,10 @@ __device__ __forceinline__ void load_unit(UnitBuf<T, MB, CHUNK_SCALES>& b, const
   if (HAS_ZP) b.zword = p.zeros[(long)g * (p.size_n / 8) + strip * 8 + zero_point_word(col16)];
 }
 
-template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX, bool FP4 = false>
+template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX, bool FP4 = false, bool NV = false>
 __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const StreamParams params) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq4Of<T, FP4>::type D4;   // integer codes, or float4_e2m1f
+  typedef typename Dq4Of<T, FP4, NV>::type D4;   // integer codes, or float4_e2m1f (NV: scales per 16 rows)
   typedef typename D4::Col Col;
   __shared__ float4 red[4][MB * 4][64];
   // Several 64-row slabs can share a launch when no strip is shared between
@@ -387,7 +393,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
 
   UnitBuf<T, MB, FP4> cur, nxt;
   int mine = u_begin + wave;
-  if (mine < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM, FP4>(cur, p, mine, lane, grouped);
+  if (mine < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM, FP4, NV>(cur, p, mine, lane, grouped);
 
   int seg_begin = u_begin;
   while (seg_begin < u_end) {
@@ -404,7 +410,7 @@ __global__ __launch_bounds__(kWaves * 64) void marlin_stream_kernel(const Stream
 
     while (mine < seg_end) {
       const int next = mine + kWaves;
-      if (next < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM, FP4>(nxt, p, next, lane, grouped);
+      if (next < u_end) load_unit<T, MB, HAS_ZP, HAS_PERM, FP4, NV>(nxt, p, next, lane, grouped);
       Col cols[4];
       const bool chunk_scales = FP4 && grouped;   // the scales of every chunk came with the unit
       if (!chunk_scales) {
@@ -1214,6 +1220,7 @@ __global__ __launch_bounds__(64) void marlin_fixup_kernel(const StreamParams p) 
   const int m = 16 * mb + (lane & 15);
   if (m >= p.size_m) return;
   const int n_in = 4 * (lane >> 4);
+  const float gs = p.global_scale ? *p.global_scale : 1.f;
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
     const int nl = 16 * j + n_in;
@@ -1222,7 +1229,7 @@ __global__ __launch_bounds__(64) void marlin_fixup_kernel(const StreamParams p) 
 #pragma unroll
       for (int r = 0; r < 4; ++r) b[r] = Dq<T>::to_float(p.bias[strip * kStripN + scale_slot(nl + r, false)]);
     }
-    const floatx4_t v = acc[j];
+    const floatx4_t v = acc[j] * gs;
     uint2 o;
     o.x = (uint32_t)Dq<T>::from_float(v.x + b[0]) | ((uint32_t)Dq<T>::from_float(v.y + b[1]) << 16);
     o.y = (uint32_t)Dq<T>::from_float(v.z + b[2]) | ((uint32_t)Dq<T>::from_float(v.w + b[3]) << 16);
@@ -1232,7 +1239,7 @@ __global__ __launch_bounds__(64) void marlin_fixup_kernel(const StreamParams p) 
 
 // Writes W[K][N]: the values the GEMM kernels feed to the matrix cores.
 // With g_idx (symmetric weights only) the group of every row is looked up there.
-template <typename T, bool HAS_ZP, bool FP4 = false>
+template <typename T, bool HAS_ZP, bool FP4 = false, bool NV = false>
 __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __restrict__ b,
                                                             const uint16_t* __restrict__ scales,
                                                             const uint32_t* __restrict__ zeros,
@@ -1250,8 +1257,9 @@ __global__ __launch_bounds__(256) void marlin_dequant_kernel(const uint4* __rest
   for (long ch = (long)blockIdx.x * 4 + (threadIdx.x >> 6); ch < total_chunks; ch += (long)gridDim.x * 4) {
     const int strip = (int)(ch / chunks_per_strip);
     const int chunk = (int)(ch % chunks_per_strip);
-    const int g = grouped && !g_idx ? (chunk * kChunkK) / group_size : 0;
-    typedef typename Dq4Of<T, FP4>::type D4;
+    // NV: groups of 16 rows; a lane's eight rows lie in one of the chunk's two
+    const int g = NV ? 2 * chunk + (kb >> 1) : (grouped && !g_idx ? (chunk * kChunkK) / group_size : 0);
+    typedef typename Dq4Of<T, FP4, NV>::type D4;
     typename D4::Col cols[4];
     load_cols<T, HAS_ZP, D4>(cols, scales, zeros, size_n, strip, g, col16, grouped);
     int row_groups[8] = {0, 0, 0, 0, 0, 0, 0, 0};
@@ -1382,14 +1390,14 @@ void launch_stream_mb(const StreamParams& p, bool has_perm, hipStream_t st) {
   }
 }
 
-// float4_e2m1f codes: no zero points, no act-order
-template <typename T>
+// float4_e2m1f codes: no zero points, no act-order (NV: NVFP4, scales per 16 rows)
+template <typename T, bool NV = false>
 void launch_stream_fp4(const StreamParams& p, hipStream_t st) {
   switch ((p.size_m + 15) / 16) {
-    case 1: marlin_stream_kernel<T, 1, false, false, false, true><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    case 2: marlin_stream_kernel<T, 2, false, false, false, true><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    case 3: marlin_stream_kernel<T, 3, false, false, false, true><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
-    default: marlin_stream_kernel<T, 4, false, false, false, true><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 1: marlin_stream_kernel<T, 1, false, false, false, true, NV><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 2: marlin_stream_kernel<T, 2, false, false, false, true, NV><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    case 3: marlin_stream_kernel<T, 3, false, false, false, true, NV><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
+    default: marlin_stream_kernel<T, 4, false, false, false, true, NV><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p); break;
   }
 }
 
@@ -1492,12 +1500,13 @@ struct Checked {
   int group_size;
   int bits;         // 4 or 8
   bool fp8;         // 8-bit floating-point codes (float8_e4m3fn)
-  bool fp4;         // 4-bit floating-point codes (float4_e2m1f) with power-of-two scales per 32 rows
+  bool fp4;         // 4-bit floating-point codes (float4_e2m1f) with power-of-two scales per 32 rows (MXFP4) ...
+  bool nvfp4;       // ... or with scales of the activation type per 16 rows and a global scale (NVFP4)
 };
 
 int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_t* b_zeros,
                  const int32_t* g_idx, const int32_t* perm, int dtype, int64_t b_type_id,
-                 int64_t size_n, int64_t size_k, int64_t num_groups, int is_k_full) {
+                 int64_t size_n, int64_t size_k, int64_t num_groups, int is_k_full, bool nvfp4 = false) {
   SONAR_REQUIRE(b_layout == SONAR_LAYOUT_GFX950, "unknown b_layout = %d", b_layout);
   SONAR_REQUIRE(dtype == SONAR_DTYPE_F16 || dtype == SONAR_DTYPE_BF16, "unsupported `a` scalar_type");
   SONAR_REQUIRE(size_k > 0 && size_k % kChunkK == 0 && size_k < (1LL << 30),
@@ -1514,6 +1523,8 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
                 (long)b_type_id);
   out.fp8 = b_type_id == SONAR_TYPE_FLOAT8_E4M3FN;
   out.fp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F;
+  out.nvfp4 = nvfp4;
+  if (nvfp4) SONAR_REQUIRE(out.fp4, "a global scale goes with float4_e2m1f weights only (NVFP4)");
   out.bits = (b_type_id == SONAR_TYPE_UINT8B128 || out.fp8) ? 8 : 4;
   out.has_zp = b_zeros != nullptr;
   if (out.has_zp)
@@ -1523,6 +1534,17 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
                   "b_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   out.has_perm = perm != nullptr;
+  if (out.nvfp4) {
+    // generate_kernels.py:94-101: NVFP4, either activation type, one scale per 16 rows
+    SONAR_REQUIRE(!out.has_perm, "act-order is not supported with float4_e2m1f weights");
+    SONAR_REQUIRE(size_k == 16 * num_groups,
+                  "float4_e2m1f weights with a global scale (NVFP4) take one scale per group of 16 rows; got "
+                  "size_k = %ld, num_groups = %ld", (long)size_k, (long)num_groups);
+    SONAR_REQUIRE(((uintptr_t)b_scales) % 16 == 0, "b_scales must be 16-byte aligned");
+    out.row_groups = false;
+    out.group_size = 16;
+    return SONAR_OK;
+  }
   if (out.fp4) {
     // generate_kernels.py:102-110: MXFP4, bfloat16 activations, one power-of-two scale per 32 rows
     SONAR_REQUIRE(!out.has_perm, "act-order is not supported with float4_e2m1f weights");
@@ -1682,19 +1704,17 @@ extern "C" size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n
   return stream_scratch_bytes() + plan_partial_bytes(plan_gemm(size_m, size_n, size_k, true), size_m, size_n);
 }
 
-extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
-                                 const uint32_t* b_q_weight, int b_layout, const void* b_bias,
-                                 const void* b_scales, const uint32_t* b_zeros, const int32_t* g_idx,
-                                 const int32_t* perm, int32_t* workspace, int64_t workspace_len,
-                                 void* scratch, size_t scratch_bytes, int dtype, int64_t b_type_id,
-                                 int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
-                                 int is_k_full, int use_atomic_add, int use_fp32_reduce, void* stream) {
-  (void)use_atomic_add;
-  (void)use_fp32_reduce;
+namespace {
+// The dense GEMM behind sonar_marlin_gemm (global_scale == nullptr) and sonar_marlin_gemm_nvfp4.
+int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t* b_q_weight, int b_layout,
+                    const void* b_bias, const void* b_scales, const float* global_scale, const uint32_t* b_zeros,
+                    const int32_t* g_idx, const int32_t* perm, int32_t* workspace, int64_t workspace_len,
+                    void* scratch, size_t scratch_bytes, int dtype, int64_t b_type_id, int64_t size_m,
+                    int64_t size_n, int64_t size_k, int64_t num_groups, int is_k_full, void* stream) {
   SONAR_REQUIRE(size_m >= 0 && size_m < (1LL << 30), "size_m = %ld out of range", (long)size_m);
   Checked chk;
   if (int rc = check_common(chk, b_layout, b_scales, b_zeros, g_idx, perm, dtype, b_type_id, size_n,
-                            size_k, num_groups, is_k_full))
+                            size_k, num_groups, is_k_full, global_scale != nullptr))
     return rc;
   if (size_m == 0) return SONAR_OK;
   SONAR_REQUIRE(a && c && b_q_weight, "a, c and b_q_weight must not be NULL");
@@ -1738,6 +1758,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
   StreamParams p = {};
   p.b = reinterpret_cast<const uint4*>(b_q_weight);
   p.bias = static_cast<const uint16_t*>(b_bias);
+  p.global_scale = global_scale;
   p.scales = static_cast<const uint16_t*>(b_scales);
   p.zeros = b_zeros;
   p.perm = perm;
@@ -1792,7 +1813,7 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                 (long)size_n);
   p.total_units = (int)total_units;
   static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
-  const bool async_tile = tile_async_applies(chk.has_perm, num_groups, chk.group_size);
+  const bool async_tile = chk.nvfp4 || tile_async_applies(chk.has_perm, num_groups, chk.group_size);
   const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
   // the row -> group lookup and 8-bit codes exist in the streaming kernels only
   // (MXFP4 only through the asynchronous tile kernel: the older one has no float4 dequantiser)
@@ -1819,8 +1840,8 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
 
   if (use_tile) {
     const size_t used = stream_scratch_bytes();
-    return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, b_zeros, perm, dtype, size_m, size_n,
-                     size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used,
+    return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, perm, dtype, size_m,
+                     size_n, size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used,
                      scratch_bytes > used ? scratch_bytes - used : 0, chk.fp4, chk.bits, chk.fp8, st);
   }
 
@@ -1914,6 +1935,9 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
       if (chk.bits == 8) {
         if (dtype == SONAR_DTYPE_F16) launch_stream8_mb<_Float16>(p, chk.fp8, st);
         else launch_stream8_mb<__bf16>(p, chk.fp8, st);
+      } else if (chk.nvfp4) {
+        if (dtype == SONAR_DTYPE_F16) launch_stream_fp4<_Float16, true>(p, st);
+        else launch_stream_fp4<__bf16, true>(p, st);
       } else if (chk.fp4) {
         launch_stream_fp4<__bf16>(p, st);
       } else if (dtype == SONAR_DTYPE_F16) {
@@ -1932,6 +1956,34 @@ extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
     }
   }
   return SONAR_OK;
+}
+
+}  // namespace
+
+extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
+                                 const uint32_t* b_q_weight, int b_layout, const void* b_bias,
+                                 const void* b_scales, const uint32_t* b_zeros, const int32_t* g_idx,
+                                 const int32_t* perm, int32_t* workspace, int64_t workspace_len,
+                                 void* scratch, size_t scratch_bytes, int dtype, int64_t b_type_id,
+                                 int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
+                                 int is_k_full, int use_atomic_add, int use_fp32_reduce, void* stream) {
+  (void)use_atomic_add;
+  (void)use_fp32_reduce;
+  return marlin_gemm_any(a, a_row_stride, c, b_q_weight, b_layout, b_bias, b_scales, nullptr, b_zeros, g_idx, perm,
+                         workspace, workspace_len, scratch, scratch_bytes, dtype, b_type_id, size_m, size_n,
+                         size_k, num_groups, is_k_full, stream);
+}
+
+extern "C" int sonar_marlin_gemm_nvfp4(const void* a, int64_t a_row_stride, void* c,
+                                       const uint32_t* b_q_weight, int b_layout, const void* b_bias,
+                                       const void* b_scales, const float* global_scale, int32_t* workspace,
+                                       int64_t workspace_len, void* scratch, size_t scratch_bytes, int dtype,
+                                       int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
+                                       void* stream) {
+  SONAR_REQUIRE(global_scale != nullptr, "the global_scale parameter must be passed for nvfp4 format.");
+  return marlin_gemm_any(a, a_row_stride, c, b_q_weight, b_layout, b_bias, b_scales, global_scale, nullptr, nullptr,
+                         nullptr, workspace, workspace_len, scratch, scratch_bytes, dtype, SONAR_TYPE_FLOAT4_E2M1F,
+                         size_m, size_n, size_k, num_groups, 1, stream);
 }
 
 // ---------------------------------------------------------------------------
@@ -1983,8 +2035,10 @@ extern "C" int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout, co
                                     int dtype, int64_t b_type_id, int64_t size_n, int64_t size_k,
                                     int64_t num_groups, int is_k_full, void* stream) {
   Checked chk;
+  // float4 codes with one scale per 16 rows are NVFP4 (without its global scale: value x block scale)
+  const bool nvfp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F && size_k == 16 * num_groups;
   if (int rc = check_common(chk, b_layout, b_scales, b_zeros, g_idx, g_idx, dtype, b_type_id, size_n,
-                            size_k, num_groups, is_k_full))
+                            size_k, num_groups, is_k_full, nvfp4))
     return rc;
   SONAR_REQUIRE(b_q_weight && w_out, "b_q_weight and w_out must not be NULL");
   const long total_chunks = (size_n / kStripN) * (size_k / kChunkK);
@@ -2011,7 +2065,10 @@ extern "C" int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout, co
     return launch_status("marlin_dequant8_kernel");
   }
   const int32_t* gi = chk.row_groups ? g_idx : nullptr;
-  if (chk.fp4) {
+  if (chk.nvfp4) {
+    if (dtype == SONAR_DTYPE_F16) marlin_dequant_kernel<_Float16, false, true, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);
+    else marlin_dequant_kernel<__bf16, false, true, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);
+  } else if (chk.fp4) {
     marlin_dequant_kernel<__bf16, false, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);
   } else if (dtype == SONAR_DTYPE_F16) {
     if (chk.has_zp) marlin_dequant_kernel<_Float16, true><<<(int)blocks, 256, 0, st>>>(b, s, b_zeros, gi, w, n, k, ng, gs, total_chunks);

@@ -40,6 +40,7 @@ struct TileParams {
   uint16_t* c;
   const uint4* b;
   const uint16_t* bias;
+  const float* global_scale;   // NVFP4: one number the output is multiplied by; else nullptr
   const uint16_t* scales;
   const uint32_t* zeros;
   const int32_t* perm;
@@ -327,10 +328,14 @@ constexpr int async_copies(bool g32) { return g32 ? 8 : 7; }
 constexpr int strip_stage8(bool g32) { return 4 * kBlockBytes + (g32 ? 512 : 256); }
 constexpr int async_lds8(bool g32) { return kAsyncA + (kTileN / kStripN) * kAsyncStages * strip_stage8(g32); }
 
-template <typename T, bool HAS_ZP, bool GROUPED, bool G32 = false, bool FP4 = false, int W8 = 0>
+// NV (with G32 and FP4): NVFP4, groups of 16 rows.  The scale rows of a stage then hold four
+// groups of 128 bytes (a copy fetches two rows, one per half of the wavefront), and a lane,
+// whose eight rows of a k block lie in one group, reads the row of group 2 b + kb / 2.
+template <typename T, bool HAS_ZP, bool GROUPED, bool G32 = false, bool FP4 = false, int W8 = 0, bool NV = false>
 __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq4Of<T, FP4>::type D4;   // integer codes, or float4_e2m1f (MXFP4: with G32)
+  typedef typename Dq4Of<T, FP4, NV>::type D4;   // integer codes, or float4_e2m1f (MXFP4 / NVFP4: with G32)
+  static_assert(!NV || (G32 && FP4 && !HAS_ZP && W8 == 0), "NVFP4 is float4 codes with groups of 16 rows");
   typedef typename Dq8Of<T, W8 == 2>::type D8;   // 8-bit integer or floating-point codes (W8 != 0)
   typedef typename std::conditional<W8 != 0, typename D8::Col, typename D4::Col>::type Col;
   static_assert(W8 == 0 || (!HAS_ZP && !FP4), "8-bit codes are symmetric");
@@ -406,6 +411,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   } else {
     s_src = reinterpret_cast<const char*>(p.scales + expert * p.expert_s_stride + strip * kStripN) + 4 * (lane & 31);
     s_group_stride = (long)p.size_n * 2;
+    if (NV) s_src += (lane >> 5) * s_group_stride;   // the upper half of the wavefront fetches the next group's row
   }
   // the weight ring: private to the wavefront, or shared by the two wavefronts of a strip (8-bit codes)
   char* wring = smem + kAsyncA + (W8 ? wn : wave) * (kAsyncStages * kWaveStage);
@@ -434,7 +440,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     }
     // the scale rows (with a shared ring both wavefronts of the strip copy them: the same bytes twice)
     if (G32) {   // idx 6 / 7: the rows of groups 2 kt and 2 kt + 1
-      __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)(2 * kt + (idx - 6)) * s_group_stride),
+      __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)((NV ? 4 : 2) * kt + (NV ? 2 : 1) * (idx - 6)) *
+                                                                 s_group_stride),
                                        (lds_void_t*)(sw + kWeightBytes + 256 * (idx - 6)), 4, 0, 0);
       return;
     }
@@ -488,7 +495,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   auto raw_start = [&](int slot, int b, bool with_scales) {
     const uint32_t w_at = w_lds + slot * kWaveStage;
     const uint32_t q_at = w_at + (W8 ? 2 * b : b) * kBlockBytes + lane * 16;
-    const uint32_t r_at = w_at + (G32 ? 256 * b : 0);   // this k block's scale row
+    const uint32_t r_at = w_at + (NV ? 128 * (2 * b + (kb >> 1)) : (G32 ? 256 * b : 0));   // this k block's scale row
     if constexpr (W8 != 0) asm volatile("ds_read_b128 %0, %1 offset:1024" : "=&v"(qhigh) : "v"(q_at) : "memory");
     if (with_scales) {
       asm volatile(
@@ -500,7 +507,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
           "ds_read_b32 %5, %11"
           : "=&v"(qraw), "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
           : "v"(q_at), "v"(r_at + s_off[0]), "v"(r_at + s_off[1]), "v"(r_at + s_off[2]), "v"(r_at + s_off[3]),
-            "v"(r_at + z_off)
+            "v"(NV ? r_at + s_off[0] : r_at + z_off)
           : "memory");
     } else {
       asm volatile("ds_read_b128 %0, %1" : "=&v"(qraw) : "v"(q_at) : "memory");
@@ -682,6 +689,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
     }
   }
   const uint16_t* bias_src = p.bias ? p.bias + expert * p.expert_bias_stride + strip * kStripN : nullptr;
+  float gs = 1.f;   // NVFP4: the global scale multiplies the sum before anything else (marlin_template.h:1661-1665)
+  if (NV && p.global_scale) gs = p.global_scale[GROUPED ? expert : 0];
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb) {
     const int n = strip * kStripN + 16 * nb + 4 * kb;
@@ -693,7 +702,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 #pragma unroll
     for (int mb = 0; mb < 8; ++mb) {
       if (c_row[mb] < 0) continue;
-      const floatx4_t v = acc[nb][mb];
+      const floatx4_t v = NV ? acc[nb][mb] * gs : acc[nb][mb];
       uint16_t o[4] = {Dq<T>::from_float(v.x + bias[0]), Dq<T>::from_float(v.y + bias[1]),
                        Dq<T>::from_float(v.z + bias[2]), Dq<T>::from_float(v.w + bias[3])};
       if (GROUPED && p.mul_topk) {
@@ -732,6 +741,7 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const TileParams p) {
     acc += floatx4_t{v.x, v.y, v.z, v.w};
   }
   if (m >= p.size_m) return;
+  if (p.global_scale) acc = acc * p.global_scale[0];
   const int nl = 16 * nb + 4 * kb;
   float bias[4] = {0.f, 0.f, 0.f, 0.f};
   if (p.bias) {
@@ -796,6 +806,19 @@ int launch_tile_async_fp4(const TileParams& p, hipStream_t st) {
     attr_set = true;
   }
   marlin_tile_async_kernel<__bf16, false, false, true, true><<<tile_grid(p), kTileWaves * 64, async_lds(true), st>>>(p);
+  return SONAR_OK;
+}
+
+// NVFP4: either activation type, groups of 16 rows, a global scale
+template <typename T>
+int launch_tile_async_nvfp4(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, false, false, true, true, 0, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, async_lds(true)));
+    attr_set = true;
+  }
+  marlin_tile_async_kernel<T, false, false, true, true, 0, true><<<tile_grid(p), kTileWaves * 64, async_lds(true), st>>>(p);
   return SONAR_OK;
 }
 
@@ -879,10 +902,11 @@ bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size) {
 // Called by sonar_marlin_gemm for size_m > 64.  Shapes and pointers have been
 // validated by the caller; size_k % 64 == 0 is required here.
 int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
-              const void* scales, const uint32_t* zeros, const int32_t* perm, int dtype, int64_t size_m,
-              int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
+              const void* scales, const float* global_scale, const uint32_t* zeros, const int32_t* perm, int dtype,
+              int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
               size_t partial_bytes, bool fp4, int bits, bool fp8, hipStream_t st) {
   TileParams p;
+  p.global_scale = global_scale;
   p.a = static_cast<const uint16_t*>(a);
   p.lda = a_row_stride;
   p.c = static_cast<uint16_t*>(c);
@@ -912,7 +936,8 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   const bool zp = zeros != nullptr, pm = perm != nullptr;
   int rc;
   static const bool no_async = getenv("SONAR_MARLIN_NO_ASYNC_TILE") != nullptr;  // debugging aid
-  if (tile_async_applies(pm, num_groups, group_size) && (!no_async || fp4)) {   // float4 codes exist here only
+  const bool nvfp4 = fp4 && global_scale != nullptr;   // the caller has checked: groups of 16 rows
+  if ((nvfp4 || tile_async_applies(pm, num_groups, group_size)) && (!no_async || fp4)) {   // float4 codes exist here only
     const GemmPlan plan = plan_gemm(size_m, size_n, size_k, true);
     if (plan.k_splits > 1 && partial != nullptr && partial_bytes >= plan_partial_bytes(plan, size_m, size_n)) {
       p.k_splits = plan.k_splits;
@@ -928,7 +953,9 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
         if (p.k_splits == 1) p.partial = nullptr;
       }
     }
-    if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
+    if (nvfp4)
+      rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16>(p, st) : launch_tile_async_nvfp4<__bf16>(p, st);
+    else if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
       rc = launch_tile_async_fp4(p, st);
     else if (bits == 8)   // symmetric 8-bit codes: the caller has checked
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, false>(p, fp8, st)
@@ -984,6 +1011,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                                                                              (int)num_experts, table, max_tiles);
   if (int rc = launch_status("moe_tile_table_kernel")) return rc;
   TileParams p;
+  p.global_scale = nullptr;
   p.a = static_cast<const uint16_t*>(a);
   p.lda = size_k;
   p.c = static_cast<uint16_t*>(c);

@@ -231,6 +231,43 @@ Tensor mx_scales_as_bf16(const Tensor& b_scales, int64_t exponent_offset) {
   return out;
 }
 
+// NVFP4 block scales as the reference's callers pass them (bytes of the special 8-bit format
+// of nvfp4_marlin_process_scales, in marlin_permute_scales order with every four neighbours in
+// the order 0, 2, 1, 3; marlin_utils_fp4.py:61-120) -> numbers of the activation type in plain
+// marlin_permute_scales order, which the kernels read: a byte b stands for the half-precision
+// number with the bits b << 7 (dequant.h:520-549), and the dequantised code of the reference
+// carries 2^-14 (half) or 2^-126 (bfloat16), which is folded in here.  Cached like the weights.
+Tensor nvfp4_scales_as_16bit(const Tensor& b_scales, at::ScalarType a_type) {
+  const void* key = b_scales.const_data_ptr();
+  const int64_t tag = a_type == at::kHalf ? -16 : -17;   // stored in size_n: which conversion this entry holds
+  hipStream_t stream = (hipStream_t)current_stream(b_scales);
+  {
+    std::lock_guard<std::mutex> lock(g_cache_mutex);
+    auto it = g_cache.find(key);
+    if (it != g_cache.end() && !it->second.source.expired() &&
+        it->second.source._unsafe_get_target() == b_scales.unsafeGetTensorImpl() && it->second.size_k == -1 &&
+        it->second.size_n == tag && it->second.version == version_of(b_scales)) {
+      wait_for_conversion(it->second, stream);
+      return it->second.native;
+    }
+  }
+  refuse_during_capture(stream, "This tensor of float8_e4m3fn block scales");
+  TORCH_CHECK(b_scales.numel() % 4 == 0, "b_scales.numel() must be a multiple of 4");
+  const Tensor bytes = b_scales.view(at::kByte);
+  const Tensor order = at::tensor({0, 2, 1, 3}, at::TensorOptions().dtype(at::kLong).device(b_scales.device()));
+  const Tensor plain = bytes.reshape({-1, 4}).index_select(1, order).reshape(bytes.sizes());
+  const Tensor as_half = (plain.to(at::kShort) * 128).view(at::kHalf);   // the bits b << 7
+  Tensor out = (as_half.to(at::kFloat) * (a_type == at::kHalf ? 0x1p-14 : 0x1p-126)).to(a_type);
+  std::lock_guard<std::mutex> lock(g_cache_mutex);
+  evict_stale_locked(b_scales, key);
+  invalidate_range_locked(key, b_scales.nbytes());
+  NativeEntry entry{c10::weak_intrusive_ptr<c10::TensorImpl>(b_scales.getIntrusivePtr()), out, -1, tag,
+                    -1, version_of(b_scales), b_scales.nbytes(), stream, nullptr};
+  record_conversion(entry, stream);
+  g_cache.insert_or_assign(key, entry);
+  return out;
+}
+
 bool is_mx_scale_type(const Tensor& t) {
   return t.scalar_type() == at::kFloat8_e8m0fnu || t.scalar_type() == at::kByte;
 }
@@ -353,8 +390,16 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
   const int dtype = dtype_code(a);
   check_b_type(b_type_id);
   TORCH_CHECK_NOT_IMPLEMENTED(!a_scales.has_value(), "a_scales can only be used for 8bit activation.");
-  TORCH_CHECK_NOT_IMPLEMENTED(!global_scale.has_value(), "global_scale can only be used for nvfp4 format.");
   TORCH_CHECK_NOT_IMPLEMENTED(!is_zp_float, "is_zp_float = True is not built");
+  // marlin.cu:784-796
+  const bool nvfp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F && b_scales.scalar_type() == at::kFloat8_e4m3fn;
+  if (global_scale.has_value() && global_scale->numel() > 0) {
+    TORCH_CHECK(nvfp4, "global_scale can only be used for nvfp4 format.");
+    TORCH_CHECK(global_scale->is_cuda() && global_scale->scalar_type() == at::kFloat,
+                "scalar type of global_scale must be float");
+  } else {
+    TORCH_CHECK(!nvfp4, "the global_scale parameter must be passed for nvfp4 format.");
+  }
 
   TORCH_CHECK(a.dim() == 2, "a must be 2-D");
   TORCH_CHECK(a.size(0) == size_m, "Shape mismatch: a.size(0) = ", a.size(0), ", size_m = ", size_m);
@@ -384,9 +429,10 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
   if (mxfp8) {
     TORCH_CHECK(a.scalar_type() == at::kBFloat16, "float8_e4m3fn weights with float8_e8m0fnu scales (MXFP8) "
                 "need bfloat16 activations");
-  } else if (fp4) {   // marlin.cu:600-611; the fp8 block scales of NVFP4 are not built
-    TORCH_CHECK_NOT_IMPLEMENTED(b_scales.scalar_type() != at::kFloat8_e4m3fn,
-                                "float4_e2m1f weights with float8_e4m3fn scales (NVFP4) are not built");
+  } else if (nvfp4) {   // marlin.cu:600-611
+    TORCH_CHECK(g_idx_or_none.has_value() ? g_idx_or_none->numel() == 0 : true,
+                "act-order is not supported with float4_e2m1f weights");
+  } else if (fp4) {
     TORCH_CHECK(is_mx_scale_type(b_scales),
                 "When b_type = float4_e2m1f, b_scale scalar type must be",
                 "float8_e4m3fn (for NVFP4) or float8_e8m0fnu (for MXFP4).");
@@ -468,6 +514,18 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
   if (perm != nullptr) scratch_bytes += (size_t)size_m * size_k * 2;  // room for the column-permuted copy of A
   Tensor scratch = at::empty({(int64_t)scratch_bytes}, a.options().dtype(at::kByte));
 
+  if (nvfp4) {
+    TORCH_CHECK(size_k == 16 * num_groups, "float4_e2m1f weights with float8_e4m3fn scales (NVFP4) take one scale "
+                "per group of 16 rows; got size_k = ", size_k, ", b_scales.size(0) = ", num_groups);
+    raise_if_failed(sonar_marlin_gemm_nvfp4(
+        a.const_data_ptr(), a.stride(0), c.mutable_data_ptr(),
+        static_cast<const uint32_t*>(native.const_data_ptr()), SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none),
+        nvfp4_scales_as_16bit(b_scales, a.scalar_type()).const_data_ptr(),
+        static_cast<const float*>(global_scale->const_data_ptr()),
+        static_cast<int32_t*>(workspace.mutable_data_ptr()), workspace.numel(), scratch.mutable_data_ptr(),
+        scratch_bytes, dtype, size_m, size_n, size_k, num_groups, current_stream(a)));
+    return c;
+  }
   raise_if_failed(sonar_marlin_gemm(
       a.const_data_ptr(), a.stride(0), c.mutable_data_ptr(),
       static_cast<const uint32_t*>(native.const_data_ptr()), SONAR_LAYOUT_GFX950,

@@ -1,12 +1,16 @@
-"""MXFP4 weights (float4_e2m1f codes, one power-of-two scale per 32 rows, bf16
-activations) through the Marlin ops.  Mirrors the MXFP4 half of
-aphrodite/model_executor/layers/quantization/utils/marlin_utils_fp4.py:34-36,
-123-135, 153-290, 293-322, 556-649, 701-753 of the reference: the checkpoint
-bytes (two codes each, low nibble first along K) are GPTQ words as they stand
-and go through gptq_marlin_repack with num_bits = 4; the scales (exponent bytes
-e, value 2^(e - 127)) are permuted as for any Marlin layer, every four
-neighbours are put in the order 0, 2, 1, 3, and they travel as float8_e8m0fnu.
-NVFP4 (float8_e4m3fn scales per 16 rows and a global scale) is not built.
+"""4-bit floating-point weights (float4_e2m1f codes) through the Marlin ops.
+Mirrors aphrodite/model_executor/layers/quantization/utils/marlin_utils_fp4.py
+of the reference for dense layers of both formats and MXFP4 experts: :34-151,
+153-290, 556-649, 652-753.  The checkpoint bytes (two codes each, low nibble
+first along K) are GPTQ words as they stand and go through gptq_marlin_repack
+with num_bits = 4.  MXFP4: one power-of-two scale per 32 rows (exponent bytes e,
+value 2^(e - 127)), bf16 activations; the scales are permuted as for any Marlin
+layer, every four neighbours are put in the order 0, 2, 1, 3, and they travel
+as float8_e8m0fnu.  NVFP4: one float8_e4m3fn scale per 16 rows and an fp32
+global scale, fp16 or bf16 activations; the scales travel as bytes of the
+reference's special 8-bit format (nvfp4_marlin_process_scales) and the global
+scale carries the exponent bias of the kernel-side reading.  NVFP4 experts
+(prepare_nvfp4_moe_layer_for_marlin) are not built.
 """
 from __future__ import annotations
 
@@ -19,6 +23,7 @@ from .marlin_utils import (USE_FP32_REDUCE_DEFAULT, marlin_make_workspace_new, m
 from .scalar_type import scalar_types
 
 MXFP4_GROUP_SIZE = 32
+FP4_MARLIN_SUPPORTED_GROUP_SIZES = [16]   # marlin_utils_fp4.py:29 (NVFP4)
 
 
 def is_fp4_marlin_supported() -> bool:
@@ -35,14 +40,59 @@ def mxfp4_marlin_process_scales(marlin_scales: torch.Tensor, input_dtype: torch.
     return reordered.to(torch.float8_e8m0fnu)
 
 
+def _nvfp4_compute_scale_factor(marlin_scales: torch.Tensor, a_dtype: torch.dtype | None = None) -> float:
+    """marlin_utils_fp4.py:37-58: the power of two (>= 1) after which the largest
+    scale times 2^7 is just below 448 * 2^7; 1 for half activations."""
+    if a_dtype is not None and a_dtype == torch.half:
+        return 1.0
+    ws_float = marlin_scales.float() * (2 ** 7)
+    nonzero = ws_float > 0
+    if nonzero.any():
+        max_val = ws_float[nonzero].max()
+        if max_val < 448 * (2 ** 7):
+            return (448 * (2 ** 7) / max_val).log2().floor().exp2().item()
+    return 1.0
+
+
+def nvfp4_marlin_process_scales(marlin_scales: torch.Tensor, scale_factor: float | None = None,
+                                a_dtype: torch.dtype | None = None) -> tuple[torch.Tensor, float]:
+    """marlin_utils_fp4.py:61-120: the (non-negative) block scales, already in
+    marlin_permute_scales order, as bytes of the special format the kernel
+    reads: (0, 2, 1, 3) inside every four, times the scale factor, times 2^7,
+    what is below 2 to zero, then bits 14..7 of the half-precision number.
+    Returns (bytes as float8_e4m3fn, scale_factor)."""
+    marlin_scales = marlin_scales.to(torch.half)
+    marlin_scales = marlin_scales.view(-1, 4)[:, [0, 2, 1, 3]].view(marlin_scales.size(0), -1)
+    if scale_factor is None:
+        scale_factor = _nvfp4_compute_scale_factor(marlin_scales, a_dtype)
+    if scale_factor > 1.0:
+        marlin_scales = (marlin_scales.float() * scale_factor).to(torch.half)
+    marlin_scales = marlin_scales * (2 ** 7)
+    marlin_scales[marlin_scales < 2] = 0
+    marlin_scales = marlin_scales.view(torch.int16) << 1
+    marlin_scales = marlin_scales.view(torch.float8_e4m3fn)
+    return marlin_scales[:, 1::2].contiguous(), scale_factor
+
+
+def nvfp4_marlin_process_global_scale(global_scale: torch.Tensor, a_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """marlin_utils_fp4.py:138-151: times 2^(exponent bias of the code read as a
+    16-bit float, minus the 7 the block scales carry)."""
+    if a_dtype is None:
+        a_dtype = global_scale.dtype
+    assert a_dtype in [torch.half, torch.bfloat16]
+    target_exponent = 5 if a_dtype == torch.half else 8
+    exponent_bias = 2 ** (target_exponent - 1) - 2 ** (2 - 1)
+    return global_scale * (2.0 ** (exponent_bias - 7))
+
+
 def apply_fp4_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
                             weight_global_scale: torch.Tensor | None, workspace: torch.Tensor, size_n: int,
                             size_k: int, bias: torch.Tensor | None = None, input_dtype: torch.dtype | None = None,
                             use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
-    """marlin_utils_fp4.py:153-214."""
-    if weight_global_scale is not None:
-        raise NotImplementedError("NVFP4 (a global scale) is not built; MXFP4 only")
+    """marlin_utils_fp4.py:153-214; with a global scale the weights are NVFP4."""
     if input_dtype is not None and input_dtype.itemsize == 1:
+        if weight_global_scale is not None:
+            raise RuntimeError("NVFP4 weight + INT8/FP8 activation is not supported.")
         raise NotImplementedError("8-bit activations are not built")
     x = input.reshape(-1, input.shape[-1])
     out_shape = input.shape[:-1] + (size_n,)
@@ -51,7 +101,8 @@ def apply_fp4_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_sc
     use_atomic_add = should_use_atomic_add_reduce(m=x.size(0), n=padded_n, k=padded_k, device=input.device,
                                                   dtype=input.dtype)
     out = ops.marlin_gemm(a=x, c=None, b_q_weight=weight, b_bias=bias, b_scales=weight_scale, a_scales=None,
-                          global_scale=None, b_zeros=None, g_idx=None, perm=None, workspace=workspace,
+                          global_scale=weight_global_scale, b_zeros=None, g_idx=None, perm=None,
+                          workspace=workspace,
                           b_q_type=scalar_types.float4_e2m1f, size_m=x.size(0), size_n=padded_n, size_k=padded_k,
                           use_atomic_add=use_atomic_add, use_fp32_reduce=use_fp32_reduce)
     return marlin_unpad_output(out, size_n, padded_n).reshape(out_shape)
@@ -63,15 +114,20 @@ def _set(layer, name: str, value: torch.Tensor) -> None:
 
 
 def prepare_fp4_layer_for_marlin(layer, input_dtype: torch.dtype | None = None) -> None:
-    """marlin_utils_fp4.py:217-290 for MXFP4.  The layer holds `weight` (N, K/2)
-    uint8, `weight_scale` (N, K/32) exponent bytes, `params_dtype` (bfloat16),
-    `output_size_per_partition`, `input_size_per_partition`, optionally `bias`."""
-    if hasattr(layer, "weight_global_scale"):
-        raise NotImplementedError("NVFP4 (a global scale) is not built; MXFP4 only")
+    """marlin_utils_fp4.py:217-290.  The layer holds `weight` (N, K/2) uint8,
+    `params_dtype`, `output_size_per_partition`, `input_size_per_partition`,
+    optionally `bias`, and either `weight_scale` (N, K/32) exponent bytes
+    (MXFP4, bfloat16) or `weight_scale` (N, K/16) float8_e4m3fn with
+    `weight_global_scale` (NVFP4)."""
+    is_nvfp4 = hasattr(layer, "weight_global_scale")
     if input_dtype is not None and input_dtype.itemsize == 1:
+        if is_nvfp4:
+            raise RuntimeError("NVFP4 weight + INT8/FP8 activation is not supported.")
         raise NotImplementedError("8-bit activations are not built")
+    group_size = 16 if is_nvfp4 else MXFP4_GROUP_SIZE
     part_n, part_k = layer.output_size_per_partition, layer.input_size_per_partition
-    padded_n, padded_k = marlin_padded_nk(part_n, part_k, MXFP4_GROUP_SIZE)
+    padded_n, padded_k = marlin_padded_nk(part_n, part_k, group_size)
+    param_dtype = layer.params_dtype
     assert layer.weight.shape == (part_n, part_k // 2)
     device = layer.weight.device
     layer.workspace = marlin_make_workspace_new(device)
@@ -79,10 +135,19 @@ def prepare_fp4_layer_for_marlin(layer, input_dtype: torch.dtype | None = None) 
     qweight = marlin_pad_qweight(layer.weight.view(torch.int32).T.contiguous(), part_n, part_k, padded_n, padded_k)
     _set(layer, "weight", ops.gptq_marlin_repack(qweight, perm, padded_k, padded_n, 4))
 
-    scales = layer.weight_scale.T.contiguous().view(torch.float8_e8m0fnu).to(layer.params_dtype)
-    scales = marlin_pad_scales(scales, part_n, part_k, padded_n, padded_k, MXFP4_GROUP_SIZE)
-    scales = marlin_permute_scales(scales, padded_k, padded_n, MXFP4_GROUP_SIZE)
-    _set(layer, "weight_scale", mxfp4_marlin_process_scales(scales))
+    scales = layer.weight_scale.T.contiguous()
+    if not is_nvfp4:
+        scales = scales.view(torch.float8_e8m0fnu)
+    scales = scales.to(param_dtype)
+    scales = marlin_pad_scales(scales, part_n, part_k, padded_n, padded_k, group_size)
+    scales = marlin_permute_scales(scales, padded_k, padded_n, group_size)
+    if is_nvfp4:
+        scales, scale_factor = nvfp4_marlin_process_scales(scales, a_dtype=param_dtype)
+        _set(layer, "weight_scale", scales)
+        global_scale = nvfp4_marlin_process_global_scale(layer.weight_global_scale.to(torch.float32), param_dtype)
+        _set(layer, "weight_global_scale", global_scale / scale_factor)
+    else:
+        _set(layer, "weight_scale", mxfp4_marlin_process_scales(scales))
 
     if getattr(layer, "bias", None) is not None:
         assert layer.bias.shape == (part_n,)
@@ -143,3 +208,33 @@ def rand_marlin_weight_mxfp4_like(weight: torch.Tensor, group_size: int, input_d
     marlin_qweight = ops.gptq_marlin_repack(codes.view(torch.int32).T.contiguous(), perm, size_k, size_n, 4)
     marlin_scales = marlin_permute_scales(scales.T.to(weight.dtype), size_k, size_n, group_size)
     return weight_ref.T, marlin_qweight, mxfp4_marlin_process_scales(marlin_scales)
+
+
+def rand_marlin_weight_nvfp4_like(weight: torch.Tensor, group_size: int, input_dtype: torch.dtype | None = None):
+    """The reference's test helper (marlin_utils_fp4.py:652-698): block scales
+    from the magnitudes of `weight` (N, K), global scale max / 448, random codes;
+    returns (dequantised reference (K, N), Marlin weight, Marlin scale bytes,
+    processed global scale)."""
+    assert input_dtype is None or input_dtype.itemsize != 1, "NVFP4 weight + INT8/FP8 activation is not supported."
+    assert group_size > 0
+    size_n, size_k = weight.shape
+    device = weight.device
+    scales = weight.view(size_n, -1, group_size).abs().max(-1)[0] / 6
+    global_scale = scales.max() / 448
+    scales = (scales / global_scale).to(torch.float8_e4m3fn)
+    codes = torch.randint(0, 256, (size_n, size_k // 2), dtype=torch.uint8, device=device)
+
+    def values(nibble_high: torch.Tensor) -> torch.Tensor:
+        # sign and the three other bits at the top of a byte: as float8_e4m3fn that is value * 2^-6
+        as_fp8 = (nibble_high & 0b10000000) | ((nibble_high & 0b01110000) >> 2)
+        return as_fp8.view(torch.float8_e4m3fn).to(weight.dtype) * (2 ** 6)
+
+    odd, even = values(codes), values(codes << 4)   # k odd: high nibble; k even: low nibble
+    weight_ref = torch.cat([even.unsqueeze(2), odd.unsqueeze(2)], 2).view(size_n, size_k)
+    weight_ref = weight_ref * global_scale.to(weight.dtype) * scales.repeat_interleave(group_size, 1).to(weight.dtype)
+    perm = torch.empty(0, dtype=torch.int, device=device)
+    marlin_qweight = ops.gptq_marlin_repack(codes.view(torch.int32).T.contiguous(), perm, size_k, size_n, 4)
+    marlin_scales = marlin_permute_scales(scales.T.to(weight.dtype), size_k, size_n, group_size)
+    marlin_scales, scale_factor = nvfp4_marlin_process_scales(marlin_scales)
+    global_scale = nvfp4_marlin_process_global_scale(global_scale).to(torch.float32)
+    return weight_ref.T, marlin_qweight, marlin_scales, global_scale / scale_factor

@@ -779,7 +779,7 @@ def test_mxfp4_random_weight_helper_and_marlin_gemm(m, k, n):
     with pytest.raises(RuntimeError, match="bfloat16"):
         ops.marlin_gemm(a.half(), None, qweight, None, scales, None, None, None, None, None, workspace,
                         scalar_types.float4_e2m1f, m, n, k)
-    with pytest.raises(NotImplementedError, match="NVFP4"):
+    with pytest.raises(RuntimeError, match="global_scale parameter must be passed for nvfp4"):
         ops.marlin_gemm(a, None, qweight, None, scales.view(torch.float8_e4m3fn), None, None, None, None, None,
                         workspace, scalar_types.float4_e2m1f, m, n, k)
 
@@ -807,6 +807,72 @@ def test_prepare_mxfp4_layer_and_apply(k, n):
     x32 = mo.make_activations(4, 6, k, "bf16", std=0.5)
     y = f4.apply_fp4_marlin_linear(gu.dev_bits16(x32, "bf16").view(2, 3, k), layer.weight, layer.weight_scale, None,
                                    layer.workspace, n, k, layer.bias)
+    torch.cuda.synchronize()
+    assert y.shape == (2, 3, n)
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y.view(6, n)), mo.gemm_reference(x32, w_ref, bias32))
+    assert ok, worst
+
+
+# ---------------------------------------------------------------- NVFP4 weights (float4_e2m1f, e4m3 block scales, global scale)
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
+@pytest.mark.parametrize("m,k,n", [(1, 512, 256), (33, 1024, 320), (16, 2880, 5760), (200, 256, 512), (700, 1024, 768)])
+def test_nvfp4_random_weight_helper_and_marlin_gemm(m, k, n, dtype):
+    """The reference's NVFP4 case of its Marlin GEMM test (test_marlin_gemm.py with
+    rand_marlin_weight_nvfp4_like): the op takes the scale bytes and the processed
+    global scale as the reference's callers hold them; compared with the matmul on
+    the dequantised weight."""
+    from sonar_amd import marlin_utils_fp4 as f4
+    from sonar_amd import ops
+    from sonar_amd.marlin_utils import marlin_make_workspace_new
+    from sonar_amd.scalar_type import scalar_types
+    torch.manual_seed(m + k)
+    weight = torch.randn((n, k), dtype=dtype, device=gu.DEV)
+    a = (0.5 * torch.randn((m, k), device=gu.DEV)).to(dtype)
+    w_ref, qweight, scales, global_scale = f4.rand_marlin_weight_nvfp4_like(weight, 16)
+    assert qweight.shape == (k // 16, 2 * n) and scales.shape == (k // 16, n)
+    assert scales.dtype == torch.float8_e4m3fn and global_scale.dtype == torch.float32
+    workspace = marlin_make_workspace_new(a.device)
+    out = ops.marlin_gemm(a, None, qweight, None, scales, None, global_scale.reshape(1), None, None, None, workspace,
+                          scalar_types.float4_e2m1f, m, n, k)
+    again = ops.marlin_gemm(a, None, qweight, None, scales, None, global_scale.reshape(1), None, None, None,
+                            workspace, scalar_types.float4_e2m1f, m, n, k)     # converted scales come from the cache
+    torch.cuda.synchronize()
+    assert torch.equal(out, again)
+    want = (a.float() @ w_ref.float()).cpu().numpy()
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(out), want)
+    assert ok, worst
+    with pytest.raises(RuntimeError, match="global_scale can only be used for nvfp4"):
+        ops.marlin_gemm(a, None, qweight, None, scales.view(torch.float8_e8m0fnu), None, global_scale.reshape(1),
+                        None, None, None, workspace, scalar_types.float4_e2m1f, m, n, k)
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("k,n", [(512, 384), (384, 320)])   # 320 columns: padded to 384 inside
+def test_prepare_nvfp4_layer_and_apply(k, n, dtype):
+    """An NVFP4 checkpoint layer (weight (N, K/2) bytes, low nibble first; scales
+    (N, K/16) float8_e4m3fn; a global scale) -> prepare_fp4_layer_for_marlin ->
+    apply_fp4_marlin_linear, against value * scale * global scale on the same bytes."""
+    from sonar_amd import marlin_utils_fp4 as f4
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    rng = np.random.default_rng(k + n)
+    codes = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    sbytes = torch.from_numpy(rng.integers(0x28, 0x70, size=(k // 16, n)).astype(np.uint8))
+    scales = sbytes.view(torch.float8_e4m3fn).float().numpy()
+    g = 0.0021
+    w_ref = mo.fp4_e2m1_values()[codes] * np.repeat(scales, 16, axis=0) * np.float32(g)
+    by_n = codes.T                                            # (N, K)
+    packed = np.ascontiguousarray((by_n[:, 0::2] | (by_n[:, 1::2] << 4)).astype(np.uint8))
+    layer = types.SimpleNamespace(output_size_per_partition=n, input_size_per_partition=k, params_dtype=tdt)
+    layer.weight = torch.from_numpy(packed).to(gu.DEV)
+    layer.weight_scale = sbytes.T.contiguous().view(torch.float8_e4m3fn).to(gu.DEV)
+    layer.weight_global_scale = torch.tensor(g, dtype=torch.float32, device=gu.DEV)
+    bias32 = mo.round_to_dtype(1e-2 * rng.standard_normal(n).astype(np.float32), dtype)
+    layer.bias = gu.dev_bits16(bias32, dtype)
+    f4.prepare_fp4_layer_for_marlin(layer)
+    assert layer.weight_scale.dtype == torch.float8_e4m3fn and layer.weight_global_scale.dtype == torch.float32
+    x32 = mo.make_activations(4, 6, k, dtype, std=0.5)
+    y = f4.apply_fp4_marlin_linear(gu.dev_bits16(x32, dtype).view(2, 3, k), layer.weight, layer.weight_scale,
+                                   layer.weight_global_scale.reshape(1), layer.workspace, n, k, layer.bias)
     torch.cuda.synchronize()
     assert y.shape == (2, 3, n)
     ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y.view(6, n)), mo.gemm_reference(x32, w_ref, bias32))

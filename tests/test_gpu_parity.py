@@ -556,6 +556,110 @@ def test_mxfp4_weights_dequant_bit_exact_and_gemm_within_tolerance(gu, m, k, n, 
     assert ok, f"max_err={max_err} max_ref={max_ref}"
 
 
+def _layer_nvfp4(gu, seed, k, n, dtype):
+    """An NVFP4 layer on the device: float4_e2m1f codes in GPTQ words -> repack op ->
+    streaming order; float8_e4m3fn block scales per 16 rows through the reference's
+    chain (marlin_permute_scales, nvfp4_marlin_process_scales) and back to the
+    numbers of the activation type the C entry points take; a processed global
+    scale; plus the oracle's dequantised matrix (without the global scale)."""
+    import torch
+    rng = np.random.default_rng(seed)
+    codes = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    codes[:16, 0] = np.arange(16)                      # every code in one column
+    e4m3 = torch.from_numpy(rng.integers(0x20, 0x7F, size=(k // 16, n)).astype(np.uint8))   # 2^-3 .. 448
+    scales = e4m3.view(torch.float8_e4m3fn).float().numpy()
+    scales[0, :4] = [0.0, 2.0 ** -9, 448.0, 1.0]       # zero, the smallest number (cut to zero for fp16), the largest
+    permuted = mo.marlin_permute_scales(scales, k, n, 16)
+    scale_bytes, sf = mo.nvfp4_process_scales(permuted, dtype)
+    kernel_scales = mo.nvfp4_kernel_scales(scale_bytes, dtype)
+    w_ref = mo.dequantize_nvfp4(codes, mo.marlin_unpermute_scales(kernel_scales, k, n, 16), dtype)
+    global_scale = mo.nvfp4_process_global_scale(0.0123, dtype, sf)
+    marlin = gu.gptq_repack(gu.dev_i32(mo.gptq_pack(codes)), None, k, n)
+    return dict(native=gu.to_gfx950(marlin, k, n), marlin=marlin, scales=gu.dev_bits16(kernel_scales, dtype),
+                scale_bytes=scale_bytes, groups=k // 16, w_ref=w_ref, global_scale=float(global_scale),
+                gs_dev=torch.tensor([float(global_scale)], dtype=torch.float32, device=gu.DEV))
+
+
+NVFP4_CASES = [
+    # m, k, n, bias
+    (1, 128, 64, False),
+    (7, 512, 256, True),
+    (16, 4096, 1024, False),
+    (33, 1024, 320, True),
+    (64, 256, 4096, False),
+    (100, 1024, 512, False),      # 64-row slabs of the streaming kernel (few tiles)
+    (300, 512, 192, True),
+    (600, 2048, 1536, True),      # tile kernel, K split, partial tiles summed by the second kernel
+    (4096, 4096, 1024, False),    # tile kernel, whole tiles
+]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("m,k,n,bias", NVFP4_CASES)
+def test_nvfp4_weights_dequant_bit_exact_and_gemm_within_tolerance(gu, m, k, n, bias, dtype):
+    """float4_e2m1f weights with float8_e4m3fn scales per 16 rows and a global scale,
+    either activation type (generate_kernels.py:94-100; dequant.h:397-470, 518-549;
+    marlin_template.h:1661-1665)."""
+    from sonar_amd import _lib
+    lib = _lib.load()
+    L = _layer_nvfp4(gu, 11 * m + k, k, n, dtype)
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    w = torch.empty((k, n), dtype=tdt, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_dequant(gu.ptr(L["native"]), _lib.LAYOUT_GFX950, gu.ptr(L["scales"]), None,
+                                        None, gu.ptr(w), gu.dtype_code(dtype), _lib.TYPE_FLOAT4_E2M1F,
+                                        n, k, L["groups"], 1, gu.stream()))
+    torch.cuda.synchronize()
+    got = w.view(torch.int16).cpu().numpy().view(np.uint16)
+    want = mo.to_bits16(L["w_ref"], dtype)
+    # every bit but the sign of a zero (a negative code times a zero scale is +0 here, -0 in the oracle)
+    assert np.array_equal(np.where((got & 0x7FFF) == 0, 0, got), np.where((want & 0x7FFF) == 0, 0, want))
+
+    bias32 = bias_dev = None
+    if bias:
+        bias32 = mo.round_to_dtype(1e-2 * np.random.default_rng(m).standard_normal(n).astype(np.float32), dtype)
+        bias_dev = gu.dev_bits16(mo.marlin_permute_bias(bias32), dtype)
+    a32 = mo.make_activations(m + 1, m, k, dtype, std=0.5)
+    a = gu.dev_bits16(a32, dtype)
+    c = torch.full((m, n), float("nan"), dtype=tdt, device=gu.DEV)
+    workspace = torch.zeros(torch.cuda.get_device_properties(0).multi_processor_count, dtype=torch.int32,
+                            device=gu.DEV)
+    scratch = torch.empty(max(lib.sonar_marlin_gemm_scratch_bytes(m, n, k), 16), dtype=torch.uint8, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_gemm_nvfp4(
+        gu.ptr(a), k, gu.ptr(c), gu.ptr(L["native"]), _lib.LAYOUT_GFX950, gu.ptr(bias_dev), gu.ptr(L["scales"]),
+        gu.ptr(L["gs_dev"]), gu.ptr(workspace), workspace.numel(), gu.ptr(scratch), scratch.numel(),
+        gu.dtype_code(dtype), m, n, k, L["groups"], gu.stream()))
+    torch.cuda.synchronize()
+    ref = mo.gemm_reference(a32, L["w_ref"]).astype(np.float64) * L["global_scale"]
+    if bias:
+        ref = ref + bias32
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), ref.astype(np.float32))
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+    assert int(workspace.abs().sum().item()) == 0
+
+
+def test_nvfp4_rejected_configurations(gu):
+    """NVFP4 takes one scale per 16 rows and needs its global scale."""
+    from sonar_amd import _lib
+    lib = _lib.load()
+    k, n, m = 256, 128, 4
+    L = _layer_nvfp4(gu, 3, k, n, "bf16")
+    a = gu.dev_bits16(mo.make_activations(1, m, k, "bf16"), "bf16")
+    c = torch.empty((m, n), dtype=torch.bfloat16, device=gu.DEV)
+    workspace = torch.zeros(torch.cuda.get_device_properties(0).multi_processor_count, dtype=torch.int32,
+                            device=gu.DEV)
+    scratch = torch.empty(max(lib.sonar_marlin_gemm_scratch_bytes(m, n, k), 16), dtype=torch.uint8, device=gu.DEV)
+
+    def call(groups, gs):
+        return lib.sonar_marlin_gemm_nvfp4(
+            gu.ptr(a), k, gu.ptr(c), gu.ptr(L["native"]), _lib.LAYOUT_GFX950, None, gu.ptr(L["scales"]), gs,
+            gu.ptr(workspace), workspace.numel(), gu.ptr(scratch), scratch.numel(), gu.dtype_code("bf16"), m, n, k,
+            groups, gu.stream())
+    assert call(k // 32, gu.ptr(L["gs_dev"])) != 0 and "16 rows" in lib.sonar_marlin_last_error().decode()
+    assert call(k // 16, None) != 0 and "global_scale" in lib.sonar_marlin_last_error().decode()
+    assert call(k // 16, gu.ptr(L["gs_dev"])) == 0
+    torch.cuda.synchronize()
+
+
 def test_mxfp4_weights_rejected_configurations(gu):
     """MXFP4 exists for bfloat16 activations and groups of 32 rows only
     (generate_kernels.py:102-110), without act-order."""

@@ -481,6 +481,65 @@ def test_mxfp4_dequant_and_scale_reorder():
     assert y[0].tolist() == [0, 2, 1, 3, 4, 6, 5, 7] and np.array_equal(mo.mxfp4_process_scales(y), x)
 
 
+# ---------------------------------------------------------------- NVFP4 weights (float4_e2m1f, e4m3 scales, global scale)
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+def test_nvfp4_scale_bytes_against_both_kernel_readings(dtype):
+    """Every non-negative float8_e4m3fn scale (torch's own conversion on the CPU)
+    through nvfp4_process_scales and back through the kernel-side reading of a
+    byte (dequant.h:520-549): scale * scale_factor * 2^7, or 0 below 2."""
+    import torch
+    from fractions import Fraction
+    codes = torch.arange(0, 0x7F, dtype=torch.uint8)                 # 0 .. 448, no NaN
+    scales = codes.view(torch.float8_e4m3fn).float().numpy().reshape(1, -1)
+    scales = np.concatenate([scales, np.zeros((1, 1), np.float32)], axis=1)      # 128 columns
+    b, sf = mo.nvfp4_process_scales(scales, dtype)
+    assert sf == 1.0   # the largest scale is 448 already
+    back = mo.nvfp4_scale_bytes_as_16bit_float(b, dtype).astype(np.float64)
+    back = back.reshape(-1, 4)[:, [0, 2, 1, 3]].reshape(back.shape)   # the reorder is its own inverse
+    want = np.where(scales.astype(np.float64) * 128 < 2, 0.0, scales.astype(np.float64) * 128)
+    assert np.array_equal(back, want)
+    # the byte is bits 14..7 of the half-precision number: hand values
+    one = mo.nvfp4_process_scales(np.full((1, 4), 1.0, np.float32), "fp16")[0]
+    assert int(one[0, 0]) == (int(np.float16(128.0).view(np.uint16)) >> 7)    # 128.0 = 0x5800 -> 0xB0
+    assert int(one[0, 0]) == 0xB0
+    # kernel scales: value * 2^-bias, exact in the activation type
+    ks = mo.nvfp4_kernel_scales(b, dtype)
+    bias = mo.NVFP4_EXPONENT_BIAS[dtype]
+    assert np.array_equal(ks.astype(np.float64), want * 2.0 ** -bias)
+    assert np.array_equal(mo.round_to_dtype(ks, dtype), ks)
+    # the whole chain in exact arithmetic: value(code) * kernel scale * processed global scale
+    # == value(code) * scale * global scale, for every code and a sample of scales
+    g = 0.3712158203125
+    pg = mo.nvfp4_process_global_scale(g, dtype, sf)
+    assert Fraction(float(pg)) == Fraction(float(np.float32(g))) * Fraction(2) ** (bias - 7)
+    v = mo.fp4_e2m1_values()
+    for col in (8, 9, 57, 100, 126):
+        if want[0, col] == 0:
+            continue
+        for code in range(16):
+            w = mo.dequantize_nvfp4(np.full((16, 128), code), ks, dtype)[0, col]
+            assert Fraction(float(w)) * Fraction(float(pg)) == \
+                Fraction(float(v[code])) * Fraction(float(scales[0, col])) * Fraction(float(np.float32(g)))
+
+
+def test_nvfp4_scale_factor_and_small_scales():
+    """marlin_utils_fp4.py:37-58, 112-114: bf16 lifts small scales by a power of two
+    so that the largest is just below 448 (fp16 never does); what stays below
+    2^-6 after that is cut to zero."""
+    s = np.array([[0.5, 0.001953125, 3.0, 0.0]], dtype=np.float32)          # 2^-9 is the smallest e4m3 number
+    b16, sf16 = mo.nvfp4_process_scales(s, "fp16")
+    assert sf16 == 1.0
+    back = mo.nvfp4_scale_bytes_as_16bit_float(b16, "fp16")[0, [0, 2, 1, 3]]
+    assert back.tolist() == [64.0, 0.0, 384.0, 0.0]                          # 2^-9 * 128 = 0.25 < 2: cut
+    b, sf = mo.nvfp4_process_scales(s, "bf16")
+    assert sf == 128.0                                                        # 448 / 3 = 149.3 -> 2^7
+    back = mo.nvfp4_scale_bytes_as_16bit_float(b, "bf16")[0, [0, 2, 1, 3]]
+    assert back.tolist() == [64.0 * 128, 0.25 * 128, 384.0 * 128, 0.0]
+    assert mo.nvfp4_scale_factor(np.array([448.0], np.float32), "bf16") == 1.0
+    assert float(mo.nvfp4_process_global_scale(2.0, "bf16", 128.0)) == 2.0 * 2.0 ** 119 / 128
+    assert float(mo.nvfp4_process_global_scale(2.0, "fp16")) == 2.0 * 2.0 ** 7
+
+
 def test_moe_gemm_reference_against_per_slot_brute_force():
     """moe_gemm_reference (the oracle of the grouped GEMM) follows sorted_ids / expert_ids
     block by block.  Brute force from the routing itself, slot by slot, without any of
