@@ -237,6 +237,22 @@ int sonar_moe_wna16_marlin_gemm(
     int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
     int is_k_full, int use_atomic_add, int use_fp32_reduce, void* stream);
 
+/* The grouped GEMM for NVFP4 experts (moe/marlin_moe_wna16/ops.cu of the reference called
+ * with b_q_type = float4_e2m1f, float8_e4m3fn block scales and a global_scale per expert):
+ * b_scales dtype[E][size_k / 16][N] as for sonar_marlin_gemm_nvfp4, global_scale float[E] in
+ * device memory (row r of C is multiplied by the global scale of its block's expert before
+ * the bias and the routing weight).  No zero points, no act-order; the other arguments as for
+ * sonar_moe_wna16_marlin_gemm. */
+int sonar_moe_wna16_marlin_gemm_nvfp4(
+    const void* a, void* c, const uint32_t* b_q_weight, int b_layout,
+    const void* b_bias, const void* b_scales, const float* global_scale,
+    void* scratch, size_t scratch_bytes, const int32_t* sorted_token_ids,
+    int64_t sorted_len, const int32_t* expert_ids,
+    const int32_t* num_tokens_past_padded, const float* topk_weights,
+    int64_t moe_block_size, int64_t top_k, int mul_topk_weights,
+    int64_t num_experts, int dtype, int64_t size_m, int64_t size_n,
+    int64_t size_k, int64_t num_groups, void* stream);
+
 /* The small kernels around the two grouped GEMMs of a mixture-of-experts layer.
  * They have counterparts in every build of the reference (also on ROCm):
  *   sonar_moe_align_block_size -> _moe_C::moe_align_block_size

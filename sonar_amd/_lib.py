@@ -54,6 +54,10 @@ PROTOTYPES = {
         c_void_p, c_int64, c_void_p, c_size_t, c_void_p, c_int64, c_void_p, c_void_p, c_void_p,
         c_int64, c_int64, c_int, c_int64, c_int, c_int64, c_int64, c_int64, c_int64, c_int64,
         c_int, c_int, c_int, c_void_p]),
+    "sonar_moe_wna16_marlin_gemm_nvfp4": (c_int, [
+        c_void_p, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_size_t, c_void_p, c_int64,
+        c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int64, c_int, c_int64, c_int64, c_int64, c_int64,
+        c_void_p]),
     "sonar_moe_align_block_size": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p,
                                            c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sonar_silu_and_mul": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),

@@ -20,7 +20,7 @@ namespace sonar {
 
 // gemm_tile.hip: the MFMA-tiled grouped kernel for 64-slot blocks
 int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, const void* scales,
-                  const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
+                  const float* global_scale, const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
                   int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
                   int64_t num_groups, int group_size, int a_by_slot, bool fp4, int bits, bool fp8, hipStream_t st);
@@ -43,6 +43,7 @@ struct MoeParams {
   uint16_t* c;
   const uint4* b;
   const uint16_t* bias;
+  const float* global_scale;   // NVFP4: one number per expert that its output is multiplied by; else nullptr
   const uint16_t* scales;
   const uint32_t* zeros;
   const int32_t* perm;
@@ -85,6 +86,7 @@ __device__ __forceinline__ void moe_scatter(const MoeParams& p, const floatx4_t 
                                             long expert_l, int strip, int lane) {
   const int col16 = lane & 15;
   const uint16_t* bias = p.bias ? p.bias + expert_l * p.size_n + strip * kStripN : nullptr;
+  const float gs = p.global_scale ? p.global_scale[expert_l] : 1.f;   // marlin_template.h(moe):1661-1665
   const int n_in = 4 * (lane >> 4);
 #pragma unroll
   for (int mb = 0; mb < MB; ++mb) {
@@ -97,7 +99,7 @@ __device__ __forceinline__ void moe_scatter(const MoeParams& p, const floatx4_t 
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const int nl = 16 * j + n_in;
-      const floatx4_t v = acc[mb][j];
+      const floatx4_t v = acc[mb][j] * gs;
       float r[4] = {v.x, v.y, v.z, v.w};
       uint16_t o[4];
 #pragma unroll
@@ -130,10 +132,11 @@ struct MoeUnit {
 // HAS_GIDX (with HAS_PERM, symmetric weights): an act-order shard that does not
 // hold whole groups (is_k_full = false); every row finds its scale through g_idx
 // (marlin_moe_wna16/ops.cu:343-351).
-template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX, bool FP4 = false>
+// NV (with FP4): NVFP4, groups of 16 rows: a lane's eight rows of a chunk lie in group kb / 2 of its two.
+template <typename T, int MB, bool HAS_ZP, bool HAS_PERM, bool HAS_GIDX, bool FP4 = false, bool NV = false>
 __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoeParams p) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq4Of<T, FP4>::type D4;   // integer codes, or float4_e2m1f
+  typedef typename Dq4Of<T, FP4, NV>::type D4;   // integer codes, or float4_e2m1f
   typedef typename D4::Col Col;
   __shared__ float4 red[4][MB * 4][64];
   __shared__ int slot_id[16 * MB];
@@ -199,7 +202,8 @@ __global__ __launch_bounds__(kMoeWaves * 64) void marlin_moe_kernel(const MoePar
 #pragma unroll
       for (int cc = 0; cc < 4; ++cc)
         if (cc < p.unit_chunks)
-          u.sv[FP4 ? cc : 0] = *reinterpret_cast<const uint4*>(srow + (long)cc * p.size_n + 8 * (col16 & 7));
+          u.sv[FP4 ? cc : 0] = *reinterpret_cast<const uint4*>(srow + (long)(NV ? 2 * cc + (kb >> 1) : cc) * p.size_n +
+                                                              8 * (col16 & 7));
       return;
     }
 #pragma unroll
@@ -492,14 +496,14 @@ void launch_moe8_mb(const MoeParams& p, bool fp8, int grid, hipStream_t st) {
   }
 }
 
-// float4_e2m1f codes: no zero points, no act-order
-template <typename T>
+// float4_e2m1f codes: no zero points, no act-order (NV: NVFP4, scales per 16 rows)
+template <typename T, bool NV = false>
 void launch_moe_fp4(const MoeParams& p, int grid, hipStream_t st) {
   switch ((p.block_size + 15) / 16) {
-    case 1: marlin_moe_kernel<T, 1, false, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
-    case 2: marlin_moe_kernel<T, 2, false, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
-    case 3: marlin_moe_kernel<T, 3, false, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
-    default: marlin_moe_kernel<T, 4, false, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
+    case 1: marlin_moe_kernel<T, 1, false, false, false, true, NV><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
+    case 2: marlin_moe_kernel<T, 2, false, false, false, true, NV><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
+    case 3: marlin_moe_kernel<T, 3, false, false, false, true, NV><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
+    default: marlin_moe_kernel<T, 4, false, false, false, true, NV><<<grid, kMoeWaves * 64, 0, st>>>(p); break;
   }
 }
 
@@ -527,19 +531,17 @@ extern "C" size_t sonar_moe_marlin_gemm_scratch_bytes(int64_t sorted_len, int64_
   return moe_block_size == 64 ? moe_tile_table_bytes(sorted_len, 0) : 0;
 }
 
-extern "C" int sonar_moe_wna16_marlin_gemm(
+namespace {
+// The grouped GEMM behind sonar_moe_wna16_marlin_gemm (global_scale == nullptr) and its NVFP4 form.
+int moe_gemm_any(
     const void* a, void* c, const uint32_t* b_q_weight, int b_layout, const void* b_bias,
-    const void* b_scales, const uint32_t* b_zeros, const int32_t* g_idx, const int32_t* perm,
-    int32_t* workspace, int64_t workspace_len, void* scratch, size_t scratch_bytes,
+    const void* b_scales, const float* global_scale, const uint32_t* b_zeros, const int32_t* g_idx,
+    const int32_t* perm, void* scratch, size_t scratch_bytes,
     const int32_t* sorted_token_ids, int64_t sorted_len, const int32_t* expert_ids,
     const int32_t* num_tokens_past_padded, const float* topk_weights, int64_t moe_block_size,
     int64_t top_k, int mul_topk_weights, int64_t num_experts, int dtype, int64_t b_type_id,
-    int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int is_k_full,
-    int use_atomic_add, int use_fp32_reduce, void* stream) {
-  (void)workspace;
-  (void)workspace_len;
-  (void)use_atomic_add;
-  (void)use_fp32_reduce;
+    int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int is_k_full, void* stream) {
+  const bool nvfp4 = global_scale != nullptr;
   SONAR_REQUIRE(b_layout == SONAR_LAYOUT_GFX950, "unknown b_layout = %d", b_layout);
   SONAR_REQUIRE(dtype == SONAR_DTYPE_F16 || dtype == SONAR_DTYPE_BF16, "unsupported `a` scalar_type");
   // marlin_moe_wna16/ops.cu:560-566
@@ -571,7 +573,15 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                   "b_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   bool has_perm = perm != nullptr;
-  if (fp4) {
+  if (nvfp4) {
+    // moe/marlin_moe_wna16/generate_kernels.py:94-101: NVFP4, either activation type, a scale per 16 rows
+    SONAR_REQUIRE(fp4, "a global scale goes with float4_e2m1f weights only (NVFP4)");
+    SONAR_REQUIRE(!has_perm, "act-order is not supported with float4_e2m1f weights");
+    SONAR_REQUIRE(size_k == 16 * num_groups,
+                  "float4_e2m1f weights with a global scale (NVFP4) take one scale per group of 16 rows; got "
+                  "size_k = %ld, num_groups = %ld", (long)size_k, (long)num_groups);
+    SONAR_REQUIRE(((uintptr_t)b_scales) % 16 == 0, "b_scales must be 16-byte aligned");
+  } else if (fp4) {
     // moe/marlin_moe_wna16/generate_kernels.py:102-110: MXFP4, bfloat16 activations, a scale per 32 rows
     SONAR_REQUIRE(!has_perm, "act-order is not supported with float4_e2m1f weights");
     SONAR_REQUIRE(dtype == SONAR_DTYPE_BF16, "float4_e2m1f weights with power-of-two block scales (MXFP4) "
@@ -602,7 +612,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     SONAR_REQUIRE(size_k % num_groups == 0, "size_k = %ld, is not divisible by num_groups = %ld",
                   (long)size_k, (long)num_groups);
     group_size = (int)(size_k / num_groups);
-    SONAR_REQUIRE(group_size % kChunkK == 0, "group_size = %d must be a multiple of %d", group_size,
+    SONAR_REQUIRE(nvfp4 || group_size % kChunkK == 0, "group_size = %d must be a multiple of %d", group_size,
                   kChunkK);
   }
   if (size_m == 0 || sorted_len == 0) return SONAR_OK;
@@ -649,7 +659,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
                 "act-order with 8-bit expert weights needs sorted_len * size_k * 2 more scratch bytes "
                 "(the column-permuted copy of A per slot)");
   // Few rows per expert: the decode kernel, one workgroup per strip and 32 slots of a block
-  if (!bits8 && !row_groups &&
+  if (!bits8 && !row_groups && !nvfp4 &&
       moe_fast_applies(has_perm, moe_block_size, sorted_len, num_experts, a_rows, size_n, size_k, num_groups,
                        group_size))
     return moe_fast_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
@@ -658,9 +668,9 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
   static const bool no_tile = getenv("SONAR_MARLIN_NO_MOE_TILE") != nullptr;  // debugging aid
   // Full blocks of 64 slots mean many rows per expert: the MFMA-tiled kernel
   if (moe_block_size == 64 && !has_perm && !row_groups && !no_tile && size_k % 64 == 0 &&
-      (num_groups == 1 || group_size % 64 == 0 || group_size == 32) && scratch != nullptr &&
+      (num_groups == 1 || group_size % 64 == 0 || group_size == 32 || nvfp4) && scratch != nullptr &&
       scratch_bytes >= moe_tile_table_bytes(sorted_len, num_experts) && ((uintptr_t)scratch) % 4 == 0)
-    return moe_tile_gemm(a, c, b_q_weight, b_bias, b_scales, b_zeros, sorted_token_ids, sorted_len, expert_ids,
+    return moe_tile_gemm(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, sorted_token_ids, sorted_len, expert_ids,
                          num_tokens_past_padded, topk_weights, top_k, mul_topk_weights ? 1 : 0, num_experts,
                          static_cast<int32_t*>(scratch), dtype, size_m, size_n, size_k, num_groups, group_size,
                          a_by_slot, fp4, bits8 ? 8 : 4, fp8, st);
@@ -670,6 +680,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
   p.c = static_cast<uint16_t*>(c);
   p.b = reinterpret_cast<const uint4*>(b_q_weight);
   p.bias = static_cast<const uint16_t*>(b_bias);
+  p.global_scale = global_scale;
   p.scales = static_cast<const uint16_t*>(b_scales);
   p.zeros = b_zeros;
   p.perm = perm;
@@ -705,6 +716,11 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     else launch_moe8_mb<__bf16>(p, fp8, (int)grid, st);
     return launch_status("marlin_moe8_kernel");
   }
+  if (nvfp4) {
+    if (dtype == SONAR_DTYPE_F16) launch_moe_fp4<_Float16, true>(p, (int)grid, st);
+    else launch_moe_fp4<__bf16, true>(p, (int)grid, st);
+    return launch_status("marlin_moe_kernel");
+  }
   if (fp4) {
     launch_moe_fp4<__bf16>(p, (int)grid, st);
     return launch_status("marlin_moe_kernel");
@@ -717,4 +733,38 @@ extern "C" int sonar_moe_wna16_marlin_gemm(
     else launch_moe_mb<__bf16, false>(p, has_perm, (int)grid, st);
   }
   return launch_status("marlin_moe_kernel");
+}
+}  // namespace
+
+extern "C" int sonar_moe_wna16_marlin_gemm(
+    const void* a, void* c, const uint32_t* b_q_weight, int b_layout, const void* b_bias,
+    const void* b_scales, const uint32_t* b_zeros, const int32_t* g_idx, const int32_t* perm,
+    int32_t* workspace, int64_t workspace_len, void* scratch, size_t scratch_bytes,
+    const int32_t* sorted_token_ids, int64_t sorted_len, const int32_t* expert_ids,
+    const int32_t* num_tokens_past_padded, const float* topk_weights, int64_t moe_block_size,
+    int64_t top_k, int mul_topk_weights, int64_t num_experts, int dtype, int64_t b_type_id,
+    int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int is_k_full,
+    int use_atomic_add, int use_fp32_reduce, void* stream) {
+  (void)workspace;
+  (void)workspace_len;
+  (void)use_atomic_add;
+  (void)use_fp32_reduce;
+  return moe_gemm_any(a, c, b_q_weight, b_layout, b_bias, b_scales, nullptr, b_zeros, g_idx, perm, scratch,
+                      scratch_bytes, sorted_token_ids, sorted_len, expert_ids, num_tokens_past_padded, topk_weights,
+                      moe_block_size, top_k, mul_topk_weights, num_experts, dtype, b_type_id, size_m, size_n, size_k,
+                      num_groups, is_k_full, stream);
+}
+
+extern "C" int sonar_moe_wna16_marlin_gemm_nvfp4(
+    const void* a, void* c, const uint32_t* b_q_weight, int b_layout, const void* b_bias,
+    const void* b_scales, const float* global_scale, void* scratch, size_t scratch_bytes,
+    const int32_t* sorted_token_ids, int64_t sorted_len, const int32_t* expert_ids,
+    const int32_t* num_tokens_past_padded, const float* topk_weights, int64_t moe_block_size,
+    int64_t top_k, int mul_topk_weights, int64_t num_experts, int dtype, int64_t size_m, int64_t size_n,
+    int64_t size_k, int64_t num_groups, void* stream) {
+  SONAR_REQUIRE(global_scale != nullptr, "the global_scale parameter must be passed for nvfp4 format.");
+  return moe_gemm_any(a, c, b_q_weight, b_layout, b_bias, b_scales, global_scale, nullptr, nullptr, nullptr, scratch,
+                      scratch_bytes, sorted_token_ids, sorted_len, expert_ids, num_tokens_past_padded, topk_weights,
+                      moe_block_size, top_k, mul_topk_weights, num_experts, dtype, SONAR_TYPE_FLOAT4_E2M1F, size_m,
+                      size_n, size_k, num_groups, 1, stream);
 }

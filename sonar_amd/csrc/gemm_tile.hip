@@ -809,16 +809,17 @@ int launch_tile_async_fp4(const TileParams& p, hipStream_t st) {
   return SONAR_OK;
 }
 
-// NVFP4: either activation type, groups of 16 rows, a global scale
-template <typename T>
+// NVFP4: either activation type, groups of 16 rows, a global scale (one per expert when GROUPED)
+template <typename T, bool GROUPED = false>
 int launch_tile_async_nvfp4(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, false, false, true, true, 0, true>,
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_async_kernel<T, false, GROUPED, true, true, 0, true>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, async_lds(true)));
     attr_set = true;
   }
-  marlin_tile_async_kernel<T, false, false, true, true, 0, true><<<tile_grid(p), kTileWaves * 64, async_lds(true), st>>>(p);
+  marlin_tile_async_kernel<T, false, GROUPED, true, true, 0, true>
+      <<<tile_grid(p), kTileWaves * 64, async_lds(true), st>>>(p);
   return SONAR_OK;
 }
 
@@ -1001,7 +1002,7 @@ size_t moe_tile_table_bytes(int64_t sorted_len, int64_t num_experts) {
 // Called by sonar_moe_wna16_marlin_gemm for 64-slot blocks without act-order
 // when group_size % 64 == 0 (or one group) and size_k % 64 == 0.
 int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, const void* scales,
-                  const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
+                  const float* global_scale, const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
                   int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
                   int64_t num_groups, int group_size, int a_by_slot, bool fp4, int bits, bool fp8, hipStream_t st) {
@@ -1011,7 +1012,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                                                                              (int)num_experts, table, max_tiles);
   if (int rc = launch_status("moe_tile_table_kernel")) return rc;
   TileParams p;
-  p.global_scale = nullptr;
+  p.global_scale = global_scale;   // NVFP4: one per expert
   p.a = static_cast<const uint16_t*>(a);
   p.lda = size_k;
   p.c = static_cast<uint16_t*>(c);
@@ -1045,7 +1046,10 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.expert_z_stride = (long)(num_groups * (size_n / 8));
   p.expert_bias_stride = (long)size_n;
   int rc;
-  if (fp4)
+  if (fp4 && global_scale != nullptr)
+    rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16, true>(p, st)
+                                  : launch_tile_async_nvfp4<__bf16, true>(p, st);
+  else if (fp4)
     rc = launch_tile_grouped_fp4(p, st);
   else if (bits == 8)
     rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, true>(p, fp8, st)

@@ -554,8 +554,17 @@ Tensor moe_wna16_marlin_gemm(
   const int dtype = dtype_code(a);
   check_b_type(b_type_id);
   TORCH_CHECK_NOT_IMPLEMENTED(!a_scales.has_value(), "a_scales can only be used for 8bit activation.");
-  TORCH_CHECK_NOT_IMPLEMENTED(!global_scale.has_value(), "global_scale can only be used for nvfp4 format.");
   TORCH_CHECK_NOT_IMPLEMENTED(!is_zp_float, "is_zp_float = True is not built");
+  // marlin_moe_wna16/ops.cu: the global scale goes with NVFP4 and only with it
+  const bool nvfp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F && b_scales.scalar_type() == at::kFloat8_e4m3fn;
+  if (global_scale.has_value() && global_scale->numel() > 0) {
+    TORCH_CHECK(nvfp4, "global_scale can only be used for nvfp4 format.");
+    TORCH_CHECK(global_scale->is_cuda() && global_scale->scalar_type() == at::kFloat &&
+                    global_scale->is_contiguous(), "scalar type of global_scale must be float");
+    TORCH_CHECK(global_scale->numel() == b_q_weight.size(0), "global_scale must hold one number per expert");
+  } else {
+    TORCH_CHECK(!nvfp4, "the global_scale parameter must be passed for nvfp4 format.");
+  }
   TORCH_CHECK(moe_block_size == 8 || moe_block_size % 16 == 0, "unsupported moe_block_size=", moe_block_size);
   TORCH_CHECK(moe_block_size >= 8 && moe_block_size <= 64, "unsupported moe_block_size=", moe_block_size);
 
@@ -582,9 +591,10 @@ Tensor moe_wna16_marlin_gemm(
   if (mxfp8) {
     TORCH_CHECK(a.scalar_type() == at::kBFloat16, "float8_e4m3fn weights with float8_e8m0fnu scales (MXFP8) "
                 "need bfloat16 activations");
+  } else if (nvfp4) {
+    TORCH_CHECK(b_scales.size(1) * 16 == size_k, "float4_e2m1f weights with float8_e4m3fn scales (NVFP4) take one "
+                "scale per group of 16 rows; got size_k = ", size_k, ", b_scales.size(1) = ", b_scales.size(1));
   } else if (fp4) {
-    TORCH_CHECK_NOT_IMPLEMENTED(b_scales.scalar_type() != at::kFloat8_e4m3fn,
-                                "float4_e2m1f weights with float8_e4m3fn scales (NVFP4) are not built");
     TORCH_CHECK(is_mx_scale_type(b_scales),
                 "When b_type = float4_e2m1f, b_scale scalar type must be",
                 "float8_e4m3fn (for NVFP4) or float8_e8m0fnu (for MXFP4).");
@@ -658,6 +668,21 @@ Tensor moe_wna16_marlin_gemm(
   Tensor scratch;
   if (scratch_bytes > 0) scratch = at::empty({(int64_t)scratch_bytes}, a.options().dtype(at::kByte));
 
+  if (nvfp4) {
+    TORCH_CHECK(perm == nullptr, "act-order is not supported with float4_e2m1f weights");
+    raise_if_failed(sonar_moe_wna16_marlin_gemm_nvfp4(
+        a.const_data_ptr(), c.mutable_data_ptr(), static_cast<const uint32_t*>(native.const_data_ptr()),
+        SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none),
+        nvfp4_scales_as_16bit(b_scales, a.scalar_type()).const_data_ptr(),
+        static_cast<const float*>(global_scale->const_data_ptr()),
+        scratch_bytes > 0 ? scratch.mutable_data_ptr() : nullptr, scratch_bytes,
+        static_cast<const int32_t*>(sorted_token_ids.const_data_ptr()), sorted_token_ids.numel(),
+        static_cast<const int32_t*>(expert_ids.const_data_ptr()),
+        static_cast<const int32_t*>(num_tokens_past_padded.const_data_ptr()),
+        static_cast<const float*>(topk_weights.const_data_ptr()), moe_block_size, top_k, mul_topk_weights ? 1 : 0,
+        experts, dtype, size_m, size_n, size_k, num_groups, current_stream(a)));
+    return c;
+  }
   raise_if_failed(sonar_moe_wna16_marlin_gemm(
       a.const_data_ptr(), c.mutable_data_ptr(), static_cast<const uint32_t*>(native.const_data_ptr()),
       SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none),

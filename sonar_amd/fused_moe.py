@@ -185,8 +185,8 @@ def _check_unbuilt(activation, clamp_limit, gemm1_alpha, gemm1_beta, input_dtype
         raise NotImplementedError("activation_situ_beta / activation_situ_linear_beta are not built")
     if input_dtype is not None:
         raise NotImplementedError("8-bit activations (input_dtype) are not built")
-    if any(g is not None for g in global_scales):
-        raise NotImplementedError("global scales (NVFP4 / 8-bit activations) are not built")
+    if any(g is not None for g in global_scales[:2]):
+        raise NotImplementedError("input_global_scale1 / input_global_scale2 (8-bit activations) are not built")
 
 
 def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, num_topk,
@@ -222,7 +222,7 @@ def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, t
     cache2 = intermediate_cache2.view(-1)[:M * num_topk * N].view(M * num_topk, N)
 
     cache1 = ops.moe_wna16_marlin_gemm(
-        hidden_states, cache1, w1, bias1, w1_scale, None, None, w1_zeros, g_idx1, sort_indices1, workspace,
+        hidden_states, cache1, w1, bias1, w1_scale, None, global_scale1, w1_zeros, g_idx1, sort_indices1, workspace,
         sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, moe_block_size=block_size_m,
         top_k=num_topk, mul_topk_weights=apply_router_weight_on_input, b_q_type=quant_type, size_m=M,
         size_n=2 * N, size_k=K, is_k_full=is_k_full, use_atomic_add=False, use_fp32_reduce=True,
@@ -234,7 +234,7 @@ def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, t
     if output is None:
         output = cache3
     return ops.moe_wna16_marlin_gemm(
-        cache2, output, w2, bias2, w2_scale, None, None, w2_zeros, g_idx2, sort_indices2, workspace,
+        cache2, output, w2, bias2, w2_scale, None, global_scale2, w2_zeros, g_idx2, sort_indices2, workspace,
         sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, moe_block_size=block_size_m,
         top_k=1, mul_topk_weights=not apply_router_weight_on_input, b_q_type=quant_type,
         size_m=M * num_topk, size_n=K, size_k=N, is_k_full=is_k_full, use_atomic_add=False,
@@ -265,7 +265,8 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
     w2: (E, N/16, 2K); scales (E, groups, 2N) / (E, groups, K); topk_weights
     fp32 [M, top_k]; topk_ids [M, top_k].  Returns [M, K].  Parameters and their order are
     the reference's; of its activations only SILU is built (anything else, and clamp_limit /
-    gemm1_alpha / gemm1_beta / global scales / input_dtype, raise NotImplementedError).
+    gemm1_alpha / gemm1_beta / input global scales / input_dtype, raise NotImplementedError;
+    global_scale1 / global_scale2 are the per-expert global scales of NVFP4 experts).
     `activation_func(activation, out, in)` and `moe_sum(moe_output [M, top_k, K], output)`
     replace the built-in HIP kernels when given, as in the reference."""
     _check_unbuilt(activation, clamp_limit, gemm1_alpha, gemm1_beta, input_dtype,
@@ -273,7 +274,7 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
                    activation_situ_beta, activation_situ_linear_beta)
     if quant_type_id not in _SUPPORTED:
         raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8, uint8b128, "
-                                  "float8_e4m3fn and float4_e2m1f (MXFP4) expert weights are built")
+                                  "float8_e4m3fn and float4_e2m1f (MXFP4, NVFP4) expert weights are built")
     quant_type = _SUPPORTED[quant_type_id]
     M, K = hidden_states.shape
     E = w1.shape[0]
@@ -300,7 +301,7 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
         hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, topk, quant_type,
         apply_router_weight_on_input, expert_map, block_size_m, sorted_token_ids, expert_ids,
         num_tokens_post_padded, activation=activation, activation_func=activation_func, topk_ids=topk_ids,
-        g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1, sort_indices2=sort_indices2,
+        global_scale1=global_scale1, global_scale2=global_scale2, g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1, sort_indices2=sort_indices2,
         w1_zeros=w1_zeros, w2_zeros=w2_zeros, workspace=workspace,
         intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2, output=None,
         is_k_full=is_k_full).view(-1, topk, K)
@@ -336,7 +337,7 @@ def batched_fused_marlin_moe(hidden_states: torch.Tensor, expert_num_tokens: tor
     are not written."""
     if quant_type_id not in _SUPPORTED:
         raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8, uint8b128, "
-                                  "float8_e4m3fn and float4_e2m1f (MXFP4) expert weights are built")
+                                  "float8_e4m3fn and float4_e2m1f (MXFP4, NVFP4) expert weights are built")
     assert hidden_states.ndim == 3, f"hidden states must be batched. e.g. [B, MAX_TOKENS, K].But got {hidden_states.size()}"
     B, max_tokens, K = hidden_states.shape
     E = w1.shape[0]

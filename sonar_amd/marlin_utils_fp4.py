@@ -1,7 +1,7 @@
 """4-bit floating-point weights (float4_e2m1f codes) through the Marlin ops.
 Mirrors aphrodite/model_executor/layers/quantization/utils/marlin_utils_fp4.py
-of the reference for dense layers of both formats and MXFP4 experts: :34-151,
-153-290, 556-649, 652-753.  The checkpoint bytes (two codes each, low nibble
+of the reference for dense layers and experts of both formats: :34-151,
+153-290, 325-448, 556-649, 652-753.  The checkpoint bytes (two codes each, low nibble
 first along K) are GPTQ words as they stand and go through gptq_marlin_repack
 with num_bits = 4.  MXFP4: one power-of-two scale per 32 rows (exponent bytes e,
 value 2^(e - 127)), bf16 activations; the scales are permuted as for any Marlin
@@ -9,8 +9,7 @@ layer, every four neighbours are put in the order 0, 2, 1, 3, and they travel
 as float8_e8m0fnu.  NVFP4: one float8_e4m3fn scale per 16 rows and an fp32
 global scale, fp16 or bf16 activations; the scales travel as bytes of the
 reference's special 8-bit format (nvfp4_marlin_process_scales) and the global
-scale carries the exponent bias of the kernel-side reading.  NVFP4 experts
-(prepare_nvfp4_moe_layer_for_marlin) are not built.
+scale carries the exponent bias of the kernel-side reading.
 """
 from __future__ import annotations
 
@@ -182,6 +181,66 @@ def prepare_moe_mxfp4_layer_for_marlin(layer, w13: torch.Tensor, w2: torch.Tenso
 
     return (repack(w13, 2 * n, k), repack(w2, k, n), permute(w13_scale, 2 * n, k), permute(w2_scale, k, n),
             permute_bias(w13_bias), permute_bias(w2_bias))
+
+
+def prepare_nvfp4_moe_layer_for_marlin(layer, w13: torch.Tensor, w13_scale: torch.Tensor, w13_scale_2: torch.Tensor,
+                                       w2: torch.Tensor, w2_scale: torch.Tensor, w2_scale_2: torch.Tensor,
+                                       is_act_and_mul: bool = True):
+    """marlin_utils_fp4.py:325-448.  w13 (E, shards * N, K/2), w2 (E, K, N/2) uint8;
+    block scales (E, shards * N, K/16), (E, K, N/16) float8_e4m3fn; global scales
+    (E,) fp32; `layer` holds num_experts, hidden_size,
+    intermediate_size_per_partition and params_dtype.  N is padded to the tile
+    size with zero rows / columns.  All experts of a matrix share one scale
+    factor.  Returns (w13, w13_scale, w13_scale_2, w2, w2_scale, w2_scale_2)."""
+    group_size = 16
+    e, k, n = layer.num_experts, layer.hidden_size, layer.intermediate_size_per_partition
+    shards = 2 if is_act_and_mul else 1
+    if k % 128 == 0:
+        padded_n = (n + 63) // 64 * 64
+    else:
+        assert k % 64 == 0, f"hidden_size = {k} unsupported by Marlin tiles"
+        padded_n = (n + 127) // 128 * 128
+    param_dtype = layer.params_dtype
+    device = w13.device
+
+    def pad_w13(x: torch.Tensor) -> torch.Tensor:
+        if padded_n == n:
+            return x
+        x = torch.nn.functional.pad(x.view(e, shards, n, x.size(-1)), (0, 0, 0, padded_n - n))
+        return x.reshape(e, shards * padded_n, -1)
+
+    def pad_w2(x: torch.Tensor, packing: int) -> torch.Tensor:
+        return x if padded_n == n else torch.nn.functional.pad(x, (0, (padded_n - n) // packing))
+
+    layer.workspace = marlin_make_workspace_new(device, 4)
+    perm = torch.empty(0, dtype=torch.int, device=device)
+
+    def repack(weight: torch.Tensor, is_w13: bool) -> torch.Tensor:
+        if is_w13:
+            assert weight.shape == (e, n * shards, k // 2)
+            weight, size_n, size_k = pad_w13(weight), padded_n * shards, k
+        else:
+            assert weight.shape == (e, k, n // 2)
+            weight, size_n, size_k = pad_w2(weight, 2), k, padded_n
+        return torch.stack([ops.gptq_marlin_repack(weight[i].contiguous().view(torch.int32).T.contiguous(), perm,
+                                                   size_k, size_n, 4) for i in range(e)])
+
+    def permute_scales(scales: torch.Tensor, g_scales: torch.Tensor, is_w13: bool):
+        scales = scales.to(param_dtype)
+        if is_w13:
+            scales, size_n, size_k = pad_w13(scales), padded_n * shards, k
+        else:
+            scales, size_n, size_k = pad_w2(scales, group_size), k, padded_n
+        factor = _nvfp4_compute_scale_factor(scales, param_dtype)   # one for all experts: they share the processing
+        out = [nvfp4_marlin_process_scales(marlin_permute_scales(scales[i].T, size_k, size_n, group_size),
+                                           scale_factor=factor, a_dtype=param_dtype)[0] for i in range(e)]
+        g_scales = nvfp4_marlin_process_global_scale(g_scales.to(torch.float32), param_dtype) / factor
+        return torch.stack(out), g_scales
+
+    mw13, mw2 = repack(w13, True), repack(w2, False)
+    s13, g13 = permute_scales(w13_scale, w13_scale_2, True)
+    s2, g2 = permute_scales(w2_scale, w2_scale_2, False)
+    return mw13, s13, g13, mw2, s2, g2
 
 
 def rand_marlin_weight_mxfp4_like(weight: torch.Tensor, group_size: int, input_dtype: torch.dtype | None = None):

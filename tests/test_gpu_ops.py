@@ -921,6 +921,54 @@ def test_prepare_moe_mxfp4_layer_and_fused_marlin_moe(cfg):
     assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)
 
 
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("cfg", [
+    # m, experts, topk, hidden, intermediate
+    (5, 4, 2, 256, 128),
+    (70, 4, 2, 256, 256),
+    (200, 8, 2, 128, 96),      # intermediate size padded to 128 inside
+    (1500, 4, 2, 256, 128),    # 64-slot blocks: the tiled grouped kernel
+], ids=str)
+def test_prepare_nvfp4_moe_layer_and_fused_marlin_moe(cfg, dtype):
+    """NVFP4 expert weights (w13 (E, 2N, K/2), w2 (E, K, N/2) bytes, float8_e4m3fn block
+    scales per 16, a global scale per expert) -> prepare_nvfp4_moe_layer_for_marlin ->
+    fused_marlin_moe, against the per-token reference on value * scale * global scale."""
+    from sonar_amd import marlin_utils_fp4 as f4
+    from sonar_amd.fused_moe import fused_marlin_moe
+    from sonar_amd.scalar_type import scalar_types
+    m, e, topk, hidden, inter = cfg
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    rng = np.random.default_rng(hidden + inter + m)
+    layer = types.SimpleNamespace(params_dtype=tdt, num_experts=e, hidden_size=hidden,
+                                  intermediate_size_per_partition=inter)
+
+    def expert_set(rows, cols):   # checkpoint shape (E, rows = N of the GEMM, cols = K of the GEMM)
+        codes = rng.integers(0, 16, size=(e, rows, cols), dtype=np.int32)
+        sb = torch.from_numpy(rng.integers(0x30, 0x60, size=(e, rows, cols // 16)).astype(np.uint8))
+        sc = sb.view(torch.float8_e4m3fn).float().numpy()
+        g = (0.02 + 0.01 * rng.random(e)).astype(np.float32)
+        packed = np.ascontiguousarray((codes[:, :, 0::2] | (codes[:, :, 1::2] << 4)).astype(np.uint8))
+        ref = [(mo.fp4_e2m1_values()[codes[i]] * np.repeat(sc[i], 16, axis=1) * g[i]).T.astype(np.float32)
+               for i in range(e)]
+        return (torch.from_numpy(packed).to(gu.DEV), sb.view(torch.float8_e4m3fn).to(gu.DEV),
+                torch.from_numpy(g).to(gu.DEV), ref)
+
+    w13, s13, g13, ref13 = expert_set(2 * inter, hidden)
+    w2, s2, g2, ref2 = expert_set(hidden, inter)
+    mw13, ms13, mg13, mw2, ms2, mg2 = f4.prepare_nvfp4_moe_layer_for_marlin(layer, w13, s13, g13, w2, s2, g2)
+    assert ms13.dtype == torch.float8_e4m3fn and mg13.dtype == torch.float32 and mg13.shape == (e,)
+    topk_ids, topk_w = _route(m, e, topk, m)
+    x32 = mo.round_to_dtype(0.5 * mo.make_activations(m, m, hidden, dtype), dtype)
+    y = fused_marlin_moe(gu.dev_bits16(x32, dtype), mw13, mw2, None, None, ms13, ms2,
+                         torch.from_numpy(topk_w).to(gu.DEV), torch.from_numpy(topk_ids).to(gu.DEV),
+                         scalar_types.float4_e2m1f.id, global_scale1=mg13, global_scale2=mg2)
+    torch.cuda.synchronize()
+    want = _moe_reference(x32, ref13, ref2, topk_ids, topk_w, dtype, None, None)
+    got = gu.host_f32(y)
+    max_ref = np.abs(want).max()
+    assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)
+
+
 # ---------------------------------------------------------------- MXFP8 weights (float8_e4m3fn, e8m0 block scales)
 def _mxfp8_reference(codes_kn, exps_gn):
     """Oracle matrix for fp8 codes (K, N) and exponent bytes (K/32, N), bf16."""
