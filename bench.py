@@ -155,13 +155,14 @@ def variants_sweep(torch, ops, gen, time_graph):
     of A, weights repacked in sorted-group order), AWQ (per-group zero points),
     8-bit weights (uint8b128), fp8 weights (float8_e4m3fn, scales with the
     exponent bias folded in), MXFP8 and MXFP4 weights (float8_e4m3fn /
-    float4_e2m1f, exponent-byte scales per 32 rows, bf16 activations)."""
+    float4_e2m1f, exponent-byte scales per 32 rows, bf16 activations), NVFP4
+    weights (float4_e2m1f, float8_e4m3fn scales per 16 rows, a global scale)."""
     from sonar_amd import marlin_utils
     from sonar_amd.scalar_type import scalar_types
     dev = "cuda:0"
     k, n = 4096, 11008
     out = []
-    for name in ("act_order", "awq", "w8a16", "fp8", "mxfp8", "mxfp4"):
+    for name in ("act_order", "awq", "w8a16", "fp8", "mxfp8", "mxfp4", "nvfp4"):
         layers = []
         words = 4 * n if name in ("w8a16", "fp8", "mxfp8") else 2 * n     # 8-bit codes: four per word
         act_dtype = torch.bfloat16 if name in ("mxfp4", "mxfp8") else torch.float16
@@ -178,6 +179,11 @@ def variants_sweep(torch, ops, gen, time_graph):
                 layers.append((qw, sc * 0.0625, empty, empty, empty, ws, scalar_types.uint8b128))
             elif name == "fp8":
                 layers.append((qw, sc * 0.0625 * 256, empty, empty, empty, ws, scalar_types.float8_e4m3fn))
+            elif name == "nvfp4":
+                # scale bytes of the kernel-side format: top bit set, as nvfp4_marlin_process_scales leaves them
+                sb = torch.randint(0x90, 0xC0, (k // 16, n), dtype=torch.uint8, device=dev, generator=gen)
+                gs = torch.full((1,), 2.0 ** -3, dtype=torch.float32, device=dev)
+                layers.append((qw, sb.view(torch.float8_e4m3fn), gs, empty, empty, ws, scalar_types.float4_e2m1f))
             elif name in ("mxfp4", "mxfp8"):
                 e8 = torch.randint(110, 120, (k // 32, n), dtype=torch.uint8, device=dev, generator=gen)
                 wt = scalar_types.float4_e2m1f if name == "mxfp4" else scalar_types.float8_e4m3fn
@@ -189,8 +195,12 @@ def variants_sweep(torch, ops, gen, time_graph):
         for m in (1, 512):
             a = torch.randn((m, k), device=dev, generator=gen).to(act_dtype)
 
-            def one(i=0, a=a, m=m):
+            def one(i=0, a=a, m=m, name=name):
                 qw, sc, zp, g_idx, perm, ws, wt = layers[i % len(layers)]
+                if name == "nvfp4":   # the third entry is the global scale
+                    ops.marlin_gemm(a, None, qw, None, sc, None, zp, None, g_idx, perm, ws, wt, m, n, k, True,
+                                    False, True, False)
+                    return
                 ops.marlin_gemm(a, None, qw, None, sc, None, None, zp, g_idx, perm, ws, wt, m, n, k, True,
                                 False, True, False)
             s = time_graph(torch, one, 24 if m == 1 else 6)
@@ -199,6 +209,8 @@ def variants_sweep(torch, ops, gen, time_graph):
                 nb += k * n // 2                        # a byte per weight instead of half
             if name in ("mxfp4", "mxfp8"):
                 nb += (k // 32 - 2 * (k // GROUP)) * n  # a byte per 32 rows instead of two per 128
+            if name == "nvfp4":
+                nb += (k // 16 - 2 * (k // GROUP)) * n  # a byte per 16 rows
             fl = 2 * m * k * n
             out.append({"variant": name, "m": m, "k": k, "n": n, "us": round(s * 1e6, 2),
                         "GBps": round(nb / s / 1e9, 1), "TFLOPs": round(fl / s / 1e12, 2),

@@ -200,6 +200,28 @@ struct DqF4 : DqF4Generic<T> {};
 // generic form, which multiplies in fp32 and converts once, rounds nothing either.
 template <typename T>
 struct DqNvF4 : DqF4Generic<T> {};
+// fp16: the code read as an fp16 number (value * 2^-14) times the scale * 2^14 in one packed
+// multiply, the reference's own arithmetic (dequant.h:397-420, 520-531): scale * 2^14 is what
+// the reference reads a scale byte as, at most 448 * 2^7.
+template <>
+struct DqNvF4<_Float16> {
+  typedef Dq<_Float16>::vec8 vec8;
+  struct Col {
+    uint32_t s2;   // scale * 2^14, twice
+  };
+  static __device__ __forceinline__ Col make_col(uint16_t scale_bits, int) {
+    const _Float16 s = __builtin_bit_cast(_Float16, scale_bits) * (_Float16)16384.0f;
+    const uint32_t b = __builtin_bit_cast(uint16_t, s);
+    return Col{b | (b << 16)};
+  }
+  static __device__ __forceinline__ uint32_t pair(uint32_t y, uint32_t s2) {
+    const half2_t h = __builtin_bit_cast(half2_t, (y & 0x80008000u) | ((y & 0x70007000u) >> 3));
+    return __builtin_bit_cast(uint32_t, h * __builtin_bit_cast(half2_t, s2));
+  }
+  static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c, uint32_t) {
+    return __builtin_bit_cast(vec8, u32x4_t{pair(q << 12, c.s2), pair(q << 8, c.s2), pair(q << 4, c.s2), pair(q, c.s2)});
+  }
+};
 
 // bf16: the matrix-core generation this is written for converts two 4-bit
 // floats of a byte to bf16 and applies a power-of-two scale in one instruction
@@ -226,6 +248,34 @@ struct DqF4<__bf16> {
                                             __builtin_amdgcn_perm(r13, r02, 0x07060302u),
                                             __builtin_amdgcn_perm(r57, r46, 0x05040100u),
                                             __builtin_amdgcn_perm(r57, r46, 0x07060302u)});
+  }
+};
+
+// bf16: the hardware conversion with a unit scale gives the code's value; the two values of a
+// register (two rows of one column) are widened, multiplied by the scale in fp32 and cut back
+// (the product has at most five significant bits: nothing is lost).
+template <>
+struct DqNvF4<__bf16> {
+  typedef Dq<__bf16>::vec8 vec8;
+  struct Col {
+    float s;   // the block scale
+  };
+  static __device__ __forceinline__ Col make_col(uint16_t scale_bits, int) {
+    return Col{Dq<__bf16>::to_float(scale_bits)};
+  }
+  static __device__ __forceinline__ uint32_t scaled(uint32_t r, float s) {
+    const float lo = __uint_as_float(r << 16) * s, hi = __uint_as_float(r & 0xFFFF0000u) * s;
+    return __builtin_amdgcn_perm(__float_as_uint(hi), __float_as_uint(lo), 0x07060302u);
+  }
+  static __device__ __forceinline__ vec8 word(uint32_t q, const Col& c, uint32_t) {
+    const uint32_t r02 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, 1.0f, 0));
+    const uint32_t r46 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, 1.0f, 1));
+    const uint32_t r13 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, 1.0f, 2));
+    const uint32_t r57 = __builtin_bit_cast(uint32_t, __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(q, 1.0f, 3));
+    return __builtin_bit_cast(vec8, u32x4_t{scaled(__builtin_amdgcn_perm(r13, r02, 0x05040100u), c.s),
+                                            scaled(__builtin_amdgcn_perm(r13, r02, 0x07060302u), c.s),
+                                            scaled(__builtin_amdgcn_perm(r57, r46, 0x05040100u), c.s),
+                                            scaled(__builtin_amdgcn_perm(r57, r46, 0x07060302u), c.s)});
   }
 };
 
