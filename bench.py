@@ -132,6 +132,50 @@ def memory_yardsticks(torch):
     return out
 
 
+def launch_floors(torch, time_graph):
+    """What one launch costs and how long the chip takes to stream the weights of
+    each GEMM of the layer when nothing is computed, with the yardstick kernels of
+    sonar_amd/csrc/bench_floor.hip (not part of the product path): an empty kernel
+    as a node of a HIP graph, and a kernel that copies a matrix's bytes into LDS
+    with the decode kernel's own asynchronous copies on all compute units, over
+    six regions of 1 GiB in turn so that nothing comes from a cache."""
+    import ctypes
+    from sonar_amd import build
+    if not os.path.exists(build.BENCH_PATH):
+        return None
+    lib = ctypes.CDLL(build.BENCH_PATH)
+    lib.sonar_bench_empty.argtypes = [ctypes.c_int, ctypes.c_void_p]
+    lib.sonar_bench_stream.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
+    cus = torch.cuda.get_device_properties(0).multi_processor_count
+    buf = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 256)
+    region = (1 << 30) // 6 // 4096 * 4096
+
+    def raw_stream():
+        return torch.cuda.current_stream().cuda_stream
+
+    def check(rc):
+        if rc != 0:
+            raise RuntimeError("bench_floor launch failed: %d" % rc)
+
+    out = {"empty_kernel_us": round(time_graph(torch, lambda i=0: check(lib.sonar_bench_empty(cus, raw_stream())),
+                                               24) * 1e6, 2),
+           "stream": []}
+    total = 0.0
+    for name, k, n in LAYER_SHAPES:
+        nbytes = k * n // 2 + (k // GROUP) * n * 2          # packed weights and scales
+        assert nbytes <= region
+
+        def one(i=0, nbytes=nbytes):
+            check(lib.sonar_bench_stream(buf.data_ptr() + (i % 6) * region, nbytes, cus, raw_stream()))
+        s = time_graph(torch, one, 24)
+        total += s
+        out["stream"].append({"gemm": name, "bytes": nbytes, "us": round(s * 1e6, 2),
+                              "GBps": round(nbytes / s / 1e9, 1)})
+    out["stream_step_us"] = round(total * 1e6, 2)
+    del buf
+    return out
+
+
 def cpu_baseline(threads: int):
     """The layer's CPU path (int4 dequantise + fp32 torch.matmul) from the
     oracle, on the o_proj shape at M = 16."""
@@ -515,6 +559,9 @@ def main() -> int:
         out["moe"] = moe_sweep(torch, gen, time_graph)
 
     out["yardsticks"] = memory_yardsticks(torch)
+    floors = launch_floors(torch, time_graph)
+    if floors is not None:
+        out["floors"] = floors
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(min(os.cpu_count() or 1, 16))
     print(json.dumps(out))

@@ -13,6 +13,7 @@ CSRC = os.path.join(PKG, "csrc")
 LIB_DIR = os.path.join(PKG, "lib")
 LIB_PATH = os.path.join(LIB_DIR, "libsonar_marlin.so")
 OPS_PATH = os.path.join(LIB_DIR, "libsonar_marlin_torch.so")
+BENCH_PATH = os.path.join(LIB_DIR, "libsonar_bench.so")   # bench.py's yardstick kernels, not part of the product
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
 HIP_SOURCES = ["repack.hip", "gemm_stream.hip", "gemm_tile.hip", "gemm_moe.hip", "moe_aux.hip"]
@@ -55,6 +56,16 @@ def build_hip_library(verbose: bool = False, only=None) -> str:
     return LIB_PATH
 
 
+def build_bench_library(verbose: bool = False) -> str:
+    """Compiles the yardstick kernels bench.py times beside the GEMMs (an empty kernel, a
+    kernel that only streams bytes) into a library of their own."""
+    os.makedirs(LIB_DIR, exist_ok=True)
+    out = _run([HIPCC, *HIP_FLAGS, "-shared", "-o", BENCH_PATH, os.path.join(CSRC, "bench_floor.hip")])
+    if verbose and out.strip():
+        print(out)
+    return BENCH_PATH
+
+
 def build_torch_ops(verbose: bool = False) -> str:
     """Compiles the C++ torch op registration layer with the host compiler and
     links it against the HIP library."""
@@ -84,6 +95,7 @@ def build_all(verbose: bool = False):
     paths = [build_hip_library(verbose)]
     if os.path.exists(os.path.join(CSRC, "torch_bindings.cpp")):
         paths.append(build_torch_ops(verbose))
+    paths.append(build_bench_library(verbose))
     return paths
 
 
