@@ -53,6 +53,18 @@ reference checkout).  How each function is pinned (none is "parity unpinned"):
                            scales 2^(e - 127) against torch's float8_e8m0fnu
                            conversion; the (0, 2, 1, 3) reorder is its own
                            inverse
+* 8-bit activations        the 32 x 32 tile order (is_a_8bit) by the same two
+                           derivations (get_weight_perm(4, True) recipe against
+                           the repack kernel's arithmetic,
+                           gptq_marlin_repack.cu:129-216), bijection, round
+                           trips; the fp8 preprocess against the two formulas
+                           the reference's tests state
+                           (test_marlin_gemm.py:148-188) and its inverse; the
+                           int8 GEMM against a per-element python loop with
+                           the textbook dequantised matmul as the limit case
+                           (all group scales equal); per_token_quant_int8
+                           against hand values and the round trip bound
+                           |x - q*s| <= s/2
 * NVFP4 weights            the scale bytes (nvfp4_process_scales) decoded by both
                            of the kernel's readings (dequant.h:520-549: b << 7
                            as fp16, and sign / exponent / mantissa moved into a
@@ -281,6 +293,246 @@ def awq_marlin_repack(b_q_weight: np.ndarray, size_k: int, size_n: int) -> np.nd
     q = awq_unpack(b_q_weight)
     assert q.shape == (size_k, size_n)
     return marlin_pack(q)
+
+
+# --------------------------------------------------------------------------
+# 4-bit weights for 8-bit activations (is_a_8bit): 32(k) x 32(n) tiles
+# --------------------------------------------------------------------------
+
+A8_ORDER = np.array([0, 4, 1, 5, 2, 6, 3, 7])  # marlin_utils_test.py:108
+
+
+def marlin_weight_perm_recipe_a8() -> np.ndarray:
+    """The 1024-entry gather table of a 32(k) x 32(n) tile for 4-bit weights
+    and 8-bit activations, built the way get_weight_perm(4, is_a_8bit=True)
+    builds it (marlin_utils_test.py:71-88,106-120)."""
+    table = []
+    for lane in range(32):
+        col = lane // 4
+        one = []
+        for block in (0, 1):
+            for row in ([4 * (lane % 4) + t for t in range(4)]
+                        + [4 * (lane % 4 + 4) + t for t in range(4)]):
+                one.append(16 * row + col + 8 * block)
+        for j in range(2):
+            table.extend(p + 512 * j for p in one)
+    perm = np.array(table)
+    return perm.reshape(-1, 8)[:, A8_ORDER].ravel()
+
+
+def marlin_pack_recipe_a8(q: np.ndarray) -> np.ndarray:
+    """(K,N) codes -> Marlin (K/16, 2N) int32 for 8-bit activations following
+    marlin_permute_weights(is_a_8bit=True) + marlin_weights
+    (marlin_utils_test.py:31-66)."""
+    k, n = q.shape
+    assert k % 32 == 0 and n % 64 == 0
+    perm = marlin_weight_perm_recipe_a8()
+    t = q.reshape(k // 32, 32, n // 16, 16).transpose(0, 2, 1, 3).reshape(k // 16, n * 16)
+    t = t.reshape(-1, perm.size)[:, perm].reshape(t.shape)
+    u = t.astype(np.uint32).reshape(k // 16, n * 2, 8)
+    out = np.zeros((k // 16, n * 2), dtype=np.uint32)
+    for i in range(8):
+        out |= u[:, :, i] << np.uint32(4 * i)
+    return out.view(np.int32)
+
+
+def _a8_word_sources(lane: int, warp: int):
+    """Rows and column (inside a 32 x 32 tile) of the eight nibble slots of
+    word lane*4 + warp, from the repack kernel's arithmetic
+    (gptq_marlin_repack.cu:129-141,176-216 with is_a_8bit): column
+    16*(warp/2) + 8*(warp%2) + lane/4; vals[i] = row 4*(lane%4) + i, vals[4+i]
+    = that row + 16; slot s holds vals[{0,4,1,5,2,6,3,7}[s]]."""
+    col = 16 * (warp // 2) + 8 * (warp % 2) + lane // 4
+    rows = []
+    for slot in range(8):
+        i = (0, 4, 1, 5, 2, 6, 3, 7)[slot]
+        rows.append(4 * (lane % 4) + (i % 4) + 16 * (i // 4))
+    return rows, col
+
+
+def marlin_pack_closed_form_a8(q: np.ndarray) -> np.ndarray:
+    """Same layout from the repack kernels' per-thread arithmetic: tile
+    (kt, nt) of 32 x 32 is 128 words at (kt*n_tiles + nt)*128, word
+    lane*4 + warp."""
+    k, n = q.shape
+    assert k % 32 == 0 and n % 64 == 0
+    kt_n, nt_n = k // 32, n // 32
+    tile = q.reshape(kt_n, 32, nt_n, 32).astype(np.uint32)  # [kt][r][nt][c]
+    out = np.zeros((kt_n, nt_n, 32, 4), dtype=np.uint32)
+    for lane in range(32):
+        for warp in range(4):
+            rows, col = _a8_word_sources(lane, warp)
+            word = np.zeros((kt_n, nt_n), dtype=np.uint32)
+            for slot in range(8):
+                word |= tile[:, rows[slot], :, col] << np.uint32(4 * slot)
+            out[:, :, lane, warp] = word
+    return out.reshape(k // 16, n * 2).view(np.int32)
+
+
+marlin_pack_a8 = marlin_pack_closed_form_a8
+
+
+def marlin_unpack_a8(packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    """Inverse of marlin_pack_a8."""
+    kt_n, nt_n = size_k // 32, size_n // 32
+    u = packed.view(np.uint32).reshape(kt_n, nt_n, 32, 4)
+    q = np.empty((kt_n, 32, nt_n, 32), dtype=np.int32)
+    for lane in range(32):
+        for warp in range(4):
+            rows, col = _a8_word_sources(lane, warp)
+            for slot in range(8):
+                q[:, rows[slot], :, col] = (u[:, :, lane, warp] >> np.uint32(4 * slot)) & np.uint32(0xF)
+    return q.reshape(size_k, size_n)
+
+
+def gptq_marlin_repack_a8(b_q_weight: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    """gptq_marlin_repack with is_a_8bit (no act-order: the kernel has
+    static_assert(!is_a_8bit) under has_perm, gptq_marlin_repack.cu:147)."""
+    q = unpack_rows(b_q_weight)
+    assert q.shape == (size_k, size_n)
+    return marlin_pack_a8(q)
+
+
+def awq_marlin_repack_a8(b_q_weight: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    q = awq_unpack(b_q_weight)
+    assert q.shape == (size_k, size_n)
+    return marlin_pack_a8(q)
+
+
+def marlin_a8_to_gfx950(marlin_packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    return gfx950_pack(marlin_unpack_a8(marlin_packed, size_k, size_n))
+
+
+def int4_fp8_preprocess(q: np.ndarray, zeros: np.ndarray | None = None,
+                        group_size: int | None = None) -> np.ndarray:
+    """marlin_int4_fp8_preprocess.cu:13-66 on unpacked codes (the op works
+    nibble by nibble, so the packing does not matter): sign and magnitude of
+    code - z in a nibble; q >= z: q - z, else 15 - q.  z = 8 without zero
+    points.  tests/kernels/quantization/test_marlin_gemm.py:148-188 states
+    the same two formulas."""
+    q = q.astype(np.int32)
+    if zeros is None:
+        return np.where(q >= 8, q - 8, 15 - q).astype(np.int32)
+    z = np.repeat(zeros.astype(np.int32), group_size, axis=0)
+    return np.where(q >= z, q - z, 15 - q).astype(np.int32)
+
+
+def int4_fp8_preprocess_inverse(p: np.ndarray) -> np.ndarray:
+    """Codes back from the preprocessed nibbles (no zero points)."""
+    p = p.astype(np.int32)
+    return np.where(p < 8, p + 8, 15 - p).astype(np.int32)
+
+
+def marlin_permute_scales_a8(s: np.ndarray, size_k: int, size_n: int, group_size: int) -> np.ndarray:
+    """marlin_utils.py:415-426 with is_a_8bit: always the single permutation."""
+    return np.ascontiguousarray(s.reshape(-1, 32)[:, SCALE_PERM_SINGLE].reshape(-1, size_n))
+
+
+def marlin_unpermute_scales_a8(s: np.ndarray, size_k: int, size_n: int, group_size: int) -> np.ndarray:
+    out = np.empty_like(s).reshape(-1, 32)
+    out[:, SCALE_PERM_SINGLE] = s.reshape(-1, 32)
+    return np.ascontiguousarray(out.reshape(-1, size_n))
+
+
+def marlin_zero_points_a8(zp: np.ndarray, num_groups: int, size_n: int) -> np.ndarray:
+    """marlin_utils.py:456-477 with is_a_8bit: the scale permutation without
+    the column interleave."""
+    t = zp.reshape(-1, 64)[:, SCALE_PERM].reshape(num_groups, size_n)
+    return pack_cols(t)
+
+
+def marlin_unpack_zero_points_a8(zp_packed: np.ndarray, num_groups: int, size_n: int) -> np.ndarray:
+    u = unpack_cols(zp_packed).reshape(-1, 64)
+    out = np.empty_like(u)
+    out[:, SCALE_PERM] = u
+    return out.reshape(num_groups, size_n)
+
+
+def awq_to_marlin_zero_points_a8(q_zp_packed: np.ndarray, num_groups: int, size_n: int) -> np.ndarray:
+    return marlin_zero_points_a8(awq_unpack(q_zp_packed), num_groups, size_n)
+
+
+def marlin_act_int8_process_scales(s32: np.ndarray):
+    """marlin_utils.py:436-440: group scales as 16-bit integers
+    round(s / max * 4096) and the factor max / 4096 that goes into the
+    activation scales.  Returns (int16 array, float32 factor)."""
+    top = np.float32(s32.max())
+    factor = np.float32(np.float32(1.0 / 4096.0) * top)
+    ints = np.rint((s32.astype(np.float32) / top) * np.float32(4096.0)).astype(np.int16)
+    return ints, factor
+
+
+def per_token_quant_int8(x32: np.ndarray):
+    """int8_utils.py:70-93: scale = absmax / 127 per row (absmax at least
+    1e-10), codes round-half-away(x * (127 / absmax)).  Returns (int8 (M,K),
+    float32 (M,1))."""
+    x = x32.astype(np.float32)
+    absmax = np.maximum(np.max(np.abs(x), axis=1, keepdims=True), np.float32(1e-10)).astype(np.float32)
+    scale = (absmax / np.float32(127.0)).astype(np.float32)
+    y = x * (np.float32(127.0) / absmax).astype(np.float32)
+    codes = (np.sign(y) * np.floor(np.abs(y) + np.float32(0.5))).astype(np.int8)
+    return codes, scale
+
+
+def gemm_w4a8_int8(a_q: np.ndarray, a_scales: np.ndarray, q: np.ndarray, group_size: int,
+                   scales, dtype: str, zeros: np.ndarray | None = None,
+                   bias32: np.ndarray | None = None) -> np.ndarray:
+    """W4A8 with int8 activations (marlin_template.h:1302-1362,1869-1903,
+    1955-1978).  Grouped (scales = the 16-bit integers of
+    marlin_act_int8_process_scales, (groups, N)):
+        c = sum_g scales[g][n] * sum_{k in g} a[m][k] * (q[k][n] - z)
+    in 32-bit integer arithmetic (wrapping), out = float(c) * a_scales[m].
+    Channelwise (group_size -1, scales = fp32 values of `dtype`, (1, N)):
+        out = (float(sum_k a * (q - z)) * a_scales[m]) * scales[n].
+    Then + bias in fp32 and one rounding to `dtype`.  z = 8 or the group's
+    zero point.  Integer sums do not depend on the order, so a kernel matches
+    this bit for bit."""
+    m, k = a_q.shape
+    n = q.shape[1]
+    grouped = group_size not in (-1, k)
+    gs = group_size if grouped else k
+    groups = k // gs
+    if zeros is None:
+        centred = q.astype(np.int64) - 8
+    else:
+        centred = q.astype(np.int64) - np.repeat(zeros.astype(np.int64), gs, axis=0)
+    a = a_q.astype(np.int64)
+    total = np.zeros((m, n), dtype=np.int64)
+    for g in range(groups):
+        part = a[:, g * gs:(g + 1) * gs] @ centred[g * gs:(g + 1) * gs, :]
+        part = ((part + 2**31) % 2**32) - 2**31
+        if grouped:
+            part = part * np.asarray(scales)[g].astype(np.uint16).astype(np.int64)[None, :]
+        total = ((total + part + 2**31) % 2**32) - 2**31
+    out = total.astype(np.int32).astype(np.float32) * a_scales.reshape(m, 1).astype(np.float32)
+    if not grouped:
+        out = out * np.asarray(scales, dtype=np.float32).reshape(1, n)
+    if bias32 is not None:
+        out = out + bias32.astype(np.float32)[None, :]
+    return round_to_dtype(out.astype(np.float32), dtype)
+
+
+def gemm_w4a8_fp8(a_fp8_32: np.ndarray, a_scales: np.ndarray, q: np.ndarray, group_size: int,
+                  scales32: np.ndarray, zeros: np.ndarray | None = None,
+                  bias32: np.ndarray | None = None) -> np.ndarray:
+    """W4A8 with float8_e4m3fn activations (a_fp8_32: their values as fp32):
+    out = (sum_g s[g][n] * sum_{k in g} a[m][k] * (q[k][n] - z)) * a_scales[m]
+    (+ bias), in float64 here: a floating-point kernel is compared within a
+    tolerance.  The reference keeps the weights as (q - z) * 2^-9 in fp8 and
+    the scales times 512 (marlin_utils_test.py:156-158): the same product."""
+    m, k = a_fp8_32.shape
+    n = q.shape[1]
+    grouped = group_size not in (-1, k)
+    gs = group_size if grouped else k
+    if zeros is None:
+        centred = q.astype(np.float64) - 8.0
+    else:
+        centred = q.astype(np.float64) - np.repeat(zeros.astype(np.float64), gs, axis=0)
+    w = centred * np.repeat(scales32.astype(np.float64), gs, axis=0)
+    out = (a_fp8_32.astype(np.float64) @ w) * a_scales.reshape(m, 1).astype(np.float64)
+    if bias32 is not None:
+        out = out + bias32.astype(np.float64)[None, :]
+    return out.astype(np.float32)
 
 
 # --------------------------------------------------------------------------

@@ -583,3 +583,157 @@ def test_moe_gemm_reference_against_per_slot_brute_force():
     kept = np.setdiff1d(np.arange(m * top_k), dropped)
     full = mo.moe_gemm_reference(a, w, sorted_ids, expert_ids, int(past[0]), bs, top_k, m, None, "fp16")
     assert np.array_equal(got[kept], full[kept])
+
+
+# ------------------------------------------------- 8-bit activations (W4A8)
+@pytest.mark.parametrize("k,n", [(32, 64), (96, 128), (160, 192)])
+def test_marlin_a8_layout_two_derivations_agree(k, n):
+    rng = np.random.default_rng(k + n)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    recipe = mo.marlin_pack_recipe_a8(q)
+    closed = mo.marlin_pack_closed_form_a8(q)
+    assert recipe.shape == (k // 16, 2 * n)
+    assert np.array_equal(recipe, closed)
+    assert np.array_equal(mo.marlin_unpack_a8(closed, k, n), q)
+    # a different order from the 16-bit one (a mix-up of the two would pass nothing above)
+    assert not np.array_equal(closed, mo.marlin_pack(q))
+    # the gather table is a permutation of the 1024 tile elements
+    perm = mo.marlin_weight_perm_recipe_a8()
+    assert sorted(perm.tolist()) == list(range(1024))
+
+
+def test_marlin_a8_layout_single_positions():
+    # one code set at (k, n): the word and nibble the repack kernel's arithmetic gives by hand:
+    # tile (k/32, n/32), lane 4*(n%8) + (k%16)/4, warp (n%32)/8, slot 2*(k%4) + (k%32)/16
+    for k, n in [(0, 0), (5, 9), (17, 31), (40, 70), (63, 127)]:
+        q = np.zeros((64, 128), dtype=np.int32)
+        q[k, n] = 15
+        w = mo.marlin_pack_a8(q).view(np.uint32).reshape(-1)
+        idx = np.nonzero(w)[0]
+        assert idx.size == 1
+        tile = (k // 32) * (128 // 32) + n // 32
+        lane = 4 * (n % 8) + (k % 16) // 4
+        warp = (n % 32) // 8
+        slot = 2 * (k % 4) + (k % 32) // 16
+        assert idx[0] == tile * 128 + lane * 4 + warp
+        assert w[idx[0]] == 15 << (4 * slot)
+
+
+def test_repack_a8_identities_and_gfx950():
+    rng = np.random.default_rng(3)
+    q = rng.integers(0, 16, size=(64, 128), dtype=np.int32)
+    m = mo.marlin_pack_a8(q)
+    assert np.array_equal(mo.gptq_marlin_repack_a8(mo.pack_rows(q), 64, 128), m)
+    assert np.array_equal(mo.awq_marlin_repack_a8(mo.awq_pack(q), 64, 128), m)
+    assert np.array_equal(mo.marlin_a8_to_gfx950(m, 64, 128), mo.gfx950_pack(q))
+
+
+def test_scales_and_zero_points_a8():
+    rng = np.random.default_rng(4)
+    s = rng.uniform(1, 2, size=(4, 128)).astype(np.float32)
+    p = mo.marlin_permute_scales_a8(s, 512, 128, 128)
+    # always the single permutation: equal to the 16-bit channelwise one row by row
+    for g in range(4):
+        assert np.array_equal(p[g:g + 1], mo.marlin_permute_scales(s[g:g + 1], 128, 128, -1))
+    assert np.array_equal(mo.marlin_unpermute_scales_a8(p, 512, 128, 128), s)
+    zp = rng.integers(0, 16, size=(4, 128), dtype=np.int32)
+    packed = mo.marlin_zero_points_a8(zp, 4, 128)
+    assert np.array_equal(mo.marlin_unpack_zero_points_a8(packed, 4, 128), zp)
+    # column n of a 64 block: word n % 8, nibble n / 8 (the transpose, no interleave)
+    one = np.zeros((1, 64), dtype=np.int32)
+    one[0, 19] = 7
+    w = mo.marlin_zero_points_a8(one, 1, 64).view(np.uint32).reshape(-1)
+    assert w[19 % 8] == 7 << (4 * (19 // 8)) and np.count_nonzero(w) == 1
+    assert np.array_equal(mo.awq_to_marlin_zero_points_a8(mo.awq_pack(zp), 4, 128), packed)
+
+
+def test_int4_fp8_preprocess_formulas_and_inverse():
+    # the two formulas of tests/kernels/quantization/test_marlin_gemm.py:148-188
+    q = np.arange(16, dtype=np.int32).reshape(16, 1)
+    assert mo.int4_fp8_preprocess(q).reshape(-1).tolist() == \
+        [15, 14, 13, 12, 11, 10, 9, 8, 0, 1, 2, 3, 4, 5, 6, 7]
+    assert np.array_equal(mo.int4_fp8_preprocess_inverse(mo.int4_fp8_preprocess(q)), q)
+    rng = np.random.default_rng(5)
+    qq = rng.integers(0, 16, size=(64, 8), dtype=np.int32)
+    zz = rng.integers(0, 16, size=(2, 8), dtype=np.int32)
+    want = qq - np.repeat(zz, 32, axis=0)
+    want[want < 0] = (15 - qq)[want < 0]
+    assert np.array_equal(mo.int4_fp8_preprocess(qq, zz, 32), want)
+    # sign and magnitude: the kernel reads nibble p as -(8 - q) = -((p & 7) + 1) when p >= 8
+    p = mo.int4_fp8_preprocess(q).reshape(-1)
+    value = np.where(p < 8, p, -((p & 7) + 1))
+    assert np.array_equal(value, np.arange(16) - 8)
+
+
+def test_per_token_quant_int8_hand_values_and_bound():
+    x = np.array([[127.0, -63.5, 0.4, -0.5], [1e-12, 0, 0, 0], [2.0, 1.0, -1.0, 0.5]], dtype=np.float32)
+    codes, scale = mo.per_token_quant_int8(x)
+    assert codes[0].tolist() == [127, -64, 0, -1]          # halves round away from zero
+    assert np.isclose(scale[0, 0], 1.0)
+    assert scale[1, 0] == np.float32(1e-10) / np.float32(127)  # the floor of absmax
+    assert codes[2].tolist() == [127, 64, -64, 32]          # 63.5 -> 64, 31.75 -> 32
+    rng = np.random.default_rng(6)
+    y = rng.normal(size=(8, 256)).astype(np.float32)
+    c, s = mo.per_token_quant_int8(y)
+    assert np.all(np.abs(y - c.astype(np.float32) * s) <= s * 0.5001)
+    assert np.all(np.max(np.abs(c), axis=1) == 127)
+
+
+def test_marlin_act_int8_process_scales():
+    s = np.array([[0.5, 1.0], [0.25, 0.1234]], dtype=np.float32)
+    ints, factor = mo.marlin_act_int8_process_scales(s)
+    assert ints.tolist() == [[2048, 4096], [1024, 505]]     # 0.1234 * 4096 = 505.4
+    assert factor == np.float32(1.0 / 4096)
+
+
+@pytest.mark.parametrize("group_size,zp", [(-1, False), (32, False), (64, True), (128, True)])
+def test_gemm_w4a8_int8_against_python_loop(group_size, zp):
+    rng = np.random.default_rng(7 + (group_size % 97))
+    m, k, n = 3, 128, 8
+    a = rng.integers(-127, 128, size=(m, k)).astype(np.int8)
+    a_s = rng.uniform(0.01, 0.02, size=(m, 1)).astype(np.float32)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    gs = k if group_size == -1 else group_size
+    groups = k // gs
+    zeros = rng.integers(0, 16, size=(groups, n), dtype=np.int32) if zp else None
+    if group_size == -1:
+        scales = mo.round_to_dtype(rng.uniform(1e-3, 1e-2, size=(1, n)).astype(np.float32), "fp16")
+    else:
+        scales = rng.integers(1, 4097, size=(groups, n)).astype(np.int16)
+    got = mo.gemm_w4a8_int8(a, a_s, q, group_size, scales, "fp16", zeros)
+    for mm in range(m):
+        for nn in range(n):
+            total = 0
+            for g in range(groups):
+                part = 0
+                for kk in range(g * gs, (g + 1) * gs):
+                    z = 8 if zeros is None else int(zeros[g, nn])
+                    part += int(a[mm, kk]) * (int(q[kk, nn]) - z)
+                total += part * (int(scales[g, nn]) if group_size != -1 else 1)
+            want = np.float32(total) * a_s[mm, 0]
+            if group_size == -1:
+                want = want * scales[0, nn]
+            assert got[mm, nn] == np.float32(want).astype(np.float16).astype(np.float32)
+
+
+def test_gemm_w4a8_limit_cases():
+    # all integer group scales equal to c: the result is c * (a @ (q - 8)), the textbook product
+    rng = np.random.default_rng(8)
+    a = rng.integers(-127, 128, size=(4, 64)).astype(np.int8)
+    q = rng.integers(0, 16, size=(64, 16), dtype=np.int32)
+    ones = np.ones((4, 1), dtype=np.float32)
+    got = mo.gemm_w4a8_int8(a, ones, q, 32, np.full((2, 16), 3, dtype=np.int16), "bf16")
+    want = mo.round_to_dtype((3 * (a.astype(np.int64) @ (q.astype(np.int64) - 8))).astype(np.float32), "bf16")
+    assert np.array_equal(got, want)
+    # 32-bit wrap-around of the integer accumulator is part of the definition
+    big = mo.gemm_w4a8_int8(np.full((1, 128), 127, dtype=np.int8), np.ones((1, 1), np.float32),
+                            np.full((128, 1), 15, dtype=np.int32), 64,
+                            np.full((2, 1), -1, dtype=np.int16), "bf16")  # -1 is read as 65535
+    wrapped = (2 * 127 * 7 * 64 * 65535 + 2**31) % 2**32 - 2**31
+    assert wrapped != 2 * 127 * 7 * 64 * 65535
+    assert big[0, 0] == mo.round_to_dtype(np.array([wrapped], dtype=np.float32), "bf16")[0]
+    # fp8 activations: equal to the dequantised matmul
+    af = rng.integers(-8, 9, size=(2, 64)).astype(np.float32)
+    s = rng.uniform(0.5, 1, size=(2, 16)).astype(np.float32)
+    w = (q - 8) * np.repeat(s, 32, axis=0)
+    assert np.allclose(mo.gemm_w4a8_fp8(af, np.ones((2, 1), np.float32), q, 32, s), af @ w, rtol=1e-6)
