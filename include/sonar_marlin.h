@@ -20,6 +20,12 @@
  *        csrc/libtorch_stable/quantization/marlin/marlin.cu:546-897
  *   sonar_marlin_gemm_nvfp4   -> the same op called with b_q_type = float4_e2m1f, float8_e4m3fn
  *        block scales and a global_scale (marlin.cu:600-611,784-796)
+ *   sonar_marlin_gemm_a8      -> the same op called with int8 or float8_e4m3fn activations and
+ *        a_scales (marlin.cu:567-598,666-679; marlin_template.h:1302-1400,1869-1903)
+ *   sonar_gptq_marlin_repack_a8 / sonar_awq_marlin_repack_a8 -> the repack ops with is_a_8bit
+ *        (gptq_marlin_repack.cu:14-268, awq_marlin_repack.cu:14-212)
+ *   sonar_marlin_int4_fp8_preprocess -> _C::marlin_int4_fp8_preprocess
+ *        csrc/libtorch_stable/quantization/marlin/marlin_int4_fp8_preprocess.cu:13-121
  *   sonar_moe_wna16_marlin_gemm -> _moe_C::moe_wna16_marlin_gemm
  *        csrc/libtorch_stable/moe/torch_bindings.cpp:76-89,
  *        csrc/libtorch_stable/moe/marlin_moe_wna16/ops.cu:544-897
@@ -46,6 +52,10 @@ extern "C" {
 /* activation / output / scale element types */
 #define SONAR_DTYPE_F16 0
 #define SONAR_DTYPE_BF16 1
+
+/* 8-bit activation types of sonar_marlin_gemm_a8 */
+#define SONAR_ADTYPE_INT8 0
+#define SONAR_ADTYPE_FP8 1        /* float8_e4m3fn */
 
 /* weight orders accepted by the GEMM entry points */
 #define SONAR_LAYOUT_GFX950 0      /* output of sonar_marlin_to_gfx950 */
@@ -103,6 +113,31 @@ int sonar_marlin8_to_gfx950(const uint32_t* marlin, uint32_t* out,
 int sonar_gfx950_to_marlin8(const uint32_t* gfx950, uint32_t* out,
                             int64_t size_k, int64_t size_n, void* stream);
 
+/* The repack ops with is_a_8bit = true (gptq_marlin_repack.cu:14-268, awq_marlin_repack.cu:14-212):
+ * 4-bit codes into the order the reference's kernels read with 8-bit activations, tiles of
+ * 32 (k) x 32 (n).  in as for the ops above, out (K/16, 2N) int32.  size_k % 32 == 0,
+ * size_n % 64 == 0, num_bits 4 (8 is SONAR_E_UNSUPPORTED: the GEMM has no 8-bit weights with 8-bit
+ * activations); no perm (the reference's kernel refuses act-order with is_a_8bit). */
+int sonar_gptq_marlin_repack_a8(const uint32_t* b_q_weight, uint32_t* out,
+                                int64_t size_k, int64_t size_n, int num_bits, void* stream);
+int sonar_awq_marlin_repack_a8(const uint32_t* b_q_weight, uint32_t* out,
+                               int64_t size_k, int64_t size_n, int num_bits, void* stream);
+/* That order <-> the streaming order of the gfx950 kernels (the same one as for 16-bit
+ * activations).  No counterpart in the reference. */
+int sonar_marlin_a8_to_gfx950(const uint32_t* marlin, uint32_t* out,
+                              int64_t size_k, int64_t size_n, void* stream);
+int sonar_gfx950_to_marlin_a8(const uint32_t* gfx950, uint32_t* out,
+                              int64_t size_k, int64_t size_n, void* stream);
+
+/* marlin_int4_fp8_preprocess (marlin_int4_fp8_preprocess.cu:13-121): every 4-bit code q of
+ * qweight becomes sign and magnitude of q - z in a nibble: q >= z ? q - z : 15 - q.  qzeros NULL:
+ * z = 8, qweight is rows * words_per_row words in any order.  qzeros given (AWQ): qweight is
+ * (rows = size_k, words_per_row = size_n / 8), qzeros (size_k / group_size, size_n / 8), both in the
+ * checkpoint's order.  out may be qweight. */
+int sonar_marlin_int4_fp8_preprocess(const uint32_t* qweight, const uint32_t* qzeros, uint32_t* out,
+                                     int64_t rows, int64_t words_per_row, int64_t group_size,
+                                     void* stream);
+
 /* Dequantised weight matrix W[K][N] (row-major, dtype elements) exactly as the
  * GEMM kernels form it in registers: round_to_dtype((code - z) * s), for
  * float8_e4m3fn round_to_dtype(value(code) * scale).  Uses the
@@ -151,6 +186,38 @@ int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                       int64_t size_m, int64_t size_n, int64_t size_k,
                       int64_t num_groups, int is_k_full, int use_atomic_add,
                       int use_fp32_reduce, void* stream);
+
+/* W4A8 (marlin.cu:567-598,666-679 of the reference; marlin_template.h:1302-1400,1869-1903,
+ * 1955-1978): 4-bit weights, 8-bit activations with one fp32 scale per row, on the 8-bit matrix
+ * cores.
+ *   a            int8 (a_dtype SONAR_ADTYPE_INT8) or float8_e4m3fn bytes (SONAR_ADTYPE_FP8),
+ *                [M][a_row_stride], 16-byte aligned, a_row_stride % 8 == 0
+ *   a_scales     float[M]
+ *   c            dtype[M][N]; dtype is also the type of b_scales (channelwise) and b_bias
+ *   b_q_weight   K*N/8 words in b_layout order.  With fp8 activations the nibbles are the ones
+ *                marlin_int4_fp8_preprocess leaves (sign and magnitude), as the reference's callers
+ *                store them
+ *   b_scales     [num_groups][N] in marlin_permute_scales(is_a_8bit=True) order (the single
+ *                permutation inside every 32 columns).  int8 activations and num_groups > 1: 16-bit
+ *                unsigned integers (marlin_act_int8_process_scales); otherwise numbers of dtype; with
+ *                fp8 activations they carry the factor 512 the reference's callers apply
+ *   b_zeros      int32[num_groups][N/8] in marlin_zero_points(is_a_8bit=True) order, iff uint4
+ *   b_bias       dtype[N] in marlin_permute_bias order, or NULL
+ *   scratch      sonar_marlin_gemm_a8_scratch_bytes() bytes
+ * int8:  C = round(float(sum_g s[g][n] * sum_{k in g} a[m][k] * (q[k][n] - z)) * a_scales[m] + bias),
+ *        the sums in wrapping 32-bit integers (exact, whatever the order); channelwise:
+ *        round((float(sum_k a (q - z)) * a_scales[m]) * s[n] + bias).
+ * fp8:   the same with fp32 sums and the weights (q - z) * 2^-9.
+ * num_groups 1 (channelwise) or size_k / 32, / 64, / 128; size_k % 32 == 0, size_n % 64 == 0; no
+ * act-order (the reference builds no such kernel).  b_type_id uint4b8 or uint4. */
+size_t sonar_marlin_gemm_a8_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k,
+                                          int64_t num_groups);
+int sonar_marlin_gemm_a8(const void* a, int64_t a_row_stride, int a_dtype, void* c,
+                         const uint32_t* b_q_weight, int b_layout, const void* b_bias,
+                         const void* b_scales, const float* a_scales, const uint32_t* b_zeros,
+                         void* scratch, size_t scratch_bytes, int dtype, int64_t b_type_id,
+                         int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
+                         void* stream);
 
 /* NVFP4 (marlin.cu:600-611,784-796 of the reference; marlin_template.h:1661-1665;
  * marlin_utils_fp4.py:59-151): float4_e2m1f codes (b_q_weight as for the other 4-bit types),

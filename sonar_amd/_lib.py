@@ -13,6 +13,8 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "lib
 DTYPE_F16 = 0
 DTYPE_BF16 = 1
 LAYOUT_GFX950 = 0
+ADTYPE_INT8 = 0
+ADTYPE_FP8 = 1
 TYPE_UINT4B8 = 1125899907892224
 TYPE_UINT4 = 1125899906843648
 TYPE_UINT8B128 = 1125899923621888
@@ -34,6 +36,15 @@ PROTOTYPES = {
     "sonar_gfx950_to_marlin": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "sonar_marlin8_to_gfx950": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "sonar_gfx950_to_marlin8": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "sonar_gptq_marlin_repack_a8": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
+    "sonar_awq_marlin_repack_a8": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
+    "sonar_marlin_a8_to_gfx950": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "sonar_gfx950_to_marlin_a8": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "sonar_marlin_int4_fp8_preprocess": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
+    "sonar_marlin_gemm_a8_scratch_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
+    "sonar_marlin_gemm_a8": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
+                                     c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int64, c_int64, c_int64,
+                                     c_int64, c_int64, c_void_p]),
     "sonar_marlin_dequant": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                      c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "sonar_marlin_gemm_scratch_bytes": (c_size_t, [c_int64, c_int64, c_int64]),

@@ -1,0 +1,405 @@
+// W4A8: 4-bit weights with 8-bit activations (int8 or float8_e4m3fn, one fp32
+// scale per activation row) on the 8-bit matrix cores
+// (v_mfma_i32_16x16x32_i8 / v_mfma_f32_16x16x32_fp8_fp8).  The path of the
+// reference's Marlin kernel with is_a_8bit
+// (csrc/libtorch_stable/quantization/marlin/marlin_template.h:1302-1400,
+// 1869-1903,1955-1978; dequant.h:492-606).
+//
+// A workgroup of four wavefronts owns one 64-column strip of the weight
+// stream, up to 64 activation rows and a range of K.  The wavefronts take the
+// scale groups of that range in turn (a group is 1, 2 or 4 chunks of 32 rows;
+// channelwise weights are walked in runs of 4 chunks), so the sum over one
+// group stays inside one wavefront: it is multiplied by the group's scale and
+// added to the wavefront's running total, in 32-bit integers for int8
+// activations (the scales are then 16-bit integers) and in fp32 for fp8.  The
+// four totals meet in LDS; wavefront w finishes column block w.  With K split
+// over several workgroups the raw totals go to scratch and a second kernel
+// adds them, so integer results never depend on the split.
+#include "common.hpp"
+#include "dequant.hpp"
+
+namespace sonar {
+namespace {
+
+typedef int intx4_t __attribute__((ext_vector_type(4)));
+
+struct A8Params {
+  const uint8_t* a;        // [M][a_row_stride] bytes
+  long a_row_stride;
+  void* c;                 // T [M][N]
+  const uint32_t* w;       // gfx950 order
+  const uint16_t* scales;  // [groups][N], single-permuted inside every 32 columns
+  const uint32_t* zeros;   // [groups][N/8] or null
+  const float* a_scales;   // [M]
+  const uint16_t* bias;    // T [N], permuted like the scales, or null
+  uint32_t* partial;       // [splits][M][N] raw totals when splits > 1
+  int m, n, chunks;
+  int unit_chunks;         // chunks per group (4 for channelwise)
+  int units;               // ceil(chunks / unit_chunks)
+  int units_per_split;
+  int splits;
+};
+
+template <typename T>
+__device__ __forceinline__ float from_bits(uint16_t b) {
+  return (float)__builtin_bit_cast(T, b);
+}
+template <typename T>
+__device__ __forceinline__ uint16_t to_bits(float f) {
+  return __builtin_bit_cast(uint16_t, (T)f);
+}
+
+// Raw 32 bits of a total and back (by value: an element of a vector type is not an object
+// __builtin_bit_cast can take).
+__device__ __forceinline__ uint32_t raw_bits(int v) { return (uint32_t)v; }
+__device__ __forceinline__ uint32_t raw_bits(float v) { return __float_as_uint(v); }
+__device__ __forceinline__ void from_raw(uint32_t b, int& v) { v = (int)b; }
+__device__ __forceinline__ void from_raw(uint32_t b, float& v) { v = __uint_as_float(b); }
+
+// Activation type: what the matrix core accumulates in and how a weight word
+// becomes two operand registers.  The eight codes of a word sit at the nibbles
+// {row 0, 2, 4, 6, 1, 3, 5, 7}; the low nibbles of the four bytes are rows
+// (0, 4, 1, 5), the high ones rows (2, 6, 3, 7): that is the byte order of the
+// B operand, and the A operand is shuffled to match.
+struct ActInt8 {
+  typedef intx4_t acc_t;
+  typedef int scalar_t;
+  static constexpr bool kInteger = true;
+  static __device__ __forceinline__ acc_t mfma(long a, long b, acc_t c) {
+    return __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, c, 0, 0, 0);
+  }
+  // uint4b8: the code with its top bit flipped is the 4-bit two's complement of
+  // code - 8; in the high nibble of a byte it reads as 16 * (code - 8).
+  static constexpr int kShift = 4;
+  static __device__ __forceinline__ long word(uint32_t w) {
+    const uint32_t x = w ^ 0x88888888u;
+    const uint32_t lo = (x << 4) & 0xf0f0f0f0u;
+    const uint32_t hi = x & 0xf0f0f0f0u;
+    return (long)(((uint64_t)hi << 32) | lo);
+  }
+  // uint4 with zero point z: ((q | 0x80) - z) ^ 0x80 is the two's complement
+  // byte of q - z, with no borrow between bytes (dequant.h:572-583).
+  static __device__ __forceinline__ long word_zp(uint32_t w, uint32_t z4) {
+    const uint32_t lo = (((w & 0x0f0f0f0fu) | 0x80808080u) - z4) ^ 0x80808080u;
+    const uint32_t hi = ((((w >> 4) & 0x0f0f0f0fu) | 0x80808080u) - z4) ^ 0x80808080u;
+    return (long)(((uint64_t)hi << 32) | lo);
+  }
+};
+
+struct ActFp8 {
+  typedef floatx4_t acc_t;
+  typedef float scalar_t;
+  static constexpr bool kInteger = false;
+  static __device__ __forceinline__ acc_t mfma(long a, long b, acc_t c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, b, c, 0, 0, 0);
+  }
+  static constexpr int kShift = 0;
+  // The nibble holds sign and magnitude as marlin_int4_fp8_preprocess leaves
+  // them: p < 8: +p, else -((p & 7) + 1).  As a float8_e4m3fn byte with a zero
+  // exponent field the magnitude m reads m * 2^-9 (8 carries into the exponent:
+  // 2^-6); the scales carry the factor 512 (dequant.h:504-515).
+  static __device__ __forceinline__ uint32_t four(uint32_t p) {
+    const uint32_t s = p & 0x08080808u;
+    return ((p & 0x07070707u) | (s << 4)) + (s >> 3);
+  }
+  static __device__ __forceinline__ long word(uint32_t w) {
+    return (long)(((uint64_t)four((w >> 4) & 0x0f0f0f0fu) << 32) | four(w & 0x0f0f0f0fu));
+  }
+  // With zero points the nibble is q >= z ? q - z : 15 - q (dequant.h:585-606).
+  static __device__ __forceinline__ uint32_t four_zp(uint32_t p, uint32_t z, uint32_t z4) {
+    const uint32_t q0 = p | 0x70707070u;
+    const uint32_t s = (q0 + z4) & 0x80808080u;
+    return ((q0 + (s >> 7) * (z + 1)) & 0x0f0f0f0fu) | s;
+  }
+  static __device__ __forceinline__ long word_zp(uint32_t w, uint32_t z4) {
+    const uint32_t z = z4 & 0xffu;
+    return (long)(((uint64_t)four_zp((w >> 4) & 0x0f0f0f0fu, z, z4) << 32) | four_zp(w & 0x0f0f0f0fu, z, z4));
+  }
+};
+
+// Raw total -> output value: the activation row's scale, for channelwise
+// weights the column's scale, the bias, one rounding.
+template <typename ACT, typename T, bool GROUPED>
+__device__ __forceinline__ uint16_t finish(typename ACT::scalar_t total, float a_scale, float col_scale,
+                                           float bias) {
+  // every step rounds to fp32 as written (the reference's epilogue does: marlin_template.h:1869-1903,
+  // 1955-1978); contraction would fuse them into the final conversion and round once
+#pragma clang fp contract(off)
+  float f = (float)total * a_scale;
+  if (!GROUPED) f *= col_scale;
+  f += bias;
+  return to_bits<T>(f);
+}
+
+template <typename ACT, typename T, int MB, bool HAS_ZP, bool GROUPED>
+__global__ __launch_bounds__(256) void marlin_a8_kernel(A8Params p) {
+  typedef typename ACT::acc_t acc_t;
+  typedef typename ACT::scalar_t scalar_t;
+  __shared__ uint32_t red[4][MB * 16][64];
+
+  const int strip = blockIdx.x, slab = blockIdx.y, split = blockIdx.z;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int m0 = slab * (MB * 16);
+
+  acc_t acc[MB][4];
+#pragma unroll
+  for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[rb][j] = acc_t{0, 0, 0, 0};
+
+  // this lane's row of A in every row block (rows past M read row M - 1, their results are dropped)
+  const uint8_t* a_row[MB];
+#pragma unroll
+  for (int rb = 0; rb < MB; ++rb) {
+    int row = m0 + 16 * rb + l16;
+    if (row >= p.m) row = p.m - 1;
+    a_row[rb] = p.a + (long)row * p.a_row_stride + 8 * kb;
+  }
+  const uint32_t* w_lane = p.w + (long)strip * p.chunks * kChunkWords + lane * 4;
+  int s_col[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) s_col[j] = strip * kStripN + scale_slot(16 * j + l16, false);
+
+  const int u_begin = split * p.units_per_split;
+  const int u_end = min(u_begin + p.units_per_split, p.units);
+  for (int u = u_begin + wave; u < u_end; u += 4) {
+    acc_t tmp[MB][4];
+#pragma unroll
+    for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) tmp[rb][j] = acc_t{0, 0, 0, 0};
+    const int g = GROUPED ? u : 0;
+    uint32_t z4[4] = {0, 0, 0, 0};
+    if (HAS_ZP) {
+      // column 16j + l16 of the strip: word l16 % 8 of the strip's eight, nibble 2j + l16 / 8
+      const uint32_t zw = p.zeros[(long)g * (p.n / 8) + strip * 8 + (l16 & 7)];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) z4[j] = ((zw >> (4 * (2 * j + (l16 >> 3)))) & 0xFu) * 0x01010101u;
+    }
+    const int c_begin = u * p.unit_chunks;
+    const int c_end = min(c_begin + p.unit_chunks, p.chunks);
+    for (int c = c_begin; c < c_end; ++c) {
+      const u32x4_t w4 = *reinterpret_cast<const u32x4_t*>(w_lane + (long)c * kChunkWords);
+      long a[MB];
+#pragma unroll
+      for (int rb = 0; rb < MB; ++rb) {
+        const uint2 v = *reinterpret_cast<const uint2*>(a_row[rb] + (long)c * kChunkK);
+        const uint32_t lo = __builtin_amdgcn_perm(v.y, v.x, 0x05010400u);   // bytes k = 0, 4, 1, 5
+        const uint32_t hi = __builtin_amdgcn_perm(v.y, v.x, 0x07030602u);   // bytes k = 2, 6, 3, 7
+        a[rb] = (long)(((uint64_t)hi << 32) | lo);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const long b = HAS_ZP ? ACT::word_zp(w4[j], z4[j]) : ACT::word(w4[j]);
+#pragma unroll
+        for (int rb = 0; rb < MB; ++rb) tmp[rb][j] = ACT::mfma(a[rb], b, tmp[rb][j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      scalar_t s = 1;
+      if (GROUPED) {
+        const uint16_t bits = p.scales[(long)g * p.n + s_col[j]];
+        if constexpr (ACT::kInteger) s = (int)bits;   // read as unsigned (marlin_template.h:1341-1348)
+        else s = from_bits<T>(bits);
+      }
+#pragma unroll
+      for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if constexpr (ACT::kInteger)
+            acc[rb][j][i] += (tmp[rb][j][i] >> (HAS_ZP ? 0 : ACT::kShift)) * s;
+          else
+            acc[rb][j][i] += tmp[rb][j][i] * s;
+        }
+    }
+  }
+
+  // the four wavefronts' totals meet in LDS; wavefront w sums column block w
+#pragma unroll
+  for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const scalar_t v = acc[rb][j][i];
+        red[wave][(rb * 4 + j) * 4 + i][lane] = raw_bits(v);
+      }
+  __syncthreads();
+  const int col = strip * kStripN + 16 * wave + l16;
+  float col_scale = 1.0f, bias = 0.0f;
+  if (p.splits == 1) {
+    const int slot = strip * kStripN + scale_slot(16 * wave + l16, false);
+    if (!GROUPED) col_scale = from_bits<T>(p.scales[slot]);
+    if (p.bias) bias = from_bits<T>(p.bias[slot]);
+  }
+#pragma unroll
+  for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      scalar_t total = 0;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) {
+        scalar_t part;
+        from_raw(red[ww][(rb * 4 + wave) * 4 + i][lane], part);
+        total += part;
+      }
+      const int row = m0 + 16 * rb + 4 * kb + i;
+      if (row >= p.m) continue;
+      if (p.splits == 1)
+        reinterpret_cast<uint16_t*>(p.c)[(long)row * p.n + col] =
+            finish<ACT, T, GROUPED>(total, p.a_scales[row], col_scale, bias);
+      else
+        p.partial[((long)split * p.m + row) * p.n + col] = raw_bits(total);
+    }
+}
+
+// Adds the raw totals of the K splits and finishes them.
+template <typename ACT, typename T, bool GROUPED>
+__global__ __launch_bounds__(256) void marlin_a8_finish_kernel(A8Params p) {
+  typedef typename ACT::scalar_t scalar_t;
+  const long total_elems = (long)p.m * p.n;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_elems;
+       idx += (long)gridDim.x * blockDim.x) {
+    const int row = (int)(idx / p.n), col = (int)(idx % p.n);
+    scalar_t total = 0;
+    for (int s = 0; s < p.splits; ++s) {
+      scalar_t part;
+      from_raw(p.partial[(long)s * total_elems + idx], part);
+      total += part;
+    }
+    const int slot = (col & ~63) + scale_slot(col & 63, false);
+    const float col_scale = GROUPED ? 1.0f : from_bits<T>(p.scales[slot]);
+    const float bias = p.bias ? from_bits<T>(p.bias[slot]) : 0.0f;
+    reinterpret_cast<uint16_t*>(p.c)[idx] = finish<ACT, T, GROUPED>(total, p.a_scales[row], col_scale, bias);
+  }
+}
+
+struct A8Plan {
+  int mb, slabs, splits, units, unit_chunks, units_per_split;
+};
+
+A8Plan plan_a8(int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups) {
+  A8Plan plan;
+  plan.mb = size_m > 48 ? 4 : (int)((size_m + 15) / 16);
+  plan.slabs = (int)((size_m + plan.mb * 16 - 1) / (plan.mb * 16));
+  const int chunks = (int)(size_k / kChunkK);
+  plan.unit_chunks = num_groups > 1 ? (int)(size_k / num_groups) / kChunkK : 4;
+  plan.units = (chunks + plan.unit_chunks - 1) / plan.unit_chunks;
+  // about four workgroups per compute unit, each wavefront with at least two groups
+  const long wgs = (long)(size_n / kStripN) * plan.slabs;
+  int splits = (int)((1024 + wgs - 1) / wgs);
+  if (splits > plan.units / 8) splits = plan.units / 8;
+  if (splits > 32) splits = 32;
+  if (splits < 1) splits = 1;
+  plan.units_per_split = (plan.units + splits - 1) / splits;
+  plan.splits = (plan.units + plan.units_per_split - 1) / plan.units_per_split;
+  return plan;
+}
+
+template <typename ACT, typename T, int MB, bool HAS_ZP>
+void launch_a8_mb(const A8Params& p, bool grouped, dim3 grid, hipStream_t st) {
+  if (grouped) marlin_a8_kernel<ACT, T, MB, HAS_ZP, true><<<grid, 256, 0, st>>>(p);
+  else marlin_a8_kernel<ACT, T, MB, HAS_ZP, false><<<grid, 256, 0, st>>>(p);
+}
+
+template <typename ACT, typename T>
+void launch_a8(const A8Params& p, const A8Plan& plan, bool grouped, hipStream_t st) {
+  const dim3 grid(p.n / kStripN, plan.slabs, plan.splits);
+  const bool zp = p.zeros != nullptr;
+#define SONAR_A8_CASE(MB)                                             \
+  case MB:                                                            \
+    if (zp) launch_a8_mb<ACT, T, MB, true>(p, grouped, grid, st);     \
+    else launch_a8_mb<ACT, T, MB, false>(p, grouped, grid, st);       \
+    break;
+  switch (plan.mb) {
+    SONAR_A8_CASE(1)
+    SONAR_A8_CASE(2)
+    SONAR_A8_CASE(3)
+    SONAR_A8_CASE(4)
+  }
+#undef SONAR_A8_CASE
+  if (plan.splits > 1) {
+    long blocks = ((long)p.m * p.n + 255) / 256;
+    if (blocks > 4096) blocks = 4096;
+    if (grouped) marlin_a8_finish_kernel<ACT, T, true><<<(int)blocks, 256, 0, st>>>(p);
+    else marlin_a8_finish_kernel<ACT, T, false><<<(int)blocks, 256, 0, st>>>(p);
+  }
+}
+
+}  // namespace
+}  // namespace sonar
+
+using namespace sonar;
+
+extern "C" size_t sonar_marlin_gemm_a8_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k,
+                                                     int64_t num_groups) {
+  if (size_m <= 0 || size_n <= 0 || size_k < kChunkK || num_groups < 1) return 0;
+  const A8Plan plan = plan_a8(size_m, size_n, size_k, num_groups);
+  return plan.splits > 1 ? (size_t)plan.splits * size_m * size_n * 4 : 0;
+}
+
+extern "C" int sonar_marlin_gemm_a8(const void* a, int64_t a_row_stride, int a_dtype, void* c, const uint32_t* b_q_weight,
+                                    int b_layout, const void* b_bias, const void* b_scales, const float* a_scales,
+                                    const uint32_t* b_zeros, void* scratch, size_t scratch_bytes, int dtype,
+                                    int64_t b_type_id, int64_t size_m, int64_t size_n, int64_t size_k,
+                                    int64_t num_groups, void* stream) {
+  SONAR_REQUIRE(b_layout == SONAR_LAYOUT_GFX950, "unknown b_layout = %d", b_layout);
+  SONAR_REQUIRE(a_dtype == SONAR_ADTYPE_INT8 || a_dtype == SONAR_ADTYPE_FP8, "unknown a_dtype = %d", a_dtype);
+  SONAR_REQUIRE(dtype == SONAR_DTYPE_F16 || dtype == SONAR_DTYPE_BF16, "unknown dtype = %d", dtype);
+  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4)
+    return fail(SONAR_E_UNSUPPORTED, "8-bit activations are built for b_type uint4b8 and uint4 only (W8A8 is not "
+                "supported by the marlin kernel; float4_e2m1f weights with fp8 activations are not built)");
+  SONAR_REQUIRE(size_m >= 0 && size_n > 0 && size_k > 0, "size_m = %ld, size_n = %ld, size_k = %ld", (long)size_m,
+                (long)size_n, (long)size_k);
+  SONAR_REQUIRE(size_n % kStripN == 0, "size_n = %ld is not divisible by %d", (long)size_n, kStripN);
+  SONAR_REQUIRE(size_k % kChunkK == 0, "size_k = %ld is not divisible by %d", (long)size_k, kChunkK);
+  SONAR_REQUIRE(size_m < (1LL << 30) && size_n < (1LL << 30) && size_k < (1LL << 30), "sizes too large");
+  SONAR_REQUIRE(num_groups >= 1 && size_k % num_groups == 0, "size_k = %ld is not divisible by num_groups = %ld",
+                (long)size_k, (long)num_groups);
+  const int64_t group_size = size_k / num_groups;
+  if (num_groups > 1)
+    SONAR_REQUIRE(group_size == 32 || group_size == 64 || group_size == 128,
+                  "Invalid group_size = %ld: 8-bit activations take -1, 32, 64 or 128", (long)group_size);
+  SONAR_REQUIRE((b_zeros != nullptr) == (b_type_id == SONAR_TYPE_UINT4),
+                "b_zeros must be given for uint4 weights and only for them");
+  if (size_m == 0) return SONAR_OK;
+  SONAR_REQUIRE(a && c && b_q_weight && b_scales && a_scales, "a, c, b_q_weight, b_scales and a_scales must not be NULL");
+  SONAR_REQUIRE(a_row_stride >= size_k && a_row_stride % 8 == 0, "A.stride(0) = %ld must be at least size_k and "
+                "divisible by 8", (long)a_row_stride);
+  SONAR_REQUIRE((uintptr_t)a % 16 == 0, "A must aligned to 16 bytes");
+
+  const A8Plan plan = plan_a8(size_m, size_n, size_k, num_groups);
+  A8Params p;
+  p.a = (const uint8_t*)a;
+  p.a_row_stride = a_row_stride;
+  p.c = c;
+  p.w = b_q_weight;
+  p.scales = (const uint16_t*)b_scales;
+  p.zeros = b_zeros;
+  p.a_scales = a_scales;
+  p.bias = (const uint16_t*)b_bias;
+  p.partial = (uint32_t*)scratch;
+  p.m = (int)size_m;
+  p.n = (int)size_n;
+  p.chunks = (int)(size_k / kChunkK);
+  p.unit_chunks = plan.unit_chunks;
+  p.units = plan.units;
+  p.units_per_split = plan.units_per_split;
+  p.splits = plan.splits;
+  if (plan.splits > 1)
+    SONAR_REQUIRE(scratch && scratch_bytes >= (size_t)plan.splits * size_m * size_n * 4,
+                  "scratch of %zu bytes is too small: sonar_marlin_gemm_a8_scratch_bytes() = %zu", scratch_bytes,
+                  (size_t)plan.splits * size_m * size_n * 4);
+  const bool grouped = num_groups > 1;
+  hipStream_t st = (hipStream_t)stream;
+  if (a_dtype == SONAR_ADTYPE_INT8) {
+    if (dtype == SONAR_DTYPE_F16) launch_a8<ActInt8, _Float16>(p, plan, grouped, st);
+    else launch_a8<ActInt8, __bf16>(p, plan, grouped, st);
+  } else {
+    if (dtype == SONAR_DTYPE_F16) launch_a8<ActFp8, _Float16>(p, plan, grouped, st);
+    else launch_a8<ActFp8, __bf16>(p, plan, grouped, st);
+  }
+  return launch_status("marlin_a8_kernel");
+}

@@ -245,6 +245,107 @@ __global__ __launch_bounds__(256) void marlin8_gfx950_kernel(const uint32_t* __r
   }
 }
 
+// ---- 4-bit codes for 8-bit activations (is_a_8bit): tiles of 32 (k) x 32 (n),
+// 128 words each, tile (kt, nt) at (kt * (N / 32) + nt) * 128.  Word lane*4 + w:
+// column 8w + lane/4; nibble slot s holds row 4*(lane%4) + s/2 + 16*(s%2)
+// (gptq_marlin_repack.cu:129-141,176-216).
+constexpr int kA8Tile = 32;
+
+__device__ __forceinline__ void a8_word_sources(int word, int slot, int& row, int& col) {
+  const int lane = word >> 2;
+  row = 4 * (lane & 3) + (slot >> 1) + 16 * (slot & 1);
+  col = 8 * (word & 3) + (lane >> 2);
+}
+
+// Word index and nibble slot of W[k][n] in that order.
+__device__ __forceinline__ long a8_position(int k, int n, int n_tiles, int& slot) {
+  const int r = k % kA8Tile, c = n % kA8Tile;
+  slot = 2 * (r & 3) + (r >> 4);
+  return ((long)(k / kA8Tile) * n_tiles + n / kA8Tile) * kMarlinTileWords + (4 * (c & 7) + ((r & 15) >> 2)) * 4 +
+         (c >> 3);
+}
+
+// SOURCE 0: GPTQ (K/8, N) words; 1: AWQ (K, N/8) words; 2: the gfx950 order.
+template <int SOURCE>
+__global__ __launch_bounds__(256) void to_marlin_a8_kernel(const uint32_t* __restrict__ in,
+                                                          uint32_t* __restrict__ out, int size_k, int size_n,
+                                                          long total_words) {
+  const int n_tiles = size_n / kA8Tile;
+  const int chunks = size_k / kChunkK;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_words;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long tile = idx / kMarlinTileWords;
+    const int word = (int)(idx % kMarlinTileWords);
+    uint32_t packed = 0;
+#pragma unroll
+    for (int slot = 0; slot < 8; ++slot) {
+      int row, col;
+      a8_word_sources(word, slot, row, col);
+      const int k = (int)(tile / n_tiles) * kA8Tile + row;
+      const int n = (int)(tile % n_tiles) * kA8Tile + col;
+      uint32_t code;
+      if (SOURCE == 0) {
+        code = in[(long)(k >> 3) * size_n + n] >> (4 * (k & 7));
+      } else if (SOURCE == 1) {
+        const int p = ((n & 7) >> 1) + 4 * (n & 1);
+        code = in[(long)k * (size_n / 8) + (n >> 3)] >> (4 * p);
+      } else {
+        const int t = k & 7;
+        const int lane = 16 * ((k % kChunkK) >> 3) + (n & 15);
+        code = in[(((long)(n / kStripN) * chunks + k / kChunkK) * 64 + lane) * 4 + ((n % kStripN) >> 4)] >>
+               (4 * ((t >> 1) + 4 * (t & 1)));
+      }
+      packed |= (code & 0xFu) << (4 * slot);
+    }
+    out[idx] = packed;
+  }
+}
+
+// One thread per gfx950 word (rows 32c + 8*(L/16) + t of column 64s + 16j + L%16).
+__global__ __launch_bounds__(256) void marlin_a8_to_gfx950_kernel(const uint32_t* __restrict__ in,
+                                                                 uint32_t* __restrict__ out, int size_k,
+                                                                 int size_n, long total_words) {
+  const int n_tiles = size_n / kA8Tile;
+  const int chunks = size_k / kChunkK;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_words;
+       idx += (long)gridDim.x * blockDim.x) {
+    const int j = (int)(idx & 3);
+    const int lane = (int)((idx >> 2) & 63);
+    const long chunk_id = idx >> 8;
+    const int n = (int)(chunk_id / chunks) * kStripN + 16 * j + (lane & 15);
+    const int k0 = (int)(chunk_id % chunks) * kChunkK + 8 * (lane >> 4);
+    uint32_t packed = 0;
+#pragma unroll
+    for (int t = 0; t < 8; ++t) {
+      int slot;
+      const long src = a8_position(k0 + t, n, n_tiles, slot);
+      packed |= ((in[src] >> (4 * slot)) & 0xFu) << (4 * ((t >> 1) + 4 * (t & 1)));
+    }
+    out[idx] = packed;
+  }
+}
+
+// marlin_int4_fp8_preprocess.cu:13-66: nibble by nibble, code -> sign and
+// magnitude of code - z (z = 8 without zero points): q >= z ? q - z : 15 - q.
+__global__ __launch_bounds__(256) void int4_fp8_preprocess_kernel(const uint32_t* __restrict__ in,
+                                                                 const uint32_t* __restrict__ zeros,
+                                                                 uint32_t* __restrict__ out, long words_per_row,
+                                                                 int group_size, long total_words) {
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_words;
+       idx += (long)gridDim.x * blockDim.x) {
+    uint32_t val = in[idx];
+    uint32_t zero = zeros ? zeros[(idx / words_per_row) / group_size * words_per_row + idx % words_per_row]
+                          : 0x88888888u;
+    uint32_t res = 0;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const uint32_t q = (val >> (4 * i)) & 0xFu, z = (zero >> (4 * i)) & 0xFu;
+      res |= (q >= z ? q - z : 15u - q) << (4 * i);
+    }
+    out[idx] = res;
+  }
+}
+
 int grid_for(long total_words) {
   long blocks = (total_words + 255) / 256;
   if (blocks > 256L * 32) blocks = 256L * 32;
@@ -352,4 +453,77 @@ extern "C" int sonar_gfx950_to_marlin8(const uint32_t* gfx950, uint32_t* out, in
   marlin8_gfx950_kernel<false><<<grid_for(total), 256, 0, (hipStream_t)stream>>>(gfx950, out, (int)size_k,
                                                                                 (int)size_n, total);
   return launch_status("marlin8_gfx950_kernel");
+}
+
+// ---- the weight order for 8-bit activations --------------------------------
+namespace {
+int check_a8_shape(int64_t size_k, int64_t size_n, int num_bits) {
+  if (int rc = check_repack_shape(size_k, size_n, num_bits)) return rc;
+  if (num_bits != 4)
+    return fail(SONAR_E_UNSUPPORTED, "Unsupported repack config: num_bits = %d with is_a_8bit (the GEMM has no "
+                "8-bit weights with 8-bit activations)", num_bits);
+  SONAR_REQUIRE(size_k % kA8Tile == 0, "size_k = %ld is not divisible by %d (the tile of 8-bit activations)",
+                (long)size_k, kA8Tile);
+  return SONAR_OK;
+}
+}  // namespace
+
+extern "C" int sonar_gptq_marlin_repack_a8(const uint32_t* b_q_weight, uint32_t* out, int64_t size_k,
+                                           int64_t size_n, int num_bits, void* stream) {
+  if (int rc = check_a8_shape(size_k, size_n, num_bits)) return rc;
+  SONAR_REQUIRE(b_q_weight && out, "b_q_weight and out must not be NULL");
+  const long total = size_k * size_n / 8;
+  to_marlin_a8_kernel<0><<<grid_for(total), 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k,
+                                                                          (int)size_n, total);
+  return launch_status("to_marlin_a8_kernel");
+}
+
+extern "C" int sonar_awq_marlin_repack_a8(const uint32_t* b_q_weight, uint32_t* out, int64_t size_k,
+                                          int64_t size_n, int num_bits, void* stream) {
+  if (int rc = check_a8_shape(size_k, size_n, num_bits)) return rc;
+  SONAR_REQUIRE(b_q_weight && out, "b_q_weight and out must not be NULL");
+  const long total = size_k * size_n / 8;
+  to_marlin_a8_kernel<1><<<grid_for(total), 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k,
+                                                                          (int)size_n, total);
+  return launch_status("to_marlin_a8_kernel");
+}
+
+extern "C" int sonar_marlin_a8_to_gfx950(const uint32_t* marlin, uint32_t* out, int64_t size_k, int64_t size_n,
+                                         void* stream) {
+  if (int rc = check_a8_shape(size_k, size_n, 4)) return rc;
+  SONAR_REQUIRE(marlin && out && marlin != out, "marlin and out must be distinct non-NULL buffers");
+  const long total = size_k * size_n / 8;
+  marlin_a8_to_gfx950_kernel<<<grid_for(total), 256, 0, (hipStream_t)stream>>>(marlin, out, (int)size_k,
+                                                                              (int)size_n, total);
+  return launch_status("marlin_a8_to_gfx950_kernel");
+}
+
+extern "C" int sonar_gfx950_to_marlin_a8(const uint32_t* gfx950, uint32_t* out, int64_t size_k, int64_t size_n,
+                                         void* stream) {
+  if (int rc = check_a8_shape(size_k, size_n, 4)) return rc;
+  SONAR_REQUIRE(gfx950 && out && gfx950 != out, "gfx950 and out must be distinct non-NULL buffers");
+  const long total = size_k * size_n / 8;
+  to_marlin_a8_kernel<2><<<grid_for(total), 256, 0, (hipStream_t)stream>>>(gfx950, out, (int)size_k,
+                                                                          (int)size_n, total);
+  return launch_status("to_marlin_a8_kernel");
+}
+
+extern "C" int sonar_marlin_int4_fp8_preprocess(const uint32_t* qweight, const uint32_t* qzeros, uint32_t* out,
+                                                int64_t rows, int64_t words_per_row, int64_t group_size,
+                                                void* stream) {
+  SONAR_REQUIRE(qweight && out, "qweight and out must not be NULL");
+  SONAR_REQUIRE(rows > 0 && words_per_row > 0, "rows = %ld and words_per_row = %ld must be positive", (long)rows,
+                (long)words_per_row);
+  if (qzeros) {
+    SONAR_REQUIRE(rows % 32 == 0, "size_k % 32 != 0");
+    SONAR_REQUIRE(group_size > 0 && rows % group_size == 0, "qweight.size(0) % qzeros.size(0) != 0");
+    SONAR_REQUIRE(group_size % 8 == 0, "group_size % 8 != 0");
+  } else {
+    SONAR_REQUIRE(rows * words_per_row * 8 % 256 == 0, "qweight.numel() * 8 % 256 != 0");
+    group_size = 1;
+  }
+  const long total = rows * words_per_row;
+  int4_fp8_preprocess_kernel<<<grid_for(total), 256, 0, (hipStream_t)stream>>>(qweight, qzeros, out, words_per_row,
+                                                                              (int)group_size, total);
+  return launch_status("int4_fp8_preprocess_kernel");
 }

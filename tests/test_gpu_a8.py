@@ -1,0 +1,201 @@
+"""W4A8 through the C ABI against the CPU oracle: the weight order for 8-bit
+activations and the fp8 preprocess bit for bit, the int8 GEMM bit for bit
+(integer sums, one rounding), the fp8 GEMM within the tolerance of the other
+floating-point paths (1e-2 of max|ref|)."""
+import ctypes
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import marlin_oracle as mo
+from sonar_amd import _lib
+from tests.gpu_util import DEV, dev_bits16, dev_i32, host_f32, ptr, stream, dtype_code
+
+pytestmark = pytest.mark.gpu
+
+
+def _repack_a8(words, k, n, awq=False):
+    lib = _lib.load()
+    out = torch.empty((k // 16, 2 * n), dtype=torch.int32, device=DEV)
+    fn = lib.sonar_awq_marlin_repack_a8 if awq else lib.sonar_gptq_marlin_repack_a8
+    _lib.check(fn(ptr(words), ptr(out), k, n, 4, stream()))
+    return out
+
+
+def _a8_to_gfx950(marlin, k, n):
+    out = torch.empty(k * n // 8, dtype=torch.int32, device=DEV)
+    _lib.check(_lib.load().sonar_marlin_a8_to_gfx950(ptr(marlin), ptr(out), k, n, stream()))
+    return out
+
+
+# sizes of the reference's repack test: K = 128 * k_factor, N = 64 / 256 * n_factor
+# (tests/kernels/quantization/test_marlin_gemm.py:58-66,196-247)
+@pytest.mark.parametrize("k,n", [(128 * 8, 64 * 4), (128 * 5, 256 * 7), (128 * 11, 64 * 13), (32, 64)])
+def test_repack_a8_bit_exact(k, n):
+    rng = np.random.default_rng(k + n)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    want = mo.marlin_pack_a8(q)
+    got = _repack_a8(dev_i32(mo.gptq_pack(q)), k, n)
+    assert np.array_equal(got.cpu().numpy(), want)
+    got_awq = _repack_a8(dev_i32(mo.awq_pack(q)), k, n, awq=True)
+    assert np.array_equal(got_awq.cpu().numpy(), want)
+    native = _a8_to_gfx950(got, k, n)
+    assert np.array_equal(native.cpu().numpy(), mo.gfx950_pack(q))
+    back = torch.empty_like(got)
+    _lib.check(_lib.load().sonar_gfx950_to_marlin_a8(ptr(native), ptr(back), k, n, stream()))
+    assert torch.equal(back, got)
+
+
+def test_repack_a8_rejections():
+    lib = _lib.load()
+    w = torch.zeros(64 * 64 // 4, dtype=torch.int32, device=DEV)
+    out = torch.zeros(64 * 64 // 4, dtype=torch.int32, device=DEV)
+    assert lib.sonar_gptq_marlin_repack_a8(ptr(w), ptr(out), 64, 64, 8, stream()) == _lib.E_UNSUPPORTED
+    assert lib.sonar_gptq_marlin_repack_a8(ptr(w), ptr(out), 48, 64, 4, stream()) == _lib.E_INVALID
+    assert b"32" in lib.sonar_marlin_last_error()
+    assert lib.sonar_awq_marlin_repack_a8(ptr(w), ptr(out), 64, 32, 4, stream()) == _lib.E_INVALID
+
+
+def test_int4_fp8_preprocess_bit_exact():
+    lib = _lib.load()
+    rng = np.random.default_rng(11)
+    k, n, gs = 256, 128, 64
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    # without zero points: any packing (here the Marlin order for 8-bit activations)
+    packed = mo.marlin_pack_a8(q)
+    d = dev_i32(packed)
+    out = torch.empty_like(d)
+    _lib.check(lib.sonar_marlin_int4_fp8_preprocess(ptr(d), None, ptr(out), d.shape[0], d.shape[1], 0, stream()))
+    assert np.array_equal(out.cpu().numpy(), mo.marlin_pack_a8(mo.int4_fp8_preprocess(q)))
+    _lib.check(lib.sonar_marlin_int4_fp8_preprocess(ptr(d), None, ptr(d), d.shape[0], d.shape[1], 0, stream()))
+    assert torch.equal(d, out)                      # in place
+    # AWQ: qweight (K, N/8) and qzeros (K/group, N/8) in the checkpoint's packing
+    z = rng.integers(0, 16, size=(k // gs, n), dtype=np.int32)
+    dq, dz = dev_i32(mo.awq_pack(q)), dev_i32(mo.awq_pack(z))
+    out = torch.empty_like(dq)
+    _lib.check(lib.sonar_marlin_int4_fp8_preprocess(ptr(dq), ptr(dz), ptr(out), k, n // 8, gs, stream()))
+    assert np.array_equal(out.cpu().numpy(), mo.awq_pack(mo.int4_fp8_preprocess(q, z, gs)))
+
+
+class A8Layer:
+    def __init__(self, seed, k, n, group_size, dtype, zero_points, act, bias=False):
+        rng = np.random.default_rng(seed)
+        self.k, self.n, self.dtype, self.act, self.group_size = k, n, dtype, act, group_size
+        self.q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+        self.groups = 1 if group_size == -1 else k // group_size
+        self.zeros = rng.integers(0, 16, size=(self.groups, n), dtype=np.int32) if zero_points else None
+        s = mo.round_to_dtype(rng.uniform(1e-3, 1e-2, size=(self.groups, n)).astype(np.float32), dtype)
+        self.factor = np.float32(1.0)
+        if act == "int8" and self.groups > 1:
+            ints, self.factor = mo.marlin_act_int8_process_scales(s)
+            self.scales = ints
+            dev_s = torch.from_numpy(mo.marlin_permute_scales_a8(ints, k, n, group_size).copy()).to(DEV)
+        else:
+            if act == "fp8":
+                s = mo.round_to_dtype(s * np.float32(512.0), dtype)   # the factor of the fp8 weights
+            self.scales = s
+            dev_s = dev_bits16(mo.marlin_permute_scales_a8(s, k, n, group_size), dtype)
+        self.dev_scales = dev_s
+        codes = self.q
+        if act == "fp8":
+            codes = mo.int4_fp8_preprocess(self.q, self.zeros, k // self.groups)
+        self.native = _a8_to_gfx950(_repack_a8(dev_i32(mo.gptq_pack(codes)), k, n), k, n)
+        self.dev_zeros = dev_i32(mo.marlin_zero_points_a8(self.zeros, self.groups, n)) if zero_points else None
+        self.bias32, self.dev_bias = None, None
+        if bias:
+            self.bias32 = mo.round_to_dtype(rng.standard_normal(n).astype(np.float32), dtype)
+            self.dev_bias = dev_bits16(mo.marlin_permute_bias(self.bias32), dtype)
+        self.b_type = _lib.TYPE_UINT4 if zero_points else _lib.TYPE_UINT4B8
+
+    def gemm(self, a_dev, a_scales_dev, m):
+        lib = _lib.load()
+        tdt = torch.float16 if self.dtype == "fp16" else torch.bfloat16
+        c = torch.full((m, self.n), float("nan"), dtype=tdt, device=DEV)
+        nbytes = lib.sonar_marlin_gemm_a8_scratch_bytes(m, self.n, self.k, self.groups)
+        scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=DEV)
+        _lib.check(lib.sonar_marlin_gemm_a8(
+            ptr(a_dev), a_dev.stride(0) if m else self.k, _lib.ADTYPE_INT8 if self.act == "int8" else _lib.ADTYPE_FP8,
+            ptr(c), ptr(self.native), _lib.LAYOUT_GFX950, ptr(self.dev_bias), ptr(self.dev_scales),
+            ptr(a_scales_dev), ptr(self.dev_zeros), ptr(scratch), scratch.numel(), dtype_code(self.dtype),
+            self.b_type, m, self.n, self.k, self.groups, stream()))
+        return c
+
+
+INT8_CASES = [
+    # k, n, group, zp, dtype, bias, M list
+    (256, 128, -1, False, "fp16", False, [1, 16, 33]),
+    (256, 128, 32, False, "bf16", True, [7, 64]),
+    (1024, 256, 64, False, "fp16", False, [1, 100]),
+    (1024, 256, 128, False, "bf16", False, [5, 257]),
+    (512, 192, -1, True, "bf16", True, [3, 48]),
+    (512, 192, 32, True, "fp16", False, [17, 65]),
+    (1024, 64, 64, True, "bf16", False, [2]),
+    (8192, 64, 128, False, "fp16", True, [1, 20]),     # K split over workgroups
+    (4096, 128, -1, False, "bf16", False, [9]),         # channelwise, K split
+    (1056, 128, -1, False, "fp16", False, [4]),         # K a multiple of 32 only
+]
+
+
+@pytest.mark.parametrize("k,n,group,zp,dtype,bias,ms", INT8_CASES)
+def test_w4a8_int8_gemm_bit_exact(k, n, group, zp, dtype, bias, ms):
+    layer = A8Layer(100 + k + n + group, k, n, group, dtype, zp, "int8", bias)
+    for m in ms:
+        rng = np.random.default_rng(m)
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        a_q, a_s = mo.per_token_quant_int8(x)
+        a_s = (a_s * layer.factor).astype(np.float32)
+        got = layer.gemm(torch.from_numpy(a_q).to(DEV), torch.from_numpy(a_s.reshape(-1)).to(DEV), m)
+        want = mo.gemm_w4a8_int8(a_q, a_s, layer.q, group, layer.scales, dtype, layer.zeros, layer.bias32)
+        assert np.array_equal(host_f32(got), want), (m, np.abs(host_f32(got) - want).max())
+
+
+FP8_CASES = [
+    (256, 128, -1, False, "fp16", False, [1, 16]),
+    (512, 128, 32, False, "bf16", True, [7, 64]),
+    (1024, 256, 64, False, "fp16", False, [33]),
+    (1024, 256, 128, False, "bf16", False, [100]),
+    (512, 192, 64, True, "fp16", False, [5, 40]),
+    (512, 64, -1, True, "bf16", True, [2]),
+    (8192, 64, 128, False, "bf16", False, [3]),
+]
+
+
+@pytest.mark.parametrize("k,n,group,zp,dtype,bias,ms", FP8_CASES)
+def test_w4a8_fp8_gemm_within_tolerance(k, n, group, zp, dtype, bias, ms):
+    layer = A8Layer(200 + k + n + group, k, n, group, dtype, zp, "fp8", bias)
+    for m in ms:
+        g = torch.Generator().manual_seed(m)
+        x = torch.randn((m, k), generator=g)
+        a_s = (x.abs().amax(dim=1, keepdim=True) / 448.0).clamp_min(1e-10)
+        a_fp8 = (x / a_s).to(torch.float8_e4m3fn)
+        got = layer.gemm(a_fp8.view(torch.uint8).to(DEV), a_s.reshape(-1).to(DEV), m)
+        # the scales as the kernel holds them (times 512), the weights as (q - z) * 2^-9
+        want = mo.gemm_w4a8_fp8(a_fp8.float().numpy(), a_s.numpy(), layer.q, group,
+                                layer.scales / np.float32(512.0), layer.zeros, layer.bias32)
+        ok, max_err, max_ref = mo.gemm_tolerance_ok(host_f32(got), want)
+        assert ok, (m, max_err, max_ref)
+
+
+def test_w4a8_rejections():
+    lib = _lib.load()
+    layer = A8Layer(1, 256, 64, 64, "fp16", False, "int8")
+    a = torch.zeros((4, 256), dtype=torch.int8, device=DEV)
+    s = torch.ones(4, device=DEV)
+    c = torch.empty((4, 64), dtype=torch.float16, device=DEV)
+
+    def call(**kw):
+        args = dict(a=a, stride=256, adt=_lib.ADTYPE_INT8, b_type=_lib.TYPE_UINT4B8, zeros=None, groups=4, k=256)
+        args.update(kw)
+        return lib.sonar_marlin_gemm_a8(ptr(args["a"]), args["stride"], args["adt"], ptr(c), ptr(layer.native),
+                                        _lib.LAYOUT_GFX950, None, ptr(layer.dev_scales), ptr(s), ptr(args["zeros"]),
+                                        None, 0, _lib.DTYPE_F16, args["b_type"], 4, 64, args["k"], args["groups"],
+                                        stream())
+
+    assert call() == _lib.OK
+    assert call(b_type=_lib.TYPE_UINT8B128) == _lib.E_UNSUPPORTED      # W8A8 is not a Marlin mode
+    assert call(adt=7) == _lib.E_INVALID
+    assert call(groups=16) == _lib.E_INVALID                           # group size 16
+    assert call(b_type=_lib.TYPE_UINT4) == _lib.E_INVALID              # zero points missing
+    assert call(stride=260) == _lib.E_INVALID
+    assert call(a=None) == _lib.E_INVALID
