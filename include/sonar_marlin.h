@@ -24,6 +24,9 @@
  *        a_scales (marlin.cu:567-598,666-679; marlin_template.h:1302-1400,1869-1903)
  *   sonar_gptq_marlin_repack_a8 / sonar_awq_marlin_repack_a8 -> the repack ops with is_a_8bit
  *        (gptq_marlin_repack.cu:14-268, awq_marlin_repack.cu:14-212)
+ *   sonar_per_token_quant_int8 / _fp8 -> per_token_quant_int8 (a Triton kernel in the reference,
+ *        layers/quantization/utils/int8_utils.py:70-120) and QuantFP8 per token
+ *        (layers/quantization/input_quant_fp8.py:188-204), which marlin_quant_input calls
  *   sonar_marlin_int4_fp8_preprocess -> _C::marlin_int4_fp8_preprocess
  *        csrc/libtorch_stable/quantization/marlin/marlin_int4_fp8_preprocess.cu:13-121
  *   sonar_moe_wna16_marlin_gemm -> _moe_C::moe_wna16_marlin_gemm
@@ -52,6 +55,7 @@ extern "C" {
 /* activation / output / scale element types */
 #define SONAR_DTYPE_F16 0
 #define SONAR_DTYPE_BF16 1
+#define SONAR_DTYPE_F32 2          /* input of the per-token quantisers only */
 
 /* 8-bit activation types of sonar_marlin_gemm_a8 */
 #define SONAR_ADTYPE_INT8 0
@@ -186,6 +190,17 @@ int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                       int64_t size_m, int64_t size_n, int64_t size_k,
                       int64_t num_groups, int is_k_full, int use_atomic_add,
                       int use_fp32_reduce, void* stream);
+
+/* Per-token quantisation of the activations for sonar_marlin_gemm_a8: one fp32 scale per row.
+ * int8 (per_token_quant_int8, layers/quantization/utils/int8_utils.py:70-120): scale =
+ * max(absmax, 1e-10) / 127, code = x * (127 / absmax) rounded half away from zero.
+ * fp8 (QuantFP8 per token, layers/quantization/input_quant_fp8.py:188-204): scale =
+ * max(absmax / 448, 1 / (448 * 512)), code = float8_e4m3fn(clamp(x * (1 / scale), -448, 448)).
+ *   x   dtype[rows][row_stride] (SONAR_DTYPE_F16, _BF16 or _F32); q [rows][cols]; scales float[rows] */
+int sonar_per_token_quant_int8(const void* x, int dtype, int64_t row_stride, int8_t* q,
+                               float* scales, int64_t rows, int64_t cols, void* stream);
+int sonar_per_token_quant_fp8(const void* x, int dtype, int64_t row_stride, uint8_t* q,
+                              float* scales, int64_t rows, int64_t cols, void* stream);
 
 /* W4A8 (marlin.cu:567-598,666-679 of the reference; marlin_template.h:1302-1400,1869-1903,
  * 1955-1978): 4-bit weights, 8-bit activations with one fp32 scale per row, on the 8-bit matrix

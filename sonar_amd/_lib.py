@@ -12,6 +12,7 @@ _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "lib
 
 DTYPE_F16 = 0
 DTYPE_BF16 = 1
+DTYPE_F32 = 2
 LAYOUT_GFX950 = 0
 ADTYPE_INT8 = 0
 ADTYPE_FP8 = 1
@@ -41,6 +42,8 @@ PROTOTYPES = {
     "sonar_marlin_a8_to_gfx950": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "sonar_gfx950_to_marlin_a8": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "sonar_marlin_int4_fp8_preprocess": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int64, c_void_p]),
+    "sonar_per_token_quant_int8": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
+    "sonar_per_token_quant_fp8": (c_int, [c_void_p, c_int, c_int64, c_void_p, c_void_p, c_int64, c_int64, c_void_p]),
     "sonar_marlin_gemm_a8_scratch_bytes": (c_size_t, [c_int64, c_int64, c_int64, c_int64]),
     "sonar_marlin_gemm_a8": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int64, c_int64, c_int64,

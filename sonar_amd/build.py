@@ -16,7 +16,7 @@ OPS_PATH = os.path.join(LIB_DIR, "libsonar_marlin_torch.so")
 BENCH_PATH = os.path.join(LIB_DIR, "libsonar_bench.so")   # bench.py's yardstick kernels, not part of the product
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 
-HIP_SOURCES = ["repack.hip", "gemm_stream.hip", "gemm_tile.hip", "gemm_moe.hip", "moe_aux.hip", "gemm_a8.hip"]
+HIP_SOURCES = ["repack.hip", "gemm_stream.hip", "gemm_tile.hip", "gemm_moe.hip", "moe_aux.hip", "gemm_a8.hip", "quant_input.hip"]
 HIP_FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fno-gpu-rdc",
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",

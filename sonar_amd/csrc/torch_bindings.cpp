@@ -33,9 +33,11 @@
 #include <ATen/hip/impl/HIPStreamMasqueradingAsCUDA.h>
 #include <torch/library.h>
 
+#include <algorithm>
 #include <iterator>
 #include <mutex>
 #include <optional>
+#include <tuple>
 #include <unordered_map>
 
 #include "sonar_marlin.h"
@@ -158,15 +160,18 @@ void evict_stale_locked(const Tensor& t, const void* key) {
 }
 
 // b_q_weight: (K/16, 2N) or (E, K/16, 2N) int32 in Marlin order; (K/16, 4N) for 8-bit codes.
-Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, int64_t experts, int bits = 4) {
+// `a8`: the 4-bit order of 8-bit activations (32 x 32 tiles).
+Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, int64_t experts, int bits = 4,
+                      bool a8 = false) {
   const void* key = b_q_weight.const_data_ptr();
   hipStream_t stream = (hipStream_t)current_stream(b_q_weight);
+  const int64_t key_k = a8 ? -1000 - size_k : size_k;   // the cache entry says which order it was converted from
   {
     std::lock_guard<std::mutex> lock(g_cache_mutex);
     auto it = g_cache.find(key);
     if (it != g_cache.end() && !it->second.source.expired() &&
         it->second.source._unsafe_get_target() == b_q_weight.unsafeGetTensorImpl() &&
-        it->second.size_k == size_k && it->second.size_n == size_n && it->second.experts == experts &&
+        it->second.size_k == key_k && it->second.size_n == size_n && it->second.experts == experts &&
         it->second.version == version_of(b_q_weight)) {
       wait_for_conversion(it->second, stream);
       return it->second.native;
@@ -178,14 +183,16 @@ Tensor native_weights(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, 
   const uint32_t* src = static_cast<const uint32_t*>(b_q_weight.const_data_ptr());
   uint32_t* dst = static_cast<uint32_t*>(native.mutable_data_ptr());
   for (int64_t e = 0; e < experts; ++e)
-    raise_if_failed(bits == 8 ? sonar_marlin8_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
-                                                        current_stream(b_q_weight))
-                              : sonar_marlin_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
-                                                       current_stream(b_q_weight)));
+    raise_if_failed(a8        ? sonar_marlin_a8_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
+                                                          current_stream(b_q_weight))
+                    : bits == 8 ? sonar_marlin8_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
+                                                          current_stream(b_q_weight))
+                                : sonar_marlin_to_gfx950(src + e * words, dst + e * words, size_k, size_n,
+                                                         current_stream(b_q_weight)));
   std::lock_guard<std::mutex> lock(g_cache_mutex);
   evict_stale_locked(b_q_weight, key);
   invalidate_range_locked(key, b_q_weight.nbytes());
-  NativeEntry entry{c10::weak_intrusive_ptr<c10::TensorImpl>(b_q_weight.getIntrusivePtr()), native, size_k, size_n,
+  NativeEntry entry{c10::weak_intrusive_ptr<c10::TensorImpl>(b_q_weight.getIntrusivePtr()), native, key_k, size_n,
                     experts, version_of(b_q_weight), b_q_weight.nbytes(), stream, nullptr};
   record_conversion(entry, stream);
   g_cache.insert_or_assign(key, entry);
@@ -302,7 +309,6 @@ const void* opt_ptr(const OptTensor& t) {
 // ---------------------------------------------------------------- repack
 Tensor gptq_marlin_repack(const Tensor& b_q_weight, const Tensor& perm, int64_t size_k,
                           int64_t size_n, int64_t num_bits, bool is_a_8bit) {
-  TORCH_CHECK_NOT_IMPLEMENTED(!is_a_8bit, "is_a_8bit = True (W4A8) is not built; activations are 16-bit");
   TORCH_CHECK(num_bits == 4 || num_bits == 8, "num_bits must be 4 or 8. Got = ", num_bits);
   const int64_t pack_factor = 32 / num_bits;
   TORCH_CHECK(size_k % 16 == 0, "size_k = ", size_k, " is not divisible by tile_k_size = ", 16);
@@ -324,6 +330,16 @@ Tensor gptq_marlin_repack(const Tensor& b_q_weight, const Tensor& perm, int64_t 
 
   c10::hip::HIPGuardMasqueradingAsCUDA guard(b_q_weight.device());
   Tensor out = at::empty({size_k / 16, size_n * 16 / pack_factor}, b_q_weight.options());
+  if (is_a_8bit) {
+    // gptq_marlin_repack.cu:147 (static_assert(!is_a_8bit) under has_perm), :354-357
+    TORCH_CHECK(!has_perm, "Unsupported repack config: num_bits = ", num_bits, ", has_perm = ", has_perm,
+                ", is_a_8bit = ", is_a_8bit);
+    raise_if_failed(sonar_gptq_marlin_repack_a8(static_cast<const uint32_t*>(b_q_weight.const_data_ptr()),
+                                                static_cast<uint32_t*>(out.mutable_data_ptr()), size_k, size_n,
+                                                (int)num_bits, current_stream(b_q_weight)));
+    forget_memory_of(out);
+    return out;
+  }
   raise_if_failed(sonar_gptq_marlin_repack(
       static_cast<const uint32_t*>(b_q_weight.const_data_ptr()),
       has_perm ? static_cast<const int32_t*>(perm.const_data_ptr()) : nullptr,
@@ -335,7 +351,6 @@ Tensor gptq_marlin_repack(const Tensor& b_q_weight, const Tensor& perm, int64_t 
 
 Tensor awq_marlin_repack(const Tensor& b_q_weight, int64_t size_k, int64_t size_n, int64_t num_bits,
                          bool is_a_8bit) {
-  TORCH_CHECK_NOT_IMPLEMENTED(!is_a_8bit, "is_a_8bit = True (W4A8) is not built; activations are 16-bit");
   TORCH_CHECK(num_bits == 4 || num_bits == 8, "num_bits must be 4 or 8. Got = ", num_bits);
   const int64_t pack_factor = 32 / num_bits;
   TORCH_CHECK(size_k % 16 == 0, "size_k = ", size_k, " is not divisible by tile_k_size = ", 16);
@@ -350,9 +365,9 @@ Tensor awq_marlin_repack(const Tensor& b_q_weight, int64_t size_k, int64_t size_
 
   c10::hip::HIPGuardMasqueradingAsCUDA guard(b_q_weight.device());
   Tensor out = at::empty({size_k / 16, size_n * 16 / pack_factor}, b_q_weight.options());
-  raise_if_failed(sonar_awq_marlin_repack(static_cast<const uint32_t*>(b_q_weight.const_data_ptr()),
-                                          static_cast<uint32_t*>(out.mutable_data_ptr()), size_k,
-                                          size_n, (int)num_bits, current_stream(b_q_weight)));
+  raise_if_failed((is_a_8bit ? sonar_awq_marlin_repack_a8 : sonar_awq_marlin_repack)(
+      static_cast<const uint32_t*>(b_q_weight.const_data_ptr()), static_cast<uint32_t*>(out.mutable_data_ptr()),
+      size_k, size_n, (int)num_bits, current_stream(b_q_weight)));
   forget_memory_of(out);
   return out;
 }
@@ -370,6 +385,42 @@ Tensor marlin_to_gfx950(const Tensor& b_q_weight, int64_t size_k, int64_t size_n
   return out;
 }
 
+// marlin_int4_fp8_preprocess.cu:68-117
+Tensor marlin_int4_fp8_preprocess(const Tensor& qweight, const OptTensor& qzeros_or_none, bool inplace) {
+  TORCH_CHECK(qweight.is_cuda(), "qweight is not on GPU");
+  TORCH_CHECK(qweight.scalar_type() == at::kInt, "qweight.dtype != torch.int32");
+  TORCH_CHECK(qweight.is_contiguous(), "qweight is not contiguous");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(qweight.device());
+  Tensor output = inplace ? qweight : at::empty_like(qweight);
+  if (qweight.numel() == 0) return output;
+  if (!qzeros_or_none.has_value()) {
+    TORCH_CHECK(qweight.numel() * 8 % 256 == 0, "qweight.numel() * 8 % 256 != 0");
+    raise_if_failed(sonar_marlin_int4_fp8_preprocess(static_cast<const uint32_t*>(qweight.const_data_ptr()), nullptr,
+                                                     static_cast<uint32_t*>(output.mutable_data_ptr()),
+                                                     qweight.numel(), 1, 0, current_stream(qweight)));
+  } else {
+    const Tensor& qzeros = qzeros_or_none.value();
+    TORCH_CHECK(qweight.dim() == 2 && qzeros.dim() == 2, "qweight and qzeros must be 2-D");
+    TORCH_CHECK(qweight.size(0) % 32 == 0, "size_k % 32 != 0");
+    TORCH_CHECK(qzeros.is_cuda(), "qzeros is not on GPU");
+    TORCH_CHECK(qzeros.scalar_type() == at::kInt, "qweight.dtype != torch.int32");
+    TORCH_CHECK(qzeros.device() == qweight.device(), "qzeros is not on the same device with qweight");
+    TORCH_CHECK(qzeros.is_contiguous(), "qzeros is not contiguous");
+    TORCH_CHECK(qweight.size(1) == qzeros.size(1), "qweight.size(1) != qzeros.size(1)");
+    TORCH_CHECK(qzeros.size(0) > 0 && qweight.size(0) % qzeros.size(0) == 0,
+                "qweight.size(0) % qzeros.size(0) != 0");
+    const int64_t group_size = qweight.size(0) / qzeros.size(0);
+    TORCH_CHECK(group_size % 8 == 0, "group_size % 8 != 0");
+    raise_if_failed(sonar_marlin_int4_fp8_preprocess(static_cast<const uint32_t*>(qweight.const_data_ptr()),
+                                                     static_cast<const uint32_t*>(qzeros.const_data_ptr()),
+                                                     static_cast<uint32_t*>(output.mutable_data_ptr()),
+                                                     qweight.size(0), qweight.size(1), group_size,
+                                                     current_stream(qweight)));
+  }
+  forget_memory_of(output);
+  return output;
+}
+
 // ---------------------------------------------------------------- dense GEMM
 void check_b_type(int64_t b_type_id) {
   TORCH_CHECK_NOT_IMPLEMENTED(
@@ -380,6 +431,113 @@ void check_b_type(int64_t b_type_id) {
       "weights are supported");
 }
 
+// 8-bit activations (marlin.cu:567-598,666-679,878-882): int8 or float8_e4m3fn `a` with one fp32
+// scale per row; c takes the type of b_scales.
+Tensor marlin_gemm_a8(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_q_weight,
+                      const OptTensor& b_bias_or_none, const Tensor& b_scales, const OptTensor& a_scales,
+                      const OptTensor& global_scale, const OptTensor& b_zeros_or_none,
+                      const OptTensor& g_idx_or_none, int64_t b_type_id, int64_t size_m, int64_t size_n,
+                      int64_t size_k, bool is_zp_float) {
+  const int a_dtype = a.scalar_type() == at::kChar ? SONAR_ADTYPE_INT8 : SONAR_ADTYPE_FP8;
+  check_b_type(b_type_id);
+  TORCH_CHECK_NOT_IMPLEMENTED(b_type_id != SONAR_TYPE_FLOAT4_E2M1F,
+                              "float4_e2m1f weights with float8_e4m3fn activations (W4A8-FP4) are not built");
+  if (a_dtype == SONAR_ADTYPE_INT8) {   // marlin_utils.py:672-676
+    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4,
+                "W8A8-INT8 is not supported by marlin kernel.");
+  } else {
+    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4,
+                "INT8 weight + FP8 activation is not supported.");
+  }
+  TORCH_CHECK(b_scales.scalar_type() == at::kHalf || b_scales.scalar_type() == at::kBFloat16,
+              "b_scales must be float16 or bfloat16 with 8-bit activations (their type is the type of c)");
+  const int dtype = b_scales.scalar_type() == at::kHalf ? SONAR_DTYPE_F16 : SONAR_DTYPE_BF16;
+  TORCH_CHECK(a_scales.has_value() && a_scales->numel() > 0,
+              "the a_scales parameter must be passed for 8bit activation.");
+  TORCH_CHECK(a_scales->is_cuda() && a_scales->scalar_type() == at::kFloat, "scalar type of a_scales must be float");
+  TORCH_CHECK(a_scales->is_contiguous() && a_scales->numel() == size_m, "a_scales must hold one scale per row of a; "
+              "got ", a_scales->numel(), " for size_m = ", size_m);
+  TORCH_CHECK(!(global_scale.has_value() && global_scale->numel() > 0),
+              "global_scale can only be used for nvfp4 format.");
+  TORCH_CHECK_NOT_IMPLEMENTED(!is_zp_float, "is_zp_float = True is not built");
+  TORCH_CHECK(!(g_idx_or_none.has_value() && g_idx_or_none->numel() > 0),
+              "act-order is not supported with 8-bit activations (the reference builds no such kernel)");
+
+  TORCH_CHECK(a.dim() == 2, "a must be 2-D");
+  TORCH_CHECK(a.size(0) == size_m, "Shape mismatch: a.size(0) = ", a.size(0), ", size_m = ", size_m);
+  TORCH_CHECK(a.size(1) == size_k, "Shape mismatch: a.size(1) = ", a.size(1), ", size_k = ", size_k);
+  TORCH_CHECK(size_k % 16 == 0, "size_k = ", size_k, " is not divisible by tile_size = ", 16);
+  TORCH_CHECK(b_q_weight.dim() == 2 && size_k / 16 == b_q_weight.size(0),
+              "Shape mismatch: b_q_weight.size(0) = ", b_q_weight.size(0), ", size_k = ", size_k,
+              ", tile_size = ", 16);
+  TORCH_CHECK(b_q_weight.size(1) % 16 == 0, "b_q_weight.size(1) = ", b_q_weight.size(1),
+              " is not divisible by tile_size = ", 16);
+  const int64_t actual_size_n = b_q_weight.size(1) / 16 * 8;
+  TORCH_CHECK(size_n == actual_size_n, "size_n = ", size_n, ", actual_size_n = ", actual_size_n);
+  TORCH_CHECK(a.is_cuda(), "A is not on GPU");
+  TORCH_CHECK(size_m == 0 || a.stride(1) == 1, "A.stride(1) is not 1");
+  TORCH_CHECK(size_m == 0 || a.stride(0) % 8 == 0, "A.stride(0) must divisible by 8");
+  TORCH_CHECK(((uint64_t)a.const_data_ptr()) % 16 == 0, "A must aligned to 16 bytes");
+  TORCH_CHECK(b_q_weight.is_cuda(), "b_q_weight is not on GPU");
+  TORCH_CHECK(b_q_weight.is_contiguous(), "b_q_weight is not contiguous");
+  TORCH_CHECK(b_q_weight.scalar_type() == at::kInt, "b_q_weight type is not kInt");
+  TORCH_CHECK(b_scales.is_cuda(), "b_scales is not on GPU");
+  TORCH_CHECK(b_scales.is_contiguous(), "b_scales is not contiguous");
+
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
+  Tensor c;
+  if (c_or_none.has_value()) {
+    c = c_or_none.value();
+    TORCH_CHECK(c.is_cuda(), "c is not on GPU");
+    TORCH_CHECK(c.is_contiguous(), "c is not contiguous");
+    TORCH_CHECK(c.size(0) == size_m, "Shape mismatch: c.size(0) = ", c.size(0), ", size_m = ", size_m);
+    TORCH_CHECK(c.size(1) == size_n, "Shape mismatch: c.size(1) = ", c.size(1), ", size_n = ", size_n);
+    TORCH_CHECK(c.scalar_type() == b_scales.scalar_type(), "c must have the type of b_scales with 8-bit activations");
+  } else {
+    c = at::empty({size_m, size_n}, b_scales.options());
+  }
+  if (size_m == 0) return c;
+
+  TORCH_CHECK(b_scales.dim() == 2, "b_scales rank = ", b_scales.dim(), " is not 2");
+  TORCH_CHECK(b_scales.size(1) == size_n, "b_scales dim 1 = ", b_scales.size(1), " is not size_n = ", size_n);
+  const int64_t num_groups = b_scales.size(0);
+  if (b_bias_or_none.has_value()) {
+    const Tensor& b = b_bias_or_none.value();
+    TORCH_CHECK(b.is_cuda(), "b_bias is not on GPU");
+    TORCH_CHECK(b.is_contiguous(), "b_bias is not contiguous");
+    TORCH_CHECK(b.size(0) == size_n, "b_bias.size(0) != size_n");
+    TORCH_CHECK(b.scalar_type() == c.scalar_type(), "b_bias must have the dtype of c");
+  }
+  const bool has_zp = b_zeros_or_none.has_value() && b_zeros_or_none->size(-1) > 0;
+  if (has_zp) {
+    const Tensor& z = b_zeros_or_none.value();
+    TORCH_CHECK(z.is_cuda(), "b_zeros is not on GPU");
+    TORCH_CHECK(z.is_contiguous(), "b_zeros is not contiguous");
+    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4, "b_type must be u4 or u8 when has_zp = True. Got = uint4b8");
+    TORCH_CHECK(z.dim() == 2, "b_zeros rank = ", z.dim(), " is not 2");
+    TORCH_CHECK(z.size(0) == num_groups, "b_zeros dim 0 = ", z.size(0), " is not num_groups = ", num_groups);
+    TORCH_CHECK(z.size(1) == size_n / 8, "b_zeros dim 1 = ", z.size(1), " is not size_n / pack_factor = ", size_n / 8);
+    TORCH_CHECK(z.scalar_type() == at::kInt, "b_zeros must be int32");
+  } else {
+    TORCH_CHECK(b_type_id != SONAR_TYPE_UINT4,
+                "b_type must be uint4b8, uint8b128, int4, int8, float8_e4m3fn or float4_e2m1f when "
+                "has_zp = False. Got = uint4");
+  }
+  TORCH_CHECK(size_n % 64 == 0, "size_n = ", size_n, ", is not divisible by min_thread_n = ", 64);
+  TORCH_CHECK(size_k % 32 == 0, "size_k = ", size_k, " is not divisible by 32 (the k tile of 8-bit activations)");
+
+  Tensor native = native_weights(b_q_weight, size_k, size_n, 1, 4, /*a8=*/true);
+  const size_t scratch_bytes = sonar_marlin_gemm_a8_scratch_bytes(size_m, size_n, size_k, num_groups);
+  Tensor scratch = at::empty({(int64_t)std::max<size_t>(scratch_bytes, 16)}, a.options().dtype(at::kByte));
+  raise_if_failed(sonar_marlin_gemm_a8(
+      a.const_data_ptr(), a.stride(0), a_dtype, c.mutable_data_ptr(),
+      static_cast<const uint32_t*>(native.const_data_ptr()), SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none),
+      b_scales.const_data_ptr(), static_cast<const float*>(a_scales->const_data_ptr()),
+      has_zp ? static_cast<const uint32_t*>(b_zeros_or_none->const_data_ptr()) : nullptr, scratch.mutable_data_ptr(),
+      scratch_bytes, dtype, b_type_id, size_m, size_n, size_k, num_groups, current_stream(a)));
+  return c;
+}
+
 Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_q_weight,
                    const OptTensor& b_bias_or_none, const Tensor& b_scales, const OptTensor& a_scales,
                    const OptTensor& global_scale, const OptTensor& b_zeros_or_none,
@@ -387,9 +545,13 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
                    const Tensor& workspace, int64_t b_type_id, int64_t size_m, int64_t size_n,
                    int64_t size_k, bool is_k_full, bool use_atomic_add, bool use_fp32_reduce,
                    bool is_zp_float) {
+  if (a.scalar_type() == at::kChar || a.scalar_type() == at::kFloat8_e4m3fn)
+    return marlin_gemm_a8(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, a_scales, global_scale,
+                          b_zeros_or_none, g_idx_or_none, b_type_id, size_m, size_n, size_k, is_zp_float);
+  TORCH_CHECK(a.scalar_type() == at::kHalf || a.scalar_type() == at::kBFloat16, "unsupported `a` scalar_type");
   const int dtype = dtype_code(a);
   check_b_type(b_type_id);
-  TORCH_CHECK_NOT_IMPLEMENTED(!a_scales.has_value(), "a_scales can only be used for 8bit activation.");
+  TORCH_CHECK(!(a_scales.has_value() && a_scales->numel() > 0), "a_scales can only be used for 8bit activation.");
   TORCH_CHECK_NOT_IMPLEMENTED(!is_zp_float, "is_zp_float = True is not built");
   // marlin.cu:784-796
   const bool nvfp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F && b_scales.scalar_type() == at::kFloat8_e4m3fn;
@@ -748,6 +910,40 @@ void moe_sum(const Tensor& input, Tensor& output) {
                                 input.size(2), dtype_code(input), current_stream(input)));
 }
 
+// Per-token quantisation of the activations of the W4A8 GEMM: (codes of x's shape, float32
+// scales (..., 1)).
+std::tuple<Tensor, Tensor> per_token_quant(const Tensor& x, bool fp8) {
+  TORCH_CHECK(x.is_cuda(), "x is not on GPU");
+  TORCH_CHECK(x.dim() >= 1 && x.size(-1) > 0, "x must have a non-empty last dimension");
+  int dtype;
+  if (x.scalar_type() == at::kHalf) dtype = SONAR_DTYPE_F16;
+  else if (x.scalar_type() == at::kBFloat16) dtype = SONAR_DTYPE_BF16;
+  else if (x.scalar_type() == at::kFloat) dtype = SONAR_DTYPE_F32;
+  else TORCH_CHECK(false, "per-token quantisation takes float16, bfloat16 or float32; got ", x.scalar_type());
+  const int64_t cols = x.size(-1);
+  const Tensor x2 = x.reshape({-1, cols});
+  const Tensor src = x2.stride(1) == 1 ? x2 : x2.contiguous();
+  const int64_t rows = src.size(0);
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(x.device());
+  Tensor q = at::empty(x.sizes(), x.options().dtype(fp8 ? at::kFloat8_e4m3fn : at::kChar));
+  auto scale_shape = x.sizes().vec();
+  scale_shape.back() = 1;
+  Tensor scales = at::empty(scale_shape, x.options().dtype(at::kFloat));
+  if (fp8)
+    raise_if_failed(sonar_per_token_quant_fp8(src.const_data_ptr(), dtype, rows ? src.stride(0) : cols,
+                                              static_cast<uint8_t*>(q.mutable_data_ptr()),
+                                              static_cast<float*>(scales.mutable_data_ptr()), rows, cols,
+                                              current_stream(x)));
+  else
+    raise_if_failed(sonar_per_token_quant_int8(src.const_data_ptr(), dtype, rows ? src.stride(0) : cols,
+                                               static_cast<int8_t*>(q.mutable_data_ptr()),
+                                               static_cast<float*>(scales.mutable_data_ptr()), rows, cols,
+                                               current_stream(x)));
+  return {q, scales};
+}
+std::tuple<Tensor, Tensor> per_token_quant_int8(const Tensor& x) { return per_token_quant(x, false); }
+std::tuple<Tensor, Tensor> per_token_quant_fp8(const Tensor& x) { return per_token_quant(x, true); }
+
 }  // namespace
 
 // Ops every build of the reference already has under _C / _moe_C (they are not
@@ -759,11 +955,15 @@ TORCH_LIBRARY(sonar_amd, m) {
       "Tensor! experts_ids, Tensor! num_tokens_post_pad, Tensor? maybe_expert_map) -> ()");
   m.def("silu_and_mul(Tensor! result, Tensor input) -> ()");
   m.def("moe_sum(Tensor input, Tensor! output) -> ()");
+  m.def("per_token_quant_int8(Tensor x) -> (Tensor, Tensor)");
+  m.def("per_token_quant_fp8(Tensor x) -> (Tensor, Tensor)");
 }
 TORCH_LIBRARY_IMPL(sonar_amd, CUDA, m) {
   m.impl("moe_align_block_size", &moe_align_block_size);
   m.impl("silu_and_mul", &silu_and_mul);
   m.impl("moe_sum", &moe_sum);
+  m.impl("per_token_quant_int8", &per_token_quant_int8);
+  m.impl("per_token_quant_fp8", &per_token_quant_fp8);
 }
 
 TORCH_LIBRARY_FRAGMENT(_C, m) {
@@ -791,6 +991,7 @@ TORCH_LIBRARY_FRAGMENT(_C, m) {
       "awq_marlin_repack(Tensor b_q_weight, SymInt size_k, "
       "SymInt size_n, int num_bits, bool is_a_8bit) -> Tensor");
   // not in the reference: Marlin order -> gfx950 streaming order, and cache control
+  m.def("marlin_int4_fp8_preprocess(Tensor qweight, Tensor? qzeros_or_none, bool inplace) -> Tensor");
   m.def("marlin_to_gfx950(Tensor b_q_weight, SymInt size_k, SymInt size_n) -> Tensor");
   m.def("marlin_weight_cache_clear() -> int", &marlin_weight_cache_clear);
   m.def("marlin_weight_cache_invalidate(Tensor t) -> int", &marlin_weight_cache_invalidate);
@@ -801,6 +1002,7 @@ TORCH_LIBRARY_IMPL(_C, CUDA, m) {
   m.impl("gptq_marlin_gemm", &marlin_gemm);
   m.impl("gptq_marlin_repack", &gptq_marlin_repack);
   m.impl("awq_marlin_repack", &awq_marlin_repack);
+  m.impl("marlin_int4_fp8_preprocess", &marlin_int4_fp8_preprocess);
   m.impl("marlin_to_gfx950", &marlin_to_gfx950);
 }
 

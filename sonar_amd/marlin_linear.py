@@ -17,12 +17,12 @@ import torch
 
 from . import ops
 from .marlin_utils import (MARLIN_SUPPORTED_GROUP_SIZES, apply_gptq_marlin_linear,
-                           check_marlin_supports_shape, marlin_is_k_full, marlin_make_empty_g_idx,
+                           check_marlin_supports_shape, marlin_act_int8_process_scales, marlin_is_k_full, marlin_make_empty_g_idx,
                            marlin_make_workspace_new, marlin_pad_dim, marlin_pad_qweight,
                            marlin_pad_scales, marlin_padded_nk, marlin_permute_bias,
                            marlin_permute_scales, marlin_sort_g_idx, marlin_zero_points,
                            query_marlin_supported_quant_types, unpack_cols)
-from .scalar_type import ScalarType
+from .scalar_type import ScalarType, scalar_types
 
 
 _AWQ_SLOT_OF_COLUMN = (0, 4, 1, 5, 2, 6, 3, 7)   # nibble slot of column j of an AWQ-packed int32
@@ -96,8 +96,10 @@ class MarlinLinearKernel:
 
     @classmethod
     def can_implement(cls, c: MPLinearLayerConfig) -> tuple[bool, str | None]:
-        if c.act_type not in (torch.float16, torch.bfloat16):
-            return False, f"activation type {c.act_type} not supported: fp16 / bf16 only"
+        if c.act_type not in (torch.float16, torch.bfloat16, torch.int8, torch.float8_e4m3fn):
+            return False, f"activation type {c.act_type} not supported: fp16, bf16, int8 or float8_e4m3fn"
+        if c.act_type.itemsize == 1 and c.has_g_idx:
+            return False, "act-order is not supported with 8-bit activations"
         quant_types = query_marlin_supported_quant_types(c.zero_points)
         if c.weight_type not in quant_types:
             return False, (f"Quant type ({c.weight_type}) not supported by  Marlin, supported types "
@@ -117,6 +119,9 @@ class MarlinLinearKernel:
     def process_weights_after_loading(self, layer) -> None:
         c = self.config
         device = getattr(layer, self.w_q_name).device
+        is_a_8bit = c.act_type is not None and c.act_type.itemsize == 1
+        if is_a_8bit:   # marlin.py:92-93
+            assert c.weight_type == scalar_types.uint4b8, "W8A8 is not supported by marlin kernel."
         row_parallel = c.partition_weight_shape[0] != c.full_weight_shape[0]
         self.is_k_full = marlin_is_k_full(c.has_g_idx, row_parallel)
         size_k, size_n = c.partition_weight_shape
@@ -152,7 +157,8 @@ class MarlinLinearKernel:
                 zp = unpack_cols(zp, c.weight_type.size_bits, grouped_k, size_n)
             zp = marlin_pad_scales(zp, size_n, size_k, padded_n, padded_k, c.group_size)
             setattr(layer, self.w_zp_name,
-                    marlin_zero_points(zp, padded_grouped_k, padded_n, c.weight_type.size_bits))
+                    marlin_zero_points(zp, padded_grouped_k, padded_n, c.weight_type.size_bits,
+                                       is_a_8bit=is_a_8bit))
         else:
             setattr(layer, self.w_zp_name, marlin_make_empty_g_idx(device))
 
@@ -161,12 +167,22 @@ class MarlinLinearKernel:
         setattr(layer, self.w_q_name, ops.gptq_marlin_repack(
             marlin_pad_qweight(w_q.contiguous(), size_n, size_k, padded_n, padded_k),
             perm=layer.g_idx_sort_indices, size_k=padded_k, size_n=padded_n,
-            num_bits=c.weight_type.size_bits, is_a_8bit=False))
+            num_bits=c.weight_type.size_bits, is_a_8bit=is_a_8bit))
+        if c.act_type == torch.float8_e4m3fn:   # marlin.py:95-97: sign-and-magnitude codes, scales times 512
+            ops.marlin_int4_fp8_preprocess(getattr(layer, self.w_q_name), inplace=True)
         w_s = getattr(layer, self.w_s_name)
         w_s = _input_major(w_s, w_s.numel() // size_n, size_n)
-        setattr(layer, self.w_s_name, marlin_permute_scales(
+        if c.act_type == torch.float8_e4m3fn:
+            w_s = w_s * 512
+        w_s = marlin_permute_scales(
             marlin_pad_scales(w_s.contiguous(), size_n, size_k, padded_n, padded_k, c.group_size),
-            size_k=padded_k, size_n=padded_n, group_size=c.group_size))
+            size_k=padded_k, size_n=padded_n, group_size=c.group_size, is_a_8bit=is_a_8bit)
+        num_groups = 1 if c.group_size == -1 else size_k // c.group_size
+        layer.input_global_scale = None
+        if c.act_type == torch.int8 and num_groups > 1:   # marlin.py:156-163
+            w_s, input_global_scale = marlin_act_int8_process_scales(w_s)
+            layer.input_global_scale = torch.nn.Parameter(input_global_scale, requires_grad=False)
+        setattr(layer, self.w_s_name, w_s)
         if getattr(layer, "bias", None) is not None:
             layer.bias = marlin_permute_bias(marlin_pad_dim(layer.bias, size_n, padded_n))
 
@@ -177,4 +193,5 @@ class MarlinLinearKernel:
             weight_zp=getattr(layer, self.w_zp_name), g_idx=getattr(layer, self.w_gidx_name),
             g_idx_sort_indices=layer.g_idx_sort_indices, workspace=self.workspace, wtype=c.weight_type,
             input_size_per_partition=c.partition_weight_shape[0],
-            output_size_per_partition=c.partition_weight_shape[1], is_k_full=self.is_k_full, bias=bias)
+            output_size_per_partition=c.partition_weight_shape[1], is_k_full=self.is_k_full,
+            input_global_scale=getattr(layer, "input_global_scale", None), bias=bias, input_dtype=c.act_type)

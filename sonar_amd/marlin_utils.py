@@ -8,6 +8,7 @@ with torch index ops so tensors stay on their device."""
 from __future__ import annotations
 
 import math
+import os
 
 import torch
 
@@ -243,9 +244,8 @@ def get_scale_perms():
 
 def marlin_permute_scales(s: torch.Tensor, size_k: int, size_n: int, group_size: int,
                           is_a_8bit: bool = False) -> torch.Tensor:
-    assert not is_a_8bit, "8-bit activations are not built"
     scale_perm, scale_perm_single = get_scale_perms()
-    if group_size < size_k and group_size != -1:
+    if group_size < size_k and group_size != -1 and not is_a_8bit:
         s = s.reshape((-1, len(scale_perm)))[:, scale_perm]
     else:
         s = s.reshape((-1, len(scale_perm_single)))[:, scale_perm_single]
@@ -259,6 +259,16 @@ def marlin_permute_bias(s: torch.Tensor) -> torch.Tensor:
     return s.reshape(*origin_shape).contiguous()
 
 
+def marlin_act_int8_process_scales(s: torch.Tensor):
+    """Group scales for int8 activations (marlin_utils.py:436-440): 16-bit integers
+    round(s / max * 4096) stored in a tensor of the scales' dtype, and the factor
+    max / 4096 that the caller multiplies into the activation scales."""
+    a_scales_scale_factor = 1 / 4096 * s.max().float()
+    s = s / s.max() * 4096
+    s = s.round().to(torch.int16).view(s.dtype)
+    return s, a_scales_scale_factor
+
+
 def marlin_moe_permute_scales(s: torch.Tensor, size_k: int, size_n: int, group_size: int,
                               is_a_8bit: bool = False) -> torch.Tensor:
     output = torch.empty_like(s)
@@ -270,10 +280,12 @@ def marlin_moe_permute_scales(s: torch.Tensor, size_k: int, size_n: int, group_s
 def marlin_zero_points(zp: torch.Tensor, size_k: int, size_n: int, num_bits: int,
                        is_a_8bit: bool = False) -> torch.Tensor:
     """`size_k` here is the number of groups (rows of zp), as in the reference."""
-    assert num_bits == 4 and not is_a_8bit
+    assert num_bits == 4
     scale_perm, _ = get_scale_perms()
     zp = zp.reshape((-1, len(scale_perm)))[:, scale_perm]
-    zp = zp.reshape((-1, 8))[:, _INTERLEAVE_4BIT].reshape((-1, size_n)).contiguous()
+    if not is_a_8bit:   # the column interleave of the 16-bit dequantiser (marlin_utils.py:472-473)
+        zp = zp.reshape((-1, 8))[:, _INTERLEAVE_4BIT]
+    zp = zp.reshape((-1, size_n)).contiguous()
     return pack_cols(zp, num_bits, size_k, size_n)
 
 
@@ -313,6 +325,42 @@ def should_use_atomic_add_reduce(m: int, n: int, k: int, device: torch.device, d
     return False
 
 
+# ---------------------------------------------------------------- 8-bit activations
+def per_token_quant_int8(x: torch.Tensor):
+    """int8_utils.py:95-120: (int8 of x's shape, float32 scales (..., 1))."""
+    return ops.per_token_quant_int8(x)
+
+
+def per_token_quant_fp8(x: torch.Tensor):
+    """What get__quant_fp8_method()(x) returns in the reference (marlin_utils.py:596-603)."""
+    return ops.per_token_quant_fp8(x)
+
+
+def get_marlin_input_dtype(prefix: str | None = None):
+    """The activation type the environment asks for (marlin_utils.py:606-623):
+    APHRODITE_MARLIN_INPUT_DTYPE = int8 | fp8, else None (16-bit).  The reference lets
+    fp8 through only where the tensor cores have it (SM 8.9 / 12.x); gfx950 has fp8 matrix
+    cores, so it is allowed here."""
+    want = os.environ.get("APHRODITE_MARLIN_INPUT_DTYPE")
+    if want is None:
+        return None
+    if want.lower() == "int8":
+        return torch.int8
+    if want.lower() == "fp8":
+        return torch.float8_e4m3fn
+    return None
+
+
+def marlin_quant_input(x: torch.Tensor, quant_dtype: torch.dtype):
+    """marlin_utils.py:626-633."""
+    x = x.reshape(-1, x.shape[-1])
+    if quant_dtype == torch.int8:
+        return per_token_quant_int8(x)
+    if quant_dtype == torch.float8_e4m3fn:
+        return per_token_quant_fp8(x)
+    raise ValueError(f"unsupported quant_dtype {quant_dtype}")
+
+
 # ---------------------------------------------------------------- the linear call
 def apply_gptq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_scale: torch.Tensor,
                              weight_zp: torch.Tensor, g_idx: torch.Tensor,
@@ -323,15 +371,22 @@ def apply_gptq_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_s
                              bias: torch.Tensor | None = None,
                              use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT,
                              input_dtype: torch.dtype | None = None) -> torch.Tensor:
-    if input_dtype is not None and input_dtype.itemsize == 1:
-        raise NotImplementedError("8-bit activations (W4A8) are not built")
     reshaped_x = input.reshape(-1, input.shape[-1])
     out_shape = input.shape[:-1] + (output_size_per_partition,)
     padded_n, padded_k = marlin_repacked_nk(weight, wtype.size_bits)
     reshaped_x = marlin_pad_dim(reshaped_x, input_size_per_partition, padded_k)
     use_atomic_add = should_use_atomic_add_reduce(reshaped_x.size(0), padded_n, padded_k, input.device,
                                                   input.dtype)
-    output = ops.marlin_gemm(reshaped_x, None, weight, bias, weight_scale, None, None, weight_zp, g_idx,
+    a_scales = None
+    if input_dtype == torch.int8:      # marlin_utils.py:671-680
+        assert wtype == scalar_types.uint4b8, "W8A8-INT8 is not supported by marlin kernel."
+        reshaped_x, a_scales = marlin_quant_input(reshaped_x, input_dtype)
+        if input_global_scale is not None:
+            a_scales = a_scales * input_global_scale
+    elif input_dtype == torch.float8_e4m3fn:
+        assert wtype == scalar_types.uint4b8, "INT8 weight + FP8 activation is not supported."
+        reshaped_x, a_scales = marlin_quant_input(reshaped_x, input_dtype)
+    output = ops.marlin_gemm(reshaped_x, None, weight, bias, weight_scale, a_scales, None, weight_zp, g_idx,
                              g_idx_sort_indices, workspace, wtype, size_m=reshaped_x.shape[0],
                              size_n=padded_n, size_k=padded_k, is_k_full=is_k_full,
                              use_atomic_add=use_atomic_add, use_fp32_reduce=use_fp32_reduce,

@@ -41,6 +41,19 @@ def _register_fakes() -> None:
         return torch.empty((size_k // 16, size_n * 16 // pack_factor), dtype=b_q_weight.dtype,
                            device=b_q_weight.device)
 
+    @reg("_C::marlin_int4_fp8_preprocess")
+    def _(qweight, qzeros_or_none=None, inplace=False):
+        return torch.empty_like(qweight)
+
+    def quant_fake(code_dtype):
+        def fake(x):
+            return (torch.empty(x.shape, dtype=code_dtype, device=x.device),
+                    torch.empty(x.shape[:-1] + (1,), dtype=torch.float32, device=x.device))
+        return fake
+
+    reg("sonar_amd::per_token_quant_int8")(quant_fake(torch.int8))
+    reg("sonar_amd::per_token_quant_fp8")(quant_fake(torch.float8_e4m3fn))
+
     @reg("_C::marlin_to_gfx950")
     def _(b_q_weight, size_k, size_n):
         return torch.empty_like(b_q_weight)
@@ -101,6 +114,26 @@ def awq_marlin_moe_repack(b_q_weight: torch.Tensor, perm: torch.Tensor, size_k: 
     for e in range(num_experts):
         output[e] = torch.ops._C.awq_marlin_repack(b_q_weight[e], size_k, size_n, num_bits, is_a_8bit)
     return output
+
+
+def marlin_int4_fp8_preprocess(qweight: torch.Tensor, qzeros_or_none: torch.Tensor | None = None,
+                               inplace: bool = False) -> torch.Tensor:
+    """aphrodite/_custom_ops.py:1464-1469: 4-bit codes -> sign and magnitude of code - zero
+    point, the form the fp8-activation kernels read."""
+    return torch.ops._C.marlin_int4_fp8_preprocess(qweight, qzeros_or_none, inplace)
+
+
+def per_token_quant_int8(x: torch.Tensor):
+    """One scale per row, max(absmax, 1e-10) / 127, and int8 codes rounded half away from zero
+    (the reference's Triton kernel, layers/quantization/utils/int8_utils.py:70-120).  Returns
+    (int8 of x's shape, float32 (..., 1))."""
+    return torch.ops.sonar_amd.per_token_quant_int8(x)
+
+
+def per_token_quant_fp8(x: torch.Tensor):
+    """Dynamic per-token float8_e4m3fn quantisation (QuantFP8(False, GroupShape.PER_TOKEN),
+    layers/quantization/input_quant_fp8.py:188-204): scale = max(absmax / 448, 1 / (448 * 512))."""
+    return torch.ops.sonar_amd.per_token_quant_fp8(x)
 
 
 def marlin_gemm(a: torch.Tensor, c: torch.Tensor | None, b_q_weight: torch.Tensor,

@@ -87,3 +87,33 @@ def test_opcheck_moe_wna16_marlin_gemm(layer, with_c):
     args = (a, c, w, None, s, None, None, None, None, None, layer["ws"], sorted_ids, expert_ids, past, topk_w, bs,
             top_k, False, scalar_types.uint4b8.id, m, n, k, True, False, True, False, -1, -1, -1)
     opcheck(torch.ops._moe_C.moe_wna16_marlin_gemm, args, c_given=with_c)
+
+
+def test_opcheck_w4a8_ops(layer):
+    """The ops of the 8-bit-activation path: repack with is_a_8bit, marlin_int4_fp8_preprocess
+    (out of place, as the schema promises no mutation) and marlin_gemm with int8 / fp8 `a`."""
+    from sonar_amd import marlin_utils
+    from sonar_amd.scalar_type import scalar_types
+    k, n = layer["k"], layer["n"]
+    opcheck(torch.ops._C.gptq_marlin_repack, (layer["qw"], layer["empty"], k, n, 4, True))
+    qa = torch.from_numpy(mo.awq_pack(layer["q"])).to(DEV)
+    opcheck(torch.ops._C.awq_marlin_repack, (qa, k, n, 4, True))
+    marlin8 = torch.ops._C.gptq_marlin_repack(layer["qw"], layer["empty"], k, n, 4, True)
+    opcheck(torch.ops._C.marlin_int4_fp8_preprocess, (marlin8, None, False))
+    scales = marlin_utils.marlin_permute_scales(
+        torch.rand((k // 128, n), device=DEV, dtype=torch.float16) * 1e-2, k, n, 128, is_a_8bit=True)
+    int_scales, _ = marlin_utils.marlin_act_int8_process_scales(scales)
+    m = 8
+    x = torch.randn((m, k), device=DEV, dtype=torch.float16)
+    for quant, s in ((marlin_utils.per_token_quant_int8, int_scales), (marlin_utils.per_token_quant_fp8, scales)):
+        a, a_s = quant(x)
+        args = (a, None, marlin8, None, s, a_s, None, layer["empty"], layer["empty"], layer["empty"], layer["ws"],
+                scalar_types.uint4b8.id, m, n, k, True, False, True, False)
+        if a.dtype == torch.int8:
+            opcheck(torch.ops._C.marlin_gemm, args)
+        else:
+            # the schema check perturbs its inputs with arithmetic torch does not have for float8_e4m3fn
+            torch.library.opcheck(torch.ops._C.marlin_gemm, args, test_utils=OPCHECK_TEST_UTILS[1:],
+                                  raise_exception=True)
+    opcheck(torch.ops.sonar_amd.per_token_quant_int8, (x,))
+    opcheck(torch.ops.sonar_amd.per_token_quant_fp8, (x,))

@@ -1038,3 +1038,122 @@ def test_prepare_mxfp8_moe_layer_and_fused_marlin_moe(cfg):
     got = gu.host_f32(y)
     max_ref = np.abs(want).max()
     assert np.abs(got - want).max() <= 2e-2 * max_ref, (np.abs(got - want).max(), max_ref)
+
+
+# ---------------------------------------------------------------- 8-bit activations (W4A8)
+def test_marlin_int4_fp8_preprocess_reference_formulas():
+    """The reference's own two tests of the op (tests/kernels/quantization/test_marlin_gemm.py:148-188)."""
+    from sonar_amd import ops
+    qweight_unpacked = torch.randint(0, 16, size=(2048, 2048), dtype=torch.int32, device="cuda")
+    qweight_packed = (qweight_unpacked[:, ::2] * 16 + qweight_unpacked[:, 1::2]).to(torch.int8).view(torch.int32)
+    res = ops.marlin_int4_fp8_preprocess(qweight_packed)
+    want = torch.where(qweight_unpacked >= 8, qweight_unpacked - 8, 15 - qweight_unpacked)
+    want = (want[:, ::2] * 16 + want[:, 1::2]).to(torch.int8).view(torch.int32)
+    assert (res == want).all()
+    assert res.data_ptr() != qweight_packed.data_ptr()
+    same = ops.marlin_int4_fp8_preprocess(qweight_packed, inplace=True)
+    assert same.data_ptr() == qweight_packed.data_ptr() and (qweight_packed == want).all()
+
+    group_size = 128
+    qzeros_unpacked = torch.randint(0, 16, size=(2048 // group_size, 2048), dtype=torch.int32, device="cuda")
+    qweight_packed = (qweight_unpacked[:, ::2] * 16 + qweight_unpacked[:, 1::2]).to(torch.int8).view(torch.int32)
+    qzeros_packed = (qzeros_unpacked[:, ::2] * 16 + qzeros_unpacked[:, 1::2]).to(torch.int8).view(torch.int32)
+    res = ops.marlin_int4_fp8_preprocess(qweight_packed, qzeros_packed)
+    want = qweight_unpacked - qzeros_unpacked.repeat_interleave(group_size, 0)
+    want[want < 0] = 15 - qweight_unpacked[want < 0]
+    want = (want[:, ::2] * 16 + want[:, 1::2]).to(torch.int8).view(torch.int32)
+    assert (res == want).all()
+
+
+@pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16, torch.float32])
+def test_per_token_quant_ops_bit_exact(dtype):
+    """int8 against the oracle, fp8 against the same formula in torch's fp32 arithmetic on the
+    CPU (IEEE division and multiplication, round-to-nearest-even conversion)."""
+    from oracle import marlin_oracle as mo
+    from sonar_amd.marlin_utils import marlin_quant_input, per_token_quant_fp8, per_token_quant_int8
+    x = torch.randn((3, 11, 520), device="cuda", dtype=dtype) * 3
+    x[0, 0] = 0                                           # a row of zeros: the floors of the scales
+    q, s = per_token_quant_int8(x)
+    want_q, want_s = mo.per_token_quant_int8(x.float().cpu().numpy().reshape(33, 520))
+    assert q.dtype == torch.int8 and s.dtype == torch.float32 and q.shape == x.shape and s.shape == (3, 11, 1)
+    assert np.array_equal(q.cpu().numpy().reshape(33, 520), want_q)
+    assert np.array_equal(s.cpu().numpy().reshape(33, 1), want_s)
+    f, fs = per_token_quant_fp8(x)
+    xc = x.float().cpu()
+    want_fs = (xc.abs().amax(dim=-1, keepdim=True) / 448.0).clamp(min=1.0 / (448.0 * 512.0))
+    want_f = (xc * want_fs.reciprocal()).clamp(-448.0, 448.0).to(torch.float8_e4m3fn)
+    assert f.dtype == torch.float8_e4m3fn and fs.shape == (3, 11, 1)
+    assert torch.equal(fs.cpu(), want_fs)
+    assert torch.equal(f.cpu().view(torch.uint8), want_f.view(torch.uint8))
+    # a view with a row stride, and the reference's dispatcher
+    wide = torch.randn((8, 1024), device="cuda", dtype=dtype)
+    q2, s2 = marlin_quant_input(wide[:, :512], torch.int8)
+    q3, s3 = per_token_quant_int8(wide[:, :512].contiguous())
+    assert torch.equal(q2, q3) and torch.equal(s2, s3)
+    with pytest.raises(ValueError, match="unsupported quant_dtype"):
+        marlin_quant_input(wide, torch.float16)
+
+
+@pytest.mark.parametrize("act_type", [torch.int8, torch.float8_e4m3fn])
+@pytest.mark.parametrize("group_size", [-1, 128])
+def test_linear_kernel_with_8bit_activations(act_type, group_size):
+    """MarlinLinearKernel with act_type int8 / fp8 (marlin.py:88-163,214-235): repack with
+    is_a_8bit, fp8 preprocess and scales times 512, integer group scales and
+    input_global_scale; the output follows the 16-bit kernel's within the quantisation error
+    of the activations."""
+    from sonar_amd.marlin_linear import MarlinLinearKernel, MPLinearLayerConfig
+    from sonar_amd.scalar_type import scalar_types
+    from tests.quant_utils import gptq_pack, gptq_quantize_weights
+    k, n, m = 512, 256, 24
+    w = torch.randn((k, n), device="cuda", dtype=torch.float16)
+    w_ref, q_w, s, _, _ = gptq_quantize_weights(w, scalar_types.uint4b8, k if group_size == -1 else group_size, False)
+    outs = {}
+    for act in (torch.float16, act_type):
+        cfg = MPLinearLayerConfig(full_weight_shape=(k, n), partition_weight_shape=(k, n),
+                                  weight_type=scalar_types.uint4b8, act_type=act, group_size=group_size,
+                                  zero_points=False, has_g_idx=False)
+        layer = types.SimpleNamespace(qweight=gptq_pack(q_w, 4, k, n), scales=s.clone(), bias=None)
+        kernel = MarlinLinearKernel(cfg, w_zp_param_name=None, w_gidx_param_name=None)
+        kernel.process_weights_after_loading(layer)
+        if act == torch.int8:
+            assert (layer.input_global_scale is not None) == (group_size != -1)
+        torch.manual_seed(0)
+        x = torch.randn((m, k), device="cuda", dtype=torch.float16)
+        outs[act] = kernel.apply_weights(layer, x)
+        assert outs[act].dtype == torch.float16 and outs[act].shape == (m, n)
+    ref = torch.matmul(x, w_ref)
+    rel = lambda o: (torch.mean(torch.abs(o - ref)) / torch.mean(torch.abs(ref))).item()
+    assert rel(outs[torch.float16]) < 0.01
+    assert rel(outs[act_type]) < 0.04
+
+
+def test_w4a8_op_rejections():
+    from sonar_amd import ops
+    from sonar_amd.marlin_utils import marlin_make_workspace_new, per_token_quant_int8
+    from sonar_amd.scalar_type import scalar_types
+    from tests.marlin_utils_for_tests import marlin_quantize
+    k, n, m = 256, 128, 4
+    w = torch.randn((k, n), device="cuda", dtype=torch.float16)
+    w_ref, q_w, s, g_idx, sort_idx, _ = marlin_quantize(w, scalar_types.uint4b8, 128, False, input_dtype=torch.int8)
+    ws = marlin_make_workspace_new(w.device)
+    a, a_s = per_token_quant_int8(torch.randn((m, k), device="cuda", dtype=torch.float16))
+
+    def call(a=a, a_s=a_s, b_type=scalar_types.uint4b8, scales=s, gs=None, g=None, p=None):
+        return ops.marlin_gemm(a, None, q_w, None, scales, a_s, gs, None, g, p, ws, b_type, m, n, k)
+
+    assert call().shape == (m, n)
+    with pytest.raises(RuntimeError, match="a_scales parameter must be passed for 8bit activation"):
+        call(a_s=None)
+    with pytest.raises(RuntimeError, match="W8A8-INT8 is not supported"):
+        call(b_type=scalar_types.uint8b128)
+    with pytest.raises(RuntimeError, match="global_scale can only be used for nvfp4"):
+        call(gs=torch.ones(1, device="cuda"))
+    with pytest.raises(RuntimeError, match="act-order is not supported with 8-bit activations"):
+        perm = torch.randperm(k, device="cuda").int()
+        call(g=torch.zeros(k, dtype=torch.int32, device="cuda"), p=perm)
+    with pytest.raises(RuntimeError, match="a_scales can only be used for 8bit activation"):
+        ops.marlin_gemm(torch.randn((m, k), device="cuda", dtype=torch.float16), None, q_w, None, s, a_s, None, None,
+                        None, None, ws, scalar_types.uint4b8, m, n, k)
+    with pytest.raises(RuntimeError, match="Unsupported repack config"):
+        ops.gptq_marlin_repack(torch.zeros((k // 8, n), dtype=torch.int32, device="cuda"),
+                               torch.randperm(k, device="cuda").int(), k, n, 4, True)

@@ -8,8 +8,8 @@ laid out in Marlin order by the index recipe of `marlin_utils_test.py`
   * `marlin_gemm` must agree with `torch.matmul(a, w_ref)` under the
     reference's criterion mean|out - ref| / mean|ref| < 0.04 (test_marlin_gemm,
     test_marlin_gemm_with_bias), over the reference's grid of shapes, group
-    sizes, weight types (integer, fp8, MXFP4), act-order and is_k_full for 16-bit
-    activations.
+    sizes, weight types (integer, fp8, MXFP4), act-order and is_k_full, for 16-bit
+    activations and for int8 / float8_e4m3fn activations with 4-bit weights.
 No oracle here: the expected values come from torch on the GPU, as in the
 reference."""
 from __future__ import annotations
@@ -33,6 +33,10 @@ DENSE_CONFIGS = [
     {"b_type": scalar_types.uint8b128, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]}, # GPTQ int8
     {"b_type": scalar_types.float8_e4m3fn, "group_blocks": [-1, 8]},                              # FP8
     {"b_type": scalar_types.float4_e2m1f, "a_type": [torch.bfloat16], "group_blocks": [2]},       # MXFP4
+    {"a_quant": torch.int8, "b_type": scalar_types.uint4, "group_blocks": [-1, 2, 4, 8]},         # AWQ int4, int8 A
+    {"a_quant": torch.int8, "b_type": scalar_types.uint4b8, "group_blocks": [-1, 2, 4, 8]},       # GPTQ int4, int8 A
+    {"a_quant": torch.float8_e4m3fn, "b_type": scalar_types.uint4b8, "group_blocks": [-1, 2, 4, 8]},  # fp8 A
+    {"a_quant": torch.float8_e4m3fn, "b_type": scalar_types.uint4, "group_blocks": [-1, 2, 4, 8]},
 ]
 
 
@@ -47,28 +51,36 @@ def rand_data(shape, dtype=torch.float16):
 @pytest.mark.parametrize("n_chunk", MARLIN_N_CHUNKS)
 @pytest.mark.parametrize("quant_type", [scalar_types.uint4b8, scalar_types.uint8b128], ids=str)
 @pytest.mark.parametrize("act_order", [False, True])
+@pytest.mark.parametrize("is_a_8bit", [True, False])
 @pytest.mark.parametrize("nk_factors", MARLIN_REPACK_NK_FACTORS)
-def test_gptq_marlin_repack(n_chunk, quant_type, act_order, nk_factors):
+def test_gptq_marlin_repack(n_chunk, quant_type, act_order, is_a_8bit, nk_factors):
     from sonar_amd import ops
     from tests.marlin_utils_for_tests import get_weight_perm, marlin_weights
     from tests.quant_utils import gptq_pack, gptq_quantize_weights, sort_weights
     n_factor, k_factor = nk_factors
     size_k, size_n, group_size = 128 * k_factor, n_chunk * n_factor, 128
+    if act_order and is_a_8bit:
+        return   # the reference's filter (test_marlin_gemm.py:205-212)
+    if is_a_8bit and quant_type.size_bits == 8:
+        pytest.skip("8-bit weights in the order of 8-bit activations are not built: no GEMM takes them "
+                    "(W8A8 is not a Marlin mode)")
     b_weight = rand_data((size_k, size_n))
     w_ref, q_w, s, g_idx, rand_perm = gptq_quantize_weights(b_weight, quant_type, group_size, act_order)
     q_w_gptq = gptq_pack(q_w, quant_type.size_bits, size_k, size_n)
     sort_indices = torch.empty(0, dtype=torch.int, device=b_weight.device)
     if act_order:
         q_w, g_idx, sort_indices = sort_weights(q_w, g_idx)
-    expected = marlin_weights(q_w, size_k, size_n, quant_type.size_bits, get_weight_perm(quant_type.size_bits))
-    got = ops.gptq_marlin_repack(q_w_gptq, sort_indices, size_k, size_n, quant_type.size_bits, False)
+    expected = marlin_weights(q_w, size_k, size_n, quant_type.size_bits,
+                              get_weight_perm(quant_type.size_bits, is_a_8bit), is_a_8bit)
+    got = ops.gptq_marlin_repack(q_w_gptq, sort_indices, size_k, size_n, quant_type.size_bits, is_a_8bit)
     torch.cuda.synchronize()
     assert torch.equal(expected, got)
 
 
 @pytest.mark.parametrize("n_chunk", MARLIN_N_CHUNKS)
+@pytest.mark.parametrize("is_a_8bit", [True, False])
 @pytest.mark.parametrize("nk_factors", MARLIN_REPACK_NK_FACTORS)
-def test_awq_marlin_repack(n_chunk, nk_factors):
+def test_awq_marlin_repack(n_chunk, is_a_8bit, nk_factors):
     from sonar_amd import ops
     from tests.marlin_utils_for_tests import get_weight_perm, marlin_weights
     from tests.quant_utils import awq_pack, quantize_weights
@@ -78,8 +90,8 @@ def test_awq_marlin_repack(n_chunk, nk_factors):
     b_weight = rand_data((size_k, size_n))
     w_ref, q_w, s, zp = quantize_weights(b_weight, quant_type, 128, zero_points=True)
     q_w_awq = awq_pack(q_w, 4, size_k, size_n)
-    expected = marlin_weights(q_w, size_k, size_n, 4, get_weight_perm(4))
-    got = ops.awq_marlin_repack(q_w_awq, size_k, size_n, 4, False)
+    expected = marlin_weights(q_w, size_k, size_n, 4, get_weight_perm(4, is_a_8bit), is_a_8bit)
+    got = ops.awq_marlin_repack(q_w_awq, size_k, size_n, 4, is_a_8bit)
     torch.cuda.synchronize()
     assert torch.equal(expected, got)
 
@@ -105,13 +117,14 @@ def _gemm_cases():
                 continue
             if not act_order and is_k_full:
                 continue
-            cases.append((cfg["b_type"], dtype, group_size, size_m, size_n, size_k, act_order, is_k_full))
+            cases.append((cfg.get("a_quant"), cfg["b_type"], dtype, group_size, size_m, size_n, size_k, act_order,
+                          is_k_full))
     return cases
 
 
-@pytest.mark.parametrize("b_type,dtype,group_size,size_m,size_n,size_k,act_order,is_k_full", _gemm_cases(),
+@pytest.mark.parametrize("a_quant,b_type,dtype,group_size,size_m,size_n,size_k,act_order,is_k_full", _gemm_cases(),
                          ids=lambda v: str(v).replace("torch.", ""))
-def test_marlin_gemm(b_type, dtype, group_size, size_m, size_n, size_k, act_order, is_k_full):
+def test_marlin_gemm(a_quant, b_type, dtype, group_size, size_m, size_n, size_k, act_order, is_k_full):
     from sonar_amd import ops
     from sonar_amd.marlin_utils import marlin_make_workspace_new
     from sonar_amd.marlin_utils_fp4 import rand_marlin_weight_mxfp4_like
@@ -119,8 +132,10 @@ def test_marlin_gemm(b_type, dtype, group_size, size_m, size_n, size_k, act_orde
     from tests.marlin_utils_for_tests import awq_marlin_quantize, marlin_quantize
     a_input = rand_data((size_m, size_k), dtype=dtype)
     b_weight = rand_data((size_k, size_n), dtype=dtype)
+    from sonar_amd.marlin_utils import per_token_quant_fp8, per_token_quant_int8
     if b_type == scalar_types.uint4:
-        w_ref, marlin_q_w, marlin_s, marlin_zp = awq_marlin_quantize(b_weight, b_type, group_size)
+        w_ref, marlin_q_w, marlin_s, marlin_zp = awq_marlin_quantize(b_weight, b_type, group_size,
+                                                                     input_dtype=a_quant)
         g_idx = sort_indices = None
     elif b_type == scalar_types.float8_e4m3fn:
         w_ref, marlin_q_w, marlin_s = marlin_quant_fp8_torch(b_weight.T.contiguous(), group_size)
@@ -129,14 +144,25 @@ def test_marlin_gemm(b_type, dtype, group_size, size_m, size_n, size_k, act_orde
         w_ref, marlin_q_w, marlin_s = rand_marlin_weight_mxfp4_like(b_weight.T, group_size)
         g_idx = sort_indices = marlin_zp = None
     else:
-        w_ref, marlin_q_w, marlin_s, g_idx, sort_indices, _ = marlin_quantize(b_weight, b_type, group_size, act_order)
+        w_ref, marlin_q_w, marlin_s, g_idx, sort_indices, _ = marlin_quantize(b_weight, b_type, group_size, act_order,
+                                                                              input_dtype=a_quant)
         marlin_zp = None
     workspace = marlin_make_workspace_new(w_ref.device)
+    a_scales, a_input_ref = None, a_input
+    if a_quant == torch.int8:                      # test_marlin_gemm.py:446-455
+        a_input, a_scales = per_token_quant_int8(a_input)
+        a_input_ref = (a_input.to(a_scales.dtype) * a_scales.view(-1, 1)).to(dtype)
+        if group_size != -1:
+            a_scales = (a_scales / 4096 * marlin_s.max()).float()
+            marlin_s = (marlin_s / marlin_s.max() * 4096).round().to(torch.int16).view(dtype)
+    elif a_quant == torch.float8_e4m3fn:           # test_marlin_gemm.py:456-459
+        a_input, a_scales = per_token_quant_fp8(a_input)
+        a_input_ref = (a_input.to(a_scales.dtype) * a_scales.view(-1, 1)).to(dtype)
     output = torch.empty((size_m, size_n), dtype=dtype, device=a_input.device)
-    output = ops.marlin_gemm(a_input, output, marlin_q_w, None, marlin_s, None, None, marlin_zp, g_idx, sort_indices,
-                             workspace, b_type, a_input.shape[0], b_weight.shape[1], a_input.shape[1],
+    output = ops.marlin_gemm(a_input, output, marlin_q_w, None, marlin_s, a_scales, None, marlin_zp, g_idx,
+                             sort_indices, workspace, b_type, a_input.shape[0], b_weight.shape[1], a_input.shape[1],
                              is_k_full=is_k_full, use_atomic_add=False, use_fp32_reduce=True, is_zp_float=False)
-    output_ref = torch.matmul(a_input, w_ref)
+    output_ref = torch.matmul(a_input_ref, w_ref)
     torch.cuda.synchronize()
     assert compute_max_diff(output, output_ref) < 0.04
 

@@ -691,7 +691,7 @@ def test_gemm_w4a8_int8_against_python_loop(group_size, zp):
     rng = np.random.default_rng(7 + (group_size % 97))
     m, k, n = 3, 128, 8
     a = rng.integers(-127, 128, size=(m, k)).astype(np.int8)
-    a_s = rng.uniform(0.01, 0.02, size=(m, 1)).astype(np.float32)
+    a_s = rng.uniform(1e-6, 2e-6, size=(m, 1)).astype(np.float32) * (1e3 if group_size == -1 else 1)
     q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
     gs = k if group_size == -1 else group_size
     groups = k // gs
@@ -713,6 +713,7 @@ def test_gemm_w4a8_int8_against_python_loop(group_size, zp):
             want = np.float32(total) * a_s[mm, 0]
             if group_size == -1:
                 want = want * scales[0, nn]
+            assert np.isfinite(got[mm, nn]) and got[mm, nn] != 0
             assert got[mm, nn] == np.float32(want).astype(np.float16).astype(np.float32)
 
 
