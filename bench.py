@@ -41,6 +41,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 MEASURED_TRAFFIC_M16 = 32_400_000
 REPLAYS = 21                # graph replays per timing; the median is reported
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
+MFMA_PEAK_8BIT_TFLOPS = 5000.0   # MI355X dense int8 / fp8
 GROUP = 128
 LAYER_SHAPES = [("qkv", 4096, 6144), ("o", 4096, 4096), ("gate_up", 4096, 28672), ("down", 14336, 4096)]
 
@@ -200,13 +201,17 @@ def variants_sweep(torch, ops, gen, time_graph):
     8-bit weights (uint8b128), fp8 weights (float8_e4m3fn, scales with the
     exponent bias folded in), MXFP8 and MXFP4 weights (float8_e4m3fn /
     float4_e2m1f, exponent-byte scales per 32 rows, bf16 activations), NVFP4
-    weights (float4_e2m1f, float8_e4m3fn scales per 16 rows, a global scale)."""
+    weights (float4_e2m1f, float8_e4m3fn scales per 16 rows, a global scale),
+    W4A8 (uint4b8 weights in the order of 8-bit activations; int8 activations with
+    16-bit integer group scales, float8_e4m3fn activations with the weights as
+    marlin_int4_fp8_preprocess leaves them; one fp32 scale per activation row;
+    frac_mfma is then against the 8-bit peak)."""
     from sonar_amd import marlin_utils
     from sonar_amd.scalar_type import scalar_types
     dev = "cuda:0"
     k, n = 4096, 11008
     out = []
-    for name in ("act_order", "awq", "w8a16", "fp8", "mxfp8", "mxfp4", "nvfp4"):
+    for name in ("act_order", "awq", "w8a16", "fp8", "mxfp8", "mxfp4", "nvfp4", "w4a8_int8", "w4a8_fp8"):
         layers = []
         words = 4 * n if name in ("w8a16", "fp8", "mxfp8") else 2 * n     # 8-bit codes: four per word
         act_dtype = torch.bfloat16 if name in ("mxfp4", "mxfp8") else torch.float16
@@ -221,6 +226,11 @@ def variants_sweep(torch, ops, gen, time_graph):
                 layers.append((qw, sc, empty, g_idx, perm, ws, scalar_types.uint4b8))
             elif name == "w8a16":
                 layers.append((qw, sc * 0.0625, empty, empty, empty, ws, scalar_types.uint8b128))
+            elif name == "w4a8_int8":
+                ints = torch.randint(1, 4097, (k // GROUP, n), dtype=torch.int16, device=dev, generator=gen)
+                layers.append((qw, ints.view(torch.float16), empty, empty, empty, ws, scalar_types.uint4b8))
+            elif name == "w4a8_fp8":
+                layers.append((qw, sc * 512, empty, empty, empty, ws, scalar_types.uint4b8))
             elif name == "fp8":
                 layers.append((qw, sc * 0.0625 * 256, empty, empty, empty, ws, scalar_types.float8_e4m3fn))
             elif name == "nvfp4":
@@ -238,9 +248,17 @@ def variants_sweep(torch, ops, gen, time_graph):
                 layers.append((qw, sc, zp, empty, empty, ws, scalar_types.uint4))
         for m in (1, 512):
             a = torch.randn((m, k), device=dev, generator=gen).to(act_dtype)
+            a_scales = None
+            if name.startswith("w4a8"):
+                a, a_scales = (ops.per_token_quant_int8 if name == "w4a8_int8" else ops.per_token_quant_fp8)(a)
+                a_scales = a_scales * (2.0 ** -12 if name == "w4a8_int8" else 1.0)
 
-            def one(i=0, a=a, m=m, name=name):
+            def one(i=0, a=a, m=m, name=name, a_scales=a_scales):
                 qw, sc, zp, g_idx, perm, ws, wt = layers[i % len(layers)]
+                if a_scales is not None:
+                    ops.marlin_gemm(a, None, qw, None, sc, a_scales, None, None, None, None, ws, wt, m, n, k, True,
+                                    False, True, False)
+                    return
                 if name == "nvfp4":   # the third entry is the global scale
                     ops.marlin_gemm(a, None, qw, None, sc, None, zp, None, g_idx, perm, ws, wt, m, n, k, True,
                                     False, True, False)
@@ -255,11 +273,14 @@ def variants_sweep(torch, ops, gen, time_graph):
                 nb += (k // 32 - 2 * (k // GROUP)) * n  # a byte per 32 rows instead of two per 128
             if name == "nvfp4":
                 nb += (k // 16 - 2 * (k // GROUP)) * n  # a byte per 16 rows
+            if a_scales is not None:
+                nb += 4 * m - m * k                     # a byte per activation instead of two, a scale per row
             fl = 2 * m * k * n
+            peak = MFMA_PEAK_8BIT_TFLOPS if a_scales is not None else MFMA_PEAK_TFLOPS
             out.append({"variant": name, "m": m, "k": k, "n": n, "us": round(s * 1e6, 2),
                         "GBps": round(nb / s / 1e9, 1), "TFLOPs": round(fl / s / 1e12, 2),
                         "frac_hbm": round(nb / s / 1e9 / HBM_PEAK_GBPS, 4),
-                        "frac_mfma": round(fl / s / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+                        "frac_mfma": round(fl / s / 1e12 / peak, 4)})
             print("variant", json.dumps(out[-1]), file=sys.stderr, flush=True)
     return out
 

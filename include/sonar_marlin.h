@@ -234,6 +234,24 @@ int sonar_marlin_gemm_a8(const void* a, int64_t a_row_stride, int a_dtype, void*
                          int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
                          void* stream);
 
+/* The grouped (mixture-of-experts) form of sonar_marlin_gemm_a8: _moe_C::moe_wna16_marlin_gemm called
+ * with int8 / float8_e4m3fn activations and a_scales (moe/marlin_moe_wna16/marlin_template.h:471-560,
+ * 622-650,2020-2060).  Row id of sorted_token_ids: row id / top_k of a and of a_scales, row id of c
+ * and of topk_weights.
+ *   a          [size_m][size_k] bytes, contiguous, 8-byte aligned;  a_scales float[size_m]
+ *   c          dtype[size_m * top_k][size_n]; rows of blocks whose expert id is outside
+ *              [0, num_experts) are left untouched
+ *   b_q_weight, b_scales, b_zeros, b_bias: as for sonar_marlin_gemm_a8 with a leading expert dimension
+ * Every (block, 64-column strip) is one workgroup over the whole of K; no scratch.  The other
+ * arguments as for sonar_moe_wna16_marlin_gemm. */
+int sonar_moe_wna16_marlin_gemm_a8(
+    const void* a, int a_dtype, void* c, const uint32_t* b_q_weight, int b_layout,
+    const void* b_bias, const void* b_scales, const float* a_scales, const uint32_t* b_zeros,
+    const int32_t* sorted_token_ids, int64_t sorted_len, const int32_t* expert_ids,
+    const int32_t* num_tokens_past_padded, const float* topk_weights, int64_t moe_block_size,
+    int64_t top_k, int mul_topk_weights, int64_t num_experts, int dtype, int64_t b_type_id,
+    int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, void* stream);
+
 /* NVFP4 (marlin.cu:600-611,784-796 of the reference; marlin_template.h:1661-1665;
  * marlin_utils_fp4.py:59-151): float4_e2m1f codes (b_q_weight as for the other 4-bit types),
  * one block scale per 16 rows and column, and one global scale.

@@ -1145,6 +1145,36 @@ def moe_gemm_reference(a32: np.ndarray, w32_per_expert, sorted_ids: np.ndarray,
     return out
 
 
+def moe_gemm_w4a8_int8(a_q: np.ndarray, a_scales: np.ndarray, experts, sorted_ids: np.ndarray,
+                       expert_ids: np.ndarray, num_post_pad: int, block_size: int, top_k: int,
+                       topk_weights: np.ndarray | None, dtype: str) -> np.ndarray:
+    """moe_wna16_marlin_gemm with int8 activations: for every valid slot id of block b,
+    C[id] = gemm_w4a8_int8(row id // top_k of A with its scale, expert expert_ids[b]),
+    then optionally times dtype(topk_weights[id]) in dtype arithmetic
+    (moe/marlin_moe_wna16/marlin_template.h:471-560,622-650,1883-1909).  `experts`: one
+    dict per expert with q, group_size, scales, zeros (or None), bias32 (or None)."""
+    size_m = a_q.shape[0]
+    n = experts[0]["q"].shape[1]
+    out = np.zeros((size_m * top_k, n), dtype=np.float32)
+    for b in range(num_post_pad // block_size):
+        e = int(expert_ids[b])
+        if e < 0 or e >= len(experts):
+            continue
+        ids = sorted_ids[b * block_size:(b + 1) * block_size]
+        ids = ids[ids < size_m * top_k]
+        if ids.size == 0:
+            continue
+        rows = ids // top_k
+        ex = experts[e]
+        c = gemm_w4a8_int8(a_q[rows], a_scales.reshape(-1)[rows], ex["q"], ex["group_size"], ex["scales"], dtype,
+                           ex.get("zeros"), ex.get("bias32"))
+        if topk_weights is not None:
+            wts = round_to_dtype(topk_weights.reshape(-1)[ids].astype(np.float32), dtype)
+            c = round_to_dtype(c * wts[:, None], dtype)
+        out[ids, :] = c
+    return out
+
+
 # --------------------------------------------------------------------------
 # CPU baseline of the layer: int4 dequantise + torch.matmul in fp32
 # --------------------------------------------------------------------------

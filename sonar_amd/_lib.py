@@ -48,6 +48,10 @@ PROTOTYPES = {
     "sonar_marlin_gemm_a8": (c_int, [c_void_p, c_int64, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p,
                                      c_void_p, c_void_p, c_void_p, c_size_t, c_int, c_int64, c_int64, c_int64,
                                      c_int64, c_int64, c_void_p]),
+    "sonar_moe_wna16_marlin_gemm_a8": (c_int, [
+        c_void_p, c_int, c_void_p, c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_void_p, c_int64,
+        c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_int64, c_int, c_int64, c_int64, c_int64, c_int64,
+        c_int64, c_void_p]),
     "sonar_marlin_dequant": (c_int, [c_void_p, c_int, c_void_p, c_void_p, c_void_p, c_void_p, c_int,
                                      c_int64, c_int64, c_int64, c_int64, c_int, c_void_p]),
     "sonar_marlin_gemm_scratch_bytes": (c_size_t, [c_int64, c_int64, c_int64]),

@@ -131,6 +131,105 @@ __device__ __forceinline__ uint16_t finish(typename ACT::scalar_t total, float a
   return to_bits<T>(f);
 }
 
+// The sum over this wavefront's share of K: groups (units) u_begin + wave, + 4, ... of
+// [u_begin, u_end).  a_row[rb]: this lane's row of A in row block rb, already offset by the
+// lane's 8 bytes inside a chunk; w_lane: the lane's 16 bytes of chunk 0 of the strip;
+// scales / zeros: row 0 of the matrix's (the expert's) scales and zero points.
+template <typename ACT, typename T, int MB, bool HAS_ZP, bool GROUPED>
+__device__ __forceinline__ void a8_accumulate(typename ACT::acc_t (&acc)[MB][4], const uint8_t* const (&a_row)[MB],
+                                              const uint32_t* w_lane, const uint16_t* scales,
+                                              const uint32_t* zeros, int n, int strip, int chunks, int unit_chunks,
+                                              int u_begin, int u_end, int wave, int l16) {
+  typedef typename ACT::acc_t acc_t;
+  typedef typename ACT::scalar_t scalar_t;
+  int s_col[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) s_col[j] = strip * kStripN + scale_slot(16 * j + l16, false);
+  for (int u = u_begin + wave; u < u_end; u += 4) {
+    acc_t tmp[MB][4];
+#pragma unroll
+    for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) tmp[rb][j] = acc_t{0, 0, 0, 0};
+    const int g = GROUPED ? u : 0;
+    uint32_t z4[4] = {0, 0, 0, 0};
+    if (HAS_ZP) {
+      // column 16j + l16 of the strip: word l16 % 8 of the strip's eight, nibble 2j + l16 / 8
+      const uint32_t zw = zeros[(long)g * (n / 8) + strip * 8 + (l16 & 7)];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) z4[j] = ((zw >> (4 * (2 * j + (l16 >> 3)))) & 0xFu) * 0x01010101u;
+    }
+    const int c_begin = u * unit_chunks;
+    const int c_end = min(c_begin + unit_chunks, chunks);
+    for (int c = c_begin; c < c_end; ++c) {
+      const u32x4_t w4 = *reinterpret_cast<const u32x4_t*>(w_lane + (long)c * kChunkWords);
+      long a[MB];
+#pragma unroll
+      for (int rb = 0; rb < MB; ++rb) {
+        const uint2 v = *reinterpret_cast<const uint2*>(a_row[rb] + (long)c * kChunkK);
+        const uint32_t lo = __builtin_amdgcn_perm(v.y, v.x, 0x05010400u);   // bytes k = 0, 4, 1, 5
+        const uint32_t hi = __builtin_amdgcn_perm(v.y, v.x, 0x07030602u);   // bytes k = 2, 6, 3, 7
+        a[rb] = (long)(((uint64_t)hi << 32) | lo);
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const long b = HAS_ZP ? ACT::word_zp(w4[j], z4[j]) : ACT::word(w4[j]);
+#pragma unroll
+        for (int rb = 0; rb < MB; ++rb) tmp[rb][j] = ACT::mfma(a[rb], b, tmp[rb][j]);
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      scalar_t s = 1;
+      if (GROUPED) {
+        const uint16_t bits = scales[(long)g * n + s_col[j]];
+        if constexpr (ACT::kInteger) s = (int)bits;   // read as unsigned (marlin_template.h:1341-1348)
+        else s = from_bits<T>(bits);
+      }
+#pragma unroll
+      for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if constexpr (ACT::kInteger)
+            acc[rb][j][i] += (tmp[rb][j][i] >> (HAS_ZP ? 0 : ACT::kShift)) * s;
+          else
+            acc[rb][j][i] += tmp[rb][j][i] * s;
+        }
+    }
+  }
+}
+
+// The four wavefronts' totals meet in LDS; afterwards wavefront w holds, in total[rb][i], the
+// sums of column block w: row 16 rb + 4 (lane / 16) + i, column 16 w + lane % 16 of the tile.
+template <typename ACT, int MB>
+__device__ __forceinline__ void a8_reduce(const typename ACT::acc_t (&acc)[MB][4], uint32_t (&red)[4][MB * 16][64],
+                                          typename ACT::scalar_t (&total)[MB][4], int wave, int lane) {
+  typedef typename ACT::scalar_t scalar_t;
+#pragma unroll
+  for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const scalar_t v = acc[rb][j][i];
+        red[wave][(rb * 4 + j) * 4 + i][lane] = raw_bits(v);
+      }
+  __syncthreads();
+#pragma unroll
+  for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      scalar_t sum = 0;
+#pragma unroll
+      for (int ww = 0; ww < 4; ++ww) {
+        scalar_t part;
+        from_raw(red[ww][(rb * 4 + wave) * 4 + i][lane], part);
+        sum += part;
+      }
+      total[rb][i] = sum;
+    }
+}
+
 template <typename ACT, typename T, int MB, bool HAS_ZP, bool GROUPED>
 __global__ __launch_bounds__(256) void marlin_a8_kernel(A8Params p) {
   typedef typename ACT::acc_t acc_t;
@@ -157,76 +256,13 @@ __global__ __launch_bounds__(256) void marlin_a8_kernel(A8Params p) {
     a_row[rb] = p.a + (long)row * p.a_row_stride + 8 * kb;
   }
   const uint32_t* w_lane = p.w + (long)strip * p.chunks * kChunkWords + lane * 4;
-  int s_col[4];
-#pragma unroll
-  for (int j = 0; j < 4; ++j) s_col[j] = strip * kStripN + scale_slot(16 * j + l16, false);
-
   const int u_begin = split * p.units_per_split;
   const int u_end = min(u_begin + p.units_per_split, p.units);
-  for (int u = u_begin + wave; u < u_end; u += 4) {
-    acc_t tmp[MB][4];
-#pragma unroll
-    for (int rb = 0; rb < MB; ++rb)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) tmp[rb][j] = acc_t{0, 0, 0, 0};
-    const int g = GROUPED ? u : 0;
-    uint32_t z4[4] = {0, 0, 0, 0};
-    if (HAS_ZP) {
-      // column 16j + l16 of the strip: word l16 % 8 of the strip's eight, nibble 2j + l16 / 8
-      const uint32_t zw = p.zeros[(long)g * (p.n / 8) + strip * 8 + (l16 & 7)];
-#pragma unroll
-      for (int j = 0; j < 4; ++j) z4[j] = ((zw >> (4 * (2 * j + (l16 >> 3)))) & 0xFu) * 0x01010101u;
-    }
-    const int c_begin = u * p.unit_chunks;
-    const int c_end = min(c_begin + p.unit_chunks, p.chunks);
-    for (int c = c_begin; c < c_end; ++c) {
-      const u32x4_t w4 = *reinterpret_cast<const u32x4_t*>(w_lane + (long)c * kChunkWords);
-      long a[MB];
-#pragma unroll
-      for (int rb = 0; rb < MB; ++rb) {
-        const uint2 v = *reinterpret_cast<const uint2*>(a_row[rb] + (long)c * kChunkK);
-        const uint32_t lo = __builtin_amdgcn_perm(v.y, v.x, 0x05010400u);   // bytes k = 0, 4, 1, 5
-        const uint32_t hi = __builtin_amdgcn_perm(v.y, v.x, 0x07030602u);   // bytes k = 2, 6, 3, 7
-        a[rb] = (long)(((uint64_t)hi << 32) | lo);
-      }
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const long b = HAS_ZP ? ACT::word_zp(w4[j], z4[j]) : ACT::word(w4[j]);
-#pragma unroll
-        for (int rb = 0; rb < MB; ++rb) tmp[rb][j] = ACT::mfma(a[rb], b, tmp[rb][j]);
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      scalar_t s = 1;
-      if (GROUPED) {
-        const uint16_t bits = p.scales[(long)g * p.n + s_col[j]];
-        if constexpr (ACT::kInteger) s = (int)bits;   // read as unsigned (marlin_template.h:1341-1348)
-        else s = from_bits<T>(bits);
-      }
-#pragma unroll
-      for (int rb = 0; rb < MB; ++rb)
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          if constexpr (ACT::kInteger)
-            acc[rb][j][i] += (tmp[rb][j][i] >> (HAS_ZP ? 0 : ACT::kShift)) * s;
-          else
-            acc[rb][j][i] += tmp[rb][j][i] * s;
-        }
-    }
-  }
+  a8_accumulate<ACT, T, MB, HAS_ZP, GROUPED>(acc, a_row, w_lane, p.scales, p.zeros, p.n, strip, p.chunks,
+                                             p.unit_chunks, u_begin, u_end, wave, l16);
+  scalar_t total[MB][4];
+  a8_reduce<ACT, MB>(acc, red, total, wave, lane);
 
-  // the four wavefronts' totals meet in LDS; wavefront w sums column block w
-#pragma unroll
-  for (int rb = 0; rb < MB; ++rb)
-#pragma unroll
-    for (int j = 0; j < 4; ++j)
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const scalar_t v = acc[rb][j][i];
-        red[wave][(rb * 4 + j) * 4 + i][lane] = raw_bits(v);
-      }
-  __syncthreads();
   const int col = strip * kStripN + 16 * wave + l16;
   float col_scale = 1.0f, bias = 0.0f;
   if (p.splits == 1) {
@@ -238,20 +274,92 @@ __global__ __launch_bounds__(256) void marlin_a8_kernel(A8Params p) {
   for (int rb = 0; rb < MB; ++rb)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      scalar_t total = 0;
-#pragma unroll
-      for (int ww = 0; ww < 4; ++ww) {
-        scalar_t part;
-        from_raw(red[ww][(rb * 4 + wave) * 4 + i][lane], part);
-        total += part;
-      }
       const int row = m0 + 16 * rb + 4 * kb + i;
       if (row >= p.m) continue;
       if (p.splits == 1)
         reinterpret_cast<uint16_t*>(p.c)[(long)row * p.n + col] =
-            finish<ACT, T, GROUPED>(total, p.a_scales[row], col_scale, bias);
+            finish<ACT, T, GROUPED>(total[rb][i], p.a_scales[row], col_scale, bias);
       else
-        p.partial[((long)split * p.m + row) * p.n + col] = raw_bits(total);
+        p.partial[((long)split * p.m + row) * p.n + col] = raw_bits(total[rb][i]);
+    }
+}
+
+// Grouped (mixture-of-experts) form: workgroup (strip, block) takes the rows
+// sorted_token_ids[block * block_size ...] (row id / top_k of A, row id of C and of
+// topk_weights, a_scales[id / top_k]; ids >= size_m * top_k are padding) and the expert
+// expert_ids[block] (moe/marlin_moe_wna16/marlin_template.h:471-560,622-650), over the whole of K.
+struct MoeA8Params {
+  A8Params g;              // m = size_m (rows of A); a_scales per row of A
+  const int32_t* sorted_ids;
+  const int32_t* expert_ids;
+  const int32_t* num_post_pad;
+  const float* topk_weights;
+  int block_size, top_k, mul_topk, num_experts, groups, sorted_len;
+};
+
+template <typename ACT, typename T, int MB, bool HAS_ZP, bool GROUPED>
+__global__ __launch_bounds__(256) void marlin_moe_a8_kernel(MoeA8Params q) {
+  typedef typename ACT::acc_t acc_t;
+  typedef typename ACT::scalar_t scalar_t;
+  __shared__ uint32_t red[4][MB * 16][64];
+  __shared__ int slot_id[16 * MB];
+  const A8Params& p = q.g;
+
+  const int strip = blockIdx.x, block = blockIdx.y;
+  const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+  const int l16 = lane & 15, kb = lane >> 4;
+  // the whole workgroup leaves together: nothing below is reached by a part of it
+  if (block * q.block_size >= q.num_post_pad[0]) return;
+  const int expert = q.expert_ids[block];
+  if (expert < 0 || expert >= q.num_experts) return;
+
+  const int rows_total = p.m * q.top_k;
+  if (threadIdx.x < 16 * MB) {
+    int id = -1;
+    const int at = block * q.block_size + (int)threadIdx.x;
+    if ((int)threadIdx.x < q.block_size && at < q.sorted_len) {
+      id = q.sorted_ids[at];
+      if (id < 0 || id >= rows_total) id = -1;
+    }
+    slot_id[threadIdx.x] = id;
+  }
+  __syncthreads();
+
+  acc_t acc[MB][4];
+#pragma unroll
+  for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[rb][j] = acc_t{0, 0, 0, 0};
+  const uint8_t* a_row[MB];
+#pragma unroll
+  for (int rb = 0; rb < MB; ++rb) {
+    const int id = slot_id[16 * rb + l16];
+    a_row[rb] = p.a + (long)(id < 0 ? 0 : id / q.top_k) * p.a_row_stride + 8 * kb;   // padding reads row 0
+  }
+  const long words_per_expert = (long)p.chunks * kChunkWords * (p.n / kStripN);
+  const uint32_t* w_lane = p.w + expert * words_per_expert + (long)strip * p.chunks * kChunkWords + lane * 4;
+  const uint16_t* scales = p.scales + (long)expert * q.groups * p.n;
+  const uint32_t* zeros = HAS_ZP ? p.zeros + (long)expert * q.groups * (p.n / 8) : nullptr;
+  a8_accumulate<ACT, T, MB, HAS_ZP, GROUPED>(acc, a_row, w_lane, scales, zeros, p.n, strip, p.chunks,
+                                             p.unit_chunks, 0, p.units, wave, l16);
+  scalar_t total[MB][4];
+  a8_reduce<ACT, MB>(acc, red, total, wave, lane);
+
+  const int col = strip * kStripN + 16 * wave + l16;
+  const int slot = strip * kStripN + scale_slot(16 * wave + l16, false);
+  const float col_scale = GROUPED ? 1.0f : from_bits<T>(scales[slot]);
+  const float bias = p.bias ? from_bits<T>(p.bias[(long)expert * p.n + slot]) : 0.0f;
+#pragma unroll
+  for (int rb = 0; rb < MB; ++rb)
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int id = slot_id[16 * rb + 4 * kb + i];
+      if (id < 0) continue;
+      uint16_t o = finish<ACT, T, GROUPED>(total[rb][i], p.a_scales[id / q.top_k], col_scale, bias);
+      // the routing weight is rounded to the output type and the product is formed and rounded in
+      // that type (marlin_template.h:1893-1897), as in the 16-bit grouped kernels
+      if (q.mul_topk) o = to_bits<T>(from_bits<T>(o) * from_bits<T>(to_bits<T>(q.topk_weights[id])));
+      reinterpret_cast<uint16_t*>(p.c)[(long)id * p.n + col] = o;
     }
 }
 
@@ -328,10 +436,100 @@ void launch_a8(const A8Params& p, const A8Plan& plan, bool grouped, hipStream_t 
   }
 }
 
+template <typename ACT, typename T, int MB>
+void launch_moe_a8_mb(const MoeA8Params& q, bool grouped, bool zp, dim3 grid, hipStream_t st) {
+  if (grouped) {
+    if (zp) marlin_moe_a8_kernel<ACT, T, MB, true, true><<<grid, 256, 0, st>>>(q);
+    else marlin_moe_a8_kernel<ACT, T, MB, false, true><<<grid, 256, 0, st>>>(q);
+  } else {
+    if (zp) marlin_moe_a8_kernel<ACT, T, MB, true, false><<<grid, 256, 0, st>>>(q);
+    else marlin_moe_a8_kernel<ACT, T, MB, false, false><<<grid, 256, 0, st>>>(q);
+  }
+}
+
+template <typename ACT, typename T>
+void launch_moe_a8(const MoeA8Params& q, bool grouped, int blocks, hipStream_t st) {
+  const dim3 grid(q.g.n / kStripN, blocks, 1);
+  const bool zp = q.g.zeros != nullptr;
+  switch ((q.block_size + 15) / 16) {
+    case 1: launch_moe_a8_mb<ACT, T, 1>(q, grouped, zp, grid, st); break;
+    case 2: launch_moe_a8_mb<ACT, T, 2>(q, grouped, zp, grid, st); break;
+    case 3: launch_moe_a8_mb<ACT, T, 3>(q, grouped, zp, grid, st); break;
+    default: launch_moe_a8_mb<ACT, T, 4>(q, grouped, zp, grid, st); break;
+  }
+}
+
+// Checks shared by the dense and the grouped entry point.
+int check_a8(int a_dtype, int dtype, int b_layout, int64_t b_type_id, int64_t size_m, int64_t size_n, int64_t size_k,
+             int64_t num_groups, const uint32_t* b_zeros) {
+  if (int rc = check_a8(a_dtype, dtype, b_layout, b_type_id, size_m, size_n, size_k, num_groups, b_zeros)) return rc;
+  return SONAR_OK;
+}
+
 }  // namespace
 }  // namespace sonar
 
 using namespace sonar;
+
+extern "C" int sonar_moe_wna16_marlin_gemm_a8(
+    const void* a, int a_dtype, void* c, const uint32_t* b_q_weight, int b_layout, const void* b_bias,
+    const void* b_scales, const float* a_scales, const uint32_t* b_zeros, const int32_t* sorted_token_ids,
+    int64_t sorted_len, const int32_t* expert_ids, const int32_t* num_tokens_past_padded, const float* topk_weights,
+    int64_t moe_block_size, int64_t top_k, int mul_topk_weights, int64_t num_experts, int dtype, int64_t b_type_id,
+    int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, void* stream) {
+  if (int rc = check_a8(a_dtype, dtype, b_layout, b_type_id, size_m, size_n, size_k, num_groups, b_zeros)) return rc;
+  SONAR_REQUIRE(moe_block_size == 8 || (moe_block_size % 16 == 0 && moe_block_size >= 16 && moe_block_size <= 64),
+                "unsupported moe_block_size = %ld", (long)moe_block_size);
+  SONAR_REQUIRE(top_k >= 1 && num_experts >= 1, "top_k = %ld, num_experts = %ld", (long)top_k, (long)num_experts);
+  SONAR_REQUIRE(sorted_len >= 0 && sorted_len < (1LL << 31), "sorted_token_ids has %ld entries", (long)sorted_len);
+  SONAR_REQUIRE(!mul_topk_weights || topk_weights, "topk_weights must be given with mul_topk_weights");
+  if (size_m == 0 || sorted_len == 0) return SONAR_OK;
+  SONAR_REQUIRE(a && c && b_q_weight && b_scales && a_scales && sorted_token_ids && expert_ids &&
+                    num_tokens_past_padded,
+                "a, c, b_q_weight, b_scales, a_scales, sorted_token_ids, expert_ids and num_tokens_past_padded "
+                "must not be NULL");
+  SONAR_REQUIRE((uintptr_t)a % 8 == 0, "A must be aligned to 8 bytes");
+  const int64_t blocks = (sorted_len + moe_block_size - 1) / moe_block_size;
+  SONAR_REQUIRE(blocks <= 65535, "too many blocks of sorted tokens: %ld", (long)blocks);
+  MoeA8Params q;
+  A8Params& p = q.g;
+  p.a = (const uint8_t*)a;
+  p.a_row_stride = size_k;
+  p.c = c;
+  p.w = b_q_weight;
+  p.scales = (const uint16_t*)b_scales;
+  p.zeros = b_zeros;
+  p.a_scales = a_scales;
+  p.bias = (const uint16_t*)b_bias;
+  p.partial = nullptr;
+  p.m = (int)size_m;
+  p.n = (int)size_n;
+  p.chunks = (int)(size_k / kChunkK);
+  p.unit_chunks = num_groups > 1 ? (int)(size_k / num_groups) / kChunkK : 4;
+  p.units = (p.chunks + p.unit_chunks - 1) / p.unit_chunks;
+  p.units_per_split = p.units;
+  p.splits = 1;
+  q.sorted_ids = sorted_token_ids;
+  q.expert_ids = expert_ids;
+  q.num_post_pad = num_tokens_past_padded;
+  q.topk_weights = topk_weights;
+  q.block_size = (int)moe_block_size;
+  q.top_k = (int)top_k;
+  q.mul_topk = mul_topk_weights ? 1 : 0;
+  q.num_experts = (int)num_experts;
+  q.groups = (int)num_groups;
+  q.sorted_len = (int)sorted_len;
+  const bool grouped = num_groups > 1;
+  hipStream_t st = (hipStream_t)stream;
+  if (a_dtype == SONAR_ADTYPE_INT8) {
+    if (dtype == SONAR_DTYPE_F16) launch_moe_a8<ActInt8, _Float16>(q, grouped, (int)blocks, st);
+    else launch_moe_a8<ActInt8, __bf16>(q, grouped, (int)blocks, st);
+  } else {
+    if (dtype == SONAR_DTYPE_F16) launch_moe_a8<ActFp8, _Float16>(q, grouped, (int)blocks, st);
+    else launch_moe_a8<ActFp8, __bf16>(q, grouped, (int)blocks, st);
+  }
+  return launch_status("marlin_moe_a8_kernel");
+}
 
 extern "C" size_t sonar_marlin_gemm_a8_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k,
                                                      int64_t num_groups) {

@@ -701,6 +701,110 @@ Tensor marlin_gemm(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_
 }
 
 // ---------------------------------------------------------------- grouped GEMM
+// 8-bit activations (moe/marlin_moe_wna16/ops.cu: the same type resolution as marlin.cu:567-598).
+Tensor moe_wna16_marlin_gemm_a8(const Tensor& a, const OptTensor& c_or_none, const Tensor& b_q_weight,
+                                const OptTensor& b_bias_or_none, const Tensor& b_scales, const OptTensor& a_scales,
+                                const OptTensor& global_scale, const OptTensor& b_zeros_or_none,
+                                const OptTensor& g_idx_or_none, const Tensor& sorted_token_ids,
+                                const Tensor& expert_ids, const Tensor& num_tokens_past_padded,
+                                const Tensor& topk_weights, int64_t moe_block_size, int64_t top_k,
+                                bool mul_topk_weights, int64_t b_type_id, int64_t size_m, int64_t size_n,
+                                int64_t size_k, bool is_zp_float) {
+  const int a_dtype = a.scalar_type() == at::kChar ? SONAR_ADTYPE_INT8 : SONAR_ADTYPE_FP8;
+  check_b_type(b_type_id);
+  TORCH_CHECK_NOT_IMPLEMENTED(b_type_id != SONAR_TYPE_FLOAT4_E2M1F,
+                              "float4_e2m1f weights with float8_e4m3fn activations (W4A8-FP4) are not built");
+  TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4,
+              a_dtype == SONAR_ADTYPE_INT8 ? "W8A8-INT8 is not supported by marlin kernel."
+                                           : "INT8 weight + FP8 activation is not supported.");
+  TORCH_CHECK(b_scales.scalar_type() == at::kHalf || b_scales.scalar_type() == at::kBFloat16,
+              "b_scales must be float16 or bfloat16 with 8-bit activations (their type is the type of c)");
+  const int dtype = b_scales.scalar_type() == at::kHalf ? SONAR_DTYPE_F16 : SONAR_DTYPE_BF16;
+  TORCH_CHECK(a_scales.has_value() && a_scales->numel() > 0,
+              "the a_scales parameter must be passed for 8bit activation.");
+  TORCH_CHECK(a_scales->is_cuda() && a_scales->scalar_type() == at::kFloat && a_scales->is_contiguous(),
+              "scalar type of a_scales must be float");
+  TORCH_CHECK(a_scales->numel() == size_m, "a_scales must hold one scale per row of a; got ", a_scales->numel(),
+              " for size_m = ", size_m);
+  TORCH_CHECK(!(global_scale.has_value() && global_scale->numel() > 0),
+              "global_scale can only be used for nvfp4 format.");
+  TORCH_CHECK_NOT_IMPLEMENTED(!is_zp_float, "is_zp_float = True is not built");
+  TORCH_CHECK(!(g_idx_or_none.has_value() && g_idx_or_none->numel() > 0),
+              "act-order is not supported with 8-bit activations (the reference builds no such kernel)");
+  TORCH_CHECK(moe_block_size == 8 || moe_block_size % 16 == 0, "unsupported moe_block_size=", moe_block_size);
+  TORCH_CHECK(moe_block_size >= 8 && moe_block_size <= 64, "unsupported moe_block_size=", moe_block_size);
+  TORCH_CHECK(a.dim() == 2 && a.size(0) == size_m, "Shape mismatch: a.size(0) = ", a.size(0),
+              ", size_m = ", size_m);
+  TORCH_CHECK(a.size(1) == size_k, "Shape mismatch: a.size(1) = ", a.size(1), ", size_k = ", size_k);
+  TORCH_CHECK(a.is_cuda() && a.is_contiguous(), "A is not a contiguous GPU tensor");
+  TORCH_CHECK(b_q_weight.dim() == 3, "b_q_weight must be (E, K/16, 2N)");
+  const int64_t experts = b_q_weight.size(0);
+  TORCH_CHECK(size_k % 32 == 0 && size_k / 16 == b_q_weight.size(1),
+              "Shape mismatch: b_q_weight.size(1) = ", b_q_weight.size(1), ", size_k = ", size_k,
+              ", tile_size = ", 16);
+  TORCH_CHECK(b_q_weight.size(2) % 16 == 0 && b_q_weight.size(2) / 16 * 8 == size_n,
+              "size_n = ", size_n, ", actual_size_n = ", b_q_weight.size(2) / 16 * 8);
+  TORCH_CHECK(b_q_weight.is_cuda() && b_q_weight.is_contiguous() && b_q_weight.scalar_type() == at::kInt,
+              "b_q_weight must be a contiguous int32 GPU tensor");
+  TORCH_CHECK(b_scales.is_cuda() && b_scales.is_contiguous(), "b_scales is not a contiguous GPU tensor");
+  TORCH_CHECK(b_scales.dim() == 3 && b_scales.size(0) == experts, "b_scales rank = ", b_scales.dim(), " is not 3");
+  TORCH_CHECK(b_scales.size(2) == size_n, "b_scales dim 2 = ", b_scales.size(2), " is not size_n = ", size_n);
+  const int64_t num_groups = b_scales.size(1);
+
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(a.device());
+  Tensor c;
+  if (c_or_none.has_value()) {
+    c = c_or_none.value();
+    TORCH_CHECK(c.is_cuda() && c.is_contiguous(), "c is not a contiguous GPU tensor");
+    TORCH_CHECK(c.size(0) == size_m * top_k, "Shape mismatch: c.size(0) = ", c.size(0),
+                ", size_m * topk = ", size_m * top_k);
+    TORCH_CHECK(c.size(1) == size_n, "Shape mismatch: c.size(1) = ", c.size(1), ", size_n = ", size_n);
+    TORCH_CHECK(c.scalar_type() == b_scales.scalar_type(), "c must have the type of b_scales with 8-bit activations");
+  } else {
+    c = at::empty({size_m * top_k, size_n}, b_scales.options());
+  }
+  if (size_m == 0) return c;
+  if (b_bias_or_none.has_value()) {
+    const Tensor& b = b_bias_or_none.value();
+    TORCH_CHECK(b.is_cuda() && b.is_contiguous(), "b_bias is not a contiguous GPU tensor");
+    TORCH_CHECK(b.size(-1) == size_n, "b_bias.size(-1) != size_n");
+    TORCH_CHECK(b.scalar_type() == c.scalar_type(), "b_bias must have the dtype of c");
+  }
+  const bool has_zp = b_zeros_or_none.has_value() && b_zeros_or_none->size(-1) > 0;
+  if (has_zp) {
+    const Tensor& z = b_zeros_or_none.value();
+    TORCH_CHECK(z.is_cuda() && z.is_contiguous() && z.scalar_type() == at::kInt,
+                "b_zeros must be a contiguous int32 GPU tensor");
+    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4, "b_type must be u4 or u8 when has_zp = True. Got = uint4b8");
+    TORCH_CHECK(z.dim() == 3 && z.size(1) == num_groups && z.size(2) == size_n / 8,
+                "b_zeros must be (E, num_groups, size_n / 8)");
+  } else {
+    TORCH_CHECK(b_type_id != SONAR_TYPE_UINT4,
+                "b_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False. Got = uint4");
+  }
+  TORCH_CHECK(sorted_token_ids.is_cuda() && sorted_token_ids.scalar_type() == at::kInt &&
+                  sorted_token_ids.is_contiguous(), "sorted_token_ids must be a contiguous int32 GPU tensor");
+  TORCH_CHECK(expert_ids.is_cuda() && expert_ids.scalar_type() == at::kInt && expert_ids.is_contiguous(),
+              "expert_ids must be a contiguous int32 GPU tensor");
+  TORCH_CHECK(num_tokens_past_padded.is_cuda() && num_tokens_past_padded.scalar_type() == at::kInt,
+              "num_tokens_past_padded must be an int32 GPU tensor");
+  TORCH_CHECK(topk_weights.is_cuda() && topk_weights.scalar_type() == at::kFloat &&
+                  topk_weights.is_contiguous(), "topk_weights must be a contiguous float32 GPU tensor");
+
+  Tensor native = native_weights(b_q_weight, size_k, size_n, experts, 4, /*a8=*/true);
+  raise_if_failed(sonar_moe_wna16_marlin_gemm_a8(
+      a.const_data_ptr(), a_dtype, c.mutable_data_ptr(), static_cast<const uint32_t*>(native.const_data_ptr()),
+      SONAR_LAYOUT_GFX950, opt_ptr(b_bias_or_none), b_scales.const_data_ptr(),
+      static_cast<const float*>(a_scales->const_data_ptr()),
+      has_zp ? static_cast<const uint32_t*>(b_zeros_or_none->const_data_ptr()) : nullptr,
+      static_cast<const int32_t*>(sorted_token_ids.const_data_ptr()), sorted_token_ids.numel(),
+      static_cast<const int32_t*>(expert_ids.const_data_ptr()),
+      static_cast<const int32_t*>(num_tokens_past_padded.const_data_ptr()),
+      static_cast<const float*>(topk_weights.const_data_ptr()), moe_block_size, top_k, mul_topk_weights ? 1 : 0,
+      experts, dtype, b_type_id, size_m, size_n, size_k, num_groups, current_stream(a)));
+  return c;
+}
+
 Tensor moe_wna16_marlin_gemm(
     Tensor& a, const OptTensor& c_or_none, Tensor& b_q_weight, const OptTensor& b_bias_or_none,
     Tensor& b_scales, const OptTensor& a_scales, const OptTensor& global_scale,
@@ -713,9 +817,15 @@ Tensor moe_wna16_marlin_gemm(
   (void)thread_k;
   (void)thread_n;
   (void)blocks_per_sm;
+  if (a.scalar_type() == at::kChar || a.scalar_type() == at::kFloat8_e4m3fn)
+    return moe_wna16_marlin_gemm_a8(a, c_or_none, b_q_weight, b_bias_or_none, b_scales, a_scales, global_scale,
+                                    b_zeros_or_none, g_idx_or_none, sorted_token_ids, expert_ids,
+                                    num_tokens_past_padded, topk_weights, moe_block_size, top_k, mul_topk_weights,
+                                    b_type_id, size_m, size_n, size_k, is_zp_float);
+  TORCH_CHECK(a.scalar_type() == at::kHalf || a.scalar_type() == at::kBFloat16, "unsupported `a` scalar_type");
   const int dtype = dtype_code(a);
   check_b_type(b_type_id);
-  TORCH_CHECK_NOT_IMPLEMENTED(!a_scales.has_value(), "a_scales can only be used for 8bit activation.");
+  TORCH_CHECK(!(a_scales.has_value() && a_scales->numel() > 0), "a_scales can only be used for 8bit activation.");
   TORCH_CHECK_NOT_IMPLEMENTED(!is_zp_float, "is_zp_float = True is not built");
   // marlin_moe_wna16/ops.cu: the global scale goes with NVFP4 and only with it
   const bool nvfp4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F && b_scales.scalar_type() == at::kFloat8_e4m3fn;

@@ -18,7 +18,7 @@ import math
 import torch
 
 from . import ops
-from .marlin_utils import marlin_make_workspace_new
+from .marlin_utils import marlin_make_workspace_new, marlin_quant_input
 from .scalar_type import ScalarType, scalar_types
 
 _SUPPORTED = {t.id: t for t in (scalar_types.uint4, scalar_types.uint4b8, scalar_types.uint8b128,
@@ -183,10 +183,12 @@ def _check_unbuilt(activation, clamp_limit, gemm1_alpha, gemm1_beta, input_dtype
         raise NotImplementedError("clamp_limit / gemm1_alpha / gemm1_beta (SWIGLUOAI parameters) are not built")
     if activation_situ_beta is not None or activation_situ_linear_beta is not None:
         raise NotImplementedError("activation_situ_beta / activation_situ_linear_beta are not built")
-    if input_dtype is not None:
-        raise NotImplementedError("8-bit activations (input_dtype) are not built")
-    if any(g is not None for g in global_scales[:2]):
-        raise NotImplementedError("input_global_scale1 / input_global_scale2 (8-bit activations) are not built")
+    if input_dtype is not None and input_dtype not in (torch.int8, torch.float8_e4m3fn, torch.float16,
+                                                       torch.bfloat16):
+        raise ValueError(f"unsupported input_dtype {input_dtype}")
+    if input_dtype != torch.int8 and any(g is not None for g in global_scales[:2]):
+        raise ValueError("input_global_scale1 / input_global_scale2 go with int8 activations (input_dtype = "
+                         "torch.int8) only")
 
 
 def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, num_topk,
@@ -221,8 +223,17 @@ def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, t
     cache3 = intermediate_cache13[:M * num_topk * K].view(M * num_topk, K)
     cache2 = intermediate_cache2.view(-1)[:M * num_topk * N].view(M * num_topk, N)
 
+    # 8-bit activations: one scale per token row, times the factor of the integer group scales
+    # (marlin_moe.py:126-133,181-187)
+    a_scales1 = a_scales2 = None
+    gate_up_input = hidden_states
+    if input_dtype in (torch.int8, torch.float8_e4m3fn):
+        gate_up_input, a_scales1 = marlin_quant_input(hidden_states, input_dtype)
+        if input_dtype == torch.int8 and input_global_scale1 is not None:
+            a_scales1 = a_scales1 * input_global_scale1
     cache1 = ops.moe_wna16_marlin_gemm(
-        hidden_states, cache1, w1, bias1, w1_scale, None, global_scale1, w1_zeros, g_idx1, sort_indices1, workspace,
+        gate_up_input, cache1, w1, bias1, w1_scale, a_scales1, global_scale1, w1_zeros, g_idx1, sort_indices1,
+        workspace,
         sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, moe_block_size=block_size_m,
         top_k=num_topk, mul_topk_weights=apply_router_weight_on_input, b_q_type=quant_type, size_m=M,
         size_n=2 * N, size_k=K, is_k_full=is_k_full, use_atomic_add=False, use_fp32_reduce=True,
@@ -233,8 +244,12 @@ def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, t
         silu_and_mul(cache2, cache1.view(-1, 2 * N))
     if output is None:
         output = cache3
+    if input_dtype in (torch.int8, torch.float8_e4m3fn):
+        cache2, a_scales2 = marlin_quant_input(cache2, input_dtype)
+        if input_dtype == torch.int8 and input_global_scale2 is not None:
+            a_scales2 = a_scales2 * input_global_scale2
     return ops.moe_wna16_marlin_gemm(
-        cache2, output, w2, bias2, w2_scale, None, global_scale2, w2_zeros, g_idx2, sort_indices2, workspace,
+        cache2, output, w2, bias2, w2_scale, a_scales2, global_scale2, w2_zeros, g_idx2, sort_indices2, workspace,
         sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, moe_block_size=block_size_m,
         top_k=1, mul_topk_weights=not apply_router_weight_on_input, b_q_type=quant_type,
         size_m=M * num_topk, size_n=K, size_k=N, is_k_full=is_k_full, use_atomic_add=False,
@@ -265,8 +280,11 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
     w2: (E, N/16, 2K); scales (E, groups, 2N) / (E, groups, K); topk_weights
     fp32 [M, top_k]; topk_ids [M, top_k].  Returns [M, K].  Parameters and their order are
     the reference's; of its activations only SILU is built (anything else, and clamp_limit /
-    gemm1_alpha / gemm1_beta / input global scales / input_dtype, raise NotImplementedError;
-    global_scale1 / global_scale2 are the per-expert global scales of NVFP4 experts).
+    gemm1_alpha / gemm1_beta, raise NotImplementedError; global_scale1 / global_scale2 are the
+    per-expert global scales of NVFP4 experts).  input_dtype torch.int8 / torch.float8_e4m3fn:
+    the tokens and the activation's output are quantised per row and both GEMMs run on the 8-bit
+    matrix cores (4-bit expert weights repacked with is_a_8bit; input_global_scale1 / 2 are the
+    factors marlin_act_int8_process_scales returns for the integer group scales).
     `activation_func(activation, out, in)` and `moe_sum(moe_output [M, top_k, K], output)`
     replace the built-in HIP kernels when given, as in the reference."""
     _check_unbuilt(activation, clamp_limit, gemm1_alpha, gemm1_beta, input_dtype,
@@ -293,6 +311,8 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
     else:
         m_est = math.ceil(M * E / global_num_experts)   # expected tokens for the local experts
     block_size_m = moe_block_size(m_est, topk, E)
+    if input_dtype is not None and input_dtype.itemsize == 1:
+        block_size_m = max(block_size_m, 16)             # marlin_moe.py:328-329
     sorted_token_ids, expert_ids, num_tokens_post_padded = moe_align_block_size(
         topk_ids, block_size_m, global_num_experts, expert_map, ignore_invalid_experts=True)
 
@@ -301,10 +321,12 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
         hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, topk, quant_type,
         apply_router_weight_on_input, expert_map, block_size_m, sorted_token_ids, expert_ids,
         num_tokens_post_padded, activation=activation, activation_func=activation_func, topk_ids=topk_ids,
-        global_scale1=global_scale1, global_scale2=global_scale2, g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1, sort_indices2=sort_indices2,
+        input_global_scale1=input_global_scale1, input_global_scale2=input_global_scale2,
+        global_scale1=global_scale1, global_scale2=global_scale2, g_idx1=g_idx1, g_idx2=g_idx2,
+        sort_indices1=sort_indices1, sort_indices2=sort_indices2,
         w1_zeros=w1_zeros, w2_zeros=w2_zeros, workspace=workspace,
         intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2, output=None,
-        is_k_full=is_k_full).view(-1, topk, K)
+        input_dtype=input_dtype, is_k_full=is_k_full).view(-1, topk, K)
     if output is None:
         output = torch.empty_like(hidden_states)
     if expert_map is not None:
@@ -322,19 +344,27 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
 def batched_fused_marlin_moe(hidden_states: torch.Tensor, expert_num_tokens: torch.Tensor, w1: torch.Tensor,
                              w2: torch.Tensor, bias1: torch.Tensor | None, bias2: torch.Tensor | None,
                              w1_scale: torch.Tensor, w2_scale: torch.Tensor, quant_type_id: int,
-                             apply_router_weight_on_input: bool = False,
+                             apply_router_weight_on_input: bool = False, global_num_experts: int = -1,
+                             activation="silu", expert_map: torch.Tensor | None = None,
+                             input_global_scale1: torch.Tensor | None = None,
+                             input_global_scale2: torch.Tensor | None = None,
+                             global_scale1: torch.Tensor | None = None, global_scale2: torch.Tensor | None = None,
                              g_idx1: torch.Tensor | None = None, g_idx2: torch.Tensor | None = None,
                              sort_indices1: torch.Tensor | None = None, sort_indices2: torch.Tensor | None = None,
                              w1_zeros: torch.Tensor | None = None, w2_zeros: torch.Tensor | None = None,
                              workspace: torch.Tensor | None = None,
                              intermediate_cache13: torch.Tensor | None = None,
                              intermediate_cache2: torch.Tensor | None = None, is_k_full: bool = True,
-                             output: torch.Tensor | None = None) -> torch.Tensor:
-    """The layer on tokens already batched by expert (marlin_moe.py:395-560):
-    hidden_states [E, max_tokens, K], of which the first expert_num_tokens[e] rows
-    of batch e are valid.  Every row belongs to one expert, so top_k = 1 and the
-    routing weights are ones.  Returns [E, max_tokens, K]; rows of invalid tokens
-    are not written."""
+                             output: torch.Tensor | None = None, input_dtype: torch.dtype | None = None,
+                             clamp_limit: float | None = None, gemm1_alpha: float = 1.0, gemm1_beta: float = 0.0,
+                             activation_func=None, activation_situ_beta: float | None = None,
+                             activation_situ_linear_beta: float | None = None) -> torch.Tensor:
+    """The layer on tokens already batched by expert (marlin_moe.py:395-560; same
+    parameters in the same order): hidden_states [E, max_tokens, K], of which the first
+    expert_num_tokens[e] rows of batch e are valid.  Every row belongs to one expert, so
+    top_k = 1 and the routing weights are ones.  Returns [E, max_tokens, K]; rows of invalid
+    tokens are not written.  global_num_experts and expert_map are accepted for signature
+    parity (the batches are the local experts already)."""
     if quant_type_id not in _SUPPORTED:
         raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8, uint8b128, "
                                   "float8_e4m3fn and float4_e2m1f (MXFP4, NVFP4) expert weights are built")
@@ -353,6 +383,8 @@ def batched_fused_marlin_moe(hidden_states: torch.Tensor, expert_num_tokens: tor
         if max_tokens / b_m < 0.9:
             block_size_m = b_m
             break
+    if input_dtype is not None and input_dtype.itemsize == 1:
+        block_size_m = max(block_size_m, 16)             # marlin_moe.py:507-508
     sorted_token_ids, expert_ids, num_tokens_post_padded = batched_moe_align_block_size(
         max_tokens, block_size_m, expert_num_tokens)
     M = B * max_tokens
@@ -360,8 +392,12 @@ def batched_fused_marlin_moe(hidden_states: torch.Tensor, expert_num_tokens: tor
     out = _fused_marlin_moe(
         hidden_states.view(-1, K), w1, w2, bias1, bias2, w1_scale, w2_scale, topk_weights, 1,
         _SUPPORTED[quant_type_id], apply_router_weight_on_input, None, block_size_m, sorted_token_ids,
-        expert_ids, num_tokens_post_padded, g_idx1=g_idx1, g_idx2=g_idx2, sort_indices1=sort_indices1,
-        sort_indices2=sort_indices2, w1_zeros=w1_zeros, w2_zeros=w2_zeros, workspace=workspace,
-        intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2,
-        output=output.view(-1, K) if output is not None else None, is_k_full=is_k_full)
+        expert_ids, num_tokens_post_padded, activation=activation, activation_func=activation_func,
+        input_global_scale1=input_global_scale1, input_global_scale2=input_global_scale2,
+        global_scale1=global_scale1, global_scale2=global_scale2, g_idx1=g_idx1, g_idx2=g_idx2,
+        sort_indices1=sort_indices1, sort_indices2=sort_indices2, w1_zeros=w1_zeros, w2_zeros=w2_zeros,
+        workspace=workspace, intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2,
+        output=output.view(-1, K) if output is not None else None, input_dtype=input_dtype, is_k_full=is_k_full,
+        clamp_limit=clamp_limit, gemm1_alpha=gemm1_alpha, gemm1_beta=gemm1_beta,
+        activation_situ_beta=activation_situ_beta, activation_situ_linear_beta=activation_situ_linear_beta)
     return out.view(B, max_tokens, K)

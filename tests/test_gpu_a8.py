@@ -199,3 +199,90 @@ def test_w4a8_rejections():
     assert call(b_type=_lib.TYPE_UINT4) == _lib.E_INVALID              # zero points missing
     assert call(stride=260) == _lib.E_INVALID
     assert call(a=None) == _lib.E_INVALID
+
+
+# ---------------------------------------------------------------- grouped (mixture of experts)
+MOE_A8_CASES = [
+    # m, k, n, experts, top_k, block, group, zp, dtype, bias, mul_topk
+    (1, 256, 128, 4, 2, 16, 64, False, "fp16", False, False),
+    (33, 512, 192, 5, 2, 16, 128, False, "bf16", True, True),
+    (70, 256, 128, 3, 3, 32, -1, False, "fp16", False, True),
+    (19, 512, 64, 6, 2, 8, 32, True, "bf16", False, False),
+    (100, 1024, 128, 4, 1, 64, 128, True, "fp16", True, False),
+    (47, 256, 256, 7, 4, 48, 64, False, "bf16", False, True),
+]
+
+
+@pytest.mark.parametrize("m,k,n,e,top_k,block,group,zp,dtype,bias,mul_topk", MOE_A8_CASES)
+@pytest.mark.parametrize("act", ["int8", "fp8"])
+def test_moe_w4a8_gemm(act, m, k, n, e, top_k, block, group, zp, dtype, bias, mul_topk):
+    """The grouped entry point: int8 bit for bit against the oracle, fp8 within tolerance.  One
+    expert id is set to -1 (held elsewhere): its rows must stay untouched."""
+    lib = _lib.load()
+    rng = np.random.default_rng(m * 7 + k + e)
+    layers = [A8Layer(300 + i + k + n, k, n, group, dtype, zp, act, bias) for i in range(e)]
+    # the integer group scales of all experts share one factor (the layer-wide maximum) in the
+    # reference; the per-expert factors of these test layers go into per-row scales instead
+    topk_ids = np.stack([rng.permutation(e)[:top_k] for _ in range(m)]).astype(np.int32)
+    sorted_ids, expert_ids, post_pad = mo.moe_align_block_size(topk_ids, block, e)
+    post_pad = int(post_pad[0])
+    expert_ids = expert_ids.copy()
+    skipped = int(expert_ids[0])
+    expert_ids[expert_ids == skipped] = -1 if e > 1 and m > 1 else skipped
+    topk_w = rng.uniform(0.1, 1.0, size=(m, top_k)).astype(np.float32)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    if act == "int8":
+        a_q, a_s = mo.per_token_quant_int8(x)
+        a_s = (a_s * layers[0].factor).astype(np.float32)      # one factor: the experts below share scales' scale
+        a_dev = torch.from_numpy(a_q).to(DEV)
+    else:
+        xt = torch.from_numpy(x)
+        a_s_t = (xt.abs().amax(dim=1, keepdim=True) / 448.0).clamp_min(1e-10)
+        a_fp8 = (xt / a_s_t).to(torch.float8_e4m3fn)
+        a_s = a_s_t.numpy()
+        a_dev = a_fp8.view(torch.uint8).to(DEV)
+    w_all = torch.stack([l.native for l in layers]).contiguous()
+    s_all = torch.stack([l.dev_scales for l in layers]).contiguous()
+    z_all = torch.stack([l.dev_zeros for l in layers]).contiguous() if zp else None
+    b_all = torch.stack([l.dev_bias for l in layers]).contiguous() if bias else None
+    c = torch.full((m * top_k, n), 7.0, dtype=tdt, device=DEV)
+    # device copies held in names: a temporary would hand its memory to the next allocation
+    d_as = torch.from_numpy(a_s.reshape(-1).copy()).to(DEV)
+    d_sorted, d_experts = dev_i32(sorted_ids), dev_i32(expert_ids)
+    d_past = dev_i32(np.array([post_pad], dtype=np.int32))
+    d_tw = torch.from_numpy(topk_w.reshape(-1).copy()).to(DEV)
+    _lib.check(lib.sonar_moe_wna16_marlin_gemm_a8(
+        ptr(a_dev), _lib.ADTYPE_INT8 if act == "int8" else _lib.ADTYPE_FP8, ptr(c), ptr(w_all), _lib.LAYOUT_GFX950,
+        ptr(b_all), ptr(s_all), ptr(d_as), ptr(z_all), ptr(d_sorted), sorted_ids.size, ptr(d_experts), ptr(d_past),
+        ptr(d_tw), block, top_k, int(mul_topk), e, dtype_code(dtype), layers[0].b_type, m, n, k, layers[0].groups,
+        stream()))
+    torch.cuda.synchronize()
+    got = host_f32(c)
+    written = np.zeros(m * top_k, dtype=bool)
+    for b in range(post_pad // block):
+        if expert_ids[b] >= 0:
+            ids = sorted_ids[b * block:(b + 1) * block]
+            written[ids[ids < m * top_k]] = True
+    assert np.all(got[~written] == 7.0)
+    if act == "int8":
+        experts = [dict(q=l.q, group_size=group, scales=l.scales, zeros=l.zeros, bias32=l.bias32) for l in layers]
+        want = mo.moe_gemm_w4a8_int8(a_q, a_s, experts, sorted_ids, expert_ids, post_pad, block, top_k,
+                                     topk_w if mul_topk else None, dtype)
+        assert np.array_equal(got[written], want[written]), np.abs(got[written] - want[written]).max()
+    else:
+        want = np.zeros_like(got)
+        for b in range(post_pad // block):
+            ex = int(expert_ids[b])
+            if ex < 0:
+                continue
+            ids = sorted_ids[b * block:(b + 1) * block]
+            ids = ids[ids < m * top_k]
+            l = layers[ex]
+            r = mo.gemm_w4a8_fp8(a_fp8.float().numpy()[ids // top_k], a_s.reshape(-1)[ids // top_k], l.q, group,
+                                 l.scales / np.float32(512.0), l.zeros, l.bias32)
+            if mul_topk:
+                r = r * topk_w.reshape(-1)[ids][:, None]
+            want[ids] = r
+        ok, max_err, max_ref = mo.gemm_tolerance_ok(got[written], want[written])
+        assert ok, (max_err, max_ref)

@@ -200,6 +200,10 @@ MOE_CONFIGS = [
     {"b_type": scalar_types.uint8b128, "support_act_order": True, "group_blocks": [-1, 2, 4, 8]},
     {"b_type": scalar_types.float8_e4m3fn, "group_blocks": [-1, 8]},
     {"b_type": scalar_types.float4_e2m1f, "a_type": torch.bfloat16, "group_blocks": [2]},
+    {"a_quant": torch.int8, "b_type": scalar_types.uint4, "group_blocks": [-1, 2, 4, 8]},
+    {"a_quant": torch.int8, "b_type": scalar_types.uint4b8, "group_blocks": [-1, 2, 4, 8]},
+    {"a_quant": torch.float8_e4m3fn, "b_type": scalar_types.uint4b8, "group_blocks": [-1, 2, 4, 8]},
+    {"a_quant": torch.float8_e4m3fn, "b_type": scalar_types.uint4, "group_blocks": [-1, 2, 4, 8]},
 ]
 MARLIN_MOE_SCENARIOS = [
     # (m, n, k, e, topk, ep_size, act_order, is_k_full)
@@ -229,12 +233,12 @@ def _moe_cases():
                     continue
                 if group_size in (k, n):
                     continue
-                cases.append((cfg["b_type"], cfg.get("a_type", torch.float16), group_size, m, n, k, e, topk, ep_size,
-                              act_order, is_k_full))
+                cases.append((cfg.get("a_quant"), cfg["b_type"], cfg.get("a_type", torch.float16), group_size, m, n, k,
+                              e, topk, ep_size, act_order, is_k_full))
     return cases
 
 
-def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None):
+def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None, input_dtype=None):
     """MarlinMoEWeightData.make (test_moe.py:774-892): every expert's (N, K)
     matrix quantised and laid out on its own, then stacked."""
     from sonar_amd.marlin_utils import marlin_permute_bias
@@ -245,7 +249,8 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None):
     out = {"w_ref": [], "qweight": [], "scales": [], "zeros": [], "g_idx": [], "sort_indices": [], "bias": []}
     for i in range(w.shape[0]):
         if quant_type == scalar_types.uint4:
-            w_ref, qweight, scales, zeros = awq_marlin_quantize(w[i].transpose(1, 0), quant_type, group_size)
+            w_ref, qweight, scales, zeros = awq_marlin_quantize(w[i].transpose(1, 0), quant_type, group_size,
+                                                                input_dtype=input_dtype)
             out["zeros"].append(zeros)
         elif quant_type == scalar_types.float8_e4m3fn:
             w_ref, qweight, scales = marlin_quant_fp8_torch(w[i].contiguous(), group_size)
@@ -253,7 +258,7 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None):
             w_ref, qweight, scales = rand_marlin_weight_mxfp4_like(w[i], group_size)
         else:
             w_ref, qweight, scales, g_idx, sort_indices, _ = marlin_quantize(
-                w[i].transpose(1, 0), quant_type, group_size, act_order, torch.randperm(k))
+                w[i].transpose(1, 0), quant_type, group_size, act_order, torch.randperm(k), input_dtype=input_dtype)
             out["g_idx"].append(g_idx)
             out["sort_indices"].append(sort_indices)
         out["w_ref"].append(w_ref.T)
@@ -261,17 +266,33 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None):
         out["scales"].append(scales)
         if bias is not None:
             out["bias"].append(marlin_permute_bias(bias[i]))
-    return {name: (torch.stack(v).contiguous() if v else None) for name, v in out.items()}
+    res = {name: (torch.stack(v).contiguous() if v else None) for name, v in out.items()}
+    res["a_scales_factor"] = None
+    if input_dtype == torch.int8 and group_size != -1:        # test_moe.py:876-880
+        scales = res["scales"]
+        res["a_scales_factor"] = 1 / 4096 * scales.max().float()
+        res["scales"] = (scales / scales.max() * 4096).round().to(torch.int16).view(w.dtype)
+    return res
 
 
-def _torch_experts(a, w1, w2, topk_weight, topk_ids, expert_map=None, b1=None, b2=None):
+def _torch_experts(a, w1, w2, topk_weight, topk_ids, expert_map=None, b1=None, b2=None, quant_dtype=None):
     """Plain mixture of experts on (E, 2N, K) / (E, K, N) matrices: for every
     token and routed expert silu(x W1_gate^T) * (x W1_up^T) through W2^T, summed
-    with the routing weights; experts mapped to -1 contribute nothing."""
+    with the routing weights; experts mapped to -1 contribute nothing.  With
+    `quant_dtype` (int8 / float8_e4m3fn) the input of either product is quantised per row
+    and dequantised first (torch_experts with quant_input_only, tests/kernels/utils.py:845-893)."""
+    from sonar_amd.marlin_utils import marlin_quant_input
+
+    def through_quant(x):
+        if quant_dtype is None:
+            return x
+        q, s = marlin_quant_input(x, quant_dtype)
+        return (q.float() * s.view(-1, 1)).to(x.dtype)
+
     m, k = a.shape
     n = w2.shape[-1]
     out = torch.zeros((m, k), dtype=torch.float32, device=a.device)
-    a32 = a.float()
+    a32 = through_quant(a).float()
     for ex in torch.unique(topk_ids).tolist():
         local = ex if expert_map is None else int(expert_map[ex])
         if local < 0:
@@ -281,7 +302,7 @@ def _torch_experts(a, w1, w2, topk_weight, topk_ids, expert_map=None, b1=None, b
         if b1 is not None:
             h = h + b1[local].float()
         h = h.to(a.dtype).float()
-        act = (torch.nn.functional.silu(h[:, :n]) * h[:, n:]).to(a.dtype).float()
+        act = through_quant((torch.nn.functional.silu(h[:, :n]) * h[:, n:]).to(a.dtype)).float()
         y = act @ w2[local].float().T
         if b2 is not None:
             y = y + b2[local].float()
@@ -289,9 +310,9 @@ def _torch_experts(a, w1, w2, topk_weight, topk_ids, expert_map=None, b1=None, b
     return out.to(a.dtype)
 
 
-@pytest.mark.parametrize("b_type,dtype,group_size,m,n,k,e,topk,ep_size,act_order,is_k_full", _moe_cases(),
+@pytest.mark.parametrize("a_quant,b_type,dtype,group_size,m,n,k,e,topk,ep_size,act_order,is_k_full", _moe_cases(),
                          ids=lambda v: str(v).replace("torch.", ""))
-def test_fused_marlin_moe(b_type, dtype, group_size, m, n, k, e, topk, ep_size, act_order, is_k_full):
+def test_fused_marlin_moe(a_quant, b_type, dtype, group_size, m, n, k, e, topk, ep_size, act_order, is_k_full):
     from sonar_amd.fused_moe import fused_marlin_moe
     torch.manual_seed(1)
     a = torch.randn((m, k), device="cuda", dtype=dtype) / 10
@@ -304,19 +325,24 @@ def test_fused_marlin_moe(b_type, dtype, group_size, m, n, k, e, topk, ep_size, 
         e_map = torch.full((e,), -1, device="cuda", dtype=torch.int32)
         e_map[e_ids] = torch.arange(local_e, device="cuda", dtype=torch.int32)
         w1, w2 = w1[e_ids], w2[e_ids]
-    d1 = _marlin_moe_weights(w1, b_type, group_size, act_order)
-    d2 = _marlin_moe_weights(w2, b_type, group_size, act_order)
+    d1 = _marlin_moe_weights(w1, b_type, group_size, act_order, input_dtype=a_quant)
+    d2 = _marlin_moe_weights(w2, b_type, group_size, act_order, input_dtype=a_quant)
     score = torch.randn((m, e), device="cuda", dtype=dtype)
     topk_weights, topk_ids = torch.topk(torch.softmax(score, dim=-1, dtype=torch.float32), topk)
-    want = _torch_experts(a, d1["w_ref"], d2["w_ref"], topk_weights, topk_ids, e_map)
+    want = _torch_experts(a, d1["w_ref"], d2["w_ref"], topk_weights, topk_ids, e_map, quant_dtype=a_quant)
     got = fused_marlin_moe(a, d1["qweight"], d2["qweight"], None, None, d1["scales"], d2["scales"], topk_weights,
                            topk_ids.to(torch.int32), global_num_experts=e, expert_map=e_map, g_idx1=d1["g_idx"],
-                           g_idx2=d2["g_idx"], sort_indices1=d1["sort_indices"], sort_indices2=d2["sort_indices"],
-                           w1_zeros=d1["zeros"], w2_zeros=d2["zeros"], quant_type_id=b_type.id, is_k_full=is_k_full)
+                           g_idx2=d2["g_idx"], input_global_scale1=d1["a_scales_factor"],
+                           input_global_scale2=d2["a_scales_factor"], sort_indices1=d1["sort_indices"],
+                           sort_indices2=d2["sort_indices"], w1_zeros=d1["zeros"], w2_zeros=d2["zeros"],
+                           input_dtype=a_quant, quant_type_id=b_type.id, is_k_full=is_k_full)
     torch.cuda.synchronize()
     torch.testing.assert_close(got, want, atol=4e-2, rtol=0)
-    # and this build's own bar for two chained GEMMs: 2e-2 of the largest reference value
-    assert float((got.float() - want.float()).abs().max()) <= 2e-2 * float(want.float().abs().max())
+    # and this build's own bar for two chained GEMMs: 2e-2 of the largest reference value; twice that
+    # with 8-bit activations, where an intermediate value that differs in its last bit can land in
+    # the next quantisation step (1 / 16 of its size for float8_e4m3fn)
+    bar = 2e-2 if a_quant is None else 4e-2
+    assert float((got.float() - want.float()).abs().max()) <= bar * float(want.float().abs().max())
 
 
 @pytest.mark.parametrize("m", [1, 256])
