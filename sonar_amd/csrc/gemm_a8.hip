@@ -22,6 +22,7 @@ namespace sonar {
 namespace {
 
 typedef int intx4_t __attribute__((ext_vector_type(4)));
+typedef int intx8_t __attribute__((ext_vector_type(8)));
 
 struct A8Params {
   const uint8_t* a;        // [M][a_row_stride] bytes
@@ -84,6 +85,14 @@ struct ActInt8 {
     const uint32_t hi = ((((w >> 4) & 0x0f0f0f0fu) | 0x80808080u) - z4) ^ 0x80808080u;
     return (long)(((uint64_t)hi << 32) | lo);
   }
+  // The full-rate instruction takes two chunks (K = 64) at a time.
+  static constexpr int kWideChunks = 2;
+  typedef intx4_t wide_t;
+  static __device__ __forceinline__ acc_t mfma_wide(wide_t a, wide_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_i32_16x16x64_i8(a, b, c, 0, 0, 0);
+  }
+  // byte offset, inside a row of the LDS tile, of the 8 bytes (chunk c of the step, k block kb)
+  static __device__ __forceinline__ int unit_offset(int c, int kb) { return (c >> 1) * 64 + kb * 16 + (c & 1) * 8; }
 };
 
 struct ActFp8 {
@@ -115,6 +124,13 @@ struct ActFp8 {
     const uint32_t z = z4 & 0xffu;
     return (long)(((uint64_t)four_zp((w >> 4) & 0x0f0f0f0fu, z, z4) << 32) | four_zp(w & 0x0f0f0f0fu, z, z4));
   }
+  // The full-rate instruction takes four chunks (K = 128) at a time; its block scales are 1.
+  static constexpr int kWideChunks = 4;
+  typedef intx8_t wide_t;
+  static __device__ __forceinline__ acc_t mfma_wide(wide_t a, wide_t b, acc_t c) {
+    return __builtin_amdgcn_mfma_scale_f32_16x16x128_f8f6f4(a, b, c, 0, 0, 0, 127, 0, 127);
+  }
+  static __device__ __forceinline__ int unit_offset(int c, int kb) { return kb * 32 + c * 8; }
 };
 
 // Raw total -> output value: the activation row's scale, for channelwise
@@ -363,6 +379,220 @@ __global__ __launch_bounds__(256) void marlin_moe_a8_kernel(MoeA8Params q) {
     }
 }
 
+// ---- the tiled kernel for many rows -----------------------------------------
+// A workgroup owns a 128 x 128 tile of C; its four wavefronts own 64 x 64 quarters (wavefront
+// (wr, wc): rows 64 wr, the 64-column strip 2 tile + wc) and walk K in steps of 128 (four
+// chunks).  The activations of a step (128 rows x 128 bytes) go through LDS, two buffers, one
+// barrier a step; on the way in every 8 bytes are shuffled into the byte order of the B
+// operand and laid out so that a lane finds the bytes of one full-rate instruction side by
+// side (rows 144 bytes apart: no bank conflicts).  The weights stay in registers, one step
+// ahead.  GC: chunks per scale group (1, 2, 4) or 0 for channelwise scales.  Groups that
+// span the K of a full-rate instruction use it (v_mfma_i32_16x16x64_i8,
+// v_mfma_f32_16x16x128_f8f6f4); smaller groups take the K = 32 forms.
+constexpr int kA8TileM = 128, kA8TileN = 128, kA8StepK = 128, kA8StepChunks = 4, kA8RowBytes = 144;
+
+template <typename ACT, typename T, bool HAS_ZP, int GC>
+__global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
+  typedef typename ACT::acc_t acc_t;
+  typedef typename ACT::scalar_t scalar_t;
+  typedef typename ACT::wide_t wide_t;
+  constexpr int WIDE = ACT::kWideChunks;
+  constexpr bool kUseWide = GC == 0 || GC >= WIDE;
+  constexpr int kGroupsPerStep = GC == 0 ? 1 : kA8StepChunks / GC;
+  // channelwise uint4b8 weights take the zero-point form with z = 8: no factor 16 to shift out
+  constexpr bool kZpForm = HAS_ZP || (ACT::kInteger && GC == 0);
+  constexpr int kShift = (ACT::kInteger && !kZpForm) ? ACT::kShift : 0;
+  __shared__ __align__(16) uint8_t tile[2][kA8TileM * kA8RowBytes];
+
+  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int l16 = lane & 15, kb = lane >> 4;
+  const int wr = wave >> 1, wc = wave & 1;
+  const int m0 = blockIdx.y * kA8TileM;
+  const int strip = blockIdx.x * 2 + wc;
+  const int s_begin = blockIdx.z * p.units_per_split;
+  const int s_end = min(s_begin + p.units_per_split, p.units);
+
+  // copy role: thread t brings 64 bytes of row t / 2 of the tile
+  const int c_row = tid >> 1, c_half = tid & 1;
+  int src_row = m0 + c_row;
+  if (src_row >= p.m) src_row = p.m - 1;                  // results of such rows are dropped
+  const uint8_t* a_src = p.a + (long)src_row * p.a_row_stride + c_half * 64;
+  const int dst_row = c_row * kA8RowBytes;
+  const uint32_t* w_lane = p.w + (long)strip * p.chunks * kChunkWords + lane * 4;
+  int s_col[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) s_col[j] = strip * kStripN + scale_slot(16 * j + l16, false);
+
+  acc_t acc[4][4], tmp[4][4];
+#pragma unroll
+  for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[rb][j] = tmp[rb][j] = acc_t{0, 0, 0, 0};
+
+  uint4 ra[4];
+  u32x4_t wq[kA8StepChunks], wq_next[kA8StepChunks];
+  auto load_a = [&](int step) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      ra[i] = *reinterpret_cast<const uint4*>(a_src + (long)step * kA8StepK + 16 * i);
+  };
+  auto load_w = [&](int step, u32x4_t (&dst)[kA8StepChunks]) {
+#pragma unroll
+    for (int c = 0; c < kA8StepChunks; ++c)
+      dst[c] = *reinterpret_cast<const u32x4_t*>(w_lane + (long)(step * kA8StepChunks + c) * kChunkWords);
+  };
+  auto store_a = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const int c = c_half * 2 + (i >> 1), kb0 = 2 * (i & 1);
+      uint2 u0, u1;
+      u0.x = __builtin_amdgcn_perm(ra[i].y, ra[i].x, 0x05010400u);   // bytes k = 0, 4, 1, 5
+      u0.y = __builtin_amdgcn_perm(ra[i].y, ra[i].x, 0x07030602u);   // bytes k = 2, 6, 3, 7
+      u1.x = __builtin_amdgcn_perm(ra[i].w, ra[i].z, 0x05010400u);
+      u1.y = __builtin_amdgcn_perm(ra[i].w, ra[i].z, 0x07030602u);
+      *reinterpret_cast<uint2*>(&tile[buf][dst_row + ACT::unit_offset(c, kb0)]) = u0;
+      *reinterpret_cast<uint2*>(&tile[buf][dst_row + ACT::unit_offset(c, kb0 + 1)]) = u1;
+    }
+  };
+  // group g is complete in tmp: into acc with its scale
+  auto apply_group = [&](int g) {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const uint16_t bits = p.scales[(long)g * p.n + s_col[j]];
+      scalar_t sc;
+      if constexpr (ACT::kInteger) sc = (int)bits;
+      else sc = from_bits<T>(bits);
+#pragma unroll
+      for (int rb = 0; rb < 4; ++rb) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if constexpr (ACT::kInteger) acc[rb][j][i] += __mul24(tmp[rb][j][i] >> kShift, sc);
+          else acc[rb][j][i] += tmp[rb][j][i] * sc;
+        }
+        tmp[rb][j] = acc_t{0, 0, 0, 0};
+      }
+    }
+  };
+
+  if (s_begin < s_end) {
+    load_a(s_begin);
+    load_w(s_begin, wq);
+    store_a(0);
+  }
+  __syncthreads();
+  for (int step = s_begin; step < s_end; ++step) {
+    const int buf = (step - s_begin) & 1;
+    const bool more = step + 1 < s_end;
+    if (more) {
+      load_a(step + 1);
+      load_w(step + 1, wq_next);
+    }
+    // zero points of the groups of this step: word l16 % 8 of the strip's eight, nibble 2j + l16 / 8
+    uint32_t zw[kGroupsPerStep];
+    if (HAS_ZP) {
+#pragma unroll
+      for (int gi = 0; gi < kGroupsPerStep; ++gi) {
+        const int g = GC == 0 ? 0 : step * kGroupsPerStep + gi;
+        zw[gi] = p.zeros[(long)g * (p.n / 8) + strip * 8 + (l16 & 7)];
+      }
+    }
+    const uint8_t* rows = &tile[buf][(64 * wr + l16) * kA8RowBytes];
+#pragma unroll
+    for (int w0 = 0; w0 < kA8StepChunks; w0 += WIDE) {
+      // B operands of the WIDE chunks, every column block
+      long bq[WIDE][4];
+#pragma unroll
+      for (int c = 0; c < WIDE; ++c) {
+        const int gi = GC == 0 ? 0 : (w0 + c) / GC;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          uint32_t z4 = 0x08080808u;
+          if (HAS_ZP) z4 = ((zw[gi] >> (4 * (2 * j + (l16 >> 3)))) & 0xFu) * 0x01010101u;
+          bq[c][j] = kZpForm ? ACT::word_zp(wq[w0 + c][j], z4) : ACT::word(wq[w0 + c][j]);
+        }
+      }
+      // this lane's bytes of the WIDE chunks of row 16 rb + l16: side by side in LDS
+      auto read_a = [&](int rb, uint32_t (&av)[2 * WIDE]) {
+#pragma unroll
+        for (int h = 0; h < WIDE / 2; ++h) {
+          const uint4 v = *reinterpret_cast<const uint4*>(rows + rb * 16 * kA8RowBytes +
+                                                          ACT::unit_offset(w0 + 2 * h, kb));
+          av[4 * h + 0] = v.x; av[4 * h + 1] = v.y; av[4 * h + 2] = v.z; av[4 * h + 3] = v.w;
+        }
+      };
+      if constexpr (kUseWide) {
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) {
+          uint32_t av[2 * WIDE];
+          read_a(rb, av);
+          wide_t a;
+#pragma unroll
+          for (int d = 0; d < 2 * WIDE; ++d) a[d] = (int)av[d];
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            wide_t b;
+#pragma unroll
+            for (int c = 0; c < WIDE; ++c) {
+              b[2 * c] = (int)(uint32_t)bq[c][j];
+              b[2 * c + 1] = (int)(uint32_t)((uint64_t)bq[c][j] >> 32);
+            }
+            if constexpr (GC == 0) acc[rb][j] = ACT::mfma_wide(a, b, acc[rb][j]);
+            else tmp[rb][j] = ACT::mfma_wide(a, b, tmp[rb][j]);
+          }
+        }
+        if constexpr (GC != 0) {
+          if ((w0 + WIDE) % GC == 0) apply_group((step * kA8StepChunks + w0 + WIDE) / GC - 1);
+        }
+      } else {
+        // groups smaller than the full-rate K: chunk by chunk, the group's scale behind its last chunk
+        uint32_t av[4][2 * WIDE];
+#pragma unroll
+        for (int rb = 0; rb < 4; ++rb) read_a(rb, av[rb]);
+#pragma unroll
+        for (int c = 0; c < WIDE; ++c) {
+#pragma unroll
+          for (int rb = 0; rb < 4; ++rb) {
+            const long a = (long)(((uint64_t)av[rb][2 * c + 1] << 32) | av[rb][2 * c]);
+#pragma unroll
+            for (int j = 0; j < 4; ++j) tmp[rb][j] = ACT::mfma(a, bq[c][j], tmp[rb][j]);
+          }
+          if ((w0 + c + 1) % GC == 0) apply_group((step * kA8StepChunks + w0 + c + 1) / GC - 1);
+        }
+      }
+    }
+    if (more) {
+      store_a(buf ^ 1);
+#pragma unroll
+      for (int c = 0; c < kA8StepChunks; ++c) wq[c] = wq_next[c];
+    }
+    __syncthreads();
+  }
+
+  // epilogue: lane holds rows 64 wr + 16 rb + 4 kb + i, column 16 j + l16 of its strip
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int col = strip * kStripN + 16 * j + l16;
+    float col_scale = 1.0f, bias = 0.0f;
+    if (p.splits == 1) {
+      if (GC == 0) col_scale = from_bits<T>(p.scales[s_col[j]]);
+      if (p.bias) bias = from_bits<T>(p.bias[s_col[j]]);
+    }
+#pragma unroll
+    for (int rb = 0; rb < 4; ++rb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        const int row = m0 + 64 * wr + 16 * rb + 4 * kb + i;
+        if (row >= p.m) continue;
+        const scalar_t total = acc[rb][j][i];
+        if (p.splits == 1)
+          reinterpret_cast<uint16_t*>(p.c)[(long)row * p.n + col] =
+              finish<ACT, T, GC != 0>(total, p.a_scales[row], col_scale, bias);
+        else
+          p.partial[((long)blockIdx.z * p.m + row) * p.n + col] = raw_bits(total);
+      }
+  }
+}
+
 // Adds the raw totals of the K splits and finishes them.
 template <typename ACT, typename T, bool GROUPED>
 __global__ __launch_bounds__(256) void marlin_a8_finish_kernel(A8Params p) {
@@ -385,11 +615,31 @@ __global__ __launch_bounds__(256) void marlin_a8_finish_kernel(A8Params p) {
 }
 
 struct A8Plan {
+  bool tile;   // the tiled kernel: units are steps of 128 rows of the weights
   int mb, slabs, splits, units, unit_chunks, units_per_split;
 };
 
 A8Plan plan_a8(int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups) {
   A8Plan plan;
+  // groups of 32 rows stay with the kernel above: one scale per K = 32 instruction leaves the tiled
+  // kernel more scale arithmetic than matrix work, and its registers do not hold it
+  plan.tile = size_m > 64 && size_k % kA8StepK == 0 && size_n % kA8TileN == 0 &&
+              (num_groups == 1 || size_k / num_groups >= 64);
+  if (plan.tile) {
+    plan.mb = 0;
+    plan.slabs = (int)((size_m + kA8TileM - 1) / kA8TileM);
+    plan.unit_chunks = num_groups > 1 ? (int)(size_k / num_groups) / kChunkK : 0;
+    plan.units = (int)(size_k / kA8StepK);
+    // fewer tiles than two per compute unit: split K, at least eight steps a workgroup
+    const long tiles = (long)(size_n / kA8TileN) * plan.slabs;
+    int splits = (int)(512 / tiles);
+    if (splits > plan.units / 8) splits = plan.units / 8;
+    if (splits > 16) splits = 16;
+    if (splits < 1) splits = 1;
+    plan.units_per_split = (plan.units + splits - 1) / splits;
+    plan.splits = (plan.units + plan.units_per_split - 1) / plan.units_per_split;
+    return plan;
+  }
   plan.mb = size_m > 48 ? 4 : (int)((size_m + 15) / 16);
   plan.slabs = (int)((size_m + plan.mb * 16 - 1) / (plan.mb * 16));
   const int chunks = (int)(size_k / kChunkK);
@@ -412,10 +662,31 @@ void launch_a8_mb(const A8Params& p, bool grouped, dim3 grid, hipStream_t st) {
   else marlin_a8_kernel<ACT, T, MB, HAS_ZP, false><<<grid, 256, 0, st>>>(p);
 }
 
+template <typename ACT, typename T, bool HAS_ZP>
+void launch_a8_tile_gc(const A8Params& p, int gc, dim3 grid, hipStream_t st) {
+  switch (gc) {
+    case 0: marlin_a8_tile_kernel<ACT, T, HAS_ZP, 0><<<grid, 256, 0, st>>>(p); break;
+    case 2: marlin_a8_tile_kernel<ACT, T, HAS_ZP, 2><<<grid, 256, 0, st>>>(p); break;
+    default: marlin_a8_tile_kernel<ACT, T, HAS_ZP, 4><<<grid, 256, 0, st>>>(p); break;
+  }
+}
+
 template <typename ACT, typename T>
 void launch_a8(const A8Params& p, const A8Plan& plan, bool grouped, hipStream_t st) {
-  const dim3 grid(p.n / kStripN, plan.slabs, plan.splits);
   const bool zp = p.zeros != nullptr;
+  if (plan.tile) {
+    const dim3 grid(p.n / kA8TileN, plan.slabs, plan.splits);
+    if (zp) launch_a8_tile_gc<ACT, T, true>(p, plan.unit_chunks, grid, st);
+    else launch_a8_tile_gc<ACT, T, false>(p, plan.unit_chunks, grid, st);
+    if (plan.splits > 1) {
+      long blocks = ((long)p.m * p.n + 255) / 256;
+      if (blocks > 4096) blocks = 4096;
+      if (grouped) marlin_a8_finish_kernel<ACT, T, true><<<(int)blocks, 256, 0, st>>>(p);
+      else marlin_a8_finish_kernel<ACT, T, false><<<(int)blocks, 256, 0, st>>>(p);
+    }
+    return;
+  }
+  const dim3 grid(p.n / kStripN, plan.slabs, plan.splits);
 #define SONAR_A8_CASE(MB)                                             \
   case MB:                                                            \
     if (zp) launch_a8_mb<ACT, T, MB, true>(p, grouped, grid, st);     \
@@ -462,7 +733,25 @@ void launch_moe_a8(const MoeA8Params& q, bool grouped, int blocks, hipStream_t s
 // Checks shared by the dense and the grouped entry point.
 int check_a8(int a_dtype, int dtype, int b_layout, int64_t b_type_id, int64_t size_m, int64_t size_n, int64_t size_k,
              int64_t num_groups, const uint32_t* b_zeros) {
-  if (int rc = check_a8(a_dtype, dtype, b_layout, b_type_id, size_m, size_n, size_k, num_groups, b_zeros)) return rc;
+  SONAR_REQUIRE(b_layout == SONAR_LAYOUT_GFX950, "unknown b_layout = %d", b_layout);
+  SONAR_REQUIRE(a_dtype == SONAR_ADTYPE_INT8 || a_dtype == SONAR_ADTYPE_FP8, "unknown a_dtype = %d", a_dtype);
+  SONAR_REQUIRE(dtype == SONAR_DTYPE_F16 || dtype == SONAR_DTYPE_BF16, "unknown dtype = %d", dtype);
+  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4)
+    return fail(SONAR_E_UNSUPPORTED, "8-bit activations are built for b_type uint4b8 and uint4 only (W8A8 is not "
+                "supported by the marlin kernel; float4_e2m1f weights with fp8 activations are not built)");
+  SONAR_REQUIRE(size_m >= 0 && size_n > 0 && size_k > 0, "size_m = %ld, size_n = %ld, size_k = %ld", (long)size_m,
+                (long)size_n, (long)size_k);
+  SONAR_REQUIRE(size_n % kStripN == 0, "size_n = %ld is not divisible by %d", (long)size_n, kStripN);
+  SONAR_REQUIRE(size_k % kChunkK == 0, "size_k = %ld is not divisible by %d", (long)size_k, kChunkK);
+  SONAR_REQUIRE(size_m < (1LL << 30) && size_n < (1LL << 30) && size_k < (1LL << 30), "sizes too large");
+  SONAR_REQUIRE(num_groups >= 1 && size_k % num_groups == 0, "size_k = %ld is not divisible by num_groups = %ld",
+                (long)size_k, (long)num_groups);
+  const int64_t group_size = size_k / num_groups;
+  if (num_groups > 1)
+    SONAR_REQUIRE(group_size == 32 || group_size == 64 || group_size == 128,
+                  "Invalid group_size = %ld: 8-bit activations take -1, 32, 64 or 128", (long)group_size);
+  SONAR_REQUIRE((b_zeros != nullptr) == (b_type_id == SONAR_TYPE_UINT4),
+                "b_zeros must be given for uint4 weights and only for them");
   return SONAR_OK;
 }
 
@@ -543,25 +832,7 @@ extern "C" int sonar_marlin_gemm_a8(const void* a, int64_t a_row_stride, int a_d
                                     const uint32_t* b_zeros, void* scratch, size_t scratch_bytes, int dtype,
                                     int64_t b_type_id, int64_t size_m, int64_t size_n, int64_t size_k,
                                     int64_t num_groups, void* stream) {
-  SONAR_REQUIRE(b_layout == SONAR_LAYOUT_GFX950, "unknown b_layout = %d", b_layout);
-  SONAR_REQUIRE(a_dtype == SONAR_ADTYPE_INT8 || a_dtype == SONAR_ADTYPE_FP8, "unknown a_dtype = %d", a_dtype);
-  SONAR_REQUIRE(dtype == SONAR_DTYPE_F16 || dtype == SONAR_DTYPE_BF16, "unknown dtype = %d", dtype);
-  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4)
-    return fail(SONAR_E_UNSUPPORTED, "8-bit activations are built for b_type uint4b8 and uint4 only (W8A8 is not "
-                "supported by the marlin kernel; float4_e2m1f weights with fp8 activations are not built)");
-  SONAR_REQUIRE(size_m >= 0 && size_n > 0 && size_k > 0, "size_m = %ld, size_n = %ld, size_k = %ld", (long)size_m,
-                (long)size_n, (long)size_k);
-  SONAR_REQUIRE(size_n % kStripN == 0, "size_n = %ld is not divisible by %d", (long)size_n, kStripN);
-  SONAR_REQUIRE(size_k % kChunkK == 0, "size_k = %ld is not divisible by %d", (long)size_k, kChunkK);
-  SONAR_REQUIRE(size_m < (1LL << 30) && size_n < (1LL << 30) && size_k < (1LL << 30), "sizes too large");
-  SONAR_REQUIRE(num_groups >= 1 && size_k % num_groups == 0, "size_k = %ld is not divisible by num_groups = %ld",
-                (long)size_k, (long)num_groups);
-  const int64_t group_size = size_k / num_groups;
-  if (num_groups > 1)
-    SONAR_REQUIRE(group_size == 32 || group_size == 64 || group_size == 128,
-                  "Invalid group_size = %ld: 8-bit activations take -1, 32, 64 or 128", (long)group_size);
-  SONAR_REQUIRE((b_zeros != nullptr) == (b_type_id == SONAR_TYPE_UINT4),
-                "b_zeros must be given for uint4 weights and only for them");
+  if (int rc = check_a8(a_dtype, dtype, b_layout, b_type_id, size_m, size_n, size_k, num_groups, b_zeros)) return rc;
   if (size_m == 0) return SONAR_OK;
   SONAR_REQUIRE(a && c && b_q_weight && b_scales && a_scales, "a, c, b_q_weight, b_scales and a_scales must not be NULL");
   SONAR_REQUIRE(a_row_stride >= size_k && a_row_stride % 8 == 0, "A.stride(0) = %ld must be at least size_k and "

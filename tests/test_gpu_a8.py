@@ -134,6 +134,16 @@ INT8_CASES = [
     (8192, 64, 128, False, "fp16", True, [1, 20]),     # K split over workgroups
     (4096, 128, -1, False, "bf16", False, [9]),         # channelwise, K split
     (1056, 128, -1, False, "fp16", False, [4]),         # K a multiple of 32 only
+    # the tiled kernel (more than 64 rows, N a multiple of 128, K of 128, groups of 64 rows or more)
+    (1024, 256, -1, False, "fp16", True, [65, 200]),
+    (1024, 256, 64, False, "bf16", False, [128, 300]),
+    (512, 384, 128, False, "fp16", True, [129]),
+    (1024, 128, -1, True, "bf16", False, [100]),
+    (512, 256, 64, True, "fp16", True, [257]),
+    (1024, 256, 128, True, "fp16", False, [96]),
+    (8192, 128, 128, False, "fp16", False, [128]),      # K split over workgroups
+    (8192, 128, -1, False, "bf16", True, [70]),
+    (1024, 256, 32, False, "fp16", False, [100]),       # groups of 32: the slab kernel
 ]
 
 
@@ -158,6 +168,14 @@ FP8_CASES = [
     (512, 192, 64, True, "fp16", False, [5, 40]),
     (512, 64, -1, True, "bf16", True, [2]),
     (8192, 64, 128, False, "bf16", False, [3]),
+    # the tiled kernel
+    (1024, 256, -1, False, "fp16", True, [65, 200]),
+    (1024, 256, 128, False, "bf16", False, [128, 300]),
+    (1024, 256, 64, False, "fp16", False, [100]),
+    (512, 384, 128, True, "fp16", True, [129]),
+    (1024, 128, -1, True, "bf16", False, [100]),
+    (512, 256, 64, True, "bf16", False, [257]),
+    (8192, 128, 128, False, "fp16", False, [128]),
 ]
 
 
