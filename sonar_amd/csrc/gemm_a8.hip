@@ -399,8 +399,9 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
   constexpr int WIDE = ACT::kWideChunks;
   constexpr bool kUseWide = GC == 0 || GC >= WIDE;
   constexpr int kGroupsPerStep = GC == 0 ? 1 : kA8StepChunks / GC;
-  // channelwise uint4b8 weights take the zero-point form with z = 8: no factor 16 to shift out
-  constexpr bool kZpForm = HAS_ZP || (ACT::kInteger && GC == 0);
+  // uint4b8 weights enter as 16 (q - 8); the factor leaves with the group's scale, or, for channelwise
+  // scales, in the epilogue (the host sends K beyond 2^16 to the slab kernel: 2^16 * 127 * 128 < 2^31)
+  constexpr bool kZpForm = HAS_ZP;
   constexpr int kShift = (ACT::kInteger && !kZpForm) ? ACT::kShift : 0;
   __shared__ __align__(16) uint8_t tile[2][kA8TileM * kA8RowBytes];
 
@@ -469,23 +470,26 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
           if constexpr (ACT::kInteger) acc[rb][j][i] += __mul24(tmp[rb][j][i] >> kShift, sc);
           else acc[rb][j][i] += tmp[rb][j][i] * sc;
         }
-        tmp[rb][j] = acc_t{0, 0, 0, 0};
       }
     }
   };
 
   if (s_begin < s_end) {
-    load_a(s_begin);
     load_w(s_begin, wq);
+    load_a(s_begin);
     store_a(0);
   }
+  // Nothing is outstanding when the loop starts: otherwise the compiler's wait counts, which must
+  // also hold for this first entry, make every later step wait for the loads it has only just
+  // issued for the step after it.  (vmcnt = 0; the other counters untouched.)
+  __builtin_amdgcn_s_waitcnt(0x0F70);
   __syncthreads();
   for (int step = s_begin; step < s_end; ++step) {
     const int buf = (step - s_begin) & 1;
     const bool more = step + 1 < s_end;
     if (more) {
-      load_a(step + 1);
       load_w(step + 1, wq_next);
+      load_a(step + 1);
     }
     // zero points of the groups of this step: word l16 % 8 of the strip's eight, nibble 2j + l16 / 8
     uint32_t zw[kGroupsPerStep];
@@ -536,7 +540,9 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
               b[2 * c] = (int)(uint32_t)bq[c][j];
               b[2 * c + 1] = (int)(uint32_t)((uint64_t)bq[c][j] >> 32);
             }
+            // the first instruction of a group starts from zero: tmp needs no clearing
             if constexpr (GC == 0) acc[rb][j] = ACT::mfma_wide(a, b, acc[rb][j]);
+            else if (w0 % GC == 0) tmp[rb][j] = ACT::mfma_wide(a, b, acc_t{0, 0, 0, 0});
             else tmp[rb][j] = ACT::mfma_wide(a, b, tmp[rb][j]);
           }
         }
@@ -554,7 +560,8 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
           for (int rb = 0; rb < 4; ++rb) {
             const long a = (long)(((uint64_t)av[rb][2 * c + 1] << 32) | av[rb][2 * c]);
 #pragma unroll
-            for (int j = 0; j < 4; ++j) tmp[rb][j] = ACT::mfma(a, bq[c][j], tmp[rb][j]);
+            for (int j = 0; j < 4; ++j)
+              tmp[rb][j] = ACT::mfma(a, bq[c][j], (w0 + c) % GC == 0 ? acc_t{0, 0, 0, 0} : tmp[rb][j]);
           }
           if ((w0 + c + 1) % GC == 0) apply_group((step * kA8StepChunks + w0 + c + 1) / GC - 1);
         }
@@ -583,7 +590,8 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
       for (int i = 0; i < 4; ++i) {
         const int row = m0 + 64 * wr + 16 * rb + 4 * kb + i;
         if (row >= p.m) continue;
-        const scalar_t total = acc[rb][j][i];
+        scalar_t total = acc[rb][j][i];
+        if constexpr (ACT::kInteger && GC == 0) total >>= kShift;
         if (p.splits == 1)
           reinterpret_cast<uint16_t*>(p.c)[(long)row * p.n + col] =
               finish<ACT, T, GC != 0>(total, p.a_scales[row], col_scale, bias);
@@ -624,7 +632,7 @@ A8Plan plan_a8(int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_group
   // groups of 32 rows stay with the kernel above: one scale per K = 32 instruction leaves the tiled
   // kernel more scale arithmetic than matrix work, and its registers do not hold it
   plan.tile = size_m > 64 && size_k % kA8StepK == 0 && size_n % kA8TileN == 0 &&
-              (num_groups == 1 || size_k / num_groups >= 64);
+              (num_groups == 1 ? size_k <= 65536 : size_k / num_groups >= 64);
   if (plan.tile) {
     plan.mb = 0;
     plan.slabs = (int)((size_m + kA8TileM - 1) / kA8TileM);
