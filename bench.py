@@ -196,7 +196,7 @@ def cpu_baseline(threads: int):
 
 
 def variants_sweep(torch, ops, gen, time_graph):
-    """K = 4096, N = 11008 at M = 1 and 512: act-order (perm gathers the columns
+    """K = 4096, N = 11008 at M = 1 and 512 (W4A8 also at 4096): act-order (perm gathers the columns
     of A, weights repacked in sorted-group order), AWQ (per-group zero points),
     8-bit weights (uint8b128), fp8 weights (float8_e4m3fn, scales with the
     exponent bias folded in), MXFP8 and MXFP4 weights (float8_e4m3fn /
@@ -246,7 +246,7 @@ def variants_sweep(torch, ops, gen, time_graph):
                 zp = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // GROUP, n // 8), dtype=torch.int32, device=dev,
                                    generator=gen)
                 layers.append((qw, sc, zp, empty, empty, ws, scalar_types.uint4))
-        for m in (1, 512):
+        for m in (1, 512) + ((4096,) if name.startswith("w4a8") else ()):
             a = torch.randn((m, k), device=dev, generator=gen).to(act_dtype)
             a_scales = None
             if name.startswith("w4a8"):

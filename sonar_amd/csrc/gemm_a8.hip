@@ -147,11 +147,11 @@ __device__ __forceinline__ uint16_t finish(typename ACT::scalar_t total, float a
   return to_bits<T>(f);
 }
 
-// The sum over this wavefront's share of K: groups (units) u_begin + wave, + 4, ... of
+// The sum over this wavefront's share of K: groups (units) u_begin + wave, + WAVES, ... of
 // [u_begin, u_end).  a_row[rb]: this lane's row of A in row block rb, already offset by the
 // lane's 8 bytes inside a chunk; w_lane: the lane's 16 bytes of chunk 0 of the strip;
 // scales / zeros: row 0 of the matrix's (the expert's) scales and zero points.
-template <typename ACT, typename T, int MB, bool HAS_ZP, bool GROUPED>
+template <typename ACT, typename T, int MB, bool HAS_ZP, bool GROUPED, int WAVES = 4>
 __device__ __forceinline__ void a8_accumulate(typename ACT::acc_t (&acc)[MB][4], const uint8_t* const (&a_row)[MB],
                                               const uint32_t* w_lane, const uint16_t* scales,
                                               const uint32_t* zeros, int n, int strip, int chunks, int unit_chunks,
@@ -161,7 +161,7 @@ __device__ __forceinline__ void a8_accumulate(typename ACT::acc_t (&acc)[MB][4],
   int s_col[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) s_col[j] = strip * kStripN + scale_slot(16 * j + l16, false);
-  for (int u = u_begin + wave; u < u_end; u += 4) {
+  for (int u = u_begin + wave; u < u_end; u += WAVES) {
     acc_t tmp[MB][4];
 #pragma unroll
     for (int rb = 0; rb < MB; ++rb)
@@ -215,10 +215,11 @@ __device__ __forceinline__ void a8_accumulate(typename ACT::acc_t (&acc)[MB][4],
   }
 }
 
-// The four wavefronts' totals meet in LDS; afterwards wavefront w holds, in total[rb][i], the
+// The wavefronts' totals meet in LDS; afterwards wavefront w < 4 holds, in total[rb][i], the
 // sums of column block w: row 16 rb + 4 (lane / 16) + i, column 16 w + lane % 16 of the tile.
-template <typename ACT, int MB>
-__device__ __forceinline__ void a8_reduce(const typename ACT::acc_t (&acc)[MB][4], uint32_t (&red)[4][MB * 16][64],
+template <typename ACT, int MB, int WAVES = 4>
+__device__ __forceinline__ void a8_reduce(const typename ACT::acc_t (&acc)[MB][4],
+                                          uint32_t (&red)[WAVES][MB * 16][64],
                                           typename ACT::scalar_t (&total)[MB][4], int wave, int lane) {
   typedef typename ACT::scalar_t scalar_t;
 #pragma unroll
@@ -231,13 +232,14 @@ __device__ __forceinline__ void a8_reduce(const typename ACT::acc_t (&acc)[MB][4
         red[wave][(rb * 4 + j) * 4 + i][lane] = raw_bits(v);
       }
   __syncthreads();
+  if (wave >= 4) return;
 #pragma unroll
   for (int rb = 0; rb < MB; ++rb)
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       scalar_t sum = 0;
 #pragma unroll
-      for (int ww = 0; ww < 4; ++ww) {
+      for (int ww = 0; ww < WAVES; ++ww) {
         scalar_t part;
         from_raw(red[ww][(rb * 4 + wave) * 4 + i][lane], part);
         sum += part;
@@ -246,11 +248,19 @@ __device__ __forceinline__ void a8_reduce(const typename ACT::acc_t (&acc)[MB][4
     }
 }
 
+// Few rows leave registers and LDS for more wavefronts: 16 for one row block, 8 for two, so that
+// a workgroup walks K sixteen or eight ways and fewer calls need K split over workgroups.
+template <int MB>
+struct A8Waves {
+  static constexpr int value = MB == 1 ? 16 : (MB == 2 ? 8 : 4);
+};
+
 template <typename ACT, typename T, int MB, bool HAS_ZP, bool GROUPED>
-__global__ __launch_bounds__(256) void marlin_a8_kernel(A8Params p) {
+__global__ __launch_bounds__(64 * A8Waves<MB>::value) void marlin_a8_kernel(A8Params p) {
   typedef typename ACT::acc_t acc_t;
   typedef typename ACT::scalar_t scalar_t;
-  __shared__ uint32_t red[4][MB * 16][64];
+  constexpr int WAVES = A8Waves<MB>::value;
+  __shared__ uint32_t red[WAVES][MB * 16][64];
 
   const int strip = blockIdx.x, slab = blockIdx.y, split = blockIdx.z;
   const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -274,10 +284,11 @@ __global__ __launch_bounds__(256) void marlin_a8_kernel(A8Params p) {
   const uint32_t* w_lane = p.w + (long)strip * p.chunks * kChunkWords + lane * 4;
   const int u_begin = split * p.units_per_split;
   const int u_end = min(u_begin + p.units_per_split, p.units);
-  a8_accumulate<ACT, T, MB, HAS_ZP, GROUPED>(acc, a_row, w_lane, p.scales, p.zeros, p.n, strip, p.chunks,
-                                             p.unit_chunks, u_begin, u_end, wave, l16);
+  a8_accumulate<ACT, T, MB, HAS_ZP, GROUPED, WAVES>(acc, a_row, w_lane, p.scales, p.zeros, p.n, strip, p.chunks,
+                                                    p.unit_chunks, u_begin, u_end, wave, l16);
   scalar_t total[MB][4];
-  a8_reduce<ACT, MB>(acc, red, total, wave, lane);
+  a8_reduce<ACT, MB, WAVES>(acc, red, total, wave, lane);
+  if (wave >= 4) return;
 
   const int col = strip * kStripN + 16 * wave + l16;
   float col_scale = 1.0f, bias = 0.0f;
@@ -631,7 +642,7 @@ A8Plan plan_a8(int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_group
   A8Plan plan;
   // groups of 32 rows stay with the kernel above: one scale per K = 32 instruction leaves the tiled
   // kernel more scale arithmetic than matrix work, and its registers do not hold it
-  plan.tile = size_m > 64 && size_k % kA8StepK == 0 && size_n % kA8TileN == 0 &&
+  plan.tile = size_m > 32 && size_k % kA8StepK == 0 && size_n % kA8TileN == 0 &&
               (num_groups == 1 ? size_k <= 65536 : size_k / num_groups >= 64);
   if (plan.tile) {
     plan.mb = 0;
@@ -653,10 +664,11 @@ A8Plan plan_a8(int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_group
   const int chunks = (int)(size_k / kChunkK);
   plan.unit_chunks = num_groups > 1 ? (int)(size_k / num_groups) / kChunkK : 4;
   plan.units = (chunks + plan.unit_chunks - 1) / plan.unit_chunks;
-  // about four workgroups per compute unit, each wavefront with at least two groups
+  // about ten wavefronts per compute unit, each with at least two groups
+  const int waves = plan.mb == 1 ? 16 : (plan.mb == 2 ? 8 : 4);
   const long wgs = (long)(size_n / kStripN) * plan.slabs;
-  int splits = (int)((1024 + wgs - 1) / wgs);
-  if (splits > plan.units / 8) splits = plan.units / 8;
+  int splits = (int)(2560 / (wgs * waves));
+  if (splits > plan.units / (2 * waves)) splits = plan.units / (2 * waves);
   if (splits > 32) splits = 32;
   if (splits < 1) splits = 1;
   plan.units_per_split = (plan.units + splits - 1) / splits;
@@ -666,8 +678,9 @@ A8Plan plan_a8(int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_group
 
 template <typename ACT, typename T, int MB, bool HAS_ZP>
 void launch_a8_mb(const A8Params& p, bool grouped, dim3 grid, hipStream_t st) {
-  if (grouped) marlin_a8_kernel<ACT, T, MB, HAS_ZP, true><<<grid, 256, 0, st>>>(p);
-  else marlin_a8_kernel<ACT, T, MB, HAS_ZP, false><<<grid, 256, 0, st>>>(p);
+  constexpr int threads = 64 * A8Waves<MB>::value;
+  if (grouped) marlin_a8_kernel<ACT, T, MB, HAS_ZP, true><<<grid, threads, 0, st>>>(p);
+  else marlin_a8_kernel<ACT, T, MB, HAS_ZP, false><<<grid, threads, 0, st>>>(p);
 }
 
 template <typename ACT, typename T, bool HAS_ZP>
