@@ -664,10 +664,10 @@ A8Plan plan_a8(int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_group
   const int chunks = (int)(size_k / kChunkK);
   plan.unit_chunks = num_groups > 1 ? (int)(size_k / num_groups) / kChunkK : 4;
   plan.units = (chunks + plan.unit_chunks - 1) / plan.unit_chunks;
-  // about ten wavefronts per compute unit, each with at least two groups
+  // about sixteen wavefronts per compute unit, each with at least two groups
   const int waves = plan.mb == 1 ? 16 : (plan.mb == 2 ? 8 : 4);
   const long wgs = (long)(size_n / kStripN) * plan.slabs;
-  int splits = (int)(2560 / (wgs * waves));
+  int splits = (int)(4096 / (wgs * waves));
   if (splits > plan.units / (2 * waves)) splits = plan.units / (2 * waves);
   if (splits > 32) splits = 32;
   if (splits < 1) splits = 1;
