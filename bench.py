@@ -342,19 +342,45 @@ def moe_sweep(torch, gen, time_graph):
                                       expert_ids, past, tw, bs, 1, True, scalar_types.float4_e2m1f, t * topk, hidden,
                                       inter, True, False, True, False)
 
+        # the same codes in the order of 8-bit activations, int8 tokens with a scale a row, 16-bit integer
+        # group scales; blocks of at least 16 slots (marlin_moe.py:328-329)
+        bs8 = max(bs, 16)
+        sorted8, experts8, past8 = (sorted_ids, expert_ids, past) if bs8 == bs else \
+            fused_moe.moe_align_block_size(ti, bs8, e)
+        i1 = torch.randint(1, 4097, (e, hidden // GROUP, 2 * inter), dtype=torch.int16, device=dev,
+                           generator=gen).view(dt)
+        i2 = torch.randint(1, 4097, (e, inter // GROUP, hidden), dtype=torch.int16, device=dev, generator=gen).view(dt)
+        xq, xs = ops.per_token_quant_int8(x)
+        h2q, h2s = ops.per_token_quant_int8(h2)
+        xs, h2s = xs * 2.0 ** -12, h2s * 2.0 ** -12
+
+        def gemm1_a8(i=0):
+            ops.moe_wna16_marlin_gemm(xq, h1, w1, None, i1, xs, None, None, None, None, ws, sorted8, experts8, past8,
+                                      tw, bs8, topk, False, scalar_types.uint4b8, t, 2 * inter, hidden, True, False,
+                                      True, False)
+
+        def gemm2_a8(i=0):
+            ops.moe_wna16_marlin_gemm(h2q, y, w2, None, i2, h2s, None, None, None, None, ws, sorted8, experts8, past8,
+                                      tw, bs8, 1, True, scalar_types.uint4b8, t * topk, hidden, inter, True, False,
+                                      True, False)
+
         reps = 8 if t == 16 else 2
         cases = [("gate_up", gemm1, hidden, 2 * inter, t, GROUP, 2), ("down", gemm2, inter, hidden, t * topk, GROUP, 2),
                  ("gate_up (mxfp4)", gemm1_mx, hidden, 2 * inter, t, 32, 1),
-                 ("down (mxfp4)", gemm2_mx, inter, hidden, t * topk, 32, 1)]
+                 ("down (mxfp4)", gemm2_mx, inter, hidden, t * topk, 32, 1),
+                 ("gate_up (w4a8 int8)", gemm1_a8, hidden, 2 * inter, t, GROUP, 2),
+                 ("down (w4a8 int8)", gemm2_a8, inter, hidden, t * topk, GROUP, 2)]
         for name, fn, k, n, rows, group, scale_bytes in cases:
             s = time_graph(torch, fn, reps)
             weights = routed * (k * n // 2 + (k // group) * n * scale_bytes)
-            nb = weights + rows * k * 2 + t * topk * n * 2 + sorted_ids.numel() * 4 + expert_ids.numel() * 4
+            a8 = "w4a8" in name
+            nb = weights + rows * k * (1 if a8 else 2) + t * topk * n * 2 + sorted_ids.numel() * 4 + \
+                expert_ids.numel() * 4
             fl = 2 * t * topk * n * k
             out.append({"tokens": t, "gemm": name, "block_size": bs, "experts_routed": routed,
                         "us": round(s * 1e6, 1), "GBps": round(nb / s / 1e9, 1), "TFLOPs": round(fl / s / 1e12, 2),
                         "frac_hbm": round(nb / s / 1e9 / HBM_PEAK_GBPS, 4),
-                        "frac_mfma": round(fl / s / 1e12 / MFMA_PEAK_TFLOPS, 4)})
+                        "frac_mfma": round(fl / s / 1e12 / (MFMA_PEAK_8BIT_TFLOPS if a8 else MFMA_PEAK_TFLOPS), 4)})
             print("moe", json.dumps(out[-1]), file=sys.stderr, flush=True)
         torch.cuda.synchronize()
         t0 = time.perf_counter()

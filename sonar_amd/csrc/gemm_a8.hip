@@ -402,8 +402,12 @@ __global__ __launch_bounds__(256) void marlin_moe_a8_kernel(MoeA8Params q) {
 // v_mfma_f32_16x16x128_f8f6f4); smaller groups take the K = 32 forms.
 constexpr int kA8TileM = 128, kA8TileN = 128, kA8StepK = 128, kA8StepChunks = 4, kA8RowBytes = 144;
 
-template <typename ACT, typename T, bool HAS_ZP, int GC>
-__global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
+// MOE: the grouped form.  A workgroup is one block of up to 64 sorted slots times 256 columns;
+// wavefront w owns strip 4 tile + w, so the four share the rows in LDS and none repeats another's
+// dequantisation.  Rows are gathered through sorted_token_ids, the whole of K in one workgroup.
+template <typename ACT, typename T, bool HAS_ZP, int GC, bool MOE = false>
+__global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(MoeA8Params q) {
+  const A8Params& p = q.g;
   typedef typename ACT::acc_t acc_t;
   typedef typename ACT::scalar_t scalar_t;
   typedef typename ACT::wide_t wide_t;
@@ -414,23 +418,55 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
   // scales, in the epilogue (the host sends K beyond 2^16 to the slab kernel: 2^16 * 127 * 128 < 2^31)
   constexpr bool kZpForm = HAS_ZP;
   constexpr int kShift = (ACT::kInteger && !kZpForm) ? ACT::kShift : 0;
-  __shared__ __align__(16) uint8_t tile[2][kA8TileM * kA8RowBytes];
+  constexpr int kRows = MOE ? 64 : kA8TileM;
+  constexpr int kLoads = MOE ? 2 : 4;                       // 16-byte loads of a thread per step
+  __shared__ __align__(16) uint8_t tile[2][kRows * kA8RowBytes];
+  __shared__ int slot_id[64];
 
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int l16 = lane & 15, kb = lane >> 4;
-  const int wr = wave >> 1, wc = wave & 1;
-  const int m0 = blockIdx.y * kA8TileM;
-  const int strip = blockIdx.x * 2 + wc;
-  const int s_begin = blockIdx.z * p.units_per_split;
-  const int s_end = min(s_begin + p.units_per_split, p.units);
+  const int wr = MOE ? 0 : wave >> 1, wc = MOE ? wave : wave & 1;
+  const int m0 = MOE ? 0 : blockIdx.y * kA8TileM;
+  const int strip = blockIdx.x * (MOE ? 4 : 2) + wc;
+  const int s_begin = MOE ? 0 : blockIdx.z * p.units_per_split;
+  const int s_end = MOE ? p.units : min(s_begin + p.units_per_split, p.units);
 
-  // copy role: thread t brings 64 bytes of row t / 2 of the tile
-  const int c_row = tid >> 1, c_half = tid & 1;
-  int src_row = m0 + c_row;
-  if (src_row >= p.m) src_row = p.m - 1;                  // results of such rows are dropped
-  const uint8_t* a_src = p.a + (long)src_row * p.a_row_stride + c_half * 64;
+  int expert = 0;
+  if (MOE) {
+    // the whole workgroup leaves together: nothing below is reached by a part of it
+    const int block = blockIdx.y;
+    if (block * q.block_size >= q.num_post_pad[0]) return;
+    expert = q.expert_ids[block];
+    if (expert < 0 || expert >= q.num_experts) return;
+    if (tid < 64) {
+      int id = -1;
+      const int at = block * q.block_size + tid;
+      if (tid < q.block_size && at < q.sorted_len) {
+        id = q.sorted_ids[at];
+        if (id < 0 || id >= p.m * q.top_k) id = -1;
+      }
+      slot_id[tid] = id;
+    }
+    __syncthreads();
+  }
+
+  // copy role: thread t brings 64 bytes of row t / 2 of the tile (MOE: 32 bytes of row t / 4)
+  const int c_row = MOE ? tid >> 2 : tid >> 1;
+  const int c_off = MOE ? (tid & 3) * 32 : (tid & 1) * 64;  // first byte inside the 128 of a step
+  int src_row;
+  if (MOE) {
+    const int id = slot_id[c_row];
+    src_row = id < 0 ? 0 : id / q.top_k;                    // padding reads row 0, its results are dropped
+  } else {
+    src_row = m0 + c_row;
+    if (src_row >= p.m) src_row = p.m - 1;                  // results of such rows are dropped
+  }
+  const uint8_t* a_src = p.a + (long)src_row * p.a_row_stride + c_off;
   const int dst_row = c_row * kA8RowBytes;
-  const uint32_t* w_lane = p.w + (long)strip * p.chunks * kChunkWords + lane * 4;
+  const long expert_words = MOE ? (long)expert * p.chunks * kChunkWords * (p.n / kStripN) : 0;
+  const uint32_t* w_lane = p.w + expert_words + (long)strip * p.chunks * kChunkWords + lane * 4;
+  const uint16_t* scales = p.scales + (MOE ? (long)expert * q.groups * p.n : 0);
+  const uint32_t* zeros = HAS_ZP ? p.zeros + (MOE ? (long)expert * q.groups * (p.n / 8) : 0) : nullptr;
   int s_col[4];
 #pragma unroll
   for (int j = 0; j < 4; ++j) s_col[j] = strip * kStripN + scale_slot(16 * j + l16, false);
@@ -441,11 +477,11 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) acc[rb][j] = tmp[rb][j] = acc_t{0, 0, 0, 0};
 
-  uint4 ra[4];
+  uint4 ra[kLoads];
   u32x4_t wq[kA8StepChunks], wq_next[kA8StepChunks];
   auto load_a = [&](int step) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
+    for (int i = 0; i < kLoads; ++i)
       ra[i] = *reinterpret_cast<const uint4*>(a_src + (long)step * kA8StepK + 16 * i);
   };
   auto load_w = [&](int step, u32x4_t (&dst)[kA8StepChunks]) {
@@ -455,8 +491,9 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
   };
   auto store_a = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      const int c = c_half * 2 + (i >> 1), kb0 = 2 * (i & 1);
+    for (int i = 0; i < kLoads; ++i) {
+      const int off = c_off + 16 * i;                       // 16 bytes = k blocks kb0, kb0 + 1 of chunk c
+      const int c = off >> 5, kb0 = ((off >> 4) & 1) * 2;
       uint2 u0, u1;
       u0.x = __builtin_amdgcn_perm(ra[i].y, ra[i].x, 0x05010400u);   // bytes k = 0, 4, 1, 5
       u0.y = __builtin_amdgcn_perm(ra[i].y, ra[i].x, 0x07030602u);   // bytes k = 2, 6, 3, 7
@@ -470,7 +507,7 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
   auto apply_group = [&](int g) {
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const uint16_t bits = p.scales[(long)g * p.n + s_col[j]];
+      const uint16_t bits = scales[(long)g * p.n + s_col[j]];
       scalar_t sc;
       if constexpr (ACT::kInteger) sc = (int)bits;
       else sc = from_bits<T>(bits);
@@ -508,7 +545,7 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
 #pragma unroll
       for (int gi = 0; gi < kGroupsPerStep; ++gi) {
         const int g = GC == 0 ? 0 : step * kGroupsPerStep + gi;
-        zw[gi] = p.zeros[(long)g * (p.n / 8) + strip * 8 + (l16 & 7)];
+        zw[gi] = zeros[(long)g * (p.n / 8) + strip * 8 + (l16 & 7)];
       }
     }
     const uint8_t* rows = &tile[buf][(64 * wr + l16) * kA8RowBytes];
@@ -592,17 +629,25 @@ __global__ __launch_bounds__(256, 2) void marlin_a8_tile_kernel(A8Params p) {
     const int col = strip * kStripN + 16 * j + l16;
     float col_scale = 1.0f, bias = 0.0f;
     if (p.splits == 1) {
-      if (GC == 0) col_scale = from_bits<T>(p.scales[s_col[j]]);
-      if (p.bias) bias = from_bits<T>(p.bias[s_col[j]]);
+      if (GC == 0) col_scale = from_bits<T>(scales[s_col[j]]);
+      if (p.bias) bias = from_bits<T>(p.bias[(MOE ? (long)expert * p.n : 0) + s_col[j]]);
     }
 #pragma unroll
     for (int rb = 0; rb < 4; ++rb)
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int row = m0 + 64 * wr + 16 * rb + 4 * kb + i;
-        if (row >= p.m) continue;
         scalar_t total = acc[rb][j][i];
         if constexpr (ACT::kInteger && GC == 0) total >>= kShift;
+        if constexpr (MOE) {
+          const int id = slot_id[16 * rb + 4 * kb + i];
+          if (id < 0) continue;
+          uint16_t o = finish<ACT, T, GC != 0>(total, p.a_scales[id / q.top_k], col_scale, bias);
+          if (q.mul_topk) o = to_bits<T>(from_bits<T>(o) * from_bits<T>(to_bits<T>(q.topk_weights[id])));
+          reinterpret_cast<uint16_t*>(p.c)[(long)id * p.n + col] = o;
+          continue;
+        }
+        const int row = m0 + 64 * wr + 16 * rb + 4 * kb + i;
+        if (row >= p.m) continue;
         if (p.splits == 1)
           reinterpret_cast<uint16_t*>(p.c)[(long)row * p.n + col] =
               finish<ACT, T, GC != 0>(total, p.a_scales[row], col_scale, bias);
@@ -683,12 +728,12 @@ void launch_a8_mb(const A8Params& p, bool grouped, dim3 grid, hipStream_t st) {
   else marlin_a8_kernel<ACT, T, MB, HAS_ZP, false><<<grid, threads, 0, st>>>(p);
 }
 
-template <typename ACT, typename T, bool HAS_ZP>
-void launch_a8_tile_gc(const A8Params& p, int gc, dim3 grid, hipStream_t st) {
+template <typename ACT, typename T, bool HAS_ZP, bool MOE>
+void launch_a8_tile_gc(const MoeA8Params& q, int gc, dim3 grid, hipStream_t st) {
   switch (gc) {
-    case 0: marlin_a8_tile_kernel<ACT, T, HAS_ZP, 0><<<grid, 256, 0, st>>>(p); break;
-    case 2: marlin_a8_tile_kernel<ACT, T, HAS_ZP, 2><<<grid, 256, 0, st>>>(p); break;
-    default: marlin_a8_tile_kernel<ACT, T, HAS_ZP, 4><<<grid, 256, 0, st>>>(p); break;
+    case 0: marlin_a8_tile_kernel<ACT, T, HAS_ZP, 0, MOE><<<grid, 256, 0, st>>>(q); break;
+    case 2: marlin_a8_tile_kernel<ACT, T, HAS_ZP, 2, MOE><<<grid, 256, 0, st>>>(q); break;
+    default: marlin_a8_tile_kernel<ACT, T, HAS_ZP, 4, MOE><<<grid, 256, 0, st>>>(q); break;
   }
 }
 
@@ -697,8 +742,10 @@ void launch_a8(const A8Params& p, const A8Plan& plan, bool grouped, hipStream_t 
   const bool zp = p.zeros != nullptr;
   if (plan.tile) {
     const dim3 grid(p.n / kA8TileN, plan.slabs, plan.splits);
-    if (zp) launch_a8_tile_gc<ACT, T, true>(p, plan.unit_chunks, grid, st);
-    else launch_a8_tile_gc<ACT, T, false>(p, plan.unit_chunks, grid, st);
+    MoeA8Params q = {};
+    q.g = p;
+    if (zp) launch_a8_tile_gc<ACT, T, true, false>(q, plan.unit_chunks, grid, st);
+    else launch_a8_tile_gc<ACT, T, false, false>(q, plan.unit_chunks, grid, st);
     if (plan.splits > 1) {
       long blocks = ((long)p.m * p.n + 255) / 256;
       if (blocks > 4096) blocks = 4096;
@@ -741,8 +788,20 @@ void launch_moe_a8_mb(const MoeA8Params& q, bool grouped, bool zp, dim3 grid, hi
 
 template <typename ACT, typename T>
 void launch_moe_a8(const MoeA8Params& q, bool grouped, int blocks, hipStream_t st) {
-  const dim3 grid(q.g.n / kStripN, blocks, 1);
   const bool zp = q.g.zeros != nullptr;
+  // blocks of more than 32 slots on shapes the tiled kernel takes (groups of 64 rows or more)
+  const int gc = grouped ? q.g.unit_chunks : 0;
+  if (q.block_size > 32 && q.g.n % 256 == 0 && q.g.chunks % kA8StepChunks == 0 && gc != 1 &&
+      (grouped || q.g.chunks <= 2048)) {
+    MoeA8Params t = q;
+    t.g.units = q.g.chunks / kA8StepChunks;
+    t.g.units_per_split = t.g.units;
+    const dim3 grid(q.g.n / 256, blocks, 1);
+    if (zp) launch_a8_tile_gc<ACT, T, true, true>(t, gc, grid, st);
+    else launch_a8_tile_gc<ACT, T, false, true>(t, gc, grid, st);
+    return;
+  }
+  const dim3 grid(q.g.n / kStripN, blocks, 1);
   switch ((q.block_size + 15) / 16) {
     case 1: launch_moe_a8_mb<ACT, T, 1>(q, grouped, zp, grid, st); break;
     case 2: launch_moe_a8_mb<ACT, T, 2>(q, grouped, zp, grid, st); break;

@@ -67,7 +67,32 @@ def layer8_fixture(seed, k, n, g, dtype, m):
             "c_ref": mo.gemm_reference(a, w)}
 
 
+def w4a8_fixture(seed, k, n, g, dtype, m):
+    """4-bit weights with int8 activations: the order of 8-bit activations, integer group
+    scales, per-token quantised activations and the exact result of the integer GEMM."""
+    rng = np.random.default_rng(seed)
+    q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    zeros = rng.integers(0, 16, size=(k // g, n), dtype=np.int32)
+    scales = mo.round_to_dtype(rng.uniform(1e-3, 1e-2, size=(k // g, n)).astype(np.float32), dtype)
+    ints, factor = mo.marlin_act_int8_process_scales(scales)
+    marlin = mo.gptq_marlin_repack_a8(mo.gptq_pack(q), k, n)
+    x = rng.standard_normal((m, k)).astype(np.float32)
+    a_q, a_s = mo.per_token_quant_int8(x)
+    a_s = (a_s * factor).astype(np.float32)
+    return {"size_k": np.int64(k), "size_n": np.int64(n), "group_size": np.int64(g), "size_m": np.int64(m),
+            "q": q.astype(np.uint8), "gptq_packed": mo.gptq_pack(q), "awq_packed": mo.awq_pack(q),
+            "marlin_a8": marlin, "gfx950": mo.marlin_a8_to_gfx950(marlin, k, n),
+            "fp8_preprocessed": mo.int4_fp8_preprocess(q).astype(np.uint8),
+            "zeros": zeros.astype(np.uint8), "zeros_marlin_a8": mo.marlin_zero_points_a8(zeros, k // g, n),
+            "int_scales": ints, "int_scales_marlin_a8": mo.marlin_permute_scales_a8(ints, k, n, g),
+            "x": x, "a_q": a_q, "a_scales": a_s,
+            "c_bits": mo.to_bits16(mo.gemm_w4a8_int8(a_q, a_s, q, g, ints, dtype), dtype),
+            "c_zp_bits": mo.to_bits16(mo.gemm_w4a8_int8(a_q, a_s, q, g, ints, dtype, zeros), dtype)}
+
+
 def main():
+    np.savez_compressed(os.path.join(HERE, "w4a8_int8_fp16_k256_n128_g64.npz"),
+                        **w4a8_fixture(105, 256, 128, 64, "fp16", 9))
     np.savez_compressed(os.path.join(HERE, "gptq8_bf16_k128_n64_g64.npz"),
                         **layer8_fixture(104, 128, 64, 64, "bf16", 6))
     np.savez_compressed(os.path.join(HERE, "gptq_fp16_k128_n128_g64.npz"),

@@ -209,3 +209,55 @@ def test_hip_kernels_reproduce_fp8_and_mxfp4_tables(dtype):
     _lib.check(lib.sonar_marlin_dequant(gu.ptr(native), _lib.LAYOUT_GFX950, gu.ptr(scales), None, None, gu.ptr(w),
                                         gu.dtype_code("bf16"), _lib.TYPE_FLOAT4_E2M1F, n, k, k // 32, 1, gu.stream()))
     assert np.array_equal(w.view(torch.int16).cpu().numpy().view(np.uint16), f["dequant_bits"])
+
+
+def test_oracle_reproduces_w4a8_fixture():
+    f = load("w4a8_int8_fp16_k256_n128_g64.npz")
+    k, n, g = int(f["size_k"]), int(f["size_n"]), int(f["group_size"])
+    q, zeros = f["q"].astype(np.int32), f["zeros"].astype(np.int32)
+    assert np.array_equal(mo.gptq_marlin_repack_a8(f["gptq_packed"], k, n), f["marlin_a8"])
+    assert np.array_equal(mo.awq_marlin_repack_a8(f["awq_packed"], k, n), f["marlin_a8"])
+    assert np.array_equal(mo.marlin_pack_recipe_a8(q), f["marlin_a8"])
+    assert np.array_equal(mo.marlin_a8_to_gfx950(f["marlin_a8"], k, n), f["gfx950"])
+    assert np.array_equal(mo.gfx950_pack(q), f["gfx950"])        # the same stream as for 16-bit activations
+    assert np.array_equal(mo.int4_fp8_preprocess(q), f["fp8_preprocessed"])
+    assert np.array_equal(mo.marlin_zero_points_a8(zeros, k // g, n), f["zeros_marlin_a8"])
+    assert np.array_equal(mo.marlin_permute_scales_a8(f["int_scales"], k, n, g), f["int_scales_marlin_a8"])
+    a_q, a_s = mo.per_token_quant_int8(f["x"])
+    assert np.array_equal(a_q, f["a_q"])
+    for zp, key in ((None, "c_bits"), (zeros, "c_zp_bits")):
+        c = mo.gemm_w4a8_int8(f["a_q"], f["a_scales"], q, g, f["int_scales"], "fp16", zp)
+        assert np.array_equal(mo.to_bits16(c, "fp16"), f[key])
+
+
+@pytest.mark.gpu
+def test_hip_kernels_reproduce_w4a8_fixture():
+    import torch
+
+    from sonar_amd import _lib
+    from tests import gpu_util as gu
+    f = load("w4a8_int8_fp16_k256_n128_g64.npz")
+    k, n, g, m = int(f["size_k"]), int(f["size_n"]), int(f["group_size"]), int(f["size_m"])
+    lib = _lib.load()
+    marlin = torch.empty((k // 16, 2 * n), dtype=torch.int32, device=gu.DEV)
+    src = gu.dev_i32(f["gptq_packed"])
+    _lib.check(lib.sonar_gptq_marlin_repack_a8(gu.ptr(src), gu.ptr(marlin), k, n, 4, gu.stream()))
+    assert np.array_equal(marlin.cpu().numpy().view(np.uint32), U32(f["marlin_a8"]))
+    native = torch.empty(k * n // 8, dtype=torch.int32, device=gu.DEV)
+    _lib.check(lib.sonar_marlin_a8_to_gfx950(gu.ptr(marlin), gu.ptr(native), k, n, gu.stream()))
+    assert np.array_equal(native.cpu().numpy().view(np.uint32), U32(f["gfx950"].reshape(-1)))
+    x = torch.from_numpy(f["x"]).to(gu.DEV)
+    a_q = torch.empty((m, k), dtype=torch.int8, device=gu.DEV)
+    a_s = torch.empty(m, dtype=torch.float32, device=gu.DEV)
+    _lib.check(lib.sonar_per_token_quant_int8(gu.ptr(x), _lib.DTYPE_F32, k, gu.ptr(a_q), gu.ptr(a_s), m, k,
+                                              gu.stream()))
+    assert np.array_equal(a_q.cpu().numpy(), f["a_q"])
+    scales = torch.from_numpy(f["int_scales_marlin_a8"].copy()).to(gu.DEV)
+    a_scales = torch.from_numpy(f["a_scales"].reshape(-1).copy()).to(gu.DEV)
+    zeros = gu.dev_i32(f["zeros_marlin_a8"])
+    for zp, b_type, key in ((None, _lib.TYPE_UINT4B8, "c_bits"), (zeros, _lib.TYPE_UINT4, "c_zp_bits")):
+        c = torch.empty((m, n), dtype=torch.float16, device=gu.DEV)
+        _lib.check(lib.sonar_marlin_gemm_a8(gu.ptr(a_q), k, _lib.ADTYPE_INT8, gu.ptr(c), gu.ptr(native),
+                                            _lib.LAYOUT_GFX950, None, gu.ptr(scales), gu.ptr(a_scales), gu.ptr(zp),
+                                            None, 0, _lib.DTYPE_F16, b_type, m, n, k, k // g, gu.stream()))
+        assert np.array_equal(c.view(torch.int16).cpu().numpy().view(np.uint16), f[key])

@@ -228,6 +228,11 @@ MOE_A8_CASES = [
     (19, 512, 64, 6, 2, 8, 32, True, "bf16", False, False),
     (100, 1024, 128, 4, 1, 64, 128, True, "fp16", True, False),
     (47, 256, 256, 7, 4, 48, 64, False, "bf16", False, True),
+    # blocks of more than 32 slots, N a multiple of 256: the tiled kernel's grouped form
+    (300, 1024, 512, 4, 2, 64, 128, False, "fp16", True, True),
+    (150, 512, 256, 3, 2, 64, -1, False, "bf16", False, False),
+    (90, 512, 256, 5, 3, 48, 64, True, "fp16", False, True),
+    (200, 256, 512, 6, 1, 64, 128, True, "bf16", True, False),
 ]
 
 
