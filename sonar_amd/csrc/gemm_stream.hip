@@ -1830,6 +1830,13 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
                          total_units * n_strips < (1LL << 31);
   p.parts = p.total_units < cus ? p.total_units : cus;
   if (strip_per_workgroup && row_slabs) p.parts = (int)n_strips;
+  // One row block on a matrix with about as many strips as compute units: a workgroup per strip, so that
+  // no strip is shared and the fix-up launch goes (K = 4096, N = 11008, M = 1: 8-bit codes 18.4 -> 15.0 us,
+  // NVFP4 17.2 -> 14.0 us).  (Sixteen wavefronts a workgroup on top of that: 26 us, the unit buffers of
+  // the general kernels do not fit 128 registers.)
+  // From 48 rows on the even split over all compute units is ahead again (8-bit codes, M = 64: 29.1
+  // against 31.2 us).
+  if (size_m <= 16 && n_strips >= cus / 2 && n_strips <= 4 * cus) p.parts = (int)n_strips;
   p.slabs = 1;
   p.grid_parts = p.parts;
   p.tickets = nullptr;
