@@ -119,9 +119,9 @@ int sonar_gfx950_to_marlin8(const uint32_t* gfx950, uint32_t* out,
 
 /* The repack ops with is_a_8bit = true (gptq_marlin_repack.cu:14-268, awq_marlin_repack.cu:14-212):
  * 4-bit codes into the order the reference's kernels read with 8-bit activations, tiles of
- * 32 (k) x 32 (n).  in as for the ops above, out (K/16, 2N) int32.  size_k % 32 == 0,
- * size_n % 64 == 0, num_bits 4 (8 is SONAR_E_UNSUPPORTED: the GEMM has no 8-bit weights with 8-bit
- * activations); no perm (the reference's kernel refuses act-order with is_a_8bit). */
+ * 32 (k) x 32 (n).  in as for the ops above, out (K/16, 2N) int32 ((K/16, 4N) for 8-bit codes, GPTQ
+ * source only; no GEMM takes that order, here or in the reference).  size_k % 32 == 0,
+ * size_n % 64 == 0; no perm (the reference's kernel refuses act-order with is_a_8bit). */
 int sonar_gptq_marlin_repack_a8(const uint32_t* b_q_weight, uint32_t* out,
                                 int64_t size_k, int64_t size_n, int num_bits, void* stream);
 int sonar_awq_marlin_repack_a8(const uint32_t* b_q_weight, uint32_t* out,

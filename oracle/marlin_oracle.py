@@ -399,6 +399,49 @@ def awq_marlin_repack_a8(b_q_weight: np.ndarray, size_k: int, size_n: int) -> np
     return marlin_pack_a8(q)
 
 
+def marlin_pack8_recipe_a8(q: np.ndarray) -> np.ndarray:
+    """8-bit codes in the order of 8-bit activations, by the recipe: the same gather table as
+    for 4-bit codes before its interleave (get_weight_perm(8, True): interleave [0, 1, 2, 3],
+    marlin_utils_test.py:111-115), four codes a word.  (K, N) -> (K/16, 4N) int32.  No GEMM of
+    the reference takes this order (W8A8 is not a Marlin mode); the repack op produces it."""
+    k, n = q.shape
+    assert k % 32 == 0 and n % 64 == 0
+    perm = marlin_weight_perm_recipe_a8().reshape(-1, 8)[:, np.argsort(A8_ORDER)].ravel()   # interleave undone
+    t = q.reshape(k // 32, 32, n // 16, 16).transpose(0, 2, 1, 3).reshape(k // 16, n * 16)
+    t = t.reshape(-1, perm.size)[:, perm].reshape(t.shape)
+    u = t.astype(np.uint32).reshape(k // 16, n * 4, 4)
+    out = np.zeros((k // 16, n * 4), dtype=np.uint32)
+    for i in range(4):
+        out |= u[:, :, i] << np.uint32(8 * i)
+    return out.view(np.int32)
+
+
+def marlin_pack8_closed_form_a8(q: np.ndarray) -> np.ndarray:
+    """The same from the repack kernel's arithmetic (gptq_marlin_repack.cu:129-141,176-236 with
+    is_a_8bit, num_bits 8): tile (kt, nt) of 32 x 32 is 256 words; word lane*8 + 2*warp + h holds
+    column 8*warp + lane/4, rows 4*(lane%4) + {0,1,2,3} + 16h at bytes 0..3."""
+    k, n = q.shape
+    assert k % 32 == 0 and n % 64 == 0
+    kt_n, nt_n = k // 32, n // 32
+    tile = q.reshape(kt_n, 32, nt_n, 32).astype(np.uint32)
+    out = np.zeros((kt_n, nt_n, 32, 4, 2), dtype=np.uint32)
+    for lane in range(32):
+        for warp in range(4):
+            col = 8 * warp + lane // 4
+            for h in range(2):
+                word = np.zeros((kt_n, nt_n), dtype=np.uint32)
+                for i in range(4):
+                    word |= tile[:, 4 * (lane % 4) + i + 16 * h, :, col] << np.uint32(8 * i)
+                out[:, :, lane, warp, h] = word
+    return out.reshape(k // 16, n * 4).view(np.int32)
+
+
+def gptq_marlin_repack8_a8(b_q_weight: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
+    q = unpack_rows8(b_q_weight)
+    assert q.shape == (size_k, size_n)
+    return marlin_pack8_closed_form_a8(q)
+
+
 def marlin_a8_to_gfx950(marlin_packed: np.ndarray, size_k: int, size_n: int) -> np.ndarray:
     return gfx950_pack(marlin_unpack_a8(marlin_packed, size_k, size_n))
 

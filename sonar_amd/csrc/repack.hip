@@ -301,6 +301,25 @@ __global__ __launch_bounds__(256) void to_marlin_a8_kernel(const uint32_t* __res
   }
 }
 
+// 8-bit codes in that order (gptq_marlin_repack.cu:216-236 with is_a_8bit): a 32 x 32 tile is 256
+// words; word lane*8 + 2*w + h: column 8w + lane/4, rows 4*(lane%4) + {0..3} + 16h at bytes 0..3.
+// No GEMM takes it (the reference has no 8-bit weights with 8-bit activations either); the
+// repack op produces it.  Source: GPTQ (K/4, N) words.
+__global__ __launch_bounds__(256) void gptq8_to_marlin_a8_kernel(const uint32_t* __restrict__ in,
+                                                                uint32_t* __restrict__ out, int size_k, int size_n,
+                                                                long total_words) {
+  const int n_tiles = size_n / kA8Tile;
+  for (long idx = (long)blockIdx.x * blockDim.x + threadIdx.x; idx < total_words;
+       idx += (long)gridDim.x * blockDim.x) {
+    const long tile = idx / 256;
+    const int word = (int)(idx % 256);
+    const int lane = word >> 3, w = (word >> 1) & 3, h = word & 1;
+    const int n = (int)(tile % n_tiles) * kA8Tile + 8 * w + (lane >> 2);
+    const int k0 = (int)(tile / n_tiles) * kA8Tile + 4 * (lane & 3) + 16 * h;   // a multiple of 4: one source word
+    out[idx] = in[(long)(k0 >> 2) * size_n + n];
+  }
+}
+
 // One thread per gfx950 word (rows 32c + 8*(L/16) + t of column 64s + 16j + L%16).
 __global__ __launch_bounds__(256) void marlin_a8_to_gfx950_kernel(const uint32_t* __restrict__ in,
                                                                  uint32_t* __restrict__ out, int size_k,
@@ -459,9 +478,6 @@ extern "C" int sonar_gfx950_to_marlin8(const uint32_t* gfx950, uint32_t* out, in
 namespace {
 int check_a8_shape(int64_t size_k, int64_t size_n, int num_bits) {
   if (int rc = check_repack_shape(size_k, size_n, num_bits)) return rc;
-  if (num_bits != 4)
-    return fail(SONAR_E_UNSUPPORTED, "Unsupported repack config: num_bits = %d with is_a_8bit (the GEMM has no "
-                "8-bit weights with 8-bit activations)", num_bits);
   SONAR_REQUIRE(size_k % kA8Tile == 0, "size_k = %ld is not divisible by %d (the tile of 8-bit activations)",
                 (long)size_k, kA8Tile);
   return SONAR_OK;
@@ -472,6 +488,12 @@ extern "C" int sonar_gptq_marlin_repack_a8(const uint32_t* b_q_weight, uint32_t*
                                            int64_t size_n, int num_bits, void* stream) {
   if (int rc = check_a8_shape(size_k, size_n, num_bits)) return rc;
   SONAR_REQUIRE(b_q_weight && out, "b_q_weight and out must not be NULL");
+  if (num_bits == 8) {
+    const long words = size_k * size_n / 4;
+    gptq8_to_marlin_a8_kernel<<<grid_for(words), 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k,
+                                                                               (int)size_n, words);
+    return launch_status("gptq8_to_marlin_a8_kernel");
+  }
   const long total = size_k * size_n / 8;
   to_marlin_a8_kernel<0><<<grid_for(total), 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k,
                                                                           (int)size_n, total);
@@ -481,6 +503,7 @@ extern "C" int sonar_gptq_marlin_repack_a8(const uint32_t* b_q_weight, uint32_t*
 extern "C" int sonar_awq_marlin_repack_a8(const uint32_t* b_q_weight, uint32_t* out, int64_t size_k,
                                           int64_t size_n, int num_bits, void* stream) {
   if (int rc = check_a8_shape(size_k, size_n, num_bits)) return rc;
+  if (num_bits != 4) return fail(SONAR_E_UNSUPPORTED, "awq_marlin_repack: 8-bit AWQ weights are not built");
   SONAR_REQUIRE(b_q_weight && out, "b_q_weight and out must not be NULL");
   const long total = size_k * size_n / 8;
   to_marlin_a8_kernel<1><<<grid_for(total), 256, 0, (hipStream_t)stream>>>(b_q_weight, out, (int)size_k,

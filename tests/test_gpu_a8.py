@@ -47,11 +47,23 @@ def test_repack_a8_bit_exact(k, n):
     assert torch.equal(back, got)
 
 
+@pytest.mark.parametrize("k,n", [(128 * 5, 256 * 7), (32, 64)])
+def test_repack8_a8_bit_exact(k, n):
+    """8-bit codes in the order of 8-bit activations (produced for parity with the repack op; no GEMM
+    takes it)."""
+    rng = np.random.default_rng(k * 3 + n)
+    q = rng.integers(0, 256, size=(k, n), dtype=np.int32)
+    out = torch.empty((k // 16, 4 * n), dtype=torch.int32, device=DEV)
+    src = dev_i32(mo.pack_rows8(q))
+    _lib.check(_lib.load().sonar_gptq_marlin_repack_a8(ptr(src), ptr(out), k, n, 8, stream()))
+    assert np.array_equal(out.cpu().numpy(), mo.marlin_pack8_closed_form_a8(q))
+
+
 def test_repack_a8_rejections():
     lib = _lib.load()
     w = torch.zeros(64 * 64 // 4, dtype=torch.int32, device=DEV)
     out = torch.zeros(64 * 64 // 4, dtype=torch.int32, device=DEV)
-    assert lib.sonar_gptq_marlin_repack_a8(ptr(w), ptr(out), 64, 64, 8, stream()) == _lib.E_UNSUPPORTED
+    assert lib.sonar_awq_marlin_repack_a8(ptr(w), ptr(out), 64, 64, 8, stream()) == _lib.E_UNSUPPORTED
     assert lib.sonar_gptq_marlin_repack_a8(ptr(w), ptr(out), 48, 64, 4, stream()) == _lib.E_INVALID
     assert b"32" in lib.sonar_marlin_last_error()
     assert lib.sonar_awq_marlin_repack_a8(ptr(w), ptr(out), 64, 32, 4, stream()) == _lib.E_INVALID

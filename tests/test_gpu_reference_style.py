@@ -61,9 +61,6 @@ def test_gptq_marlin_repack(n_chunk, quant_type, act_order, is_a_8bit, nk_factor
     size_k, size_n, group_size = 128 * k_factor, n_chunk * n_factor, 128
     if act_order and is_a_8bit:
         return   # the reference's filter (test_marlin_gemm.py:205-212)
-    if is_a_8bit and quant_type.size_bits == 8:
-        pytest.skip("8-bit weights in the order of 8-bit activations are not built: no GEMM takes them "
-                    "(W8A8 is not a Marlin mode)")
     b_weight = rand_data((size_k, size_n))
     w_ref, q_w, s, g_idx, rand_perm = gptq_quantize_weights(b_weight, quant_type, group_size, act_order)
     q_w_gptq = gptq_pack(q_w, quant_type.size_bits, size_k, size_n)

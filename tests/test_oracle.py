@@ -738,3 +738,21 @@ def test_gemm_w4a8_limit_cases():
     s = rng.uniform(0.5, 1, size=(2, 16)).astype(np.float32)
     w = (q - 8) * np.repeat(s, 32, axis=0)
     assert np.allclose(mo.gemm_w4a8_fp8(af, np.ones((2, 1), np.float32), q, 32, s), af @ w, rtol=1e-6)
+
+
+def test_marlin8_a8_layout_two_derivations_agree():
+    rng = np.random.default_rng(21)
+    q = rng.integers(0, 256, size=(96, 128), dtype=np.int32)
+    recipe, closed = mo.marlin_pack8_recipe_a8(q), mo.marlin_pack8_closed_form_a8(q)
+    assert recipe.shape == (6, 512) and np.array_equal(recipe, closed)
+    assert np.array_equal(mo.gptq_marlin_repack8_a8(mo.pack_rows8(q), 96, 128), closed)
+    assert not np.array_equal(closed, mo.marlin_pack8_closed_form(q))     # not the 16-bit order
+    # one code at (k, n): tile (k/32, n/32), lane 4*(n%8) + (k%16)/4, warp (n%32)/8, half (k%32)/16, byte k%4
+    for k, n in [(0, 0), (21, 13), (63, 127)]:
+        one = np.zeros((64, 128), dtype=np.int32)
+        one[k, n] = 255
+        w = mo.marlin_pack8_closed_form_a8(one).view(np.uint32).reshape(-1)
+        idx = np.nonzero(w)[0]
+        tile = (k // 32) * 4 + n // 32
+        assert idx.tolist() == [tile * 256 + (4 * (n % 8) + (k % 16) // 4) * 8 + 2 * ((n % 32) // 8) + (k % 32) // 16]
+        assert w[idx[0]] == 255 << (8 * (k % 4))
