@@ -224,7 +224,11 @@ int sonar_per_token_quant_fp8(const void* x, int dtype, int64_t row_stride, uint
  *        round((float(sum_k a (q - z)) * a_scales[m]) * s[n] + bias).
  * fp8:   the same with fp32 sums and the weights (q - z) * 2^-9.
  * num_groups 1 (channelwise) or size_k / 32, / 64, / 128; size_k % 32 == 0, size_n % 64 == 0; no
- * act-order (the reference builds no such kernel).  b_type_id uint4b8 or uint4. */
+ * act-order (the reference builds no such kernel).  b_type_id uint4b8 or uint4, or float4_e2m1f
+ * with float8_e4m3fn activations (MXFP4 weights, "W4A8-FP4", dequant.h:474-490, marlin.cu:576-590):
+ * b_scales then are exponent bytes [K/32][N] in the same order, each 6 above the checkpoint's
+ * (mxfp4_marlin_process_scales with an fp8 input type), no zero points, and
+ * C = round((sum_g 2^(e[g][n] - 127 - 6) * sum_{k in g} a[m][k] * value(code[k][n])) * a_scales[m] + bias). */
 size_t sonar_marlin_gemm_a8_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k,
                                           int64_t num_groups);
 int sonar_marlin_gemm_a8(const void* a, int64_t a_row_stride, int a_dtype, void* c,

@@ -64,7 +64,10 @@ reference checkout).  How each function is pinned (none is "parity unpinned"):
                            the textbook dequantised matmul as the limit case
                            (all group scales equal); per_token_quant_int8
                            against hand values and the round trip bound
-                           |x - q*s| <= s/2
+                           |x - q*s| <= s/2; MXFP4 with fp8 activations: the
+                           byte a code becomes (dequant.h:474-490) decoded as
+                           float8_e4m3fn equals 2^-6 times the code's value for
+                           all 16 codes, which the scale bytes' + 6 undoes
 * NVFP4 weights            the scale bytes (nvfp4_process_scales) decoded by both
                            of the kernel's readings (dequant.h:520-549: b << 7
                            as fp16, and sign / exponent / mantissa moved into a
@@ -801,6 +804,47 @@ def dequantize_mxfp4(codes: np.ndarray, exponent_bytes: np.ndarray, dtype: str =
     k, n = codes.shape
     rows = np.arange(k) // 32
     return round_to_dtype(fp4_e2m1_values()[codes] * mx_scale_values(exponent_bytes)[rows, :], dtype)
+
+
+def mxfp4_process_scales_a8(permuted_bytes: np.ndarray) -> np.ndarray:
+    """marlin_utils_fp4.py:125-135 for float8_e4m3fn activations: no reorder
+    inside the fours, every exponent byte plus 6 (the kernel holds a code as a
+    float8_e4m3fn byte worth 2^-6 times the float4_e2m1f value: exponent bias
+    7 against 1).  Bytes above 249 are refused, as the reference's assert does."""
+    b = np.asarray(permuted_bytes).astype(np.int32)
+    assert b.max() <= 249
+    return (b + 6).astype(np.uint8)
+
+
+def fp4_code_as_fp8_byte(code: np.ndarray) -> np.ndarray:
+    """dequant.h:474-490: sign to bit 7, the two exponent bits and the mantissa
+    bit to bits 4..2 of a float8_e4m3fn byte."""
+    c = np.asarray(code).astype(np.uint8)
+    return (((c & 8) << 4) | ((c & 7) << 2)).astype(np.uint8)
+
+
+def fp8_e4m3fn_value(byte: np.ndarray) -> np.ndarray:
+    """float8_e4m3fn: sign, 4 exponent bits (bias 7), 3 mantissa bits,
+    subnormals at exponent 0 (NaN at 0x7f / 0xff not used here)."""
+    b = np.asarray(byte).astype(np.int32)
+    e, m = (b >> 3) & 15, b & 7
+    mag = np.where(e == 0, m / 8.0 * 2.0 ** -6, (1 + m / 8.0) * 2.0 ** (e - 7.0))
+    return np.where(b & 0x80, -mag, mag).astype(np.float32)
+
+
+def gemm_w4a8_fp4(a_fp8_32: np.ndarray, a_scales: np.ndarray, codes: np.ndarray, exponent_bytes: np.ndarray,
+                  bias32: np.ndarray | None = None) -> np.ndarray:
+    """MXFP4 weights with float8_e4m3fn activations: out = (a @ w) * a_scales
+    (+ bias) with w[k][n] = value(code) * 2^(e[k // 32][n] - 127), in float64
+    (a floating-point kernel, compared within a tolerance).  `exponent_bytes`
+    are the checkpoint's, before mxfp4_process_scales_a8."""
+    m, k = a_fp8_32.shape
+    w = fp4_e2m1_values()[codes].astype(np.float64) * np.repeat(
+        mx_scale_values(exponent_bytes).astype(np.float64), 32, axis=0)
+    out = (a_fp8_32.astype(np.float64) @ w) * a_scales.reshape(m, 1).astype(np.float64)
+    if bias32 is not None:
+        out = out + bias32.astype(np.float64)[None, :]
+    return out.astype(np.float32)
 
 
 # --------------------------------------------------------------------------

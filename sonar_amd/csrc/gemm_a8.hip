@@ -66,6 +66,7 @@ struct ActInt8 {
   typedef intx4_t acc_t;
   typedef int scalar_t;
   static constexpr bool kInteger = true;
+  static constexpr bool kE8Scales = false;
   static __device__ __forceinline__ acc_t mfma(long a, long b, acc_t c) {
     return __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, c, 0, 0, 0);
   }
@@ -99,6 +100,7 @@ struct ActFp8 {
   typedef floatx4_t acc_t;
   typedef float scalar_t;
   static constexpr bool kInteger = false;
+  static constexpr bool kE8Scales = false;
   static __device__ __forceinline__ acc_t mfma(long a, long b, acc_t c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_fp8_fp8(a, b, c, 0, 0, 0);
   }
@@ -133,6 +135,29 @@ struct ActFp8 {
   static __device__ __forceinline__ int unit_offset(int c, int kb) { return kb * 32 + c * 8; }
 };
 
+// float4_e2m1f codes with fp8 activations (MXFP4 weights, "W4A8-FP4": dequant.h:474-490): sign,
+// two exponent bits and the mantissa bit moved into a float8_e4m3fn byte read 2^-6 times the fp4
+// value (the zero exponent field gives the subnormal 0.5); the exponent-byte scales carry the 6
+// (mxfp4_marlin_process_scales, marlin_utils_fp4.py:129-135).  Groups of 32 rows, no zero points.
+struct ActFp8F4 : ActFp8 {
+  static constexpr bool kE8Scales = true;
+  static __device__ __forceinline__ uint32_t four_f4(uint32_t x) {   // nibbles in the high halves of x's bytes
+    return (x & 0x80808080u) | ((x & 0x70707070u) >> 2);
+  }
+  static __device__ __forceinline__ long word(uint32_t w) {
+    return (long)(((uint64_t)four_f4(w) << 32) | four_f4(w << 4));
+  }
+  static __device__ __forceinline__ long word_zp(uint32_t w, uint32_t) { return word(w); }
+};
+// Scale of a group as the kernel multiplies it: 16-bit integer, number of the output type, or (E8)
+// an exponent byte 2^(b - 127).
+template <typename ACT, typename T, bool E8>
+__device__ __forceinline__ typename ACT::scalar_t group_scale(const void* scales, long index) {
+  if constexpr (E8) return __uint_as_float((uint32_t)static_cast<const uint8_t*>(scales)[index] << 23);
+  else if constexpr (ACT::kInteger) return (int)static_cast<const uint16_t*>(scales)[index];   // read as unsigned
+  else return from_bits<T>(static_cast<const uint16_t*>(scales)[index]);
+}
+
 // Raw total -> output value: the activation row's scale, for channelwise
 // weights the column's scale, the bias, one rounding.
 template <typename ACT, typename T, bool GROUPED>
@@ -151,9 +176,9 @@ __device__ __forceinline__ uint16_t finish(typename ACT::scalar_t total, float a
 // [u_begin, u_end).  a_row[rb]: this lane's row of A in row block rb, already offset by the
 // lane's 8 bytes inside a chunk; w_lane: the lane's 16 bytes of chunk 0 of the strip;
 // scales / zeros: row 0 of the matrix's (the expert's) scales and zero points.
-template <typename ACT, typename T, int MB, bool HAS_ZP, bool GROUPED, int WAVES = 4>
+template <typename ACT, typename T, int MB, bool HAS_ZP, bool GROUPED, int WAVES = 4, bool E8 = false>
 __device__ __forceinline__ void a8_accumulate(typename ACT::acc_t (&acc)[MB][4], const uint8_t* const (&a_row)[MB],
-                                              const uint32_t* w_lane, const uint16_t* scales,
+                                              const uint32_t* w_lane, const void* scales,
                                               const uint32_t* zeros, int n, int strip, int chunks, int unit_chunks,
                                               int u_begin, int u_end, int wave, int l16) {
   typedef typename ACT::acc_t acc_t;
@@ -197,11 +222,7 @@ __device__ __forceinline__ void a8_accumulate(typename ACT::acc_t (&acc)[MB][4],
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       scalar_t s = 1;
-      if (GROUPED) {
-        const uint16_t bits = scales[(long)g * n + s_col[j]];
-        if constexpr (ACT::kInteger) s = (int)bits;   // read as unsigned (marlin_template.h:1341-1348)
-        else s = from_bits<T>(bits);
-      }
+      if (GROUPED) s = group_scale<ACT, T, E8>(scales, (long)g * n + s_col[j]);   // marlin_template.h:1341-1382
 #pragma unroll
       for (int rb = 0; rb < MB; ++rb)
 #pragma unroll
@@ -284,8 +305,8 @@ __global__ __launch_bounds__(64 * A8Waves<MB>::value) void marlin_a8_kernel(A8Pa
   const uint32_t* w_lane = p.w + (long)strip * p.chunks * kChunkWords + lane * 4;
   const int u_begin = split * p.units_per_split;
   const int u_end = min(u_begin + p.units_per_split, p.units);
-  a8_accumulate<ACT, T, MB, HAS_ZP, GROUPED, WAVES>(acc, a_row, w_lane, p.scales, p.zeros, p.n, strip, p.chunks,
-                                                    p.unit_chunks, u_begin, u_end, wave, l16);
+  a8_accumulate<ACT, T, MB, HAS_ZP, GROUPED, WAVES, ACT::kE8Scales>(acc, a_row, w_lane, p.scales, p.zeros, p.n, strip,
+                                                                    p.chunks, p.unit_chunks, u_begin, u_end, wave, l16);
   scalar_t total[MB][4];
   a8_reduce<ACT, MB, WAVES>(acc, red, total, wave, lane);
   if (wave >= 4) return;
@@ -365,10 +386,13 @@ __global__ __launch_bounds__(256) void marlin_moe_a8_kernel(MoeA8Params q) {
   }
   const long words_per_expert = (long)p.chunks * kChunkWords * (p.n / kStripN);
   const uint32_t* w_lane = p.w + expert * words_per_expert + (long)strip * p.chunks * kChunkWords + lane * 4;
-  const uint16_t* scales = p.scales + (long)expert * q.groups * p.n;
+  const long scale_offset = (long)expert * q.groups * p.n;   // exponent-byte scales: one byte each
+  const uint16_t* scales = ACT::kE8Scales ? reinterpret_cast<const uint16_t*>(
+                                                reinterpret_cast<const uint8_t*>(p.scales) + scale_offset)
+                                          : p.scales + scale_offset;
   const uint32_t* zeros = HAS_ZP ? p.zeros + (long)expert * q.groups * (p.n / 8) : nullptr;
-  a8_accumulate<ACT, T, MB, HAS_ZP, GROUPED>(acc, a_row, w_lane, scales, zeros, p.n, strip, p.chunks,
-                                             p.unit_chunks, 0, p.units, wave, l16);
+  a8_accumulate<ACT, T, MB, HAS_ZP, GROUPED, 4, ACT::kE8Scales>(acc, a_row, w_lane, scales, zeros, p.n, strip,
+                                                                p.chunks, p.unit_chunks, 0, p.units, wave, l16);
   scalar_t total[MB][4];
   a8_reduce<ACT, MB>(acc, red, total, wave, lane);
 
@@ -740,7 +764,7 @@ void launch_a8_tile_gc(const MoeA8Params& q, int gc, dim3 grid, hipStream_t st) 
 template <typename ACT, typename T>
 void launch_a8(const A8Params& p, const A8Plan& plan, bool grouped, hipStream_t st) {
   const bool zp = p.zeros != nullptr;
-  if (plan.tile) {
+  if constexpr (!ACT::kE8Scales) if (plan.tile) {
     const dim3 grid(p.n / kA8TileN, plan.slabs, plan.splits);
     MoeA8Params q = {};
     q.g = p;
@@ -791,7 +815,7 @@ void launch_moe_a8(const MoeA8Params& q, bool grouped, int blocks, hipStream_t s
   const bool zp = q.g.zeros != nullptr;
   // blocks of more than 32 slots on shapes the tiled kernel takes (groups of 64 rows or more)
   const int gc = grouped ? q.g.unit_chunks : 0;
-  if (q.block_size > 32 && q.g.n % 256 == 0 && q.g.chunks % kA8StepChunks == 0 && gc != 1 &&
+  if constexpr (!ACT::kE8Scales) if (q.block_size > 32 && q.g.n % 256 == 0 && q.g.chunks % kA8StepChunks == 0 && gc != 1 &&
       (grouped || q.g.chunks <= 2048)) {
     MoeA8Params t = q;
     t.g.units = q.g.chunks / kA8StepChunks;
@@ -816,9 +840,17 @@ int check_a8(int a_dtype, int dtype, int b_layout, int64_t b_type_id, int64_t si
   SONAR_REQUIRE(b_layout == SONAR_LAYOUT_GFX950, "unknown b_layout = %d", b_layout);
   SONAR_REQUIRE(a_dtype == SONAR_ADTYPE_INT8 || a_dtype == SONAR_ADTYPE_FP8, "unknown a_dtype = %d", a_dtype);
   SONAR_REQUIRE(dtype == SONAR_DTYPE_F16 || dtype == SONAR_DTYPE_BF16, "unknown dtype = %d", dtype);
-  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4)
-    return fail(SONAR_E_UNSUPPORTED, "8-bit activations are built for b_type uint4b8 and uint4 only (W8A8 is not "
-                "supported by the marlin kernel; float4_e2m1f weights with fp8 activations are not built)");
+  const bool f4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F;
+  if (b_type_id != SONAR_TYPE_UINT4B8 && b_type_id != SONAR_TYPE_UINT4 && !f4)
+    return fail(SONAR_E_UNSUPPORTED, "8-bit activations are built for b_type uint4b8, uint4 and float4_e2m1f only "
+                "(W8A8 is not supported by the marlin kernel)");
+  if (f4) {
+    if (a_dtype != SONAR_ADTYPE_FP8) return fail(SONAR_E_UNSUPPORTED, "MXFP4 weight + INT8 activation is not supported.");
+    SONAR_REQUIRE(num_groups >= 1 && size_k == 32 * num_groups, "float4_e2m1f weights with 8-bit activations take "
+                  "one exponent-byte scale per 32 rows; got size_k = %ld, num_groups = %ld", (long)size_k,
+                  (long)num_groups);
+    SONAR_REQUIRE(b_zeros == nullptr, "float4_e2m1f weights have no zero points");
+  }
   SONAR_REQUIRE(size_m >= 0 && size_n > 0 && size_k > 0, "size_m = %ld, size_n = %ld, size_k = %ld", (long)size_m,
                 (long)size_n, (long)size_k);
   SONAR_REQUIRE(size_n % kStripN == 0, "size_n = %ld is not divisible by %d", (long)size_n, kStripN);
@@ -833,6 +865,11 @@ int check_a8(int a_dtype, int dtype, int b_layout, int64_t b_type_id, int64_t si
   SONAR_REQUIRE((b_zeros != nullptr) == (b_type_id == SONAR_TYPE_UINT4),
                 "b_zeros must be given for uint4 weights and only for them");
   return SONAR_OK;
+}
+
+// One 32-row group of float4 weights is a "grouped" call even when K = 32.
+bool a8_grouped(int64_t b_type_id, int64_t num_groups) {
+  return num_groups > 1 || b_type_id == SONAR_TYPE_FLOAT4_E2M1F;
 }
 
 }  // namespace
@@ -888,9 +925,12 @@ extern "C" int sonar_moe_wna16_marlin_gemm_a8(
   q.num_experts = (int)num_experts;
   q.groups = (int)num_groups;
   q.sorted_len = (int)sorted_len;
-  const bool grouped = num_groups > 1;
+  const bool grouped = a8_grouped(b_type_id, num_groups);
   hipStream_t st = (hipStream_t)stream;
-  if (a_dtype == SONAR_ADTYPE_INT8) {
+  if (b_type_id == SONAR_TYPE_FLOAT4_E2M1F) {
+    if (dtype == SONAR_DTYPE_F16) launch_moe_a8<ActFp8F4, _Float16>(q, grouped, (int)blocks, st);
+    else launch_moe_a8<ActFp8F4, __bf16>(q, grouped, (int)blocks, st);
+  } else if (a_dtype == SONAR_ADTYPE_INT8) {
     if (dtype == SONAR_DTYPE_F16) launch_moe_a8<ActInt8, _Float16>(q, grouped, (int)blocks, st);
     else launch_moe_a8<ActInt8, __bf16>(q, grouped, (int)blocks, st);
   } else {
@@ -941,9 +981,12 @@ extern "C" int sonar_marlin_gemm_a8(const void* a, int64_t a_row_stride, int a_d
     SONAR_REQUIRE(scratch && scratch_bytes >= (size_t)plan.splits * size_m * size_n * 4,
                   "scratch of %zu bytes is too small: sonar_marlin_gemm_a8_scratch_bytes() = %zu", scratch_bytes,
                   (size_t)plan.splits * size_m * size_n * 4);
-  const bool grouped = num_groups > 1;
+  const bool grouped = a8_grouped(b_type_id, num_groups);
   hipStream_t st = (hipStream_t)stream;
-  if (a_dtype == SONAR_ADTYPE_INT8) {
+  if (b_type_id == SONAR_TYPE_FLOAT4_E2M1F) {
+    if (dtype == SONAR_DTYPE_F16) launch_a8<ActFp8F4, _Float16>(p, plan, grouped, st);
+    else launch_a8<ActFp8F4, __bf16>(p, plan, grouped, st);
+  } else if (a_dtype == SONAR_ADTYPE_INT8) {
     if (dtype == SONAR_DTYPE_F16) launch_a8<ActInt8, _Float16>(p, plan, grouped, st);
     else launch_a8<ActInt8, __bf16>(p, plan, grouped, st);
   } else {

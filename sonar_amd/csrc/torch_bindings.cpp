@@ -440,18 +440,27 @@ Tensor marlin_gemm_a8(const Tensor& a, const OptTensor& c_or_none, const Tensor&
                       int64_t size_k, bool is_zp_float) {
   const int a_dtype = a.scalar_type() == at::kChar ? SONAR_ADTYPE_INT8 : SONAR_ADTYPE_FP8;
   check_b_type(b_type_id);
-  TORCH_CHECK_NOT_IMPLEMENTED(b_type_id != SONAR_TYPE_FLOAT4_E2M1F,
-                              "float4_e2m1f weights with float8_e4m3fn activations (W4A8-FP4) are not built");
-  if (a_dtype == SONAR_ADTYPE_INT8) {   // marlin_utils.py:672-676
+  // MXFP4 weights with fp8 activations ("W4A8-FP4", marlin.cu:576-590): exponent-byte scales per 32
+  // rows, the output type is that of c, which must be passed
+  const bool f4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F;
+  if (f4) {
+    TORCH_CHECK(a_dtype == SONAR_ADTYPE_FP8, "MXFP4 weight + INT8 activation is not supported.");
+    TORCH_CHECK(is_mx_scale_type(b_scales), "float4_e2m1f weights with 8-bit activations take float8_e8m0fnu "
+                "scales (MXFP4); NVFP4 weight + INT8/FP8 activation is not supported.");
+    TORCH_CHECK(c_or_none.has_value(), "c must be passed for W4A8-FP4");
+    TORCH_CHECK(c_or_none->scalar_type() == at::kHalf || c_or_none->scalar_type() == at::kBFloat16,
+                "unsupported c dtype");
+  } else if (a_dtype == SONAR_ADTYPE_INT8) {   // marlin_utils.py:672-676
     TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4,
                 "W8A8-INT8 is not supported by marlin kernel.");
   } else {
     TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4,
                 "INT8 weight + FP8 activation is not supported.");
   }
-  TORCH_CHECK(b_scales.scalar_type() == at::kHalf || b_scales.scalar_type() == at::kBFloat16,
+  const at::ScalarType c_type = f4 ? c_or_none->scalar_type() : b_scales.scalar_type();
+  TORCH_CHECK(c_type == at::kHalf || c_type == at::kBFloat16,
               "b_scales must be float16 or bfloat16 with 8-bit activations (their type is the type of c)");
-  const int dtype = b_scales.scalar_type() == at::kHalf ? SONAR_DTYPE_F16 : SONAR_DTYPE_BF16;
+  const int dtype = c_type == at::kHalf ? SONAR_DTYPE_F16 : SONAR_DTYPE_BF16;
   TORCH_CHECK(a_scales.has_value() && a_scales->numel() > 0,
               "the a_scales parameter must be passed for 8bit activation.");
   TORCH_CHECK(a_scales->is_cuda() && a_scales->scalar_type() == at::kFloat, "scalar type of a_scales must be float");
@@ -492,7 +501,7 @@ Tensor marlin_gemm_a8(const Tensor& a, const OptTensor& c_or_none, const Tensor&
     TORCH_CHECK(c.is_contiguous(), "c is not contiguous");
     TORCH_CHECK(c.size(0) == size_m, "Shape mismatch: c.size(0) = ", c.size(0), ", size_m = ", size_m);
     TORCH_CHECK(c.size(1) == size_n, "Shape mismatch: c.size(1) = ", c.size(1), ", size_n = ", size_n);
-    TORCH_CHECK(c.scalar_type() == b_scales.scalar_type(), "c must have the type of b_scales with 8-bit activations");
+    TORCH_CHECK(c.scalar_type() == c_type, "c must have the type of b_scales with 8-bit activations");
   } else {
     c = at::empty({size_m, size_n}, b_scales.options());
   }
@@ -712,14 +721,21 @@ Tensor moe_wna16_marlin_gemm_a8(const Tensor& a, const OptTensor& c_or_none, con
                                 int64_t size_k, bool is_zp_float) {
   const int a_dtype = a.scalar_type() == at::kChar ? SONAR_ADTYPE_INT8 : SONAR_ADTYPE_FP8;
   check_b_type(b_type_id);
-  TORCH_CHECK_NOT_IMPLEMENTED(b_type_id != SONAR_TYPE_FLOAT4_E2M1F,
-                              "float4_e2m1f weights with float8_e4m3fn activations (W4A8-FP4) are not built");
-  TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4,
-              a_dtype == SONAR_ADTYPE_INT8 ? "W8A8-INT8 is not supported by marlin kernel."
-                                           : "INT8 weight + FP8 activation is not supported.");
-  TORCH_CHECK(b_scales.scalar_type() == at::kHalf || b_scales.scalar_type() == at::kBFloat16,
+  const bool f4 = b_type_id == SONAR_TYPE_FLOAT4_E2M1F;   // MXFP4 experts with fp8 tokens: c gives the output type
+  if (f4) {
+    TORCH_CHECK(a_dtype == SONAR_ADTYPE_FP8, "MXFP4 weight + INT8 activation is not supported.");
+    TORCH_CHECK(is_mx_scale_type(b_scales), "float4_e2m1f weights with 8-bit activations take float8_e8m0fnu "
+                "scales (MXFP4); NVFP4 weight + INT8/FP8 activation is not supported.");
+    TORCH_CHECK(c_or_none.has_value(), "c must be passed for W4A8-FP4");
+  } else {
+    TORCH_CHECK(b_type_id == SONAR_TYPE_UINT4B8 || b_type_id == SONAR_TYPE_UINT4,
+                a_dtype == SONAR_ADTYPE_INT8 ? "W8A8-INT8 is not supported by marlin kernel."
+                                             : "INT8 weight + FP8 activation is not supported.");
+  }
+  const at::ScalarType c_type = f4 ? c_or_none->scalar_type() : b_scales.scalar_type();
+  TORCH_CHECK(c_type == at::kHalf || c_type == at::kBFloat16,
               "b_scales must be float16 or bfloat16 with 8-bit activations (their type is the type of c)");
-  const int dtype = b_scales.scalar_type() == at::kHalf ? SONAR_DTYPE_F16 : SONAR_DTYPE_BF16;
+  const int dtype = c_type == at::kHalf ? SONAR_DTYPE_F16 : SONAR_DTYPE_BF16;
   TORCH_CHECK(a_scales.has_value() && a_scales->numel() > 0,
               "the a_scales parameter must be passed for 8bit activation.");
   TORCH_CHECK(a_scales->is_cuda() && a_scales->scalar_type() == at::kFloat && a_scales->is_contiguous(),
@@ -759,7 +775,7 @@ Tensor moe_wna16_marlin_gemm_a8(const Tensor& a, const OptTensor& c_or_none, con
     TORCH_CHECK(c.size(0) == size_m * top_k, "Shape mismatch: c.size(0) = ", c.size(0),
                 ", size_m * topk = ", size_m * top_k);
     TORCH_CHECK(c.size(1) == size_n, "Shape mismatch: c.size(1) = ", c.size(1), ", size_n = ", size_n);
-    TORCH_CHECK(c.scalar_type() == b_scales.scalar_type(), "c must have the type of b_scales with 8-bit activations");
+    TORCH_CHECK(c.scalar_type() == c_type, "c must have the type of b_scales with 8-bit activations");
   } else {
     c = at::empty({size_m * top_k, size_n}, b_scales.options());
   }

@@ -16,9 +16,10 @@ from __future__ import annotations
 import torch
 
 from . import ops
-from .marlin_utils import (USE_FP32_REDUCE_DEFAULT, marlin_make_workspace_new, marlin_pad_dim, marlin_pad_qweight,
-                           marlin_pad_scales, marlin_padded_nk, marlin_permute_bias, marlin_permute_scales,
-                           marlin_repacked_nk, marlin_unpad_output, should_use_atomic_add_reduce)
+from .marlin_utils import (USE_FP32_REDUCE_DEFAULT, get_marlin_input_dtype, marlin_make_workspace_new,
+                           marlin_pad_dim, marlin_pad_qweight, marlin_pad_scales, marlin_padded_nk,
+                           marlin_permute_bias, marlin_permute_scales, marlin_quant_input, marlin_repacked_nk,
+                           marlin_unpad_output, should_use_atomic_add_reduce)
 from .scalar_type import scalar_types
 
 MXFP4_GROUP_SIZE = 32
@@ -31,12 +32,17 @@ def is_fp4_marlin_supported() -> bool:
 
 
 def mxfp4_marlin_process_scales(marlin_scales: torch.Tensor, input_dtype: torch.dtype | None = None) -> torch.Tensor:
-    """marlin_utils_fp4.py:123-135 for 16-bit activations: (0, 2, 1, 3) inside
-    every four, then the exponent bytes."""
-    if input_dtype is not None and input_dtype.itemsize == 1:
-        raise NotImplementedError("8-bit activations are not built")
-    reordered = marlin_scales.view(-1, 4)[:, [0, 2, 1, 3]].view(marlin_scales.size(0), -1)
-    return reordered.to(torch.float8_e8m0fnu)
+    """marlin_utils_fp4.py:123-135: for 16-bit activations (0, 2, 1, 3) inside every four, then
+    the exponent bytes; for float8_e4m3fn activations the bytes in place, plus 6 (the fp4 codes
+    enter the fp8 matrix instruction as value * 2^-6)."""
+    if input_dtype is None or input_dtype.itemsize == 2:
+        marlin_scales = marlin_scales.view(-1, 4)[:, [0, 2, 1, 3]].view(marlin_scales.size(0), -1)
+    marlin_scales = marlin_scales.to(torch.float8_e8m0fnu)
+    if input_dtype == torch.float8_e4m3fn:
+        as_bytes = marlin_scales.view(torch.uint8)
+        assert as_bytes.max() <= 249
+        marlin_scales = (as_bytes + 6).view(torch.float8_e8m0fnu)   # exponent bias fp4 -> fp8: 2^3 - 2^1
+    return marlin_scales
 
 
 def _nvfp4_compute_scale_factor(marlin_scales: torch.Tensor, a_dtype: torch.dtype | None = None) -> float:
@@ -89,17 +95,23 @@ def apply_fp4_marlin_linear(input: torch.Tensor, weight: torch.Tensor, weight_sc
                             size_k: int, bias: torch.Tensor | None = None, input_dtype: torch.dtype | None = None,
                             use_fp32_reduce: bool = USE_FP32_REDUCE_DEFAULT) -> torch.Tensor:
     """marlin_utils_fp4.py:153-214; with a global scale the weights are NVFP4."""
-    if input_dtype is not None and input_dtype.itemsize == 1:
-        if weight_global_scale is not None:
-            raise RuntimeError("NVFP4 weight + INT8/FP8 activation is not supported.")
-        raise NotImplementedError("8-bit activations are not built")
     x = input.reshape(-1, input.shape[-1])
     out_shape = input.shape[:-1] + (size_n,)
     padded_n, padded_k = marlin_repacked_nk(weight, num_bits=4)
     x = marlin_pad_dim(x, size_k, padded_k)
     use_atomic_add = should_use_atomic_add_reduce(m=x.size(0), n=padded_n, k=padded_k, device=input.device,
                                                   dtype=input.dtype)
-    out = ops.marlin_gemm(a=x, c=None, b_q_weight=weight, b_bias=bias, b_scales=weight_scale, a_scales=None,
+    a_scales, c = None, None
+    if input_dtype is not None and input_dtype.itemsize == 1:   # marlin_utils_fp4.py:185-191
+        if weight_global_scale is not None:
+            raise RuntimeError("NVFP4 weight + INT8/FP8 activation is not supported.")
+        if input_dtype != torch.float8_e4m3fn:
+            raise RuntimeError("MXFP4 weight + INT8 activation is not supported.")
+        # the op takes the output type from c in this mode (marlin.cu:576-590); the reference passes
+        # c = None here, which its op refuses
+        c = torch.empty((x.size(0), padded_n), dtype=input.dtype, device=input.device)
+        x, a_scales = marlin_quant_input(x, torch.float8_e4m3fn)
+    out = ops.marlin_gemm(a=x, c=c, b_q_weight=weight, b_bias=bias, b_scales=weight_scale, a_scales=a_scales,
                           global_scale=weight_global_scale, b_zeros=None, g_idx=None, perm=None,
                           workspace=workspace,
                           b_q_type=scalar_types.float4_e2m1f, size_m=x.size(0), size_n=padded_n, size_k=padded_k,
@@ -119,10 +131,12 @@ def prepare_fp4_layer_for_marlin(layer, input_dtype: torch.dtype | None = None) 
     (MXFP4, bfloat16) or `weight_scale` (N, K/16) float8_e4m3fn with
     `weight_global_scale` (NVFP4)."""
     is_nvfp4 = hasattr(layer, "weight_global_scale")
-    if input_dtype is not None and input_dtype.itemsize == 1:
+    is_a_8bit = input_dtype is not None and input_dtype.itemsize == 1
+    if is_a_8bit:
         if is_nvfp4:
             raise RuntimeError("NVFP4 weight + INT8/FP8 activation is not supported.")
-        raise NotImplementedError("8-bit activations are not built")
+        if input_dtype != torch.float8_e4m3fn:
+            raise RuntimeError("MXFP4 weight + INT8 activation is not supported.")
     group_size = 16 if is_nvfp4 else MXFP4_GROUP_SIZE
     part_n, part_k = layer.output_size_per_partition, layer.input_size_per_partition
     padded_n, padded_k = marlin_padded_nk(part_n, part_k, group_size)
@@ -132,21 +146,21 @@ def prepare_fp4_layer_for_marlin(layer, input_dtype: torch.dtype | None = None) 
     layer.workspace = marlin_make_workspace_new(device)
     perm = torch.empty(0, dtype=torch.int, device=device)
     qweight = marlin_pad_qweight(layer.weight.view(torch.int32).T.contiguous(), part_n, part_k, padded_n, padded_k)
-    _set(layer, "weight", ops.gptq_marlin_repack(qweight, perm, padded_k, padded_n, 4))
+    _set(layer, "weight", ops.gptq_marlin_repack(qweight, perm, padded_k, padded_n, 4, is_a_8bit))
 
     scales = layer.weight_scale.T.contiguous()
     if not is_nvfp4:
         scales = scales.view(torch.float8_e8m0fnu)
     scales = scales.to(param_dtype)
     scales = marlin_pad_scales(scales, part_n, part_k, padded_n, padded_k, group_size)
-    scales = marlin_permute_scales(scales, padded_k, padded_n, group_size)
+    scales = marlin_permute_scales(scales, padded_k, padded_n, group_size, is_a_8bit=is_a_8bit)
     if is_nvfp4:
         scales, scale_factor = nvfp4_marlin_process_scales(scales, a_dtype=param_dtype)
         _set(layer, "weight_scale", scales)
         global_scale = nvfp4_marlin_process_global_scale(layer.weight_global_scale.to(torch.float32), param_dtype)
         _set(layer, "weight_global_scale", global_scale / scale_factor)
     else:
-        _set(layer, "weight_scale", mxfp4_marlin_process_scales(scales))
+        _set(layer, "weight_scale", mxfp4_marlin_process_scales(scales, input_dtype=input_dtype))
 
     if getattr(layer, "bias", None) is not None:
         assert layer.bias.shape == (part_n,)
@@ -159,19 +173,25 @@ def prepare_moe_mxfp4_layer_for_marlin(layer, w13: torch.Tensor, w2: torch.Tenso
     """marlin_utils_fp4.py:556-649.  w13 (E, 2N, K/2), w2 (E, K, N/2) uint8; scales
     (E, 2N, K/32), (E, K, N/32) exponent bytes; `layer.params_dtype` is the
     activation type.  Returns (w13, w2, w13_scale, w2_scale, w13_bias, w2_bias)
-    for fused_marlin_moe; nothing on the layer changes."""
+    for fused_marlin_moe; nothing on the layer changes.  The activation type of the GEMM comes from
+    get_marlin_input_dtype(): float8_e4m3fn gives the 8-bit-activation layouts."""
+    input_dtype = get_marlin_input_dtype()
+    if input_dtype is not None and input_dtype.itemsize == 1 and input_dtype != torch.float8_e4m3fn:
+        raise RuntimeError("MXFP4 weight + INT8 activation is not supported.")
+    is_a_8bit = input_dtype is not None and input_dtype.itemsize == 1
     e, n, k = w13.shape[0], w13.shape[1] // 2, w13.shape[2] * 2
     perm = torch.empty(0, dtype=torch.int, device=w13.device)
 
     def repack(weight: torch.Tensor, size_n: int, size_k: int) -> torch.Tensor:
         assert weight.shape == (e, size_n, size_k // 2)
-        return torch.stack([ops.gptq_marlin_repack(weight[i].view(torch.int32).T.contiguous(), perm, size_k, size_n, 4)
-                            for i in range(e)])
+        return torch.stack([ops.gptq_marlin_repack(weight[i].view(torch.int32).T.contiguous(), perm, size_k, size_n, 4,
+                                                   is_a_8bit) for i in range(e)])
 
     def permute(scales: torch.Tensor, size_n: int, size_k: int) -> torch.Tensor:
         scales = scales.view(torch.float8_e8m0fnu).to(layer.params_dtype)
         return torch.stack([mxfp4_marlin_process_scales(
-            marlin_permute_scales(scales[i].T, size_k, size_n, MXFP4_GROUP_SIZE)) for i in range(e)])
+            marlin_permute_scales(scales[i].T, size_k, size_n, MXFP4_GROUP_SIZE, is_a_8bit=is_a_8bit),
+            input_dtype=input_dtype) for i in range(e)])
 
     def permute_bias(bias: torch.Tensor | None) -> torch.Tensor | None:
         if bias is None:
@@ -247,7 +267,9 @@ def rand_marlin_weight_mxfp4_like(weight: torch.Tensor, group_size: int, input_d
     """The reference's test helper (marlin_utils_fp4.py:701-753): random codes of
     the shape of `weight` (N, K) and random exponents 110..119; returns
     (dequantised reference (K, N), Marlin weight, Marlin scales)."""
-    assert input_dtype is None or input_dtype.itemsize != 1, "8-bit activations are not built"
+    is_a_8bit = input_dtype is not None and input_dtype.itemsize == 1
+    if is_a_8bit:
+        assert input_dtype == torch.float8_e4m3fn, "MXFP4 weight + INT8 activation is not supported."
     assert group_size > 0
     size_n, size_k = weight.shape
     device = weight.device
@@ -264,9 +286,11 @@ def rand_marlin_weight_mxfp4_like(weight: torch.Tensor, group_size: int, input_d
     weight_ref = torch.cat([even.unsqueeze(2), odd.unsqueeze(2)], 2).view(size_n, size_k)
     weight_ref = weight_ref * scales.repeat_interleave(group_size, 1).to(weight.dtype)
     perm = torch.empty(0, dtype=torch.int, device=device)
-    marlin_qweight = ops.gptq_marlin_repack(codes.view(torch.int32).T.contiguous(), perm, size_k, size_n, 4)
-    marlin_scales = marlin_permute_scales(scales.T.to(weight.dtype), size_k, size_n, group_size)
-    return weight_ref.T, marlin_qweight, mxfp4_marlin_process_scales(marlin_scales)
+    marlin_qweight = ops.gptq_marlin_repack(codes.view(torch.int32).T.contiguous(), perm, size_k, size_n, 4,
+                                            is_a_8bit)
+    marlin_scales = marlin_permute_scales(scales.T.to(weight.dtype), size_k, size_n, group_size,
+                                          is_a_8bit=is_a_8bit)
+    return weight_ref.T, marlin_qweight, mxfp4_marlin_process_scales(marlin_scales, input_dtype=input_dtype)
 
 
 def rand_marlin_weight_nvfp4_like(weight: torch.Tensor, group_size: int, input_dtype: torch.dtype | None = None):

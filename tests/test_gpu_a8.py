@@ -207,6 +207,61 @@ def test_w4a8_fp8_gemm_within_tolerance(k, n, group, zp, dtype, bias, ms):
         assert ok, (m, max_err, max_ref)
 
 
+FP4_CASES = [
+    # k, n, dtype, bias, M list
+    (256, 128, "bf16", False, [1, 16]),
+    (512, 192, "fp16", True, [7, 33]),
+    (1024, 256, "bf16", True, [64, 100]),
+    (8192, 64, "bf16", False, [3]),
+    (1024, 256, "fp16", False, [257]),
+]
+
+
+@pytest.mark.parametrize("k,n,dtype,bias,ms", FP4_CASES)
+def test_w4a8_fp4_gemm_within_tolerance(k, n, dtype, bias, ms):
+    """MXFP4 weights (float4_e2m1f codes, an exponent byte per column and 32 rows) with
+    float8_e4m3fn activations."""
+    lib = _lib.load()
+    rng = np.random.default_rng(k + n)
+    codes = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    e8 = rng.integers(110, 125, size=(k // 32, n)).astype(np.uint8)
+    native = _a8_to_gfx950(_repack_a8(dev_i32(mo.gptq_pack(codes)), k, n), k, n)
+    dev_s = torch.from_numpy(mo.mxfp4_process_scales_a8(mo.marlin_permute_scales_a8(e8, k, n, 32))).to(DEV)
+    bias32 = dev_bias = None
+    if bias:
+        bias32 = mo.round_to_dtype((rng.standard_normal(n) * 1e-3).astype(np.float32), dtype)
+        dev_bias = dev_bits16(mo.marlin_permute_bias(bias32), dtype)
+    tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+    for m in ms:
+        g = torch.Generator().manual_seed(m)
+        x = torch.randn((m, k), generator=g)
+        a_s = (x.abs().amax(dim=1, keepdim=True) / 448.0).clamp_min(1e-10)
+        a_fp8 = (x / a_s).to(torch.float8_e4m3fn)
+        a_dev, s_dev = a_fp8.view(torch.uint8).to(DEV), a_s.reshape(-1).to(DEV)
+        c = torch.full((m, n), float("nan"), dtype=tdt, device=DEV)
+        nbytes = lib.sonar_marlin_gemm_a8_scratch_bytes(m, n, k, k // 32)
+        scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=DEV)
+        _lib.check(lib.sonar_marlin_gemm_a8(
+            ptr(a_dev), k, _lib.ADTYPE_FP8, ptr(c), ptr(native), _lib.LAYOUT_GFX950, ptr(dev_bias), ptr(dev_s),
+            ptr(s_dev), None, ptr(scratch), scratch.numel(), dtype_code(dtype), _lib.TYPE_FLOAT4_E2M1F, m, n, k,
+            k // 32, stream()))
+        want = mo.gemm_w4a8_fp4(a_fp8.float().numpy(), a_s.numpy(), codes, e8, bias32)
+        ok, max_err, max_ref = mo.gemm_tolerance_ok(host_f32(c), want)
+        assert ok, (m, max_err, max_ref)
+    # int8 activations, zero points and groups other than 32 rows are refused
+    a = torch.zeros((4, k), dtype=torch.int8, device=DEV)
+    c = torch.empty((4, n), dtype=tdt, device=DEV)
+
+    def call(adt=_lib.ADTYPE_FP8, zeros=None, groups=k // 32):
+        return lib.sonar_marlin_gemm_a8(ptr(a), k, adt, ptr(c), ptr(native), _lib.LAYOUT_GFX950, None, ptr(dev_s),
+                                        ptr(s_dev), ptr(zeros), None, 0, dtype_code(dtype), _lib.TYPE_FLOAT4_E2M1F,
+                                        4, n, k, groups, stream())
+
+    assert call(adt=_lib.ADTYPE_INT8) == _lib.E_UNSUPPORTED
+    assert call(zeros=dev_s) == _lib.E_INVALID
+    assert call(groups=k // 64) == _lib.E_INVALID
+
+
 def test_w4a8_rejections():
     lib = _lib.load()
     layer = A8Layer(1, 256, 64, 64, "fp16", False, "int8")

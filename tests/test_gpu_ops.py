@@ -813,6 +813,52 @@ def test_prepare_mxfp4_layer_and_apply(k, n):
     assert ok, worst
 
 
+@pytest.mark.parametrize("k,n", [(512, 384), (384, 320)])
+def test_prepare_mxfp4_layer_and_apply_with_fp8_activations(k, n):
+    """The same checkpoint layer prepared for float8_e4m3fn activations (the weight order and the scale
+    order of 8-bit activations, exponent bytes plus 6): apply_fp4_marlin_linear quantises the input
+    per row; against the oracle's product on the quantised-then-dequantised input."""
+    from sonar_amd import marlin_utils as mu
+    from sonar_amd import marlin_utils_fp4 as f4
+    rng = np.random.default_rng(k + n)
+    codes = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+    e = rng.integers(108, 122, size=(k // 32, n)).astype(np.uint8)
+    by_n = codes.T
+    packed = np.ascontiguousarray((by_n[:, 0::2] | (by_n[:, 1::2] << 4)).astype(np.uint8))
+    layer = types.SimpleNamespace(output_size_per_partition=n, input_size_per_partition=k,
+                                  params_dtype=torch.bfloat16)
+    layer.weight = torch.from_numpy(packed).to(gu.DEV)
+    layer.weight_scale = torch.from_numpy(np.ascontiguousarray(e.T)).to(gu.DEV)
+    bias32 = mo.round_to_dtype(1e-2 * rng.standard_normal(n).astype(np.float32), "bf16")
+    layer.bias = gu.dev_bits16(bias32, "bf16")
+    with pytest.raises(RuntimeError, match="MXFP4 weight \\+ INT8 activation is not supported."):
+        f4.prepare_fp4_layer_for_marlin(layer, input_dtype=torch.int8)
+    f4.prepare_fp4_layer_for_marlin(layer, input_dtype=torch.float8_e4m3fn)
+    assert layer.weight_scale.dtype == torch.float8_e8m0fnu
+    x32 = mo.make_activations(4, 6, k, "bf16", std=0.5)
+    x = gu.dev_bits16(x32, "bf16")
+    y = f4.apply_fp4_marlin_linear(x.view(2, 3, k), layer.weight, layer.weight_scale, None, layer.workspace, n, k,
+                                   layer.bias, input_dtype=torch.float8_e4m3fn)
+    torch.cuda.synchronize()
+    assert y.shape == (2, 3, n) and y.dtype == torch.bfloat16
+    a_q, a_s = mu.per_token_quant_fp8(x)
+    want = mo.gemm_w4a8_fp4(a_q.float().cpu().numpy(), a_s.cpu().numpy(), codes, e, bias32)
+    ok, *worst = mo.gemm_tolerance_ok(gu.host_f32(y.view(6, n)), want)
+    assert ok, worst
+    with pytest.raises(RuntimeError, match="MXFP4 weight \\+ INT8 activation is not supported."):
+        f4.apply_fp4_marlin_linear(x, layer.weight, layer.weight_scale, None, layer.workspace, n, k,
+                                   input_dtype=torch.int8)
+    with pytest.raises(RuntimeError, match="NVFP4 weight \\+ INT8/FP8 activation is not supported."):
+        f4.apply_fp4_marlin_linear(x, layer.weight, layer.weight_scale, torch.ones(1, device=gu.DEV),
+                                   layer.workspace, n, k, input_dtype=torch.float8_e4m3fn)
+    # the op itself: c names the output type in this mode
+    from sonar_amd import ops
+    from sonar_amd.scalar_type import scalar_types as st
+    with pytest.raises(RuntimeError, match="c must be passed for W4A8-FP4"):
+        ops.marlin_gemm(a_q, None, layer.weight, None, layer.weight_scale, a_s, None, None, None, None,
+                        layer.workspace, st.float4_e2m1f, 6, layer.weight.size(1) // 2, k)
+
+
 # ---------------------------------------------------------------- NVFP4 weights (float4_e2m1f, e4m3 block scales, global scale)
 @pytest.mark.parametrize("dtype", [torch.float16, torch.bfloat16])
 @pytest.mark.parametrize("m,k,n", [(1, 512, 256), (33, 1024, 320), (16, 2880, 5760), (200, 256, 512), (700, 1024, 768)])

@@ -37,6 +37,8 @@ DENSE_CONFIGS = [
     {"a_quant": torch.int8, "b_type": scalar_types.uint4b8, "group_blocks": [-1, 2, 4, 8]},       # GPTQ int4, int8 A
     {"a_quant": torch.float8_e4m3fn, "b_type": scalar_types.uint4b8, "group_blocks": [-1, 2, 4, 8]},  # fp8 A
     {"a_quant": torch.float8_e4m3fn, "b_type": scalar_types.uint4, "group_blocks": [-1, 2, 4, 8]},
+    {"a_quant": torch.float8_e4m3fn, "b_type": scalar_types.float4_e2m1f, "a_type": [torch.bfloat16],
+     "group_blocks": [2]},                                                                      # MXFP4, fp8 A
 ]
 
 
@@ -138,7 +140,7 @@ def test_marlin_gemm(a_quant, b_type, dtype, group_size, size_m, size_n, size_k,
         w_ref, marlin_q_w, marlin_s = marlin_quant_fp8_torch(b_weight.T.contiguous(), group_size)
         g_idx = sort_indices = marlin_zp = None
     elif b_type == scalar_types.float4_e2m1f:
-        w_ref, marlin_q_w, marlin_s = rand_marlin_weight_mxfp4_like(b_weight.T, group_size)
+        w_ref, marlin_q_w, marlin_s = rand_marlin_weight_mxfp4_like(b_weight.T, group_size, input_dtype=a_quant)
         g_idx = sort_indices = marlin_zp = None
     else:
         w_ref, marlin_q_w, marlin_s, g_idx, sort_indices, _ = marlin_quantize(b_weight, b_type, group_size, act_order,
@@ -201,6 +203,8 @@ MOE_CONFIGS = [
     {"a_quant": torch.int8, "b_type": scalar_types.uint4b8, "group_blocks": [-1, 2, 4, 8]},
     {"a_quant": torch.float8_e4m3fn, "b_type": scalar_types.uint4b8, "group_blocks": [-1, 2, 4, 8]},
     {"a_quant": torch.float8_e4m3fn, "b_type": scalar_types.uint4, "group_blocks": [-1, 2, 4, 8]},
+    {"a_quant": torch.float8_e4m3fn, "b_type": scalar_types.float4_e2m1f, "a_type": torch.bfloat16,
+     "group_blocks": [2]},
 ]
 MARLIN_MOE_SCENARIOS = [
     # (m, n, k, e, topk, ep_size, act_order, is_k_full)
@@ -252,7 +256,7 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None, input_d
         elif quant_type == scalar_types.float8_e4m3fn:
             w_ref, qweight, scales = marlin_quant_fp8_torch(w[i].contiguous(), group_size)
         elif quant_type == scalar_types.float4_e2m1f:
-            w_ref, qweight, scales = rand_marlin_weight_mxfp4_like(w[i], group_size)
+            w_ref, qweight, scales = rand_marlin_weight_mxfp4_like(w[i], group_size, input_dtype=input_dtype)
         else:
             w_ref, qweight, scales, g_idx, sort_indices, _ = marlin_quantize(
                 w[i].transpose(1, 0), quant_type, group_size, act_order, torch.randperm(k), input_dtype=input_dtype)

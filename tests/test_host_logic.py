@@ -509,8 +509,10 @@ def test_mxfp4_host_helpers():
     assert out.dtype == torch.float8_e8m0fnu
     assert out.view(torch.uint8).tolist() == [[120, 122, 121, 123, 124, 126, 125, 127]]
     assert np.array_equal(out.view(torch.uint8).numpy(), mo.mxfp4_process_scales(e.numpy()))
-    with pytest.raises(NotImplementedError):
-        f4.mxfp4_marlin_process_scales(s, input_dtype=torch.float8_e4m3fn)
+    a8 = f4.mxfp4_marlin_process_scales(s, input_dtype=torch.float8_e4m3fn)   # in place, plus 6
+    assert a8.dtype == torch.float8_e8m0fnu
+    assert a8.view(torch.uint8).tolist() == [[v + 6 for v in e.view(-1).tolist()]]
+    assert np.array_equal(a8.view(torch.uint8).numpy(), mo.mxfp4_process_scales_a8(e.numpy()))
     from sonar_amd import marlin_utils_fp8 as f8   # MXFP8: the same reorder (marlin_utils_fp8.py:381-386)
     assert torch.equal(f8.mxfp8_marlin_process_scales(s).view(torch.uint8), out.view(torch.uint8))
     assert mu.check_marlin_supported(st.float4_e2m1f, 32)

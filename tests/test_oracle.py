@@ -756,3 +756,32 @@ def test_marlin8_a8_layout_two_derivations_agree():
         tile = (k // 32) * 4 + n // 32
         assert idx.tolist() == [tile * 256 + (4 * (n % 8) + (k % 16) // 4) * 8 + 2 * ((n % 32) // 8) + (k % 32) // 16]
         assert w[idx[0]] == 255 << (8 * (k % 4))
+
+
+def test_fp4_code_as_fp8_byte_is_value_times_2_pow_minus_6():
+    """The byte the 8-bit-activation kernels make of a float4_e2m1f code, decoded as float8_e4m3fn,
+    is 2^-6 times the code's value for all 16 codes; the scale bytes carry the 6."""
+    codes = np.arange(16)
+    got = mo.fp8_e4m3fn_value(mo.fp4_code_as_fp8_byte(codes))
+    assert np.array_equal(got * np.float32(64.0), mo.fp4_e2m1_values())
+    # the float8_e4m3fn decoder itself, against torch's
+    import torch
+    every = np.array([b for b in range(256) if b & 0x7f != 0x7f], dtype=np.uint8)
+    assert np.array_equal(mo.fp8_e4m3fn_value(every),
+                          torch.from_numpy(every).view(torch.float8_e4m3fn).float().numpy())
+    b = np.array([[10, 100], [121, 240]], dtype=np.uint8)
+    assert np.array_equal(mo.mxfp4_process_scales_a8(b), b + 6)
+    assert np.array_equal(mo.mx_scale_values(mo.mxfp4_process_scales_a8(b)) / 64, mo.mx_scale_values(b))
+    with pytest.raises(AssertionError):
+        mo.mxfp4_process_scales_a8(np.array([250], dtype=np.uint8))
+
+
+def test_gemm_w4a8_fp4_against_dequantised_matmul():
+    rng = np.random.default_rng(5)
+    k, n, m = 64, 8, 3
+    codes = rng.integers(0, 16, size=(k, n))
+    e = rng.integers(120, 130, size=(k // 32, n)).astype(np.uint8)
+    a = rng.standard_normal((m, k)).astype(np.float32)
+    a_s = rng.uniform(0.5, 2, size=m).astype(np.float32)
+    want = (a.astype(np.float64) @ mo.dequantize_mxfp4(codes, e, "bf16").astype(np.float64)) * a_s[:, None]
+    assert np.allclose(mo.gemm_w4a8_fp4(a, a_s, codes, e), want, rtol=1e-6)
