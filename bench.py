@@ -556,7 +556,7 @@ def main() -> int:
                                 "frac_mfma": round(fl / s / 1e12 / MFMA_PEAK_TFLOPS, 4)})
         out["roofline_mfma"] = {"bound": "mfma", "achieved": round(pflops / ps / 1e12, 1), "peak": MFMA_PEAK_TFLOPS,
                                 "unit": "TFLOP/s", "frac": round(pflops / ps / 1e12 / MFMA_PEAK_TFLOPS, 4),
-                                "kernel": "marlin_tile_async_kernel<f16> (+ tile_reduce_kernel where K is split)",
+                                "kernel": "marlin_tile_wide_kernel<f16> (+ tile_reduce_kernel where K is split)",
                                 "workload": "the four GEMMs of the layer at M=4096, fp16 activations ~ N(0,0.5), "
                                             + ("4 plain launches of the step" if args.eager else
                                                f"4 steps per graph, median of {REPLAYS} replays"),

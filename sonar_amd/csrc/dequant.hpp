@@ -85,6 +85,20 @@ struct Dq<_Float16> {
     const half2_t w0 = d0 * c.s, w1 = d1 * c.s, w2 = d2 * c.s, w3 = d3 * c.s;
     return vec8{w0.x, w0.y, w1.x, w1.y, w2.x, w2.y, w3.x, w3.y};
   }
+  // word() one instruction at a time, for kernels that place the instructions themselves: pair
+  // `part` (0..3) of the word is stage3(stage2(stage1(part < 2 ? q : q >> 8, part, magic), c, part), c)
+  typedef half2_t Mid;
+  static __device__ __forceinline__ uint32_t stage1(uint32_t q, int part, uint32_t magic) {
+    return and_or(q, (part & 1) ? 0x00f000f0u : 0x000f000fu, magic);
+  }
+  static __device__ __forceinline__ Mid stage2(uint32_t x, const Col& c, int part) {
+    const half2_t r16 = half2_t{(_Float16)0.0625f, (_Float16)0.0625f};
+    if (part & 1) return __builtin_elementwise_fma(__builtin_bit_cast(half2_t, x), r16, c.c1);
+    return __builtin_bit_cast(half2_t, x) - c.c0;
+  }
+  static __device__ __forceinline__ uint32_t stage3(Mid y, const Col& c) {
+    return __builtin_bit_cast(uint32_t, y * c.s);
+  }
   static __device__ __forceinline__ floatx4_t mfma(vec8 w, vec8 a, floatx4_t acc) {
     return __builtin_amdgcn_mfma_f32_16x16x32_f16(w, a, acc, 0, 0, 0);
   }
@@ -134,6 +148,19 @@ struct Dq<__bf16> {
     const bf16x2_t w2 = pair(lo1, c.s, c.c0);
     const bf16x2_t w3 = pair(hi1, c.s16, c.c1);
     return vec8{w0.x, w0.y, w1.x, w1.y, w2.x, w2.y, w3.x, w3.y};
+  }
+  // word() in three stages (see Dq<_Float16>)
+  typedef floatx2_t Mid;
+  static __device__ __forceinline__ uint32_t stage1(uint32_t q, int part, uint32_t magic) {
+    return and_or(q, (part & 1) ? 0x00f000f0u : 0x000f000fu, magic);
+  }
+  static __device__ __forceinline__ Mid stage2(uint32_t x, const Col& c, int part) {
+    const half2_t h = __builtin_bit_cast(half2_t, x);
+    const float mul = (part & 1) ? c.s16 : c.s, add = (part & 1) ? c.c1 : c.c0;
+    return floatx2_t{__builtin_fmaf((float)h.x, mul, add), __builtin_fmaf((float)h.y, mul, add)};
+  }
+  static __device__ __forceinline__ uint32_t stage3(Mid y, const Col&) {
+    return __builtin_bit_cast(uint32_t, __builtin_convertvector(y, bf16x2_t));
   }
   static __device__ __forceinline__ floatx4_t mfma(vec8 w, vec8 a, floatx4_t acc) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(w, a, acc, 0, 0, 0);

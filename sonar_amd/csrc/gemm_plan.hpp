@@ -51,6 +51,8 @@ inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool a
   plan.tile = true;
   plan.k_splits = splits;
   plan.k_steps_per_split = (k_steps + splits - 1) / splits;
+  // ranges of a multiple of four steps where K allows it (the wide tile kernel takes only those)
+  if (k_steps % 4 == 0) plan.k_steps_per_split = (plan.k_steps_per_split + 3) / 4 * 4;
   plan.k_splits = (k_steps + plan.k_steps_per_split - 1) / plan.k_steps_per_split;  // no empty split
   plan.whole_tiles = plan.k_splits > 1 ? whole_tiles : tiles;
   return plan;

@@ -595,6 +595,9 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
   // and the copies for steps past the end fetch the last step again, into a
   // slot nobody reads any more.  So seven copies are outstanding at every wait.
   asm volatile("s_waitcnt vmcnt(%0)" ::"n"(kAsyncCopies) : "memory");  // stage k_first has landed
+  // a shared ring: the blocks of k block 0 are the copies of the strip's wavefront of group 0,
+  // which the wavefront of group 1 may read only behind a barrier that follows that wait
+  if constexpr (W8 != 0) phase_end();
   raw_start(0, 0, true);
   phase_end();
   {
@@ -713,6 +716,332 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
       packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
       packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
       *reinterpret_cast<uint2*>(p.c + c_row[mb] * p.size_n + n) = packed;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// The wide form of the asynchronous tile kernel: the same 256 x 256 tile and K
+// step, four wavefronts instead of eight, one per SIMD with the whole register
+// file (256 accumulator registers for 256 rows x 64 columns: a strip over all
+// rows of the tile).  A chunk of weights is dequantised once per workgroup
+// instead of once per group of rows and feeds 64 MFMAs; with no second
+// wavefront on the SIMD the other work (dequantising the next chunk, the LDS
+// reads of A two row blocks ahead, the copies of a later stage) sits between
+// the MFMAs of the wavefront's own instruction stream, one to two instructions
+// behind each MFMA, where the matrix pipeline hides them.
+//   * A: a ring of four 32-KiB stages filled by LDS-DMA, wavefront w copying
+//     row blocks 4w..4w+3 (eight 1-KiB regions, the layout of the kernel above).
+//   * W: the two chunks of a step go from memory straight into registers (one
+//     16-byte load per lane and chunk), a ring of four register sets.
+//   * scales / zero points: one 256-byte row per step through a private LDS
+//     ring of eight rows, fetched a step earlier than the rest.
+// The eleven memory operations a wavefront issues per step (8 + 1 + 2: stage
+// kt + 3 of A and W, the scale row of step kt + 4) go out in the second half of
+// step kt.  One barrier per step, between its halves: before it a wavefront
+// waits until only the eleven youngest operations are outstanding, so behind it
+// stage kt + 1 has landed for everyone and the slot of stage kt - 1 is free.
+// The MFMAs are written as asm statements with the accumulator as a tied
+// operand: 224 accumulator registers in AGPRs, 32 in VGPRs, every one updated in
+// place (left to the register allocator, the 256 accumulators of this loop get
+// copied between registers all the time).  The compiler therefore does not see
+// MFMAs here and pads no matrix-core hazard: none arises inside the loop (an
+// accumulator is touched again 64 MFMAs later, operands are written long before
+// they are read), and the results are read after the pipeline has drained
+// (s_nop below).
+// 4-bit integer codes, groups of 64 * 2^i rows or one group, K ranges of a
+// multiple of four steps, no act-order, dense calls.
+constexpr int kWideStages = 4;
+constexpr int kWideScaleRows = 8;
+constexpr int kWideA = kWideStages * kStageA;                      // 128 KiB
+constexpr int kWideLds = kWideA + 4 * kWideScaleRows * 256;        // + the scale rows of four wavefronts
+constexpr int kWideOps = 11;
+
+template <typename T, bool HAS_ZP>
+__global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void marlin_tile_wide_kernel(
+    const TileParams p) {
+  typedef typename Dq<T>::vec8 vec8;
+  typedef typename Dq<T>::Col Col;
+  typedef typename Dq<T>::Mid Mid;
+  extern __shared__ __attribute__((aligned(1024))) char smem[];
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int col16 = lane & 15;
+  const int kb = lane >> 4;
+  const uint32_t magic = magic_register();
+  const bool grouped = p.num_groups > 1;
+
+  int tile, tile_m, tile_n, split;
+  bool whole_k;
+  if (!tile_of_workgroup(p, tile, split, whole_k)) return;
+  tile_coords(p, tile, tile_m, tile_n);
+  const int m0 = tile_m * kTileM;
+  const int strip0 = tile_n * (kTileN / kStripN);
+  const int strips_here = min(kTileN / kStripN, p.size_n / kStripN - strip0);
+  const bool active = wave < strips_here;
+  // a wavefront past the last strip works on the last strip again and stores nothing
+  const int strip = strip0 + (active ? wave : strips_here - 1);
+
+  // ---- sources (regions of A as in marlin_tile_async_kernel; wavefront w fills regions 8w..8w+7)
+  const char* a_src[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    const int region = 8 * wave + i;
+    const int r8 = lane >> 3;
+    int row = m0 + 16 * (region >> 1) + 8 * (region & 1) + r8;
+    if (row >= p.size_m) row = p.size_m - 1;   // rows past M are computed and never stored
+    a_src[i] = reinterpret_cast<const char*>(p.a) + ((long)row * p.lda + 8 * ((lane & 7) ^ r8)) * 2;
+  }
+  const uint4* b_src = p.b + (size_t)(unsigned)(strip * p.chunks_per_strip) * 64 + lane;
+  const char* s_src;
+  long s_group_stride;
+  if (HAS_ZP && lane >= 32) {
+    s_src = reinterpret_cast<const char*>(p.zeros + strip * 8 + (lane & 7));
+    s_group_stride = (long)(p.size_n / 8) * 4;
+  } else {
+    s_src = reinterpret_cast<const char*>(p.scales + strip * kStripN) + 4 * (lane & 31);
+    s_group_stride = (long)p.size_n * 2;
+  }
+  // steps per group as a shift (the host checks: group_size = 64 * 2^i)
+  const int group_shift = grouped ? 31 - __builtin_clz(p.group_size / kTileK) : 0;
+  char* sring = smem + kWideA + wave * (kWideScaleRows * 256);
+  const uint32_t a_lds = (uint32_t)(uintptr_t)(lds_void_t*)smem;
+  const uint32_t s_lds = (uint32_t)(uintptr_t)(lds_void_t*)sring;
+
+  // K steps [k_first, k_tiles) of this workgroup
+  const int k_first = whole_k ? 0 : split * p.k_steps_per_split;
+  const int k_tiles = whole_k ? p.size_k / kTileK : min(p.size_k / kTileK, k_first + p.k_steps_per_split);
+
+  u32x4_t wq[kWideStages][2];   // packed chunks in flight or waiting
+  // the scale row of step kt (clamped to the last step) into its ring position
+  auto issue_scales = [&](int kt) __attribute__((always_inline)) {
+    const int k = min(kt, k_tiles - 1);
+    const int grp = grouped ? k >> group_shift : 0;
+    __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)grp * s_group_stride),
+                                     (lds_void_t*)(sring + ((kt - k_first) & (kWideScaleRows - 1)) * 256), 4, 0, 0);
+  };
+  // memory operation `idx` (0..10) issued for step kt into ring position `slot`: 0..7 the
+  // blocks of A of step kt, 8 the scale row of step kt + 1, 9 and 10 the chunks of step kt
+  auto issue_one = [&](int kt, int slot, int idx) __attribute__((always_inline)) {
+    const int k = min(kt, k_tiles - 1);
+    if (idx < 8) {
+      __builtin_amdgcn_global_load_lds((glb_void_t*)(a_src[idx] + (long)k * (kTileK * 2)),
+                                       (lds_void_t*)(smem + slot * kStageA + (8 * wave + idx) * kBlockBytes), 16, 0, 0);
+    } else if (idx == 8) {
+      issue_scales(kt + 1);
+    } else {
+      const uint4* g = b_src + (size_t)(2 * k + (idx - 9)) * 64;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(wq[slot][idx - 9]) : "v"(g) : "memory");
+    }
+  };
+
+  uint32_t s_off[4];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) s_off[j] = 2 * scale_slot(16 * j + col16, grouped);
+  const uint32_t z_off = 128 + 4 * zero_point_word(col16);
+  // operand lane (kb, col16) of row block 0, k block b of stage 0: piece 4 b + kb of row col16
+  uint32_t a_base[2];
+#pragma unroll
+  for (int b = 0; b < 2; ++b)
+    a_base[b] = a_lds + (col16 >> 3) * kBlockBytes + (col16 & 7) * 128 + (((4 * b + kb) ^ (col16 & 7)) * 16);
+
+  floatx4_t acc[4][16];
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+    for (int mb = 0; mb < 16; ++mb) {
+      acc[nb][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
+      // the zeros sit where the MFMAs will hold the accumulator, so that the value has one home
+      // on every path to the stores
+      if (mb < 14) asm volatile("" : "+a"(acc[nb][mb]));
+      else asm volatile("" : "+v"(acc[nb][mb]));
+    }
+
+  constexpr int kAhead = 4;   // operands of A are read this many row blocks ahead
+  u32x4_t av[8];          // row block rb in av[rb & 7]
+  uint32_t wb[2][4][4];   // dequantised chunk of k block b: four operand blocks of 16 columns, four pairs each
+  uint32_t sb0 = 0, sb1 = 0, sb2 = 0, sb3 = 0, zw = 0;
+  Col cols[2][4];         // by the parity of the step
+
+#define SONAR_WIDE_READ(dst, base, off) \
+  asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(dst) : "v"(base), "i"(off) : "memory")
+#define SONAR_WIDE_LANDED(n, reg) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(reg) : "n"(n) : "memory")
+
+  auto scales_start = [&](int kt) __attribute__((always_inline)) {
+    const uint32_t r_at = s_lds + ((kt - k_first) & (kWideScaleRows - 1)) * 256;
+    asm volatile(
+        "ds_read_u16 %0, %5\n\t"
+        "ds_read_u16 %1, %6\n\t"
+        "ds_read_u16 %2, %7\n\t"
+        "ds_read_u16 %3, %8\n\t"
+        "ds_read_b32 %4, %9"
+        : "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
+        : "v"(r_at + s_off[0]), "v"(r_at + s_off[1]), "v"(r_at + s_off[2]), "v"(r_at + s_off[3]), "v"(r_at + z_off)
+        : "memory");
+  };
+  auto make_col = [&](int set, int j) __attribute__((always_inline)) {
+    const uint32_t sbits = j == 0 ? sb0 : j == 1 ? sb1 : j == 2 ? sb2 : sb3;
+    int z = 8;
+    if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
+    cols[set][j] = Dq<T>::make_col((uint16_t)sbits, z);
+  };
+  auto word_of = [](const u32x4_t& q, int j) __attribute__((always_inline)) -> uint32_t {
+    return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
+  };
+  // acc[j][rb] += W block j (16 columns) x A row block rb, in place; row blocks 14 and 15 in VGPRs
+  auto mfma = [&](int B, int j, int rb) __attribute__((always_inline)) {
+    const u32x4_t w = u32x4_t{wb[B][j][0], wb[B][j][1], wb[B][j][2], wb[B][j][3]};
+    if constexpr (std::is_same<T, _Float16>::value) {
+      if (rb < 14) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[j][rb]) : "v"(w), "v"(av[rb & 7]));
+      else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[j][rb]) : "v"(w), "v"(av[rb & 7]));
+    } else {
+      if (rb < 14) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[j][rb]) : "v"(w), "v"(av[rb & 7]));
+      else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc[j][rb]) : "v"(w), "v"(av[rb & 7]));
+    }
+  };
+
+  // One k block of step kt: 16 row blocks of four MFMAs.  R: ring position of the step's
+  // stage, B: the k block.  Behind the MFMAs of a row block, one instruction each: pair
+  // rb % 4 of word rb / 4 of the next half step's chunk; then B = 0: the scales of step kt + 1
+  // become per-column constants; B = 1: one memory operation of step kt + 3.
+  auto chunk = [&](const int R, const int B, const int kt) __attribute__((always_inline)) {
+    const int NR = B ? (R + 1) & 3 : R;   // stage and k block of the half step after this one
+    const int NB = B ^ 1;
+    const int set = B ? (R + 1) & 1 : R & 1;   // constants of the step the next half step belongs to
+    const uint32_t a_cur = a_base[B] + R * kStageA;
+    const uint32_t a_next = a_base[NB] + NR * kStageA;
+    const u32x4_t& q4 = B ? wq[NR][0] : wq[R][1];
+#pragma unroll
+    for (int rb = 0; rb < 16; ++rb) {
+      const int j = rb >> 2, part = rb & 3;
+      // reads started after the one of this row block: those of the next kAhead - 1 row blocks,
+      // and in the first half the five scale reads of slot 0
+      if (B == 0 && rb >= 1 && rb <= kAhead) SONAR_WIDE_LANDED(kAhead - 1 + 5, av[rb & 7]);
+      else SONAR_WIDE_LANDED(kAhead - 1, av[rb & 7]);
+      if (rb + kAhead < 16) SONAR_WIDE_READ(av[(rb + kAhead) & 7], a_cur, (rb + kAhead) * 2048);
+      else SONAR_WIDE_READ(av[(rb + kAhead) & 7], a_next, (rb + kAhead - 16) * 2048);
+      if (B == 0 && rb == 0) scales_start(kt + 1);
+      const uint32_t qw = word_of(q4, j);
+      mfma(B, 0, rb);
+      const uint32_t x = Dq<T>::stage1(part < 2 ? qw : qw >> 8, part, magic);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma(B, 1, rb);
+      const Mid y = Dq<T>::stage2(x, cols[set][j], part);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma(B, 2, rb);
+      wb[NB][j][part] = Dq<T>::stage3(y, cols[set][j]);
+      __builtin_amdgcn_sched_barrier(0);
+      mfma(B, 3, rb);
+      if (B == 0) {
+        if (rb > kAhead && rb <= kAhead + 4) make_col((R + 1) & 1, rb - kAhead - 1);
+      } else if (rb < kWideOps) {
+        issue_one(kt + 3, (R + 3) & 3, rb);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
+  auto step = [&](const int R, int kt) __attribute__((always_inline)) {
+    chunk(R, 0, kt);
+    // stage kt + 1 (its blocks of A, its two chunks) and the scale row of step kt + 2 have landed
+    // once only the operations issued in step kt - 1 are outstanding
+    asm volatile("s_waitcnt vmcnt(%2)"
+                 : "+v"(wq[(R + 1) & 3][0]), "+v"(wq[(R + 1) & 3][1])
+                 : "n"(kWideOps)
+                 : "memory");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_sched_barrier(0);
+    chunk(R, 1, kt);
+  };
+
+  // ---- prologue: the scale row of the first step, then what steps k_first - 3 .. k_first - 1 would have issued
+  issue_scales(k_first);
+#pragma unroll
+  for (int idx = 0; idx < kWideOps; ++idx) issue_one(k_first, 0, idx);
+#pragma unroll
+  for (int idx = 0; idx < kWideOps; ++idx) issue_one(k_first + 1, 1, idx);
+#pragma unroll
+  for (int idx = 0; idx < kWideOps; ++idx) issue_one(k_first + 2, 2, idx);
+  asm volatile("s_waitcnt vmcnt(%2)" : "+v"(wq[0][0]), "+v"(wq[0][1]) : "n"(2 * kWideOps) : "memory");
+  __builtin_amdgcn_s_barrier();
+  scales_start(k_first);
+  asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw) : : "memory");
+#pragma unroll
+  for (int j = 0; j < 4; ++j) make_col(0, j);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const u32x4_t w = __builtin_bit_cast(u32x4_t, Dq<T>::word(word_of(wq[0][0], j), cols[0][j], magic));
+    wb[0][j][0] = w.x;
+    wb[0][j][1] = w.y;
+    wb[0][j][2] = w.z;
+    wb[0][j][3] = w.w;
+  }
+#pragma unroll
+  for (int rb = 0; rb < kAhead; ++rb) SONAR_WIDE_READ(av[rb], a_base[0], rb * 2048);
+  __builtin_amdgcn_sched_barrier(0);
+
+  // the host gives this kernel K ranges of a multiple of four steps (the ring positions are static)
+  for (int kt = k_first; kt < k_tiles; kt += 4) {
+    step(0, kt);
+    step(1, kt + 1);
+    step(2, kt + 2);
+    step(3, kt + 3);
+  }
+  // nothing in flight may outlive the wavefront (the copies of the steps past the end, the two
+  // operand reads of the last half step), and the matrix pipeline drains before the results are read
+  asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
+  // the registers those operations were still to fill stay untouched up to here
+#pragma unroll
+  for (int i = 0; i < kWideStages; ++i) {
+    asm volatile("" : "+v"(wq[i][0]) : : "memory");
+    asm volatile("" : "+v"(wq[i][1]) : : "memory");
+  }
+#pragma unroll
+  for (int i = 0; i < 8; ++i) asm volatile("" : "+v"(av[i]) : : "memory");
+  asm volatile("" : "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw) : : "memory");
+  __builtin_amdgcn_sched_barrier(0);
+#undef SONAR_WIDE_LANDED
+#undef SONAR_WIDE_READ
+
+  if (!active) return;
+  if (!whole_k) {
+    // partial tile of this K range, in the order tile_reduce_kernel reads: 1-KiB blocks
+    // (half of the rows, strip, column block, row block)
+    const int first_split = whole_tiles(p);
+    const int split_tiles = p.tiles_m * p.tiles_n - first_split;
+    float4* dst = p.partial + ((size_t)(split * split_tiles + tile - first_split) * 256 + wave * 32) * 64 + lane;
+#pragma unroll
+    for (int nb = 0; nb < 4; ++nb)
+#pragma unroll
+      for (int mb = 0; mb < 16; ++mb) {
+        if (mb < 14) asm volatile("" : "+a"(acc[nb][mb]));   // still in its AGPRs here
+        const floatx4_t v = acc[nb][mb];
+        dst[((mb >> 3) * 128 + nb * 8 + (mb & 7)) * 64] = make_float4(v.x, v.y, v.z, v.w);
+        __builtin_amdgcn_sched_barrier(0);   // one accumulator at a time leaves the AGPRs
+      }
+    return;
+  }
+  const uint16_t* bias_src = p.bias ? p.bias + strip * kStripN : nullptr;
+#pragma unroll
+  for (int nb = 0; nb < 4; ++nb) {
+    const int n = strip * kStripN + 16 * nb + 4 * kb;
+    float bias[4] = {0.f, 0.f, 0.f, 0.f};
+    if (bias_src) {
+#pragma unroll
+      for (int r = 0; r < 4; ++r) bias[r] = Dq<T>::to_float(bias_src[scale_slot(16 * nb + 4 * kb + r, false)]);
+    }
+#pragma unroll
+    for (int mb = 0; mb < 16; ++mb) {
+      const int row = m0 + 16 * mb + col16;
+      if (mb < 14) asm volatile("" : "+a"(acc[nb][mb]));   // still in its AGPRs here
+      if (row >= p.size_m) continue;
+      const floatx4_t v = acc[nb][mb];
+      uint2 packed;
+      packed.x = (uint32_t)Dq<T>::from_float(v.x + bias[0]) | ((uint32_t)Dq<T>::from_float(v.y + bias[1]) << 16);
+      packed.y = (uint32_t)Dq<T>::from_float(v.z + bias[2]) | ((uint32_t)Dq<T>::from_float(v.w + bias[3]) << 16);
+      *reinterpret_cast<uint2*>(p.c + (long)row * p.size_n + n) = packed;
+      __builtin_amdgcn_sched_barrier(0);   // one accumulator at a time leaves the AGPRs
     }
   }
 }
@@ -857,6 +1186,18 @@ int launch_tile_async8(const TileParams& p, bool fp8, hipStream_t st) {
 }
 
 template <typename T, bool HAS_ZP>
+int launch_tile_wide(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, HAS_ZP>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, kWideLds));
+    attr_set = true;
+  }
+  marlin_tile_wide_kernel<T, HAS_ZP><<<tile_grid(p), 256, kWideLds, st>>>(p);
+  return SONAR_OK;
+}
+
+template <typename T, bool HAS_ZP>
 int launch_tile_async(const TileParams& p, hipStream_t st) {
   return (p.num_groups > 1 && p.group_size == 32) ? launch_tile_async_groups<T, HAS_ZP, true>(p, st)
                                                   : launch_tile_async_groups<T, HAS_ZP, false>(p, st);
@@ -893,6 +1234,19 @@ int launch_tile(const TileParams& p, hipStream_t st) {
   return SONAR_OK;
 }
 
+}  // namespace
+
+namespace {
+// The wide form: K ranges of a multiple of four steps, groups of 64 * 2^i rows or one group.
+bool wide_applies(const TileParams& p) {
+  static const bool no_wide = getenv("SONAR_MARLIN_NO_WIDE_TILE") != nullptr;   // debugging aid
+  if (no_wide) return false;
+  const int k_steps = p.size_k / kTileK;
+  if (k_steps % 4 != 0 || (p.k_splits > 1 && p.k_steps_per_split % 4 != 0)) return false;
+  if (p.num_groups == 1) return true;
+  const int per_group = p.group_size / kTileK;   // steps per group: a power of two
+  return p.group_size % kTileK == 0 && (per_group & (per_group - 1)) == 0;
+}
 }  // namespace
 
 // The asynchronous tile kernel needs groups of 32 rows or a multiple of 64 and no gather of A.
@@ -961,6 +1315,10 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     else if (bits == 8)   // symmetric 8-bit codes: the caller has checked
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, false>(p, fp8, st)
                                     : launch_tile_async8<__bf16, false>(p, fp8, st);
+    else if (wide_applies(p) && dtype == SONAR_DTYPE_F16)
+      rc = zp ? launch_tile_wide<_Float16, true>(p, st) : launch_tile_wide<_Float16, false>(p, st);
+    else if (wide_applies(p))
+      rc = zp ? launch_tile_wide<__bf16, true>(p, st) : launch_tile_wide<__bf16, false>(p, st);
     else if (dtype == SONAR_DTYPE_F16)
       rc = zp ? launch_tile_async<_Float16, true>(p, st) : launch_tile_async<_Float16, false>(p, st);
     else

@@ -241,8 +241,9 @@ def test_kernels_with_hand_counted_waits_do_not_spill():
     if not os.path.exists(hipcc):
         pytest.skip("hipcc not available")
     root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
-    watched = {"gemm_tile.hip": "marlin_tile_async_kernel", "gemm_stream.hip": "marlin_stream_fast_kernel"}
-    for src, kernel in watched.items():
+    watched = [("gemm_tile.hip", "marlin_tile_async_kernel"), ("gemm_tile.hip", "marlin_tile_wide_kernel"),
+               ("gemm_stream.hip", "marlin_stream_fast_kernel")]
+    for src, kernel in watched:
         out = subprocess.run(
             [hipcc, "-O3", "--offload-arch=gfx950", "-std=c++17", "-Xclang", "-target-feature", "-Xclang",
              "-packed-fp32-ops", "-I", os.path.join(root, "include"), "-I", os.path.join(root, "sonar_amd", "csrc"),
