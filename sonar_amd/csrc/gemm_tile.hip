@@ -750,14 +750,14 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 // they are read), and the results are read after the pipeline has drained
 // (s_nop below).
 // 4-bit integer codes, groups of 64 * 2^i rows or one group, K ranges of a
-// multiple of four steps, no act-order, dense calls.
+// multiple of four steps, no act-order; dense and grouped (mixture-of-experts) calls.
 constexpr int kWideStages = 4;
 constexpr int kWideScaleRows = 8;
 constexpr int kWideA = kWideStages * kStageA;                      // 128 KiB
 constexpr int kWideLds = kWideA + 4 * kWideScaleRows * 256;        // + the scale rows of four wavefronts
 constexpr int kWideOps = 11;
 
-template <typename T, bool HAS_ZP>
+template <typename T, bool HAS_ZP, bool GROUPED = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void marlin_tile_wide_kernel(
     const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
@@ -777,6 +777,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   bool whole_k;
   if (!tile_of_workgroup(p, tile, split, whole_k)) return;
   tile_coords(p, tile, tile_m, tile_n);
+  // Grouped calls: row tile t is up to four consecutive 64-slot blocks of one expert, listed in
+  // tile_table; rows are slots of sorted_ids (as in marlin_tile_async_kernel).
+  int first_slot = 0, tile_rows = kTileM;
+  long expert = 0;
+  if (GROUPED) {
+    if (tile_m >= p.tile_table[0]) return;
+    first_slot = p.tile_table[1 + 3 * tile_m] * 64;
+    tile_rows = p.tile_table[2 + 3 * tile_m] * 64;
+    expert = p.tile_table[3 + 3 * tile_m];
+  }
   const int m0 = tile_m * kTileM;
   const int strip0 = tile_n * (kTileN / kStripN);
   const int strips_here = min(kTileN / kStripN, p.size_n / kStripN - strip0);
@@ -790,18 +800,26 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int i = 0; i < 8; ++i) {
     const int region = 8 * wave + i;
     const int r8 = lane >> 3;
-    int row = m0 + 16 * (region >> 1) + 8 * (region & 1) + r8;
-    if (row >= p.size_m) row = p.size_m - 1;   // rows past M are computed and never stored
+    const int in_tile = 16 * (region >> 1) + 8 * (region & 1) + r8;
+    int row;
+    if (GROUPED) {
+      const int id = in_tile < tile_rows ? p.sorted_ids[first_slot + in_tile] : p.rows_total;
+      // padding slots read row 0, never stored
+      row = (unsigned)id < (unsigned)p.rows_total ? (p.a_by_slot ? first_slot + in_tile : id / p.top_k) : 0;
+    } else {
+      row = m0 + in_tile;
+      if (row >= p.size_m) row = p.size_m - 1;   // rows past M are computed and never stored
+    }
     a_src[i] = reinterpret_cast<const char*>(p.a) + ((long)row * p.lda + 8 * ((lane & 7) ^ r8)) * 2;
   }
-  const uint4* b_src = p.b + (size_t)(unsigned)(strip * p.chunks_per_strip) * 64 + lane;
+  const uint4* b_src = p.b + expert * p.expert_b_stride + (size_t)(unsigned)(strip * p.chunks_per_strip) * 64 + lane;
   const char* s_src;
   long s_group_stride;
   if (HAS_ZP && lane >= 32) {
-    s_src = reinterpret_cast<const char*>(p.zeros + strip * 8 + (lane & 7));
+    s_src = reinterpret_cast<const char*>(p.zeros + expert * p.expert_z_stride + strip * 8 + (lane & 7));
     s_group_stride = (long)(p.size_n / 8) * 4;
   } else {
-    s_src = reinterpret_cast<const char*>(p.scales + strip * kStripN) + 4 * (lane & 31);
+    s_src = reinterpret_cast<const char*>(p.scales + expert * p.expert_s_stride + strip * kStripN) + 4 * (lane & 31);
     s_group_stride = (long)p.size_n * 2;
   }
   // steps per group as a shift (the host checks: group_size = 64 * 2^i)
@@ -1005,7 +1023,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #undef SONAR_WIDE_READ
 
   if (!active) return;
-  if (!whole_k) {
+  if (!GROUPED && !whole_k) {
     // partial tile of this K range, in the order tile_reduce_kernel reads: 1-KiB blocks
     // (half of the rows, strip, column block, row block)
     const int first_split = whole_tiles(p);
@@ -1022,25 +1040,46 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       }
     return;
   }
-  const uint16_t* bias_src = p.bias ? p.bias + strip * kStripN : nullptr;
+  const uint16_t* bias_src = p.bias ? p.bias + expert * p.expert_bias_stride + strip * kStripN : nullptr;
+  float bias[4][4];
 #pragma unroll
-  for (int nb = 0; nb < 4; ++nb) {
-    const int n = strip * kStripN + 16 * nb + 4 * kb;
-    float bias[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bias_src) {
+  for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-      for (int r = 0; r < 4; ++r) bias[r] = Dq<T>::to_float(bias_src[scale_slot(16 * nb + 4 * kb + r, false)]);
+    for (int r = 0; r < 4; ++r)
+      bias[nb][r] = bias_src ? Dq<T>::to_float(bias_src[scale_slot(16 * nb + 4 * kb + r, false)]) : 0.f;
+#pragma unroll
+  for (int mb = 0; mb < 16; ++mb) {
+    // the row of C this lane writes for this row block
+    const int r = 16 * mb + col16;
+    long c_row = -1;
+    float row_w = 1.f;
+    if (GROUPED) {
+      const int id = r < tile_rows ? p.sorted_ids[first_slot + r] : p.rows_total;
+      if ((unsigned)id < (unsigned)p.rows_total) {
+        c_row = id;
+        // the routing weight is rounded to the activation type and the product is
+        // formed and rounded in that type (marlin_template.h(moe):1893-1897)
+        if (p.mul_topk) row_w = Dq<T>::to_float(Dq<T>::from_float(p.topk_weights[id]));
+      }
+    } else if (m0 + r < p.size_m) {
+      c_row = m0 + r;
     }
 #pragma unroll
-    for (int mb = 0; mb < 16; ++mb) {
-      const int row = m0 + 16 * mb + col16;
+    for (int nb = 0; nb < 4; ++nb) {
       if (mb < 14) asm volatile("" : "+a"(acc[nb][mb]));   // still in its AGPRs here
-      if (row >= p.size_m) continue;
-      const floatx4_t v = acc[nb][mb];
-      uint2 packed;
-      packed.x = (uint32_t)Dq<T>::from_float(v.x + bias[0]) | ((uint32_t)Dq<T>::from_float(v.y + bias[1]) << 16);
-      packed.y = (uint32_t)Dq<T>::from_float(v.z + bias[2]) | ((uint32_t)Dq<T>::from_float(v.w + bias[3]) << 16);
-      *reinterpret_cast<uint2*>(p.c + (long)row * p.size_n + n) = packed;
+      if (c_row >= 0) {
+        const floatx4_t v = acc[nb][mb];
+        uint16_t o[4] = {Dq<T>::from_float(v.x + bias[nb][0]), Dq<T>::from_float(v.y + bias[nb][1]),
+                         Dq<T>::from_float(v.z + bias[nb][2]), Dq<T>::from_float(v.w + bias[nb][3])};
+        if (GROUPED && p.mul_topk) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i) o[i] = Dq<T>::from_float(Dq<T>::to_float(o[i]) * row_w);
+        }
+        uint2 packed;
+        packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+        packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+        *reinterpret_cast<uint2*>(p.c + c_row * p.size_n + strip * kStripN + 16 * nb + 4 * kb) = packed;
+      }
       __builtin_amdgcn_sched_barrier(0);   // one accumulator at a time leaves the AGPRs
     }
   }
@@ -1185,15 +1224,15 @@ int launch_tile_async8(const TileParams& p, bool fp8, hipStream_t st) {
              : launch_tile_async8_groups<T, GROUPED, false, 1>(p, st);
 }
 
-template <typename T, bool HAS_ZP>
+template <typename T, bool HAS_ZP, bool GROUPED = false>
 int launch_tile_wide(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, HAS_ZP>,
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, HAS_ZP, GROUPED>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, kWideLds));
     attr_set = true;
   }
-  marlin_tile_wide_kernel<T, HAS_ZP><<<tile_grid(p), 256, kWideLds, st>>>(p);
+  marlin_tile_wide_kernel<T, HAS_ZP, GROUPED><<<tile_grid(p), 256, kWideLds, st>>>(p);
   return SONAR_OK;
 }
 
@@ -1412,12 +1451,16 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   else if (bits == 8)
     rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, true>(p, fp8, st)
                                   : launch_tile_async8<__bf16, true>(p, fp8, st);
+  else if (wide_applies(p) && dtype == SONAR_DTYPE_F16)
+    rc = zeros ? launch_tile_wide<_Float16, true, true>(p, st) : launch_tile_wide<_Float16, false, true>(p, st);
+  else if (wide_applies(p))
+    rc = zeros ? launch_tile_wide<__bf16, true, true>(p, st) : launch_tile_wide<__bf16, false, true>(p, st);
   else if (dtype == SONAR_DTYPE_F16)
     rc = zeros ? launch_tile_grouped<_Float16, true>(p, st) : launch_tile_grouped<_Float16, false>(p, st);
   else
     rc = zeros ? launch_tile_grouped<__bf16, true>(p, st) : launch_tile_grouped<__bf16, false>(p, st);
   if (rc) return rc;
-  return launch_status("marlin_tile_async_kernel (grouped)");
+  return launch_status("tile kernel (grouped)");
 }
 
 }  // namespace sonar
