@@ -8,22 +8,24 @@ namespace sonar {
 
 struct GemmPlan {
   bool tile;        // MFMA-tiled kernel (else the streaming kernels, in 64-row slabs)
-  int k_splits;     // workgroups per split 256 x 256 tile along K (tile kernel only)
+  int tile_rows;    // rows of a tile: 256, or 128 (the wide tile kernel's form for calls with few tiles)
+  int k_splits;     // workgroups per split tile along K (tile kernel only)
   int k_steps_per_split;
   // With k_splits > 1: the first `whole_tiles` tiles of the tile numbering are
   // each computed by one workgroup over the whole of K, the rest are split.
   int64_t whole_tiles;
 };
 
-inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool async_tile) {
-  GemmPlan plan = {false, 1, 0, 0};
+inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool async_tile, int tile_rows = 256) {
+  GemmPlan plan = {false, tile_rows, 1, 0, 0};
   if (size_m <= 64 || size_k % 64 != 0) return plan;
-  const int64_t tiles = ((size_m + 255) / 256) * ((size_n + 255) / 256);
+  const int64_t tiles = ((size_m + tile_rows - 1) / tile_rows) * ((size_n + 255) / 256);
   const int k_steps = (int)(size_k / 64);
   plan.k_steps_per_split = k_steps;
   // Few tiles leave compute units idle: split K so that about 256 workgroups
   // run, each with at least eight K steps.  Partial tiles cost 256 KiB of
-  // fp32 traffic each way, so up to 128 rows the streaming kernels stay ahead.
+  // fp32 traffic each way (128 with 128-row tiles), so up to 128 rows the streaming kernels
+  // stay ahead.
   int splits = 1;
   if (async_tile && tiles < 256) {
     splits = (int)(256 / tiles);
@@ -60,8 +62,24 @@ inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool a
 
 inline size_t plan_partial_bytes(const GemmPlan& plan, int64_t size_m, int64_t size_n) {
   if (!plan.tile || plan.k_splits <= 1) return 0;
-  const int64_t tiles = ((size_m + 255) / 256) * ((size_n + 255) / 256);
-  return (size_t)plan.k_splits * (size_t)(tiles - plan.whole_tiles) * 256 * 1024;
+  const int64_t tiles = ((size_m + plan.tile_rows - 1) / plan.tile_rows) * ((size_n + 255) / 256);
+  return (size_t)plan.k_splits * (size_t)(tiles - plan.whole_tiles) * plan.tile_rows * 1024;
+}
+
+// The 128-row form pays when 256-row tiles would leave more than half of the compute units to
+// K ranges of the same tile: twice the tiles, half the ranges, half the partial-tile bytes.  With
+// a long K the partial tiles are a small part of the work and the larger tile stays ahead
+// (measured: K = 14336, M = 1024, N = 4096: 108 us against 119).
+inline bool plan_prefers_128_rows(int64_t size_m, int64_t size_n, int64_t size_k) {
+  const int64_t tiles256 = ((size_m + 255) / 256) * ((size_n + 255) / 256);
+  return size_m > 128 && tiles256 <= 128 && size_k <= 8192;
+}
+
+// Scratch for the partial tiles of either tiling.
+inline size_t plan_partial_bytes_any(int64_t size_m, int64_t size_n, int64_t size_k) {
+  const size_t a = plan_partial_bytes(plan_gemm(size_m, size_n, size_k, true, 256), size_m, size_n);
+  const size_t b = plan_partial_bytes(plan_gemm(size_m, size_n, size_k, true, 128), size_m, size_n);
+  return a > b ? a : b;
 }
 
 }  // namespace sonar

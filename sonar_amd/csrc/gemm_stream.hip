@@ -1701,7 +1701,7 @@ size_t stream_scratch_bytes() { return (size_t)2 * cu_count() * kSlotFloat4 * si
 
 extern "C" size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k) {
   // partial tiles of the streaming kernels, then those of a split-K tile launch
-  return stream_scratch_bytes() + plan_partial_bytes(plan_gemm(size_m, size_n, size_k, true), size_m, size_n);
+  return stream_scratch_bytes() + plan_partial_bytes_any(size_m, size_n, size_k);
 }
 
 namespace {

@@ -48,6 +48,7 @@ struct TileParams {
   int num_groups, group_size;
   int chunks_per_strip;
   int tiles_m, tiles_n;
+  int tile_rows;               // rows of a tile: 256 (128: marlin_tile_wide_kernel with 8 row blocks)
   int tile_band;               // rows of tiles per band of the tile numbering (tile_of_workgroup)
   // split K (k_splits > 1): workgroup (tile, split) of a split tile covers K steps
   // [split * k_steps_per_split, ...) and leaves its fp32 tile in `partial` for tile_reduce_kernel
@@ -753,16 +754,23 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 // multiple of four steps, no act-order; dense and grouped (mixture-of-experts) calls.
 constexpr int kWideStages = 4;
 constexpr int kWideScaleRows = 8;
-constexpr int kWideA = kWideStages * kStageA;                      // 128 KiB
-constexpr int kWideLds = kWideA + 4 * kWideScaleRows * 256;        // + the scale rows of four wavefronts
-constexpr int kWideOps = 11;
+// RB: row blocks of 16 rows a wavefront owns: 16 (a 256-row tile) or 8 (a 128-row tile, for
+// calls with few tiles: twice the tiles, half the K ranges and half the partial-tile traffic).
+constexpr int wide_stage(int rb) { return rb * 2 * kBlockBytes; }                    // one stage of A
+constexpr int wide_a(int rb) { return kWideStages * wide_stage(rb); }                // 128 / 64 KiB
+constexpr int wide_lds(int rb) { return wide_a(rb) + 4 * kWideScaleRows * 256; }     // + the scale rows of four wavefronts
+constexpr int wide_ops(int rb) { return rb / 2 + 3; }   // per wavefront and step: its blocks of A, the scale row, two chunks
 
-template <typename T, bool HAS_ZP, bool GROUPED = false>
+template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void marlin_tile_wide_kernel(
     const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq<T>::Col Col;
   typedef typename Dq<T>::Mid Mid;
+  static_assert(RB == 16 || (RB == 8 && !GROUPED), "256-row tiles, or 128-row tiles for dense calls");
+  constexpr int kRows = 16 * RB;
+  constexpr int kStage = wide_stage(RB), kWideA = wide_a(RB), kWideOps = wide_ops(RB);
+  constexpr int kAgprBlocks = RB == 16 ? 14 : RB;   // row blocks whose accumulators sit in AGPRs
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
   const int tid = threadIdx.x;
@@ -779,7 +787,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   tile_coords(p, tile, tile_m, tile_n);
   // Grouped calls: row tile t is up to four consecutive 64-slot blocks of one expert, listed in
   // tile_table; rows are slots of sorted_ids (as in marlin_tile_async_kernel).
-  int first_slot = 0, tile_rows = kTileM;
+  int first_slot = 0, tile_rows = kRows;
   long expert = 0;
   if (GROUPED) {
     if (tile_m >= p.tile_table[0]) return;
@@ -787,18 +795,18 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     tile_rows = p.tile_table[2 + 3 * tile_m] * 64;
     expert = p.tile_table[3 + 3 * tile_m];
   }
-  const int m0 = tile_m * kTileM;
+  const int m0 = tile_m * kRows;
   const int strip0 = tile_n * (kTileN / kStripN);
   const int strips_here = min(kTileN / kStripN, p.size_n / kStripN - strip0);
   const bool active = wave < strips_here;
   // a wavefront past the last strip works on the last strip again and stores nothing
   const int strip = strip0 + (active ? wave : strips_here - 1);
 
-  // ---- sources (regions of A as in marlin_tile_async_kernel; wavefront w fills regions 8w..8w+7)
-  const char* a_src[8];
+  // ---- sources (regions of A as in marlin_tile_async_kernel; wavefront w fills RB / 2 regions)
+  const char* a_src[RB / 2];
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const int region = 8 * wave + i;
+  for (int i = 0; i < RB / 2; ++i) {
+    const int region = (RB / 2) * wave + i;
     const int r8 = lane >> 3;
     const int in_tile = 16 * (region >> 1) + 8 * (region & 1) + r8;
     int row;
@@ -840,18 +848,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)grp * s_group_stride),
                                      (lds_void_t*)(sring + ((kt - k_first) & (kWideScaleRows - 1)) * 256), 4, 0, 0);
   };
-  // memory operation `idx` (0..10) issued for step kt into ring position `slot`: 0..7 the
-  // blocks of A of step kt, 8 the scale row of step kt + 1, 9 and 10 the chunks of step kt
+  // memory operation `idx` (0..kWideOps-1) issued for step kt into ring position `slot`: first the
+  // blocks of A of step kt, then the scale row of step kt + 1, then the two chunks of step kt
   auto issue_one = [&](int kt, int slot, int idx) __attribute__((always_inline)) {
     const int k = min(kt, k_tiles - 1);
-    if (idx < 8) {
+    if (idx < RB / 2) {
       __builtin_amdgcn_global_load_lds((glb_void_t*)(a_src[idx] + (long)k * (kTileK * 2)),
-                                       (lds_void_t*)(smem + slot * kStageA + (8 * wave + idx) * kBlockBytes), 16, 0, 0);
-    } else if (idx == 8) {
+                                       (lds_void_t*)(smem + slot * kStage + ((RB / 2) * wave + idx) * kBlockBytes),
+                                       16, 0, 0);
+    } else if (idx == RB / 2) {
       issue_scales(kt + 1);
     } else {
-      const uint4* g = b_src + (size_t)(2 * k + (idx - 9)) * 64;
-      asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(wq[slot][idx - 9]) : "v"(g) : "memory");
+      const int c = idx - RB / 2 - 1;
+      const uint4* g = b_src + (size_t)(2 * k + c) * 64;
+      asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(wq[slot][c]) : "v"(g) : "memory");
     }
   };
 
@@ -865,15 +875,15 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int b = 0; b < 2; ++b)
     a_base[b] = a_lds + (col16 >> 3) * kBlockBytes + (col16 & 7) * 128 + (((4 * b + kb) ^ (col16 & 7)) * 16);
 
-  floatx4_t acc[4][16];
+  floatx4_t acc[4][RB];
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-    for (int mb = 0; mb < 16; ++mb) {
+    for (int mb = 0; mb < RB; ++mb) {
       acc[nb][mb] = floatx4_t{0.f, 0.f, 0.f, 0.f};
       // the zeros sit where the MFMAs will hold the accumulator, so that the value has one home
       // on every path to the stores
-      if (mb < 14) asm volatile("" : "+a"(acc[nb][mb]));
+      if (mb < kAgprBlocks) asm volatile("" : "+a"(acc[nb][mb]));
       else asm volatile("" : "+v"(acc[nb][mb]));
     }
 
@@ -908,52 +918,61 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   auto word_of = [](const u32x4_t& q, int j) __attribute__((always_inline)) -> uint32_t {
     return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
   };
-  // acc[j][rb] += W block j (16 columns) x A row block rb, in place; row blocks 14 and 15 in VGPRs
+  // acc[j][rb] += W block j (16 columns) x A row block rb, in place; with 16 row blocks the last two in VGPRs
   auto mfma = [&](int B, int j, int rb) __attribute__((always_inline)) {
     const u32x4_t w = u32x4_t{wb[B][j][0], wb[B][j][1], wb[B][j][2], wb[B][j][3]};
     if constexpr (std::is_same<T, _Float16>::value) {
-      if (rb < 14) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[j][rb]) : "v"(w), "v"(av[rb & 7]));
+      if (rb < kAgprBlocks) asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+a"(acc[j][rb]) : "v"(w), "v"(av[rb & 7]));
       else asm volatile("v_mfma_f32_16x16x32_f16 %0, %1, %2, %0" : "+v"(acc[j][rb]) : "v"(w), "v"(av[rb & 7]));
     } else {
-      if (rb < 14) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[j][rb]) : "v"(w), "v"(av[rb & 7]));
+      if (rb < kAgprBlocks) asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+a"(acc[j][rb]) : "v"(w), "v"(av[rb & 7]));
       else asm volatile("v_mfma_f32_16x16x32_bf16 %0, %1, %2, %0" : "+v"(acc[j][rb]) : "v"(w), "v"(av[rb & 7]));
     }
   };
 
-  // One k block of step kt: 16 row blocks of four MFMAs.  R: ring position of the step's
-  // stage, B: the k block.  Behind the MFMAs of a row block, one instruction each: pair
-  // rb % 4 of word rb / 4 of the next half step's chunk; then B = 0: the scales of step kt + 1
-  // become per-column constants; B = 1: one memory operation of step kt + 3.
+  // One k block of step kt: RB row blocks of four MFMAs.  R: ring position of the step's
+  // stage, B: the k block.  Behind the MFMAs of a row block, one instruction each: one pair
+  // (with 8 row blocks: two) of the 16 of the next half step's chunk; then B = 0: the scales of
+  // step kt + 1 become per-column constants; B = 1: one memory operation of step kt + 3.
   auto chunk = [&](const int R, const int B, const int kt) __attribute__((always_inline)) {
     const int NR = B ? (R + 1) & 3 : R;   // stage and k block of the half step after this one
     const int NB = B ^ 1;
     const int set = B ? (R + 1) & 1 : R & 1;   // constants of the step the next half step belongs to
-    const uint32_t a_cur = a_base[B] + R * kStageA;
-    const uint32_t a_next = a_base[NB] + NR * kStageA;
+    const uint32_t a_cur = a_base[B] + R * kStage;
+    const uint32_t a_next = a_base[NB] + NR * kStage;
     const u32x4_t& q4 = B ? wq[NR][0] : wq[R][1];
+    constexpr int kPairs = 16 / RB;   // pairs of weights dequantised per row block
 #pragma unroll
-    for (int rb = 0; rb < 16; ++rb) {
-      const int j = rb >> 2, part = rb & 3;
+    for (int rb = 0; rb < RB; ++rb) {
+      const int j = (kPairs * rb) >> 2, part = (kPairs * rb) & 3;
       // reads started after the one of this row block: those of the next kAhead - 1 row blocks,
       // and in the first half the five scale reads of slot 0
       if (B == 0 && rb >= 1 && rb <= kAhead) SONAR_WIDE_LANDED(kAhead - 1 + 5, av[rb & 7]);
       else SONAR_WIDE_LANDED(kAhead - 1, av[rb & 7]);
-      if (rb + kAhead < 16) SONAR_WIDE_READ(av[(rb + kAhead) & 7], a_cur, (rb + kAhead) * 2048);
-      else SONAR_WIDE_READ(av[(rb + kAhead) & 7], a_next, (rb + kAhead - 16) * 2048);
+      if (rb + kAhead < RB) SONAR_WIDE_READ(av[(rb + kAhead) & 7], a_cur, (rb + kAhead) * 2048);
+      else SONAR_WIDE_READ(av[(rb + kAhead) & 7], a_next, (rb + kAhead - RB) * 2048);
       if (B == 0 && rb == 0) scales_start(kt + 1);
       const uint32_t qw = word_of(q4, j);
       mfma(B, 0, rb);
       const uint32_t x = Dq<T>::stage1(part < 2 ? qw : qw >> 8, part, magic);
+      uint32_t x2 = 0;
+      if (kPairs == 2) x2 = Dq<T>::stage1(part < 2 ? qw : qw >> 8, part + 1, magic);
       __builtin_amdgcn_sched_barrier(0);
       mfma(B, 1, rb);
       const Mid y = Dq<T>::stage2(x, cols[set][j], part);
+      Mid y2 = y;
+      if (kPairs == 2) y2 = Dq<T>::stage2(x2, cols[set][j], part + 1);
       __builtin_amdgcn_sched_barrier(0);
       mfma(B, 2, rb);
       wb[NB][j][part] = Dq<T>::stage3(y, cols[set][j]);
+      if (kPairs == 2) wb[NB][j][part + 1] = Dq<T>::stage3(y2, cols[set][j]);
       __builtin_amdgcn_sched_barrier(0);
       mfma(B, 3, rb);
       if (B == 0) {
-        if (rb > kAhead && rb <= kAhead + 4) make_col((R + 1) & 1, rb - kAhead - 1);
+        // the scale reads of slot 0 have landed behind the wait of slot kAhead + 1
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          if (rb == (kAhead + 1 + c < RB ? kAhead + 1 + c : RB - 1)) make_col((R + 1) & 1, c);
       } else if (rb < kWideOps) {
         issue_one(kt + 3, (R + 3) & 3, rb);
       }
@@ -1028,12 +1047,12 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     // (half of the rows, strip, column block, row block)
     const int first_split = whole_tiles(p);
     const int split_tiles = p.tiles_m * p.tiles_n - first_split;
-    float4* dst = p.partial + ((size_t)(split * split_tiles + tile - first_split) * 256 + wave * 32) * 64 + lane;
+    float4* dst = p.partial + ((size_t)(split * split_tiles + tile - first_split) * kRows + wave * 32) * 64 + lane;
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
-      for (int mb = 0; mb < 16; ++mb) {
-        if (mb < 14) asm volatile("" : "+a"(acc[nb][mb]));   // still in its AGPRs here
+      for (int mb = 0; mb < RB; ++mb) {
+        if (mb < kAgprBlocks) asm volatile("" : "+a"(acc[nb][mb]));   // still in its AGPRs here
         const floatx4_t v = acc[nb][mb];
         dst[((mb >> 3) * 128 + nb * 8 + (mb & 7)) * 64] = make_float4(v.x, v.y, v.z, v.w);
         __builtin_amdgcn_sched_barrier(0);   // one accumulator at a time leaves the AGPRs
@@ -1048,7 +1067,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int r = 0; r < 4; ++r)
       bias[nb][r] = bias_src ? Dq<T>::to_float(bias_src[scale_slot(16 * nb + 4 * kb + r, false)]) : 0.f;
 #pragma unroll
-  for (int mb = 0; mb < 16; ++mb) {
+  for (int mb = 0; mb < RB; ++mb) {
     // the row of C this lane writes for this row block
     const int r = 16 * mb + col16;
     long c_row = -1;
@@ -1066,7 +1085,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb) {
-      if (mb < 14) asm volatile("" : "+a"(acc[nb][mb]));   // still in its AGPRs here
+      if (mb < kAgprBlocks) asm volatile("" : "+a"(acc[nb][mb]));   // still in its AGPRs here
       if (c_row >= 0) {
         const floatx4_t v = acc[nb][mb];
         uint16_t o[4] = {Dq<T>::from_float(v.x + bias[nb][0]), Dq<T>::from_float(v.y + bias[nb][1]),
@@ -1091,21 +1110,24 @@ template <typename T>
 __global__ __launch_bounds__(256) void tile_reduce_kernel(const TileParams p) {
   const int lane = threadIdx.x & 63;
   const int col16 = lane & 15, kb = lane >> 4;
-  const long unit = (long)blockIdx.x * 4 + (threadIdx.x >> 6);   // (tile, wavefront, accumulator tile)
+  const long unit = (long)blockIdx.x * 4 + (threadIdx.x >> 6);   // (tile, 1-KiB block of the partial tile)
   const int first_split = whole_tiles(p);
   const int tiles = p.tiles_m * p.tiles_n - first_split;  // split tiles
-  if (unit >= (long)tiles * 256) return;
-  const int tile = (int)(unit >> 8);
-  const int wave = (int)(unit >> 5) & 7;
-  const int nb = (int)(unit & 31) >> 3, mb = (int)unit & 7;
+  const int blocks = p.tile_rows;                          // blocks per partial tile: 256 or 128
+  if (unit >= (long)tiles * blocks) return;
+  const int tile = (int)(unit / blocks);
+  const int within = (int)(unit - (long)tile * blocks);
+  // block = 128 (half of the rows) + 32 strip + 8 column block + row block
+  const int half = within >> 7, wave = (within >> 5) & 3;
+  const int nb = (within >> 3) & 3, mb = within & 7;
   int tile_m, tile_n;
   tile_coords(p, first_split + tile, tile_m, tile_n);
-  const int strip = tile_n * (kTileN / kStripN) + (wave & 3);
-  const int m = tile_m * kTileM + 128 * (wave >> 2) + 16 * mb + col16;
+  const int strip = tile_n * (kTileN / kStripN) + wave;
+  const int m = tile_m * p.tile_rows + 128 * half + 16 * mb + col16;
   if (strip * kStripN >= p.size_n) return;
   floatx4_t acc = floatx4_t{0.f, 0.f, 0.f, 0.f};
   for (int s = 0; s < p.k_splits; ++s) {
-    const float4 v = p.partial[((size_t)(s * tiles + tile) * 256 + (unit & 255)) * 64 + lane];
+    const float4 v = p.partial[((size_t)(s * tiles + tile) * blocks + within) * 64 + lane];
     acc += floatx4_t{v.x, v.y, v.z, v.w};
   }
   if (m >= p.size_m) return;
@@ -1224,16 +1246,23 @@ int launch_tile_async8(const TileParams& p, bool fp8, hipStream_t st) {
              : launch_tile_async8_groups<T, GROUPED, false, 1>(p, st);
 }
 
-template <typename T, bool HAS_ZP, bool GROUPED = false>
-int launch_tile_wide(const TileParams& p, hipStream_t st) {
+template <typename T, bool HAS_ZP, bool GROUPED, int RB>
+int launch_tile_wide_rows(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, HAS_ZP, GROUPED>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, kWideLds));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, HAS_ZP, GROUPED, RB>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(RB)));
     attr_set = true;
   }
-  marlin_tile_wide_kernel<T, HAS_ZP, GROUPED><<<tile_grid(p), 256, kWideLds, st>>>(p);
+  marlin_tile_wide_kernel<T, HAS_ZP, GROUPED, RB><<<tile_grid(p), 256, wide_lds(RB), st>>>(p);
   return SONAR_OK;
+}
+template <typename T, bool HAS_ZP, bool GROUPED = false>
+int launch_tile_wide(const TileParams& p, hipStream_t st) {
+  if constexpr (!GROUPED) {
+    if (p.tile_rows == 128) return launch_tile_wide_rows<T, HAS_ZP, false, 8>(p, st);
+  }
+  return launch_tile_wide_rows<T, HAS_ZP, GROUPED, 16>(p, st);
 }
 
 template <typename T, bool HAS_ZP>
@@ -1315,6 +1344,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   p.num_groups = (int)num_groups;
   p.group_size = group_size;
   p.chunks_per_strip = (int)(size_k / kChunkK);
+  p.tile_rows = kTileM;
   p.tiles_m = (int)((size_m + kTileM - 1) / kTileM);
   p.tile_band = 4;
   p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);
@@ -1332,7 +1362,22 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   static const bool no_async = getenv("SONAR_MARLIN_NO_ASYNC_TILE") != nullptr;  // debugging aid
   const bool nvfp4 = fp4 && global_scale != nullptr;   // the caller has checked: groups of 16 rows
   if ((nvfp4 || tile_async_applies(pm, num_groups, group_size)) && (!no_async || fp4)) {   // float4 codes exist here only
-    const GemmPlan plan = plan_gemm(size_m, size_n, size_k, true);
+    GemmPlan plan = plan_gemm(size_m, size_n, size_k, true);
+    // few tiles and a call the wide kernel takes: 128-row tiles
+    static const bool no_128 = getenv("SONAR_MARLIN_NO_128_ROW_TILES") != nullptr;   // debugging aid
+    if (!no_128 && bits == 4 && !fp4 && plan_prefers_128_rows(size_m, size_n, size_k)) {
+      const GemmPlan plan128 = plan_gemm(size_m, size_n, size_k, true, 128);
+      TileParams probe = p;
+      probe.k_splits = plan128.k_splits;
+      probe.k_steps_per_split = plan128.k_steps_per_split;
+      if (plan128.tile && wide_applies(probe) &&
+          (plan128.k_splits == 1 || (partial != nullptr && partial_bytes >= plan_partial_bytes(plan128, size_m, size_n)))) {
+        plan = plan128;
+        p.tile_rows = 128;
+        p.tiles_m = (int)((size_m + 127) / 128);
+        p.tile_band = 8;   // the same rows of A per band as four 256-row tiles
+      }
+    }
     if (plan.k_splits > 1 && partial != nullptr && partial_bytes >= plan_partial_bytes(plan, size_m, size_n)) {
       p.k_splits = plan.k_splits;
       p.k_steps_per_split = plan.k_steps_per_split;
@@ -1347,6 +1392,8 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
         if (p.k_splits == 1) p.partial = nullptr;
       }
     }
+    if (p.tile_rows != kTileM && !wide_applies(p))
+      return fail(SONAR_E_INVALID, "internal: 128-row tiles exist in the wide tile kernel only");
     if (nvfp4)
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16>(p, st) : launch_tile_async_nvfp4<__bf16>(p, st);
     else if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
@@ -1365,7 +1412,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     if (rc) return rc;
     if (int rc2 = launch_status("marlin_tile_async_kernel")) return rc2;
     if (p.k_splits > 1) {
-      const int blocks = (p.tiles_m * p.tiles_n - p.whole_tiles) * 64;
+      const int blocks = (p.tiles_m * p.tiles_n - p.whole_tiles) * (p.tile_rows / 4);
       if (dtype == SONAR_DTYPE_F16) tile_reduce_kernel<_Float16><<<blocks, 256, 0, st>>>(p);
       else tile_reduce_kernel<__bf16><<<blocks, 256, 0, st>>>(p);
       return launch_status("tile_reduce_kernel");
@@ -1424,6 +1471,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.num_groups = (int)num_groups;
   p.group_size = group_size;
   p.chunks_per_strip = (int)(size_k / kChunkK);
+  p.tile_rows = kTileM;
   p.tiles_m = max_tiles;
   p.tile_band = max_tiles > 0 ? max_tiles : 1;  // row tiles of different experts share no panel of W: whole columns
   p.k_splits = 1;
