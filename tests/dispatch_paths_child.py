@@ -25,6 +25,7 @@ DENSE = [
     (300, 1024, 768, 128, "bf16", False, True),
     (600, 1024, 768, 64, "fp16", True, False),
     (1100, 512, 1024, -1, "bf16", False, False),
+    (2100, 512, 4096, 128, "bf16", True, True),     # 144 tiles of 256 rows: the wide tile kernel's 256-row form
 ]
 
 

@@ -21,6 +21,8 @@ SWITCHES = [
     "SONAR_MARLIN_NO_ROW_PAIRS",     # blocks of 16 rows only
     "SONAR_MARLIN_NO_HALF_WG",       # 8-wavefront workgroups only
     "SONAR_MARLIN_NO_TILE",          # the streaming kernels in 64-row slabs for every M
+    "SONAR_MARLIN_NO_WIDE_TILE",     # the eight-wavefront tile kernel where the wide one would run
+    "SONAR_MARLIN_NO_128_ROW_TILES", # the wide tile kernel with 256-row tiles only
     "SONAR_MARLIN_NO_ASYNC_TILE",    # the register-staged tile kernel
     "SONAR_MARLIN_MAX_K_SPLITS=1",   # no split K in the tile kernel
     "SONAR_MARLIN_NO_MOE_TILE",      # the grouped streaming kernel for 64-slot blocks
