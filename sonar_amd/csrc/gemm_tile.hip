@@ -783,8 +783,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
   int tile, tile_m, tile_n, split;
   bool whole_k;
-  if (!tile_of_workgroup(p, tile, split, whole_k)) return;
-  tile_coords(p, tile, tile_m, tile_n);
+  if (GROUPED) {
+    // The launch is sized for the most row tiles the routing could make; the tiles there are
+    // (tile_table[0]) are numbered here in bands of four row tiles, so that the 32 workgroups an
+    // XCD holds share 4 panels of A and 8 panels of W (of one expert where the routing is even),
+    // and every XCD gets its share of them.
+    TileParams live = p;
+    live.tiles_m = p.tile_table[0];
+    live.tile_band = 4;
+    if (live.tiles_m <= 0 || !tile_of_workgroup(live, tile, split, whole_k)) return;
+    tile_coords(live, tile, tile_m, tile_n);
+  } else {
+    if (!tile_of_workgroup(p, tile, split, whole_k)) return;
+    tile_coords(p, tile, tile_m, tile_n);
+  }
   // Grouped calls: row tile t is up to four consecutive 64-slot blocks of one expert, listed in
   // tile_table; rows are slots of sorted_ids (as in marlin_tile_async_kernel).
   int first_slot = 0, tile_rows = kRows;
@@ -1473,7 +1485,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.chunks_per_strip = (int)(size_k / kChunkK);
   p.tile_rows = kTileM;
   p.tiles_m = max_tiles;
-  p.tile_band = max_tiles > 0 ? max_tiles : 1;  // row tiles of different experts share no panel of W: whole columns
+  p.tile_band = max_tiles > 0 ? max_tiles : 1;  // whole columns of row tiles (the wide kernel numbers its tiles itself)
   p.k_splits = 1;
   p.whole_tiles = 0;  // read only with k_splits > 1
   p.k_steps_per_split = (int)(size_k / kTileK);
