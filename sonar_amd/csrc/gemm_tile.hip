@@ -750,26 +750,31 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 // accumulator is touched again 64 MFMAs later, operands are written long before
 // they are read), and the results are read after the pipeline has drained
 // (s_nop below).
-// 4-bit integer codes, groups of 64 * 2^i rows or one group, K ranges of a
-// multiple of four steps, no act-order; dense and grouped (mixture-of-experts) calls.
+// 4-bit integer codes with groups of 64 * 2^i rows or one group, or MXFP4 (float4_e2m1f codes,
+// bf16, a scale per 32 rows: one hardware conversion and half a byte permute behind each row
+// block); K ranges of a multiple of four steps, no act-order; dense and grouped
+// (mixture-of-experts) calls.
 constexpr int kWideStages = 4;
-constexpr int kWideScaleRows = 8;
+constexpr int kWideScaleRows = 16;   // a ring of 16 rows per wavefront: eight steps of one row, or of two (MXFP4)
 // RB: row blocks of 16 rows a wavefront owns: 16 (a 256-row tile) or 8 (a 128-row tile, for
 // calls with few tiles: twice the tiles, half the K ranges and half the partial-tile traffic).
 constexpr int wide_stage(int rb) { return rb * 2 * kBlockBytes; }                    // one stage of A
 constexpr int wide_a(int rb) { return kWideStages * wide_stage(rb); }                // 128 / 64 KiB
 constexpr int wide_lds(int rb) { return wide_a(rb) + 4 * kWideScaleRows * 256; }     // + the scale rows of four wavefronts
-constexpr int wide_ops(int rb) { return rb / 2 + 3; }   // per wavefront and step: its blocks of A, the scale row, two chunks
+// memory operations per wavefront and step: its blocks of A, the scale row (MXFP4: two, one per k block), two chunks
+constexpr int wide_ops(int rb, bool fp4 = false) { return rb / 2 + (fp4 ? 4 : 3); }
 
-template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16>
+template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16, bool FP4 = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void marlin_tile_wide_kernel(
     const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq<T>::Col Col;
+  typedef typename Dq4Of<T, FP4>::type D4;   // integer codes, or float4_e2m1f with a scale per 32 rows (MXFP4: bf16)
+  typedef typename D4::Col Col;
   typedef typename Dq<T>::Mid Mid;
+  static_assert(!FP4 || (std::is_same<T, __bf16>::value && !HAS_ZP && RB == 16), "MXFP4: bf16, no zero points, 256-row tiles");
   static_assert(RB == 16 || (RB == 8 && !GROUPED), "256-row tiles, or 128-row tiles for dense calls");
   constexpr int kRows = 16 * RB;
-  constexpr int kStage = wide_stage(RB), kWideA = wide_a(RB), kWideOps = wide_ops(RB);
+  constexpr int kStage = wide_stage(RB), kWideA = wide_a(RB), kWideOps = wide_ops(RB, FP4);
   constexpr int kAgprBlocks = RB == 16 ? 14 : RB;   // row blocks whose accumulators sit in AGPRs
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -853,12 +858,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int k_tiles = whole_k ? p.size_k / kTileK : min(p.size_k / kTileK, k_first + p.k_steps_per_split);
 
   u32x4_t wq[kWideStages][2];   // packed chunks in flight or waiting
-  // the scale row of step kt (clamped to the last step) into its ring position
-  auto issue_scales = [&](int kt) __attribute__((always_inline)) {
+  // the scale row of step kt (clamped to the last step) into its ring position; MXFP4: the row of
+  // k block h of the step (groups of 32 rows), ring position 2 (kt - k_first) + h
+  auto issue_scales = [&](int kt, int h) __attribute__((always_inline)) {
     const int k = min(kt, k_tiles - 1);
-    const int grp = grouped ? k >> group_shift : 0;
+    const int grp = FP4 ? 2 * k + h : (grouped ? k >> group_shift : 0);
+    const int at = FP4 ? 2 * (kt - k_first) + h : kt - k_first;
     __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)grp * s_group_stride),
-                                     (lds_void_t*)(sring + ((kt - k_first) & (kWideScaleRows - 1)) * 256), 4, 0, 0);
+                                     (lds_void_t*)(sring + (at & (kWideScaleRows - 1)) * 256), 4, 0, 0);
   };
   // memory operation `idx` (0..kWideOps-1) issued for step kt into ring position `slot`: first the
   // blocks of A of step kt, then the scale row of step kt + 1, then the two chunks of step kt
@@ -868,10 +875,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       __builtin_amdgcn_global_load_lds((glb_void_t*)(a_src[idx] + (long)k * (kTileK * 2)),
                                        (lds_void_t*)(smem + slot * kStage + ((RB / 2) * wave + idx) * kBlockBytes),
                                        16, 0, 0);
-    } else if (idx == RB / 2) {
-      issue_scales(kt + 1);
+    } else if (idx < RB / 2 + (FP4 ? 2 : 1)) {
+      issue_scales(kt + 1, idx - RB / 2);
     } else {
-      const int c = idx - RB / 2 - 1;
+      const int c = idx - RB / 2 - (FP4 ? 2 : 1);
       const uint4* g = b_src + (size_t)(2 * k + c) * 64;
       asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(wq[slot][c]) : "v"(g) : "memory");
     }
@@ -903,14 +910,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   u32x4_t av[8];          // row block rb in av[rb & 7]
   uint32_t wb[2][4][4];   // dequantised chunk of k block b: four operand blocks of 16 columns, four pairs each
   uint32_t sb0 = 0, sb1 = 0, sb2 = 0, sb3 = 0, zw = 0;
-  Col cols[2][4];         // by the parity of the step
+  Col cols[2][4];         // by the parity of the step (MXFP4: of the k block)
 
 #define SONAR_WIDE_READ(dst, base, off) \
   asm volatile("ds_read_b128 %0, %1 offset:%2" : "=&v"(dst) : "v"(base), "i"(off) : "memory")
 #define SONAR_WIDE_LANDED(n, reg) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(reg) : "n"(n) : "memory")
 
-  auto scales_start = [&](int kt) __attribute__((always_inline)) {
-    const uint32_t r_at = s_lds + ((kt - k_first) & (kWideScaleRows - 1)) * 256;
+  auto scales_start = [&](int kt, int h) __attribute__((always_inline)) {
+    const uint32_t r_at = s_lds + ((FP4 ? 2 * (kt - k_first) + h : kt - k_first) & (kWideScaleRows - 1)) * 256;
     asm volatile(
         "ds_read_u16 %0, %5\n\t"
         "ds_read_u16 %1, %6\n\t"
@@ -925,7 +932,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const uint32_t sbits = j == 0 ? sb0 : j == 1 ? sb1 : j == 2 ? sb2 : sb3;
     int z = 8;
     if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
-    cols[set][j] = Dq<T>::make_col((uint16_t)sbits, z);
+    cols[set][j] = D4::make_col((uint16_t)sbits, z);
   };
   auto word_of = [](const u32x4_t& q, int j) __attribute__((always_inline)) -> uint32_t {
     return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
@@ -949,45 +956,74 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   auto chunk = [&](const int R, const int B, const int kt) __attribute__((always_inline)) {
     const int NR = B ? (R + 1) & 3 : R;   // stage and k block of the half step after this one
     const int NB = B ^ 1;
-    const int set = B ? (R + 1) & 1 : R & 1;   // constants of the step the next half step belongs to
+    // constants of the step the next half step belongs to (MXFP4: of the next k block)
+    const int set = FP4 ? NB : (B ? (R + 1) & 1 : R & 1);
     const uint32_t a_cur = a_base[B] + R * kStage;
     const uint32_t a_next = a_base[NB] + NR * kStage;
     const u32x4_t& q4 = B ? wq[NR][0] : wq[R][1];
     constexpr int kPairs = 16 / RB;   // pairs of weights dequantised per row block
+    uint32_t r_lo = 0;     // MXFP4: rows (0, 2) or (4, 6) of the word in hand, waiting for their odd partners
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       const int j = (kPairs * rb) >> 2, part = (kPairs * rb) & 3;
       // reads started after the one of this row block: those of the next kAhead - 1 row blocks,
-      // and in the first half the five scale reads of slot 0
-      if (B == 0 && rb >= 1 && rb <= kAhead) SONAR_WIDE_LANDED(kAhead - 1 + 5, av[rb & 7]);
+      // and the five scale reads of slot 0 (first half; MXFP4: either half)
+      if ((B == 0 || FP4) && rb >= 1 && rb <= kAhead) SONAR_WIDE_LANDED(kAhead - 1 + 5, av[rb & 7]);
       else SONAR_WIDE_LANDED(kAhead - 1, av[rb & 7]);
+      // behind this wait the scale reads of slot 0 have landed: from here on the registers they fill
+      // hold the scales (without this the compiler is free to use them any time after slot 0)
+      if ((B == 0 || FP4) && rb == (kAhead + 1 < RB ? kAhead + 1 : RB - 1))
+        asm volatile("" : "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw) : : "memory");
       if (rb + kAhead < RB) SONAR_WIDE_READ(av[(rb + kAhead) & 7], a_cur, (rb + kAhead) * 2048);
       else SONAR_WIDE_READ(av[(rb + kAhead) & 7], a_next, (rb + kAhead - RB) * 2048);
-      if (B == 0 && rb == 0) scales_start(kt + 1);
+      // the scales of the step after this one (MXFP4: of its k block B, two half steps ahead)
+      if (rb == 0 && (B == 0 || FP4)) scales_start(kt + 1, B);
       const uint32_t qw = word_of(q4, j);
-      mfma(B, 0, rb);
-      const uint32_t x = Dq<T>::stage1(part < 2 ? qw : qw >> 8, part, magic);
-      uint32_t x2 = 0;
-      if (kPairs == 2) x2 = Dq<T>::stage1(part < 2 ? qw : qw >> 8, part + 1, magic);
-      __builtin_amdgcn_sched_barrier(0);
-      mfma(B, 1, rb);
-      const Mid y = Dq<T>::stage2(x, cols[set][j], part);
-      Mid y2 = y;
-      if (kPairs == 2) y2 = Dq<T>::stage2(x2, cols[set][j], part + 1);
-      __builtin_amdgcn_sched_barrier(0);
-      mfma(B, 2, rb);
-      wb[NB][j][part] = Dq<T>::stage3(y, cols[set][j]);
-      if (kPairs == 2) wb[NB][j][part + 1] = Dq<T>::stage3(y2, cols[set][j]);
-      __builtin_amdgcn_sched_barrier(0);
-      mfma(B, 3, rb);
-      if (B == 0) {
-        // the scale reads of slot 0 have landed behind the wait of slot kAhead + 1
+      if constexpr (FP4) {
+        // one hardware conversion per row block (two rows of the column each: (0,2), (1,3), (4,6),
+        // (5,7)); behind the second and the fourth, the two byte permutes that put four rows in order
+        mfma(B, 0, rb);
+        const float sc = cols[set][j].s;
+        const uint32_t r = __builtin_bit_cast(
+            uint32_t, part == 0   ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, sc, 0)
+                      : part == 1 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, sc, 2)
+                      : part == 2 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, sc, 1)
+                                  : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, sc, 3));
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 1, rb);
+        if (part & 1) wb[NB][j][part - 1] = __builtin_amdgcn_perm(r, r_lo, 0x05040100u);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 2, rb);
+        if (part & 1) wb[NB][j][part] = __builtin_amdgcn_perm(r, r_lo, 0x07060302u);
+        else r_lo = r;
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 3, rb);
+      } else {
+        mfma(B, 0, rb);
+        const uint32_t x = Dq<T>::stage1(part < 2 ? qw : qw >> 8, part, magic);
+        uint32_t x2 = 0;
+        if (kPairs == 2) x2 = Dq<T>::stage1(part < 2 ? qw : qw >> 8, part + 1, magic);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 1, rb);
+        const Mid y = Dq<T>::stage2(x, cols[set][j], part);
+        Mid y2 = y;
+        if (kPairs == 2) y2 = Dq<T>::stage2(x2, cols[set][j], part + 1);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 2, rb);
+        wb[NB][j][part] = Dq<T>::stage3(y, cols[set][j]);
+        if (kPairs == 2) wb[NB][j][part + 1] = Dq<T>::stage3(y2, cols[set][j]);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 3, rb);
+      }
+      if (B == 0 || FP4) {
+        // the scale reads of slot 0 have landed behind the wait of slot kAhead + 1; they become the
+        // constants of the step after this one (MXFP4: of its k block B, whose set the chunk being
+        // dequantised here does not use)
 #pragma unroll
         for (int c = 0; c < 4; ++c)
-          if (rb == (kAhead + 1 + c < RB ? kAhead + 1 + c : RB - 1)) make_col((R + 1) & 1, c);
-      } else if (rb < kWideOps) {
-        issue_one(kt + 3, (R + 3) & 3, rb);
+          if (rb == (kAhead + 1 + c < RB ? kAhead + 1 + c : RB - 1)) make_col(FP4 ? B : (R + 1) & 1, c);
       }
+      if (B == 1 && rb < kWideOps) issue_one(kt + 3, (R + 3) & 3, rb);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -1005,7 +1041,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   };
 
   // ---- prologue: the scale row of the first step, then what steps k_first - 3 .. k_first - 1 would have issued
-  issue_scales(k_first);
+  issue_scales(k_first, 0);
+  if (FP4) issue_scales(k_first, 1);
 #pragma unroll
   for (int idx = 0; idx < kWideOps; ++idx) issue_one(k_first, 0, idx);
 #pragma unroll
@@ -1014,13 +1051,19 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int idx = 0; idx < kWideOps; ++idx) issue_one(k_first + 2, 2, idx);
   asm volatile("s_waitcnt vmcnt(%2)" : "+v"(wq[0][0]), "+v"(wq[0][1]) : "n"(2 * kWideOps) : "memory");
   __builtin_amdgcn_s_barrier();
-  scales_start(k_first);
+  if (FP4) {   // the constants of k block 1 of the first step; those of k block 0 below
+    scales_start(k_first, 1);
+    asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw) : : "memory");
+#pragma unroll
+    for (int j = 0; j < 4; ++j) make_col(1, j);
+  }
+  scales_start(k_first, 0);
   asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw) : : "memory");
 #pragma unroll
   for (int j = 0; j < 4; ++j) make_col(0, j);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const u32x4_t w = __builtin_bit_cast(u32x4_t, Dq<T>::word(word_of(wq[0][0], j), cols[0][j], magic));
+    const u32x4_t w = __builtin_bit_cast(u32x4_t, D4::word(word_of(wq[0][0], j), cols[0][j], magic));
     wb[0][j][0] = w.x;
     wb[0][j][1] = w.y;
     wb[0][j][2] = w.z;
@@ -1269,6 +1312,18 @@ int launch_tile_wide_rows(const TileParams& p, hipStream_t st) {
   marlin_tile_wide_kernel<T, HAS_ZP, GROUPED, RB><<<tile_grid(p), 256, wide_lds(RB), st>>>(p);
   return SONAR_OK;
 }
+// MXFP4: bf16, groups of 32 rows, float4_e2m1f codes
+template <bool GROUPED>
+int launch_tile_wide_fp4(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<__bf16, false, GROUPED, 16, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
+    attr_set = true;
+  }
+  marlin_tile_wide_kernel<__bf16, false, GROUPED, 16, true><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
+  return SONAR_OK;
+}
 template <typename T, bool HAS_ZP, bool GROUPED = false>
 int launch_tile_wide(const TileParams& p, hipStream_t st) {
   if constexpr (!GROUPED) {
@@ -1326,6 +1381,12 @@ bool wide_applies(const TileParams& p) {
   if (p.num_groups == 1) return true;
   const int per_group = p.group_size / kTileK;   // steps per group: a power of two
   return p.group_size % kTileK == 0 && (per_group & (per_group - 1)) == 0;
+}
+// ... and for MXFP4 (groups of 32 rows, the caller has checked): the K ranges only.
+bool wide_applies_fp4(const TileParams& p) {
+  static const bool no_wide = getenv("SONAR_MARLIN_NO_WIDE_TILE") != nullptr;
+  const int k_steps = p.size_k / kTileK;
+  return !no_wide && k_steps % 4 == 0 && (p.k_splits == 1 || p.k_steps_per_split % 4 == 0) && p.tile_rows == kTileM;
 }
 }  // namespace
 
@@ -1409,7 +1470,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     if (nvfp4)
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16>(p, st) : launch_tile_async_nvfp4<__bf16>(p, st);
     else if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
-      rc = launch_tile_async_fp4(p, st);
+      rc = wide_applies_fp4(p) ? launch_tile_wide_fp4<false>(p, st) : launch_tile_async_fp4(p, st);
     else if (bits == 8)   // symmetric 8-bit codes: the caller has checked
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, false>(p, fp8, st)
                                     : launch_tile_async8<__bf16, false>(p, fp8, st);
@@ -1507,7 +1568,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
     rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16, true>(p, st)
                                   : launch_tile_async_nvfp4<__bf16, true>(p, st);
   else if (fp4)
-    rc = launch_tile_grouped_fp4(p, st);
+    rc = wide_applies_fp4(p) ? launch_tile_wide_fp4<true>(p, st) : launch_tile_grouped_fp4(p, st);
   else if (bits == 8)
     rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, true>(p, fp8, st)
                                   : launch_tile_async8<__bf16, true>(p, fp8, st);
