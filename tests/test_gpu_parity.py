@@ -241,6 +241,37 @@ def test_marlin_gemm_tiled_within_tolerance(gu, dtype, m, k, n, g, zp, act, bias
     assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
 
 
+WIDE_TILE_CASES = [
+    # m, k, n, group, zp, bias: the forms of the one-wavefront-per-SIMD tile kernel (K a multiple of 256,
+    # groups of 64 * 2^i rows or one group).  At most 128 tiles of 256 rows: 128-row tiles
+    (300, 256, 256, 64, False, False),        # one pass of the four-step loop
+    (300, 1024, 768, 128, True, True),        # 9 tiles of 128 rows, two ranges of K
+    (520, 2048, 512, 256, False, True),       # groups of four steps
+    (1100, 512, 1024, -1, True, False),       # channelwise, zero points, no split
+    (140, 8192, 256, 128, False, False),      # long K, eight ranges
+    # more than 128 tiles of 256 rows: 256-row tiles
+    (2100, 256, 4096, 64, True, True),        # 144 tiles, one pass of the loop
+    (2100, 1024, 4096, 128, False, False),
+    (2304, 512, 3840, -1, False, True),       # 9 x 15 tiles, the last column tile full
+    (2050, 1024, 4160, 128, True, False),     # a ragged last column tile (one strip) and a ragged last row tile
+    # K = 10240 > 8192 keeps 256-row tiles although there are few
+    (300, 10240, 512, 128, False, True),
+]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("m,k,n,g,zp,bias", WIDE_TILE_CASES)
+def test_wide_tile_kernel_forms_within_tolerance(gu, dtype, m, k, n, g, zp, bias):
+    layer = gu.DeviceLayer(77 + m + k, k, n, g, dtype, zero_points=zp, act_order=False, bias=bias)
+    a32 = mo.make_activations(m + 3, m, k, dtype, std=0.5)
+    a = gu.dev_bits16(a32, dtype)
+    c = layer.gemm(a, m)
+    ok, max_err, max_ref = mo.gemm_tolerance_ok(gu.host_f32(c), mo.gemm_reference(a32, layer.w_ref, layer.bias32))
+    assert ok, f"max_err={max_err} max_ref={max_ref}"
+    c2 = layer.gemm(a, m)
+    assert torch.equal(c.view(torch.int16), c2.view(torch.int16))   # split K is summed in a fixed order
+
+
 @pytest.mark.parametrize("dtype", ["fp16", "bf16"])
 @pytest.mark.parametrize("m,k,n", [(1, 4096, 11008), (16, 512, 256), (48, 1024, 512), (512, 4096, 1024)])
 def test_act_order_with_permuted_copy_of_a(gu, dtype, m, k, n):
