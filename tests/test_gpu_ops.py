@@ -930,6 +930,7 @@ def test_prepare_nvfp4_layer_and_apply(k, n, dtype):
     (5, 4, 2, 256, 128, False),
     (70, 4, 2, 256, 256, True),
     (200, 8, 2, 128, 128, False),
+    (700, 4, 2, 512, 256, True),     # 64-slot blocks, K a multiple of 256: the wide tile kernel's grouped MXFP4 form
 ], ids=str)
 def test_prepare_moe_mxfp4_layer_and_fused_marlin_moe(cfg):
     """MXFP4 expert weights (w13 (E, 2N, K/2), w2 (E, K, N/2) bytes, exponent-byte
