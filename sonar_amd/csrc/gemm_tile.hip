@@ -750,7 +750,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 // accumulator is touched again 64 MFMAs later, operands are written long before
 // they are read), and the results are read after the pipeline has drained
 // (s_nop below).
-// 4-bit integer codes with groups of 64 * 2^i rows or one group, or MXFP4 (float4_e2m1f codes,
+// 4-bit or symmetric 8-bit codes with groups of 64 * 2^i rows or one group, or MXFP4 (float4_e2m1f codes,
 // bf16, a scale per 32 rows: one hardware conversion and half a byte permute behind each row
 // block); K ranges of a multiple of four steps, no act-order; dense and grouped
 // (mixture-of-experts) calls.
@@ -761,20 +761,25 @@ constexpr int kWideScaleRows = 16;   // a ring of 16 rows per wavefront: eight s
 constexpr int wide_stage(int rb) { return rb * 2 * kBlockBytes; }                    // one stage of A
 constexpr int wide_a(int rb) { return kWideStages * wide_stage(rb); }                // 128 / 64 KiB
 constexpr int wide_lds(int rb) { return wide_a(rb) + 4 * kWideScaleRows * 256; }     // + the scale rows of four wavefronts
-// memory operations per wavefront and step: its blocks of A, the scale row (MXFP4: two, one per k block), two chunks
-constexpr int wide_ops(int rb, bool fp4 = false) { return rb / 2 + (fp4 ? 4 : 3); }
+// memory operations per wavefront and step: its blocks of A, the scale row (MXFP4: two, one per k block), two
+// chunks (8-bit codes: four blocks)
+constexpr int wide_ops(int rb, bool fp4 = false, bool w8 = false) { return rb / 2 + (fp4 ? 2 : 1) + (w8 ? 4 : 2); }
 
-template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16, bool FP4 = false>
+template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16, bool FP4 = false, int W8 = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void marlin_tile_wide_kernel(
     const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
   typedef typename Dq4Of<T, FP4>::type D4;   // integer codes, or float4_e2m1f with a scale per 32 rows (MXFP4: bf16)
-  typedef typename D4::Col Col;
+  typedef typename Dq8Of<T, W8 == 2>::type D8;   // 8-bit integer (W8 = 1) or floating-point (W8 = 2) codes
+  typedef typename std::conditional<W8 != 0, typename D8::Col, typename D4::Col>::type Col;
   typedef typename Dq<T>::Mid Mid;
+  static_assert(W8 == 0 || (!HAS_ZP && !FP4 && RB == 16), "8-bit codes: symmetric, 256-row tiles");
+  constexpr int kChunkLoads = W8 ? 2 : 1;   // 16-byte loads per lane and k block: 8-bit codes come as a block of
+                                            // the low four and a block of the high four of a lane's eight rows
   static_assert(!FP4 || (std::is_same<T, __bf16>::value && !HAS_ZP && RB == 16), "MXFP4: bf16, no zero points, 256-row tiles");
   static_assert(RB == 16 || (RB == 8 && !GROUPED), "256-row tiles, or 128-row tiles for dense calls");
   constexpr int kRows = 16 * RB;
-  constexpr int kStage = wide_stage(RB), kWideA = wide_a(RB), kWideOps = wide_ops(RB, FP4);
+  constexpr int kStage = wide_stage(RB), kWideA = wide_a(RB), kWideOps = wide_ops(RB, FP4, W8 != 0);
   constexpr int kAgprBlocks = RB == 16 ? 14 : RB;   // row blocks whose accumulators sit in AGPRs
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -837,7 +842,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     }
     a_src[i] = reinterpret_cast<const char*>(p.a) + ((long)row * p.lda + 8 * ((lane & 7) ^ r8)) * 2;
   }
-  const uint4* b_src = p.b + expert * p.expert_b_stride + (size_t)(unsigned)(strip * p.chunks_per_strip) * 64 + lane;
+  const uint4* b_src = p.b + expert * p.expert_b_stride +
+                       (size_t)(unsigned)(strip * p.chunks_per_strip) * (64 * kChunkLoads) + lane;
   const char* s_src;
   long s_group_stride;
   if (HAS_ZP && lane >= 32) {
@@ -857,7 +863,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const int k_first = whole_k ? 0 : split * p.k_steps_per_split;
   const int k_tiles = whole_k ? p.size_k / kTileK : min(p.size_k / kTileK, k_first + p.k_steps_per_split);
 
-  u32x4_t wq[kWideStages][2];   // packed chunks in flight or waiting
+  u32x4_t wq[kWideStages][2 * kChunkLoads];   // packed chunks in flight or waiting (8-bit: [2 b + h], h = high rows)
   // the scale row of step kt (clamped to the last step) into its ring position; MXFP4: the row of
   // k block h of the step (groups of 32 rows), ring position 2 (kt - k_first) + h
   auto issue_scales = [&](int kt, int h) __attribute__((always_inline)) {
@@ -879,7 +885,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       issue_scales(kt + 1, idx - RB / 2);
     } else {
       const int c = idx - RB / 2 - (FP4 ? 2 : 1);
-      const uint4* g = b_src + (size_t)(2 * k + c) * 64;
+      const uint4* g = b_src + (size_t)(2 * kChunkLoads * k + c) * 64;
       asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(wq[slot][c]) : "v"(g) : "memory");
     }
   };
@@ -932,7 +938,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const uint32_t sbits = j == 0 ? sb0 : j == 1 ? sb1 : j == 2 ? sb2 : sb3;
     int z = 8;
     if (HAS_ZP) z = (int)((zw >> zero_point_shift(16 * j + col16)) & 0xFu);
-    cols[set][j] = D4::make_col((uint16_t)sbits, z);
+    if constexpr (W8 != 0) cols[set][j] = D8::make_col((uint16_t)sbits);
+    else cols[set][j] = D4::make_col((uint16_t)sbits, z);
   };
   auto word_of = [](const u32x4_t& q, int j) __attribute__((always_inline)) -> uint32_t {
     return j == 0 ? q.x : j == 1 ? q.y : j == 2 ? q.z : q.w;
@@ -960,7 +967,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int set = FP4 ? NB : (B ? (R + 1) & 1 : R & 1);
     const uint32_t a_cur = a_base[B] + R * kStage;
     const uint32_t a_next = a_base[NB] + NR * kStage;
-    const u32x4_t& q4 = B ? wq[NR][0] : wq[R][1];
+    const u32x4_t& q4 = B ? wq[NR][0] : wq[R][kChunkLoads];                         // 8-bit: the low four rows
+    const u32x4_t& q4h = B ? wq[NR][kChunkLoads - 1] : wq[R][2 * kChunkLoads - 1];   // 8-bit: the high four rows
     constexpr int kPairs = 16 / RB;   // pairs of weights dequantised per row block
     uint32_t r_lo = 0;     // MXFP4: rows (0, 2) or (4, 6) of the word in hand, waiting for their odd partners
 #pragma unroll
@@ -979,7 +987,20 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       // the scales of the step after this one (MXFP4: of its k block B, two half steps ahead)
       if (rb == 0 && (B == 0 || FP4)) scales_start(kt + 1, B);
       const uint32_t qw = word_of(q4, j);
-      if constexpr (FP4) {
+      if constexpr (W8 != 0) {
+        // behind every second row block, half a column block (four rows of 16 columns) in one piece
+        mfma(B, 0, rb);
+        if ((rb & 1) == 0) {
+          const int jj = rb >> 2, half = (rb >> 1) & 1;
+          const uint2 w = D8::word4(word_of(half ? q4h : q4, jj), cols[set][jj], magic);
+          wb[NB][jj][2 * half] = w.x;
+          wb[NB][jj][2 * half + 1] = w.y;
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 1, rb);
+        mfma(B, 2, rb);
+        mfma(B, 3, rb);
+      } else if constexpr (FP4) {
         // one hardware conversion per row block (two rows of the column each: (0,2), (1,3), (4,6),
         // (5,7)); behind the second and the fourth, the two byte permutes that put four rows in order
         mfma(B, 0, rb);
@@ -1035,6 +1056,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                  : "+v"(wq[(R + 1) & 3][0]), "+v"(wq[(R + 1) & 3][1])
                  : "n"(kWideOps)
                  : "memory");
+    if constexpr (W8 != 0) asm volatile("" : "+v"(wq[(R + 1) & 3][2]), "+v"(wq[(R + 1) & 3][3]) : : "memory");
     __builtin_amdgcn_s_barrier();
     __builtin_amdgcn_sched_barrier(0);
     chunk(R, 1, kt);
@@ -1050,6 +1072,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #pragma unroll
   for (int idx = 0; idx < kWideOps; ++idx) issue_one(k_first + 2, 2, idx);
   asm volatile("s_waitcnt vmcnt(%2)" : "+v"(wq[0][0]), "+v"(wq[0][1]) : "n"(2 * kWideOps) : "memory");
+  if constexpr (W8 != 0) asm volatile("" : "+v"(wq[0][2]), "+v"(wq[0][3]) : : "memory");
   __builtin_amdgcn_s_barrier();
   if (FP4) {   // the constants of k block 1 of the first step; those of k block 0 below
     scales_start(k_first, 1);
@@ -1063,7 +1086,14 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int j = 0; j < 4; ++j) make_col(0, j);
 #pragma unroll
   for (int j = 0; j < 4; ++j) {
-    const u32x4_t w = __builtin_bit_cast(u32x4_t, D4::word(word_of(wq[0][0], j), cols[0][j], magic));
+    u32x4_t w;
+    if constexpr (W8 != 0) {
+      const uint2 lo = D8::word4(word_of(wq[0][0], j), cols[0][j], magic);
+      const uint2 hi = D8::word4(word_of(wq[0][1], j), cols[0][j], magic);
+      w = u32x4_t{lo.x, lo.y, hi.x, hi.y};
+    } else {
+      w = __builtin_bit_cast(u32x4_t, D4::word(word_of(wq[0][0], j), cols[0][j], magic));
+    }
     wb[0][j][0] = w.x;
     wb[0][j][1] = w.y;
     wb[0][j][2] = w.z;
@@ -1085,10 +1115,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   asm volatile("s_waitcnt vmcnt(0) lgkmcnt(0)\n\ts_nop 15\n\ts_nop 15" ::: "memory");
   // the registers those operations were still to fill stay untouched up to here
 #pragma unroll
-  for (int i = 0; i < kWideStages; ++i) {
-    asm volatile("" : "+v"(wq[i][0]) : : "memory");
-    asm volatile("" : "+v"(wq[i][1]) : : "memory");
-  }
+  for (int i = 0; i < kWideStages; ++i)
+#pragma unroll
+    for (int c = 0; c < 2 * kChunkLoads; ++c) asm volatile("" : "+v"(wq[i][c]) : : "memory");
 #pragma unroll
   for (int i = 0; i < 8; ++i) asm volatile("" : "+v"(av[i]) : : "memory");
   asm volatile("" : "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw) : : "memory");
@@ -1324,6 +1353,21 @@ int launch_tile_wide_fp4(const TileParams& p, hipStream_t st) {
   marlin_tile_wide_kernel<__bf16, false, GROUPED, 16, true><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
   return SONAR_OK;
 }
+// 8-bit codes: uint8b128 or float8_e4m3fn (groups of 64 * 2^i rows or one group)
+template <typename T, bool GROUPED>
+int launch_tile_wide8(const TileParams& p, bool fp8, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, false, GROUPED, 16, false, 1>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, false, GROUPED, 16, false, 2>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
+    attr_set = true;
+  }
+  if (fp8) marlin_tile_wide_kernel<T, false, GROUPED, 16, false, 2><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
+  else marlin_tile_wide_kernel<T, false, GROUPED, 16, false, 1><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
+  return SONAR_OK;
+}
 template <typename T, bool HAS_ZP, bool GROUPED = false>
 int launch_tile_wide(const TileParams& p, hipStream_t st) {
   if constexpr (!GROUPED) {
@@ -1471,6 +1515,9 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16>(p, st) : launch_tile_async_nvfp4<__bf16>(p, st);
     else if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
       rc = wide_applies_fp4(p) ? launch_tile_wide_fp4<false>(p, st) : launch_tile_async_fp4(p, st);
+    else if (bits == 8 && wide_applies(p) && p.tile_rows == kTileM)
+      rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide8<_Float16, false>(p, fp8, st)
+                                    : launch_tile_wide8<__bf16, false>(p, fp8, st);
     else if (bits == 8)   // symmetric 8-bit codes: the caller has checked
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, false>(p, fp8, st)
                                     : launch_tile_async8<__bf16, false>(p, fp8, st);
@@ -1569,6 +1616,9 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                                   : launch_tile_async_nvfp4<__bf16, true>(p, st);
   else if (fp4)
     rc = wide_applies_fp4(p) ? launch_tile_wide_fp4<true>(p, st) : launch_tile_grouped_fp4(p, st);
+  else if (bits == 8 && wide_applies(p))
+    rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide8<_Float16, true>(p, fp8, st)
+                                  : launch_tile_wide8<__bf16, true>(p, fp8, st);
   else if (bits == 8)
     rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, true>(p, fp8, st)
                                   : launch_tile_async8<__bf16, true>(p, fp8, st);
