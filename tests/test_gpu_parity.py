@@ -256,6 +256,9 @@ WIDE_TILE_CASES = [
     (2050, 1024, 4160, 128, True, False),     # a ragged last column tile (one strip) and a ragged last row tile
     # K = 10240 > 8192 keeps 256-row tiles although there are few
     (300, 10240, 512, 128, False, True),
+    # 65..128 rows with a long K: the tile kernel (256-row tiles, K split) instead of 64-row slabs
+    (100, 8192, 512, 128, False, True),
+    (128, 14336, 256, 128, True, False),
 ]
 
 
