@@ -753,7 +753,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 // 4-bit or symmetric 8-bit codes with groups of 64 * 2^i rows or one group, or MXFP4 (float4_e2m1f codes,
 // bf16, a scale per 32 rows: one hardware conversion and half a byte permute behind each row
 // block); K ranges of a multiple of four steps, no act-order; dense and grouped
-// (mixture-of-experts) calls.
+// (mixture-of-experts) calls.  K ranges that are not a multiple of four steps are padded with
+// steps of zeros (taken only where that is a small part of the range).
 constexpr int kWideStages = 4;
 constexpr int kWideScaleRows = 16;   // a ring of 16 rows per wavefront: eight steps of one row, or of two (MXFP4)
 // RB: row blocks of 16 rows a wavefront owns: 16 (a 256-row tile) or 8 (a 128-row tile, for
@@ -764,6 +765,11 @@ constexpr int wide_lds(int rb) { return wide_a(rb) + 4 * kWideScaleRows * 256; }
 // memory operations per wavefront and step: its blocks of A, the scale row (MXFP4: two, one per k block), two
 // chunks (8-bit codes: four blocks)
 constexpr int wide_ops(int rb, bool fp4 = false, bool w8 = false) { return rb / 2 + (fp4 ? 2 : 1) + (w8 ? 4 : 2); }
+
+// One 128-byte line of zeros: what the copies of A fetch for the steps past the end of a K range that
+// is not a multiple of four steps (the loop always runs whole passes of four; those steps then add
+// zeros times the last step's weights).
+__device__ __attribute__((aligned(128))) const uint32_t kWideZeroLine[32] = {};
 
 template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16, bool FP4 = false, int W8 = 0>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void marlin_tile_wide_kernel(
@@ -878,7 +884,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   auto issue_one = [&](int kt, int slot, int idx) __attribute__((always_inline)) {
     const int k = min(kt, k_tiles - 1);
     if (idx < RB / 2) {
-      __builtin_amdgcn_global_load_lds((glb_void_t*)(a_src[idx] + (long)k * (kTileK * 2)),
+      // (the comparison is uniform: a pair of selects per copy)
+      const char* src = kt < k_tiles ? a_src[idx] + (long)k * (kTileK * 2)
+                                     : reinterpret_cast<const char*>(kWideZeroLine) + 16 * (lane & 7);
+      __builtin_amdgcn_global_load_lds((glb_void_t*)src,
                                        (lds_void_t*)(smem + slot * kStage + ((RB / 2) * wave + idx) * kBlockBytes),
                                        16, 0, 0);
     } else if (idx < RB / 2 + (FP4 ? 2 : 1)) {
@@ -1103,7 +1112,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   for (int rb = 0; rb < kAhead; ++rb) SONAR_WIDE_READ(av[rb], a_base[0], rb * 2048);
   __builtin_amdgcn_sched_barrier(0);
 
-  // the host gives this kernel K ranges of a multiple of four steps (the ring positions are static)
+  // whole passes of four steps (the ring positions are static); steps past the end of the range
+  // multiply zeros
   for (int kt = k_first; kt < k_tiles; kt += 4) {
     step(0, kt);
     step(1, kt + 1);
@@ -1416,12 +1426,15 @@ int launch_tile(const TileParams& p, hipStream_t st) {
 }  // namespace
 
 namespace {
-// The wide form: K ranges of a multiple of four steps, groups of 64 * 2^i rows or one group.
+// The wide form: groups of 64 * 2^i rows or one group; K ranges of a multiple of four steps, or long ones.
+// Steps of zeros the wide kernel adds to a K range of `range` steps (at most a tenth of the range is accepted).
+int wide_padding(int range) { return (4 - range % 4) % 4; }
 bool wide_applies(const TileParams& p) {
   static const bool no_wide = getenv("SONAR_MARLIN_NO_WIDE_TILE") != nullptr;   // debugging aid
   if (no_wide) return false;
-  const int k_steps = p.size_k / kTileK;
-  if (k_steps % 4 != 0 || (p.k_splits > 1 && p.k_steps_per_split % 4 != 0)) return false;
+  // K ranges are rounded up to four steps with steps of zeros: not where that is a large part of the work
+  const int range = p.k_splits > 1 ? p.k_steps_per_split : p.size_k / kTileK;
+  if (wide_padding(range) * 10 > range) return false;
   if (p.num_groups == 1) return true;
   const int per_group = p.group_size / kTileK;   // steps per group: a power of two
   return p.group_size % kTileK == 0 && (per_group & (per_group - 1)) == 0;
@@ -1429,8 +1442,10 @@ bool wide_applies(const TileParams& p) {
 // ... and for MXFP4 (groups of 32 rows, the caller has checked): the K ranges only.
 bool wide_applies_fp4(const TileParams& p) {
   static const bool no_wide = getenv("SONAR_MARLIN_NO_WIDE_TILE") != nullptr;
-  const int k_steps = p.size_k / kTileK;
-  return !no_wide && k_steps % 4 == 0 && (p.k_splits == 1 || p.k_steps_per_split % 4 == 0) && p.tile_rows == kTileM;
+  const int range = p.k_splits > 1 ? p.k_steps_per_split : p.size_k / kTileK;
+  // (no padding here: the eight-wavefront kernel is as fast on these codes, and ahead once steps are wasted:
+  // K = 2880, N = 5760, M = 4096: 143 us against 156)
+  return !no_wide && wide_padding(range) == 0 && p.tile_rows == kTileM;
 }
 }  // namespace
 

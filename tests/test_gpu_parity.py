@@ -256,6 +256,9 @@ WIDE_TILE_CASES = [
     (2050, 1024, 4160, 128, True, False),     # a ragged last column tile (one strip) and a ragged last row tile
     # K = 10240 > 8192 keeps 256-row tiles although there are few
     (300, 10240, 512, 128, False, True),
+    # K ranges that are not a multiple of four steps: padded with steps of zeros
+    (2100, 2880, 4096, 64, False, True),      # 45 steps, one range
+    (520, 1344, 5120, 64, True, False),       # 21 steps in two ranges of 11 and 10 (128-row tiles)
     # 65..128 rows with a long K: the tile kernel (256-row tiles, K split) instead of 64-row slabs
     (100, 8192, 512, 128, False, True),
     (128, 14336, 256, 128, True, False),
