@@ -728,7 +728,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 // rows of the tile).  A chunk of weights is dequantised once per workgroup
 // instead of once per group of rows and feeds 64 MFMAs; with no second
 // wavefront on the SIMD the other work (dequantising the next chunk, the LDS
-// reads of A two row blocks ahead, the copies of a later stage) sits between
+// reads of A four row blocks ahead, the copies of a later stage) sits between
 // the MFMAs of the wavefront's own instruction stream, one to two instructions
 // behind each MFMA, where the matrix pipeline hides them.
 //   * A: a ring of four 32-KiB stages filled by LDS-DMA, wavefront w copying
@@ -736,7 +736,7 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 //   * W: the two chunks of a step go from memory straight into registers (one
 //     16-byte load per lane and chunk), a ring of four register sets.
 //   * scales / zero points: one 256-byte row per step through a private LDS
-//     ring of eight rows, fetched a step earlier than the rest.
+//     ring of sixteen rows, fetched a step earlier than the rest.
 // The eleven memory operations a wavefront issues per step (8 + 1 + 2: stage
 // kt + 3 of A and W, the scale row of step kt + 4) go out in the second half of
 // step kt.  One barrier per step, between its halves: before it a wavefront
@@ -752,9 +752,9 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 // (s_nop below).
 // 4-bit or symmetric 8-bit codes with groups of 64 * 2^i rows or one group, or MXFP4 (float4_e2m1f codes,
 // bf16, a scale per 32 rows: one hardware conversion and half a byte permute behind each row
-// block); K ranges of a multiple of four steps, no act-order; dense and grouped
-// (mixture-of-experts) calls.  K ranges that are not a multiple of four steps are padded with
-// steps of zeros (taken only where that is a small part of the range).
+// block); no act-order; dense and grouped (mixture-of-experts) calls.  K ranges that are not a
+// multiple of four steps are padded with steps of zeros (integer codes; taken only where that
+// is a small part of the range).
 constexpr int kWideStages = 4;
 constexpr int kWideScaleRows = 16;   // a ring of 16 rows per wavefront: eight steps of one row, or of two (MXFP4)
 // RB: row blocks of 16 rows a wavefront owns: 16 (a 256-row tile) or 8 (a 128-row tile, for
