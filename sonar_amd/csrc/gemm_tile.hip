@@ -750,13 +750,14 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 // accumulator is touched again 64 MFMAs later, operands are written long before
 // they are read), and the results are read after the pipeline has drained
 // (s_nop below).
-// 4-bit or symmetric 8-bit codes with groups of 64 * 2^i rows or one group, or MXFP4 (float4_e2m1f codes,
+// 4-bit or symmetric 8-bit codes with groups of 64 * 2^i rows or one group, MXFP4 (float4_e2m1f codes,
 // bf16, a scale per 32 rows: one hardware conversion and half a byte permute behind each row
-// block); no act-order; dense and grouped (mixture-of-experts) calls.  K ranges that are not a
+// block), or 8-bit codes with a scale per 32 rows (MXFP8); no act-order; dense and grouped
+// (mixture-of-experts) calls.  K ranges that are not a
 // multiple of four steps are padded with steps of zeros (integer codes; taken only where that
 // is a small part of the range).
 constexpr int kWideStages = 4;
-constexpr int kWideScaleRows = 16;   // a ring of 16 rows per wavefront: eight steps of one row, or of two (MXFP4)
+constexpr int kWideScaleRows = 16;   // a ring of 16 rows per wavefront: eight steps of one row, or of two (groups of 32 rows)
 // RB: row blocks of 16 rows a wavefront owns: 16 (a 256-row tile) or 8 (a 128-row tile, for
 // calls with few tiles: twice the tiles, half the K ranges and half the partial-tile traffic).
 constexpr int wide_stage(int rb) { return rb * 2 * kBlockBytes; }                    // one stage of A
@@ -771,7 +772,8 @@ constexpr int wide_ops(int rb, bool fp4 = false, bool w8 = false) { return rb / 
 // zeros times the last step's weights).
 __device__ __attribute__((aligned(128))) const uint32_t kWideZeroLine[32] = {};
 
-template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16, bool FP4 = false, int W8 = 0>
+// G32: a scale per 32 rows (one row of scales per k block): MXFP4 always, 8-bit codes when asked (MXFP8)
+template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16, bool FP4 = false, int W8 = 0, bool G32 = FP4>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void marlin_tile_wide_kernel(
     const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
@@ -780,12 +782,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   typedef typename std::conditional<W8 != 0, typename D8::Col, typename D4::Col>::type Col;
   typedef typename Dq<T>::Mid Mid;
   static_assert(W8 == 0 || (!HAS_ZP && !FP4 && RB == 16), "8-bit codes: symmetric, 256-row tiles");
+  static_assert(G32 == FP4 || (G32 && W8 != 0), "groups of 32 rows: MXFP4 and 8-bit codes");
   constexpr int kChunkLoads = W8 ? 2 : 1;   // 16-byte loads per lane and k block: 8-bit codes come as a block of
                                             // the low four and a block of the high four of a lane's eight rows
   static_assert(!FP4 || (std::is_same<T, __bf16>::value && !HAS_ZP && RB == 16), "MXFP4: bf16, no zero points, 256-row tiles");
   static_assert(RB == 16 || (RB == 8 && !GROUPED), "256-row tiles, or 128-row tiles for dense calls");
   constexpr int kRows = 16 * RB;
-  constexpr int kStage = wide_stage(RB), kWideA = wide_a(RB), kWideOps = wide_ops(RB, FP4, W8 != 0);
+  constexpr int kStage = wide_stage(RB), kWideA = wide_a(RB), kWideOps = wide_ops(RB, G32, W8 != 0);
   constexpr int kAgprBlocks = RB == 16 ? 14 : RB;   // row blocks whose accumulators sit in AGPRs
   extern __shared__ __attribute__((aligned(1024))) char smem[];
 
@@ -874,8 +877,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // k block h of the step (groups of 32 rows), ring position 2 (kt - k_first) + h
   auto issue_scales = [&](int kt, int h) __attribute__((always_inline)) {
     const int k = min(kt, k_tiles - 1);
-    const int grp = FP4 ? 2 * k + h : (grouped ? k >> group_shift : 0);
-    const int at = FP4 ? 2 * (kt - k_first) + h : kt - k_first;
+    const int grp = G32 ? 2 * k + h : (grouped ? k >> group_shift : 0);
+    const int at = G32 ? 2 * (kt - k_first) + h : kt - k_first;
     __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)grp * s_group_stride),
                                      (lds_void_t*)(sring + (at & (kWideScaleRows - 1)) * 256), 4, 0, 0);
   };
@@ -890,10 +893,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       __builtin_amdgcn_global_load_lds((glb_void_t*)src,
                                        (lds_void_t*)(smem + slot * kStage + ((RB / 2) * wave + idx) * kBlockBytes),
                                        16, 0, 0);
-    } else if (idx < RB / 2 + (FP4 ? 2 : 1)) {
+    } else if (idx < RB / 2 + (G32 ? 2 : 1)) {
       issue_scales(kt + 1, idx - RB / 2);
     } else {
-      const int c = idx - RB / 2 - (FP4 ? 2 : 1);
+      const int c = idx - RB / 2 - (G32 ? 2 : 1);
       const uint4* g = b_src + (size_t)(2 * kChunkLoads * k + c) * 64;
       asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(wq[slot][c]) : "v"(g) : "memory");
     }
@@ -932,7 +935,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #define SONAR_WIDE_LANDED(n, reg) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(reg) : "n"(n) : "memory")
 
   auto scales_start = [&](int kt, int h) __attribute__((always_inline)) {
-    const uint32_t r_at = s_lds + ((FP4 ? 2 * (kt - k_first) + h : kt - k_first) & (kWideScaleRows - 1)) * 256;
+    const uint32_t r_at = s_lds + ((G32 ? 2 * (kt - k_first) + h : kt - k_first) & (kWideScaleRows - 1)) * 256;
     asm volatile(
         "ds_read_u16 %0, %5\n\t"
         "ds_read_u16 %1, %6\n\t"
@@ -973,7 +976,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const int NR = B ? (R + 1) & 3 : R;   // stage and k block of the half step after this one
     const int NB = B ^ 1;
     // constants of the step the next half step belongs to (MXFP4: of the next k block)
-    const int set = FP4 ? NB : (B ? (R + 1) & 1 : R & 1);
+    const int set = G32 ? NB : (B ? (R + 1) & 1 : R & 1);
     const uint32_t a_cur = a_base[B] + R * kStage;
     const uint32_t a_next = a_base[NB] + NR * kStage;
     const u32x4_t& q4 = B ? wq[NR][0] : wq[R][kChunkLoads];                         // 8-bit: the low four rows
@@ -985,16 +988,16 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       const int j = (kPairs * rb) >> 2, part = (kPairs * rb) & 3;
       // reads started after the one of this row block: those of the next kAhead - 1 row blocks,
       // and the five scale reads of slot 0 (first half; MXFP4: either half)
-      if ((B == 0 || FP4) && rb >= 1 && rb <= kAhead) SONAR_WIDE_LANDED(kAhead - 1 + 5, av[rb & 7]);
+      if ((B == 0 || G32) && rb >= 1 && rb <= kAhead) SONAR_WIDE_LANDED(kAhead - 1 + 5, av[rb & 7]);
       else SONAR_WIDE_LANDED(kAhead - 1, av[rb & 7]);
       // behind this wait the scale reads of slot 0 have landed: from here on the registers they fill
       // hold the scales (without this the compiler is free to use them any time after slot 0)
-      if ((B == 0 || FP4) && rb == (kAhead + 1 < RB ? kAhead + 1 : RB - 1))
+      if ((B == 0 || G32) && rb == (kAhead + 1 < RB ? kAhead + 1 : RB - 1))
         asm volatile("" : "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw) : : "memory");
       if (rb + kAhead < RB) SONAR_WIDE_READ(av[(rb + kAhead) & 7], a_cur, (rb + kAhead) * 2048);
       else SONAR_WIDE_READ(av[(rb + kAhead) & 7], a_next, (rb + kAhead - RB) * 2048);
       // the scales of the step after this one (MXFP4: of its k block B, two half steps ahead)
-      if (rb == 0 && (B == 0 || FP4)) scales_start(kt + 1, B);
+      if (rb == 0 && (B == 0 || G32)) scales_start(kt + 1, B);
       const uint32_t qw = word_of(q4, j);
       if constexpr (W8 != 0) {
         // behind every second row block, half a column block (four rows of 16 columns) in one piece
@@ -1045,13 +1048,13 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         __builtin_amdgcn_sched_barrier(0);
         mfma(B, 3, rb);
       }
-      if (B == 0 || FP4) {
+      if (B == 0 || G32) {
         // the scale reads of slot 0 have landed behind the wait of slot kAhead + 1; they become the
         // constants of the step after this one (MXFP4: of its k block B, whose set the chunk being
         // dequantised here does not use)
 #pragma unroll
         for (int c = 0; c < 4; ++c)
-          if (rb == (kAhead + 1 + c < RB ? kAhead + 1 + c : RB - 1)) make_col(FP4 ? B : (R + 1) & 1, c);
+          if (rb == (kAhead + 1 + c < RB ? kAhead + 1 + c : RB - 1)) make_col(G32 ? B : (R + 1) & 1, c);
       }
       if (B == 1 && rb < kWideOps) issue_one(kt + 3, (R + 3) & 3, rb);
       __builtin_amdgcn_sched_barrier(0);
@@ -1073,7 +1076,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
   // ---- prologue: the scale row of the first step, then what steps k_first - 3 .. k_first - 1 would have issued
   issue_scales(k_first, 0);
-  if (FP4) issue_scales(k_first, 1);
+  if (G32) issue_scales(k_first, 1);
 #pragma unroll
   for (int idx = 0; idx < kWideOps; ++idx) issue_one(k_first, 0, idx);
 #pragma unroll
@@ -1083,7 +1086,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   asm volatile("s_waitcnt vmcnt(%2)" : "+v"(wq[0][0]), "+v"(wq[0][1]) : "n"(2 * kWideOps) : "memory");
   if constexpr (W8 != 0) asm volatile("" : "+v"(wq[0][2]), "+v"(wq[0][3]) : : "memory");
   __builtin_amdgcn_s_barrier();
-  if (FP4) {   // the constants of k block 1 of the first step; those of k block 0 below
+  if (G32) {   // the constants of k block 1 of the first step; those of k block 0 below
     scales_start(k_first, 1);
     asm volatile("s_waitcnt lgkmcnt(0)" : "+v"(sb0), "+v"(sb1), "+v"(sb2), "+v"(sb3), "+v"(zw) : : "memory");
 #pragma unroll
@@ -1363,20 +1366,26 @@ int launch_tile_wide_fp4(const TileParams& p, hipStream_t st) {
   marlin_tile_wide_kernel<__bf16, false, GROUPED, 16, true><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
   return SONAR_OK;
 }
-// 8-bit codes: uint8b128 or float8_e4m3fn (groups of 64 * 2^i rows or one group)
-template <typename T, bool GROUPED>
-int launch_tile_wide8(const TileParams& p, bool fp8, hipStream_t st) {
+// 8-bit codes: uint8b128 or float8_e4m3fn (groups of 64 * 2^i rows or one group; G32: of 32 rows, MXFP8)
+inline bool wide8_groups_of_32(const TileParams& p) { return p.num_groups > 1 && p.group_size == 32; }
+template <typename T, bool GROUPED, int W8, bool G32>
+int launch_tile_wide8_groups(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, false, GROUPED, 16, false, 1>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, false, GROUPED, 16, false, 2>,
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, false, GROUPED, 16, false, W8, G32>,
                                   hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
     attr_set = true;
   }
-  if (fp8) marlin_tile_wide_kernel<T, false, GROUPED, 16, false, 2><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
-  else marlin_tile_wide_kernel<T, false, GROUPED, 16, false, 1><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
+  marlin_tile_wide_kernel<T, false, GROUPED, 16, false, W8, G32><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
   return SONAR_OK;
+}
+template <typename T, bool GROUPED>
+int launch_tile_wide8(const TileParams& p, bool fp8, hipStream_t st) {
+  const bool g32 = wide8_groups_of_32(p);
+  if (fp8) return g32 ? launch_tile_wide8_groups<T, GROUPED, 2, true>(p, st)
+                      : launch_tile_wide8_groups<T, GROUPED, 2, false>(p, st);
+  return g32 ? launch_tile_wide8_groups<T, GROUPED, 1, true>(p, st)
+             : launch_tile_wide8_groups<T, GROUPED, 1, false>(p, st);
 }
 template <typename T, bool HAS_ZP, bool GROUPED = false>
 int launch_tile_wide(const TileParams& p, hipStream_t st) {
@@ -1447,6 +1456,10 @@ bool wide_applies_fp4(const TileParams& p) {
   // K = 2880, N = 5760, M = 4096: 143 us against 156)
   return !no_wide && wide_padding(range) == 0 && p.tile_rows == kTileM;
 }
+// ... and for 8-bit codes: groups of 32 rows under the rule of MXFP4, other groups under that of the 4-bit codes.
+bool wide_applies8(const TileParams& p) {
+  return p.tile_rows == kTileM && (wide8_groups_of_32(p) ? wide_applies_fp4(p) : wide_applies(p));
+}
 }  // namespace
 
 // The asynchronous tile kernel needs groups of 32 rows or a multiple of 64 and no gather of A.
@@ -1493,7 +1506,8 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   int rc;
   static const bool no_async = getenv("SONAR_MARLIN_NO_ASYNC_TILE") != nullptr;  // debugging aid
   const bool nvfp4 = fp4 && global_scale != nullptr;   // the caller has checked: groups of 16 rows
-  if ((nvfp4 || tile_async_applies(pm, num_groups, group_size)) && (!no_async || fp4)) {   // float4 codes exist here only
+  if ((nvfp4 || tile_async_applies(pm, num_groups, group_size)) &&
+      (!no_async || fp4 || bits == 8)) {   // float4 and 8-bit codes exist here only
     GemmPlan plan = plan_gemm(size_m, size_n, size_k, true);
     // few tiles and a call the wide kernel takes: 128-row tiles
     static const bool no_128 = getenv("SONAR_MARLIN_NO_128_ROW_TILES") != nullptr;   // debugging aid
@@ -1530,7 +1544,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16>(p, st) : launch_tile_async_nvfp4<__bf16>(p, st);
     else if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
       rc = wide_applies_fp4(p) ? launch_tile_wide_fp4<false>(p, st) : launch_tile_async_fp4(p, st);
-    else if (bits == 8 && wide_applies(p) && p.tile_rows == kTileM)
+    else if (bits == 8 && wide_applies8(p))
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide8<_Float16, false>(p, fp8, st)
                                     : launch_tile_wide8<__bf16, false>(p, fp8, st);
     else if (bits == 8)   // symmetric 8-bit codes: the caller has checked
@@ -1631,7 +1645,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                                   : launch_tile_async_nvfp4<__bf16, true>(p, st);
   else if (fp4)
     rc = wide_applies_fp4(p) ? launch_tile_wide_fp4<true>(p, st) : launch_tile_grouped_fp4(p, st);
-  else if (bits == 8 && wide_applies(p))
+  else if (bits == 8 && wide_applies8(p))
     rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide8<_Float16, true>(p, fp8, st)
                                   : launch_tile_wide8<__bf16, true>(p, fp8, st);
   else if (bits == 8)

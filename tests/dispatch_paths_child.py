@@ -66,6 +66,17 @@ def dense_mxfp4() -> None:
             sys.exit(1)
 
 
+def dense_8bit() -> None:
+    """8-bit codes on both tile kernels: one group, groups of 128 and of 32 rows (the test
+    functions raise on a mismatch)."""
+    from tests import test_gpu_parity as tp
+    for (dtype, m, k, n, g) in [("bf16", 1024, 1024, 832, 32), ("fp16", 700, 1280, 4160, 32),
+                                ("fp16", 300, 2048, 512, 128), ("bf16", 260, 1024, 4160, -1)]:
+        tp.test_fp8_weights_dequant_bit_exact_and_gemm_within_tolerance(gu, dtype, m, k, n, g, True)
+        tp.test_w8a16_dequant_bit_exact_and_gemm_within_tolerance(gu, dtype, m, k, n, g, False, False)
+        print("8-bit", dtype, m, k, n, g, "ok", flush=True)
+
+
 def grouped() -> None:
     from tests import test_gpu_moe as tm
     for case in [(300, 4, 2, 256, 256, 128, "fp16", False, False, False, 64, True),
@@ -81,5 +92,6 @@ def grouped() -> None:
 if __name__ == "__main__":
     dense()
     dense_mxfp4()
+    dense_8bit()
     grouped()
     print("all paths ok", flush=True)

@@ -1052,11 +1052,13 @@ def test_prepare_mxfp8_layer_and_apply(m, k, n):
                                      layer.workspace, n, k, None)
 
 
-@pytest.mark.parametrize("cfg", [(5, 4, 2, 256, 128), (70, 4, 2, 256, 256), (9, 4, 2, 256, 96)], ids=str)
+@pytest.mark.parametrize("cfg", [(5, 4, 2, 256, 128), (70, 4, 2, 256, 256), (9, 4, 2, 256, 96),
+                                 (700, 4, 2, 512, 256)], ids=str)
 def test_prepare_mxfp8_moe_layer_and_fused_marlin_moe(cfg):
     """MXFP8 expert weights -> prepare_mxfp8_moe_layer_for_marlin -> fused_marlin_moe,
     against the per-token reference on the same bytes (the third case pads the
-    intermediate size 96 -> 128)."""
+    intermediate size 96 -> 128; the fourth runs on 64-slot blocks: the tile kernels'
+    grouped form)."""
     from sonar_amd import marlin_utils_fp8 as f8
     from sonar_amd.fused_moe import fused_marlin_moe
     from sonar_amd.scalar_type import scalar_types

@@ -387,6 +387,9 @@ W8_CASES = [
     (260, 1024, 4160, -1, False, False),     # one group
     (512, 2048, 320, 32, False, True),       # groups of 32 rows
     (300, 2048, 512, 128, True, False),      # act-order through the permuted copy of A
+    (1024, 1024, 832, 32, False, False),     # groups of 32 rows, whole tiles over all of K
+    (700, 1280, 4160, 32, False, True),      # ... K ranges of 20 steps, ragged tiles both ways
+    (300, 1216, 512, 32, False, False),      # ... 19 steps: not a multiple of four (the eight-wavefront kernel)
 ]
 
 
@@ -468,6 +471,9 @@ FP8_CASES = [
     (300, 2048, 512, 128, True),
     (1024, 1024, 832, -1, False),
     (512, 2048, 320, 32, True),
+    (1024, 1024, 832, 32, False),     # groups of 32 rows, whole tiles over all of K
+    (700, 1280, 4160, 32, True),      # ... K ranges of 20 steps, ragged tiles both ways
+    (300, 1216, 512, 32, False),      # ... 19 steps: not a multiple of four (the eight-wavefront kernel)
 ]
 
 
