@@ -752,8 +752,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 // (s_nop below).
 // 4-bit or symmetric 8-bit codes with groups of 64 * 2^i rows or one group, MXFP4 (float4_e2m1f codes,
 // bf16, a scale per 32 rows: one hardware conversion and half a byte permute behind each row
-// block), or 8-bit codes with a scale per 32 rows (MXFP8); no act-order; dense and grouped
-// (mixture-of-experts) calls.  K ranges that are not a
+// block), or integer / 8-bit floating-point codes with a scale per 32 rows (MXFP8 among them); no
+// act-order; dense and grouped (mixture-of-experts) calls.  K ranges that are not a
 // multiple of four steps are padded with steps of zeros (integer codes; taken only where that
 // is a small part of the range).
 constexpr int kWideStages = 4;
@@ -772,7 +772,7 @@ constexpr int wide_ops(int rb, bool fp4 = false, bool w8 = false) { return rb / 
 // zeros times the last step's weights).
 __device__ __attribute__((aligned(128))) const uint32_t kWideZeroLine[32] = {};
 
-// G32: a scale per 32 rows (one row of scales per k block): MXFP4 always, 8-bit codes when asked (MXFP8)
+// G32: a scale (and zero point) per 32 rows, i.e. one row of them per k block: MXFP4 always, integer codes when asked
 template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16, bool FP4 = false, int W8 = 0, bool G32 = FP4>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void marlin_tile_wide_kernel(
     const TileParams p) {
@@ -782,7 +782,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   typedef typename std::conditional<W8 != 0, typename D8::Col, typename D4::Col>::type Col;
   typedef typename Dq<T>::Mid Mid;
   static_assert(W8 == 0 || (!HAS_ZP && !FP4 && RB == 16), "8-bit codes: symmetric, 256-row tiles");
-  static_assert(G32 == FP4 || (G32 && W8 != 0), "groups of 32 rows: MXFP4 and 8-bit codes");
+  static_assert(!FP4 || G32, "MXFP4 has a scale per 32 rows");
+  static_assert(!G32 || RB == 16, "groups of 32 rows: 256-row tiles");
   constexpr int kChunkLoads = W8 ? 2 : 1;   // 16-byte loads per lane and k block: 8-bit codes come as a block of
                                             // the low four and a block of the high four of a lane's eight rows
   static_assert(!FP4 || (std::is_same<T, __bf16>::value && !HAS_ZP && RB == 16), "MXFP4: bf16, no zero points, 256-row tiles");
@@ -1367,7 +1368,7 @@ int launch_tile_wide_fp4(const TileParams& p, hipStream_t st) {
   return SONAR_OK;
 }
 // 8-bit codes: uint8b128 or float8_e4m3fn (groups of 64 * 2^i rows or one group; G32: of 32 rows, MXFP8)
-inline bool wide8_groups_of_32(const TileParams& p) { return p.num_groups > 1 && p.group_size == 32; }
+inline bool wide_groups_of_32(const TileParams& p) { return p.num_groups > 1 && p.group_size == 32; }
 template <typename T, bool GROUPED, int W8, bool G32>
 int launch_tile_wide8_groups(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
@@ -1381,14 +1382,27 @@ int launch_tile_wide8_groups(const TileParams& p, hipStream_t st) {
 }
 template <typename T, bool GROUPED>
 int launch_tile_wide8(const TileParams& p, bool fp8, hipStream_t st) {
-  const bool g32 = wide8_groups_of_32(p);
+  const bool g32 = wide_groups_of_32(p);
   if (fp8) return g32 ? launch_tile_wide8_groups<T, GROUPED, 2, true>(p, st)
                       : launch_tile_wide8_groups<T, GROUPED, 2, false>(p, st);
   return g32 ? launch_tile_wide8_groups<T, GROUPED, 1, true>(p, st)
              : launch_tile_wide8_groups<T, GROUPED, 1, false>(p, st);
 }
+// 4-bit integer codes with groups of 32 rows
+template <typename T, bool HAS_ZP, bool GROUPED>
+int launch_tile_wide_g32(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, HAS_ZP, GROUPED, 16, false, 0, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
+    attr_set = true;
+  }
+  marlin_tile_wide_kernel<T, HAS_ZP, GROUPED, 16, false, 0, true><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
+  return SONAR_OK;
+}
 template <typename T, bool HAS_ZP, bool GROUPED = false>
 int launch_tile_wide(const TileParams& p, hipStream_t st) {
+  if (wide_groups_of_32(p)) return launch_tile_wide_g32<T, HAS_ZP, GROUPED>(p, st);
   if constexpr (!GROUPED) {
     if (p.tile_rows == 128) return launch_tile_wide_rows<T, HAS_ZP, false, 8>(p, st);
   }
@@ -1436,6 +1450,7 @@ int launch_tile(const TileParams& p, hipStream_t st) {
 
 namespace {
 // The wide form: groups of 64 * 2^i rows or one group; K ranges of a multiple of four steps, or long ones.
+// Groups of 32 rows: 256-row tiles and whole passes only.
 // Steps of zeros the wide kernel adds to a K range of `range` steps (at most a tenth of the range is accepted).
 int wide_padding(int range) { return (4 - range % 4) % 4; }
 bool wide_applies(const TileParams& p) {
@@ -1443,6 +1458,7 @@ bool wide_applies(const TileParams& p) {
   if (no_wide) return false;
   // K ranges are rounded up to four steps with steps of zeros: not where that is a large part of the work
   const int range = p.k_splits > 1 ? p.k_steps_per_split : p.size_k / kTileK;
+  if (wide_groups_of_32(p)) return wide_padding(range) == 0 && p.tile_rows == kTileM;
   if (wide_padding(range) * 10 > range) return false;
   if (p.num_groups == 1) return true;
   const int per_group = p.group_size / kTileK;   // steps per group: a power of two
@@ -1456,10 +1472,8 @@ bool wide_applies_fp4(const TileParams& p) {
   // K = 2880, N = 5760, M = 4096: 143 us against 156)
   return !no_wide && wide_padding(range) == 0 && p.tile_rows == kTileM;
 }
-// ... and for 8-bit codes: groups of 32 rows under the rule of MXFP4, other groups under that of the 4-bit codes.
-bool wide_applies8(const TileParams& p) {
-  return p.tile_rows == kTileM && (wide8_groups_of_32(p) ? wide_applies_fp4(p) : wide_applies(p));
-}
+// ... and for 8-bit codes: 256-row tiles only.
+bool wide_applies8(const TileParams& p) { return p.tile_rows == kTileM && wide_applies(p); }
 }  // namespace
 
 // The asynchronous tile kernel needs groups of 32 rows or a multiple of 64 and no gather of A.
@@ -1514,6 +1528,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     if (!no_128 && bits == 4 && !fp4 && plan_prefers_128_rows(size_m, size_n, size_k)) {
       const GemmPlan plan128 = plan_gemm(size_m, size_n, size_k, true, 128);
       TileParams probe = p;
+      probe.tile_rows = 128;
       probe.k_splits = plan128.k_splits;
       probe.k_steps_per_split = plan128.k_steps_per_split;
       if (plan128.tile && wide_applies(probe) &&

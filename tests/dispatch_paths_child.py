@@ -26,6 +26,7 @@ DENSE = [
     (600, 1024, 768, 64, "fp16", True, False),
     (1100, 512, 1024, -1, "bf16", False, False),
     (2100, 512, 4096, 128, "bf16", True, True),     # 144 tiles of 256 rows: the wide tile kernel's 256-row form
+    (600, 1024, 768, 32, "fp16", True, False),      # groups of 32 rows in either tile kernel
 ]
 
 

@@ -243,7 +243,7 @@ def test_marlin_gemm_tiled_within_tolerance(gu, dtype, m, k, n, g, zp, act, bias
 
 WIDE_TILE_CASES = [
     # m, k, n, group, zp, bias: the forms of the one-wavefront-per-SIMD tile kernel (K a multiple of 256,
-    # groups of 64 * 2^i rows or one group).  At most 128 tiles of 256 rows: 128-row tiles
+    # groups of 32 or 64 * 2^i rows or one group).  At most 128 tiles of 256 rows: 128-row tiles
     (300, 256, 256, 64, False, False),        # one pass of the four-step loop
     (300, 1024, 768, 128, True, True),        # 9 tiles of 128 rows, two ranges of K
     (520, 2048, 512, 256, False, True),       # groups of four steps
@@ -262,6 +262,11 @@ WIDE_TILE_CASES = [
     # 65..128 rows with a long K: the tile kernel (256-row tiles, K split) instead of 64-row slabs
     (100, 8192, 512, 128, False, True),
     (128, 14336, 256, 128, True, False),
+    # groups of 32 rows: a row of scales (and zero points) per k block, 256-row tiles
+    (300, 1024, 768, 32, True, True),         # two ranges of K
+    (2100, 512, 4096, 32, False, False),      # 144 tiles
+    (1030, 2048, 4160, 32, True, False),      # ragged both ways, K split
+    (600, 1216, 512, 32, False, True),        # 19 steps: the eight-wavefront kernel
 ]
 
 
