@@ -772,12 +772,16 @@ constexpr int wide_ops(int rb, bool fp4 = false, bool w8 = false) { return rb / 
 // zeros times the last step's weights).
 __device__ __attribute__((aligned(128))) const uint32_t kWideZeroLine[32] = {};
 
-// G32: a scale (and zero point) per 32 rows, i.e. one row of them per k block: MXFP4 always, integer codes when asked
-template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16, bool FP4 = false, int W8 = 0, bool G32 = FP4>
+// G32: a scale (and zero point) per 32 rows, i.e. one row of them per k block: MXFP4 always, integer codes when asked.
+// NV (with FP4): NVFP4, a scale per 16 rows: the row of a k block then holds two groups of 128 bytes (the copy
+// fetches one per half of the wavefront), and a lane, whose eight rows of a k block lie in one group, reads group
+// kb / 2; the global scale multiplies the sums at the end.
+template <typename T, bool HAS_ZP, bool GROUPED = false, int RB = 16, bool FP4 = false, int W8 = 0, bool G32 = FP4,
+          bool NV = false>
 __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) void marlin_tile_wide_kernel(
     const TileParams p) {
   typedef typename Dq<T>::vec8 vec8;
-  typedef typename Dq4Of<T, FP4>::type D4;   // integer codes, or float4_e2m1f with a scale per 32 rows (MXFP4: bf16)
+  typedef typename Dq4Of<T, FP4, NV>::type D4;   // integer codes, or float4_e2m1f (MXFP4: bf16; NVFP4)
   typedef typename Dq8Of<T, W8 == 2>::type D8;   // 8-bit integer (W8 = 1) or floating-point (W8 = 2) codes
   typedef typename std::conditional<W8 != 0, typename D8::Col, typename D4::Col>::type Col;
   typedef typename Dq<T>::Mid Mid;
@@ -786,7 +790,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   static_assert(!G32 || RB == 16, "groups of 32 rows: 256-row tiles");
   constexpr int kChunkLoads = W8 ? 2 : 1;   // 16-byte loads per lane and k block: 8-bit codes come as a block of
                                             // the low four and a block of the high four of a lane's eight rows
-  static_assert(!FP4 || (std::is_same<T, __bf16>::value && !HAS_ZP && RB == 16), "MXFP4: bf16, no zero points, 256-row tiles");
+  static_assert(!FP4 || ((NV || std::is_same<T, __bf16>::value) && !HAS_ZP && RB == 16),
+                "MXFP4: bf16; float4 codes: no zero points, 256-row tiles");
+  static_assert(!NV || FP4, "NVFP4 is float4 codes");
   static_assert(RB == 16 || (RB == 8 && !GROUPED), "256-row tiles, or 128-row tiles for dense calls");
   constexpr int kRows = 16 * RB;
   constexpr int kStage = wide_stage(RB), kWideA = wide_a(RB), kWideOps = wide_ops(RB, G32, W8 != 0);
@@ -862,6 +868,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   } else {
     s_src = reinterpret_cast<const char*>(p.scales + expert * p.expert_s_stride + strip * kStripN) + 4 * (lane & 31);
     s_group_stride = (long)p.size_n * 2;
+    if (NV) s_src += (lane >> 5) * s_group_stride;   // the upper half of the wavefront fetches the next group's row
   }
   // steps per group as a shift (the host checks: group_size = 64 * 2^i)
   const int group_shift = grouped ? 31 - __builtin_clz(p.group_size / kTileK) : 0;
@@ -878,7 +885,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   // k block h of the step (groups of 32 rows), ring position 2 (kt - k_first) + h
   auto issue_scales = [&](int kt, int h) __attribute__((always_inline)) {
     const int k = min(kt, k_tiles - 1);
-    const int grp = G32 ? 2 * k + h : (grouped ? k >> group_shift : 0);
+    const int grp = G32 ? (NV ? 2 : 1) * (2 * k + h) : (grouped ? k >> group_shift : 0);
     const int at = G32 ? 2 * (kt - k_first) + h : kt - k_first;
     __builtin_amdgcn_global_load_lds((glb_void_t*)(s_src + (long)grp * s_group_stride),
                                      (lds_void_t*)(sring + (at & (kWideScaleRows - 1)) * 256), 4, 0, 0);
@@ -936,7 +943,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #define SONAR_WIDE_LANDED(n, reg) asm volatile("s_waitcnt lgkmcnt(%1)" : "+v"(reg) : "n"(n) : "memory")
 
   auto scales_start = [&](int kt, int h) __attribute__((always_inline)) {
-    const uint32_t r_at = s_lds + ((G32 ? 2 * (kt - k_first) + h : kt - k_first) & (kWideScaleRows - 1)) * 256;
+    const uint32_t r_at = s_lds + ((G32 ? 2 * (kt - k_first) + h : kt - k_first) & (kWideScaleRows - 1)) * 256 +
+                          (NV ? 128 * (kb >> 1) : 0);
     asm volatile(
         "ds_read_u16 %0, %5\n\t"
         "ds_read_u16 %1, %6\n\t"
@@ -944,7 +952,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         "ds_read_u16 %3, %8\n\t"
         "ds_read_b32 %4, %9"
         : "=&v"(sb0), "=&v"(sb1), "=&v"(sb2), "=&v"(sb3), "=&v"(zw)
-        : "v"(r_at + s_off[0]), "v"(r_at + s_off[1]), "v"(r_at + s_off[2]), "v"(r_at + s_off[3]), "v"(r_at + z_off)
+        : "v"(r_at + s_off[0]), "v"(r_at + s_off[1]), "v"(r_at + s_off[2]), "v"(r_at + s_off[3]),
+          "v"(NV ? r_at + s_off[0] : r_at + z_off)
         : "memory");
   };
   auto make_col = [&](int set, int j) __attribute__((always_inline)) {
@@ -984,6 +993,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     const u32x4_t& q4h = B ? wq[NR][kChunkLoads - 1] : wq[R][2 * kChunkLoads - 1];   // 8-bit: the high four rows
     constexpr int kPairs = 16 / RB;   // pairs of weights dequantised per row block
     uint32_t r_lo = 0;     // MXFP4: rows (0, 2) or (4, 6) of the word in hand, waiting for their odd partners
+    uint32_t nv_lo = 0, nv_hi = 0;   // NVFP4, bf16: the same rows as fp32 products
 #pragma unroll
     for (int rb = 0; rb < RB; ++rb) {
       const int j = (kPairs * rb) >> 2, part = (kPairs * rb) & 3;
@@ -1013,6 +1023,47 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
         mfma(B, 1, rb);
         mfma(B, 2, rb);
         mfma(B, 3, rb);
+      } else if constexpr (NV && std::is_same<T, _Float16>::value) {
+        // the pair of codes read as fp16 numbers (value * 2^-14) times scale * 2^14 in one packed multiply
+        // (DqNvF4<_Float16>::pair, a piece behind each MFMA)
+        mfma(B, 0, rb);
+        const uint32_t y = part == 3 ? qw : qw << (12 - 4 * part);
+        const uint32_t mag = (y >> 3) & 0x0E000E00u;
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 1, rb);
+        const uint32_t hbits = (y & 0x80008000u) | mag;
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 2, rb);
+        wb[NB][j][part] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, hbits) *
+                                                           __builtin_bit_cast(half2_t, cols[set][j].s2));
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 3, rb);
+      } else if constexpr (NV) {
+        // bf16: one hardware conversion with a unit scale per row block (rows (0,2), (1,3), (4,6), (5,7) of the
+        // column), the two values times the scale in fp32; behind the second and the fourth, the two byte
+        // permutes that cut the products back to bf16 and put four rows in order (DqNvF4<__bf16>::word)
+        mfma(B, 0, rb);
+        const float sc = cols[set][j].s;
+        const uint32_t r = __builtin_bit_cast(
+            uint32_t, part == 0   ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, 1.0f, 0)
+                      : part == 1 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, 1.0f, 2)
+                      : part == 2 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, 1.0f, 1)
+                                  : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, 1.0f, 3));
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 1, rb);
+        const float f_lo = __uint_as_float(r << 16), f_hi = __uint_as_float(r & 0xFFFF0000u);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 2, rb);
+        const uint32_t p_lo = __float_as_uint(f_lo * sc), p_hi = __float_as_uint(f_hi * sc);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 3, rb);
+        if (part & 1) {
+          wb[NB][j][part - 1] = __builtin_amdgcn_perm(p_lo, nv_lo, 0x07060302u);
+          wb[NB][j][part] = __builtin_amdgcn_perm(p_hi, nv_hi, 0x07060302u);
+        } else {
+          nv_lo = p_lo;
+          nv_hi = p_hi;
+        }
       } else if constexpr (FP4) {
         // one hardware conversion per row block (two rows of the column each: (0,2), (1,3), (4,6),
         // (5,7)); behind the second and the fourth, the two byte permutes that put four rows in order
@@ -1158,6 +1209,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     return;
   }
   const uint16_t* bias_src = p.bias ? p.bias + expert * p.expert_bias_stride + strip * kStripN : nullptr;
+  float gs = 1.f;   // NVFP4: the global scale multiplies the sum before anything else (marlin_template.h:1661-1665)
+  if (NV && p.global_scale) gs = p.global_scale[GROUPED ? expert : 0];
   float bias[4][4];
 #pragma unroll
   for (int nb = 0; nb < 4; ++nb)
@@ -1185,7 +1238,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
     for (int nb = 0; nb < 4; ++nb) {
       if (mb < kAgprBlocks) asm volatile("" : "+a"(acc[nb][mb]));   // still in its AGPRs here
       if (c_row >= 0) {
-        const floatx4_t v = acc[nb][mb];
+        const floatx4_t v = NV ? acc[nb][mb] * gs : acc[nb][mb];
         uint16_t o[4] = {Dq<T>::from_float(v.x + bias[nb][0]), Dq<T>::from_float(v.y + bias[nb][1]),
                          Dq<T>::from_float(v.z + bias[nb][2]), Dq<T>::from_float(v.w + bias[nb][3])};
         if (GROUPED && p.mul_topk) {
@@ -1365,6 +1418,18 @@ int launch_tile_wide_fp4(const TileParams& p, hipStream_t st) {
     attr_set = true;
   }
   marlin_tile_wide_kernel<__bf16, false, GROUPED, 16, true><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
+  return SONAR_OK;
+}
+// NVFP4: either activation type, groups of 16 rows, a global scale (one per expert when GROUPED)
+template <typename T, bool GROUPED>
+int launch_tile_wide_nvfp4(const TileParams& p, hipStream_t st) {
+  static bool attr_set = false;
+  if (!attr_set) {
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, false, GROUPED, 16, true, 0, true, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
+    attr_set = true;
+  }
+  marlin_tile_wide_kernel<T, false, GROUPED, 16, true, 0, true, true><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
   return SONAR_OK;
 }
 // 8-bit codes: uint8b128 or float8_e4m3fn (groups of 64 * 2^i rows or one group; G32: of 32 rows, MXFP8)
@@ -1555,7 +1620,10 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     }
     if (p.tile_rows != kTileM && !wide_applies(p))
       return fail(SONAR_E_INVALID, "internal: 128-row tiles exist in the wide tile kernel only");
-    if (nvfp4)
+    if (nvfp4 && wide_applies_fp4(p))
+      rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide_nvfp4<_Float16, false>(p, st)
+                                    : launch_tile_wide_nvfp4<__bf16, false>(p, st);
+    else if (nvfp4)
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16>(p, st) : launch_tile_async_nvfp4<__bf16>(p, st);
     else if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
       rc = wide_applies_fp4(p) ? launch_tile_wide_fp4<false>(p, st) : launch_tile_async_fp4(p, st);
@@ -1655,7 +1723,10 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.expert_z_stride = (long)(num_groups * (size_n / 8));
   p.expert_bias_stride = (long)size_n;
   int rc;
-  if (fp4 && global_scale != nullptr)
+  if (fp4 && global_scale != nullptr && wide_applies_fp4(p))
+    rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide_nvfp4<_Float16, true>(p, st)
+                                  : launch_tile_wide_nvfp4<__bf16, true>(p, st);
+  else if (fp4 && global_scale != nullptr)
     rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16, true>(p, st)
                                   : launch_tile_async_nvfp4<__bf16, true>(p, st);
   else if (fp4)

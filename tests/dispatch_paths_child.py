@@ -76,6 +76,10 @@ def dense_8bit() -> None:
         tp.test_fp8_weights_dequant_bit_exact_and_gemm_within_tolerance(gu, dtype, m, k, n, g, True)
         tp.test_w8a16_dequant_bit_exact_and_gemm_within_tolerance(gu, dtype, m, k, n, g, False, False)
         print("8-bit", dtype, m, k, n, g, "ok", flush=True)
+    # NVFP4 on both tile kernels
+    for (dtype, m, k, n) in [("fp16", 600, 2048, 1536), ("bf16", 2100, 512, 4160)]:
+        tp.test_nvfp4_weights_dequant_bit_exact_and_gemm_within_tolerance(gu, m, k, n, True, dtype)
+        print("nvfp4", dtype, m, k, n, "ok", flush=True)
 
 
 def grouped() -> None:

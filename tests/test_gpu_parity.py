@@ -639,6 +639,8 @@ NVFP4_CASES = [
     (300, 512, 192, True),
     (600, 2048, 1536, True),      # tile kernel, K split, partial tiles summed by the second kernel
     (4096, 4096, 1024, False),    # tile kernel, whole tiles
+    (2100, 512, 4160, True),      # ... 153 tiles, ragged both ways
+    (300, 1216, 512, False),      # ... 19 steps: not a multiple of four (the eight-wavefront kernel)
 ]
 
 
