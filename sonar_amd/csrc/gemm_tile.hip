@@ -752,7 +752,8 @@ __global__ __launch_bounds__(kTileWaves * 64) void marlin_tile_async_kernel(cons
 // (s_nop below).
 // 4-bit or symmetric 8-bit codes with groups of 64 * 2^i rows or one group, MXFP4 (float4_e2m1f codes,
 // bf16, a scale per 32 rows: one hardware conversion and half a byte permute behind each row
-// block), or integer / 8-bit floating-point codes with a scale per 32 rows (MXFP8 among them); no
+// block), integer / 8-bit floating-point codes with a scale per 32 rows (MXFP8 among them), or NVFP4
+// (float4_e2m1f codes with a scale per 16 rows and a global scale, either activation type); no
 // act-order; dense and grouped (mixture-of-experts) calls.  K ranges that are not a
 // multiple of four steps are padded with steps of zeros (integer codes; taken only where that
 // is a small part of the range).
