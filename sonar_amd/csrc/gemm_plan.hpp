@@ -16,7 +16,17 @@ struct GemmPlan {
   int64_t whole_tiles;
 };
 
-inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool async_tile, int tile_rows = 256) {
+// 97..128 rows on a matrix with more strips than compute units (N > 16384) and K <= 8192: the wide tile
+// kernel's 128-row form with K in two ranges is ahead of blocks of rows in the decode kernel (measured at
+// K = 4096, N = 28672: M = 128: 45 us against 55; M = 72 and 96: level; with 64 to 96 strips, N = 4096 / 6144,
+// the decode kernel is two times ahead).  `wide128`: the call is one that form takes (4-bit integer codes
+// with groups of 64 * 2^i rows or one group, no act-order gather).
+inline bool plan_rows_97_128(int64_t size_m, int64_t size_n, int64_t size_k, bool wide128) {
+  return wide128 && size_m > 96 && size_m <= 128 && size_n > 16384 && size_k <= 8192 && size_k % 256 == 0;
+}
+
+inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool async_tile, int tile_rows = 256,
+                          bool rows_97_128 = false) {
   GemmPlan plan = {false, tile_rows, 1, 0, 0};
   if (size_m <= 64 || size_k % 64 != 0) return plan;
   const int64_t tiles = ((size_m + tile_rows - 1) / tile_rows) * ((size_n + 255) / 256);
@@ -50,7 +60,7 @@ inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool a
   }
   // (with a long K the partial tiles are a small part of the work: measured at K = 14336, N = 4096,
   // M = 96 / 128: 47 / 53 us in slabs)
-  if (size_m <= 128 && !(async_tile && size_k >= 8192 && splits > 1)) return plan;
+  if (size_m <= 128 && !(async_tile && (size_k >= 8192 || rows_97_128) && splits > 1)) return plan;
   if (splits == 1 && size_m <= 512 && tiles < 64) return plan;  // slabs use every compute unit
   plan.tile = true;
   plan.k_splits = splits;
@@ -72,15 +82,16 @@ inline size_t plan_partial_bytes(const GemmPlan& plan, int64_t size_m, int64_t s
 // K ranges of the same tile: twice the tiles, half the ranges, half the partial-tile bytes.  With
 // a long K the partial tiles are a small part of the work and the larger tile stays ahead
 // (measured: K = 14336, M = 1024, N = 4096: 108 us against 119).
-inline bool plan_prefers_128_rows(int64_t size_m, int64_t size_n, int64_t size_k) {
+inline bool plan_prefers_128_rows(int64_t size_m, int64_t size_n, int64_t size_k, bool rows_97_128 = false) {
   const int64_t tiles256 = ((size_m + 255) / 256) * ((size_n + 255) / 256);
-  return size_m > 128 && tiles256 <= 128 && size_k <= 8192;
+  return (size_m > 128 || rows_97_128) && tiles256 <= 128 && size_k <= 8192;
 }
 
 // Scratch for the partial tiles of either tiling.
 inline size_t plan_partial_bytes_any(int64_t size_m, int64_t size_n, int64_t size_k) {
-  const size_t a = plan_partial_bytes(plan_gemm(size_m, size_n, size_k, true, 256), size_m, size_n);
-  const size_t b = plan_partial_bytes(plan_gemm(size_m, size_n, size_k, true, 128), size_m, size_n);
+  const bool r = plan_rows_97_128(size_m, size_n, size_k, true);
+  const size_t a = plan_partial_bytes(plan_gemm(size_m, size_n, size_k, true, 256, r), size_m, size_n);
+  const size_t b = plan_partial_bytes(plan_gemm(size_m, size_n, size_k, true, 128, r), size_m, size_n);
   return a > b ? a : b;
 }
 

@@ -1801,7 +1801,14 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
   const bool few_row_blocks = n_strips * ((size_m + 31) / 32) <= 4 * (int64_t)cus;
   // (groups of 32 / 64 rows take the 16-row kernel up to 16 rows only: measured at K = 4096, N = 11008,
   // M = 64: 43 / 30 us in blocks of rows against 30 / 27 in the general kernel)
-  const bool slab_fast = !no_slabs && fast_shape && size_m > 16 && unit_group_shift >= -1 &&
+  static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
+  const bool async_tile = chk.nvfp4 || tile_async_applies(chk.has_perm, num_groups, chk.group_size);
+  // (97..128 rows on more strips than compute units: 128-row tiles, see plan_rows_97_128)
+  const int steps_per_group = chk.group_size / 64;
+  const bool wide128 = chk.bits == 4 && !chk.fp4 && !chk.has_perm && !chk.row_groups &&
+                       (num_groups == 1 || (chk.group_size % 64 == 0 && (steps_per_group & (steps_per_group - 1)) == 0));
+  const bool rows_97_128 = !no_tile && async_tile && plan_rows_97_128(size_m, size_n, size_k, wide128);
+  const bool slab_fast = !no_slabs && fast_shape && size_m > 16 && unit_group_shift >= -1 && !rows_97_128 &&
                          (size_m <= 64 || (strip_per_workgroup && (size_m <= 128 || few_row_blocks)));
 
   p.unit_chunks = p.chunks_per_strip % 4 == 0 ? 4 : (p.chunks_per_strip % 2 == 0 ? 2 : 1);
@@ -1812,9 +1819,7 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
   SONAR_REQUIRE(total_units * cus < (1LL << 31), "size_k * size_n = %ld x %ld is too large", (long)size_k,
                 (long)size_n);
   p.total_units = (int)total_units;
-  static const bool no_tile = getenv("SONAR_MARLIN_NO_TILE") != nullptr;  // debugging aid
-  const bool async_tile = chk.nvfp4 || tile_async_applies(chk.has_perm, num_groups, chk.group_size);
-  const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile);
+  const GemmPlan plan = plan_gemm(size_m, size_n, size_k, async_tile, 256, rows_97_128);
   // the row -> group lookup and 8-bit codes exist in the streaming kernels only
   // (MXFP4 only through the asynchronous tile kernel: the older one has no float4 dequantiser)
   // (8-bit codes and MXFP4 only through the asynchronous tile kernel: the older one has neither dequantiser)

@@ -1588,11 +1588,15 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   const bool nvfp4 = fp4 && global_scale != nullptr;   // the caller has checked: groups of 16 rows
   if ((nvfp4 || tile_async_applies(pm, num_groups, group_size)) &&
       (!no_async || fp4 || bits == 8)) {   // float4 and 8-bit codes exist here only
-    GemmPlan plan = plan_gemm(size_m, size_n, size_k, true);
+    const int steps_per_group = group_size / kTileK;
+    const bool wide128 = bits == 4 && !fp4 && !pm &&
+                         (num_groups == 1 || (group_size % kTileK == 0 && (steps_per_group & (steps_per_group - 1)) == 0));
+    const bool rows_97_128 = plan_rows_97_128(size_m, size_n, size_k, wide128);
+    GemmPlan plan = plan_gemm(size_m, size_n, size_k, true, 256, rows_97_128);
     // few tiles and a call the wide kernel takes: 128-row tiles
     static const bool no_128 = getenv("SONAR_MARLIN_NO_128_ROW_TILES") != nullptr;   // debugging aid
-    if (!no_128 && bits == 4 && !fp4 && plan_prefers_128_rows(size_m, size_n, size_k)) {
-      const GemmPlan plan128 = plan_gemm(size_m, size_n, size_k, true, 128);
+    if (!no_128 && bits == 4 && !fp4 && plan_prefers_128_rows(size_m, size_n, size_k, rows_97_128)) {
+      const GemmPlan plan128 = plan_gemm(size_m, size_n, size_k, true, 128, rows_97_128);
       TileParams probe = p;
       probe.tile_rows = 128;
       probe.k_splits = plan128.k_splits;

@@ -262,6 +262,9 @@ WIDE_TILE_CASES = [
     # 65..128 rows with a long K: the tile kernel (256-row tiles, K split) instead of 64-row slabs
     (100, 8192, 512, 128, False, True),
     (128, 14336, 256, 128, True, False),
+    # 97..128 rows on more strips than compute units: 128-row tiles, K in two ranges
+    (128, 512, 16640, 128, False, True),
+    (100, 1024, 16448, -1, True, False),
     # groups of 32 rows: a row of scales (and zero points) per k block, 256-row tiles
     (300, 1024, 768, 32, True, True),         # two ranges of K
     (2100, 512, 4096, 32, False, False),      # 144 tiles
