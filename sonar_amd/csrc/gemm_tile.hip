@@ -764,8 +764,8 @@ constexpr int kWideScaleRows = 16;   // a ring of 16 rows per wavefront: eight s
 constexpr int wide_stage(int rb) { return rb * 2 * kBlockBytes; }                    // one stage of A
 constexpr int wide_a(int rb) { return kWideStages * wide_stage(rb); }                // 128 / 64 KiB
 constexpr int wide_lds(int rb) { return wide_a(rb) + 4 * kWideScaleRows * 256; }     // + the scale rows of four wavefronts
-// memory operations per wavefront and step: its blocks of A, the scale row (MXFP4: two, one per k block), two
-// chunks (8-bit codes: four blocks)
+// memory operations per wavefront and step: its blocks of A, the scale row (groups of 32 / 16 rows: two, one per
+// k block), two chunks (8-bit codes: four blocks)
 constexpr int wide_ops(int rb, bool fp4 = false, bool w8 = false) { return rb / 2 + (fp4 ? 2 : 1) + (w8 ? 4 : 2); }
 
 // One 128-byte line of zeros: what the copies of A fetch for the steps past the end of a K range that
@@ -786,7 +786,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   typedef typename Dq8Of<T, W8 == 2>::type D8;   // 8-bit integer (W8 = 1) or floating-point (W8 = 2) codes
   typedef typename std::conditional<W8 != 0, typename D8::Col, typename D4::Col>::type Col;
   typedef typename Dq<T>::Mid Mid;
-  static_assert(W8 == 0 || (!HAS_ZP && !FP4 && RB == 16), "8-bit codes: symmetric, 256-row tiles");
+  static_assert(W8 == 0 || (!HAS_ZP && !FP4), "8-bit codes: symmetric");
+  static_assert(wide_ops(RB, G32, W8 != 0) <= 2 * RB, "a step's memory operations go out behind its row blocks");
   static_assert(!FP4 || G32, "MXFP4 has a scale per 32 rows");
   static_assert(!G32 || RB == 16, "groups of 32 rows: 256-row tiles");
   constexpr int kChunkLoads = W8 ? 2 : 1;   // 16-byte loads per lane and k block: 8-bit codes come as a block of
@@ -1014,8 +1015,9 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
       if constexpr (W8 != 0) {
         // behind every second row block, half a column block (four rows of 16 columns) in one piece
         mfma(B, 0, rb);
-        if ((rb & 1) == 0) {
-          const int jj = rb >> 2, half = (rb >> 1) & 1;
+        if (RB == 8 || (rb & 1) == 0) {   // (with 8 row blocks: behind every row block)
+          const int piece = RB == 8 ? rb : rb >> 1;
+          const int jj = piece >> 1, half = piece & 1;
           const uint2 w = D8::word4(word_of(half ? q4h : q4, jj), cols[set][jj], magic);
           wb[NB][jj][2 * half] = w.x;
           wb[NB][jj][2 * half + 1] = w.y;
@@ -1110,6 +1112,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
           if (rb == (kAhead + 1 + c < RB ? kAhead + 1 + c : RB - 1)) make_col(G32 ? B : (R + 1) & 1, c);
       }
       if (B == 1 && rb < kWideOps) issue_one(kt + 3, (R + 3) & 3, rb);
+      // (8-bit codes with 8 row blocks: nine operations, the ninth behind the first row block too)
+      if (B == 1 && RB + rb < kWideOps) issue_one(kt + 3, (R + 3) & 3, RB + rb);
       __builtin_amdgcn_sched_barrier(0);
     }
   };
@@ -1435,20 +1439,25 @@ int launch_tile_wide_nvfp4(const TileParams& p, hipStream_t st) {
 }
 // 8-bit codes: uint8b128 or float8_e4m3fn (groups of 64 * 2^i rows or one group; G32: of 32 rows, MXFP8)
 inline bool wide_groups_of_32(const TileParams& p) { return p.num_groups > 1 && p.group_size == 32; }
-template <typename T, bool GROUPED, int W8, bool G32>
+template <typename T, bool GROUPED, int W8, bool G32, int RB = 16>
 int launch_tile_wide8_groups(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, false, GROUPED, 16, false, W8, G32>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, false, GROUPED, RB, false, W8, G32>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(RB)));
     attr_set = true;
   }
-  marlin_tile_wide_kernel<T, false, GROUPED, 16, false, W8, G32><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
+  marlin_tile_wide_kernel<T, false, GROUPED, RB, false, W8, G32><<<tile_grid(p), 256, wide_lds(RB), st>>>(p);
   return SONAR_OK;
 }
 template <typename T, bool GROUPED>
 int launch_tile_wide8(const TileParams& p, bool fp8, hipStream_t st) {
   const bool g32 = wide_groups_of_32(p);
+  if constexpr (!GROUPED) {   // 128-row tiles (dense calls with few tiles; never with groups of 32 rows)
+    if (p.tile_rows == 128)
+      return fp8 ? launch_tile_wide8_groups<T, false, 2, false, 8>(p, st)
+                 : launch_tile_wide8_groups<T, false, 1, false, 8>(p, st);
+  }
   if (fp8) return g32 ? launch_tile_wide8_groups<T, GROUPED, 2, true>(p, st)
                       : launch_tile_wide8_groups<T, GROUPED, 2, false>(p, st);
   return g32 ? launch_tile_wide8_groups<T, GROUPED, 1, true>(p, st)
@@ -1538,8 +1547,8 @@ bool wide_applies_fp4(const TileParams& p) {
   // K = 2880, N = 5760, M = 4096: 143 us against 156)
   return !no_wide && wide_padding(range) == 0 && p.tile_rows == kTileM;
 }
-// ... and for 8-bit codes: 256-row tiles only.
-bool wide_applies8(const TileParams& p) { return p.tile_rows == kTileM && wide_applies(p); }
+// ... and for 8-bit codes (the same rule: 128-row tiles but for groups of 32 rows).
+bool wide_applies8(const TileParams& p) { return wide_applies(p); }
 }  // namespace
 
 // The asynchronous tile kernel needs groups of 32 rows or a multiple of 64 and no gather of A.
@@ -1595,7 +1604,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     GemmPlan plan = plan_gemm(size_m, size_n, size_k, true, 256, rows_97_128);
     // few tiles and a call the wide kernel takes: 128-row tiles
     static const bool no_128 = getenv("SONAR_MARLIN_NO_128_ROW_TILES") != nullptr;   // debugging aid
-    if (!no_128 && bits == 4 && !fp4 && plan_prefers_128_rows(size_m, size_n, size_k, rows_97_128)) {
+    if (!no_128 && !fp4 && plan_prefers_128_rows(size_m, size_n, size_k, rows_97_128)) {
       const GemmPlan plan128 = plan_gemm(size_m, size_n, size_k, true, 128, rows_97_128);
       TileParams probe = p;
       probe.tile_rows = 128;

@@ -395,6 +395,8 @@ W8_CASES = [
     (260, 1024, 4160, -1, False, False),     # one group
     (512, 2048, 320, 32, False, True),       # groups of 32 rows
     (300, 2048, 512, 128, True, False),      # act-order through the permuted copy of A
+    (520, 2048, 512, 256, False, True),      # few tiles: 128-row tiles, groups of four steps
+    (1100, 512, 1024, -1, False, False),     # ... one group, no K split
     (1024, 1024, 832, 32, False, False),     # groups of 32 rows, whole tiles over all of K
     (700, 1280, 4160, 32, False, True),      # ... K ranges of 20 steps, ragged tiles both ways
     (300, 1216, 512, 32, False, False),      # ... 19 steps: not a multiple of four (the eight-wavefront kernel)
@@ -479,6 +481,8 @@ FP8_CASES = [
     (300, 2048, 512, 128, True),
     (1024, 1024, 832, -1, False),
     (512, 2048, 320, 32, True),
+    (520, 2048, 512, 128, True),      # few tiles: 128-row tiles
+    (1100, 512, 1024, -1, False),     # ... one group, no K split
     (1024, 1024, 832, 32, False),     # groups of 32 rows, whole tiles over all of K
     (700, 1280, 4160, 32, True),      # ... K ranges of 20 steps, ragged tiles both ways
     (300, 1216, 512, 32, False),      # ... 19 steps: not a multiple of four (the eight-wavefront kernel)
