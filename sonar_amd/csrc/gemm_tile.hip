@@ -789,12 +789,11 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   static_assert(W8 == 0 || (!HAS_ZP && !FP4), "8-bit codes: symmetric");
   static_assert(wide_ops(RB, G32, W8 != 0) <= 2 * RB, "a step's memory operations go out behind its row blocks");
   static_assert(!FP4 || G32, "MXFP4 has a scale per 32 rows");
-  static_assert(!G32 || RB == 16, "groups of 32 rows: 256-row tiles");
   constexpr int kChunkLoads = W8 ? 2 : 1;   // 16-byte loads per lane and k block: 8-bit codes come as a block of
                                             // the low four and a block of the high four of a lane's eight rows
-  static_assert(!FP4 || ((NV || std::is_same<T, __bf16>::value) && !HAS_ZP && RB == 16),
-                "MXFP4: bf16; float4 codes: no zero points, 256-row tiles");
-  static_assert(!NV || FP4, "NVFP4 is float4 codes");
+  static_assert(!FP4 || ((NV || std::is_same<T, __bf16>::value) && !HAS_ZP), "MXFP4: bf16; float4 codes: no zero points");
+  static_assert(!NV || (FP4 && RB == 16), "NVFP4 is float4 codes; 256-row tiles");
+  static_assert(!(W8 != 0 && G32) || RB == 16, "8-bit codes with groups of 32 rows: 256-row tiles");
   static_assert(RB == 16 || (RB == 8 && !GROUPED), "256-row tiles, or 128-row tiles for dense calls");
   constexpr int kRows = 16 * RB;
   constexpr int kStage = wide_stage(RB), kWideA = wide_a(RB), kWideOps = wide_ops(RB, G32, W8 != 0);
@@ -1041,6 +1040,23 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
                                                            __builtin_bit_cast(half2_t, cols[set][j].s2));
         __builtin_amdgcn_sched_barrier(0);
         mfma(B, 3, rb);
+      } else if constexpr (FP4 && kPairs == 2) {
+        // MXFP4 with 8 row blocks: the conversions of an even and an odd part (rows (0,2) and (1,3), or (4,6) and
+        // (5,7)) and their two byte permutes behind one row block
+        mfma(B, 0, rb);
+        const float sc = cols[set][j].s;
+        const uint32_t r_e = __builtin_bit_cast(uint32_t, part == 0 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, sc, 0)
+                                                                    : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, sc, 1));
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 1, rb);
+        const uint32_t r_o = __builtin_bit_cast(uint32_t, part == 0 ? __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, sc, 2)
+                                                                    : __builtin_amdgcn_cvt_scalef32_pk_bf16_fp4(qw, sc, 3));
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 2, rb);
+        wb[NB][j][part] = __builtin_amdgcn_perm(r_o, r_e, 0x05040100u);
+        __builtin_amdgcn_sched_barrier(0);
+        mfma(B, 3, rb);
+        wb[NB][j][part + 1] = __builtin_amdgcn_perm(r_o, r_e, 0x07060302u);
       } else if constexpr (NV) {
         // bf16: one hardware conversion with a unit scale per row block (rows (0,2), (1,3), (4,6), (5,7) of the
         // column), the two values times the scale in fp32; behind the second and the fourth, the two byte
@@ -1414,28 +1430,40 @@ int launch_tile_wide_rows(const TileParams& p, hipStream_t st) {
   return SONAR_OK;
 }
 // MXFP4: bf16, groups of 32 rows, float4_e2m1f codes
-template <bool GROUPED>
-int launch_tile_wide_fp4(const TileParams& p, hipStream_t st) {
+template <bool GROUPED, int RB>
+int launch_tile_wide_fp4_rows(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<__bf16, false, GROUPED, 16, true>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<__bf16, false, GROUPED, RB, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(RB)));
     attr_set = true;
   }
-  marlin_tile_wide_kernel<__bf16, false, GROUPED, 16, true><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
+  marlin_tile_wide_kernel<__bf16, false, GROUPED, RB, true><<<tile_grid(p), 256, wide_lds(RB), st>>>(p);
   return SONAR_OK;
 }
+template <bool GROUPED>
+int launch_tile_wide_fp4(const TileParams& p, hipStream_t st) {
+  if constexpr (!GROUPED) {
+    if (p.tile_rows == 128) return launch_tile_wide_fp4_rows<false, 8>(p, st);
+  }
+  return launch_tile_wide_fp4_rows<GROUPED, 16>(p, st);
+}
 // NVFP4: either activation type, groups of 16 rows, a global scale (one per expert when GROUPED)
-template <typename T, bool GROUPED>
-int launch_tile_wide_nvfp4(const TileParams& p, hipStream_t st) {
+template <typename T, bool GROUPED, int RB>
+int launch_tile_wide_nvfp4_rows(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, false, GROUPED, 16, true, 0, true, true>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, false, GROUPED, RB, true, 0, true, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(RB)));
     attr_set = true;
   }
-  marlin_tile_wide_kernel<T, false, GROUPED, 16, true, 0, true, true><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
+  marlin_tile_wide_kernel<T, false, GROUPED, RB, true, 0, true, true><<<tile_grid(p), 256, wide_lds(RB), st>>>(p);
   return SONAR_OK;
+}
+template <typename T, bool GROUPED>
+int launch_tile_wide_nvfp4(const TileParams& p, hipStream_t st) {
+  if (p.tile_rows != kTileM) return fail(SONAR_E_INVALID, "internal: NVFP4 runs on 256-row tiles");
+  return launch_tile_wide_nvfp4_rows<T, GROUPED, 16>(p, st);
 }
 // 8-bit codes: uint8b128 or float8_e4m3fn (groups of 64 * 2^i rows or one group; G32: of 32 rows, MXFP8)
 inline bool wide_groups_of_32(const TileParams& p) { return p.num_groups > 1 && p.group_size == 32; }
@@ -1453,7 +1481,8 @@ int launch_tile_wide8_groups(const TileParams& p, hipStream_t st) {
 template <typename T, bool GROUPED>
 int launch_tile_wide8(const TileParams& p, bool fp8, hipStream_t st) {
   const bool g32 = wide_groups_of_32(p);
-  if constexpr (!GROUPED) {   // 128-row tiles (dense calls with few tiles; never with groups of 32 rows)
+  if constexpr (!GROUPED) {   // 128-row tiles (dense calls with few tiles)
+    if (p.tile_rows == 128 && g32) return fail(SONAR_E_INVALID, "internal: 8-bit codes with groups of 32 rows run on 256-row tiles");
     if (p.tile_rows == 128)
       return fp8 ? launch_tile_wide8_groups<T, false, 2, false, 8>(p, st)
                  : launch_tile_wide8_groups<T, false, 1, false, 8>(p, st);
@@ -1464,16 +1493,23 @@ int launch_tile_wide8(const TileParams& p, bool fp8, hipStream_t st) {
              : launch_tile_wide8_groups<T, GROUPED, 1, false>(p, st);
 }
 // 4-bit integer codes with groups of 32 rows
-template <typename T, bool HAS_ZP, bool GROUPED>
-int launch_tile_wide_g32(const TileParams& p, hipStream_t st) {
+template <typename T, bool HAS_ZP, bool GROUPED, int RB>
+int launch_tile_wide_g32_rows(const TileParams& p, hipStream_t st) {
   static bool attr_set = false;
   if (!attr_set) {
-    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, HAS_ZP, GROUPED, 16, false, 0, true>,
-                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(16)));
+    SONAR_HIP(hipFuncSetAttribute((const void*)marlin_tile_wide_kernel<T, HAS_ZP, GROUPED, RB, false, 0, true>,
+                                  hipFuncAttributeMaxDynamicSharedMemorySize, wide_lds(RB)));
     attr_set = true;
   }
-  marlin_tile_wide_kernel<T, HAS_ZP, GROUPED, 16, false, 0, true><<<tile_grid(p), 256, wide_lds(16), st>>>(p);
+  marlin_tile_wide_kernel<T, HAS_ZP, GROUPED, RB, false, 0, true><<<tile_grid(p), 256, wide_lds(RB), st>>>(p);
   return SONAR_OK;
+}
+template <typename T, bool HAS_ZP, bool GROUPED>
+int launch_tile_wide_g32(const TileParams& p, hipStream_t st) {
+  if constexpr (!GROUPED) {
+    if (p.tile_rows == 128) return launch_tile_wide_g32_rows<T, HAS_ZP, false, 8>(p, st);
+  }
+  return launch_tile_wide_g32_rows<T, HAS_ZP, GROUPED, 16>(p, st);
 }
 template <typename T, bool HAS_ZP, bool GROUPED = false>
 int launch_tile_wide(const TileParams& p, hipStream_t st) {
@@ -1525,7 +1561,7 @@ int launch_tile(const TileParams& p, hipStream_t st) {
 
 namespace {
 // The wide form: groups of 64 * 2^i rows or one group; K ranges of a multiple of four steps, or long ones.
-// Groups of 32 rows: 256-row tiles and whole passes only.
+// Groups of 32 rows: whole passes only.
 // Steps of zeros the wide kernel adds to a K range of `range` steps (at most a tenth of the range is accepted).
 int wide_padding(int range) { return (4 - range % 4) % 4; }
 bool wide_applies(const TileParams& p) {
@@ -1533,7 +1569,7 @@ bool wide_applies(const TileParams& p) {
   if (no_wide) return false;
   // K ranges are rounded up to four steps with steps of zeros: not where that is a large part of the work
   const int range = p.k_splits > 1 ? p.k_steps_per_split : p.size_k / kTileK;
-  if (wide_groups_of_32(p)) return wide_padding(range) == 0 && p.tile_rows == kTileM;
+  if (wide_groups_of_32(p)) return wide_padding(range) == 0;
   if (wide_padding(range) * 10 > range) return false;
   if (p.num_groups == 1) return true;
   const int per_group = p.group_size / kTileK;   // steps per group: a power of two
@@ -1545,9 +1581,9 @@ bool wide_applies_fp4(const TileParams& p) {
   const int range = p.k_splits > 1 ? p.k_steps_per_split : p.size_k / kTileK;
   // (no padding here: the eight-wavefront kernel is as fast on these codes, and ahead once steps are wasted:
   // K = 2880, N = 5760, M = 4096: 143 us against 156)
-  return !no_wide && wide_padding(range) == 0 && p.tile_rows == kTileM;
+  return !no_wide && wide_padding(range) == 0;
 }
-// ... and for 8-bit codes (the same rule: 128-row tiles but for groups of 32 rows).
+// ... and for 8-bit codes (the same rule).
 bool wide_applies8(const TileParams& p) { return wide_applies(p); }
 }  // namespace
 
@@ -1604,13 +1640,16 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     GemmPlan plan = plan_gemm(size_m, size_n, size_k, true, 256, rows_97_128);
     // few tiles and a call the wide kernel takes: 128-row tiles
     static const bool no_128 = getenv("SONAR_MARLIN_NO_128_ROW_TILES") != nullptr;   // debugging aid
-    if (!no_128 && !fp4 && plan_prefers_128_rows(size_m, size_n, size_k, rows_97_128)) {
+    // (not for NVFP4 and 8-bit codes with groups of 32 rows, whose heavier dequantisation wants the 16 row blocks
+    // to hide behind: M = 512, K = 4096, N = 11008: NVFP4 69.9 us against 68.7, MXFP8 91.8 against 82.2)
+    const bool rows128_ok = !nvfp4 && !(bits == 8 && num_groups > 1 && group_size == 32);
+    if (!no_128 && rows128_ok && plan_prefers_128_rows(size_m, size_n, size_k, rows_97_128)) {
       const GemmPlan plan128 = plan_gemm(size_m, size_n, size_k, true, 128, rows_97_128);
       TileParams probe = p;
       probe.tile_rows = 128;
       probe.k_splits = plan128.k_splits;
       probe.k_steps_per_split = plan128.k_steps_per_split;
-      if (plan128.tile && wide_applies(probe) &&
+      if (plan128.tile && (fp4 ? wide_applies_fp4(probe) : wide_applies(probe)) &&
           (plan128.k_splits == 1 || (partial != nullptr && partial_bytes >= plan_partial_bytes(plan128, size_m, size_n)))) {
         plan = plan128;
         p.tile_rows = 128;
@@ -1632,7 +1671,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
         if (p.k_splits == 1) p.partial = nullptr;
       }
     }
-    if (p.tile_rows != kTileM && !wide_applies(p))
+    if (p.tile_rows != kTileM && !(fp4 ? wide_applies_fp4(p) : wide_applies(p)))
       return fail(SONAR_E_INVALID, "internal: 128-row tiles exist in the wide tile kernel only");
     if (nvfp4 && wide_applies_fp4(p))
       rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide_nvfp4<_Float16, false>(p, st)
