@@ -137,18 +137,24 @@ def launch_floors(torch, time_graph):
     """What one launch costs and how long the chip takes to stream the weights of
     each GEMM of the layer when nothing is computed, with the yardstick kernels of
     sonar_amd/csrc/bench_floor.hip (not part of the product path): an empty kernel
-    as a node of a HIP graph, and a kernel that copies a matrix's bytes into LDS
-    with the decode kernel's own asynchronous copies on all compute units, over
-    six regions of 1 GiB in turn so that nothing comes from a cache."""
+    as a node of a HIP graph, and kernels that only fetch a matrix's bytes on all
+    compute units, over six regions of 1 GiB / 6 in turn so that nothing comes from
+    a cache, in four load styles: the decode kernel's own asynchronous copies into
+    LDS without and with the non-temporal bit (`stream`, `stream_nt`: the decode kernel
+    copies its weights with it), plain 16-byte loads into registers at eight wavefronts
+    per SIMD (`stream_reg`), and the same with the non-temporal bit (`stream_reg_nt`)."""
     import ctypes
     from sonar_amd import build
     if not os.path.exists(build.BENCH_PATH):
         return None
     lib = ctypes.CDLL(build.BENCH_PATH)
     lib.sonar_bench_empty.argtypes = [ctypes.c_int, ctypes.c_void_p]
-    lib.sonar_bench_stream.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_void_p]
+    lib.sonar_bench_stream.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_void_p]
+    lib.sonar_bench_stream_reg.argtypes = [ctypes.c_void_p, ctypes.c_size_t, ctypes.c_int, ctypes.c_int,
+                                           ctypes.c_void_p, ctypes.c_void_p]
     cus = torch.cuda.get_device_properties(0).multi_processor_count
     buf = torch.empty(1 << 30, dtype=torch.uint8, device="cuda:0").random_(0, 256)
+    sink = torch.zeros(16, dtype=torch.uint8, device="cuda:0")
     region = (1 << 30) // 6 // 4096 * 4096
 
     def raw_stream():
@@ -159,20 +165,29 @@ def launch_floors(torch, time_graph):
             raise RuntimeError("bench_floor launch failed: %d" % rc)
 
     out = {"empty_kernel_us": round(time_graph(torch, lambda i=0: check(lib.sonar_bench_empty(cus, raw_stream())),
-                                               24) * 1e6, 2),
-           "stream": []}
-    total = 0.0
-    for name, k, n in LAYER_SHAPES:
-        nbytes = k * n // 2 + (k // GROUP) * n * 2          # packed weights and scales
-        assert nbytes <= region
+                                               24) * 1e6, 2)}
+    styles = {
+        "stream": lambda src, nbytes: lib.sonar_bench_stream(src, nbytes, cus, 0, raw_stream()),
+        "stream_nt": lambda src, nbytes: lib.sonar_bench_stream(src, nbytes, cus, 1, raw_stream()),
+        "stream_reg": lambda src, nbytes: lib.sonar_bench_stream_reg(src, nbytes, 2 * cus, 0, sink.data_ptr(),
+                                                                     raw_stream()),
+        "stream_reg_nt": lambda src, nbytes: lib.sonar_bench_stream_reg(src, nbytes, 2 * cus, 1, sink.data_ptr(),
+                                                                        raw_stream()),
+    }
+    for style, launch in styles.items():
+        out[style] = []
+        total = 0.0
+        for name, k, n in LAYER_SHAPES:
+            nbytes = k * n // 2 + (k // GROUP) * n * 2          # packed weights and scales
+            assert nbytes <= region
 
-        def one(i=0, nbytes=nbytes):
-            check(lib.sonar_bench_stream(buf.data_ptr() + (i % 6) * region, nbytes, cus, raw_stream()))
-        s = time_graph(torch, one, 24)
-        total += s
-        out["stream"].append({"gemm": name, "bytes": nbytes, "us": round(s * 1e6, 2),
-                              "GBps": round(nbytes / s / 1e9, 1)})
-    out["stream_step_us"] = round(total * 1e6, 2)
+            def one(i=0, nbytes=nbytes, launch=launch):
+                check(launch(buf.data_ptr() + (i % 6) * region, nbytes))
+            s = time_graph(torch, one, 24)
+            total += s
+            out[style].append({"gemm": name, "bytes": nbytes, "us": round(s * 1e6, 2),
+                               "GBps": round(nbytes / s / 1e9, 1)})
+        out[style + "_step_us"] = round(total * 1e6, 2)
     del buf
     return out
 
