@@ -36,9 +36,13 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 # (profiles/marlin_stream_fast_kernel_llama3-8b-layer_m16_hbm-traffic.txt): FETCH_SIZE scaled
 # by 2.000 and WRITE_SIZE by 1.000, the factors that make the `--calibrate` pass (256 MiB
 # read, 256 MiB written) come out right.  Average over the four GEMMs of the layer.  Counters
-# cannot be read from inside a run: the figure belongs to the launch shapes of that profile
-# (192 / 256 / 448 / 256 workgroups) and is reported for M = 16 with six weight copies only.
+# cannot be read from inside a run: the figure belongs to the launches of that profile
+# (PROFILED_LAUNCHES: workgroups, threads per workgroup, pieces per strip, non-temporal weight
+# copies, as sonar_marlin_last_decode_launch reports them) and is reported only while the run's
+# own launches are the same, for M = 16 with six weight copies; otherwise `traffic` is null.
 MEASURED_TRAFFIC_M16 = 32_400_000
+PROFILED_LAUNCHES = {"qkv": [192, 512, 2, 0], "o": [256, 512, 4, 0], "gate_up": [448, 256, 1, 1],
+                     "down": [256, 512, 4, 1]}
 REPLAYS = 21                # graph replays per timing; the median is reported
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 MFMA_PEAK_8BIT_TFLOPS = 5000.0   # MI355X dense int8 / fp8
@@ -194,20 +198,32 @@ def launch_floors(torch, time_graph):
 
 def cpu_baseline(threads: int):
     """The layer's CPU path (int4 dequantise + fp32 torch.matmul) from the
-    oracle, on the o_proj shape at M = 16."""
+    oracle at M = 16: `value` on the o_proj shape (BASELINE configuration 1), and
+    the same on the other three projection shapes under `layer` (a bounded sample:
+    one layer's four GEMMs, 2 + 5 runs each, 20 to 30 s of CPU work)."""
     import numpy as np
 
     from oracle import marlin_oracle as mo
-    k, n, m = 4096, 4096, 16
-    layer = mo.make_layer(0, k, n, GROUP, "fp16")
-    a = mo.make_activations(1, m, k, "fp16")
-    t_full, t_mm, _ = mo.cpu_layer_baseline(mo.gptq_pack(layer["q"]), layer["scales"], a, GROUP, threads,
-                                            repeats=5, warmup=2)
-    nbytes = algorithmic_bytes(m, k, n)
-    return {"value": round(nbytes / t_full / 1e9, 3), "unit": "GB/s", "cores": threads, "kind": "port",
+    m = 16
+    rows = []
+    for name, k, n in LAYER_SHAPES:
+        rng = np.random.default_rng(k + n)
+        q = rng.integers(0, 16, size=(k, n), dtype=np.int32)
+        scales = mo.round_to_dtype(rng.uniform(1e-3, 1e-2, size=(k // GROUP, n)).astype(np.float32), "fp16")
+        a = mo.make_activations(1, m, k, "fp16")
+        t_full, t_mm, _ = mo.cpu_layer_baseline(mo.gptq_pack(q), scales, a, GROUP, threads, repeats=5, warmup=2)
+        nbytes = algorithmic_bytes(m, k, n)
+        rows.append({"gemm": name, "k": k, "n": n, "m": m, "ms": round(t_full * 1e3, 2),
+                     "matmul_alone_ms": round(t_mm * 1e3, 2), "GBps": round(nbytes / t_full / 1e9, 3),
+                     "gflops": round(2 * m * n * k / t_full / 1e9, 2)})
+        del q, scales
+    o = next(r for r in rows if r["gemm"] == "o")
+    return {"value": o["GBps"], "unit": "GB/s", "cores": threads, "kind": "port",
             "sample": "o_proj 4096x4096, M=16, fp16: dequantise+matmul fp32, median of 5 "
-                      f"({t_full * 1e3:.1f} ms; matmul alone {t_mm * 1e3:.1f} ms)",
-            "gflops": round(2 * m * n * k / t_full / 1e9, 2)}
+                      f"({o['ms']:.1f} ms; matmul alone {o['matmul_alone_ms']:.1f} ms); `layer`: the same on "
+                      "all four projection shapes",
+            "gflops": o["gflops"], "layer": rows,
+            "layer_ms": round(sum(r["ms"] for r in rows), 2)}
 
 
 def variants_sweep(torch, ops, gen, time_graph):
@@ -460,6 +476,18 @@ def main() -> int:
         step(i)
     torch.cuda.synchronize()
 
+    # the launch every GEMM of the step makes (read back from the library, one eager call each)
+    import ctypes
+    from sonar_amd import _lib
+    lib = _lib.load()
+    launch_shapes = {}
+    for idx, (name, k, n) in enumerate(LAYER_SHAPES):
+        copies[0][idx].run(ops, acts[k], wtype)
+        shape = (ctypes.c_int32 * 4)()
+        lib.sonar_marlin_last_decode_launch(shape, 4)
+        launch_shapes[name] = list(shape)
+    torch.cuda.synchronize()
+
     if args.calibrate:
         x = torch.zeros(64 * 1024 * 1024, dtype=torch.int32, device="cuda:0")
         for _ in range(3):
@@ -525,7 +553,9 @@ def main() -> int:
         "tflops": round(step_flops / step_s / 1e12, 2),
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_M16 if (m == 16 and args.copies == 6) else None,
+                     "traffic": MEASURED_TRAFFIC_M16 if (m == 16 and args.copies == 6 and
+                                                         launch_shapes == PROFILED_LAUNCHES) else None,
+                     "launches": launch_shapes,
                      "kernel": kernel,
                      "bytes_per_launch": step_bytes // launches,
                      "us_per_launch": round(step_s / launches * 1e6, 3)},
@@ -624,6 +654,10 @@ def main() -> int:
     floors = launch_floors(torch, time_graph)
     if floors is not None:
         out["floors"] = floors
+        # how far the step is from a kernel that only streams the same weights (the faster of the copy styles)
+        floor_us = min(floors[k] for k in floors if k.endswith("_step_us"))
+        out["roofline"]["stream_floor_us"] = floor_us
+        out["roofline"]["step_over_stream_floor"] = round(step_s * 1e6 / floor_us, 3)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline(min(os.cpu_count() or 1, 16))
     print(json.dumps(out))

@@ -87,6 +87,16 @@ extern "C" {
 const char* sonar_marlin_last_error(void);
 const char* sonar_marlin_version(void);
 
+/* The launch the calling thread's last sonar_marlin_gemm / _nvfp4 / _noalloc call made with the
+ * decode kernel (no counterpart in the reference; for benchmarks that quote per-launch counter
+ * figures and must know that the launch shapes are still the profiled ones).  Fills
+ *   out[0]  workgroups of the launch (0: the last call did not run the decode kernel)
+ *   out[1]  threads per workgroup
+ *   out[2]  pieces every strip was cut into along K
+ *   out[3]  1 when the weight copies carried the non-temporal bit
+ * and returns the number of entries written (at most n). */
+int sonar_marlin_last_decode_launch(int32_t* out, int n);
+
 /* GPTQ (K/8, N) int32, nibble k%8 of word [k/8][n] = code of W[k][n]
  * -> Marlin (K/16, 2N) int32; with num_bits == 8: (K/4, N) int32, byte k%4
  * -> Marlin (K/16, 4N) int32.  perm (int32[K], may be NULL) selects source
@@ -287,9 +297,13 @@ int sonar_marlin_gemm_nvfp4(const void* a, int64_t a_row_stride, void* c,
  * partial tiles of strips or tiles whose K range is shared between workgroups; with act-order the
  * column-permuted copy of A when it fits) is a static array in device memory of 24 MiB, one
  * per GPU, held until the process ends.  The call allocates and frees nothing.  A call whose
- * sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k) exceeds 24 MiB fails with
- * SONAR_E_INVALID and launches nothing (every size_m <= 128 fits for any matrix; beyond that
- * only calls whose K range is split over many workgroups can exceed it).  All calls on one
+ * sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k) exceeds 24 MiB (K split over many
+ * workgroups of the tile kernels: 65 to 128 rows on K >= 8192, or 97 to 128 rows on N = 28672,
+ * take 56 MiB) still runs: the 8 MiB of the streaming kernels always fit, and the tile kernels
+ * split K only as far as their partial tiles fit (another order of summation than
+ * sonar_marlin_gemm's, slower, the same tolerance).  What cannot make do is refused with
+ * SONAR_E_INVALID before anything is launched: act-order with 8-bit weights or with
+ * is_k_full = 0 needs the copy of A (size_m * size_k * 2 bytes) inside the array.  All calls on one
  * GPU share that GPU's array: calls that overlap in time on one GPU (two streams, two
  * threads) race and give wrong results; calls on one stream, or ordered by events, do not.
  * Nothing in the array has to be zero between calls.  The first call on a device looks the

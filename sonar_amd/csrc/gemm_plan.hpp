@@ -22,7 +22,9 @@ struct GemmPlan {
 // the decode kernel is two times ahead).  `wide128`: the call is one that form takes (4-bit integer codes
 // with groups of 64 * 2^i rows or one group, no act-order gather).
 inline bool plan_rows_97_128(int64_t size_m, int64_t size_n, int64_t size_k, bool wide128) {
-  return wide128 && size_m > 96 && size_m <= 128 && size_n > 16384 && size_k <= 8192 && size_k % 256 == 0;
+  // (up to 128 tiles of 256 columns: beyond that K is not split and the tile kernel is not planned)
+  return wide128 && size_m > 96 && size_m <= 128 && size_n > 16384 && size_n <= 32768 && size_k <= 8192 &&
+         size_k % 256 == 0;
 }
 
 inline GemmPlan plan_gemm(int64_t size_m, int64_t size_n, int64_t size_k, bool async_tile, int tile_rows = 256,

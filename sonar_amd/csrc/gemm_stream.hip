@@ -1713,6 +1713,7 @@ using namespace sonar;
 
 namespace {
 size_t stream_scratch_bytes() { return (size_t)2 * cu_count() * kSlotFloat4 * sizeof(float4); }
+thread_local int32_t g_last_decode_launch[4] = {0, 0, 0, 0};
 }  // namespace
 
 
@@ -1727,7 +1728,11 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
                     const void* b_bias, const void* b_scales, const float* global_scale, const uint32_t* b_zeros,
                     const int32_t* g_idx, const int32_t* perm, int32_t* workspace, int64_t workspace_len,
                     void* scratch, size_t scratch_bytes, int dtype, int64_t b_type_id, int64_t size_m,
-                    int64_t size_n, int64_t size_k, int64_t num_groups, int is_k_full, void* stream) {
+                    int64_t size_n, int64_t size_k, int64_t num_groups, int is_k_full, void* stream,
+                    bool make_do = false) {
+  // `make_do`: the scratch buffer is of a fixed size (sonar_marlin_gemm_noalloc): beyond the
+  // partial tiles of the streaming kernels, which always fit, the call uses what room there is
+  // (no K split in the tile kernels without room for their partial tiles).
   SONAR_REQUIRE(size_m >= 0 && size_m < (1LL << 30), "size_m = %ld out of range", (long)size_m);
   Checked chk;
   if (int rc = check_common(chk, b_layout, b_scales, b_zeros, g_idx, perm, dtype, b_type_id, size_n,
@@ -1744,13 +1749,22 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
   // (all zero again when the kernel ends; nobody ever waits on one).
   SONAR_REQUIRE(workspace && workspace_len >= cus,
                 "workspace.numel = %ld is below min_workspace_size = %d", (long)workspace_len, cus);
-  SONAR_REQUIRE(scratch && scratch_bytes >= sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k),
+  SONAR_REQUIRE(scratch && scratch_bytes >= (make_do ? stream_scratch_bytes()
+                                                     : sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k)),
                 "scratch of %zu bytes is too small", scratch_bytes);
 
+  g_last_decode_launch[0] = 0;
   hipStream_t st = (hipStream_t)stream;
   // Act-order with room in the scratch buffer for a copy of A: permute the
   // columns of A once and run the plain grouped kernels on the copy.
-  const size_t base_scratch = sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k);
+  size_t base_scratch = sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k);
+  if (make_do) {   // the copy of A goes before the tile kernels' partial tiles when both do not fit
+    const size_t copy_bytes = chk.has_perm ? (size_t)size_m * size_k * 2 : 0;
+    const size_t left = scratch_bytes > stream_scratch_bytes() + copy_bytes
+                            ? scratch_bytes - stream_scratch_bytes() - copy_bytes : 0;
+    if (base_scratch > stream_scratch_bytes() + left) base_scratch = stream_scratch_bytes() + left;
+    base_scratch &= ~(size_t)255;
+  }
   if (chk.has_perm && scratch_bytes >= base_scratch + (size_t)size_m * size_k * 2) {
     uint16_t* a_tmp = reinterpret_cast<uint16_t*>(static_cast<char*>(scratch) + base_scratch);
     const long vecs = (long)size_m * (size_k / 8);
@@ -1840,8 +1854,13 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
   // the row -> group lookup and 8-bit codes exist in the streaming kernels only
   // (MXFP4 only through the asynchronous tile kernel: the older one has no float4 dequantiser)
   // (8-bit codes and MXFP4 only through the asynchronous tile kernel: the older one has neither dequantiser)
+  // (a fixed scratch buffer without room for the partial tiles of up to 128 rows: the tile kernel
+  // is planned for those only because K can be split, so they go to the streaming kernels)
+  const size_t tile_room = base_scratch > stream_scratch_bytes() ? base_scratch - stream_scratch_bytes() : 0;
+  const bool tile_starved = make_do && size_m <= 128 && plan.k_splits > 1 &&
+                            tile_room < plan_partial_bytes_any(size_m, size_n, size_k);
   const bool use_tile = plan.tile && !no_tile && !chk.row_groups && ((chk.bits == 4 && !chk.fp4) || async_tile) &&
-                        !(slab_fast && p.unit_chunks == 4);
+                        !(slab_fast && p.unit_chunks == 4) && !tile_starved;
   // More than 64 rows in the general kernels (8-bit codes, is_k_full = false,
   // the tile path switched off) on a matrix of short strips: one workgroup per
   // strip as well, so that every 64-row slab can run in the same launch and the
@@ -1870,8 +1889,8 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
   if (use_tile) {
     const size_t used = stream_scratch_bytes();
     return tile_gemm(a, a_row_stride, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, perm, dtype, size_m,
-                     size_n, size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used,
-                     scratch_bytes > used ? scratch_bytes - used : 0, chk.fp4, chk.bits, chk.fp8, st);
+                     size_n, size_k, num_groups, chk.group_size, static_cast<char*>(scratch) + used, tile_room,
+                     chk.fp4, chk.bits, chk.fp8, st);
   }
 
   // The fast kernel: up to 16 rows, or more rows in blocks of 16 or 32 (slab_fast), all in
@@ -1927,6 +1946,10 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
       p.xcd_ranges = p.slabs == 1 && p.parts % 8 == 0;
     }
     p.nt_weights = p.slabs == 1 && size_k * size_n / 2 >= 20 * 1000 * 1000;
+    g_last_decode_launch[0] = p.grid_parts * p.slabs;
+    g_last_decode_launch[1] = half ? 256 : 512;
+    g_last_decode_launch[2] = 1 << shift;
+    g_last_decode_launch[3] = p.nt_weights;
     int rc;
     if (chk.fp4)   // groups of 32 rows: never in blocks of rows (slab_fast is off), so one block of 16 rows
       rc = launch_fast_fp4<false>(p, half, st);
@@ -1990,6 +2013,12 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
 
 }  // namespace
 
+extern "C" int sonar_marlin_last_decode_launch(int32_t* out, int n) {
+  int i = 0;
+  for (; out != nullptr && i < n && i < 4; ++i) out[i] = g_last_decode_launch[i];
+  return i;
+}
+
 extern "C" int sonar_marlin_gemm(const void* a, int64_t a_row_stride, void* c,
                                  const uint32_t* b_q_weight, int b_layout, const void* b_bias,
                                  const void* b_scales, const uint32_t* b_zeros, const int32_t* g_idx,
@@ -2045,19 +2074,13 @@ extern "C" int sonar_marlin_gemm_noalloc(const void* a, int64_t a_row_stride, vo
     SONAR_REQUIRE(base != nullptr, "hipGetSymbolAddress returned no address for the static scratch array");
     __atomic_store_n(&g_static_scratch[dev], base, __ATOMIC_RELEASE);
   }
-  const size_t need = sonar_marlin_gemm_scratch_bytes(size_m, size_n, size_k);
-  if (need > kStaticScratchBytes)
-    return fail(SONAR_E_INVALID,
-                "sonar_marlin_gemm_noalloc: size_m, size_n, size_k = %ld, %ld, %ld need %zu bytes of scratch, "
-                "the static array holds %zu; call sonar_marlin_gemm with a buffer of the caller's",
-                (long)size_m, (long)size_n, (long)size_k, need, kStaticScratchBytes);
-  // an act-order call also gets room for the column-permuted copy of A when that fits
-  size_t give = need;
-  if (perm != nullptr && need + (size_t)size_m * (size_t)size_k * 2 <= kStaticScratchBytes)
-    give = need + (size_t)size_m * (size_t)size_k * 2;
-  return sonar_marlin_gemm(a, a_row_stride, c, b_q_weight, b_layout, b_bias, b_scales, b_zeros, g_idx, perm,
-                           workspace, workspace_len, base, give, dtype, b_type_id, size_m, size_n, size_k,
-                           num_groups, is_k_full, use_atomic_add, use_fp32_reduce, stream);
+  // The whole array: the call takes what it needs of it and makes do where that is less than
+  // sonar_marlin_gemm_scratch_bytes() (the partial tiles of the streaming kernels, 8 MiB, always
+  // fit; a tile launch whose partial tiles do not runs without splitting K).
+  static_assert(kStaticScratchBytes >= ((size_t)16 << 20), "room for the streaming kernels' partial tiles");
+  return marlin_gemm_any(a, a_row_stride, c, b_q_weight, b_layout, b_bias, b_scales, nullptr, b_zeros, g_idx, perm,
+                         workspace, workspace_len, base, kStaticScratchBytes, dtype, b_type_id, size_m, size_n,
+                         size_k, num_groups, is_k_full, stream, true);
 }
 
 extern "C" int sonar_marlin_dequant(const uint32_t* b_q_weight, int b_layout, const void* b_scales,

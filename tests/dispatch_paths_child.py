@@ -27,6 +27,7 @@ DENSE = [
     (1100, 512, 1024, -1, "bf16", False, False),
     (2100, 512, 4096, 128, "bf16", True, True),     # 144 tiles of 256 rows: the wide tile kernel's 256-row form
     (600, 1024, 768, 32, "fp16", True, False),      # groups of 32 rows in either tile kernel
+    (128, 1024, 40960, 128, "fp16", False, False),  # 97..128 rows on more than 512 strips: one launch of row blocks
 ]
 
 

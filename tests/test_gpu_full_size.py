@@ -6,9 +6,11 @@ oracle is applied to sampled output columns only: the GPTQ words of those column
 are unpacked and dequantised on the CPU (oracle.unpack_rows / oracle.dequantize)
 and multiplied with the activations in fp32.  Every real launch shape of the
 decode sweep (M = 1 .. 64 on the four Llama-3-8B projections), of the prefill
-sweep (M = 1024, 8192) and of the Mixtral-sized grouped GEMM at 4096 tokens
-meets the oracle this way.  Tolerance: max|err| <= 1e-2 max|ref| and
-|err| <= 1e-2 max|ref| + 1e-2 |ref| (oracle.gemm_tolerance_ok)."""
+sweep (M = 256, 1024, 4096, 8192 on the same four), of the Mixtral-sized grouped
+GEMMs at 16 and 4096 tokens and of the W4A8 shapes the benchmark times (K = 4096,
+N = 11008 dense; Mixtral-sized experts grouped) meets the oracle this way.
+Tolerance: max|err| <= 1e-2 max|ref| and |err| <= 1e-2 max|ref| + 1e-2 |ref|
+(oracle.gemm_tolerance_ok); int8 activations: bit for bit."""
 from __future__ import annotations
 
 import numpy as np
@@ -106,10 +108,11 @@ def test_decode_sweep_meets_the_oracle_on_sampled_columns(name, m):
     assert torch.equal(c.view(torch.int16), c2.view(torch.int16))
 
 
-@pytest.mark.parametrize("m", [1024, 8192])
-@pytest.mark.parametrize("name", ["gate_up", "down"])
+@pytest.mark.parametrize("m", [256, 1024, 4096, 8192])
+@pytest.mark.parametrize("name", list(LLAMA))
 def test_prefill_sweep_meets_the_oracle_on_sampled_columns(name, m):
-    """Benchmark configuration 3: fp16 activations ~ N(0, 0.5)."""
+    """Benchmark configuration 3: fp16 activations ~ N(0, 0.5), every M of the sweep on every
+    projection shape (the launches the benchmark's MFMA figure is made of among them)."""
     layer = big_layer(name, "fp16")
     gen = torch.Generator(device=gu.DEV).manual_seed(m)
     a = (torch.randn((m, layer.k), device=gu.DEV, generator=gen) * 0.5).to(torch.float16)
@@ -119,16 +122,29 @@ def test_prefill_sweep_meets_the_oracle_on_sampled_columns(name, m):
     check_columns(layer, a, c, m, sampled_columns(layer.n, 6, m))
 
 
+_experts = {}
+
+
+def mixtral_experts(k, n):
+    """Eight experts of one Mixtral-sized matrix, kept for the cases that share them."""
+    if (k, n) not in _experts:
+        _experts.clear()                      # one set at a time: 0.5 GB of device memory each
+        _layers.clear()
+        _experts[(k, n)] = [BigLayer(50 + i, k, n, "bf16") for i in range(8)]
+    return _experts[(k, n)]
+
+
+@pytest.mark.parametrize("tokens", [16, 4096])
 @pytest.mark.parametrize("k,n,top_k,mul", [(4096, 28672, 2, False), (14336, 4096, 1, True)])
-def test_mixtral_sized_grouped_gemm_at_4096_tokens(k, n, top_k, mul):
-    """Benchmark configuration 5 at T = 4096 on the real expert shapes (w13: K = 4096,
-    N = 28672 with top-2 routing; w2: K = 14336, N = 4096 on the 8192 routed rows with
-    the routing weights multiplied in): 64-slot blocks, the tiled grouped kernel.  Every
-    routed row is checked on sampled columns against the oracle, and sampled rows
-    against the dense GEMM of that row with its expert."""
+def test_mixtral_sized_grouped_gemm(k, n, top_k, mul, tokens):
+    """Benchmark configuration 5 at T = 16 and T = 4096 on the real expert shapes (w13: K = 4096,
+    N = 28672 with top-2 routing; w2: K = 14336, N = 4096 on the routed rows with the routing
+    weights multiplied in): 8-slot blocks in the grouped decode kernel, 64-slot blocks in the
+    tiled grouped kernel.  Every routed row is checked on sampled columns against the oracle,
+    and sampled rows against the dense GEMM of that row with its expert."""
     from sonar_amd import fused_moe, marlin_utils
-    tokens, e = 4096, 8
-    experts = [BigLayer(50 + i, k, n, "bf16") for i in range(e)]
+    e = 8
+    experts = mixtral_experts(k, n)
     native = torch.stack([x.native for x in experts]).contiguous()
     scales = torch.stack([x.scales for x in experts]).contiguous()
     gen = torch.Generator(device=gu.DEV).manual_seed(9)
@@ -136,7 +152,7 @@ def test_mixtral_sized_grouped_gemm_at_4096_tokens(k, n, top_k, mul):
     tw2, ti2 = torch.topk(torch.softmax(logits, dim=1), 2, dim=1)
     ti2 = ti2.to(torch.int32)
     bs = fused_moe.moe_block_size(tokens, 2, e)
-    assert bs == 64
+    assert bs == (64 if tokens == 4096 else 8)
     sorted_ids, expert_ids, past = fused_moe.moe_align_block_size(ti2, bs, e)
     rows_a = tokens if top_k == 2 else tokens * 2     # the second GEMM of a layer takes one row per routed slot
     a = (torch.randn((rows_a, k), device=gu.DEV, generator=gen) * 0.5).to(torch.bfloat16)
@@ -184,3 +200,127 @@ def test_mixtral_sized_grouped_gemm_at_4096_tokens(k, n, top_k, mul):
             dense = (dense.to(torch.bfloat16) * tw[r].to(torch.bfloat16)).float()
         err = float((dense - c[r].float()).abs().max())
         assert err <= 1e-2 * scale, (int(r), err, scale)
+
+
+# ---------------------------------------------------------------------------
+# W4A8 at the sizes the benchmark times
+class BigA8Layer:
+    """uint4b8 weights drawn on the device in the order of 8-bit activations, groups of 128 rows."""
+
+    def __init__(self, seed, k, n, dtype, act):
+        from tests.test_gpu_a8 import _a8_to_gfx950, _repack_a8
+        self.k, self.n, self.dtype, self.act = k, n, dtype, act
+        self.tdt = torch.float16 if dtype == "fp16" else torch.bfloat16
+        gen = torch.Generator(device=gu.DEV).manual_seed(seed)
+        self.qweight = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 8, n), dtype=torch.int32, device=gu.DEV,
+                                     generator=gen)
+        words = self.qweight
+        if act == "fp8":     # sign-and-magnitude nibbles, as marlin_int4_fp8_preprocess leaves them
+            words = torch.empty_like(self.qweight)
+            _lib.check(_lib.load().sonar_marlin_int4_fp8_preprocess(gu.ptr(self.qweight), None, gu.ptr(words),
+                                                                     k // 8, n, 0, gu.stream()))
+        self.native = _a8_to_gfx950(_repack_a8(words, k, n), k, n)
+        rng = np.random.default_rng(seed)
+        s = mo.round_to_dtype(rng.uniform(1e-3, 1e-2, size=(k // GROUP, n)).astype(np.float32), dtype)
+        self.factor = np.float32(1.0)
+        if act == "int8":
+            self.scales, self.factor = mo.marlin_act_int8_process_scales(s)      # 16-bit integers
+            self.dev_scales = torch.from_numpy(mo.marlin_permute_scales_a8(self.scales, k, n, GROUP).copy()).to(gu.DEV)
+        else:
+            self.scales = mo.round_to_dtype(s * np.float32(512.0), dtype)
+            self.dev_scales = gu.dev_bits16(mo.marlin_permute_scales_a8(self.scales, k, n, GROUP), dtype)
+
+    def q_columns(self, cols):
+        idx = torch.as_tensor(cols, device=gu.DEV)
+        return mo.unpack_rows(self.qweight[:, idx].cpu().numpy())
+
+    def gemm(self, a_dev, a_scales_dev, m):
+        lib = _lib.load()
+        c = torch.full((m, self.n), float("nan"), dtype=self.tdt, device=gu.DEV)
+        nbytes = lib.sonar_marlin_gemm_a8_scratch_bytes(m, self.n, self.k, self.k // GROUP)
+        scratch = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=gu.DEV)
+        _lib.check(lib.sonar_marlin_gemm_a8(
+            gu.ptr(a_dev), self.k, _lib.ADTYPE_INT8 if self.act == "int8" else _lib.ADTYPE_FP8, gu.ptr(c),
+            gu.ptr(self.native), _lib.LAYOUT_GFX950, None, gu.ptr(self.dev_scales), gu.ptr(a_scales_dev), None,
+            gu.ptr(scratch), scratch.numel(), gu.dtype_code(self.dtype), _lib.TYPE_UINT4B8, m, self.n, self.k,
+            self.k // GROUP, gu.stream()))
+        return c
+
+
+@pytest.mark.parametrize("m", [1, 64, 512, 4096])
+def test_w4a8_int8_at_benchmark_size_bit_exact_on_sampled_columns(m):
+    """K = 4096, N = 11008 (the shape bench.py times W4A8 on): the slab kernel and the tiled
+    kernel with many tiles and no K split, bit for bit against the oracle."""
+    k, n = 4096, 11008
+    layer = BigA8Layer(700, k, n, "fp16", "int8")
+    rng = np.random.default_rng(m)
+    a_q, a_s = mo.per_token_quant_int8(rng.standard_normal((m, k)).astype(np.float32))
+    a_s = (a_s * layer.factor).astype(np.float32)
+    got = layer.gemm(torch.from_numpy(a_q).to(gu.DEV), torch.from_numpy(a_s.reshape(-1)).to(gu.DEV), m)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(got.float()).all())
+    cols = sampled_columns(n, 8, m)
+    want = mo.gemm_w4a8_int8(a_q, a_s, layer.q_columns(cols), GROUP, layer.scales[:, cols], "fp16")
+    have = got[:, torch.as_tensor(cols, device=gu.DEV)].float().cpu().numpy()
+    assert np.array_equal(have, want), np.abs(have - want).max()
+
+
+@pytest.mark.parametrize("m", [64, 4096])
+def test_w4a8_fp8_at_benchmark_size_on_sampled_columns(m):
+    k, n = 4096, 11008
+    layer = BigA8Layer(701, k, n, "bf16", "fp8")
+    g = torch.Generator().manual_seed(m)
+    x = torch.randn((m, k), generator=g)
+    a_s = (x.abs().amax(dim=1, keepdim=True) / 448.0).clamp_min(1e-10)
+    a_fp8 = (x / a_s).to(torch.float8_e4m3fn)
+    got = layer.gemm(a_fp8.view(torch.uint8).to(gu.DEV), a_s.reshape(-1).to(gu.DEV), m)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(got.float()).all())
+    cols = sampled_columns(n, 8, m)
+    want = mo.gemm_w4a8_fp8(a_fp8.float().numpy(), a_s.numpy(), layer.q_columns(cols), GROUP,
+                            layer.scales[:, cols] / np.float32(512.0))
+    have = got[:, torch.as_tensor(cols, device=gu.DEV)].float().cpu().numpy()
+    ok, err, big = mo.gemm_tolerance_ok(have, want)
+    assert ok, (err, big)
+
+
+def test_w4a8_int8_grouped_at_mixtral_size_bit_exact_on_sampled_columns():
+    """The grouped W4A8 entry point on 64-slot blocks at the size bench.py times (8 experts of
+    K = 4096, N = 28672, 4096 tokens, top 2): every routed row on sampled columns, bit for bit."""
+    from sonar_amd import fused_moe
+    _layers.clear()
+    _experts.clear()
+    tokens, e, k, n, top_k = 4096, 8, 4096, 28672, 2
+    experts = [BigA8Layer(720 + i, k, n, "bf16", "int8") for i in range(e)]
+    # one factor for all experts, as the reference's layer-wide maximum gives
+    factor = experts[0].factor
+    native = torch.stack([x.native for x in experts]).contiguous()
+    scales = torch.stack([x.dev_scales for x in experts]).contiguous()
+    gen = torch.Generator(device=gu.DEV).manual_seed(11)
+    logits = torch.randn((tokens, e), device=gu.DEV, generator=gen)
+    tw2, ti2 = torch.topk(torch.softmax(logits, dim=1), top_k, dim=1)
+    ti2 = ti2.to(torch.int32)
+    bs = 64
+    sorted_ids, expert_ids, past = fused_moe.moe_align_block_size(ti2, bs, e)
+    rng = np.random.default_rng(5)
+    a_q, a_s = mo.per_token_quant_int8(rng.standard_normal((tokens, k)).astype(np.float32))
+    a_s = (a_s * factor).astype(np.float32)
+    d_a, d_as = torch.from_numpy(a_q).to(gu.DEV), torch.from_numpy(a_s.reshape(-1).copy()).to(gu.DEV)
+    c = torch.full((tokens * top_k, n), float("nan"), dtype=torch.bfloat16, device=gu.DEV)
+    tw = tw2.reshape(-1).contiguous().float()
+    lib = _lib.load()
+    _lib.check(lib.sonar_moe_wna16_marlin_gemm_a8(
+        gu.ptr(d_a), _lib.ADTYPE_INT8, gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None, gu.ptr(scales),
+        gu.ptr(d_as), None, gu.ptr(sorted_ids), sorted_ids.numel(), gu.ptr(expert_ids), gu.ptr(past), gu.ptr(tw),
+        bs, top_k, 0, e, _lib.DTYPE_BF16, _lib.TYPE_UINT4B8, tokens, n, k, k // GROUP, gu.stream()))
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(c.float()).all()), "a routed row was not written"
+    cols = sampled_columns(n, 6, 3)
+    have = c[:, torch.as_tensor(cols, device=gu.DEV)].float().cpu().numpy()
+    ids = ti2.reshape(-1).cpu().numpy()
+    want = np.zeros_like(have)
+    for ex in range(e):
+        rows = np.nonzero(ids == ex)[0]
+        want[rows] = mo.gemm_w4a8_int8(a_q[rows // top_k], a_s.reshape(-1)[rows // top_k], experts[ex].q_columns(cols),
+                                       GROUP, experts[ex].scales[:, cols], "bf16")
+    assert np.array_equal(have, want), np.abs(have - want).max()

@@ -717,6 +717,53 @@ def test_gemm_w4a8_int8_against_python_loop(group_size, zp):
             assert got[mm, nn] == np.float32(want).astype(np.float16).astype(np.float32)
 
 
+def test_moe_gemm_w4a8_int8_against_per_slot_loop():
+    """moe_gemm_w4a8_int8 (the checker of the grouped W4A8 GPU tests) walks sorted_ids /
+    expert_ids block by block.  The same result from the routing alone, one routed slot at a
+    time in plain Python integers: C[t * top_k + j] = (sum_g s[e][g][n] * sum_{k in g}
+    a[t][k] * (q[e][k][n] - z)) * a_scale[t] for e = topk_ids[t][j], rounded, times the rounded
+    routing weight, rounded.  A wrong row (id % top_k for id // top_k), a wrong expert, the
+    activation scale of another row, a block skipped or written twice, or the routing weight
+    applied before the rounding all fail it."""
+    rng = np.random.default_rng(21)
+    m, e, top_k, k, n, bs, gs = 9, 4, 2, 64, 8, 8, 32
+    a = rng.integers(-127, 128, size=(m, k)).astype(np.int8)
+    a_s = rng.uniform(1e-6, 2e-6, size=(m, 1)).astype(np.float32)
+    experts = []
+    for _ in range(e):
+        experts.append(dict(q=rng.integers(0, 16, size=(k, n), dtype=np.int32), group_size=gs,
+                            scales=rng.integers(1, 4097, size=(k // gs, n)).astype(np.int16),
+                            zeros=rng.integers(0, 16, size=(k // gs, n), dtype=np.int32), bias32=None))
+    topk_ids = np.stack([rng.permutation(e)[:top_k] for _ in range(m)]).astype(np.int32)
+    weights = rng.uniform(0.1, 1.0, size=(m, top_k)).astype(np.float32)
+    sorted_ids, expert_ids, past = mo.moe_align_block_size(topk_ids, bs, e)
+    for dtype in ("fp16", "bf16"):
+        for tw in (None, weights):
+            got = mo.moe_gemm_w4a8_int8(a, a_s, experts, sorted_ids, expert_ids, int(past[0]), bs, top_k, tw, dtype)
+            for t in range(m):
+                for j in range(top_k):
+                    ex = experts[int(topk_ids[t, j])]
+                    for col in range(n):
+                        total = 0
+                        for g in range(k // gs):
+                            part = sum(int(a[t, kk]) * (int(ex["q"][kk, col]) - int(ex["zeros"][g, col]))
+                                       for kk in range(g * gs, (g + 1) * gs))
+                            total += part * int(ex["scales"][g, col])
+                        assert -2 ** 31 <= total < 2 ** 31          # no wrap in this case
+                        want = mo.round_to_dtype(np.array([np.float32(total) * a_s[t, 0]], np.float32), dtype)[0]
+                        if tw is not None:
+                            wt = mo.round_to_dtype(np.array([tw[t, j]], np.float32), dtype)[0]
+                            want = mo.round_to_dtype(np.array([want * wt], np.float32), dtype)[0]
+                        assert want != 0 and got[t * top_k + j, col] == want, (dtype, t, j, col)
+    # a block of an expert held elsewhere (-1) writes nothing
+    skipped = expert_ids.copy()
+    skipped[0] = -1
+    got = mo.moe_gemm_w4a8_int8(a, a_s, experts, sorted_ids, skipped, int(past[0]), bs, top_k, None, "fp16")
+    dropped = sorted_ids[:bs]
+    dropped = dropped[dropped < m * top_k]
+    assert dropped.size > 0 and np.all(got[dropped] == 0)
+
+
 def test_gemm_w4a8_limit_cases():
     # all integer group scales equal to c: the result is c * (a @ (q - 8)), the textbook product
     rng = np.random.default_rng(8)
