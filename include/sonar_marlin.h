@@ -400,6 +400,31 @@ int sonar_silu_and_mul(void* out, const void* in, int64_t rows, int64_t d, int d
 int sonar_moe_sum(void* out, const void* in, int64_t tokens, int64_t topk, int64_t d, int dtype,
                   void* stream);
 
+/* The other gated activations apply_moe_activation dispatches between the two grouped GEMMs
+ * (aphrodite/model_executor/layers/fused_moe/activation.py:128-205): in is [rows][2 d] (gate half,
+ * then up half; SONAR_ACT_SWIGLUOAI: gate and up alternate), out is [rows][d], T the 16-bit type.
+ *   SONAR_ACT_SILU_CLAMP  _C::silu_and_mul_with_clamp(out, in, limit, alpha, beta)
+ *        (torch_bindings.cpp:644-649, activation_kernels.cu:28-76,154-160): SILU with clamp_limit,
+ *        and SWIGLUOAI_UNINTERLEAVE (the experts of gpt-oss in the packed gate | up order):
+ *        g = T(min(gate, limit)), u = clamp(up, -limit, limit),
+ *        out = T(float(T(g / (1 + exp(-alpha g)))) * (u + beta))
+ *   SONAR_ACT_GELU / SONAR_ACT_GELU_TANH  _C::gelu_and_mul / gelu_tanh_and_mul (activation_kernels.cu:172-215)
+ *   SONAR_ACT_SWIGLUOAI   _C::swigluoai_and_mul(out, in, alpha = 1.702, limit = 7.0)
+ *        (activation_kernels.cu:412-423): out = T((u + 1) g / (1 + exp(-alpha g))), g = min(gate, limit),
+ *        u = clamp(up, -limit, limit)
+ *   SONAR_ACT_SITU        _C::situ_and_mul(out, in, beta, linear_beta) (activation_kernels.cu:489-510):
+ *        `alpha` carries beta, `beta` carries linear_beta (<= 0: up passes through)
+ *   SONAR_ACT_SWIGLUSTEP  swiglustep_and_mul_triton (aphrodite/model_executor/layers/activation.py:27-72):
+ *        out = T(min(silu(gate), limit) * clamp(up, -limit, limit)) */
+#define SONAR_ACT_SILU_CLAMP 1
+#define SONAR_ACT_GELU 2
+#define SONAR_ACT_GELU_TANH 3
+#define SONAR_ACT_SWIGLUOAI 4
+#define SONAR_ACT_SITU 5
+#define SONAR_ACT_SWIGLUSTEP 6
+int sonar_moe_activation(void* out, const void* in, int64_t rows, int64_t d, int kind, float limit,
+                         float alpha, float beta, int dtype, void* stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -1205,6 +1205,89 @@ def moe_block_size_rule(m: int, topk: int, num_experts: int) -> int:
     return 64
 
 
+def moe_activation(name: str, x32: np.ndarray, dtype: str, clamp_limit: float | None = None, alpha: float = 1.0,
+                   beta: float = 0.0, situ_beta: float | None = None, situ_linear_beta: float | None = None) -> np.ndarray:
+    """The activation between the two grouped GEMMs of the fused mixture-of-experts layer
+    (apply_moe_activation, aphrodite/model_executor/layers/fused_moe/activation.py:128-205):
+    x32 holds values of `dtype`, [rows, 2 d] for a gated activation (gate half then up half;
+    "swigluoai": gate and up alternate), [rows, d] for one without a gate; returns [rows, d]
+    values of `dtype`.  Every rounding to `dtype` the reference's kernels make is made here,
+    exp / tanh / erf in float64 (a kernel's float32 functions may differ in the last place):
+      silu                  T(T(g / (1 + e^-g)) * u)      csrc/libtorch_stable/activation_kernels.cu:28-76,157-160
+      silu + clamp_limit,   g = T(min(gate, limit)), u = clamp(up, +-limit):
+      swigluoai_uninterleave  T(T(g / (1 + e^(-alpha g))) * (u + beta))      (:60-75; silu_and_mul_with_clamp)
+      gelu, gelu_tanh       T(T(gelu(g)) * u)             (:172-215)
+      swigluoai             g = min(gate, 7), u = clamp(up, +-7): T((u + 1) g / (1 + e^(-1.702 g)))   (:412-423)
+      situ                  T(b tanh(g / b) / (1 + e^-g) * (lb > 0 ? lb tanh(u / lb) : u))   (:489-510)
+      swiglustep            T(min(g sigmoid(g), 7) * clamp(u, +-7))    (layers/activation.py:27-52)
+      silu_no_mul, gelu_no_mul, gelu_tanh_no_mul   T(f(x));   relu2_no_mul   T(T(max(x, 0))^2)"""
+    x = np.asarray(x32, dtype=np.float64)
+
+    def rnd(v):
+        return round_to_dtype(np.asarray(v, dtype=np.float64).astype(np.float32), dtype).astype(np.float64)
+
+    def erf(v):
+        from math import erf as erf1
+        return np.vectorize(erf1)(v)
+
+    # the two GELU forms in float32 step by step, as the kernels write them: far in the negative
+    # tail 1 + erf(..) cancels, and what is left depends on the float32 sum, not on the function
+    def gelu(v):
+        f = v.astype(np.float32)
+        e = erf((f * np.float32(0.70710678118654752440)).astype(np.float64)).astype(np.float32)
+        return (f * np.float32(0.5) * (np.float32(1.0) + e)).astype(np.float64)
+
+    def gelu_tanh(v):
+        f = v.astype(np.float32)
+        inner = np.float32(0.79788456080286535588) * (f + np.float32(0.044715) * (f * f * f))
+        t = np.tanh(inner.astype(np.float64)).astype(np.float32)
+        return (np.float32(0.5) * f * (np.float32(1.0) + t)).astype(np.float64)
+
+    if name.endswith("_no_mul"):
+        if name == "silu_no_mul":
+            return rnd(x / (1.0 + np.exp(-x))).astype(np.float32)
+        if name == "gelu_no_mul":
+            return rnd(gelu(x)).astype(np.float32)
+        if name == "gelu_tanh_no_mul":
+            return rnd(gelu_tanh(x)).astype(np.float32)
+        if name == "relu2_no_mul":
+            return rnd(rnd(np.maximum(x, 0.0)) ** 2).astype(np.float32)
+        raise ValueError(name)
+    d = x.shape[-1] // 2
+    if name == "swigluoai":
+        g, u = x[..., 0::2], x[..., 1::2]
+        g = np.minimum(g, 7.0)
+        u = np.clip(u, -7.0, 7.0)
+        return rnd((u + 1.0) * g / (1.0 + np.exp(-g * np.float64(np.float32(1.702))))).astype(np.float32)
+    g, u = x[..., :d], x[..., d:]
+    if name == "silu" and clamp_limit is None:
+        return rnd(rnd(g / (1.0 + np.exp(-g))) * u).astype(np.float32)
+    if name in ("silu", "swigluoai_uninterleave"):
+        if clamp_limit is None:
+            raise ValueError("swigluoai_uninterleave needs clamp_limit")
+        a, b = (1.0, 0.0) if name == "silu" else (np.float64(np.float32(alpha)), np.float64(np.float32(beta)))
+        lim = np.float64(np.float32(clamp_limit))
+        gc = rnd(np.minimum(g, lim))
+        uc = np.clip(u, -lim, lim)
+        act = rnd(gc / (1.0 + np.exp(-gc * a)))
+        return rnd(act * (uc + b)).astype(np.float32)
+    if name == "gelu":
+        return rnd(rnd(gelu(g)) * u).astype(np.float32)
+    if name == "gelu_tanh":
+        return rnd(rnd(gelu_tanh(g)) * u).astype(np.float32)
+    if name == "situ":
+        b = np.float64(np.float32(situ_beta))
+        gate_out = b * np.tanh(g / b) / (1.0 + np.exp(-g))
+        up_out = u
+        if situ_linear_beta is not None and situ_linear_beta > 0:
+            lb = np.float64(np.float32(situ_linear_beta))
+            up_out = lb * np.tanh(u / lb)
+        return rnd(gate_out * up_out).astype(np.float32)
+    if name == "swiglustep":
+        return rnd(np.minimum(g / (1.0 + np.exp(-g)), 7.0) * np.clip(u, -7.0, 7.0)).astype(np.float32)
+    raise ValueError(name)
+
+
 def moe_gemm_reference(a32: np.ndarray, w32_per_expert, sorted_ids: np.ndarray,
                        expert_ids: np.ndarray, num_post_pad: int, block_size: int,
                        top_k: int, size_m: int, topk_weights: np.ndarray | None,

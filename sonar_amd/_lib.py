@@ -6,7 +6,7 @@ from __future__ import annotations
 
 import ctypes
 import os
-from ctypes import c_char_p, c_int, c_int64, c_size_t, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_int64, c_size_t, c_void_p
 
 _LIB_PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "lib", "libsonar_marlin.so")
 
@@ -80,6 +80,8 @@ PROTOTYPES = {
     "sonar_moe_align_block_size": (c_int, [c_void_p, c_int64, c_int64, c_int64, c_void_p, c_int64, c_void_p,
                                            c_int64, c_void_p, c_void_p, c_void_p, c_void_p]),
     "sonar_silu_and_mul": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
+    "sonar_moe_activation": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_float, c_float, c_float, c_int,
+                                     c_void_p]),
     "sonar_moe_sum": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int64, c_int, c_void_p]),
 }
 

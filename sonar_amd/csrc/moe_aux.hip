@@ -120,6 +120,94 @@ __global__ __launch_bounds__(256) void silu_and_mul_kernel(uint16_t* __restrict_
   }
 }
 
+// The gated activations of the fused mixture-of-experts layer other than plain SiLU
+// (aphrodite/model_executor/layers/fused_moe/activation.py:128-205 of the reference; the
+// arithmetic of csrc/libtorch_stable/activation_kernels.cu:28-95,154-215,412-423,489-510 and of
+// the Triton kernel aphrodite/model_executor/layers/activation.py:27-52), one (gate, up) pair
+// -> one output, every intermediate rounding where the reference has one:
+//   kClampSilu  silu_and_mul_with_clamp: g = T(min(gate, limit)), u = clamp(up, -limit, limit);
+//               T(float(T(g / (1 + exp(-alpha g)))) * (u + beta))
+//   kGelu       T(float(T(0.5 g (1 + erf(g / sqrt 2)))) * up);  kGeluTanh: the tanh form
+//   kSwigluOai  gate / up interleaved in the input: g = min(gate, limit), u = clamp(up, +-limit);
+//               T((u + 1) * g / (1 + exp(-alpha g)))
+//   kSitu       T(beta tanh(gate / beta) / (1 + exp(-gate)) * (linear_beta > 0 ? linear_beta tanh(up / linear_beta) : up))
+//               (beta in `alpha`, linear_beta in `beta`)
+//   kSwigluStep T(min(gate * sigmoid(gate), limit) * clamp(up, -limit, limit))
+enum MoeActivation { kClampSilu = 1, kGelu = 2, kGeluTanh = 3, kSwigluOai = 4, kSitu = 5, kSwigluStep = 6 };
+
+template <typename T, int KIND>
+__device__ __forceinline__ uint16_t gated_activation(uint16_t gate_bits, uint16_t up_bits, float limit, float alpha,
+                                                     float beta) {
+  const float gate = to_f32<T>(gate_bits), up = to_f32<T>(up_bits);
+  if constexpr (KIND == kClampSilu) {
+    const float g = to_f32<T>(from_f32<T>(fminf(gate, limit)));
+    const float u = fmaxf(fminf(up, limit), -limit);
+    const float act = to_f32<T>(from_f32<T>(g / (1.0f + expf(-g * alpha))));
+    return from_f32<T>(act * (u + beta));
+  } else if constexpr (KIND == kGelu) {
+    const float act = to_f32<T>(from_f32<T>(gate * 0.5f * (1.0f + erff(gate * 0.70710678118654752440f))));
+    return from_f32<T>(act * up);
+  } else if constexpr (KIND == kGeluTanh) {
+    const float inner = 0.79788456080286535588f * (gate + 0.044715f * (gate * gate * gate));
+    const float act = to_f32<T>(from_f32<T>(0.5f * gate * (1.0f + tanhf(inner))));
+    return from_f32<T>(act * up);
+  } else if constexpr (KIND == kSwigluOai) {
+    const float g = fminf(gate, limit);
+    const float u = fmaxf(fminf(up, limit), -limit);
+    return from_f32<T>((u + 1.0f) * g / (1.0f + expf(-g * alpha)));
+  } else if constexpr (KIND == kSitu) {
+    const float gate_out = alpha * tanhf(gate * (1.0f / alpha)) / (1.0f + expf(-gate));
+    const float up_out = beta > 0.0f ? beta * tanhf(up * (1.0f / beta)) : up;
+    return from_f32<T>(gate_out * up_out);
+  } else {
+    const float silu = gate / (1.0f + expf(-gate));
+    return from_f32<T>(fminf(silu, limit) * fmaxf(fminf(up, limit), -limit));
+  }
+}
+
+// in: rows x 2d (gate half then up half; kSwigluOai: gate and up alternate), out: rows x d.
+template <typename T, int KIND>
+__global__ __launch_bounds__(256) void moe_activation_kernel(uint16_t* __restrict__ out,
+                                                            const uint16_t* __restrict__ in, long rows, int d,
+                                                            float limit, float alpha, float beta) {
+  const long vec_per_row = d / 8;
+  const long total = rows * vec_per_row;
+  for (long i = (long)blockIdx.x * blockDim.x + threadIdx.x; i < total; i += (long)gridDim.x * blockDim.x) {
+    const long r = i / vec_per_row;
+    const int c = (int)(i - r * vec_per_row) * 8;
+    uint4 g, u;
+    if constexpr (KIND == kSwigluOai) {   // sixteen values: eight pairs
+      g = *reinterpret_cast<const uint4*>(in + r * 2 * d + 2 * c);
+      u = *reinterpret_cast<const uint4*>(in + r * 2 * d + 2 * c + 8);
+    } else {
+      g = *reinterpret_cast<const uint4*>(in + r * 2 * d + c);
+      u = *reinterpret_cast<const uint4*>(in + r * 2 * d + d + c);
+    }
+    const uint32_t gw[4] = {g.x, g.y, g.z, g.w}, uw[4] = {u.x, u.y, u.z, u.w};
+    uint32_t ow[4];
+#pragma unroll
+    for (int w = 0; w < 4; ++w) {
+      uint32_t o = 0;
+#pragma unroll
+      for (int h = 0; h < 2; ++h) {
+        uint16_t gb, ub;
+        if constexpr (KIND == kSwigluOai) {   // output 2 w + h of these eight: the pair in word 2 w + h of g | u
+          const int pair = 2 * w + h;
+          const uint32_t word = pair < 4 ? gw[pair] : uw[pair - 4];
+          gb = (uint16_t)word;
+          ub = (uint16_t)(word >> 16);
+        } else {
+          gb = (uint16_t)(gw[w] >> (16 * h));
+          ub = (uint16_t)(uw[w] >> (16 * h));
+        }
+        o |= (uint32_t)gated_activation<T, KIND>(gb, ub, limit, alpha, beta) << (16 * h);
+      }
+      ow[w] = o;
+    }
+    *reinterpret_cast<uint4*>(out + r * d + c) = make_uint4(ow[0], ow[1], ow[2], ow[3]);
+  }
+}
+
 // out[t][c] = T(sum_k in[t][k][c]), summed in fp32.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_sum_kernel(uint16_t* __restrict__ out, const uint16_t* __restrict__ in,
@@ -206,6 +294,43 @@ extern "C" int sonar_silu_and_mul(void* out, const void* in, int64_t rows, int64
     silu_and_mul_kernel<__bf16><<<blocks, 256, 0, st>>>(static_cast<uint16_t*>(out),
                                                         static_cast<const uint16_t*>(in), rows, (int)d);
   return launch_status("silu_and_mul_kernel");
+}
+
+namespace {
+template <typename T>
+void launch_moe_activation(int kind, int blocks, hipStream_t st, uint16_t* out, const uint16_t* in, long rows, int d,
+                           float limit, float alpha, float beta) {
+  switch (kind) {
+    case kClampSilu: moe_activation_kernel<T, kClampSilu><<<blocks, 256, 0, st>>>(out, in, rows, d, limit, alpha, beta); break;
+    case kGelu: moe_activation_kernel<T, kGelu><<<blocks, 256, 0, st>>>(out, in, rows, d, limit, alpha, beta); break;
+    case kGeluTanh: moe_activation_kernel<T, kGeluTanh><<<blocks, 256, 0, st>>>(out, in, rows, d, limit, alpha, beta); break;
+    case kSwigluOai: moe_activation_kernel<T, kSwigluOai><<<blocks, 256, 0, st>>>(out, in, rows, d, limit, alpha, beta); break;
+    case kSitu: moe_activation_kernel<T, kSitu><<<blocks, 256, 0, st>>>(out, in, rows, d, limit, alpha, beta); break;
+    default: moe_activation_kernel<T, kSwigluStep><<<blocks, 256, 0, st>>>(out, in, rows, d, limit, alpha, beta); break;
+  }
+}
+}  // namespace
+
+extern "C" int sonar_moe_activation(void* out, const void* in, int64_t rows, int64_t d, int kind, float limit,
+                                    float alpha, float beta, int dtype, void* stream) {
+  SONAR_REQUIRE(dtype == SONAR_DTYPE_F16 || dtype == SONAR_DTYPE_BF16, "unsupported dtype");
+  SONAR_REQUIRE(kind >= SONAR_ACT_SILU_CLAMP && kind <= SONAR_ACT_SWIGLUSTEP, "moe_activation: unknown kind %d", kind);
+  SONAR_REQUIRE(rows >= 0 && d > 0 && d % 8 == 0, "moe_activation: d = %ld must be a positive multiple of 8", (long)d);
+  if (kind == SONAR_ACT_SILU_CLAMP || kind == SONAR_ACT_SWIGLUOAI || kind == SONAR_ACT_SWIGLUSTEP)
+    SONAR_REQUIRE(limit > 0.0f, "moe_activation: this activation needs a positive clamp limit");
+  if (kind == SONAR_ACT_SITU) SONAR_REQUIRE(alpha > 0.0f, "moe_activation: SITU needs a positive beta");
+  if (rows == 0) return SONAR_OK;
+  SONAR_REQUIRE(out && in && ((uintptr_t)out) % 16 == 0 && ((uintptr_t)in) % 16 == 0,
+                "moe_activation: pointers must be 16-byte aligned");
+  hipStream_t st = (hipStream_t)stream;
+  const int blocks = blocks_for(rows * (d / 8));
+  if (dtype == SONAR_DTYPE_F16)
+    launch_moe_activation<_Float16>(kind, blocks, st, static_cast<uint16_t*>(out), static_cast<const uint16_t*>(in),
+                                    rows, (int)d, limit, alpha, beta);
+  else
+    launch_moe_activation<__bf16>(kind, blocks, st, static_cast<uint16_t*>(out), static_cast<const uint16_t*>(in),
+                                  rows, (int)d, limit, alpha, beta);
+  return launch_status("moe_activation_kernel");
 }
 
 extern "C" int sonar_moe_sum(void* out, const void* in, int64_t tokens, int64_t topk, int64_t d, int dtype,

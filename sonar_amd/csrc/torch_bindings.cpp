@@ -1025,6 +1025,38 @@ void silu_and_mul(Tensor& result, const Tensor& input) {
                                      d, dtype_code(input), current_stream(input)));
 }
 
+// The reference's other gated activations (fused_moe/activation.py:128-205), schemas as in
+// csrc/libtorch_stable/torch_bindings.cpp:640-680 of the reference.
+void gated_activation(Tensor& result, const Tensor& input, int kind, double limit, double alpha, double beta,
+                      const char* name) {
+  TORCH_CHECK(input.is_cuda() && input.is_contiguous() && result.is_cuda() && result.is_contiguous(), name,
+              " needs contiguous GPU tensors");
+  TORCH_CHECK(result.scalar_type() == input.scalar_type(), "result must have the dtype of input");
+  const int64_t d = input.size(-1) / 2;
+  TORCH_CHECK(input.size(-1) == 2 * d && result.size(-1) == d && result.numel() * 2 == input.numel(),
+              "result must be input with the last dimension halved");
+  c10::hip::HIPGuardMasqueradingAsCUDA guard(input.device());
+  raise_if_failed(sonar_moe_activation(result.mutable_data_ptr(), input.const_data_ptr(), input.numel() / (2 * d), d,
+                                       kind, (float)limit, (float)alpha, (float)beta, dtype_code(input),
+                                       current_stream(input)));
+}
+void silu_and_mul_with_clamp(Tensor& result, const Tensor& input, double limit, double alpha, double beta) {
+  gated_activation(result, input, SONAR_ACT_SILU_CLAMP, limit, alpha, beta, "silu_and_mul_with_clamp");
+}
+void gelu_and_mul(Tensor& out, const Tensor& input) { gated_activation(out, input, SONAR_ACT_GELU, 0, 1, 0, "gelu_and_mul"); }
+void gelu_tanh_and_mul(Tensor& out, const Tensor& input) {
+  gated_activation(out, input, SONAR_ACT_GELU_TANH, 0, 1, 0, "gelu_tanh_and_mul");
+}
+void swigluoai_and_mul(Tensor& out, const Tensor& input, double alpha, double limit) {
+  gated_activation(out, input, SONAR_ACT_SWIGLUOAI, limit, alpha, 0, "swigluoai_and_mul");
+}
+void situ_and_mul(Tensor& out, const Tensor& input, double beta, double linear_beta) {
+  gated_activation(out, input, SONAR_ACT_SITU, 0, beta, linear_beta, "situ_and_mul");
+}
+void swiglustep_and_mul(Tensor& out, const Tensor& input, double limit) {
+  gated_activation(out, input, SONAR_ACT_SWIGLUSTEP, limit, 1, 0, "swiglustep_and_mul");
+}
+
 void moe_sum(const Tensor& input, Tensor& output) {
   TORCH_CHECK(input.is_cuda() && input.is_contiguous() && output.is_cuda() && output.is_contiguous(),
               "moe_sum needs contiguous GPU tensors");
@@ -1080,6 +1112,12 @@ TORCH_LIBRARY(sonar_amd, m) {
       "moe_align_block_size(Tensor topk_ids, int num_experts, int block_size, Tensor! sorted_token_ids, "
       "Tensor! experts_ids, Tensor! num_tokens_post_pad, Tensor? maybe_expert_map) -> ()");
   m.def("silu_and_mul(Tensor! result, Tensor input) -> ()");
+  m.def("silu_and_mul_with_clamp(Tensor! result, Tensor input, float limit, float alpha=1.0, float beta=0.0) -> ()");
+  m.def("gelu_and_mul(Tensor! out, Tensor input) -> ()");
+  m.def("gelu_tanh_and_mul(Tensor! out, Tensor input) -> ()");
+  m.def("swigluoai_and_mul(Tensor! out, Tensor input, float alpha=1.702, float limit=7.0) -> ()");
+  m.def("situ_and_mul(Tensor! out, Tensor input, float beta, float linear_beta) -> ()");
+  m.def("swiglustep_and_mul(Tensor! out, Tensor input, float limit=7.0) -> ()");
   m.def("moe_sum(Tensor input, Tensor! output) -> ()");
   m.def("per_token_quant_int8(Tensor x) -> (Tensor, Tensor)");
   m.def("per_token_quant_fp8(Tensor x) -> (Tensor, Tensor)");
@@ -1087,6 +1125,12 @@ TORCH_LIBRARY(sonar_amd, m) {
 TORCH_LIBRARY_IMPL(sonar_amd, CUDA, m) {
   m.impl("moe_align_block_size", &moe_align_block_size);
   m.impl("silu_and_mul", &silu_and_mul);
+  m.impl("silu_and_mul_with_clamp", &silu_and_mul_with_clamp);
+  m.impl("gelu_and_mul", &gelu_and_mul);
+  m.impl("gelu_tanh_and_mul", &gelu_tanh_and_mul);
+  m.impl("swigluoai_and_mul", &swigluoai_and_mul);
+  m.impl("situ_and_mul", &situ_and_mul);
+  m.impl("swiglustep_and_mul", &swiglustep_and_mul);
   m.impl("moe_sum", &moe_sum);
   m.impl("per_token_quant_int8", &per_token_quant_int8);
   m.impl("per_token_quant_fp8", &per_token_quant_fp8);

@@ -171,18 +171,97 @@ def moe_sum(moe_output: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
 def _activation_name(activation) -> str:
     """`activation` as the reference passes it (a MoEActivation enum member, whose value is
     the name) or as a plain string."""
-    return str(getattr(activation, "value", activation)).lower()
+    name = str(getattr(activation, "value", activation)).lower()
+    return {"gelu_pytorch_tanh": "gelu_tanh"}.get(name, name)
 
 
-def _check_unbuilt(activation, clamp_limit, gemm1_alpha, gemm1_beta, input_dtype, global_scales,
-                   activation_situ_beta=None, activation_situ_linear_beta=None) -> None:
-    if _activation_name(activation) != "silu":
-        raise NotImplementedError(f"activation {activation!r}: only SILU (silu(gate) * up) is built; the "
-                                  "reference's GELU, RELU2, SWIGLUOAI, SITU and no-mul variants are not")
-    if clamp_limit is not None or gemm1_alpha != 1.0 or gemm1_beta != 0.0:
-        raise NotImplementedError("clamp_limit / gemm1_alpha / gemm1_beta (SWIGLUOAI parameters) are not built")
-    if activation_situ_beta is not None or activation_situ_linear_beta is not None:
-        raise NotImplementedError("activation_situ_beta / activation_situ_linear_beta are not built")
+# the reference's MoEActivation values (fused_moe/activation.py:11-38)
+_GATED = ("silu", "gelu", "gelu_tanh", "swigluoai", "situ", "swigluoai_uninterleave", "swiglustep")
+_NOT_GATED = ("silu_no_mul", "gelu_no_mul", "gelu_tanh_no_mul", "relu2_no_mul")
+
+
+def activation_is_gated(activation) -> bool:
+    """MoEActivation.is_gated: a gated activation takes [.., 2 d] and gives [.., d]."""
+    return not _activation_name(activation).endswith("_no_mul")
+
+
+def _gated_on_gpu(op, output, input, *args) -> bool:
+    d = output.shape[-1]
+    if input.is_cuda and input.is_contiguous() and output.is_contiguous() and d % 8 == 0:
+        op(output, input, *args)
+        return True
+    return False
+
+
+def apply_moe_activation(activation, output: torch.Tensor, input: torch.Tensor, *, clamp_limit=None,
+                         alpha: float = 1.0, beta: float = 0.0, topk_ids=None, expert_map=None,
+                         activation_situ_beta=None, activation_situ_linear_beta=None) -> torch.Tensor:
+    """The reference's dispatcher between the two grouped GEMMs
+    (fused_moe/activation.py:128-205): `output` [rows, d] from `input` [rows, 2 d] (gated) or
+    [rows, d].  `clamp_limit` / `alpha` / `beta` drive the clamped SwiGLU: SILU with a
+    clamp_limit and SWIGLUOAI_UNINTERLEAVE are both silu_and_mul_with_clamp.  The gated forms
+    run as HIP kernels on GPU tensors (torch expressions of the same arithmetic serve CPU
+    tensors); the forms without a gate are torch functions in the reference as well.
+    `topk_ids` / `expert_map` are accepted as in the reference: its pad-aware variant skips
+    slots that nobody reads, the values of the others are the same."""
+    name = _activation_name(activation)
+    assert input.dim() == 2 and output.dim() == 2, "input and output must be 2D"
+    d = output.shape[-1]
+    if activation_is_gated(name):
+        assert d * 2 == input.shape[-1], f"{name} expects 2x ratio: {d * 2} vs {input.shape[-1]}"
+    else:
+        assert d == input.shape[-1], f"{name} expects equal sizes: {d} vs {input.shape[-1]}"
+    f32 = torch.float32
+    g, u = input[..., :d].to(f32), input[..., d:].to(f32)
+    dt = output.dtype
+    if name == "silu" and clamp_limit is None:
+        silu_and_mul(output, input)
+    elif name in ("silu", "swigluoai_uninterleave"):
+        assert clamp_limit is not None, "SWIGLUOAI_UNINTERLEAVE requires clamp_limit"
+        a, b = (1.0, 0.0) if name == "silu" else (float(alpha), float(beta))
+        if not _gated_on_gpu(torch.ops.sonar_amd.silu_and_mul_with_clamp, output, input, float(clamp_limit), a, b):
+            gc = g.clamp(max=clamp_limit).to(dt).to(f32)
+            act = (gc / (1.0 + torch.exp(-gc * a))).to(dt).to(f32)
+            output.copy_((act * (u.clamp(-clamp_limit, clamp_limit) + b)).to(dt))
+    elif name == "gelu":
+        if not _gated_on_gpu(torch.ops.sonar_amd.gelu_and_mul, output, input):
+            output.copy_((torch.nn.functional.gelu(g).to(dt).to(f32) * u).to(dt))
+    elif name == "gelu_tanh":
+        if not _gated_on_gpu(torch.ops.sonar_amd.gelu_tanh_and_mul, output, input):
+            output.copy_((torch.nn.functional.gelu(g, approximate="tanh").to(dt).to(f32) * u).to(dt))
+    elif name == "swigluoai":      # gate and up alternate (gpt-oss checkpoints); alpha 1.702, limit 7.0
+        if not _gated_on_gpu(torch.ops.sonar_amd.swigluoai_and_mul, output, input, 1.702, 7.0):
+            gi = input[..., 0::2].to(f32).clamp(max=7.0)
+            ui = input[..., 1::2].to(f32).clamp(-7.0, 7.0)
+            output.copy_(((ui + 1.0) * gi / (1.0 + torch.exp(-gi * 1.702))).to(dt))
+    elif name == "situ":
+        assert activation_situ_beta is not None, "SITU requires activation_situ_beta"
+        lb = -1.0 if activation_situ_linear_beta is None else float(activation_situ_linear_beta)
+        if not _gated_on_gpu(torch.ops.sonar_amd.situ_and_mul, output, input, float(activation_situ_beta), lb):
+            bt = float(activation_situ_beta)
+            up = lb * torch.tanh(u / lb) if lb > 0 else u
+            output.copy_((bt * torch.tanh(g / bt) / (1.0 + torch.exp(-g)) * up).to(dt))
+    elif name == "swiglustep":
+        if not _gated_on_gpu(torch.ops.sonar_amd.swiglustep_and_mul, output, input, 7.0):
+            output.copy_(((g * torch.sigmoid(g)).clamp(max=7.0) * u.clamp(-7.0, 7.0)).to(dt))
+    elif name == "silu_no_mul":
+        output.copy_(torch.nn.functional.silu(input))
+    elif name == "gelu_no_mul":
+        output.copy_(torch.nn.functional.gelu(input))
+    elif name == "gelu_tanh_no_mul":
+        output.copy_(torch.nn.functional.gelu(input, approximate="tanh"))
+    elif name == "relu2_no_mul":
+        torch.nn.functional.relu(input, inplace=True)
+        torch.square(input, out=output)
+    else:
+        raise ValueError(f"Unsupported FusedMoe activation: {activation}")
+    return output
+
+
+def _check_arguments(activation, input_dtype, global_scales) -> None:
+    name = _activation_name(activation)
+    if name not in _GATED + _NOT_GATED:
+        raise ValueError(f"Unknown MoE activation: {activation!r}. Valid activations: {list(_GATED + _NOT_GATED)}")
     if input_dtype is not None and input_dtype not in (torch.int8, torch.float8_e4m3fn, torch.float16,
                                                        torch.bfloat16):
         raise ValueError(f"unsupported input_dtype {input_dtype}")
@@ -202,24 +281,27 @@ def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, t
                       activation_situ_beta=None, activation_situ_linear_beta=None):
     """Gate/up GEMM -> activation -> down GEMM over already routed slots
     (marlin_moe.py:57-223; same parameters in the same order).  `activation_func`, when
-    given, is called as activation_func(activation, out [M * top_k, N], in [M * top_k, 2N])
-    like the reference's apply_moe_activation; the default is the HIP silu_and_mul.
-    `expert_map` and `topk_ids` are accepted for signature parity (the routing passed in
-    already reflects them).  Returns the [M * top_k, K] per-slot outputs."""
-    _check_unbuilt(activation, clamp_limit, gemm1_alpha, gemm1_beta, input_dtype,
-                   (input_global_scale1, input_global_scale2, global_scale1, global_scale2),
-                   activation_situ_beta, activation_situ_linear_beta)
+    given, is called like the reference's apply_moe_activation: activation_func(activation,
+    out [M * top_k, N], in [M * top_k, shards * N], clamp_limit=, alpha=, beta=, topk_ids=,
+    expert_map=, activation_situ_beta=, activation_situ_linear_beta=); the default is
+    apply_moe_activation above.  A gated activation takes the gate and up projections from the
+    first GEMM (shards = 2), one without a gate takes one projection.  `expert_map` is otherwise
+    accepted for signature parity (the routing passed in already reflects it).  Returns the
+    [M * top_k, K] per-slot outputs."""
+    _check_arguments(activation, input_dtype, (input_global_scale1, input_global_scale2, global_scale1,
+                                               global_scale2))
     assert hidden_states.ndim == 2
     M, K = hidden_states.shape
     N = w2.shape[1] * 16                       # intermediate size: w2 is (E, N/16, 2K)
+    shards = 2 if activation_is_gated(activation) else 1
     dev, dt = hidden_states.device, hidden_states.dtype
     if workspace is None:
         workspace = marlin_make_workspace_new(dev, 4)
     if intermediate_cache13 is None:
-        intermediate_cache13 = torch.empty((M * num_topk * max(2 * N, K),), device=dev, dtype=dt)
+        intermediate_cache13 = torch.empty((M * num_topk * max(shards * N, K),), device=dev, dtype=dt)
     if intermediate_cache2 is None:
         intermediate_cache2 = torch.empty((M * num_topk, N), device=dev, dtype=dt)
-    cache1 = intermediate_cache13[:M * num_topk * 2 * N].view(M * num_topk, 2 * N)
+    cache1 = intermediate_cache13[:M * num_topk * shards * N].view(M * num_topk, shards * N)
     cache3 = intermediate_cache13[:M * num_topk * K].view(M * num_topk, K)
     cache2 = intermediate_cache2.view(-1)[:M * num_topk * N].view(M * num_topk, N)
 
@@ -236,12 +318,13 @@ def _fused_marlin_moe(hidden_states, w1, w2, bias1, bias2, w1_scale, w2_scale, t
         workspace,
         sorted_token_ids, expert_ids, num_tokens_post_padded, topk_weights, moe_block_size=block_size_m,
         top_k=num_topk, mul_topk_weights=apply_router_weight_on_input, b_q_type=quant_type, size_m=M,
-        size_n=2 * N, size_k=K, is_k_full=is_k_full, use_atomic_add=False, use_fp32_reduce=True,
+        size_n=shards * N, size_k=K, is_k_full=is_k_full, use_atomic_add=False, use_fp32_reduce=True,
         is_zp_float=False)
-    if activation_func is not None:
-        activation_func(activation, cache2, cache1.view(-1, 2 * N))
-    else:
-        silu_and_mul(cache2, cache1.view(-1, 2 * N))
+    # (SILU with a clamp_limit and SWIGLUOAI_UNINTERLEAVE both come out as silu_and_mul_with_clamp)
+    (activation_func or apply_moe_activation)(
+        activation, cache2, cache1.view(-1, shards * N), clamp_limit=clamp_limit, alpha=gemm1_alpha,
+        beta=gemm1_beta, topk_ids=topk_ids, expert_map=expert_map, activation_situ_beta=activation_situ_beta,
+        activation_situ_linear_beta=activation_situ_linear_beta)
     if output is None:
         output = cache3
     if input_dtype in (torch.int8, torch.float8_e4m3fn):
@@ -279,17 +362,19 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
     (marlin_moe.py:226-392).  w1: (E, K/16, 2 * 2N) gate and up projections,
     w2: (E, N/16, 2K); scales (E, groups, 2N) / (E, groups, K); topk_weights
     fp32 [M, top_k]; topk_ids [M, top_k].  Returns [M, K].  Parameters and their order are
-    the reference's; of its activations only SILU is built (anything else, and clamp_limit /
-    gemm1_alpha / gemm1_beta, raise NotImplementedError; global_scale1 / global_scale2 are the
-    per-expert global scales of NVFP4 experts).  input_dtype torch.int8 / torch.float8_e4m3fn:
+    the reference's: `activation` any of its MoEActivation values (a gated one takes w1 with the
+    gate and up projections, (E, K/16, 2 * 2N); one without a gate takes (E, K/16, 2N)), with
+    clamp_limit / gemm1_alpha / gemm1_beta for the clamped SwiGLU forms (SILU with a clamp_limit,
+    SWIGLUOAI_UNINTERLEAVE: the experts of gpt-oss) and activation_situ_beta /
+    activation_situ_linear_beta for SITU; global_scale1 / global_scale2 are the per-expert global
+    scales of NVFP4 experts.  input_dtype torch.int8 / torch.float8_e4m3fn:
     the tokens and the activation's output are quantised per row and both GEMMs run on the 8-bit
     matrix cores (4-bit expert weights repacked with is_a_8bit; input_global_scale1 / 2 are the
     factors marlin_act_int8_process_scales returns for the integer group scales).
-    `activation_func(activation, out, in)` and `moe_sum(moe_output [M, top_k, K], output)`
-    replace the built-in HIP kernels when given, as in the reference."""
-    _check_unbuilt(activation, clamp_limit, gemm1_alpha, gemm1_beta, input_dtype,
-                   (input_global_scale1, input_global_scale2, global_scale1, global_scale2),
-                   activation_situ_beta, activation_situ_linear_beta)
+    `activation_func(activation, out, in, **parameters)` and `moe_sum(moe_output [M, top_k, K],
+    output)` replace the built-in HIP kernels when given, as in the reference."""
+    _check_arguments(activation, input_dtype, (input_global_scale1, input_global_scale2, global_scale1,
+                                               global_scale2))
     if quant_type_id not in _SUPPORTED:
         raise NotImplementedError(f"quant type id {quant_type_id}: only uint4, uint4b8, uint8b128, "
                                   "float8_e4m3fn and float4_e2m1f (MXFP4, NVFP4) expert weights are built")
@@ -326,7 +411,9 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
         sort_indices1=sort_indices1, sort_indices2=sort_indices2,
         w1_zeros=w1_zeros, w2_zeros=w2_zeros, workspace=workspace,
         intermediate_cache13=intermediate_cache13, intermediate_cache2=intermediate_cache2, output=None,
-        input_dtype=input_dtype, is_k_full=is_k_full).view(-1, topk, K)
+        input_dtype=input_dtype, is_k_full=is_k_full, clamp_limit=clamp_limit, gemm1_alpha=gemm1_alpha,
+        gemm1_beta=gemm1_beta, activation_situ_beta=activation_situ_beta,
+        activation_situ_linear_beta=activation_situ_linear_beta).view(-1, topk, K)
     if output is None:
         output = torch.empty_like(hidden_states)
     if expert_map is not None:

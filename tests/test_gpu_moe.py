@@ -398,6 +398,67 @@ def test_silu_and_mul_and_moe_sum_kernels(dtype):
     assert np.array_equal(gu.host_f32(s), want)        # fp32 sum in k order, one rounding
 
 
+ACTIVATIONS = [
+    # name, kind, limit, alpha, beta, oracle keywords
+    ("silu", 1, 3.0, 1.0, 0.0, dict(clamp_limit=3.0)),
+    ("swigluoai_uninterleave", 1, 7.0, 1.702, 1.0, dict(clamp_limit=7.0, alpha=1.702, beta=1.0)),
+    ("gelu", 2, 0.0, 1.0, 0.0, {}),
+    ("gelu_tanh", 3, 0.0, 1.0, 0.0, {}),
+    ("swigluoai", 4, 7.0, 1.702, 0.0, {}),
+    ("situ", 5, 0.0, 4.0, 3.0, dict(situ_beta=4.0, situ_linear_beta=3.0)),
+    ("situ", 5, 0.0, 2.5, -1.0, dict(situ_beta=2.5, situ_linear_beta=None)),
+    ("swiglustep", 6, 7.0, 1.0, 0.0, {}),
+]
+
+
+@pytest.mark.parametrize("dtype", ["fp16", "bf16"])
+@pytest.mark.parametrize("name,kind,limit,alpha,beta,kw", ACTIVATIONS, ids=lambda v: str(v) if isinstance(v, str) else None)
+def test_gated_activation_kernels(name, kind, limit, alpha, beta, kw, dtype):
+    """sonar_moe_activation against oracle.moe_activation: values beyond the clamp limits on
+    both sides included.  The kernel's float32 exp / tanh / erf against float64 there: at most
+    one unit in the last place of an intermediate rounding, and nearly every value equal."""
+    lib = _lib.load()
+    rng = np.random.default_rng(kind * 7 + len(name))
+    rows, d = 29, 136
+    x32 = mo.round_to_dtype((rng.standard_normal((rows, 2 * d)) * 4).astype(np.float32), dtype)
+    x = gu.dev_bits16(x32, dtype)
+    out = torch.empty((rows, d), dtype=x.dtype, device=gu.DEV)
+    _lib.check(lib.sonar_moe_activation(gu.ptr(out), gu.ptr(x), rows, d, kind, limit, alpha, beta,
+                                        gu.dtype_code(dtype), gu.stream()))
+    want = mo.moe_activation(name, x32, dtype, **kw)
+    got = gu.host_f32(out)
+    ulp = 2.0 ** (-10 if dtype == "fp16" else -7)
+    assert np.all(np.isfinite(got))
+    tol = 2 * ulp * np.abs(want) + 1e-6
+    if name.startswith("gelu"):   # 1 + erf / 1 + tanh in float32: the last place of that sum, times gate * up
+        tol = tol + 2.0 ** -20 * np.abs(x32[:, :d] * x32[:, d:])
+    assert np.all(np.abs(got - want) <= tol), np.abs(got - want).max()
+    assert np.mean(got == want) > 0.95
+    # the torch op and the dispatcher of the fused layer give the same bits
+    from sonar_amd import fused_moe
+    out2 = torch.empty_like(out)
+    fused_moe.apply_moe_activation(name, out2, x, clamp_limit=kw.get("clamp_limit"), alpha=kw.get("alpha", 1.0),
+                                   beta=kw.get("beta", 0.0), activation_situ_beta=kw.get("situ_beta"),
+                                   activation_situ_linear_beta=kw.get("situ_linear_beta"))
+    assert torch.equal(out2.view(torch.int16), out.view(torch.int16))
+    # ... and its torch expressions for CPU tensors agree to the same bar
+    cpu = torch.empty((rows, d), dtype=x.dtype)
+    fused_moe.apply_moe_activation(name, cpu, x.cpu(), clamp_limit=kw.get("clamp_limit"), alpha=kw.get("alpha", 1.0),
+                                   beta=kw.get("beta", 0.0), activation_situ_beta=kw.get("situ_beta"),
+                                   activation_situ_linear_beta=kw.get("situ_linear_beta"))
+    assert np.all(np.abs(cpu.float().numpy() - want) <= tol)
+
+
+def test_gated_activation_rejections():
+    lib = _lib.load()
+    x = torch.zeros((4, 32), dtype=torch.float16, device=gu.DEV)
+    out = torch.zeros((4, 16), dtype=torch.float16, device=gu.DEV)
+    assert lib.sonar_moe_activation(gu.ptr(out), gu.ptr(x), 4, 16, 9, 1.0, 1.0, 0.0, 0, gu.stream()) == _lib.E_INVALID
+    assert lib.sonar_moe_activation(gu.ptr(out), gu.ptr(x), 4, 16, 1, 0.0, 1.0, 0.0, 0, gu.stream()) == _lib.E_INVALID
+    assert b"limit" in lib.sonar_marlin_last_error()
+    assert lib.sonar_moe_activation(gu.ptr(out), gu.ptr(x), 4, 12, 2, 0.0, 1.0, 0.0, 0, gu.stream()) == _lib.E_INVALID
+
+
 def test_moe_tiled_and_streaming_kernels_agree():
     """The same 64-slot-block call with and without the scratch the tiled kernel
     needs for its table takes two different kernels; both meet the tolerance

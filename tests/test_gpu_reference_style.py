@@ -276,7 +276,8 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None, input_d
     return res
 
 
-def _torch_experts(a, w1, w2, topk_weight, topk_ids, expert_map=None, b1=None, b2=None, quant_dtype=None):
+def _torch_experts(a, w1, w2, topk_weight, topk_ids, expert_map=None, b1=None, b2=None, quant_dtype=None,
+                   activation=None):
     """Plain mixture of experts on (E, 2N, K) / (E, K, N) matrices: for every
     token and routed expert silu(x W1_gate^T) * (x W1_up^T) through W2^T, summed
     with the routing weights; experts mapped to -1 contribute nothing.  With
@@ -303,7 +304,11 @@ def _torch_experts(a, w1, w2, topk_weight, topk_ids, expert_map=None, b1=None, b
         if b1 is not None:
             h = h + b1[local].float()
         h = h.to(a.dtype).float()
-        act = through_quant((torch.nn.functional.silu(h[:, :n]) * h[:, n:]).to(a.dtype)).float()
+        if activation is None:
+            act = (torch.nn.functional.silu(h[:, :n]) * h[:, n:]).to(a.dtype)
+        else:      # any other activation of the layer, in plain fp32 torch arithmetic
+            act = activation(h).to(a.dtype)
+        act = through_quant(act).float()
         y = act @ w2[local].float().T
         if b2 is not None:
             y = y + b2[local].float()
@@ -344,6 +349,58 @@ def test_fused_marlin_moe(a_quant, b_type, dtype, group_size, m, n, k, e, topk, 
     # the next quantisation step (1 / 16 of its size for float8_e4m3fn)
     bar = 2e-2 if a_quant is None else 4e-2
     assert float((got.float() - want.float()).abs().max()) <= bar * float(want.float().abs().max())
+
+
+def _swigluoai_packed(h, limit=7.0, alpha=1.702, beta=1.0):
+    n = h.shape[1] // 2
+    g = h[:, :n].clamp(max=limit)
+    u = h[:, n:].clamp(-limit, limit)
+    return g * torch.sigmoid(alpha * g) * (u + beta)
+
+
+MOE_ACTIVATIONS = {
+    # name -> (keywords of fused_marlin_moe, fp32 torch form on the first GEMM's output, gated)
+    "swigluoai_uninterleave": (dict(clamp_limit=7.0, gemm1_alpha=1.702, gemm1_beta=1.0), _swigluoai_packed, True),
+    "silu+clamp": (dict(clamp_limit=0.5), lambda h: _swigluoai_packed(h, 0.5, 1.0, 0.0), True),
+    "gelu": (dict(), lambda h: torch.nn.functional.gelu(h[:, :h.shape[1] // 2]) * h[:, h.shape[1] // 2:], True),
+    "swiglustep": (dict(), lambda h: torch.nn.functional.silu(h[:, :h.shape[1] // 2]).clamp(max=7.0)
+                   * h[:, h.shape[1] // 2:].clamp(-7.0, 7.0), True),
+    "relu2_no_mul": (dict(), lambda h: torch.relu(h) ** 2, False),
+    "silu_no_mul": (dict(), torch.nn.functional.silu, False),
+}
+
+
+@pytest.mark.parametrize("name", list(MOE_ACTIVATIONS))
+@pytest.mark.parametrize("b_type,group_size,dtype", [(scalar_types.uint4b8, 128, torch.half),
+                                                     (scalar_types.float4_e2m1f, 32, torch.bfloat16)],
+                         ids=["uint4b8", "mxfp4"])
+def test_fused_marlin_moe_other_activations(name, b_type, group_size, dtype):
+    """The layer with the reference's other activations (marlin_moe.py:74-75, 93-94, 163-174;
+    tests/kernels/moe/test_moe.py:1087-1161 for the one without a gate): the clamped SwiGLU of
+    gpt-oss on MXFP4 experts among them, against a torch mixture of experts with that
+    activation in fp32.  Activations whose values are scaled up here so that the clamps bite."""
+    from sonar_amd.fused_moe import fused_marlin_moe
+    kwargs, torch_form, gated = MOE_ACTIVATIONS[name]
+    torch.manual_seed(3)
+    m, n, k, e, topk = 33, 512, 256, 6, 2
+    a = torch.randn((m, k), device="cuda", dtype=dtype)
+    w1 = torch.randn((e, (2 if gated else 1) * n, k), device="cuda", dtype=dtype) / 4
+    w2 = torch.randn((e, k, n), device="cuda", dtype=dtype) / 16
+    d1 = _marlin_moe_weights(w1, b_type, group_size, False)
+    d2 = _marlin_moe_weights(w2, b_type, group_size, False)
+    score = torch.randn((m, e), device="cuda", dtype=dtype)
+    topk_weights, topk_ids = torch.topk(torch.softmax(score, dim=-1, dtype=torch.float32), topk)
+    want = _torch_experts(a, d1["w_ref"], d2["w_ref"], topk_weights, topk_ids, activation=torch_form)
+    got = fused_marlin_moe(a, d1["qweight"], d2["qweight"], None, None, d1["scales"], d2["scales"], topk_weights,
+                           topk_ids.to(torch.int32), global_num_experts=e, quant_type_id=b_type.id,
+                           activation=name.split("+")[0], **kwargs)
+    torch.cuda.synchronize()
+    assert float((got.float() - want.float()).abs().max()) <= 2e-2 * float(want.float().abs().max())
+    if name == "silu+clamp" and b_type == scalar_types.uint4b8:   # the clamp bites: the unclamped layer is elsewhere
+        plain = fused_marlin_moe(a, d1["qweight"], d2["qweight"], None, None, d1["scales"], d2["scales"],
+                                 topk_weights, topk_ids.to(torch.int32), global_num_experts=e,
+                                 quant_type_id=b_type.id)
+        assert float((plain.float() - want.float()).abs().max()) > 5e-2 * float(want.float().abs().max())
 
 
 @pytest.mark.parametrize("m", [1, 256])

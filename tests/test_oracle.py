@@ -540,6 +540,62 @@ def test_nvfp4_scale_factor_and_small_scales():
     assert float(mo.nvfp4_process_global_scale(2.0, "fp16")) == 2.0 * 2.0 ** 7
 
 
+def test_moe_activation_closed_forms_and_limits():
+    """oracle.moe_activation against values that follow from the formulas without evaluating
+    them the same way: alpha = 0 turns every sigmoid into 1/2; a gate or an up value beyond the
+    limit gives what the limit gives (gate clamped from above only, up from both sides); the
+    +1 of swigluoai and the beta of the clamped SiLU make u = -1 / u = -beta a zero; the
+    interleaved order of swigluoai against the packed order of swigluoai_uninterleave with
+    alpha 1.702, beta 1; SITU with a huge beta is SiLU; relu2 of a negative is 0."""
+    x = np.array([[2.0, -3.0, 0.5, 4.0,    1.5, 2.0, -1.0, 0.25]], dtype=np.float32)       # gate | up
+    for dtype in ("fp16", "bf16"):
+        half = mo.moe_activation("swigluoai_uninterleave", x, dtype, clamp_limit=100.0, alpha=0.0, beta=0.0)
+        assert np.array_equal(half, mo.round_to_dtype(mo.round_to_dtype(x[:, :4] / 2, dtype) * x[:, 4:], dtype))
+        with_beta = mo.moe_activation("swigluoai_uninterleave", x, dtype, clamp_limit=100.0, alpha=0.0, beta=1.0)
+        assert with_beta[0, 2] == 0.0 and with_beta[0, 0] == 2.5                          # (u + 1): -1 -> 0; 1 * 2.5
+        # clamps: gate 9 acts as gate 3 (limit 3) but gate -9 stays; up +-9 act as +-3
+        big = np.array([[9.0, -9.0, 1.0, 1.0,   1.0, 1.0, 9.0, -9.0]], dtype=np.float32)
+        lim = np.array([[3.0, -9.0, 1.0, 1.0,   1.0, 1.0, 3.0, -3.0]], dtype=np.float32)
+        for name, kw in (("silu", dict(clamp_limit=3.0)),
+                         ("swigluoai_uninterleave", dict(clamp_limit=3.0, alpha=1.702, beta=1.0))):
+            assert np.array_equal(mo.moe_activation(name, big, dtype, **kw), mo.moe_activation(name, lim, dtype, **kw))
+        assert not np.array_equal(mo.moe_activation("silu", big, dtype, clamp_limit=3.0),
+                                  mo.moe_activation("silu", big, dtype))
+        # SILU with a clamp no value reaches is plain SILU
+        assert np.array_equal(mo.moe_activation("silu", x, dtype, clamp_limit=50.0), mo.moe_activation("silu", x, dtype))
+        # swigluoai: pairs alternate; the same numbers packed, alpha 1.702, beta 1, limit 7: one rounding
+        # less in the interleaved kernel, so compare within an ulp
+        inter = np.empty_like(x)
+        inter[:, 0::2], inter[:, 1::2] = x[:, :4], x[:, 4:]
+        a = mo.moe_activation("swigluoai", inter, dtype)
+        b = mo.moe_activation("swigluoai_uninterleave", x, dtype, clamp_limit=7.0, alpha=1.702, beta=1.0)
+        ulp = 2.0 ** (-9 if dtype == "fp16" else -6)
+        assert np.all(np.abs(a - b) <= ulp * np.abs(b)) and a[0, 2] == 0.0
+        g = np.float64(2.0)
+        assert a[0, 0] == mo.round_to_dtype(np.array([2.5 * g / (1 + np.exp(-1.702 * g))], np.float32), dtype)[0]
+        # limits of swigluoai: gate 9 -> 7, up -9 -> -7 (so u + 1 = -6)
+        lim7 = mo.moe_activation("swigluoai", np.array([[9.0, -9.0]], np.float32), dtype)
+        assert lim7[0, 0] == mo.round_to_dtype(np.array([-6.0 * 7.0 / (1 + np.exp(-1.702 * 7.0))], np.float32), dtype)[0]
+        # SITU: beta -> infinity is SiLU(gate) * up in one rounding; linear_beta bounds the up half
+        situ = mo.moe_activation("situ", x, dtype, situ_beta=1e6)
+        one = mo.round_to_dtype((x[:, :4].astype(np.float64) / (1 + np.exp(-x[:, :4].astype(np.float64)))
+                                 * x[:, 4:]).astype(np.float32), dtype)
+        assert np.array_equal(situ, one)
+        bounded = mo.moe_activation("situ", np.array([[1.0, 50.0]], np.float32), dtype, situ_beta=1e6, situ_linear_beta=2.0)
+        assert bounded[0, 0] == mo.round_to_dtype(np.array([2.0 / (1 + np.exp(-1.0))], np.float32), dtype)[0]
+        # swiglustep: silu(gate) capped at 7, up within +-7
+        step = mo.moe_activation("swiglustep", np.array([[20.0, 1.0, 9.0, -9.0]], np.float32), dtype)
+        assert step[0, 0] == 49.0 and step[0, 1] == mo.round_to_dtype(np.array([-7.0 / (1 + np.exp(-1.0))], np.float32), dtype)[0]
+        # gelu: 0 -> 0, large -> identity; the tanh form agrees with erf to 1e-3
+        ge = mo.moe_activation("gelu", np.array([[0.0, 8.0, 1.0, 1.0, 3.0, 0.5, 1.0, 1.0]], np.float32), dtype)
+        assert ge[0, 0] == 0.0 and ge[0, 1] == 4.0
+        assert abs(float(mo.moe_activation("gelu_tanh", x, dtype)[0, 0]) - float(mo.moe_activation("gelu", x, dtype)[0, 0])) < 1e-2
+        # no gate
+        r2 = mo.moe_activation("relu2_no_mul", np.array([[-2.0, 3.0]], np.float32), dtype)
+        assert r2.tolist() == [[0.0, 9.0]]
+        assert mo.moe_activation("silu_no_mul", np.array([[0.0]], np.float32), dtype)[0, 0] == 0.0
+
+
 def test_moe_gemm_reference_against_per_slot_brute_force():
     """moe_gemm_reference (the oracle of the grouped GEMM) follows sorted_ids / expert_ids
     block by block.  Brute force from the routing itself, slot by slot, without any of
