@@ -50,6 +50,8 @@ struct TileParams {
   int tiles_m, tiles_n;
   int tile_rows;               // rows of a tile: 256 (128: marlin_tile_wide_kernel with 8 row blocks)
   int tile_band;               // rows of tiles per band of the tile numbering (tile_of_workgroup)
+  // the launch covers tiles [tile_begin, tile_begin + tile_count) of the numbering (tile_count 0: all of them)
+  int tile_begin, tile_count;
   // split K (k_splits > 1): workgroup (tile, split) of a split tile covers K steps
   // [split * k_steps_per_split, ...) and leaves its fp32 tile in `partial` for tile_reduce_kernel
   int k_splits, k_steps_per_split;
@@ -90,9 +92,12 @@ __device__ __forceinline__ void tile_coords(const TileParams& p, int tile, int& 
   tile_n = rem / rows;
   tile_m = band * p.tile_band + rem - tile_n * rows;
 }
-// Tiles computed by one workgroup over the whole of K (the first ones of the numbering).
+// Tiles of the launch, and those of them computed by one workgroup over the whole of K (the first ones).
+__host__ __device__ __forceinline__ int launch_tiles(const TileParams& p) {
+  return p.tile_count > 0 ? p.tile_count : p.tiles_m * p.tiles_n;
+}
 __host__ __device__ __forceinline__ int whole_tiles(const TileParams& p) {
-  return p.k_splits > 1 ? p.whole_tiles : p.tiles_m * p.tiles_n;
+  return p.k_splits > 1 ? p.whole_tiles : launch_tiles(p);
 }
 
 // Workgroup id -> (tile, K range).  Workgroups whose ids are congruent mod 8
@@ -102,7 +107,7 @@ __host__ __device__ __forceinline__ int whole_tiles(const TileParams& p) {
 // of the split tiles, so that the short workgroups start last on every XCD.
 // Returns false for the padding ids of a run.
 __device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile, int& split, bool& whole_k) {
-  const int tiles = p.tiles_m * p.tiles_n;
+  const int tiles = launch_tiles(p);
   const int whole = whole_tiles(p);
   const int split_tiles = tiles - whole;
   const int whole_per_xcd = (whole + 7) / 8;
@@ -112,7 +117,9 @@ __device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile
   if (whole_k) {
     tile = xcd * whole_per_xcd + i;
     split = 0;
-    return tile < whole;
+    const bool mine = tile < whole;
+    tile += p.tile_begin;   // (a launch over a part of the numbering never splits K)
+    return mine;
   }
   const int t = xcd * split_per_xcd + (i - whole_per_xcd);
   if (t >= split_tiles * p.k_splits) return false;
@@ -123,7 +130,7 @@ __device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile
 
 inline int tile_grid(const TileParams& p) {
   const int whole = whole_tiles(p);
-  const int split_work = (p.tiles_m * p.tiles_n - whole) * p.k_splits;
+  const int split_work = (launch_tiles(p) - whole) * p.k_splits;
   return 8 * ((whole + 7) / 8 + (split_work + 7) / 8);
 }
 
@@ -1617,6 +1624,7 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   p.tile_rows = kTileM;
   p.tiles_m = (int)((size_m + kTileM - 1) / kTileM);
   p.tile_band = 4;
+  p.tile_begin = p.tile_count = 0;
   p.tiles_n = (int)((size_n + kTileN - 1) / kTileN);
   p.k_splits = 1;
   p.whole_tiles = 0;  // read only with k_splits > 1
@@ -1673,27 +1681,61 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     }
     if (p.tile_rows != kTileM && !(fp4 ? wide_applies_fp4(p) : wide_applies(p)))
       return fail(SONAR_E_INVALID, "internal: 128-row tiles exist in the wide tile kernel only");
-    if (nvfp4 && wide_applies_fp4(p))
-      rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide_nvfp4<_Float16, false>(p, st)
-                                    : launch_tile_wide_nvfp4<__bf16, false>(p, st);
-    else if (nvfp4)
-      rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16>(p, st) : launch_tile_async_nvfp4<__bf16>(p, st);
-    else if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
-      rc = wide_applies_fp4(p) ? launch_tile_wide_fp4<false>(p, st) : launch_tile_async_fp4(p, st);
-    else if (bits == 8 && wide_applies8(p))
-      rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide8<_Float16, false>(p, fp8, st)
-                                    : launch_tile_wide8<__bf16, false>(p, fp8, st);
-    else if (bits == 8)   // symmetric 8-bit codes: the caller has checked
-      rc = dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, false>(p, fp8, st)
-                                    : launch_tile_async8<__bf16, false>(p, fp8, st);
-    else if (wide_applies(p) && dtype == SONAR_DTYPE_F16)
-      rc = zp ? launch_tile_wide<_Float16, true>(p, st) : launch_tile_wide<_Float16, false>(p, st);
-    else if (wide_applies(p))
-      rc = zp ? launch_tile_wide<__bf16, true>(p, st) : launch_tile_wide<__bf16, false>(p, st);
-    else if (dtype == SONAR_DTYPE_F16)
-      rc = zp ? launch_tile_async<_Float16, true>(p, st) : launch_tile_async<_Float16, false>(p, st);
-    else
-      rc = zp ? launch_tile_async<__bf16, true>(p, st) : launch_tile_async<__bf16, false>(p, st);
+    // the kernel a launch described by q takes
+    auto launch = [&](const TileParams& q) -> int {
+      if (nvfp4 && wide_applies_fp4(q))
+        return dtype == SONAR_DTYPE_F16 ? launch_tile_wide_nvfp4<_Float16, false>(q, st)
+                                    : launch_tile_wide_nvfp4<__bf16, false>(q, st);
+      else if (nvfp4)
+        return dtype == SONAR_DTYPE_F16 ? launch_tile_async_nvfp4<_Float16>(q, st) : launch_tile_async_nvfp4<__bf16>(q, st);
+      else if (fp4)   // the caller has checked: bf16, groups of 32 rows, no zero points
+        return wide_applies_fp4(q) ? launch_tile_wide_fp4<false>(q, st) : launch_tile_async_fp4(q, st);
+      else if (bits == 8 && wide_applies8(q))
+        return dtype == SONAR_DTYPE_F16 ? launch_tile_wide8<_Float16, false>(q, fp8, st)
+                                    : launch_tile_wide8<__bf16, false>(q, fp8, st);
+      else if (bits == 8)   // symmetric 8-bit codes: the caller has checked
+        return dtype == SONAR_DTYPE_F16 ? launch_tile_async8<_Float16, false>(q, fp8, st)
+                                    : launch_tile_async8<__bf16, false>(q, fp8, st);
+      else if (wide_applies(q) && dtype == SONAR_DTYPE_F16)
+        return zp ? launch_tile_wide<_Float16, true>(q, st) : launch_tile_wide<_Float16, false>(q, st);
+      else if (wide_applies(q))
+        return zp ? launch_tile_wide<__bf16, true>(q, st) : launch_tile_wide<__bf16, false>(q, st);
+      else if (dtype == SONAR_DTYPE_F16)
+        return zp ? launch_tile_async<_Float16, true>(q, st) : launch_tile_async<_Float16, false>(q, st);
+      else
+        return zp ? launch_tile_async<__bf16, true>(q, st) : launch_tile_async<__bf16, false>(q, st);
+    };
+    auto takes_wide = [&](const TileParams& q) {
+      return fp4 ? wide_applies_fp4(q) : (bits == 8 ? wide_applies8(q) : wide_applies(q));
+    };
+    // More tiles than compute units with a short last round (M = 4096, N = 6144: 384 tiles of 256
+    // rows = 256 + 128): instead of cutting the K ranges of that round's tiles in two and summing
+    // partial tiles in a third launch, the full rounds run as they are and the last round runs in
+    // a second launch as twice as many 128-row tiles over the whole of K: nothing goes through
+    // scratch (163 + 18 us of split tiles and their sum before).  Tile t of the 256-row numbering
+    // is tiles 2 t and 2 t + 1 of the 128-row numbering with bands twice as high.
+    static const bool no_two_sizes = getenv("SONAR_MARLIN_NO_TWO_TILE_SIZES") != nullptr;   // debugging aid
+    if (!no_two_sizes && !no_128 && rows128_ok && p.tile_rows == kTileM && plan.k_splits > 1 && plan.whole_tiles > 0 &&
+        (size_m - 1) % kTileM >= 128) {
+      TileParams big = p;
+      big.k_splits = 1;
+      big.k_steps_per_split = (int)(size_k / kTileK);
+      big.partial = nullptr;
+      big.tile_count = (int)plan.whole_tiles;
+      TileParams half = big;
+      half.tile_rows = 128;
+      half.tiles_m = 2 * p.tiles_m;
+      half.tile_band = 8;
+      half.tile_begin = 2 * (int)plan.whole_tiles;
+      half.tile_count = 2 * (p.tiles_m * p.tiles_n - (int)plan.whole_tiles);
+      if (takes_wide(big) && takes_wide(half)) {
+        if (int rc1 = launch(big)) return rc1;
+        if (int rc2 = launch_status("marlin_tile_wide_kernel")) return rc2;
+        if (int rc1 = launch(half)) return rc1;
+        return launch_status("marlin_tile_wide_kernel (128-row tiles)");
+      }
+    }
+    rc = launch(p);
     if (rc) return rc;
     if (int rc2 = launch_status("marlin_tile_async_kernel")) return rc2;
     if (p.k_splits > 1) {
@@ -1741,6 +1783,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                                                                              (int)num_experts, table, max_tiles);
   if (int rc = launch_status("moe_tile_table_kernel")) return rc;
   TileParams p;
+  p.tile_begin = p.tile_count = 0;
   p.global_scale = global_scale;   // NVFP4: one per expert
   p.a = static_cast<const uint16_t*>(a);
   p.lda = size_k;

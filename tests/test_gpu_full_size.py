@@ -134,6 +134,20 @@ def mixtral_experts(k, n):
     return _experts[(k, n)]
 
 
+def test_prefill_short_last_round_with_split_k_meets_the_oracle():
+    """M = 3900 on the qkv shape: 384 tiles of 256 rows whose last round is 128 tiles, the last row
+    of tiles less than half full: that round's tiles are cut along K and summed by
+    tile_reduce_kernel (at M = 4096 the round runs as 128-row tiles instead)."""
+    layer = big_layer("qkv", "fp16")
+    m = 3900
+    gen = torch.Generator(device=gu.DEV).manual_seed(m)
+    a = (torch.randn((m, layer.k), device=gu.DEV, generator=gen) * 0.5).to(torch.float16)
+    c = layer.gemm(a, m)
+    torch.cuda.synchronize()
+    assert bool(torch.isfinite(c.float()).all())
+    check_columns(layer, a, c, m, sampled_columns(layer.n, 6, m))
+
+
 @pytest.mark.parametrize("tokens", [16, 4096])
 @pytest.mark.parametrize("k,n,top_k,mul", [(4096, 28672, 2, False), (14336, 4096, 1, True)])
 def test_mixtral_sized_grouped_gemm(k, n, top_k, mul, tokens):
