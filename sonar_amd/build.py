@@ -24,6 +24,24 @@ HIP_FLAGS = [
 ]
 
 
+# The compiler the hand-scheduled kernels were checked with.  Their asm statements
+# (loads whose results land many instructions later, tied to their use only by a later
+# wait statement) depend on how this compiler allocates registers: another one may be
+# fine, but only the parity tests and the resource report can say so.
+CHECKED_HIPCC = "roc-7.2.0"
+
+
+def check_compiler() -> None:
+    """Refuses a compiler other than the checked one unless SONAR_ANY_HIPCC is set."""
+    proc = subprocess.run([HIPCC, "--version"], stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+    if CHECKED_HIPCC in proc.stdout or os.environ.get("SONAR_ANY_HIPCC"):
+        return
+    raise RuntimeError(
+        "%s is not the compiler these kernels were checked with (%s).  Set SONAR_ANY_HIPCC=1 to build "
+        "anyway, then run tests/test_host_logic.py (no spills in the tile kernels) and the GPU parity "
+        "tests before use.\n%s" % (HIPCC, CHECKED_HIPCC, proc.stdout))
+
+
 def _run(cmd):
     proc = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in proc.stdout.splitlines()
@@ -36,6 +54,7 @@ def _run(cmd):
 def build_hip_library(verbose: bool = False, only=None) -> str:
     """Compiles every HIP source (or, with `only`, those sources; the other objects are
     reused when they exist) and links the shared library."""
+    check_compiler()
     os.makedirs(LIB_DIR, exist_ok=True)
     only = set(only or HIP_SOURCES)
 
