@@ -23,8 +23,10 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   const float* global_scale, const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
                   int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, int bits, bool fp8, hipStream_t st);
+                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, int bits, bool fp8, void* partial,
+                  size_t partial_bytes, hipStream_t st);
 size_t moe_tile_table_bytes(int64_t sorted_len, int64_t num_experts);
+size_t moe_tile_partial_bytes(int64_t size_k);
 // gemm_stream.hip: the 16-row decode kernel in grouped form, for few rows per expert
 bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t sorted_len, int64_t num_experts,
                       int64_t a_rows, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size);
@@ -522,13 +524,19 @@ void launch_moe_mb(const MoeParams& p, bool has_perm, int grid, hipStream_t st) 
 
 using namespace sonar;
 
+// the table of row tiles, rounded up so that what follows it is aligned
+static size_t moe_table_room(int64_t sorted_len) {
+  return (moe_tile_table_bytes(sorted_len, 0) + 255) & ~(size_t)255;
+}
+
 extern "C" size_t sonar_moe_marlin_gemm_scratch_bytes(int64_t sorted_len, int64_t moe_block_size,
                                                       int64_t size_n, int64_t size_k) {
   (void)size_n;
-  (void)size_k;
-  // K is never split across workgroups, so no partial sums leave the chip; the
-  // tiled kernel for 64-slot blocks keeps its table of row tiles here (one entry per block)
-  return moe_block_size == 64 ? moe_tile_table_bytes(sorted_len, 0) : 0;
+  // Blocks of fewer than 64 slots: K is never split across workgroups, no partial sums leave
+  // the chip.  64-slot blocks: the tiled kernel keeps its table of row tiles here (one entry per
+  // block) and, behind it, the fp32 partial tiles of the tiles it splits along K.
+  if (moe_block_size != 64) return 0;
+  return moe_table_room(sorted_len) + moe_tile_partial_bytes(size_k);
 }
 
 namespace {
@@ -673,7 +681,8 @@ int moe_gemm_any(
     return moe_tile_gemm(a, c, b_q_weight, b_bias, b_scales, global_scale, b_zeros, sorted_token_ids, sorted_len, expert_ids,
                          num_tokens_past_padded, topk_weights, top_k, mul_topk_weights ? 1 : 0, num_experts,
                          static_cast<int32_t*>(scratch), dtype, size_m, size_n, size_k, num_groups, group_size,
-                         a_by_slot, fp4, bits8 ? 8 : 4, fp8, st);
+                         a_by_slot, fp4, bits8 ? 8 : 4, fp8, static_cast<char*>(scratch) + moe_table_room(sorted_len),
+                         scratch_bytes > moe_table_room(sorted_len) ? scratch_bytes - moe_table_room(sorted_len) : 0, st);
 
   MoeParams p;
   p.a = static_cast<const uint16_t*>(a);

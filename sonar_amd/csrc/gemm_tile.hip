@@ -121,6 +121,8 @@ __device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile
     tile += p.tile_begin;   // (a launch over a part of the numbering never splits K)
     return mine;
   }
+  // (a grouped launch is sized for the most tiles there could be: ids past this XCD's share do nothing)
+  if (i - whole_per_xcd >= split_per_xcd) return false;
   const int t = xcd * split_per_xcd + (i - whole_per_xcd);
   if (t >= split_tiles * p.k_splits) return false;
   split = t / split_tiles;
@@ -128,10 +130,53 @@ __device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile
   return true;
 }
 
+// Grouped calls learn the number of their tiles on the device (the routing decides it), so the
+// kernel plans the K split itself, by plan_gemm's rules: fewer tiles than compute units, or a last
+// round of workgroups that fills half of the chip or less, are cut along K into about 256
+// workgroups, in ranges of a multiple of four steps (the caller has checked that K allows it).
+constexpr int kLiveSplitTilesMax = 128;   // tiles that can be split, and
+constexpr int kLiveSplitWorkMax = 256;    // (tile, K range) pairs, i.e. partial tiles, there can be
+struct LiveSplit {
+  int whole, splits, steps;   // tiles computed over the whole of K; K ranges per split tile; steps per range
+};
+__host__ __device__ __forceinline__ LiveSplit plan_live_split(int tiles, int k_steps) {
+  LiveSplit s = {tiles, 1, k_steps};
+  int split_tiles = 0;
+  if (tiles < 256) split_tiles = tiles;
+  else if (k_steps >= 48 && tiles % 256 <= 128) split_tiles = tiles % 256;
+  if (split_tiles == 0 || split_tiles > kLiveSplitTilesMax) return s;
+  int splits = 256 / split_tiles;
+  if (splits > k_steps / 8) splits = k_steps / 8;
+  if (splits > 16) splits = 16;
+  if (splits < 2) return s;
+  const int steps = ((k_steps + splits - 1) / splits + 3) / 4 * 4;
+  splits = (k_steps + steps - 1) / steps;   // no empty range
+  if (splits < 2) return s;
+  s.whole = tiles - split_tiles;
+  s.splits = splits;
+  s.steps = steps;
+  return s;
+}
+// The tiles there are in a grouped call, with the K split planned from them when the call has room for partial tiles.
+__device__ __forceinline__ TileParams live_tiles(const TileParams& p) {
+  TileParams live = p;
+  live.tiles_m = p.tile_table[0];
+  live.tile_band = 4;
+  if (p.partial != nullptr) {
+    const LiveSplit s = plan_live_split(live.tiles_m * live.tiles_n, p.size_k / kTileK);
+    live.k_splits = s.splits;
+    live.whole_tiles = s.whole;
+    live.k_steps_per_split = s.steps;
+  }
+  return live;
+}
+
 inline int tile_grid(const TileParams& p) {
   const int whole = whole_tiles(p);
   const int split_work = (launch_tiles(p) - whole) * p.k_splits;
-  return 8 * ((whole + 7) / 8 + (split_work + 7) / 8);
+  // (a grouped call with room for partial tiles: the kernel may turn up to 128 of its tiles into 256 K ranges)
+  const int live_split = p.tile_table != nullptr && p.partial != nullptr ? kLiveSplitWorkMax : 0;
+  return 8 * ((whole + 7) / 8 + (split_work + live_split + 7) / 8);
 }
 
 template <typename T, bool HAS_ZP, bool HAS_PERM>
@@ -817,19 +862,25 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 
   int tile, tile_m, tile_n, split;
   bool whole_k;
+  int steps_per_split = p.k_steps_per_split;
+  int partial_at;   // without whole_k: index of this workgroup's partial tile, (split, split tile)
   if (GROUPED) {
     // The launch is sized for the most row tiles the routing could make; the tiles there are
     // (tile_table[0]) are numbered here in bands of four row tiles, so that the 32 workgroups an
     // XCD holds share 4 panels of A and 8 panels of W (of one expert where the routing is even),
     // and every XCD gets its share of them.
-    TileParams live = p;
-    live.tiles_m = p.tile_table[0];
-    live.tile_band = 4;
+    // With room for partial tiles the K split is planned here too (plan_live_split).
+    const TileParams live = live_tiles(p);
     if (live.tiles_m <= 0 || !tile_of_workgroup(live, tile, split, whole_k)) return;
     tile_coords(live, tile, tile_m, tile_n);
+    steps_per_split = live.k_steps_per_split;
+    const int first_split = whole_tiles(live);
+    partial_at = split * (live.tiles_m * live.tiles_n - first_split) + tile - first_split;
   } else {
     if (!tile_of_workgroup(p, tile, split, whole_k)) return;
     tile_coords(p, tile, tile_m, tile_n);
+    const int first_split = whole_tiles(p);
+    partial_at = split * (p.tiles_m * p.tiles_n - first_split) + tile - first_split;
   }
   // Grouped calls: row tile t is up to four consecutive 64-slot blocks of one expert, listed in
   // tile_table; rows are slots of sorted_ids (as in marlin_tile_async_kernel).
@@ -885,8 +936,8 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   const uint32_t s_lds = (uint32_t)(uintptr_t)(lds_void_t*)sring;
 
   // K steps [k_first, k_tiles) of this workgroup
-  const int k_first = whole_k ? 0 : split * p.k_steps_per_split;
-  const int k_tiles = whole_k ? p.size_k / kTileK : min(p.size_k / kTileK, k_first + p.k_steps_per_split);
+  const int k_first = whole_k ? 0 : split * steps_per_split;
+  const int k_tiles = whole_k ? p.size_k / kTileK : min(p.size_k / kTileK, k_first + steps_per_split);
 
   u32x4_t wq[kWideStages][2 * kChunkLoads];   // packed chunks in flight or waiting (8-bit: [2 b + h], h = high rows)
   // the scale row of step kt (clamped to the last step) into its ring position; MXFP4: the row of
@@ -1219,12 +1270,10 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
 #undef SONAR_WIDE_READ
 
   if (!active) return;
-  if (!GROUPED && !whole_k) {
+  if (!whole_k) {
     // partial tile of this K range, in the order tile_reduce_kernel reads: 1-KiB blocks
     // (half of the rows, strip, column block, row block)
-    const int first_split = whole_tiles(p);
-    const int split_tiles = p.tiles_m * p.tiles_n - first_split;
-    float4* dst = p.partial + ((size_t)(split * split_tiles + tile - first_split) * kRows + wave * 32) * 64 + lane;
+    float4* dst = p.partial + ((size_t)partial_at * kRows + wave * 32) * 64 + lane;
 #pragma unroll
     for (int nb = 0; nb < 4; ++nb)
 #pragma unroll
@@ -1321,6 +1370,60 @@ __global__ __launch_bounds__(256) void tile_reduce_kernel(const TileParams p) {
   o.x = (uint32_t)Dq<T>::from_float(acc.x + bias[0]) | ((uint32_t)Dq<T>::from_float(acc.y + bias[1]) << 16);
   o.y = (uint32_t)Dq<T>::from_float(acc.z + bias[2]) | ((uint32_t)Dq<T>::from_float(acc.w + bias[3]) << 16);
   *reinterpret_cast<uint2*>(p.c + (long)m * p.size_n + strip * kStripN + nl) = o;
+}
+
+// The same for a grouped call whose kernel has split some of its tiles along K (plan_live_split):
+// rows are slots of sorted_ids, bias and global scale the expert's, the routing weight applied as
+// in the kernel's own epilogue.  Launched for the most tiles there can be; the rest leaves at once.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams p) {
+  const int lane = threadIdx.x & 63;
+  const int col16 = lane & 15, kb = lane >> 4;
+  const int unit = blockIdx.x * 4 + (threadIdx.x >> 6);   // (split tile, 1-KiB block of the partial tile)
+  const TileParams live = live_tiles(p);
+  if (live.tiles_m <= 0 || live.k_splits < 2) return;
+  const int first_split = live.whole_tiles;
+  const int tiles = live.tiles_m * live.tiles_n - first_split;
+  if (unit >= tiles * kTileM) return;
+  const int tile = unit / kTileM;
+  const int within = unit - tile * kTileM;
+  const int half = within >> 7, wave = (within >> 5) & 3;
+  const int nb = (within >> 3) & 3, mb = within & 7;
+  int tile_m, tile_n;
+  tile_coords(live, first_split + tile, tile_m, tile_n);
+  const int strip = tile_n * (kTileN / kStripN) + wave;
+  if (strip * kStripN >= p.size_n) return;
+  const int first_slot = p.tile_table[1 + 3 * tile_m] * 64;
+  const int tile_rows = p.tile_table[2 + 3 * tile_m] * 64;
+  const long expert = p.tile_table[3 + 3 * tile_m];
+  const int r = 128 * half + 16 * mb + col16;
+  const int id = r < tile_rows ? p.sorted_ids[first_slot + r] : p.rows_total;
+  if ((unsigned)id >= (unsigned)p.rows_total) return;   // padding slot
+  floatx4_t acc = floatx4_t{0.f, 0.f, 0.f, 0.f};
+  for (int s = 0; s < live.k_splits; ++s) {
+    const float4 v = p.partial[((size_t)(s * tiles + tile) * kTileM + within) * 64 + lane];
+    acc += floatx4_t{v.x, v.y, v.z, v.w};
+  }
+  if (p.global_scale) acc = acc * p.global_scale[expert];
+  const int nl = 16 * nb + 4 * kb;
+  float bias[4] = {0.f, 0.f, 0.f, 0.f};
+  if (p.bias) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+      bias[i] = Dq<T>::to_float(p.bias[expert * p.expert_bias_stride + strip * kStripN + scale_slot(nl + i, false)]);
+  }
+  uint16_t o[4] = {Dq<T>::from_float(acc.x + bias[0]), Dq<T>::from_float(acc.y + bias[1]),
+                   Dq<T>::from_float(acc.z + bias[2]), Dq<T>::from_float(acc.w + bias[3])};
+  if (p.mul_topk) {
+    // rounded to the activation type, the product formed and rounded in that type (as in the kernel)
+    const float row_w = Dq<T>::to_float(Dq<T>::from_float(p.topk_weights[id]));
+#pragma unroll
+    for (int i = 0; i < 4; ++i) o[i] = Dq<T>::from_float(Dq<T>::to_float(o[i]) * row_w);
+  }
+  uint2 packed;
+  packed.x = (uint32_t)o[0] | ((uint32_t)o[1] << 16);
+  packed.y = (uint32_t)o[2] | ((uint32_t)o[3] << 16);
+  *reinterpret_cast<uint2*>(p.c + (long)id * p.size_n + strip * kStripN + nl) = packed;
 }
 
 // Builds the row-tile table of a grouped call: runs of blocks with the same
@@ -1769,6 +1872,13 @@ int moe_tile_max(int64_t sorted_len, int64_t num_experts) {
 size_t moe_tile_table_bytes(int64_t sorted_len, int64_t num_experts) {
   return (size_t)(1 + 3 * moe_tile_max(sorted_len, num_experts)) * sizeof(int32_t);
 }
+// Room for the fp32 partial tiles of a grouped call that splits some of its tiles along K on the
+// device (plan_live_split): 64 MiB where K allows a split, else none.
+size_t moe_tile_partial_bytes(int64_t size_k) {
+  const int64_t k_steps = size_k / kTileK;
+  if (size_k % (4 * kTileK) != 0 || k_steps < 16) return 0;
+  return (size_t)kLiveSplitWorkMax * kTileM * 1024;
+}
 
 // Called by sonar_moe_wna16_marlin_gemm for 64-slot blocks without act-order
 // when group_size % 64 == 0 (or one group) and size_k % 64 == 0.
@@ -1776,7 +1886,8 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   const float* global_scale, const uint32_t* zeros, const int32_t* sorted_ids, int64_t sorted_len, const int32_t* expert_ids,
                   const int32_t* num_post_pad, const float* topk_weights, int64_t top_k, int mul_topk,
                   int64_t num_experts, int32_t* table, int dtype, int64_t size_m, int64_t size_n, int64_t size_k,
-                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, int bits, bool fp8, hipStream_t st) {
+                  int64_t num_groups, int group_size, int a_by_slot, bool fp4, int bits, bool fp8, void* partial,
+                  size_t partial_bytes, hipStream_t st) {
   const int max_tiles = moe_tile_max(sorted_len, num_experts);
   const int blocks_max = (int)((sorted_len + 63) / 64);
   moe_tile_table_kernel<<<1, 256, (size_t)blocks_max * sizeof(int32_t), st>>>(expert_ids, num_post_pad, blocks_max, 64,
@@ -1818,6 +1929,14 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   p.expert_s_stride = (long)(num_groups * size_n);
   p.expert_z_stride = (long)(num_groups * (size_n / 8));
   p.expert_bias_stride = (long)size_n;
+  // The wide kernel splits the tiles of a short last round (or all of them when they are few) along
+  // K, given room for their partial tiles; moe_tile_reduce_kernel sums them.
+  static const bool no_live_split = getenv("SONAR_MARLIN_NO_MOE_K_SPLIT") != nullptr;   // debugging aid
+  const bool wide = fp4 ? wide_applies_fp4(p) : (bits == 8 ? wide_applies8(p) : wide_applies(p));
+  const size_t partial_need = moe_tile_partial_bytes(size_k);
+  if (wide && !no_live_split && partial != nullptr && partial_need > 0 && partial_bytes >= partial_need &&
+      ((uintptr_t)partial) % 16 == 0)
+    p.partial = static_cast<float4*>(partial);
   int rc;
   if (fp4 && global_scale != nullptr && wide_applies_fp4(p))
     rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide_nvfp4<_Float16, true>(p, st)
@@ -1842,7 +1961,15 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   else
     rc = zeros ? launch_tile_grouped<__bf16, true>(p, st) : launch_tile_grouped<__bf16, false>(p, st);
   if (rc) return rc;
-  return launch_status("tile kernel (grouped)");
+  if (int rc2 = launch_status("tile kernel (grouped)")) return rc2;
+  if (p.partial != nullptr) {
+    const int64_t tiles = std::min<int64_t>((int64_t)max_tiles * p.tiles_n, kLiveSplitTilesMax);
+    const int blocks = (int)(tiles * (kTileM / 4));
+    if (dtype == SONAR_DTYPE_F16) moe_tile_reduce_kernel<_Float16><<<blocks, 256, 0, st>>>(p);
+    else moe_tile_reduce_kernel<__bf16><<<blocks, 256, 0, st>>>(p);
+    return launch_status("moe_tile_reduce_kernel");
+  }
+  return SONAR_OK;
 }
 
 }  // namespace sonar

@@ -87,6 +87,7 @@ def grouped() -> None:
     from tests import test_gpu_moe as tm
     for case in [(300, 4, 2, 256, 256, 128, "fp16", False, False, False, 64, True),
                  (700, 8, 2, 512, 128, 64, "bf16", True, False, True, 64, False),
+                 (900, 3, 2, 2048, 256, 128, "bf16", True, False, True, 64, False),   # K split on the device
                  (40, 4, 2, 256, 128, 128, "fp16", False, False, False, 16, True),
                  (3, 8, 2, 512, 256, 128, "bf16", True, False, True, 8, False),
                  (130, 4, 2, 256, 320, -1, "fp16", False, False, True, 32, True),

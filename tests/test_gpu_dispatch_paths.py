@@ -27,6 +27,7 @@ SWITCHES = [
     "SONAR_MARLIN_MAX_K_SPLITS=1",   # no split K in the tile kernel
     "SONAR_MARLIN_NO_MOE_TILE",      # the grouped streaming kernel for 64-slot blocks
     "SONAR_MARLIN_NO_MOE_FAST",      # ... and for blocks of up to 32 slots
+    "SONAR_MARLIN_NO_MOE_K_SPLIT",   # the grouped wide tile kernel never cuts its tiles along K
     "SONAR_MARLIN_NO_MOE_PERMUTED_COPY",   # act-order experts: the gathering kernel although scratch has room
 ]
 

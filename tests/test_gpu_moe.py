@@ -103,6 +103,14 @@ MOE_CASES = [
     (90, 8, 2, 384, 128, -1, "fp16", False, False, False, 64, False),
     (1100, 2, 1, 128, 512, 128, "bf16", False, False, True, 64, False),
     (900, 2, 2, 256, 512, 32, "fp16", True, False, True, 64, True),      # groups of 32 rows in the tile kernel
+    # K of 16 steps or more in whole passes of four: the wide kernel cuts its few tiles along K on the device
+    # (fp32 partial tiles through scratch, moe_tile_reduce_kernel); act-order through the permuted copy
+    (700, 4, 2, 1024, 320, 128, "fp16", False, False, False, 64, True),
+    (900, 3, 2, 2048, 256, 128, "bf16", True, False, True, 64, False),
+    (640, 5, 2, 1280, 192, 64, "bf16", False, False, True, 64, True),
+    (650, 2, 2, 1024, 256, 128, "fp16", False, True, False, 64, True),
+    # more tiles than compute units with a short last round (9 row tiles x 33 = 297) and K of 48 steps
+    (1100, 3, 2, 3072, 8448, 128, "bf16", False, False, True, 64, True),
 ]
 
 
@@ -252,7 +260,9 @@ def test_moe_matches_dense_gemm_per_expert():
     (16, 4096, 28672, "uint4b8"), (64, 14336, 4096, "uint4b8"), (256, 4096, 28672, "uint4b8"),
     (600, 14336, 4096, "uint4b8"),
     # 8-bit codes: blocks of 64 slots run the tile kernel's 8-bit form, smaller ones the general grouped kernel
-    (700, 4096, 2048, "uint8b128"), (2048, 2048, 1024, "fp8"), (64, 2048, 1024, "uint8b128")])
+    (700, 4096, 2048, "uint8b128"), (2048, 2048, 1024, "fp8"), (64, 2048, 1024, "uint8b128"),
+    # MXFP4 in the tile kernel with few tiles, and with a short last round of them (384 = 256 + 128): both cut along K
+    (700, 4096, 2048, "mxfp4"), (2100, 14336, 4096, "mxfp4")])
 def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     """Mixtral-8x7B expert shapes (8 experts, top 2, the block size of the
     reference's rule), where the CPU oracle is too slow: every routed slot must
@@ -264,10 +274,14 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     e, top_k, dtype = 8, 2, torch.bfloat16
     gen = torch.Generator(device=gu.DEV).manual_seed(tokens + n)
     lib = _lib.load()
-    b_type = {"uint4b8": _lib.TYPE_UINT4B8, "uint8b128": _lib.TYPE_UINT8B128, "fp8": _lib.TYPE_FLOAT8_E4M3FN}[wtype]
-    words = k * n // (8 if wtype == "uint4b8" else 4)
+    b_type = {"uint4b8": _lib.TYPE_UINT4B8, "uint8b128": _lib.TYPE_UINT8B128, "fp8": _lib.TYPE_FLOAT8_E4M3FN,
+              "mxfp4": _lib.TYPE_FLOAT4_E2M1F}[wtype]
+    words = k * n // (8 if wtype in ("uint4b8", "mxfp4") else 4)
+    groups = k // (32 if wtype == "mxfp4" else 128)
     native = torch.randint(-2 ** 31, 2 ** 31 - 1, (e, words), dtype=torch.int32, device=gu.DEV, generator=gen)
-    scales = torch.rand((e, k // 128, n), device=gu.DEV, generator=gen) * 9e-3 + 1e-3
+    scales = torch.rand((e, groups, n), device=gu.DEV, generator=gen) * 9e-3 + 1e-3
+    if wtype == "mxfp4":   # powers of two
+        scales = torch.exp2(torch.randint(-9, -5, (e, groups, n), device=gu.DEV, generator=gen).float())
     if wtype == "uint8b128":
         scales = scales / 16
     if wtype == "fp8":   # the exponent bias of the codes is folded into the scales: 2^120 for bf16
@@ -286,7 +300,7 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     _lib.check(lib.sonar_moe_wna16_marlin_gemm(
         gu.ptr(a), gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None, gu.ptr(scales), None, None, None,
         gu.ptr(workspace), workspace.numel(), gu.ptr(scr), nbytes, gu.ptr(sid), sid.numel(), gu.ptr(eid),
-        gu.ptr(npp), None, bs, top_k, 0, e, _lib.DTYPE_BF16, b_type, tokens, n, k, k // 128, 1, 0, 1,
+        gu.ptr(npp), None, bs, top_k, 0, e, _lib.DTYPE_BF16, b_type, tokens, n, k, groups, 1, 0, 1,
         gu.stream()))
     torch.cuda.synchronize()
     assert bool(torch.isfinite(c.float()).all())
@@ -303,7 +317,7 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
         _lib.check(lib.sonar_marlin_gemm(
             gu.ptr(rows), k, gu.ptr(dense), gu.ptr(native[ex]), _lib.LAYOUT_GFX950, None, gu.ptr(scales[ex]), None,
             None, None, gu.ptr(workspace), workspace.numel(), gu.ptr(dscr), dscr.numel(), _lib.DTYPE_BF16,
-            b_type, m, n, k, k // 128, 1, 0, 1, gu.stream()))
+            b_type, m, n, k, groups, 1, 0, 1, gu.stream()))
         got = c[torch.from_numpy(slots).to(gu.DEV)].float()
         err = float((got - dense.float()).abs().max())
         assert err <= 1e-2 * scale, (ex, err, scale)
