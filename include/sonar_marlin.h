@@ -330,8 +330,8 @@ int sonar_marlin_gemm_noalloc(const void* a, int64_t a_row_stride, void* c,
  *                in b_layout order; b_type_id uint4b8, uint4, uint8b128, float8_e4m3fn
  *                or float4_e2m1f (scales as described at the type ids)
  *   b_scales     dtype[num_experts][num_groups][N]; b_zeros / b_bias likewise
- *   scratch      sonar_moe_marlin_gemm_scratch_bytes(): for 64-slot blocks the table of
- *                row tiles and 64 MiB for fp32 partial tiles (the tile kernel cuts few
+ *   scratch      sonar_moe_marlin_gemm_scratch_bytes(): for 64-slot blocks the tables of
+ *                row tiles and 96 MiB for fp32 partial tiles (the tile kernel cuts few
  *                tiles, or those of a short last round, along K; with less, down to
  *                the table alone, it runs without that); act-order calls run 4 to
  *                20 times faster with sorted_len * K * 2 bytes more behind that

@@ -161,7 +161,7 @@ __host__ __device__ __forceinline__ LiveSplit plan_live_split(int tiles, int k_s
 __device__ __forceinline__ TileParams live_tiles(const TileParams& p) {
   TileParams live = p;
   live.tiles_m = p.tile_table[0];
-  live.tile_band = 4;
+  live.tile_band = p.tile_rows == kTileM ? 4 : 8;   // the same rows of A per band with either tile size
   if (p.partial != nullptr) {
     const LiveSplit s = plan_live_split(live.tiles_m * live.tiles_n, p.size_k / kTileK);
     live.k_splits = s.splits;
@@ -846,7 +846,7 @@ __global__ __launch_bounds__(256) __attribute__((amdgpu_waves_per_eu(1, 1))) voi
   static_assert(!FP4 || ((NV || std::is_same<T, __bf16>::value) && !HAS_ZP), "MXFP4: bf16; float4 codes: no zero points");
   static_assert(!NV || (FP4 && RB == 16), "NVFP4 is float4 codes; 256-row tiles");
   static_assert(!(W8 != 0 && G32) || RB == 16, "8-bit codes with groups of 32 rows: 256-row tiles");
-  static_assert(RB == 16 || (RB == 8 && !GROUPED), "256-row tiles, or 128-row tiles for dense calls");
+  static_assert(RB == 16 || RB == 8, "256-row tiles or 128-row tiles");
   constexpr int kRows = 16 * RB;
   constexpr int kStage = wide_stage(RB), kWideA = wide_a(RB), kWideOps = wide_ops(RB, G32, W8 != 0);
   constexpr int kAgprBlocks = RB == 16 ? 14 : RB;   // row blocks whose accumulators sit in AGPRs
@@ -1384,9 +1384,10 @@ __global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams p
   if (live.tiles_m <= 0 || live.k_splits < 2) return;
   const int first_split = live.whole_tiles;
   const int tiles = live.tiles_m * live.tiles_n - first_split;
-  if (unit >= tiles * kTileM) return;
-  const int tile = unit / kTileM;
-  const int within = unit - tile * kTileM;
+  const int blocks = p.tile_rows;   // 1-KiB blocks per partial tile: 256 or 128
+  if (unit >= tiles * blocks) return;
+  const int tile = unit / blocks;
+  const int within = unit - tile * blocks;
   const int half = within >> 7, wave = (within >> 5) & 3;
   const int nb = (within >> 3) & 3, mb = within & 7;
   int tile_m, tile_n;
@@ -1401,7 +1402,7 @@ __global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams p
   if ((unsigned)id >= (unsigned)p.rows_total) return;   // padding slot
   floatx4_t acc = floatx4_t{0.f, 0.f, 0.f, 0.f};
   for (int s = 0; s < live.k_splits; ++s) {
-    const float4 v = p.partial[((size_t)(s * tiles + tile) * kTileM + within) * 64 + lane];
+    const float4 v = p.partial[((size_t)(s * tiles + tile) * blocks + within) * 64 + lane];
     acc += floatx4_t{v.x, v.y, v.z, v.w};
   }
   if (p.global_scale) acc = acc * p.global_scale[expert];
@@ -1427,33 +1428,45 @@ __global__ __launch_bounds__(256) void moe_tile_reduce_kernel(const TileParams p
 }
 
 // Builds the row-tile table of a grouped call: runs of blocks with the same
-// expert are cut into tiles of up to four blocks.  One workgroup; expert_ids
-// is staged in LDS and scanned by one thread (a few hundred entries).
+// expert are cut into tiles of up to four blocks.  With `table_small` the one or
+// two blocks a run ends in go there instead, to be computed as a 128-row tile at
+// half the cost.  One workgroup; expert_ids is staged in LDS and scanned by one
+// thread (a few hundred entries).
 __global__ __launch_bounds__(256) void moe_tile_table_kernel(const int32_t* __restrict__ expert_ids,
                                                             const int32_t* __restrict__ num_post_pad,
                                                             int num_blocks_max, int block_size, int num_experts,
-                                                            int32_t* __restrict__ table, int max_tiles) {
+                                                            int32_t* __restrict__ table,
+                                                            int32_t* __restrict__ table_small, int max_tiles) {
   extern __shared__ int32_t ids[];
   int blocks = num_post_pad[0] / block_size;
   if (blocks > num_blocks_max) blocks = num_blocks_max;
   for (int b = threadIdx.x; b < blocks; b += blockDim.x) ids[b] = expert_ids[b];
   __syncthreads();
   if (threadIdx.x != 0) return;
-  int tiles = 0;
+  int tiles = 0, small = 0;
   int b = 0;
-  while (b < blocks && tiles < max_tiles) {
+  while (b < blocks) {
     const int e = ids[b];
-    int n = 1;
-    while (n < 4 && b + n < blocks && ids[b + n] == e) ++n;
+    int run = 1;
+    while (b + run < blocks && ids[b + run] == e) ++run;
     if (e >= 0 && e < num_experts) {
-      table[1 + 3 * tiles] = b;
-      table[2 + 3 * tiles] = n;
-      table[3 + 3 * tiles] = e;
-      ++tiles;
+      for (int at = 0; at < run; at += 4) {
+        const int n = min(4, run - at);
+        const bool to_small = table_small != nullptr && n <= 2;
+        int32_t* t = to_small ? table_small : table;
+        int& count = to_small ? small : tiles;
+        if (count < max_tiles) {
+          t[1 + 3 * count] = b + at;
+          t[2 + 3 * count] = n;
+          t[3 + 3 * count] = e;
+          ++count;
+        }
+      }
     }
-    b += n;
+    b += run;
   }
   table[0] = tiles;
+  if (table_small != nullptr) table_small[0] = small;
 }
 
 template <typename T, bool HAS_ZP, bool G32>
@@ -1553,9 +1566,7 @@ int launch_tile_wide_fp4_rows(const TileParams& p, hipStream_t st) {
 }
 template <bool GROUPED>
 int launch_tile_wide_fp4(const TileParams& p, hipStream_t st) {
-  if constexpr (!GROUPED) {
-    if (p.tile_rows == 128) return launch_tile_wide_fp4_rows<false, 8>(p, st);
-  }
+  if (p.tile_rows == 128) return launch_tile_wide_fp4_rows<GROUPED, 8>(p, st);
   return launch_tile_wide_fp4_rows<GROUPED, 16>(p, st);
 }
 // NVFP4: either activation type, groups of 16 rows, a global scale (one per expert when GROUPED)
@@ -1591,12 +1602,11 @@ int launch_tile_wide8_groups(const TileParams& p, hipStream_t st) {
 template <typename T, bool GROUPED>
 int launch_tile_wide8(const TileParams& p, bool fp8, hipStream_t st) {
   const bool g32 = wide_groups_of_32(p);
-  if constexpr (!GROUPED) {   // 128-row tiles (dense calls with few tiles)
-    if (p.tile_rows == 128 && g32) return fail(SONAR_E_INVALID, "internal: 8-bit codes with groups of 32 rows run on 256-row tiles");
-    if (p.tile_rows == 128)
-      return fp8 ? launch_tile_wide8_groups<T, false, 2, false, 8>(p, st)
-                 : launch_tile_wide8_groups<T, false, 1, false, 8>(p, st);
-  }
+  // 128-row tiles (dense calls with few tiles; the short ends of an expert's rows)
+  if (p.tile_rows == 128 && g32) return fail(SONAR_E_INVALID, "internal: 8-bit codes with groups of 32 rows run on 256-row tiles");
+  if (p.tile_rows == 128)
+    return fp8 ? launch_tile_wide8_groups<T, GROUPED, 2, false, 8>(p, st)
+               : launch_tile_wide8_groups<T, GROUPED, 1, false, 8>(p, st);
   if (fp8) return g32 ? launch_tile_wide8_groups<T, GROUPED, 2, true>(p, st)
                       : launch_tile_wide8_groups<T, GROUPED, 2, false>(p, st);
   return g32 ? launch_tile_wide8_groups<T, GROUPED, 1, true>(p, st)
@@ -1618,15 +1628,15 @@ template <typename T, bool HAS_ZP, bool GROUPED>
 int launch_tile_wide_g32(const TileParams& p, hipStream_t st) {
   if constexpr (!GROUPED) {
     if (p.tile_rows == 128) return launch_tile_wide_g32_rows<T, HAS_ZP, false, 8>(p, st);
+  } else if (p.tile_rows == 128) {
+    return fail(SONAR_E_INVALID, "internal: grouped calls with groups of 32 rows run on 256-row tiles");
   }
   return launch_tile_wide_g32_rows<T, HAS_ZP, GROUPED, 16>(p, st);
 }
 template <typename T, bool HAS_ZP, bool GROUPED = false>
 int launch_tile_wide(const TileParams& p, hipStream_t st) {
   if (wide_groups_of_32(p)) return launch_tile_wide_g32<T, HAS_ZP, GROUPED>(p, st);
-  if constexpr (!GROUPED) {
-    if (p.tile_rows == 128) return launch_tile_wide_rows<T, HAS_ZP, false, 8>(p, st);
-  }
+  if (p.tile_rows == 128) return launch_tile_wide_rows<T, HAS_ZP, GROUPED, 8>(p, st);
   return launch_tile_wide_rows<T, HAS_ZP, GROUPED, 16>(p, st);
 }
 
@@ -1869,15 +1879,23 @@ int moe_tile_max(int64_t sorted_len, int64_t num_experts) {
   (void)num_experts;
   return (int)((sorted_len + 63) / 64);
 }
+// (two tables: the tiles of up to four blocks, and the one- or two-block ends of the experts' rows
+// that the wide kernel computes as 128-row tiles)
+static size_t moe_one_table_bytes(int64_t sorted_len) {
+  return ((size_t)(1 + 3 * moe_tile_max(sorted_len, 0)) * sizeof(int32_t) + 255) & ~(size_t)255;
+}
 size_t moe_tile_table_bytes(int64_t sorted_len, int64_t num_experts) {
-  return (size_t)(1 + 3 * moe_tile_max(sorted_len, num_experts)) * sizeof(int32_t);
+  (void)num_experts;
+  return 2 * moe_one_table_bytes(sorted_len);
 }
 // Room for the fp32 partial tiles of a grouped call that splits some of its tiles along K on the
-// device (plan_live_split): 64 MiB where K allows a split, else none.
+// device (plan_live_split): 64 MiB for the 256-row tiles and 32 MiB for the 128-row tiles where K
+// allows a split, else none.
+static size_t moe_partial_bytes_of(int tile_rows) { return (size_t)kLiveSplitWorkMax * tile_rows * 1024; }
 size_t moe_tile_partial_bytes(int64_t size_k) {
   const int64_t k_steps = size_k / kTileK;
   if (size_k % (4 * kTileK) != 0 || k_steps < 16) return 0;
-  return (size_t)kLiveSplitWorkMax * kTileM * 1024;
+  return moe_partial_bytes_of(kTileM) + moe_partial_bytes_of(128);
 }
 
 // Called by sonar_moe_wna16_marlin_gemm for 64-slot blocks without act-order
@@ -1890,9 +1908,6 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
                   size_t partial_bytes, hipStream_t st) {
   const int max_tiles = moe_tile_max(sorted_len, num_experts);
   const int blocks_max = (int)((sorted_len + 63) / 64);
-  moe_tile_table_kernel<<<1, 256, (size_t)blocks_max * sizeof(int32_t), st>>>(expert_ids, num_post_pad, blocks_max, 64,
-                                                                             (int)num_experts, table, max_tiles);
-  if (int rc = launch_status("moe_tile_table_kernel")) return rc;
   TileParams p;
   p.tile_begin = p.tile_count = 0;
   p.global_scale = global_scale;   // NVFP4: one per expert
@@ -1937,6 +1952,44 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   if (wide && !no_live_split && partial != nullptr && partial_need > 0 && partial_bytes >= partial_need &&
       ((uintptr_t)partial) % 16 == 0)
     p.partial = static_cast<float4*>(partial);
+  // ... and computes the one or two blocks an expert's rows end in as a 128-row tile, in a launch of
+  // its own (the forms that have 128-row tiles: not NVFP4, not groups of 32 rows but MXFP4's)
+  static const bool no_small = getenv("SONAR_MARLIN_NO_MOE_128_ROW_TILES") != nullptr;   // debugging aid
+  const bool nvfp4 = fp4 && global_scale != nullptr;
+  const bool two_sizes = wide && !no_small && !nvfp4 && (fp4 || !wide_groups_of_32(p));
+  int32_t* table_small = two_sizes ? table + moe_one_table_bytes(sorted_len) / sizeof(int32_t) : nullptr;
+  moe_tile_table_kernel<<<1, 256, (size_t)blocks_max * sizeof(int32_t), st>>>(expert_ids, num_post_pad, blocks_max, 64,
+                                                                             (int)num_experts, table, table_small,
+                                                                             max_tiles);
+  if (int rc = launch_status("moe_tile_table_kernel")) return rc;
+  auto reduce = [&](const TileParams& q) -> int {
+    if (q.partial == nullptr) return SONAR_OK;
+    const int64_t tiles = std::min<int64_t>((int64_t)max_tiles * q.tiles_n, kLiveSplitTilesMax);
+    const int blocks = (int)(tiles * (q.tile_rows / 4));
+    if (dtype == SONAR_DTYPE_F16) moe_tile_reduce_kernel<_Float16><<<blocks, 256, 0, st>>>(q);
+    else moe_tile_reduce_kernel<__bf16><<<blocks, 256, 0, st>>>(q);
+    return launch_status("moe_tile_reduce_kernel");
+  };
+  if (two_sizes) {
+    TileParams q = p;
+    q.tile_rows = 128;
+    q.tile_table = table_small;
+    if (p.partial != nullptr)
+      q.partial = reinterpret_cast<float4*>(static_cast<char*>(partial) + moe_partial_bytes_of(kTileM));
+    int rc;
+    if (fp4)
+      rc = launch_tile_wide_fp4<true>(q, st);
+    else if (bits == 8)
+      rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide8<_Float16, true>(q, fp8, st)
+                                    : launch_tile_wide8<__bf16, true>(q, fp8, st);
+    else if (dtype == SONAR_DTYPE_F16)
+      rc = zeros ? launch_tile_wide<_Float16, true, true>(q, st) : launch_tile_wide<_Float16, false, true>(q, st);
+    else
+      rc = zeros ? launch_tile_wide<__bf16, true, true>(q, st) : launch_tile_wide<__bf16, false, true>(q, st);
+    if (rc) return rc;
+    if (int rc2 = launch_status("tile kernel (grouped, 128-row tiles)")) return rc2;
+    if (int rc2 = reduce(q)) return rc2;
+  }
   int rc;
   if (fp4 && global_scale != nullptr && wide_applies_fp4(p))
     rc = dtype == SONAR_DTYPE_F16 ? launch_tile_wide_nvfp4<_Float16, true>(p, st)
@@ -1962,14 +2015,7 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
     rc = zeros ? launch_tile_grouped<__bf16, true>(p, st) : launch_tile_grouped<__bf16, false>(p, st);
   if (rc) return rc;
   if (int rc2 = launch_status("tile kernel (grouped)")) return rc2;
-  if (p.partial != nullptr) {
-    const int64_t tiles = std::min<int64_t>((int64_t)max_tiles * p.tiles_n, kLiveSplitTilesMax);
-    const int blocks = (int)(tiles * (kTileM / 4));
-    if (dtype == SONAR_DTYPE_F16) moe_tile_reduce_kernel<_Float16><<<blocks, 256, 0, st>>>(p);
-    else moe_tile_reduce_kernel<__bf16><<<blocks, 256, 0, st>>>(p);
-    return launch_status("moe_tile_reduce_kernel");
-  }
-  return SONAR_OK;
+  return reduce(p);
 }
 
 }  // namespace sonar

@@ -212,22 +212,28 @@ def apply_moe_activation(activation, output: torch.Tensor, input: torch.Tensor, 
     else:
         assert d == input.shape[-1], f"{name} expects equal sizes: {d} vs {input.shape[-1]}"
     f32 = torch.float32
-    g, u = input[..., :d].to(f32), input[..., d:].to(f32)
     dt = output.dtype
+
+    def halves():   # gate and up in fp32, for the torch expressions only (a pass over the tensor each)
+        return input[..., :d].to(f32), input[..., d:].to(f32)
+
     if name == "silu" and clamp_limit is None:
         silu_and_mul(output, input)
     elif name in ("silu", "swigluoai_uninterleave"):
         assert clamp_limit is not None, "SWIGLUOAI_UNINTERLEAVE requires clamp_limit"
         a, b = (1.0, 0.0) if name == "silu" else (float(alpha), float(beta))
         if not _gated_on_gpu(torch.ops.sonar_amd.silu_and_mul_with_clamp, output, input, float(clamp_limit), a, b):
+            g, u = halves()
             gc = g.clamp(max=clamp_limit).to(dt).to(f32)
             act = (gc / (1.0 + torch.exp(-gc * a))).to(dt).to(f32)
             output.copy_((act * (u.clamp(-clamp_limit, clamp_limit) + b)).to(dt))
     elif name == "gelu":
         if not _gated_on_gpu(torch.ops.sonar_amd.gelu_and_mul, output, input):
+            g, u = halves()
             output.copy_((torch.nn.functional.gelu(g).to(dt).to(f32) * u).to(dt))
     elif name == "gelu_tanh":
         if not _gated_on_gpu(torch.ops.sonar_amd.gelu_tanh_and_mul, output, input):
+            g, u = halves()
             output.copy_((torch.nn.functional.gelu(g, approximate="tanh").to(dt).to(f32) * u).to(dt))
     elif name == "swigluoai":      # gate and up alternate (gpt-oss checkpoints); alpha 1.702, limit 7.0
         if not _gated_on_gpu(torch.ops.sonar_amd.swigluoai_and_mul, output, input, 1.702, 7.0):
@@ -238,11 +244,13 @@ def apply_moe_activation(activation, output: torch.Tensor, input: torch.Tensor, 
         assert activation_situ_beta is not None, "SITU requires activation_situ_beta"
         lb = -1.0 if activation_situ_linear_beta is None else float(activation_situ_linear_beta)
         if not _gated_on_gpu(torch.ops.sonar_amd.situ_and_mul, output, input, float(activation_situ_beta), lb):
+            g, u = halves()
             bt = float(activation_situ_beta)
             up = lb * torch.tanh(u / lb) if lb > 0 else u
             output.copy_((bt * torch.tanh(g / bt) / (1.0 + torch.exp(-g)) * up).to(dt))
     elif name == "swiglustep":
         if not _gated_on_gpu(torch.ops.sonar_amd.swiglustep_and_mul, output, input, 7.0):
+            g, u = halves()
             output.copy_(((g * torch.sigmoid(g)).clamp(max=7.0) * u.clamp(-7.0, 7.0)).to(dt))
     elif name == "silu_no_mul":
         output.copy_(torch.nn.functional.silu(input))

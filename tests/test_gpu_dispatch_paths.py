@@ -28,6 +28,7 @@ SWITCHES = [
     "SONAR_MARLIN_NO_MOE_TILE",      # the grouped streaming kernel for 64-slot blocks
     "SONAR_MARLIN_NO_MOE_FAST",      # ... and for blocks of up to 32 slots
     "SONAR_MARLIN_NO_MOE_K_SPLIT",   # the grouped wide tile kernel never cuts its tiles along K
+    "SONAR_MARLIN_NO_MOE_128_ROW_TILES",   # ... and computes the short ends of the experts' rows as 256-row tiles
     "SONAR_MARLIN_NO_MOE_PERMUTED_COPY",   # act-order experts: the gathering kernel although scratch has room
 ]
 
