@@ -92,7 +92,7 @@ def check_columns(layer, a, c, m, cols, rows=None):
     assert ok, (err, big)
 
 
-@pytest.mark.parametrize("m", [1, 2, 4, 8, 16, 32, 64])
+@pytest.mark.parametrize("m", [1, 2, 4, 8, 16, 32, 48, 64])
 @pytest.mark.parametrize("name", list(LLAMA))
 def test_decode_sweep_meets_the_oracle_on_sampled_columns(name, m):
     """Benchmark configuration 2: bf16, every M of the sweep on every projection shape."""

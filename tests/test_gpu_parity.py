@@ -123,6 +123,11 @@ GEMM_CASES = [
     (33, 14336, 1024, 128, False, False, True),
     (64, 2048, 512, 128, True, False, False),
     (40, 4096, 640, -1, False, False, False),
+    # 33..64 rows on more strips than half the compute units: two workgroups of two blocks of rows per strip
+    (40, 1024, 8320, 128, True, False, True),
+    (64, 512, 16384, -1, False, False, False),
+    (33, 2048, 8448, 128, False, False, True),
+    (49, 256, 8256, 256, True, False, False),
 ]
 
 
