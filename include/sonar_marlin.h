@@ -428,6 +428,20 @@ int sonar_moe_sum(void* out, const void* in, int64_t tokens, int64_t topk, int64
 int sonar_moe_activation(void* out, const void* in, int64_t rows, int64_t d, int kind, float limit,
                          float alpha, float beta, int dtype, void* stream);
 
+/* Diagnostics for host-side tests; no counterpart in the reference.  The tile kernels'
+ * launches for a dense call (4-bit integer codes, no act-order, room for every partial
+ * tile), or for a grouped call whose routing made `row_tiles` row tiles of `tile_rows`
+ * rows out of at most `max_row_tiles`: one row of six int32 per workgroup that has
+ * work (launch, rows of a tile, row tile, column tile, first K step, end of its K
+ * steps), from the planning and mapping code the launches and the kernels run.
+ * Returns the number of such workgroups (rows beyond out_rows are counted, not
+ * written), -1 for arguments out of range.  Runs on the host; needs no GPU. */
+int64_t sonar_debug_tile_schedule(int64_t size_m, int64_t size_n, int64_t size_k,
+                                  int64_t num_groups, int32_t* out, int64_t out_rows);
+int64_t sonar_debug_moe_tile_schedule(int64_t row_tiles, int64_t max_row_tiles, int64_t size_n,
+                                      int64_t size_k, int tile_rows, int with_partial,
+                                      int32_t* out, int64_t out_rows);
+
 #ifdef __cplusplus
 }
 #endif

@@ -32,6 +32,8 @@ PROTOTYPES = {
     "sonar_marlin_last_error": (c_char_p, []),
     "sonar_marlin_version": (c_char_p, []),
     "sonar_marlin_last_decode_launch": (c_int, [c_void_p, c_int]),
+    "sonar_debug_tile_schedule": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_void_p, c_int64]),
+    "sonar_debug_moe_tile_schedule": (c_int64, [c_int64, c_int64, c_int64, c_int64, c_int, c_int, c_void_p, c_int64]),
     "sonar_gptq_marlin_repack": (c_int, [c_void_p, c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "sonar_awq_marlin_repack": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_int, c_void_p]),
     "sonar_marlin_to_gfx950": (c_int, [c_void_p, c_void_p, c_int64, c_int64, c_void_p]),

@@ -85,7 +85,7 @@ __device__ __forceinline__ uint4 load_a16(const TileParams& p, int row, int k0) 
 // Tiles are numbered band by band (tile_band rows of tiles), inside a band
 // column by column: with bands of 4 rows, 32 consecutive tiles are 4 panels
 // of A x 8 panels of W.
-__device__ __forceinline__ void tile_coords(const TileParams& p, int tile, int& tile_m, int& tile_n) {
+__host__ __device__ __forceinline__ void tile_coords(const TileParams& p, int tile, int& tile_m, int& tile_n) {
   const int band = tile / (p.tile_band * p.tiles_n);
   const int rem = tile - band * p.tile_band * p.tiles_n;
   const int rows = min(p.tile_band, p.tiles_m - band * p.tile_band);
@@ -106,13 +106,14 @@ __host__ __device__ __forceinline__ int whole_tiles(const TileParams& p) {
 // few panels of W, and after those a contiguous run of the (tile, split) pairs
 // of the split tiles, so that the short workgroups start last on every XCD.
 // Returns false for the padding ids of a run.
-__device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile, int& split, bool& whole_k) {
+__host__ __device__ __forceinline__ bool tile_of_block(const TileParams& p, int block, int& tile, int& split,
+                                                       bool& whole_k) {
   const int tiles = launch_tiles(p);
   const int whole = whole_tiles(p);
   const int split_tiles = tiles - whole;
   const int whole_per_xcd = (whole + 7) / 8;
   const int split_per_xcd = (split_tiles * p.k_splits + 7) / 8;
-  const int xcd = blockIdx.x & 7, i = blockIdx.x >> 3;
+  const int xcd = block & 7, i = block >> 3;
   whole_k = i < whole_per_xcd;
   if (whole_k) {
     tile = xcd * whole_per_xcd + i;
@@ -128,6 +129,9 @@ __device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile
   split = t / split_tiles;
   tile = whole + t - split * split_tiles;
   return true;
+}
+__device__ __forceinline__ bool tile_of_workgroup(const TileParams& p, int& tile, int& split, bool& whole_k) {
+  return tile_of_block(p, blockIdx.x, tile, split, whole_k);
 }
 
 // Grouped calls learn the number of their tiles on the device (the routing decides it), so the
@@ -157,10 +161,11 @@ __host__ __device__ __forceinline__ LiveSplit plan_live_split(int tiles, int k_s
   s.steps = steps;
   return s;
 }
-// The tiles there are in a grouped call, with the K split planned from them when the call has room for partial tiles.
-__device__ __forceinline__ TileParams live_tiles(const TileParams& p) {
+// The tiles there are in a grouped call (`row_tiles` of them down the rows), with the K split
+// planned from them when the call has room for partial tiles.
+__host__ __device__ __forceinline__ TileParams live_tiles_of(const TileParams& p, int row_tiles) {
   TileParams live = p;
-  live.tiles_m = p.tile_table[0];
+  live.tiles_m = row_tiles;
   live.tile_band = p.tile_rows == kTileM ? 4 : 8;   // the same rows of A per band with either tile size
   if (p.partial != nullptr) {
     const LiveSplit s = plan_live_split(live.tiles_m * live.tiles_n, p.size_k / kTileK);
@@ -170,6 +175,7 @@ __device__ __forceinline__ TileParams live_tiles(const TileParams& p) {
   }
   return live;
 }
+__device__ __forceinline__ TileParams live_tiles(const TileParams& p) { return live_tiles_of(p, p.tile_table[0]); }
 
 inline int tile_grid(const TileParams& p) {
   const int whole = whole_tiles(p);
@@ -1712,22 +1718,98 @@ bool tile_async_applies(bool has_perm, int64_t num_groups, int group_size) {
   return !has_perm && (num_groups == 1 || group_size % kTileK == 0 || group_size == 32);
 }
 
-// Called by sonar_marlin_gemm for size_m > 64.  Shapes and pointers have been
-// validated by the caller; size_k % 64 == 0 is required here.
-int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
-              const void* scales, const float* global_scale, const uint32_t* zeros, const int32_t* perm, int dtype,
-              int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
-              size_t partial_bytes, bool fp4, int bits, bool fp8, hipStream_t st) {
-  TileParams p;
-  p.global_scale = global_scale;
-  p.a = static_cast<const uint16_t*>(a);
-  p.lda = a_row_stride;
-  p.c = static_cast<uint16_t*>(c);
-  p.b = reinterpret_cast<const uint4*>(b);
-  p.bias = static_cast<const uint16_t*>(bias);
-  p.scales = static_cast<const uint16_t*>(scales);
-  p.zeros = zeros;
-  p.perm = perm;
+namespace {
+// What tile_gemm launches for a call the asynchronous tile kernels take: one launch (with
+// tile_reduce_kernel behind it when K is split), or two launches of the wide kernel.
+struct TileLaunches {
+  int count;          // 1 or 2; 0: an internal error
+  TileParams launch[2];
+};
+
+// `p` arrives with the shape, the pointers and one 256-row launch over the whole of K filled in.
+TileLaunches plan_tile_launches(TileParams p, int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
+                                int group_size, void* partial, size_t partial_bytes, bool fp4, bool nvfp4, int bits,
+                                bool has_perm) {
+  TileLaunches out;
+  out.count = 1;
+  const int steps_per_group = group_size / kTileK;
+  const bool wide128 = bits == 4 && !fp4 && !has_perm &&
+                       (num_groups == 1 || (group_size % kTileK == 0 && (steps_per_group & (steps_per_group - 1)) == 0));
+  const bool rows_97_128 = plan_rows_97_128(size_m, size_n, size_k, wide128);
+  GemmPlan plan = plan_gemm(size_m, size_n, size_k, true, 256, rows_97_128);
+  // few tiles and a call the wide kernel takes: 128-row tiles
+  static const bool no_128 = getenv("SONAR_MARLIN_NO_128_ROW_TILES") != nullptr;   // debugging aid
+  // (not for NVFP4 and 8-bit codes with groups of 32 rows, whose heavier dequantisation wants the 16 row blocks
+  // to hide behind: M = 512, K = 4096, N = 11008: NVFP4 69.9 us against 68.7, MXFP8 91.8 against 82.2)
+  const bool rows128_ok = !nvfp4 && !(bits == 8 && num_groups > 1 && group_size == 32);
+  if (!no_128 && rows128_ok && plan_prefers_128_rows(size_m, size_n, size_k, rows_97_128)) {
+    const GemmPlan plan128 = plan_gemm(size_m, size_n, size_k, true, 128, rows_97_128);
+    TileParams probe = p;
+    probe.tile_rows = 128;
+    probe.k_splits = plan128.k_splits;
+    probe.k_steps_per_split = plan128.k_steps_per_split;
+    if (plan128.tile && (fp4 ? wide_applies_fp4(probe) : wide_applies(probe)) &&
+        (plan128.k_splits == 1 || (partial != nullptr && partial_bytes >= plan_partial_bytes(plan128, size_m, size_n)))) {
+      plan = plan128;
+      p.tile_rows = 128;
+      p.tiles_m = (int)((size_m + 127) / 128);
+      p.tile_band = 8;   // the same rows of A per band as four 256-row tiles
+    }
+  }
+  if (plan.k_splits > 1 && partial != nullptr && partial_bytes >= plan_partial_bytes(plan, size_m, size_n)) {
+    p.k_splits = plan.k_splits;
+    p.k_steps_per_split = plan.k_steps_per_split;
+    p.whole_tiles = (int)plan.whole_tiles;
+    p.partial = static_cast<float4*>(partial);
+    static const char* max_splits = getenv("SONAR_MARLIN_MAX_K_SPLITS");  // debugging aid
+    if (max_splits && atoi(max_splits) >= 1 && p.k_splits > atoi(max_splits)) {
+      const int k_steps = (int)(size_k / kTileK);
+      p.k_splits = atoi(max_splits);
+      p.k_steps_per_split = (k_steps + p.k_splits - 1) / p.k_splits;
+      p.k_splits = (k_steps + p.k_steps_per_split - 1) / p.k_steps_per_split;
+      if (p.k_splits == 1) p.partial = nullptr;
+    }
+  }
+  out.launch[0] = p;
+  if (p.tile_rows != kTileM && !(fp4 ? wide_applies_fp4(p) : wide_applies(p))) {
+    out.count = 0;   // 128-row tiles exist in the wide tile kernel only
+    return out;
+  }
+  auto takes_wide = [&](const TileParams& q) {
+    return fp4 ? wide_applies_fp4(q) : (bits == 8 ? wide_applies8(q) : wide_applies(q));
+  };
+  // More tiles than compute units with a short last round (M = 4096, N = 6144: 384 tiles of 256
+  // rows = 256 + 128): instead of cutting the K ranges of that round's tiles in two and summing
+  // partial tiles in a third launch, the full rounds run as they are and the last round runs in
+  // a second launch as twice as many 128-row tiles over the whole of K: nothing goes through
+  // scratch (163 + 18 us of split tiles and their sum before).  Tile t of the 256-row numbering
+  // is tiles 2 t and 2 t + 1 of the 128-row numbering with bands twice as high.
+  static const bool no_two_sizes = getenv("SONAR_MARLIN_NO_TWO_TILE_SIZES") != nullptr;   // debugging aid
+  if (!no_two_sizes && !no_128 && rows128_ok && p.tile_rows == kTileM && plan.k_splits > 1 && plan.whole_tiles > 0 &&
+      (size_m - 1) % kTileM >= 128) {
+    TileParams big = p;
+    big.k_splits = 1;
+    big.k_steps_per_split = (int)(size_k / kTileK);
+    big.partial = nullptr;
+    big.tile_count = (int)plan.whole_tiles;
+    TileParams half = big;
+    half.tile_rows = 128;
+    half.tiles_m = 2 * p.tiles_m;
+    half.tile_band = 8;
+    half.tile_begin = 2 * (int)plan.whole_tiles;
+    half.tile_count = 2 * (p.tiles_m * p.tiles_n - (int)plan.whole_tiles);
+    if (takes_wide(big) && takes_wide(half)) {
+      out.count = 2;
+      out.launch[0] = big;
+      out.launch[1] = half;
+    }
+  }
+  return out;
+}
+
+// The shape of a dense call as one 256-row launch over the whole of K (no pointers).
+TileParams dense_tile_shape(int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size) {
+  TileParams p = {};
   p.size_m = (int)size_m;
   p.size_n = (int)size_n;
   p.size_k = (int)size_k;
@@ -1742,57 +1824,35 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
   p.k_splits = 1;
   p.whole_tiles = 0;  // read only with k_splits > 1
   p.k_steps_per_split = (int)(size_k / kTileK);
-  p.partial = nullptr;
-  p.sorted_ids = nullptr;
-  p.topk_weights = nullptr;
-  p.tile_table = nullptr;
-  p.rows_total = p.top_k = p.mul_topk = p.a_by_slot = 0;
-  p.expert_b_stride = p.expert_s_stride = p.expert_z_stride = p.expert_bias_stride = 0;
+  return p;
+}
+}  // namespace
+
+// Called by sonar_marlin_gemm for size_m > 64.  Shapes and pointers have been
+// validated by the caller; size_k % 64 == 0 is required here.
+int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, const void* bias,
+              const void* scales, const float* global_scale, const uint32_t* zeros, const int32_t* perm, int dtype,
+              int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups, int group_size, void* partial,
+              size_t partial_bytes, bool fp4, int bits, bool fp8, hipStream_t st) {
+  TileParams p = dense_tile_shape(size_m, size_n, size_k, num_groups, group_size);
+  p.global_scale = global_scale;
+  p.a = static_cast<const uint16_t*>(a);
+  p.lda = a_row_stride;
+  p.c = static_cast<uint16_t*>(c);
+  p.b = reinterpret_cast<const uint4*>(b);
+  p.bias = static_cast<const uint16_t*>(bias);
+  p.scales = static_cast<const uint16_t*>(scales);
+  p.zeros = zeros;
+  p.perm = perm;
   const bool zp = zeros != nullptr, pm = perm != nullptr;
   int rc;
   static const bool no_async = getenv("SONAR_MARLIN_NO_ASYNC_TILE") != nullptr;  // debugging aid
   const bool nvfp4 = fp4 && global_scale != nullptr;   // the caller has checked: groups of 16 rows
   if ((nvfp4 || tile_async_applies(pm, num_groups, group_size)) &&
       (!no_async || fp4 || bits == 8)) {   // float4 and 8-bit codes exist here only
-    const int steps_per_group = group_size / kTileK;
-    const bool wide128 = bits == 4 && !fp4 && !pm &&
-                         (num_groups == 1 || (group_size % kTileK == 0 && (steps_per_group & (steps_per_group - 1)) == 0));
-    const bool rows_97_128 = plan_rows_97_128(size_m, size_n, size_k, wide128);
-    GemmPlan plan = plan_gemm(size_m, size_n, size_k, true, 256, rows_97_128);
-    // few tiles and a call the wide kernel takes: 128-row tiles
-    static const bool no_128 = getenv("SONAR_MARLIN_NO_128_ROW_TILES") != nullptr;   // debugging aid
-    // (not for NVFP4 and 8-bit codes with groups of 32 rows, whose heavier dequantisation wants the 16 row blocks
-    // to hide behind: M = 512, K = 4096, N = 11008: NVFP4 69.9 us against 68.7, MXFP8 91.8 against 82.2)
-    const bool rows128_ok = !nvfp4 && !(bits == 8 && num_groups > 1 && group_size == 32);
-    if (!no_128 && rows128_ok && plan_prefers_128_rows(size_m, size_n, size_k, rows_97_128)) {
-      const GemmPlan plan128 = plan_gemm(size_m, size_n, size_k, true, 128, rows_97_128);
-      TileParams probe = p;
-      probe.tile_rows = 128;
-      probe.k_splits = plan128.k_splits;
-      probe.k_steps_per_split = plan128.k_steps_per_split;
-      if (plan128.tile && (fp4 ? wide_applies_fp4(probe) : wide_applies(probe)) &&
-          (plan128.k_splits == 1 || (partial != nullptr && partial_bytes >= plan_partial_bytes(plan128, size_m, size_n)))) {
-        plan = plan128;
-        p.tile_rows = 128;
-        p.tiles_m = (int)((size_m + 127) / 128);
-        p.tile_band = 8;   // the same rows of A per band as four 256-row tiles
-      }
-    }
-    if (plan.k_splits > 1 && partial != nullptr && partial_bytes >= plan_partial_bytes(plan, size_m, size_n)) {
-      p.k_splits = plan.k_splits;
-      p.k_steps_per_split = plan.k_steps_per_split;
-      p.whole_tiles = (int)plan.whole_tiles;
-      p.partial = static_cast<float4*>(partial);
-      static const char* max_splits = getenv("SONAR_MARLIN_MAX_K_SPLITS");  // debugging aid
-      if (max_splits && atoi(max_splits) >= 1 && p.k_splits > atoi(max_splits)) {
-        const int k_steps = (int)(size_k / kTileK);
-        p.k_splits = atoi(max_splits);
-        p.k_steps_per_split = (k_steps + p.k_splits - 1) / p.k_splits;
-        p.k_splits = (k_steps + p.k_steps_per_split - 1) / p.k_steps_per_split;
-        if (p.k_splits == 1) p.partial = nullptr;
-      }
-    }
-    if (p.tile_rows != kTileM && !(fp4 ? wide_applies_fp4(p) : wide_applies(p)))
+    const TileLaunches plan = plan_tile_launches(p, size_m, size_n, size_k, num_groups, group_size, partial,
+                                                 partial_bytes, fp4, nvfp4, bits, pm);
+    if (plan.count == 0)
       return fail(SONAR_E_INVALID, "internal: 128-row tiles exist in the wide tile kernel only");
     // the kernel a launch described by q takes
     auto launch = [&](const TileParams& q) -> int {
@@ -1818,36 +1878,13 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
       else
         return zp ? launch_tile_async<__bf16, true>(q, st) : launch_tile_async<__bf16, false>(q, st);
     };
-    auto takes_wide = [&](const TileParams& q) {
-      return fp4 ? wide_applies_fp4(q) : (bits == 8 ? wide_applies8(q) : wide_applies(q));
-    };
-    // More tiles than compute units with a short last round (M = 4096, N = 6144: 384 tiles of 256
-    // rows = 256 + 128): instead of cutting the K ranges of that round's tiles in two and summing
-    // partial tiles in a third launch, the full rounds run as they are and the last round runs in
-    // a second launch as twice as many 128-row tiles over the whole of K: nothing goes through
-    // scratch (163 + 18 us of split tiles and their sum before).  Tile t of the 256-row numbering
-    // is tiles 2 t and 2 t + 1 of the 128-row numbering with bands twice as high.
-    static const bool no_two_sizes = getenv("SONAR_MARLIN_NO_TWO_TILE_SIZES") != nullptr;   // debugging aid
-    if (!no_two_sizes && !no_128 && rows128_ok && p.tile_rows == kTileM && plan.k_splits > 1 && plan.whole_tiles > 0 &&
-        (size_m - 1) % kTileM >= 128) {
-      TileParams big = p;
-      big.k_splits = 1;
-      big.k_steps_per_split = (int)(size_k / kTileK);
-      big.partial = nullptr;
-      big.tile_count = (int)plan.whole_tiles;
-      TileParams half = big;
-      half.tile_rows = 128;
-      half.tiles_m = 2 * p.tiles_m;
-      half.tile_band = 8;
-      half.tile_begin = 2 * (int)plan.whole_tiles;
-      half.tile_count = 2 * (p.tiles_m * p.tiles_n - (int)plan.whole_tiles);
-      if (takes_wide(big) && takes_wide(half)) {
-        if (int rc1 = launch(big)) return rc1;
-        if (int rc2 = launch_status("marlin_tile_wide_kernel")) return rc2;
-        if (int rc1 = launch(half)) return rc1;
-        return launch_status("marlin_tile_wide_kernel (128-row tiles)");
-      }
+    if (plan.count == 2) {
+      if (int rc1 = launch(plan.launch[0])) return rc1;
+      if (int rc2 = launch_status("marlin_tile_wide_kernel")) return rc2;
+      if (int rc1 = launch(plan.launch[1])) return rc1;
+      return launch_status("marlin_tile_wide_kernel (128-row tiles)");
     }
+    p = plan.launch[0];
     rc = launch(p);
     if (rc) return rc;
     if (int rc2 = launch_status("marlin_tile_async_kernel")) return rc2;
@@ -2019,3 +2056,69 @@ int moe_tile_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
 }
 
 }  // namespace sonar
+
+// ---------------------------------------------------------------------------
+// Diagnostics for host-side tests (no counterpart in the reference): which tile and which K
+// steps every workgroup id of the tile kernels' launches works on, from the same planning and
+// mapping code the launches and the kernels run.  One row of six int32 per workgroup that has
+// work: launch, rows of a tile, row tile, column tile, first K step, end of its K steps.
+namespace {
+int64_t schedule_rows(const sonar::TileParams& p, const sonar::TileParams& mapped, int launch, int32_t* out,
+                      int64_t out_rows, int64_t at) {
+  using namespace sonar;
+  const int grid = tile_grid(p);
+  const int k_steps = p.size_k / kTileK;
+  for (int block = 0; block < grid; ++block) {
+    int tile, split, tile_m, tile_n;
+    bool whole_k;
+    if (!tile_of_block(mapped, block, tile, split, whole_k)) continue;
+    tile_coords(mapped, tile, tile_m, tile_n);
+    if (at < out_rows) {
+      int32_t* row = out + 6 * at;
+      row[0] = launch;
+      row[1] = mapped.tile_rows;
+      row[2] = tile_m;
+      row[3] = tile_n;
+      row[4] = whole_k ? 0 : split * mapped.k_steps_per_split;
+      row[5] = whole_k ? k_steps : std::min(k_steps, row[4] + mapped.k_steps_per_split);
+    }
+    ++at;
+  }
+  return at;
+}
+}  // namespace
+
+// A dense call (4-bit integer codes, no act-order) with room for every partial tile.
+extern "C" int64_t sonar_debug_tile_schedule(int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_groups,
+                                             int32_t* out, int64_t out_rows) {
+  using namespace sonar;
+  if (size_m <= 0 || size_n <= 0 || size_k <= 0 || size_k % kTileK != 0 || num_groups < 1 || size_k % num_groups != 0)
+    return -1;
+  const int group_size = (int)(size_k / num_groups);
+  static float4 never_read;
+  const TileLaunches plan =
+      plan_tile_launches(dense_tile_shape(size_m, size_n, size_k, num_groups, group_size), size_m, size_n, size_k,
+                         num_groups, group_size, &never_read, ~(size_t)0, false, false, 4, false);
+  int64_t at = 0;
+  for (int l = 0; l < plan.count; ++l) at = schedule_rows(plan.launch[l], plan.launch[l], l, out, out_rows, at);
+  return at;
+}
+
+// A grouped call whose routing made `row_tiles` row tiles of `tile_rows` rows, launched for up to
+// `max_row_tiles` of them; `with_partial`: the call has room for partial tiles.
+extern "C" int64_t sonar_debug_moe_tile_schedule(int64_t row_tiles, int64_t max_row_tiles, int64_t size_n,
+                                                 int64_t size_k, int tile_rows, int with_partial, int32_t* out,
+                                                 int64_t out_rows) {
+  using namespace sonar;
+  if (row_tiles < 0 || row_tiles > max_row_tiles || size_n <= 0 || size_k <= 0 || size_k % kTileK != 0 ||
+      (tile_rows != kTileM && tile_rows != 128))
+    return -1;
+  static float4 never_read;
+  static int32_t no_table;
+  TileParams p = dense_tile_shape(max_row_tiles * tile_rows, size_n, size_k, 1, (int)size_k);
+  p.tile_rows = tile_rows;
+  p.tiles_m = (int)max_row_tiles;
+  p.tile_table = &no_table;
+  if (with_partial && moe_tile_partial_bytes(size_k) > 0) p.partial = &never_read;
+  return schedule_rows(p, live_tiles_of(p, (int)row_tiles), 0, out, out_rows, 0);
+}
