@@ -380,7 +380,7 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
     matrix cores (4-bit expert weights repacked with is_a_8bit; input_global_scale1 / 2 are the
     factors marlin_act_int8_process_scales returns for the integer group scales).
     `activation_func(activation, out, in, **parameters)` and `moe_sum(moe_output [M, top_k, K],
-    output)` replace the built-in HIP kernels when given, as in the reference."""
+    output, topk_ids, expert_map)` replace the built-in HIP kernels when given, as in the reference."""
     _check_arguments(activation, input_dtype, (input_global_scale1, input_global_scale2, global_scale1,
                                                global_scale2))
     if quant_type_id not in _SUPPORTED:
@@ -430,8 +430,8 @@ def fused_marlin_moe(hidden_states: torch.Tensor, w1: torch.Tensor, w2: torch.Te
         inside = (ids >= 0) & (ids < global_num_experts)
         local = inside & (expert_map.to(torch.int64)[ids.clamp(0, global_num_experts - 1)] >= 0)
         moe_output = torch.where(local.unsqueeze(-1), moe_output, torch.zeros_like(moe_output))
-    if sum_rows is not None:
-        sum_rows(moe_output.contiguous(), output)
+    if sum_rows is not None:   # called as the reference calls it (marlin_moe.py:391)
+        sum_rows(moe_output.contiguous(), output, topk_ids, expert_map)
         return output
     return globals()["moe_sum"](moe_output.contiguous(), output)
 

@@ -588,6 +588,54 @@ def test_batched_fused_marlin_moe_against_per_token_reference(cfg):
         assert np.all(got[b, counts[b]:] == 7.0), "rows of invalid tokens must not be written"
 
 
+@pytest.mark.parametrize("zp", [False, True])
+def test_marlin_experts_classes_run_the_layer(zp):
+    """MarlinExperts / BatchedMarlinExperts (marlin_moe.py:707-1096) called the way the reference's
+    modular kernel calls them (workspaces of workspace_shapes(), output buffer given): the same
+    bits as fused_marlin_moe / batched_fused_marlin_moe on the same inputs."""
+    from sonar_amd import marlin_experts as me
+    from sonar_amd.fused_moe import batched_fused_marlin_moe, fused_marlin_moe
+    from sonar_amd.scalar_type import scalar_types
+    m, e, topk, hidden, inter, dtype = 37, 4, 2, 256, 128, "bf16"
+    (w1, s1, z1, _), (w2, s2, z2, _) = _moe_layer(61, e, hidden, inter, 128, dtype, zp)
+    quant = me.ExpertsQuantConfig(use_int4_w4a16=True, w1_scale=s1, w2_scale=s2, w1_zp=z1, w2_zp=z2)
+    experts = me.MarlinExperts(me.ExpertsMoeConfig(), quant)
+    assert experts.quant_type_id == (scalar_types.uint4.id if zp else scalar_types.uint4b8.id)
+    topk_ids, topk_w = _route(m, e, topk, m)
+    tw, ti = torch.from_numpy(topk_w).to(gu.DEV), torch.from_numpy(topk_ids).to(gu.DEV)
+    x = gu.dev_bits16(mo.round_to_dtype(0.5 * mo.make_activations(3, m, hidden, dtype), dtype), dtype)
+    E, M, N, K, k = experts.moe_problem_size(x, w1, w2, ti)
+    assert (E, M, N, K, k) == (e, m, inter, hidden, topk)
+    ws13, ws2, out_shape = experts.workspace_shapes(M, N, K, k, e, e, None, "silu")
+    buf13 = torch.empty(ws13, dtype=x.dtype, device=gu.DEV)
+    buf2 = torch.empty(ws2, dtype=x.dtype, device=gu.DEV)
+    out = torch.full(out_shape, 9.0, dtype=x.dtype, device=gu.DEV)
+    experts.apply(out, x, w1, w2, tw, ti, "silu", e, None, None, None, buf13, buf2, None, False)
+    want = fused_marlin_moe(x, w1, w2, None, None, s1, s2, tw, ti, experts.quant_type_id, w1_zeros=z1, w2_zeros=z2)
+    torch.cuda.synchronize()
+    assert torch.equal(out, want)
+
+    max_tokens, dispatchers = 20, 1
+    batched = me.BatchedMarlinExperts(me.ExpertsMoeConfig(), quant, max_tokens, dispatchers)
+    counts = torch.tensor([max_tokens, 3, 0, 11], dtype=torch.int32, device=gu.DEV)
+    xb = gu.dev_bits16(mo.round_to_dtype(0.5 * mo.make_activations(4, e * max_tokens, hidden, dtype), dtype),
+                       dtype).view(e, max_tokens, hidden)
+    ws13, ws2, out_shape = batched.workspace_shapes(max_tokens, inter, hidden, 1, e, e, None, "silu")
+    assert out_shape == (e, max_tokens, hidden)
+    buf13 = torch.empty(ws13, dtype=x.dtype, device=gu.DEV)
+    buf2 = torch.empty(ws2, dtype=x.dtype, device=gu.DEV)
+    outb = torch.full(out_shape, 9.0, dtype=x.dtype, device=gu.DEV)
+
+    class Meta:
+        expert_num_tokens = counts
+
+    batched.apply(outb, xb, w1, w2, None, None, "silu", e, None, None, None, buf13, buf2, Meta, False)
+    wantb = batched_fused_marlin_moe(xb, counts, w1, w2, None, None, s1, s2, batched.quant_type_id, w1_zeros=z1,
+                                     w2_zeros=z2, output=torch.full(out_shape, 9.0, dtype=x.dtype, device=gu.DEV))
+    torch.cuda.synchronize()
+    assert torch.equal(outb, wantb)
+
+
 def test_fused_marlin_moe_replays_in_a_hip_graph():
     """The layer reads no device value on the host, so it can be recorded; every
     replay must reproduce the eager result, also after the routing changed."""

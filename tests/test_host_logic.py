@@ -519,3 +519,47 @@ def test_mxfp4_host_helpers():
     assert mu.check_marlin_supported(st.float4_e2m1f, 32)
     assert not mu.check_marlin_supported(st.float4_e2m1f, 32, has_zp=True)
     assert f4.is_fp4_marlin_supported()
+
+
+def test_marlin_experts_configuration_logic():
+    """MarlinExpertsBase (marlin_moe.py:568-704): the weight type from the configuration flags,
+    the problem size from the packed tensors, the workspaces of both activation formats, the
+    activations it accepts."""
+    import torch
+    from sonar_amd import marlin_experts as me
+    from sonar_amd.scalar_type import scalar_types
+    moe = me.ExpertsMoeConfig()
+    ids = {
+        "use_int4_w4a16": scalar_types.uint4b8.id, "use_int8_w8a16": scalar_types.uint8b128.id,
+        "use_fp8_w8a16": scalar_types.float8_e4m3fn.id, "use_mxfp4_w4a16": scalar_types.float4_e2m1f.id,
+        "use_nvfp4_w4a16": scalar_types.float4_e2m1f.id,
+    }
+    for flag, want in ids.items():
+        assert me.MarlinExperts(moe, me.ExpertsQuantConfig(**{flag: True})).quant_type_id == want
+    zp = me.ExpertsQuantConfig(use_int4_w4a16=True, w1_zp=torch.zeros(1, dtype=torch.int32))
+    assert me.MarlinExperts(moe, zp).quant_type_id == scalar_types.uint4.id
+    with pytest.raises(AssertionError, match="Supports only"):
+        me.MarlinExperts(moe, me.ExpertsQuantConfig())
+    q = me.ExpertsQuantConfig(use_int4_w4a16=True, gemm1_clamp_limit=7.0, gemm1_alpha=1.702)
+    ex = me.MarlinExperts(moe, q)
+    assert (ex.gemm1_clamp_limit, ex.gemm1_alpha, ex.gemm1_beta) == (7.0, 1.702, 0.0)
+    # (E, K / 16, 2 * 2N) and (E, N / 16, 2K) packed tensors
+    e, k, n, m, topk = 8, 4096, 14336, 5, 2
+    w1 = torch.empty((e, k // 16, 4 * n), dtype=torch.int32, device="meta")
+    w2 = torch.empty((e, n // 16, 2 * k), dtype=torch.int32, device="meta")
+    a = torch.empty((m, k), dtype=torch.float16, device="meta")
+    ti = torch.empty((m, topk), dtype=torch.int32, device="meta")
+    assert ex.moe_problem_size(a, w1, w2, ti) == (e, m, n, k, topk)
+    assert ex.moe_problem_size(torch.empty((e, 9, k), device="meta"), w1, w2, ti) == (e, 9, n, k, topk)
+    # marlin_moe.py:741-744: swapped against fused_marlin_moe's intermediate caches
+    assert ex.workspace_shapes(m, n, k, topk, e, e, None, "silu") == \
+        ((m * topk, max(n, k)), (m * topk * max(2 * n, k),), (m, k))
+    b = me.BatchedMarlinExperts(moe, q, max_num_tokens=32, num_dispatchers=2)
+    assert b.workspace_shapes(m, n, k, topk, e, e, None, "silu") == \
+        ((e * 64, max(k, 2 * n)), (e * 64, n), (e, 64, k))
+    assert ex.activation_format() == "standard" and b.activation_format() == "batched_experts"
+    for name in ("silu", "gelu", "gelu_tanh", "situ", "swigluoai", "swigluoai_uninterleave", "swiglustep",
+                 "silu_no_mul", "gelu_no_mul", "gelu_tanh_no_mul", "relu2_no_mul"):
+        assert ex._supports_activation(name), name
+    assert not ex._supports_activation("relu")
+    assert ex._supports_no_act_and_mul()
