@@ -1631,14 +1631,16 @@ bool moe_fast_applies(bool has_perm, int64_t moe_block_size, int64_t sorted_len,
   if (shift <= -2 && moe_block_size > 16) return false;   // groups of 32 / 64 rows: one block of 16 rows only
   if (moe_block_size < 64) return true;
   // 64-slot blocks also have the tile kernel, which wins once the experts have
-  // rows enough to fill its 256-row tiles.  Measured on Mixtral shapes (8
-  // experts, top 2): 1016 slots (256 tokens): 285 / 128 us here against 459 /
-  // 349 in the tile kernel (gate_up / down); 1528 slots: 559 / 237 against 493 /
-  // 355; 2552 slots: 977 / 406 against 753 / 369.  The tile kernel launches at
-  // least experts x N / 256 workgroups; where that is under one per compute
-  // unit (down) it stays behind for longer.
+  // rows enough for its tiles.  Measured on Mixtral shapes (8 experts, top 2;
+  // gate_up / down, this kernel against the tile kernel with its 128-row tiles
+  // and its K split): 888 slots (192 tokens): 250 / 103 us against 271 / 137;
+  // 952 slots: 265 / 122 against 267 / 134; 1016 slots (256 tokens): 305 / 123
+  // against 272 / 132; 1144 slots: down 150 against 137; 1272 slots: down 178
+  // against 141.  The tile kernel launches at least experts x N / 256
+  // workgroups; where that is under one per compute unit (down) it stays
+  // behind a little longer.
   const int64_t tile_workgroups = num_experts * ((size_n + 255) / 256);
-  return sorted_len <= (tile_workgroups < cu_count() ? 1600 : 1100);
+  return sorted_len <= (tile_workgroups < cu_count() ? 1100 : 1000);
 }
 
 // Called by sonar_moe_wna16_marlin_gemm when moe_fast_applies: one workgroup
