@@ -82,11 +82,13 @@ inline size_t plan_partial_bytes(const GemmPlan& plan, int64_t size_m, int64_t s
 
 // The 128-row form pays when 256-row tiles would leave more than half of the compute units to
 // K ranges of the same tile: twice the tiles, half the ranges, half the partial-tile bytes.  With
-// a long K the partial tiles are a small part of the work and the larger tile stays ahead
-// (measured: K = 14336, M = 1024, N = 4096: 108 us against 119).
+// a long K the partial tiles are a smaller part of the work and the larger tile is ahead again
+// from 48 tiles on (measured at K = 14336, N = 4096, 128-row against 256-row tiles: M = 256:
+// 44.4 against 50.9 us; 384: 62.0 against 75.4; 512: 72.7 against 74.6; 768: 109 against 101;
+// 1024: 126 against 120).
 inline bool plan_prefers_128_rows(int64_t size_m, int64_t size_n, int64_t size_k, bool rows_97_128 = false) {
   const int64_t tiles256 = ((size_m + 255) / 256) * ((size_n + 255) / 256);
-  return (size_m > 128 || rows_97_128) && tiles256 <= 128 && size_k <= 8192;
+  return (size_m > 128 || rows_97_128) && tiles256 <= (size_k <= 8192 ? 128 : 32);
 }
 
 // Scratch for the partial tiles of either tiling.
