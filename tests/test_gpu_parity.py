@@ -123,6 +123,10 @@ GEMM_CASES = [
     (33, 14336, 1024, 128, False, False, True),
     (64, 2048, 512, 128, True, False, False),
     (40, 4096, 640, -1, False, False, False),
+    # 65..128 rows on a long K: 128-row tiles of the wide tile kernel, K in ranges
+    (72, 8192, 1280, 128, True, False, False),
+    (128, 14336, 768, 128, False, False, True),
+    (65, 11008, 512, -1, False, False, False),
     # 33..64 rows on more strips than half the compute units: two workgroups of two blocks of rows per strip
     (40, 1024, 8320, 128, True, False, True),
     (64, 512, 16384, -1, False, False, False),
