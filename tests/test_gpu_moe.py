@@ -109,6 +109,9 @@ MOE_CASES = [
     (900, 3, 2, 2048, 256, 128, "bf16", True, False, True, 64, False),
     (640, 5, 2, 1280, 192, 64, "bf16", False, False, True, 64, True),
     (650, 2, 2, 1024, 256, 128, "fp16", False, True, False, 64, True),
+    # fp16 with zero points on 64-slot blocks: 256- and 128-row tiles, without and with the K split
+    (600, 4, 2, 512, 256, 128, "fp16", True, False, True, 64, True),
+    (500, 3, 2, 1024, 320, 64, "fp16", True, False, False, 64, False),
     # more tiles than compute units with a short last round (9 row tiles x 33 = 297) and K of 48 steps
     (1100, 3, 2, 3072, 8448, 128, "bf16", False, False, True, 64, True),
 ]
@@ -262,7 +265,9 @@ def test_moe_matches_dense_gemm_per_expert():
     # 8-bit codes: blocks of 64 slots run the tile kernel's 8-bit form, smaller ones the general grouped kernel
     (700, 4096, 2048, "uint8b128"), (2048, 2048, 1024, "fp8"), (64, 2048, 1024, "uint8b128"),
     # MXFP4 in the tile kernel with few tiles, and with a short last round of them (384 = 256 + 128): both cut along K
-    (700, 4096, 2048, "mxfp4"), (2100, 14336, 4096, "mxfp4")])
+    (700, 4096, 2048, "mxfp4"), (2100, 14336, 4096, "mxfp4"),
+    # the fp16 instantiations of the grouped tile kernel's 8-bit and 4-bit forms (256- and 128-row tiles)
+    (700, 2048, 1024, "uint8b128/fp16"), (700, 2048, 1024, "fp8/fp16"), (700, 2048, 1024, "uint4b8/fp16")])
 def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     """Mixtral-8x7B expert shapes (8 experts, top 2, the block size of the
     reference's rule), where the CPU oracle is too slow: every routed slot must
@@ -272,6 +277,9 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     of 8, 32 and 64 slots, i.e. the grouped decode kernel with one and two
     blocks of rows, its two-halves form and the tile kernel."""
     e, top_k, dtype = 8, 2, torch.bfloat16
+    if wtype.endswith("/fp16"):
+        wtype, dtype = wtype[:-5], torch.float16
+    dtype_code = _lib.DTYPE_BF16 if dtype == torch.bfloat16 else _lib.DTYPE_F16
     gen = torch.Generator(device=gu.DEV).manual_seed(tokens + n)
     lib = _lib.load()
     b_type = {"uint4b8": _lib.TYPE_UINT4B8, "uint8b128": _lib.TYPE_UINT8B128, "fp8": _lib.TYPE_FLOAT8_E4M3FN,
@@ -284,8 +292,8 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
         scales = torch.exp2(torch.randint(-9, -5, (e, groups, n), device=gu.DEV, generator=gen).float())
     if wtype == "uint8b128":
         scales = scales / 16
-    if wtype == "fp8":   # the exponent bias of the codes is folded into the scales: 2^120 for bf16
-        scales = scales * 2.0 ** 120
+    if wtype == "fp8":   # the exponent bias of the codes is folded into the scales: 2^120 for bf16, 2^8 for fp16
+        scales = scales * (2.0 ** 120 if dtype == torch.bfloat16 else 2.0 ** 8)
     scales = scales.to(dtype)
     a = torch.randn((tokens, k), device=gu.DEV, generator=gen).to(dtype)
     topk_ids, topk_w = route(tokens, tokens, e, top_k)
@@ -300,7 +308,7 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     _lib.check(lib.sonar_moe_wna16_marlin_gemm(
         gu.ptr(a), gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None, gu.ptr(scales), None, None, None,
         gu.ptr(workspace), workspace.numel(), gu.ptr(scr), nbytes, gu.ptr(sid), sid.numel(), gu.ptr(eid),
-        gu.ptr(npp), None, bs, top_k, 0, e, _lib.DTYPE_BF16, b_type, tokens, n, k, groups, 1, 0, 1,
+        gu.ptr(npp), None, bs, top_k, 0, e, dtype_code, b_type, tokens, n, k, groups, 1, 0, 1,
         gu.stream()))
     torch.cuda.synchronize()
     assert bool(torch.isfinite(c.float()).all())
@@ -316,7 +324,7 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
         dscr = torch.empty(max(lib.sonar_marlin_gemm_scratch_bytes(m, n, k), 16), dtype=torch.uint8, device=gu.DEV)
         _lib.check(lib.sonar_marlin_gemm(
             gu.ptr(rows), k, gu.ptr(dense), gu.ptr(native[ex]), _lib.LAYOUT_GFX950, None, gu.ptr(scales[ex]), None,
-            None, None, gu.ptr(workspace), workspace.numel(), gu.ptr(dscr), dscr.numel(), _lib.DTYPE_BF16,
+            None, None, gu.ptr(workspace), workspace.numel(), gu.ptr(dscr), dscr.numel(), dtype_code,
             b_type, m, n, k, groups, 1, 0, 1, gu.stream()))
         got = c[torch.from_numpy(slots).to(gu.DEV)].float()
         err = float((got - dense.float()).abs().max())
