@@ -109,6 +109,10 @@ MOE_CASES = [
     (900, 3, 2, 2048, 256, 128, "bf16", True, False, True, 64, False),
     (640, 5, 2, 1280, 192, 64, "bf16", False, False, True, 64, True),
     (650, 2, 2, 1024, 256, 128, "fp16", False, True, False, 64, True),
+    # groups of 32 rows in the grouped tile kernel: the other activation type, with and without zero points
+    (700, 2, 2, 256, 512, 32, "bf16", False, False, False, 64, True),
+    (700, 2, 2, 256, 512, 32, "fp16", False, False, True, 64, False),
+    (700, 2, 2, 512, 256, 32, "bf16", True, False, False, 64, True),
     # fp16 with zero points on 64-slot blocks: 256- and 128-row tiles, without and with the K split
     (600, 4, 2, 512, 256, 128, "fp16", True, False, True, 64, True),
     (500, 3, 2, 1024, 320, 64, "fp16", True, False, False, 64, False),
@@ -267,7 +271,9 @@ def test_moe_matches_dense_gemm_per_expert():
     # MXFP4 in the tile kernel with few tiles, and with a short last round of them (384 = 256 + 128): both cut along K
     (700, 4096, 2048, "mxfp4"), (2100, 14336, 4096, "mxfp4"),
     # the fp16 instantiations of the grouped tile kernel's 8-bit and 4-bit forms (256- and 128-row tiles)
-    (700, 2048, 1024, "uint8b128/fp16"), (700, 2048, 1024, "fp8/fp16"), (700, 2048, 1024, "uint4b8/fp16")])
+    (700, 2048, 1024, "uint8b128/fp16"), (700, 2048, 1024, "fp8/fp16"), (700, 2048, 1024, "uint4b8/fp16"),
+    # 8-bit codes with a scale per 32 rows (the layout of MXFP8), either activation type
+    (700, 2048, 1024, "uint8b128g32"), (700, 2048, 1024, "uint8b128g32/fp16"), (700, 2048, 1024, "fp8g32/fp16")])
 def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     """Mixtral-8x7B expert shapes (8 experts, top 2, the block size of the
     reference's rule), where the CPU oracle is too slow: every routed slot must
@@ -280,12 +286,15 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     if wtype.endswith("/fp16"):
         wtype, dtype = wtype[:-5], torch.float16
     dtype_code = _lib.DTYPE_BF16 if dtype == torch.bfloat16 else _lib.DTYPE_F16
+    group = 128
+    if wtype.endswith("g32"):
+        wtype, group = wtype[:-3], 32
     gen = torch.Generator(device=gu.DEV).manual_seed(tokens + n)
     lib = _lib.load()
     b_type = {"uint4b8": _lib.TYPE_UINT4B8, "uint8b128": _lib.TYPE_UINT8B128, "fp8": _lib.TYPE_FLOAT8_E4M3FN,
               "mxfp4": _lib.TYPE_FLOAT4_E2M1F}[wtype]
     words = k * n // (8 if wtype in ("uint4b8", "mxfp4") else 4)
-    groups = k // (32 if wtype == "mxfp4" else 128)
+    groups = k // (32 if wtype == "mxfp4" else group)
     native = torch.randint(-2 ** 31, 2 ** 31 - 1, (e, words), dtype=torch.int32, device=gu.DEV, generator=gen)
     scales = torch.rand((e, groups, n), device=gu.DEV, generator=gen) * 9e-3 + 1e-3
     if wtype == "mxfp4":   # powers of two
