@@ -748,8 +748,22 @@ A8Plan plan_a8(int64_t size_m, int64_t size_n, int64_t size_k, int64_t num_group
 template <typename ACT, typename T, int MB, bool HAS_ZP>
 void launch_a8_mb(const A8Params& p, bool grouped, dim3 grid, hipStream_t st) {
   constexpr int threads = 64 * A8Waves<MB>::value;
-  if (grouped) marlin_a8_kernel<ACT, T, MB, HAS_ZP, true><<<grid, threads, 0, st>>>(p);
-  else marlin_a8_kernel<ACT, T, MB, HAS_ZP, false><<<grid, threads, 0, st>>>(p);
+  if constexpr (ACT::kE8Scales) {   // float4 codes: always groups of 32 rows, never zero points
+    static_assert(!HAS_ZP, "float4_e2m1f weights have no zero points");
+    marlin_a8_kernel<ACT, T, MB, false, true><<<grid, threads, 0, st>>>(p);
+  } else {
+    if (grouped) marlin_a8_kernel<ACT, T, MB, HAS_ZP, true><<<grid, threads, 0, st>>>(p);
+    else marlin_a8_kernel<ACT, T, MB, HAS_ZP, false><<<grid, threads, 0, st>>>(p);
+  }
+}
+
+// The sum of the K ranges of a split call.
+template <typename ACT, typename T>
+void launch_a8_finish(const A8Params& p, bool grouped, hipStream_t st) {
+  long blocks = ((long)p.m * p.n + 255) / 256;
+  if (blocks > 4096) blocks = 4096;
+  if (grouped || ACT::kE8Scales) marlin_a8_finish_kernel<ACT, T, true><<<(int)blocks, 256, 0, st>>>(p);
+  else if constexpr (!ACT::kE8Scales) marlin_a8_finish_kernel<ACT, T, false><<<(int)blocks, 256, 0, st>>>(p);
 }
 
 template <typename ACT, typename T, bool HAS_ZP, bool MOE>
@@ -770,19 +784,19 @@ void launch_a8(const A8Params& p, const A8Plan& plan, bool grouped, hipStream_t 
     q.g = p;
     if (zp) launch_a8_tile_gc<ACT, T, true, false>(q, plan.unit_chunks, grid, st);
     else launch_a8_tile_gc<ACT, T, false, false>(q, plan.unit_chunks, grid, st);
-    if (plan.splits > 1) {
-      long blocks = ((long)p.m * p.n + 255) / 256;
-      if (blocks > 4096) blocks = 4096;
-      if (grouped) marlin_a8_finish_kernel<ACT, T, true><<<(int)blocks, 256, 0, st>>>(p);
-      else marlin_a8_finish_kernel<ACT, T, false><<<(int)blocks, 256, 0, st>>>(p);
-    }
+    if (plan.splits > 1) launch_a8_finish<ACT, T>(p, grouped, st);
     return;
   }
   const dim3 grid(p.n / kStripN, plan.slabs, plan.splits);
-#define SONAR_A8_CASE(MB)                                             \
-  case MB:                                                            \
-    if (zp) launch_a8_mb<ACT, T, MB, true>(p, grouped, grid, st);     \
-    else launch_a8_mb<ACT, T, MB, false>(p, grouped, grid, st);       \
+#define SONAR_A8_CASE(MB)                                                          \
+  case MB:                                                                         \
+    if constexpr (!ACT::kE8Scales) {                                               \
+      if (zp) {                                                                    \
+        launch_a8_mb<ACT, T, MB, true>(p, grouped, grid, st);                      \
+        break;                                                                     \
+      }                                                                            \
+    }                                                                              \
+    launch_a8_mb<ACT, T, MB, false>(p, grouped, grid, st);                         \
     break;
   switch (plan.mb) {
     SONAR_A8_CASE(1)
@@ -791,17 +805,14 @@ void launch_a8(const A8Params& p, const A8Plan& plan, bool grouped, hipStream_t 
     SONAR_A8_CASE(4)
   }
 #undef SONAR_A8_CASE
-  if (plan.splits > 1) {
-    long blocks = ((long)p.m * p.n + 255) / 256;
-    if (blocks > 4096) blocks = 4096;
-    if (grouped) marlin_a8_finish_kernel<ACT, T, true><<<(int)blocks, 256, 0, st>>>(p);
-    else marlin_a8_finish_kernel<ACT, T, false><<<(int)blocks, 256, 0, st>>>(p);
-  }
+  if (plan.splits > 1) launch_a8_finish<ACT, T>(p, grouped, st);
 }
 
 template <typename ACT, typename T, int MB>
 void launch_moe_a8_mb(const MoeA8Params& q, bool grouped, bool zp, dim3 grid, hipStream_t st) {
-  if (grouped) {
+  if constexpr (ACT::kE8Scales) {   // float4 codes: always groups of 32 rows, never zero points
+    marlin_moe_a8_kernel<ACT, T, MB, false, true><<<grid, 256, 0, st>>>(q);
+  } else if (grouped) {
     if (zp) marlin_moe_a8_kernel<ACT, T, MB, true, true><<<grid, 256, 0, st>>>(q);
     else marlin_moe_a8_kernel<ACT, T, MB, false, true><<<grid, 256, 0, st>>>(q);
   } else {
@@ -850,6 +861,10 @@ int check_a8(int a_dtype, int dtype, int b_layout, int64_t b_type_id, int64_t si
                   "one exponent-byte scale per 32 rows; got size_k = %ld, num_groups = %ld", (long)size_k,
                   (long)num_groups);
     SONAR_REQUIRE(b_zeros == nullptr, "float4_e2m1f weights have no zero points");
+    // generate_kernels.py:152-161: c_type kBFloat16 only
+    if (dtype != SONAR_DTYPE_BF16)
+      return fail(SONAR_E_UNSUPPORTED, "float4_e2m1f weights with float8_e4m3fn activations (MXFP4) are built for "
+                  "bfloat16 outputs only");
   }
   SONAR_REQUIRE(size_m >= 0 && size_n > 0 && size_k > 0, "size_m = %ld, size_n = %ld, size_k = %ld", (long)size_m,
                 (long)size_n, (long)size_k);
@@ -928,8 +943,7 @@ extern "C" int sonar_moe_wna16_marlin_gemm_a8(
   const bool grouped = a8_grouped(b_type_id, num_groups);
   hipStream_t st = (hipStream_t)stream;
   if (b_type_id == SONAR_TYPE_FLOAT4_E2M1F) {
-    if (dtype == SONAR_DTYPE_F16) launch_moe_a8<ActFp8F4, _Float16>(q, grouped, (int)blocks, st);
-    else launch_moe_a8<ActFp8F4, __bf16>(q, grouped, (int)blocks, st);
+    launch_moe_a8<ActFp8F4, __bf16>(q, grouped, (int)blocks, st);   // bfloat16 outputs only (check_a8)
   } else if (a_dtype == SONAR_ADTYPE_INT8) {
     if (dtype == SONAR_DTYPE_F16) launch_moe_a8<ActInt8, _Float16>(q, grouped, (int)blocks, st);
     else launch_moe_a8<ActInt8, __bf16>(q, grouped, (int)blocks, st);
@@ -984,8 +998,7 @@ extern "C" int sonar_marlin_gemm_a8(const void* a, int64_t a_row_stride, int a_d
   const bool grouped = a8_grouped(b_type_id, num_groups);
   hipStream_t st = (hipStream_t)stream;
   if (b_type_id == SONAR_TYPE_FLOAT4_E2M1F) {
-    if (dtype == SONAR_DTYPE_F16) launch_a8<ActFp8F4, _Float16>(p, plan, grouped, st);
-    else launch_a8<ActFp8F4, __bf16>(p, plan, grouped, st);
+    launch_a8<ActFp8F4, __bf16>(p, plan, grouped, st);   // bfloat16 outputs only (check_a8)
   } else if (a_dtype == SONAR_ADTYPE_INT8) {
     if (dtype == SONAR_DTYPE_F16) launch_a8<ActInt8, _Float16>(p, plan, grouped, st);
     else launch_a8<ActInt8, __bf16>(p, plan, grouped, st);

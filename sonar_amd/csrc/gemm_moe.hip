@@ -470,8 +470,8 @@ void launch_moe(const MoeParams& p, bool has_perm, int grid, hipStream_t st) {
     if constexpr (!HAS_ZP) marlin_moe_kernel<T, MB, false, true, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
   } else if (p.g_idx) {   // rows already permuted into a copy of A, groups still looked up per row
     if constexpr (!HAS_ZP) marlin_moe_kernel<T, MB, false, false, true><<<grid, kMoeWaves * 64, 0, st>>>(p);
-  } else if (has_perm) {
-    marlin_moe_kernel<T, MB, HAS_ZP, true, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
+  } else if (has_perm) {   // symmetric weights only (checked by the entry point)
+    if constexpr (!HAS_ZP) marlin_moe_kernel<T, MB, false, true, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
   } else {
     marlin_moe_kernel<T, MB, HAS_ZP, false, false><<<grid, kMoeWaves * 64, 0, st>>>(p);
   }
@@ -581,6 +581,11 @@ int moe_gemm_any(
                   "b_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   bool has_perm = perm != nullptr;
+  // moe/marlin_moe_wna16/generate_kernels.py:66-72: uint4 weights with zero points come without the act-order form
+  // (group_blocks 0), and the op then finds no kernel
+  if (has_zp && has_perm)
+    return fail(SONAR_E_UNSUPPORTED, "Unsupported shapes: has_act_order = 1 with zero points (b_type uint4): "
+                "act-order is built for uint4b8 and uint8b128 weights only");
   if (nvfp4) {
     // moe/marlin_moe_wna16/generate_kernels.py:94-101: NVFP4, either activation type, a scale per 16 rows
     SONAR_REQUIRE(fp4, "a global scale goes with float4_e2m1f weights only (NVFP4)");
@@ -609,8 +614,6 @@ int moe_gemm_any(
   const bool row_groups = has_perm && !is_k_full;
   if (has_perm) {
     SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
-    if (row_groups && has_zp)
-      return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False and zero points is not built");
   }
   int group_size = (int)size_k;
   if (row_groups) {

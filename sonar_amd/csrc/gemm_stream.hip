@@ -1390,8 +1390,8 @@ template <typename T, int MB, bool HAS_ZP>
 void launch_stream(const StreamParams& p, bool has_perm, hipStream_t st) {
   if (p.g_idx) {  // row -> group lookup: symmetric weights, activations already permuted
     if constexpr (!HAS_ZP) marlin_stream_kernel<T, MB, false, false, true><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p);
-  } else if (has_perm) {
-    marlin_stream_kernel<T, MB, HAS_ZP, true, false><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p);
+  } else if (has_perm) {   // symmetric weights only (check_common)
+    if constexpr (!HAS_ZP) marlin_stream_kernel<T, MB, false, true, false><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p);
   } else {
     marlin_stream_kernel<T, MB, HAS_ZP, false, false><<<p.grid_parts * p.slabs, kWaves * 64, 0, st>>>(p);
   }
@@ -1551,6 +1551,11 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
                   "b_type must be uint4b8, uint8b128 or float8_e4m3fn when has_zp = False (uint4 needs b_zeros)");
   SONAR_REQUIRE((g_idx == nullptr) == (perm == nullptr), "g_idx and perm must be given together");
   out.has_perm = perm != nullptr;
+  // generate_kernels.py:66-72: uint4 weights with zero points come without the act-order form
+  // (group_blocks 0), and marlin.cu:509-519 then finds no kernel
+  if (out.has_zp && out.has_perm)
+    return fail(SONAR_E_UNSUPPORTED, "Unsupported shapes: has_act_order = 1 with zero points (b_type uint4): "
+                "act-order is built for uint4b8 and uint8b128 weights only");
   if (out.nvfp4) {
     // generate_kernels.py:94-101: NVFP4, either activation type, one scale per 16 rows
     SONAR_REQUIRE(!out.has_perm, "act-order is not supported with float4_e2m1f weights");
@@ -1583,8 +1588,6 @@ int check_common(Checked& out, int b_layout, const void* b_scales, const uint32_
   if (out.has_perm) SONAR_REQUIRE(num_groups > 1, "For act_order, num_groups must be > 1");
   if (out.row_groups) {
     // marlin.cu:343-351,763-769: group_size = 0, every row looks its group up
-    if (out.has_zp)
-      return fail(SONAR_E_UNSUPPORTED, "act-order with is_k_full = False and zero points is not built");
     out.group_size = 0;
   } else if (num_groups > 1) {
     SONAR_REQUIRE(size_k % num_groups == 0, "size_k = %ld, is not divisible by num_groups = %ld",

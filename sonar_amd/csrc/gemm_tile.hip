@@ -1897,11 +1897,12 @@ int tile_gemm(const void* a, int64_t a_row_stride, void* c, const uint32_t* b, c
     return SONAR_OK;
   }
   if (bits == 8) return fail(SONAR_E_INVALID, "internal: 8-bit codes exist in the asynchronous tile kernel only");
+  if (zp && pm) return fail(SONAR_E_INVALID, "internal: act-order with zero points");   // refused by the entry point
   if (dtype == SONAR_DTYPE_F16) {
-    rc = zp ? (pm ? launch_tile<_Float16, true, true>(p, st) : launch_tile<_Float16, true, false>(p, st))
+    rc = zp ? launch_tile<_Float16, true, false>(p, st)
             : (pm ? launch_tile<_Float16, false, true>(p, st) : launch_tile<_Float16, false, false>(p, st));
   } else {
-    rc = zp ? (pm ? launch_tile<__bf16, true, true>(p, st) : launch_tile<__bf16, true, false>(p, st))
+    rc = zp ? launch_tile<__bf16, true, false>(p, st)
             : (pm ? launch_tile<__bf16, false, true>(p, st) : launch_tile<__bf16, false, false>(p, st));
   }
   if (rc) return rc;
