@@ -23,6 +23,7 @@ DENSE = [
     (33, 14336, 1024, 128, "bf16", False, True),
     (200, 512, 4096, 128, "fp16", False, False),
     (300, 1024, 768, 128, "bf16", False, True),
+    (300, 1024, 768, 128, "fp16", False, False),
     (600, 1024, 768, 64, "fp16", True, False),
     (1100, 512, 1024, -1, "bf16", False, False),
     (2100, 512, 4096, 128, "bf16", True, True),     # 144 tiles of 256 rows: the wide tile kernel's 256-row form
@@ -94,6 +95,10 @@ def grouped() -> None:
                  (50, 4, 2, 512, 128, 128, "bf16", False, True, False, 16, True)]:     # act-order
         print("grouped", case, flush=True)
         tm.test_moe_gemm_within_tolerance(case)   # raises on a mismatch
+    # NVFP4 experts on 64-slot blocks: the tile kernels, or the general grouped kernel when they are switched off
+    from tests import test_gpu_ops as to
+    to.test_prepare_nvfp4_moe_layer_and_fused_marlin_moe((1500, 4, 2, 256, 128), "fp16")
+    print("grouped nvfp4 ok", flush=True)
 
 
 if __name__ == "__main__":

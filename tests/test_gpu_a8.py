@@ -156,6 +156,12 @@ INT8_CASES = [
     (8192, 128, 128, False, "fp16", False, [128]),      # K split over workgroups
     (8192, 128, -1, False, "bf16", True, [70]),
     (1024, 256, 32, False, "fp16", False, [100]),       # groups of 32: the slab kernel
+    # 33..48 rows on a matrix the tiled kernel does not take (N = 192): three blocks of 16 rows
+    (512, 192, -1, False, "fp16", False, [40]),
+    (512, 192, 64, False, "fp16", True, [40]),
+    (512, 192, -1, True, "fp16", False, [40]),
+    (512, 192, 32, True, "fp16", True, [40]),
+    (8192, 128, -1, False, "fp16", True, [9]),          # channelwise, K split
 ]
 
 
@@ -188,6 +194,13 @@ FP8_CASES = [
     (1024, 128, -1, True, "bf16", False, [100]),
     (512, 256, 64, True, "bf16", False, [257]),
     (8192, 128, 128, False, "fp16", False, [128]),
+    # 33..48 rows on a matrix the tiled kernel does not take (N = 192): three blocks of 16 rows
+    (512, 192, -1, False, "fp16", False, [40]),
+    (512, 192, 64, False, "fp16", True, [40]),
+    (512, 192, -1, True, "fp16", False, [40]),
+    # channelwise, K split over workgroups
+    (8192, 128, -1, False, "fp16", True, [9]),
+    (8192, 128, -1, False, "bf16", False, [9]),
 ]
 
 
@@ -208,12 +221,12 @@ def test_w4a8_fp8_gemm_within_tolerance(k, n, group, zp, dtype, bias, ms):
 
 
 FP4_CASES = [
-    # k, n, dtype, bias, M list
+    # k, n, dtype, bias, M list   (bfloat16 outputs only: generate_kernels.py:152-161)
     (256, 128, "bf16", False, [1, 16]),
-    (512, 192, "fp16", True, [7, 33]),
+    (512, 192, "bf16", True, [7, 20, 33]),
     (1024, 256, "bf16", True, [64, 100]),
     (8192, 64, "bf16", False, [3]),
-    (1024, 256, "fp16", False, [257]),
+    (1024, 256, "bf16", False, [257]),
 ]
 
 
@@ -252,14 +265,15 @@ def test_w4a8_fp4_gemm_within_tolerance(k, n, dtype, bias, ms):
     a = torch.zeros((4, k), dtype=torch.int8, device=DEV)
     c = torch.empty((4, n), dtype=tdt, device=DEV)
 
-    def call(adt=_lib.ADTYPE_FP8, zeros=None, groups=k // 32):
+    def call(adt=_lib.ADTYPE_FP8, zeros=None, groups=k // 32, out=dtype_code(dtype)):
         return lib.sonar_marlin_gemm_a8(ptr(a), k, adt, ptr(c), ptr(native), _lib.LAYOUT_GFX950, None, ptr(dev_s),
-                                        ptr(s_dev), ptr(zeros), None, 0, dtype_code(dtype), _lib.TYPE_FLOAT4_E2M1F,
+                                        ptr(s_dev), ptr(zeros), None, 0, out, _lib.TYPE_FLOAT4_E2M1F,
                                         4, n, k, groups, stream())
 
     assert call(adt=_lib.ADTYPE_INT8) == _lib.E_UNSUPPORTED
     assert call(zeros=dev_s) == _lib.E_INVALID
     assert call(groups=k // 64) == _lib.E_INVALID
+    assert call(out=_lib.DTYPE_F16) == _lib.E_UNSUPPORTED      # no float16 outputs
 
 
 def test_w4a8_rejections():
@@ -300,6 +314,14 @@ MOE_A8_CASES = [
     (150, 512, 256, 3, 2, 64, -1, False, "bf16", False, False),
     (90, 512, 256, 5, 3, 48, 64, True, "fp16", False, True),
     (200, 256, 512, 6, 1, 64, 128, True, "bf16", True, False),
+    (200, 512, 256, 4, 2, 64, -1, True, "bf16", False, True),      # ... channelwise with zero points
+    (200, 512, 256, 4, 2, 64, 64, True, "bf16", True, False),      # ... groups of 64 rows
+    (200, 512, 256, 4, 2, 64, 128, False, "bf16", False, True),    # ... groups of 128 rows
+] + [
+    # one scale per column on a matrix the tiled kernel does not take (N = 128): the general grouped kernel
+    # with one to four blocks of 16 rows, either output type, with and without zero points
+    (2 * block, 256, 128, 3, 2, block, -1, zp, dtype, block == 32, block != 48)
+    for dtype in ("fp16", "bf16") for block in (16, 32, 48, 64) for zp in (False, True)
 ]
 
 

@@ -118,6 +118,35 @@ MOE_CASES = [
     (500, 3, 2, 1024, 320, 64, "fp16", True, False, False, 64, False),
     # more tiles than compute units with a short last round (9 row tiles x 33 = 297) and K of 48 steps
     (1100, 3, 2, 3072, 8448, 128, "bf16", False, False, True, 64, True),
+    # blocks of 16 slots on more (block, strip) pairs than compute units: the decode kernel's workgroups of
+    # four wavefronts, with one, two and four groups per 128 rows, both activation types, with and without
+    # zero points
+    (200, 4, 2, 256, 1024, 128, "fp16", False, False, False, 16, True),
+    (200, 4, 2, 256, 1024, 128, "fp16", True, False, True, 16, False),
+    (200, 4, 2, 256, 1024, 128, "bf16", True, False, False, 16, True),
+    (200, 4, 2, 256, 1024, 64, "fp16", False, False, True, 16, True),
+    (200, 4, 2, 256, 1024, 64, "fp16", True, False, False, 16, True),
+    (200, 4, 2, 256, 1024, 64, "bf16", False, False, False, 16, False),
+    (200, 4, 2, 256, 1024, 64, "bf16", True, False, True, 16, True),
+    (200, 4, 2, 256, 1024, 32, "fp16", False, False, False, 16, True),
+    (200, 4, 2, 256, 1024, 32, "fp16", True, False, True, 16, True),
+    (200, 4, 2, 256, 1024, 32, "bf16", False, False, True, 16, False),
+    (200, 4, 2, 256, 1024, 32, "bf16", True, False, False, 16, True),
+    # ... blocks of 32 slots (two blocks of rows per workgroup) with zero points, and eight wavefronts on two groups
+    (200, 4, 2, 256, 1024, 128, "bf16", True, False, False, 32, True),
+    (10, 4, 2, 256, 256, 64, "bf16", True, False, True, 16, True),
+    # 64-slot blocks, more slots than the decode kernel takes, K of 10 steps (not a whole number of the wide
+    # kernel's passes of four): the eight-wavefront grouped tile kernel, with groups of 128, 64 and 32 rows
+    (700, 2, 2, 640, 256, 128, "fp16", False, False, True, 64, True),
+    (700, 2, 2, 640, 256, 64, "fp16", True, False, False, 64, False),
+    (700, 2, 2, 640, 256, 32, "bf16", False, False, False, 64, True),
+    (700, 2, 2, 640, 256, 32, "bf16", True, False, True, 64, True),
+    (700, 2, 2, 640, 256, 32, "fp16", False, False, True, 64, False),
+    (700, 2, 2, 640, 256, 32, "fp16", True, False, False, 64, True),
+    # K = 192 is not a whole number of the decode kernel's 128-row units: the general grouped kernel
+    (9, 4, 2, 192, 128, 64, "fp16", True, False, False, 16, True),
+    # act-order on blocks of 48 slots: the gathering kernel with three blocks of rows, then the permuted copy
+    (100, 3, 2, 512, 128, 128, "fp16", False, True, False, 48, True),
 ]
 
 
@@ -174,13 +203,17 @@ def test_random_moe_cases_against_oracle(case):
     test_moe_gemm_within_tolerance(case)
 
 
-@pytest.mark.parametrize("cfg", [(9, 4, 2, 16, "fp16", True), (70, 3, 2, 32, "bf16", False), (200, 2, 1, 64, "fp16", True)],
+@pytest.mark.parametrize("copy", [False, True], ids=["gather", "permuted_copy"])
+@pytest.mark.parametrize("cfg", [(9, 4, 2, 16, "fp16", True), (70, 3, 2, 32, "bf16", False), (200, 2, 1, 64, "fp16", True),
+                                 (9, 4, 2, 16, "bf16", False), (70, 3, 2, 32, "fp16", True), (100, 2, 2, 48, "fp16", True),
+                                 (100, 2, 2, 48, "bf16", True), (200, 2, 1, 64, "bf16", False)],
                          ids=str)
-def test_moe_act_order_shard_without_whole_groups(cfg):
+def test_moe_act_order_shard_without_whole_groups(cfg, copy):
     """Row-parallel shards of act-order experts (is_k_full = False; the
     reference's scenario (133, 256, 256, 5, 2, 1, act_order, k_full = False),
     tests/kernels/moe/test_moe.py:688-710): the shard's rows lie in all groups
-    and every row finds its scale through g_idx."""
+    and every row finds its scale through g_idx.  `copy`: with room for a
+    column-permuted copy of A per slot the kernels run without the gather."""
     m, e, top_k, bs, dtype, mul = cfg
     k_full, n, g = 1024, 192, 128
     lo, hi = 384, 768
@@ -210,9 +243,13 @@ def test_moe_act_order_shard_without_whole_groups(cfg):
     npp = gu.dev_i32(np.array([int(past[0])], dtype=np.int32))
     tw = torch.from_numpy(topk_w.astype(np.float32).reshape(-1)).to(gu.DEV)
     workspace = torch.zeros(1024, dtype=torch.int32, device=gu.DEV)
+    scr, nbytes = None, 0
+    if copy:
+        nbytes = (lib.sonar_moe_marlin_gemm_scratch_bytes(sid.numel(), bs, n, k) + 255) // 256 * 256 + sid.numel() * k * 2
+        scr = torch.empty(nbytes, dtype=torch.uint8, device=gu.DEV)
     _lib.check(lib.sonar_moe_wna16_marlin_gemm(
         gu.ptr(a), gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None, gu.ptr(scales), None, gu.ptr(g_dev),
-        gu.ptr(perm), gu.ptr(workspace), workspace.numel(), None, 0, gu.ptr(sid), sid.numel(), gu.ptr(eid),
+        gu.ptr(perm), gu.ptr(workspace), workspace.numel(), gu.ptr(scr), nbytes, gu.ptr(sid), sid.numel(), gu.ptr(eid),
         gu.ptr(npp), gu.ptr(tw), bs, top_k, int(mul), e, gu.dtype_code(dtype), _lib.TYPE_UINT4B8, m, n, k,
         k_full // g, 0, 0, 1, gu.stream()))
     torch.cuda.synchronize()
@@ -270,10 +307,26 @@ def test_moe_matches_dense_gemm_per_expert():
     (700, 4096, 2048, "uint8b128"), (2048, 2048, 1024, "fp8"), (64, 2048, 1024, "uint8b128"),
     # MXFP4 in the tile kernel with few tiles, and with a short last round of them (384 = 256 + 128): both cut along K
     (700, 4096, 2048, "mxfp4"), (2100, 14336, 4096, "mxfp4"),
+    # ... and in the decode kernel on more (block, strip) pairs than compute units (workgroups of four wavefronts)
+    (16, 4096, 4096, "mxfp4"),
     # the fp16 instantiations of the grouped tile kernel's 8-bit and 4-bit forms (256- and 128-row tiles)
     (700, 2048, 1024, "uint8b128/fp16"), (700, 2048, 1024, "fp8/fp16"), (700, 2048, 1024, "uint4b8/fp16"),
     # 8-bit codes with a scale per 32 rows (the layout of MXFP8), either activation type
-    (700, 2048, 1024, "uint8b128g32"), (700, 2048, 1024, "uint8b128g32/fp16"), (700, 2048, 1024, "fp8g32/fp16")])
+    (700, 2048, 1024, "uint8b128g32"), (700, 2048, 1024, "uint8b128g32/fp16"), (700, 2048, 1024, "fp8g32/fp16"),
+    # K of 10 steps, not a whole number of the wide kernel's passes: the eight-wavefront grouped tile kernel's 8-bit forms
+    (700, 640, 512, "uint8b128"), (700, 640, 512, "fp8"), (700, 640, 512, "uint8b128/fp16"), (700, 640, 512, "fp8/fp16"),
+    (700, 640, 512, "uint8b128g32"), (700, 640, 512, "fp8g32"), (700, 640, 512, "uint8b128g32/fp16"),
+    (700, 640, 512, "fp8g32/fp16"),
+    # blocks of 8, 32 and 48 slots of 8-bit codes: the general grouped kernel with one, two and three blocks of rows
+    (8, 512, 256, "uint8b128"), (8, 512, 256, "uint8b128g32"), (100, 512, 256, "uint8b128g32"),
+    (150, 512, 256, "uint8b128g32"), (8, 512, 256, "fp8g32/fp16"), (100, 512, 256, "fp8g32/fp16"),
+    (150, 512, 256, "fp8g32/fp16"),
+    # MXFP4 on a K that is not a whole number of the decode kernel's units (the gpt-oss expert shape): the general kernel
+    (8, 2880, 5760, "mxfp4"),
+    # 64-slot blocks without the scratch the tile kernel needs: the general grouped kernel with four blocks of rows
+    (300, 512, 256, "uint8b128!"), (300, 512, 256, "uint8b128g32!"), (300, 512, 256, "uint8b128/fp16!"),
+    (300, 512, 256, "uint8b128g32/fp16!"), (300, 512, 256, "fp8/fp16!"), (300, 512, 256, "fp8g32/fp16!"),
+    (300, 512, 256, "mxfp4!")])
 def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     """Mixtral-8x7B expert shapes (8 experts, top 2, the block size of the
     reference's rule), where the CPU oracle is too slow: every routed slot must
@@ -283,6 +336,8 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     of 8, 32 and 64 slots, i.e. the grouped decode kernel with one and two
     blocks of rows, its two-halves form and the tile kernel."""
     e, top_k, dtype = 8, 2, torch.bfloat16
+    with_scratch = not wtype.endswith("!")
+    wtype = wtype.rstrip("!")
     if wtype.endswith("/fp16"):
         wtype, dtype = wtype[:-5], torch.float16
     dtype_code = _lib.DTYPE_BF16 if dtype == torch.bfloat16 else _lib.DTYPE_F16
@@ -312,8 +367,8 @@ def test_full_size_grouped_gemm_agrees_with_dense_rows(tokens, k, n, wtype):
     npp = gu.dev_i32(np.array([int(past[0])], dtype=np.int32))
     c = torch.zeros((tokens * top_k, n), dtype=dtype, device=gu.DEV)
     workspace = torch.zeros(1024, dtype=torch.int32, device=gu.DEV)
-    nbytes = lib.sonar_moe_marlin_gemm_scratch_bytes(sid.numel(), bs, n, k)
-    scr = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=gu.DEV)
+    nbytes = lib.sonar_moe_marlin_gemm_scratch_bytes(sid.numel(), bs, n, k) if with_scratch else 0
+    scr = torch.empty(max(nbytes, 16), dtype=torch.uint8, device=gu.DEV) if with_scratch else None
     _lib.check(lib.sonar_moe_wna16_marlin_gemm(
         gu.ptr(a), gu.ptr(c), gu.ptr(native), _lib.LAYOUT_GFX950, None, gu.ptr(scales), None, None, None,
         gu.ptr(workspace), workspace.numel(), gu.ptr(scr), nbytes, gu.ptr(sid), sid.numel(), gu.ptr(eid),
@@ -490,16 +545,18 @@ def test_gated_activation_rejections():
     assert lib.sonar_moe_activation(gu.ptr(out), gu.ptr(x), 4, 12, 2, 0.0, 1.0, 0.0, 0, gu.stream()) == _lib.E_INVALID
 
 
-def test_moe_tiled_and_streaming_kernels_agree():
-    """The same 64-slot-block call with and without the scratch the tiled kernel
-    needs for its table takes two different kernels; both meet the tolerance
-    against the reference and each other."""
-    m, e, top_k, k, n, bs = 260, 4, 2, 512, 256, 64
-    ex = Experts(91, e, k, n, 128, "bf16")
+@pytest.mark.parametrize("dtype,zp", [("bf16", False), ("fp16", False), ("fp16", True), ("bf16", True)])
+def test_moe_tiled_and_streaming_kernels_agree(dtype, zp):
+    """The same 64-slot-block call (more slots than the decode kernel takes) with
+    and without the scratch the tiled kernel needs for its table takes two
+    different kernels; both meet the tolerance against the reference and each
+    other."""
+    m, e, top_k, k, n, bs = 700, 4, 2, 512, 256, 64
+    ex = Experts(91, e, k, n, 128, dtype, zero_points=zp)
     topk_ids, topk_w = route(7, m, e, top_k)
     sorted_ids, expert_ids, past = mo.moe_align_block_size(topk_ids, bs, e)
-    a32 = mo.make_activations(4, m, k, "bf16")
-    a = gu.dev_bits16(a32, "bf16")
+    a32 = mo.make_activations(4, m, k, dtype)
+    a = gu.dev_bits16(a32, dtype)
     tiled = gu.host_f32(ex.gemm(a, sorted_ids, expert_ids, int(past[0]), topk_w, bs, top_k, m, True, scratch=True))
     streamed = gu.host_f32(ex.gemm(a, sorted_ids, expert_ids, int(past[0]), topk_w, bs, top_k, m, True, scratch=False))
     want = ex.reference(a32, sorted_ids, expert_ids, int(past[0]), bs, top_k, m, topk_w)

@@ -1023,6 +1023,7 @@ def test_prepare_moe_mxfp4_layer_and_fused_marlin_moe(cfg):
     (70, 4, 2, 256, 256),
     (200, 8, 2, 128, 96),      # intermediate size padded to 128 inside
     (1500, 4, 2, 256, 128),    # 64-slot blocks: the tiled grouped kernel
+    (40, 4, 2, 256, 128),      # 32-slot blocks: two blocks of rows per workgroup of the general grouped kernel
 ], ids=str)
 def test_prepare_nvfp4_moe_layer_and_fused_marlin_moe(cfg, dtype):
     """NVFP4 expert weights (w13 (E, 2N, K/2), w2 (E, K, N/2) bytes, float8_e4m3fn block

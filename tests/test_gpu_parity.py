@@ -132,6 +132,18 @@ GEMM_CASES = [
     (64, 512, 16384, -1, False, False, False),
     (33, 2048, 8448, 128, False, False, True),
     (49, 256, 8256, 256, True, False, False),
+    # up to 16 rows on more strips than compute units: workgroups of four wavefronts, with one, two and four
+    # groups per 128 rows
+    (9, 256, 16448, 128, True, False, False),
+    (16, 256, 16448, 64, False, False, True),
+    (13, 512, 16448, 64, True, False, False),
+    (16, 256, 16448, 32, False, False, False),
+    (5, 512, 16448, 32, True, False, True),
+    # K = 320 is not a whole number of the decode kernel's 128-row units: the general kernel with zero points,
+    # one, two and three blocks of 16 rows
+    (7, 320, 192, 64, True, False, False),
+    (20, 320, 192, -1, True, False, True),
+    (40, 320, 192, 64, True, False, False),
 ]
 
 
@@ -216,6 +228,11 @@ def test_error_paths(gu):
     layer.workspace = torch.zeros(4, dtype=torch.int32, device=gu.DEV)
     with pytest.raises(_lib.SonarMarlinError, match="workspace"):
         layer.gemm(a, 1)
+    # act-order with zero points: the reference generates no such kernel (generate_kernels.py:66-72) and
+    # fails with "Unsupported shapes" (marlin.cu:509-519)
+    layer = gu.DeviceLayer(2, 256, 64, 128, "fp16", zero_points=True, act_order=True)
+    with pytest.raises(NotImplementedError, match="Unsupported shapes"):
+        layer.gemm(torch.zeros((1, 256), dtype=torch.float16, device=gu.DEV), 1)
 
 
 TILE_CASES = [
@@ -233,6 +250,8 @@ TILE_CASES = [
     (1000, 2048, 1024, 32, False, False, True),
     # 9 x 29 = 261 tiles: 256 whole ones, then the last 5 split six ways along K
     (2200, 3072, 7360, 128, True, False, True),
+    # K of five steps: not a whole number of the wide kernel's passes of four, the eight-wavefront kernel
+    (600, 320, 512, 64, False, False, True),
 ]
 
 
@@ -274,11 +293,12 @@ WIDE_TILE_CASES = [
     # 97..128 rows on more strips than compute units: 128-row tiles, K in two ranges
     (128, 512, 16640, 128, False, True),
     (100, 1024, 16448, -1, True, False),
-    # groups of 32 rows: a row of scales (and zero points) per k block, 256-row tiles
-    (300, 1024, 768, 32, True, True),         # two ranges of K
-    (2100, 512, 4096, 32, False, False),      # 144 tiles
+    # groups of 32 rows: a row of scales (and zero points) per k block
+    (300, 1024, 768, 32, True, True),         # 128-row tiles, two ranges of K
+    (2100, 512, 4096, 32, False, False),      # 144 tiles of 256 rows
     (1030, 2048, 4160, 32, True, False),      # ragged both ways, K split
     (600, 1216, 512, 32, False, True),        # 19 steps: the eight-wavefront kernel
+    (2100, 256, 4160, 32, True, True),        # 153 tiles of 256 rows with zero points, ragged both ways
 ]
 
 
@@ -409,6 +429,7 @@ W8_CASES = [
     (1024, 1024, 832, 32, False, False),     # groups of 32 rows, whole tiles over all of K
     (700, 1280, 4160, 32, False, True),      # ... K ranges of 20 steps, ragged tiles both ways
     (300, 1216, 512, 32, False, False),      # ... 19 steps: not a multiple of four (the eight-wavefront kernel)
+    (2100, 512, 4160, 128, False, True),     # more than 128 tiles of 256 rows: 256-row tiles, ragged both ways
 ]
 
 
@@ -486,6 +507,7 @@ FP8_CASES = [
     (1, 4096, 4096, 128, False),
     (16, 1024, 256, 32, False),       # groups of 32 rows: MXFP8
     (100, 512, 192, 32, True),
+    (20, 512, 192, 32, False),        # ... two blocks of 16 rows
     # the MFMA tile kernel's form for 8-bit floating-point codes
     (300, 2048, 512, 128, True),
     (1024, 1024, 832, -1, False),
@@ -495,6 +517,7 @@ FP8_CASES = [
     (1024, 1024, 832, 32, False),     # groups of 32 rows, whole tiles over all of K
     (700, 1280, 4160, 32, True),      # ... K ranges of 20 steps, ragged tiles both ways
     (300, 1216, 512, 32, False),      # ... 19 steps: not a multiple of four (the eight-wavefront kernel)
+    (2100, 512, 4160, -1, True),      # more than 128 tiles of 256 rows: 256-row tiles, ragged both ways
 ]
 
 
@@ -583,6 +606,8 @@ MXFP4_CASES = [
     (1, 2880, 5760, False),     # gpt-oss expert shape: K is 90 groups of 32 rows
     (1024, 2880, 5760, True),   # the same through the tile kernel (K = 45 steps of 64 rows)
     (4096, 4096, 1024, False),  # tile kernel, several rounds of tiles
+    (2100, 512, 4160, True),    # ... 153 tiles of 256 rows, ragged both ways
+    (16, 256, 16448, False),    # more strips than compute units: the decode kernel's workgroups of four wavefronts
 ]
 
 

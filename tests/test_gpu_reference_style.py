@@ -236,6 +236,11 @@ def _moe_cases():
                     continue
                 cases.append((cfg.get("a_quant"), cfg["b_type"], cfg.get("a_type", torch.float16), group_size, m, n, k,
                               e, topk, ep_size, act_order, is_k_full))
+    # beyond the reference's list: act-order shards (is_k_full = False) of 8-bit experts on routing blocks of
+    # 8, 32, 48 and 64 slots, either activation type
+    for dtype in (torch.float16, torch.bfloat16):
+        for m in (1, 40, 90, 133):
+            cases.append((None, scalar_types.uint8b128, dtype, 64, m, 256, 256, 5, 2, 1, True, False))
     return cases
 
 
