@@ -144,7 +144,7 @@ INT8_CASES = [
     (512, 192, 32, True, "fp16", False, [17, 65]),
     (1024, 64, 64, True, "bf16", False, [2]),
     (8192, 64, 128, False, "fp16", True, [1, 20]),     # K split over workgroups
-    (4096, 128, -1, False, "bf16", False, [9]),         # channelwise, K split
+    (4096, 128, -1, False, "bf16", False, [9]),         # channelwise, a long K in one range
     (1056, 128, -1, False, "fp16", False, [4]),         # K a multiple of 32 only
     # the tiled kernel (more than 64 rows, N a multiple of 128, K of 128, groups of 64 rows or more)
     (1024, 256, -1, False, "fp16", True, [65, 200]),

@@ -264,6 +264,41 @@ def test_kernels_with_hand_counted_waits_do_not_spill():
         assert seen >= 4, f"no resource report for {kernel}"
 
 
+KERNEL_FORMS = {
+    "awq_to_marlin_kernel": 1, "gfx950_to_marlin_kernel": 1, "gptq8_to_marlin_a8_kernel": 1,
+    "gptq8_to_marlin_kernel": 2, "gptq_to_marlin_kernel": 2, "int4_fp8_preprocess_kernel": 1,
+    "marlin8_gfx950_kernel": 2, "marlin_a8_finish_kernel": 9, "marlin_a8_kernel": 68,
+    "marlin_a8_tile_kernel": 48, "marlin_a8_to_gfx950_kernel": 1, "marlin_dequant8_kernel": 4,
+    "marlin_dequant_kernel": 7, "marlin_fixup_kernel": 8, "marlin_moe8_kernel": 40, "marlin_moe_a8_kernel": 68,
+    "marlin_moe_kernel": 52, "marlin_stream8_kernel": 40, "marlin_stream_fast_kernel": 68,
+    "marlin_stream_kernel": 44, "marlin_tile_async_kernel": 38, "marlin_tile_kernel": 6,
+    "marlin_tile_wide_kernel": 60, "marlin_to_gfx950_kernel": 1, "moe_activation_kernel": 12,
+    "moe_align_count_kernel": 1, "moe_align_place_kernel": 1, "moe_permute_rows_kernel": 1,
+    "moe_sum_kernel": 2, "moe_tile_reduce_kernel": 2, "moe_tile_table_kernel": 1, "per_token_quant_kernel": 6,
+    "permute_columns_kernel": 1, "silu_and_mul_kernel": 2, "tile_reduce_kernel": 2, "to_marlin_a8_kernel": 3,
+}
+
+
+def test_library_holds_the_kernel_forms_the_gpu_tests_launch():
+    """The instantiations of every __global__ function in the built library,
+    counted from its host-side launch stubs.  Each of the forms counted here is
+    launched by at least one GPU parity case (compared against a kernel trace of
+    the whole GPU suite); a count that changes means a form was added or dropped:
+    give a new form a parity case before raising the number."""
+    import collections
+    import re
+    import shutil
+    import subprocess
+    from sonar_amd import _lib
+    nm = shutil.which("nm") or shutil.which("llvm-nm")
+    if nm is None:
+        pytest.skip("nm not available")
+    _lib.load()
+    syms = subprocess.run([nm, _lib._LIB_PATH], capture_output=True, text=True, timeout=120).stdout
+    seen = collections.Counter(m.group(1) for m in re.finditer(r"__device_stub__\d*([a-z_0-9]+kernel)", syms))
+    assert dict(seen) == KERNEL_FORMS
+
+
 def test_awq_checkpoint_conversion_matches_gptq_packing():
     """AutoAWQ tensors through convert_awq_to_standard_format give what packing the
     same codes the GPTQ way gives (layers/quantization/auto_awq.py:93-153)."""
