@@ -176,11 +176,14 @@ size_t sonar_marlin_gemm_scratch_bytes(int64_t size_m, int64_t size_n, int64_t s
  *   b_zeros      int32[num_groups][N/8] in marlin_zero_points order, or NULL
  *                (required iff b_type_id == SONAR_TYPE_UINT4)
  *   g_idx, perm  int32[K] each or both NULL; with both given the call is an
- *                act-order call: perm maps weight row k to column perm[k] of
- *                A; g_idx[k] is the group of weight row k, read only when
- *                is_k_full == 0 (a shard that does not hold whole groups:
- *                b_scales then has every group of the unsharded matrix,
- *                num_groups need not divide K, b_zeros must be NULL, and the
+ *                act-order call (symmetric weights only: with b_zeros it is
+ *                refused with SONAR_E_UNSUPPORTED, "Unsupported shapes", as
+ *                the reference has no such kernel,
+ *                marlin/generate_kernels.py:66-72): perm maps weight row k to
+ *                column perm[k] of A; g_idx[k] is the group of weight row k,
+ *                read only when is_k_full == 0 (a shard that does not hold
+ *                whole groups: b_scales then has every group of the unsharded
+ *                matrix, num_groups need not divide K, and the
  *                size_m * size_k * 2 extra scratch bytes below are required)
  *   workspace    int32[workspace_len], all zero on entry, all zero on exit;
  *                workspace_len >= number of compute units
@@ -237,7 +240,8 @@ int sonar_per_token_quant_fp8(const void* x, int dtype, int64_t row_stride, uint
  * act-order (the reference builds no such kernel).  b_type_id uint4b8 or uint4, or float4_e2m1f
  * with float8_e4m3fn activations (MXFP4 weights, "W4A8-FP4", dequant.h:474-490, marlin.cu:576-590):
  * b_scales then are exponent bytes [K/32][N] in the same order, each 6 above the checkpoint's
- * (mxfp4_marlin_process_scales with an fp8 input type), no zero points, and
+ * (mxfp4_marlin_process_scales with an fp8 input type), no zero points, dtype bfloat16 only
+ * (marlin/generate_kernels.py:152-161; float16 is refused with SONAR_E_UNSUPPORTED), and
  * C = round((sum_g 2^(e[g][n] - 127 - 6) * sum_{k in g} a[m][k] * value(code[k][n])) * a_scales[m] + bias). */
 size_t sonar_marlin_gemm_a8_scratch_bytes(int64_t size_m, int64_t size_n, int64_t size_k,
                                           int64_t num_groups);
@@ -337,8 +341,9 @@ int sonar_marlin_gemm_noalloc(const void* a, int64_t a_row_stride, void* c,
  *                20 times faster with sorted_len * K * 2 bytes more behind that
  *                size rounded up to 256 (a column-permuted copy of A per slot;
  *                required for act-order with uint8b128)
- *   g_idx, perm  int32[num_experts][K] or NULL; with is_k_full == 0 (shards that
- *                hold no whole group; no zero points) g_idx is the group of
+ *   g_idx, perm  int32[num_experts][K] or NULL (act-order: symmetric weights only, refused
+ *                with SONAR_E_UNSUPPORTED together with b_zeros); with is_k_full == 0 (shards that
+ *                hold no whole group) g_idx is the group of
  *                every sorted row and num_groups the groups of the whole matrix
  *   sorted_token_ids int32[sorted_len], expert_ids int32[ceil(sorted_len/bs)],
  *   num_tokens_past_padded int32[1] (read on the device), topk_weights
