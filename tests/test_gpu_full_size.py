@@ -122,6 +122,40 @@ def test_prefill_sweep_meets_the_oracle_on_sampled_columns(name, m):
     check_columns(layer, a, c, m, sampled_columns(layer.n, 6, m))
 
 
+@pytest.mark.parametrize("name,m,dtype", [
+    ("o", 16, "bf16"),        # decode kernel, four pieces per strip summed through tickets in the workspace
+    ("down", 16, "bf16"),     # ... with non-temporal weight copies
+    ("gate_up", 48, "bf16"),  # ... blocks of rows, more workgroups than compute units
+    ("o", 256, "fp16"),       # tile kernel, 128-row tiles cut along K, partial tiles summed by a second kernel
+    ("qkv", 4096, "fp16"),    # tile kernel, two launches (256-row tiles, then the short last round as 128-row tiles)
+])
+def test_gemm_replayed_from_a_hip_graph_gives_the_eager_bits(name, m, dtype):
+    """The launches of one call captured into a HIP graph and replayed three times, with an eager
+    call of another size on the same workspace between the replays: every replay gives the bits of
+    the eager call and leaves the workspace zero (nothing in the library's launches depends on
+    state the host set up for one launch only)."""
+    layer = big_layer(name, dtype)
+    gen = torch.Generator(device=gu.DEV).manual_seed(m + 7)
+    a = (torch.randn((m, layer.k), device=gu.DEV, generator=gen) * 0.5).to(layer.tdt)
+    want = layer.gemm(a, m)
+    torch.cuda.synchronize()
+    stream = torch.cuda.Stream()
+    with torch.cuda.stream(stream):
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            got = layer.gemm(a, m)
+        for _ in range(3):
+            other_m = max(1, m // 2 - 1)
+            other = layer.gemm(a[:other_m], other_m)      # eager work between the replays
+            graph.replay()
+            stream.synchronize()
+            assert torch.equal(got.view(torch.int16), want.view(torch.int16))
+            assert bool(torch.isfinite(other.float()).all())
+            assert int(layer.workspace.abs().sum().item()) == 0
+            got.zero_()
+    torch.cuda.synchronize()
+
+
 _experts = {}
 
 
