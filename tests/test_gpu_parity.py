@@ -176,11 +176,14 @@ def test_gemm_row_strided_activations(gu, m, k, n):
     assert ok, (max_err, max_ref)
 
 
-@pytest.mark.parametrize("m", [32, 300])
-def test_gemm_subset_input_like_the_reference(gu, m):
+@pytest.mark.parametrize("m,n", [(32, 2048), (300, 2048),
+                                 # the same window through the decode kernel (one block of rows, and blocks of
+                                 # rows on 64 strips) and through 256-row tiles
+                                 (9, 2048), (16, 4096), (40, 4096), (2100, 4096)])
+def test_gemm_subset_input_like_the_reference(gu, m, n):
     """tests/kernels/quantization/test_marlin_gemm.py:494-537: A is the window
     [8:m+8, 8:k+8] of a matrix twice as large (row stride 2k, 16-byte offset)."""
-    k, n = 1024, 2048
+    k = 1024
     layer = gu.DeviceLayer(8, k, n, 128, "fp16")
     big32 = mo.make_activations(6, 2 * m, 2 * k, "fp16")
     a = gu.dev_bits16(big32, "fp16")[8:m + 8, 8:k + 8]
