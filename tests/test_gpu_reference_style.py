@@ -248,11 +248,12 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None, input_d
     """MarlinMoEWeightData.make (test_moe.py:774-892): every expert's (N, K)
     matrix quantised and laid out on its own, then stacked."""
     from sonar_amd.marlin_utils import marlin_permute_bias
-    from sonar_amd.marlin_utils_fp4 import rand_marlin_weight_mxfp4_like
+    from sonar_amd.marlin_utils_fp4 import rand_marlin_weight_mxfp4_like, rand_marlin_weight_nvfp4_like
     from sonar_amd.marlin_utils_fp8 import marlin_quant_fp8_torch
     from tests.marlin_utils_for_tests import awq_marlin_quantize, marlin_quantize
     k = w.shape[-1]
-    out = {"w_ref": [], "qweight": [], "scales": [], "zeros": [], "g_idx": [], "sort_indices": [], "bias": []}
+    out = {"w_ref": [], "qweight": [], "scales": [], "zeros": [], "g_idx": [], "sort_indices": [], "bias": [],
+           "global_scale": []}
     for i in range(w.shape[0]):
         if quant_type == scalar_types.uint4:
             w_ref, qweight, scales, zeros = awq_marlin_quantize(w[i].transpose(1, 0), quant_type, group_size,
@@ -260,6 +261,10 @@ def _marlin_moe_weights(w, quant_type, group_size, act_order, bias=None, input_d
             out["zeros"].append(zeros)
         elif quant_type == scalar_types.float8_e4m3fn:
             w_ref, qweight, scales = marlin_quant_fp8_torch(w[i].contiguous(), group_size)
+        elif quant_type == scalar_types.float4_e2m1f and group_size == 16:      # NVFP4 (test_moe.py:806-816)
+            w_ref, qweight, scales, global_scale = rand_marlin_weight_nvfp4_like(w[i], group_size,
+                                                                                 input_dtype=input_dtype)
+            out["global_scale"].append(global_scale.reshape(()))
         elif quant_type == scalar_types.float4_e2m1f:
             w_ref, qweight, scales = rand_marlin_weight_mxfp4_like(w[i], group_size, input_dtype=input_dtype)
         else:
@@ -406,6 +411,32 @@ def test_fused_marlin_moe_other_activations(name, b_type, group_size, dtype):
                                  topk_weights, topk_ids.to(torch.int32), global_num_experts=e,
                                  quant_type_id=b_type.id)
         assert float((plain.float() - want.float()).abs().max()) > 5e-2 * float(want.float().abs().max())
+
+
+@pytest.mark.parametrize("m", [1, 64, 256])
+@pytest.mark.parametrize("n,k", [(1024, 1024), (2048, 2048)])
+@pytest.mark.parametrize("e,topk", [(8, 2), (64, 4)])
+def test_fused_marlin_moe_non_gated(m, n, k, e, topk):
+    """tests/kernels/moe/test_moe.py:1083-1161: NVFP4 experts (groups of 16, a global scale per
+    expert) with relu2_no_mul, whose w1 is (e, n, k) and not (e, 2n, k); atol 1e-1."""
+    from sonar_amd.fused_moe import fused_marlin_moe
+    torch.manual_seed(42)
+    quant_type, dtype = scalar_types.float4_e2m1f, torch.bfloat16
+    a = torch.randn((m, k), device="cuda", dtype=dtype) / 10
+    w1 = torch.randn((e, n, k), device="cuda", dtype=dtype) / 10
+    w2 = torch.randn((e, k, n), device="cuda", dtype=dtype) / 10
+    d1 = _marlin_moe_weights(w1, quant_type, 16, False)
+    d2 = _marlin_moe_weights(w2, quant_type, 16, False)
+    score = torch.randn((m, e), device="cuda", dtype=dtype)
+    topk_weights, topk_ids = torch.topk(torch.softmax(score, dim=-1, dtype=torch.float32), topk)
+    want = _torch_experts(a, d1["w_ref"], d2["w_ref"], topk_weights, topk_ids,
+                          activation=lambda h: torch.relu(h) ** 2)
+    got = fused_marlin_moe(a, d1["qweight"], d2["qweight"], None, None, d1["scales"], d2["scales"], topk_weights,
+                           topk_ids.to(torch.int32), global_num_experts=e, expert_map=None,
+                           global_scale1=d1["global_scale"], global_scale2=d2["global_scale"],
+                           quant_type_id=quant_type.id, is_k_full=True, activation="relu2_no_mul")
+    torch.cuda.synchronize()
+    torch.testing.assert_close(got, want, atol=1e-1, rtol=0)
 
 
 @pytest.mark.parametrize("m", [1, 256])
