@@ -20,11 +20,14 @@ SWITCHES = [
     "SONAR_MARLIN_NO_SLABS",         # no blocks of rows in the 16-row kernel
     "SONAR_MARLIN_NO_ROW_PAIRS",     # blocks of 16 rows only
     "SONAR_MARLIN_NO_HALF_WG",       # 8-wavefront workgroups only
+    "SONAR_MARLIN_SPLIT=1",          # no strip shared between workgroups
+    "SONAR_MARLIN_NO_INLINE_SUM",    # shared strips summed by the fix-up launch
     "SONAR_MARLIN_NO_TILE",          # the streaming kernels in 64-row slabs for every M
     "SONAR_MARLIN_NO_WIDE_TILE",     # the eight-wavefront tile kernel where the wide one would run
     "SONAR_MARLIN_NO_128_ROW_TILES", # the wide tile kernel with 256-row tiles only
     "SONAR_MARLIN_NO_ASYNC_TILE",    # the register-staged tile kernel
     "SONAR_MARLIN_MAX_K_SPLITS=1",   # no split K in the tile kernel
+    "SONAR_MARLIN_NO_TWO_TILE_SIZES",  # a short last round of tiles cut along K instead of a second launch of 128-row tiles
     "SONAR_MARLIN_NO_MOE_TILE",      # the grouped streaming kernel for 64-slot blocks
     "SONAR_MARLIN_NO_MOE_FAST",      # ... and for blocks of up to 32 slots
     "SONAR_MARLIN_NO_MOE_K_SPLIT",   # the grouped wide tile kernel never cuts its tiles along K
