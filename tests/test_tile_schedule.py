@@ -42,14 +42,12 @@ def _check_cover(rows, tiles_by_rows, tiles_n, k_steps):
 LLAMA = {"qkv": (4096, 6144), "o": (4096, 4096), "gate_up": (4096, 28672), "down": (14336, 4096)}
 
 
-@pytest.mark.parametrize("m", [65, 100, 128, 200, 256, 300, 512, 1000, 1024, 2048, 3900, 4096, 5000, 8192])
-@pytest.mark.parametrize("name", list(LLAMA))
-def test_dense_launches_cover_every_tile_and_k_step_once(name, m):
-    k, n = LLAMA[name]
-    rows = _rows("sonar_debug_tile_schedule", m, n, k, k // 128)
+def _check_dense(m, n, k, groups):
+    """Returns what the call got: "none", "one launch" or "two launches"."""
+    rows = _rows("sonar_debug_tile_schedule", m, n, k, groups)
     if len(rows) == 0:      # the call is not planned for the tile kernels (few rows on few strips)
         assert m <= 512
-        return
+        return "none"
     tiles_n = (n + 255) // 256
     launches = sorted(set(rows[:, 0].tolist()))
     sizes = sorted(set(rows[:, 1].tolist()))
@@ -57,7 +55,7 @@ def test_dense_launches_cover_every_tile_and_k_step_once(name, m):
         assert len(sizes) == 1
         r = sizes[0]
         _check_cover(rows, {r: set(range((m + r - 1) // r))}, tiles_n, k // 64)
-        return
+        return "one launch"
     # two launches: whole rounds of 256-row tiles, then the rest as 128-row tiles; every row of C is
     # covered by exactly one of the two sizes, per column tile
     assert launches == [0, 1] and sizes == [128, 256]
@@ -71,6 +69,48 @@ def test_dense_launches_cover_every_tile_and_k_step_once(name, m):
         else:
             cover[tm, tn] += 1
     assert np.all(cover == 1)
+    return "two launches"
+
+
+@pytest.mark.parametrize("m", [65, 100, 128, 200, 256, 300, 512, 1000, 1024, 2048, 3900, 4096, 5000, 8192])
+@pytest.mark.parametrize("name", list(LLAMA))
+def test_dense_launches_cover_every_tile_and_k_step_once(name, m):
+    k, n = LLAMA[name]
+    _check_dense(m, n, k, k // 128)
+
+
+def test_dense_launches_of_random_shapes_cover_every_tile_and_k_step_once():
+    """Seeded draws over rows, columns (multiples of 64), K (multiples of 64) and group sizes, small and
+    large: one launch of either tile size, with and without ranges of K, and the two-launch form."""
+    rng = np.random.default_rng(11)
+    kinds = {}
+    for i in range(600):
+        if i % 2:
+            m, n = int(rng.integers(65, 9000)), 64 * int(rng.integers(1, 513))
+        else:
+            m, n = int(rng.integers(65, 1200)), 64 * int(rng.integers(1, 100))
+        k = 64 * int(rng.integers(1, 257))
+        choices = [1] + [k // g for g in (32, 64, 128, 256) if k % g == 0 and k // g > 1]
+        kind = _check_dense(m, n, k, int(rng.choice(choices)))
+        kinds[kind] = kinds.get(kind, 0) + 1
+    assert kinds.get("one launch", 0) > 100 and kinds.get("two launches", 0) > 10, kinds
+
+
+def test_grouped_launches_of_random_shapes_cover_the_live_tiles_once():
+    rng = np.random.default_rng(12)
+    cut = 0
+    for _ in range(600):
+        max_row_tiles = int(rng.integers(1, 200))
+        row_tiles = int(rng.integers(0, max_row_tiles + 1))
+        n, k = 64 * int(rng.integers(1, 460)), 64 * int(rng.integers(1, 257))
+        tile_rows, with_partial = int(rng.choice([256, 128])), int(rng.integers(0, 2))
+        rows = _rows("sonar_debug_moe_tile_schedule", row_tiles, max_row_tiles, n, k, tile_rows, with_partial)
+        if row_tiles == 0:
+            assert len(rows) == 0
+            continue
+        _check_cover(rows, {tile_rows: set(range(row_tiles))}, (n + 255) // 256, k // 64)
+        cut += bool(np.any(rows[:, 5] - rows[:, 4] != k // 64))
+    assert cut > 5      # some of the draws are launches with tiles cut along K
 
 
 def test_qkv_at_4096_rows_is_the_two_launch_case():
