@@ -5,8 +5,11 @@ A step is one pass over the four W4A16 projection GEMMs of a Llama-3-8B decoder
 layer (qkv 4096x6144, o 4096x4096, gate_up 4096x28672, down 14336x4096;
 int4 weights, group size 128) at M = 16 bf16 activation rows, through the same
 torch ops the reference's callers use.  Weights of `--copies` distinct layers
-(more bytes than the 256 MB last-level cache) are visited round-robin so every
-step streams its weights from HBM.  The K timed steps are recorded in one HIP
+are visited round-robin so that every step streams its weights from HBM: 24 by
+default, because the two large matrices are copied with the non-temporal bit
+and leave the 256 MB last-level cache to the two small ones, whose 24 copies
+(519 MB) are what it would have to hold between two uses (with 6 copies the
+step measures 4 % faster than with 12, 24 or 48, which agree).  The K timed steps are recorded in one HIP
 graph; the graph is replayed `REPLAYS` times, each replay between two events on
 the launching stream, and the line reports the median replay (with the 10th
 and 90th percentile beside it).
@@ -30,7 +33,7 @@ if ROOT not in sys.path:
     sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
-# HBM bytes per GEMM launch of the default workload (M = 16, 6 weight copies), from one
+# HBM bytes per GEMM launch of the default workload (M = 16, 24 weight copies), from one
 # `rocprofv3 --pmc FETCH_SIZE` and one `--pmc WRITE_SIZE` run of
 # `bench.py --no-prefill --eager --calibrate`
 # (profiles/marlin_stream_fast_kernel_llama3-8b-layer_m16_hbm-traffic.txt): FETCH_SIZE scaled
@@ -39,11 +42,12 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 # cannot be read from inside a run: the figure belongs to the launches of that profile
 # (PROFILED_LAUNCHES: workgroups, threads per workgroup, pieces per strip, non-temporal weight
 # copies, as sonar_marlin_last_decode_launch reports them) and is reported only while the run's
-# own launches are the same, for M = 16 with six weight copies; otherwise `traffic` is null.
+# own launches are the same, for M = 16 with the default number of weight copies; otherwise `traffic` is null.
 MEASURED_TRAFFIC_M16 = 32_400_000
 PROFILED_LAUNCHES = {"qkv": [192, 512, 2, 0], "o": [256, 512, 4, 0], "gate_up": [448, 256, 1, 1],
                      "down": [256, 512, 4, 1]}
 REPLAYS = 21                # graph replays per timing; the median is reported
+DEFAULT_COPIES = 24          # distinct layers visited round-robin (see the module docstring)
 MFMA_PEAK_TFLOPS = 2500.0   # MI355X dense fp16 / bf16
 MFMA_PEAK_8BIT_TFLOPS = 5000.0   # MI355X dense int8 / fp8
 GROUP = 128
@@ -85,8 +89,9 @@ def time_graph(torch, fn, reps, replays=REPLAYS, spread=False):
     call (with `spread`: median, 10th and 90th percentile)."""
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
-        # every weight copy fn cycles through gets its one-time layout conversion here,
-        # outside the graph (fn(i) uses copy i modulo the number of copies, at most 8)
+        # the first weight copies fn cycles through get their one-time layout conversion here,
+        # outside the graph (fn(i) uses copy i modulo the number of copies; the decode step's
+        # copies have all been through the warm-up steps before)
         for i in range(min(reps, 8)):
             fn(i)
         stream.synchronize()
@@ -432,7 +437,7 @@ def main() -> int:
     ap.add_argument("--steps", type=int, default=200)
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--m", type=int, default=16, help="activation rows of the decode step (1..64)")
-    ap.add_argument("--copies", type=int, default=6)
+    ap.add_argument("--copies", type=int, default=DEFAULT_COPIES)
     ap.add_argument("--sweep", action="store_true")
     ap.add_argument("--no-cpu", action="store_true")
     ap.add_argument("--no-prefill", action="store_true", help="skip the M = 4096 half of the metric")
@@ -553,7 +558,7 @@ def main() -> int:
         "tflops": round(step_flops / step_s / 1e12, 2),
         "roofline": {"bound": "hbm", "achieved": round(gbps, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
                      "frac": round(gbps / HBM_PEAK_GBPS, 4),
-                     "traffic": MEASURED_TRAFFIC_M16 if (m == 16 and args.copies == 6 and
+                     "traffic": MEASURED_TRAFFIC_M16 if (m == 16 and args.copies == DEFAULT_COPIES and
                                                          launch_shapes == PROFILED_LAUNCHES) else None,
                      "launches": launch_shapes,
                      "kernel": kernel,

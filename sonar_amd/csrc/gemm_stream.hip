@@ -1950,7 +1950,8 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
       p.ticket_stride = room >= 4 ? 4 : (int)room;
       p.xcd_ranges = p.slabs == 1 && p.parts % 8 == 0;
     }
-    p.nt_weights = p.slabs == 1 && size_k * size_n / 2 >= 20 * 1000 * 1000;
+    static const bool no_nt = getenv("SONAR_MARLIN_NO_NT_WEIGHTS") != nullptr;
+    p.nt_weights = !no_nt && p.slabs == 1 && size_k * size_n / 2 >= 20 * 1000 * 1000;
     g_last_decode_launch[0] = p.grid_parts * p.slabs;
     g_last_decode_launch[1] = half ? 256 : 512;
     g_last_decode_launch[2] = 1 << shift;

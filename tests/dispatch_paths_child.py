@@ -106,7 +106,18 @@ def grouped() -> None:
     print("grouped nvfp4 ok", flush=True)
 
 
+def dense_large() -> None:
+    """The two large projections of the benchmark's layer at 16 rows: the matrices whose weight copies
+    carry the non-temporal bit unless it is switched off (sampled columns against the oracle)."""
+    from tests import test_gpu_full_size as tf
+    for name in ("gate_up", "down"):
+        tf.test_decode_sweep_meets_the_oracle_on_sampled_columns(name, 16)
+        print("dense large", name, "ok", flush=True)
+
+
 if __name__ == "__main__":
+    if "SONAR_MARLIN_NO_NT_WEIGHTS" in os.environ:
+        dense_large()
     dense()
     dense_mxfp4()
     dense_8bit()

@@ -20,6 +20,7 @@ SWITCHES = [
     "SONAR_MARLIN_NO_SLABS",         # no blocks of rows in the 16-row kernel
     "SONAR_MARLIN_NO_ROW_PAIRS",     # blocks of 16 rows only
     "SONAR_MARLIN_NO_HALF_WG",       # 8-wavefront workgroups only
+    "SONAR_MARLIN_NO_NT_WEIGHTS",    # no non-temporal bit on the weight copies of large matrices
     "SONAR_MARLIN_SPLIT=1",          # no strip shared between workgroups
     "SONAR_MARLIN_NO_INLINE_SUM",    # shared strips summed by the fix-up launch
     "SONAR_MARLIN_NO_TILE",          # the streaming kernels in 64-row slabs for every M
