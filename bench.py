@@ -89,10 +89,9 @@ def time_graph(torch, fn, reps, replays=REPLAYS, spread=False):
     call (with `spread`: median, 10th and 90th percentile)."""
     stream = torch.cuda.Stream()
     with torch.cuda.stream(stream):
-        # the first weight copies fn cycles through get their one-time layout conversion here,
-        # outside the graph (fn(i) uses copy i modulo the number of copies; the decode step's
-        # copies have all been through the warm-up steps before)
-        for i in range(min(reps, 8)):
+        # every weight copy fn cycles through gets its one-time layout conversion here,
+        # outside the graph (fn(i) uses copy i modulo the number of copies, at most 32)
+        for i in range(min(reps, 32)):
             fn(i)
         stream.synchronize()
         graph = torch.cuda.CUDAGraph()
@@ -251,7 +250,7 @@ def variants_sweep(torch, ops, gen, time_graph):
         layers = []
         words = 4 * n if name in ("w8a16", "fp8", "mxfp8") else 2 * n     # 8-bit codes: four per word
         act_dtype = torch.bfloat16 if name in ("mxfp4", "mxfp8") else torch.float16
-        for _ in range(6):
+        for _ in range(16):   # 16 x 22.5 MB of 4-bit codes: more than the 256 MB last-level cache holds
             qw = torch.randint(-2 ** 31, 2 ** 31 - 1, (k // 16, words), dtype=torch.int32, device=dev, generator=gen)
             sc = (torch.rand((k // GROUP, n), device=dev, generator=gen) * 9e-3 + 1e-3).to(torch.float16)
             ws = marlin_utils.marlin_make_workspace_new(torch.device(dev))
