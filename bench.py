@@ -44,7 +44,7 @@ HBM_PEAK_GBPS = 8000.0      # MI355X HBM3E
 # copies, as sonar_marlin_last_decode_launch reports them) and is reported only while the run's
 # own launches are the same, for M = 16 with the default number of weight copies; otherwise `traffic` is null.
 MEASURED_TRAFFIC_M16 = 32_400_000
-PROFILED_LAUNCHES = {"qkv": [192, 512, 2, 0], "o": [256, 512, 4, 0], "gate_up": [448, 256, 1, 1],
+PROFILED_LAUNCHES = {"qkv": [192, 512, 2, 1], "o": [256, 512, 4, 0], "gate_up": [448, 256, 1, 1],
                      "down": [256, 512, 4, 1]}
 REPLAYS = 21                # graph replays per timing; the median is reported
 DEFAULT_COPIES = 24          # distinct layers visited round-robin (see the module docstring)

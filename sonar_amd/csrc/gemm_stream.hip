@@ -681,14 +681,16 @@ __device__ __forceinline__ void copy_weights(const StreamParams& p, const FastLa
                                              char* slot, int lane, int unit_group_shift) {
   const uint4* gq = p.b + (size_t)(unsigned)(strip * p.chunks_per_strip + unit * 4) * 64 + lane;
   lds_void_t* lq = (lds_void_t*)slot;
-  // `nt_weights` (a launch whose workgroups each read their weights once, on a matrix of 20 MB or
-  // more): the copies carry the non-temporal bit, which streams the weights past the L2 and
+  // `nt_weights` (a launch whose workgroups each read their weights once, on a matrix of 10 MB or
+  // more): the copies carry the non-temporal bit, which streams the weights past the caches and
   // leaves the activations and the partial tiles there.  Measured on the four GEMMs of a
-  // Llama-3-8B layer at M = 16, one box, three runs each: no copy with the bit 41.97 us a layer,
-  // the gate / up matrix (59 MB) only 40.96, that and the down matrix (29 MB) 39.76, all four
-  // 40.13 (a copy-only kernel with plain loads on the gate / up matrix: 5.3 -> 5.9 TB/s).
-  // With several blocks of rows the later ones count on finding the chunk in the L2, and those
-  // copies stay plain.
+  // Llama-3-8B layer at M = 16, one box, over 24 sets of weights in turn (no matrix is used again
+  // before 2.7 GB of others): no copy with the bit 42.7 us a layer, the gate / up (59 MB) and the
+  // down matrix (29 MB) 41.6 - 42.2, those and the qkv matrix (12.6 MB) 41.0, all four 41.1
+  // (a copy-only kernel with plain loads on the gate / up matrix: 5.3 -> 5.9 TB/s).  The size
+  // stands for "the model's weights do not fit the caches": matrices of a few MB may well be
+  // found there by the next call.  With several blocks of rows the later ones count on finding
+  // the chunk in the L2, and those copies stay plain.
   constexpr int kNonTemporal = 2;
   if (p.nt_weights) {
     __builtin_amdgcn_global_load_lds((glb_void_t*)gq, lq, 16, 0, kNonTemporal);
@@ -1951,7 +1953,7 @@ int marlin_gemm_any(const void* a, int64_t a_row_stride, void* c, const uint32_t
       p.xcd_ranges = p.slabs == 1 && p.parts % 8 == 0;
     }
     static const bool no_nt = getenv("SONAR_MARLIN_NO_NT_WEIGHTS") != nullptr;
-    p.nt_weights = !no_nt && p.slabs == 1 && size_k * size_n / 2 >= 20 * 1000 * 1000;
+    p.nt_weights = !no_nt && p.slabs == 1 && size_k * size_n / 2 >= 10 * 1000 * 1000;
     g_last_decode_launch[0] = p.grid_parts * p.slabs;
     g_last_decode_launch[1] = half ? 256 : 512;
     g_last_decode_launch[2] = 1 << shift;
