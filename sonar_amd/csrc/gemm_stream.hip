@@ -1701,6 +1701,14 @@ int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   fast_group_shift(num_groups, group_size, unit_group_shift);
   const bool half = (int64_t)p.slabs * n_strips > cu_count();   // small workgroups, three per compute unit
   const int row_blocks = moe_block_size <= 16 ? 1 : 2;
+  // Non-temporal weight copies as in the dense call, where no other workgroup counts on finding the
+  // chunks in the L2: blocks of up to 32 slots (the two halves of a larger block read the same strip).
+  // Mixtral-8x7B experts, two sets of weights in turn, gate / up and down GEMM and the whole layer:
+  // 16 tokens 97.4 / 47.7 / 153.9 -> 90.1 / 48.0 / 143.2 us, 32 tokens 107.9 / 51.8 / 173.5 ->
+  // 108.4 / 46.2 / 161.5, 64 tokens 153.2 / 63.3 / 218.9 -> 150.1 / 62.4 / 215.4; with blocks of 48
+  // slots (128 tokens) the down GEMM went from 90.5 to 104.8 us, with 64 slots nothing moved.
+  static const bool no_nt = getenv("SONAR_MARLIN_NO_NT_WEIGHTS") != nullptr;
+  p.nt_weights = !no_nt && p.sub_blocks == 1 && num_experts * size_k * size_n / 2 >= 10 * 1000 * 1000;
   int rc;
   if (fp4)   // bf16, groups of 32 rows, blocks of at most 16 slots: moe_fast_applies has seen to it
     rc = launch_fast_fp4<true>(p, half, st);
