@@ -1708,7 +1708,10 @@ int moe_fast_gemm(const void* a, void* c, const uint32_t* b, const void* bias, c
   // 108.4 / 46.2 / 161.5, 64 tokens 153.2 / 63.3 / 218.9 -> 150.1 / 62.4 / 215.4; with blocks of 48
   // slots (128 tokens) the down GEMM went from 90.5 to 104.8 us, with 64 slots nothing moved.
   static const bool no_nt = getenv("SONAR_MARLIN_NO_NT_WEIGHTS") != nullptr;
-  p.nt_weights = !no_nt && p.sub_blocks == 1 && num_experts * size_k * size_n / 2 >= 10 * 1000 * 1000;
+  // (and at most two blocks an expert: beyond that the blocks of an expert read its strips again and again,
+  // and the caches are all that keeps those reads from memory)
+  p.nt_weights = !no_nt && p.sub_blocks == 1 && p.slabs <= 2 * num_experts &&
+                 num_experts * size_k * size_n / 2 >= 10 * 1000 * 1000;
   int rc;
   if (fp4)   // bf16, groups of 32 rows, blocks of at most 16 slots: moe_fast_applies has seen to it
     rc = launch_fast_fp4<true>(p, half, st);
